@@ -1,0 +1,383 @@
+"""Pins the CPU oracle (oracle/illatio_oracle.c) without running the reference: closed
+forms, an independent numpy reading of the formats, brute force on integers, and the
+reference's own criterion for the row dots (inspect/iquant-test.lisp:45-53: kernel vs a
+double-precision dot of dequantized values, |diff| / sum|terms| < 1e-6)."""
+import json
+import os
+
+import numpy as np
+import pytest
+
+import np_formats as npf
+import oracle_lib as orc
+from illatio_amd import synth
+
+TYPES = [synth.Q8_0, synth.Q4_K, synth.Q6_K, synth.Q2_K, synth.IQ2_XXS]
+HERE = os.path.dirname(os.path.abspath(__file__))
+
+
+# ---- fp16 (half.lisp) ---------------------------------------------------------------------
+def test_half_to_single_exhaustive():
+    bits = np.arange(65536, dtype=np.uint16)
+    want = bits.view(np.float16).astype(np.float32)
+    got = np.array([orc.half_to_single(int(b)) for b in bits], dtype=np.float32)
+    nan = np.isnan(want)
+    assert np.array_equal(np.isnan(got), nan)
+    assert np.array_equal(got[~nan].view(np.uint32), want[~nan].view(np.uint32))
+
+
+def test_single_to_half_rne():
+    rng = synth.make_rng(11)
+    halves = np.arange(0x7c00, dtype=np.uint16).view(np.float16).astype(np.float32)
+    mids = ((halves[:-1].astype(np.float64) + halves[1:].astype(np.float64)) / 2).astype(np.float32)  # exact ties
+    cand = [halves, mids, np.nextafter(mids, np.float32(np.inf)), np.nextafter(mids, np.float32(-np.inf)),
+            np.array([65504.0, 65519.99, 65520.0, 65536.0, 1e10, 5.9604645e-8, 2.9802322e-8, 2.9802326e-8,
+                      1e-10, 0.0, np.inf], np.float32),
+            rng.standard_normal(20000).astype(np.float32) * np.float32(10.0) ** rng.integers(-9, 6, 20000).astype(np.float32),
+            np.arange(1, 2000, dtype=np.uint32).view(np.float32)]           # single subnormals
+    x = np.concatenate(cand)
+    x = np.concatenate([x, -x])
+    with np.errstate(over="ignore"):
+        want = x.astype(np.float16).view(np.uint16)
+    got = np.array([orc.single_to_half(v) for v in x], dtype=np.uint16)
+    assert np.array_equal(got, want)
+    assert orc.single_to_half(float("nan")) & 0x7c00 == 0x7c00 and orc.single_to_half(float("nan")) & 0x3ff
+
+
+# ---- IQ2_XXS tables --------------------------------------------------------------------------
+def test_iq2xxs_tables_invariants_and_headers():
+    grid, signs = npf.tables()
+    assert grid.size == 256 and signs.size == 128
+    by = (grid[:, None] >> (np.arange(8, dtype=np.uint64) * np.uint64(8))) & np.uint64(0xFF)
+    assert set(np.unique(by).tolist()) == {8, 25, 43}
+    assert len(set(grid.tolist())) == 256
+    for s in range(128):
+        assert signs[s] == s + 128 * (bin(s).count("1") & 1)
+    # both C headers carry the fixture's values
+    import re
+    root = os.path.dirname(HERE)
+    for rel in ("oracle/iq2xxs_tables.h", "illatio_amd/csrc/ilt_iq2xxs_tables.h"):
+        text = open(os.path.join(root, rel)).read()
+        g = [int(h, 16) for h in re.findall(r"0x([0-9a-f]{16})ULL", text)]
+        assert g == grid.tolist(), rel
+        body = text[text.index("ksigns_iq2xs[128]"):]
+        s = [int(v) for v in re.findall(r"\b(\d{1,3})\b", body[body.index("{"):body.index("}")])]
+        assert s == signs.tolist(), rel
+
+
+@pytest.mark.skipif(not os.path.isdir("/root/reference/src"), reason="reference tree not present")
+def test_iq2xxs_tables_match_reference_copies():
+    import importlib.util
+    spec = importlib.util.spec_from_file_location("mk", os.path.join(HERE, "golden", "make_iq2xxs_tables.py"))
+    mk = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mk)
+    grid, signs = npf.tables()
+    lg, ls = mk.lisp_tables("/root/reference/src/iquant.lisp")
+    assert lg == grid.tolist() and ls == signs.tolist()
+    for rel in ("src/cuda/ds4f.cu", "src/metal/ds4f.metal"):
+        cg, cs = mk.c_tables(os.path.join("/root/reference", rel))
+        assert cg == grid.tolist() and cs[:128] == signs.tolist()
+
+
+# ---- scale-min-k4 ------------------------------------------------------------------------------
+def test_scale_min_k4_bitfields():
+    # closed form: 8 six-bit scales then 8 six-bit mins packed in 12 bytes; the low four of
+    # each live in bytes 0..7's low 6 bits, the high four split 4 bits + 2 bits.
+    rng = synth.make_rng(5)
+    for _ in range(300):
+        sc = rng.integers(0, 64, 8)
+        mn = rng.integers(0, 64, 8)
+        q = np.zeros(12, np.uint8)
+        for j in range(4):
+            q[j] = sc[j] | ((sc[j + 4] >> 4) << 6)
+            q[j + 4] = mn[j] | ((mn[j + 4] >> 4) << 6)
+            q[j + 8] = (sc[j + 4] & 0xF) | ((mn[j + 4] & 0xF) << 4)
+        for j in range(8):
+            assert orc.scale_min_k4(j, q) == (sc[j], mn[j])
+
+
+# ---- decoders: bit-exact against the numpy reading, and hand-built blocks ---------------------
+@pytest.mark.parametrize("qtype", TYPES)
+def test_dequant_matches_numpy_reading(qtype):
+    rng = synth.make_rng(100 + qtype)
+    cols = 512
+    w = synth.weights(qtype, 24, cols, rng)
+    got = orc.dequant_rows(qtype, w, cols)
+    want = npf.dequant(qtype, w, cols)
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
+def _one_hot_block(qtype):
+    bb = synth.BLOCK_BYTES[qtype]
+    return np.zeros((1, bb), np.uint8)
+
+
+def test_dequant_hand_built_blocks():
+    h1 = np.array([1.0], np.float16).view(np.uint8)       # fp16 1.0
+    # Q8_0: d=1, q[5] = -3
+    b = _one_hot_block(synth.Q8_0); b[0, 0:2] = h1; b[0, 2 + 5] = np.uint8(256 - 3)
+    y = orc.dequant_rows(synth.Q8_0, b, 32)[0]
+    assert y[5] == -3.0 and np.count_nonzero(y) == 1
+    # Q4_K: d=1, scale of group 3 = 2 (byte 4+3), high nibble of qs[32*1 + 7] = 9 -> weight 64*1+32+7
+    b = _one_hot_block(synth.Q4_K); b[0, 0:2] = h1; b[0, 4 + 3] = 2; b[0, 16 + 32 + 7] = 9 << 4
+    y = orc.dequant_rows(synth.Q4_K, b, 256)[0]
+    assert y[64 + 32 + 7] == 18.0 and np.count_nonzero(y) == 1
+    # Q4_K: dmin=1, min of group 5 = 17 = 0b010001: low 4 bits in byte 4+8+1 high nibble, top 2 in byte 4+5 bits 6-7
+    b = _one_hot_block(synth.Q4_K); b[0, 2:4] = h1; b[0, 4 + 9] = (17 & 0xF) << 4; b[0, 4 + 5] = (17 >> 4) << 6
+    y = orc.dequant_rows(synth.Q4_K, b, 256)[0]
+    assert np.all(y[160:192] == -17.0) and np.count_nonzero(y) == 32
+    # Q6_K: d=1, sc[8+4+1] = -2, weight 128+64+16+3: high nibble of ql[64+16+3], bits 4-5 of qh[32+16+3]
+    b = _one_hot_block(synth.Q6_K); b[0, 208:210] = h1; b[0, 192 + 13] = np.uint8(256 - 2)
+    b[0, 64 + 19] = 0x5 << 4; b[0, 128 + 32 + 19] = 0x2 << 4
+    y = orc.dequant_rows(synth.Q6_K, b, 256)[0]
+    assert y[128 + 64 + 19] == -2.0 * ((0x5 | (0x2 << 4)) - 32)
+    assert np.all(np.delete(y[128 + 64 + 16:128 + 64 + 32], 3) == -2.0 * -32)
+    # Q2_K: d=1, scale byte 8+2*2+1 low nibble 3, quant (bits 4-5) of qs[32+16+9] = 2 -> weight 128+64+16+9
+    b = _one_hot_block(synth.Q2_K); b[0, 80:82] = h1; b[0, 8 + 5] = 3; b[0, 16 + 32 + 16 + 9] = 2 << 4
+    y = orc.dequant_rows(synth.Q2_K, b, 256)[0]
+    assert y[128 + 64 + 16 + 9] == 6.0 and np.count_nonzero(y) == 1
+    # IQ2_XXS: d=1, sub-block 2, LS=3, grid index 1 (=0x080808080808082b) at l=1, sign pattern 1 at l=1
+    grid, signs = npf.tables()
+    b = _one_hot_block(synth.IQ2_XXS); b[0, 0:2] = h1
+    so = 2 + 8 * 2
+    b[0, so + 1] = 1
+    aux = (3 << 28) | (1 << 7)
+    b[0, so + 4:so + 8] = np.array([aux], "<u4").view(np.uint8)
+    y = orc.dequant_rows(synth.IQ2_XXS, b, 256)[0]
+    db = np.float32(1.0) * np.float32(3.5) * np.float32(0.25)
+    seg = y[64 + 8:64 + 16]
+    assert seg[0] == -db * 43 and np.all(seg[1:7] == db * 8) and seg[7] == -db * 8  # ksigns[1] = 129: bits 0 and 7
+    assert np.all(y[64:72] == db * 8)
+
+
+# ---- quantizers ---------------------------------------------------------------------------------
+def test_quantize_q8_closed_form_and_cases():
+    rng = synth.make_rng(3)
+    x = synth.activations(32 * 40, rng)
+    x[0:32] = 0.0                                   # zero block
+    x[32:64] = 0.0; x[40] = -2.5                    # single non-zero
+    x[64:96] = np.arange(32, dtype=np.float32) - 16  # ties: amax 16 -> id = 127/16; 0.5*... exact halves rare
+    for f16 in (True, False):
+        q, s = orc.quantize_q8(x, f16)
+        xb = x.reshape(-1, 32)
+        amax = np.abs(xb).max(axis=1)
+        d = amax / np.float32(127.0)
+        with np.errstate(divide="ignore"):
+            idv = np.where(d == 0, np.float32(0), np.float32(1.0) / d).astype(np.float32)
+        want_q = np.rint(xb * idv[:, None]).astype(np.int8)
+        assert np.array_equal(q.reshape(-1, 32), want_q)
+        want_s = d.astype(np.float16).astype(np.float32) if f16 else d
+        assert np.array_equal(s.view(np.uint32), want_s.view(np.uint32))
+        assert np.all(q[0:32] == 0) and s[0] == 0
+        assert q[40] == -127 and np.count_nonzero(q[32:64]) == 1
+    # round-half-even on exact ties: d = 2/127 -> id = 63.5; x = k/127 -> x*id = k/2
+    x = np.zeros(32, np.float32); x[0] = 2.0
+    idv = np.float32(1.0) / (np.float32(2.0) / np.float32(127.0))
+    for k in range(1, 9):
+        x[k] = np.float32(k + 0.5) / idv
+    q, _ = orc.quantize_q8(x, True)
+    assert np.array_equal(q[1:9], np.rint((x[1:9] * idv)).astype(np.int8))
+
+
+def test_quantize_q8k_closed_form_and_cases():
+    rng = synth.make_rng(4)
+    x = synth.activations(256 * 6, rng)
+    x[0:256] = 0.0                                        # zero block: d = 0, q = 0
+    x[256 + 17] = -9.0                                    # max on a negative value -> iscale positive
+    x[512 + 3] = 7.0; x[512 + 200] = -7.0                 # duplicate magnitude: the first (positive) wins
+    q, d, bs = orc.quantize_q8k(x)
+    assert d[0] == 0 and np.all(q[0:256] == 0) and np.all(bs[0:16] == 0)
+    assert q[256 + 17] == -127 and d[1] == np.float32(1.0) / (np.float32(-127.0) / np.float32(-9.0))
+    assert q[512 + 3] == -127 and q[512 + 200] == 127 and d[2] < 0
+    for b in range(1, 6):
+        xb = x[256 * b:256 * b + 256]
+        i = int(np.argmax(np.abs(xb)))                    # numpy argmax: first of equals
+        isc = np.float32(-127.0) / xb[i]
+        want = np.minimum(127, np.rint(isc * xb)).astype(np.int8)
+        assert np.array_equal(q[256 * b:256 * b + 256], want)
+        assert d[b] == np.float32(1.0) / isc
+        assert np.array_equal(bs[16 * b:16 * b + 16], want.astype(np.int32).reshape(16, 16).sum(axis=1))
+        assert np.max(np.abs(xb - d[b] * want.astype(np.float32))) <= abs(d[b]) * 0.5 * 1.0001 + 1e-6
+
+
+# ---- integer block sums by brute force; floats against a double-precision dot ----------------------
+def _quantized_act(qtype, cols, rng):
+    x = (rng.random(cols, dtype=np.float32) * 2 - 1).astype(np.float32)      # U(-1,1) as iquant-test.lisp:37-38
+    if qtype == synth.Q8_0:
+        q, s = orc.quantize_q8(x, True)
+        return x, q, s, None, np.repeat(s, 32)
+    q, d, bs = orc.quantize_q8k(x)
+    return x, q, d, bs, np.repeat(d, 256)
+
+
+@pytest.mark.parametrize("qtype", TYPES)
+def test_row_dot_integers_and_double_dot(qtype):
+    rng = synth.make_rng(200 + qtype)
+    cols, rows = 2048, 48
+    w = synth.weights(qtype, rows, cols, rng)
+    x, xq, xs, bs, xscale = _quantized_act(qtype, cols, rng)
+    f = npf.decode(qtype, w, cols)
+    deq = npf.dequant(qtype, w, cols).astype(np.float64)
+    xi = xq.astype(np.int64)
+    worst = 0.0
+    for r in range(rows):
+        q = f["q"][r].astype(np.int64)
+        res = orc.row_dot(qtype, w[r], cols, xq, xs, bs, ints=True)
+        if qtype == synth.Q8_0:
+            assert np.array_equal(res[1], (q * xi).reshape(-1, 32).sum(axis=1))
+        elif qtype == synth.Q4_K:
+            assert np.array_equal(res[1], (q * f["isc"][r] * xi).reshape(-1, 256).sum(axis=1))
+            assert np.array_equal(res[2], (f["imn"][r].astype(np.int64) * xi).reshape(-1, 256).sum(axis=1))
+        elif qtype == synth.Q6_K:
+            assert np.array_equal(res[1], (q * f["isc"][r] * xi).reshape(-1, 256).sum(axis=1))
+            assert np.array_equal(res[2], (f["isc"][r].astype(np.int64) * xi).reshape(-1, 256).sum(axis=1))
+        elif qtype == synth.Q2_K:
+            assert np.array_equal(res[1], (q * f["isc"][r] * xi).reshape(-1, 256).sum(axis=1))
+            assert np.array_equal(res[2], (f["imn"][r].astype(np.int64) * xi).reshape(-1, 256).sum(axis=1))
+        else:
+            assert np.array_equal(res[1], (q * xi).reshape(-1, 32).sum(axis=1))
+        terms = deq[r] * xscale.astype(np.float64) * xi
+        rel = abs(float(res[0]) - terms.sum()) / np.abs(terms).sum()
+        worst = max(worst, rel)
+        if qtype in (synth.Q2_K, synth.IQ2_XXS):
+            v2 = orc.row_dot(qtype, w[r], cols, xq, xs, bs, order="avx2")
+            assert abs(float(v2) - terms.sum()) / np.abs(terms).sum() < 1e-6
+    assert worst < 1e-6, worst
+
+
+def test_row_dot_sign_and_term_sensitivity():
+    """A dropped min term, a wrong sign or a swapped d/dmin moves the result far beyond 1e-6:
+    the double-dot check above would catch it.  Here: zero activations give zero, and scaling
+    the activation scale scales the result exactly (power of two)."""
+    rng = synth.make_rng(9)
+    cols = 1024
+    for qtype in TYPES:
+        w = synth.weights(qtype, 2, cols, rng)
+        x, xq, xs, bs, _ = _quantized_act(qtype, cols, rng)
+        v = orc.row_dot(qtype, w[0], cols, xq, xs, bs)
+        v4 = orc.row_dot(qtype, w[0], cols, xq, xs * np.float32(4.0), bs)
+        assert np.float32(v4) == np.float32(v) * np.float32(4.0)
+        z = orc.row_dot(qtype, w[0], cols, np.zeros_like(xq), xs, None if bs is None else np.zeros_like(bs))
+        assert z == 0.0
+
+
+@pytest.mark.parametrize("qtype", TYPES)
+def test_matmul_is_per_token_row_dot(qtype):
+    """batch.lisp:10-12: a batched product is bit-identical to one token at a time, at any thread count."""
+    rng = synth.make_rng(300 + qtype)
+    rows, cols, ntok = 64, 512, 5
+    w = synth.weights(qtype, rows, cols, rng)
+    x = synth.activations((ntok, cols), rng)
+    a = orc.matmul(qtype, w, rows, cols, x, nthreads=1)
+    b = orc.matmul(qtype, w, rows, cols, x, nthreads=3)
+    assert np.array_equal(a.view(np.uint32), b.view(np.uint32))
+    for t in range(ntok):
+        one = orc.matmul(qtype, w, rows, cols, x[t])
+        assert np.array_equal(one.view(np.uint32), a[t].view(np.uint32))
+    if qtype == synth.Q8_0:
+        q, s = orc.quantize_q8(x[2], True)
+        v = orc.row_dot(qtype, w[7], cols, q, s)
+    else:
+        q, d, bs = orc.quantize_q8k(x[2])
+        v = orc.row_dot(qtype, w[7], cols, q, d, bs)
+    assert np.float32(v) == a[2, 7]
+
+
+# ---- silu / softplus: against correctly rounded values ----------------------------------------------
+def test_activation_functions_correctly_rounded():
+    rng = synth.make_rng(6)
+    xs = np.concatenate([rng.standard_normal(4000).astype(np.float32) * 4, np.array([0, -0.0, 20, 20.5, -20, -20.5, 30, -30, 88, -88], np.float32)])
+    ld = np.longdouble
+    for x in xs:
+        e = np.exp(ld(-abs(x)))
+        sig = (ld(1) / (ld(1) + e)) if x >= 0 else e / (ld(1) + e)
+        # the reference rounds exp to single first, then divides in single
+        ef = np.float32(np.exp(ld(-x) if x >= 0 else ld(x)))
+        want = (np.float32(1) / (np.float32(1) + ef)) if x >= 0 else ef / (np.float32(1) + ef)
+        assert np.float32(orc.sigmoid(x)) == want
+        assert abs(float(want) - float(sig)) <= 1.2e-7
+        assert np.float32(orc.silu(x)) == np.float32(x) * want
+        if x > 20:
+            sp = np.float32(x)
+        elif x < -20:
+            sp = np.float32(np.exp(ld(x)))
+        else:
+            sp = np.float32(np.log(ld(np.float32(1) + np.float32(np.exp(ld(x))))))
+        assert np.float32(orc.softplus(x)) == sp
+
+
+# ---- routing -------------------------------------------------------------------------------------
+def test_route_against_stable_sort():
+    rng = synth.make_rng(7)
+    for trial in range(60):
+        ne, nu = (256, 6) if trial % 2 else (16, 3)
+        logits = rng.standard_normal(ne).astype(np.float32)
+        if trial % 3 == 0:
+            logits[rng.integers(0, ne, ne // 2)] = logits[0]            # many exact ties
+        bias = None if trial % 4 else (rng.standard_normal(ne).astype(np.float32) * 0.1)
+        sel, w = orc.route(logits, nu, 1.5, bias)
+        p = np.array([np.sqrt(np.float32(orc.softplus(v))) for v in logits], np.float32)
+        s = p if bias is None else p + bias
+        order = sorted(range(ne), key=lambda i: (-float(s[i]), i))[:nu]
+        assert sel.tolist() == order
+        tot = np.float32(0)
+        for i in order:
+            tot = np.float32(tot + p[i])
+        want = (p[order] / tot) * np.float32(1.5)
+        assert np.array_equal(w, want.astype(np.float32))
+        assert abs(float(w.sum()) - 1.5) < 1e-5
+
+
+# ---- the experts ----------------------------------------------------------------------------------
+def _experts(rng, ne, d, ff):
+    gate = synth.weights(synth.IQ2_XXS, ne * ff, d, rng)
+    up = synth.weights(synth.IQ2_XXS, ne * ff, d, rng)
+    down = synth.weights(synth.Q2_K, ne * d, ff, rng)
+    return gate, up, down
+
+
+def test_moe_routed_composition_and_order():
+    rng = synth.make_rng(8)
+    ne, d, ff, nu = 8, 512, 256, 3
+    gate, up, down = _experts(rng, ne, d, ff)
+    norm = synth.activations(d, rng)
+    sel = np.array([5, 1, 6], np.int32)
+    w = np.array([0.7, 0.5, 0.3], np.float32)
+    for clamp in (0.0, 0.05):
+        moe, mid = orc.moe_routed(gate, up, down, d, ff, sel, w, clamp, norm)
+        xq, xd, xbs = orc.quantize_q8k(norm)
+        for slot in (0, 2):
+            e = sel[slot]
+            for r in (0, 17, ff - 1):
+                g = np.float32(orc.row_dot(synth.IQ2_XXS, gate[e * ff + r], d, xq, xd))
+                u = np.float32(orc.row_dot(synth.IQ2_XXS, up[e * ff + r], d, xq, xd))
+                if clamp > 1e-6:
+                    g = min(g, np.float32(clamp)); u = max(np.float32(-clamp), min(u, np.float32(clamp)))
+                want = (np.float32(orc.silu(g)) * u) * w[slot]
+                assert mid[slot, r] == want
+        for r in (0, 100, d - 1):
+            acc = np.float32(0)
+            for slot in range(nu):
+                q, dd, bs = orc.quantize_q8k(mid[slot])
+                acc = np.float32(acc + np.float32(orc.row_dot(synth.Q2_K, down[sel[slot] * d + r], ff, q, dd, bs)))
+            assert moe[r] == acc
+        m3, _ = orc.moe_routed(gate, up, down, d, ff, sel, w, clamp, norm, nthreads=3)
+        assert np.array_equal(m3.view(np.uint32), moe.view(np.uint32))
+
+
+def test_moe_chunk_equals_token_at_a_time():
+    """ds4f.lisp:1128-1130: a layer-major chunk gives the decode's bits."""
+    rng = synth.make_rng(10)
+    ne, d, ff, nu, n = 8, 512, 256, 3, 7
+    gate, up, down = _experts(rng, ne, d, ff)
+    sg = synth.weights(synth.Q8_0, ff, d, rng); su = synth.weights(synth.Q8_0, ff, d, rng)
+    sd = synth.weights(synth.Q8_0, d, ff, rng)
+    norms = synth.activations((n, d), rng)
+    logits = synth.zipf_router_logits(n, ne, rng)
+    shared = np.stack([orc.moe_shared(sg, su, sd, d, ff, 0.0, norms[t]) for t in range(n)])
+    out, sel, w, counts = orc.moe_chunk(gate, up, down, d, ff, ne, nu, 1.5, 0.0, logits, norms, shared, nthreads=2)
+    assert counts.sum() == n * nu and np.array_equal(counts, np.bincount(sel.ravel(), minlength=ne))
+    for t in range(n):
+        one, s1, w1 = orc.moe_token(gate, up, down, sg, su, sd, d, ff, ne, nu, 1.5, 0.0, logits[t], norms[t])
+        assert s1.tolist() == sel[t].tolist() and np.array_equal(w1, w[t])
+        assert np.array_equal(one.view(np.uint32), out[t].view(np.uint32))
