@@ -1,0 +1,351 @@
+// The C ABI of libillatio_hip.so (declared in include/illatio_hip.h): the driver calls the
+// reference's src/cuda.lisp makes, typed entry points for the kernels, and launch by name.
+// Host code only validates shapes and picks launch geometry; it does no arithmetic on data.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <string.h>
+
+#include "../../include/illatio_hip.h"
+#include "ilt_kernels.h"
+
+#define ILT_TRY(expr) do { hipError_t e_ = (expr); if (e_ != hipSuccess) return (int)e_; } while (0)
+#define ILT_REQUIRE(cond) do { if (!(cond)) return (int)hipErrorInvalidValue; } while (0)
+
+static inline hipStream_t S(uint64_t s) { return (hipStream_t)(uintptr_t)s; }
+static inline hipEvent_t E(uint64_t e) { return (hipEvent_t)(uintptr_t)e; }
+
+static int block_weights(int fmt) { return fmt == ILT_Q8_0 ? 32 : 256; }
+static int block_bytes(int fmt) {
+  switch (fmt) { case ILT_Q8_0: return 34; case ILT_Q2_K: return 84; case ILT_Q4_K: return 144;
+                 case ILT_Q6_K: return 210; case ILT_IQ2_XXS: return 66; }
+  return 0;
+}
+// kquant.cu's numbering of the K-quants (cuda-dense.lisp:18-20) -> GGUF's
+static int kquant_type(int code) { return code == 0 ? ILT_Q4_K : code == 2 ? ILT_Q6_K : 0; }
+
+namespace {
+struct Args {
+  void** p;
+  template <class T> T ptr(int i) const { return (T)(uintptr_t)(*(const uint64_t*)p[i]); }
+  int i32(int i) const { return *(const int32_t*)p[i]; }
+  long long i64(int i) const { return *(const int64_t*)p[i]; }
+  float f32(int i) const { return *(const float*)p[i]; }
+};
+}  // namespace
+
+extern "C" {
+
+int ilt_init(void) { return (int)hipInit(0); }
+
+int ilt_device_count(int* n) { ILT_REQUIRE(n); return (int)hipGetDeviceCount(n); }
+
+int ilt_device_get_info(int index, ilt_device_info* out) {
+  ILT_REQUIRE(out);
+  hipDeviceProp_t p;
+  ILT_TRY(hipGetDeviceProperties(&p, index));
+  memset(out, 0, sizeof(*out));
+  snprintf(out->name, sizeof(out->name), "%s (%s)", p.name, p.gcnArchName);
+  out->arch = 90;
+  out->total_memory = p.totalGlobalMem;
+  out->max_shared = (int)p.sharedMemPerBlock;
+  out->compute_units = p.multiProcessorCount;
+  out->wave_size = p.warpSize;
+  out->numa_node = -1;
+  char path[128];
+  snprintf(path, sizeof(path), "/sys/bus/pci/devices/%04x:%02x:%02x.0/numa_node", p.pciDomainID, p.pciBusID, p.pciDeviceID);
+  if (FILE* f = fopen(path, "r")) { int node; if (fscanf(f, "%d", &node) == 1) out->numa_node = node; fclose(f); }
+  return ILT_OK;
+}
+
+int ilt_set_device(int index) { return (int)hipSetDevice(index); }
+
+const char* ilt_error_string(int code) {
+  if (code == ILT_OK) return "no error";
+  return hipGetErrorString((hipError_t)code);
+}
+
+int ilt_stream_create(uint64_t* stream, unsigned flags) {
+  ILT_REQUIRE(stream);
+  hipStream_t s;
+  ILT_TRY(hipStreamCreateWithFlags(&s, (flags & 1) ? hipStreamNonBlocking : hipStreamDefault));
+  *stream = (uint64_t)(uintptr_t)s;
+  return ILT_OK;
+}
+int ilt_stream_destroy(uint64_t stream) { return (int)hipStreamDestroy(S(stream)); }
+int ilt_stream_sync(uint64_t stream) { return (int)hipStreamSynchronize(S(stream)); }
+int ilt_stream_wait_event(uint64_t stream, uint64_t event) { return (int)hipStreamWaitEvent(S(stream), E(event), 0); }
+
+int ilt_event_create(uint64_t* event, unsigned flags) {
+  ILT_REQUIRE(event);
+  hipEvent_t e;
+  ILT_TRY(hipEventCreateWithFlags(&e, (flags & 2) ? hipEventDisableTiming : hipEventDefault));
+  *event = (uint64_t)(uintptr_t)e;
+  return ILT_OK;
+}
+int ilt_event_destroy(uint64_t event) { return (int)hipEventDestroy(E(event)); }
+int ilt_event_record(uint64_t event, uint64_t stream) { return (int)hipEventRecord(E(event), S(stream)); }
+int ilt_event_query(uint64_t event) {
+  hipError_t e = hipEventQuery(E(event));
+  if (e == hipErrorNotReady) { (void)hipGetLastError(); return ILT_NOT_READY; }
+  return (int)e;
+}
+int ilt_event_elapsed_ms(uint64_t start, uint64_t stop, float* ms) { ILT_REQUIRE(ms); return (int)hipEventElapsedTime(ms, E(start), E(stop)); }
+
+int ilt_malloc(uint64_t* dptr, uint64_t bytes) {
+  ILT_REQUIRE(dptr);
+  void* p = nullptr;
+  ILT_TRY(hipMalloc(&p, bytes < 256 ? 256 : bytes));
+  *dptr = (uint64_t)(uintptr_t)p;
+  return ILT_OK;
+}
+int ilt_free(uint64_t dptr) { return dptr ? (int)hipFree((void*)(uintptr_t)dptr) : ILT_OK; }
+int ilt_memset_async(uint64_t dptr, int byte, uint64_t bytes, uint64_t stream) {
+  return (int)hipMemsetAsync((void*)(uintptr_t)dptr, byte, bytes, S(stream));
+}
+int ilt_mem_info(uint64_t* free_bytes, uint64_t* total_bytes) {
+  ILT_REQUIRE(free_bytes && total_bytes);
+  size_t f = 0, t = 0;
+  ILT_TRY(hipMemGetInfo(&f, &t));
+  *free_bytes = f; *total_bytes = t;
+  return ILT_OK;
+}
+int ilt_memcpy_htod_async(uint64_t dst, const void* src, uint64_t bytes, uint64_t stream) {
+  return (int)hipMemcpyAsync((void*)(uintptr_t)dst, src, bytes, hipMemcpyHostToDevice, S(stream));
+}
+int ilt_memcpy_dtoh_async(void* dst, uint64_t src, uint64_t bytes, uint64_t stream) {
+  return (int)hipMemcpyAsync(dst, (const void*)(uintptr_t)src, bytes, hipMemcpyDeviceToHost, S(stream));
+}
+int ilt_memcpy_dtod_async(uint64_t dst, uint64_t src, uint64_t bytes, uint64_t stream) {
+  return (int)hipMemcpyAsync((void*)(uintptr_t)dst, (const void*)(uintptr_t)src, bytes, hipMemcpyDeviceToDevice, S(stream));
+}
+int ilt_host_alloc(uint64_t* hptr, uint64_t bytes, unsigned flags) {
+  ILT_REQUIRE(hptr);
+  void* p = nullptr;
+  unsigned f = 0;
+  if (flags & 1) f |= hipHostMallocPortable;
+  if (flags & 2) f |= hipHostMallocMapped;
+  ILT_TRY(hipHostMalloc(&p, bytes < 64 ? 64 : bytes, f));
+  *hptr = (uint64_t)(uintptr_t)p;
+  return ILT_OK;
+}
+int ilt_host_free(uint64_t hptr) { return (int)hipHostFree((void*)(uintptr_t)hptr); }
+int ilt_host_register(void* p, uint64_t bytes, unsigned flags) {
+  unsigned f = 0;
+  if (flags & 1) f |= hipHostRegisterPortable;
+  if (flags & 2) f |= hipHostRegisterMapped;
+  return (int)hipHostRegister(p, bytes, f);
+}
+int ilt_host_unregister(void* p) { return (int)hipHostUnregister(p); }
+
+// ---- kernels ----------------------------------------------------------------------------------
+
+int ilt_repack_q8(uint64_t stream, const void* raw, void* qs, void* d, int64_t nblocks) {
+  ILT_REQUIRE(nblocks >= 0 && (nblocks == 0 || (raw && qs && d)));
+  return (int)ilt_k_repack_q8((const uint8_t*)raw, (int8_t*)qs, (uint16_t*)d, nblocks, S(stream));
+}
+
+int ilt_repack_q6k(uint64_t stream, const void* raw, void* out, int64_t nblocks) {
+  ILT_REQUIRE(nblocks >= 0 && (nblocks == 0 || (raw && out)));
+  return (int)ilt_k_copy_bytes((const uint8_t*)raw, (uint8_t*)out, nblocks * 210, S(stream));
+}
+
+int ilt_quant_q8(uint64_t stream, const float* x, int8_t* xq, float* xs, int32_t* xsum, int64_t nblocks) {
+  ILT_REQUIRE(nblocks >= 0 && (nblocks == 0 || (x && xq && xs)));
+  return (int)ilt_k_quant_q8(x, xq, xs, xsum, nblocks, 1, S(stream));
+}
+
+int ilt_d4_quant(uint64_t stream, const float* x, int8_t* xq, float* xs, int nblocks) {
+  ILT_REQUIRE(nblocks >= 0 && (nblocks == 0 || (x && xq && xs)));
+  return (int)ilt_k_quant_q8(x, xq, xs, nullptr, nblocks, 0, S(stream));
+}
+
+int ilt_quant_q8k(uint64_t stream, const float* x, int8_t* xq, float* xd, int32_t* bsums, int64_t nblocks) {
+  ILT_REQUIRE(nblocks >= 0 && (nblocks == 0 || (x && xq && xd && bsums)));
+  return (int)ilt_k_quant_q8k(x, xq, xd, bsums, nblocks, S(stream));
+}
+
+static int gemv_dense(uint64_t stream, int fmt, const void* w, const uint16_t* wd, const int8_t* xq, const float* xs,
+                      const int32_t* bsums, float* out, const float* bias, int rows, int cols, int acc, int group_rows) {
+  ILT_REQUIRE(fmt && rows >= 0 && cols > 0 && cols % block_weights(fmt) == 0);
+  if (rows == 0) return ILT_OK;
+  ILT_REQUIRE(w && xq && xs && out && (fmt == ILT_Q8_0 ? wd != nullptr : bsums != nullptr));
+  ILT_REQUIRE(((uintptr_t)w & 15) == 0 && ((uintptr_t)xq & 15) == 0);
+  IltGemvParams p = {};
+  p.w = (const uint8_t*)w; p.wd = wd; p.rows = rows; p.cols = cols;
+  p.row_bytes = fmt == ILT_Q8_0 ? cols : cols / 256 * block_bytes(fmt);
+  p.xq = xq; p.xs = xs; p.bsums = bsums; p.y = out; p.bias = bias; p.acc = acc;
+  p.rw = ilt_gemv_pick_rw(fmt, rows, cols, 1);
+  if (group_rows > 0 && group_rows < rows) {
+    ILT_REQUIRE(rows % group_rows == 0);
+    while (p.rw > 1 && group_rows % p.rw) p.rw >>= 1;
+    p.group_rows = group_rows;
+  }
+  return (int)ilt_gemv_launch(fmt, p, 1, S(stream));
+}
+
+int ilt_mv_q8(uint64_t stream, const int8_t* wq, const uint16_t* wd, const int8_t* xq, const float* xs, float* out,
+              const float* bias, int rows, int cols, int acc) {
+  return gemv_dense(stream, ILT_Q8_0, wq, wd, xq, xs, nullptr, out, bias, rows, cols, acc, 0);
+}
+
+int ilt_mv_q8_3(uint64_t stream, const int8_t* q0, const uint16_t* d0, const int8_t* q1, const uint16_t* d1,
+                const int8_t* q2, const uint16_t* d2, const int8_t* xq, const float* xs, float* o0, float* o1, float* o2,
+                const float* b0, const float* b1, const float* b2, int r0, int r1, int r2, int cols) {
+  int e = gemv_dense(stream, ILT_Q8_0, q0, d0, xq, xs, nullptr, o0, b0, r0, cols, 0, 0);
+  if (e) return e;
+  e = gemv_dense(stream, ILT_Q8_0, q1, d1, xq, xs, nullptr, o1, b1, r1, cols, 0, 0);
+  if (e) return e;
+  return gemv_dense(stream, ILT_Q8_0, q2, d2, xq, xs, nullptr, o2, b2, r2, cols, 0, 0);
+}
+
+int ilt_mv_k(uint64_t stream, int type, const void* w, const int8_t* xq, const float* xd, const int32_t* bsums, float* out,
+             const float* bias, int rows, int cols, int acc) {
+  return gemv_dense(stream, kquant_type(type), w, nullptr, xq, xd, bsums, out, bias, rows, cols, acc, 0);
+}
+
+int ilt_d4_mvq8(uint64_t stream, int rows, int cols, int group_rows, const int8_t* wq, const uint16_t* wd,
+                const int8_t* xq, const float* xs, float* y) {
+  ILT_REQUIRE(group_rows > 0);
+  return gemv_dense(stream, ILT_Q8_0, wq, wd, xq, xs, nullptr, y, nullptr, rows, cols, 0, group_rows);
+}
+
+static int gemv_experts(uint64_t stream, int fmt, int ncols, int nrows, int row_bytes, int64_t add, int x_stride,
+                        int y_stride, const uint64_t* ptrs, int nz, const int8_t* xq, const float* xd,
+                        const int32_t* bsums, float* dst) {
+  ILT_REQUIRE(nrows >= 0 && nz >= 0 && ncols > 0 && ncols % 256 == 0 && row_bytes == ncols / 256 * block_bytes(fmt));
+  if (nrows == 0 || nz == 0) return ILT_OK;
+  ILT_REQUIRE(ptrs && xq && xd && (bsums || fmt == ILT_IQ2_XXS) && dst && add >= 0 && (add & 1) == 0 && x_stride % 256 == 0 && x_stride >= 0);
+  IltGemvParams p = {};
+  p.ptrs = ptrs; p.add = add; p.rows = nrows; p.cols = ncols; p.row_bytes = row_bytes;
+  p.xq = xq; p.xs = xd; p.bsums = bsums; p.x_stride = x_stride; p.y = dst; p.y_stride = y_stride;
+  p.rw = ilt_gemv_pick_rw(fmt, nrows, ncols, nz);
+  return (int)ilt_gemv_launch(fmt, p, nz, S(stream));
+}
+
+int ilt_d4_mv_iq2_xxs(uint64_t stream, int ncols, int nrows, int row_bytes, int64_t add, int x_stride, int y_stride,
+                      const uint64_t* ptrs, int nz, const int8_t* xq, const float* xd, float* dst) {
+  return gemv_experts(stream, ILT_IQ2_XXS, ncols, nrows, row_bytes, add, x_stride, y_stride, ptrs, nz, xq, xd,
+                      nullptr, dst);
+}
+
+int ilt_d4_mv_q2_k(uint64_t stream, int ncols, int nrows, int row_bytes, int64_t add, int x_stride, int y_stride,
+                   const uint64_t* ptrs, int nz, const int8_t* xq, const float* xd, const int32_t* bsums, float* dst) {
+  return gemv_experts(stream, ILT_Q2_K, ncols, nrows, row_bytes, add, x_stride, y_stride, ptrs, nz, xq, xd, bsums, dst);
+}
+
+int ilt_dequant_rows(uint64_t stream, int gguf_type, const void* w, const uint16_t* wd, const int32_t* rows_idx,
+                     int64_t nrows, int cols, float* out) {
+  ILT_REQUIRE(block_bytes(gguf_type) && cols > 0 && cols % block_weights(gguf_type) == 0 && nrows >= 0);
+  if (nrows == 0) return ILT_OK;
+  ILT_REQUIRE(w && out && (gguf_type != ILT_Q8_0 || wd));
+  const long long rb = gguf_type == ILT_Q8_0 ? cols : (long long)cols / 256 * block_bytes(gguf_type);
+  return (int)ilt_k_dequant_rows(gguf_type, (const uint8_t*)w, wd, rows_idx, nrows, cols, rb, out, S(stream));
+}
+
+int ilt_embed_q8(uint64_t stream, const int8_t* qs, const uint16_t* d, const int32_t* tokens, float* out, int cols, int n) {
+  return ilt_dequant_rows(stream, ILT_Q8_0, qs, d, tokens, n, cols, out);
+}
+
+int ilt_embed_k(uint64_t stream, int type, const void* w, const int32_t* tokens, float* out, int cols, int n) {
+  ILT_REQUIRE(kquant_type(type));
+  return ilt_dequant_rows(stream, kquant_type(type), w, nullptr, tokens, n, cols, out);
+}
+
+int ilt_d4_route(uint64_t stream, int ne, int nu, int hash, float scale, int has_bias, const float* logits,
+                 const float* bias, const int32_t* tid2eid, const uint32_t* tokens, uint32_t* sel, float* wout, int ntok) {
+  ILT_REQUIRE(ntok >= 0 && (ntok == 0 || (logits && sel && wout)));
+  ILT_REQUIRE(!has_bias || bias);
+  ILT_REQUIRE(hash != 1 || (tid2eid && tokens));
+  return (int)ilt_k_route(ne, nu, hash, scale, has_bias, logits, bias, tid2eid, tokens, sel, wout, ntok, S(stream));
+}
+
+int ilt_d4_group_zero(uint64_t stream, int ne, uint32_t* counts) {
+  ILT_REQUIRE(ne > 0 && counts);
+  return (int)ilt_k_group_zero(ne, counts, S(stream));
+}
+int ilt_d4_group_count(uint64_t stream, int n, int ne, int nu, const uint32_t* sel, uint32_t* counts, uint32_t* rank) {
+  ILT_REQUIRE(n >= 0 && (n == 0 || (sel && counts && rank)));
+  return (int)ilt_k_group_count(n, ne, nu, sel, counts, rank, S(stream));
+}
+int ilt_d4_group_scan(uint64_t stream, int n, int ne, int nu, const uint32_t* counts, uint32_t* bases) {
+  ILT_REQUIRE(ne > 0 && counts && bases);
+  return (int)ilt_k_group_scan(n, ne, nu, counts, bases, S(stream));
+}
+int ilt_d4_group_scatter(uint64_t stream, int n, int ne, int nu, const uint32_t* sel, const uint32_t* rank,
+                         const uint32_t* bases, const float* w, uint32_t* rmap, uint32_t* smap, float* wrow) {
+  ILT_REQUIRE(n >= 0 && nu > 0 && (n == 0 || (sel && rank && bases && w && rmap && smap && wrow)));
+  return (int)ilt_k_group_scatter(n, ne, nu, sel, rank, bases, w, rmap, smap, wrow, S(stream));
+}
+int ilt_d4_gather_rows(uint64_t stream, int d, int nrows, const float* src, const uint32_t* map, float* x) {
+  ILT_REQUIRE(d > 0 && nrows >= 0 && (nrows == 0 || (src && map && x)));
+  return (int)ilt_k_gather_rows(d, nrows, src, map, x, S(stream));
+}
+int ilt_d4_swiglu_w(uint64_t stream, int n, int ff, float clamp, const float* g, const float* u, const float* w,
+                    float* mid, int8_t* xq, float* xs) {
+  ILT_REQUIRE(n >= 0 && ff > 0 && (n == 0 || (g && u && w && mid)) && (!xq || xs));
+  return (int)ilt_k_swiglu_w(n, ff, clamp, g, u, w, mid, xq, xs, S(stream));
+}
+int ilt_d4_moe_sum(uint64_t stream, int d, int k, const float* down, const float* shared_, float* moe, const uint32_t* perm) {
+  ILT_REQUIRE(d > 0 && k >= 0 && down && moe);
+  return (int)ilt_k_moe_sum(d, k, down, shared_, moe, perm, S(stream));
+}
+int ilt_d4_moe_sum_rows(uint64_t stream, int d, int nu, int ntok, const float* down, const uint32_t* map,
+                        const float* shared_, float* moe) {
+  ILT_REQUIRE(d > 0 && nu > 0 && ntok >= 0 && (ntok == 0 || (down && map && moe)));
+  return (int)ilt_k_moe_sum_rows(d, nu, ntok, down, map, shared_, moe, S(stream));
+}
+
+// ---- launch by name ---------------------------------------------------------------------------
+int ilt_launch(const char* kernel, unsigned gx, unsigned gy, unsigned gz, unsigned bx, unsigned by, unsigned bz,
+               unsigned shared_bytes, uint64_t stream, void** params) {
+  ILT_REQUIRE(kernel && params);
+  (void)gy; (void)bx; (void)by; (void)bz; (void)shared_bytes;
+  const Args a = { params };
+  typedef const int8_t* ci8; typedef const uint16_t* cu16; typedef const float* cf; typedef const uint32_t* cu32;
+#define K(name) if (!strcmp(kernel, name))
+  K("repack_q8") return ilt_repack_q8(stream, a.ptr<const void*>(0), a.ptr<void*>(1), a.ptr<void*>(2), a.i64(3));
+  K("repack_q6k") return ilt_repack_q6k(stream, a.ptr<const void*>(0), a.ptr<void*>(1), a.i64(2));
+  K("quant_q8") return ilt_quant_q8(stream, a.ptr<cf>(0), a.ptr<int8_t*>(1), a.ptr<float*>(2), a.ptr<int32_t*>(3), a.i64(4));
+  K("d4_quant") return ilt_d4_quant(stream, a.ptr<cf>(0), a.ptr<int8_t*>(1), a.ptr<float*>(2), a.i32(3));
+  K("quant_q8k") return ilt_quant_q8k(stream, a.ptr<cf>(0), a.ptr<int8_t*>(1), a.ptr<float*>(2), a.ptr<int32_t*>(3), a.i64(4));
+  K("mv_q8") return ilt_mv_q8(stream, a.ptr<ci8>(0), a.ptr<cu16>(1), a.ptr<ci8>(2), a.ptr<cf>(3), a.ptr<float*>(4),
+                              a.ptr<cf>(5), a.i32(6), a.i32(7), a.i32(8));
+  K("mv_q8_3") return ilt_mv_q8_3(stream, a.ptr<ci8>(0), a.ptr<cu16>(1), a.ptr<ci8>(2), a.ptr<cu16>(3), a.ptr<ci8>(4),
+                                  a.ptr<cu16>(5), a.ptr<ci8>(6), a.ptr<cf>(7), a.ptr<float*>(8), a.ptr<float*>(9),
+                                  a.ptr<float*>(10), a.ptr<cf>(11), a.ptr<cf>(12), a.ptr<cf>(13), a.i32(14), a.i32(15),
+                                  a.i32(16), a.i32(17));
+  K("mv_k") return ilt_mv_k(stream, a.i32(0), a.ptr<const void*>(1), a.ptr<ci8>(2), a.ptr<cf>(3), a.ptr<const int32_t*>(4),
+                            a.ptr<float*>(5), a.ptr<cf>(6), a.i32(7), a.i32(8), a.i32(9));
+  K("d4_mvq8") return ilt_d4_mvq8(stream, a.i32(0), a.i32(1), a.i32(2), a.ptr<ci8>(3), a.ptr<cu16>(4), a.ptr<ci8>(5),
+                                  a.ptr<cf>(6), a.ptr<float*>(7));
+  K("d4_mv_iq2_xxs") {
+    ILT_REQUIRE(a.ptr<const void*>(7) == nullptr);
+    return ilt_d4_mv_iq2_xxs(stream, a.i32(0), a.i32(1), a.i32(2), a.i64(3), a.i32(4), a.i32(5), a.ptr<const uint64_t*>(6),
+                             (int)gz, a.ptr<ci8>(8), a.ptr<cf>(10), a.ptr<float*>(9));
+  }
+  K("d4_mv_q2_k") {
+    ILT_REQUIRE(a.ptr<const void*>(7) == nullptr);
+    return ilt_d4_mv_q2_k(stream, a.i32(0), a.i32(1), a.i32(2), a.i64(3), a.i32(4), a.i32(5), a.ptr<const uint64_t*>(6),
+                          (int)gz, a.ptr<ci8>(8), a.ptr<cf>(10), a.ptr<const int32_t*>(11), a.ptr<float*>(9));
+  }
+  K("embed_q8") return ilt_embed_q8(stream, a.ptr<ci8>(0), a.ptr<cu16>(1), a.ptr<const int32_t*>(2), a.ptr<float*>(3), a.i32(4), (int)gx);
+  K("embed_k") return ilt_embed_k(stream, a.i32(0), a.ptr<const void*>(1), a.ptr<const int32_t*>(2), a.ptr<float*>(3), a.i32(4), (int)gx);
+  K("d4_route") return ilt_d4_route(stream, a.i32(0), a.i32(1), a.i32(2), a.f32(3), a.i32(4), a.ptr<cf>(5), a.ptr<cf>(6),
+                                    a.ptr<const int32_t*>(7), a.ptr<cu32>(8), a.ptr<uint32_t*>(9), a.ptr<float*>(10), (int)gx);
+  K("d4_group_zero") return ilt_d4_group_zero(stream, a.i32(0), a.ptr<uint32_t*>(1));
+  K("d4_group_count") return ilt_d4_group_count(stream, a.i32(0), a.i32(1), a.i32(2), a.ptr<cu32>(3), a.ptr<uint32_t*>(4), a.ptr<uint32_t*>(5));
+  K("d4_group_scan") return ilt_d4_group_scan(stream, a.i32(0), a.i32(1), a.i32(2), a.ptr<cu32>(3), a.ptr<uint32_t*>(4));
+  K("d4_group_scatter") return ilt_d4_group_scatter(stream, a.i32(0), a.i32(1), a.i32(2), a.ptr<cu32>(3), a.ptr<cu32>(4),
+                                                    a.ptr<cu32>(5), a.ptr<cf>(6), a.ptr<uint32_t*>(7), a.ptr<uint32_t*>(8), a.ptr<float*>(9));
+  K("d4_gather_rows") return ilt_d4_gather_rows(stream, a.i32(0), a.i32(1), a.ptr<cf>(2), a.ptr<cu32>(3), a.ptr<float*>(4));
+  K("d4_swiglu_w") return ilt_d4_swiglu_w(stream, a.i32(0), a.i32(1), a.f32(2), a.ptr<cf>(3), a.ptr<cf>(4), a.ptr<cf>(5),
+                                          a.ptr<float*>(6), a.ptr<int8_t*>(7), a.ptr<float*>(8));
+  K("d4_moe_sum") return ilt_d4_moe_sum(stream, a.i32(0), a.i32(1), a.ptr<cf>(2), a.ptr<cf>(3), a.ptr<float*>(4), a.ptr<cu32>(5));
+  K("d4_moe_sum_rows") return ilt_d4_moe_sum_rows(stream, a.i32(0), a.i32(1), a.i32(2), a.ptr<cf>(3), a.ptr<cu32>(4),
+                                                  a.ptr<cf>(5), a.ptr<float*>(6));
+#undef K
+  return (int)hipErrorNotFound;
+}
+
+}  // extern "C"

@@ -1,0 +1,87 @@
+// Device-side helpers shared by the gfx950 kernels: wave64 lane exchange through
+// DPP, exact fp16 widening, packed int8 dot products.
+#ifndef ILT_DEVICE_H
+#define ILT_DEVICE_H
+
+#include <hip/hip_runtime.h>
+#include <hip/hip_fp16.h>
+#include <stdint.h>
+
+#define ILT_WAVE 64
+
+typedef int8_t i8;
+typedef uint8_t u8;
+typedef uint16_t u16;
+typedef uint32_t u32;
+typedef uint64_t u64;
+
+// DPP controls (CDNA ISA): quad_perm 0x00-0xff, row_shl:n 0x100+n (lane i reads lane
+// i+n of its 16-lane row), row_shr:n 0x110+n, row_half_mirror 0x141 (reverse within 8).
+#define ILT_DPP_XOR1 0xB1
+#define ILT_DPP_XOR2 0x4E
+#define ILT_DPP_HALF_MIRROR 0x141
+#define ILT_DPP_ROW_MIRROR 0x140
+#define ILT_DPP_SHL(n) (0x100 + (n))
+
+template <int CTRL>
+__device__ __forceinline__ int ilt_dpp(int v) {
+  return __builtin_amdgcn_update_dpp(0, v, CTRL, 0xf, 0xf, true);
+}
+template <int CTRL>
+__device__ __forceinline__ float ilt_dppf(float v) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, true));
+}
+
+// Integer sums over aligned groups of 2/4/8/16 lanes; every lane of the group ends
+// with the total.  Integers: any order gives the same bits.
+__device__ __forceinline__ int ilt_sum2(int v) { return v + ilt_dpp<ILT_DPP_XOR1>(v); }
+__device__ __forceinline__ int ilt_sum4(int v) { v = ilt_sum2(v); return v + ilt_dpp<ILT_DPP_XOR2>(v); }
+__device__ __forceinline__ int ilt_sum8(int v) { v = ilt_sum4(v); return v + ilt_dpp<ILT_DPP_HALF_MIRROR>(v); }
+__device__ __forceinline__ int ilt_sum16(int v) { v = ilt_sum8(v); return v + ilt_dpp<ILT_DPP_ROW_MIRROR>(v); }
+
+__device__ __forceinline__ float ilt_max16(float v) {
+  v = fmaxf(v, ilt_dppf<ILT_DPP_XOR1>(v));
+  v = fmaxf(v, ilt_dppf<ILT_DPP_XOR2>(v));
+  v = fmaxf(v, ilt_dppf<ILT_DPP_HALF_MIRROR>(v));
+  v = fmaxf(v, ilt_dppf<ILT_DPP_ROW_MIRROR>(v));
+  return v;
+}
+
+// binary16 bits -> binary32, exact (subnormals included).
+__device__ __forceinline__ float ilt_h2f(u16 h) { return __half2float(__ushort_as_half(h)); }
+
+// four int8 x int8 products added to c (v_dot4_i32_i8); exact.
+__device__ __forceinline__ int ilt_dot4(int a, int b, int c) { return __builtin_amdgcn_sdot4(a, b, c, false); }
+
+__device__ __forceinline__ int ilt_dot16(const int4& a, const int4& b, int c) {
+  c = ilt_dot4(a.x, b.x, c); c = ilt_dot4(a.y, b.y, c); c = ilt_dot4(a.z, b.z, c); return ilt_dot4(a.w, b.w, c);
+}
+
+// Loads that may be 2-byte aligned (GGUF blocks of 34, 66, 84 and 210 bytes are not
+// 16-byte multiples); gfx950 performs them in hardware.
+__device__ __forceinline__ int4 ilt_ld16(const u8* p) {
+  int4 v; __builtin_memcpy(&v, __builtin_assume_aligned(p, 2), 16); return v;
+}
+__device__ __forceinline__ int2 ilt_ld8(const u8* p) {
+  int2 v; __builtin_memcpy(&v, __builtin_assume_aligned(p, 2), 8); return v;
+}
+__device__ __forceinline__ u32 ilt_ld4(const u8* p) {
+  u32 v; __builtin_memcpy(&v, __builtin_assume_aligned(p, 2), 4); return v;
+}
+__device__ __forceinline__ u16 ilt_ld2(const u8* p) {
+  u16 v; __builtin_memcpy(&v, __builtin_assume_aligned(p, 2), 2); return v;
+}
+
+// SBCL evaluates single-float exp and log by widening to double, calling libm and
+// rounding back (the CPU path's silu, softplus); the kernels do the same.
+__device__ __forceinline__ float ilt_expf_via_double(float x) { return (float)exp((double)x); }
+__device__ __forceinline__ float ilt_logf_via_double(float x) { return (float)log((double)x); }
+
+__device__ __forceinline__ float ilt_sigmoid(float x) {
+  if (x >= 0.0f) return 1.0f / (1.0f + ilt_expf_via_double(-x));
+  float e = ilt_expf_via_double(x);
+  return e / (1.0f + e);
+}
+__device__ __forceinline__ float ilt_silu(float x) { return x * ilt_sigmoid(x); }
+
+#endif  // ILT_DEVICE_H

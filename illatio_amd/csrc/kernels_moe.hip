@@ -1,0 +1,236 @@
+// The MoE expert path's small kernels for gfx950: routing, grouping (token, slot) rows
+// by expert, the gather, the gated activation and the slot-ordered sums.  Names,
+// argument meaning and results follow the reference's kernels
+// (src/cuda/ds4f_chunk.cu:393-508, src/cuda/ds4f.cu:645-655, 902-910); the floats follow
+// its CPU path (src/ds4f.lisp:248-254, 950-978, 1013-1036).
+#include "ilt_device.h"
+#include "ilt_kernels.h"
+
+namespace {
+
+__device__ __forceinline__ float softplus(float x) {
+  if (x > 20.0f) return x;
+  if (x < -20.0f) return ilt_expf_via_double(x);
+  return ilt_logf_via_double(1.0f + ilt_expf_via_double(x));
+}
+
+// d4-route: a workgroup a token, a thread an expert.  p = sqrt(softplus(logit)); the top
+// NU of p (+ bias), the earlier expert first of equal ones; weights p/sum(p)*scale with
+// the sum taken in slot order and floored at 2^-14.  hash 1: the experts come from
+// tid2eid[token].
+__global__ void route_kernel(int ne, int nu, int hash, float scale, int has_bias, const float* __restrict__ logits,
+                             const float* __restrict__ bias, const int* __restrict__ tid2eid,
+                             const u32* __restrict__ tokens, u32* __restrict__ sel, float* __restrict__ wout) {
+  extern __shared__ float sh[];
+  float* probs = sh;                    // ne
+  float* sv = sh + ne;                  // ne
+  u64* wbest = (u64*)(sh + 2 * ne);     // up to 16 waves
+  u32* picked = (u32*)(wbest + 16);     // nu
+  const int t = blockIdx.x, e = threadIdx.x;
+  if (e < ne) {
+    const float p = sqrtf(softplus(logits[(long long)t * ne + e]));
+    probs[e] = p;
+    sv[e] = has_bias ? p + bias[(has_bias == 2 ? (long long)t * ne : 0) + e] : p;
+  }
+  __syncthreads();
+  if (hash == 1) {
+    if (e < nu) picked[e] = (u32)tid2eid[(long long)tokens[t] * nu + e];
+  } else {
+    for (int k = 0; k < nu; k++) {
+      // order-preserving key of a float, then the complement of the index: the largest key
+      // is the largest score, the earliest expert among equals
+      u64 key = 0;
+      if (e < ne) {
+        const u32 b = __float_as_uint(sv[e]);
+        const u32 ord = (b & 0x80000000u) ? ~b : (b | 0x80000000u);
+        key = ((u64)ord << 32) | (u32)(0x7FFFFFFF - e);
+        if (sv[e] != sv[e]) key = 0;    // a NaN never wins
+      }
+#pragma unroll
+      for (int off = 32; off > 0; off >>= 1) {
+        const u32 hi = __shfl_xor((u32)(key >> 32), off), lo = __shfl_xor((u32)key, off);
+        const u64 o = ((u64)hi << 32) | lo;
+        key = o > key ? o : key;
+      }
+      if ((e & 63) == 0) wbest[e >> 6] = key;
+      __syncthreads();
+      if (e == 0) {
+        u64 best = wbest[0];
+        for (int w = 1; w < (int)(blockDim.x + 63) / 64; w++) best = wbest[w] > best ? wbest[w] : best;
+        const u32 bi = 0x7FFFFFFF - (u32)(best & 0xFFFFFFFFu);
+        picked[k] = bi;
+        sv[bi] = -INFINITY;
+      }
+      __syncthreads();
+    }
+  }
+  __syncthreads();
+  if (e == 0) {
+    float sum = 0.0f;
+    for (int i = 0; i < nu; i++) sum = sum + probs[picked[i]];
+    if (sum < 6.103515625e-5f) sum = 6.103515625e-5f;
+    for (int i = 0; i < nu; i++) {
+      sel[(long long)t * nu + i] = picked[i];
+      wout[(long long)t * nu + i] = (probs[picked[i]] / sum) * scale;
+    }
+  }
+}
+
+__global__ void group_zero_kernel(int ne, u32* counts) {
+  const int e = blockIdx.x * blockDim.x + threadIdx.x;
+  if (e < ne) counts[e] = 0u;
+}
+
+// rank[row] = the row's place among its expert's rows.  The order inside an expert is
+// whatever the atomics give; every later step goes through rmap/smap, so results do not
+// depend on it.
+__global__ void group_count_kernel(int n, const u32* __restrict__ sel, u32* counts, u32* __restrict__ rank) {
+  const int gid = blockIdx.x * blockDim.x + threadIdx.x;
+  if (gid >= n) return;
+  rank[gid] = atomicAdd(counts + sel[gid], 1u);
+}
+
+// bases[e] = rows before expert e's.  One workgroup of 1024; ne <= 1024.
+__global__ __launch_bounds__(1024) void group_scan_kernel(int ne, const u32* __restrict__ counts, u32* __restrict__ bases) {
+  __shared__ u32 sh[1024];
+  const int e = threadIdx.x;
+  sh[e] = e < ne ? counts[e] : 0u;
+  __syncthreads();
+  for (int off = 1; off < 1024; off <<= 1) {
+    const u32 v = e >= off ? sh[e - off] : 0u;
+    __syncthreads();
+    sh[e] += v;
+    __syncthreads();
+  }
+  if (e < ne) bases[e] = sh[e] - counts[e];
+}
+
+__global__ void group_scatter_kernel(int n, int nu, const u32* __restrict__ sel, const u32* __restrict__ rank,
+                                     const u32* __restrict__ bases, const float* __restrict__ w,
+                                     u32* __restrict__ rmap, u32* __restrict__ smap, float* __restrict__ wrow) {
+  const int gid = blockIdx.x * blockDim.x + threadIdx.x;
+  if (gid >= n) return;
+  const u32 row = bases[sel[gid]] + rank[gid];
+  rmap[row] = gid / nu; smap[gid] = row; wrow[row] = w[gid];
+}
+
+__global__ void gather_rows_kernel(int d, int nrows, const float* __restrict__ src, const u32* __restrict__ map,
+                                   float* __restrict__ x) {
+  const long long gid = ((long long)blockIdx.x * blockDim.x + threadIdx.x) * 4;
+  if (gid >= (long long)nrows * d) return;
+  const int r = (int)(gid / d), j = (int)(gid % d);
+  *(float4*)(x + gid) = *(const float4*)(src + (long long)map[r] * d + j);
+}
+
+// mid[r][j] = (silu(g) * u) * w[r], g and u clamped first when clamp > 1e-6
+// (d4-routed!, ds4f.lisp:1016-1019); quantized to Q8_0 with a float scale as well when xq
+// is given (the shared expert's down projection takes Q8_0 activations).
+__global__ __launch_bounds__(256) void swiglu_w_kernel(long long total, int ff, float clamp, const float* __restrict__ g,
+                                                       const float* __restrict__ u, const float* __restrict__ w,
+                                                       float* __restrict__ mid, i8* __restrict__ xq, float* __restrict__ xs) {
+  const long long i = (long long)blockIdx.x * 256 + threadIdx.x;
+  const bool live = i < total;
+  float v = 0.0f;
+  if (live) {
+    float gv = g[i], uv = u[i];
+    if (clamp > 1e-6f) { gv = fminf(gv, clamp); uv = fmaxf(-clamp, fminf(uv, clamp)); }
+    v = (ilt_silu(gv) * uv) * w[i / ff];
+    mid[i] = v;
+  }
+  if (xq) {
+    float amax = ilt_max16(fabsf(v));
+    amax = fmaxf(amax, __shfl_xor(amax, 16));
+    const float d = amax / 127.0f;
+    const float id = d == 0.0f ? 0.0f : 1.0f / d;
+    if (live) {
+      xq[i] = (i8)(int)rintf(v * id);
+      if ((threadIdx.x & 31) == 0) xs[i >> 5] = d;
+    }
+  }
+}
+
+__global__ void moe_sum_kernel(int d, int k, const float* __restrict__ down, const float* __restrict__ shared_,
+                               float* __restrict__ moe, const u32* __restrict__ perm) {
+  const int r = blockIdx.x * blockDim.x + threadIdx.x;
+  if (r >= d) return;
+  float acc = 0.0f;
+  for (int i = 0; i < k; i++) acc = acc + down[(long long)(perm ? perm[i] : i) * d + r];
+  moe[r] = shared_ ? acc + shared_[r] : acc;
+}
+
+__global__ void moe_sum_rows_kernel(int d, int nu, int ntok, const float* __restrict__ down, const u32* __restrict__ map,
+                                    const float* __restrict__ shared_, float* __restrict__ moe) {
+  const long long gid = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (gid >= (long long)ntok * d) return;
+  const int t = (int)(gid / d), j = (int)(gid % d);
+  float acc = 0.0f;
+  for (int s = 0; s < nu; s++) acc = acc + down[(long long)map[(long long)t * nu + s] * d + j];
+  moe[gid] = shared_ ? acc + shared_[gid] : acc;
+}
+
+}  // namespace
+
+hipError_t ilt_k_route(int ne, int nu, int hash, float scale, int has_bias, const float* logits, const float* bias,
+                       const int* tid2eid, const uint32_t* tokens, uint32_t* sel, float* wout, int ntok, hipStream_t st) {
+  if (ntok <= 0) return hipSuccess;
+  if (ne < 1 || ne > 1024 || nu < 1 || nu > ne || hash < 0 || hash > 1) return hipErrorInvalidValue;
+  const int threads = (ne + 63) / 64 * 64;
+  const size_t smem = 4 * (size_t)(2 * ne) + 8 * 16 + 4 * (size_t)nu;
+  hipLaunchKernelGGL(route_kernel, dim3(ntok), dim3(threads), smem, st, ne, nu, hash, scale, has_bias, logits, bias,
+                     tid2eid, tokens, sel, wout);
+  return hipGetLastError();
+}
+
+hipError_t ilt_k_group_zero(int ne, uint32_t* counts, hipStream_t st) {
+  hipLaunchKernelGGL(group_zero_kernel, dim3((ne + 255) / 256), dim3(256), 0, st, ne, counts);
+  return hipGetLastError();
+}
+
+hipError_t ilt_k_group_count(int n, int ne, int nu, const uint32_t* sel, uint32_t* counts, uint32_t* rank, hipStream_t st) {
+  if (n <= 0) return hipSuccess;
+  hipLaunchKernelGGL(group_count_kernel, dim3((n + 255) / 256), dim3(256), 0, st, n, sel, counts, rank);
+  return hipGetLastError();
+}
+
+hipError_t ilt_k_group_scan(int n, int ne, int nu, const uint32_t* counts, uint32_t* bases, hipStream_t st) {
+  if (ne > 1024) return hipErrorInvalidValue;
+  hipLaunchKernelGGL(group_scan_kernel, dim3(1), dim3(1024), 0, st, ne, counts, bases);
+  return hipGetLastError();
+}
+
+hipError_t ilt_k_group_scatter(int n, int ne, int nu, const uint32_t* sel, const uint32_t* rank, const uint32_t* bases,
+                               const float* w, uint32_t* rmap, uint32_t* smap, float* wrow, hipStream_t st) {
+  if (n <= 0) return hipSuccess;
+  hipLaunchKernelGGL(group_scatter_kernel, dim3((n + 255) / 256), dim3(256), 0, st, n, nu, sel, rank, bases, w, rmap, smap, wrow);
+  return hipGetLastError();
+}
+
+hipError_t ilt_k_gather_rows(int d, int nrows, const float* src, const uint32_t* map, float* x, hipStream_t st) {
+  if (nrows <= 0) return hipSuccess;
+  if (d % 4) return hipErrorInvalidValue;
+  const long long n4 = (long long)nrows * d / 4;
+  hipLaunchKernelGGL(gather_rows_kernel, dim3((unsigned)((n4 + 255) / 256)), dim3(256), 0, st, d, nrows, src, map, x);
+  return hipGetLastError();
+}
+
+hipError_t ilt_k_swiglu_w(int n, int ff, float clamp, const float* g, const float* u, const float* w, float* mid,
+                          int8_t* xq, float* xs, hipStream_t st) {
+  const long long total = (long long)n * ff;
+  if (total <= 0) return hipSuccess;
+  if (xq && (total % 32)) return hipErrorInvalidValue;
+  hipLaunchKernelGGL(swiglu_w_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st, total, ff, clamp, g, u, w, mid, xq, xs);
+  return hipGetLastError();
+}
+
+hipError_t ilt_k_moe_sum(int d, int k, const float* down, const float* shared_, float* moe, const uint32_t* perm, hipStream_t st) {
+  hipLaunchKernelGGL(moe_sum_kernel, dim3((d + 255) / 256), dim3(256), 0, st, d, k, down, shared_, moe, perm);
+  return hipGetLastError();
+}
+
+hipError_t ilt_k_moe_sum_rows(int d, int nu, int ntok, const float* down, const uint32_t* map, const float* shared_,
+                              float* moe, hipStream_t st) {
+  const long long n = (long long)ntok * d;
+  if (n <= 0) return hipSuccess;
+  hipLaunchKernelGGL(moe_sum_rows_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, d, nu, ntok, down, map, shared_, moe);
+  return hipGetLastError();
+}

@@ -1,0 +1,191 @@
+// Activation quantizers, the Q8_0 upload repack, and row dequantizers for gfx950.
+// Every result is bit-for-bit what the reference's CPU path stores
+// (tensor.lisp:245-262, kquant.lisp:130-167, 466-497, iquant.lisp:161-230).
+#include "ilt_device.h"
+#include "ilt_iq2xxs_tables.h"
+#include "ilt_kernels.h"
+
+namespace {
+
+__device__ const u64 q_grid_dev[256] = { ILT_IQ2XXS_GRID_VALUES };
+
+// Q8_0 activations (quantize-q8!): a block of 32 per half wave.  d = amax/127; the
+// stored scale is d through fp16 when f16_scale; q = round-half-even(x * (1/d)) with the
+// unrounded d.  xsum (optional) gets the block's integer sum.
+__global__ __launch_bounds__(256) void quant_q8_kernel(const float* __restrict__ x, i8* __restrict__ xq,
+                                                       float* __restrict__ xs, int* __restrict__ xsum,
+                                                       long long nblocks, int f16_scale) {
+  const long long i = (long long)blockIdx.x * 256 + threadIdx.x;
+  const long long b = i >> 5;
+  const bool live = b < nblocks;
+  const float v = live ? x[i] : 0.0f;
+  float amax = ilt_max16(fabsf(v));
+  amax = fmaxf(amax, __shfl_xor(amax, 16));
+  const float d = amax / 127.0f;
+  const float id = d == 0.0f ? 0.0f : 1.0f / d;
+  const int q = (int)rintf(v * id);
+  int sum = ilt_sum16(q);
+  sum += __shfl_xor(sum, 16);
+  if (!live) return;
+  xq[i] = (i8)q;
+  if ((threadIdx.x & 31) == 0) {
+    xs[b] = f16_scale ? __half2float(__float2half_rn(d)) : d;
+    if (xsum) xsum[b] = sum;
+  }
+}
+
+// Q8_K activations (quantize-q8k!): a block of 256 per workgroup.  The
+// largest-magnitude value, the first of equals, sets iscale = -127/max;
+// q = min(127, round-half-even(iscale*x)); d = 1/iscale; sums of each 16 quants.
+__global__ __launch_bounds__(256) void quant_q8k_kernel(const float* __restrict__ x, i8* __restrict__ xq,
+                                                        float* __restrict__ xd, int* __restrict__ bsums) {
+  __shared__ u64 wkey[4];
+  __shared__ float smx;
+  const long long b = blockIdx.x;
+  const int t = threadIdx.x;
+  const float v = x[b * 256 + t];
+  // |v|'s bits order as |v| does; the low word prefers the earlier index
+  u64 key = ((u64)__float_as_uint(fabsf(v)) << 32) | (u32)(255 - t);
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) {
+    const u32 hi = __shfl_xor((u32)(key >> 32), off), lo = __shfl_xor((u32)key, off);
+    const u64 o = ((u64)hi << 32) | lo;
+    key = o > key ? o : key;
+  }
+  if ((t & 63) == 0) wkey[t >> 6] = key;
+  __syncthreads();
+  u64 best = wkey[0];
+#pragma unroll
+  for (int w = 1; w < 4; w++) best = wkey[w] > best ? wkey[w] : best;
+  if (t == 255 - (int)(best & 0xFFFFFFFFu)) smx = v;
+  __syncthreads();
+  const float mx = smx;
+  int q = 0;
+  float iscale = 0.0f;
+  if ((best >> 32) != 0) {
+    iscale = -127.0f / mx;
+    q = min(127, (int)rintf(iscale * v));
+  }
+  xq[b * 256 + t] = (i8)q;
+  const int s = ilt_sum16(q);
+  if ((t & 15) == 0) bsums[b * 16 + (t >> 4)] = s;
+  if (t == 0) xd[b] = (best >> 32) != 0 ? 1.0f / iscale : 0.0f;
+}
+
+// GGUF Q8_0 blocks (f16 d, 32 int8) split into an int8 array and an f16 scale array.
+__global__ __launch_bounds__(256) void repack_q8_kernel(const u8* __restrict__ raw, i8* __restrict__ qs,
+                                                        u16* __restrict__ d, long long nblocks) {
+  const long long i = (long long)blockIdx.x * 256 + threadIdx.x;   // one thread per 2 bytes of quants
+  const long long b = i >> 4;
+  if (b >= nblocks) return;
+  const int k = (int)(i & 15);
+  const u8* blk = raw + b * 34;
+  *(u16*)(qs + b * 32 + 2 * k) = *(const u16*)(blk + 2 + 2 * k);
+  if (k == 0) d[b] = *(const u16*)blk;
+}
+
+__global__ __launch_bounds__(256) void copy_bytes_kernel(const u8* __restrict__ src, u8* __restrict__ dst, long long bytes) {
+  const long long i = ((long long)blockIdx.x * 256 + threadIdx.x) * 2;
+  if (i + 1 < bytes) *(u16*)(dst + i) = *(const u16*)(src + i);
+  else if (i < bytes) dst[i] = src[i];
+}
+
+// ---- rows as floats (embed_q8 / embed_k; q8mat-row!, kmat-row!, *-row-floats!) ------------------
+__device__ __forceinline__ void scale_min_k4_bytes(int j, const u8* q, int& sc, int& m) {
+  if (j < 4) { sc = q[j] & 63; m = q[j + 4] & 63; }
+  else { sc = (q[j + 4] & 0xF) | ((q[j - 4] >> 6) << 4); m = (q[j + 4] >> 4) | ((q[j] >> 6) << 4); }
+}
+
+__device__ float dequant_one(int fmt, const u8* wrow, const u16* wdrow, int col) {
+  if (fmt == ILT_Q8_0) {
+    // split layout: wrow = int8 quants of the row, wdrow = its f16 scales
+    return ilt_h2f(wdrow[col >> 5]) * (float)((const i8*)wrow)[col];
+  }
+  const int i = col >> 8, idx = col & 255;
+  if (fmt == ILT_Q4_K) {
+    const u8* blk = wrow + (long)i * 144;
+    const int g = idx >> 5, l = idx & 31;
+    int sc, m; scale_min_k4_bytes(g, blk + 4, sc, m);
+    const u8 byte = blk[16 + (g >> 1) * 32 + l];
+    const int q = (g & 1) ? (byte >> 4) : (byte & 0xF);
+    const float d1 = ilt_h2f(ilt_ld2(blk)) * (float)sc, m1 = ilt_h2f(ilt_ld2(blk + 2)) * (float)m;
+    return d1 * (float)q - m1;
+  }
+  if (fmt == ILT_Q6_K) {
+    const u8* blk = wrow + (long)i * 210;
+    const int c = idx >> 7, r = idx & 127, part = r >> 5, l = r & 31;
+    const int lowbyte = blk[64 * c + (part & 1) * 32 + l];
+    const int low = part < 2 ? (lowbyte & 0xF) : (lowbyte >> 4);
+    const int q = low | (((blk[128 + 32 * c + l] >> (2 * part)) & 3) << 4);
+    const int sc = ((const i8*)blk)[192 + 8 * c + 2 * part + (l >> 4)];
+    return (ilt_h2f(ilt_ld2(blk + 208)) * (float)sc) * (float)(q - 32);
+  }
+  if (fmt == ILT_Q2_K) {
+    const u8* blk = wrow + (long)i * 84;
+    const int h = idx >> 7, k = (idx >> 5) & 3, half = (idx >> 4) & 1, l = idx & 15;
+    const u8 sb = blk[8 * h + 2 * k + half];
+    const float dl = ilt_h2f(ilt_ld2(blk + 80)) * (float)(sb & 15), ml = ilt_h2f(ilt_ld2(blk + 82)) * (float)(sb >> 4);
+    return dl * (float)((blk[16 + 32 * h + 16 * half + l] >> (2 * k)) & 3) - ml;
+  }
+  // IQ2_XXS
+  const u8* blk = wrow + (long)i * 66;
+  const int ib = idx >> 5, l = (idx >> 3) & 3, jj = idx & 7;
+  const u8* so = blk + 2 + 8 * ib;
+  const u32 aux = (u32)so[4] | ((u32)so[5] << 8) | ((u32)so[6] << 16) | ((u32)so[7] << 24);
+  const float db = (ilt_h2f(ilt_ld2(blk)) * (0.5f + (float)(aux >> 28))) * 0.25f;
+  const u64 g = q_grid_dev[so[l]];
+  u32 s = (aux >> (7 * l)) & 127;
+  s |= (__popc(s) & 1) << 7;
+  return (db * (float)((g >> (8 * jj)) & 0xFF)) * (((s >> jj) & 1) ? -1.0f : 1.0f);
+}
+
+// out[n][col] = W[rows_idx[n]][col] (rows_idx null: row n).
+__global__ __launch_bounds__(256) void dequant_rows_kernel(int fmt, const u8* __restrict__ w, const u16* __restrict__ wd,
+                                                           const int* __restrict__ rows_idx, int cols,
+                                                           long long row_bytes, float* __restrict__ out) {
+  const long long n = blockIdx.y;
+  const long long r = rows_idx ? rows_idx[n] : n;
+  const u8* wrow = w + r * row_bytes;
+  const u16* wdrow = wd ? wd + r * (cols >> 5) : nullptr;
+  for (int col = blockIdx.x * 256 + threadIdx.x; col < cols; col += gridDim.x * 256)
+    out[n * cols + col] = dequant_one(fmt, wrow, wdrow, col);
+}
+
+}  // namespace
+
+hipError_t ilt_k_quant_q8(const float* x, int8_t* xq, float* xs, int* xsum, long long nblocks, int f16_scale, hipStream_t st) {
+  if (nblocks <= 0) return hipSuccess;
+  hipLaunchKernelGGL(quant_q8_kernel, dim3((unsigned)((nblocks * 32 + 255) / 256)), dim3(256), 0, st, x, xq, xs, xsum, nblocks, f16_scale);
+  return hipGetLastError();
+}
+
+hipError_t ilt_k_quant_q8k(const float* x, int8_t* xq, float* xd, int* bsums, long long nblocks, hipStream_t st) {
+  if (nblocks <= 0) return hipSuccess;
+  hipLaunchKernelGGL(quant_q8k_kernel, dim3((unsigned)nblocks), dim3(256), 0, st, x, xq, xd, bsums);
+  return hipGetLastError();
+}
+
+hipError_t ilt_k_repack_q8(const uint8_t* raw, int8_t* qs, uint16_t* d, long long nblocks, hipStream_t st) {
+  if (nblocks <= 0) return hipSuccess;
+  hipLaunchKernelGGL(repack_q8_kernel, dim3((unsigned)((nblocks * 16 + 255) / 256)), dim3(256), 0, st, raw, qs, d, nblocks);
+  return hipGetLastError();
+}
+
+hipError_t ilt_k_copy_bytes(const uint8_t* src, uint8_t* dst, long long bytes, hipStream_t st) {
+  if (bytes <= 0) return hipSuccess;
+  hipLaunchKernelGGL(copy_bytes_kernel, dim3((unsigned)((bytes / 2 + 256) / 256)), dim3(256), 0, st, src, dst, bytes);
+  return hipGetLastError();
+}
+
+hipError_t ilt_k_dequant_rows(int fmt, const uint8_t* w, const uint16_t* wd, const int* rows_idx, long long nrows,
+                              int cols, long long row_bytes, float* out, hipStream_t st) {
+  if (nrows <= 0) return hipSuccess;
+  const unsigned gx = (unsigned)min((cols + 255) / 256, 64);
+  for (long long n0 = 0; n0 < nrows; n0 += 65535) {
+    const unsigned gy = (unsigned)min(nrows - n0, (long long)65535);
+    hipLaunchKernelGGL(dequant_rows_kernel, dim3(gx, gy), dim3(256), 0, st, fmt, w, wd,
+                       rows_idx ? rows_idx + n0 : nullptr, cols, row_bytes, out + n0 * cols);
+    if (!rows_idx) w += 65535 * row_bytes, wd = wd ? wd + 65535LL * (cols >> 5) : nullptr;
+  }
+  return hipGetLastError();
+}

@@ -1,0 +1,122 @@
+"""Dense matrices on the device: the host side of the reference's src/cuda-dense.lisp for
+the quantized products (UPLOAD-GMAT :75-100, CMAT-MUL :220-248, QKV-MUL :309-324), driving
+the kernels through LAUNCH exactly as the Lisp host does.
+
+Where the reference's CUDA path quantizes activations into Q8_0-style blocks for every
+format, this path quantizes them as the reference's CPU path does -- Q8_0 for Q8_0
+matrices, Q8_K for K-quants (matrix-act-kind, kquant.lisp:532-533) -- so results match
+the CPU path bit for bit.
+"""
+import numpy as np
+
+from . import hip
+from .synth import BLOCK_BYTES, BLOCK_WEIGHTS, Q4_K, Q6_K, Q8_0
+
+KQUANT_CODE = {Q4_K: 0, Q6_K: 2}      # kquant-code, cuda-dense.lisp:18-20
+
+
+class CMat:
+    """A matrix on the device (CMAT): TYPE, ROWS, COLS, QS (and D, Q8_0's scales)."""
+
+    def __init__(self, name, qtype, rows, cols, qs, d=None):
+        self.name, self.type, self.rows, self.cols, self.qs, self.d = name, qtype, rows, cols, qs, d
+
+    def kquant_p(self):
+        return self.type in KQUANT_CODE
+
+    def free(self):
+        hip.hip_free(self.qs)
+        hip.hip_free(self.d)
+
+
+def upload_gmat(dev, name, qtype, rows, cols, raw_bytes):
+    """RAW_BYTES (the matrix's GGUF blocks, a uint8 array) to DEV: Q8_0 split into int8s and
+    scales by repack_q8; Q6_K through repack_q6k (which here keeps the 210-byte blocks);
+    Q4_K as it is."""
+    if qtype not in (Q8_0, Q4_K, Q6_K):
+        raise ValueError(f"the dense path multiplies Q8_0, Q4_K and Q6_K; {name} is type {qtype}")
+    if cols % BLOCK_WEIGHTS[qtype]:
+        raise ValueError(f"{name}: {cols} columns is not a whole number of blocks")
+    raw_bytes = np.ascontiguousarray(raw_bytes, dtype=np.uint8).ravel()
+    n = rows * cols
+    nbytes = n // BLOCK_WEIGHTS[qtype] * BLOCK_BYTES[qtype]
+    assert raw_bytes.size == nbytes
+    if qtype == Q8_0:
+        nb = n // 32
+        raw = hip.hip_upload_new(dev, raw_bytes)
+        qs, d = hip.hip_alloc(dev, n, zero=False), hip.hip_alloc(dev, 2 * nb, zero=False)
+        hip.launch(dev, "repack_q8", (nb + 7) // 8, (32, 8), [raw, qs, d, hip.I64(nb)])
+        hip.hip_sync(dev)
+        hip.hip_free(raw)
+        return CMat(name, qtype, rows, cols, qs, d)
+    if qtype == Q6_K:
+        nb = n // 256
+        raw = hip.hip_upload_new(dev, raw_bytes)
+        qs = hip.hip_alloc(dev, 224 * nb, zero=False)
+        hip.launch(dev, "repack_q6k", (nb + 7) // 8, (32, 8), [raw, qs, hip.I64(nb)])
+        hip.hip_sync(dev)
+        hip.hip_free(raw)
+        return CMat(name, qtype, rows, cols, qs)
+    return CMat(name, qtype, rows, cols, hip.hip_upload_new(dev, raw_bytes))
+
+
+class QAct:
+    """Quantized activations on the device for N tokens of COLS: Q8_0 (xq, xs) and/or Q8_K
+    (kq, kd, ksum), the formats a QACT holds (kquant.lisp:504-514)."""
+
+    def __init__(self, dev, n, cols, kinds=("q8", "q8k")):
+        self.dev, self.n, self.cols = dev, n, cols
+        self.xq = self.xs = self.kq = self.kd = self.ksum = None
+        if "q8" in kinds:
+            self.xq, self.xs = hip.hip_alloc(dev, n * cols), hip.hip_alloc(dev, 4 * n * cols // 32)
+        if "q8k" in kinds:
+            self.kq, self.kd = hip.hip_alloc(dev, n * cols), hip.hip_alloc(dev, 4 * n * cols // 256)
+            self.ksum = hip.hip_alloc(dev, 4 * n * cols // 16)
+
+    def free(self):
+        for b in (self.xq, self.xs, self.kq, self.kd, self.ksum):
+            hip.hip_free(b)
+
+
+def quantize_act(dev, x, act, n=None, f16_scale=True):
+    """X (a DBuf of N x COLS floats) into ACT, in each format it holds (QUANTIZE-ACT!)."""
+    n = act.n if n is None else n
+    if act.xq is not None:
+        nb = n * act.cols // 32
+        if f16_scale:
+            hip.launch(dev, "quant_q8", (nb * 32 + 255) // 256, 256, [x, act.xq, act.xs, None, hip.I64(nb)])
+        else:
+            hip.launch(dev, "d4_quant", (nb * 32 + 255) // 256, 256, [x, act.xq, act.xs, nb])
+    if act.kq is not None:
+        nb = n * act.cols // 256
+        hip.launch(dev, "quant_q8k", nb, 256, [x, act.kq, act.kd, act.ksum, hip.I64(nb)])
+    return act
+
+
+def cmat_mul(dev, w, act, y, n=1, bias=None, acc=False):
+    """Y = W X for N tokens (token t's X at t*cols, its Y at t*rows), or Y += it when ACC
+    (CMAT-MUL): the matrix-vector kernel for one token, the tiled product for more."""
+    rows, cols = w.rows, w.cols
+    a = 1 if acc else 0
+    if w.kquant_p():
+        code = KQUANT_CODE[w.type]
+        if n == 1:
+            hip.launch(dev, "mv_k", (rows + 3) // 4, 128, [code, w.qs, act.kq, act.kd, act.ksum, y, bias, rows, cols, a])
+        else:
+            hip.launch(dev, "mm_k", ((n + 63) // 64, (rows + 63) // 64), 256,
+                       [code, w.qs, act.kq, act.kd, act.ksum, y, bias, rows, cols, n, a])
+    elif n == 1:
+        hip.launch(dev, "mv_q8", (rows + 3) // 4, 128, [w.qs, w.d, act.xq, act.xs, y, bias, rows, cols, a])
+    else:
+        hip.launch(dev, "mm_q8", ((n + 63) // 64, (rows + 63) // 64), 256,
+                   [w.qs, w.d, act.xq, act.xs, y, bias, rows, cols, n, a])
+    return y
+
+
+def embed(dev, emb, tokens, x, n, d):
+    """Rows TOKENS (a device vector of N ids) of the embedding EMB as floats in X (EMBED)."""
+    if emb.kquant_p():
+        hip.launch(dev, "embed_k", n, 128, [KQUANT_CODE[emb.type], emb.qs, tokens, x, d])
+    else:
+        hip.launch(dev, "embed_q8", n, 256, [emb.qs, emb.d, tokens, x, d])
+    return x

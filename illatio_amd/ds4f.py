@@ -1,0 +1,136 @@
+"""The routed and shared experts of one FFN on the device: the host side of the
+reference's DK-FFN-TAIL (src/cuda-ds4f.lisp:908-956, one token) and DK-FFN-ROUTED-CHUNK
+(src/cuda-ds4f-prefill.lisp:315-356, a chunk), driving the kernels through LAUNCH.
+
+An expert slot holds gate | up | down contiguously (cuda-ds4f.lisp:162-166): kernels get a
+table of slot addresses and a byte offset (0, gate-bytes, 2 gate-bytes).  With 288 GB of
+HBM every expert is resident, so there is no pool, no read-through and no CPU expert: slot
+e is expert e.
+
+Activations are quantized as the reference's CPU path quantizes them (Q8_K for the routed
+experts, D4-ROUTED!, ds4f.lisp:994-1037; Q8_0 with a float scale for the shared expert,
+D4-SHARED!, :1039-1048), not left as floats as its CUDA kernels take them.
+"""
+import numpy as np
+
+from . import hip
+from .synth import IQ2_XXS, Q2_K, Q8_0, row_bytes
+
+
+class ExpertPool:
+    """NE experts on DEV, slot e = gate | up | down of expert e, 256-byte aligned."""
+
+    def __init__(self, dev, ne, d, ff, gate, up, down):
+        self.dev, self.ne, self.d, self.ff = dev, ne, d, ff
+        self.grb, self.drb = row_bytes(IQ2_XXS, d), row_bytes(Q2_K, ff)
+        self.gate_bytes, self.down_bytes = ff * self.grb, d * self.drb
+        self.slot_bytes = (2 * self.gate_bytes + self.down_bytes + 255) // 256 * 256
+        host = np.zeros((ne, self.slot_bytes), np.uint8)
+        host[:, :self.gate_bytes] = np.asarray(gate, np.uint8).reshape(ne, self.gate_bytes)
+        host[:, self.gate_bytes:2 * self.gate_bytes] = np.asarray(up, np.uint8).reshape(ne, self.gate_bytes)
+        host[:, 2 * self.gate_bytes:2 * self.gate_bytes + self.down_bytes] = np.asarray(down, np.uint8).reshape(ne, self.down_bytes)
+        self.pool = hip.hip_upload_new(dev, host)
+
+    def slot_ptr(self, e):
+        return self.pool.ptr + int(e) * self.slot_bytes
+
+    def free(self):
+        hip.hip_free(self.pool)
+
+
+class SharedExpert:
+    """The shared expert's three Q8_0 matrices, repacked (d4-upload-weights)."""
+
+    def __init__(self, dev, d, ff, sgate, sup, sdown):
+        from .dense import upload_gmat
+        self.d, self.ff = d, ff
+        self.gate = upload_gmat(dev, "ffn_gate_shexp", Q8_0, ff, d, sgate)
+        self.up = upload_gmat(dev, "ffn_up_shexp", Q8_0, ff, d, sup)
+        self.down = upload_gmat(dev, "ffn_down_shexp", Q8_0, d, ff, sdown)
+
+    def free(self):
+        for m in (self.gate, self.up, self.down):
+            m.free()
+
+
+def _q8k(dev, x, n_elems):
+    kq, kd = hip.hip_alloc(dev, n_elems), hip.hip_alloc(dev, 4 * n_elems // 256)
+    ks = hip.hip_alloc(dev, 4 * n_elems // 16)
+    hip.launch(dev, "quant_q8k", n_elems // 256, 256, [x, kq, kd, ks, hip.I64(n_elems // 256)])
+    return kq, kd, ks
+
+
+def ffn_shared(dev, sh, norm2, clamp, n=1):
+    """The shared expert of N tokens' NORM2 (DK-FFN-HEAD's second half): returns SOUT."""
+    d, ff = sh.d, sh.ff
+    qn_q, qn_s = hip.hip_alloc(dev, n * d), hip.hip_alloc(dev, 4 * n * d // 32)
+    sg, su, smid = (hip.hip_alloc(dev, 4 * n * ff) for _ in range(3))
+    qm_q, qm_s = hip.hip_alloc(dev, n * ff), hip.hip_alloc(dev, 4 * n * ff // 32)
+    sout = hip.hip_alloc(dev, 4 * n * d)
+    one = hip.hip_upload_new(dev, np.ones(n, np.float32))
+    hip.launch(dev, "d4_quant", (n * d + 255) // 256, 256, [norm2, qn_q, qn_s, n * d // 32])
+    if n == 1:
+        hip.launch(dev, "d4_mvq8", (ff + 3) // 4, 128, [ff, d, ff, sh.gate.qs, sh.gate.d, qn_q, qn_s, sg])
+        hip.launch(dev, "d4_mvq8", (ff + 3) // 4, 128, [ff, d, ff, sh.up.qs, sh.up.d, qn_q, qn_s, su])
+    else:
+        for w, y in ((sh.gate, sg), (sh.up, su)):
+            hip.launch(dev, "mm_q8", ((n + 63) // 64, (ff + 63) // 64), 256, [w.qs, w.d, qn_q, qn_s, y, None, ff, d, n, 0])
+    hip.launch(dev, "d4_swiglu_w", (n * ff + 255) // 256, 256, [n, ff, float(clamp), sg, su, one, smid, qm_q, qm_s])
+    if n == 1:
+        hip.launch(dev, "d4_mvq8", (d + 3) // 4, 128, [d, ff, d, sh.down.qs, sh.down.d, qm_q, qm_s, sout])
+    else:
+        hip.launch(dev, "mm_q8", ((n + 63) // 64, (d + 63) // 64), 256, [sh.down.qs, sh.down.d, qm_q, qm_s, sout, None, d, ff, n, 0])
+    hip.hip_sync(dev)
+    for b in (qn_q, qn_s, sg, su, smid, qm_q, qm_s, one):
+        hip.hip_free(b)
+    return sout
+
+
+def ffn_tail(dev, pool, sel, w, norm2, sout, clamp, keep=None):
+    """One token's routed experts SEL (weights W) on NORM2, summed in SEL's order with the
+    shared expert's SOUT (DK-FFN-TAIL): gate and up in one launch over 2k matrices, the
+    gated activation, each slot's Q8_K quantization, down, the ordered sum.  Returns MOE."""
+    d, ff, k = pool.d, pool.ff, len(sel)
+    gb = pool.gate_bytes
+    ptrs = hip.hip_upload_new(dev, np.array([pool.slot_ptr(e) for e in sel] + [pool.slot_ptr(e) + gb for e in sel], np.uint64))
+    bw = hip.hip_upload_new(dev, np.asarray(w, np.float32))
+    bgu, bm = hip.hip_alloc(dev, 4 * 2 * k * ff), hip.hip_alloc(dev, 4 * k * ff)
+    bd, moe = hip.hip_alloc(dev, 4 * k * d), hip.hip_alloc(dev, 4 * d)
+    xq, xd, xs = _q8k(dev, norm2, d)
+    hip.launch(dev, "d4_mv_iq2_xxs", ((ff + 7) // 8, 1, 2 * k), 64,
+               [d, ff, pool.grb, hip.I64(0), 0, ff, ptrs, None, xq, bgu, xd, xs])
+    hip.launch(dev, "d4_swiglu_w", (k * ff + 255) // 256, 256, [k, ff, float(clamp), bgu, bgu.at(4 * k * ff), bw, bm, None, None])
+    mq, md, ms = _q8k(dev, bm, k * ff)
+    hip.launch(dev, "d4_mv_q2_k", ((d + 7) // 8, 1, k), 64,
+               [ff, d, pool.drb, hip.I64(2 * gb), ff, d, ptrs, None, mq, bd, md, ms])
+    hip.launch(dev, "d4_moe_sum", (d + 255) // 256, 256, [d, k, bd, sout, moe, None])
+    hip.hip_sync(dev)
+    if keep is not None:
+        keep["mid"] = hip.hip_floats(bm, k * ff).reshape(k, ff)
+        keep["gu"] = hip.hip_floats(bgu, 2 * k * ff).reshape(2, k, ff)
+        keep["down"] = hip.hip_floats(bd, k * d).reshape(k, d)
+    for b in (ptrs, bw, bgu, bm, bd, xq, xd, xs, mq, md, ms):
+        hip.hip_free(b)
+    return moe
+
+
+def route(dev, logits, n, ne, nu, scale, bias=None):
+    """D4_ROUTE for N tokens' LOGITS (a DBuf): returns (sel, w) DBufs of N x NU."""
+    sel, w = hip.hip_alloc(dev, 4 * n * nu), hip.hip_alloc(dev, 4 * n * nu)
+    hip.launch(dev, "d4_route", n, ne, [ne, nu, 0, float(scale), 1 if bias is not None else 0, logits, bias, None, None, sel, w],
+               shared=4 * (2 * ne + 64 + nu))
+    return sel, w
+
+
+def group_rows(dev, sel, w, n, ne, nu):
+    """The N x NU (token, slot) rows grouped by expert (D4_GROUP_*): returns a dict of DBufs
+    counts, bases (per expert), rmap (row -> token), smap ((token, slot) -> row), wrow."""
+    rows = n * nu
+    g = {k: hip.hip_alloc(dev, 4 * (ne if k in ("counts", "bases") else rows)) for k in
+         ("counts", "bases", "rank", "rmap", "smap", "wrow")}
+    hip.launch(dev, "d4_group_zero", (ne + 255) // 256, min(ne, 256), [ne, g["counts"]])
+    hip.launch(dev, "d4_group_count", (rows + 255) // 256, 256, [rows, ne, nu, sel, g["counts"], g["rank"]])
+    hip.launch(dev, "d4_group_scan", 1, ne, [rows, ne, nu, g["counts"], g["bases"]])
+    hip.launch(dev, "d4_group_scatter", (rows + 255) // 256, 256,
+               [rows, ne, nu, sel, g["rank"], g["bases"], w, g["rmap"], g["smap"], g["wrow"]])
+    return g

@@ -1,0 +1,173 @@
+/*
+ * illatio_hip.h -- C ABI of libillatio_hip.so: illatio's quantized matrix-product path
+ * on one MI355X (gfx950).
+ *
+ * The library stands where the reference binds libcuda + NVRTC through SBCL's alien
+ * interface (src/cuda.lisp).  Part 1 mirrors the driver calls that file makes, one
+ * function each; part 2 is one typed entry point per kernel on the quantized
+ * matrix-product path, named after the reference kernel it replaces and taking that
+ * kernel's arguments in that kernel's order (grid and block shapes are chosen here, for
+ * 64-lane waves, not by the caller); part 3 launches those kernels by name from the
+ * reference's 8-byte-slot argument block, as its LAUNCH does.
+ *
+ * Conventions (src/cuda.lisp:34-57): every function returns an int, 0 on success,
+ * otherwise a HIP error code whose text ilt_error_string gives; nothing aborts or
+ * throws across the boundary.  Handles (streams, events) and device addresses are plain
+ * 64-bit values.  The library owns no memory: it allocates and frees only on request.
+ * Stream 0 is the device's default stream.
+ *
+ * Numerics.  Results are those of the reference's CPU path (src/tensor.lisp,
+ * src/kquant.lisp, src/iquant.lisp, src/ds4f.lisp), not of its CUDA kernels: the
+ * decode products and the int8 prefill products return the CPU path's bits.  So the
+ * K-quant, IQ2_XXS and Q2_K kernels take Q8_K activations (ilt_quant_q8k), where the
+ * reference's CUDA kernels take Q8_0-style blocks or floats.
+ */
+#ifndef ILLATIO_HIP_H
+#define ILLATIO_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define ILT_OK 0
+#define ILT_NOT_READY 600 /* ilt_event_query: work before the event is still running */
+
+/* Weight formats, numbered as GGUF numbers them (src/gguf.lisp:31-40). */
+#define ILT_TYPE_Q8_0 8
+#define ILT_TYPE_Q2_K 10
+#define ILT_TYPE_Q4_K 12
+#define ILT_TYPE_Q6_K 14
+#define ILT_TYPE_IQ2_XXS 16
+
+/* ---- 1. the device: what src/cuda.lisp asks of the driver --------------------------- */
+
+/* The fields of the reference's CUDEV (src/cuda.lisp:61-70). arch is reported as 90 so
+   that callers' (>= arch 80) tests choose the matrix-core paths (cuda-dense.lisp:218). */
+typedef struct ilt_device_info {
+  char name[256];
+  int arch;
+  uint64_t total_memory;
+  int max_shared;      /* LDS bytes one workgroup may use */
+  int numa_node;       /* -1 when unknown */
+  int compute_units;
+  int wave_size;
+} ilt_device_info;
+
+int ilt_init(void);                                     /* cuInit, cuda.lisp:76 */
+int ilt_device_count(int* n);                           /* cuDeviceGetCount, :78 */
+int ilt_device_get_info(int index, ilt_device_info* out); /* cuDeviceGet/GetName/GetAttribute/TotalMem, :100-135 */
+int ilt_set_device(int index);                          /* cuCtxSetCurrent, :90-92 */
+const char* ilt_error_string(int code);                 /* cuGetErrorString, :34-39 */
+
+int ilt_stream_create(uint64_t* stream, unsigned flags); /* cuStreamCreate, :133, :380-386; flags 1 = non-blocking */
+int ilt_stream_destroy(uint64_t stream);
+int ilt_stream_sync(uint64_t stream);                   /* cuStreamSynchronize, :318-319, :414 */
+int ilt_stream_wait_event(uint64_t stream, uint64_t event); /* cuStreamWaitEvent, :408-411 */
+int ilt_event_create(uint64_t* event, unsigned flags);  /* cuEventCreate, :388-393; flags 2 = no timing */
+int ilt_event_destroy(uint64_t event);                  /* cuEventDestroy, :395-396 */
+int ilt_event_record(uint64_t event, uint64_t stream);  /* cuEventRecord, :398-399 */
+int ilt_event_query(uint64_t event);                    /* cuEventQuery, :433-440: 0 done, ILT_NOT_READY pending */
+int ilt_event_elapsed_ms(uint64_t start, uint64_t stop, float* ms); /* for measurement; no reference counterpart */
+
+int ilt_malloc(uint64_t* dptr, uint64_t bytes);         /* cuMemAlloc, :239-249 (at least 256 bytes) */
+int ilt_free(uint64_t dptr);                            /* cuMemFree, :261-267 */
+int ilt_memset_async(uint64_t dptr, int byte, uint64_t bytes, uint64_t stream); /* cuMemsetD8Async, :269-273 */
+int ilt_mem_info(uint64_t* free_bytes, uint64_t* total_bytes); /* cuMemGetInfo, :275-281 */
+int ilt_memcpy_htod_async(uint64_t dst, const void* src, uint64_t bytes, uint64_t stream); /* :283-291, :416-421 */
+int ilt_memcpy_dtoh_async(void* dst, uint64_t src, uint64_t bytes, uint64_t stream);       /* :302-309, :430-431 */
+int ilt_memcpy_dtod_async(uint64_t dst, uint64_t src, uint64_t bytes, uint64_t stream);    /* :423-428 */
+int ilt_host_alloc(uint64_t* hptr, uint64_t bytes, unsigned flags); /* cuMemHostAlloc, :371-378; flags 1 portable, 2 mapped */
+int ilt_host_free(uint64_t hptr);                       /* cuMemFreeHost, :380 */
+int ilt_host_register(void* p, uint64_t bytes, unsigned flags); /* cuMemHostRegister, :359-366 */
+int ilt_host_unregister(void* p);                       /* cuMemHostUnregister, :368-369 */
+
+/* ---- 2. the kernels --------------------------------------------------------------------
+ * Pointers are device addresses.  "|0" marks an argument that may be null.             */
+
+/* Upload-time repacks (cuda-dense.lisp:87-100).
+   repack_q8 (src/cuda/dense.cu:42): GGUF Q8_0 blocks -> int8 quants + f16 scales.
+   repack_q6k (src/cuda/kquant.cu:195): the reference pads Q6_K blocks to 224 bytes; here
+   the 210-byte blocks are read where they lie, so this copies them unchanged (out needs
+   210*nblocks bytes; the reference's 224*nblocks is enough). */
+int ilt_repack_q8(uint64_t stream, const void* raw, void* qs, void* d, int64_t nblocks);
+int ilt_repack_q6k(uint64_t stream, const void* raw, void* out, int64_t nblocks);
+
+/* Activation quantizers.
+   quant_q8 (dense.cu:84; CPU: quantize-q8!, tensor.lisp:245-262 with *q8-f16-scale* T):
+     blocks of 32, scale stored rounded through fp16; xsum|0 gets each block's integer sum.
+   d4_quant (ds4f.cu:35; *q8-f16-scale* NIL, ds4f.lisp:1052-1053): the scale kept a float.
+   quant_q8k (no CUDA counterpart; CPU: quantize-q8k!, kquant.lisp:130-167): blocks of
+     256, xd one float per block, bsums one int32 per 16 quants. */
+int ilt_quant_q8(uint64_t stream, const float* x, int8_t* xq, float* xs, int32_t* xsum, int64_t nblocks);
+int ilt_d4_quant(uint64_t stream, const float* x, int8_t* xq, float* xs, int nblocks);
+int ilt_quant_q8k(uint64_t stream, const float* x, int8_t* xq, float* xd, int32_t* bsums, int64_t nblocks);
+
+/* Decode products, y[r] = W[r].x (+ bias[r]); acc: y += that.
+   mv_q8 (dense.cu:194; CPU: matvec!, tensor.lisp:321-352): W repacked by ilt_repack_q8.
+   mv_k (kquant.cu:169; CPU: q4k-row-dot / q6k-row-dot, kquant.lisp:171-236): type 0 Q4_K,
+     2 Q6_K (kquant-code, cuda-dense.lisp:18-20); w the GGUF blocks; xq/xd/bsums from
+     ilt_quant_q8k.
+   mv_q8_3 (dense.cu:210): three products sharing x in one call.
+   d4_mvq8 (ds4f.cu:50): Q8_0, row r against the activations of group r/group_rows. */
+int ilt_mv_q8(uint64_t stream, const int8_t* wq, const uint16_t* wd, const int8_t* xq, const float* xs, float* out,
+              const float* bias, int rows, int cols, int acc);
+int ilt_mv_q8_3(uint64_t stream, const int8_t* q0, const uint16_t* d0, const int8_t* q1, const uint16_t* d1,
+                const int8_t* q2, const uint16_t* d2, const int8_t* xq, const float* xs, float* o0, float* o1, float* o2,
+                const float* b0, const float* b1, const float* b2, int r0, int r1, int r2, int cols);
+int ilt_mv_k(uint64_t stream, int type, const void* w, const int8_t* xq, const float* xd, const int32_t* bsums, float* out,
+             const float* bias, int rows, int cols, int acc);
+int ilt_d4_mvq8(uint64_t stream, int rows, int cols, int group_rows, const int8_t* wq, const uint16_t* wd,
+                const int8_t* xq, const float* xs, float* y);
+
+/* The indexed expert products (ds4f.cu:769, 837; CPU: iq2xxs-row-dot, q2k-row-dot,
+   iquant.lisp:126-215).  For each z < nz: W = the nrows x ncols matrix at ptrs[z] + add
+   (row_bytes apart), x = the Q8_K activations at element z*x_stride, y = dst + z*y_stride.
+   The reference's grid z (cuda-ds4f.lisp:937-941) is nz here. */
+int ilt_d4_mv_iq2_xxs(uint64_t stream, int ncols, int nrows, int row_bytes, int64_t add, int x_stride, int y_stride,
+                      const uint64_t* ptrs, int nz, const int8_t* xq, const float* xd, float* dst);
+int ilt_d4_mv_q2_k(uint64_t stream, int ncols, int nrows, int row_bytes, int64_t add, int x_stride, int y_stride,
+                   const uint64_t* ptrs, int nz, const int8_t* xq, const float* xd, const int32_t* bsums, float* dst);
+
+/* Rows as floats (dense.cu:53 embed_q8, kquant.cu:202 embed_k; CPU: q8mat-row!, kmat-row!,
+   iq2xxs-row-floats!, q2k-row-floats!): out[n] = row tokens[n] (row n when tokens is null)
+   of W, bit-exact.  ilt_dequant_rows takes a GGUF type (any of the five; Q8_0 repacked,
+   wd its scales). */
+int ilt_embed_q8(uint64_t stream, const int8_t* qs, const uint16_t* d, const int32_t* tokens, float* out, int cols, int n);
+int ilt_embed_k(uint64_t stream, int type, const void* w, const int32_t* tokens, float* out, int cols, int n);
+int ilt_dequant_rows(uint64_t stream, int gguf_type, const void* w, const uint16_t* wd, const int32_t* rows_idx,
+                     int64_t nrows, int cols, float* out);
+
+/* The expert path's small kernels (ds4f.cu:645, 902; ds4f_chunk.cu:393-508; CPU:
+   d4-route, d4-routed!, ds4f.lisp:950-1037, 1169-1239).  d4_route routes ntok tokens
+   (the reference's grid x).  hash 0: top-nu; 1: tid2eid table.  has_bias 0/1/2 as there. */
+int ilt_d4_route(uint64_t stream, int ne, int nu, int hash, float scale, int has_bias, const float* logits,
+                 const float* bias, const int32_t* tid2eid, const uint32_t* tokens, uint32_t* sel, float* wout, int ntok);
+int ilt_d4_group_zero(uint64_t stream, int ne, uint32_t* counts);
+int ilt_d4_group_count(uint64_t stream, int n, int ne, int nu, const uint32_t* sel, uint32_t* counts, uint32_t* rank);
+int ilt_d4_group_scan(uint64_t stream, int n, int ne, int nu, const uint32_t* counts, uint32_t* bases);
+int ilt_d4_group_scatter(uint64_t stream, int n, int ne, int nu, const uint32_t* sel, const uint32_t* rank,
+                         const uint32_t* bases, const float* w, uint32_t* rmap, uint32_t* smap, float* wrow);
+int ilt_d4_gather_rows(uint64_t stream, int d, int nrows, const float* src, const uint32_t* map, float* x);
+int ilt_d4_swiglu_w(uint64_t stream, int n, int ff, float clamp, const float* g, const float* u, const float* w,
+                    float* mid, int8_t* xq, float* xs);
+int ilt_d4_moe_sum(uint64_t stream, int d, int k, const float* down, const float* shared_, float* moe, const uint32_t* perm);
+int ilt_d4_moe_sum_rows(uint64_t stream, int d, int nu, int ntok, const float* down, const uint32_t* map,
+                        const float* shared_, float* moe);
+
+/* ---- 3. launch by name (src/cuda.lisp:323-352) -------------------------------------------
+ * params[i] points at argument i's 8-byte slot: a pointer as 64 bits, an int in the low
+ * 32 bits, a float in the low 32 bits, a long long as 64 bits.  Kernel names and argument
+ * orders are the reference's (its src/cuda/ *.cu); the grid and block passed in are read
+ * only where an argument count lives in them (d4_route: tokens = gx; d4_mv_*: experts =
+ * gz).  For d4_mv_iq2_xxs / d4_mv_q2_k the slots "src1, counts, bases" carry the Q8_K
+ * activations "xq, xd, bsums" and srcs must be null.  Unknown names return
+ * hipErrorNotFound. */
+int ilt_launch(const char* kernel, unsigned gx, unsigned gy, unsigned gz, unsigned bx, unsigned by, unsigned bz,
+               unsigned shared_bytes, uint64_t stream, void** params);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* ILLATIO_HIP_H */

@@ -1,0 +1,212 @@
+"""GPU parity of the quantizers, the upload repack, the row dequantizers and the decode
+products against the CPU oracle, through the C ABI (via the Lisp-shaped LAUNCH).  Integer
+and byte results are compared bit for bit; so are the float products, because the kernels
+add a row's block terms in the CPU path's order."""
+import numpy as np
+import pytest
+
+import oracle_lib as orc
+from illatio_amd import synth
+
+pytestmark = pytest.mark.gpu
+
+TYPES = [synth.Q8_0, synth.Q4_K, synth.Q6_K, synth.Q2_K, synth.IQ2_XXS]
+
+
+@pytest.fixture(scope="module")
+def dev():
+    from illatio_amd import hip
+    return hip.open_hip(0)
+
+
+def bits(a):
+    return np.ascontiguousarray(a, np.float32).view(np.uint32)
+
+
+def special_activations(cols, rng):
+    x = synth.activations(cols, rng)
+    x[0:32] = 0.0                      # a zero Q8_0 block
+    if cols >= 512:
+        x[256:512] = 0.0               # a zero Q8_K block
+    x[40] = -7.5                       # block maximum on a negative value
+    x[70] = 3.25; x[90] = -3.25        # equal magnitudes: the first wins
+    return x
+
+
+@pytest.mark.parametrize("n", [32, 2560, 4864, 32 * 1000 + 32])
+def test_quant_q8_bit_exact(dev, n):
+    from illatio_amd import hip
+    rng = synth.make_rng(n)
+    x = special_activations(n, rng) if n >= 128 else synth.activations(n, rng)
+    xb = hip.hip_upload_new(dev, x)
+    for f16 in (True, False):
+        q, s, sm = hip.hip_alloc(dev, n), hip.hip_alloc(dev, 4 * n // 32), hip.hip_alloc(dev, 4 * n // 32)
+        if f16:
+            hip.launch(dev, "quant_q8", (n + 255) // 256, 256, [xb, q, s, sm, hip.I64(n // 32)])
+        else:
+            hip.launch(dev, "d4_quant", (n + 255) // 256, 256, [xb, q, s, n // 32])
+        wq, ws = orc.quantize_q8(x, f16)
+        assert np.array_equal(hip.hip_download(q, np.int8, n), wq)
+        assert np.array_equal(bits(hip.hip_floats(s, n // 32)), bits(ws))
+        if f16:
+            assert np.array_equal(hip.hip_download(sm, np.int32, n // 32), wq.astype(np.int32).reshape(-1, 32).sum(axis=1))
+        for b in (q, s, sm):
+            hip.hip_free(b)
+    hip.hip_free(xb)
+
+
+@pytest.mark.parametrize("n", [256, 2560, 9728, 256 * 96])
+def test_quant_q8k_bit_exact(dev, n):
+    from illatio_amd import hip
+    rng = synth.make_rng(n + 1)
+    x = special_activations(n, rng)
+    xb = hip.hip_upload_new(dev, x)
+    q, d, bs = hip.hip_alloc(dev, n), hip.hip_alloc(dev, 4 * n // 256), hip.hip_alloc(dev, 4 * n // 16)
+    hip.launch(dev, "quant_q8k", n // 256, 256, [xb, q, d, bs, hip.I64(n // 256)])
+    wq, wd, wbs = orc.quantize_q8k(x)
+    assert np.array_equal(hip.hip_download(q, np.int8, n), wq)
+    assert np.array_equal(bits(hip.hip_floats(d, n // 256)), bits(wd))
+    assert np.array_equal(hip.hip_download(bs, np.int32, n // 16), wbs)
+    for b in (xb, q, d, bs):
+        hip.hip_free(b)
+
+
+def upload(dev, qtype, rows, cols, w):
+    """The matrix as the kernels read it: Q8_0 repacked, the rest in GGUF blocks."""
+    from illatio_amd import dense, hip
+    if qtype in (synth.Q8_0, synth.Q4_K, synth.Q6_K):
+        return dense.upload_gmat(dev, "w", qtype, rows, cols, w)
+    return dense.CMat("w", qtype, rows, cols, hip.hip_upload_new(dev, w))
+
+
+@pytest.mark.parametrize("qtype", TYPES)
+def test_dequant_rows_bit_exact(dev, qtype):
+    from illatio_amd import hip
+    import ctypes as C
+    rng = synth.make_rng(40 + qtype)
+    rows, cols = 40, 1024
+    w = synth.weights(qtype, rows, cols, rng)
+    m = upload(dev, qtype, rows, cols, w)
+    idx = np.array([3, 0, 39, 17, 3], np.int32)
+    ib = hip.hip_upload_new(dev, idx)
+    out = hip.hip_alloc(dev, 4 * len(idx) * cols)
+    hip.call("ilt_dequant_rows", C.c_uint64(dev.stream), C.c_int(qtype), C.c_uint64(m.qs.ptr),
+             C.c_uint64(m.d.ptr if m.d else 0), C.c_uint64(ib.ptr), C.c_int64(len(idx)), C.c_int(cols), C.c_uint64(out.ptr))
+    got = hip.hip_floats(out, len(idx) * cols).reshape(len(idx), cols)
+    want = orc.dequant_rows(qtype, w, cols)[idx]
+    assert np.array_equal(bits(got), bits(want))
+    if qtype in (synth.Q8_0, synth.Q4_K, synth.Q6_K):
+        from illatio_amd import dense
+        out2 = hip.hip_alloc(dev, 4 * len(idx) * cols)
+        dense.embed(dev, m, ib, out2, len(idx), cols)
+        assert np.array_equal(bits(hip.hip_floats(out2, len(idx) * cols).reshape(len(idx), cols)), bits(want))
+        hip.hip_free(out2)
+    for b in (ib, out):
+        hip.hip_free(b)
+    m.free()
+
+
+DENSE_SHAPES = {
+    synth.Q8_0: [(4864, 896), (896, 4864), (36, 64), (1, 32)],       # BASELINE config 1, then ragged
+    synth.Q4_K: [(4096, 2560), (2560, 4096), (1024, 2560), (100, 9728), (3, 256)],
+    synth.Q6_K: [(1024, 2560), (2560, 9728), (64, 5120), (37, 512)],
+}
+
+
+@pytest.mark.parametrize("qtype", [synth.Q8_0, synth.Q4_K, synth.Q6_K])
+def test_dense_gemv_matches_cpu_path_bit_for_bit(dev, qtype):
+    from illatio_amd import dense, hip
+    for rows, cols in DENSE_SHAPES[qtype]:
+        rng = synth.make_rng(1000 * qtype + rows + cols)
+        w = synth.weights(qtype, rows, cols, rng)
+        x = special_activations(cols, rng) if cols >= 512 else synth.activations(cols, rng)
+        bias = synth.activations(rows, rng)
+        m = upload(dev, qtype, rows, cols, w)
+        act = dense.QAct(dev, 1, cols, ("q8",) if qtype == synth.Q8_0 else ("q8k",))
+        xb, bb = hip.hip_upload_new(dev, x), hip.hip_upload_new(dev, bias)
+        y = hip.hip_alloc(dev, 4 * rows)
+        dense.quantize_act(dev, xb, act)
+        dense.cmat_mul(dev, m, act, y)
+        want = orc.matmul(qtype, w, rows, cols, x)
+        got = hip.hip_floats(y, rows)
+        assert np.array_equal(bits(got), bits(want)), (qtype, rows, cols, np.abs(got - want).max())
+        # + bias, then accumulate on top: y = (W.x + b) + (W.x + b)
+        dense.cmat_mul(dev, m, act, y, bias=bb)
+        wb = want + bias
+        assert np.array_equal(bits(hip.hip_floats(y, rows)), bits(wb))
+        dense.cmat_mul(dev, m, act, y, bias=bb, acc=True)
+        assert np.array_equal(bits(hip.hip_floats(y, rows)), bits(wb + wb))
+        for b in (xb, bb, y):
+            hip.hip_free(b)
+        act.free(); m.free()
+
+
+def test_d4_mvq8_grouped_rows(dev):
+    """Row r against the activations of group r / group_rows (ds4f.cu:50-62)."""
+    from illatio_amd import dense, hip
+    rng = synth.make_rng(77)
+    rows, cols, groups = 96, 256, 3
+    w = synth.weights(synth.Q8_0, rows, cols, rng)
+    x = synth.activations((groups, cols), rng)
+    m = upload(dev, synth.Q8_0, rows, cols, w)
+    xb = hip.hip_upload_new(dev, x)
+    q, s = hip.hip_alloc(dev, groups * cols), hip.hip_alloc(dev, 4 * groups * cols // 32)
+    y = hip.hip_alloc(dev, 4 * rows)
+    hip.launch(dev, "d4_quant", (groups * cols + 255) // 256, 256, [xb, q, s, groups * cols // 32])
+    hip.launch(dev, "d4_mvq8", (rows + 3) // 4, 128, [rows, cols, rows // groups, m.qs, m.d, q, s, y])
+    got = hip.hip_floats(y, rows)
+    gr = rows // groups
+    for g in range(groups):
+        want = orc.matmul(synth.Q8_0, w[g * gr:(g + 1) * gr], gr, cols, x[g], f16_scale=False)
+        assert np.array_equal(bits(got[g * gr:(g + 1) * gr]), bits(want))
+    for b in (xb, q, s, y):
+        hip.hip_free(b)
+    m.free()
+
+
+@pytest.mark.parametrize("qtype,rows,cols", [(synth.IQ2_XXS, 2048, 4096), (synth.Q2_K, 4096, 2048),
+                                              (synth.IQ2_XXS, 50, 512), (synth.Q2_K, 9, 256)])
+def test_indexed_expert_gemv_bit_for_bit(dev, qtype, rows, cols):
+    """ptrs[z] + add addressing, per-z activations (x_stride) and outputs (y_stride)."""
+    from illatio_amd import hip
+    rng = synth.make_rng(qtype * 7 + rows)
+    nexp, nz = 5, 3
+    rb = synth.row_bytes(qtype, cols)
+    pad = 512
+    slot = (pad + rows * rb + 255) // 256 * 256
+    w = synth.weights(qtype, nexp * rows, cols, rng).reshape(nexp, rows * rb)
+    host = np.zeros((nexp, slot), np.uint8)
+    host[:, pad:pad + rows * rb] = w
+    pool = hip.hip_upload_new(dev, host)
+    chosen = [4, 0, 2]
+    ptrs = hip.hip_upload_new(dev, np.array([pool.ptr + e * slot for e in chosen], np.uint64))
+    for x_stride in (0, cols):
+        x = special_activations(cols * nz, rng).reshape(nz, cols) if cols >= 512 else synth.activations((nz, cols), rng)
+        xb = hip.hip_upload_new(dev, x)
+        kq, kd, ks = hip.hip_alloc(dev, nz * cols), hip.hip_alloc(dev, 4 * nz * cols // 256), hip.hip_alloc(dev, 4 * nz * cols // 16)
+        hip.launch(dev, "quant_q8k", nz * cols // 256, 256, [xb, kq, kd, ks, hip.I64(nz * cols // 256)])
+        y = hip.hip_alloc(dev, 4 * nz * rows)
+        name = "d4_mv_iq2_xxs" if qtype == synth.IQ2_XXS else "d4_mv_q2_k"
+        hip.launch(dev, name, ((rows + 7) // 8, 1, nz), 64,
+                   [cols, rows, rb, hip.I64(pad), x_stride, rows, ptrs, None, kq, y, kd, ks])
+        got = hip.hip_floats(y, nz * rows).reshape(nz, rows)
+        for z, e in enumerate(chosen):
+            want = orc.matmul(qtype, w[e].reshape(rows, rb), rows, cols, x[z if x_stride else 0])
+            assert np.array_equal(bits(got[z]), bits(want)), (qtype, z, np.abs(got[z] - want).max())
+        for b in (xb, kq, kd, ks, y):
+            hip.hip_free(b)
+    hip.hip_free(pool); hip.hip_free(ptrs)
+
+
+def test_invalid_arguments_are_errors_not_faults(dev):
+    from illatio_amd import hip
+    b = hip.hip_alloc(dev, 4096)
+    with pytest.raises(hip.HipError):
+        hip.launch(dev, "mv_q8", 1, 128, [b, b, b, b, b, None, 4, 48, 0])        # cols not a multiple of 32
+    with pytest.raises(hip.HipError):
+        hip.launch(dev, "mv_k", 1, 128, [1, b, b, b, b, b, None, 4, 256, 0])      # Q5_K is not built
+    with pytest.raises(hip.HipError):
+        hip.launch(dev, "no_such_kernel", 1, 1, [])
+    with pytest.raises(hip.HipError):
+        hip.launch(dev, "mv_q8", 1, 128, [None, b, b, b, b, None, 4, 32, 0])      # null weights
+    hip.hip_free(b)
