@@ -1,0 +1,155 @@
+"""GPU parity of the MoE expert path's kernels against the CPU oracle: routing (indices
+and weights bit for bit), the grouping of (token, slot) rows by expert, the gather, the
+gated activation, and one token's whole routed + shared FFN (DK-FFN-TAIL's sequence)."""
+import numpy as np
+import pytest
+
+import oracle_lib as orc
+from illatio_amd import synth
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def dev():
+    from illatio_amd import hip
+    return hip.open_hip(0)
+
+
+def bits(a):
+    return np.ascontiguousarray(a, np.float32).view(np.uint32)
+
+
+@pytest.mark.parametrize("ne,nu,n", [(256, 6, 64), (16, 3, 5), (64, 8, 33)])
+def test_route_indices_and_weights_bit_exact(dev, ne, nu, n):
+    from illatio_amd import ds4f, hip
+    rng = synth.make_rng(ne + n)
+    logits = synth.zipf_router_logits(n, ne, rng)
+    logits[1, :] = 0.25                                    # every expert equal: the first nu win, in order
+    logits[2, ne // 2:] = logits[2, 0]                     # many exact ties
+    logits[3, :4] = [30.0, -30.0, 21.0, -21.0]             # softplus's outer branches
+    for bias in (None, (rng.standard_normal(ne) * 0.05).astype(np.float32)):
+        lb = hip.hip_upload_new(dev, logits)
+        bb = None if bias is None else hip.hip_upload_new(dev, bias)
+        sel, w = ds4f.route(dev, lb, n, ne, nu, 1.5, bb)
+        gs = hip.hip_download(sel, np.uint32, n * nu).reshape(n, nu)
+        gw = hip.hip_floats(w, n * nu).reshape(n, nu)
+        for t in range(n):
+            ws, ww = orc.route(logits[t], nu, 1.5, bias)
+            assert gs[t].tolist() == ws.tolist(), (t, gs[t], ws)
+            assert np.array_equal(bits(gw[t]), bits(ww)), t
+        if bias is None:
+            assert gs[1].tolist() == list(range(nu))
+        for b in (lb, bb, sel, w):
+            hip.hip_free(b)
+
+
+def test_group_rows_invariants_and_gather(dev):
+    from illatio_amd import ds4f, hip
+    rng = synth.make_rng(5)
+    n, ne, nu, d = 300, 256, 6, 64
+    logits = synth.zipf_router_logits(n, ne, rng)
+    lb = hip.hip_upload_new(dev, logits)
+    sel, w = ds4f.route(dev, lb, n, ne, nu, 1.5)
+    g = ds4f.group_rows(dev, sel, w, n, ne, nu)
+    rows = n * nu
+    hs = hip.hip_download(sel, np.uint32, rows)
+    hw = hip.hip_floats(w, rows)
+    counts = hip.hip_download(g["counts"], np.uint32, ne)
+    bases = hip.hip_download(g["bases"], np.uint32, ne)
+    rmap = hip.hip_download(g["rmap"], np.uint32, rows)
+    smap = hip.hip_download(g["smap"], np.uint32, rows)
+    wrow = hip.hip_floats(g["wrow"], rows)
+    assert np.array_equal(counts, np.bincount(hs, minlength=ne))
+    assert np.array_equal(bases, np.concatenate([[0], np.cumsum(counts)[:-1]]))
+    assert sorted(smap.tolist()) == list(range(rows))                      # a permutation
+    assert np.array_equal(rmap[smap], np.arange(rows) // nu)               # row -> its token
+    assert np.array_equal(bits(wrow[smap]), bits(hw))
+    e_of_row = np.searchsorted(np.cumsum(counts), np.arange(rows), side="right")
+    assert np.array_equal(e_of_row[smap], hs)                              # each row inside its expert's range
+    src = synth.activations((n, d), rng)
+    sb = hip.hip_upload_new(dev, src)
+    x = hip.hip_alloc(dev, 4 * rows * d)
+    hip.launch(dev, "d4_gather_rows", (rows * d + 255) // 256, 256, [d, rows, sb, g["rmap"], x])
+    assert np.array_equal(bits(hip.hip_floats(x, rows * d).reshape(rows, d)), bits(src[rmap]))
+    # the slot-ordered sum over rows, with the shared expert's rows added after
+    down = synth.activations((rows, d), rng)
+    shared = synth.activations((n, d), rng)
+    db, shb, moe = hip.hip_upload_new(dev, down), hip.hip_upload_new(dev, shared), hip.hip_alloc(dev, 4 * n * d)
+    hip.launch(dev, "d4_moe_sum_rows", (n * d + 255) // 256, 256, [d, nu, n, db, g["smap"], shb, moe])
+    want = np.zeros((n, d), np.float32)
+    for s in range(nu):
+        want = want + down[smap.reshape(n, nu)[:, s]]
+    want = want + shared
+    assert np.array_equal(bits(hip.hip_floats(moe, n * d).reshape(n, d)), bits(want))
+    for b in [lb, sel, w, sb, x, db, shb, moe] + list(g.values()):
+        hip.hip_free(b)
+
+
+@pytest.mark.parametrize("clamp", [0.0, 0.7])
+def test_swiglu_w_matches_cpu_silu(dev, clamp):
+    from illatio_amd import hip
+    rng = synth.make_rng(9)
+    n, ff = 6, 512
+    g = (synth.activations((n, ff), rng) * 3).astype(np.float32)
+    u = synth.activations((n, ff), rng)
+    g[0, :6] = [0.0, -0.0, 25.0, -25.0, 88.0, -100.0]
+    w = (rng.random(n, dtype=np.float32) + 0.1).astype(np.float32)
+    gb, ub, wb = (hip.hip_upload_new(dev, a) for a in (g, u, w))
+    mid, xq, xs = hip.hip_alloc(dev, 4 * n * ff), hip.hip_alloc(dev, n * ff), hip.hip_alloc(dev, 4 * n * ff // 32)
+    hip.launch(dev, "d4_swiglu_w", (n * ff + 255) // 256, 256, [n, ff, float(clamp), gb, ub, wb, mid, xq, xs])
+    got = hip.hip_floats(mid, n * ff).reshape(n, ff)
+    want = np.empty_like(got)
+    for r in range(n):
+        for j in range(ff):
+            gv, uv = g[r, j], u[r, j]
+            if clamp > 1e-6:
+                gv = min(gv, np.float32(clamp)); uv = max(np.float32(-clamp), min(uv, np.float32(clamp)))
+            want[r, j] = (np.float32(orc.silu(gv)) * uv) * w[r]
+    assert np.array_equal(bits(got), bits(want)), np.abs(got - want).max()
+    wq, ws = orc.quantize_q8(want, f16_scale=False)
+    assert np.array_equal(hip.hip_download(xq, np.int8, n * ff), wq)
+    assert np.array_equal(bits(hip.hip_floats(xs, n * ff // 32)), bits(ws))
+    for b in (gb, ub, wb, mid, xq, xs):
+        hip.hip_free(b)
+
+
+def _moe_weights(rng, ne, d, ff):
+    gate = synth.weights(synth.IQ2_XXS, ne * ff, d, rng)
+    up = synth.weights(synth.IQ2_XXS, ne * ff, d, rng)
+    down = synth.weights(synth.Q2_K, ne * d, ff, rng)
+    sg = synth.weights(synth.Q8_0, ff, d, rng)
+    su = synth.weights(synth.Q8_0, ff, d, rng)
+    sd = synth.weights(synth.Q8_0, d, ff, rng)
+    return gate, up, down, sg, su, sd
+
+
+@pytest.mark.parametrize("ne,d,ff,nu,clamp", [(8, 512, 256, 3, 0.0), (8, 512, 256, 3, 0.05), (12, 4096, 2048, 6, 0.0)])
+def test_moe_decode_step_bit_exact(dev, ne, d, ff, nu, clamp):
+    """BASELINE config 4's sequence at a reduced expert count (12 resident experts of the
+    full 4096 x 2048 shape), and a small shape with the clamp on: route -> gate/up -> gated
+    activation -> per-slot Q8_K -> down -> ordered sum + shared expert."""
+    from illatio_amd import ds4f, hip
+    rng = synth.make_rng(ne * 1000 + d)
+    gate, up, down, sg, su, sd = _moe_weights(rng, ne, d, ff)
+    pool = ds4f.ExpertPool(dev, ne, d, ff, gate, up, down)
+    sh = ds4f.SharedExpert(dev, d, ff, sg, su, sd)
+    for trial in range(2):
+        norm = synth.activations(d, rng)
+        logits = synth.activations(ne, rng)
+        want, wsel, ww = orc.moe_token(gate, up, down, sg, su, sd, d, ff, ne, nu, 1.5, clamp, logits, norm)
+        lb, nb = hip.hip_upload_new(dev, logits), hip.hip_upload_new(dev, norm)
+        sel, w = ds4f.route(dev, lb, 1, ne, nu, 1.5)
+        hsel, hw = hip.hip_download(sel, np.uint32, nu), hip.hip_floats(w, nu)
+        assert hsel.tolist() == wsel.tolist() and np.array_equal(bits(hw), bits(ww))
+        sout = ds4f.ffn_shared(dev, sh, nb, clamp)
+        assert np.array_equal(bits(hip.hip_floats(sout, d)), bits(orc.moe_shared(sg, su, sd, d, ff, clamp, norm)))
+        keep = {}
+        moe = ds4f.ffn_tail(dev, pool, hsel, hw, nb, sout, clamp, keep)
+        _, wmid = orc.moe_routed(gate, up, down, d, ff, wsel, ww, clamp, norm)
+        assert np.array_equal(bits(keep["mid"]), bits(wmid)), np.abs(keep["mid"] - wmid).max()
+        got = hip.hip_floats(moe, d)
+        assert np.array_equal(bits(got), bits(want)), np.abs(got - want).max()
+        for b in (lb, nb, sel, w, sout, moe):
+            hip.hip_free(b)
+    pool.free(); sh.free()
