@@ -296,6 +296,46 @@ int ilt_d4_moe_sum_rows(uint64_t stream, int d, int nu, int ntok, const float* d
   return (int)ilt_k_moe_sum_rows(d, nu, ntok, down, map, shared_, moe, S(stream));
 }
 
+int ilt_mm_q8(uint64_t stream, const int8_t* wq, const uint16_t* wd, const int8_t* xq, const float* xs, float* y,
+              const float* bias, int rows, int cols, int n, int acc) {
+  ILT_REQUIRE(rows >= 0 && n >= 0 && cols > 0 && cols % 32 == 0);
+  if (rows == 0 || n == 0) return ILT_OK;
+  ILT_REQUIRE(wq && wd && xq && xs && y && ((uintptr_t)wq & 15) == 0 && ((uintptr_t)xq & 15) == 0 && cols % 16 == 0);
+  return (int)ilt_k_gemm_i8(ILT_Q8_0, (const uint8_t*)wq, wd, cols, rows, cols, xq, xs, nullptr, n, y, bias, acc, S(stream));
+}
+
+int ilt_mm_k(uint64_t stream, int type, const void* w, const int8_t* xq, const float* xd, const int32_t* bsums, float* y,
+             const float* bias, int rows, int cols, int n, int acc) {
+  const int fmt = kquant_type(type);
+  ILT_REQUIRE(fmt && rows >= 0 && n >= 0 && cols > 0 && cols % 256 == 0);
+  if (rows == 0 || n == 0) return ILT_OK;
+  ILT_REQUIRE(w && xq && xd && bsums && y && ((uintptr_t)w & 15) == 0 && ((uintptr_t)xq & 15) == 0);
+  return (int)ilt_k_gemm_i8(fmt, (const uint8_t*)w, nullptr, (long long)cols / 256 * block_bytes(fmt), rows, cols, xq, xd,
+                            bsums, n, y, bias, acc, S(stream));
+}
+
+static int mm_id(uint64_t stream, int fmt, int ncols, int nrows, int row_bytes, int64_t add, const uint64_t* ptrs,
+                 const uint32_t* counts, const uint32_t* bases, int ne, int64_t total_rows, const int8_t* xq,
+                 const float* xd, const int32_t* bsums, float* y) {
+  ILT_REQUIRE(ncols > 0 && ncols % 256 == 0 && nrows >= 0 && ne >= 0 && ne <= 256 && total_rows >= 0);
+  ILT_REQUIRE(row_bytes == ncols / 256 * block_bytes(fmt) && add >= 0 && (add & 1) == 0);
+  if (nrows == 0 || ne == 0 || total_rows == 0) return ILT_OK;
+  ILT_REQUIRE(ptrs && counts && bases && xq && xd && y && (bsums || fmt == ILT_IQ2_XXS) && ((uintptr_t)xq & 15) == 0);
+  return (int)ilt_k_gemm_i8_id(fmt, ptrs, add, counts, bases, ne, row_bytes, nrows, ncols, xq, xd, bsums, total_rows, y, S(stream));
+}
+
+int ilt_d4_mm_id_iq2_xxs(uint64_t stream, int ncols, int nrows, int row_bytes, int64_t add, const uint64_t* ptrs,
+                         const uint32_t* counts, const uint32_t* bases, int ne, int64_t total_rows,
+                         const int8_t* xq, const float* xd, float* y) {
+  return mm_id(stream, ILT_IQ2_XXS, ncols, nrows, row_bytes, add, ptrs, counts, bases, ne, total_rows, xq, xd, nullptr, y);
+}
+
+int ilt_d4_mm_id_q2_k(uint64_t stream, int ncols, int nrows, int row_bytes, int64_t add, const uint64_t* ptrs,
+                      const uint32_t* counts, const uint32_t* bases, int ne, int64_t total_rows,
+                      const int8_t* xq, const float* xd, const int32_t* bsums, float* y) {
+  return mm_id(stream, ILT_Q2_K, ncols, nrows, row_bytes, add, ptrs, counts, bases, ne, total_rows, xq, xd, bsums, y);
+}
+
 // ---- launch by name ---------------------------------------------------------------------------
 int ilt_launch(const char* kernel, unsigned gx, unsigned gy, unsigned gz, unsigned bx, unsigned by, unsigned bz,
                unsigned shared_bytes, uint64_t stream, void** params) {
@@ -317,6 +357,21 @@ int ilt_launch(const char* kernel, unsigned gx, unsigned gy, unsigned gz, unsign
                                   a.i32(16), a.i32(17));
   K("mv_k") return ilt_mv_k(stream, a.i32(0), a.ptr<const void*>(1), a.ptr<ci8>(2), a.ptr<cf>(3), a.ptr<const int32_t*>(4),
                             a.ptr<float*>(5), a.ptr<cf>(6), a.i32(7), a.i32(8), a.i32(9));
+  if (!strcmp(kernel, "mm_q8") || !strcmp(kernel, "mm_q8_mma"))
+    return ilt_mm_q8(stream, a.ptr<ci8>(0), a.ptr<cu16>(1), a.ptr<ci8>(2), a.ptr<cf>(3), a.ptr<float*>(4), a.ptr<cf>(5),
+                     a.i32(6), a.i32(7), a.i32(8), a.i32(9));
+  K("mm_k") return ilt_mm_k(stream, a.i32(0), a.ptr<const void*>(1), a.ptr<ci8>(2), a.ptr<cf>(3), a.ptr<const int32_t*>(4),
+                            a.ptr<float*>(5), a.ptr<cf>(6), a.i32(7), a.i32(8), a.i32(9), a.i32(10));
+  if (!strcmp(kernel, "mm_q4k_mma") || !strcmp(kernel, "mm_q6k_mma"))
+    return ilt_mm_k(stream, kernel[4] == '4' ? 0 : 2, a.ptr<const void*>(0), a.ptr<ci8>(1), a.ptr<cf>(2),
+                    a.ptr<const int32_t*>(3), a.ptr<float*>(4), a.ptr<cf>(5), a.i32(6), a.i32(7), a.i32(8), a.i32(9));
+  K("d4_mm_id_iq2_xxs")
+    return ilt_d4_mm_id_iq2_xxs(stream, a.i32(0), a.i32(1), a.i32(2), a.i64(5), a.ptr<const uint64_t*>(6), a.ptr<cu32>(7),
+                                a.ptr<cu32>(8), (int)gz, a.i64(13), a.ptr<ci8>(9), a.ptr<cf>(11), a.ptr<float*>(10));
+  K("d4_mm_id_q2_k")
+    return ilt_d4_mm_id_q2_k(stream, a.i32(0), a.i32(1), a.i32(2), a.i64(5), a.ptr<const uint64_t*>(6), a.ptr<cu32>(7),
+                             a.ptr<cu32>(8), (int)gz, a.i64(13), a.ptr<ci8>(9), a.ptr<cf>(11), a.ptr<const int32_t*>(12),
+                             a.ptr<float*>(10));
   K("d4_mvq8") return ilt_d4_mvq8(stream, a.i32(0), a.i32(1), a.i32(2), a.ptr<ci8>(3), a.ptr<cu16>(4), a.ptr<ci8>(5),
                                   a.ptr<cf>(6), a.ptr<float*>(7));
   K("d4_mv_iq2_xxs") {

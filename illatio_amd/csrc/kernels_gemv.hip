@@ -23,7 +23,7 @@ constexpr int kThreads = 256;
 __device__ const u64 ilt_iq2xxs_grid_dev[256] = { ILT_IQ2XXS_GRID_VALUES };
 
 template <int FMT> struct Fmt;
-template <> struct Fmt<ILT_Q8_0>    { static constexpr int LPB = 2, TERMS = 1, BW = 32,  BB = 32; };
+template <> struct Fmt<ILT_Q8_0>    { static constexpr int LPB = 2, TERMS = 1, BW = 32; };
 template <> struct Fmt<ILT_Q4_K>    { static constexpr int LPB = 8, TERMS = 2, BW = 256; };
 template <> struct Fmt<ILT_Q6_K>    { static constexpr int LPB = 8, TERMS = 1, BW = 256; };
 template <> struct Fmt<ILT_Q2_K>    { static constexpr int LPB = 8, TERMS = 2, BW = 256; };

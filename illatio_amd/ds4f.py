@@ -134,3 +134,43 @@ def group_rows(dev, sel, w, n, ne, nu):
     hip.launch(dev, "d4_group_scatter", (rows + 255) // 256, 256,
                [rows, ne, nu, sel, g["rank"], g["bases"], w, g["rmap"], g["smap"], g["wrow"]])
     return g
+
+
+def ffn_routed_chunk(dev, pool, logits, norm2, sout, n, ne, nu, scale, clamp, bias=None, keep=None):
+    """A chunk of N tokens past the router (DK-FFN-ROUTED-CHUNK): each token's experts and
+    weights (d4_route), the (token, slot) rows grouped by expert, the rows gathered and
+    quantized, every expert's gate, up and down as one grouped product each over its rows
+    (d4_mm_id_*), the gated activation between, then each token's rows summed in slot order
+    with the shared expert's SOUT.  LOGITS (N x NE), NORM2 (N x D) and SOUT (N x D) are
+    DBufs; returns MOE (N x D)."""
+    d, ff = pool.d, pool.ff
+    rows = n * nu
+    gb = pool.gate_bytes
+    sel, w = route(dev, logits, n, ne, nu, scale, bias)
+    g = group_rows(dev, sel, w, n, ne, nu)
+    ptrs = hip.hip_upload_new(dev, np.array([pool.slot_ptr(e) for e in range(ne)], np.uint64))
+    x = hip.hip_alloc(dev, 4 * rows * d)
+    hip.launch(dev, "d4_gather_rows", (rows * d + 255) // 256, 256, [d, rows, norm2, g["rmap"], x])
+    xq, xd, xs = _q8k(dev, x, rows * d)
+    gg, gu, mid = (hip.hip_alloc(dev, 4 * rows * ff) for _ in range(3))
+    down, moe = hip.hip_alloc(dev, 4 * rows * d), hip.hip_alloc(dev, 4 * n * d)
+
+    def mm_id(kernel, ncols, nrows, rb, add, xin, yout):
+        hip.launch(dev, kernel, ((n + 63) // 64, (nrows + 63) // 64, ne), 128,
+                   [ncols, nrows, rb, ncols, nrows, hip.I64(add), ptrs, g["counts"], g["bases"], xin[0], yout,
+                    xin[1], xin[2], hip.I64(rows)])
+
+    mm_id("d4_mm_id_iq2_xxs", d, ff, pool.grb, 0, (xq, xd, None), gg)
+    mm_id("d4_mm_id_iq2_xxs", d, ff, pool.grb, gb, (xq, xd, None), gu)
+    hip.launch(dev, "d4_swiglu_w", (rows * ff + 255) // 256, 256, [rows, ff, float(clamp), gg, gu, g["wrow"], mid, None, None])
+    mq, md, ms = _q8k(dev, mid, rows * ff)
+    mm_id("d4_mm_id_q2_k", ff, d, pool.drb, 2 * gb, (mq, md, ms), down)
+    hip.launch(dev, "d4_moe_sum_rows", (n * d + 255) // 256, 256, [d, nu, n, down, g["smap"], sout, moe])
+    hip.hip_sync(dev)
+    if keep is not None:
+        keep["sel"] = hip.hip_download(sel, np.uint32, rows).reshape(n, nu)
+        keep["w"] = hip.hip_floats(w, rows).reshape(n, nu)
+        keep["counts"] = hip.hip_download(g["counts"], np.uint32, ne)
+    for b in [sel, w, ptrs, x, xq, xd, xs, gg, gu, mid, mq, md, ms, down] + list(g.values()):
+        hip.hip_free(b)
+    return moe

@@ -156,14 +156,39 @@ int ilt_d4_moe_sum(uint64_t stream, int d, int k, const float* down, const float
 int ilt_d4_moe_sum_rows(uint64_t stream, int d, int nu, int ntok, const float* down, const uint32_t* map,
                         const float* shared_, float* moe);
 
+/* Prefill products on the int8 matrix cores, y[t*rows + r] = W[r].x_t (+ bias[r]) for n
+   tokens, each (row, token) with the decode kernel's bits (CPU: MATMUL!, batch.lisp:128-205,
+   "bit-identical to feeding the tokens one at a time", :10-12).
+   mm_q8 (dense.cu:251, 642, 884 mm_q8 / mm_q8_mma / mm_q8_mma2): W repacked by ilt_repack_q8,
+     activations from ilt_quant_q8 (or ilt_d4_quant), token t's at t*cols.
+   mm_k (kquant.cu:223, 458-466 mm_k / mm_q4k_mma / mm_q6k_mma): type 0 Q4_K, 2 Q6_K;
+     activations from ilt_quant_q8k.
+   d4_mm_id_* (ds4f_mm.cu:256-257): the grouped expert product.  Expert z's matrix is at
+     ptrs[z] + add; it multiplies rows bases[z] .. bases[z]+counts[z]-1 of the gathered,
+     Q8_K-quantized activations (xq/xd/bsums, ncols apart) into the same rows of y (nrows
+     apart).  ne experts (at most 256), total_rows = the sum of counts. */
+int ilt_mm_q8(uint64_t stream, const int8_t* wq, const uint16_t* wd, const int8_t* xq, const float* xs, float* y,
+              const float* bias, int rows, int cols, int n, int acc);
+int ilt_mm_k(uint64_t stream, int type, const void* w, const int8_t* xq, const float* xd, const int32_t* bsums, float* y,
+             const float* bias, int rows, int cols, int n, int acc);
+int ilt_d4_mm_id_iq2_xxs(uint64_t stream, int ncols, int nrows, int row_bytes, int64_t add, const uint64_t* ptrs,
+                         const uint32_t* counts, const uint32_t* bases, int ne, int64_t total_rows,
+                         const int8_t* xq, const float* xd, float* y);
+int ilt_d4_mm_id_q2_k(uint64_t stream, int ncols, int nrows, int row_bytes, int64_t add, const uint64_t* ptrs,
+                      const uint32_t* counts, const uint32_t* bases, int ne, int64_t total_rows,
+                      const int8_t* xq, const float* xd, const int32_t* bsums, float* y);
+
 /* ---- 3. launch by name (src/cuda.lisp:323-352) -------------------------------------------
  * params[i] points at argument i's 8-byte slot: a pointer as 64 bits, an int in the low
  * 32 bits, a float in the low 32 bits, a long long as 64 bits.  Kernel names and argument
  * orders are the reference's (its src/cuda/ *.cu); the grid and block passed in are read
  * only where an argument count lives in them (d4_route: tokens = gx; d4_mv_*: experts =
  * gz).  For d4_mv_iq2_xxs / d4_mv_q2_k the slots "src1, counts, bases" carry the Q8_K
- * activations "xq, xd, bsums" and srcs must be null.  Unknown names return
- * hipErrorNotFound. */
+ * activations "xq, xd, bsums" and srcs must be null.  mm_q8, mm_q8_mma, mm_k, mm_q4k_mma and
+ * mm_q6k_mma take the reference's lists.  d4_mm_id_iq2_xxs / d4_mm_id_q2_k take the
+ * reference's eleven slots (ncols, nrows, row_bytes, x_stride, y_stride, add, ptrs, counts,
+ * bases, x, y) with x = xq, followed by three more: xd, bsums, total_rows (long long);
+ * experts = gz.  Unknown names return hipErrorNotFound. */
 int ilt_launch(const char* kernel, unsigned gx, unsigned gy, unsigned gz, unsigned bx, unsigned by, unsigned bz,
                unsigned shared_bytes, uint64_t stream, void** params);
 

@@ -1,0 +1,89 @@
+"""GPU parity of the prefill products (int8 matrix cores) with the CPU oracle, through the
+C ABI.  The reference's CPU MATMUL! gives each (row, token) the decode product's bits
+(batch.lisp:10-12); so do these kernels, so every comparison is bit for bit -- dense
+(Q8_0, Q4_K, Q6_K) and the grouped expert product (IQ2_XXS, Q2_K) of a prefill chunk."""
+import numpy as np
+import pytest
+
+import oracle_lib as orc
+from illatio_amd import synth
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def dev():
+    from illatio_amd import hip
+    return hip.open_hip(0)
+
+
+def bits(a):
+    return np.ascontiguousarray(a, np.float32).view(np.uint32)
+
+
+CASES = [
+    (synth.Q8_0, 4864, 896, 70),        # BASELINE config 1's matrices, a ragged token count
+    (synth.Q8_0, 896, 4864, 5),
+    (synth.Q8_0, 100, 64, 129),         # rows and columns that fill no tile
+    (synth.Q4_K, 1024, 2560, 64),
+    (synth.Q4_K, 200, 512, 3),
+    (synth.Q6_K, 640, 5120, 96),        # BASELINE config 3's format and width, fewer rows
+    (synth.Q6_K, 65, 256, 65),
+]
+
+
+@pytest.mark.parametrize("qtype,rows,cols,n", CASES)
+def test_dense_prefill_equals_cpu_matmul_bit_for_bit(dev, qtype, rows, cols, n):
+    from illatio_amd import dense, hip
+    rng = synth.make_rng(qtype * 31 + rows + n)
+    w = synth.weights(qtype, rows, cols, rng)
+    x = synth.activations((n, cols), rng)
+    x[0, :256] = 0.0
+    bias = synth.activations(rows, rng)
+    m = dense.upload_gmat(dev, "w", qtype, rows, cols, w)
+    act = dense.QAct(dev, n, cols, ("q8",) if qtype == synth.Q8_0 else ("q8k",))
+    xb, bb = hip.hip_upload_new(dev, x), hip.hip_upload_new(dev, bias)
+    y = hip.hip_alloc(dev, 4 * n * rows)
+    dense.quantize_act(dev, xb, act)
+    dense.cmat_mul(dev, m, act, y, n=n)
+    want = orc.matmul(qtype, w, rows, cols, x, nthreads=8)
+    got = hip.hip_floats(y, n * rows).reshape(n, rows)
+    assert np.array_equal(bits(got), bits(want)), (np.abs(got - want).max(), np.argwhere(bits(got) != bits(want))[:5])
+    dense.cmat_mul(dev, m, act, y, n=n, bias=bb, acc=True)
+    assert np.array_equal(bits(hip.hip_floats(y, n * rows).reshape(n, rows)), bits(want + (want + bias[None, :])))
+    # the tiled product and the matrix-vector kernel agree on token 0
+    y1 = hip.hip_alloc(dev, 4 * rows)
+    dense.cmat_mul(dev, m, act, y1, n=1)
+    assert np.array_equal(bits(hip.hip_floats(y1, rows)), bits(want[0]))
+    for b in (xb, bb, y, y1):
+        hip.hip_free(b)
+    act.free(); m.free()
+
+
+@pytest.mark.parametrize("ne,d,ff,nu,n,clamp", [(8, 512, 256, 3, 37, 0.0), (16, 1024, 512, 4, 150, 0.6),
+                                                 (12, 4096, 2048, 6, 96, 0.0)])
+def test_moe_prefill_chunk_bit_exact(dev, ne, d, ff, nu, n, clamp):
+    """BASELINE config 5's sequence (route -> group -> gather -> grouped gate, up -> gated
+    activation -> grouped down -> slot-ordered sum + shared) at reduced expert and token
+    counts, Zipf-skewed routing, against the CPU path's chunk (ds4f.lisp:1169-1239)."""
+    from illatio_amd import ds4f, hip
+    rng = synth.make_rng(ne + d + n)
+    gate = synth.weights(synth.IQ2_XXS, ne * ff, d, rng)
+    up = synth.weights(synth.IQ2_XXS, ne * ff, d, rng)
+    down = synth.weights(synth.Q2_K, ne * d, ff, rng)
+    norms = synth.activations((n, d), rng)
+    logits = synth.zipf_router_logits(n, ne, rng)
+    shared = synth.activations((n, d), rng)
+    want, wsel, ww, wcounts = orc.moe_chunk(gate, up, down, d, ff, ne, nu, 1.5, clamp, logits, norms, shared, nthreads=8)
+    pool = ds4f.ExpertPool(dev, ne, d, ff, gate, up, down)
+    lb, nb, sb = (hip.hip_upload_new(dev, a) for a in (logits, norms, shared))
+    keep = {}
+    moe = ds4f.ffn_routed_chunk(dev, pool, lb, nb, sb, n, ne, nu, 1.5, clamp, keep=keep)
+    assert np.array_equal(keep["sel"], wsel.astype(np.uint32))
+    assert np.array_equal(bits(keep["w"]), bits(ww))
+    assert np.array_equal(keep["counts"], wcounts.astype(np.uint32))
+    got = hip.hip_floats(moe, n * d).reshape(n, d)
+    assert np.array_equal(bits(got), bits(want)), (np.abs(got - want).max(), np.argwhere(bits(got) != bits(want))[:5])
+    for b in (lb, nb, sb, moe):
+        hip.hip_free(b)
+    pool.free()
