@@ -48,6 +48,10 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--layers", type=int, default=LAYERS, help=argparse.SUPPRESS)
+    ap.add_argument("--mode", default="fused", choices=["fused", "fused-q", "single"],
+                    help="fused: Q/K/V in one launch, gate+up in one, activations quantized inside the product "
+                         "kernels; fused-q: the same launches after separate quantizer launches; "
+                         "single: one launch per matrix after separate quantizer launches")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU; --gpus N with N above 1 is not supported "
@@ -80,28 +84,53 @@ def main():
     ev = [hip.hip_event_create(dev, timing=True) for _ in range(2)]
     probes = []          # (kernel label, bytes, start event, stop event) when profiling
 
-    def mv(w, act, y, label, nbytes, probe):
+    wbytes = {name: synth.row_bytes(qt, cols) * rows for name, qt, rows, cols, _ in specs}
+
+    def timed(fn, nbytes, probe):
         if probe:
             e0, e1 = hip.hip_event_create(dev, True), hip.hip_event_create(dev, True)
             hip.hip_event_record(e0, dev.stream)
-        dense.cmat_mul(dev, w, act, y)
+        fn()
         if probe:
             hip.hip_event_record(e1, dev.stream)
-            probes.append((label, nbytes, e0, e1))
+            probes.append(("gemv_kernel", nbytes, e0, e1))
+
+    fused, inq = args.mode != "single", args.mode == "fused"
 
     def step(probe=False):
         for L in layers:
-            dense.quantize_act(dev, xbuf["x"], acts["x"])
-            for name, qt, rows, cols, src in specs:
-                if name == "wo":
-                    dense.quantize_act(dev, xbuf["att"], acts["att"])
-                if name == "gate":
+            if fused:
+                xf = xbuf["x"] if inq else None
+                if not inq:
                     dense.quantize_act(dev, xbuf["x"], acts["x"])
-                if name == "down":
-                    dense.quantize_act(dev, xbuf["mid"], acts["mid"])
-                mv(L[name], acts[src], ybuf[name], synth.TYPE_NAMES[qt], synth.row_bytes(qt, cols) * rows + cols + 4 * rows, probe)
-        dense.quantize_act(dev, xbuf["x"], acts["x"])
-        mv(head, acts["x"], logits, "q6_k", head_host.size + D + 4 * VOCAB, probe)
+                timed(lambda: dense.qkv_mul(dev, L["wq"], L["wk"], L["wv"], acts["x"], ybuf["wq"], ybuf["wk"], ybuf["wv"], xf=xf),
+                      wbytes["wq"] + wbytes["wk"] + wbytes["wv"] + D + 4 * (QD + 2 * KVD), probe)
+                if not inq:
+                    dense.quantize_act(dev, xbuf["att"], acts["att"])
+                timed(lambda: dense.mv_multi(dev, [(L["wo"], ybuf["wo"], None)], acts["att"], xf=xbuf["att"] if inq else None),
+                      wbytes["wo"] + QD + 4 * D, probe)
+                if not inq:
+                    dense.quantize_act(dev, xbuf["x"], acts["x"])
+                timed(lambda: dense.glu_mul(dev, L["gate"], L["up"], acts["x"], ybuf["gate"], xf=xf),
+                      wbytes["gate"] + wbytes["up"] + D + 4 * FFN, probe)
+                # the down projection's input is 9728 wide: quantized once, not by every workgroup
+                dense.quantize_act(dev, xbuf["mid"], acts["mid"])
+                timed(lambda: dense.cmat_mul(dev, L["down"], acts["mid"], ybuf["down"]), wbytes["down"] + FFN + 4 * D, probe)
+            else:
+                dense.quantize_act(dev, xbuf["x"], acts["x"])
+                for name, qt, rows, cols, src in specs:
+                    if name == "wo":
+                        dense.quantize_act(dev, xbuf["att"], acts["att"])
+                    if name == "gate":
+                        dense.quantize_act(dev, xbuf["x"], acts["x"])
+                    if name == "down":
+                        dense.quantize_act(dev, xbuf["mid"], acts["mid"])
+                    timed(lambda: dense.cmat_mul(dev, L[name], acts[src], ybuf[name]), wbytes[name] + cols + 4 * rows, probe)
+        if inq:
+            timed(lambda: dense.mv_multi(dev, [(head, logits, None)], xf=xbuf["x"]), head_host.size + D + 4 * VOCAB, probe)
+        else:
+            dense.quantize_act(dev, xbuf["x"], acts["x"])
+            timed(lambda: dense.cmat_mul(dev, head, acts["x"], logits), head_host.size + D + 4 * VOCAB, probe)
 
     for _ in range(args.warmup):
         step()
@@ -132,7 +161,7 @@ def main():
     achieved = dbytes / (dms * 1e-3) / 1e9
     roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                 "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
-                "kernel": f"gemv_kernel<{dom}>", "launches": dn, "avg_launch_us": round(dms / dn * 1e3, 2),
+                "kernel": "gemv_kernel<0> (dense Q4_K/Q6_K decode product)", "launches": dn, "avg_launch_us": round(dms / dn * 1e3, 2),
                 "avg_bytes_per_launch": dbytes // dn,
                 "other_kernels": {k: {"GB/s": round(v[1] / (v[0] * 1e-3) / 1e9, 1), "launches": v[2]}
                                   for k, v in per.items() if k != dom}}
@@ -148,7 +177,7 @@ def main():
             pass
         xs = {k: synth.activations(n, synth.make_rng(7)) for k, n in xin.items()}
         sample_bytes, t_cpu, reps = 0, 0.0, 0
-        while t_cpu < 10.0 and reps < 64:
+        while t_cpu < 10.0 and reps < 4000:
             for name, qt, rows, cols, src in specs:
                 t1 = time.perf_counter()
                 orc.matmul(qt, host[name], rows, cols, xs[src], nthreads=cores)
@@ -166,7 +195,7 @@ def main():
            "dtype": "int8 block dots, fp32 combine", "data": "synthetic",
            "config": {"workload": f"qwen3-4b-shape decode: the {nl * 7 + 1} quantized matvecs of one token "
                                   f"({nl} layers x 7 + output head), Q4_K/Q6_K, batch 1",
-                      "bytes_per_step": step_bytes, "layers": nl},
+                      "bytes_per_step": step_bytes, "layers": nl, "launch_mode": args.mode},
            "pct_of_hbm_peak": round(100 * gbs / HBM_PEAK_GBS, 2),
            "matvec_only_tok_per_s": round(1e3 / ms_per_step, 1),
            "device_ms_per_step": round(dev_ms / args.steps, 4),

@@ -16,9 +16,10 @@ static inline hipStream_t S(uint64_t s) { return (hipStream_t)(uintptr_t)s; }
 static inline hipEvent_t E(uint64_t e) { return (hipEvent_t)(uintptr_t)e; }
 
 static int block_weights(int fmt) { return fmt == ILT_Q8_0 ? 32 : 256; }
+// bytes of one block as the kernels read it (Q6_K: the padded device block)
 static int block_bytes(int fmt) {
   switch (fmt) { case ILT_Q8_0: return 34; case ILT_Q2_K: return 84; case ILT_Q4_K: return 144;
-                 case ILT_Q6_K: return 210; case ILT_IQ2_XXS: return 66; }
+                 case ILT_Q6_K: return ILT_Q6K_STRIDE; case ILT_IQ2_XXS: return 66; }
   return 0;
 }
 // kquant.cu's numbering of the K-quants (cuda-dense.lisp:18-20) -> GGUF's
@@ -147,7 +148,7 @@ int ilt_repack_q8(uint64_t stream, const void* raw, void* qs, void* d, int64_t n
 
 int ilt_repack_q6k(uint64_t stream, const void* raw, void* out, int64_t nblocks) {
   ILT_REQUIRE(nblocks >= 0 && (nblocks == 0 || (raw && out)));
-  return (int)ilt_k_copy_bytes((const uint8_t*)raw, (uint8_t*)out, nblocks * 210, S(stream));
+  return (int)ilt_k_repack_q6k((const uint8_t*)raw, (uint8_t*)out, nblocks, S(stream));
 }
 
 int ilt_quant_q8(uint64_t stream, const float* x, int8_t* xq, float* xs, int32_t* xsum, int64_t nblocks) {
@@ -165,49 +166,98 @@ int ilt_quant_q8k(uint64_t stream, const float* x, int8_t* xq, float* xd, int32_
   return (int)ilt_k_quant_q8k(x, xq, xd, bsums, nblocks, S(stream));
 }
 
-static int gemv_dense(uint64_t stream, int fmt, const void* w, const uint16_t* wd, const int8_t* xq, const float* xs,
-                      const int32_t* bsums, float* out, const float* bias, int rows, int cols, int acc, int group_rows) {
-  ILT_REQUIRE(fmt && rows >= 0 && cols > 0 && cols % block_weights(fmt) == 0);
-  if (rows == 0) return ILT_OK;
-  ILT_REQUIRE(w && xq && xs && out && (fmt == ILT_Q8_0 ? wd != nullptr : bsums != nullptr));
-  ILT_REQUIRE(((uintptr_t)w & 15) == 0 && ((uintptr_t)xq & 15) == 0);
+// One launch over up to four dense matrices sharing the activations (given quantized, or
+// as floats to be quantized by the kernel).
+static int gemv_multi(uint64_t stream, int nmat, const int* fmts, const void* const* ws, const uint16_t* const* wds,
+                      float* const* ys, const float* const* biases, const int* rows, int cols, const int8_t* xq,
+                      const float* xs, const int32_t* bsums, const float* xf, int f16_scale, int acc, int glu,
+                      int group_rows) {
+  ILT_REQUIRE(nmat >= 1 && nmat <= 4 && cols > 0);
+  const bool q8 = fmts[0] == ILT_Q8_0;
   IltGemvParams p = {};
-  p.w = (const uint8_t*)w; p.wd = wd; p.rows = rows; p.cols = cols;
-  p.row_bytes = fmt == ILT_Q8_0 ? cols : cols / 256 * block_bytes(fmt);
-  p.xq = xq; p.xs = xs; p.bsums = bsums; p.y = out; p.bias = bias; p.acc = acc;
-  p.rw = ilt_gemv_pick_rw(fmt, rows, cols, 1);
-  if (group_rows > 0 && group_rows < rows) {
-    ILT_REQUIRE(rows % group_rows == 0);
-    while (p.rw > 1 && group_rows % p.rw) p.rw >>= 1;
+  int live = 0;
+  for (int i = 0; i < nmat; i++) {
+    const int fmt = fmts[i];
+    ILT_REQUIRE((fmt == ILT_Q8_0 || fmt == ILT_Q4_K || fmt == ILT_Q6_K) && (fmt == ILT_Q8_0) == q8);
+    ILT_REQUIRE(rows[i] >= 0 && cols % block_weights(fmt) == 0);
+    if (rows[i] == 0) { ILT_REQUIRE(!glu); continue; }
+    ILT_REQUIRE(ws[i] && ys[i] && ((uintptr_t)ws[i] & 15) == 0 && (fmt != ILT_Q8_0 || wds[i]));
+    IltGemvMat& m = p.mat[live++];
+    m.w = (const uint8_t*)ws[i]; m.wd = wds[i]; m.y = ys[i]; m.bias = biases ? biases[i] : nullptr;
+    m.rows = rows[i]; m.fmt = fmt;
+    m.row_bytes = fmt == ILT_Q8_0 ? cols : (long long)cols / 256 * block_bytes(fmt);
+  }
+  if (live == 0) return ILT_OK;
+  if (glu) ILT_REQUIRE(live == 2 && p.mat[0].rows == p.mat[1].rows && !acc);
+  if (xf) ILT_REQUIRE(((uintptr_t)xf & 15) == 0);
+  else ILT_REQUIRE(xq && xs && (q8 || bsums) && ((uintptr_t)xq & 15) == 0);
+  p.nmat = live; p.cols = cols; p.xq = xq; p.xs = xs; p.bsums = bsums; p.xf = xf; p.f16_scale = f16_scale;
+  p.acc = acc; p.glu = glu;
+  if (group_rows > 0 && group_rows < p.mat[0].rows) {
+    ILT_REQUIRE(live == 1 && p.mat[0].rows % group_rows == 0);
     p.group_rows = group_rows;
   }
-  return (int)ilt_gemv_launch(fmt, p, 1, S(stream));
+  return (int)ilt_gemv_launch(p, 1, S(stream));
+}
+
+static int gemv_dense(uint64_t stream, int fmt, const void* w, const uint16_t* wd, const int8_t* xq, const float* xs,
+                      const int32_t* bsums, const float* xf, int f16_scale, float* out, const float* bias, int rows,
+                      int cols, int acc, int group_rows) {
+  ILT_REQUIRE(fmt);
+  return gemv_multi(stream, 1, &fmt, &w, &wd, &out, &bias, &rows, cols, xq, xs, bsums, xf, f16_scale, acc, 0, group_rows);
 }
 
 int ilt_mv_q8(uint64_t stream, const int8_t* wq, const uint16_t* wd, const int8_t* xq, const float* xs, float* out,
               const float* bias, int rows, int cols, int acc) {
-  return gemv_dense(stream, ILT_Q8_0, wq, wd, xq, xs, nullptr, out, bias, rows, cols, acc, 0);
+  return gemv_dense(stream, ILT_Q8_0, wq, wd, xq, xs, nullptr, nullptr, 0, out, bias, rows, cols, acc, 0);
 }
 
 int ilt_mv_q8_3(uint64_t stream, const int8_t* q0, const uint16_t* d0, const int8_t* q1, const uint16_t* d1,
                 const int8_t* q2, const uint16_t* d2, const int8_t* xq, const float* xs, float* o0, float* o1, float* o2,
                 const float* b0, const float* b1, const float* b2, int r0, int r1, int r2, int cols) {
-  int e = gemv_dense(stream, ILT_Q8_0, q0, d0, xq, xs, nullptr, o0, b0, r0, cols, 0, 0);
-  if (e) return e;
-  e = gemv_dense(stream, ILT_Q8_0, q1, d1, xq, xs, nullptr, o1, b1, r1, cols, 0, 0);
-  if (e) return e;
-  return gemv_dense(stream, ILT_Q8_0, q2, d2, xq, xs, nullptr, o2, b2, r2, cols, 0, 0);
+  const int fmts[3] = {ILT_Q8_0, ILT_Q8_0, ILT_Q8_0}, rows[3] = {r0, r1, r2};
+  const void* ws[3] = {q0, q1, q2}; const uint16_t* wds[3] = {d0, d1, d2};
+  float* ys[3] = {o0, o1, o2}; const float* bs[3] = {b0, b1, b2};
+  return gemv_multi(stream, 3, fmts, ws, wds, ys, bs, rows, cols, xq, xs, nullptr, nullptr, 0, 0, 0, 0);
+}
+
+int ilt_mv_q8_glu(uint64_t stream, const int8_t* gq, const uint16_t* gd, const int8_t* uq, const uint16_t* ud,
+                  const int8_t* xq, const float* xs, float* out, int rows, int cols) {
+  const int fmts[2] = {ILT_Q8_0, ILT_Q8_0}, r[2] = {rows, rows};
+  const void* ws[2] = {gq, uq}; const uint16_t* wds[2] = {gd, ud};
+  float* ys[2] = {out, out};
+  return gemv_multi(stream, 2, fmts, ws, wds, ys, nullptr, r, cols, xq, xs, nullptr, nullptr, 0, 0, 1, 0);
 }
 
 int ilt_mv_k(uint64_t stream, int type, const void* w, const int8_t* xq, const float* xd, const int32_t* bsums, float* out,
              const float* bias, int rows, int cols, int acc) {
-  return gemv_dense(stream, kquant_type(type), w, nullptr, xq, xd, bsums, out, bias, rows, cols, acc, 0);
+  return gemv_dense(stream, kquant_type(type), w, nullptr, xq, xd, bsums, nullptr, 0, out, bias, rows, cols, acc, 0);
+}
+
+int ilt_mv_k_glu(uint64_t stream, int gtype, const void* gw, int utype, const void* uw, const int8_t* xq, const float* xd,
+                 const int32_t* bsums, float* out, int rows, int cols) {
+  const int fmts[2] = {kquant_type(gtype), kquant_type(utype)}, r[2] = {rows, rows};
+  ILT_REQUIRE(fmts[0] && fmts[1]);
+  const void* ws[2] = {gw, uw}; const uint16_t* wds[2] = {nullptr, nullptr};
+  float* ys[2] = {out, out};
+  return gemv_multi(stream, 2, fmts, ws, wds, ys, nullptr, r, cols, xq, xd, bsums, nullptr, 0, 0, 1, 0);
+}
+
+int ilt_mv_multi(uint64_t stream, int nmat, const ilt_mv_desc* descs, int cols, const int8_t* xq, const float* xs,
+                 const int32_t* bsums, const float* xf, int f16_scale, int acc, int glu) {
+  ILT_REQUIRE(descs && nmat >= 1 && nmat <= 4);
+  int fmts[4], rows[4]; const void* ws[4]; const uint16_t* wds[4]; float* ys[4]; const float* bs[4];
+  for (int i = 0; i < nmat; i++) {
+    fmts[i] = descs[i].gguf_type; rows[i] = descs[i].rows; ws[i] = descs[i].w; wds[i] = descs[i].wd;
+    ys[i] = descs[i].y; bs[i] = descs[i].bias;
+  }
+  return gemv_multi(stream, nmat, fmts, ws, wds, ys, bs, rows, cols, xq, xs, bsums, xf, f16_scale, acc, glu, 0);
 }
 
 int ilt_d4_mvq8(uint64_t stream, int rows, int cols, int group_rows, const int8_t* wq, const uint16_t* wd,
                 const int8_t* xq, const float* xs, float* y) {
   ILT_REQUIRE(group_rows > 0);
-  return gemv_dense(stream, ILT_Q8_0, wq, wd, xq, xs, nullptr, y, nullptr, rows, cols, 0, group_rows);
+  return gemv_dense(stream, ILT_Q8_0, wq, wd, xq, xs, nullptr, nullptr, 0, y, nullptr, rows, cols, 0, group_rows);
 }
 
 static int gemv_experts(uint64_t stream, int fmt, int ncols, int nrows, int row_bytes, int64_t add, int x_stride,
@@ -216,11 +266,12 @@ static int gemv_experts(uint64_t stream, int fmt, int ncols, int nrows, int row_
   ILT_REQUIRE(nrows >= 0 && nz >= 0 && ncols > 0 && ncols % 256 == 0 && row_bytes == ncols / 256 * block_bytes(fmt));
   if (nrows == 0 || nz == 0) return ILT_OK;
   ILT_REQUIRE(ptrs && xq && xd && (bsums || fmt == ILT_IQ2_XXS) && dst && add >= 0 && (add & 1) == 0 && x_stride % 256 == 0 && x_stride >= 0);
+  ILT_REQUIRE(nz <= 65535 && ((uintptr_t)xq & 15) == 0);
   IltGemvParams p = {};
-  p.ptrs = ptrs; p.add = add; p.rows = nrows; p.cols = ncols; p.row_bytes = row_bytes;
-  p.xq = xq; p.xs = xd; p.bsums = bsums; p.x_stride = x_stride; p.y = dst; p.y_stride = y_stride;
-  p.rw = ilt_gemv_pick_rw(fmt, nrows, ncols, nz);
-  return (int)ilt_gemv_launch(fmt, p, nz, S(stream));
+  p.nmat = 1; p.mat[0].rows = nrows; p.mat[0].row_bytes = row_bytes; p.mat[0].fmt = fmt; p.mat[0].y = dst;
+  p.ptrs = ptrs; p.add = add; p.cols = ncols;
+  p.xq = xq; p.xs = xd; p.bsums = bsums; p.x_stride = x_stride; p.y_stride = y_stride;
+  return (int)ilt_gemv_launch(p, nz, S(stream));
 }
 
 int ilt_d4_mv_iq2_xxs(uint64_t stream, int ncols, int nrows, int row_bytes, int64_t add, int x_stride, int y_stride,
@@ -372,6 +423,10 @@ int ilt_launch(const char* kernel, unsigned gx, unsigned gy, unsigned gz, unsign
     return ilt_d4_mm_id_q2_k(stream, a.i32(0), a.i32(1), a.i32(2), a.i64(5), a.ptr<const uint64_t*>(6), a.ptr<cu32>(7),
                              a.ptr<cu32>(8), (int)gz, a.i64(13), a.ptr<ci8>(9), a.ptr<cf>(11), a.ptr<const int32_t*>(12),
                              a.ptr<float*>(10));
+  K("mv_q8_glu") return ilt_mv_q8_glu(stream, a.ptr<ci8>(0), a.ptr<cu16>(1), a.ptr<ci8>(2), a.ptr<cu16>(3), a.ptr<ci8>(4),
+                                      a.ptr<cf>(5), a.ptr<float*>(6), a.i32(7), a.i32(8));
+  K("mv_k_glu") return ilt_mv_k_glu(stream, a.i32(0), a.ptr<const void*>(1), a.i32(2), a.ptr<const void*>(3), a.ptr<ci8>(4),
+                                    a.ptr<cf>(5), a.ptr<const int32_t*>(6), a.ptr<float*>(7), a.i32(8), a.i32(9));
   K("d4_mvq8") return ilt_d4_mvq8(stream, a.i32(0), a.i32(1), a.i32(2), a.ptr<ci8>(3), a.ptr<cu16>(4), a.ptr<ci8>(5),
                                   a.ptr<cf>(6), a.ptr<float*>(7));
   K("d4_mv_iq2_xxs") {

@@ -57,8 +57,29 @@ __device__ __forceinline__ int ilt_dot16(const int4& a, const int4& b, int c) {
   c = ilt_dot4(a.x, b.x, c); c = ilt_dot4(a.y, b.y, c); c = ilt_dot4(a.z, b.z, c); return ilt_dot4(a.w, b.w, c);
 }
 
-// Loads that may be 2-byte aligned (GGUF blocks of 34, 66, 84 and 210 bytes are not
-// 16-byte multiples); gfx950 performs them in hardware.
+// Address spaces spelled out.  A pointer rebuilt from an integer (an expert's slot
+// address), or carried through a struct, is "generic" to the compiler; generic loads are
+// FLAT instructions, which count against the LDS counter as well as the memory counter and
+// so cannot stay in flight across an LDS read.  These helpers load through address space 1
+// (global) and store through address space 3 (LDS) whatever the pointer's history.
+#define ILT_GLOBAL __attribute__((address_space(1)))
+#define ILT_LDS __attribute__((address_space(3)))
+
+typedef int ilt_v4i __attribute__((ext_vector_type(4)));
+typedef int ilt_v2i __attribute__((ext_vector_type(2)));
+typedef float ilt_v2f __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ int4 ilt_lds_ld16(const void* p) {
+  const ilt_v4i v = *(const ILT_LDS ilt_v4i*)p; return make_int4(v.x, v.y, v.z, v.w);
+}
+__device__ __forceinline__ int2 ilt_lds_ld8(const void* p) {
+  const ilt_v2i v = *(const ILT_LDS ilt_v2i*)p; return make_int2(v.x, v.y);
+}
+__device__ __forceinline__ float ilt_lds_ldf(const void* p) { return *(const ILT_LDS float*)p; }
+__device__ __forceinline__ void ilt_lds_stf(void* p, float v) { *(ILT_LDS float*)p = v; }
+__device__ __forceinline__ void ilt_lds_stf2(void* p, float a, float b) { ilt_v2f v = {a, b}; *(ILT_LDS ilt_v2f*)p = v; }
+
+// Global loads that may be only 2-byte aligned (GGUF blocks of 34, 66, 84 and 210 bytes are
+// not 16-byte multiples); gfx950 performs them in hardware.
 __device__ __forceinline__ int4 ilt_ld16(const u8* p) {
   int4 v; __builtin_memcpy(&v, __builtin_assume_aligned(p, 2), 16); return v;
 }
@@ -71,6 +92,23 @@ __device__ __forceinline__ u32 ilt_ld4(const u8* p) {
 __device__ __forceinline__ u16 ilt_ld2(const u8* p) {
   u16 v; __builtin_memcpy(&v, __builtin_assume_aligned(p, 2), 2); return v;
 }
+
+// Buffer loads: a wave-uniform descriptor (base, byte count) plus a per-lane byte offset.
+// They count against the memory counter only, so they stay in flight across LDS traffic,
+// and a read past the byte count returns zeros instead of faulting.
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t ilt_rsrc(const void* base, u32 bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, bytes, 0x00020000);
+}
+__device__ __forceinline__ int4 ilt_bld16(__amdgpu_buffer_rsrc_t r, u32 off) {
+  const ilt_v4i v = __builtin_amdgcn_raw_buffer_load_b128(r, off, 0, 0);
+  return make_int4(v.x, v.y, v.z, v.w);
+}
+__device__ __forceinline__ int2 ilt_bld8(__amdgpu_buffer_rsrc_t r, u32 off) {
+  const ilt_v2i v = __builtin_amdgcn_raw_buffer_load_b64(r, off, 0, 0);
+  return make_int2(v.x, v.y);
+}
+__device__ __forceinline__ u32 ilt_bld4(__amdgpu_buffer_rsrc_t r, u32 off) { return __builtin_amdgcn_raw_buffer_load_b32(r, off, 0, 0); }
+__device__ __forceinline__ u16 ilt_bld2(__amdgpu_buffer_rsrc_t r, u32 off) { return __builtin_amdgcn_raw_buffer_load_b16(r, off, 0, 0); }
 
 // SBCL evaluates single-float exp and log by widening to double, calling libm and
 // rounding back (the CPU path's silu, softplus); the kernels do the same.

@@ -12,30 +12,50 @@
 #define ILT_Q6_K 14
 #define ILT_IQ2_XXS 16
 
-struct IltGemvParams {
+// Q6_K on the device: the 210-byte GGUF block followed by two bytes of padding, so that
+// every block (and every 16-byte piece of it) starts on a 4-byte boundary.
+#define ILT_Q6K_STRIDE 212
+
+struct IltGemvMat {
   const uint8_t* w;          // the matrix (Q8_0: its int8 quants), rows one after another
-  const uint64_t* ptrs;      // or, per grid z, the device address of an expert's slot ...
-  long long add;             // ... plus this byte offset into it
   const uint16_t* wd;        // Q8_0 only: the f16 block scales
-  int rows, cols, row_bytes;
-  const int8_t* xq;          // quantized activations
-  const float* xs;           // their block scales (per 32 for Q8_0, per 256 otherwise)
-  const int* bsums;          // Q8_K: sums of each 16 quants
-  int x_stride;              // activations of grid z start at z * x_stride elements
-  float* y;                  // output; grid z's at z * y_stride
-  int y_stride;
+  float* y;                  // output rows
   const float* bias;         // added after the sum, or null
-  int acc;                   // y += result
-  int rw;                    // rows per workgroup
-  int group_rows;            // >0: row r reads the activations of group r/group_rows (cols apart)
+  long long row_bytes;
+  int rows;
+  int fmt;                   // ILT_Q8_0, ILT_Q4_K, ILT_Q6_K (dense); the expert kernels ignore it
+  int batch0, nbat;          // this matrix's first batch among the launch's, and how many (set at launch)
 };
 
-int ilt_gemv_pick_rw(int fmt, int rows, int cols, int nz);
-hipError_t ilt_gemv_launch(int fmt, const IltGemvParams& p, int nz, hipStream_t st);
+struct IltGemvParams {
+  IltGemvMat mat[4];         // up to four matrices sharing the activations
+  int nmat;
+  const uint64_t* ptrs;      // experts: grid y's matrix is at ptrs[y] + add (mat[0].w unused)
+  long long add;
+  int cols;
+  const int8_t* xq;          // quantized activations ...
+  const float* xs;           //   their block scales (per 32 for Q8_0, per 256 otherwise)
+  const int* bsums;          //   Q8_K: sums of each 16 quants
+  const float* xf;           // ... or the activations as floats, quantized by each workgroup
+  int f16_scale;             // Q8_0 from floats: store the scale through fp16 (*q8-f16-scale*)
+  int x_stride;              // activations of grid y start at y * x_stride elements
+  int y_stride;              // outputs of grid y start at y * y_stride
+  int acc;                   // y += result
+  int glu;                   // mat[0] = gate, mat[1] = up: y = silu(gate.x) * (up.x) into mat[0].y
+  int group_rows;            // >0: row r reads the activations of group r/group_rows (cols apart)
+  int nbatches;              // batches of rows in the launch (per group, per grid y; set at launch)
+  int wgs_per_group;         // grouped rows: workgroups sharing one group (set at launch)
+  int batch;                 // rows a wave takes through phase A at a time (set at launch)
+  uint32_t s_magic;          // ceil(2^32 / blocks per row)
+};
+
+// The kernel is chosen by the matrices' formats (mat[i].fmt): one format, or Q4_K and Q6_K mixed.
+hipError_t ilt_gemv_launch(IltGemvParams& p, int nz, hipStream_t st);
 
 hipError_t ilt_k_quant_q8(const float* x, int8_t* xq, float* xs, int* xsum, long long nblocks, int f16_scale, hipStream_t st);
 hipError_t ilt_k_quant_q8k(const float* x, int8_t* xq, float* xd, int* bsums, long long nblocks, hipStream_t st);
 hipError_t ilt_k_repack_q8(const uint8_t* raw, int8_t* qs, uint16_t* d, long long nblocks, hipStream_t st);
+hipError_t ilt_k_repack_q6k(const uint8_t* raw, uint8_t* out, long long nblocks, hipStream_t st);
 hipError_t ilt_k_copy_bytes(const uint8_t* src, uint8_t* dst, long long bytes, hipStream_t st);
 hipError_t ilt_k_dequant_rows(int fmt, const uint8_t* w, const uint16_t* wd, const int* rows_idx, long long nrows,
                               int cols, long long row_bytes, float* out, hipStream_t st);

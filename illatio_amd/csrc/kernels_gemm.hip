@@ -95,7 +95,7 @@ __device__ __forceinline__ void stage_w(Smem& S, const u8* __restrict__ w, const
   } else if (FMT == ILT_Q6_K) {
     const int row = t >> 2, c = (t >> 1) & 1, pp = t & 1;
     const bool live = r0 + row < rows;
-    const u8* blk = w + (long)(live ? r0 + row : r0) * row_bytes + (long)sb * 210;
+    const u8* blk = w + (long)(live ? r0 + row : r0) * row_bytes + (long)sb * ILT_Q6K_STRIDE;
     const int m = live ? -1 : 0;
 #pragma unroll
     for (int h = 0; h < 2; h++) {

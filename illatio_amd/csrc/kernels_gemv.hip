@@ -1,17 +1,20 @@
 // Decode GEMV kernels for gfx950: y = W.x for W in GGUF Q8_0 / Q4_K / Q6_K / Q2_K /
-// IQ2_XXS blocks, x already quantized as the reference's CPU path quantizes it
-// (Q8_0 blocks for Q8_0 weights, Q8_K blocks for the rest).
+// IQ2_XXS blocks, x quantized as the reference's CPU path quantizes it (Q8_0 blocks for
+// Q8_0 weights, Q8_K blocks for the rest) -- either beforehand or here, by each workgroup
+// as it stages x into LDS.
 //
-// Every kernel has the same two phases.
-//   A. A workgroup owns RW consecutive rows, i.e. one contiguous run of RW*S blocks
-//      (S blocks per row).  Groups of LPB lanes walk that run block by block, so a
-//      wave's loads cover consecutive bytes.  Each group forms the block's exact
-//      integer sums (v_dot4_i32_i8, DPP adds) and one lane turns them into the
-//      block's float terms, exactly as the CPU kernels do
-//      (tensor.lisp:329-336, kquant.lisp:180-236, iquant.lisp:138-215), into LDS.
-//   B. One lane per row adds its row's terms in block order: the CPU's sequential
-//      sum, so the result has the CPU path's bits.
-// The activations live in LDS for the whole workgroup.
+// A workgroup (4 waves) stages the activations once and then takes chunks of rows in turn
+// (a persistent grid); inside a chunk each wave owns RWW consecutive rows, i.e. one
+// contiguous run of RWW*S blocks.  Two phases per wave and chunk:
+//   A. Groups of LPB lanes (4; 2 for Q8_0) walk the run block by block, so a wave's
+//      128-bit loads cover consecutive bytes, two steps in flight.  Each group forms the
+//      block's exact integer sums (v_dot4_i32_i8, DPP adds) and one lane turns them into
+//      the block's float terms exactly as the CPU kernels do (tensor.lisp:329-336,
+//      kquant.lisp:180-236, iquant.lisp:138-215), into the wave's own piece of LDS.
+//   B. One lane per row adds its row's terms in block order: the CPU's sequential sum, so
+//      the result has the CPU path's bits.
+// One launch may cover several matrices that share x (Q, K, V; gate and up), and may end
+// in silu(gate)*up (swiglu!, model.lisp:364-378).
 #include "ilt_device.h"
 #include "ilt_iq2xxs_tables.h"
 #include "ilt_kernels.h"
@@ -19,115 +22,75 @@
 namespace {
 
 constexpr int kThreads = 256;
+constexpr int kWaves = 4;
+constexpr int XP = 256 + 16;   // LDS pitch of one Q8_K activation block: spreads banks
 
 __device__ const u64 ilt_iq2xxs_grid_dev[256] = { ILT_IQ2XXS_GRID_VALUES };
 
 template <int FMT> struct Fmt;
-template <> struct Fmt<ILT_Q8_0>    { static constexpr int LPB = 2, TERMS = 1, BW = 32; };
-template <> struct Fmt<ILT_Q4_K>    { static constexpr int LPB = 8, TERMS = 2, BW = 256; };
-template <> struct Fmt<ILT_Q6_K>    { static constexpr int LPB = 8, TERMS = 1, BW = 256; };
-template <> struct Fmt<ILT_Q2_K>    { static constexpr int LPB = 8, TERMS = 2, BW = 256; };
-template <> struct Fmt<ILT_IQ2_XXS> { static constexpr int LPB = 8, TERMS = 1, BW = 256; };
+// LPB lanes per block; TERMS floats per block
+template <> struct Fmt<ILT_Q8_0>    { static constexpr int LPB = 2, TERMS = 1; };
+template <> struct Fmt<ILT_Q4_K>    { static constexpr int LPB = 4, TERMS = 2; };
+template <> struct Fmt<ILT_Q6_K>    { static constexpr int LPB = 4, TERMS = 1; };
+template <> struct Fmt<ILT_Q2_K>    { static constexpr int LPB = 4, TERMS = 2; };
+template <> struct Fmt<ILT_IQ2_XXS> { static constexpr int LPB = 4, TERMS = 1; };
 
 struct Lds {
-  const i8* xq;        // cols int8
-  const float* xs;     // one scale per block (32 or 256 activations)
-  const int* bsums;    // sums of 16 quants (Q8_K only)
+  const i8* xq;        // Q8_0: cols bytes; Q8_K: XP bytes per block of 256
+  const float* xs;     // one scale per activation block
+  const int* bsums;    // Q8_K: sums of 16 quants
   const u64* grid;     // IQ2_XXS codebook
-  float* terms;
 };
-
-// ggml's get_scale_min_k4 on the 12 scale bytes held in three words.
-__device__ __forceinline__ void scale_min_k4(int g, u32 s0, u32 s1, u32 s2, int& sc, int& m) {
-  const int sh = 8 * (g & 3);
-  const u32 a = (s0 >> sh) & 0xFF, b = (s1 >> sh) & 0xFF, c = (s2 >> sh) & 0xFF;
-  if (g < 4) { sc = a & 63; m = b & 63; }
-  else { sc = (c & 0xF) | ((a >> 6) << 4); m = (c >> 4) | ((b >> 6) << 4); }
-}
 
 __device__ __forceinline__ int4 and4(const int4& v, int m) { return make_int4(v.x & m, v.y & m, v.z & m, v.w & m); }
 __device__ __forceinline__ int4 shr4(const int4& v, int n) {
   return make_int4((u32)v.x >> n, (u32)v.y >> n, (u32)v.z >> n, (u32)v.w >> n);
 }
-
-// ---- phase A, one block per group of LPB lanes ---------------------------------------------
-template <int FMT> __device__ __forceinline__ void block_terms(const u8* w, const u16* wd, long f, int s, int j, const Lds& L);
-
-template <> __device__ __forceinline__ void block_terms<ILT_Q8_0>(const u8* w, const u16* wd, long f, int s, int j, const Lds& L) {
-  const int4 q = *(const int4*)(w + f * 32 + 16 * j);
-  const int4 x = *(const int4*)(L.xq + s * 32 + 16 * j);
-  const int acc = ilt_sum2(ilt_dot16(q, x, 0));
-  if (j == 0) L.terms[f] = (float)acc * (ilt_h2f(wd[f]) * L.xs[s]);
+__device__ __forceinline__ int4 or_shl4(const int4& a, const int4& b, int m, int n) {   // a | ((b & m) << n)
+  return make_int4(a.x | ((b.x & m) << n), a.y | ((b.y & m) << n), a.z | ((b.z & m) << n), a.w | ((b.w & m) << n));
 }
+__device__ __forceinline__ int sel4(const int4& v, int i) { return i == 0 ? v.x : i == 1 ? v.y : i == 2 ? v.z : v.w; }
 
-template <> __device__ __forceinline__ void block_terms<ILT_Q4_K>(const u8* w, const u16*, long f, int s, int j, const Lds& L) {
-  const u8* blk = w + f * 144;
-  const int4 hdr = *(const int4*)blk;
-  const int4 q = *(const int4*)(blk + 16 + 16 * j);
-  const int k = j >> 1;
-  const i8* xb = L.xq + s * 256 + 64 * k + 16 * (j & 1);
-  const int lo = ilt_dot16(and4(q, 0x0F0F0F0F), *(const int4*)xb, 0);
-  const int hi = ilt_dot16(and4(shr4(q, 4), 0x0F0F0F0F), *(const int4*)(xb + 32), 0);
-  int sc0, sc1, m0, m1, mj, scj;
-  scale_min_k4(2 * k, hdr.y, hdr.z, hdr.w, sc0, m0);
-  scale_min_k4(2 * k + 1, hdr.y, hdr.z, hdr.w, sc1, m1);
-  scale_min_k4(j, hdr.y, hdr.z, hdr.w, scj, mj);
-  const int2 bs = *(const int2*)(L.bsums + s * 16 + 2 * j);
-  const int isum = ilt_sum8(lo * sc0 + hi * sc1);
-  const int imin = ilt_sum8(mj * (bs.x + bs.y));
-  if (j == 0) {
-    const float ydi = L.xs[s];
-    const float d = ydi * ilt_h2f((u16)(hdr.x & 0xFFFF)), dmin = ydi * ilt_h2f((u16)((u32)hdr.x >> 16));
-    L.terms[2 * f] = dmin * (float)imin;
-    L.terms[2 * f + 1] = d * (float)isum;
-  }
+// ---- the raw bytes a lane needs for one block (issued early, consumed a step later) ------------
+template <int FMT> struct Raw;
+template <> struct Raw<ILT_Q8_0> { int4 q; u16 d; };
+template <> struct Raw<ILT_Q4_K> { int4 hdr, qa, qb; };
+template <> struct Raw<ILT_Q6_K> { int4 ql0, ql1, qh0, qh1, sc; u16 d; };
+template <> struct Raw<ILT_Q2_K> { int4 q, sb; u32 dd; };
+template <> struct Raw<ILT_IQ2_XXS> { int4 q; u16 d; };
+
+// rw: the wave's rows (for Q8_0 their int8 quants); rd: Q8_0's scales.  f: block within them.
+template <int FMT> __device__ __forceinline__ void load_raw(Raw<FMT>& r, __amdgpu_buffer_rsrc_t rw, __amdgpu_buffer_rsrc_t rd, u32 f, int j);
+template <> __device__ __forceinline__ void load_raw<ILT_Q8_0>(Raw<ILT_Q8_0>& r, __amdgpu_buffer_rsrc_t rw, __amdgpu_buffer_rsrc_t rd, u32 f, int j) {
+  r.q = ilt_bld16(rw, f * 32 + 16 * j);
+  r.d = ilt_bld2(rd, f * 2);
 }
-
-template <> __device__ __forceinline__ void block_terms<ILT_Q6_K>(const u8* w, const u16*, long f, int s, int j, const Lds& L) {
-  const u8* blk = w + f * 210;
-  const int c = j >> 2, isb = (j >> 1) & 1, l16 = j & 1;
-  const int4 ql = ilt_ld16(blk + 64 * c + 32 * isb + 16 * l16);
-  const int4 qh = ilt_ld16(blk + 128 + 32 * c + 16 * l16);
-  const i8* sc = (const i8*)(blk + 192);
-  const int sclo = sc[8 * c + 2 * isb + l16], schi = sc[8 * c + 4 + 2 * isb + l16];
-  const int scA = sc[2 * j], scB = sc[2 * j + 1];
-  const int4 hl = shr4(qh, 2 * isb), hh = shr4(qh, 4 + 2 * isb);
-  int4 lo = and4(ql, 0x0F0F0F0F), hi = and4(shr4(ql, 4), 0x0F0F0F0F);
-  lo.x |= (hl.x & 0x03030303) << 4; lo.y |= (hl.y & 0x03030303) << 4; lo.z |= (hl.z & 0x03030303) << 4; lo.w |= (hl.w & 0x03030303) << 4;
-  hi.x |= (hh.x & 0x03030303) << 4; hi.y |= (hh.y & 0x03030303) << 4; hi.z |= (hh.z & 0x03030303) << 4; hi.w |= (hh.w & 0x03030303) << 4;
-  const i8* xb = L.xq + s * 256 + 128 * c + 32 * isb + 16 * l16;
-  const int dlo = ilt_dot16(lo, *(const int4*)xb, 0), dhi = ilt_dot16(hi, *(const int4*)(xb + 64), 0);
-  const int2 bs = *(const int2*)(L.bsums + s * 16 + 2 * j);
-  const int isum = ilt_sum8(dlo * sclo + dhi * schi);
-  const int imins = ilt_sum8(bs.x * scA + bs.y * scB);
-  if (j == 0) L.terms[f] = (ilt_h2f(ilt_ld2(blk + 208)) * L.xs[s]) * (float)(isum - 32 * imins);
+template <> __device__ __forceinline__ void load_raw<ILT_Q4_K>(Raw<ILT_Q4_K>& r, __amdgpu_buffer_rsrc_t rw, __amdgpu_buffer_rsrc_t, u32 f, int j) {
+  const u32 b = f * 144;
+  r.hdr = ilt_bld16(rw, b);
+  r.qa = ilt_bld16(rw, b + 16 + 32 * j);
+  r.qb = ilt_bld16(rw, b + 32 + 32 * j);
 }
-
-template <> __device__ __forceinline__ void block_terms<ILT_Q2_K>(const u8* w, const u16*, long f, int s, int j, const Lds& L) {
-  const u8* blk = w + f * 84;
-  const int h = j >> 2, half = (j >> 1) & 1, lh = j & 1;
-  const int2 q = ilt_ld8(blk + 16 + 32 * h + 16 * half + 8 * lh);
-  const int2 sb = ilt_ld8(blk + 8 * h);
-  const i8* xb = L.xq + s * 256 + 128 * h + 16 * half + 8 * lh;
-  int isum = 0;
-#pragma unroll
-  for (int k = 0; k < 4; k++) {
-    const int2 x = *(const int2*)(xb + 32 * k);
-    const int dot = ilt_dot4(((u32)q.y >> (2 * k)) & 0x03030303, x.y, ilt_dot4(((u32)q.x >> (2 * k)) & 0x03030303, x.x, 0));
-    const u32 sw = ((u32)(k < 2 ? sb.x : sb.y) >> (16 * (k & 1) + 8 * half)) & 0xF;
-    isum += (int)sw * dot;
-  }
-  const u32 mb = ilt_ld2(blk + 2 * j);
-  const int2 bs = *(const int2*)(L.bsums + s * 16 + 2 * j);
-  const int mins = ilt_sum8((int)((mb >> 4) & 0xF) * bs.x + (int)(mb >> 12) * bs.y);
-  isum = ilt_sum8(isum);
-  if (j == 0) {
-    const float ydb = L.xs[s];
-    const u32 dd = ilt_ld4(blk + 80);
-    const float d = ydb * ilt_h2f((u16)(dd & 0xFFFF)), dmin = (-ydb) * ilt_h2f((u16)(dd >> 16));
-    L.terms[2 * f] = dmin * (float)mins;
-    L.terms[2 * f + 1] = d * (float)isum;
-  }
+template <> __device__ __forceinline__ void load_raw<ILT_Q6_K>(Raw<ILT_Q6_K>& r, __amdgpu_buffer_rsrc_t rw, __amdgpu_buffer_rsrc_t, u32 f, int j) {
+  const u32 b = f * ILT_Q6K_STRIDE;
+  const int c = j >> 1, pp = j & 1;
+  r.ql0 = ilt_bld16(rw, b + 64 * c + 32 * pp);
+  r.ql1 = ilt_bld16(rw, b + 64 * c + 32 * pp + 16);
+  r.qh0 = ilt_bld16(rw, b + 128 + 32 * c);
+  r.qh1 = ilt_bld16(rw, b + 128 + 32 * c + 16);
+  r.sc = ilt_bld16(rw, b + 192);
+  r.d = ilt_bld2(rw, b + 208);
+}
+template <> __device__ __forceinline__ void load_raw<ILT_Q2_K>(Raw<ILT_Q2_K>& r, __amdgpu_buffer_rsrc_t rw, __amdgpu_buffer_rsrc_t, u32 f, int j) {
+  const u32 b = f * 84;
+  r.q = ilt_bld16(rw, b + 16 + 16 * j);       // h = j>>1, half = j&1: qs[32h + 16half ..]
+  r.sb = ilt_bld16(rw, b);
+  r.dd = ilt_bld4(rw, b + 80);
+}
+template <> __device__ __forceinline__ void load_raw<ILT_IQ2_XXS>(Raw<ILT_IQ2_XXS>& r, __amdgpu_buffer_rsrc_t rw, __amdgpu_buffer_rsrc_t, u32 f, int j) {
+  const u32 b = f * 66;
+  r.q = ilt_bld16(rw, b + 2 + 16 * j);        // sub-blocks 2j and 2j+1: (grid idx, aux) twice
+  r.d = ilt_bld2(rw, b);
 }
 
 // One IQ2_XXS sub-block (32 weights): its integer dot with 32 activations.  The sign of
@@ -137,125 +100,486 @@ __device__ __forceinline__ int iq2xxs_sub_dot(u32 g, u32 aux, const i8* xb, cons
   int pos = 0, neg = 0;
 #pragma unroll
   for (int l = 0; l < 4; l++) {
-    const uint2 mag = *(const uint2*)(grid + ((g >> (8 * l)) & 0xFF));
+    const int2 mag = ilt_lds_ld8(grid + ((g >> (8 * l)) & 0xFF));
     u32 s = (aux >> (7 * l)) & 127;
     s |= (__popc(s) & 1) << 7;
     const u32 mlo = (((s & 0xF) * 0x00204081u) & 0x01010101u) * 0xFFu;
     const u32 mhi = (((s >> 4) * 0x00204081u) & 0x01010101u) * 0xFFu;
-    const int2 x = *(const int2*)(xb + 8 * l);
+    const int2 x = ilt_lds_ld8(xb + 8 * l);
     pos = ilt_dot4((int)mag.y, x.y, ilt_dot4((int)mag.x, x.x, pos));
-    neg = ilt_dot4((int)(mag.y & mhi), x.y, ilt_dot4((int)(mag.x & mlo), x.x, neg));
+    neg = ilt_dot4((int)((u32)mag.y & mhi), x.y, ilt_dot4((int)((u32)mag.x & mlo), x.x, neg));
   }
   return pos - 2 * neg;
 }
 
-template <> __device__ __forceinline__ void block_terms<ILT_IQ2_XXS>(const u8* w, const u16*, long f, int s, int j, const Lds& L) {
-  const u8* blk = w + f * 66;
-  const int2 sb = ilt_ld8(blk + 2 + 8 * j);
-  const u32 aux = (u32)sb.y;
-  const int isum = iq2xxs_sub_dot((u32)sb.x, aux, L.xq + s * 256 + 32 * j, L.grid);
-  const float term = (float)isum * (0.5f + (float)(aux >> 28));
-  // lane 0 gathers the even sub-blocks' terms in order, lane 1 the odd ones'
-  float a = 0.0f + term;
-  a = a + ilt_dppf<ILT_DPP_SHL(2)>(term);
-  a = a + ilt_dppf<ILT_DPP_SHL(4)>(term);
-  a = a + ilt_dppf<ILT_DPP_SHL(6)>(term);
-  const float b = ilt_dppf<ILT_DPP_SHL(1)>(a);
-  if (j == 0) L.terms[f] = (ilt_h2f(ilt_ld2(blk)) * L.xs[s]) * (a + b);
+// ---- phase A for one block: the group's lanes reduce, lane j == 0 writes the terms --------------
+template <int FMT> __device__ __forceinline__ void block_terms(const Raw<FMT>& r, int s, int j, const Lds& L, float* t);
+
+template <> __device__ __forceinline__ void block_terms<ILT_Q8_0>(const Raw<ILT_Q8_0>& r, int s, int j, const Lds& L, float* t) {
+  const int4 x = ilt_lds_ld16(L.xq + s * 32 + 16 * j);
+  const int acc = ilt_sum2(ilt_dot16(r.q, x, 0));
+  if (j == 0) ilt_lds_stf(t, (float)acc * (ilt_h2f(r.d) * ilt_lds_ldf(L.xs + s)));
+}
+
+template <> __device__ __forceinline__ void block_terms<ILT_Q4_K>(const Raw<ILT_Q4_K>& r, int s, int j, const Lds& L, float* t) {
+  const i8* xb = L.xq + s * XP + 64 * j;
+  int lo = ilt_dot16(and4(r.qa, 0x0F0F0F0F), ilt_lds_ld16(xb), 0);
+  lo = ilt_dot16(and4(r.qb, 0x0F0F0F0F), ilt_lds_ld16(xb + 16), lo);
+  int hi = ilt_dot16(and4(shr4(r.qa, 4), 0x0F0F0F0F), ilt_lds_ld16(xb + 32), 0);
+  hi = ilt_dot16(and4(shr4(r.qb, 4), 0x0F0F0F0F), ilt_lds_ld16(xb + 48), hi);
+  // get_scale_min_k4 for groups 2j and 2j+1 at once, on 16-bit fields of the 12 scale bytes
+  const int sh = 16 * (j & 1);
+  const u32 a = ((u32)r.hdr.y >> sh) & 0xFFFF, b = ((u32)r.hdr.z >> sh) & 0xFFFF, c = ((u32)r.hdr.w >> sh) & 0xFFFF;
+  int sc0, sc1, m0, m1;
+  if (j < 2) { sc0 = a & 63; sc1 = (a >> 8) & 63; m0 = b & 63; m1 = (b >> 8) & 63; }
+  else {
+    sc0 = (c & 0xF) | (((a >> 6) & 3) << 4); sc1 = ((c >> 8) & 0xF) | (((a >> 14) & 3) << 4);
+    m0 = ((c >> 4) & 0xF) | (((b >> 6) & 3) << 4); m1 = ((c >> 12) & 0xF) | (((b >> 14) & 3) << 4);
+  }
+  const int4 bs = ilt_lds_ld16(L.bsums + s * 16 + 4 * j);
+  const int isum = ilt_sum4(lo * sc0 + hi * sc1);
+  const int imin = ilt_sum4(m0 * (bs.x + bs.y) + m1 * (bs.z + bs.w));
+  if (j == 0) {
+    const float ydi = ilt_lds_ldf(L.xs + s);
+    const float d = ydi * ilt_h2f((u16)(r.hdr.x & 0xFFFF)), dmin = ydi * ilt_h2f((u16)((u32)r.hdr.x >> 16));
+    ilt_lds_stf2(t, dmin * (float)imin, d * (float)isum);
+  }
+}
+
+template <> __device__ __forceinline__ void block_terms<ILT_Q6_K>(const Raw<ILT_Q6_K>& r, int s, int j, const Lds& L, float* t) {
+  const int c = j >> 1, pp = j & 1;
+  const i8* xb = L.xq + s * XP + 128 * c + 32 * pp;
+  const int s0 = 2 * pp, s1 = 2 * pp + 4;
+  // low nibbles: weights 128c + 32pp + l; high nibbles: the same + 64 (l = 0..31)
+  const int4 lo0 = or_shl4(and4(r.ql0, 0x0F0F0F0F), shr4(r.qh0, s0), 0x03030303, 4);
+  const int4 lo1 = or_shl4(and4(r.ql1, 0x0F0F0F0F), shr4(r.qh1, s0), 0x03030303, 4);
+  const int4 hi0 = or_shl4(and4(shr4(r.ql0, 4), 0x0F0F0F0F), shr4(r.qh0, s1), 0x03030303, 4);
+  const int4 hi1 = or_shl4(and4(shr4(r.ql1, 4), 0x0F0F0F0F), shr4(r.qh1, s1), 0x03030303, 4);
+  const int dl0 = ilt_dot16(lo0, ilt_lds_ld16(xb), 0), dl1 = ilt_dot16(lo1, ilt_lds_ld16(xb + 16), 0);
+  const int dh0 = ilt_dot16(hi0, ilt_lds_ld16(xb + 64), 0), dh1 = ilt_dot16(hi1, ilt_lds_ld16(xb + 80), 0);
+  // int8 scales: groups 8c+2pp+{0,1} for the low nibbles, 8c+4+2pp+{0,1} for the high
+  const u32 wl = (u32)(c ? r.sc.z : r.sc.x) >> (16 * pp), wh = (u32)(c ? r.sc.w : r.sc.y) >> (16 * pp);
+  int isum = dl0 * (int)(i8)(wl & 0xFF) + dl1 * (int)(i8)((wl >> 8) & 0xFF);
+  isum += dh0 * (int)(i8)(wh & 0xFF) + dh1 * (int)(i8)((wh >> 8) & 0xFF);
+  const u32 wj = (u32)sel4(r.sc, j);
+  const int4 bs = ilt_lds_ld16(L.bsums + s * 16 + 4 * j);
+  int imins = bs.x * (int)(i8)(wj & 0xFF) + bs.y * (int)(i8)((wj >> 8) & 0xFF);
+  imins += bs.z * (int)(i8)((wj >> 16) & 0xFF) + bs.w * (int)(i8)(wj >> 24);
+  isum = ilt_sum4(isum);
+  imins = ilt_sum4(imins);
+  if (j == 0) ilt_lds_stf(t, (ilt_h2f(r.d) * ilt_lds_ldf(L.xs + s)) * (float)(isum - 32 * imins));
+}
+
+template <> __device__ __forceinline__ void block_terms<ILT_Q2_K>(const Raw<ILT_Q2_K>& r, int s, int j, const Lds& L, float* t) {
+  const int h = j >> 1, half = j & 1;
+  const i8* xb = L.xq + s * XP + 128 * h + 16 * half;
+  const u32 wa = (u32)(h ? r.sb.z : r.sb.x) >> (8 * half), wb = (u32)(h ? r.sb.w : r.sb.y) >> (8 * half);
+  int isum = 0;
+#pragma unroll
+  for (int k = 0; k < 4; k++) {
+    const int dot = ilt_dot16(and4(shr4(r.q, 2 * k), 0x03030303), ilt_lds_ld16(xb + 32 * k), 0);
+    const u32 sw = ((k < 2 ? wa : wb) >> (16 * (k & 1))) & 0xF;
+    isum += (int)sw * dot;
+  }
+  const u32 wj = (u32)sel4(r.sb, j);
+  const int4 bs = ilt_lds_ld16(L.bsums + s * 16 + 4 * j);
+  int mins = (int)((wj >> 4) & 0xF) * bs.x + (int)((wj >> 12) & 0xF) * bs.y;
+  mins += (int)((wj >> 20) & 0xF) * bs.z + (int)(wj >> 28) * bs.w;
+  isum = ilt_sum4(isum);
+  mins = ilt_sum4(mins);
+  if (j == 0) {
+    const float ydb = ilt_lds_ldf(L.xs + s);
+    const float d = ydb * ilt_h2f((u16)(r.dd & 0xFFFF)), dmin = (-ydb) * ilt_h2f((u16)(r.dd >> 16));
+    ilt_lds_stf2(t, dmin * (float)mins, d * (float)isum);
+  }
+}
+
+template <> __device__ __forceinline__ void block_terms<ILT_IQ2_XXS>(const Raw<ILT_IQ2_XXS>& r, int s, int j, const Lds& L, float* t) {
+  const i8* xb = L.xq + s * XP + 64 * j;
+  const u32 aux0 = (u32)r.q.y, aux1 = (u32)r.q.w;
+  const float te = (float)iq2xxs_sub_dot((u32)r.q.x, aux0, xb, L.grid) * (0.5f + (float)(aux0 >> 28));
+  const float to = (float)iq2xxs_sub_dot((u32)r.q.z, aux1, xb + 32, L.grid) * (0.5f + (float)(aux1 >> 28));
+  // lane 0 adds the even sub-blocks' terms in order, then the odd ones' (ds4's order)
+  float a = 0.0f + te, b = 0.0f + to;
+  a = a + ilt_dppf<ILT_DPP_SHL(1)>(te); b = b + ilt_dppf<ILT_DPP_SHL(1)>(to);
+  a = a + ilt_dppf<ILT_DPP_SHL(2)>(te); b = b + ilt_dppf<ILT_DPP_SHL(2)>(to);
+  a = a + ilt_dppf<ILT_DPP_SHL(3)>(te); b = b + ilt_dppf<ILT_DPP_SHL(3)>(to);
+  if (j == 0) ilt_lds_stf(t, (ilt_h2f(r.d) * ilt_lds_ldf(L.xs + s)) * (a + b));
 }
 
 // ---- phase B: a row's terms in block order -------------------------------------------------
+// The adds are a chain; the LDS reads are not, so they go eight blocks ahead of it.
 template <int FMT> __device__ __forceinline__ float row_sum(const float* t, int S) {
+  constexpr int TERMS = Fmt<FMT>::TERMS;
   float sum = 0.0f;
-  if (FMT == ILT_Q4_K) { for (int s = 0; s < S; s++) { sum = sum - t[2 * s]; sum = sum + t[2 * s + 1]; } }
-  else if (FMT == ILT_Q2_K) { for (int s = 0; s < S; s++) { sum = sum + t[2 * s]; sum = sum + t[2 * s + 1]; } }
-  else { for (int s = 0; s < S; s++) sum = sum + t[s]; }
+  int s = 0;
+  for (; s + 8 <= S; s += 8) {
+    float v[8 * TERMS];
+#pragma unroll
+    for (int k = 0; k < 8 * TERMS; k++) v[k] = ilt_lds_ldf(t + s * TERMS + k);
+#pragma unroll
+    for (int k = 0; k < 8; k++) {
+      if (FMT == ILT_Q4_K) { sum = sum - v[2 * k]; sum = sum + v[2 * k + 1]; }
+      else if (FMT == ILT_Q2_K) { sum = sum + v[2 * k]; sum = sum + v[2 * k + 1]; }
+      else sum = sum + v[k];
+    }
+  }
+  for (; s < S; s++) {
+    if (FMT == ILT_Q4_K) { sum = sum - ilt_lds_ldf(t + 2 * s); sum = sum + ilt_lds_ldf(t + 2 * s + 1); }
+    else if (FMT == ILT_Q2_K) { sum = sum + ilt_lds_ldf(t + 2 * s); sum = sum + ilt_lds_ldf(t + 2 * s + 1); }
+    else sum = sum + ilt_lds_ldf(t + s);
+  }
   if (FMT == ILT_IQ2_XXS) sum = 0.25f * sum;
   return sum;
 }
 
+__device__ __forceinline__ const void* uniform_ptr(const void* p) {   // the same in every lane: say so
+  const u64 a = (u64)p;
+  const u32 lo = __builtin_amdgcn_readfirstlane((u32)a), hi = __builtin_amdgcn_readfirstlane((u32)(a >> 32));
+  return (const void*)(((u64)hi << 32) | lo);
+}
+
+// A wave's rows [row0, row0+nrows) of one matrix: terms into t (nrows*S*TERMS floats, the wave's own).
+// No branch inside the run of full steps: the next step's loads (index clamped into the
+// run, so always in bounds) are issued before the current step is computed, two register
+// sets taking turns; the ragged last step's lanes find their block already loaded.
+// The first step's loads of a run, on their own: a wave issues them for its first batch
+// before the activations are staged, so the two latencies overlap.
 template <int FMT>
-__global__ __launch_bounds__(kThreads) void gemv_kernel(IltGemvParams p) {
+__device__ __forceinline__ void first_load(Raw<FMT>& r, const u8* w, const u16* wd, long row0, int nrows, int S,
+                                           long row_bytes, int lane) {
   using F = Fmt<FMT>;
-  extern __shared__ __align__(16) unsigned char smem[];
-  const int S = p.cols / F::BW;
-  const int z = blockIdx.z;
-  // LDS: xq | bsums | xs | (grid) | terms
-  i8* lxq = (i8*)smem;
-  int* lbs = (int*)(smem + p.cols);
-  const int nbs = (FMT == ILT_Q8_0 || FMT == ILT_IQ2_XXS) ? 0 : p.cols / 16;
-  float* lxs = (float*)(lbs + nbs);
-  u64* lgrid = (u64*)(((uintptr_t)(lxs + S) + 7) & ~(uintptr_t)7);
-  float* terms = (float*)(lgrid + (FMT == ILT_IQ2_XXS ? 256 : 0));
-
-  const long xoff = (long)z * p.x_stride + (p.group_rows > 0 ? (long)(blockIdx.x * p.rw / p.group_rows) * p.cols : 0);
-  const i8* gxq = p.xq + xoff;
-  for (int i = threadIdx.x * 16; i < p.cols; i += kThreads * 16) *(int4*)(lxq + i) = *(const int4*)(gxq + i);
-  for (int i = threadIdx.x; i < S; i += kThreads) lxs[i] = p.xs[xoff / F::BW + i];
-  for (int i = threadIdx.x; i < nbs; i += kThreads) lbs[i] = p.bsums[xoff / 16 + i];
-  if (FMT == ILT_IQ2_XXS) lgrid[threadIdx.x] = ilt_iq2xxs_grid_dev[threadIdx.x];
-  __syncthreads();
-
-  const int r0 = blockIdx.x * p.rw;
-  const int nrows = min(p.rw, p.rows - r0);
-  const u8* wbase = p.ptrs ? (const u8*)(p.ptrs[z] + p.add) : p.w;
-  const u8* w = wbase + (long)r0 * p.row_bytes;
-  const u16* wd = p.wd ? p.wd + (long)r0 * S : nullptr;
-  const Lds L = { lxq, lxs, lbs, lgrid, terms };
-
-  const int j = threadIdx.x % F::LPB;
+  const int j = lane % F::LPB, gl = lane / F::LPB;
   const int nblk = nrows * S;
-  // whole groups stay together: every lane of a group sees the same f
-  for (int f = threadIdx.x / F::LPB; f < nblk; f += kThreads / F::LPB)
-    block_terms<FMT>(w, wd, f, f % S, j, L);
-  __syncthreads();
+  const __amdgpu_buffer_rsrc_t wr = ilt_rsrc(uniform_ptr(w + row0 * row_bytes), __builtin_amdgcn_readfirstlane((u32)(nrows * row_bytes)));
+  const __amdgpu_buffer_rsrc_t wdr = ilt_rsrc(uniform_ptr(wd ? wd + row0 * S : nullptr), wd ? __builtin_amdgcn_readfirstlane((u32)nblk * 2) : 0);
+  load_raw<FMT>(r, wr, wdr, min(gl, nblk - 1), j);
+}
 
-  for (int r = threadIdx.x; r < nrows; r += kThreads) {
-    float v = row_sum<FMT>(terms + (long)r * S * F::TERMS, S);
-    const long o = (long)z * p.y_stride + r0 + r;
-    if (p.bias) v = v + p.bias[r0 + r];
-    if (p.acc) v = p.y[o] + v;
-    p.y[o] = v;
+template <int FMT>
+__device__ __forceinline__ void wave_rows(const u8* w, const u16* wd, long row0, int nrows, int S, u32 s_magic,
+                                          long row_bytes, const Lds& L, float* t, int lane, const Raw<FMT>* pre) {
+  using F = Fmt<FMT>;
+  constexpr int GPW = ILT_WAVE / F::LPB;           // blocks per wave step
+  const int j = lane % F::LPB, gl = lane / F::LPB;
+  const int nblk = nrows * S, last = nblk - 1;
+  const __amdgpu_buffer_rsrc_t wr = ilt_rsrc(uniform_ptr(w + row0 * row_bytes), __builtin_amdgcn_readfirstlane((u32)(nrows * row_bytes)));
+  const __amdgpu_buffer_rsrc_t wdr = ilt_rsrc(uniform_ptr(wd ? wd + row0 * S : nullptr), wd ? __builtin_amdgcn_readfirstlane((u32)nblk * 2) : 0);
+  const int nfull = nblk / GPW;
+#define ILT_COMPUTE(reg, ff)                                                           \
+  {                                                                                    \
+    const int f_ = (ff);                                                               \
+    const int s_ = S > 1 ? f_ - (int)__umulhi((u32)f_, s_magic) * S : 0;               \
+    block_terms<FMT>(reg, s_, j, L, t + (long)f_ * F::TERMS);                          \
+  }
+  int f = gl;
+  Raw<FMT> ra, rb;
+  if (pre) ra = *pre; else load_raw<FMT>(ra, wr, wdr, min(f, last), j);
+  int k = 0;
+  for (; k + 2 <= nfull; k += 2) {
+    load_raw<FMT>(rb, wr, wdr, min(f + GPW, last), j);
+    ILT_COMPUTE(ra, f)
+    load_raw<FMT>(ra, wr, wdr, min(f + 2 * GPW, last), j);
+    ILT_COMPUTE(rb, f + GPW)
+    f += 2 * GPW;
+  }
+  if (k < nfull) {
+    load_raw<FMT>(rb, wr, wdr, min(f + GPW, last), j);
+    ILT_COMPUTE(ra, f)
+    f += GPW;
+    if (f < nblk) ILT_COMPUTE(rb, f)
+  } else if (f < nblk) {
+    ILT_COMPUTE(ra, f)
+  }
+#undef ILT_COMPUTE
+}
+
+// silu(g)*u as swiglu! computes it (model.lisp:374): x / (1 + exp(-x)), exp through double
+__device__ __forceinline__ float dense_glu(float g, float u) { return (g / (1.0f + ilt_expf_via_double(-g))) * u; }
+
+// ---- activation staging: copy quantized x, or quantize fp32 x here --------------------------------
+__device__ __forceinline__ float wave_max(float v) {     // the same value in every lane
+  v = ilt_max16(v);
+  const float a = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 0));
+  const float b = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 16));
+  const float c = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 32));
+  const float d = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 48));
+  return fmaxf(fmaxf(a, b), fmaxf(c, d));
+}
+
+// Q8_K (quantize-q8k!, kquant.lisp:130-167): a wave a block of 256, four values a lane; the
+// largest-magnitude value, the first of equals, sets iscale = -127/max.  The loads of up
+// to four of the wave's blocks go out together.
+__device__ __forceinline__ void stage_q8k_from_f32(const float* __restrict__ x, int nblk, i8* lxq, float* lxs, int* lbs) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  for (int b0 = wave; b0 < nblk; b0 += 4 * kWaves) {
+    float4 vs[4];
+#pragma unroll
+    for (int u = 0; u < 4; u++) {
+      const int b = b0 + u * kWaves;
+      vs[u] = b < nblk ? *(const float4*)(x + b * 256 + 4 * lane) : make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+#pragma unroll
+    for (int u = 0; u < 4; u++) {
+      const int b = b0 + u * kWaves;
+      if (b >= nblk) break;
+      const float4 v = vs[u];
+      const float amax = wave_max(fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w))));
+      int q0 = 0, q1 = 0, q2 = 0, q3 = 0;
+      float d = 0.0f;
+      if (amax != 0.0f) {
+        // the first position holding the maximum: lowest lane per component, then lowest index
+        const u64 m0 = __ballot(fabsf(v.x) == amax), m1 = __ballot(fabsf(v.y) == amax);
+        const u64 m2 = __ballot(fabsf(v.z) == amax), m3 = __ballot(fabsf(v.w) == amax);
+        int idx = 1 << 20;
+        if (m0) idx = min(idx, 4 * (int)__builtin_ctzll(m0));
+        if (m1) idx = min(idx, 4 * (int)__builtin_ctzll(m1) + 1);
+        if (m2) idx = min(idx, 4 * (int)__builtin_ctzll(m2) + 2);
+        if (m3) idx = min(idx, 4 * (int)__builtin_ctzll(m3) + 3);
+        const int src = __builtin_amdgcn_readfirstlane(idx >> 2), e = __builtin_amdgcn_readfirstlane(idx & 3);
+        const float pick = e == 0 ? v.x : e == 1 ? v.y : e == 2 ? v.z : v.w;
+        const float mx = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(pick), src));
+        const float iscale = -127.0f / mx;
+        q0 = min(127, (int)rintf(iscale * v.x)); q1 = min(127, (int)rintf(iscale * v.y));
+        q2 = min(127, (int)rintf(iscale * v.z)); q3 = min(127, (int)rintf(iscale * v.w));
+        d = 1.0f / iscale;
+      }
+      *(int*)(lxq + b * XP + 4 * lane) = (q0 & 0xFF) | ((q1 & 0xFF) << 8) | ((q2 & 0xFF) << 16) | ((q3 & 0xFF) << 24);
+      const int s = ilt_sum4(q0 + q1 + q2 + q3);
+      if ((lane & 3) == 0) lbs[b * 16 + (lane >> 2)] = s;
+      if (lane == 0) lxs[b] = d;
+    }
+  }
+}
+
+// Q8_0 (quantize-q8!, tensor.lisp:245-262): 8 lanes a block of 32.
+__device__ __forceinline__ void stage_q8_from_f32(const float* __restrict__ x, int nblk, int f16_scale, i8* lxq, float* lxs) {
+  const int n8 = nblk * 8;
+  for (int c0 = 0; c0 < n8; c0 += kThreads) {
+    const int c = c0 + threadIdx.x;
+    const float4 v = c < n8 ? *(const float4*)(x + 4 * c) : make_float4(0.f, 0.f, 0.f, 0.f);
+    float amax = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
+    amax = fmaxf(amax, ilt_dppf<ILT_DPP_XOR1>(amax));
+    amax = fmaxf(amax, ilt_dppf<ILT_DPP_XOR2>(amax));
+    amax = fmaxf(amax, ilt_dppf<ILT_DPP_HALF_MIRROR>(amax));
+    const float d = amax / 127.0f;
+    const float id = d == 0.0f ? 0.0f : 1.0f / d;
+    const int q0 = (int)rintf(v.x * id), q1 = (int)rintf(v.y * id), q2 = (int)rintf(v.z * id), q3 = (int)rintf(v.w * id);
+    if (c < n8) {
+      *(int*)(lxq + 4 * c) = (q0 & 0xFF) | ((q1 & 0xFF) << 8) | ((q2 & 0xFF) << 16) | ((q3 & 0xFF) << 24);
+      if ((c & 7) == 0) lxs[c >> 3] = f16_scale ? __half2float(__float2half_rn(d)) : d;
+    }
   }
 }
 
 template <int FMT>
-size_t gemv_smem(const IltGemvParams& p) {
-  using F = Fmt<FMT>;
-  const int S = p.cols / F::BW;
-  size_t b = p.cols + 4 * S + ((FMT == ILT_Q8_0 || FMT == ILT_IQ2_XXS) ? 0 : p.cols / 16 * 4) + 8;
-  if (FMT == ILT_IQ2_XXS) b += 2048;
-  return b + (size_t)p.rw * S * F::TERMS * 4;
+__device__ __forceinline__ void run_rows(const IltGemvMat& m, const IltGemvParams& p, long row0, int nrows, int S,
+                                         const Lds& L, float* t, int lane, int z, const Raw<FMT>* pre) {
+  const u8* w = p.ptrs ? (const u8*)(p.ptrs[z] + p.add) : m.w;
+  wave_rows<FMT>(w, m.wd, row0, nrows, S, p.s_magic, m.row_bytes, L, t, lane, pre);
 }
 
-template <int FMT>
-hipError_t launch(const IltGemvParams& p, int nz, hipStream_t st) {
-  dim3 grid((p.rows + p.rw - 1) / p.rw, 1, nz);
-  const size_t smem = gemv_smem<FMT>(p);
-  hipLaunchKernelGGL(gemv_kernel<FMT>, grid, dim3(kThreads), smem, st, p);
-  return hipGetLastError();
+// FSET: one format (its GGUF number), or 0 = the launch's matrices mix Q4_K and Q6_K
+// The preloaded first step: one register set for the launch's format (two when they mix)
+template <int FSET> struct Pre {
+  Raw<(FSET ? FSET : ILT_Q4_K)> a;
+  Raw<(FSET ? FSET : ILT_Q6_K)> b;      // used only when FSET == 0, for a Q6_K matrix
+};
+
+template <int FSET>
+__device__ __forceinline__ void run_any(const IltGemvMat& m, const IltGemvParams& p, long row0, int nrows, int S,
+                                        const Lds& L, float* t, int lane, int z, const Pre<FSET>* pre) {
+  if (FSET != 0) run_rows<(FSET ? FSET : ILT_Q4_K)>(m, p, row0, nrows, S, L, t, lane, z, pre ? &pre->a : nullptr);
+  else if (m.fmt == ILT_Q4_K) run_rows<ILT_Q4_K>(m, p, row0, nrows, S, L, t, lane, z, (const Raw<ILT_Q4_K>*)(pre ? &pre->a : nullptr));
+  else run_rows<ILT_Q6_K>(m, p, row0, nrows, S, L, t, lane, z, (const Raw<ILT_Q6_K>*)(pre ? &pre->b : nullptr));
+}
+
+__device__ __forceinline__ float sum_any(int fmt, const float* t, int S) {
+  switch (fmt) {
+    case ILT_Q8_0: return row_sum<ILT_Q8_0>(t, S);
+    case ILT_Q4_K: return row_sum<ILT_Q4_K>(t, S);
+    case ILT_Q6_K: return row_sum<ILT_Q6_K>(t, S);
+    case ILT_Q2_K: return row_sum<ILT_Q2_K>(t, S);
+    default: return row_sum<ILT_IQ2_XXS>(t, S);
+  }
+}
+
+// FSET: the format of every matrix of the launch, or 0 when they mix Q4_K and Q6_K.  The
+// expert formats (IQ2_XXS, Q2_K) take grid y = expert.
+template <int FSET>
+__global__ __launch_bounds__(kThreads) void gemv_kernel(IltGemvParams p) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  const int z = blockIdx.y;
+  constexpr bool q8 = FSET == ILT_Q8_0;
+  const int S = q8 ? p.cols / 32 : p.cols / 256;
+  // LDS: xq | bsums | xs | (grid) | terms (per wave)
+  i8* lxq = (i8*)smem;
+  const int xq_bytes = q8 ? p.cols : S * XP;
+  int* lbs = (int*)(smem + xq_bytes);
+  const int nbs = (q8 || FSET == ILT_IQ2_XXS) ? 0 : p.cols / 16;
+  float* lxs = (float*)(lbs + nbs);
+  u64* lgrid = (u64*)(((uintptr_t)(lxs + S) + 7) & ~(uintptr_t)7);
+  float* terms = (float*)(lgrid + (FSET == ILT_IQ2_XXS ? 256 : 0));
+
+  // grouped rows (d4_mvq8): wgs_per_group workgroups share one group's rows and activations
+  const int group = p.group_rows > 0 ? blockIdx.x / p.wgs_per_group : 0;
+  const int wg_in = p.group_rows > 0 ? blockIdx.x % p.wgs_per_group : blockIdx.x;
+  const int nwg = p.group_rows > 0 ? p.wgs_per_group : gridDim.x;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int RB = p.batch;                             // rows per batch
+
+  // Batches of RB rows (never across two matrices) are dealt out to the grid's waves in turn,
+  // so at any time the waves' reads lie close together in memory.
+  const int nw = nwg * kWaves, wid = wg_in * kWaves + wave;
+  const long grow0 = (long)group * p.group_rows;      // first row of this group (0 when ungrouped)
+  auto locate = [&](int b, int& mi, long& row0, int& nrows) {
+    mi = 0;
+    if (!p.glu) while (mi + 1 < p.nmat && b >= p.mat[mi + 1].batch0) mi++;
+    // batch bl of nbat deals out the rows evenly: [rows*bl/nbat, rows*(bl+1)/nbat)
+    const long rows = p.group_rows > 0 ? p.group_rows : p.mat[mi].rows;
+    const long bl = b - p.mat[mi].batch0, nbat = p.mat[mi].nbat;
+    row0 = rows * bl / nbat;
+    nrows = (int)(rows * (bl + 1) / nbat - row0);
+    row0 += grow0;
+  };
+
+  // the first batch's first loads go out now, so they are on their way while x is staged
+  Pre<FSET> pre;
+  if (wid < p.nbatches) {
+    int mi; long row0; int nrows;
+    locate(wid, mi, row0, nrows);
+    const IltGemvMat& m = p.mat[mi];
+    const u8* w0 = p.ptrs ? (const u8*)(p.ptrs[z] + p.add) : m.w;
+    if (FSET != 0 || m.fmt == ILT_Q4_K) first_load<(FSET ? FSET : ILT_Q4_K)>(pre.a, w0, m.wd, row0, nrows, S, m.row_bytes, lane);
+    else first_load<(FSET ? FSET : ILT_Q6_K)>(pre.b, w0, m.wd, row0, nrows, S, m.row_bytes, lane);
+    // and a touch of every 64-byte line of the batch's first 16 KB, so the later steps hit in L2
+    const u8* wb = w0 + row0 * m.row_bytes;
+    const long bytes = (long)nrows * m.row_bytes;
+    int warm = 0;
+    for (long o = 64L * lane; o < bytes && o < 16384; o += 64 * 64) warm ^= *(const int*)(wb + (o & ~3L));
+    asm volatile("" :: "v"(warm));
+  }
+
+  // ---- stage the activations ----
+  const long xoff = (long)z * p.x_stride + (long)group * p.cols;
+  if (p.xf) {
+    if (q8) stage_q8_from_f32(p.xf + xoff, S, p.f16_scale, lxq, lxs);
+    else stage_q8k_from_f32(p.xf + xoff, S, lxq, lxs, lbs);
+  } else {
+    const i8* gxq = p.xq + xoff;
+    if (q8) {
+      for (int i = threadIdx.x * 16; i < p.cols; i += kThreads * 16) *(int4*)(lxq + i) = *(const int4*)(gxq + i);
+      for (int i = threadIdx.x; i < S; i += kThreads) lxs[i] = p.xs[xoff / 32 + i];
+    } else {
+      for (int i = threadIdx.x; i < S * 16; i += kThreads)
+        *(int4*)(lxq + (i >> 4) * XP + 16 * (i & 15)) = *(const int4*)(gxq + 16 * i);
+      for (int i = threadIdx.x; i < S; i += kThreads) lxs[i] = p.xs[xoff / 256 + i];
+      for (int i = threadIdx.x; i < nbs; i += kThreads) lbs[i] = p.bsums[xoff / 16 + i];
+    }
+  }
+  if (FSET == ILT_IQ2_XXS) lgrid[threadIdx.x] = ilt_iq2xxs_grid_dev[threadIdx.x];
+  __syncthreads();
+
+  const Lds L = { lxq, lxs, lbs, lgrid };
+  const int tpr = q8 ? S : S * 2;                     // floats of terms per row (the larger TERMS)
+  float* tw = terms + (long)wave * RB * tpr * (p.glu ? 2 : 1);
+
+  for (int b = wid; b < p.nbatches; b += nw) {
+    int mi; long row0; int nrows;
+    locate(b, mi, row0, nrows);
+    const IltGemvMat& m = p.mat[mi];
+    const int fmt = FSET != 0 ? FSET : m.fmt;
+    run_any<FSET>(m, p, row0, nrows, S, L, tw, lane, z, b == wid ? &pre : nullptr);
+    if (p.glu) run_any<FSET>(p.mat[1], p, row0, nrows, S, L, tw + (long)RB * tpr, lane, z, nullptr);   // up's same rows
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    if (lane < nrows) {
+      const int tper = (fmt == ILT_Q4_K || fmt == ILT_Q2_K) ? 2 : 1;
+      float v = FSET != 0 ? row_sum<(FSET ? FSET : ILT_Q4_K)>(tw + (long)lane * S * tper, S) : sum_any(fmt, tw + (long)lane * S * tper, S);
+      const long r = row0 + lane;
+      if (p.glu) {
+        const int ufmt = FSET != 0 ? FSET : p.mat[1].fmt;
+        const float uv = sum_any(ufmt, tw + (long)RB * tpr + (long)lane * S * (ufmt == ILT_Q4_K ? 2 : 1), S);
+        m.y[r] = dense_glu(v, uv);
+      } else {
+        float* y = m.y + (long)z * p.y_stride;
+        if (m.bias) v = v + m.bias[r];
+        if (p.acc) v = y[r] + v;
+        y[r] = v;
+      }
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+  }
+}
+
+size_t gemv_smem(int fset, const IltGemvParams& p) {
+  const bool q8 = fset == ILT_Q8_0;
+  const int S = q8 ? p.cols / 32 : p.cols / 256;
+  size_t b = q8 ? (size_t)p.cols : (size_t)S * XP;
+  b += (q8 || fset == ILT_IQ2_XXS) ? 0 : (size_t)p.cols / 16 * 4;
+  b += 4 * (size_t)S + 8;
+  if (fset == ILT_IQ2_XXS) b += 2048;
+  return b + (size_t)kWaves * p.batch * S * (q8 ? 1 : 2) * 4 * (p.glu ? 2 : 1);
 }
 
 }  // namespace
 
-// Rows per workgroup: enough workgroups to cover the chip several times over, but no
-// more rows than LDS terms allow and at least 4 so the activations' staging is shared.
-int ilt_gemv_pick_rw(int fmt, int rows, int cols, int nz) {
-  const int bw = fmt == ILT_Q8_0 ? 32 : 256;
-  const int S = cols / bw, terms = (fmt == ILT_Q4_K || fmt == ILT_Q2_K) ? 2 : 1;
-  int rw = 32;
-  while (rw > 4 && (long)((rows + rw - 1) / rw) * nz < 2048) rw >>= 1;
-  while (rw > 1 && (size_t)rw * S * terms * 4 > 48 * 1024) rw >>= 1;
-  return rw;
-}
-
-hipError_t ilt_gemv_launch(int fmt, const IltGemvParams& p, int nz, hipStream_t st) {
-  switch (fmt) {
-    case ILT_Q8_0: return launch<ILT_Q8_0>(p, nz, st);
-    case ILT_Q4_K: return launch<ILT_Q4_K>(p, nz, st);
-    case ILT_Q6_K: return launch<ILT_Q6_K>(p, nz, st);
-    case ILT_Q2_K: return launch<ILT_Q2_K>(p, nz, st);
-    case ILT_IQ2_XXS: return launch<ILT_IQ2_XXS>(p, nz, st);
+hipError_t ilt_gemv_launch(IltGemvParams& p, int nz, hipStream_t st) {
+  int fset = p.mat[0].fmt;
+  for (int i = 1; i < p.nmat; i++) if (p.mat[i].fmt != fset) fset = 0;
+  const bool q8 = fset == ILT_Q8_0;
+  const int S = q8 ? p.cols / 32 : p.cols / 256;
+  const int nm = p.glu ? 1 : p.nmat;
+  long total_rows = 0;
+  for (int i = 0; i < nm; i++) total_rows += p.mat[i].rows;
+  const int ngroups = p.group_rows > 0 ? (int)(total_rows / p.group_rows) : 1;
+  const long rows_each = p.group_rows > 0 ? p.group_rows : total_rows;     // rows that share one x
+  // The grid is a whole number of workgroups per CU (256 CUs), 1024 workgroups at most, split
+  // over grid y and the row groups; every wave gets the same number of batches, and a
+  // matrix's batches share its rows out evenly.  A batch is 16 rows at most (one lane each
+  // in phase B) and no more than the terms' share of LDS (32 KB) allows.
+  const size_t row_terms = (size_t)kWaves * S * (q8 ? 1 : 2) * 4 * (p.glu ? 2 : 1);
+  int rb_max = 16;
+  if ((size_t)rb_max * row_terms > 32768) rb_max = (int)(32768 / row_terms);
+  if (rb_max < 1) rb_max = 1;
+  const long all_rows = rows_each * nz * ngroups;
+  int m = 4;
+  while (m > 1 && all_rows < 3L * 1024 * m) m--;               // at least three rows a wave on average
+  int waves_each = 1024 * m / (nz * ngroups) / kWaves * kWaves;  // waves per (grid y, group)
+  if (waves_each < kWaves) waves_each = kWaves;
+  if (waves_each > rows_each) waves_each = (int)((rows_each + kWaves - 1) / kWaves * kWaves);
+  const int rounds = (int)((rows_each + (long)waves_each * rb_max - 1) / ((long)waves_each * rb_max));
+  long nb_total = (long)waves_each * rounds;
+  if (nb_total > rows_each) nb_total = rows_each;
+  p.batch = rb_max;
+  int nb = 0;
+  for (int i = 0; i < p.nmat; i++) {
+    p.mat[i].batch0 = nb;
+    if (i >= nm) { p.mat[i].nbat = p.mat[0].nbat; continue; }
+    const long r = p.group_rows > 0 ? p.group_rows : p.mat[i].rows;
+    long nbi = (nb_total * r + rows_each - 1) / rows_each;       // this matrix's share of the batches
+    if (nbi < (r + rb_max - 1) / rb_max) nbi = (r + rb_max - 1) / rb_max;
+    if (nbi > r) nbi = r;
+    p.mat[i].nbat = (int)nbi;
+    nb += (int)nbi;
   }
-  return hipErrorInvalidValue;
+  p.nbatches = nb;                                                          // per group, per grid y
+  p.s_magic = (uint32_t)(0x100000000ULL / (uint64_t)S) + 1;   // floor(f/S) = umulhi(f, magic) while f*S < 2^32
+  const int wgs = waves_each / kWaves;
+  p.wgs_per_group = wgs;
+  dim3 grid(wgs * ngroups, nz);
+  const size_t smem = gemv_smem(fset, p);
+  if (smem > 64 * 1024) return hipErrorInvalidValue;
+  switch (fset) {
+    case 0: hipLaunchKernelGGL(gemv_kernel<0>, grid, dim3(kThreads), smem, st, p); break;
+    case ILT_Q8_0: hipLaunchKernelGGL(gemv_kernel<ILT_Q8_0>, grid, dim3(kThreads), smem, st, p); break;
+    case ILT_Q4_K: hipLaunchKernelGGL(gemv_kernel<ILT_Q4_K>, grid, dim3(kThreads), smem, st, p); break;
+    case ILT_Q6_K: hipLaunchKernelGGL(gemv_kernel<ILT_Q6_K>, grid, dim3(kThreads), smem, st, p); break;
+    case ILT_Q2_K: hipLaunchKernelGGL(gemv_kernel<ILT_Q2_K>, grid, dim3(kThreads), smem, st, p); break;
+    case ILT_IQ2_XXS: hipLaunchKernelGGL(gemv_kernel<ILT_IQ2_XXS>, grid, dim3(kThreads), smem, st, p); break;
+    default: return hipErrorInvalidValue;
+  }
+  return hipGetLastError();
 }

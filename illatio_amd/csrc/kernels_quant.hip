@@ -84,6 +84,15 @@ __global__ __launch_bounds__(256) void repack_q8_kernel(const u8* __restrict__ r
   if (k == 0) d[b] = *(const u16*)blk;
 }
 
+// GGUF Q6_K blocks (210 bytes) to the device block: the same bytes, then two of padding.
+__global__ __launch_bounds__(256) void repack_q6k_kernel(const u8* __restrict__ raw, u8* __restrict__ out, long long nblocks) {
+  const long long i = (long long)blockIdx.x * 256 + threadIdx.x;   // one thread per 2 bytes
+  const long long b = i / (ILT_Q6K_STRIDE / 2);
+  if (b >= nblocks) return;
+  const int k = (int)(i % (ILT_Q6K_STRIDE / 2));
+  *(u16*)(out + b * ILT_Q6K_STRIDE + 2 * k) = k < 105 ? *(const u16*)(raw + b * 210 + 2 * k) : (u16)0;
+}
+
 __global__ __launch_bounds__(256) void copy_bytes_kernel(const u8* __restrict__ src, u8* __restrict__ dst, long long bytes) {
   const long long i = ((long long)blockIdx.x * 256 + threadIdx.x) * 2;
   if (i + 1 < bytes) *(u16*)(dst + i) = *(const u16*)(src + i);
@@ -112,7 +121,7 @@ __device__ float dequant_one(int fmt, const u8* wrow, const u16* wdrow, int col)
     return d1 * (float)q - m1;
   }
   if (fmt == ILT_Q6_K) {
-    const u8* blk = wrow + (long)i * 210;
+    const u8* blk = wrow + (long)i * ILT_Q6K_STRIDE;
     const int c = idx >> 7, r = idx & 127, part = r >> 5, l = r & 31;
     const int lowbyte = blk[64 * c + (part & 1) * 32 + l];
     const int low = part < 2 ? (lowbyte & 0xF) : (lowbyte >> 4);
@@ -168,6 +177,13 @@ hipError_t ilt_k_quant_q8k(const float* x, int8_t* xq, float* xd, int* bsums, lo
 hipError_t ilt_k_repack_q8(const uint8_t* raw, int8_t* qs, uint16_t* d, long long nblocks, hipStream_t st) {
   if (nblocks <= 0) return hipSuccess;
   hipLaunchKernelGGL(repack_q8_kernel, dim3((unsigned)((nblocks * 16 + 255) / 256)), dim3(256), 0, st, raw, qs, d, nblocks);
+  return hipGetLastError();
+}
+
+hipError_t ilt_k_repack_q6k(const uint8_t* raw, uint8_t* out, long long nblocks, hipStream_t st) {
+  if (nblocks <= 0) return hipSuccess;
+  const long long n = nblocks * (ILT_Q6K_STRIDE / 2);
+  hipLaunchKernelGGL(repack_q6k_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, raw, out, nblocks);
   return hipGetLastError();
 }
 

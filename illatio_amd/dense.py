@@ -7,6 +7,8 @@ format, this path quantizes them as the reference's CPU path does -- Q8_0 for Q8
 matrices, Q8_K for K-quants (matrix-act-kind, kquant.lisp:532-533) -- so results match
 the CPU path bit for bit.
 """
+import ctypes as C
+
 import numpy as np
 
 from . import hip
@@ -31,7 +33,7 @@ class CMat:
 
 def upload_gmat(dev, name, qtype, rows, cols, raw_bytes):
     """RAW_BYTES (the matrix's GGUF blocks, a uint8 array) to DEV: Q8_0 split into int8s and
-    scales by repack_q8; Q6_K through repack_q6k (which here keeps the 210-byte blocks);
+    scales by repack_q8; Q6_K through repack_q6k (here: 210-byte blocks padded to 212);
     Q4_K as it is."""
     if qtype not in (Q8_0, Q4_K, Q6_K):
         raise ValueError(f"the dense path multiplies Q8_0, Q4_K and Q6_K; {name} is type {qtype}")
@@ -111,6 +113,46 @@ def cmat_mul(dev, w, act, y, n=1, bias=None, acc=False):
         hip.launch(dev, "mm_q8", ((n + 63) // 64, (rows + 63) // 64), 256,
                    [w.qs, w.d, act.xq, act.xs, y, bias, rows, cols, n, a])
     return y
+
+
+class MvDesc(C.Structure):
+    _fields_ = [("gguf_type", C.c_int), ("rows", C.c_int), ("w", C.c_uint64), ("wd", C.c_uint64),
+                ("y", C.c_uint64), ("bias", C.c_uint64)]
+
+
+def mv_multi(dev, parts, act=None, xf=None, f16_scale=True, acc=False, glu=False):
+    """PARTS, up to four (W Y BIAS) sharing X, in one launch (CMAT-MUL-N's idea, for one
+    token): X quantized in ACT, or the floats XF, which the kernel then quantizes itself."""
+    descs = (MvDesc * len(parts))()
+    for i, (w, y, bias) in enumerate(parts):
+        descs[i] = MvDesc(w.type, w.rows, w.qs.ptr, w.d.ptr if w.d else 0, y.ptr, bias.ptr if bias else 0)
+    w0 = parts[0][0]
+    if xf is not None:
+        xq = xs = bs = 0
+    elif w0.kquant_p():
+        xq, xs, bs = act.kq.ptr, act.kd.ptr, act.ksum.ptr
+    else:
+        xq, xs, bs = act.xq.ptr, act.xs.ptr, 0
+    hip.call("ilt_mv_multi", C.c_uint64(dev.stream), C.c_int(len(parts)), descs, C.c_int(w0.cols), C.c_uint64(xq),
+             C.c_uint64(xs), C.c_uint64(bs), C.c_uint64(xf.ptr if xf is not None else 0), C.c_int(1 if f16_scale else 0),
+             C.c_int(1 if acc else 0), C.c_int(1 if glu else 0))
+
+
+def qkv_mul(dev, wq, wk, wv, act, q, k, v, bq=None, bk=None, bv=None, xf=None):
+    """Q, K and V's products of one token in one launch (QKV-MUL, cuda-dense.lisp:309-324)."""
+    mv_multi(dev, [(wq, q, bq), (wk, k, bk), (wv, v, bv)], act, xf)
+
+
+def glu_mul(dev, g, u, act, fa, xf=None):
+    """silu(G x) * (U x) into FA for one token (GLU-MUL, cuda-dense.lisp:326-339)."""
+    if xf is not None:
+        return mv_multi(dev, [(g, fa, None), (u, fa, None)], None, xf, glu=True)
+    f, d = g.rows, g.cols
+    if g.kquant_p():
+        hip.launch(dev, "mv_k_glu", (f + 3) // 4, 128,
+                   [KQUANT_CODE[g.type], g.qs, KQUANT_CODE[u.type], u.qs, act.kq, act.kd, act.ksum, fa, f, d])
+    else:
+        hip.launch(dev, "mv_q8_glu", (f + 3) // 4, 128, [g.qs, g.d, u.qs, u.d, act.xq, act.xs, fa, f, d])
 
 
 def embed(dev, emb, tokens, x, n, d):

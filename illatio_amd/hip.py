@@ -13,7 +13,7 @@ import os
 import numpy as np
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libillatio_hip.so")
+LIB_PATH = os.environ.get("ILLATIO_HIP_LIB") or os.path.join(_HERE, "libillatio_hip.so")
 
 NOT_READY = 600
 

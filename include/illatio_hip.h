@@ -88,9 +88,12 @@ int ilt_host_unregister(void* p);                       /* cuMemHostUnregister, 
 
 /* Upload-time repacks (cuda-dense.lisp:87-100).
    repack_q8 (src/cuda/dense.cu:42): GGUF Q8_0 blocks -> int8 quants + f16 scales.
-   repack_q6k (src/cuda/kquant.cu:195): the reference pads Q6_K blocks to 224 bytes; here
-   the 210-byte blocks are read where they lie, so this copies them unchanged (out needs
-   210*nblocks bytes; the reference's 224*nblocks is enough). */
+   repack_q6k (src/cuda/kquant.cu:195): the reference pads Q6_K blocks to 224 bytes for
+   16-byte alignment; gfx950 only needs 4-byte alignment for full-rate 128-bit loads, so
+   the device block is the 210 GGUF bytes plus 2 of padding (ILT_Q6K_DEVICE_BLOCK = 212;
+   out needs 212*nblocks bytes, the reference's 224*nblocks is enough).  Every kernel that
+   takes a Q6_K matrix takes this layout. */
+#define ILT_Q6K_DEVICE_BLOCK 212
 int ilt_repack_q8(uint64_t stream, const void* raw, void* qs, void* d, int64_t nblocks);
 int ilt_repack_q6k(uint64_t stream, const void* raw, void* out, int64_t nblocks);
 
@@ -120,6 +123,32 @@ int ilt_mv_k(uint64_t stream, int type, const void* w, const int8_t* xq, const f
              const float* bias, int rows, int cols, int acc);
 int ilt_d4_mvq8(uint64_t stream, int rows, int cols, int group_rows, const int8_t* wq, const uint16_t* wd,
                 const int8_t* xq, const float* xs, float* y);
+
+/* Gate and up in one launch ending in swiglu! (model.lisp:364-378): out[r] =
+   (g / (1 + exp(-g))) * u with g = gate[r].x, u = up[r].x, each the decode product's bits.
+   mv_q8_glu (dense.cu:230), mv_k_glu (kquant.cu:183). */
+int ilt_mv_q8_glu(uint64_t stream, const int8_t* gq, const uint16_t* gd, const int8_t* uq, const uint16_t* ud,
+                  const int8_t* xq, const float* xs, float* out, int rows, int cols);
+int ilt_mv_k_glu(uint64_t stream, int gtype, const void* gw, int utype, const void* uw, const int8_t* xq, const float* xd,
+                 const int32_t* bsums, float* out, int rows, int cols);
+
+/* Up to four matrices that share x in one launch (the reference has this for Q8_0 only,
+   mv_q8_3; its K-quant QKV is three launches, cuda-dense.lisp:321-323).  All Q8_0, or any mix
+   of Q4_K and Q6_K.  The activations come quantized (xq, xs, bsums as for mv_q8 / mv_k), or,
+   with xf non-null, as floats that every workgroup quantizes for itself exactly as
+   quantize-q8! (scale through fp16 when f16_scale) / quantize-q8k! would: the product then
+   needs no quantizer launch before it.  glu: descs[0] = gate, descs[1] = up, result into
+   descs[0].y.  No counterpart in the reference beyond mv_q8_3. */
+typedef struct ilt_mv_desc {
+  int gguf_type;          /* ILT_TYPE_Q8_0, ILT_TYPE_Q4_K or ILT_TYPE_Q6_K */
+  int rows;
+  const void* w;          /* Q8_0: int8 quants (repacked) */
+  const uint16_t* wd;     /* Q8_0: f16 scales; else null */
+  float* y;
+  const float* bias;      /* or null */
+} ilt_mv_desc;
+int ilt_mv_multi(uint64_t stream, int nmat, const ilt_mv_desc* descs, int cols, const int8_t* xq, const float* xs,
+                 const int32_t* bsums, const float* xf, int f16_scale, int acc, int glu);
 
 /* The indexed expert products (ds4f.cu:769, 837; CPU: iq2xxs-row-dot, q2k-row-dot,
    iquant.lisp:126-215).  For each z < nz: W = the nrows x ncols matrix at ptrs[z] + add

@@ -484,6 +484,9 @@ float orc_softplus(float x) {
   return sb_log(1.0f + sb_exp(x));
 }
 
+/* ---- src/model.lisp:364-378 (swiglu!): silu(x) = x / (1 + e^-x), times b ------------------------------ */
+float orc_swiglu(float x, float b) { return (x / (1.0f + sb_exp(-x))) * b; }
+
 /* ---- src/ds4f.lisp:950-978 (d4-route), the top-N_USED branch --------------------------------------- */
 /* sel: nu expert indices in descending-score order; w: their weights.  bias may be NULL. */
 void orc_route(const float* logits, const float* bias, int ne, int nu, float scale, int32_t* sel, float* w) {

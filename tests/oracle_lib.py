@@ -32,8 +32,9 @@ def lib():
         L.orc_single_to_half.argtypes = [C.c_float]
         for name in ("orc_q8_0_row_dot", "orc_q4k_row_dot", "orc_q6k_row_dot", "orc_iq2xxs_row_dot",
                      "orc_iq2xxs_row_dot_avx2", "orc_q2k_row_dot", "orc_q2k_row_dot_avx2",
-                     "orc_sigmoid", "orc_silu", "orc_softplus"):
+                     "orc_sigmoid", "orc_silu", "orc_softplus", "orc_swiglu"):
             getattr(L, name).restype = C.c_float
+        L.orc_swiglu.argtypes = [C.c_float, C.c_float]
         for name in ("orc_sigmoid", "orc_silu", "orc_softplus"):
             getattr(L, name).argtypes = [C.c_float]
         for name in ("orc_block_bytes", "orc_block_weights"):
@@ -156,6 +157,14 @@ def silu(x):
 
 def sigmoid(x):
     return lib().orc_sigmoid(float(np.float32(x)))
+
+
+def swiglu(g, u):
+    """silu(g) * u as the dense models compute it (swiglu!, model.lisp:364-378), elementwise."""
+    g = np.ascontiguousarray(g, np.float32).ravel()
+    u = np.ascontiguousarray(u, np.float32).ravel()
+    f = lib().orc_swiglu
+    return np.array([f(float(a), float(b)) for a, b in zip(g, u)], np.float32)
 
 
 def softplus(x):

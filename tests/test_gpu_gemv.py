@@ -210,3 +210,64 @@ def test_invalid_arguments_are_errors_not_faults(dev):
     with pytest.raises(hip.HipError):
         hip.launch(dev, "mv_q8", 1, 128, [None, b, b, b, b, None, 4, 32, 0])      # null weights
     hip.hip_free(b)
+
+
+@pytest.mark.parametrize("kind", ["k", "q8"])
+def test_fused_launches_match_single_products(dev, kind):
+    """Q, K, V in one launch; gate and up ending in swiglu!; and the same with the kernel
+    quantizing the float activations itself -- all with the single products' bits."""
+    from illatio_amd import dense, hip
+    rng = synth.make_rng(555 if kind == "k" else 556)
+    cols = 2560 if kind == "k" else 896
+    shapes = [(synth.Q4_K, 4096), (synth.Q4_K, 1024), (synth.Q6_K, 1024)] if kind == "k" else \
+             [(synth.Q8_0, 896), (synth.Q8_0, 128), (synth.Q8_0, 132)]
+    ws = [synth.weights(t, r, cols, rng) for t, r in shapes]
+    ms = [upload(dev, t, r, cols, w) for (t, r), w in zip(shapes, ws)]
+    x = special_activations(cols, rng)
+    xb = hip.hip_upload_new(dev, x)
+    act = dense.QAct(dev, 1, cols, ("q8k",) if kind == "k" else ("q8",))
+    dense.quantize_act(dev, xb, act)
+    biases = [None, synth.activations(shapes[1][1], rng), None]
+    bbs = [None if b is None else hip.hip_upload_new(dev, b) for b in biases]
+    want = [orc.matmul(t, w, r, cols, x) + (0 if b is None else b) for (t, r), w, b in zip(shapes, ws, biases)]
+    for xf in (None, xb):
+        ys = [hip.hip_alloc(dev, 4 * r) for _, r in shapes]
+        dense.qkv_mul(dev, ms[0], ms[1], ms[2], act, ys[0], ys[1], ys[2], bbs[0], bbs[1], bbs[2], xf=xf)
+        for y, wv, (_, r) in zip(ys, want, shapes):
+            assert np.array_equal(bits(hip.hip_floats(y, r)), bits(wv)), ("qkv", kind, xf is not None)
+        for y in ys:
+            hip.hip_free(y)
+    # gate/up: two matrices of equal rows (mixed K-quant formats allowed)
+    gshape = [(synth.Q4_K, 1000), (synth.Q6_K, 1000)] if kind == "k" else [(synth.Q8_0, 500), (synth.Q8_0, 500)]
+    gw = [synth.weights(t, r, cols, rng) for t, r in gshape]
+    gm = [upload(dev, t, r, cols, w) for (t, r), w in zip(gshape, gw)]
+    g = orc.matmul(gshape[0][0], gw[0], gshape[0][1], cols, x)
+    u = orc.matmul(gshape[1][0], gw[1], gshape[1][1], cols, x)
+    g[:3] = g[:3]  # values as they come; the extreme gates are covered below
+    wglu = orc.swiglu(g, u)
+    for xf in (None, xb):
+        fa = hip.hip_alloc(dev, 4 * gshape[0][1])
+        dense.glu_mul(dev, gm[0], gm[1], act, fa, xf=xf)
+        assert np.array_equal(bits(hip.hip_floats(fa, gshape[0][1])), bits(wglu)), ("glu", kind, xf is not None)
+        hip.hip_free(fa)
+    for b in [xb] + [b for b in bbs if b is not None]:
+        hip.hip_free(b)
+    act.free()
+    for m in ms + gm:
+        m.free()
+
+
+def test_in_kernel_quantization_single_matrix(dev):
+    """xf: the float activations quantized by every workgroup as quantize-q8k! / quantize-q8!."""
+    from illatio_amd import dense, hip
+    rng = synth.make_rng(909)
+    for qtype, rows, cols in ((synth.Q6_K, 2560, 9728), (synth.Q4_K, 64, 256), (synth.Q8_0, 896, 4864), (synth.Q8_0, 8, 32)):
+        w = synth.weights(qtype, rows, cols, rng)
+        x = special_activations(cols, rng) if cols >= 512 else synth.activations(cols, rng)
+        m = upload(dev, qtype, rows, cols, w)
+        xb, y = hip.hip_upload_new(dev, x), hip.hip_alloc(dev, 4 * rows)
+        for f16 in ((True, False) if qtype == synth.Q8_0 else (True,)):
+            dense.mv_multi(dev, [(m, y, None)], xf=xb, f16_scale=f16)
+            want = orc.matmul(qtype, w, rows, cols, x, f16_scale=f16)
+            assert np.array_equal(bits(hip.hip_floats(y, rows)), bits(want)), (qtype, rows, cols, f16)
+        hip.hip_free(xb); hip.hip_free(y); m.free()
