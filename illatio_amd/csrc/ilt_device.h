@@ -99,6 +99,13 @@ __device__ __forceinline__ u16 ilt_ld2(const u8* p) {
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t ilt_rsrc(const void* base, u32 bytes) {
   return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, bytes, 0x00020000);
 }
+// A pointer that is the same in every lane, said so to the compiler (a descriptor built from
+// a value it cannot prove uniform is applied lane by lane in a loop).
+__device__ __forceinline__ const void* ilt_uniform_ptr(const void* p) {
+  const u64 a = (u64)p;
+  const u32 lo = __builtin_amdgcn_readfirstlane((u32)a), hi = __builtin_amdgcn_readfirstlane((u32)(a >> 32));
+  return (const void*)(((u64)hi << 32) | lo);
+}
 __device__ __forceinline__ int4 ilt_bld16(__amdgpu_buffer_rsrc_t r, u32 off) {
   const ilt_v4i v = __builtin_amdgcn_raw_buffer_load_b128(r, off, 0, 0);
   return make_int4(v.x, v.y, v.z, v.w);
@@ -109,6 +116,13 @@ __device__ __forceinline__ int2 ilt_bld8(__amdgpu_buffer_rsrc_t r, u32 off) {
 }
 __device__ __forceinline__ u32 ilt_bld4(__amdgpu_buffer_rsrc_t r, u32 off) { return __builtin_amdgcn_raw_buffer_load_b32(r, off, 0, 0); }
 __device__ __forceinline__ u16 ilt_bld2(__amdgpu_buffer_rsrc_t r, u32 off) { return __builtin_amdgcn_raw_buffer_load_b16(r, off, 0, 0); }
+__device__ __forceinline__ u8 ilt_bld1(__amdgpu_buffer_rsrc_t r, u32 off) { return __builtin_amdgcn_raw_buffer_load_b8(r, off, 0, 0); }
+
+// 16 bytes per lane from global memory straight into LDS, no register in between: lane i's
+// piece lands at lds_base + 16*i (lds_base the same in every lane).  Counted by vmcnt.
+__device__ __forceinline__ void ilt_g2lds16(const void* src, void* lds_base) {
+  __builtin_amdgcn_global_load_lds((const ILT_GLOBAL void*)src, (ILT_LDS void*)lds_base, 16, 0, 0);
+}
 
 // SBCL evaluates single-float exp and log by widening to double, calling libm and
 // rounding back (the CPU path's silu, softplus); the kernels do the same.

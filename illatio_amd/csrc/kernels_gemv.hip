@@ -233,11 +233,6 @@ template <int FMT> __device__ __forceinline__ float row_sum(const float* t, int 
   return sum;
 }
 
-__device__ __forceinline__ const void* uniform_ptr(const void* p) {   // the same in every lane: say so
-  const u64 a = (u64)p;
-  const u32 lo = __builtin_amdgcn_readfirstlane((u32)a), hi = __builtin_amdgcn_readfirstlane((u32)(a >> 32));
-  return (const void*)(((u64)hi << 32) | lo);
-}
 
 // A wave's rows [row0, row0+nrows) of one matrix: terms into t (nrows*S*TERMS floats, the wave's own).
 // No branch inside the run of full steps: the next step's loads (index clamped into the
@@ -251,8 +246,8 @@ __device__ __forceinline__ void first_load(Raw<FMT>& r, const u8* w, const u16* 
   using F = Fmt<FMT>;
   const int j = lane % F::LPB, gl = lane / F::LPB;
   const int nblk = nrows * S;
-  const __amdgpu_buffer_rsrc_t wr = ilt_rsrc(uniform_ptr(w + row0 * row_bytes), __builtin_amdgcn_readfirstlane((u32)(nrows * row_bytes)));
-  const __amdgpu_buffer_rsrc_t wdr = ilt_rsrc(uniform_ptr(wd ? wd + row0 * S : nullptr), wd ? __builtin_amdgcn_readfirstlane((u32)nblk * 2) : 0);
+  const __amdgpu_buffer_rsrc_t wr = ilt_rsrc(ilt_uniform_ptr(w + row0 * row_bytes), __builtin_amdgcn_readfirstlane((u32)(nrows * row_bytes)));
+  const __amdgpu_buffer_rsrc_t wdr = ilt_rsrc(ilt_uniform_ptr(wd ? wd + row0 * S : nullptr), wd ? __builtin_amdgcn_readfirstlane((u32)nblk * 2) : 0);
   load_raw<FMT>(r, wr, wdr, min(gl, nblk - 1), j);
 }
 
@@ -263,8 +258,8 @@ __device__ __forceinline__ void wave_rows(const u8* w, const u16* wd, long row0,
   constexpr int GPW = ILT_WAVE / F::LPB;           // blocks per wave step
   const int j = lane % F::LPB, gl = lane / F::LPB;
   const int nblk = nrows * S, last = nblk - 1;
-  const __amdgpu_buffer_rsrc_t wr = ilt_rsrc(uniform_ptr(w + row0 * row_bytes), __builtin_amdgcn_readfirstlane((u32)(nrows * row_bytes)));
-  const __amdgpu_buffer_rsrc_t wdr = ilt_rsrc(uniform_ptr(wd ? wd + row0 * S : nullptr), wd ? __builtin_amdgcn_readfirstlane((u32)nblk * 2) : 0);
+  const __amdgpu_buffer_rsrc_t wr = ilt_rsrc(ilt_uniform_ptr(w + row0 * row_bytes), __builtin_amdgcn_readfirstlane((u32)(nrows * row_bytes)));
+  const __amdgpu_buffer_rsrc_t wdr = ilt_rsrc(ilt_uniform_ptr(wd ? wd + row0 * S : nullptr), wd ? __builtin_amdgcn_readfirstlane((u32)nblk * 2) : 0);
   const int nfull = nblk / GPW;
 #define ILT_COMPUTE(reg, ff)                                                           \
   {                                                                                    \

@@ -12,7 +12,7 @@ import ctypes as C
 import numpy as np
 
 from . import hip
-from .synth import BLOCK_BYTES, BLOCK_WEIGHTS, Q4_K, Q6_K, Q8_0
+from .synth import BLOCK_BYTES, BLOCK_WEIGHTS, IQ2_XXS, Q2_K, Q4_K, Q6_K, Q8_0
 
 KQUANT_CODE = {Q4_K: 0, Q6_K: 2}      # kquant-code, cuda-dense.lisp:18-20
 
@@ -112,6 +112,16 @@ def cmat_mul(dev, w, act, y, n=1, bias=None, acc=False):
     else:
         hip.launch(dev, "mm_q8", ((n + 63) // 64, (rows + 63) // 64), 256,
                    [w.qs, w.d, act.xq, act.xs, y, bias, rows, cols, n, a])
+    return y
+
+
+def cmat_mul_bf16(dev, w, x, y, n, bias=None, acc=False):
+    """Y = W X for N tokens on the bf16 matrix cores, X a DBuf of N x COLS floats: no
+    activation quantizer runs; within 2e-2 of CMAT-MUL's result rather than equal to it."""
+    if w.type not in (Q2_K, Q4_K, Q6_K, IQ2_XXS):
+        raise ValueError(f"the bf16 product multiplies Q2_K, Q4_K, Q6_K and IQ2_XXS; {w.name} is type {w.type}")
+    hip.launch(dev, "mm_k_bf16", ((n + 127) // 128, (w.rows + 127) // 128), 256,
+               [w.type, w.qs, x, y, bias, w.rows, w.cols, n, 1 if acc else 0])
     return y
 
 

@@ -136,6 +136,44 @@ def group_rows(dev, sel, w, n, ne, nu):
     return g
 
 
+def ffn_routed_chunk_bf16(dev, pool, logits, norm2, sout, n, ne, nu, scale, clamp, bias=None, keep=None):
+    """FFN-ROUTED-CHUNK with the three grouped products on the bf16 matrix cores: the same
+    routing, grouping, gated activation and slot-ordered sum, no activation quantizers.
+    Within 2e-2 of the CPU path's chunk; the routing and grouping stay exact."""
+    d, ff = pool.d, pool.ff
+    rows = n * nu
+    gb = pool.gate_bytes
+    sel, w = route(dev, logits, n, ne, nu, scale, bias)
+    g = group_rows(dev, sel, w, n, ne, nu)
+    ptrs = hip.hip_upload_new(dev, np.array([pool.slot_ptr(e) for e in range(ne)], np.uint64))
+    x = hip.hip_alloc(dev, 4 * rows * d)
+    hip.launch(dev, "d4_gather_rows", (rows * d + 255) // 256, 256, [d, rows, norm2, g["rmap"], x])
+    gg, gu, mid = (hip.hip_alloc(dev, 4 * rows * ff) for _ in range(3))
+    down, moe = hip.hip_alloc(dev, 4 * rows * d), hip.hip_alloc(dev, 4 * n * d)
+
+    def mm_id(qtype, ncols, nrows, rb, add, xin, yout):
+        hip.launch(dev, "d4_mm_id_bf16", (rows // 128 + ne, (nrows + 127) // 128), 256,
+                   [qtype, ncols, nrows, rb, hip.I64(add), ptrs, g["counts"], g["bases"], ne, hip.I64(rows), xin, yout])
+
+    mm_id(IQ2_XXS, d, ff, pool.grb, 0, x, gg)
+    mm_id(IQ2_XXS, d, ff, pool.grb, gb, x, gu)
+    hip.launch(dev, "d4_swiglu_w", (rows * ff + 255) // 256, 256, [rows, ff, float(clamp), gg, gu, g["wrow"], mid, None, None])
+    mm_id(Q2_K, ff, d, pool.drb, 2 * gb, mid, down)
+    hip.launch(dev, "d4_moe_sum_rows", (n * d + 255) // 256, 256, [d, nu, n, down, g["smap"], sout, moe])
+    hip.hip_sync(dev)
+    if keep is not None:
+        keep["sel"] = hip.hip_download(sel, np.uint32, rows).reshape(n, nu)
+        keep["w"] = hip.hip_floats(w, rows).reshape(n, nu)
+        keep["counts"] = hip.hip_download(g["counts"], np.uint32, ne)
+        keep["bases"] = hip.hip_download(g["bases"], np.uint32, ne)
+        keep["x"], keep["mid"] = hip.hip_floats(x, rows * d).reshape(rows, d), hip.hip_floats(mid, rows * ff).reshape(rows, ff)
+        keep["gate"], keep["up"] = (hip.hip_floats(b, rows * ff).reshape(rows, ff) for b in (gg, gu))
+        keep["down"] = hip.hip_floats(down, rows * d).reshape(rows, d)
+    for b in [sel, w, ptrs, x, gg, gu, mid, down] + list(g.values()):
+        hip.hip_free(b)
+    return moe
+
+
 def ffn_routed_chunk(dev, pool, logits, norm2, sout, n, ne, nu, scale, clamp, bias=None, keep=None):
     """A chunk of N tokens past the router (DK-FFN-ROUTED-CHUNK): each token's experts and
     weights (d4_route), the (token, slot) rows grouped by expert, the rows gathered and

@@ -1,0 +1,162 @@
+"""GPU checks of the bf16 matrix-core prefill products, through the C ABI.
+
+Two kinds.  (1) One-hot activations read the dequantized matrix back through the product:
+token t = column c's unit vector gives y[t][r] = bf16(W[r][c]) with nothing else added, so
+every weight's position, scale and sign is compared exactly with the CPU dequantizer's
+value rounded to bf16.  (2) Random activations against the CPU path (quantized activations,
+integer block dots) and against a double-precision product of the dequantized weights with
+the float activations.  The tolerance of this path is 2e-2 of the largest output magnitude
+against the CPU path; against the double product the bf16 roundings alone remain, and the
+rms error must stay under 5e-3 of the rms output."""
+import numpy as np
+import pytest
+
+import oracle_lib as orc
+from illatio_amd import synth
+
+pytestmark = pytest.mark.gpu
+
+TOL_VS_CPU = 2e-2      # max |gpu - cpu| / max |cpu|
+TOL_RMS_VS_EXACT = 5e-3
+TOL_CHAIN_VS_EXACT = 3e-2   # three products and a clamped gate compounded, against the exact chain
+
+
+@pytest.fixture(scope="module")
+def dev():
+    from illatio_amd import hip
+    return hip.open_hip(0)
+
+
+def bf16_round(a):
+    """float32 -> nearest bf16 (ties to even), returned as float32."""
+    b = np.ascontiguousarray(a, np.float32).view(np.uint32).astype(np.uint64)
+    b = (b + 0x7FFF + ((b >> 16) & 1)) & 0xFFFF0000
+    return b.astype(np.uint32).view(np.float32)
+
+
+def upload(dev, qtype, rows, cols, w):
+    from illatio_amd import dense, hip
+    if qtype in (synth.Q4_K, synth.Q6_K):
+        return dense.upload_gmat(dev, "w", qtype, rows, cols, w)
+    return dense.CMat("w", qtype, rows, cols, hip.hip_upload_new(dev, w))
+
+
+FORMATS = [synth.Q4_K, synth.Q6_K, synth.Q2_K, synth.IQ2_XXS]
+
+
+@pytest.mark.parametrize("qtype", FORMATS)
+@pytest.mark.parametrize("rows,cols", [(130, 512), (64, 256)])
+def test_one_hot_tokens_read_back_the_dequantized_matrix(dev, qtype, rows, cols):
+    from illatio_amd import dense, hip
+    rng = synth.make_rng(qtype + rows)
+    w = synth.weights(qtype, rows, cols, rng)
+    x = np.eye(cols, dtype=np.float32)
+    m = upload(dev, qtype, rows, cols, w)
+    xb, y = hip.hip_upload_new(dev, x), hip.hip_alloc(dev, 4 * cols * rows)
+    dense.cmat_mul_bf16(dev, m, xb, y, cols)
+    got = hip.hip_floats(y, cols * rows).reshape(cols, rows)
+    want = bf16_round(orc.dequant_rows(qtype, w, cols).reshape(rows, cols)).T
+    # compared as numbers: a weight that dequantizes to -0.0 comes back as 0.0 + -0.0 = 0.0
+    assert np.array_equal(got, want), np.argwhere(got != want)[:8]
+    hip.hip_free(xb); hip.hip_free(y); m.free()
+
+
+@pytest.mark.parametrize("qtype,rows,cols,n", [
+    (synth.Q6_K, 640, 5120, 200),        # BASELINE config 3's format and width, fewer rows, ragged tokens
+    (synth.Q6_K, 1000, 1024, 128),
+    (synth.Q4_K, 1024, 2560, 77),
+    (synth.Q2_K, 300, 2048, 129),
+    (synth.IQ2_XXS, 256, 4096, 64),
+])
+def test_dense_bf16_product_within_tolerance(dev, qtype, rows, cols, n):
+    from illatio_amd import dense, hip
+    rng = synth.make_rng(qtype * 7 + rows + n)
+    w = synth.weights(qtype, rows, cols, rng)
+    x = synth.activations((n, cols), rng)
+    bias = synth.activations(rows, rng)
+    m = upload(dev, qtype, rows, cols, w)
+    xb, bb, y = hip.hip_upload_new(dev, x), hip.hip_upload_new(dev, bias), hip.hip_alloc(dev, 4 * n * rows)
+    dense.cmat_mul_bf16(dev, m, xb, y, n)
+    got = hip.hip_floats(y, n * rows).reshape(n, rows)
+    cpu = orc.matmul(qtype, w, rows, cols, x, nthreads=8)
+    exact = x.astype(np.float64) @ orc.dequant_rows(qtype, w, cols).reshape(rows, cols).astype(np.float64).T
+    assert np.abs(got - cpu).max() <= TOL_VS_CPU * np.abs(cpu).max()
+    assert np.sqrt(np.mean((got - exact) ** 2)) <= TOL_RMS_VS_EXACT * np.sqrt(np.mean(exact ** 2))
+    # accumulate + bias: y += W x + bias
+    dense.cmat_mul_bf16(dev, m, xb, y, n, bias=bb, acc=True)
+    got2 = hip.hip_floats(y, n * rows).reshape(n, rows)
+    assert np.array_equal(got2, got + (got + bias[None, :]))
+    for b in (xb, bb, y):
+        hip.hip_free(b)
+    m.free()
+
+
+def exact_chunk(G, U, Dn, sel, ww, norms, clamp):
+    """The routed experts of a chunk in double precision from the dequantized weights and
+    the float activations (no activation quantization, no bf16): what both paths approximate."""
+    n, nu = sel.shape
+    out = np.zeros((n, Dn.shape[1]))
+    for t in range(n):
+        x = norms[t].astype(np.float64)
+        for s in range(nu):
+            e = int(sel[t, s])
+            g, u = G[e] @ x, U[e] @ x
+            if clamp > 0:
+                g, u = np.minimum(g, clamp), np.clip(u, -clamp, clamp)
+            out[t] += Dn[e] @ ((g / (1 + np.exp(-g))) * u * float(ww[t, s]))
+    return out
+
+
+@pytest.mark.parametrize("ne,d,ff,nu,n,clamp", [(8, 512, 256, 3, 37, 0.0), (16, 1024, 512, 4, 300, 0.6),
+                                                 (12, 4096, 2048, 6, 96, 0.0)])
+def test_moe_prefill_chunk_bf16_within_tolerance(dev, ne, d, ff, nu, n, clamp):
+    """The prefill chunk of test_gpu_gemm.py with the three grouped products on the bf16
+    matrix cores.  Routing, counts and weights stay equal to the CPU path's.  Each grouped
+    product is within 2e-2 of the CPU product (quantized activations, integer block dots)
+    of the same input rows.  Over the whole chain the CPU path's own activation quantization
+    is the larger error (2-7% of the largest output at these shapes, against an exact
+    double-precision chain), so the chain is held to this: the bf16 chunk is no farther
+    from the exact chain than the CPU path's chunk is."""
+    from illatio_amd import ds4f, hip
+    rng = synth.make_rng(ne + d + n)
+    gate = synth.weights(synth.IQ2_XXS, ne * ff, d, rng)
+    up = synth.weights(synth.IQ2_XXS, ne * ff, d, rng)
+    down = synth.weights(synth.Q2_K, ne * d, ff, rng)
+    norms = synth.activations((n, d), rng)
+    logits = synth.zipf_router_logits(n, ne, rng)
+    shared = synth.activations((n, d), rng)
+    want, wsel, ww, wcounts = orc.moe_chunk(gate, up, down, d, ff, ne, nu, 1.5, clamp, logits, norms, shared, nthreads=8)
+    pool = ds4f.ExpertPool(dev, ne, d, ff, gate, up, down)
+    lb, nb, sb = (hip.hip_upload_new(dev, a) for a in (logits, norms, shared))
+    keep = {}
+    moe = ds4f.ffn_routed_chunk_bf16(dev, pool, lb, nb, sb, n, ne, nu, 1.5, clamp, keep=keep)
+    assert np.array_equal(keep["sel"], wsel.astype(np.uint32))
+    assert np.array_equal(keep["w"].view(np.uint32), np.ascontiguousarray(ww, np.float32).view(np.uint32))
+    assert np.array_equal(keep["counts"], wcounts.astype(np.uint32))
+    got = hip.hip_floats(moe, n * d).reshape(n, d)
+
+    # every expert's three products against the CPU product of the same rows
+    grb, drb = synth.row_bytes(synth.IQ2_XXS, d), synth.row_bytes(synth.Q2_K, ff)
+    gate_e, up_e, down_e = gate.reshape(ne, ff * grb), up.reshape(ne, ff * grb), down.reshape(ne, d * drb)
+    cpu = {k: np.zeros_like(keep[k]) for k in ("gate", "up", "down")}
+    for e in range(ne):
+        b, c = int(keep["bases"][e]), int(keep["counts"][e])
+        if c == 0:
+            continue
+        cpu["gate"][b:b + c] = orc.matmul(synth.IQ2_XXS, gate_e[e], ff, d, keep["x"][b:b + c], nthreads=8)
+        cpu["up"][b:b + c] = orc.matmul(synth.IQ2_XXS, up_e[e], ff, d, keep["x"][b:b + c], nthreads=8)
+        cpu["down"][b:b + c] = orc.matmul(synth.Q2_K, down_e[e], d, ff, keep["mid"][b:b + c], nthreads=8)
+    for k in ("gate", "up", "down"):
+        assert np.abs(keep[k] - cpu[k]).max() <= TOL_VS_CPU * np.abs(cpu[k]).max(), k
+
+    # the chain against the exact one
+    G = orc.dequant_rows(synth.IQ2_XXS, gate, d).reshape(ne, ff, d).astype(np.float64)
+    U = orc.dequant_rows(synth.IQ2_XXS, up, d).reshape(ne, ff, d).astype(np.float64)
+    Dn = orc.dequant_rows(synth.Q2_K, down, ff).reshape(ne, d, ff).astype(np.float64)
+    exact = exact_chunk(G, U, Dn, wsel, ww, norms, clamp) + shared
+    err_gpu, err_cpu = np.abs(got - exact).max(), np.abs(want - exact).max()
+    assert err_gpu <= err_cpu, (err_gpu, err_cpu)
+    assert err_gpu <= TOL_CHAIN_VS_EXACT * np.abs(exact - shared).max(), (err_gpu, np.abs(exact - shared).max())
+    for b in (lb, nb, sb, moe):
+        hip.hip_free(b)
+    pool.free()
