@@ -389,27 +389,34 @@ int ilt_d4_mm_id_q2_k(uint64_t stream, int ncols, int nrows, int row_bytes, int6
 
 static int bf16_type(int t) { return (t == ILT_Q2_K || t == ILT_Q4_K || t == ILT_Q6_K || t == ILT_IQ2_XXS) ? t : 0; }
 
-int ilt_mm_k_bf16(uint64_t stream, int gguf_type, const void* w, const float* x, float* y, const float* bias,
+int ilt_cvt_bf16(uint64_t stream, const float* x, uint16_t* xb, int64_t n) {
+  ILT_REQUIRE(n >= 0 && n % 8 == 0);
+  if (n == 0) return ILT_OK;
+  ILT_REQUIRE(x && xb && ((uintptr_t)x & 15) == 0 && ((uintptr_t)xb & 15) == 0);
+  return (int)ilt_k_cvt_bf16(x, xb, n, S(stream));
+}
+
+int ilt_mm_k_bf16(uint64_t stream, int gguf_type, const void* w, const uint16_t* xb, float* y, const float* bias,
                   int rows, int cols, int n, int acc) {
   const int fmt = bf16_type(gguf_type);
   ILT_REQUIRE(fmt && rows >= 0 && n >= 0 && cols > 0 && cols % 256 == 0);
   if (rows == 0 || n == 0) return ILT_OK;
   const long long row_bytes = (long long)cols / 256 * block_bytes(fmt);
-  ILT_REQUIRE(w && x && y && ((uintptr_t)w & 1) == 0 && ((uintptr_t)x & 15) == 0);
-  ILT_REQUIRE(row_bytes * rows < 0xFFFFFFF0LL && 4LL * cols * 128 < 0xFFFFFFF0LL);
-  return (int)ilt_k_gemm_bf16(fmt, (const uint8_t*)w, row_bytes, rows, cols, x, n, y, bias, acc, S(stream));
+  ILT_REQUIRE(w && xb && y && ((uintptr_t)w & 1) == 0 && ((uintptr_t)xb & 15) == 0);
+  ILT_REQUIRE(row_bytes * rows < 0xFFFFFFF0LL);
+  return (int)ilt_k_gemm_bf16(fmt, (const uint8_t*)w, row_bytes, rows, cols, xb, n, y, bias, acc, S(stream));
 }
 
 int ilt_d4_mm_id_bf16(uint64_t stream, int gguf_type, int ncols, int nrows, int row_bytes, int64_t add, const uint64_t* ptrs,
                       const uint32_t* counts, const uint32_t* bases, int ne, int64_t total_rows,
-                      const float* x, float* y) {
+                      const uint16_t* xb, float* y) {
   const int fmt = bf16_type(gguf_type);
   ILT_REQUIRE(fmt && ncols > 0 && ncols % 256 == 0 && nrows >= 0 && ne >= 0 && ne <= 256 && total_rows >= 0);
   ILT_REQUIRE(row_bytes == ncols / 256 * block_bytes(fmt) && add >= 0 && (add & 1) == 0);
   if (nrows == 0 || ne == 0 || total_rows == 0) return ILT_OK;
-  ILT_REQUIRE(ptrs && counts && bases && x && y && ((uintptr_t)x & 15) == 0 && total_rows < (1LL << 31));
-  ILT_REQUIRE((long long)row_bytes * nrows < 0xFFFFFFF0LL && 4LL * ncols * 128 < 0xFFFFFFF0LL);
-  return (int)ilt_k_gemm_bf16_id(fmt, ptrs, add, counts, bases, ne, row_bytes, nrows, ncols, x, total_rows, y, S(stream));
+  ILT_REQUIRE(ptrs && counts && bases && xb && y && ((uintptr_t)xb & 15) == 0 && total_rows < (1LL << 31));
+  ILT_REQUIRE((long long)row_bytes * nrows < 0xFFFFFFF0LL);
+  return (int)ilt_k_gemm_bf16_id(fmt, ptrs, add, counts, bases, ne, row_bytes, nrows, ncols, xb, total_rows, y, S(stream));
 }
 
 // ---- launch by name ---------------------------------------------------------------------------
@@ -441,11 +448,12 @@ int ilt_launch(const char* kernel, unsigned gx, unsigned gy, unsigned gz, unsign
   if (!strcmp(kernel, "mm_q4k_mma") || !strcmp(kernel, "mm_q6k_mma"))
     return ilt_mm_k(stream, kernel[4] == '4' ? 0 : 2, a.ptr<const void*>(0), a.ptr<ci8>(1), a.ptr<cf>(2),
                     a.ptr<const int32_t*>(3), a.ptr<float*>(4), a.ptr<cf>(5), a.i32(6), a.i32(7), a.i32(8), a.i32(9));
-  K("mm_k_bf16") return ilt_mm_k_bf16(stream, a.i32(0), a.ptr<const void*>(1), a.ptr<cf>(2), a.ptr<float*>(3), a.ptr<cf>(4),
+  K("cvt_bf16") return ilt_cvt_bf16(stream, a.ptr<cf>(0), a.ptr<uint16_t*>(1), a.i64(2));
+  K("mm_k_bf16") return ilt_mm_k_bf16(stream, a.i32(0), a.ptr<const void*>(1), a.ptr<cu16>(2), a.ptr<float*>(3), a.ptr<cf>(4),
                                       a.i32(5), a.i32(6), a.i32(7), a.i32(8));
   K("d4_mm_id_bf16")
     return ilt_d4_mm_id_bf16(stream, a.i32(0), a.i32(1), a.i32(2), a.i32(3), a.i64(4), a.ptr<const uint64_t*>(5), a.ptr<cu32>(6),
-                             a.ptr<cu32>(7), a.i32(8), a.i64(9), a.ptr<cf>(10), a.ptr<float*>(11));
+                             a.ptr<cu32>(7), a.i32(8), a.i64(9), a.ptr<cu16>(10), a.ptr<float*>(11));
   K("d4_mm_id_iq2_xxs")
     return ilt_d4_mm_id_iq2_xxs(stream, a.i32(0), a.i32(1), a.i32(2), a.i64(5), a.ptr<const uint64_t*>(6), a.ptr<cu32>(7),
                                 a.ptr<cu32>(8), (int)gz, a.i64(13), a.ptr<ci8>(9), a.ptr<cf>(11), a.ptr<float*>(10));

@@ -81,12 +81,14 @@ hipError_t ilt_k_gemm_i8_id(int fmt, const uint64_t* ptrs, long long add, const 
                             int ne, long long row_bytes, int rows, int cols, const int8_t* xq, const float* xs,
                             const int* bsums, long long total_rows, float* y, hipStream_t st);
 
-// bf16 matrix-core products on float activations (weights dequantized to bf16 in LDS);
-// Q4_K, Q6_K (212-byte device blocks), Q2_K, IQ2_XXS.  Within 2e-2 of the CPU path.
-hipError_t ilt_k_gemm_bf16(int fmt, const uint8_t* w, long long row_bytes, int rows, int cols, const float* x, int ntok,
+// bf16 matrix-core products on bf16 activations (ilt_k_cvt_bf16 rounds floats, n a multiple
+// of 8); weights dequantized to bf16 in LDS: Q4_K, Q6_K (212-byte device blocks), Q2_K,
+// IQ2_XXS.  Within 2e-2 of the CPU path.
+hipError_t ilt_k_cvt_bf16(const float* x, uint16_t* xb, long long n, hipStream_t st);
+hipError_t ilt_k_gemm_bf16(int fmt, const uint8_t* w, long long row_bytes, int rows, int cols, const uint16_t* xb, int ntok,
                            float* y, const float* bias, int acc, hipStream_t st);
 hipError_t ilt_k_gemm_bf16_id(int fmt, const uint64_t* ptrs, long long add, const uint32_t* counts, const uint32_t* bases,
-                              int ne, long long row_bytes, int rows, int cols, const float* x, long long total_rows,
+                              int ne, long long row_bytes, int rows, int cols, const uint16_t* xb, long long total_rows,
                               float* y, hipStream_t st);
 
 #endif  // ILT_KERNELS_H

@@ -115,13 +115,21 @@ def cmat_mul(dev, w, act, y, n=1, bias=None, acc=False):
     return y
 
 
-def cmat_mul_bf16(dev, w, x, y, n, bias=None, acc=False):
-    """Y = W X for N tokens on the bf16 matrix cores, X a DBuf of N x COLS floats: no
-    activation quantizer runs; within 2e-2 of CMAT-MUL's result rather than equal to it."""
+def cvt_bf16(dev, x, n_elems, out=None):
+    """N_ELEMS floats of X (a DBuf) rounded to bf16, into OUT or a new DBuf: the bf16
+    product's counterpart of QUANTIZE-ACT!."""
+    out = out if out is not None else hip.hip_alloc(dev, 2 * n_elems, zero=False)
+    hip.launch(dev, "cvt_bf16", (n_elems // 8 + 255) // 256, 256, [x, out, hip.I64(n_elems)])
+    return out
+
+
+def cmat_mul_bf16(dev, w, xb, y, n, bias=None, acc=False):
+    """Y = W X for N tokens on the bf16 matrix cores, XB a DBuf of N x COLS bf16 (CVT-BF16):
+    no activation quantizer runs; within 2e-2 of CMAT-MUL's result rather than equal to it."""
     if w.type not in (Q2_K, Q4_K, Q6_K, IQ2_XXS):
         raise ValueError(f"the bf16 product multiplies Q2_K, Q4_K, Q6_K and IQ2_XXS; {w.name} is type {w.type}")
     hip.launch(dev, "mm_k_bf16", ((n + 127) // 128, (w.rows + 127) // 128), 256,
-               [w.type, w.qs, x, y, bias, w.rows, w.cols, n, 1 if acc else 0])
+               [w.type, w.qs, xb, y, bias, w.rows, w.cols, n, 1 if acc else 0])
     return y
 
 

@@ -13,7 +13,7 @@ D4-SHARED!, :1039-1048), not left as floats as its CUDA kernels take them.
 """
 import numpy as np
 
-from . import hip
+from . import dense, hip
 from .synth import IQ2_XXS, Q2_K, Q8_0, row_bytes
 
 
@@ -148,6 +148,7 @@ def ffn_routed_chunk_bf16(dev, pool, logits, norm2, sout, n, ne, nu, scale, clam
     ptrs = hip.hip_upload_new(dev, np.array([pool.slot_ptr(e) for e in range(ne)], np.uint64))
     x = hip.hip_alloc(dev, 4 * rows * d)
     hip.launch(dev, "d4_gather_rows", (rows * d + 255) // 256, 256, [d, rows, norm2, g["rmap"], x])
+    xb = dense.cvt_bf16(dev, x, rows * d)
     gg, gu, mid = (hip.hip_alloc(dev, 4 * rows * ff) for _ in range(3))
     down, moe = hip.hip_alloc(dev, 4 * rows * d), hip.hip_alloc(dev, 4 * n * d)
 
@@ -155,10 +156,11 @@ def ffn_routed_chunk_bf16(dev, pool, logits, norm2, sout, n, ne, nu, scale, clam
         hip.launch(dev, "d4_mm_id_bf16", (rows // 128 + ne, (nrows + 127) // 128), 256,
                    [qtype, ncols, nrows, rb, hip.I64(add), ptrs, g["counts"], g["bases"], ne, hip.I64(rows), xin, yout])
 
-    mm_id(IQ2_XXS, d, ff, pool.grb, 0, x, gg)
-    mm_id(IQ2_XXS, d, ff, pool.grb, gb, x, gu)
+    mm_id(IQ2_XXS, d, ff, pool.grb, 0, xb, gg)
+    mm_id(IQ2_XXS, d, ff, pool.grb, gb, xb, gu)
     hip.launch(dev, "d4_swiglu_w", (rows * ff + 255) // 256, 256, [rows, ff, float(clamp), gg, gu, g["wrow"], mid, None, None])
-    mm_id(Q2_K, ff, d, pool.drb, 2 * gb, mid, down)
+    mb = dense.cvt_bf16(dev, mid, rows * ff)
+    mm_id(Q2_K, ff, d, pool.drb, 2 * gb, mb, down)
     hip.launch(dev, "d4_moe_sum_rows", (n * d + 255) // 256, 256, [d, nu, n, down, g["smap"], sout, moe])
     hip.hip_sync(dev)
     if keep is not None:
@@ -169,7 +171,7 @@ def ffn_routed_chunk_bf16(dev, pool, logits, norm2, sout, n, ne, nu, scale, clam
         keep["x"], keep["mid"] = hip.hip_floats(x, rows * d).reshape(rows, d), hip.hip_floats(mid, rows * ff).reshape(rows, ff)
         keep["gate"], keep["up"] = (hip.hip_floats(b, rows * ff).reshape(rows, ff) for b in (gg, gu))
         keep["down"] = hip.hip_floats(down, rows * d).reshape(rows, d)
-    for b in [sel, w, ptrs, x, gg, gu, mid, down] + list(g.values()):
+    for b in [sel, w, ptrs, x, xb, mb, gg, gu, mid, down] + list(g.values()):
         hip.hip_free(b)
     return moe
 

@@ -207,21 +207,24 @@ int ilt_d4_mm_id_q2_k(uint64_t stream, int ncols, int nrows, int row_bytes, int6
                       const uint32_t* counts, const uint32_t* bases, int ne, int64_t total_rows,
                       const int8_t* xq, const float* xd, const int32_t* bsums, float* y);
 
-/* The same products on the bf16 matrix cores, from float activations: W is dequantized to
-   bf16 value by value as the CPU's *-row-floats! do (kquant.lisp:466-497 Q4_K, :530-569
-   Q6_K, :411-445 Q2_K; iquant.lisp:161-230 IQ2_XXS) and x rounded to bf16, with fp32
-   accumulation.  No activation quantizer runs, so this is the faster prefill path; its
-   results are within 2e-2 (relative to the largest output) of the CPU path, not bit-exact.
+/* The same products on the bf16 matrix cores: W is dequantized to bf16 value by value as the
+   CPU's *-row-floats! do (kquant.lisp:466-497 Q4_K, :530-569 Q6_K, :411-445 Q2_K;
+   iquant.lisp:161-230 IQ2_XXS), the activations are floats rounded to bf16 by cvt_bf16
+   (in place of an activation quantizer), the accumulation is fp32.  This is the faster
+   prefill path; its results are within 2e-2 (relative to the largest output) of the CPU
+   path, not bit-exact.
+   cvt_bf16: n floats (a multiple of 8, 16-byte aligned) to n bf16.
    mm_k_bf16: gguf_type 10 Q2_K, 12 Q4_K, 14 Q6_K (212-byte device blocks of
-     ilt_repack_q6k), 16 IQ2_XXS; x is n tokens of cols floats, 16-byte aligned;
+     ilt_repack_q6k), 16 IQ2_XXS; xb is n tokens of cols bf16, 16-byte aligned;
      y[t*rows + r] (+= when acc, + bias[r]).  The matrix is at most 4 GiB.
-   d4_mm_id_bf16: the grouped expert product of ds4f_mm.cu:256-257 on the gathered float
-     rows x (ncols apart), same gguf_type codes, other arguments as d4_mm_id_*. */
-int ilt_mm_k_bf16(uint64_t stream, int gguf_type, const void* w, const float* x, float* y, const float* bias,
+   d4_mm_id_bf16: the grouped expert product of ds4f_mm.cu:256-257 on the gathered rows
+     xb (bf16, ncols apart), same gguf_type codes, other arguments as d4_mm_id_*. */
+int ilt_cvt_bf16(uint64_t stream, const float* x, uint16_t* xb, int64_t n);
+int ilt_mm_k_bf16(uint64_t stream, int gguf_type, const void* w, const uint16_t* xb, float* y, const float* bias,
                   int rows, int cols, int n, int acc);
 int ilt_d4_mm_id_bf16(uint64_t stream, int gguf_type, int ncols, int nrows, int row_bytes, int64_t add, const uint64_t* ptrs,
                       const uint32_t* counts, const uint32_t* bases, int ne, int64_t total_rows,
-                      const float* x, float* y);
+                      const uint16_t* xb, float* y);
 
 /* ---- 3. launch by name (src/cuda.lisp:323-352) -------------------------------------------
  * params[i] points at argument i's 8-byte slot: a pointer as 64 bits, an int in the low

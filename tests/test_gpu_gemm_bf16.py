@@ -52,13 +52,14 @@ def test_one_hot_tokens_read_back_the_dequantized_matrix(dev, qtype, rows, cols)
     w = synth.weights(qtype, rows, cols, rng)
     x = np.eye(cols, dtype=np.float32)
     m = upload(dev, qtype, rows, cols, w)
-    xb, y = hip.hip_upload_new(dev, x), hip.hip_alloc(dev, 4 * cols * rows)
+    xf, y = hip.hip_upload_new(dev, x), hip.hip_alloc(dev, 4 * cols * rows)
+    xb = dense.cvt_bf16(dev, xf, x.size)
     dense.cmat_mul_bf16(dev, m, xb, y, cols)
     got = hip.hip_floats(y, cols * rows).reshape(cols, rows)
     want = bf16_round(orc.dequant_rows(qtype, w, cols).reshape(rows, cols)).T
     # compared as numbers: a weight that dequantizes to -0.0 comes back as 0.0 + -0.0 = 0.0
     assert np.array_equal(got, want), np.argwhere(got != want)[:8]
-    hip.hip_free(xb); hip.hip_free(y); m.free()
+    hip.hip_free(xf); hip.hip_free(xb); hip.hip_free(y); m.free()
 
 
 @pytest.mark.parametrize("qtype,rows,cols,n", [
@@ -67,6 +68,10 @@ def test_one_hot_tokens_read_back_the_dequantized_matrix(dev, qtype, rows, cols)
     (synth.Q4_K, 1024, 2560, 77),
     (synth.Q2_K, 300, 2048, 129),
     (synth.IQ2_XXS, 256, 4096, 64),
+    (synth.Q6_K, 8200, 512, 4000),       # 1024 tiles and more: the 256-token tile runs; ragged both ways
+    (synth.Q4_K, 8200, 256, 4100),
+    (synth.Q2_K, 8200, 256, 4100),
+    (synth.IQ2_XXS, 8200, 256, 4100),
 ])
 def test_dense_bf16_product_within_tolerance(dev, qtype, rows, cols, n):
     from illatio_amd import dense, hip
@@ -75,10 +80,12 @@ def test_dense_bf16_product_within_tolerance(dev, qtype, rows, cols, n):
     x = synth.activations((n, cols), rng)
     bias = synth.activations(rows, rng)
     m = upload(dev, qtype, rows, cols, w)
-    xb, bb, y = hip.hip_upload_new(dev, x), hip.hip_upload_new(dev, bias), hip.hip_alloc(dev, 4 * n * rows)
+    xf, bb, y = hip.hip_upload_new(dev, x), hip.hip_upload_new(dev, bias), hip.hip_alloc(dev, 4 * n * rows)
+    xb = dense.cvt_bf16(dev, xf, x.size)
+    assert np.array_equal(hip.hip_download(xb, np.uint16, x.size), (bf16_round(x).view(np.uint32) >> 16).astype(np.uint16).ravel())
     dense.cmat_mul_bf16(dev, m, xb, y, n)
     got = hip.hip_floats(y, n * rows).reshape(n, rows)
-    cpu = orc.matmul(qtype, w, rows, cols, x, nthreads=8)
+    cpu = orc.matmul(qtype, w, rows, cols, x, nthreads=16)
     exact = x.astype(np.float64) @ orc.dequant_rows(qtype, w, cols).reshape(rows, cols).astype(np.float64).T
     assert np.abs(got - cpu).max() <= TOL_VS_CPU * np.abs(cpu).max()
     assert np.sqrt(np.mean((got - exact) ** 2)) <= TOL_RMS_VS_EXACT * np.sqrt(np.mean(exact ** 2))
@@ -86,7 +93,7 @@ def test_dense_bf16_product_within_tolerance(dev, qtype, rows, cols, n):
     dense.cmat_mul_bf16(dev, m, xb, y, n, bias=bb, acc=True)
     got2 = hip.hip_floats(y, n * rows).reshape(n, rows)
     assert np.array_equal(got2, got + (got + bias[None, :]))
-    for b in (xb, bb, y):
+    for b in (xf, xb, bb, y):
         hip.hip_free(b)
     m.free()
 
