@@ -6,27 +6,31 @@
 // kernels_gemm.hip).  Each weight is dequantized exactly as the reference's
 // *-row-floats! / kmat-row! do (kquant.lisp:466-497, iquant.lisp:161-230) before rounding.
 //
-// A workgroup (256 threads, 4 waves) computes 128 rows x TN tokens (TN 256, or 128 for few
-// tokens and for the expert groups) in steps of 32 columns:
+// A workgroup of 2*TM threads computes TM rows x TN tokens (256x256, 128x256 or 128x128,
+// the larger the tile the less is fetched and dequantized per product; the smaller ones for
+// few tokens and for the expert groups) in steps of 32 columns:
 //   - the activations' 32-column slab goes from global memory straight into LDS
 //     (global_load_lds_dwordx4), two steps ahead, into a ring of three slabs;
-//   - every thread holds the raw bytes of 16 weights of one row one step ahead in registers,
-//     dequantizes them and writes them as bf16 into one of two weight slabs;
-//   - one barrier per step; then wave w multiplies rows 64*(w/2).. by tokens (TN/2)*(w%2)..
+//   - thread (row, e) dequantizes columns 16e..16e+15 of its row in every step.  It holds
+//     the raw bytes of half a super-block (four steps) of its row in registers, in two sets
+//     loaded four steps before first use; it dequantizes the next step's weights and writes
+//     them as bf16 into one of two weight slabs while the current step's MFMAs run;
+//   - one barrier per step; wave w multiplies rows 64*(w/2).. by tokens (TN/2)*(w%2)..
 //     as patches of 32x32.  The MFMA's M side is the tokens and its N side the rows, so a
 //     lane's 16 results of a patch are one row for 16 tokens and a store instruction writes
 //     32 consecutive rows of a token.
-// Both kinds of slab hold 64 bytes per row as four 16-byte pieces, piece p of row r at
-// 4*r + (p ^ ((r>>2)&3)): rows 0..15 of one piece index cover all 64 banks once, with no
-// padding (the direct loads write 1 KB per wave instruction contiguously, so the swizzle
-// is applied by choosing which global piece each lane fetches).
-// Two workgroups share a CU, so one's dequantization overlaps the other's MFMAs.
+// Both kinds of slab hold 64 bytes per row as four 16-byte pieces, unpadded and swizzled
+// (slab_off): the direct loads write 1 KB per wave instruction contiguously, so the swizzle
+// is applied by choosing which global piece each lane fetches.
 // Tiles are numbered so that the workgroups resident on one XCD (every eighth workgroup id)
-// form a block of 8 row tiles x 8 token tiles and share W and x slabs through that XCD's L2.
-// The grouped expert product (d4_mm_id_*) walks the token tiles of every expert's rows in turn.
+// form a block of 8 row tiles x several token tiles and share W and x slabs through that
+// XCD's L2.  The grouped expert product (d4_mm_id_*) walks the token tiles of every
+// expert's rows in turn.
 #include "ilt_device.h"
 #include "ilt_iq2xxs_tables.h"
 #include "ilt_kernels.h"
+#include <stdlib.h>
+#include <type_traits>
 
 namespace {
 
@@ -35,9 +39,8 @@ typedef __bf16 v2bf __attribute__((ext_vector_type(2)));
 typedef float v16f __attribute__((ext_vector_type(16)));
 typedef float v2f __attribute__((ext_vector_type(2)));
 
-constexpr int TM = 128, KS = 32;       // rows per tile, columns per step
+constexpr int KS = 32;                 // columns per step
 constexpr int GR = 8;                  // row tiles per block of tiles sharing an L2
-constexpr int WSLAB = TM * KS * 2;     // bytes of a weight slab
 
 __device__ const u64 bf_grid_dev[256] = { ILT_IQ2XXS_GRID_VALUES };
 
@@ -47,86 +50,94 @@ __device__ __forceinline__ u32 pack_bf16(float a, float b) {
   u32 u; __builtin_memcpy(&u, &r, 4); return u;
 }
 
-// The raw bytes of a thread's 16 weights (row = t/2, columns 16*(t%2).. of the step's 32).
+// The raw bytes a thread needs for four steps (half a super-block, 128 columns) of its row:
+// thread (row, e) dequantizes columns 16e..16e+15 of every 32-column step.  Loaded once per
+// four steps, so that a load instruction's 32 rows fetch 32 bytes each rather than 16 or 2.
 template <int FMT> struct WRaw;
-template <> struct WRaw<ILT_Q4_K> { int4 hdr, q; };
-template <> struct WRaw<ILT_Q6_K> { int4 ql, qh; u32 sc, d; };
-template <> struct WRaw<ILT_Q2_K> { int4 q; u32 sc, dd; };
-template <> struct WRaw<ILT_IQ2_XXS> { int2 q; u32 d; };
+template <> struct WRaw<ILT_Q4_K> { int4 hdr, q[2]; static constexpr int LOADS = 3; };
+template <> struct WRaw<ILT_Q6_K> { int4 ql[2], qh; int2 sc; u32 d; static constexpr int LOADS = 5; };
+template <> struct WRaw<ILT_Q2_K> { int4 q; int2 sc; u32 dd; static constexpr int LOADS = 3; };
+template <> struct WRaw<ILT_IQ2_XXS> { int4 q[2]; u32 d; static constexpr int LOADS = 3; };
 
-template <int FMT> __device__ __forceinline__ void load_w(WRaw<FMT>& r, __amdgpu_buffer_rsrc_t rw, u32 rowoff, int ks, int e);
+// hb: the half super-block (hb>>1 the super-block, c = hb&1 its half)
+template <int FMT> __device__ __forceinline__ void load_w(WRaw<FMT>& r, __amdgpu_buffer_rsrc_t rw, u32 rowoff, int hb, int e);
 
-template <> __device__ __forceinline__ void load_w<ILT_Q4_K>(WRaw<ILT_Q4_K>& r, __amdgpu_buffer_rsrc_t rw, u32 rowoff, int ks, int e) {
-  const u32 b = rowoff + (u32)(ks >> 3) * 144;
+template <> __device__ __forceinline__ void load_w<ILT_Q4_K>(WRaw<ILT_Q4_K>& r, __amdgpu_buffer_rsrc_t rw, u32 rowoff, int hb, int e) {
+  const u32 b = rowoff + (u32)(hb >> 1) * 144;
   r.hdr = ilt_bld16(rw, b);
-  r.q = ilt_bld16(rw, b + 16 + 32 * ((ks >> 1) & 3) + 16 * e);
+  r.q[0] = ilt_bld16(rw, b + 16 + 64 * (hb & 1) + 16 * e);
+  r.q[1] = ilt_bld16(rw, b + 48 + 64 * (hb & 1) + 16 * e);
 }
-template <> __device__ __forceinline__ void load_w<ILT_Q6_K>(WRaw<ILT_Q6_K>& r, __amdgpu_buffer_rsrc_t rw, u32 rowoff, int ks, int e) {
-  const u32 b = rowoff + (u32)(ks >> 3) * ILT_Q6K_STRIDE;
-  const int c = (ks >> 2) & 1, part = ks & 3;
-  r.ql = ilt_bld16(rw, b + 64 * c + 32 * (part & 1) + 16 * e);
+template <> __device__ __forceinline__ void load_w<ILT_Q6_K>(WRaw<ILT_Q6_K>& r, __amdgpu_buffer_rsrc_t rw, u32 rowoff, int hb, int e) {
+  const u32 b = rowoff + (u32)(hb >> 1) * ILT_Q6K_STRIDE;
+  const int c = hb & 1;
+  r.ql[0] = ilt_bld16(rw, b + 64 * c + 16 * e);
+  r.ql[1] = ilt_bld16(rw, b + 64 * c + 32 + 16 * e);
   r.qh = ilt_bld16(rw, b + 128 + 32 * c + 16 * e);
-  r.sc = ilt_bld1(rw, b + 192 + 8 * c + 2 * part + e);
+  r.sc = ilt_bld8(rw, b + 192 + 8 * c);
   r.d = ilt_bld2(rw, b + 208);
 }
-template <> __device__ __forceinline__ void load_w<ILT_Q2_K>(WRaw<ILT_Q2_K>& r, __amdgpu_buffer_rsrc_t rw, u32 rowoff, int ks, int e) {
-  const u32 b = rowoff + (u32)(ks >> 3) * 84;
-  const int h = (ks >> 2) & 1, j = ks & 3;
-  r.q = ilt_bld16(rw, b + 16 + 32 * h + 16 * e);
-  r.sc = ilt_bld1(rw, b + 8 * h + 2 * j + e);
+template <> __device__ __forceinline__ void load_w<ILT_Q2_K>(WRaw<ILT_Q2_K>& r, __amdgpu_buffer_rsrc_t rw, u32 rowoff, int hb, int e) {
+  const u32 b = rowoff + (u32)(hb >> 1) * 84;
+  r.q = ilt_bld16(rw, b + 16 + 32 * (hb & 1) + 16 * e);
+  r.sc = ilt_bld8(rw, b + 8 * (hb & 1));
   r.dd = ilt_bld4(rw, b + 80);
 }
-template <> __device__ __forceinline__ void load_w<ILT_IQ2_XXS>(WRaw<ILT_IQ2_XXS>& r, __amdgpu_buffer_rsrc_t rw, u32 rowoff, int ks, int e) {
-  const u32 b = rowoff + (u32)(ks >> 3) * 66;
-  r.q = ilt_bld8(rw, b + 2 + 8 * (ks & 7));
+template <> __device__ __forceinline__ void load_w<ILT_IQ2_XXS>(WRaw<ILT_IQ2_XXS>& r, __amdgpu_buffer_rsrc_t rw, u32 rowoff, int hb, int e) {
+  const u32 b = rowoff + (u32)(hb >> 1) * 66;
+  r.q[0] = ilt_bld16(rw, b + 2 + 32 * (hb & 1));
+  r.q[1] = ilt_bld16(rw, b + 18 + 32 * (hb & 1));
   r.d = ilt_bld2(rw, b);
 }
 
-// 16 weights as floats, in column order, each computed as the CPU dequantizers compute it.
-template <int FMT> __device__ __forceinline__ void dequant16(const WRaw<FMT>& r, int ks, int e, const u64* grid, float* o);
+__device__ __forceinline__ u32 word_of(const int4& v, int i) { return (u32)(i == 0 ? v.x : i == 1 ? v.y : i == 2 ? v.z : v.w); }
 
-template <> __device__ __forceinline__ void dequant16<ILT_Q4_K>(const WRaw<ILT_Q4_K>& r, int ks, int e, const u64*, float* o) {
-  const int g = ks & 7, sh = 8 * (g & 3), hl = ks & 1;
+// 16 weights as floats, in column order, each computed as the CPU dequantizers compute it.
+// j: the step within the half super-block (a constant after unrolling); c: which half.
+template <int FMT> __device__ __forceinline__ void dequant16(const WRaw<FMT>& r, int j, int c, int e, const u64* grid, float* o);
+
+template <> __device__ __forceinline__ void dequant16<ILT_Q4_K>(const WRaw<ILT_Q4_K>& r, int j, int c, int e, const u64*, float* o) {
+  const int sh = 8 * j, hl = j & 1;              // group g = 4c + j of the super-block
   const u32 x0 = ((u32)r.hdr.y >> sh) & 0xFF, x1 = ((u32)r.hdr.z >> sh) & 0xFF, x2 = ((u32)r.hdr.w >> sh) & 0xFF;
-  const u32 sc = g < 4 ? (x0 & 63) : ((x2 & 0xF) | ((x0 >> 6) << 4));
-  const u32 mn = g < 4 ? (x1 & 63) : ((x2 >> 4) | ((x1 >> 6) << 4));
+  const u32 sc = c == 0 ? (x0 & 63) : ((x2 & 0xF) | ((x0 >> 6) << 4));
+  const u32 mn = c == 0 ? (x1 & 63) : ((x2 >> 4) | ((x1 >> 6) << 4));
   const float d1 = ilt_h2f((u16)(r.hdr.x & 0xFFFF)) * (float)sc, m1 = ilt_h2f((u16)((u32)r.hdr.x >> 16)) * (float)mn;
-  const u32 w[4] = {(u32)r.q.x, (u32)r.q.y, (u32)r.q.z, (u32)r.q.w};
+  const int4& q = r.q[j >> 1];
 #pragma unroll
   for (int i = 0; i < 4; i++) {
-    const u32 v = (w[i] >> (4 * hl)) & 0x0F0F0F0F;
+    const u32 v = (word_of(q, i) >> (4 * hl)) & 0x0F0F0F0F;
 #pragma unroll
     for (int k = 0; k < 4; k++) o[4 * i + k] = d1 * (float)((v >> (8 * k)) & 0xFF) - m1;
   }
 }
 
-template <> __device__ __forceinline__ void dequant16<ILT_Q6_K>(const WRaw<ILT_Q6_K>& r, int ks, int e, const u64*, float* o) {
-  const int part = ks & 3, h = part >> 1;
-  const float s = ilt_h2f((u16)r.d) * (float)(i8)(r.sc & 0xFF);
-  const u32 ql[4] = {(u32)r.ql.x, (u32)r.ql.y, (u32)r.ql.z, (u32)r.ql.w};
-  const u32 qh[4] = {(u32)r.qh.x, (u32)r.qh.y, (u32)r.qh.z, (u32)r.qh.w};
+template <> __device__ __forceinline__ void dequant16<ILT_Q6_K>(const WRaw<ILT_Q6_K>& r, int j, int c, int e, const u64*, float* o) {
+  const int h = j >> 1;                          // 32-weight part j of the half: ql[j&1]'s nibble h, qh's bit pair j
+  const u32 scw = (u32)(j < 2 ? r.sc.x : r.sc.y) >> (16 * (j & 1) + 8 * e);
+  const float s = ilt_h2f((u16)r.d) * (float)(i8)(scw & 0xFF);
+  const int4& ql = r.ql[j & 1];
 #pragma unroll
   for (int i = 0; i < 4; i++) {
-    const u32 v = ((ql[i] >> (4 * h)) & 0x0F0F0F0F) | (((qh[i] >> (2 * part)) & 0x03030303) << 4);
+    const u32 v = ((word_of(ql, i) >> (4 * h)) & 0x0F0F0F0F) | (((word_of(r.qh, i) >> (2 * j)) & 0x03030303) << 4);
 #pragma unroll
     for (int k = 0; k < 4; k++) o[4 * i + k] = s * (float)((int)((v >> (8 * k)) & 0xFF) - 32);
   }
 }
 
-template <> __device__ __forceinline__ void dequant16<ILT_Q2_K>(const WRaw<ILT_Q2_K>& r, int ks, int e, const u64*, float* o) {
-  const int j = ks & 3;
-  const float dl = ilt_h2f((u16)(r.dd & 0xFFFF)) * (float)(r.sc & 15), ml = ilt_h2f((u16)(r.dd >> 16)) * (float)((r.sc >> 4) & 15);
-  const u32 w[4] = {(u32)r.q.x, (u32)r.q.y, (u32)r.q.z, (u32)r.q.w};
+template <> __device__ __forceinline__ void dequant16<ILT_Q2_K>(const WRaw<ILT_Q2_K>& r, int j, int c, int e, const u64*, float* o) {
+  const u32 scw = ((u32)(j < 2 ? r.sc.x : r.sc.y) >> (16 * (j & 1) + 8 * e)) & 0xFF;
+  const float dl = ilt_h2f((u16)(r.dd & 0xFFFF)) * (float)(scw & 15), ml = ilt_h2f((u16)(r.dd >> 16)) * (float)(scw >> 4);
 #pragma unroll
   for (int i = 0; i < 4; i++) {
-    const u32 v = (w[i] >> (2 * j)) & 0x03030303;
+    const u32 v = (word_of(r.q, i) >> (2 * j)) & 0x03030303;
 #pragma unroll
     for (int k = 0; k < 4; k++) o[4 * i + k] = dl * (float)((v >> (8 * k)) & 0xFF) - ml;
   }
 }
 
-template <> __device__ __forceinline__ void dequant16<ILT_IQ2_XXS>(const WRaw<ILT_IQ2_XXS>& r, int ks, int e, const u64* grid, float* o) {
-  const u32 g = (u32)r.q.x >> (16 * e), aux = (u32)r.q.y;
+template <> __device__ __forceinline__ void dequant16<ILT_IQ2_XXS>(const WRaw<ILT_IQ2_XXS>& r, int j, int c, int e, const u64* grid, float* o) {
+  const int4& q = r.q[j >> 1];                   // the half's 32-weight group j: 8 bytes
+  const u32 g = word_of(q, 2 * (j & 1)) >> (16 * e), aux = word_of(q, 2 * (j & 1) + 1);
   const float db = (ilt_h2f((u16)r.d) * (0.5f + (float)(aux >> 28))) * 0.25f;
 #pragma unroll
   for (int l = 0; l < 2; l++) {
@@ -150,21 +161,28 @@ struct BfParams {
   float* y; const float* bias; int acc; int ntok;
 };
 
-template <int TN> struct Smem {
+template <int TM, int TN> struct Smem {
   __align__(16) u8 xs[3][TN * KS * 2];
-  __align__(16) u8 ws[2][WSLAB];
+  __align__(16) u8 ws[2][TM * KS * 2];
   u64 grid[256];
   u32 scan[256];
   int tile_z, tile_t0, tile_n;
 };
 
-// piece p (16 bytes) of row r of a slab
-__device__ __forceinline__ u32 slab_off(int r, int p) { return (u32)(4 * r + (p ^ ((r >> 2) & 3))) * 16; }
+// Piece p (16 bytes) of row r of a slab.  Rows are 64 bytes, so 8 consecutive rows span 128
+// bytes-wide LDS twice over and 16 rows a 256-byte-wide one four times; the piece index is
+// xor-ed with bits of the row such that the same piece of 8 (or 16) consecutive rows falls
+// in 8 (or 16) different 16-byte columns.
+__device__ __forceinline__ u32 slab_swz(int r) { return (((r >> 1) ^ (r >> 3)) & 1) | (((r >> 2) & 1) << 1); }
+__device__ __forceinline__ u32 slab_off(int r, int p) { return (u32)(4 * r + (p ^ slab_swz(r))) * 16; }
 
-template <int FMT, int TN>
-__global__ __launch_bounds__(256, TN == 256 ? 2 : 3) void gemm_bf16_kernel(BfParams p) {
-  __shared__ Smem<TN> S;
-  constexpr int NA = TN / 64;        // 32-token patches per wave; also direct-load instructions per wave and step
+// TM rows x TN tokens per workgroup of 2*TM threads; wave w: rows 64*(w/2).., tokens (TN/2)*(w%2)..
+template <int FMT, int TM, int TN>
+__global__ __launch_bounds__(2 * TM, TM == 256 ? 1 : TN == 256 ? 2 : 3) void gemm_bf16_kernel(BfParams p) {
+  __shared__ Smem<TM, TN> S;
+  constexpr int NA = TN / 64;            // 32-token patches per wave
+  constexpr int NI = 2 * TN / TM;        // direct-load instructions per wave and step
+  constexpr int WL = WRaw<FMT>::LOADS;
   const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
   const int NR = (p.rows + TM - 1) / TM;
 
@@ -173,12 +191,12 @@ __global__ __launch_bounds__(256, TN == 256 ? 2 : 3) void gemm_bf16_kernel(BfPar
   {
     int NT;
     if (p.ptrs) {
-      S.scan[t] = t < p.ne ? (p.counts[t] + TN - 1) / TN : 0;
+      if (t < 256) S.scan[t] = t < p.ne ? (p.counts[t] + TN - 1) / TN : 0;
       __syncthreads();
       for (int off = 1; off < 256; off <<= 1) {
-        const u32 v = t >= off ? S.scan[t - off] : 0;
+        const u32 v = (t < 256 && t >= off) ? S.scan[t - off] : 0;
         __syncthreads();
-        S.scan[t] += v;
+        if (t < 256) S.scan[t] += v;
         __syncthreads();
       }
       NT = (int)S.scan[255];
@@ -210,18 +228,22 @@ __global__ __launch_bounds__(256, TN == 256 ? 2 : 3) void gemm_bf16_kernel(BfPar
     }
   }
   const int r0 = rt * TM;
-  if (FMT == ILT_IQ2_XXS) { S.grid[t] = bf_grid_dev[t]; __syncthreads(); }
+  if (FMT == ILT_IQ2_XXS) {
+    if (t < 256) S.grid[t] = bf_grid_dev[t];
+    __syncthreads();
+  }
 
   // ---- this thread's shares of a step ----
   const int wrow = t >> 1, e = t & 1;                      // 16 weights of row wrow
   const __amdgpu_buffer_rsrc_t rw = ilt_rsrc(ilt_uniform_ptr(w), (u32)min((long long)p.rows * p.row_bytes, 0xFFFFFFF0LL));
   const u32 wrowoff = (u32)((long long)min(r0 + wrow, p.rows - 1) * p.row_bytes);
   const u32 wdst = slab_off(wrow, 2 * e);                  // its two pieces: 2e and 2e+1 (the second at wdst ^ 16)
-  const u8* xsrc[NA];                                      // the x pieces it sends to LDS
+  const u8* xbase = (const u8*)ilt_uniform_ptr(p.x + tok0 * (long)p.cols);
+  u32 xoff[NI];                                            // the x pieces it sends to LDS
 #pragma unroll
-  for (int i = 0; i < NA; i++) {
-    const int P = (wave * NA + i) * 64 + lane, tok = P >> 2, kp = (P & 3) ^ ((tok >> 2) & 3);
-    xsrc[i] = (const u8*)(p.x + (tok0 + min(tok, ntok - 1)) * (long)p.cols) + 16 * kp;
+  for (int i = 0; i < NI; i++) {
+    const int P = (wave * NI + i) * 64 + lane, tok = P >> 2, kp = (P & 3) ^ (int)slab_swz(tok);
+    xoff[i] = (u32)min(tok, ntok - 1) * (u32)p.cols * 2 + 16 * kp;
   }
 
   v16f acc[NA][2];
@@ -240,37 +262,52 @@ __global__ __launch_bounds__(256, TN == 256 ? 2 : 3) void gemm_bf16_kernel(BfPar
 #pragma unroll
   for (int b = 0; b < 2; b++) boff[b] = slab_off(wr0 + 32 * b + l32, lh);
 
-  const int nk = p.cols / KS;
+  const int nk = p.cols / KS, nh = nk / 4;                 // steps, half super-blocks
   auto issue_x = [&](int stage, int ks) {
 #pragma unroll
-    for (int i = 0; i < NA; i++) ilt_g2lds16(xsrc[i] + (long)ks * (KS * 2), S.xs[stage] + (wave * NA + i) * 1024);
+    for (int i = 0; i < NI; i++) ilt_g2lds16(xbase + ks * (KS * 2) + xoff[i], S.xs[stage] + (wave * NI + i) * 1024);
+  };
+  auto dequant_to = [&](const WRaw<FMT>& raw, int j, int c, int slab) {   // step j of a half's weights into a slab
+    float o[16];
+    dequant16<FMT>(raw, j, c, e, S.grid, o);
+    u32 pk[8];
+#pragma unroll
+    for (int i = 0; i < 8; i++) pk[i] = pack_bf16(o[2 * i], o[2 * i + 1]);
+    u8* ws = S.ws[slab];
+    *(int4*)(ws + wdst) = make_int4(pk[0], pk[1], pk[2], pk[3]);
+    *(int4*)(ws + (wdst ^ 16)) = make_int4(pk[4], pk[5], pk[6], pk[7]);
   };
 
-  WRaw<FMT> wraw;
-  load_w<FMT>(wraw, rw, wrowoff, 0, e);
+  // Two register sets of raw weights, each a half super-block (4 steps): rawa holds half 0
+  // of a super-block, rawb half 1.  Step ks multiplies slab ks while it dequantizes step
+  // ks+1's weights into the other weight slab; a set is reloaded, with the half two ahead,
+  // right after its last step is dequantized, four steps before it is needed again.
+  WRaw<FMT> rawa, rawb;
+  load_w<FMT>(rawa, rw, wrowoff, 0, e);
   issue_x(0, 0);
-  issue_x(1, min(1, nk - 1));
+  load_w<FMT>(rawb, rw, wrowoff, 1, e);
+  issue_x(1, 1);
   int st0 = 0, st1 = 1, st2 = 2;                           // ring: the step's slab, the next step's, the one after
+  dequant_to(rawa, 0, 0, 0);
 
-  for (int ks = 0; ks < nk; ks++) {
-    {
-      float o[16];
-      dequant16<FMT>(wraw, ks, e, S.grid, o);
-      u32 pk[8];
-#pragma unroll
-      for (int i = 0; i < 8; i++) pk[i] = pack_bf16(o[2 * i], o[2 * i + 1]);
-      u8* ws = S.ws[ks & 1];
-      *(int4*)(ws + wdst) = make_int4(pk[0], pk[1], pk[2], pk[3]);
-      *(int4*)(ws + (wdst ^ 16)) = make_int4(pk[4], pk[5], pk[6], pk[7]);
-    }
-    // all but the newest NA loads have landed: this step's x slab has (it was sent two steps ago)
-    if (NA == 4) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
-    else asm volatile("s_waitcnt vmcnt(2)" ::: "memory");
+  // J: the step's place in its super-block (0..7), a constant in the unrolled body
+  auto step = [&](int ks, auto Jc) {
+    constexpr int J = decltype(Jc)::value;
+    // All loads but the previous step's have landed: this step's x slab has (sent two steps
+    // ago).  The barrier also publishes the weight slab written during the previous step,
+    // and says that x slab ks-1 and the other weight slab are read no more.
+    constexpr int prev = NI + ((J == 0 || J == 4) ? WL : 0);   // steps 3 and 7 of a super-block also reload a set
+    asm volatile("s_waitcnt vmcnt(%0)" :: "n"(prev) : "memory");
     __syncthreads();
-    load_w<FMT>(wraw, rw, wrowoff, min(ks + 1, nk - 1), e);
+    if (J == 3) load_w<FMT>(rawa, rw, wrowoff, min((ks >> 2) + 2, nh - 1), e);   // rawa's last use was step 2's dequantization
+    if (J == 7) load_w<FMT>(rawb, rw, wrowoff, min((ks >> 2) + 2, nh - 1), e);
     issue_x(st2, min(ks + 2, nk - 1));
+    __builtin_amdgcn_sched_barrier(0);
     const u8* xs = S.xs[st0];
-    const u8* ws = S.ws[ks & 1];
+    const u8* ws = S.ws[J & 1];
+    // step ks+1's weights: J+1 = 1..3 from rawa, 4..7 from rawb, 8 = the next super-block's 0 from rawa
+    // (past the last step: a slab nobody reads)
+    constexpr int J1 = (J + 1) & 7;
 #pragma unroll
     for (int kk = 0; kk < 2; kk++) {
       v8bf af[NA], bf[2];
@@ -278,12 +315,23 @@ __global__ __launch_bounds__(256, TN == 256 ? 2 : 3) void gemm_bf16_kernel(BfPar
       for (int a = 0; a < NA; a++) af[a] = *(const v8bf*)(xs + (aoff[a] ^ (32 * kk)));
 #pragma unroll
       for (int b = 0; b < 2; b++) bf[b] = *(const v8bf*)(ws + (boff[b] ^ (32 * kk)));
+      if (kk == 0) dequant_to(J1 < 4 ? rawa : rawb, J1 & 3, J1 >> 2, J1 & 1);
 #pragma unroll
       for (int a = 0; a < NA; a++)
 #pragma unroll
         for (int b = 0; b < 2; b++) acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[a], bf[b], acc[a][b], 0, 0, 0);
     }
     const int s = st0; st0 = st1; st1 = st2; st2 = s;
+  };
+  for (int ks = 0; ks < nk; ks += 8) {     // one super-block of 256 columns
+    step(ks + 0, std::integral_constant<int, 0>{});
+    step(ks + 1, std::integral_constant<int, 1>{});
+    step(ks + 2, std::integral_constant<int, 2>{});
+    step(ks + 3, std::integral_constant<int, 3>{});
+    step(ks + 4, std::integral_constant<int, 4>{});
+    step(ks + 5, std::integral_constant<int, 5>{});
+    step(ks + 6, std::integral_constant<int, 6>{});
+    step(ks + 7, std::integral_constant<int, 7>{});
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // the tail's redundant loads: nothing may land in LDS after the workgroup ends
 
@@ -316,21 +364,21 @@ __global__ __launch_bounds__(256) void cvt_bf16_kernel(const float* __restrict__
   ((int4*)xb)[i] = make_int4(pack_bf16(a.x, a.y), pack_bf16(a.z, a.w), pack_bf16(b.x, b.y), pack_bf16(b.z, b.w));
 }
 
-template <int FMT, int TN>
+template <int FMT, int TM, int TN>
 hipError_t launch_bf16(const BfParams& p, long long token_tiles, hipStream_t st) {
   const long long total = token_tiles * ((p.rows + TM - 1) / TM), per = (total + 7) / 8;
   if (per * 8 > 0x7FFFFFFFLL) return hipErrorInvalidValue;
-  hipLaunchKernelGGL((gemm_bf16_kernel<FMT, TN>), dim3((unsigned)(per * 8)), dim3(256), 0, st, p);
+  hipLaunchKernelGGL((gemm_bf16_kernel<FMT, TM, TN>), dim3((unsigned)(per * 8)), dim3(2 * TM), 0, st, p);
   return hipGetLastError();
 }
 
-template <int TN>
+template <int TM, int TN>
 hipError_t dispatch_bf16(int fmt, const BfParams& p, long long token_tiles, hipStream_t st) {
   switch (fmt) {
-    case ILT_Q4_K: return launch_bf16<ILT_Q4_K, TN>(p, token_tiles, st);
-    case ILT_Q6_K: return launch_bf16<ILT_Q6_K, TN>(p, token_tiles, st);
-    case ILT_Q2_K: return launch_bf16<ILT_Q2_K, TN>(p, token_tiles, st);
-    case ILT_IQ2_XXS: return launch_bf16<ILT_IQ2_XXS, TN>(p, token_tiles, st);
+    case ILT_Q4_K: return launch_bf16<ILT_Q4_K, TM, TN>(p, token_tiles, st);
+    case ILT_Q6_K: return launch_bf16<ILT_Q6_K, TM, TN>(p, token_tiles, st);
+    case ILT_Q2_K: return launch_bf16<ILT_Q2_K, TM, TN>(p, token_tiles, st);
+    case ILT_IQ2_XXS: return launch_bf16<ILT_IQ2_XXS, TM, TN>(p, token_tiles, st);
   }
   return hipErrorInvalidValue;
 }
@@ -349,10 +397,15 @@ hipError_t ilt_k_gemm_bf16(int fmt, const uint8_t* w, long long row_bytes, int r
   if (ntok <= 0 || rows <= 0) return hipSuccess;
   BfParams p = {};
   p.w = w; p.rows = rows; p.cols = cols; p.row_bytes = row_bytes; p.x = xb; p.y = y; p.bias = bias; p.acc = acc; p.ntok = ntok;
-  // 256-token tiles halve the dequantization per product, but need enough tiles to fill 512 workgroup slots
-  const long long nr = (rows + TM - 1) / TM;
-  if ((long long)((ntok + 255) / 256) * nr >= 1024) return dispatch_bf16<256>(fmt, p, (ntok + 255) / 256, st);
-  return dispatch_bf16<128>(fmt, p, (ntok + 127) / 128, st);
+  // Larger tiles dequantize and fetch less per product, but need enough tiles to fill the chip:
+  // 256x256 runs one workgroup per CU (256 slots), 128x256 two, 128x128 three.
+  const long long t256 = (ntok + 255) / 256, r256 = (rows + 255) / 256, r128 = (rows + 127) / 128;
+  const char* force = getenv("ILT_BF16_TILE");     // "1", "2", "3": the 128x128, 128x256, 256x256 tile whatever the shape (tests)
+  int tile = force ? atoi(force) : 0;
+  if (tile < 1 || tile > 3) tile = t256 * r256 >= 512 ? 3 : t256 * r128 >= 1024 ? 2 : 1;
+  if (tile == 3) return dispatch_bf16<256, 256>(fmt, p, t256, st);
+  if (tile == 2) return dispatch_bf16<128, 256>(fmt, p, t256, st);
+  return dispatch_bf16<128, 128>(fmt, p, (ntok + 127) / 128, st);
 }
 
 hipError_t ilt_k_gemm_bf16_id(int fmt, const uint64_t* ptrs, long long add, const uint32_t* counts, const uint32_t* bases,
@@ -363,5 +416,5 @@ hipError_t ilt_k_gemm_bf16_id(int fmt, const uint64_t* ptrs, long long add, cons
   BfParams p = {};
   p.ptrs = ptrs; p.add = add; p.counts = counts; p.bases = bases; p.ne = ne;
   p.rows = rows; p.cols = cols; p.row_bytes = row_bytes; p.x = xb; p.y = y; p.ntok = (int)total_rows;
-  return dispatch_bf16<128>(fmt, p, total_rows / 128 + ne, st);
+  return dispatch_bf16<128, 128>(fmt, p, total_rows / 128 + ne, st);
 }

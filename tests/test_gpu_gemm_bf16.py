@@ -44,10 +44,12 @@ def upload(dev, qtype, rows, cols, w):
 FORMATS = [synth.Q4_K, synth.Q6_K, synth.Q2_K, synth.IQ2_XXS]
 
 
+@pytest.mark.parametrize("tile", [1, 2, 3])          # the 128x128, 128x256 and 256x256 workgroup tiles
 @pytest.mark.parametrize("qtype", FORMATS)
-@pytest.mark.parametrize("rows,cols", [(130, 512), (64, 256)])
-def test_one_hot_tokens_read_back_the_dequantized_matrix(dev, qtype, rows, cols):
+@pytest.mark.parametrize("rows,cols", [(130, 512), (300, 256)])
+def test_one_hot_tokens_read_back_the_dequantized_matrix(dev, monkeypatch, qtype, rows, cols, tile):
     from illatio_amd import dense, hip
+    monkeypatch.setenv("ILT_BF16_TILE", str(tile))
     rng = synth.make_rng(qtype + rows)
     w = synth.weights(qtype, rows, cols, rng)
     x = np.eye(cols, dtype=np.float32)
@@ -68,13 +70,15 @@ def test_one_hot_tokens_read_back_the_dequantized_matrix(dev, qtype, rows, cols)
     (synth.Q4_K, 1024, 2560, 77),
     (synth.Q2_K, 300, 2048, 129),
     (synth.IQ2_XXS, 256, 4096, 64),
-    (synth.Q6_K, 8200, 512, 4000),       # 1024 tiles and more: the 256-token tile runs; ragged both ways
-    (synth.Q4_K, 8200, 256, 4100),
-    (synth.Q2_K, 8200, 256, 4100),
-    (synth.IQ2_XXS, 8200, 256, 4100),
+    (synth.Q6_K, 8200, 512, 4000),       # enough tiles that the largest tile is chosen by itself; ragged both ways
 ])
-def test_dense_bf16_product_within_tolerance(dev, qtype, rows, cols, n):
+@pytest.mark.parametrize("tile", [0, 2, 3])          # 0: chosen by shape; 2, 3: the 128x256 and 256x256 tiles forced
+def test_dense_bf16_product_within_tolerance(dev, monkeypatch, qtype, rows, cols, n, tile):
     from illatio_amd import dense, hip
+    if tile:
+        monkeypatch.setenv("ILT_BF16_TILE", str(tile))
+    else:
+        monkeypatch.delenv("ILT_BF16_TILE", raising=False)
     rng = synth.make_rng(qtype * 7 + rows + n)
     w = synth.weights(qtype, rows, cols, rng)
     x = synth.activations((n, cols), rng)
