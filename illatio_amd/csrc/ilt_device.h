@@ -124,6 +124,19 @@ __device__ __forceinline__ void ilt_g2lds16(const void* src, void* lds_base) {
   __builtin_amdgcn_global_load_lds((const ILT_GLOBAL void*)src, (ILT_LDS void*)lds_base, 16, 0, 0);
 }
 
+// A 16-byte LDS store the compiler does not see as one.  After a direct global-to-LDS load
+// it makes every LDS store wait for vmcnt(0), i.e. for loads sent off to arrive steps later;
+// a kernel that keeps such loads in flight stores through this and waits for its stores
+// itself (ilt_barrier_lds) before the barrier that publishes them.
+__device__ __forceinline__ void ilt_lds_st16_untracked(void* p, int a, int b, int c, int d) {
+  const ilt_v4i v = {a, b, c, d};
+  asm volatile("ds_write_b128 %0, %1" :: "v"((u32)(uintptr_t)(ILT_LDS void*)p), "v"(v) : "memory");
+}
+// This wave's LDS traffic done, then the workgroup barrier -- without __syncthreads()'s fence,
+// which would also wait for every global load in flight (vmcnt(0)), the direct-to-LDS ones
+// included.  The caller waits (s_waitcnt vmcnt(n)) for the loads the barrier must publish.
+__device__ __forceinline__ void ilt_barrier_lds() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+
 // SBCL evaluates single-float exp and log by widening to double, calling libm and
 // rounding back (the CPU path's silu, softplus); the kernels do the same.
 __device__ __forceinline__ float ilt_expf_via_double(float x) { return (float)exp((double)x); }

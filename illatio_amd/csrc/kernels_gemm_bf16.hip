@@ -176,13 +176,19 @@ template <int TM, int TN> struct Smem {
 __device__ __forceinline__ u32 slab_swz(int r) { return (((r >> 1) ^ (r >> 3)) & 1) | (((r >> 2) & 1) << 1); }
 __device__ __forceinline__ u32 slab_off(int r, int p) { return (u32)(4 * r + (p ^ slab_swz(r))) * 16; }
 
-// TM rows x TN tokens per workgroup of 2*TM threads; wave w: rows 64*(w/2).., tokens (TN/2)*(w%2)..
-template <int FMT, int TM, int TN>
-__global__ __launch_bounds__(2 * TM, TM == 256 ? 1 : TN == 256 ? 2 : 3) void gemm_bf16_kernel(BfParams p) {
+// TM rows x TN tokens per workgroup; wave w: rows 32*NB*(w/2).., tokens (TN/2)*(w%2)..: NA x NB
+// patches of 32x32.  NB = 2: 2*TM threads, two per row; NB = 4: TM threads, one per row, a
+// wave alone on its SIMD with 128x128 results in 256 accumulator registers.
+template <int TM, int NB> constexpr int bf16_threads() { return 64 * 2 * (TM / (32 * NB)); }
+
+template <int FMT, int TM, int TN, int NB>
+__global__ __launch_bounds__((bf16_threads<TM, NB>()), (TM == 256 ? 1 : TN == 256 ? 2 : 3)) void gemm_bf16_kernel(BfParams p) {
   __shared__ Smem<TM, TN> S;
+  constexpr int THREADS = bf16_threads<TM, NB>();
+  constexpr int NE = 2 * TM / THREADS;   // 16-column units of a row a thread dequantizes per step: 1 or 2
   constexpr int NA = TN / 64;            // 32-token patches per wave
-  constexpr int NI = 2 * TN / TM;        // direct-load instructions per wave and step
-  constexpr int WL = WRaw<FMT>::LOADS;
+  constexpr int NI = 4 * TN / THREADS;   // direct-load instructions per wave and step
+  constexpr int WL = WRaw<FMT>::LOADS * NE;
   const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
   const int NR = (p.rows + TM - 1) / TM;
 
@@ -234,10 +240,10 @@ __global__ __launch_bounds__(2 * TM, TM == 256 ? 1 : TN == 256 ? 2 : 3) void gem
   }
 
   // ---- this thread's shares of a step ----
-  const int wrow = t >> 1, e = t & 1;                      // 16 weights of row wrow
+  const int wrow = NE == 1 ? t >> 1 : t, e0 = NE == 1 ? t & 1 : 0;   // 16 weights (or all 32) of row wrow
   const __amdgpu_buffer_rsrc_t rw = ilt_rsrc(ilt_uniform_ptr(w), (u32)min((long long)p.rows * p.row_bytes, 0xFFFFFFF0LL));
   const u32 wrowoff = (u32)((long long)min(r0 + wrow, p.rows - 1) * p.row_bytes);
-  const u32 wdst = slab_off(wrow, 2 * e);                  // its two pieces: 2e and 2e+1 (the second at wdst ^ 16)
+  const u32 wdst = slab_off(wrow, 2 * e0);                 // unit e's two pieces: 2e and 2e+1, at (wdst ^ 32e) and that ^ 16
   const u8* xbase = (const u8*)ilt_uniform_ptr(p.x + tok0 * (long)p.cols);
   u32 xoff[NI];                                            // the x pieces it sends to LDS
 #pragma unroll
@@ -246,46 +252,53 @@ __global__ __launch_bounds__(2 * TM, TM == 256 ? 1 : TN == 256 ? 2 : 3) void gem
     xoff[i] = (u32)min(tok, ntok - 1) * (u32)p.cols * 2 + 16 * kp;
   }
 
-  v16f acc[NA][2];
+  v16f acc[NA][NB];
 #pragma unroll
   for (int a = 0; a < NA; a++)
 #pragma unroll
-    for (int b = 0; b < 2; b++)
+    for (int b = 0; b < NB; b++)
 #pragma unroll
       for (int r = 0; r < 16; r++) acc[a][b][r] = 0.0f;
 
-  const int wt0 = (TN / 2) * (wave & 1), wr0 = 64 * (wave >> 1);   // this wave's tokens and rows in the tile
+  const int wt0 = (TN / 2) * (wave & 1), wr0 = 32 * NB * (wave >> 1);   // this wave's tokens and rows in the tile
   const int l32 = lane & 31, lh = lane >> 5;
-  u32 aoff[NA], boff[2];                                   // fragment offsets for the step's first 16 columns; the second 16 at ^ 32
+  u32 aoff[NA], boff[NB];                                  // fragment offsets for the step's first 16 columns; the second 16 at ^ 32
 #pragma unroll
   for (int a = 0; a < NA; a++) aoff[a] = slab_off(wt0 + 32 * a + l32, lh);
 #pragma unroll
-  for (int b = 0; b < 2; b++) boff[b] = slab_off(wr0 + 32 * b + l32, lh);
+  for (int b = 0; b < NB; b++) boff[b] = slab_off(wr0 + 32 * b + l32, lh);
 
   const int nk = p.cols / KS, nh = nk / 4;                 // steps, half super-blocks
   auto issue_x = [&](int stage, int ks) {
 #pragma unroll
     for (int i = 0; i < NI; i++) ilt_g2lds16(xbase + ks * (KS * 2) + xoff[i], S.xs[stage] + (wave * NI + i) * 1024);
   };
-  auto dequant_to = [&](const WRaw<FMT>& raw, int j, int c, int slab) {   // step j of a half's weights into a slab
-    float o[16];
-    dequant16<FMT>(raw, j, c, e, S.grid, o);
-    u32 pk[8];
+  auto dequant_to = [&](const WRaw<FMT>* raw, int j, int c, int slab) {   // step j of a half's weights into a slab
 #pragma unroll
-    for (int i = 0; i < 8; i++) pk[i] = pack_bf16(o[2 * i], o[2 * i + 1]);
-    u8* ws = S.ws[slab];
-    *(int4*)(ws + wdst) = make_int4(pk[0], pk[1], pk[2], pk[3]);
-    *(int4*)(ws + (wdst ^ 16)) = make_int4(pk[4], pk[5], pk[6], pk[7]);
+    for (int u = 0; u < NE; u++) {
+      float o[16];
+      dequant16<FMT>(raw[u], j, c, e0 + u, S.grid, o);
+      u32 pk[8];
+#pragma unroll
+      for (int i = 0; i < 8; i++) pk[i] = pack_bf16(o[2 * i], o[2 * i + 1]);
+      u8* ws = S.ws[slab];
+      ilt_lds_st16_untracked(ws + (wdst ^ (32 * u)), pk[0], pk[1], pk[2], pk[3]);
+      ilt_lds_st16_untracked(ws + (wdst ^ (32 * u) ^ 16), pk[4], pk[5], pk[6], pk[7]);
+    }
+  };
+  auto load_raw = [&](WRaw<FMT>* raw, int hb) {
+#pragma unroll
+    for (int u = 0; u < NE; u++) load_w<FMT>(raw[u], rw, wrowoff, hb, e0 + u);
   };
 
   // Two register sets of raw weights, each a half super-block (4 steps): rawa holds half 0
   // of a super-block, rawb half 1.  Step ks multiplies slab ks while it dequantizes step
   // ks+1's weights into the other weight slab; a set is reloaded, with the half two ahead,
   // right after its last step is dequantized, four steps before it is needed again.
-  WRaw<FMT> rawa, rawb;
-  load_w<FMT>(rawa, rw, wrowoff, 0, e);
+  WRaw<FMT> rawa[NE], rawb[NE];
+  load_raw(rawa, 0);
   issue_x(0, 0);
-  load_w<FMT>(rawb, rw, wrowoff, 1, e);
+  load_raw(rawb, 1);
   issue_x(1, 1);
   int st0 = 0, st1 = 1, st2 = 2;                           // ring: the step's slab, the next step's, the one after
   dequant_to(rawa, 0, 0, 0);
@@ -298,9 +311,9 @@ __global__ __launch_bounds__(2 * TM, TM == 256 ? 1 : TN == 256 ? 2 : 3) void gem
     // and says that x slab ks-1 and the other weight slab are read no more.
     constexpr int prev = NI + ((J == 0 || J == 4) ? WL : 0);   // steps 3 and 7 of a super-block also reload a set
     asm volatile("s_waitcnt vmcnt(%0)" :: "n"(prev) : "memory");
-    __syncthreads();
-    if (J == 3) load_w<FMT>(rawa, rw, wrowoff, min((ks >> 2) + 2, nh - 1), e);   // rawa's last use was step 2's dequantization
-    if (J == 7) load_w<FMT>(rawb, rw, wrowoff, min((ks >> 2) + 2, nh - 1), e);
+    ilt_barrier_lds();                                     // no fence: later steps' loads stay in flight
+    if (J == 3) load_raw(rawa, min((ks >> 2) + 2, nh - 1));   // rawa's last use was step 2's dequantization
+    if (J == 7) load_raw(rawb, min((ks >> 2) + 2, nh - 1));
     issue_x(st2, min(ks + 2, nk - 1));
     __builtin_amdgcn_sched_barrier(0);
     const u8* xs = S.xs[st0];
@@ -310,16 +323,16 @@ __global__ __launch_bounds__(2 * TM, TM == 256 ? 1 : TN == 256 ? 2 : 3) void gem
     constexpr int J1 = (J + 1) & 7;
 #pragma unroll
     for (int kk = 0; kk < 2; kk++) {
-      v8bf af[NA], bf[2];
+      v8bf af[NA], bf[NB];
 #pragma unroll
       for (int a = 0; a < NA; a++) af[a] = *(const v8bf*)(xs + (aoff[a] ^ (32 * kk)));
 #pragma unroll
-      for (int b = 0; b < 2; b++) bf[b] = *(const v8bf*)(ws + (boff[b] ^ (32 * kk)));
+      for (int b = 0; b < NB; b++) bf[b] = *(const v8bf*)(ws + (boff[b] ^ (32 * kk)));
       if (kk == 0) dequant_to(J1 < 4 ? rawa : rawb, J1 & 3, J1 >> 2, J1 & 1);
 #pragma unroll
       for (int a = 0; a < NA; a++)
 #pragma unroll
-        for (int b = 0; b < 2; b++) acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[a], bf[b], acc[a][b], 0, 0, 0);
+        for (int b = 0; b < NB; b++) acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[a], bf[b], acc[a][b], 0, 0, 0);
     }
     const int s = st0; st0 = st1; st1 = st2; st2 = s;
   };
@@ -337,7 +350,7 @@ __global__ __launch_bounds__(2 * TM, TM == 256 ? 1 : TN == 256 ? 2 : 3) void gem
 
   // ---- store: patch (a, b): token = wt0 + 32a + 8*(r/4) + 4*lh + r%4, row = wr0 + 32b + l32 ----
 #pragma unroll
-  for (int b = 0; b < 2; b++) {
+  for (int b = 0; b < NB; b++) {
     const int row = r0 + wr0 + 32 * b + l32;
     if (row >= p.rows) continue;
     const float bv = p.bias ? p.bias[row] : 0.0f;
@@ -364,21 +377,21 @@ __global__ __launch_bounds__(256) void cvt_bf16_kernel(const float* __restrict__
   ((int4*)xb)[i] = make_int4(pack_bf16(a.x, a.y), pack_bf16(a.z, a.w), pack_bf16(b.x, b.y), pack_bf16(b.z, b.w));
 }
 
-template <int FMT, int TM, int TN>
+template <int FMT, int TM, int TN, int NB>
 hipError_t launch_bf16(const BfParams& p, long long token_tiles, hipStream_t st) {
   const long long total = token_tiles * ((p.rows + TM - 1) / TM), per = (total + 7) / 8;
   if (per * 8 > 0x7FFFFFFFLL) return hipErrorInvalidValue;
-  hipLaunchKernelGGL((gemm_bf16_kernel<FMT, TM, TN>), dim3((unsigned)(per * 8)), dim3(2 * TM), 0, st, p);
+  hipLaunchKernelGGL((gemm_bf16_kernel<FMT, TM, TN, NB>), dim3((unsigned)(per * 8)), dim3(bf16_threads<TM, NB>()), 0, st, p);
   return hipGetLastError();
 }
 
-template <int TM, int TN>
+template <int TM, int TN, int NB>
 hipError_t dispatch_bf16(int fmt, const BfParams& p, long long token_tiles, hipStream_t st) {
   switch (fmt) {
-    case ILT_Q4_K: return launch_bf16<ILT_Q4_K, TM, TN>(p, token_tiles, st);
-    case ILT_Q6_K: return launch_bf16<ILT_Q6_K, TM, TN>(p, token_tiles, st);
-    case ILT_Q2_K: return launch_bf16<ILT_Q2_K, TM, TN>(p, token_tiles, st);
-    case ILT_IQ2_XXS: return launch_bf16<ILT_IQ2_XXS, TM, TN>(p, token_tiles, st);
+    case ILT_Q4_K: return launch_bf16<ILT_Q4_K, TM, TN, NB>(p, token_tiles, st);
+    case ILT_Q6_K: return launch_bf16<ILT_Q6_K, TM, TN, NB>(p, token_tiles, st);
+    case ILT_Q2_K: return launch_bf16<ILT_Q2_K, TM, TN, NB>(p, token_tiles, st);
+    case ILT_IQ2_XXS: return launch_bf16<ILT_IQ2_XXS, TM, TN, NB>(p, token_tiles, st);
   }
   return hipErrorInvalidValue;
 }
@@ -397,15 +410,22 @@ hipError_t ilt_k_gemm_bf16(int fmt, const uint8_t* w, long long row_bytes, int r
   if (ntok <= 0 || rows <= 0) return hipSuccess;
   BfParams p = {};
   p.w = w; p.rows = rows; p.cols = cols; p.row_bytes = row_bytes; p.x = xb; p.y = y; p.bias = bias; p.acc = acc; p.ntok = ntok;
-  // Larger tiles dequantize and fetch less per product, but need enough tiles to fill the chip:
-  // 256x256 runs one workgroup per CU (256 slots), 128x256 two, 128x128 three.
-  const long long t256 = (ntok + 255) / 256, r256 = (rows + 255) / 256, r128 = (rows + 127) / 128;
-  const char* force = getenv("ILT_BF16_TILE");     // "1", "2", "3": the 128x128, 128x256, 256x256 tile whatever the shape (tests)
+  // Larger tiles fetch and dequantize less per product but leave more of the last round of
+  // workgroups idle.  Cost of a variant: rounds over the 256 CUs x tile area / its measured
+  // relative rate (128x128 0.85, 128x256 1.0, 256x256 1.1).
+  const long long t128 = (ntok + 127) / 128, t256 = (ntok + 255) / 256, r256 = (rows + 255) / 256, r128 = (rows + 127) / 128;
+  const char* force = getenv("ILT_BF16_TILE");     // "1".."4": that variant whatever the shape (tests)
   int tile = force ? atoi(force) : 0;
-  if (tile < 1 || tile > 3) tile = t256 * r256 >= 512 ? 3 : t256 * r128 >= 1024 ? 2 : 1;
-  if (tile == 3) return dispatch_bf16<256, 256>(fmt, p, t256, st);
-  if (tile == 2) return dispatch_bf16<128, 256>(fmt, p, t256, st);
-  return dispatch_bf16<128, 128>(fmt, p, (ntok + 127) / 128, st);
+  if (tile < 1 || tile > 4) {
+    const double c1 = (double)((t128 * r128 + 255) / 256) * 1.0 / 0.85;
+    const double c2 = (double)((t256 * r128 + 255) / 256) * 2.0 / 1.0;
+    const double c3 = (double)((t256 * r256 + 255) / 256) * 4.0 / 1.1;
+    tile = c3 <= c2 && c3 <= c1 ? 3 : c2 <= c1 ? 2 : 1;
+  }
+  if (tile == 4) return dispatch_bf16<256, 256, 4>(fmt, p, t256, st);
+  if (tile == 3) return dispatch_bf16<256, 256, 2>(fmt, p, t256, st);
+  if (tile == 2) return dispatch_bf16<128, 256, 2>(fmt, p, t256, st);
+  return dispatch_bf16<128, 128, 2>(fmt, p, t128, st);
 }
 
 hipError_t ilt_k_gemm_bf16_id(int fmt, const uint64_t* ptrs, long long add, const uint32_t* counts, const uint32_t* bases,
@@ -416,5 +436,5 @@ hipError_t ilt_k_gemm_bf16_id(int fmt, const uint64_t* ptrs, long long add, cons
   BfParams p = {};
   p.ptrs = ptrs; p.add = add; p.counts = counts; p.bases = bases; p.ne = ne;
   p.rows = rows; p.cols = cols; p.row_bytes = row_bytes; p.x = xb; p.y = y; p.ntok = (int)total_rows;
-  return dispatch_bf16<128, 128>(fmt, p, total_rows / 128 + ne, st);
+  return dispatch_bf16<128, 128, 2>(fmt, p, total_rows / 128 + ne, st);
 }
