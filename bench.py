@@ -1,23 +1,32 @@
 #!/usr/bin/env python3
 """bench.py -- the quantized matrix-product path on one MI355X.
 
-A step is one decoded token's worth of quantized products at the Qwen3-4B shape
-(BASELINE.json configs[1]): for each of 36 layers the activation quantizations and the
-seven matrix-vector products (Q4_K wq 4096x2560, wk 1024x2560, wo 2560x4096, gate and up
-9728x2560; Q6_K wv 1024x2560, down 2560x9728), then the Q6_K output head 151936x2560 --
-2,618,273,280 bytes of GGUF blocks streamed from HBM per step, every matrix its own
-allocation, so the working set (2.6 GB) is far beyond the 256 MB MALL.  Weights and
-activations are synthetic and seeded (illatio_amd/synth.py); inputs are resident in HBM
-before the timed region.  No attention, norm or RoPE runs in a step: those belong to the
-dense-forward harness, not to this path.
+The default workload (c2) is the one the metric is quoted on: a step is one decoded token's
+worth of quantized products at the Qwen3-4B shape (BASELINE.json configs[1]) -- for each of
+36 layers the activation quantizations and the seven matrix-vector products (Q4_K wq
+4096x2560, wk 1024x2560, wo 2560x4096, gate and up 9728x2560; Q6_K wv 1024x2560, down
+2560x9728), then the Q6_K output head 151936x2560: 2,618,273,280 bytes of GGUF blocks
+streamed from HBM per step, every matrix its own allocation, so the working set (2.6 GB)
+is far beyond the 256 MB MALL.  No attention, norm or RoPE runs in a step: those belong to
+the dense-forward harness, not to this path.
 
-Prints one JSON line: metric "Q-matvec achieved HBM GB/s ...", value = GB/s of GGUF bytes
-over the whole step, plus the roofline of the dominant kernel (timed with HIP events on the
-launch stream in a second pass over the same sequence) and the CPU oracle timed on a
-bounded sample of the same workload on this host.
+Other workloads (--workload), each BASELINE.json's config of the same number:
+  c1  Q8_0 decode GEMV 4864x896 and 896x4864, rotating over 64 copies (593 MB)
+  c3  Q6_K prefill product 17408x5120 on T tokens (--tokens, default 4096): bf16 matrix
+      cores (--path bf16, the float activations rounded to bf16 inside the step) or the
+      bit-exact int8 path (--path int8, the Q8_K activation quantizer inside the step)
+  c4  MoE decode step: 256 resident experts (IQ2_XXS gate/up, Q2_K down), top-6, the Q8_0
+      shared expert, rotating over 3 layers' pools (5.4 GB); routing tables made beforehand
+  c5  MoE prefill chunk: 4096 tokens, Zipf(1.1)-skewed top-6 routing, route -> group ->
+      gather -> grouped gate, up -> gated activation -> grouped down -> ordered sum
+Weights and activations are synthetic and seeded (illatio_amd/synth.py); inputs are resident
+in HBM before the timed region.
+
+Prints one JSON line: the metric, the roofline of the dominant kernel (timed with HIP events
+on the launch stream in a second pass over the same sequence) and the CPU oracle timed on a
+bounded sample of the same workload on this host's cores.
 """
 import argparse
-import ctypes as C
 import json
 import os
 import sys
@@ -30,92 +39,135 @@ sys.path.insert(0, ROOT)
 sys.path.insert(0, os.path.join(ROOT, "tests"))
 
 HBM_PEAK_GBS = 8000.0
+MFMA_PEAK_TFLOPS = {"bf16": 2500.0, "int8": 5000.0}
 
 D, FFN, QD, KVD, VOCAB, LAYERS = 2560, 9728, 4096, 1024, 151936, 36
 
 
-def layer_matrices():
-    from illatio_amd import synth
-    return [("wq", synth.Q4_K, QD, D, "x"), ("wk", synth.Q4_K, KVD, D, "x"), ("wv", synth.Q6_K, KVD, D, "x"),
-            ("wo", synth.Q4_K, D, QD, "att"), ("gate", synth.Q4_K, FFN, D, "x"), ("up", synth.Q4_K, FFN, D, "x"),
-            ("down", synth.Q6_K, D, FFN, "mid")]
+def host_cores():
+    cores = min(os.cpu_count() or 1, 64)
+    try:
+        cores = min(cores, len(os.sched_getaffinity(0)))
+    except AttributeError:
+        pass
+    return cores
 
 
-def main():
-    ap = argparse.ArgumentParser()
-    ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--layers", type=int, default=LAYERS, help=argparse.SUPPRESS)
-    ap.add_argument("--mode", default="fused", choices=["fused", "fused-q", "single"],
-                    help="fused: Q/K/V in one launch, gate+up in one, activations quantized inside the product "
-                         "kernels; fused-q: the same launches after separate quantizer launches; "
-                         "single: one launch per matrix after separate quantizer launches")
-    args = ap.parse_args()
-    if args.gpus != 1:
-        print("bench.py: this build runs on one GPU; --gpus N with N above 1 is not supported "
-              "(the path shards by rows / by experts, see DESIGN.md)", file=sys.stderr)
-        return 2
+class Timer:
+    """K steps timed between two syncs, wall clock and device events; then the same
+    sequence once more with an event pair around every launch that names a kernel."""
 
+    def __init__(self, dev):
+        from illatio_amd import hip
+        self.hip, self.dev, self.probes, self.probing = hip, dev, [], False
+
+    def launch(self, label, work, fn):
+        """Run FN (one kernel launch); WORK = its algorithmic bytes or flops."""
+        hip = self.hip
+        if self.probing:
+            e0, e1 = hip.hip_event_create(self.dev, True), hip.hip_event_create(self.dev, True)
+            hip.hip_event_record(e0, self.dev.stream)
+            fn()
+            hip.hip_event_record(e1, self.dev.stream)
+            self.probes.append((label, work, e0, e1))
+        else:
+            fn()
+
+    def run(self, step, steps, warmup, probe_steps=3, work_of=None):
+        """WORK_OF(kernel name, launch arguments) -> algorithmic work: when given, the probing
+        pass puts an event pair around every launch the host functions make, by kernel name."""
+        hip, dev = self.hip, self.dev
+        for i in range(warmup):
+            step(i)
+        hip.hip_sync(dev)
+        ev = [hip.hip_event_create(dev, timing=True) for _ in range(2)]
+        t0 = time.perf_counter()
+        hip.hip_event_record(ev[0], dev.stream)
+        for i in range(steps):
+            step(warmup + i)
+        hip.hip_event_record(ev[1], dev.stream)
+        self.enqueue_ms = (time.perf_counter() - t0) * 1e3 / steps     # host time to queue a step's launches
+        hip.hip_sync(dev)
+        wall_ms = (time.perf_counter() - t0) * 1e3
+        dev_ms = hip.hip_event_elapsed_ms(ev[0], ev[1])
+        self.probing = True
+        plain = hip.launch
+        if work_of:
+            def probed(d, kernel, grid, block, a, shared=0):
+                self.launch(kernel, work_of(kernel, a), lambda: plain(d, kernel, grid, block, a, shared))
+            hip.launch = probed
+        try:
+            for i in range(max(1, min(steps, probe_steps))):
+                step(warmup + steps + i)
+            hip.hip_sync(dev)
+        finally:
+            hip.launch = plain
+        self.probing = False
+        per = {}
+        for label, work, e0, e1 in self.probes:
+            t = per.setdefault(label, [0.0, 0, 0])
+            t[0] += hip.hip_event_elapsed_ms(e0, e1); t[1] += work; t[2] += 1
+            hip.hip_event_destroy(e0); hip.hip_event_destroy(e1)
+        return max(wall_ms, dev_ms) / steps, dev_ms / steps, per
+
+
+def roofline_of(per, bound, peak, unit, kernel_names):
+    """The dominant kernel's roofline entry from the per-label (ms, work, launches) sums."""
+    dom = max(per, key=lambda k: per[k][0])
+    ms, work, n = per[dom]
+    scale = 1e9 if unit == "GB/s" else 1e12
+    achieved = work / (ms * 1e-3) / scale
+    return {"bound": bound, "achieved": round(achieved, 1), "peak": peak, "unit": unit, "frac": round(achieved / peak, 4),
+            "traffic": None, "kernel": kernel_names.get(dom, dom), "launches": n, "avg_launch_us": round(ms / n * 1e3, 2),
+            "avg_work_per_launch": work // n,
+            "other_kernels": {kernel_names.get(k, k): {unit: round(v[1] / (v[0] * 1e-3) / scale, 1), "launches": v[2],
+                                                       "avg_launch_us": round(v[0] / v[2] * 1e3, 2)}
+                              for k, v in per.items() if k != dom and v[1]}}
+
+
+# ---------------------------------------------------------------------------------------------
+def workload_c2(args, dev):
     from illatio_amd import dense, hip, synth
-    dev = hip.open_hip(0)
     rng = synth.make_rng(42)
     nl = args.layers
-
-    # ---- weights: one seeded layer's bytes, uploaded to a separate allocation per layer ----
-    specs = layer_matrices()
+    specs = [("wq", synth.Q4_K, QD, D, "x"), ("wk", synth.Q4_K, KVD, D, "x"), ("wv", synth.Q6_K, KVD, D, "x"),
+             ("wo", synth.Q4_K, D, QD, "att"), ("gate", synth.Q4_K, FFN, D, "x"), ("up", synth.Q4_K, FFN, D, "x"),
+             ("down", synth.Q6_K, D, FFN, "mid")]
     host = {name: synth.weights(qt, rows, cols, rng) for name, qt, rows, cols, _ in specs}
-    layers = []
-    for li in range(nl):
-        layers.append({name: dense.upload_gmat(dev, f"blk.{li}.{name}", qt, rows, cols, host[name])
-                       for name, qt, rows, cols, _ in specs})
+    layers = [{name: dense.upload_gmat(dev, f"blk.{li}.{name}", qt, rows, cols, host[name])
+               for name, qt, rows, cols, _ in specs} for li in range(nl)]
     head_host = synth.weights(synth.Q6_K, VOCAB, D, rng)
     head = dense.upload_gmat(dev, "output", synth.Q6_K, VOCAB, D, head_host)
-    step_bytes = nl * sum(synth.row_bytes(qt, cols) * rows for _, qt, rows, cols, _ in specs) + head_host.size
+    wbytes = {name: synth.row_bytes(qt, cols) * rows for name, qt, rows, cols, _ in specs}
+    step_bytes = nl * sum(wbytes.values()) + head_host.size
 
-    # ---- activations (device resident) ----
     xin = {"x": D, "att": QD, "mid": FFN}
     xbuf = {k: hip.hip_upload_new(dev, synth.activations(n, rng)) for k, n in xin.items()}
     acts = {k: dense.QAct(dev, 1, n, ("q8k",)) for k, n in xin.items()}
     ybuf = {name: hip.hip_alloc(dev, 4 * rows) for name, _, rows, _, _ in specs}
     logits = hip.hip_alloc(dev, 4 * VOCAB)
-
-    ev = [hip.hip_event_create(dev, timing=True) for _ in range(2)]
-    probes = []          # (kernel label, bytes, start event, stop event) when profiling
-
-    wbytes = {name: synth.row_bytes(qt, cols) * rows for name, qt, rows, cols, _ in specs}
-
-    def timed(fn, nbytes, probe):
-        if probe:
-            e0, e1 = hip.hip_event_create(dev, True), hip.hip_event_create(dev, True)
-            hip.hip_event_record(e0, dev.stream)
-        fn()
-        if probe:
-            hip.hip_event_record(e1, dev.stream)
-            probes.append(("gemv_kernel", nbytes, e0, e1))
-
+    tm = Timer(dev)
     fused, inq = args.mode != "single", args.mode == "fused"
 
-    def step(probe=False):
+    def step(_):
         for L in layers:
             if fused:
                 xf = xbuf["x"] if inq else None
                 if not inq:
                     dense.quantize_act(dev, xbuf["x"], acts["x"])
-                timed(lambda: dense.qkv_mul(dev, L["wq"], L["wk"], L["wv"], acts["x"], ybuf["wq"], ybuf["wk"], ybuf["wv"], xf=xf),
-                      wbytes["wq"] + wbytes["wk"] + wbytes["wv"] + D + 4 * (QD + 2 * KVD), probe)
+                tm.launch("qkv", wbytes["wq"] + wbytes["wk"] + wbytes["wv"] + D + 4 * (QD + 2 * KVD),
+                          lambda: dense.qkv_mul(dev, L["wq"], L["wk"], L["wv"], acts["x"], ybuf["wq"], ybuf["wk"], ybuf["wv"], xf=xf))
                 if not inq:
                     dense.quantize_act(dev, xbuf["att"], acts["att"])
-                timed(lambda: dense.mv_multi(dev, [(L["wo"], ybuf["wo"], None)], acts["att"], xf=xbuf["att"] if inq else None),
-                      wbytes["wo"] + QD + 4 * D, probe)
+                tm.launch("wo", wbytes["wo"] + QD + 4 * D,
+                          lambda: dense.mv_multi(dev, [(L["wo"], ybuf["wo"], None)], acts["att"], xf=xbuf["att"] if inq else None))
                 if not inq:
                     dense.quantize_act(dev, xbuf["x"], acts["x"])
-                timed(lambda: dense.glu_mul(dev, L["gate"], L["up"], acts["x"], ybuf["gate"], xf=xf),
-                      wbytes["gate"] + wbytes["up"] + D + 4 * FFN, probe)
+                tm.launch("glu", wbytes["gate"] + wbytes["up"] + D + 4 * FFN,
+                          lambda: dense.glu_mul(dev, L["gate"], L["up"], acts["x"], ybuf["gate"], xf=xf))
                 # the down projection's input is 9728 wide: quantized once, not by every workgroup
                 dense.quantize_act(dev, xbuf["mid"], acts["mid"])
-                timed(lambda: dense.cmat_mul(dev, L["down"], acts["mid"], ybuf["down"]), wbytes["down"] + FFN + 4 * D, probe)
+                tm.launch("down", wbytes["down"] + FFN + 4 * D, lambda: dense.cmat_mul(dev, L["down"], acts["mid"], ybuf["down"]))
             else:
                 dense.quantize_act(dev, xbuf["x"], acts["x"])
                 for name, qt, rows, cols, src in specs:
@@ -125,81 +177,309 @@ def main():
                         dense.quantize_act(dev, xbuf["x"], acts["x"])
                     if name == "down":
                         dense.quantize_act(dev, xbuf["mid"], acts["mid"])
-                    timed(lambda: dense.cmat_mul(dev, L[name], acts[src], ybuf[name]), wbytes[name] + cols + 4 * rows, probe)
+                    tm.launch(name, wbytes[name] + cols + 4 * rows, lambda: dense.cmat_mul(dev, L[name], acts[src], ybuf[name]))
         if inq:
-            timed(lambda: dense.mv_multi(dev, [(head, logits, None)], xf=xbuf["x"]), head_host.size + D + 4 * VOCAB, probe)
+            tm.launch("head", head_host.size + D + 4 * VOCAB, lambda: dense.mv_multi(dev, [(head, logits, None)], xf=xbuf["x"]))
         else:
             dense.quantize_act(dev, xbuf["x"], acts["x"])
-            timed(lambda: dense.cmat_mul(dev, head, acts["x"], logits), head_host.size + D + 4 * VOCAB, probe)
+            tm.launch("head", head_host.size + D + 4 * VOCAB, lambda: dense.cmat_mul(dev, head, acts["x"], logits))
 
-    for _ in range(args.warmup):
-        step()
-    hip.hip_sync(dev)
-    t0 = time.perf_counter()
-    hip.hip_event_record(ev[0], dev.stream)
-    for _ in range(args.steps):
-        step()
-    hip.hip_event_record(ev[1], dev.stream)
-    hip.hip_sync(dev)
-    wall_ms = (time.perf_counter() - t0) * 1e3
-    dev_ms = hip.hip_event_elapsed_ms(ev[0], ev[1])
-    ms_per_step = max(wall_ms, dev_ms) / args.steps
-    gbs = step_bytes / (ms_per_step * 1e-3) / 1e9
+    ms, dev_ms, per = tm.run(step, args.steps, args.warmup)
+    # the roofline entry is the product kernel over all its launches of a step (one kernel, several shapes)
+    allk = [sum(v[0] for v in per.values()), sum(v[1] for v in per.values()), sum(v[2] for v in per.values())]
+    shapes = {k: {"GB/s": round(v[1] / (v[0] * 1e-3) / 1e9, 1), "avg_launch_us": round(v[0] / v[2] * 1e3, 2),
+                  "bytes_per_launch": v[1] // v[2]} for k, v in per.items()}
+    roof = roofline_of({"gemv": allk}, "hbm", HBM_PEAK_GBS, "GB/s",
+                       {"gemv": "gemv_kernel<FMT> (decode product: Q4_K, Q6_K and the fused Q4_K+Q6_K launch)"})
+    roof["by_launch_shape"] = shapes
+    gbs = step_bytes / (ms * 1e-3) / 1e9
 
-    # ---- roofline of the dominant kernel: HIP events around each launch, same sequence ----
-    for _ in range(max(1, min(args.steps, 5))):
-        step(probe=True)
-    hip.hip_sync(dev)
-    per = {}
-    for label, nbytes, e0, e1 in probes:
-        ms = hip.hip_event_elapsed_ms(e0, e1)
-        t = per.setdefault(label, [0.0, 0, 0])
-        t[0] += ms; t[1] += nbytes; t[2] += 1
-        hip.hip_event_destroy(e0); hip.hip_event_destroy(e1)
-    dom = max(per, key=lambda k: per[k][0])
-    dms, dbytes, dn = per[dom]
-    achieved = dbytes / (dms * 1e-3) / 1e9
-    roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
-                "kernel": "gemv_kernel<0> (dense Q4_K/Q6_K decode product)", "launches": dn, "avg_launch_us": round(dms / dn * 1e3, 2),
-                "avg_bytes_per_launch": dbytes // dn,
-                "other_kernels": {k: {"GB/s": round(v[1] / (v[0] * 1e-3) / 1e9, 1), "launches": v[2]}
-                                  for k, v in per.items() if k != dom}}
-
-    # ---- CPU baseline: the oracle (a C restatement of the reference's CPU path) on this host ----
-    cpu = None
-    if not args.no_cpu:
+    def cpu():
         import oracle_lib as orc
-        cores = min(os.cpu_count() or 1, 64)
-        try:
-            cores = min(cores, len(os.sched_getaffinity(0)))
-        except AttributeError:
-            pass
+        cores = host_cores()
         xs = {k: synth.activations(n, synth.make_rng(7)) for k, n in xin.items()}
-        sample_bytes, t_cpu, reps = 0, 0.0, 0
+        nbytes, t_cpu, reps = 0, 0.0, 0
         while t_cpu < 10.0 and reps < 4000:
             for name, qt, rows, cols, src in specs:
                 t1 = time.perf_counter()
                 orc.matmul(qt, host[name], rows, cols, xs[src], nthreads=cores)
                 t_cpu += time.perf_counter() - t1
-                sample_bytes += host[name].size
+                nbytes += host[name].size
             reps += 1
-        cpu = {"value": round(sample_bytes / t_cpu / 1e9, 3), "unit": "GB/s", "cores": cores, "kind": "port",
-               "sample": f"{reps} x one layer's seven products (activation quantization included), "
-                         f"{sample_bytes} weight bytes, {t_cpu:.1f} s",
-               "tok_per_s_equiv": round(sample_bytes / t_cpu / step_bytes, 3)}
+        return {"value": round(nbytes / t_cpu / 1e9, 3), "unit": "GB/s", "cores": cores, "kind": "port",
+                "sample": f"{reps} x one layer's seven products (activation quantization included), {nbytes} weight bytes, {t_cpu:.1f} s",
+                "tok_per_s_equiv": round(nbytes / t_cpu / step_bytes, 3)}
 
-    out = {"metric": "Q-matvec achieved HBM GB/s (% of 8 TB/s); decode tok/s at Qwen3-4B shape",
-           "value": round(gbs, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-           "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-           "dtype": "int8 block dots, fp32 combine", "data": "synthetic",
-           "config": {"workload": f"qwen3-4b-shape decode: the {nl * 7 + 1} quantized matvecs of one token "
-                                  f"({nl} layers x 7 + output head), Q4_K/Q6_K, batch 1",
-                      "bytes_per_step": step_bytes, "layers": nl, "launch_mode": args.mode},
-           "pct_of_hbm_peak": round(100 * gbs / HBM_PEAK_GBS, 2),
-           "matvec_only_tok_per_s": round(1e3 / ms_per_step, 1),
-           "device_ms_per_step": round(dev_ms / args.steps, 4),
-           "roofline": roofline, "cpu_baseline": cpu}
+    return {"value": round(gbs, 1), "unit": "GB/s", "ms_per_step": ms, "device_ms_per_step": dev_ms, "enqueue_ms": tm.enqueue_ms,
+            "dtype": "int8 block dots, fp32 combine",
+            "config": {"workload": f"c2: qwen3-4b-shape decode, the {nl * 7 + 1} quantized matvecs of one token "
+                                   f"({nl} layers x 7 + output head), Q4_K/Q6_K, batch 1",
+                       "bytes_per_step": step_bytes, "layers": nl, "launch_mode": args.mode},
+            "extra": {"pct_of_hbm_peak": round(100 * gbs / HBM_PEAK_GBS, 2), "matvec_only_tok_per_s": round(1e3 / ms, 1)},
+            "roofline": roof, "cpu": cpu}
+
+
+def workload_c1(args, dev):
+    from illatio_amd import dense, hip, synth
+    rng = synth.make_rng(11)
+    shapes = [("up", 4864, 896), ("down", 896, 4864)]
+    host = {n: synth.weights(synth.Q8_0, r, c, rng, dscale=0.02) for n, r, c in shapes}
+    ncopy = 64
+    mats = [{n: dense.upload_gmat(dev, n, synth.Q8_0, r, c, host[n]) for n, r, c in shapes} for _ in range(ncopy)]
+    xs = {n: synth.activations(c, rng) for n, r, c in shapes}
+    xb = {n: hip.hip_upload_new(dev, xs[n]) for n in xs}
+    ys = {n: hip.hip_alloc(dev, 4 * r) for n, r, c in shapes}
+    nbytes = {n: host[n].size + c // 32 * 34 + 4 * r for n, r, c in shapes}
+    step_bytes = sum(host[n].size for n in host)
+    tm = Timer(dev)
+
+    def step(i):
+        m = mats[i % ncopy]
+        for n, r, c in shapes:      # the activation quantizer runs inside the product kernel
+            tm.launch(n, nbytes[n], lambda: dense.mv_multi(dev, [(m[n], ys[n], None)], xf=xb[n]))
+
+    ms, dev_ms, per = tm.run(step, args.steps, args.warmup, probe_steps=20)
+    roof = roofline_of({"gemv": [sum(v[0] for v in per.values()), sum(v[1] for v in per.values()), sum(v[2] for v in per.values())]},
+                       "hbm", HBM_PEAK_GBS, "GB/s", {"gemv": "gemv_kernel<8> (Q8_0 decode product, activations quantized in the kernel)"})
+    gbs = step_bytes / (ms * 1e-3) / 1e9
+
+    def cpu():
+        import oracle_lib as orc
+        cores = host_cores()
+        nb, t_cpu, reps = 0, 0.0, 0
+        while t_cpu < 10.0 and reps < 20000:
+            for n, r, c in shapes:
+                t1 = time.perf_counter()
+                orc.matmul(synth.Q8_0, host[n], r, c, xs[n], nthreads=cores)
+                t_cpu += time.perf_counter() - t1
+                nb += host[n].size
+            reps += 1
+        return {"value": round(nb / t_cpu / 1e9, 3), "unit": "GB/s", "cores": cores, "kind": "port",
+                "sample": f"{reps} x both products (quantization included), {nb} weight bytes, {t_cpu:.1f} s"}
+
+    return {"value": round(gbs, 1), "unit": "GB/s", "ms_per_step": ms, "device_ms_per_step": dev_ms, "enqueue_ms": tm.enqueue_ms, "dtype": "int8 block dots, fp32 combine",
+            "config": {"workload": "c1: Q8_0 decode GEMV 4864x896 and 896x4864 (Qwen2-0.5B MLP), batch 1, rotating over 64 copies",
+                       "bytes_per_step": step_bytes},
+            "extra": {"pct_of_hbm_peak": round(100 * gbs / HBM_PEAK_GBS, 2)}, "roofline": roof, "cpu": cpu}
+
+
+def workload_c3(args, dev):
+    from illatio_amd import dense, hip, synth
+    rng = synth.make_rng(33)
+    rows, cols, T = (17408, 5120, args.tokens) if not args.transpose else (5120, 17408, args.tokens)
+    w = np.tile(synth.weights(synth.Q6_K, 256, cols, rng, dscale=0.01), (rows // 256, 1))
+    m = dense.upload_gmat(dev, "w", synth.Q6_K, rows, cols, w)
+    x = synth.activations((T, cols), rng)
+    xf = hip.hip_upload_new(dev, x)
+    y = hip.hip_alloc(dev, 4 * T * rows, zero=False)
+    flops = 2.0 * rows * cols * T
+    tm = Timer(dev)
+    if args.path == "bf16":
+        xb = hip.hip_alloc(dev, 2 * T * cols, zero=False)
+
+        def step(_):
+            tm.launch("cvt", 0, lambda: dense.cvt_bf16(dev, xf, T * cols, xb))
+            tm.launch("mm", flops, lambda: dense.cmat_mul_bf16(dev, m, xb, y, T))
+        names = {"mm": "gemm_bf16_kernel<14, TM, TN, NB> (Q6_K dequantized to bf16 in LDS, v_mfma_f32_32x32x16_bf16)"}
+    else:
+        act = dense.QAct(dev, T, cols, ("q8k",))
+
+        def step(_):
+            tm.launch("quant", 0, lambda: dense.quantize_act(dev, xf, act))
+            tm.launch("mm", flops, lambda: dense.cmat_mul(dev, m, act, y, n=T))
+        names = {"mm": "gemm_i8_kernel (Q6_K unpacked to int8 in LDS, v_mfma_i32_16x16x64_i8, bit-exact with the CPU path)"}
+    ms, dev_ms, per = tm.run(step, args.steps, args.warmup)
+    roof = roofline_of({k: v for k, v in per.items() if k == "mm"}, "mfma", MFMA_PEAK_TFLOPS[args.path], "TFLOP/s" if args.path == "bf16" else "TOP/s", names)
+    roof["unit"] = "TFLOP/s"
+    tf = flops / (ms * 1e-3) / 1e12
+
+    def cpu():
+        import oracle_lib as orc
+        cores = host_cores()
+        ts = 16
+        t1 = time.perf_counter()
+        reps = 0
+        while time.perf_counter() - t1 < 10.0:
+            orc.matmul(synth.Q6_K, w, rows, cols, x[:ts], nthreads=cores)
+            reps += 1
+        t_cpu = time.perf_counter() - t1
+        return {"value": round(2.0 * rows * cols * ts * reps / t_cpu / 1e12, 4), "unit": "TFLOP/s", "cores": cores, "kind": "port",
+                "sample": f"{reps} x the same matrix on {ts} tokens (quantization included), {t_cpu:.1f} s"}
+
+    return {"value": round(tf, 1), "unit": "TFLOP/s", "ms_per_step": ms, "device_ms_per_step": dev_ms, "enqueue_ms": tm.enqueue_ms,
+            "dtype": "bf16 x bf16, fp32 accumulate" if args.path == "bf16" else "int8 block dots, fp32 combine",
+            "metric": "prefill product TFLOP/s (% of dense MFMA peak)",
+            "config": {"workload": f"c3: Q6_K prefill product {rows}x{cols} on {T} tokens, {args.path} path "
+                                   f"(activation conversion inside the step)", "flops_per_step": flops, "tokens": T},
+            "extra": {"pct_of_mfma_peak": round(100 * tf / MFMA_PEAK_TFLOPS[args.path], 2)}, "roofline": roof, "cpu": cpu}
+
+
+def moe_weights(rng, ne_unique, ne, d, ff):
+    from illatio_amd import synth
+    reps = ne // ne_unique
+    gate = np.tile(synth.weights(synth.IQ2_XXS, ne_unique * ff, d, rng), (reps, 1))
+    up = np.tile(synth.weights(synth.IQ2_XXS, ne_unique * ff, d, rng), (reps, 1))
+    down = np.tile(synth.weights(synth.Q2_K, ne_unique * d, ff, rng), (reps, 1))
+    return gate, up, down
+
+
+def workload_c4(args, dev):
+    from illatio_amd import ds4f, hip, synth
+    import oracle_lib as orc
+    rng = synth.make_rng(44)
+    ne, nu, d, ff, nlayers = 256, 6, 4096, 2048, 3
+    gate, up, down = moe_weights(rng, 32, ne, d, ff)
+    sg, su = (synth.weights(synth.Q8_0, ff, d, rng) for _ in range(2))
+    sd = synth.weights(synth.Q8_0, d, ff, rng)
+    pools = [ds4f.ExpertPool(dev, ne, d, ff, gate, up, down) for _ in range(nlayers)]
+    shared = [ds4f.SharedExpert(dev, d, ff, sg, su, sd) for _ in range(nlayers)]
+    x = synth.activations(d, rng)
+    xb = hip.hip_upload_new(dev, x)
+    nsteps = args.steps + args.warmup + 3
+    tables, routes = [], []
+    for i in range(nsteps):                      # the reference routes on the CPU (cuda-ds4f.lisp:991-999); tables made beforehand
+        sel, w = orc.route(synth.activations(ne, rng), nu, 1.5)
+        routes.append((sel, w))
+        tables.append(ds4f.tail_tables(dev, pools[i % nlayers], sel, w))
+    ws = hip.Workspace(dev, 8 << 20)
+    iq, q2, q8 = synth.row_bytes(synth.IQ2_XXS, d), synth.row_bytes(synth.Q2_K, ff), 34
+    step_bytes = nu * (2 * ff * iq + d * q2) + 2 * ff * d // 32 * q8 + d * ff // 32 * q8
+    tm = Timer(dev)
+
+    def step(i):
+        ws.reset()
+        L = i % nlayers
+        sel, w = routes[i]
+        ds4f.ffn_tail(dev, pools[L], sel, w, xb, ds4f.ffn_shared(dev, shared[L], xb, 0.0, ws=ws), 0.0, ws=ws, tables=tables[i])
+
+    def work_of(kernel, a):          # weight bytes + quantized activations + float outputs of the product kernels
+        if kernel == "d4_mv_iq2_xxs":
+            return 2 * nu * ff * iq + d + d // 256 * 4 + 4 * 2 * nu * ff
+        if kernel == "d4_mv_q2_k":
+            return nu * (d * q2 + ff + ff // 256 * 4 + ff // 16 * 4) + 4 * nu * d
+        if kernel == "d4_mvq8":
+            return a[0] * a[1] // 32 * q8 + a[1] // 32 * 36 + 4 * a[0]
+        return 0
+
+    ms, dev_ms, per = tm.run(step, args.steps, args.warmup, probe_steps=3, work_of=work_of)
+    roof = roofline_of({k: v for k, v in per.items() if v[1]}, "hbm", HBM_PEAK_GBS, "GB/s",
+                       {"d4_mv_iq2_xxs": "gemv_kernel<16> (the 6 selected experts' IQ2_XXS gate and up, one launch over 12 matrices)",
+                        "d4_mv_q2_k": "gemv_kernel<10> (the 6 experts' Q2_K down)", "d4_mvq8": "gemv_kernel<8> (shared expert, Q8_0)"})
+    roof["launch_us_all"] = {k: round(v[0] / v[2] * 1e3, 2) for k, v in per.items()}
+    gbs = step_bytes / (ms * 1e-3) / 1e9
+
+    def cpu():
+        cores = host_cores()
+        t1, reps = time.perf_counter(), 0
+        while time.perf_counter() - t1 < 10.0:
+            sel, w = routes[reps % len(routes)]
+            orc.moe_routed(gate, up, down, d, ff, sel, w, 0.0, x, nthreads=cores)
+            orc.moe_shared(sg, su, sd, d, ff, 0.0, x, nthreads=cores)
+            reps += 1
+        t_cpu = time.perf_counter() - t1
+        return {"value": round(step_bytes * reps / t_cpu / 1e9, 3), "unit": "GB/s", "cores": cores, "kind": "port",
+                "sample": f"{reps} decode steps (6 routed experts + shared expert), {t_cpu:.1f} s"}
+
+    return {"value": round(gbs, 1), "unit": "GB/s", "ms_per_step": ms, "device_ms_per_step": dev_ms, "enqueue_ms": tm.enqueue_ms, "dtype": "int8 block dots, fp32 combine",
+            "metric": "MoE decode step achieved HBM GB/s (% of 8 TB/s)",
+            "config": {"workload": f"c4: MoE decode step, 256 resident experts (IQ2_XXS gate/up, Q2_K down) top-6 + Q8_0 shared expert, "
+                                   f"d 4096, ff 2048, batch 1, rotating over {nlayers} layers", "bytes_per_step": step_bytes},
+            "extra": {"pct_of_hbm_peak": round(100 * gbs / HBM_PEAK_GBS, 2), "launches_per_step": 12}, "roofline": roof, "cpu": cpu}
+
+
+def workload_c5(args, dev):
+    from illatio_amd import ds4f, hip, synth
+    import oracle_lib as orc
+    rng = synth.make_rng(55)
+    ne, nu, d, ff, n = 256, 6, 4096, 2048, args.tokens
+    gate, up, down = moe_weights(rng, 32, ne, d, ff)
+    pool = ds4f.ExpertPool(dev, ne, d, ff, gate, up, down)
+    norms = synth.activations((n, d), rng)
+    logits = synth.zipf_router_logits(n, ne, rng)
+    lb, nb = hip.hip_upload_new(dev, logits), hip.hip_upload_new(dev, norms)
+    sb = hip.hip_alloc(dev, 4 * n * d)
+    rows = n * nu
+    ws = hip.Workspace(dev, rows * (4 * d * 2 + 2 * d + 4 * ff * 3 + 2 * ff + d + ff + 4096) + 4 * n * d + (16 << 20))
+    flops = 2.0 * rows * 3 * ff * d
+    tm = Timer(dev)
+    fn = ds4f.ffn_routed_chunk_bf16 if args.path == "bf16" else ds4f.ffn_routed_chunk
+
+    def step(_):
+        ws.reset()
+        fn(dev, pool, lb, nb, sb, n, ne, nu, 1.5, 0.0, ws=ws)
+
+    def work_of(kernel, a):
+        if kernel == "d4_mm_id_bf16":
+            return 2.0 * rows * a[1] * a[2]
+        if kernel in ("d4_mm_id_iq2_xxs", "d4_mm_id_q2_k"):
+            return 2.0 * rows * a[0] * a[1]
+        return 0
+
+    ms, dev_ms, per = tm.run(step, args.steps, args.warmup, probe_steps=2, work_of=work_of)
+    # one grouped-product kernel template, three launches (gate, up: IQ2_XXS; down: Q2_K)
+    mm = [k for k in per if per[k][1]]
+    allmm = [sum(per[k][0] for k in mm), sum(per[k][1] for k in mm), sum(per[k][2] for k in mm)]
+    roof = roofline_of({"mm_id": allmm}, "mfma", MFMA_PEAK_TFLOPS[args.path], "TFLOP/s",
+                       {"mm_id": "gemm_bf16_kernel<16|10, 128, 128, 2> grouped (d4_mm_id_bf16: gate, up, down)" if args.path == "bf16"
+                        else "gemm_i8_kernel grouped (d4_mm_id_iq2_xxs x2, d4_mm_id_q2_k), bit-exact"})
+    roof["launch_us_all"] = {k: round(v[0] / v[2] * 1e3, 2) for k, v in per.items()}
+    tf = flops / (ms * 1e-3) / 1e12
+
+    def cpu():
+        cores = host_cores()
+        ts = 8
+        t1, reps = time.perf_counter(), 0
+        while time.perf_counter() - t1 < 10.0:
+            orc.moe_chunk(gate, up, down, d, ff, ne, nu, 1.5, 0.0, logits[:ts], norms[:ts], None, nthreads=cores)
+            reps += 1
+        t_cpu = time.perf_counter() - t1
+        return {"value": round(2.0 * ts * nu * 3 * ff * d * reps / t_cpu / 1e12, 4), "unit": "TFLOP/s", "cores": cores, "kind": "port",
+                "sample": f"{reps} chunks of {ts} tokens (48 rows each), {t_cpu:.1f} s"}
+
+    return {"value": round(tf, 1), "unit": "TFLOP/s", "ms_per_step": ms, "device_ms_per_step": dev_ms, "enqueue_ms": tm.enqueue_ms,
+            "dtype": "bf16 x bf16, fp32 accumulate" if args.path == "bf16" else "int8 block dots, fp32 combine",
+            "metric": "MoE prefill grouped product TFLOP/s (% of dense MFMA peak)",
+            "config": {"workload": f"c5: MoE prefill chunk, {n} tokens x top-6 of 256 experts (Zipf 1.1), IQ2_XXS gate/up, Q2_K down, "
+                                   f"d 4096, ff 2048, {args.path} path, routing to ordered sum", "flops_per_step": flops, "tokens": n},
+            "extra": {"pct_of_mfma_peak": round(100 * tf / MFMA_PEAK_TFLOPS[args.path], 2)}, "roofline": roof, "cpu": cpu}
+
+
+WORKLOADS = {"c1": workload_c1, "c2": workload_c2, "c3": workload_c3, "c4": workload_c4, "c5": workload_c5}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--workload", default="c2", choices=sorted(WORKLOADS))
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--layers", type=int, default=LAYERS, help=argparse.SUPPRESS)
+    ap.add_argument("--tokens", type=int, default=4096, help="c3, c5: tokens per step")
+    ap.add_argument("--transpose", action="store_true", help="c3: the 5120x17408 matrix")
+    ap.add_argument("--path", default="bf16", choices=["bf16", "int8"], help="c3, c5: which matrix-core path")
+    ap.add_argument("--mode", default="fused", choices=["fused", "fused-q", "single"],
+                    help="c2: fused = Q/K/V in one launch, gate+up in one, activations quantized inside the product "
+                         "kernels; fused-q = the same launches after separate quantizer launches; "
+                         "single = one launch per matrix after separate quantizer launches")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on one GPU; --gpus N with N above 1 is not supported "
+              "(the path shards by rows / by experts, see DESIGN.md)", file=sys.stderr)
+        return 2
+
+    from illatio_amd import hip
+    dev = hip.open_hip(0)
+    r = WORKLOADS[args.workload](args, dev)
+    out = {"metric": r.get("metric", "Q-matvec achieved HBM GB/s (% of 8 TB/s); decode tok/s at Qwen3-4B shape"),
+           "value": r["value"], "unit": r["unit"], "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+           "ms_per_step": round(r["ms_per_step"], 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+           "dtype": r["dtype"], "data": "synthetic", "config": r["config"]}
+    out.update(r["extra"])
+    out["device_ms_per_step"] = round(r["device_ms_per_step"], 4)
+    out["host_enqueue_ms_per_step"] = round(r["enqueue_ms"], 4)
+    out["roofline"] = r["roofline"]
+    out["cpu_baseline"] = None if args.no_cpu else r["cpu"]()
     print(json.dumps(out))
     return 0
 

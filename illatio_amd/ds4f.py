@@ -30,12 +30,14 @@ class ExpertPool:
         host[:, self.gate_bytes:2 * self.gate_bytes] = np.asarray(up, np.uint8).reshape(ne, self.gate_bytes)
         host[:, 2 * self.gate_bytes:2 * self.gate_bytes + self.down_bytes] = np.asarray(down, np.uint8).reshape(ne, self.down_bytes)
         self.pool = hip.hip_upload_new(dev, host)
+        self.ptrs = hip.hip_upload_new(dev, np.array([self.slot_ptr(e) for e in range(ne)], np.uint64))
 
     def slot_ptr(self, e):
         return self.pool.ptr + int(e) * self.slot_bytes
 
     def free(self):
         hip.hip_free(self.pool)
+        hip.hip_free(self.ptrs)
 
 
 class SharedExpert:
@@ -47,27 +49,33 @@ class SharedExpert:
         self.gate = upload_gmat(dev, "ffn_gate_shexp", Q8_0, ff, d, sgate)
         self.up = upload_gmat(dev, "ffn_up_shexp", Q8_0, ff, d, sup)
         self.down = upload_gmat(dev, "ffn_down_shexp", Q8_0, d, ff, sdown)
+        self.ones = None
 
     def free(self):
         for m in (self.gate, self.up, self.down):
             m.free()
+        hip.hip_free(self.ones)
 
 
-def _q8k(dev, x, n_elems):
-    kq, kd = hip.hip_alloc(dev, n_elems), hip.hip_alloc(dev, 4 * n_elems // 256)
-    ks = hip.hip_alloc(dev, 4 * n_elems // 16)
+def _q8k(dev, x, n_elems, alloc=hip.hip_alloc):
+    kq, kd = alloc(dev, n_elems), alloc(dev, 4 * n_elems // 256)
+    ks = alloc(dev, 4 * n_elems // 16)
     hip.launch(dev, "quant_q8k", n_elems // 256, 256, [x, kq, kd, ks, hip.I64(n_elems // 256)])
     return kq, kd, ks
 
 
-def ffn_shared(dev, sh, norm2, clamp, n=1):
-    """The shared expert of N tokens' NORM2 (DK-FFN-HEAD's second half): returns SOUT."""
+def ffn_shared(dev, sh, norm2, clamp, n=1, ws=None):
+    """The shared expert of N tokens' NORM2 (DK-FFN-HEAD's second half): returns SOUT.
+    With a Workspace WS nothing is allocated, freed or waited for."""
     d, ff = sh.d, sh.ff
-    qn_q, qn_s = hip.hip_alloc(dev, n * d), hip.hip_alloc(dev, 4 * n * d // 32)
-    sg, su, smid = (hip.hip_alloc(dev, 4 * n * ff) for _ in range(3))
-    qm_q, qm_s = hip.hip_alloc(dev, n * ff), hip.hip_alloc(dev, 4 * n * ff // 32)
-    sout = hip.hip_alloc(dev, 4 * n * d)
-    one = hip.hip_upload_new(dev, np.ones(n, np.float32))
+    A = ws.alloc if ws else hip.hip_alloc
+    qn_q, qn_s = A(dev, n * d), A(dev, 4 * n * d // 32)
+    sg, su, smid = (A(dev, 4 * n * ff) for _ in range(3))
+    qm_q, qm_s = A(dev, n * ff), A(dev, 4 * n * ff // 32)
+    sout = A(dev, 4 * n * d)
+    if getattr(sh, "ones", None) is None or sh.ones.bytes < 4 * n:
+        sh.ones = hip.hip_upload_new(dev, np.ones(n, np.float32))
+    one = sh.ones
     hip.launch(dev, "d4_quant", (n * d + 255) // 256, 256, [norm2, qn_q, qn_s, n * d // 32])
     if n == 1:
         hip.launch(dev, "d4_mvq8", (ff + 3) // 4, 128, [ff, d, ff, sh.gate.qs, sh.gate.d, qn_q, qn_s, sg])
@@ -80,53 +88,67 @@ def ffn_shared(dev, sh, norm2, clamp, n=1):
         hip.launch(dev, "d4_mvq8", (d + 3) // 4, 128, [d, ff, d, sh.down.qs, sh.down.d, qm_q, qm_s, sout])
     else:
         hip.launch(dev, "mm_q8", ((n + 63) // 64, (d + 63) // 64), 256, [sh.down.qs, sh.down.d, qm_q, qm_s, sout, None, d, ff, n, 0])
+    if ws:
+        return sout
     hip.hip_sync(dev)
-    for b in (qn_q, qn_s, sg, su, smid, qm_q, qm_s, one):
+    for b in (qn_q, qn_s, sg, su, smid, qm_q, qm_s):
         hip.hip_free(b)
     return sout
 
 
-def ffn_tail(dev, pool, sel, w, norm2, sout, clamp, keep=None):
-    """One token's routed experts SEL (weights W) on NORM2, summed in SEL's order with the
-    shared expert's SOUT (DK-FFN-TAIL): gate and up in one launch over 2k matrices, the
-    gated activation, each slot's Q8_K quantization, down, the ordered sum.  Returns MOE."""
-    d, ff, k = pool.d, pool.ff, len(sel)
+def tail_tables(dev, pool, sel, w):
+    """The device tables DK-FFN-TAIL's kernels take for one token: the 2k matrix addresses
+    (the selected experts' gates, then their ups) and the k weights."""
     gb = pool.gate_bytes
     ptrs = hip.hip_upload_new(dev, np.array([pool.slot_ptr(e) for e in sel] + [pool.slot_ptr(e) + gb for e in sel], np.uint64))
-    bw = hip.hip_upload_new(dev, np.asarray(w, np.float32))
-    bgu, bm = hip.hip_alloc(dev, 4 * 2 * k * ff), hip.hip_alloc(dev, 4 * k * ff)
-    bd, moe = hip.hip_alloc(dev, 4 * k * d), hip.hip_alloc(dev, 4 * d)
-    xq, xd, xs = _q8k(dev, norm2, d)
+    return ptrs, hip.hip_upload_new(dev, np.asarray(w, np.float32))
+
+
+def ffn_tail(dev, pool, sel, w, norm2, sout, clamp, keep=None, ws=None, tables=None):
+    """One token's routed experts SEL (weights W) on NORM2, summed in SEL's order with the
+    shared expert's SOUT (DK-FFN-TAIL): gate and up in one launch over 2k matrices, the
+    gated activation, each slot's Q8_K quantization, down, the ordered sum.  Returns MOE.
+    With a Workspace WS nothing is allocated, freed or waited for; TABLES = tail_tables()
+    made beforehand."""
+    d, ff, k = pool.d, pool.ff, len(sel)
+    gb = pool.gate_bytes
+    A = ws.alloc if ws else hip.hip_alloc
+    ptrs, bw = tables if tables else tail_tables(dev, pool, sel, w)
+    bgu, bm = A(dev, 4 * 2 * k * ff), A(dev, 4 * k * ff)
+    bd, moe = A(dev, 4 * k * d), A(dev, 4 * d)
+    xq, xd, xs = _q8k(dev, norm2, d, A)
     hip.launch(dev, "d4_mv_iq2_xxs", ((ff + 7) // 8, 1, 2 * k), 64,
                [d, ff, pool.grb, hip.I64(0), 0, ff, ptrs, None, xq, bgu, xd, xs])
     hip.launch(dev, "d4_swiglu_w", (k * ff + 255) // 256, 256, [k, ff, float(clamp), bgu, bgu.at(4 * k * ff), bw, bm, None, None])
-    mq, md, ms = _q8k(dev, bm, k * ff)
+    mq, md, ms = _q8k(dev, bm, k * ff, A)
     hip.launch(dev, "d4_mv_q2_k", ((d + 7) // 8, 1, k), 64,
                [ff, d, pool.drb, hip.I64(2 * gb), ff, d, ptrs, None, mq, bd, md, ms])
     hip.launch(dev, "d4_moe_sum", (d + 255) // 256, 256, [d, k, bd, sout, moe, None])
+    if ws:
+        return moe
     hip.hip_sync(dev)
     if keep is not None:
         keep["mid"] = hip.hip_floats(bm, k * ff).reshape(k, ff)
         keep["gu"] = hip.hip_floats(bgu, 2 * k * ff).reshape(2, k, ff)
         keep["down"] = hip.hip_floats(bd, k * d).reshape(k, d)
-    for b in (ptrs, bw, bgu, bm, bd, xq, xd, xs, mq, md, ms):
+    for b in (bgu, bm, bd, xq, xd, xs, mq, md, ms) + (() if tables else (ptrs, bw)):
         hip.hip_free(b)
     return moe
 
 
-def route(dev, logits, n, ne, nu, scale, bias=None):
+def route(dev, logits, n, ne, nu, scale, bias=None, alloc=hip.hip_alloc):
     """D4_ROUTE for N tokens' LOGITS (a DBuf): returns (sel, w) DBufs of N x NU."""
-    sel, w = hip.hip_alloc(dev, 4 * n * nu), hip.hip_alloc(dev, 4 * n * nu)
+    sel, w = alloc(dev, 4 * n * nu), alloc(dev, 4 * n * nu)
     hip.launch(dev, "d4_route", n, ne, [ne, nu, 0, float(scale), 1 if bias is not None else 0, logits, bias, None, None, sel, w],
                shared=4 * (2 * ne + 64 + nu))
     return sel, w
 
 
-def group_rows(dev, sel, w, n, ne, nu):
+def group_rows(dev, sel, w, n, ne, nu, alloc=hip.hip_alloc):
     """The N x NU (token, slot) rows grouped by expert (D4_GROUP_*): returns a dict of DBufs
     counts, bases (per expert), rmap (row -> token), smap ((token, slot) -> row), wrow."""
     rows = n * nu
-    g = {k: hip.hip_alloc(dev, 4 * (ne if k in ("counts", "bases") else rows)) for k in
+    g = {k: alloc(dev, 4 * (ne if k in ("counts", "bases") else rows)) for k in
          ("counts", "bases", "rank", "rmap", "smap", "wrow")}
     hip.launch(dev, "d4_group_zero", (ne + 255) // 256, min(ne, 256), [ne, g["counts"]])
     hip.launch(dev, "d4_group_count", (rows + 255) // 256, 256, [rows, ne, nu, sel, g["counts"], g["rank"]])
@@ -136,21 +158,23 @@ def group_rows(dev, sel, w, n, ne, nu):
     return g
 
 
-def ffn_routed_chunk_bf16(dev, pool, logits, norm2, sout, n, ne, nu, scale, clamp, bias=None, keep=None):
+def ffn_routed_chunk_bf16(dev, pool, logits, norm2, sout, n, ne, nu, scale, clamp, bias=None, keep=None, ws=None):
     """FFN-ROUTED-CHUNK with the three grouped products on the bf16 matrix cores: the same
     routing, grouping, gated activation and slot-ordered sum, no activation quantizers.
-    Within 2e-2 of the CPU path's chunk; the routing and grouping stay exact."""
+    Within 2e-2 of the CPU path's chunk; the routing and grouping stay exact.  With a
+    Workspace WS nothing is allocated, freed or waited for."""
     d, ff = pool.d, pool.ff
     rows = n * nu
     gb = pool.gate_bytes
-    sel, w = route(dev, logits, n, ne, nu, scale, bias)
-    g = group_rows(dev, sel, w, n, ne, nu)
-    ptrs = hip.hip_upload_new(dev, np.array([pool.slot_ptr(e) for e in range(ne)], np.uint64))
-    x = hip.hip_alloc(dev, 4 * rows * d)
+    A = ws.alloc if ws else hip.hip_alloc
+    sel, w = route(dev, logits, n, ne, nu, scale, bias, A)
+    g = group_rows(dev, sel, w, n, ne, nu, A)
+    ptrs = pool.ptrs
+    x = A(dev, 4 * rows * d)
     hip.launch(dev, "d4_gather_rows", (rows * d + 255) // 256, 256, [d, rows, norm2, g["rmap"], x])
-    xb = dense.cvt_bf16(dev, x, rows * d)
-    gg, gu, mid = (hip.hip_alloc(dev, 4 * rows * ff) for _ in range(3))
-    down, moe = hip.hip_alloc(dev, 4 * rows * d), hip.hip_alloc(dev, 4 * n * d)
+    xb = dense.cvt_bf16(dev, x, rows * d, A(dev, 2 * rows * d))
+    gg, gu, mid = (A(dev, 4 * rows * ff) for _ in range(3))
+    down, moe = A(dev, 4 * rows * d), A(dev, 4 * n * d)
 
     def mm_id(qtype, ncols, nrows, rb, add, xin, yout):
         hip.launch(dev, "d4_mm_id_bf16", (rows // 128 + ne, (nrows + 127) // 128), 256,
@@ -159,9 +183,11 @@ def ffn_routed_chunk_bf16(dev, pool, logits, norm2, sout, n, ne, nu, scale, clam
     mm_id(IQ2_XXS, d, ff, pool.grb, 0, xb, gg)
     mm_id(IQ2_XXS, d, ff, pool.grb, gb, xb, gu)
     hip.launch(dev, "d4_swiglu_w", (rows * ff + 255) // 256, 256, [rows, ff, float(clamp), gg, gu, g["wrow"], mid, None, None])
-    mb = dense.cvt_bf16(dev, mid, rows * ff)
+    mb = dense.cvt_bf16(dev, mid, rows * ff, A(dev, 2 * rows * ff))
     mm_id(Q2_K, ff, d, pool.drb, 2 * gb, mb, down)
     hip.launch(dev, "d4_moe_sum_rows", (n * d + 255) // 256, 256, [d, nu, n, down, g["smap"], sout, moe])
+    if ws:
+        return moe
     hip.hip_sync(dev)
     if keep is not None:
         keep["sel"] = hip.hip_download(sel, np.uint32, rows).reshape(n, nu)
@@ -171,29 +197,30 @@ def ffn_routed_chunk_bf16(dev, pool, logits, norm2, sout, n, ne, nu, scale, clam
         keep["x"], keep["mid"] = hip.hip_floats(x, rows * d).reshape(rows, d), hip.hip_floats(mid, rows * ff).reshape(rows, ff)
         keep["gate"], keep["up"] = (hip.hip_floats(b, rows * ff).reshape(rows, ff) for b in (gg, gu))
         keep["down"] = hip.hip_floats(down, rows * d).reshape(rows, d)
-    for b in [sel, w, ptrs, x, xb, mb, gg, gu, mid, down] + list(g.values()):
+    for b in [sel, w, x, xb, mb, gg, gu, mid, down] + list(g.values()):
         hip.hip_free(b)
     return moe
 
 
-def ffn_routed_chunk(dev, pool, logits, norm2, sout, n, ne, nu, scale, clamp, bias=None, keep=None):
+def ffn_routed_chunk(dev, pool, logits, norm2, sout, n, ne, nu, scale, clamp, bias=None, keep=None, ws=None):
     """A chunk of N tokens past the router (DK-FFN-ROUTED-CHUNK): each token's experts and
     weights (d4_route), the (token, slot) rows grouped by expert, the rows gathered and
     quantized, every expert's gate, up and down as one grouped product each over its rows
     (d4_mm_id_*), the gated activation between, then each token's rows summed in slot order
     with the shared expert's SOUT.  LOGITS (N x NE), NORM2 (N x D) and SOUT (N x D) are
-    DBufs; returns MOE (N x D)."""
+    DBufs; returns MOE (N x D).  With a Workspace WS nothing is allocated, freed or waited for."""
     d, ff = pool.d, pool.ff
     rows = n * nu
     gb = pool.gate_bytes
-    sel, w = route(dev, logits, n, ne, nu, scale, bias)
-    g = group_rows(dev, sel, w, n, ne, nu)
-    ptrs = hip.hip_upload_new(dev, np.array([pool.slot_ptr(e) for e in range(ne)], np.uint64))
-    x = hip.hip_alloc(dev, 4 * rows * d)
+    A = ws.alloc if ws else hip.hip_alloc
+    sel, w = route(dev, logits, n, ne, nu, scale, bias, A)
+    g = group_rows(dev, sel, w, n, ne, nu, A)
+    ptrs = pool.ptrs
+    x = A(dev, 4 * rows * d)
     hip.launch(dev, "d4_gather_rows", (rows * d + 255) // 256, 256, [d, rows, norm2, g["rmap"], x])
-    xq, xd, xs = _q8k(dev, x, rows * d)
-    gg, gu, mid = (hip.hip_alloc(dev, 4 * rows * ff) for _ in range(3))
-    down, moe = hip.hip_alloc(dev, 4 * rows * d), hip.hip_alloc(dev, 4 * n * d)
+    xq, xd, xs = _q8k(dev, x, rows * d, A)
+    gg, gu, mid = (A(dev, 4 * rows * ff) for _ in range(3))
+    down, moe = A(dev, 4 * rows * d), A(dev, 4 * n * d)
 
     def mm_id(kernel, ncols, nrows, rb, add, xin, yout):
         hip.launch(dev, kernel, ((n + 63) // 64, (nrows + 63) // 64, ne), 128,
@@ -203,14 +230,16 @@ def ffn_routed_chunk(dev, pool, logits, norm2, sout, n, ne, nu, scale, clamp, bi
     mm_id("d4_mm_id_iq2_xxs", d, ff, pool.grb, 0, (xq, xd, None), gg)
     mm_id("d4_mm_id_iq2_xxs", d, ff, pool.grb, gb, (xq, xd, None), gu)
     hip.launch(dev, "d4_swiglu_w", (rows * ff + 255) // 256, 256, [rows, ff, float(clamp), gg, gu, g["wrow"], mid, None, None])
-    mq, md, ms = _q8k(dev, mid, rows * ff)
+    mq, md, ms = _q8k(dev, mid, rows * ff, A)
     mm_id("d4_mm_id_q2_k", ff, d, pool.drb, 2 * gb, (mq, md, ms), down)
     hip.launch(dev, "d4_moe_sum_rows", (n * d + 255) // 256, 256, [d, nu, n, down, g["smap"], sout, moe])
+    if ws:
+        return moe
     hip.hip_sync(dev)
     if keep is not None:
         keep["sel"] = hip.hip_download(sel, np.uint32, rows).reshape(n, nu)
         keep["w"] = hip.hip_floats(w, rows).reshape(n, nu)
         keep["counts"] = hip.hip_download(g["counts"], np.uint32, ne)
-    for b in [sel, w, ptrs, x, xq, xd, xs, gg, gu, mid, mq, md, ms, down] + list(g.values()):
+    for b in [sel, w, x, xq, xd, xs, gg, gu, mid, mq, md, ms, down] + list(g.values()):
         hip.hip_free(b)
     return moe

@@ -123,9 +123,38 @@ def hip_alloc(dev, nbytes, zero=True):
 
 
 def hip_free(b):
-    if b is not None and b.ptr:
+    if b is not None and b.ptr and not isinstance(b, _Slice):
         call("ilt_free", C.c_uint64(b.ptr))
         b.ptr = 0
+
+
+class _Slice(DBuf):
+    """A DBuf carved out of a Workspace: freed with it, not by hip_free."""
+    __slots__ = ()
+
+
+class Workspace:
+    """One device allocation handed out in 256-byte-aligned pieces, for a sequence of launches
+    that must not allocate or free between them (the reference's hosts keep such buffers in
+    their state structs, e.g. DKSTATE, cuda-ds4f.lisp:395-428).  alloc has hip_alloc's
+    signature; reset() starts over; pieces are not zeroed."""
+
+    def __init__(self, dev, nbytes):
+        self.dev, self.buf, self.used = dev, hip_alloc(dev, nbytes, zero=False), 0
+
+    def alloc(self, dev, nbytes, zero=False):
+        n = (max(int(nbytes), 256) + 255) // 256 * 256
+        if self.used + n > self.buf.bytes:
+            raise MemoryError(f"workspace of {self.buf.bytes} bytes is full")
+        b = _Slice(self.buf.ptr + self.used, int(nbytes), dev)
+        self.used += n
+        return hip_zero(b) if zero else b
+
+    def reset(self):
+        self.used = 0
+
+    def free(self):
+        hip_free(self.buf)
 
 
 def hip_zero(b):
