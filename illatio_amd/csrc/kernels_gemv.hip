@@ -253,7 +253,7 @@ __device__ __forceinline__ void first_load(Raw<FMT>& r, const u8* w, const u16* 
 
 template <int FMT>
 __device__ __forceinline__ void wave_rows(const u8* w, const u16* wd, long row0, int nrows, int S, u32 s_magic,
-                                          long row_bytes, const Lds& L, float* t, int lane, const Raw<FMT>* pre) {
+                                          long row_bytes, const Lds& L, float* t, int lane, const Raw<FMT>& pre, bool use_pre) {
   using F = Fmt<FMT>;
   constexpr int GPW = ILT_WAVE / F::LPB;           // blocks per wave step
   const int j = lane % F::LPB, gl = lane / F::LPB;
@@ -269,7 +269,8 @@ __device__ __forceinline__ void wave_rows(const u8* w, const u16* wd, long row0,
   }
   int f = gl;
   Raw<FMT> ra, rb;
-  if (pre) ra = *pre; else load_raw<FMT>(ra, wr, wdr, min(f, last), j);
+  // (no pointer to the preloaded set anywhere: a set whose address is taken lives in scratch memory)
+  if (use_pre) ra = pre; else load_raw<FMT>(ra, wr, wdr, min(f, last), j);
   int k = 0;
   for (; k + 2 <= nfull; k += 2) {
     load_raw<FMT>(rb, wr, wdr, min(f + GPW, last), j);
@@ -369,9 +370,9 @@ __device__ __forceinline__ void stage_q8_from_f32(const float* __restrict__ x, i
 
 template <int FMT>
 __device__ __forceinline__ void run_rows(const IltGemvMat& m, const IltGemvParams& p, long row0, int nrows, int S,
-                                         const Lds& L, float* t, int lane, int z, const Raw<FMT>* pre) {
+                                         const Lds& L, float* t, int lane, int z, const Raw<FMT>& pre, bool use_pre) {
   const u8* w = p.ptrs ? (const u8*)(p.ptrs[z] + p.add) : m.w;
-  wave_rows<FMT>(w, m.wd, row0, nrows, S, p.s_magic, m.row_bytes, L, t, lane, pre);
+  wave_rows<FMT>(w, m.wd, row0, nrows, S, p.s_magic, m.row_bytes, L, t, lane, pre, use_pre);
 }
 
 // FSET: one format (its GGUF number), or 0 = the launch's matrices mix Q4_K and Q6_K
@@ -383,10 +384,10 @@ template <int FSET> struct Pre {
 
 template <int FSET>
 __device__ __forceinline__ void run_any(const IltGemvMat& m, const IltGemvParams& p, long row0, int nrows, int S,
-                                        const Lds& L, float* t, int lane, int z, const Pre<FSET>* pre) {
-  if (FSET != 0) run_rows<(FSET ? FSET : ILT_Q4_K)>(m, p, row0, nrows, S, L, t, lane, z, pre ? &pre->a : nullptr);
-  else if (m.fmt == ILT_Q4_K) run_rows<ILT_Q4_K>(m, p, row0, nrows, S, L, t, lane, z, (const Raw<ILT_Q4_K>*)(pre ? &pre->a : nullptr));
-  else run_rows<ILT_Q6_K>(m, p, row0, nrows, S, L, t, lane, z, (const Raw<ILT_Q6_K>*)(pre ? &pre->b : nullptr));
+                                        const Lds& L, float* t, int lane, int z, const Pre<FSET>& pre, bool use_pre) {
+  if constexpr (FSET != 0) run_rows<FSET>(m, p, row0, nrows, S, L, t, lane, z, pre.a, use_pre);
+  else if (m.fmt == ILT_Q4_K) run_rows<ILT_Q4_K>(m, p, row0, nrows, S, L, t, lane, z, pre.a, use_pre);
+  else run_rows<ILT_Q6_K>(m, p, row0, nrows, S, L, t, lane, z, pre.b, use_pre);
 }
 
 __device__ __forceinline__ float sum_any(int fmt, const float* t, int S) {
@@ -484,8 +485,8 @@ __global__ __launch_bounds__(kThreads) void gemv_kernel(IltGemvParams p) {
     locate(b, mi, row0, nrows);
     const IltGemvMat& m = p.mat[mi];
     const int fmt = FSET != 0 ? FSET : m.fmt;
-    run_any<FSET>(m, p, row0, nrows, S, L, tw, lane, z, b == wid ? &pre : nullptr);
-    if (p.glu) run_any<FSET>(p.mat[1], p, row0, nrows, S, L, tw + (long)RB * tpr, lane, z, nullptr);   // up's same rows
+    run_any<FSET>(m, p, row0, nrows, S, L, tw, lane, z, pre, b == wid);
+    if (p.glu) run_any<FSET>(p.mat[1], p, row0, nrows, S, L, tw + (long)RB * tpr, lane, z, pre, false);   // the same rows of up
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
