@@ -25,6 +25,7 @@ struct IltGemvMat {
   int rows;
   int fmt;                   // ILT_Q8_0, ILT_Q4_K, ILT_Q6_K (dense); the expert kernels ignore it
   int batch0, nbat;          // this matrix's first batch among the launch's, and how many (set at launch)
+  int rq, rr;                // rows / nbat and rows % nbat: batch i is rq rows, one more for the first rr (set at launch)
 };
 
 struct IltGemvParams {

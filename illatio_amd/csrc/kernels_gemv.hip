@@ -294,57 +294,61 @@ __device__ __forceinline__ void wave_rows(const u8* w, const u16* wd, long row0,
 __device__ __forceinline__ float dense_glu(float g, float u) { return (g / (1.0f + ilt_expf_via_double(-g))) * u; }
 
 // ---- activation staging: copy quantized x, or quantize fp32 x here --------------------------------
-__device__ __forceinline__ float wave_max(float v) {     // the same value in every lane
-  v = ilt_max16(v);
-  const float a = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 0));
-  const float b = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 16));
-  const float c = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 32));
-  const float d = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 48));
-  return fmaxf(fmaxf(a, b), fmaxf(c, d));
+// Q8_K (quantize-q8k!, kquant.lisp:130-167): 16 lanes a block of 256, so a wave quantizes four
+// blocks at once and every reduction stays inside a 16-lane DPP row.  Lane l of a row holds
+// the values 4*(l+16i)+c (i, c = 0..3).  The largest-magnitude value, the first of equals,
+// sets iscale = -127/max.
+__device__ __forceinline__ int ilt_min16(int v) {
+  v = min(v, ilt_dpp<ILT_DPP_XOR1>(v)); v = min(v, ilt_dpp<ILT_DPP_XOR2>(v));
+  v = min(v, ilt_dpp<ILT_DPP_HALF_MIRROR>(v)); return min(v, ilt_dpp<ILT_DPP_ROW_MIRROR>(v));
+}
+__device__ __forceinline__ int ilt_or16(int v) {
+  v |= ilt_dpp<ILT_DPP_XOR1>(v); v |= ilt_dpp<ILT_DPP_XOR2>(v);
+  v |= ilt_dpp<ILT_DPP_HALF_MIRROR>(v); return v | ilt_dpp<ILT_DPP_ROW_MIRROR>(v);
 }
 
-// Q8_K (quantize-q8k!, kquant.lisp:130-167): a wave a block of 256, four values a lane; the
-// largest-magnitude value, the first of equals, sets iscale = -127/max.  The loads of up
-// to four of the wave's blocks go out together.
 __device__ __forceinline__ void stage_q8k_from_f32(const float* __restrict__ x, int nblk, i8* lxq, float* lxs, int* lbs) {
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  for (int b0 = wave; b0 < nblk; b0 += 4 * kWaves) {
-    float4 vs[4];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, g = lane >> 4, l = lane & 15;
+  for (int b0 = 4 * wave; b0 < nblk; b0 += 4 * kWaves) {
+    const int b = b0 + g;
+    const bool live = b < nblk;
+    float v[16];
 #pragma unroll
-    for (int u = 0; u < 4; u++) {
-      const int b = b0 + u * kWaves;
-      vs[u] = b < nblk ? *(const float4*)(x + b * 256 + 4 * lane) : make_float4(0.f, 0.f, 0.f, 0.f);
+    for (int i = 0; i < 4; i++) {
+      const float4 t = live ? *(const float4*)(x + b * 256 + 4 * (l + 16 * i)) : make_float4(0.f, 0.f, 0.f, 0.f);
+      v[4 * i] = t.x; v[4 * i + 1] = t.y; v[4 * i + 2] = t.z; v[4 * i + 3] = t.w;
     }
+    float am = 0.0f;
 #pragma unroll
-    for (int u = 0; u < 4; u++) {
-      const int b = b0 + u * kWaves;
-      if (b >= nblk) break;
-      const float4 v = vs[u];
-      const float amax = wave_max(fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w))));
-      int q0 = 0, q1 = 0, q2 = 0, q3 = 0;
-      float d = 0.0f;
-      if (amax != 0.0f) {
-        // the first position holding the maximum: lowest lane per component, then lowest index
-        const u64 m0 = __ballot(fabsf(v.x) == amax), m1 = __ballot(fabsf(v.y) == amax);
-        const u64 m2 = __ballot(fabsf(v.z) == amax), m3 = __ballot(fabsf(v.w) == amax);
-        int idx = 1 << 20;
-        if (m0) idx = min(idx, 4 * (int)__builtin_ctzll(m0));
-        if (m1) idx = min(idx, 4 * (int)__builtin_ctzll(m1) + 1);
-        if (m2) idx = min(idx, 4 * (int)__builtin_ctzll(m2) + 2);
-        if (m3) idx = min(idx, 4 * (int)__builtin_ctzll(m3) + 3);
-        const int src = __builtin_amdgcn_readfirstlane(idx >> 2), e = __builtin_amdgcn_readfirstlane(idx & 3);
-        const float pick = e == 0 ? v.x : e == 1 ? v.y : e == 2 ? v.z : v.w;
-        const float mx = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(pick), src));
-        const float iscale = -127.0f / mx;
-        q0 = min(127, (int)rintf(iscale * v.x)); q1 = min(127, (int)rintf(iscale * v.y));
-        q2 = min(127, (int)rintf(iscale * v.z)); q3 = min(127, (int)rintf(iscale * v.w));
-        d = 1.0f / iscale;
+    for (int k = 0; k < 16; k++) am = fmaxf(am, fabsf(v[k]));
+    const float amax = ilt_max16(am);
+    // this lane's first position holding the maximum (its values are in rising position order), and the value there
+    int idx = 1 << 20;
+    float val = 0.0f;
+#pragma unroll
+    for (int k = 15; k >= 0; k--) {
+      const bool hit = fabsf(v[k]) == amax;
+      idx = hit ? 4 * (l + 16 * (k >> 2)) + (k & 3) : idx;
+      val = hit ? v[k] : val;
+    }
+    const int first = ilt_min16(idx);
+    const float mx = __int_as_float(ilt_or16(idx == first ? __float_as_int(val) : 0));
+    const bool nz = amax != 0.0f;
+    const float iscale = nz ? -127.0f / mx : 0.0f;
+    const float d = nz ? 1.0f / iscale : 0.0f;
+    int q[16];
+#pragma unroll
+    for (int k = 0; k < 16; k++) q[k] = nz ? min(127, (int)rintf(iscale * v[k])) : 0;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      const int s = ilt_sum4(q[4 * i] + q[4 * i + 1] + q[4 * i + 2] + q[4 * i + 3]);
+      if (live) {
+        *(int*)(lxq + b * XP + 4 * (l + 16 * i)) =
+            (q[4 * i] & 0xFF) | ((q[4 * i + 1] & 0xFF) << 8) | ((q[4 * i + 2] & 0xFF) << 16) | ((q[4 * i + 3] & 0xFF) << 24);
+        if ((l & 3) == 0) lbs[b * 16 + (l >> 2) + 4 * i] = s;
       }
-      *(int*)(lxq + b * XP + 4 * lane) = (q0 & 0xFF) | ((q1 & 0xFF) << 8) | ((q2 & 0xFF) << 16) | ((q3 & 0xFF) << 24);
-      const int s = ilt_sum4(q0 + q1 + q2 + q3);
-      if ((lane & 3) == 0) lbs[b * 16 + (lane >> 2)] = s;
-      if (lane == 0) lxs[b] = d;
     }
+    if (live && l == 0) lxs[b] = d;
   }
 }
 
@@ -431,16 +435,15 @@ __global__ __launch_bounds__(kThreads) void gemv_kernel(IltGemvParams p) {
   auto locate = [&](int b, int& mi, long& row0, int& nrows) {
     mi = 0;
     if (!p.glu) while (mi + 1 < p.nmat && b >= p.mat[mi + 1].batch0) mi++;
-    // batch bl of nbat deals out the rows evenly: [rows*bl/nbat, rows*(bl+1)/nbat)
-    const long rows = p.group_rows > 0 ? p.group_rows : p.mat[mi].rows;
-    const long bl = b - p.mat[mi].batch0, nbat = p.mat[mi].nbat;
-    row0 = rows * bl / nbat;
-    nrows = (int)(rows * (bl + 1) / nbat - row0);
-    row0 += grow0;
+    // the rows dealt out evenly over the matrix's batches: rq each, one more for the first rr
+    const int bl = b - p.mat[mi].batch0, rq = p.mat[mi].rq, rr = p.mat[mi].rr;
+    row0 = (long)bl * rq + min(bl, rr) + grow0;
+    nrows = rq + (bl < rr ? 1 : 0);
   };
 
   // the first batch's first loads go out now, so they are on their way while x is staged
   Pre<FSET> pre;
+  int warm[4] = {0, 0, 0, 0};
   if (wid < p.nbatches) {
     int mi; long row0; int nrows;
     locate(wid, mi, row0, nrows);
@@ -451,9 +454,12 @@ __global__ __launch_bounds__(kThreads) void gemv_kernel(IltGemvParams p) {
     // and a touch of every 64-byte line of the batch's first 16 KB, so the later steps hit in L2
     const u8* wb = w0 + row0 * m.row_bytes;
     const long bytes = (long)nrows * m.row_bytes;
-    int warm = 0;
-    for (long o = 64L * lane; o < bytes && o < 16384; o += 64 * 64) warm ^= *(const int*)(wb + (o & ~3L));
-    asm volatile("" :: "v"(warm));
+    // (the values are looked at only when the kernel ends: nothing waits for these loads here)
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      const long o = 64L * lane + 4096L * i;
+      if (o < bytes) warm[i] = *(const int*)(wb + (o & ~3L));
+    }
   }
 
   // ---- stage the activations ----
@@ -508,6 +514,7 @@ __global__ __launch_bounds__(kThreads) void gemv_kernel(IltGemvParams p) {
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
   }
+  asm volatile("" :: "v"(warm[0]), "v"(warm[1]), "v"(warm[2]), "v"(warm[3]));
 }
 
 size_t gemv_smem(int fset, const IltGemvParams& p) {
@@ -518,6 +525,30 @@ size_t gemv_smem(int fset, const IltGemvParams& p) {
   b += 4 * (size_t)S + 8;
   if (fset == ILT_IQ2_XXS) b += 2048;
   return b + (size_t)kWaves * p.batch * S * (q8 ? 1 : 2) * 4 * (p.glu ? 2 : 1);
+}
+
+// Workgroups of variant FSET with SMEM bytes of LDS that one CU holds at a time (asked of the
+// runtime once per variant and LDS size, kept per device 0..7).
+int resident_per_cu(int fset, size_t smem) {
+  static int cache[8][6][65];       // [device][variant][LDS KB], 0 = not asked yet
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 8) dev = 0;
+  const int v = fset == 0 ? 0 : fset == ILT_Q8_0 ? 1 : fset == ILT_Q4_K ? 2 : fset == ILT_Q6_K ? 3 : fset == ILT_Q2_K ? 4 : 5;
+  int& c = cache[dev][v][(smem + 1023) / 1024];
+  if (c == 0) {
+    int n = 0;
+    hipError_t e = hipErrorInvalidValue;
+    switch (v) {
+      case 0: e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, gemv_kernel<0>, kThreads, smem); break;
+      case 1: e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, gemv_kernel<ILT_Q8_0>, kThreads, smem); break;
+      case 2: e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, gemv_kernel<ILT_Q4_K>, kThreads, smem); break;
+      case 3: e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, gemv_kernel<ILT_Q6_K>, kThreads, smem); break;
+      case 4: e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, gemv_kernel<ILT_Q2_K>, kThreads, smem); break;
+      default: e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, gemv_kernel<ILT_IQ2_XXS>, kThreads, smem); break;
+    }
+    c = (e == hipSuccess && n > 0) ? n : 1;
+  }
+  return c;
 }
 
 }  // namespace
@@ -541,7 +572,13 @@ hipError_t ilt_gemv_launch(IltGemvParams& p, int nz, hipStream_t st) {
   if ((size_t)rb_max * row_terms > 32768) rb_max = (int)(32768 / row_terms);
   if (rb_max < 1) rb_max = 1;
   const long all_rows = rows_each * nz * ngroups;
-  int m = 4;
+  p.batch = rb_max;
+  const size_t smem = gemv_smem(fset, p);
+  if (smem > 64 * 1024) return hipErrorInvalidValue;
+  // no more workgroups than are resident at once (registers and LDS decide how many a CU
+  // holds): a second round of workgroups would start only when the first has finished
+  int m = resident_per_cu(fset, smem);
+  if (m > 4) m = 4;
   while (m > 1 && all_rows < 3L * 1024 * m) m--;               // at least three rows a wave on average
   int waves_each = 1024 * m / (nz * ngroups) / kWaves * kWaves;  // waves per (grid y, group)
   if (waves_each < kWaves) waves_each = kWaves;
@@ -549,16 +586,17 @@ hipError_t ilt_gemv_launch(IltGemvParams& p, int nz, hipStream_t st) {
   const int rounds = (int)((rows_each + (long)waves_each * rb_max - 1) / ((long)waves_each * rb_max));
   long nb_total = (long)waves_each * rounds;
   if (nb_total > rows_each) nb_total = rows_each;
-  p.batch = rb_max;
   int nb = 0;
   for (int i = 0; i < p.nmat; i++) {
     p.mat[i].batch0 = nb;
-    if (i >= nm) { p.mat[i].nbat = p.mat[0].nbat; continue; }
+    if (i >= nm) { p.mat[i].nbat = p.mat[0].nbat; p.mat[i].rq = p.mat[0].rq; p.mat[i].rr = p.mat[0].rr; continue; }
     const long r = p.group_rows > 0 ? p.group_rows : p.mat[i].rows;
     long nbi = (nb_total * r + rows_each - 1) / rows_each;       // this matrix's share of the batches
     if (nbi < (r + rb_max - 1) / rb_max) nbi = (r + rb_max - 1) / rb_max;
     if (nbi > r) nbi = r;
     p.mat[i].nbat = (int)nbi;
+    p.mat[i].rq = (int)(r / nbi);
+    p.mat[i].rr = (int)(r % nbi);
     nb += (int)nbi;
   }
   p.nbatches = nb;                                                          // per group, per grid y
@@ -566,8 +604,6 @@ hipError_t ilt_gemv_launch(IltGemvParams& p, int nz, hipStream_t st) {
   const int wgs = waves_each / kWaves;
   p.wgs_per_group = wgs;
   dim3 grid(wgs * ngroups, nz);
-  const size_t smem = gemv_smem(fset, p);
-  if (smem > 64 * 1024) return hipErrorInvalidValue;
   switch (fset) {
     case 0: hipLaunchKernelGGL(gemv_kernel<0>, grid, dim3(kThreads), smem, st, p); break;
     case ILT_Q8_0: hipLaunchKernelGGL(gemv_kernel<ILT_Q8_0>, grid, dim3(kThreads), smem, st, p); break;
