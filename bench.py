@@ -38,6 +38,30 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 sys.path.insert(0, os.path.join(ROOT, "tests"))
 
+# HBM bytes per launch of the product kernels, from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE
+# (KiB per dispatch; profiles/traffic_*.txt): FETCH_SIZE reads 0.500 of what a plain streaming
+# kernel of known size fetches (cvt_bf16: 83,886,080 bytes read, counter 40,971 KiB), WRITE_SIZE
+# reads 1.000 (same kernel: 41,943,040 bytes written, counter 40,960 KiB); so bytes =
+# (2 * FETCH_SIZE + WRITE_SIZE) * 1024.
+def _t(fetch_kib, write_kib):
+    return int((2 * fetch_kib + write_kib) * 1024)
+
+
+TRAFFIC = {"c1": {"up": _t(2407.5, 22.0), "down": _t(2347.5, 7.0)},
+           "c2": {"qkv": _t(4862.4, 33.3), "wo": _t(3041.5, 12.0), "glu": _t(13843.7, 48.0), "down": _t(10239.8, 12.0),
+                  "head": _t(176130.8, 638.9)},
+           "c3": {"mm": _t(519278.8, 282880.0)},
+           "c4": {"d4_mv_iq2_xxs": _t(13388.0, 96.4), "d4_mv_q2_k": _t(8223.3, 96.4), "d4_mvq8": _t(4430.6, 10.7)},
+           "c5": {"d4_mm_id_bf16": _t((2 * 366921.8 + 388488.5) / 3, (2 * 196608.0 + 393216.0) / 3)}}
+
+
+def traffic_of(workload, per):
+    """Measured HBM bytes per launch, averaged over the launches the roofline entry covers."""
+    t = TRAFFIC.get(workload, {})
+    n = sum(v[2] for k, v in per.items() if k in t)
+    return int(sum(t[k] * v[2] for k, v in per.items() if k in t) / n) if n else None
+
+
 HBM_PEAK_GBS = 8000.0
 MFMA_PEAK_TFLOPS = {"bf16": 2500.0, "int8": 5000.0}
 
@@ -192,6 +216,7 @@ def workload_c2(args, dev):
     roof = roofline_of({"gemv": allk}, "hbm", HBM_PEAK_GBS, "GB/s",
                        {"gemv": "gemv_kernel<FMT> (decode product: Q4_K, Q6_K and the fused Q4_K+Q6_K launch)"})
     roof["by_launch_shape"] = shapes
+    roof["traffic"] = traffic_of("c2", per) if (args.mode == "fused" and nl == LAYERS) else None
     gbs = step_bytes / (ms * 1e-3) / 1e9
 
     def cpu():
@@ -241,6 +266,7 @@ def workload_c1(args, dev):
     ms, dev_ms, per = tm.run(step, args.steps, args.warmup, probe_steps=20)
     roof = roofline_of({"gemv": [sum(v[0] for v in per.values()), sum(v[1] for v in per.values()), sum(v[2] for v in per.values())]},
                        "hbm", HBM_PEAK_GBS, "GB/s", {"gemv": "gemv_kernel<8> (Q8_0 decode product, activations quantized in the kernel)"})
+    roof["traffic"] = traffic_of("c1", per)
     gbs = step_bytes / (ms * 1e-3) / 1e9
 
     def cpu():
@@ -291,6 +317,8 @@ def workload_c3(args, dev):
     ms, dev_ms, per = tm.run(step, args.steps, args.warmup)
     roof = roofline_of({k: v for k, v in per.items() if k == "mm"}, "mfma", MFMA_PEAK_TFLOPS[args.path], "TFLOP/s" if args.path == "bf16" else "TOP/s", names)
     roof["unit"] = "TFLOP/s"
+    if args.path == "bf16" and T == 4096 and not args.transpose:
+        roof["traffic"] = traffic_of("c3", per)
     tf = flops / (ms * 1e-3) / 1e12
 
     def cpu():
@@ -366,6 +394,8 @@ def workload_c4(args, dev):
                        {"d4_mv_iq2_xxs": "gemv_kernel<16> (the 6 selected experts' IQ2_XXS gate and up, one launch over 12 matrices)",
                         "d4_mv_q2_k": "gemv_kernel<10> (the 6 experts' Q2_K down)", "d4_mvq8": "gemv_kernel<8> (shared expert, Q8_0)"})
     roof["launch_us_all"] = {k: round(v[0] / v[2] * 1e3, 2) for k, v in per.items()}
+    dom = max((k for k in per if per[k][1]), key=lambda k: per[k][0])
+    roof["traffic"] = TRAFFIC["c4"].get(dom)
     gbs = step_bytes / (ms * 1e-3) / 1e9
 
     def cpu():
@@ -423,6 +453,8 @@ def workload_c5(args, dev):
                        {"mm_id": "gemm_bf16_kernel<16|10, 128, 128, 2> grouped (d4_mm_id_bf16: gate, up, down)" if args.path == "bf16"
                         else "gemm_i8_kernel grouped (d4_mm_id_iq2_xxs x2, d4_mm_id_q2_k), bit-exact"})
     roof["launch_us_all"] = {k: round(v[0] / v[2] * 1e3, 2) for k, v in per.items()}
+    if args.path == "bf16" and n == 4096:
+        roof["traffic"] = TRAFFIC["c5"]["d4_mm_id_bf16"]
     tf = flops / (ms * 1e-3) / 1e12
 
     def cpu():
