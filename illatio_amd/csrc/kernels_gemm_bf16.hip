@@ -92,7 +92,10 @@ template <> __device__ __forceinline__ void load_w<ILT_IQ2_XXS>(WRaw<ILT_IQ2_XXS
 
 __device__ __forceinline__ u32 word_of(const int4& v, int i) { return (u32)(i == 0 ? v.x : i == 1 ? v.y : i == 2 ? v.z : v.w); }
 
-// 16 weights as floats, in column order, each computed as the CPU dequantizers compute it.
+// 16 weights as floats, in column order, each with the CPU dequantizers' value.  Where the CPU
+// multiplies then subtracts (d1*q - m1, dl*q - ml) the product is exact in fp32 (a 17-bit
+// scale times a 2- or 4-bit integer), and Q6_K's s*(q-32) is one rounding of an exact value;
+// so a fused multiply-add gives the same bits in half the instructions.
 // j: the step within the half super-block (a constant after unrolling); c: which half.
 template <int FMT> __device__ __forceinline__ void dequant16(const WRaw<FMT>& r, int j, int c, int e, const u64* grid, float* o);
 
@@ -107,20 +110,20 @@ template <> __device__ __forceinline__ void dequant16<ILT_Q4_K>(const WRaw<ILT_Q
   for (int i = 0; i < 4; i++) {
     const u32 v = (word_of(q, i) >> (4 * hl)) & 0x0F0F0F0F;
 #pragma unroll
-    for (int k = 0; k < 4; k++) o[4 * i + k] = d1 * (float)((v >> (8 * k)) & 0xFF) - m1;
+    for (int k = 0; k < 4; k++) o[4 * i + k] = __builtin_fmaf(d1, (float)((v >> (8 * k)) & 0xFF), -m1);   // d1*q is exact in fp32
   }
 }
 
 template <> __device__ __forceinline__ void dequant16<ILT_Q6_K>(const WRaw<ILT_Q6_K>& r, int j, int c, int e, const u64*, float* o) {
   const int h = j >> 1;                          // 32-weight part j of the half: ql[j&1]'s nibble h, qh's bit pair j
   const u32 scw = (u32)(j < 2 ? r.sc.x : r.sc.y) >> (16 * (j & 1) + 8 * e);
-  const float s = ilt_h2f((u16)r.d) * (float)(i8)(scw & 0xFF);
+  const float s = ilt_h2f((u16)r.d) * (float)(i8)(scw & 0xFF), s32 = -32.0f * s;
   const int4& ql = r.ql[j & 1];
 #pragma unroll
   for (int i = 0; i < 4; i++) {
     const u32 v = ((word_of(ql, i) >> (4 * h)) & 0x0F0F0F0F) | (((word_of(r.qh, i) >> (2 * j)) & 0x03030303) << 4);
 #pragma unroll
-    for (int k = 0; k < 4; k++) o[4 * i + k] = s * (float)((int)((v >> (8 * k)) & 0xFF) - 32);
+    for (int k = 0; k < 4; k++) o[4 * i + k] = __builtin_fmaf(s, (float)((v >> (8 * k)) & 0xFF), s32);   // = RN(s*(q-32)): one rounding either way
   }
 }
 
@@ -131,7 +134,7 @@ template <> __device__ __forceinline__ void dequant16<ILT_Q2_K>(const WRaw<ILT_Q
   for (int i = 0; i < 4; i++) {
     const u32 v = (word_of(r.q, i) >> (2 * j)) & 0x03030303;
 #pragma unroll
-    for (int k = 0; k < 4; k++) o[4 * i + k] = dl * (float)((v >> (8 * k)) & 0xFF) - ml;
+    for (int k = 0; k < 4; k++) o[4 * i + k] = __builtin_fmaf(dl, (float)((v >> (8 * k)) & 0xFF), -ml);   // dl*q is exact in fp32
   }
 }
 
@@ -161,9 +164,9 @@ struct BfParams {
   float* y; const float* bias; int acc; int ntok;
 };
 
-template <int TM, int TN> struct Smem {
-  __align__(16) u8 xs[3][TN * KS * 2];
-  __align__(16) u8 ws[2][TM * KS * 2];
+template <int TM, int TN, int NXS, int NWS> struct Smem {
+  __align__(16) u8 xs[NXS][TN * KS * 2];
+  __align__(16) u8 ws[NWS][TM * KS * 2];
   u64 grid[256];
   u32 scan[256];
   int tile_z, tile_t0, tile_n;
@@ -183,7 +186,7 @@ template <int TM, int NB> constexpr int bf16_threads() { return 64 * 2 * (TM / (
 
 template <int FMT, int TM, int TN, int NB>
 __global__ __launch_bounds__((bf16_threads<TM, NB>()), (TM == 256 ? 1 : TN == 256 ? 2 : 3)) void gemm_bf16_kernel(BfParams p) {
-  __shared__ Smem<TM, TN> S;
+  __shared__ Smem<TM, TN, (NB == 4 ? 4 : 3), (NB == 4 ? 3 : 2)> S;
   constexpr int THREADS = bf16_threads<TM, NB>();
   constexpr int NE = 2 * TM / THREADS;   // 16-column units of a row a thread dequantizes per step: 1 or 2
   constexpr int NA = TN / 64;            // 32-token patches per wave
@@ -273,24 +276,101 @@ __global__ __launch_bounds__((bf16_threads<TM, NB>()), (TM == 256 ? 1 : TN == 25
 #pragma unroll
     for (int i = 0; i < NI; i++) ilt_g2lds16(xbase + ks * (KS * 2) + xoff[i], S.xs[stage] + (wave * NI + i) * 1024);
   };
+  auto dequant_unit = [&](const WRaw<FMT>& raw, int u, int j, int c, u8* ws) {   // 16 weights of step j of a half into a slab
+    float o[16];
+    dequant16<FMT>(raw, j, c, e0 + u, S.grid, o);
+    u32 pk[8];
+#pragma unroll
+    for (int i = 0; i < 8; i++) pk[i] = pack_bf16(o[2 * i], o[2 * i + 1]);
+    ilt_lds_st16_untracked(ws + (wdst ^ (32 * u)), pk[0], pk[1], pk[2], pk[3]);
+    ilt_lds_st16_untracked(ws + (wdst ^ (32 * u) ^ 16), pk[4], pk[5], pk[6], pk[7]);
+  };
   auto dequant_to = [&](const WRaw<FMT>* raw, int j, int c, int slab) {   // step j of a half's weights into a slab
 #pragma unroll
-    for (int u = 0; u < NE; u++) {
-      float o[16];
-      dequant16<FMT>(raw[u], j, c, e0 + u, S.grid, o);
-      u32 pk[8];
-#pragma unroll
-      for (int i = 0; i < 8; i++) pk[i] = pack_bf16(o[2 * i], o[2 * i + 1]);
-      u8* ws = S.ws[slab];
-      ilt_lds_st16_untracked(ws + (wdst ^ (32 * u)), pk[0], pk[1], pk[2], pk[3]);
-      ilt_lds_st16_untracked(ws + (wdst ^ (32 * u) ^ 16), pk[4], pk[5], pk[6], pk[7]);
-    }
+    for (int u = 0; u < NE; u++) dequant_unit(raw[u], u, j, c, S.ws[slab]);
   };
   auto load_raw = [&](WRaw<FMT>* raw, int hb) {
 #pragma unroll
     for (int u = 0; u < NE; u++) load_w<FMT>(raw[u], rw, wrowoff, hb, e0 + u);
   };
 
+  if constexpr (NB == 4) {
+    // One wave per SIMD, 128x128 per wave: everything is one step deeper so that nothing waits
+    // after the barrier.  Step ks dequantizes step ks+2's weights (three weight slabs) and
+    // sends off step ks+3's x loads (four x slabs); the MFMA fragments are loaded half a step
+    // ahead: while the first 16 columns' MFMAs run, the second 16 columns' fragments are read,
+    // and under those MFMAs the next step's first fragments (its slabs were published by the
+    // barrier at the start of this step).
+    WRaw<FMT> rawa[NE], rawb[NE];
+    load_raw(rawa, 0);
+    issue_x(0, 0);
+    load_raw(rawb, 1);
+    issue_x(1, 1);
+    issue_x(2, 2);
+    dequant_to(rawa, 0, 0, 0);
+    dequant_to(rawa, 1, 0, 1);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    ilt_barrier_lds();
+    int x0 = 0, x1 = 1, x2 = 2, x3 = 3;      // x ring: the step's slab, the next step's, ..., the one being filled
+    int w0 = 0, w1 = 1, w2 = 2;              // weight ring: the step's, the next step's, the one being written
+    v8bf fa[NA], fb[NB], ga[NA], gb[NB];
+#pragma unroll
+    for (int a = 0; a < NA; a++) fa[a] = *(const v8bf*)(S.xs[0] + aoff[a]);
+#pragma unroll
+    for (int b = 0; b < NB; b++) fb[b] = *(const v8bf*)(S.ws[0] + boff[b]);
+    auto step = [&](int ks, auto Jc) {
+      constexpr int J = decltype(Jc)::value;
+      constexpr int J2 = (J + 2) & 7;        // the step whose weights are dequantized now: 0..3 from rawa, 4..7 from rawb
+      if (J == 2) load_raw(rawa, min((ks >> 2) + 2, nh - 1));   // rawa's last use was during step 1
+      if (J == 6) load_raw(rawb, min((ks >> 2) + 2, nh - 1));
+      issue_x(x3, min(ks + 3, nk - 1));
+      __builtin_amdgcn_sched_barrier(0);
+      u8* wnew = S.ws[w2];
+      {
+        const u8* xs = S.xs[x0];
+        const u8* ws = S.ws[w0];
+#pragma unroll
+        for (int a = 0; a < NA; a++) ga[a] = *(const v8bf*)(xs + (aoff[a] ^ 32));
+#pragma unroll
+        for (int b = 0; b < NB; b++) gb[b] = *(const v8bf*)(ws + (boff[b] ^ 32));
+        dequant_unit((J2 < 4 ? rawa : rawb)[0], 0, J2 & 3, J2 >> 2, wnew);
+#pragma unroll
+        for (int a = 0; a < NA; a++)
+#pragma unroll
+          for (int b = 0; b < NB; b++) acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[a], fb[b], acc[a][b], 0, 0, 0);
+      }
+      {
+        const u8* xs = S.xs[x1];
+        const u8* ws = S.ws[w1];
+#pragma unroll
+        for (int a = 0; a < NA; a++) fa[a] = *(const v8bf*)(xs + aoff[a]);
+#pragma unroll
+        for (int b = 0; b < NB; b++) fb[b] = *(const v8bf*)(ws + boff[b]);
+        dequant_unit((J2 < 4 ? rawa : rawb)[1], 1, J2 & 3, J2 >> 2, wnew);
+#pragma unroll
+        for (int a = 0; a < NA; a++)
+#pragma unroll
+          for (int b = 0; b < NB; b++) acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ga[a], gb[b], acc[a][b], 0, 0, 0);
+      }
+      { const int t_ = x0; x0 = x1; x1 = x2; x2 = x3; x3 = t_; }
+      { const int t_ = w0; w0 = w1; w1 = w2; w2 = t_; }
+      // every load older than this step's has landed: this wave's share of x slab ks+2, which
+      // the next step reads; the barrier publishes it and the weight slab written just now
+      constexpr int mine = NI + ((J == 2 || J == 6) ? WL : 0);
+      asm volatile("s_waitcnt vmcnt(%0)" :: "n"(mine) : "memory");
+      ilt_barrier_lds();
+    };
+    for (int ks = 0; ks < nk; ks += 8) {
+      step(ks + 0, std::integral_constant<int, 0>{});
+      step(ks + 1, std::integral_constant<int, 1>{});
+      step(ks + 2, std::integral_constant<int, 2>{});
+      step(ks + 3, std::integral_constant<int, 3>{});
+      step(ks + 4, std::integral_constant<int, 4>{});
+      step(ks + 5, std::integral_constant<int, 5>{});
+      step(ks + 6, std::integral_constant<int, 6>{});
+      step(ks + 7, std::integral_constant<int, 7>{});
+    }
+  } else {
   // Two register sets of raw weights, each a half super-block (4 steps): rawa holds half 0
   // of a super-block, rawb half 1.  Step ks multiplies slab ks while it dequantizes step
   // ks+1's weights into the other weight slab; a set is reloaded, with the half two ahead,
@@ -345,6 +425,7 @@ __global__ __launch_bounds__((bf16_threads<TM, NB>()), (TM == 256 ? 1 : TN == 25
     step(ks + 5, std::integral_constant<int, 5>{});
     step(ks + 6, std::integral_constant<int, 6>{});
     step(ks + 7, std::integral_constant<int, 7>{});
+  }
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // the tail's redundant loads: nothing may land in LDS after the workgroup ends
 
