@@ -16,7 +16,8 @@ Other workloads (--workload), each BASELINE.json's config of the same number:
       cores (--path bf16, the float activations rounded to bf16 inside the step) or the
       bit-exact int8 path (--path int8, the Q8_K activation quantizer inside the step)
   c4  MoE decode step: 256 resident experts (IQ2_XXS gate/up, Q2_K down), top-6, the Q8_0
-      shared expert, rotating over 3 layers' pools (5.4 GB); routing tables made beforehand
+      shared expert, rotating over 3 layers' pools (5.4 GB); routing tables made beforehand;
+      --mode fused (default): 5 launches a step; --mode single: the reference's 12
   c5  MoE prefill chunk: 4096 tokens, Zipf(1.1)-skewed top-6 routing, route -> group ->
       gather -> grouped gate, up -> gated activation -> grouped down -> ordered sum
 Weights and activations are synthetic and seeded (illatio_amd/synth.py); inputs are resident
@@ -365,10 +366,11 @@ def workload_c4(args, dev):
     xb = hip.hip_upload_new(dev, x)
     nsteps = args.steps + args.warmup + 3
     tables, routes = [], []
+    fused = args.mode == "fused"
     for i in range(nsteps):                      # the reference routes on the CPU (cuda-ds4f.lisp:991-999); tables made beforehand
         sel, w = orc.route(synth.activations(ne, rng), nu, 1.5)
         routes.append((sel, w))
-        tables.append(ds4f.tail_tables(dev, pools[i % nlayers], sel, w))
+        tables.append((ds4f.fused_tables if fused else ds4f.tail_tables)(dev, pools[i % nlayers], sel, w))
     ws = hip.Workspace(dev, 8 << 20)
     iq, q2, q8 = synth.row_bytes(synth.IQ2_XXS, d), synth.row_bytes(synth.Q2_K, ff), 34
     step_bytes = nu * (2 * ff * iq + d * q2) + 2 * ff * d // 32 * q8 + d * ff // 32 * q8
@@ -378,24 +380,31 @@ def workload_c4(args, dev):
         ws.reset()
         L = i % nlayers
         sel, w = routes[i]
-        ds4f.ffn_tail(dev, pools[L], sel, w, xb, ds4f.ffn_shared(dev, shared[L], xb, 0.0, ws=ws), 0.0, ws=ws, tables=tables[i])
+        if fused:
+            ds4f.ffn_step_fused(dev, pools[L], shared[L], sel, w, xb, 0.0, ws=ws, tables=tables[i])
+        else:
+            ds4f.ffn_tail(dev, pools[L], sel, w, xb, ds4f.ffn_shared(dev, shared[L], xb, 0.0, ws=ws), 0.0, ws=ws, tables=tables[i])
 
     def work_of(kernel, a):          # weight bytes + quantized activations + float outputs of the product kernels
-        if kernel == "d4_mv_iq2_xxs":
+        if kernel in ("d4_mv_iq2_xxs", "d4_mv_glu_iq2_xxs"):
             return 2 * nu * ff * iq + d + d // 256 * 4 + 4 * 2 * nu * ff
-        if kernel == "d4_mv_q2_k":
+        if kernel in ("d4_mv_q2_k", "d4_mv_q2_k_f32"):
             return nu * (d * q2 + ff + ff // 256 * 4 + ff // 16 * 4) + 4 * nu * d
         if kernel == "d4_mvq8":
             return a[0] * a[1] // 32 * q8 + a[1] // 32 * 36 + 4 * a[0]
+        if kernel == "d4_mvq8_glu":
+            return 2 * a[0] * a[1] // 32 * q8 + a[1] // 32 * 36 + 4 * a[0]
         return 0
 
     ms, dev_ms, per = tm.run(step, args.steps, args.warmup, probe_steps=3, work_of=work_of)
     roof = roofline_of({k: v for k, v in per.items() if v[1]}, "hbm", HBM_PEAK_GBS, "GB/s",
                        {"d4_mv_iq2_xxs": "gemv_kernel<16> (the 6 selected experts' IQ2_XXS gate and up, one launch over 12 matrices)",
-                        "d4_mv_q2_k": "gemv_kernel<10> (the 6 experts' Q2_K down)", "d4_mvq8": "gemv_kernel<8> (shared expert, Q8_0)"})
+                        "d4_mv_glu_iq2_xxs": "gemv_kernel<16> (the 6 selected experts' IQ2_XXS gate, up and gated activation, one launch)",
+                        "d4_mv_q2_k": "gemv_kernel<10> (the 6 experts' Q2_K down)", "d4_mv_q2_k_f32": "gemv_kernel<10> (the 6 experts' Q2_K down)",
+                        "d4_mvq8": "gemv_kernel<8> (shared expert, Q8_0)", "d4_mvq8_glu": "gemv_kernel<8> (shared expert gate, up, gated activation)"})
     roof["launch_us_all"] = {k: round(v[0] / v[2] * 1e3, 2) for k, v in per.items()}
     dom = max((k for k in per if per[k][1]), key=lambda k: per[k][0])
-    roof["traffic"] = TRAFFIC["c4"].get(dom)
+    roof["traffic"] = TRAFFIC["c4"].get({"d4_mv_glu_iq2_xxs": "d4_mv_iq2_xxs", "d4_mv_q2_k_f32": "d4_mv_q2_k"}.get(dom, dom))
     gbs = step_bytes / (ms * 1e-3) / 1e9
 
     def cpu():
@@ -414,7 +423,8 @@ def workload_c4(args, dev):
             "metric": "MoE decode step achieved HBM GB/s (% of 8 TB/s)",
             "config": {"workload": f"c4: MoE decode step, 256 resident experts (IQ2_XXS gate/up, Q2_K down) top-6 + Q8_0 shared expert, "
                                    f"d 4096, ff 2048, batch 1, rotating over {nlayers} layers", "bytes_per_step": step_bytes},
-            "extra": {"pct_of_hbm_peak": round(100 * gbs / HBM_PEAK_GBS, 2), "launches_per_step": 12}, "roofline": roof, "cpu": cpu}
+            "extra": {"pct_of_hbm_peak": round(100 * gbs / HBM_PEAK_GBS, 2), "launches_per_step": 5 if fused else 12,
+                      "launch_mode": args.mode}, "roofline": roof, "cpu": cpu}
 
 
 def workload_c5(args, dev):
@@ -491,7 +501,7 @@ def main():
     ap.add_argument("--transpose", action="store_true", help="c3: the 5120x17408 matrix")
     ap.add_argument("--path", default="bf16", choices=["bf16", "int8"], help="c3, c5: which matrix-core path")
     ap.add_argument("--mode", default="fused", choices=["fused", "fused-q", "single"],
-                    help="c2: fused = Q/K/V in one launch, gate+up in one, activations quantized inside the product "
+                    help="c4: fused = 5 launches a step, single = the reference's sequence of 12.  c2: fused = Q/K/V in one launch, gate+up in one, activations quantized inside the product "
                          "kernels; fused-q = the same launches after separate quantizer launches; "
                          "single = one launch per matrix after separate quantizer launches")
     args = ap.parse_args()

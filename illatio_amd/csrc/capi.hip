@@ -260,29 +260,68 @@ int ilt_d4_mvq8(uint64_t stream, int rows, int cols, int group_rows, const int8_
   return gemv_dense(stream, ILT_Q8_0, wq, wd, xq, xs, nullptr, nullptr, 0, y, nullptr, rows, cols, 0, group_rows);
 }
 
-static int gemv_experts(uint64_t stream, int fmt, int ncols, int nrows, int row_bytes, int64_t add, int x_stride,
-                        int y_stride, const uint64_t* ptrs, int nz, const int8_t* xq, const float* xd,
-                        const int32_t* bsums, float* dst) {
+// add_up >= 0: the gated pair, gate at ptrs[z] + add and up at ptrs[z] + add_up, dst = the gated activation.
+// xf: the activations as floats, quantized to Q8_K in the kernel; else xq, xd, bsums.
+static int gemv_experts(uint64_t stream, int fmt, int ncols, int nrows, int row_bytes, int64_t add, int64_t add_up,
+                        int x_stride, int y_stride, const uint64_t* ptrs, int nz, const int8_t* xq, const float* xd,
+                        const int32_t* bsums, const float* xf, const float* wts, float clamp, float* dst) {
   ILT_REQUIRE(nrows >= 0 && nz >= 0 && ncols > 0 && ncols % 256 == 0 && row_bytes == ncols / 256 * block_bytes(fmt));
   if (nrows == 0 || nz == 0) return ILT_OK;
-  ILT_REQUIRE(ptrs && xq && xd && (bsums || fmt == ILT_IQ2_XXS) && dst && add >= 0 && (add & 1) == 0 && x_stride % 256 == 0 && x_stride >= 0);
-  ILT_REQUIRE(nz <= 65535 && ((uintptr_t)xq & 15) == 0);
+  ILT_REQUIRE(ptrs && dst && add >= 0 && (add & 1) == 0 && (add_up < 0 || (add_up & 1) == 0) && x_stride % 256 == 0 && x_stride >= 0);
+  if (xf) ILT_REQUIRE(((uintptr_t)xf & 15) == 0);
+  else ILT_REQUIRE(xq && xd && (bsums || fmt == ILT_IQ2_XXS) && ((uintptr_t)xq & 15) == 0);
+  ILT_REQUIRE(nz <= 65535);
   IltGemvParams p = {};
-  p.nmat = 1; p.mat[0].rows = nrows; p.mat[0].row_bytes = row_bytes; p.mat[0].fmt = fmt; p.mat[0].y = dst;
-  p.ptrs = ptrs; p.add = add; p.cols = ncols;
-  p.xq = xq; p.xs = xd; p.bsums = bsums; p.x_stride = x_stride; p.y_stride = y_stride;
+  p.nmat = 1; p.mat[0].rows = nrows; p.mat[0].row_bytes = row_bytes; p.mat[0].fmt = fmt; p.mat[0].y = dst; p.mat[0].add = add;
+  if (add_up >= 0) {
+    p.nmat = 2; p.mat[1] = p.mat[0]; p.mat[1].add = add_up;
+    p.glu = 2; p.clamp = clamp; p.wts = wts;
+  }
+  p.ptrs = ptrs; p.cols = ncols;
+  p.xq = xq; p.xs = xd; p.bsums = bsums; p.xf = xf; p.x_stride = x_stride; p.y_stride = y_stride;
   return (int)ilt_gemv_launch(p, nz, S(stream));
 }
 
 int ilt_d4_mv_iq2_xxs(uint64_t stream, int ncols, int nrows, int row_bytes, int64_t add, int x_stride, int y_stride,
                       const uint64_t* ptrs, int nz, const int8_t* xq, const float* xd, float* dst) {
-  return gemv_experts(stream, ILT_IQ2_XXS, ncols, nrows, row_bytes, add, x_stride, y_stride, ptrs, nz, xq, xd,
-                      nullptr, dst);
+  return gemv_experts(stream, ILT_IQ2_XXS, ncols, nrows, row_bytes, add, -1, x_stride, y_stride, ptrs, nz, xq, xd,
+                      nullptr, nullptr, nullptr, 0.0f, dst);
 }
 
 int ilt_d4_mv_q2_k(uint64_t stream, int ncols, int nrows, int row_bytes, int64_t add, int x_stride, int y_stride,
                    const uint64_t* ptrs, int nz, const int8_t* xq, const float* xd, const int32_t* bsums, float* dst) {
-  return gemv_experts(stream, ILT_Q2_K, ncols, nrows, row_bytes, add, x_stride, y_stride, ptrs, nz, xq, xd, bsums, dst);
+  return gemv_experts(stream, ILT_Q2_K, ncols, nrows, row_bytes, add, -1, x_stride, y_stride, ptrs, nz, xq, xd, bsums,
+                      nullptr, nullptr, 0.0f, dst);
+}
+
+int ilt_d4_mv_glu_iq2_xxs(uint64_t stream, int ncols, int nrows, int row_bytes, int64_t add_gate, int64_t add_up,
+                          int x_stride, int y_stride, const uint64_t* ptrs, int nz, const float* x, const float* wts,
+                          float clamp, float* mid) {
+  ILT_REQUIRE(add_up >= 0 && x);
+  return gemv_experts(stream, ILT_IQ2_XXS, ncols, nrows, row_bytes, add_gate, add_up, x_stride, y_stride, ptrs, nz,
+                      nullptr, nullptr, nullptr, x, wts, clamp, mid);
+}
+
+int ilt_d4_mv_q2_k_f32(uint64_t stream, int ncols, int nrows, int row_bytes, int64_t add, int x_stride, int y_stride,
+                       const uint64_t* ptrs, int nz, const float* x, float* dst) {
+  ILT_REQUIRE(x);
+  return gemv_experts(stream, ILT_Q2_K, ncols, nrows, row_bytes, add, -1, x_stride, y_stride, ptrs, nz, nullptr, nullptr,
+                      nullptr, x, nullptr, 0.0f, dst);
+}
+
+int ilt_d4_mvq8_glu(uint64_t stream, int rows, int cols, const int8_t* gq, const uint16_t* gd, const int8_t* uq,
+                    const uint16_t* ud, const float* x, float clamp, float* mid) {
+  ILT_REQUIRE(rows >= 0 && cols > 0 && cols % 32 == 0);
+  if (rows == 0) return ILT_OK;
+  ILT_REQUIRE(gq && gd && uq && ud && x && mid && ((uintptr_t)gq & 15) == 0 && ((uintptr_t)uq & 15) == 0 && ((uintptr_t)x & 15) == 0);
+  IltGemvParams p = {};
+  p.nmat = 2;
+  for (int i = 0; i < 2; i++) {
+    p.mat[i].w = (const uint8_t*)(i ? uq : gq); p.mat[i].wd = i ? ud : gd; p.mat[i].y = mid;
+    p.mat[i].rows = rows; p.mat[i].fmt = ILT_Q8_0; p.mat[i].row_bytes = cols;
+  }
+  p.cols = cols; p.xf = x; p.f16_scale = 0; p.glu = 2; p.clamp = clamp;
+  return (int)ilt_gemv_launch(p, 1, S(stream));
 }
 
 int ilt_dequant_rows(uint64_t stream, int gguf_type, const void* w, const uint16_t* wd, const int32_t* rows_idx,
@@ -465,6 +504,14 @@ int ilt_launch(const char* kernel, unsigned gx, unsigned gy, unsigned gz, unsign
                                       a.ptr<cf>(5), a.ptr<float*>(6), a.i32(7), a.i32(8));
   K("mv_k_glu") return ilt_mv_k_glu(stream, a.i32(0), a.ptr<const void*>(1), a.i32(2), a.ptr<const void*>(3), a.ptr<ci8>(4),
                                     a.ptr<cf>(5), a.ptr<const int32_t*>(6), a.ptr<float*>(7), a.i32(8), a.i32(9));
+  K("d4_mv_glu_iq2_xxs")
+    return ilt_d4_mv_glu_iq2_xxs(stream, a.i32(0), a.i32(1), a.i32(2), a.i64(3), a.i64(4), a.i32(5), a.i32(6),
+                                 a.ptr<const uint64_t*>(7), (int)gz, a.ptr<cf>(8), a.ptr<cf>(9), a.f32(10), a.ptr<float*>(11));
+  K("d4_mv_q2_k_f32")
+    return ilt_d4_mv_q2_k_f32(stream, a.i32(0), a.i32(1), a.i32(2), a.i64(3), a.i32(4), a.i32(5), a.ptr<const uint64_t*>(6),
+                              (int)gz, a.ptr<cf>(7), a.ptr<float*>(8));
+  K("d4_mvq8_glu") return ilt_d4_mvq8_glu(stream, a.i32(0), a.i32(1), a.ptr<ci8>(2), a.ptr<cu16>(3), a.ptr<ci8>(4), a.ptr<cu16>(5),
+                                          a.ptr<cf>(6), a.f32(7), a.ptr<float*>(8));
   K("d4_mvq8") return ilt_d4_mvq8(stream, a.i32(0), a.i32(1), a.i32(2), a.ptr<ci8>(3), a.ptr<cu16>(4), a.ptr<ci8>(5),
                                   a.ptr<cf>(6), a.ptr<float*>(7));
   K("d4_mv_iq2_xxs") {

@@ -22,6 +22,7 @@ struct IltGemvMat {
   float* y;                  // output rows
   const float* bias;         // added after the sum, or null
   long long row_bytes;
+  long long add;             // experts: grid y's matrix is at ptrs[y] + add (w unused)
   int rows;
   int fmt;                   // ILT_Q8_0, ILT_Q4_K, ILT_Q6_K (dense); the expert kernels ignore it
   int batch0, nbat;          // this matrix's first batch among the launch's, and how many (set at launch)
@@ -31,8 +32,7 @@ struct IltGemvMat {
 struct IltGemvParams {
   IltGemvMat mat[4];         // up to four matrices sharing the activations
   int nmat;
-  const uint64_t* ptrs;      // experts: grid y's matrix is at ptrs[y] + add (mat[0].w unused)
-  long long add;
+  const uint64_t* ptrs;      // experts: grid y's matrices are at ptrs[y] + mat[i].add
   int cols;
   const int8_t* xq;          // quantized activations ...
   const float* xs;           //   their block scales (per 32 for Q8_0, per 256 otherwise)
@@ -42,7 +42,10 @@ struct IltGemvParams {
   int x_stride;              // activations of grid y start at y * x_stride elements
   int y_stride;              // outputs of grid y start at y * y_stride
   int acc;                   // y += result
-  int glu;                   // mat[0] = gate, mat[1] = up: y = silu(gate.x) * (up.x) into mat[0].y
+  int glu;                   // mat[0] = gate, mat[1] = up, into mat[0].y: 1 = swiglu! (model.lisp:364-378),
+                             //   2 = d4-routed!/d4-shared!'s (ds4f.lisp:1016-1019): clamp, silu(g)*u, times wts[y]
+  float clamp;               // glu 2: g = min(g, clamp), u in [-clamp, clamp] when clamp > 1e-6
+  const float* wts;          // glu 2: the weight of grid y's expert, or null
   int group_rows;            // >0: row r reads the activations of group r/group_rows (cols apart)
   int nbatches;              // batches of rows in the launch (per group, per grid y; set at launch)
   int wgs_per_group;         // grouped rows: workgroups sharing one group (set at launch)

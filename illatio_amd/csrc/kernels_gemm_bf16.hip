@@ -97,9 +97,10 @@ __device__ __forceinline__ u32 word_of(const int4& v, int i) { return (u32)(i ==
 // scale times a 2- or 4-bit integer), and Q6_K's s*(q-32) is one rounding of an exact value;
 // so a fused multiply-add gives the same bits in half the instructions.
 // j: the step within the half super-block (a constant after unrolling); c: which half.
-template <int FMT> __device__ __forceinline__ void dequant16(const WRaw<FMT>& r, int j, int c, int e, const u64* grid, float* o);
+// Words i0..i1-1 of the four (a word = 4 weights) are computed, so that a caller can spread the work.
+template <int FMT> __device__ __forceinline__ void dequant16(const WRaw<FMT>& r, int j, int c, int e, const u64* grid, float* o, int i0 = 0, int i1 = 4);
 
-template <> __device__ __forceinline__ void dequant16<ILT_Q4_K>(const WRaw<ILT_Q4_K>& r, int j, int c, int e, const u64*, float* o) {
+template <> __device__ __forceinline__ void dequant16<ILT_Q4_K>(const WRaw<ILT_Q4_K>& r, int j, int c, int e, const u64*, float* o, int i0, int i1) {
   const int sh = 8 * j, hl = j & 1;              // group g = 4c + j of the super-block
   const u32 x0 = ((u32)r.hdr.y >> sh) & 0xFF, x1 = ((u32)r.hdr.z >> sh) & 0xFF, x2 = ((u32)r.hdr.w >> sh) & 0xFF;
   const u32 sc = c == 0 ? (x0 & 63) : ((x2 & 0xF) | ((x0 >> 6) << 4));
@@ -108,42 +109,46 @@ template <> __device__ __forceinline__ void dequant16<ILT_Q4_K>(const WRaw<ILT_Q
   const int4& q = r.q[j >> 1];
 #pragma unroll
   for (int i = 0; i < 4; i++) {
+    if (i < i0 || i >= i1) continue;
     const u32 v = (word_of(q, i) >> (4 * hl)) & 0x0F0F0F0F;
 #pragma unroll
     for (int k = 0; k < 4; k++) o[4 * i + k] = __builtin_fmaf(d1, (float)((v >> (8 * k)) & 0xFF), -m1);   // d1*q is exact in fp32
   }
 }
 
-template <> __device__ __forceinline__ void dequant16<ILT_Q6_K>(const WRaw<ILT_Q6_K>& r, int j, int c, int e, const u64*, float* o) {
+template <> __device__ __forceinline__ void dequant16<ILT_Q6_K>(const WRaw<ILT_Q6_K>& r, int j, int c, int e, const u64*, float* o, int i0, int i1) {
   const int h = j >> 1;                          // 32-weight part j of the half: ql[j&1]'s nibble h, qh's bit pair j
   const u32 scw = (u32)(j < 2 ? r.sc.x : r.sc.y) >> (16 * (j & 1) + 8 * e);
   const float s = ilt_h2f((u16)r.d) * (float)(i8)(scw & 0xFF), s32 = -32.0f * s;
   const int4& ql = r.ql[j & 1];
 #pragma unroll
   for (int i = 0; i < 4; i++) {
+    if (i < i0 || i >= i1) continue;
     const u32 v = ((word_of(ql, i) >> (4 * h)) & 0x0F0F0F0F) | (((word_of(r.qh, i) >> (2 * j)) & 0x03030303) << 4);
 #pragma unroll
     for (int k = 0; k < 4; k++) o[4 * i + k] = __builtin_fmaf(s, (float)((v >> (8 * k)) & 0xFF), s32);   // = RN(s*(q-32)): one rounding either way
   }
 }
 
-template <> __device__ __forceinline__ void dequant16<ILT_Q2_K>(const WRaw<ILT_Q2_K>& r, int j, int c, int e, const u64*, float* o) {
+template <> __device__ __forceinline__ void dequant16<ILT_Q2_K>(const WRaw<ILT_Q2_K>& r, int j, int c, int e, const u64*, float* o, int i0, int i1) {
   const u32 scw = ((u32)(j < 2 ? r.sc.x : r.sc.y) >> (16 * (j & 1) + 8 * e)) & 0xFF;
   const float dl = ilt_h2f((u16)(r.dd & 0xFFFF)) * (float)(scw & 15), ml = ilt_h2f((u16)(r.dd >> 16)) * (float)(scw >> 4);
 #pragma unroll
   for (int i = 0; i < 4; i++) {
+    if (i < i0 || i >= i1) continue;
     const u32 v = (word_of(r.q, i) >> (2 * j)) & 0x03030303;
 #pragma unroll
     for (int k = 0; k < 4; k++) o[4 * i + k] = __builtin_fmaf(dl, (float)((v >> (8 * k)) & 0xFF), -ml);   // dl*q is exact in fp32
   }
 }
 
-template <> __device__ __forceinline__ void dequant16<ILT_IQ2_XXS>(const WRaw<ILT_IQ2_XXS>& r, int j, int c, int e, const u64* grid, float* o) {
+template <> __device__ __forceinline__ void dequant16<ILT_IQ2_XXS>(const WRaw<ILT_IQ2_XXS>& r, int j, int c, int e, const u64* grid, float* o, int i0, int i1) {
   const int4& q = r.q[j >> 1];                   // the half's 32-weight group j: 8 bytes
   const u32 g = word_of(q, 2 * (j & 1)) >> (16 * e), aux = word_of(q, 2 * (j & 1) + 1);
   const float db = (ilt_h2f((u16)r.d) * (0.5f + (float)(aux >> 28))) * 0.25f;
 #pragma unroll
   for (int l = 0; l < 2; l++) {
+    if (2 * l < i0 || 2 * l >= i1) continue;             // a codebook entry is two words
     const int2 mag = ilt_lds_ld8(grid + ((g >> (8 * l)) & 0xFF));
     u32 s = (aux >> (7 * (2 * e + l))) & 127;
     s |= (__popc(s) & 1) << 7;
@@ -326,32 +331,28 @@ __global__ __launch_bounds__((bf16_threads<TM, NB>()), (TM == 256 ? 1 : TN == 25
       issue_x(x3, min(ks + 3, nk - 1));
       __builtin_amdgcn_sched_barrier(0);
       u8* wnew = S.ws[w2];
-      {
-        const u8* xs = S.xs[x0];
-        const u8* ws = S.ws[w0];
+      const WRaw<FMT>* rawn = J2 < 4 ? rawa : rawb;
+      // Each half step in four pieces the compiler may not mix: two fragment reads for the
+      // next half step, a quarter of a 16-weight unit's dequantization, four MFMAs.
+      auto half = [&](const u8* xs_next, const u8* ws_next, u32 flip, v8bf* ua, v8bf* ub, v8bf* na, v8bf* nb, int u) {
+        float o[16];
 #pragma unroll
-        for (int a = 0; a < NA; a++) ga[a] = *(const v8bf*)(xs + (aoff[a] ^ 32));
+        for (int q = 0; q < 4; q++) {
+          na[q] = *(const v8bf*)(xs_next + (aoff[q] ^ flip));
+          nb[q] = *(const v8bf*)(ws_next + (boff[q] ^ flip));
+          dequant16<FMT>(rawn[u], J2 & 3, J2 >> 2, e0 + u, S.grid, o, q, q + 1);
 #pragma unroll
-        for (int b = 0; b < NB; b++) gb[b] = *(const v8bf*)(ws + (boff[b] ^ 32));
-        dequant_unit((J2 < 4 ? rawa : rawb)[0], 0, J2 & 3, J2 >> 2, wnew);
+          for (int b = 0; b < NB; b++) acc[q][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ua[q], ub[b], acc[q][b], 0, 0, 0);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+        u32 pk[8];
 #pragma unroll
-        for (int a = 0; a < NA; a++)
-#pragma unroll
-          for (int b = 0; b < NB; b++) acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[a], fb[b], acc[a][b], 0, 0, 0);
-      }
-      {
-        const u8* xs = S.xs[x1];
-        const u8* ws = S.ws[w1];
-#pragma unroll
-        for (int a = 0; a < NA; a++) fa[a] = *(const v8bf*)(xs + aoff[a]);
-#pragma unroll
-        for (int b = 0; b < NB; b++) fb[b] = *(const v8bf*)(ws + boff[b]);
-        dequant_unit((J2 < 4 ? rawa : rawb)[1], 1, J2 & 3, J2 >> 2, wnew);
-#pragma unroll
-        for (int a = 0; a < NA; a++)
-#pragma unroll
-          for (int b = 0; b < NB; b++) acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ga[a], gb[b], acc[a][b], 0, 0, 0);
-      }
+        for (int i = 0; i < 8; i++) pk[i] = pack_bf16(o[2 * i], o[2 * i + 1]);
+        ilt_lds_st16_untracked(wnew + (wdst ^ (32 * u)), pk[0], pk[1], pk[2], pk[3]);
+        ilt_lds_st16_untracked(wnew + (wdst ^ (32 * u) ^ 16), pk[4], pk[5], pk[6], pk[7]);
+      };
+      half(S.xs[x0], S.ws[w0], 32, fa, fb, ga, gb, 0);     // columns 0..15: fa, fb; reads this step's columns 16..31
+      half(S.xs[x1], S.ws[w1], 0, ga, gb, fa, fb, 1);      // columns 16..31: ga, gb; reads the next step's columns 0..15
       { const int t_ = x0; x0 = x1; x1 = x2; x2 = x3; x3 = t_; }
       { const int t_ = w0; w0 = w1; w1 = w2; w2 = t_; }
       // every load older than this step's has landed: this wave's share of x slab ks+2, which

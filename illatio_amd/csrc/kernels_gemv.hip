@@ -345,7 +345,7 @@ __device__ __forceinline__ void stage_q8k_from_f32(const float* __restrict__ x, 
       if (live) {
         *(int*)(lxq + b * XP + 4 * (l + 16 * i)) =
             (q[4 * i] & 0xFF) | ((q[4 * i + 1] & 0xFF) << 8) | ((q[4 * i + 2] & 0xFF) << 16) | ((q[4 * i + 3] & 0xFF) << 24);
-        if ((l & 3) == 0) lbs[b * 16 + (l >> 2) + 4 * i] = s;
+        if (lbs && (l & 3) == 0) lbs[b * 16 + (l >> 2) + 4 * i] = s;     // IQ2_XXS takes no 16-sums: none staged
       }
     }
     if (live && l == 0) lxs[b] = d;
@@ -375,7 +375,7 @@ __device__ __forceinline__ void stage_q8_from_f32(const float* __restrict__ x, i
 template <int FMT>
 __device__ __forceinline__ void run_rows(const IltGemvMat& m, const IltGemvParams& p, long row0, int nrows, int S,
                                          const Lds& L, float* t, int lane, int z, const Raw<FMT>& pre, bool use_pre) {
-  const u8* w = p.ptrs ? (const u8*)(p.ptrs[z] + p.add) : m.w;
+  const u8* w = p.ptrs ? (const u8*)(p.ptrs[z] + m.add) : m.w;
   wave_rows<FMT>(w, m.wd, row0, nrows, S, p.s_magic, m.row_bytes, L, t, lane, pre, use_pre);
 }
 
@@ -448,7 +448,7 @@ __global__ __launch_bounds__(kThreads) void gemv_kernel(IltGemvParams p) {
     int mi; long row0; int nrows;
     locate(wid, mi, row0, nrows);
     const IltGemvMat& m = p.mat[mi];
-    const u8* w0 = p.ptrs ? (const u8*)(p.ptrs[z] + p.add) : m.w;
+    const u8* w0 = p.ptrs ? (const u8*)(p.ptrs[z] + m.add) : m.w;
     if (FSET != 0 || m.fmt == ILT_Q4_K) first_load<(FSET ? FSET : ILT_Q4_K)>(pre.a, w0, m.wd, row0, nrows, S, m.row_bytes, lane);
     else first_load<(FSET ? FSET : ILT_Q6_K)>(pre.b, w0, m.wd, row0, nrows, S, m.row_bytes, lane);
     // and a touch of every 64-byte line of the batch's first 16 KB, so the later steps hit in L2
@@ -466,7 +466,7 @@ __global__ __launch_bounds__(kThreads) void gemv_kernel(IltGemvParams p) {
   const long xoff = (long)z * p.x_stride + (long)group * p.cols;
   if (p.xf) {
     if (q8) stage_q8_from_f32(p.xf + xoff, S, p.f16_scale, lxq, lxs);
-    else stage_q8k_from_f32(p.xf + xoff, S, lxq, lxs, lbs);
+    else stage_q8k_from_f32(p.xf + xoff, S, lxq, lxs, nbs ? lbs : nullptr);
   } else {
     const i8* gxq = p.xq + xoff;
     if (q8) {
@@ -502,8 +502,17 @@ __global__ __launch_bounds__(kThreads) void gemv_kernel(IltGemvParams p) {
       const long r = row0 + lane;
       if (p.glu) {
         const int ufmt = FSET != 0 ? FSET : p.mat[1].fmt;
-        const float uv = sum_any(ufmt, tw + (long)RB * tpr + (long)lane * S * (ufmt == ILT_Q4_K ? 2 : 1), S);
-        m.y[r] = dense_glu(v, uv);
+        const float uv = sum_any(ufmt, tw + (long)RB * tpr + (long)lane * S * ((ufmt == ILT_Q4_K || ufmt == ILT_Q2_K) ? 2 : 1), S);
+        float* y = m.y + (long)z * p.y_stride;
+        if (p.glu == 1) {
+          y[r] = dense_glu(v, uv);
+        } else {        // the experts' gated activation, as d4_swiglu_w computes it
+          float gv = v, uu = uv;
+          if (p.clamp > 1e-6f) { gv = fminf(gv, p.clamp); uu = fmaxf(-p.clamp, fminf(uu, p.clamp)); }
+          float o = ilt_silu(gv) * uu;
+          if (p.wts) o = o * p.wts[z];
+          y[r] = o;
+        }
       } else {
         float* y = m.y + (long)z * p.y_stride;
         if (m.bias) v = v + m.bias[r];

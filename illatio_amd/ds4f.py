@@ -136,6 +136,39 @@ def ffn_tail(dev, pool, sel, w, norm2, sout, clamp, keep=None, ws=None, tables=N
     return moe
 
 
+def fused_tables(dev, pool, sel, w):
+    """The device tables the fused decode step takes for one token: the k slot addresses and
+    the k weights."""
+    return (hip.hip_upload_new(dev, np.array([pool.slot_ptr(e) for e in sel], np.uint64)),
+            hip.hip_upload_new(dev, np.asarray(w, np.float32)))
+
+
+def ffn_step_fused(dev, pool, sh, sel, w, norm2, clamp, ws=None, tables=None):
+    """One token's shared expert and routed experts in five launches, with ffn_shared's and
+    ffn_tail's bits: the shared expert's gate, up and gated activation in one launch and its
+    down in one (both quantizing their float input in the kernel); the routed experts' gates,
+    ups and gated activations in one launch over k expert slots, their downs in one, then
+    the ordered sum.  Returns MOE."""
+    d, ff, k = pool.d, pool.ff, len(sel)
+    gb = pool.gate_bytes
+    A = ws.alloc if ws else hip.hip_alloc
+    ptrs, bw = tables if tables else fused_tables(dev, pool, sel, w)
+    smid, sout = A(dev, 4 * ff), A(dev, 4 * d)
+    bm, bd, moe = A(dev, 4 * k * ff), A(dev, 4 * k * d), A(dev, 4 * d)
+    hip.launch(dev, "d4_mvq8_glu", (ff + 3) // 4, 128, [ff, d, sh.gate.qs, sh.gate.d, sh.up.qs, sh.up.d, norm2, float(clamp), smid])
+    dense.mv_multi(dev, [(sh.down, sout, None)], xf=smid, f16_scale=False)
+    hip.launch(dev, "d4_mv_glu_iq2_xxs", ((ff + 7) // 8, 1, k), 64,
+               [d, ff, pool.grb, hip.I64(0), hip.I64(gb), 0, ff, ptrs, norm2, bw, float(clamp), bm])
+    hip.launch(dev, "d4_mv_q2_k_f32", ((d + 7) // 8, 1, k), 64, [ff, d, pool.drb, hip.I64(2 * gb), ff, d, ptrs, bm, bd])
+    hip.launch(dev, "d4_moe_sum", (d + 255) // 256, 256, [d, k, bd, sout, moe, None])
+    if ws:
+        return moe
+    hip.hip_sync(dev)
+    for b in (smid, sout, bm, bd) + (() if tables else (ptrs, bw)):
+        hip.hip_free(b)
+    return moe
+
+
 def route(dev, logits, n, ne, nu, scale, bias=None, alloc=hip.hip_alloc):
     """D4_ROUTE for N tokens' LOGITS (a DBuf): returns (sel, w) DBufs of N x NU."""
     sel, w = alloc(dev, 4 * n * nu), alloc(dev, 4 * n * nu)

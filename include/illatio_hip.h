@@ -159,6 +159,26 @@ int ilt_d4_mv_iq2_xxs(uint64_t stream, int ncols, int nrows, int row_bytes, int6
 int ilt_d4_mv_q2_k(uint64_t stream, int ncols, int nrows, int row_bytes, int64_t add, int x_stride, int y_stride,
                    const uint64_t* ptrs, int nz, const int8_t* xq, const float* xd, const int32_t* bsums, float* dst);
 
+/* The decode step of d4-routed! / d4-shared! (ds4f.lisp:994-1048; DK-FFN-TAIL, cuda-ds4f.lisp:
+   908-956) in fewer launches, with the same bits: the activations come as floats and every
+   workgroup quantizes them as quantize-q8k! (experts) or quantize-q8! with a float scale
+   (shared expert) does, so no quantizer launch precedes the product.
+   d4_mv_glu_iq2_xxs: for each z < nz, gate at ptrs[z] + add_gate, up at ptrs[z] + add_up,
+     x at element z*x_stride (0: one x for all), mid[z*y_stride + r] = (silu(g)*u) * wts[z]
+     with g = min(g, clamp), u in [-clamp, clamp] when clamp > 1e-6 (d4_swiglu_w's formula;
+     wts may be null).  Replaces quant + d4_mv_iq2_xxs over 2k matrices + d4_swiglu_w.
+   d4_mv_q2_k_f32: d4_mv_q2_k on float activations (each z's own, x_stride apart).
+   d4_mvq8_glu: the shared expert's gate and up (Q8_0, repacked) on float x, the same gated
+     activation with weight 1 into mid.  Its down projection is ilt_mv_multi with xf = mid
+     and f16_scale 0. */
+int ilt_d4_mv_glu_iq2_xxs(uint64_t stream, int ncols, int nrows, int row_bytes, int64_t add_gate, int64_t add_up,
+                          int x_stride, int y_stride, const uint64_t* ptrs, int nz, const float* x, const float* wts,
+                          float clamp, float* mid);
+int ilt_d4_mv_q2_k_f32(uint64_t stream, int ncols, int nrows, int row_bytes, int64_t add, int x_stride, int y_stride,
+                       const uint64_t* ptrs, int nz, const float* x, float* dst);
+int ilt_d4_mvq8_glu(uint64_t stream, int rows, int cols, const int8_t* gq, const uint16_t* gd, const int8_t* uq,
+                    const uint16_t* ud, const float* x, float clamp, float* mid);
+
 /* Rows as floats (dense.cu:53 embed_q8, kquant.cu:202 embed_k; CPU: q8mat-row!, kmat-row!,
    iq2xxs-row-floats!, q2k-row-floats!): out[n] = row tokens[n] (row n when tokens is null)
    of W, bit-exact.  ilt_dequant_rows takes a GGUF type (any of the five; Q8_0 repacked,

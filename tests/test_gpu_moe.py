@@ -150,6 +150,10 @@ def test_moe_decode_step_bit_exact(dev, ne, d, ff, nu, clamp):
         assert np.array_equal(bits(keep["mid"]), bits(wmid)), np.abs(keep["mid"] - wmid).max()
         got = hip.hip_floats(moe, d)
         assert np.array_equal(bits(got), bits(want)), np.abs(got - want).max()
-        for b in (lb, nb, sel, w, sout, moe):
+        # the same step in five launches (activations quantized inside the product kernels, gate/up/gated activation fused)
+        fused = ds4f.ffn_step_fused(dev, pool, sh, hsel, hw, nb, clamp)
+        got = hip.hip_floats(fused, d)
+        assert np.array_equal(bits(got), bits(want)), np.abs(got - want).max()
+        for b in (lb, nb, sel, w, sout, moe, fused):
             hip.hip_free(b)
     pool.free(); sh.free()
