@@ -307,17 +307,27 @@ __device__ __forceinline__ int ilt_or16(int v) {
   v |= ilt_dpp<ILT_DPP_HALF_MIRROR>(v); return v | ilt_dpp<ILT_DPP_ROW_MIRROR>(v);
 }
 
-__device__ __forceinline__ void stage_q8k_from_f32(const float* __restrict__ x, int nblk, i8* lxq, float* lxs, int* lbs) {
+// This lane's 16 values of the block its 16-lane row takes in pass PASS (zeros past the end).
+__device__ __forceinline__ void load_q8k_pass(const float* __restrict__ x, int nblk, int pass, float4* t) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, g = lane >> 4, l = lane & 15;
-  for (int b0 = 4 * wave; b0 < nblk; b0 += 4 * kWaves) {
+  const int b = 4 * wave + 4 * kWaves * pass + g;
+#pragma unroll
+  for (int i = 0; i < 4; i++) t[i] = b < nblk ? *(const float4*)(x + b * 256 + 4 * (l + 16 * i)) : make_float4(0.f, 0.f, 0.f, 0.f);
+}
+
+// FIRST: the first pass's values, loaded by the caller ahead of time (load_q8k_pass(.., 0, ..)).
+__device__ __forceinline__ void stage_q8k_from_f32(const float* __restrict__ x, int nblk, i8* lxq, float* lxs, int* lbs, const float4* first) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, g = lane >> 4, l = lane & 15;
+  int pass = 0;
+  for (int b0 = 4 * wave; b0 < nblk; b0 += 4 * kWaves, pass++) {
     const int b = b0 + g;
     const bool live = b < nblk;
+    float4 t4[4];
+    if (pass == 0) { t4[0] = first[0]; t4[1] = first[1]; t4[2] = first[2]; t4[3] = first[3]; }
+    else load_q8k_pass(x, nblk, pass, t4);
     float v[16];
 #pragma unroll
-    for (int i = 0; i < 4; i++) {
-      const float4 t = live ? *(const float4*)(x + b * 256 + 4 * (l + 16 * i)) : make_float4(0.f, 0.f, 0.f, 0.f);
-      v[4 * i] = t.x; v[4 * i + 1] = t.y; v[4 * i + 2] = t.z; v[4 * i + 3] = t.w;
-    }
+    for (int i = 0; i < 4; i++) { v[4 * i] = t4[i].x; v[4 * i + 1] = t4[i].y; v[4 * i + 2] = t4[i].z; v[4 * i + 3] = t4[i].w; }
     float am = 0.0f;
 #pragma unroll
     for (int k = 0; k < 16; k++) am = fmaxf(am, fabsf(v[k]));
@@ -441,6 +451,11 @@ __global__ __launch_bounds__(kThreads) void gemv_kernel(IltGemvParams p) {
     nrows = rq + (bl < rr ? 1 : 0);
   };
 
+  // Float activations to quantize here: their first loads go out before any weight load, since
+  // loads return in order and these (hot in L2) are needed first.
+  const long xoff = (long)z * p.x_stride + (long)group * p.cols;
+  float4 xfirst[4];
+  if (!q8 && p.xf) load_q8k_pass(p.xf + xoff, S, 0, xfirst);
   // the first batch's first loads go out now, so they are on their way while x is staged
   Pre<FSET> pre;
   int warm[4] = {0, 0, 0, 0};
@@ -463,10 +478,9 @@ __global__ __launch_bounds__(kThreads) void gemv_kernel(IltGemvParams p) {
   }
 
   // ---- stage the activations ----
-  const long xoff = (long)z * p.x_stride + (long)group * p.cols;
   if (p.xf) {
     if (q8) stage_q8_from_f32(p.xf + xoff, S, p.f16_scale, lxq, lxs);
-    else stage_q8k_from_f32(p.xf + xoff, S, lxq, lxs, nbs ? lbs : nullptr);
+    else stage_q8k_from_f32(p.xf + xoff, S, lxq, lxs, nbs ? lbs : nullptr, xfirst);
   } else {
     const i8* gxq = p.xq + xoff;
     if (q8) {
