@@ -3,7 +3,7 @@
 
 The default workload (c2) is the one the metric is quoted on: a step is one decoded token's
 worth of quantized products at the Qwen3-4B shape (BASELINE.json configs[1]) -- for each of
-36 layers the activation quantizations and the seven matrix-vector products (Q4_K wq
+36 layers the activation quantizations (inside the product kernels) and the seven matrix-vector products (Q4_K wq
 4096x2560, wk 1024x2560, wo 2560x4096, gate and up 9728x2560; Q6_K wv 1024x2560, down
 2560x9728), then the Q6_K output head 151936x2560: 2,618,273,280 bytes of GGUF blocks
 streamed from HBM per step, every matrix its own allocation, so the working set (2.6 GB)
@@ -190,9 +190,11 @@ def workload_c2(args, dev):
                     dense.quantize_act(dev, xbuf["x"], acts["x"])
                 tm.launch("glu", wbytes["gate"] + wbytes["up"] + D + 4 * FFN,
                           lambda: dense.glu_mul(dev, L["gate"], L["up"], acts["x"], ybuf["gate"], xf=xf))
-                # the down projection's input is 9728 wide: quantized once, not by every workgroup
-                dense.quantize_act(dev, xbuf["mid"], acts["mid"])
-                tm.launch("down", wbytes["down"] + FFN + 4 * D, lambda: dense.cmat_mul(dev, L["down"], acts["mid"], ybuf["down"]))
+                if inq:
+                    tm.launch("down", wbytes["down"] + FFN + 4 * D, lambda: dense.mv_multi(dev, [(L["down"], ybuf["down"], None)], xf=xbuf["mid"]))
+                else:
+                    dense.quantize_act(dev, xbuf["mid"], acts["mid"])
+                    tm.launch("down", wbytes["down"] + FFN + 4 * D, lambda: dense.cmat_mul(dev, L["down"], acts["mid"], ybuf["down"]))
             else:
                 dense.quantize_act(dev, xbuf["x"], acts["x"])
                 for name, qt, rows, cols, src in specs:
