@@ -376,6 +376,11 @@ int ilt_d4_swiglu_w(uint64_t stream, int n, int ff, float clamp, const float* g,
   ILT_REQUIRE(n >= 0 && ff > 0 && (n == 0 || (g && u && w && mid)) && (!xq || xs));
   return (int)ilt_k_swiglu_w(n, ff, clamp, g, u, w, mid, xq, xs, S(stream));
 }
+int ilt_d4_swiglu_w_bf16(uint64_t stream, int n, int ff, float clamp, const float* g, const float* u, const float* w, uint16_t* mid) {
+  ILT_REQUIRE(n >= 0 && ff > 0 && ff % 8 == 0 && (n == 0 || (g && u && w && mid)));
+  ILT_REQUIRE((((uintptr_t)g | (uintptr_t)u | (uintptr_t)mid) & 15) == 0);
+  return (int)ilt_k_swiglu_w_bf16(n, ff, clamp, g, u, w, mid, S(stream));
+}
 int ilt_d4_moe_sum(uint64_t stream, int d, int k, const float* down, const float* shared_, float* moe, const uint32_t* perm) {
   ILT_REQUIRE(d > 0 && k >= 0 && down && moe);
   return (int)ilt_k_moe_sum(d, k, down, shared_, moe, perm, S(stream));
@@ -448,14 +453,14 @@ int ilt_mm_k_bf16(uint64_t stream, int gguf_type, const void* w, const uint16_t*
 
 int ilt_d4_mm_id_bf16(uint64_t stream, int gguf_type, int ncols, int nrows, int row_bytes, int64_t add, const uint64_t* ptrs,
                       const uint32_t* counts, const uint32_t* bases, int ne, int64_t total_rows,
-                      const uint16_t* xb, float* y) {
+                      const uint16_t* xb, const uint32_t* rmap, float* y) {
   const int fmt = bf16_type(gguf_type);
   ILT_REQUIRE(fmt && ncols > 0 && ncols % 256 == 0 && nrows >= 0 && ne >= 0 && ne <= 256 && total_rows >= 0);
   ILT_REQUIRE(row_bytes == ncols / 256 * block_bytes(fmt) && add >= 0 && (add & 1) == 0);
   if (nrows == 0 || ne == 0 || total_rows == 0) return ILT_OK;
   ILT_REQUIRE(ptrs && counts && bases && xb && y && ((uintptr_t)xb & 15) == 0 && total_rows < (1LL << 31));
   ILT_REQUIRE((long long)row_bytes * nrows < 0xFFFFFFF0LL);
-  return (int)ilt_k_gemm_bf16_id(fmt, ptrs, add, counts, bases, ne, row_bytes, nrows, ncols, xb, total_rows, y, S(stream));
+  return (int)ilt_k_gemm_bf16_id(fmt, ptrs, add, counts, bases, ne, row_bytes, nrows, ncols, xb, rmap, total_rows, y, S(stream));
 }
 
 // ---- launch by name ---------------------------------------------------------------------------
@@ -492,7 +497,8 @@ int ilt_launch(const char* kernel, unsigned gx, unsigned gy, unsigned gz, unsign
                                       a.i32(5), a.i32(6), a.i32(7), a.i32(8));
   K("d4_mm_id_bf16")
     return ilt_d4_mm_id_bf16(stream, a.i32(0), a.i32(1), a.i32(2), a.i32(3), a.i64(4), a.ptr<const uint64_t*>(5), a.ptr<cu32>(6),
-                             a.ptr<cu32>(7), a.i32(8), a.i64(9), a.ptr<cu16>(10), a.ptr<float*>(11));
+                             a.ptr<cu32>(7), a.i32(8), a.i64(9), a.ptr<cu16>(10), a.ptr<cu32>(11), a.ptr<float*>(12));
+  K("d4_swiglu_w_bf16") return ilt_d4_swiglu_w_bf16(stream, a.i32(0), a.i32(1), a.f32(2), a.ptr<cf>(3), a.ptr<cf>(4), a.ptr<cf>(5), a.ptr<uint16_t*>(6));
   K("d4_mm_id_iq2_xxs")
     return ilt_d4_mm_id_iq2_xxs(stream, a.i32(0), a.i32(1), a.i32(2), a.i64(5), a.ptr<const uint64_t*>(6), a.ptr<cu32>(7),
                                 a.ptr<cu32>(8), (int)gz, a.i64(13), a.ptr<ci8>(9), a.ptr<cf>(11), a.ptr<float*>(10));

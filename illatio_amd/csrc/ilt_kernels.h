@@ -92,7 +92,8 @@ hipError_t ilt_k_cvt_bf16(const float* x, uint16_t* xb, long long n, hipStream_t
 hipError_t ilt_k_gemm_bf16(int fmt, const uint8_t* w, long long row_bytes, int rows, int cols, const uint16_t* xb, int ntok,
                            float* y, const float* bias, int acc, hipStream_t st);
 hipError_t ilt_k_gemm_bf16_id(int fmt, const uint64_t* ptrs, long long add, const uint32_t* counts, const uint32_t* bases,
-                              int ne, long long row_bytes, int rows, int cols, const uint16_t* xb, long long total_rows,
-                              float* y, hipStream_t st);
+                              int ne, long long row_bytes, int rows, int cols, const uint16_t* xb, const uint32_t* rmap,
+                              long long total_rows, float* y, hipStream_t st);
+hipError_t ilt_k_swiglu_w_bf16(int n, int ff, float clamp, const float* g, const float* u, const float* w, uint16_t* mid, hipStream_t st);
 
 #endif  // ILT_KERNELS_H

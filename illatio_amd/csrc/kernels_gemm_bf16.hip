@@ -166,6 +166,7 @@ struct BfParams {
   const u32* counts; const u32* bases; int ne;
   int rows, cols; long long row_bytes;
   const u16* x;                              // bf16 activations, cols per token (the gathered rows when grouped)
+  const u32* rmap;                           // grouped: row i of the groups is x's row rmap[i] (null: row i)
   float* y; const float* bias; int acc; int ntok;
 };
 
@@ -252,12 +253,13 @@ __global__ __launch_bounds__((bf16_threads<TM, NB>()), (TM == 256 ? 1 : TN == 25
   const __amdgpu_buffer_rsrc_t rw = ilt_rsrc(ilt_uniform_ptr(w), (u32)min((long long)p.rows * p.row_bytes, 0xFFFFFFF0LL));
   const u32 wrowoff = (u32)((long long)min(r0 + wrow, p.rows - 1) * p.row_bytes);
   const u32 wdst = slab_off(wrow, 2 * e0);                 // unit e's two pieces: 2e and 2e+1, at (wdst ^ 32e) and that ^ 16
-  const u8* xbase = (const u8*)ilt_uniform_ptr(p.x + tok0 * (long)p.cols);
+  const u8* xbase = (const u8*)ilt_uniform_ptr(p.rmap ? p.x : p.x + tok0 * (long)p.cols);
   u32 xoff[NI];                                            // the x pieces it sends to LDS
 #pragma unroll
   for (int i = 0; i < NI; i++) {
     const int P = (wave * NI + i) * 64 + lane, tok = P >> 2, kp = (P & 3) ^ (int)slab_swz(tok);
-    xoff[i] = (u32)min(tok, ntok - 1) * (u32)p.cols * 2 + 16 * kp;
+    const int tk = min(tok, ntok - 1);
+    xoff[i] = (p.rmap ? p.rmap[tok0 + tk] : (u32)tk) * (u32)p.cols * 2 + 16 * kp;
   }
 
   v16f acc[NA][NB];
@@ -511,12 +513,12 @@ hipError_t ilt_k_gemm_bf16(int fmt, const uint8_t* w, long long row_bytes, int r
 }
 
 hipError_t ilt_k_gemm_bf16_id(int fmt, const uint64_t* ptrs, long long add, const uint32_t* counts, const uint32_t* bases,
-                              int ne, long long row_bytes, int rows, int cols, const uint16_t* xb, long long total_rows,
-                              float* y, hipStream_t st) {
+                              int ne, long long row_bytes, int rows, int cols, const uint16_t* xb, const uint32_t* rmap,
+                              long long total_rows, float* y, hipStream_t st) {
   if (total_rows <= 0 || rows <= 0 || ne <= 0) return hipSuccess;
   if (ne > 256) return hipErrorInvalidValue;
   BfParams p = {};
   p.ptrs = ptrs; p.add = add; p.counts = counts; p.bases = bases; p.ne = ne;
-  p.rows = rows; p.cols = cols; p.row_bytes = row_bytes; p.x = xb; p.y = y; p.ntok = (int)total_rows;
+  p.rows = rows; p.cols = cols; p.row_bytes = row_bytes; p.x = xb; p.rmap = rmap; p.y = y; p.ntok = (int)total_rows;
   return dispatch_bf16<128, 128, 2>(fmt, p, total_rows / 128 + ne, st);
 }

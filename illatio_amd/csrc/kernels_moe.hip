@@ -149,6 +149,35 @@ __global__ __launch_bounds__(256) void swiglu_w_kernel(long long total, int ff, 
   }
 }
 
+// The same gated activation rounded to bf16 (nearest even), for the bf16 grouped product: 8 values a thread.
+__global__ __launch_bounds__(256) void swiglu_w_bf16_kernel(long long total8, int ff, float clamp, const float* __restrict__ g,
+                                                            const float* __restrict__ u, const float* __restrict__ w,
+                                                            u16* __restrict__ mid) {
+  typedef float v2f __attribute__((ext_vector_type(2)));
+  typedef __bf16 v2bf __attribute__((ext_vector_type(2)));
+  const long long i = (long long)blockIdx.x * 256 + threadIdx.x;
+  if (i >= total8) return;
+  const float4 g0 = ((const float4*)g)[2 * i], g1 = ((const float4*)g)[2 * i + 1];
+  const float4 u0 = ((const float4*)u)[2 * i], u1 = ((const float4*)u)[2 * i + 1];
+  const float wv = w[(8 * i) / ff];            // ff is a multiple of 8: the eight values share a row
+  float gv[8] = {g0.x, g0.y, g0.z, g0.w, g1.x, g1.y, g1.z, g1.w}, uv[8] = {u0.x, u0.y, u0.z, u0.w, u1.x, u1.y, u1.z, u1.w};
+  u32 pk[4];
+#pragma unroll
+  for (int k = 0; k < 4; k++) {
+    float o[2];
+#pragma unroll
+    for (int h = 0; h < 2; h++) {
+      float a = gv[2 * k + h], b = uv[2 * k + h];
+      if (clamp > 1e-6f) { a = fminf(a, clamp); b = fmaxf(-clamp, fminf(b, clamp)); }
+      o[h] = (ilt_silu(a) * b) * wv;
+    }
+    const v2f v = {o[0], o[1]};
+    const v2bf r = __builtin_convertvector(v, v2bf);
+    __builtin_memcpy(&pk[k], &r, 4);
+  }
+  ((int4*)mid)[i] = make_int4(pk[0], pk[1], pk[2], pk[3]);
+}
+
 __global__ void moe_sum_kernel(int d, int k, const float* __restrict__ down, const float* __restrict__ shared_,
                                float* __restrict__ moe, const u32* __restrict__ perm) {
   const int r = blockIdx.x * blockDim.x + threadIdx.x;
@@ -219,6 +248,14 @@ hipError_t ilt_k_swiglu_w(int n, int ff, float clamp, const float* g, const floa
   if (total <= 0) return hipSuccess;
   if (xq && (total % 32)) return hipErrorInvalidValue;
   hipLaunchKernelGGL(swiglu_w_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st, total, ff, clamp, g, u, w, mid, xq, xs);
+  return hipGetLastError();
+}
+
+hipError_t ilt_k_swiglu_w_bf16(int n, int ff, float clamp, const float* g, const float* u, const float* w, uint16_t* mid, hipStream_t st) {
+  const long long total = (long long)n * ff;
+  if (total <= 0) return hipSuccess;
+  if (ff % 8) return hipErrorInvalidValue;
+  hipLaunchKernelGGL(swiglu_w_bf16_kernel, dim3((unsigned)((total / 8 + 255) / 256)), dim3(256), 0, st, total / 8, ff, clamp, g, u, w, mid);
   return hipGetLastError();
 }
 

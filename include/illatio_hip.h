@@ -237,14 +237,19 @@ int ilt_d4_mm_id_q2_k(uint64_t stream, int ncols, int nrows, int row_bytes, int6
    mm_k_bf16: gguf_type 10 Q2_K, 12 Q4_K, 14 Q6_K (212-byte device blocks of
      ilt_repack_q6k), 16 IQ2_XXS; xb is n tokens of cols bf16, 16-byte aligned;
      y[t*rows + r] (+= when acc, + bias[r]).  The matrix is at most 4 GiB.
-   d4_mm_id_bf16: the grouped expert product of ds4f_mm.cu:256-257 on the gathered rows
-     xb (bf16, ncols apart), same gguf_type codes, other arguments as d4_mm_id_*. */
+   d4_mm_id_bf16: the grouped expert product of ds4f_mm.cu:256-257, same gguf_type codes, other
+     arguments as d4_mm_id_*.  Row i of the groups multiplies xb's row rmap[i] (d4_group_scatter's
+     row -> token map: the tokens' activations are read in place, no gathered copy), or row i
+     itself when rmap is null.
+   d4_swiglu_w_bf16: d4_swiglu_w's gated activation rounded to bf16 (ff a multiple of 8). */
 int ilt_cvt_bf16(uint64_t stream, const float* x, uint16_t* xb, int64_t n);
 int ilt_mm_k_bf16(uint64_t stream, int gguf_type, const void* w, const uint16_t* xb, float* y, const float* bias,
                   int rows, int cols, int n, int acc);
 int ilt_d4_mm_id_bf16(uint64_t stream, int gguf_type, int ncols, int nrows, int row_bytes, int64_t add, const uint64_t* ptrs,
                       const uint32_t* counts, const uint32_t* bases, int ne, int64_t total_rows,
-                      const uint16_t* xb, float* y);
+                      const uint16_t* xb, const uint32_t* rmap, float* y);
+int ilt_d4_swiglu_w_bf16(uint64_t stream, int n, int ff, float clamp, const float* g, const float* u, const float* w,
+                         uint16_t* mid);
 
 /* ---- 3. launch by name (src/cuda.lisp:323-352) -------------------------------------------
  * params[i] points at argument i's 8-byte slot: a pointer as 64 bits, an int in the low

@@ -154,8 +154,9 @@ def test_moe_prefill_chunk_bf16_within_tolerance(dev, ne, d, ff, nu, n, clamp):
         b, c = int(keep["bases"][e]), int(keep["counts"][e])
         if c == 0:
             continue
-        cpu["gate"][b:b + c] = orc.matmul(synth.IQ2_XXS, gate_e[e], ff, d, keep["x"][b:b + c], nthreads=8)
-        cpu["up"][b:b + c] = orc.matmul(synth.IQ2_XXS, up_e[e], ff, d, keep["x"][b:b + c], nthreads=8)
+        xrows = norms[keep["rmap"][b:b + c]]              # the rows the expert's tiles read through the row map
+        cpu["gate"][b:b + c] = orc.matmul(synth.IQ2_XXS, gate_e[e], ff, d, xrows, nthreads=8)
+        cpu["up"][b:b + c] = orc.matmul(synth.IQ2_XXS, up_e[e], ff, d, xrows, nthreads=8)
         cpu["down"][b:b + c] = orc.matmul(synth.Q2_K, down_e[e], d, ff, keep["mid"][b:b + c], nthreads=8)
     for k in ("gate", "up", "down"):
         assert np.abs(keep[k] - cpu[k]).max() <= TOL_VS_CPU * np.abs(cpu[k]).max(), k
