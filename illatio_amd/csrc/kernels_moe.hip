@@ -84,10 +84,22 @@ __global__ void group_zero_kernel(int ne, u32* counts) {
 // rank[row] = the row's place among its expert's rows.  The order inside an expert is
 // whatever the atomics give; every later step goes through rmap/smap, so results do not
 // depend on it.
-__global__ void group_count_kernel(int n, const u32* __restrict__ sel, u32* counts, u32* __restrict__ rank) {
+// A workgroup counts its rows per expert in LDS first, then reserves each expert's run of
+// places with one global atomic: a popular expert costs one atomic a workgroup, not one a row.
+__global__ __launch_bounds__(256) void group_count_kernel(int n, int ne, const u32* __restrict__ sel, u32* counts, u32* __restrict__ rank) {
+  __shared__ u32 h[1024];
   const int gid = blockIdx.x * blockDim.x + threadIdx.x;
-  if (gid >= n) return;
-  rank[gid] = atomicAdd(counts + sel[gid], 1u);
+  for (int e = threadIdx.x; e < ne; e += blockDim.x) h[e] = 0;
+  __syncthreads();
+  u32 e = 0, mine = 0;
+  if (gid < n) { e = sel[gid]; mine = atomicAdd(&h[e], 1u); }
+  __syncthreads();
+  for (int x = threadIdx.x; x < ne; x += blockDim.x) {
+    const u32 c = h[x];
+    if (c) h[x] = atomicAdd(counts + x, c);       // now the first place of this workgroup's rows of expert x
+  }
+  __syncthreads();
+  if (gid < n) rank[gid] = h[e] + mine;
 }
 
 // bases[e] = rows before expert e's.  One workgroup of 1024; ne <= 1024.
@@ -187,14 +199,27 @@ __global__ void moe_sum_kernel(int d, int k, const float* __restrict__ down, con
   moe[r] = shared_ ? acc + shared_[r] : acc;
 }
 
-__global__ void moe_sum_rows_kernel(int d, int nu, int ntok, const float* __restrict__ down, const u32* __restrict__ map,
-                                    const float* __restrict__ shared_, float* __restrict__ moe) {
-  const long long gid = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+// Four columns a thread (16-byte loads); the slots are added in order, all loads sent first.
+__global__ __launch_bounds__(256) void moe_sum_rows_kernel(int d, int nu, int ntok, const float* __restrict__ down, const u32* __restrict__ map,
+                                                           const float* __restrict__ shared_, float* __restrict__ moe) {
+  const long long gid = ((long long)blockIdx.x * blockDim.x + threadIdx.x) * 4;
   if (gid >= (long long)ntok * d) return;
   const int t = (int)(gid / d), j = (int)(gid % d);
-  float acc = 0.0f;
-  for (int s = 0; s < nu; s++) acc = acc + down[(long long)map[(long long)t * nu + s] * d + j];
-  moe[gid] = shared_ ? acc + shared_[gid] : acc;
+  float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+  for (int s0 = 0; s0 < nu; s0 += 8) {
+    float4 v[8];
+#pragma unroll
+    for (int s = 0; s < 8; s++)
+      if (s0 + s < nu) v[s] = *(const float4*)(down + (long long)map[(long long)t * nu + s0 + s] * d + j);
+#pragma unroll
+    for (int s = 0; s < 8; s++)
+      if (s0 + s < nu) { acc.x = acc.x + v[s].x; acc.y = acc.y + v[s].y; acc.z = acc.z + v[s].z; acc.w = acc.w + v[s].w; }
+  }
+  if (shared_) {
+    const float4 sh = *(const float4*)(shared_ + gid);
+    acc.x = acc.x + sh.x; acc.y = acc.y + sh.y; acc.z = acc.z + sh.z; acc.w = acc.w + sh.w;
+  }
+  *(float4*)(moe + gid) = acc;
 }
 
 }  // namespace
@@ -217,7 +242,8 @@ hipError_t ilt_k_group_zero(int ne, uint32_t* counts, hipStream_t st) {
 
 hipError_t ilt_k_group_count(int n, int ne, int nu, const uint32_t* sel, uint32_t* counts, uint32_t* rank, hipStream_t st) {
   if (n <= 0) return hipSuccess;
-  hipLaunchKernelGGL(group_count_kernel, dim3((n + 255) / 256), dim3(256), 0, st, n, sel, counts, rank);
+  if (ne < 1 || ne > 1024) return hipErrorInvalidValue;
+  hipLaunchKernelGGL(group_count_kernel, dim3((n + 255) / 256), dim3(256), 0, st, n, ne, sel, counts, rank);
   return hipGetLastError();
 }
 
@@ -268,6 +294,7 @@ hipError_t ilt_k_moe_sum_rows(int d, int nu, int ntok, const float* down, const 
                               float* moe, hipStream_t st) {
   const long long n = (long long)ntok * d;
   if (n <= 0) return hipSuccess;
-  hipLaunchKernelGGL(moe_sum_rows_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, d, nu, ntok, down, map, shared_, moe);
+  if (d % 4) return hipErrorInvalidValue;
+  hipLaunchKernelGGL(moe_sum_rows_kernel, dim3((unsigned)((n / 4 + 255) / 256)), dim3(256), 0, st, d, nu, ntok, down, map, shared_, moe);
   return hipGetLastError();
 }
