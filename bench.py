@@ -17,7 +17,8 @@ Other workloads (--workload), each BASELINE.json's config of the same number:
       bit-exact int8 path (--path int8, the Q8_K activation quantizer inside the step)
   c4  MoE decode step: 256 resident experts (IQ2_XXS gate/up, Q2_K down), top-6, the Q8_0
       shared expert, rotating over 3 layers' pools (5.4 GB); routing tables made beforehand;
-      --mode fused (default): 5 launches a step; --mode single: the reference's 12
+      --mode fused (default): 5 launches a step; --mode single: the reference's 12;
+      --mode device: routing on the device inside the step (6 launches, no host tables)
   c5  MoE prefill chunk: 4096 tokens, Zipf(1.1)-skewed top-6 routing, route -> group ->
       gather -> grouped gate, up -> gated activation -> grouped down -> ordered sum
 Weights and activations are synthetic and seeded (illatio_amd/synth.py); inputs are resident
@@ -172,7 +173,7 @@ def workload_c2(args, dev):
     ybuf = {name: hip.hip_alloc(dev, 4 * rows) for name, _, rows, _, _ in specs}
     logits = hip.hip_alloc(dev, 4 * VOCAB)
     tm = Timer(dev)
-    fused, inq = args.mode != "single", args.mode == "fused"
+    fused, inq = args.mode != "single", args.mode in ("fused", "device")
 
     def step(_):
         for L in layers:
@@ -219,7 +220,7 @@ def workload_c2(args, dev):
     roof = roofline_of({"gemv": allk}, "hbm", HBM_PEAK_GBS, "GB/s",
                        {"gemv": "gemv_kernel<FMT> (decode product: Q4_K, Q6_K and the fused Q4_K+Q6_K launch)"})
     roof["by_launch_shape"] = shapes
-    roof["traffic"] = traffic_of("c2", per) if (args.mode == "fused" and nl == LAYERS) else None
+    roof["traffic"] = traffic_of("c2", per) if (args.mode in ("fused", "device") and nl == LAYERS) else None
     gbs = step_bytes / (ms * 1e-3) / 1e9
 
     def cpu():
@@ -368,11 +369,16 @@ def workload_c4(args, dev):
     xb = hip.hip_upload_new(dev, x)
     nsteps = args.steps + args.warmup + 3
     tables, routes = [], []
-    fused = args.mode == "fused"
+    fused, ondev = args.mode == "fused", args.mode == "device"
+    logits = []
     for i in range(nsteps):                      # the reference routes on the CPU (cuda-ds4f.lisp:991-999); tables made beforehand
-        sel, w = orc.route(synth.activations(ne, rng), nu, 1.5)
+        lg = synth.activations(ne, rng)
+        sel, w = orc.route(lg, nu, 1.5)
         routes.append((sel, w))
-        tables.append((ds4f.fused_tables if fused else ds4f.tail_tables)(dev, pools[i % nlayers], sel, w))
+        if ondev:                                # device mode: only the router's logits are resident; d4_route runs in the step
+            logits.append(hip.hip_upload_new(dev, lg))
+        else:
+            tables.append((ds4f.fused_tables if fused else ds4f.tail_tables)(dev, pools[i % nlayers], sel, w))
     ws = hip.Workspace(dev, 8 << 20)
     iq, q2, q8 = synth.row_bytes(synth.IQ2_XXS, d), synth.row_bytes(synth.Q2_K, ff), 34
     step_bytes = nu * (2 * ff * iq + d * q2) + 2 * ff * d // 32 * q8 + d * ff // 32 * q8
@@ -382,7 +388,9 @@ def workload_c4(args, dev):
         ws.reset()
         L = i % nlayers
         sel, w = routes[i]
-        if fused:
+        if ondev:
+            ds4f.ffn_step_device(dev, pools[L], shared[L], logits[i], xb, ne, nu, 1.5, 0.0, ws=ws)
+        elif fused:
             ds4f.ffn_step_fused(dev, pools[L], shared[L], sel, w, xb, 0.0, ws=ws, tables=tables[i])
         else:
             ds4f.ffn_tail(dev, pools[L], sel, w, xb, ds4f.ffn_shared(dev, shared[L], xb, 0.0, ws=ws), 0.0, ws=ws, tables=tables[i])
@@ -425,7 +433,7 @@ def workload_c4(args, dev):
             "metric": "MoE decode step achieved HBM GB/s (% of 8 TB/s)",
             "config": {"workload": f"c4: MoE decode step, 256 resident experts (IQ2_XXS gate/up, Q2_K down) top-6 + Q8_0 shared expert, "
                                    f"d 4096, ff 2048, batch 1, rotating over {nlayers} layers", "bytes_per_step": step_bytes},
-            "extra": {"pct_of_hbm_peak": round(100 * gbs / HBM_PEAK_GBS, 2), "launches_per_step": 5 if fused else 12,
+            "extra": {"pct_of_hbm_peak": round(100 * gbs / HBM_PEAK_GBS, 2), "launches_per_step": 6 if ondev else 5 if fused else 12,
                       "launch_mode": args.mode}, "roofline": roof, "cpu": cpu}
 
 
@@ -502,8 +510,9 @@ def main():
     ap.add_argument("--tokens", type=int, default=4096, help="c3, c5: tokens per step")
     ap.add_argument("--transpose", action="store_true", help="c3: the 5120x17408 matrix")
     ap.add_argument("--path", default="bf16", choices=["bf16", "int8"], help="c3, c5: which matrix-core path")
-    ap.add_argument("--mode", default="fused", choices=["fused", "fused-q", "single"],
-                    help="c4: fused = 5 launches a step, single = the reference's sequence of 12.  c2: fused = Q/K/V in one launch, gate+up in one, activations quantized inside the product "
+    ap.add_argument("--mode", default="fused", choices=["fused", "fused-q", "single", "device"],
+                    help="c4: fused = 5 launches a step, single = the reference's sequence of 12 (both with the routing done beforehand on the host, as the "
+                         "reference routes on the CPU), device = the routing kernel inside the step and the expert kernels indexing the slot table by its result (6 launches).  c2: fused = Q/K/V in one launch, gate+up in one, activations quantized inside the product "
                          "kernels; fused-q = the same launches after separate quantizer launches; "
                          "single = one launch per matrix after separate quantizer launches")
     args = ap.parse_args()

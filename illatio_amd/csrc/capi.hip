@@ -264,7 +264,8 @@ int ilt_d4_mvq8(uint64_t stream, int rows, int cols, int group_rows, const int8_
 // xf: the activations as floats, quantized to Q8_K in the kernel; else xq, xd, bsums.
 static int gemv_experts(uint64_t stream, int fmt, int ncols, int nrows, int row_bytes, int64_t add, int64_t add_up,
                         int x_stride, int y_stride, const uint64_t* ptrs, int nz, const int8_t* xq, const float* xd,
-                        const int32_t* bsums, const float* xf, const float* wts, float clamp, float* dst) {
+                        const int32_t* bsums, const float* xf, const float* wts, float clamp, float* dst,
+                        const uint32_t* sel = nullptr) {
   ILT_REQUIRE(nrows >= 0 && nz >= 0 && ncols > 0 && ncols % 256 == 0 && row_bytes == ncols / 256 * block_bytes(fmt));
   if (nrows == 0 || nz == 0) return ILT_OK;
   ILT_REQUIRE(ptrs && dst && add >= 0 && (add & 1) == 0 && (add_up < 0 || (add_up & 1) == 0) && x_stride % 256 == 0 && x_stride >= 0);
@@ -277,7 +278,7 @@ static int gemv_experts(uint64_t stream, int fmt, int ncols, int nrows, int row_
     p.nmat = 2; p.mat[1] = p.mat[0]; p.mat[1].add = add_up;
     p.glu = 2; p.clamp = clamp; p.wts = wts;
   }
-  p.ptrs = ptrs; p.cols = ncols;
+  p.ptrs = ptrs; p.sel = sel; p.cols = ncols;
   p.xq = xq; p.xs = xd; p.bsums = bsums; p.xf = xf; p.x_stride = x_stride; p.y_stride = y_stride;
   return (int)ilt_gemv_launch(p, nz, S(stream));
 }
@@ -295,18 +296,18 @@ int ilt_d4_mv_q2_k(uint64_t stream, int ncols, int nrows, int row_bytes, int64_t
 }
 
 int ilt_d4_mv_glu_iq2_xxs(uint64_t stream, int ncols, int nrows, int row_bytes, int64_t add_gate, int64_t add_up,
-                          int x_stride, int y_stride, const uint64_t* ptrs, int nz, const float* x, const float* wts,
-                          float clamp, float* mid) {
+                          int x_stride, int y_stride, const uint64_t* ptrs, const uint32_t* sel, int nz, const float* x,
+                          const float* wts, float clamp, float* mid) {
   ILT_REQUIRE(add_up >= 0 && x);
   return gemv_experts(stream, ILT_IQ2_XXS, ncols, nrows, row_bytes, add_gate, add_up, x_stride, y_stride, ptrs, nz,
-                      nullptr, nullptr, nullptr, x, wts, clamp, mid);
+                      nullptr, nullptr, nullptr, x, wts, clamp, mid, sel);
 }
 
 int ilt_d4_mv_q2_k_f32(uint64_t stream, int ncols, int nrows, int row_bytes, int64_t add, int x_stride, int y_stride,
-                       const uint64_t* ptrs, int nz, const float* x, float* dst) {
+                       const uint64_t* ptrs, const uint32_t* sel, int nz, const float* x, float* dst) {
   ILT_REQUIRE(x);
   return gemv_experts(stream, ILT_Q2_K, ncols, nrows, row_bytes, add, -1, x_stride, y_stride, ptrs, nz, nullptr, nullptr,
-                      nullptr, x, nullptr, 0.0f, dst);
+                      nullptr, x, nullptr, 0.0f, dst, sel);
 }
 
 int ilt_d4_mvq8_glu(uint64_t stream, int rows, int cols, const int8_t* gq, const uint16_t* gd, const int8_t* uq,
@@ -512,10 +513,10 @@ int ilt_launch(const char* kernel, unsigned gx, unsigned gy, unsigned gz, unsign
                                     a.ptr<cf>(5), a.ptr<const int32_t*>(6), a.ptr<float*>(7), a.i32(8), a.i32(9));
   K("d4_mv_glu_iq2_xxs")
     return ilt_d4_mv_glu_iq2_xxs(stream, a.i32(0), a.i32(1), a.i32(2), a.i64(3), a.i64(4), a.i32(5), a.i32(6),
-                                 a.ptr<const uint64_t*>(7), (int)gz, a.ptr<cf>(8), a.ptr<cf>(9), a.f32(10), a.ptr<float*>(11));
+                                 a.ptr<const uint64_t*>(7), a.ptr<cu32>(8), (int)gz, a.ptr<cf>(9), a.ptr<cf>(10), a.f32(11), a.ptr<float*>(12));
   K("d4_mv_q2_k_f32")
     return ilt_d4_mv_q2_k_f32(stream, a.i32(0), a.i32(1), a.i32(2), a.i64(3), a.i32(4), a.i32(5), a.ptr<const uint64_t*>(6),
-                              (int)gz, a.ptr<cf>(7), a.ptr<float*>(8));
+                              a.ptr<cu32>(7), (int)gz, a.ptr<cf>(8), a.ptr<float*>(9));
   K("d4_mvq8_glu") return ilt_d4_mvq8_glu(stream, a.i32(0), a.i32(1), a.ptr<ci8>(2), a.ptr<cu16>(3), a.ptr<ci8>(4), a.ptr<cu16>(5),
                                           a.ptr<cf>(6), a.f32(7), a.ptr<float*>(8));
   K("d4_mvq8") return ilt_d4_mvq8(stream, a.i32(0), a.i32(1), a.i32(2), a.ptr<ci8>(3), a.ptr<cu16>(4), a.ptr<ci8>(5),

@@ -32,7 +32,8 @@ struct IltGemvMat {
 struct IltGemvParams {
   IltGemvMat mat[4];         // up to four matrices sharing the activations
   int nmat;
-  const uint64_t* ptrs;      // experts: grid y's matrices are at ptrs[y] + mat[i].add
+  const uint64_t* ptrs;      // experts: grid y's matrices are at ptrs[y] + mat[i].add,
+  const uint32_t* sel;       //   or at ptrs[sel[y]] + mat[i].add when sel is given (ptrs = all the slots)
   int cols;
   const int8_t* xq;          // quantized activations ...
   const float* xs;           //   their block scales (per 32 for Q8_0, per 256 otherwise)

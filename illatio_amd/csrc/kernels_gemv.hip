@@ -385,7 +385,7 @@ __device__ __forceinline__ void stage_q8_from_f32(const float* __restrict__ x, i
 template <int FMT>
 __device__ __forceinline__ void run_rows(const IltGemvMat& m, const IltGemvParams& p, long row0, int nrows, int S,
                                          const Lds& L, float* t, int lane, int z, const Raw<FMT>& pre, bool use_pre) {
-  const u8* w = p.ptrs ? (const u8*)(p.ptrs[z] + m.add) : m.w;
+  const u8* w = p.ptrs ? (const u8*)(p.ptrs[p.sel ? p.sel[z] : z] + m.add) : m.w;
   wave_rows<FMT>(w, m.wd, row0, nrows, S, p.s_magic, m.row_bytes, L, t, lane, pre, use_pre);
 }
 
@@ -463,7 +463,7 @@ __global__ __launch_bounds__(kThreads) void gemv_kernel(IltGemvParams p) {
     int mi; long row0; int nrows;
     locate(wid, mi, row0, nrows);
     const IltGemvMat& m = p.mat[mi];
-    const u8* w0 = p.ptrs ? (const u8*)(p.ptrs[z] + m.add) : m.w;
+    const u8* w0 = p.ptrs ? (const u8*)(p.ptrs[p.sel ? p.sel[z] : z] + m.add) : m.w;
     if (FSET != 0 || m.fmt == ILT_Q4_K) first_load<(FSET ? FSET : ILT_Q4_K)>(pre.a, w0, m.wd, row0, nrows, S, m.row_bytes, lane);
     else first_load<(FSET ? FSET : ILT_Q6_K)>(pre.b, w0, m.wd, row0, nrows, S, m.row_bytes, lane);
     // and a touch of every 64-byte line of the batch's first 16 KB, so the later steps hit in L2

@@ -143,29 +143,47 @@ def fused_tables(dev, pool, sel, w):
             hip.hip_upload_new(dev, np.asarray(w, np.float32)))
 
 
-def ffn_step_fused(dev, pool, sh, sel, w, norm2, clamp, ws=None, tables=None):
+def ffn_step_fused(dev, pool, sh, sel, w, norm2, clamp, ws=None, tables=None, routed=None):
     """One token's shared expert and routed experts in five launches, with ffn_shared's and
     ffn_tail's bits: the shared expert's gate, up and gated activation in one launch and its
     down in one (both quantizing their float input in the kernel); the routed experts' gates,
     ups and gated activations in one launch over k expert slots, their downs in one, then
-    the ordered sum.  Returns MOE."""
-    d, ff, k = pool.d, pool.ff, len(sel)
+    the ordered sum.  Returns MOE.  ROUTED = (sel, w) DBufs as d4_route left them on the
+    device (k of them): the kernels then index the pool's slot table by sel themselves and
+    SEL, W are not used (pass k as SEL)."""
+    d, ff = pool.d, pool.ff
+    k = sel if routed else len(sel)
     gb = pool.gate_bytes
     A = ws.alloc if ws else hip.hip_alloc
-    ptrs, bw = tables if tables else fused_tables(dev, pool, sel, w)
+    dsel = None
+    if routed:
+        ptrs, (dsel, bw), tables = pool.ptrs, routed, True
+    else:
+        ptrs, bw = tables if tables else fused_tables(dev, pool, sel, w)
     smid, sout = A(dev, 4 * ff), A(dev, 4 * d)
     bm, bd, moe = A(dev, 4 * k * ff), A(dev, 4 * k * d), A(dev, 4 * d)
     hip.launch(dev, "d4_mvq8_glu", (ff + 3) // 4, 128, [ff, d, sh.gate.qs, sh.gate.d, sh.up.qs, sh.up.d, norm2, float(clamp), smid])
     dense.mv_multi(dev, [(sh.down, sout, None)], xf=smid, f16_scale=False)
     hip.launch(dev, "d4_mv_glu_iq2_xxs", ((ff + 7) // 8, 1, k), 64,
-               [d, ff, pool.grb, hip.I64(0), hip.I64(gb), 0, ff, ptrs, norm2, bw, float(clamp), bm])
-    hip.launch(dev, "d4_mv_q2_k_f32", ((d + 7) // 8, 1, k), 64, [ff, d, pool.drb, hip.I64(2 * gb), ff, d, ptrs, bm, bd])
+               [d, ff, pool.grb, hip.I64(0), hip.I64(gb), 0, ff, ptrs, dsel, norm2, bw, float(clamp), bm])
+    hip.launch(dev, "d4_mv_q2_k_f32", ((d + 7) // 8, 1, k), 64, [ff, d, pool.drb, hip.I64(2 * gb), ff, d, ptrs, dsel, bm, bd])
     hip.launch(dev, "d4_moe_sum", (d + 255) // 256, 256, [d, k, bd, sout, moe, None])
     if ws:
         return moe
     hip.hip_sync(dev)
     for b in (smid, sout, bm, bd) + (() if tables else (ptrs, bw)):
         hip.hip_free(b)
+    return moe
+
+
+def ffn_step_device(dev, pool, sh, logits, norm2, ne, nu, scale, clamp, bias=None, ws=None):
+    """A decode step with nothing going through the host: d4_route on the device, then
+    ffn_step_fused indexing the slot table by its result (six launches)."""
+    A = ws.alloc if ws else hip.hip_alloc
+    sel, w = route(dev, logits, 1, ne, nu, scale, bias, A)
+    moe = ffn_step_fused(dev, pool, sh, nu, None, norm2, clamp, ws=ws, routed=(sel, w))
+    if not ws:
+        hip.hip_free(sel); hip.hip_free(w)
     return moe
 
 

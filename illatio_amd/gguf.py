@@ -1,0 +1,152 @@
+"""The GGUF container: header, metadata, tensor directory -- the host side of the reference's
+src/gguf.lisp (READ-GGUF :105-147, GGUF-TENSOR :149-151, tensor bytes :153-157), plus the
+step from a tensor in a file to a matrix on the device (UPLOAD-GMAT, cuda-dense.lisp:75-100).
+
+All integers little-endian.  The header and directory are parsed; tensor data stays on
+disk and is memory-mapped one tensor at a time, so a model is never held twice in memory.
+"""
+import struct
+
+import numpy as np
+
+MAGIC = 0x46554747          # "GGUF"
+
+# ggml type code -> (name, elements per block, bytes per block)   (gguf.lisp:31-44)
+GGML_TYPES = {
+    0: ("f32", 1, 4), 1: ("f16", 1, 2), 2: ("q4_0", 32, 18), 3: ("q4_1", 32, 20), 6: ("q5_0", 32, 22), 7: ("q5_1", 32, 24),
+    8: ("q8_0", 32, 34), 9: ("q8_1", 32, 36), 10: ("q2_k", 256, 84), 11: ("q3_k", 256, 110), 12: ("q4_k", 256, 144),
+    13: ("q5_k", 256, 176), 14: ("q6_k", 256, 210), 15: ("q8_k", 256, 292), 16: ("iq2_xxs", 256, 66), 17: ("iq2_xs", 256, 74),
+    18: ("iq3_xxs", 256, 98), 19: ("iq1_s", 256, 50), 20: ("iq4_nl", 32, 18), 21: ("iq3_s", 256, 110), 22: ("iq2_s", 256, 82),
+    23: ("iq4_xs", 256, 136), 24: ("i8", 1, 1), 25: ("i16", 1, 2), 26: ("i32", 1, 4), 27: ("i64", 1, 8), 28: ("f64", 1, 8),
+    29: ("iq1_m", 256, 56), 30: ("bf16", 1, 2), 39: ("mxfp4", 32, 17),
+}
+
+
+class GgufError(ValueError):
+    pass
+
+
+class TensorInfo:
+    """NAME, DIMS in ggml order (ne0 is the contiguous axis), TYPE (ggml type code), OFFSET
+    relative to the data section."""
+    __slots__ = ("name", "dims", "type", "offset")
+
+    def __init__(self, name, dims, type_, offset):
+        self.name, self.dims, self.type, self.offset = name, tuple(dims), type_, offset
+
+    @property
+    def type_name(self):
+        return GGML_TYPES[self.type][0]
+
+    def elements(self):
+        n = 1
+        for d in self.dims:
+            n *= d
+        return n
+
+    def nbytes(self):
+        _, block, nb = GGML_TYPES[self.type]
+        return self.elements() // block * nb
+
+
+class Gguf:
+    def __init__(self, path):
+        self.path, self.version, self.metadata, self.tensors, self.tensor_order = path, 0, {}, {}, []
+        self.data_offset, self.alignment = 0, 32
+
+    def meta(self, key, default=None):
+        return self.metadata.get(key, default)
+
+
+class _Reader:
+    def __init__(self, f):
+        self.f = f
+
+    def take(self, n):
+        b = self.f.read(n)
+        if len(b) != n:
+            raise GgufError("GGUF: unexpected end of file")
+        return b
+
+    def uint(self, n):
+        return int.from_bytes(self.take(n), "little", signed=False)
+
+    def sint(self, n):
+        return int.from_bytes(self.take(n), "little", signed=True)
+
+    def string(self):
+        n = self.uint(8)
+        return self.take(n).decode("utf-8", errors="replace")
+
+    def value(self, t):
+        if t in (0, 2, 4, 10):
+            return self.uint({0: 1, 2: 2, 4: 4, 10: 8}[t])
+        if t in (1, 3, 5, 11):
+            return self.sint({1: 1, 3: 2, 5: 4, 11: 8}[t])
+        if t == 6:
+            return struct.unpack("<f", self.take(4))[0]
+        if t == 7:
+            return self.uint(1) != 0
+        if t == 8:
+            return self.string()
+        if t == 9:
+            et, n = self.uint(4), self.uint(8)
+            return [self.value(et) for _ in range(n)]
+        if t == 12:
+            return struct.unpack("<d", self.take(8))[0]
+        raise GgufError(f"GGUF: unknown metadata value type {t}")
+
+
+def read_gguf(path):
+    """The header, metadata and tensor directory of the GGUF file at PATH (READ-GGUF)."""
+    with open(path, "rb") as f:
+        r = _Reader(f)
+        if r.uint(4) != MAGIC:
+            raise GgufError(f"{path} is not a GGUF file")
+        g = Gguf(path)
+        g.version = r.uint(4)
+        n_tensors, n_kv = r.uint(8), r.uint(8)
+        if g.version not in (2, 3):
+            raise GgufError(f"GGUF version {g.version} is not supported (2 and 3 are)")
+        for _ in range(n_kv):
+            key = r.string()
+            g.metadata[key] = r.value(r.uint(4))
+        g.alignment = g.meta("general.alignment", 32)
+        for _ in range(n_tensors):
+            name = r.string()
+            nd = r.uint(4)
+            dims = [r.uint(8) for _ in range(nd)]
+            code = r.uint(4)
+            if code not in GGML_TYPES:
+                raise GgufError(f"GGUF: unknown ggml tensor type {code}")
+            g.tensors[name] = TensorInfo(name, dims, code, r.uint(8))
+            g.tensor_order.append(name)
+        a, p = g.alignment, f.tell()
+        g.data_offset = a * ((p + a - 1) // a)
+    return g
+
+
+def gguf_tensor(g, name, errorp=True):
+    ti = g.tensors.get(name)
+    if ti is None and errorp:
+        raise GgufError(f"GGUF: no tensor named {name!r}")
+    return ti
+
+
+def tensor_bytes(g, ti):
+    """The tensor's raw bytes as a read-only memory map (nothing is copied until it is used)."""
+    n = ti.nbytes()
+    m = np.memmap(g.path, dtype=np.uint8, mode="r", offset=g.data_offset + ti.offset, shape=(n,)) if n else np.zeros(0, np.uint8)
+    if m.size != n:
+        raise GgufError(f"GGUF: truncated tensor {ti.name}")
+    return m
+
+
+def upload_tensor(dev, g, name):
+    """The 2-D tensor NAME of G as a matrix on DEV (UPLOAD-GMAT): rows = ne1, columns = ne0."""
+    from . import dense
+    ti = gguf_tensor(g, name)
+    if len(ti.dims) != 2:
+        raise GgufError(f"{name}: {len(ti.dims)} dimensions, a matrix has two")
+    cols, rows = ti.dims
+    return dense.upload_gmat(dev, name, ti.type, rows, cols, tensor_bytes(g, ti))

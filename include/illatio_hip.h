@@ -163,6 +163,10 @@ int ilt_d4_mv_q2_k(uint64_t stream, int ncols, int nrows, int row_bytes, int64_t
    908-956) in fewer launches, with the same bits: the activations come as floats and every
    workgroup quantizes them as quantize-q8k! (experts) or quantize-q8! with a float scale
    (shared expert) does, so no quantizer launch precedes the product.
+   With sel given, ptrs is the table of all the expert slots and slot z of the launch is expert
+   sel[z] -- d4_route's output on the device, so that no routing result goes through the host
+   (the reference's decode path syncs and routes on the CPU in every layer,
+   cuda-ds4f.lisp:991-999); with sel null, ptrs[z] is slot z's address as in d4_mv_*.
    d4_mv_glu_iq2_xxs: for each z < nz, gate at ptrs[z] + add_gate, up at ptrs[z] + add_up,
      x at element z*x_stride (0: one x for all), mid[z*y_stride + r] = (silu(g)*u) * wts[z]
      with g = min(g, clamp), u in [-clamp, clamp] when clamp > 1e-6 (d4_swiglu_w's formula;
@@ -172,10 +176,10 @@ int ilt_d4_mv_q2_k(uint64_t stream, int ncols, int nrows, int row_bytes, int64_t
      activation with weight 1 into mid.  Its down projection is ilt_mv_multi with xf = mid
      and f16_scale 0. */
 int ilt_d4_mv_glu_iq2_xxs(uint64_t stream, int ncols, int nrows, int row_bytes, int64_t add_gate, int64_t add_up,
-                          int x_stride, int y_stride, const uint64_t* ptrs, int nz, const float* x, const float* wts,
-                          float clamp, float* mid);
+                          int x_stride, int y_stride, const uint64_t* ptrs, const uint32_t* sel, int nz, const float* x,
+                          const float* wts, float clamp, float* mid);
 int ilt_d4_mv_q2_k_f32(uint64_t stream, int ncols, int nrows, int row_bytes, int64_t add, int x_stride, int y_stride,
-                       const uint64_t* ptrs, int nz, const float* x, float* dst);
+                       const uint64_t* ptrs, const uint32_t* sel, int nz, const float* x, float* dst);
 int ilt_d4_mvq8_glu(uint64_t stream, int rows, int cols, const int8_t* gq, const uint16_t* gd, const int8_t* uq,
                     const uint16_t* ud, const float* x, float clamp, float* mid);
 

@@ -1,0 +1,104 @@
+"""The GGUF reader (illatio_amd/gguf.py ~ src/gguf.lisp) against files written by
+tests/gguf_writer.py: metadata kinds, the tensor directory, alignment of the data section,
+tensor sizes of the five block formats, the reference's error cases; and, on the GPU, a file's
+tensors uploaded and multiplied with the oracle's bits."""
+import struct
+
+import numpy as np
+import pytest
+
+from illatio_amd import gguf, synth
+from gguf_writer import write_gguf
+
+
+def _tensors(rng):
+    return [("blk.0.attn_q.weight", (512, 96), synth.Q4_K, synth.weights(synth.Q4_K, 96, 512, rng)),
+            ("blk.0.attn_v.weight", (512, 40), synth.Q6_K, synth.weights(synth.Q6_K, 40, 512, rng)),
+            ("blk.0.ffn_up.weight", (128, 72), synth.Q8_0, synth.weights(synth.Q8_0, 72, 128, rng)),
+            ("blk.0.ffn_gate_exps.weight", (256, 16, 3), synth.IQ2_XXS, synth.weights(synth.IQ2_XXS, 48, 256, rng)),
+            ("blk.0.ffn_down_exps.weight", (256, 8, 3), synth.Q2_K, synth.weights(synth.Q2_K, 24, 256, rng)),
+            ("output_norm.weight", (512,), 0, np.arange(512, dtype=np.float32).view(np.uint8))]
+
+
+@pytest.mark.parametrize("alignment", [None, 64, 4096])
+def test_directory_metadata_and_bytes(tmp_path, alignment):
+    rng = synth.make_rng(3)
+    ts = _tensors(rng)
+    md = {"general.architecture": "qwen3", "qwen3.block_count": 36, "qwen3.rope.freq_base": 1000000.0, "flag": True,
+          "neg": -5, "tokenizer.ggml.tokens": ["a", "bc", "é"], "tokenizer.ggml.scores": [0.5, -1.0], "empty": []}
+    p = tmp_path / "m.gguf"
+    write_gguf(p, md, ts, alignment=alignment)
+    g = gguf.read_gguf(str(p))
+    assert g.version == 3 and g.alignment == (alignment or 32) and g.data_offset % g.alignment == 0
+    assert g.meta("general.architecture") == "qwen3" and g.meta("qwen3.block_count") == 36 and g.meta("flag") is True
+    assert g.meta("neg") == -5 and g.meta("tokenizer.ggml.tokens") == ["a", "bc", "é"] and g.meta("empty") == []
+    assert g.meta("qwen3.rope.freq_base") == 1000000.0 and g.meta("missing", 7) == 7
+    assert g.tensor_order == [t[0] for t in ts]
+    for name, dims, code, raw in ts:
+        ti = gguf.gguf_tensor(g, name)
+        assert ti.dims == tuple(dims) and ti.type == code and ti.offset % g.alignment == 0
+        assert ti.nbytes() == raw.size
+        assert np.array_equal(np.asarray(gguf.tensor_bytes(g, ti)), raw.ravel())
+    assert gguf.gguf_tensor(g, "nope", errorp=False) is None
+    with pytest.raises(gguf.GgufError):
+        gguf.gguf_tensor(g, "nope")
+
+
+def test_block_sizes_are_ggml_s():
+    for code, nbytes in ((8, 34), (10, 84), (12, 144), (14, 210), (16, 66)):
+        assert gguf.GGML_TYPES[code][2] == nbytes == synth.BLOCK_BYTES[code]
+
+
+def test_rejects_what_the_reference_rejects(tmp_path):
+    p = tmp_path / "x.gguf"
+    p.write_bytes(b"GGML" + b"\0" * 32)
+    with pytest.raises(gguf.GgufError, match="not a GGUF file"):
+        gguf.read_gguf(str(p))
+    p.write_bytes(struct.pack("<IIQQ", gguf.MAGIC, 1, 0, 0))
+    with pytest.raises(gguf.GgufError, match="version 1"):
+        gguf.read_gguf(str(p))
+    p.write_bytes(struct.pack("<IIQQ", gguf.MAGIC, 3, 1, 0) + struct.pack("<Q", 1) + b"t" + struct.pack("<IQIQ", 1, 32, 99, 0))
+    with pytest.raises(gguf.GgufError, match="unknown ggml tensor type 99"):
+        gguf.read_gguf(str(p))
+    p.write_bytes(struct.pack("<IIQQ", gguf.MAGIC, 3, 0, 1) + struct.pack("<Q", 100) + b"short")
+    with pytest.raises(gguf.GgufError, match="end of file"):
+        gguf.read_gguf(str(p))
+    write_gguf(p, {}, [("w", (256, 4), synth.Q4_K, synth.weights(synth.Q4_K, 4, 256, synth.make_rng(1)))])
+    data = p.read_bytes()
+    p.write_bytes(data[:-100])                     # the tensor's last bytes are missing
+    g = gguf.read_gguf(str(p))
+    with pytest.raises((gguf.GgufError, ValueError)):
+        gguf.tensor_bytes(g, gguf.gguf_tensor(g, "w"))
+
+
+def test_version_2_reads_like_3(tmp_path):
+    p = tmp_path / "v2.gguf"
+    write_gguf(p, {"k": 1}, [], version=2)
+    g = gguf.read_gguf(str(p))
+    assert g.version == 2 and g.meta("k") == 1 and g.tensor_order == []
+
+
+@pytest.mark.gpu
+def test_tensors_of_a_file_multiply_with_the_oracles_bits(tmp_path):
+    import oracle_lib as orc
+    from illatio_amd import dense, hip
+    dev = hip.open_hip(0)
+    rng = synth.make_rng(9)
+    ts = _tensors(rng)
+    p = tmp_path / "m.gguf"
+    write_gguf(p, {"general.architecture": "test"}, ts, alignment=64)
+    g = gguf.read_gguf(str(p))
+    for name, dims, code, raw in ts[:3]:
+        cols, rows = dims
+        m = gguf.upload_tensor(dev, g, name)
+        assert (m.rows, m.cols, m.type) == (rows, cols, code)
+        x = synth.activations(cols, rng)
+        xb, y = hip.hip_upload_new(dev, x), hip.hip_alloc(dev, 4 * rows)
+        dense.mv_multi(dev, [(m, y, None)], xf=xb)
+        want = orc.matmul(code, raw, rows, cols, x)
+        assert np.array_equal(hip.hip_floats(y, rows).view(np.uint32), want.view(np.uint32))
+        for b in (xb, y):
+            hip.hip_free(b)
+        m.free()
+    with pytest.raises(gguf.GgufError):
+        gguf.upload_tensor(dev, g, "output_norm.weight")

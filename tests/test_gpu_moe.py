@@ -154,6 +154,10 @@ def test_moe_decode_step_bit_exact(dev, ne, d, ff, nu, clamp):
         fused = ds4f.ffn_step_fused(dev, pool, sh, hsel, hw, nb, clamp)
         got = hip.hip_floats(fused, d)
         assert np.array_equal(bits(got), bits(want)), np.abs(got - want).max()
-        for b in (lb, nb, sel, w, sout, moe, fused):
+        # and with the routing left on the device (six launches, no host round trip)
+        ondev = ds4f.ffn_step_device(dev, pool, sh, lb, nb, ne, nu, 1.5, clamp)
+        got = hip.hip_floats(ondev, d)
+        assert np.array_equal(bits(got), bits(want)), np.abs(got - want).max()
+        for b in (lb, nb, sel, w, sout, moe, fused, ondev):
             hip.hip_free(b)
     pool.free(); sh.free()
