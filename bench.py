@@ -174,42 +174,52 @@ def workload_c2(args, dev):
     logits = hip.hip_alloc(dev, 4 * VOCAB)
     tm = Timer(dev)
     fused, inq = args.mode != "single", args.mode in ("fused", "device")
+    # --norm: the layer's two norms and the output norm as well (rmsnorm!, model.lisp:205-216): inside the
+    # product launches when they quantize for themselves, else as rmsnorm_q8k launches in the quantizers' place
+    nwb = hip.hip_upload_new(dev, (synth.activations(D, rng) * 0.2 + 1.0).astype(np.float32)) if args.norm else None
+    norm = (nwb, 1e-6) if (args.norm and inq) else None
+
+    def quantize_x():
+        if args.norm:
+            dense.rmsnorm_q8(dev, xbuf["x"], nwb, acts["x"], D, 1e-6)
+        else:
+            dense.quantize_act(dev, xbuf["x"], acts["x"])
 
     def step(_):
         for L in layers:
             if fused:
                 xf = xbuf["x"] if inq else None
                 if not inq:
-                    dense.quantize_act(dev, xbuf["x"], acts["x"])
+                    quantize_x()
                 tm.launch("qkv", wbytes["wq"] + wbytes["wk"] + wbytes["wv"] + D + 4 * (QD + 2 * KVD),
-                          lambda: dense.qkv_mul(dev, L["wq"], L["wk"], L["wv"], acts["x"], ybuf["wq"], ybuf["wk"], ybuf["wv"], xf=xf))
+                          lambda: dense.qkv_mul(dev, L["wq"], L["wk"], L["wv"], acts["x"], ybuf["wq"], ybuf["wk"], ybuf["wv"], xf=xf, norm=norm))
                 if not inq:
                     dense.quantize_act(dev, xbuf["att"], acts["att"])
                 tm.launch("wo", wbytes["wo"] + QD + 4 * D,
                           lambda: dense.mv_multi(dev, [(L["wo"], ybuf["wo"], None)], acts["att"], xf=xbuf["att"] if inq else None))
                 if not inq:
-                    dense.quantize_act(dev, xbuf["x"], acts["x"])
+                    quantize_x()
                 tm.launch("glu", wbytes["gate"] + wbytes["up"] + D + 4 * FFN,
-                          lambda: dense.glu_mul(dev, L["gate"], L["up"], acts["x"], ybuf["gate"], xf=xf))
+                          lambda: dense.glu_mul(dev, L["gate"], L["up"], acts["x"], ybuf["gate"], xf=xf, norm=norm))
                 if inq:
                     tm.launch("down", wbytes["down"] + FFN + 4 * D, lambda: dense.mv_multi(dev, [(L["down"], ybuf["down"], None)], xf=xbuf["mid"]))
                 else:
                     dense.quantize_act(dev, xbuf["mid"], acts["mid"])
                     tm.launch("down", wbytes["down"] + FFN + 4 * D, lambda: dense.cmat_mul(dev, L["down"], acts["mid"], ybuf["down"]))
             else:
-                dense.quantize_act(dev, xbuf["x"], acts["x"])
+                quantize_x()
                 for name, qt, rows, cols, src in specs:
                     if name == "wo":
                         dense.quantize_act(dev, xbuf["att"], acts["att"])
                     if name == "gate":
-                        dense.quantize_act(dev, xbuf["x"], acts["x"])
+                        quantize_x()
                     if name == "down":
                         dense.quantize_act(dev, xbuf["mid"], acts["mid"])
                     tm.launch(name, wbytes[name] + cols + 4 * rows, lambda: dense.cmat_mul(dev, L[name], acts[src], ybuf[name]))
         if inq:
-            tm.launch("head", head_host.size + D + 4 * VOCAB, lambda: dense.mv_multi(dev, [(head, logits, None)], xf=xbuf["x"]))
+            tm.launch("head", head_host.size + D + 4 * VOCAB, lambda: dense.mv_multi(dev, [(head, logits, None)], xf=xbuf["x"], norm=norm))
         else:
-            dense.quantize_act(dev, xbuf["x"], acts["x"])
+            quantize_x()
             tm.launch("head", head_host.size + D + 4 * VOCAB, lambda: dense.cmat_mul(dev, head, acts["x"], logits))
 
     ms, dev_ms, per = tm.run(step, args.steps, args.warmup)
@@ -243,7 +253,7 @@ def workload_c2(args, dev):
             "dtype": "int8 block dots, fp32 combine",
             "config": {"workload": f"c2: qwen3-4b-shape decode, the {nl * 7 + 1} quantized matvecs of one token "
                                    f"({nl} layers x 7 + output head), Q4_K/Q6_K, batch 1",
-                       "bytes_per_step": step_bytes, "layers": nl, "launch_mode": args.mode},
+                       "bytes_per_step": step_bytes, "layers": nl, "launch_mode": args.mode, "norms_included": bool(args.norm)},
             "extra": {"pct_of_hbm_peak": round(100 * gbs / HBM_PEAK_GBS, 2), "matvec_only_tok_per_s": round(1e3 / ms, 1)},
             "roofline": roof, "cpu": cpu}
 
@@ -510,6 +520,7 @@ def main():
     ap.add_argument("--tokens", type=int, default=4096, help="c3, c5: tokens per step")
     ap.add_argument("--transpose", action="store_true", help="c3: the 5120x17408 matrix")
     ap.add_argument("--path", default="bf16", choices=["bf16", "int8"], help="c3, c5: which matrix-core path")
+    ap.add_argument("--norm", action="store_true", help="c2: include each layer's two norms and the output norm (inside the product launches in fused mode)")
     ap.add_argument("--mode", default="fused", choices=["fused", "fused-q", "single", "device"],
                     help="c4: fused = 5 launches a step, single = the reference's sequence of 12 (both with the routing done beforehand on the host, as the "
                          "reference routes on the CPU), device = the routing kernel inside the step and the expert kernels indexing the slot table by its result (6 launches).  c2: fused = Q/K/V in one launch, gate+up in one, activations quantized inside the product "

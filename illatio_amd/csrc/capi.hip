@@ -171,7 +171,7 @@ int ilt_quant_q8k(uint64_t stream, const float* x, int8_t* xq, float* xd, int32_
 static int gemv_multi(uint64_t stream, int nmat, const int* fmts, const void* const* ws, const uint16_t* const* wds,
                       float* const* ys, const float* const* biases, const int* rows, int cols, const int8_t* xq,
                       const float* xs, const int32_t* bsums, const float* xf, int f16_scale, int acc, int glu,
-                      int group_rows) {
+                      int group_rows, const float* norm_w = nullptr, float eps = 0.0f, int norm_seq = 0) {
   ILT_REQUIRE(nmat >= 1 && nmat <= 4 && cols > 0);
   const bool q8 = fmts[0] == ILT_Q8_0;
   IltGemvParams p = {};
@@ -189,9 +189,10 @@ static int gemv_multi(uint64_t stream, int nmat, const int* fmts, const void* co
   }
   if (live == 0) return ILT_OK;
   if (glu) ILT_REQUIRE(live == 2 && p.mat[0].rows == p.mat[1].rows && !acc);
-  if (xf) ILT_REQUIRE(((uintptr_t)xf & 15) == 0);
-  else ILT_REQUIRE(xq && xs && (q8 || bsums) && ((uintptr_t)xq & 15) == 0);
+  if (xf) ILT_REQUIRE(((uintptr_t)xf & 15) == 0 && ((uintptr_t)norm_w & 15) == 0);
+  else ILT_REQUIRE(!norm_w && xq && xs && (q8 || bsums) && ((uintptr_t)xq & 15) == 0);
   p.nmat = live; p.cols = cols; p.xq = xq; p.xs = xs; p.bsums = bsums; p.xf = xf; p.f16_scale = f16_scale;
+  p.norm_w = norm_w; p.eps = eps; p.norm_seq = norm_seq;
   p.acc = acc; p.glu = glu;
   if (group_rows > 0 && group_rows < p.mat[0].rows) {
     ILT_REQUIRE(live == 1 && p.mat[0].rows % group_rows == 0);
@@ -252,6 +253,37 @@ int ilt_mv_multi(uint64_t stream, int nmat, const ilt_mv_desc* descs, int cols, 
     ys[i] = descs[i].y; bs[i] = descs[i].bias;
   }
   return gemv_multi(stream, nmat, fmts, ws, wds, ys, bs, rows, cols, xq, xs, bsums, xf, f16_scale, acc, glu, 0);
+}
+
+int ilt_mv_multi_norm(uint64_t stream, int nmat, const ilt_mv_desc* descs, int cols, const float* x, const float* norm_w,
+                      float eps, int exact_order, int f16_scale, int glu) {
+  ILT_REQUIRE(descs && nmat >= 1 && nmat <= 4 && x && norm_w);
+  int fmts[4], rows[4]; const void* ws[4]; const uint16_t* wds[4]; float* ys[4]; const float* bs[4];
+  for (int i = 0; i < nmat; i++) {
+    fmts[i] = descs[i].gguf_type; rows[i] = descs[i].rows; ws[i] = descs[i].w; wds[i] = descs[i].wd;
+    ys[i] = descs[i].y; bs[i] = descs[i].bias;
+  }
+  return gemv_multi(stream, nmat, fmts, ws, wds, ys, bs, rows, cols, nullptr, nullptr, nullptr, x, f16_scale, 0, glu, 0,
+                    norm_w, eps, exact_order ? 1 : 0);
+}
+
+static int rmsnorm_quant(uint64_t stream, int k, const float* x, const float* w, float* h, int8_t* xq, float* xs, int32_t* xsum,
+                         int dim, float eps, int n, int exact_order) {
+  ILT_REQUIRE(n >= 0 && dim > 0 && dim % (k ? 256 : 32) == 0);
+  if (n == 0) return ILT_OK;
+  ILT_REQUIRE(x && w && xq && xs && (!k || xsum) && ((uintptr_t)x & 15) == 0 && ((uintptr_t)w & 15) == 0 &&
+              ((uintptr_t)h & 15) == 0 && ((uintptr_t)xq & 3) == 0);
+  return (int)ilt_k_rmsnorm_quant(k, x, w, h, xq, xs, xsum, dim, eps, 1, exact_order ? 1 : 0, n, S(stream));
+}
+
+int ilt_rmsnorm_q8(uint64_t stream, const float* x, const float* w, float* h, int8_t* xq, float* xs, int32_t* xsum, int dim,
+                   float eps, int n, int exact_order) {
+  return rmsnorm_quant(stream, 0, x, w, h, xq, xs, xsum, dim, eps, n, exact_order);
+}
+
+int ilt_rmsnorm_q8k(uint64_t stream, const float* x, const float* w, float* h, int8_t* xq, float* xd, int32_t* bsums, int dim,
+                    float eps, int n, int exact_order) {
+  return rmsnorm_quant(stream, 1, x, w, h, xq, xd, bsums, dim, eps, n, exact_order);
 }
 
 int ilt_d4_mvq8(uint64_t stream, int rows, int cols, int group_rows, const int8_t* wq, const uint16_t* wd,
@@ -468,7 +500,7 @@ int ilt_d4_mm_id_bf16(uint64_t stream, int gguf_type, int ncols, int nrows, int 
 int ilt_launch(const char* kernel, unsigned gx, unsigned gy, unsigned gz, unsigned bx, unsigned by, unsigned bz,
                unsigned shared_bytes, uint64_t stream, void** params) {
   ILT_REQUIRE(kernel && params);
-  (void)gy; (void)bx; (void)by; (void)bz; (void)shared_bytes;
+  (void)bx; (void)by; (void)bz; (void)shared_bytes;
   const Args a = { params };
   typedef const int8_t* ci8; typedef const uint16_t* cu16; typedef const float* cf; typedef const uint32_t* cu32;
 #define K(name) if (!strcmp(kernel, name))
@@ -477,6 +509,8 @@ int ilt_launch(const char* kernel, unsigned gx, unsigned gy, unsigned gz, unsign
   K("quant_q8") return ilt_quant_q8(stream, a.ptr<cf>(0), a.ptr<int8_t*>(1), a.ptr<float*>(2), a.ptr<int32_t*>(3), a.i64(4));
   K("d4_quant") return ilt_d4_quant(stream, a.ptr<cf>(0), a.ptr<int8_t*>(1), a.ptr<float*>(2), a.i32(3));
   K("quant_q8k") return ilt_quant_q8k(stream, a.ptr<cf>(0), a.ptr<int8_t*>(1), a.ptr<float*>(2), a.ptr<int32_t*>(3), a.i64(4));
+  K("rmsnorm_q8") return ilt_rmsnorm_q8(stream, a.ptr<cf>(0), a.ptr<cf>(1), a.ptr<float*>(2), a.ptr<int8_t*>(3), a.ptr<float*>(4),
+                                        a.ptr<int32_t*>(5), a.i32(6), a.f32(7), (int)gy, 0);
   K("mv_q8") return ilt_mv_q8(stream, a.ptr<ci8>(0), a.ptr<cu16>(1), a.ptr<ci8>(2), a.ptr<cf>(3), a.ptr<float*>(4),
                               a.ptr<cf>(5), a.i32(6), a.i32(7), a.i32(8));
   K("mv_q8_3") return ilt_mv_q8_3(stream, a.ptr<ci8>(0), a.ptr<cu16>(1), a.ptr<ci8>(2), a.ptr<cu16>(3), a.ptr<ci8>(4),

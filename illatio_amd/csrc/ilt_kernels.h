@@ -39,6 +39,9 @@ struct IltGemvParams {
   const float* xs;           //   their block scales (per 32 for Q8_0, per 256 otherwise)
   const int* bsums;          //   Q8_K: sums of each 16 quants
   const float* xf;           // ... or the activations as floats, quantized by each workgroup
+  const float* norm_w;       //   floats only: quantize rmsnorm!(x) * norm_w instead of x (model.lisp:205-216)
+  float eps;                 //   the norm's epsilon
+  int norm_seq;              //   1 = always add the squares one after another (the CPU's order) instead of when needed
   int f16_scale;             // Q8_0 from floats: store the scale through fp16 (*q8-f16-scale*)
   int x_stride;              // activations of grid y start at y * x_stride elements
   int y_stride;              // outputs of grid y start at y * y_stride
@@ -59,6 +62,9 @@ hipError_t ilt_gemv_launch(IltGemvParams& p, int nz, hipStream_t st);
 
 hipError_t ilt_k_quant_q8(const float* x, int8_t* xq, float* xs, int* xsum, long long nblocks, int f16_scale, hipStream_t st);
 hipError_t ilt_k_quant_q8k(const float* x, int8_t* xq, float* xd, int* bsums, long long nblocks, hipStream_t st);
+// rmsnorm! then quantize-q8! (k 0; xsum may be null) or quantize-q8k! (k 1), a row of DIM floats a workgroup
+hipError_t ilt_k_rmsnorm_quant(int k, const float* x, const float* w, float* h, int8_t* xq, float* xs, int* xsum, int dim,
+                               float eps, int f16_scale, int seq, int nrows, hipStream_t st);
 hipError_t ilt_k_repack_q8(const uint8_t* raw, int8_t* qs, uint16_t* d, long long nblocks, hipStream_t st);
 hipError_t ilt_k_repack_q6k(const uint8_t* raw, uint8_t* out, long long nblocks, hipStream_t st);
 hipError_t ilt_k_copy_bytes(const uint8_t* src, uint8_t* dst, long long bytes, hipStream_t st);

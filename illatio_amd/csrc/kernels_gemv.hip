@@ -316,7 +316,13 @@ __device__ __forceinline__ void load_q8k_pass(const float* __restrict__ x, int n
 }
 
 // FIRST: the first pass's values, loaded by the caller ahead of time (load_q8k_pass(.., 0, ..)).
-__device__ __forceinline__ void stage_q8k_from_f32(const float* __restrict__ x, int nblk, i8* lxq, float* lxs, int* lbs, const float4* first) {
+// NW: x is weighted first as rmsnorm! weights it, (x * nscale) * nw (model.lisp:215-216), NFIRST
+// being nw's first pass; H: those floats are stored as well.  PITCH: bytes from one block's
+// quants to the next's at LXQ.
+template <int PITCH>
+__device__ __forceinline__ void stage_q8k_from_f32(const float* __restrict__ x, int nblk, i8* lxq, float* lxs, int* lbs, const float4* first,
+                                                   const float* __restrict__ nw = nullptr, const float4* nfirst = nullptr,
+                                                   float nscale = 1.0f, float* __restrict__ h = nullptr) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, g = lane >> 4, l = lane & 15;
   int pass = 0;
   for (int b0 = 4 * wave; b0 < nblk; b0 += 4 * kWaves, pass++) {
@@ -325,6 +331,16 @@ __device__ __forceinline__ void stage_q8k_from_f32(const float* __restrict__ x, 
     float4 t4[4];
     if (pass == 0) { t4[0] = first[0]; t4[1] = first[1]; t4[2] = first[2]; t4[3] = first[3]; }
     else load_q8k_pass(x, nblk, pass, t4);
+    if (nw) {
+      float4 n4[4];
+      if (pass == 0) { n4[0] = nfirst[0]; n4[1] = nfirst[1]; n4[2] = nfirst[2]; n4[3] = nfirst[3]; }
+      else load_q8k_pass(nw, nblk, pass, n4);
+#pragma unroll
+      for (int i = 0; i < 4; i++) {
+        t4[i] = make_float4((t4[i].x * nscale) * n4[i].x, (t4[i].y * nscale) * n4[i].y, (t4[i].z * nscale) * n4[i].z, (t4[i].w * nscale) * n4[i].w);
+        if (h && live) *(float4*)(h + b * 256 + 4 * (l + 16 * i)) = t4[i];
+      }
+    }
     float v[16];
 #pragma unroll
     for (int i = 0; i < 4; i++) { v[4 * i] = t4[i].x; v[4 * i + 1] = t4[i].y; v[4 * i + 2] = t4[i].z; v[4 * i + 3] = t4[i].w; }
@@ -353,7 +369,7 @@ __device__ __forceinline__ void stage_q8k_from_f32(const float* __restrict__ x, 
     for (int i = 0; i < 4; i++) {
       const int s = ilt_sum4(q[4 * i] + q[4 * i + 1] + q[4 * i + 2] + q[4 * i + 3]);
       if (live) {
-        *(int*)(lxq + b * XP + 4 * (l + 16 * i)) =
+        *(int*)(lxq + b * PITCH + 4 * (l + 16 * i)) =
             (q[4 * i] & 0xFF) | ((q[4 * i + 1] & 0xFF) << 8) | ((q[4 * i + 2] & 0xFF) << 16) | ((q[4 * i + 3] & 0xFF) << 24);
         if (lbs && (l & 3) == 0) lbs[b * 16 + (l >> 2) + 4 * i] = s;     // IQ2_XXS takes no 16-sums: none staged
       }
@@ -362,12 +378,20 @@ __device__ __forceinline__ void stage_q8k_from_f32(const float* __restrict__ x, 
   }
 }
 
-// Q8_0 (quantize-q8!, tensor.lisp:245-262): 8 lanes a block of 32.
-__device__ __forceinline__ void stage_q8_from_f32(const float* __restrict__ x, int nblk, int f16_scale, i8* lxq, float* lxs) {
+// Q8_0 (quantize-q8!, tensor.lisp:245-262): 8 lanes a block of 32.  XSUM: each block's sum of
+// quants as well.  NW, NSCALE, H as for the Q8_K staging.
+__device__ __forceinline__ void stage_q8_from_f32(const float* __restrict__ x, int nblk, int f16_scale, i8* lxq, float* lxs,
+                                                  int* xsum = nullptr, const float* __restrict__ nw = nullptr, float nscale = 1.0f,
+                                                  float* __restrict__ h = nullptr) {
   const int n8 = nblk * 8;
   for (int c0 = 0; c0 < n8; c0 += kThreads) {
     const int c = c0 + threadIdx.x;
-    const float4 v = c < n8 ? *(const float4*)(x + 4 * c) : make_float4(0.f, 0.f, 0.f, 0.f);
+    float4 v = c < n8 ? *(const float4*)(x + 4 * c) : make_float4(0.f, 0.f, 0.f, 0.f);
+    if (nw) {
+      const float4 n = c < n8 ? *(const float4*)(nw + 4 * c) : make_float4(0.f, 0.f, 0.f, 0.f);
+      v = make_float4((v.x * nscale) * n.x, (v.y * nscale) * n.y, (v.z * nscale) * n.z, (v.w * nscale) * n.w);
+      if (h && c < n8) *(float4*)(h + 4 * c) = v;
+    }
     float amax = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
     amax = fmaxf(amax, ilt_dppf<ILT_DPP_XOR1>(amax));
     amax = fmaxf(amax, ilt_dppf<ILT_DPP_XOR2>(amax));
@@ -375,11 +399,57 @@ __device__ __forceinline__ void stage_q8_from_f32(const float* __restrict__ x, i
     const float d = amax / 127.0f;
     const float id = d == 0.0f ? 0.0f : 1.0f / d;
     const int q0 = (int)rintf(v.x * id), q1 = (int)rintf(v.y * id), q2 = (int)rintf(v.z * id), q3 = (int)rintf(v.w * id);
+    const int qs = xsum ? ilt_sum8(q0 + q1 + q2 + q3) : 0;
     if (c < n8) {
       *(int*)(lxq + 4 * c) = (q0 & 0xFF) | ((q1 & 0xFF) << 8) | ((q2 & 0xFF) << 16) | ((q3 & 0xFF) << 24);
-      if ((c & 7) == 0) lxs[c >> 3] = f16_scale ? __half2float(__float2half_rn(d)) : d;
+      if ((c & 7) == 0) {
+        lxs[c >> 3] = f16_scale ? __half2float(__float2half_rn(d)) : d;
+        if (xsum) xsum[c >> 3] = qs;
+      }
     }
   }
+}
+
+// ---- rmsnorm!'s scale (model.lisp:205-214) ----------------------------------------------------
+// The CPU adds the squares (each rounded to a float first) one after another in double and
+// scales by 1 / sqrt(float(sum / n + eps)).  Here the workgroup adds them in parallel: another
+// order, so the double may differ in its last bits, by less than n * 2^-52 of its value.  Where
+// every double that close rounds to the same float, the float is the CPU's; otherwise (about
+// one row in ten thousand), or when SEQ asks for it, one thread adds them again in the CPU's order.
+__device__ __forceinline__ double sq4(const float4& v) {
+  return (((double)(v.x * v.x) + (double)(v.y * v.y)) + (double)(v.z * v.z)) + (double)(v.w * v.w);
+}
+
+// The squares of this thread's share of x[0..n) (n a multiple of 4), any share of the whole.
+__device__ __forceinline__ double norm_partial(const float* __restrict__ x, int n) {
+  double s = 0.0;
+  for (int c = threadIdx.x; c < n / 4; c += kThreads) s += sq4(*(const float4*)(x + 4 * c));
+  return s;
+}
+
+// PART: this thread's part of the sum; all threads of the workgroup call this.
+__device__ __forceinline__ float norm_scale(double part, const float* __restrict__ x, int n, float eps, int seq) {
+  __shared__ double red[kWaves];
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) part += __shfl_xor(part, off);
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = part;
+  __syncthreads();
+  double sum = red[0];
+#pragma unroll
+  for (int w = 1; w < kWaves; w++) sum += red[w];
+  double v = sum / (double)n + (double)eps;
+  const double slack = v * ((double)(n + 8) * 0x1p-51);
+  if (seq || (float)(v - slack) != (float)(v + slack)) {       // the same for every thread
+    __syncthreads();
+    if (threadIdx.x == 0) {
+      double s = 0.0;
+      for (int i = 0; i < n; i++) { const float xi = x[i]; s += (double)(xi * xi); }
+      red[0] = s;
+    }
+    __syncthreads();
+    v = red[0] / (double)n + (double)eps;
+  }
+  return 1.0f / sqrtf((float)v);
 }
 
 template <int FMT>
@@ -454,8 +524,22 @@ __global__ __launch_bounds__(kThreads) void gemv_kernel(IltGemvParams p) {
   // Float activations to quantize here: their first loads go out before any weight load, since
   // loads return in order and these (hot in L2) are needed first.
   const long xoff = (long)z * p.x_stride + (long)group * p.cols;
-  float4 xfirst[4];
+  float4 xfirst[4], nfirst[4];
   if (!q8 && p.xf) load_q8k_pass(p.xf + xoff, S, 0, xfirst);
+  // ... and when they are normalized first: the norm's weights likewise, and now the squares
+  // of what xfirst does not hold
+  double sq = 0.0;
+  if (p.norm_w) {
+    if (q8) sq = norm_partial(p.xf + xoff, p.cols);
+    else {
+      load_q8k_pass(p.norm_w, S, 0, nfirst);
+      for (int pass = 1; pass * 4 * kWaves < S; pass++) {
+        float4 t[4];
+        load_q8k_pass(p.xf + xoff, S, pass, t);
+        sq += (sq4(t[0]) + sq4(t[1])) + (sq4(t[2]) + sq4(t[3]));
+      }
+    }
+  }
   // the first batch's first loads go out now, so they are on their way while x is staged
   Pre<FSET> pre;
   int warm[4] = {0, 0, 0, 0};
@@ -479,8 +563,13 @@ __global__ __launch_bounds__(kThreads) void gemv_kernel(IltGemvParams p) {
 
   // ---- stage the activations ----
   if (p.xf) {
-    if (q8) stage_q8_from_f32(p.xf + xoff, S, p.f16_scale, lxq, lxs);
-    else stage_q8k_from_f32(p.xf + xoff, S, lxq, lxs, nbs ? lbs : nullptr, xfirst);
+    float nscale = 1.0f;
+    if (p.norm_w) {
+      if (!q8) sq += (sq4(xfirst[0]) + sq4(xfirst[1])) + (sq4(xfirst[2]) + sq4(xfirst[3]));
+      nscale = norm_scale(sq, p.xf + xoff, p.cols, p.eps, p.norm_seq);
+    }
+    if (q8) stage_q8_from_f32(p.xf + xoff, S, p.f16_scale, lxq, lxs, nullptr, p.norm_w, nscale);
+    else stage_q8k_from_f32<XP>(p.xf + xoff, S, lxq, lxs, nbs ? lbs : nullptr, xfirst, p.norm_w, nfirst, nscale);
   } else {
     const i8* gxq = p.xq + xoff;
     if (q8) {
@@ -538,6 +627,28 @@ __global__ __launch_bounds__(kThreads) void gemv_kernel(IltGemvParams p) {
     __builtin_amdgcn_wave_barrier();
   }
   asm volatile("" :: "v"(warm[0]), "v"(warm[1]), "v"(warm[2]), "v"(warm[3]));
+}
+
+// rmsnorm! and the quantizer in one launch, a workgroup a row of DIM floats (the reference's
+// rmsnorm_q8, cuda/dense.cu:144-160): H (unless null) gets the floats, XQ / XS the quants and
+// scales -- Q8_0 blocks with XSUM (unless null) their sums, or with K set Q8_K blocks with
+// XSUM their sums of 16.
+template <bool K>
+__global__ __launch_bounds__(kThreads) void rmsnorm_quant_kernel(const float* __restrict__ x, const float* __restrict__ w, float* h, i8* xq,
+                                                                 float* xs, int* xsum, int dim, float eps, int f16_scale, int seq) {
+  const long row = blockIdx.x;
+  const float* xr = x + row * dim;
+  float* hr = h ? h + row * dim : nullptr;
+  const float nscale = norm_scale(norm_partial(xr, dim), xr, dim, eps, seq);
+  if constexpr (K) {
+    const int S = dim / 256;
+    float4 xfirst[4], nfirst[4];
+    load_q8k_pass(xr, S, 0, xfirst);
+    load_q8k_pass(w, S, 0, nfirst);
+    stage_q8k_from_f32<256>(xr, S, xq + row * dim, xs + row * S, xsum + row * (dim / 16), xfirst, w, nfirst, nscale, hr);
+  } else {
+    stage_q8_from_f32(xr, dim / 32, f16_scale, xq + row * dim, xs + row * (dim / 32), xsum ? xsum + row * (dim / 32) : nullptr, w, nscale, hr);
+  }
 }
 
 size_t gemv_smem(int fset, const IltGemvParams& p) {
@@ -636,5 +747,13 @@ hipError_t ilt_gemv_launch(IltGemvParams& p, int nz, hipStream_t st) {
     case ILT_IQ2_XXS: hipLaunchKernelGGL(gemv_kernel<ILT_IQ2_XXS>, grid, dim3(kThreads), smem, st, p); break;
     default: return hipErrorInvalidValue;
   }
+  return hipGetLastError();
+}
+
+hipError_t ilt_k_rmsnorm_quant(int k, const float* x, const float* w, float* h, int8_t* xq, float* xs, int* xsum, int dim,
+                               float eps, int f16_scale, int seq, int nrows, hipStream_t st) {
+  if (nrows <= 0) return hipSuccess;
+  if (k) hipLaunchKernelGGL(rmsnorm_quant_kernel<true>, dim3(nrows), dim3(kThreads), 0, st, x, w, h, xq, xs, xsum, dim, eps, f16_scale, seq);
+  else hipLaunchKernelGGL(rmsnorm_quant_kernel<false>, dim3(nrows), dim3(kThreads), 0, st, x, w, h, xq, xs, xsum, dim, eps, f16_scale, seq);
   return hipGetLastError();
 }

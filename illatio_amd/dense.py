@@ -95,6 +95,21 @@ def quantize_act(dev, x, act, n=None, f16_scale=True):
     return act
 
 
+def rmsnorm_q8(dev, x, w, act, d, eps, n=1, h=None, exact_order=False):
+    """RMSNORM! of N rows of X (D wide) by W, quantized into ACT in each format it holds, the
+    floats into H unless None (RMSNORM-Q8, cuda-dense.lisp:260-264; Q8_K blocks when ACT holds
+    them, as the CPU path makes for K-quant matrices)."""
+    if act.xq is not None:
+        hip.call("ilt_rmsnorm_q8", C.c_uint64(dev.stream), C.c_uint64(x.ptr), C.c_uint64(w.ptr), C.c_uint64(h.ptr if h else 0),
+                 C.c_uint64(act.xq.ptr), C.c_uint64(act.xs.ptr), C.c_uint64(0), C.c_int(d), C.c_float(eps), C.c_int(n),
+                 C.c_int(1 if exact_order else 0))
+    if act.kq is not None:
+        hip.call("ilt_rmsnorm_q8k", C.c_uint64(dev.stream), C.c_uint64(x.ptr), C.c_uint64(w.ptr), C.c_uint64(h.ptr if h else 0),
+                 C.c_uint64(act.kq.ptr), C.c_uint64(act.kd.ptr), C.c_uint64(act.ksum.ptr), C.c_int(d), C.c_float(eps), C.c_int(n),
+                 C.c_int(1 if exact_order else 0))
+    return act
+
+
 def cmat_mul(dev, w, act, y, n=1, bias=None, acc=False):
     """Y = W X for N tokens (token t's X at t*cols, its Y at t*rows), or Y += it when ACC
     (CMAT-MUL): the matrix-vector kernel for one token, the tiled product for more."""
@@ -138,13 +153,22 @@ class MvDesc(C.Structure):
                 ("y", C.c_uint64), ("bias", C.c_uint64)]
 
 
-def mv_multi(dev, parts, act=None, xf=None, f16_scale=True, acc=False, glu=False):
+def mv_multi(dev, parts, act=None, xf=None, f16_scale=True, acc=False, glu=False, norm=None, exact_order=False):
     """PARTS, up to four (W Y BIAS) sharing X, in one launch (CMAT-MUL-N's idea, for one
-    token): X quantized in ACT, or the floats XF, which the kernel then quantizes itself."""
+    token): X quantized in ACT, or the floats XF, which the kernel then quantizes itself --
+    after RMSNORM! by NORM = (weights DBuf, eps) when given: norm, quantizer and products in
+    one launch."""
     descs = (MvDesc * len(parts))()
     for i, (w, y, bias) in enumerate(parts):
         descs[i] = MvDesc(w.type, w.rows, w.qs.ptr, w.d.ptr if w.d else 0, y.ptr, bias.ptr if bias else 0)
     w0 = parts[0][0]
+    if norm is not None:
+        if xf is None or acc:
+            raise ValueError("a norm takes float activations and no accumulation")
+        hip.call("ilt_mv_multi_norm", C.c_uint64(dev.stream), C.c_int(len(parts)), descs, C.c_int(w0.cols), C.c_uint64(xf.ptr),
+                 C.c_uint64(norm[0].ptr), C.c_float(norm[1]), C.c_int(1 if exact_order else 0), C.c_int(1 if f16_scale else 0),
+                 C.c_int(1 if glu else 0))
+        return
     if xf is not None:
         xq = xs = bs = 0
     elif w0.kquant_p():
@@ -156,15 +180,15 @@ def mv_multi(dev, parts, act=None, xf=None, f16_scale=True, acc=False, glu=False
              C.c_int(1 if acc else 0), C.c_int(1 if glu else 0))
 
 
-def qkv_mul(dev, wq, wk, wv, act, q, k, v, bq=None, bk=None, bv=None, xf=None):
+def qkv_mul(dev, wq, wk, wv, act, q, k, v, bq=None, bk=None, bv=None, xf=None, norm=None):
     """Q, K and V's products of one token in one launch (QKV-MUL, cuda-dense.lisp:309-324)."""
-    mv_multi(dev, [(wq, q, bq), (wk, k, bk), (wv, v, bv)], act, xf)
+    mv_multi(dev, [(wq, q, bq), (wk, k, bk), (wv, v, bv)], act, xf, norm=norm)
 
 
-def glu_mul(dev, g, u, act, fa, xf=None):
+def glu_mul(dev, g, u, act, fa, xf=None, norm=None):
     """silu(G x) * (U x) into FA for one token (GLU-MUL, cuda-dense.lisp:326-339)."""
     if xf is not None:
-        return mv_multi(dev, [(g, fa, None), (u, fa, None)], None, xf, glu=True)
+        return mv_multi(dev, [(g, fa, None), (u, fa, None)], None, xf, glu=True, norm=norm)
     f, d = g.rows, g.cols
     if g.kquant_p():
         hip.launch(dev, "mv_k_glu", (f + 3) // 4, 128,

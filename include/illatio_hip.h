@@ -150,6 +150,26 @@ typedef struct ilt_mv_desc {
 int ilt_mv_multi(uint64_t stream, int nmat, const ilt_mv_desc* descs, int cols, const int8_t* xq, const float* xs,
                  const int32_t* bsums, const float* xf, int f16_scale, int acc, int glu);
 
+/* rmsnorm! (model.lisp:205-216) and the quantizer in one launch, a row of dim floats a
+   workgroup, n rows: out = (x * scale) * w with scale = 1 / sqrt(float(sum/dim + eps)), the
+   squares rounded to floats and added in double.  h (unless null) gets the floats.
+   rmsnorm_q8 (dense.cu:144-160; cuda-dense.lisp:260-264): Q8_0 blocks as quant_q8 makes them,
+     xsum|0 their sums; launched by name, rows = grid y.
+   rmsnorm_q8k: Q8_K blocks as quant_q8k makes them (no CUDA counterpart: the reference's
+     K-quant kernels take the floats).
+   ilt_mv_multi_norm: ilt_mv_multi on the floats x, normalized like this by each workgroup
+     before it quantizes them: norm, quantizer and products in one launch (the reference:
+     rmsnorm_q8 then mv_*, cuda-dense.lisp:401-403, 415-417).
+   The bits are the CPU's although the squares are added in parallel: the kernel checks that
+   no double within the reordering's error bound of its sum rounds to another float, and
+   otherwise (or always, with exact_order 1) adds them again one after another. */
+int ilt_rmsnorm_q8(uint64_t stream, const float* x, const float* w, float* h, int8_t* xq, float* xs, int32_t* xsum, int dim,
+                   float eps, int n, int exact_order);
+int ilt_rmsnorm_q8k(uint64_t stream, const float* x, const float* w, float* h, int8_t* xq, float* xd, int32_t* bsums, int dim,
+                    float eps, int n, int exact_order);
+int ilt_mv_multi_norm(uint64_t stream, int nmat, const ilt_mv_desc* descs, int cols, const float* x, const float* norm_w,
+                      float eps, int exact_order, int f16_scale, int glu);
+
 /* The indexed expert products (ds4f.cu:769, 837; CPU: iq2xxs-row-dot, q2k-row-dot,
    iquant.lisp:126-215).  For each z < nz: W = the nrows x ncols matrix at ptrs[z] + add
    (row_bytes apart), x = the Q8_K activations at element z*x_stride, y = dst + z*y_stride.

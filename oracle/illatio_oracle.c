@@ -473,6 +473,17 @@ void orc_matmul_q(int type, const uint8_t* w, int64_t rows, int64_t cols, const 
 /* ---- src/ds4f.lisp:248-254 ------------------------------------------------------------------------ */
 static inline float sb_exp(float x) { return (float)exp((double)x); }
 static inline float sb_log(float x) { return (float)log((double)x); }
+/* rmsnorm! (model.lisp:205-216): the squares are single-float products, added one after
+   another in double; scale = 1 / sqrt(float(sum/n + eps)); out = (x * scale) * w.
+   Parity unpinned: the reference holds no vector for it; tests pin it against what the
+   formula fixes (closed forms, the float-rounded squares, the order of the two products). */
+void orc_rmsnorm(const float* x, const float* w, float* out, float eps, int64_t n) {
+  double sum = 0.0;
+  for (int64_t i = 0; i < n; i++) { volatile float sq = x[i] * x[i]; sum += (double)sq; }
+  const float scale = 1.0f / sqrtf((float)(sum / (double)n + (double)eps));
+  for (int64_t i = 0; i < n; i++) { volatile float t = x[i] * scale; out[i] = t * w[i]; }
+}
+
 float orc_sigmoid(float x) {
   if (x >= 0.0f) return 1.0f / (1.0f + sb_exp(-x));
   float e = sb_exp(x); return e / (1.0f + e);

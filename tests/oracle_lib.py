@@ -167,6 +167,13 @@ def swiglu(g, u):
     return np.array([f(float(a), float(b)) for a, b in zip(g, u)], np.float32)
 
 
+def rmsnorm(x, w, eps):
+    x, w = _c(x, np.float32), _c(w, np.float32)
+    out = np.empty_like(x)
+    lib().orc_rmsnorm(_p(x), _p(w), _p(out), C.c_float(eps), C.c_int64(x.size))
+    return out
+
+
 def softplus(x):
     return lib().orc_softplus(float(np.float32(x)))
 

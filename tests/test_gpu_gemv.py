@@ -271,3 +271,108 @@ def test_in_kernel_quantization_single_matrix(dev):
             want = orc.matmul(qtype, w, rows, cols, x, f16_scale=f16)
             assert np.array_equal(bits(hip.hip_floats(y, rows)), bits(want)), (qtype, rows, cols, f16)
         hip.hip_free(xb); hip.hip_free(y); m.free()
+
+
+# ---- rmsnorm! fused with the quantizers and with the products ---------------------------------
+
+def tie_row(n):
+    """A row whose mean square lies exactly between two floats (half the values a, half b with
+    fl(a*a) and fl(b*b) an odd number of float steps apart): the parallel sum's check cannot
+    clear it, so the kernel adds the squares again in the CPU's order."""
+    f32 = np.float32
+    a = f32(1.0)
+    A = f32(a * a)
+    b = a
+    while True:
+        b = np.nextafter(b, f32(2))
+        B = f32(b * b)
+        steps = int(B.view(np.uint32)) - int(A.view(np.uint32))
+        if steps % 2 == 1:
+            break
+    x = np.empty(n, f32)
+    x[0::2], x[1::2] = a, b
+    mid = (np.float64(A) + np.float64(B)) / 2
+    assert f32(mid) != f32(np.nextafter(mid, 0)) or f32(mid) != f32(np.nextafter(mid, 4))    # a rounding tie
+    return x
+
+
+def norm_rows(dim, n, rng):
+    x = np.stack([synth.activations(dim, rng) * s for s in np.resize([1.0, 1e-3, 40.0], n)]).astype(np.float32)
+    x[0, : dim // 2] *= np.float32(1e-5)          # a wide spread inside a row
+    if n > 2:
+        x[2] = tie_row(dim)
+    if n > 3:
+        x[3] = 0.0
+    return x
+
+
+@pytest.mark.parametrize("dim", [256, 1024, 2560, 5120, 8192])
+def test_rmsnorm_quantized_bit_exact(dev, dim):
+    """rmsnorm_q8 / rmsnorm_q8k: floats, quants, scales and sums are rmsnorm! then quantize-q8! /
+    quantize-q8k!'s, whether the squares are added in parallel (checked) or one after another."""
+    from illatio_amd import dense, hip
+    rng = synth.make_rng(dim + 5)
+    n, eps = 5, 1e-6
+    x = norm_rows(dim, n, rng)
+    w = (synth.activations(dim, rng) * 0.2 + 1.0).astype(np.float32)
+    xb, wb, hb = hip.hip_upload_new(dev, x), hip.hip_upload_new(dev, w), hip.hip_alloc(dev, 4 * n * dim)
+    act = dense.QAct(dev, n, dim)
+    want_h = np.stack([orc.rmsnorm(x[t], w, eps) for t in range(n)])
+    q8, s8 = orc.quantize_q8(want_h)
+    qk, dk, bk = orc.quantize_q8k(want_h)
+    for exact_order in (False, True):
+        for b in (hb, act.xq, act.xs, act.kq, act.kd, act.ksum):
+            hip.hip_zero(b)
+        dense.rmsnorm_q8(dev, xb, wb, act, dim, eps, n=n, h=hb, exact_order=exact_order)
+        assert np.array_equal(bits(hip.hip_floats(hb, n * dim)), bits(want_h.ravel())), (dim, exact_order)
+        assert np.array_equal(hip.hip_download(act.xq, np.int8, n * dim), q8)
+        assert np.array_equal(bits(hip.hip_floats(act.xs, n * dim // 32)), bits(s8))
+        assert np.array_equal(hip.hip_download(act.kq, np.int8, n * dim), qk)
+        assert np.array_equal(bits(hip.hip_floats(act.kd, n * dim // 256)), bits(dk))
+        assert np.array_equal(hip.hip_download(act.ksum, np.int32, n * dim // 16), bk)
+    # launched by name as the reference launches it, with the block sums
+    xsum = hip.hip_alloc(dev, 4 * n * dim // 32)
+    hip.launch(dev, "rmsnorm_q8", (1, n), 256, [xb, wb, None, act.xq, act.xs, xsum, dim, float(eps)])
+    assert np.array_equal(hip.hip_download(act.xq, np.int8, n * dim), q8)
+    assert np.array_equal(hip.hip_download(xsum, np.int32, n * dim // 32), q8.reshape(-1, 32).astype(np.int32).sum(1))
+    for b in (xb, wb, hb, xsum):
+        hip.hip_free(b)
+    act.free()
+
+
+@pytest.mark.parametrize("kind", ["q8", "k"])
+def test_norm_inside_the_product_bit_exact(dev, kind):
+    """mv_multi with a norm: rmsnorm!, the quantizer and the products of Q/K/V (and gate/up with
+    the gated activation) in one launch, with the bits of the three steps run one by one."""
+    from illatio_amd import dense, hip
+    rng = synth.make_rng(77 if kind == "k" else 78)
+    eps = 1e-6
+    for cols in ((2560, 5120) if kind == "k" else (1024, 2560)):
+        shape = [(synth.Q4_K, 512), (synth.Q6_K, 128), (synth.Q4_K, 136)] if kind == "k" else [(synth.Q8_0, 512), (synth.Q8_0, 128), (synth.Q8_0, 136)]
+        ws = [synth.weights(t, r, cols, rng) for t, r in shape]
+        ms = [upload(dev, t, r, cols, w) for (t, r), w in zip(shape, ws)]
+        nw = (synth.activations(cols, rng) * 0.3 + 1.0).astype(np.float32)
+        nwb = hip.hip_upload_new(dev, nw)
+        for x in (synth.activations(cols, rng), tie_row(cols), norm_rows(cols, 1, rng)[0]):
+            h = orc.rmsnorm(x, nw, eps)
+            xb = hip.hip_upload_new(dev, x)
+            ys = [hip.hip_alloc(dev, 4 * r) for _, r in shape]
+            for exact_order in (False, True):
+                dense.mv_multi(dev, [(m, y, None) for m, y in zip(ms, ys)], xf=xb, norm=(nwb, eps), exact_order=exact_order)
+                for (t, r), w, y in zip(shape, ws, ys):
+                    assert np.array_equal(bits(hip.hip_floats(y, r)), bits(orc.matmul(t, w, r, cols, h))), (kind, cols, t, exact_order)
+            # gate and up (equal rows) ending in the gated activation
+            fa = hip.hip_alloc(dev, 4 * shape[0][1])
+            g2 = [ms[0], ms[0]] if kind == "q8" else [ms[0], upload(dev, synth.Q6_K, 512, cols, synth.weights(synth.Q6_K, 512, cols, synth.make_rng(5)))]
+            u_w = ws[0] if kind == "q8" else synth.weights(synth.Q6_K, 512, cols, synth.make_rng(5))
+            dense.mv_multi(dev, [(g2[0], fa, None), (g2[1], fa, None)], xf=xb, norm=(nwb, eps), glu=True)
+            g = orc.matmul(shape[0][0], ws[0], 512, cols, h)
+            u = orc.matmul(synth.Q8_0 if kind == "q8" else synth.Q6_K, u_w, 512, cols, h)
+            assert np.array_equal(bits(hip.hip_floats(fa, 512)), bits(orc.swiglu(g, u))), (kind, cols)
+            if kind == "k":
+                g2[1].free()
+            for b in [xb, fa] + ys:
+                hip.hip_free(b)
+        hip.hip_free(nwb)
+        for m in ms:
+            m.free()

@@ -381,3 +381,58 @@ def test_moe_chunk_equals_token_at_a_time():
         one, s1, w1 = orc.moe_token(gate, up, down, sg, su, sd, d, ff, ne, nu, 1.5, 0.0, logits[t], norms[t])
         assert s1.tolist() == sel[t].tolist() and np.array_equal(w1, w[t])
         assert np.array_equal(one.view(np.uint32), out[t].view(np.uint32))
+
+
+# ---- rmsnorm! (model.lisp:205-216) -----------------------------------------------------------
+# The reference holds no vector for it: these pin what its text fixes, on inputs chosen so that
+# each plausible misreading (exact squares, a float sum, the weight folded into the scale,
+# eps inside the mean) gives other bits.
+
+def _rms_variants(x, w, eps):
+    """The reading under test and the misreadings, in numpy with every rounding explicit."""
+    f32, f64 = np.float32, np.float64
+    sq = (x * x).astype(f32)                              # single-float products
+    seq = f64(0)
+    for s in sq:
+        seq = seq + f64(s)
+    n = f64(x.size)
+
+    def out(total, order="xs"):
+        scale = f32(1) / np.sqrt(f32(total / n + f64(f32(eps))))     # eps is a single float
+        return ((x * scale) * w) if order == "xs" else (x * (scale * w))
+    exact_sq = f64(0)
+    for v in x:
+        exact_sq = exact_sq + f64(v) * f64(v)
+    fsum = f32(0)
+    for s in sq:
+        fsum = f32(fsum + s)
+    return {"right": out(seq), "exact squares": out(exact_sq), "float sum": out(f64(fsum)),
+            "weight folded": out(seq, "sw")}
+
+
+def test_rmsnorm_closed_form_and_misreadings():
+    f32 = np.float32
+    # all equal powers of two: sum/n is the square itself
+    x = np.full(256, 0.5, f32)
+    w = np.full(256, 3.0, f32)
+    want = (x * (f32(1) / np.sqrt(f32(np.float64(0.25) + np.float64(f32(1e-6)))))) * w
+    assert np.array_equal(orc.rmsnorm(x, w, 1e-6).view(np.uint32), want.view(np.uint32))
+    # zeros: the scale is 1/sqrt(eps), the result zeros
+    assert np.array_equal(orc.rmsnorm(np.zeros(64, f32), w[:64], 1e-5), np.zeros(64, f32))
+    # seeded rows until every misreading has been told apart at least once
+    rng = np.random.default_rng(5)
+    told = set()
+    for trial in range(400):
+        n = int(rng.choice([32, 64, 256, 1024]))
+        x = (rng.standard_normal(n) * rng.choice([1e-3, 1.0, 30.0])).astype(f32)
+        if trial % 3 == 0:
+            x[: n // 2] *= f32(1e-4)                       # a wide spread of magnitudes
+        w = rng.standard_normal(n).astype(f32)
+        eps = float(rng.choice([1e-6, 1e-5]))
+        v = _rms_variants(x, w, eps)
+        got = orc.rmsnorm(x, w, eps)
+        assert np.array_equal(got.view(np.uint32), v["right"].astype(f32).view(np.uint32)), trial
+        for k in ("exact squares", "float sum", "weight folded"):
+            if not np.array_equal(v[k].astype(f32).view(np.uint32), got.view(np.uint32)):
+                told.add(k)
+    assert told == {"exact squares", "float sum", "weight folded"}, told
