@@ -65,7 +65,7 @@ def traffic_of(workload, per):
 
 
 HBM_PEAK_GBS = 8000.0
-MFMA_PEAK_TFLOPS = {"bf16": 2500.0, "int8": 5000.0}
+MFMA_PEAK_TFLOPS = {"bf16": 2500.0, "bf16-2pass": 2500.0, "bf16-resident": 2500.0, "int8": 5000.0}
 
 D, FFN, QD, KVD, VOCAB, LAYERS = 2560, 9728, 4096, 1024, 151936, 36
 
@@ -314,7 +314,20 @@ def workload_c3(args, dev):
     y = hip.hip_alloc(dev, 4 * T * rows, zero=False)
     flops = 2.0 * rows * cols * T
     tm = Timer(dev)
-    if args.path == "bf16":
+    bf16_path = args.path.startswith("bf16")
+    if args.path in ("bf16-2pass", "bf16-resident"):
+        # the matrix dequantized to a bf16 copy (inside every step, or once beforehand and kept), then the plain bf16 product
+        xb = hip.hip_alloc(dev, dense.slabs_bytes(T, cols), zero=False)
+        wb = dense.dequant_bf16(dev, m)
+        resident = args.path == "bf16-resident"
+
+        def step(_):
+            tm.launch("cvt", 0, lambda: dense.cvt_bf16_slabs(dev, xf, T, cols, xb))
+            if not resident:
+                tm.launch("dequant", 0, lambda: dense.dequant_bf16(dev, m, wb))
+            tm.launch("mm", flops, lambda: dense.mat_mul_bf16(dev, wb, rows, cols, xb, y, T))
+        names = {"mm": "gemm_bf16_plain_kernel (both operands bf16 through LDS, v_mfma_f32_32x32x16_bf16)"}
+    elif args.path == "bf16":
         xb = hip.hip_alloc(dev, 2 * T * cols, zero=False)
 
         def step(_):
@@ -329,7 +342,7 @@ def workload_c3(args, dev):
             tm.launch("mm", flops, lambda: dense.cmat_mul(dev, m, act, y, n=T))
         names = {"mm": "gemm_i8_kernel (Q6_K unpacked to int8 in LDS, v_mfma_i32_16x16x64_i8, bit-exact with the CPU path)"}
     ms, dev_ms, per = tm.run(step, args.steps, args.warmup)
-    roof = roofline_of({k: v for k, v in per.items() if k == "mm"}, "mfma", MFMA_PEAK_TFLOPS[args.path], "TFLOP/s" if args.path == "bf16" else "TOP/s", names)
+    roof = roofline_of({k: v for k, v in per.items() if k == "mm"}, "mfma", MFMA_PEAK_TFLOPS[args.path], "TFLOP/s" if bf16_path else "TOP/s", names)
     roof["unit"] = "TFLOP/s"
     if args.path == "bf16" and T == 4096 and not args.transpose:
         roof["traffic"] = traffic_of("c3", per)
@@ -349,7 +362,7 @@ def workload_c3(args, dev):
                 "sample": f"{reps} x the same matrix on {ts} tokens (quantization included), {t_cpu:.1f} s"}
 
     return {"value": round(tf, 1), "unit": "TFLOP/s", "ms_per_step": ms, "device_ms_per_step": dev_ms, "enqueue_ms": tm.enqueue_ms,
-            "dtype": "bf16 x bf16, fp32 accumulate" if args.path == "bf16" else "int8 block dots, fp32 combine",
+            "dtype": "bf16 x bf16, fp32 accumulate" if bf16_path else "int8 block dots, fp32 combine",
             "metric": "prefill product TFLOP/s (% of dense MFMA peak)",
             "config": {"workload": f"c3: Q6_K prefill product {rows}x{cols} on {T} tokens, {args.path} path "
                                    f"(activation conversion inside the step)", "flops_per_step": flops, "tokens": T},
@@ -519,7 +532,9 @@ def main():
     ap.add_argument("--layers", type=int, default=LAYERS, help=argparse.SUPPRESS)
     ap.add_argument("--tokens", type=int, default=4096, help="c3, c5: tokens per step")
     ap.add_argument("--transpose", action="store_true", help="c3: the 5120x17408 matrix")
-    ap.add_argument("--path", default="bf16", choices=["bf16", "int8"], help="c3, c5: which matrix-core path")
+    ap.add_argument("--path", default="bf16", choices=["bf16", "bf16-2pass", "bf16-resident", "int8"],
+                    help="c3, c5: which matrix-core path; c3 only: bf16-2pass = the matrix dequantized to a bf16 copy inside the step, then the plain "
+                         "bf16 product; bf16-resident = the copy made beforehand and kept")
     ap.add_argument("--norm", action="store_true", help="c2: include each layer's two norms and the output norm (inside the product launches in fused mode)")
     ap.add_argument("--mode", default="fused", choices=["fused", "fused-q", "single", "device"],
                     help="c4: fused = 5 launches a step, single = the reference's sequence of 12 (both with the routing done beforehand on the host, as the "

@@ -480,8 +480,31 @@ int ilt_mm_k_bf16(uint64_t stream, int gguf_type, const void* w, const uint16_t*
   if (rows == 0 || n == 0) return ILT_OK;
   const long long row_bytes = (long long)cols / 256 * block_bytes(fmt);
   ILT_REQUIRE(w && xb && y && ((uintptr_t)w & 1) == 0 && ((uintptr_t)xb & 15) == 0);
-  ILT_REQUIRE(row_bytes * rows < 0xFFFFFFF0LL);
+  ILT_REQUIRE(row_bytes * rows < 0xFFFFFFF0LL && rows < (1 << 21));
   return (int)ilt_k_gemm_bf16(fmt, (const uint8_t*)w, row_bytes, rows, cols, xb, n, y, bias, acc, S(stream));
+}
+
+int ilt_cvt_bf16_slabs(uint64_t stream, const float* x, uint16_t* xs, int n, int cols) {
+  ILT_REQUIRE(n >= 0 && cols > 0 && cols % 128 == 0);
+  if (n == 0) return ILT_OK;
+  ILT_REQUIRE(x && xs && ((uintptr_t)x & 15) == 0 && ((uintptr_t)xs & 15) == 0);
+  return (int)ilt_k_cvt_bf16_slabs(x, xs, n, cols, S(stream));
+}
+
+int ilt_dequant_bf16(uint64_t stream, int gguf_type, const void* w, uint16_t* wb, int rows, int cols) {
+  const int fmt = bf16_type(gguf_type);
+  ILT_REQUIRE(fmt && rows >= 0 && cols > 0 && cols % 256 == 0);
+  if (rows == 0) return ILT_OK;
+  ILT_REQUIRE(w && wb && ((uintptr_t)w & 1) == 0 && ((uintptr_t)wb & 15) == 0);
+  return (int)ilt_k_dequant_bf16(fmt, (const uint8_t*)w, (long long)cols / 256 * block_bytes(fmt), rows, cols, wb, S(stream));
+}
+
+int ilt_mm_bf16(uint64_t stream, const uint16_t* wb, const uint16_t* xb, float* y, const float* bias, int rows, int cols, int n,
+                int acc) {
+  ILT_REQUIRE(rows >= 0 && n >= 0 && cols > 0 && cols % 128 == 0 && cols < (1 << 22) && rows < (1 << 21));
+  if (rows == 0 || n == 0) return ILT_OK;
+  ILT_REQUIRE(wb && xb && y && ((uintptr_t)wb & 15) == 0 && ((uintptr_t)xb & 15) == 0);
+  return (int)ilt_k_gemm_bf16_plain(wb, rows, cols, xb, n, y, bias, acc, S(stream));
 }
 
 int ilt_d4_mm_id_bf16(uint64_t stream, int gguf_type, int ncols, int nrows, int row_bytes, int64_t add, const uint64_t* ptrs,
@@ -492,7 +515,7 @@ int ilt_d4_mm_id_bf16(uint64_t stream, int gguf_type, int ncols, int nrows, int 
   ILT_REQUIRE(row_bytes == ncols / 256 * block_bytes(fmt) && add >= 0 && (add & 1) == 0);
   if (nrows == 0 || ne == 0 || total_rows == 0) return ILT_OK;
   ILT_REQUIRE(ptrs && counts && bases && xb && y && ((uintptr_t)xb & 15) == 0 && total_rows < (1LL << 31));
-  ILT_REQUIRE((long long)row_bytes * nrows < 0xFFFFFFF0LL);
+  ILT_REQUIRE((long long)row_bytes * nrows < 0xFFFFFFF0LL && nrows < (1 << 21));
   return (int)ilt_k_gemm_bf16_id(fmt, ptrs, add, counts, bases, ne, row_bytes, nrows, ncols, xb, rmap, total_rows, y, S(stream));
 }
 
@@ -530,6 +553,9 @@ int ilt_launch(const char* kernel, unsigned gx, unsigned gy, unsigned gz, unsign
   K("cvt_bf16") return ilt_cvt_bf16(stream, a.ptr<cf>(0), a.ptr<uint16_t*>(1), a.i64(2));
   K("mm_k_bf16") return ilt_mm_k_bf16(stream, a.i32(0), a.ptr<const void*>(1), a.ptr<cu16>(2), a.ptr<float*>(3), a.ptr<cf>(4),
                                       a.i32(5), a.i32(6), a.i32(7), a.i32(8));
+  K("cvt_bf16_slabs") return ilt_cvt_bf16_slabs(stream, a.ptr<cf>(0), a.ptr<uint16_t*>(1), a.i32(2), a.i32(3));
+  K("dequant_bf16") return ilt_dequant_bf16(stream, a.i32(0), a.ptr<const void*>(1), a.ptr<uint16_t*>(2), a.i32(3), a.i32(4));
+  K("mm_bf16") return ilt_mm_bf16(stream, a.ptr<cu16>(0), a.ptr<cu16>(1), a.ptr<float*>(2), a.ptr<cf>(3), a.i32(4), a.i32(5), a.i32(6), a.i32(7));
   K("d4_mm_id_bf16")
     return ilt_d4_mm_id_bf16(stream, a.i32(0), a.i32(1), a.i32(2), a.i32(3), a.i64(4), a.ptr<const uint64_t*>(5), a.ptr<cu32>(6),
                              a.ptr<cu32>(7), a.i32(8), a.i64(9), a.ptr<cu16>(10), a.ptr<cu32>(11), a.ptr<float*>(12));

@@ -185,6 +185,58 @@ template <int TM, int TN, int NXS, int NWS> struct Smem {
 __device__ __forceinline__ u32 slab_swz(int r) { return (((r >> 1) ^ (r >> 3)) & 1) | (((r >> 2) & 1) << 1); }
 __device__ __forceinline__ u32 slab_off(int r, int p) { return (u32)(4 * r + (p ^ slab_swz(r))) * 16; }
 
+// ---- a wave's results to y ----
+// Patch (a, b), register r of a lane: token wt0 + 32a + 8*(r/4) + 4*lh + r%4, row wr0 + 32b + l32
+// of the tile, so a store instruction writes 32 consecutive rows of two tokens.  With one
+// workgroup on a CU nothing else runs while it stores, so the loop is kept to an address add
+// and a store per value and has no branches: the stores go through a buffer descriptor that
+// ends with the tile's last token, which drops what lies past it, and a lane whose row the
+// matrix does not have starts 2 GiB out.  (rows * 1024 < 2^31, checked by the host.)
+template <int NA, int NB, bool BIAS, bool ACC>
+__device__ __forceinline__ void store_patches(const v16f (&acc)[NA][NB], const BfParams& p, __amdgpu_buffer_rsrc_t ry, int r0,
+                                              int wt0, int wr0, int l32, int lh) {
+  const u32 rows4 = (u32)p.rows * 4;
+#pragma unroll
+  for (int b = 0; b < NB; b++) {
+    const int row = r0 + wr0 + 32 * b + l32;
+    const bool ok = row < p.rows;
+    const u32 base = ok ? (u32)((wt0 + 4 * lh) * p.rows + row) * 4 : 0x80000000u;
+    float bv = 0.0f;
+    if (BIAS) bv = ok ? p.bias[row] : 0.0f;
+#pragma unroll
+    for (int a = 0; a < NA; a++) {
+      float old[16];
+      if (ACC) {
+#pragma unroll
+        for (int r = 0; r < 16; r++)
+          old[r] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(ry, base + (u32)(32 * a + 8 * (r >> 2) + (r & 3)) * rows4, 0, 0));
+      }
+#pragma unroll
+      for (int r = 0; r < 16; r++) {
+        float v = acc[a][b][r];
+        if (BIAS) v = v + bv;
+        if (ACC) v = old[r] + v;
+        __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(u32, v), ry, base + (u32)(32 * a + 8 * (r >> 2) + (r & 3)) * rows4, 0, 0);
+      }
+    }
+  }
+}
+
+template <int NA, int NB>
+__device__ __forceinline__ void store_tile(const v16f (&acc)[NA][NB], const BfParams& p, long tok0, int ntok, int r0,
+                                           int wt0, int wr0, int l32, int lh) {
+  // (ntok may come out of LDS: the same in every lane, said so to the compiler)
+  const u32 ybytes = (u32)__builtin_amdgcn_readfirstlane(ntok) * (u32)p.rows * 4;
+  const __amdgpu_buffer_rsrc_t ry = ilt_rsrc(ilt_uniform_ptr(p.y + tok0 * (long)p.rows), ybytes);
+  if (p.bias) {
+    if (p.acc) store_patches<NA, NB, true, true>(acc, p, ry, r0, wt0, wr0, l32, lh);
+    else store_patches<NA, NB, true, false>(acc, p, ry, r0, wt0, wr0, l32, lh);
+  } else {
+    if (p.acc) store_patches<NA, NB, false, true>(acc, p, ry, r0, wt0, wr0, l32, lh);
+    else store_patches<NA, NB, false, false>(acc, p, ry, r0, wt0, wr0, l32, lh);
+  }
+}
+
 // TM rows x TN tokens per workgroup; wave w: rows 32*NB*(w/2).., tokens (TN/2)*(w%2)..: NA x NB
 // patches of 32x32.  NB = 2: 2*TM threads, two per row; NB = 4: TM threads, one per row, a
 // wave alone on its SIMD with 128x128 results in 256 accumulator registers.
@@ -432,26 +484,165 @@ __global__ __launch_bounds__((bf16_threads<TM, NB>()), (TM == 256 ? 1 : TN == 25
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // the tail's redundant loads: nothing may land in LDS after the workgroup ends
 
-  // ---- store: patch (a, b): token = wt0 + 32a + 8*(r/4) + 4*lh + r%4, row = wr0 + 32b + l32 ----
+  store_tile<NA, NB>(acc, p, tok0, ntok, r0, wt0, wr0, l32, lh);
+}
+
+// ---- the two-pass product: W as plain bf16 ------------------------------------------------------
+// With thousands of tokens the in-loop dequantization above is repeated for every tile of 256
+// tokens and its VALU work competes with the MFMAs for issue slots.  With HBM to spare the
+// matrix can instead be dequantized once into a bf16 copy (kept for later products, or made
+// per product) and multiplied by a kernel whose loop holds nothing but direct loads to LDS,
+// fragment reads and MFMAs.
+
+//
+// Both operands of that kernel are stored in slabs: the 32 columns of a step for 128
+// consecutive rows (or tokens) are 8 KB in one piece, row r of the group at 64*r, the groups'
+// slabs for step 0, 1, ... one after another.  A step's direct loads then read whole 128-byte
+// lines of a few DRAM pages instead of 64 bytes from each of 256 rows' pages.  The row count is
+// padded to a multiple of 256 (the padding rows hold zeros).
+constexpr int SLAB_ROWS = 128, SLAB_BYTES = SLAB_ROWS * KS * 2;
+__device__ __forceinline__ long long slab_addr(long long row, int ks, int nk) {     // of the row's 64 bytes of step ks
+  return ((row / SLAB_ROWS) * nk + ks) * SLAB_BYTES + (row % SLAB_ROWS) * (KS * 2);
+}
+
+// A workgroup: half super-block hb of a group of 128 rows; thread (row, e) dequantizes the 4 x 16
+// weights that kernel thread (row, e) dequantizes there, and writes 32 bytes into each of four slabs.
+template <int FMT>
+__global__ __launch_bounds__(256) void dequant_bf16_kernel(const u8* __restrict__ w, long long row_bytes, int rows, int cols, u8* __restrict__ out) {
+  __shared__ u64 grid[256];
+  if (FMT == ILT_IQ2_XXS) { grid[threadIdx.x] = bf_grid_dev[threadIdx.x]; __syncthreads(); }
+  const int nh = cols / 128, nk = cols / KS;
+  const int e = threadIdx.x & 1, rl = threadIdx.x >> 1;
+  const int hb = blockIdx.x % nh;
+  const long long row = (long long)(blockIdx.x / nh) * SLAB_ROWS + rl;
+  const bool live = row < rows;
+  WRaw<FMT> raw;
+  if (live) load_w<FMT>(raw, ilt_rsrc(w + row * row_bytes, (u32)row_bytes), 0u, hb, e);
 #pragma unroll
-  for (int b = 0; b < NB; b++) {
-    const int row = r0 + wr0 + 32 * b + l32;
-    if (row >= p.rows) continue;
-    const float bv = p.bias ? p.bias[row] : 0.0f;
+  for (int j = 0; j < 4; j++) {
+    u32 pk[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    if (live) {
+      float o[16];
+      dequant16<FMT>(raw, j, hb & 1, e, grid, o);
 #pragma unroll
-    for (int a = 0; a < NA; a++) {
-#pragma unroll
-      for (int r = 0; r < 16; r++) {
-        const int tk = wt0 + 32 * a + 8 * (r >> 2) + 4 * lh + (r & 3);
-        if (tk >= ntok) continue;
-        float* yo = p.y + (tok0 + tk) * (long)p.rows + row;
-        float v = acc[a][b][r];
-        if (p.bias) v = v + bv;
-        if (p.acc) v = *yo + v;
-        *yo = v;
-      }
+      for (int k = 0; k < 8; k++) pk[k] = pack_bf16(o[2 * k], o[2 * k + 1]);
     }
+    u8* dst = out + slab_addr(row, 4 * hb + j, nk) + 32 * e;
+    *(int4*)dst = make_int4((int)pk[0], (int)pk[1], (int)pk[2], (int)pk[3]);
+    *(int4*)(dst + 16) = make_int4((int)pk[4], (int)pk[5], (int)pk[6], (int)pk[7]);
   }
+}
+
+// Floats (n tokens of cols) to bf16 in slabs; npad tokens are written, zeros past n.  Thread:
+// 8 columns (16 bytes) of a token; a wave: the 64 bytes of 16 consecutive tokens.
+__global__ __launch_bounds__(256) void cvt_bf16_slabs_kernel(const float* __restrict__ x, u8* __restrict__ out, int n, long long npad, int cols) {
+  const int nk = cols / KS;
+  const long long i = (long long)blockIdx.x * 256 + threadIdx.x;      // (group, ks, token in group, piece)
+  const int piece = (int)(i & 3), tl = (int)((i >> 2) % SLAB_ROWS);
+  const long long gk = i / (4 * SLAB_ROWS);
+  const int ks = (int)(gk % nk);
+  const long long tok = (gk / nk) * SLAB_ROWS + tl;
+  if (tok >= npad) return;
+  int4 v = make_int4(0, 0, 0, 0);
+  if (tok < n) {
+    const float4* src = (const float4*)(x + tok * cols + ks * KS + 8 * piece);
+    const float4 a = src[0], b = src[1];
+    v = make_int4(pack_bf16(a.x, a.y), pack_bf16(a.z, a.w), pack_bf16(b.x, b.y), pack_bf16(b.z, b.w));
+  }
+  *(int4*)(out + slab_addr(tok, ks, nk) + 16 * piece) = v;
+}
+
+struct PlainSmem {
+  __align__(16) u8 xs[4][256 * KS * 2];
+  __align__(16) u8 ws[4][256 * KS * 2];
+};
+
+// 256 rows x 256 tokens a workgroup of four waves, one per SIMD with 128 x 128 results in 256
+// accumulator registers.  Both operands' 32-column slabs go from global memory straight into
+// LDS, three steps ahead, each into a ring of four slabs; a step's fragments are read half a
+// step ahead of their MFMAs.  One barrier a step.  p.w, p.x: the operands in slabs.
+__global__ __launch_bounds__(256, 1) void gemm_bf16_plain_kernel(BfParams p) {
+  __shared__ PlainSmem S;
+  constexpr int T = 256, NI = 4;
+  const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+  const int NR = (p.rows + T - 1) / T, NT = (p.ntok + T - 1) / T;
+  const int total = NT * NR, per = (total + 7) / 8;
+  const int L = blockIdx.x, j = L >> 3;
+  const int s = (L & 7) * per + j;
+  if (j >= per || s >= total) return;
+  const int rg = s / (GR * NT), rem = s - rg * GR * NT, nr = min(GR, NR - rg * GR);
+  const int tt = rem / nr, rt = rg * GR + (rem - tt * nr);
+  const long tok0 = (long)tt * T;
+  const int ntok = min(T, p.ntok - (int)tok0), r0 = rt * T;
+  const int nk = p.cols / KS;
+
+  const u8* xbase = (const u8*)ilt_uniform_ptr((const u8*)p.x + slab_addr(tok0, 0, nk));
+  const u8* wbase = (const u8*)ilt_uniform_ptr(p.w + slab_addr(r0, 0, nk));
+  u32 off[NI];                                 // the same place in x's and W's slabs
+#pragma unroll
+  for (int i = 0; i < NI; i++) {
+    const int P = (wave * NI + i) * 64 + lane, r = P >> 2, kp = (P & 3) ^ (int)slab_swz(r);
+    off[i] = (u32)slab_addr(r, 0, nk) + 16 * kp;
+  }
+  v16f acc[4][4];
+#pragma unroll
+  for (int a = 0; a < 4; a++)
+#pragma unroll
+    for (int b = 0; b < 4; b++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) acc[a][b][r] = 0.0f;
+  const int wt0 = 128 * (wave & 1), wr0 = 128 * (wave >> 1);
+  const int l32 = lane & 31, lh = lane >> 5;
+  u32 aoff[4], boff[4];
+#pragma unroll
+  for (int a = 0; a < 4; a++) { aoff[a] = slab_off(wt0 + 32 * a + l32, lh); boff[a] = slab_off(wr0 + 32 * a + l32, lh); }
+
+  auto issue = [&](int stage, int ks) {
+#pragma unroll
+    for (int i = 0; i < NI; i++) ilt_g2lds16(xbase + ks * SLAB_BYTES + off[i], S.xs[stage] + (wave * NI + i) * 1024);
+#pragma unroll
+    for (int i = 0; i < NI; i++) ilt_g2lds16(wbase + ks * SLAB_BYTES + off[i], S.ws[stage] + (wave * NI + i) * 1024);
+  };
+  issue(0, 0);
+  issue(1, min(1, nk - 1));
+  issue(2, min(2, nk - 1));
+  asm volatile("s_waitcnt vmcnt(%0)" :: "n"(4 * NI) : "memory");
+  ilt_barrier_lds();
+  v8bf fa[4], fb[4], ga[4], gb[4];
+#pragma unroll
+  for (int a = 0; a < 4; a++) { fa[a] = *(const v8bf*)(S.xs[0] + aoff[a]); fb[a] = *(const v8bf*)(S.ws[0] + boff[a]); }
+
+  // ST: the step's slab, a constant after unrolling
+  auto step = [&](int ks, auto Sc) {
+    constexpr int ST = decltype(Sc)::value;
+    issue((ST + 3) & 3, min(ks + 3, nk - 1));
+    __builtin_amdgcn_sched_barrier(0);
+    auto half = [&](const u8* xs_next, const u8* ws_next, u32 flip, v8bf* ua, v8bf* ub, v8bf* na, v8bf* nb) {
+#pragma unroll
+      for (int q = 0; q < 4; q++) {
+        na[q] = *(const v8bf*)(xs_next + (aoff[q] ^ flip));
+        nb[q] = *(const v8bf*)(ws_next + (boff[q] ^ flip));
+#pragma unroll
+        for (int b = 0; b < 4; b++) acc[q][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ua[q], ub[b], acc[q][b], 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    };
+    half(S.xs[ST], S.ws[ST], 32, fa, fb, ga, gb);                          // columns 0..15; reads this step's 16..31
+    half(S.xs[(ST + 1) & 3], S.ws[(ST + 1) & 3], 0, ga, gb, fa, fb);        // columns 16..31; reads the next step's 0..15
+    // only this step's loads may still be on their way: slab ks+2, which the next step reads
+    // from its second half on, has landed; the barrier publishes it and frees slab ks
+    asm volatile("s_waitcnt vmcnt(%0)" :: "n"(2 * NI) : "memory");
+    ilt_barrier_lds();
+  };
+  for (int ks = 0; ks < nk; ks += 4) {
+    step(ks + 0, std::integral_constant<int, 0>{});
+    step(ks + 1, std::integral_constant<int, 1>{});
+    step(ks + 2, std::integral_constant<int, 2>{});
+    step(ks + 3, std::integral_constant<int, 3>{});
+  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+
+  store_tile<4, 4>(acc, p, tok0, ntok, r0, wt0, wr0, l32, lh);
 }
 
 __global__ __launch_bounds__(256) void cvt_bf16_kernel(const float* __restrict__ x, u16* __restrict__ xb, long long n8) {
@@ -521,4 +712,37 @@ hipError_t ilt_k_gemm_bf16_id(int fmt, const uint64_t* ptrs, long long add, cons
   p.ptrs = ptrs; p.add = add; p.counts = counts; p.bases = bases; p.ne = ne;
   p.rows = rows; p.cols = cols; p.row_bytes = row_bytes; p.x = xb; p.rmap = rmap; p.y = y; p.ntok = (int)total_rows;
   return dispatch_bf16<128, 128, 2>(fmt, p, total_rows / 128 + ne, st);
+}
+
+hipError_t ilt_k_cvt_bf16_slabs(const float* x, uint16_t* out, int n, int cols, hipStream_t st) {
+  if (n <= 0) return hipSuccess;
+  const long long npad = (n + 255LL) / 256 * 256, threads = npad * (cols / 8);
+  hipLaunchKernelGGL(cvt_bf16_slabs_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, st, x, (u8*)out, n, npad, cols);
+  return hipGetLastError();
+}
+
+hipError_t ilt_k_dequant_bf16(int fmt, const uint8_t* w, long long row_bytes, int rows, int cols, uint16_t* outp, hipStream_t st) {
+  if (rows <= 0) return hipSuccess;
+  u8* out = (u8*)outp;
+  const long long groups = (rows + 255LL) / 256 * 2;                    // of 128 rows, the padding included
+  const dim3 grid((unsigned)(groups * (cols / 128)));
+  switch (fmt) {
+    case ILT_Q4_K: hipLaunchKernelGGL(dequant_bf16_kernel<ILT_Q4_K>, grid, dim3(256), 0, st, w, row_bytes, rows, cols, out); break;
+    case ILT_Q6_K: hipLaunchKernelGGL(dequant_bf16_kernel<ILT_Q6_K>, grid, dim3(256), 0, st, w, row_bytes, rows, cols, out); break;
+    case ILT_Q2_K: hipLaunchKernelGGL(dequant_bf16_kernel<ILT_Q2_K>, grid, dim3(256), 0, st, w, row_bytes, rows, cols, out); break;
+    case ILT_IQ2_XXS: hipLaunchKernelGGL(dequant_bf16_kernel<ILT_IQ2_XXS>, grid, dim3(256), 0, st, w, row_bytes, rows, cols, out); break;
+    default: return hipErrorInvalidValue;
+  }
+  return hipGetLastError();
+}
+
+hipError_t ilt_k_gemm_bf16_plain(const uint16_t* wb, int rows, int cols, const uint16_t* xb, int ntok, float* y, const float* bias,
+                                 int acc, hipStream_t st) {
+  if (ntok <= 0 || rows <= 0) return hipSuccess;
+  BfParams p = {};
+  p.w = (const uint8_t*)wb; p.rows = rows; p.cols = cols; p.x = xb; p.y = y; p.bias = bias; p.acc = acc; p.ntok = ntok;
+  const long long total = (long long)((ntok + 255) / 256) * ((rows + 255) / 256), per = (total + 7) / 8;
+  if (per * 8 > 0x7FFFFFFFLL) return hipErrorInvalidValue;
+  hipLaunchKernelGGL(gemm_bf16_plain_kernel, dim3((unsigned)(per * 8)), dim3(256), 0, st, p);
+  return hipGetLastError();
 }

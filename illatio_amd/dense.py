@@ -148,6 +148,41 @@ def cmat_mul_bf16(dev, w, xb, y, n, bias=None, acc=False):
     return y
 
 
+def slabs_bytes(rows, cols):
+    """Bytes of a bf16 copy in slabs of ROWS x COLS (rows padded to a multiple of 256)."""
+    return 2 * cols * ((rows + 255) // 256 * 256)
+
+
+def slabs_to_rows(a, rows, cols):
+    """A slab copy downloaded as uint16 (32 columns of 128 rows in one piece) as ROWS x COLS."""
+    g = a.reshape(-1, cols // 32, 128, 32)
+    return g.transpose(0, 2, 1, 3).reshape(-1, cols)[:rows]
+
+
+def dequant_bf16(dev, w, out=None):
+    """The matrix W as bf16 in slabs, in OUT or a new DBuf of SLABS-BYTES, each weight the value
+    CMAT-MUL-BF16 rounds inside its loop: the first pass of the two-pass product."""
+    if w.type not in (Q2_K, Q4_K, Q6_K, IQ2_XXS):
+        raise ValueError(f"the bf16 product multiplies Q2_K, Q4_K, Q6_K and IQ2_XXS; {w.name} is type {w.type}")
+    out = out if out is not None else hip.hip_alloc(dev, slabs_bytes(w.rows, w.cols), zero=False)
+    hip.launch(dev, "dequant_bf16", (w.rows + 255) // 256 * 2 * (w.cols // 128), 256, [w.type, w.qs, out, w.rows, w.cols])
+    return out
+
+
+def cvt_bf16_slabs(dev, x, n, cols, out=None):
+    """N tokens of COLS floats (a DBuf) rounded to bf16 in slabs, into OUT or a new DBuf of SLABS-BYTES."""
+    out = out if out is not None else hip.hip_alloc(dev, slabs_bytes(n, cols), zero=False)
+    hip.launch(dev, "cvt_bf16_slabs", ((n + 255) // 256 * 256 * (cols // 8) + 255) // 256, 256, [x, out, n, cols])
+    return out
+
+
+def mat_mul_bf16(dev, wb, rows, cols, xs, y, n, bias=None, acc=False):
+    """Y = W X for N tokens, WB the matrix (DEQUANT-BF16) and XS the activations (CVT-BF16-SLABS)
+    as bf16 in slabs: the second pass."""
+    hip.launch(dev, "mm_bf16", ((n + 255) // 256, (rows + 255) // 256), 256, [wb, xs, y, bias, rows, cols, n, 1 if acc else 0])
+    return y
+
+
 class MvDesc(C.Structure):
     _fields_ = [("gguf_type", C.c_int), ("rows", C.c_int), ("w", C.c_uint64), ("wd", C.c_uint64),
                 ("y", C.c_uint64), ("bias", C.c_uint64)]

@@ -261,6 +261,16 @@ int ilt_d4_mm_id_q2_k(uint64_t stream, int ncols, int nrows, int row_bytes, int6
    mm_k_bf16: gguf_type 10 Q2_K, 12 Q4_K, 14 Q6_K (212-byte device blocks of
      ilt_repack_q6k), 16 IQ2_XXS; xb is n tokens of cols bf16, 16-byte aligned;
      y[t*rows + r] (+= when acc, + bias[r]).  The matrix is at most 4 GiB.
+   dequant_bf16 + cvt_bf16_slabs + mm_bf16: the same product in two passes, for thousands of
+     tokens or a matrix multiplied again and again.  dequant_bf16 writes the matrix as bf16
+     (each weight the value mm_k_bf16 rounds in its loop), cvt_bf16_slabs the activations;
+     mm_bf16 multiplies the two copies and returns mm_k_bf16's numbers (the same products
+     added in the same order).  Both copies are laid out in slabs -- the 32 columns
+     32s..32s+31 of rows 128g..128g+127 are 8 KB in one piece at ((g * cols/32) + s) * 8192,
+     row r of the group at 64 * (r % 128) -- with the rows (tokens) padded with zeros to a
+     multiple of 256: a copy is 2 * cols * ceil(rows / 256) * 256 bytes, 16-byte aligned;
+     cols a multiple of 128 (dequant_bf16: of 256).  With memory to spare the matrix's copy can
+     stay resident beside the quantized matrix that decode reads.
    d4_mm_id_bf16: the grouped expert product of ds4f_mm.cu:256-257, same gguf_type codes, other
      arguments as d4_mm_id_*.  Row i of the groups multiplies xb's row rmap[i] (d4_group_scatter's
      row -> token map: the tokens' activations are read in place, no gathered copy), or row i
@@ -269,6 +279,10 @@ int ilt_d4_mm_id_q2_k(uint64_t stream, int ncols, int nrows, int row_bytes, int6
 int ilt_cvt_bf16(uint64_t stream, const float* x, uint16_t* xb, int64_t n);
 int ilt_mm_k_bf16(uint64_t stream, int gguf_type, const void* w, const uint16_t* xb, float* y, const float* bias,
                   int rows, int cols, int n, int acc);
+int ilt_cvt_bf16_slabs(uint64_t stream, const float* x, uint16_t* xs, int n, int cols);
+int ilt_dequant_bf16(uint64_t stream, int gguf_type, const void* w, uint16_t* wb, int rows, int cols);
+int ilt_mm_bf16(uint64_t stream, const uint16_t* wb, const uint16_t* xb, float* y, const float* bias, int rows, int cols, int n,
+                int acc);
 int ilt_d4_mm_id_bf16(uint64_t stream, int gguf_type, int ncols, int nrows, int row_bytes, int64_t add, const uint64_t* ptrs,
                       const uint32_t* counts, const uint32_t* bases, int ne, int64_t total_rows,
                       const uint16_t* xb, const uint32_t* rmap, float* y);

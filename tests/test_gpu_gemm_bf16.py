@@ -172,3 +172,50 @@ def test_moe_prefill_chunk_bf16_within_tolerance(dev, ne, d, ff, nu, n, clamp):
     for b in (lb, nb, sb, moe):
         hip.hip_free(b)
     pool.free()
+
+
+@pytest.mark.parametrize("qtype,rows,cols,n", [
+    (synth.Q6_K, 640, 5120, 200),
+    (synth.Q4_K, 300, 256, 77),          # one ragged tile, two steps... and a single super-block of columns
+    (synth.Q2_K, 513, 1024, 300),
+    (synth.IQ2_XXS, 256, 4096, 256),
+    (synth.Q6_K, 8200, 512, 4000),       # many tiles, ragged both ways
+])
+def test_two_pass_bf16_product(dev, monkeypatch, qtype, rows, cols, n):
+    """dequant_bf16 writes each weight as the one-pass kernel rounds it; mm_bf16 on that copy adds
+    the same products in the same order, so it returns the one-pass kernel's numbers."""
+    from illatio_amd import dense, hip
+    monkeypatch.delenv("ILT_BF16_TILE", raising=False)
+    rng = synth.make_rng(qtype * 11 + rows + n)
+    w = synth.weights(qtype, rows, cols, rng)
+    x = synth.activations((n, cols), rng)
+    bias = synth.activations(rows, rng)
+    m = upload(dev, qtype, rows, cols, w)
+    wb = dense.dequant_bf16(dev, m)
+    slabs = hip.hip_download(wb, np.uint16, dense.slabs_bytes(rows, cols) // 2)
+    got_w = (dense.slabs_to_rows(slabs, rows, cols).astype(np.uint32) << 16).view(np.float32)
+    want_w = bf16_round(orc.dequant_rows(qtype, w, cols)).reshape(rows, cols)
+    assert np.array_equal(got_w, want_w), np.argwhere(got_w != want_w)[:8]       # as numbers: -0.0 == 0.0
+    assert not dense.slabs_to_rows(slabs, (rows + 255) // 256 * 256, cols)[rows:].any()      # the padding rows are zeros
+    xf, bb = hip.hip_upload_new(dev, x), hip.hip_upload_new(dev, bias)
+    y1, y2 = hip.hip_alloc(dev, 4 * n * rows), hip.hip_alloc(dev, 4 * n * rows)
+    xb = dense.cvt_bf16(dev, xf, x.size)
+    xs = dense.cvt_bf16_slabs(dev, xf, n, cols)
+    assert np.array_equal(dense.slabs_to_rows(hip.hip_download(xs, np.uint16, dense.slabs_bytes(n, cols) // 2), n, cols),
+                          hip.hip_download(xb, np.uint16, x.size).reshape(n, cols))
+    dense.cmat_mul_bf16(dev, m, xb, y1, n)
+    dense.mat_mul_bf16(dev, wb, rows, cols, xs, y2, n)
+    one = hip.hip_floats(y1, n * rows).reshape(n, rows)
+    two = hip.hip_floats(y2, n * rows).reshape(n, rows)
+    assert np.array_equal(one, two), np.argwhere(one != two)[:8]
+    cpu = orc.matmul(qtype, w, rows, cols, x, nthreads=16)
+    assert np.abs(two - cpu).max() <= TOL_VS_CPU * np.abs(cpu).max()
+    dense.mat_mul_bf16(dev, wb, rows, cols, xs, y2, n, bias=bb, acc=True)
+    assert np.array_equal(hip.hip_floats(y2, n * rows).reshape(n, rows), two + (two + bias[None, :]))
+    dense.mat_mul_bf16(dev, wb, rows, cols, xs, y2, n, acc=True)                 # each of the four store loops
+    assert np.array_equal(hip.hip_floats(y2, n * rows).reshape(n, rows), (two + (two + bias[None, :])) + two)
+    dense.mat_mul_bf16(dev, wb, rows, cols, xs, y2, n, bias=bb)
+    assert np.array_equal(hip.hip_floats(y2, n * rows).reshape(n, rows), two + bias[None, :])
+    for b in (xf, xb, xs, bb, y1, y2, wb):
+        hip.hip_free(b)
+    m.free()
