@@ -168,6 +168,7 @@ struct BfParams {
   const u16* x;                              // bf16 activations, cols per token (the gathered rows when grouped)
   const u32* rmap;                           // grouped: row i of the groups is x's row rmap[i] (null: row i)
   float* y; const float* bias; int acc; int ntok;
+  long long ldy;                             // floats from a token's results to the next token's in y (rows, unless p covers a part of the rows)
 };
 
 template <int TM, int TN, int NXS, int NWS> struct Smem {
@@ -191,16 +192,16 @@ __device__ __forceinline__ u32 slab_off(int r, int p) { return (u32)(4 * r + (p 
 // workgroup on a CU nothing else runs while it stores, so the loop is kept to an address add
 // and a store per value and has no branches: the stores go through a buffer descriptor that
 // ends with the tile's last token, which drops what lies past it, and a lane whose row the
-// matrix does not have starts 2 GiB out.  (rows * 1024 < 2^31, checked by the host.)
+// matrix does not have starts 2 GiB out.  (ldy * 1024 < 2^31, checked by the host.)
 template <int NA, int NB, bool BIAS, bool ACC>
 __device__ __forceinline__ void store_patches(const v16f (&acc)[NA][NB], const BfParams& p, __amdgpu_buffer_rsrc_t ry, int r0,
                                               int wt0, int wr0, int l32, int lh) {
-  const u32 rows4 = (u32)p.rows * 4;
+  const u32 rows4 = (u32)p.ldy * 4;
 #pragma unroll
   for (int b = 0; b < NB; b++) {
     const int row = r0 + wr0 + 32 * b + l32;
     const bool ok = row < p.rows;
-    const u32 base = ok ? (u32)((wt0 + 4 * lh) * p.rows + row) * 4 : 0x80000000u;
+    const u32 base = ok ? (u32)((wt0 + 4 * lh) * (int)p.ldy + row) * 4 : 0x80000000u;
     float bv = 0.0f;
     if (BIAS) bv = ok ? p.bias[row] : 0.0f;
 #pragma unroll
@@ -226,8 +227,8 @@ template <int NA, int NB>
 __device__ __forceinline__ void store_tile(const v16f (&acc)[NA][NB], const BfParams& p, long tok0, int ntok, int r0,
                                            int wt0, int wr0, int l32, int lh) {
   // (ntok may come out of LDS: the same in every lane, said so to the compiler)
-  const u32 ybytes = (u32)__builtin_amdgcn_readfirstlane(ntok) * (u32)p.rows * 4;
-  const __amdgpu_buffer_rsrc_t ry = ilt_rsrc(ilt_uniform_ptr(p.y + tok0 * (long)p.rows), ybytes);
+  const u32 ybytes = ((u32)(__builtin_amdgcn_readfirstlane(ntok) - 1) * (u32)p.ldy + (u32)p.rows) * 4;
+  const __amdgpu_buffer_rsrc_t ry = ilt_rsrc(ilt_uniform_ptr(p.y + tok0 * p.ldy), ybytes);
   if (p.bias) {
     if (p.acc) store_patches<NA, NB, true, true>(acc, p, ry, r0, wt0, wr0, l32, lh);
     else store_patches<NA, NB, true, false>(acc, p, ry, r0, wt0, wr0, l32, lh);
@@ -552,18 +553,20 @@ __global__ __launch_bounds__(256) void cvt_bf16_slabs_kernel(const float* __rest
   *(int4*)(out + slab_addr(tok, ks, nk) + 16 * piece) = v;
 }
 
-struct PlainSmem {
-  __align__(16) u8 xs[4][256 * KS * 2];
-  __align__(16) u8 ws[4][256 * KS * 2];
+template <int T> struct PlainSmem {
+  __align__(16) u8 xs[4][T * KS * 2];
+  __align__(16) u8 ws[4][T * KS * 2];
 };
 
-// 256 rows x 256 tokens a workgroup of four waves, one per SIMD with 128 x 128 results in 256
-// accumulator registers.  Both operands' 32-column slabs go from global memory straight into
+// T rows x T tokens a workgroup of four waves.  T = 256: a wave alone on its SIMD with 128 x 128
+// results in 256 accumulator registers; T = 128 (two workgroups a CU) for the rows left over
+// when the 256-tiles do not fill a whole number of rounds over the CUs.  Both operands' 32-column slabs go from global memory straight into
 // LDS, three steps ahead, each into a ring of four slabs; a step's fragments are read half a
 // step ahead of their MFMAs.  One barrier a step.  p.w, p.x: the operands in slabs.
-__global__ __launch_bounds__(256, 1) void gemm_bf16_plain_kernel(BfParams p) {
-  __shared__ PlainSmem S;
-  constexpr int T = 256, NI = 4;
+template <int T>
+__global__ __launch_bounds__(256, (T == 256 ? 1 : 2)) void gemm_bf16_plain_kernel(BfParams p) {
+  __shared__ PlainSmem<T> S;
+  constexpr int NI = T / 64, NP = T / 64;      // direct loads per wave, step and operand; 32 x 32 patches each way per wave
   const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
   const int NR = (p.rows + T - 1) / T, NT = (p.ntok + T - 1) / T;
   const int total = NT * NR, per = (total + 7) / 8;
@@ -584,18 +587,18 @@ __global__ __launch_bounds__(256, 1) void gemm_bf16_plain_kernel(BfParams p) {
     const int P = (wave * NI + i) * 64 + lane, r = P >> 2, kp = (P & 3) ^ (int)slab_swz(r);
     off[i] = (u32)slab_addr(r, 0, nk) + 16 * kp;
   }
-  v16f acc[4][4];
+  v16f acc[NP][NP];
 #pragma unroll
-  for (int a = 0; a < 4; a++)
+  for (int a = 0; a < NP; a++)
 #pragma unroll
-    for (int b = 0; b < 4; b++)
+    for (int b = 0; b < NP; b++)
 #pragma unroll
       for (int r = 0; r < 16; r++) acc[a][b][r] = 0.0f;
-  const int wt0 = 128 * (wave & 1), wr0 = 128 * (wave >> 1);
+  const int wt0 = (T / 2) * (wave & 1), wr0 = (T / 2) * (wave >> 1);
   const int l32 = lane & 31, lh = lane >> 5;
-  u32 aoff[4], boff[4];
+  u32 aoff[NP], boff[NP];
 #pragma unroll
-  for (int a = 0; a < 4; a++) { aoff[a] = slab_off(wt0 + 32 * a + l32, lh); boff[a] = slab_off(wr0 + 32 * a + l32, lh); }
+  for (int a = 0; a < NP; a++) { aoff[a] = slab_off(wt0 + 32 * a + l32, lh); boff[a] = slab_off(wr0 + 32 * a + l32, lh); }
 
   auto issue = [&](int stage, int ks) {
 #pragma unroll
@@ -606,11 +609,11 @@ __global__ __launch_bounds__(256, 1) void gemm_bf16_plain_kernel(BfParams p) {
   issue(0, 0);
   issue(1, min(1, nk - 1));
   issue(2, min(2, nk - 1));
-  asm volatile("s_waitcnt vmcnt(%0)" :: "n"(4 * NI) : "memory");
+  asm volatile("s_waitcnt vmcnt(%0)" :: "n"(2 * NI) : "memory");     // slabs 0 and 1: step 0 reads both
   ilt_barrier_lds();
-  v8bf fa[4], fb[4], ga[4], gb[4];
+  v8bf fa[NP], fb[NP], ga[NP], gb[NP];
 #pragma unroll
-  for (int a = 0; a < 4; a++) { fa[a] = *(const v8bf*)(S.xs[0] + aoff[a]); fb[a] = *(const v8bf*)(S.ws[0] + boff[a]); }
+  for (int a = 0; a < NP; a++) { fa[a] = *(const v8bf*)(S.xs[0] + aoff[a]); fb[a] = *(const v8bf*)(S.ws[0] + boff[a]); }
 
   // ST: the step's slab, a constant after unrolling
   auto step = [&](int ks, auto Sc) {
@@ -619,11 +622,11 @@ __global__ __launch_bounds__(256, 1) void gemm_bf16_plain_kernel(BfParams p) {
     __builtin_amdgcn_sched_barrier(0);
     auto half = [&](const u8* xs_next, const u8* ws_next, u32 flip, v8bf* ua, v8bf* ub, v8bf* na, v8bf* nb) {
 #pragma unroll
-      for (int q = 0; q < 4; q++) {
+      for (int q = 0; q < NP; q++) {
         na[q] = *(const v8bf*)(xs_next + (aoff[q] ^ flip));
         nb[q] = *(const v8bf*)(ws_next + (boff[q] ^ flip));
 #pragma unroll
-        for (int b = 0; b < 4; b++) acc[q][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ua[q], ub[b], acc[q][b], 0, 0, 0);
+        for (int b = 0; b < NP; b++) acc[q][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ua[q], ub[b], acc[q][b], 0, 0, 0);
         __builtin_amdgcn_sched_barrier(0);
       }
     };
@@ -642,7 +645,7 @@ __global__ __launch_bounds__(256, 1) void gemm_bf16_plain_kernel(BfParams p) {
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 
-  store_tile<4, 4>(acc, p, tok0, ntok, r0, wt0, wr0, l32, lh);
+  store_tile<NP, NP>(acc, p, tok0, ntok, r0, wt0, wr0, l32, lh);
 }
 
 __global__ __launch_bounds__(256) void cvt_bf16_kernel(const float* __restrict__ x, u16* __restrict__ xb, long long n8) {
@@ -685,6 +688,7 @@ hipError_t ilt_k_gemm_bf16(int fmt, const uint8_t* w, long long row_bytes, int r
   if (ntok <= 0 || rows <= 0) return hipSuccess;
   BfParams p = {};
   p.w = w; p.rows = rows; p.cols = cols; p.row_bytes = row_bytes; p.x = xb; p.y = y; p.bias = bias; p.acc = acc; p.ntok = ntok;
+  p.ldy = rows;
   // Larger tiles fetch and dequantize less per product but leave more of the last round of
   // workgroups idle.  Cost of a variant: rounds over the 256 CUs x tile area / its measured
   // relative rate (128x128 0.85, 128x256 1.0, 256x256 1.1).
@@ -711,6 +715,7 @@ hipError_t ilt_k_gemm_bf16_id(int fmt, const uint64_t* ptrs, long long add, cons
   BfParams p = {};
   p.ptrs = ptrs; p.add = add; p.counts = counts; p.bases = bases; p.ne = ne;
   p.rows = rows; p.cols = cols; p.row_bytes = row_bytes; p.x = xb; p.rmap = rmap; p.y = y; p.ntok = (int)total_rows;
+  p.ldy = rows;
   return dispatch_bf16<128, 128, 2>(fmt, p, total_rows / 128 + ne, st);
 }
 
@@ -736,13 +741,47 @@ hipError_t ilt_k_dequant_bf16(int fmt, const uint8_t* w, long long row_bytes, in
   return hipGetLastError();
 }
 
+template <int T>
+static hipError_t launch_plain(const BfParams& p, hipStream_t st) {
+  const long long total = (long long)((p.ntok + T - 1) / T) * ((p.rows + T - 1) / T), per = (total + 7) / 8;
+  if (per * 8 > 0x7FFFFFFFLL) return hipErrorInvalidValue;
+  hipLaunchKernelGGL(gemm_bf16_plain_kernel<T>, dim3((unsigned)(per * 8)), dim3(256), 0, st, p);
+  return hipGetLastError();
+}
+
 hipError_t ilt_k_gemm_bf16_plain(const uint16_t* wb, int rows, int cols, const uint16_t* xb, int ntok, float* y, const float* bias,
                                  int acc, hipStream_t st) {
   if (ntok <= 0 || rows <= 0) return hipSuccess;
   BfParams p = {};
   p.w = (const uint8_t*)wb; p.rows = rows; p.cols = cols; p.x = xb; p.y = y; p.bias = bias; p.acc = acc; p.ntok = ntok;
-  const long long total = (long long)((ntok + 255) / 256) * ((rows + 255) / 256), per = (total + 7) / 8;
-  if (per * 8 > 0x7FFFFFFFLL) return hipErrorInvalidValue;
-  hipLaunchKernelGGL(gemm_bf16_plain_kernel, dim3((unsigned)(per * 8)), dim3(256), 0, st, p);
-  return hipGetLastError();
+  p.ldy = rows;
+  // One 256 x 256 tile a CU at a time: tiles beyond a whole number of rounds over the 256 CUs
+  // would take a round of their own.  Instead the row tiles that fill whole rounds go to the
+  // 256-tiles and the rows left over to 128-tiles (512 a round, a round of them about 0.7 of a
+  // big one for half the work); with less than one round of 256-tiles, everything to 128-tiles.
+  const long long nt = (ntok + 255) / 256, nr = (rows + 255) / 256, full = nt * nr / 256;
+  const char* force = getenv("ILT_BF16_PLAIN_SPLIT");      // "0": 256-tiles only; "128": 128-tiles only (tests)
+  long long nr_big = nr;
+  if (force ? atoi(force) == 128 : full == 0) nr_big = 0;
+  else if (!(force && atoi(force) == 0) && nt * nr % 256 != 0) {
+    const long long nr1 = full * 256 / nt, rest = rows - nr1 * 256;
+    const long long small_rounds = (((rest + 127) / 128) * ((ntok + 127) / 128) + 511) / 512;
+    if (0.7 * (double)small_rounds < 1.0) nr_big = nr1;
+  }
+  if (nr_big > 0) {
+    BfParams q = p;
+    q.rows = (int)min((long long)rows, nr_big * 256);
+    const hipError_t e = launch_plain<256>(q, st);
+    if (e != hipSuccess) return e;
+  }
+  if (nr_big * 256 < rows) {
+    const long long r1 = nr_big * 256;
+    BfParams q = p;
+    q.rows = rows - (int)r1;
+    q.w = p.w + r1 * (long long)cols * 2;                // whole groups of 128 rows: their slabs follow one another
+    q.y = y + r1;
+    q.bias = bias ? bias + r1 : nullptr;
+    return launch_plain<128>(q, st);
+  }
+  return hipSuccess;
 }

@@ -181,11 +181,16 @@ def test_moe_prefill_chunk_bf16_within_tolerance(dev, ne, d, ff, nu, n, clamp):
     (synth.IQ2_XXS, 256, 4096, 256),
     (synth.Q6_K, 8200, 512, 4000),       # many tiles, ragged both ways
 ])
-def test_two_pass_bf16_product(dev, monkeypatch, qtype, rows, cols, n):
+@pytest.mark.parametrize("split", [None, "0", "128"])      # tiles chosen by shape (256-tiles + 128-tiles for the rows left over), 256 only, 128 only
+def test_two_pass_bf16_product(dev, monkeypatch, qtype, rows, cols, n, split):
     """dequant_bf16 writes each weight as the one-pass kernel rounds it; mm_bf16 on that copy adds
     the same products in the same order, so it returns the one-pass kernel's numbers."""
     from illatio_amd import dense, hip
     monkeypatch.delenv("ILT_BF16_TILE", raising=False)
+    if split is None:
+        monkeypatch.delenv("ILT_BF16_PLAIN_SPLIT", raising=False)
+    else:
+        monkeypatch.setenv("ILT_BF16_PLAIN_SPLIT", split)
     rng = synth.make_rng(qtype * 11 + rows + n)
     w = synth.weights(qtype, rows, cols, rng)
     x = synth.activations((n, cols), rng)
