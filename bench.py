@@ -52,7 +52,7 @@ def _t(fetch_kib, write_kib):
 TRAFFIC = {"c1": {"up": _t(2407.5, 22.0), "down": _t(2347.5, 7.0)},
            "c2": {"qkv": _t(4862.4, 33.3), "wo": _t(3041.5, 12.0), "glu": _t(13843.7, 48.0), "down": _t(10239.8, 12.0),
                   "head": _t(176130.8, 638.9)},
-           "c3": {"mm": _t(519278.8, 282880.0)},
+           "c3": {"bf16-1pass": _t(519278.8, 282880.0)},
            "c4": {"d4_mv_iq2_xxs": _t(13388.0, 96.4), "d4_mv_q2_k": _t(8223.3, 96.4), "d4_mvq8": _t(4430.6, 10.7)},
            "c5": {"d4_mm_id_bf16": _t((2 * 366921.8 + 388488.5) / 3, (2 * 196608.0 + 393216.0) / 3)}}
 
@@ -65,7 +65,7 @@ def traffic_of(workload, per):
 
 
 HBM_PEAK_GBS = 8000.0
-MFMA_PEAK_TFLOPS = {"bf16": 2500.0, "bf16-2pass": 2500.0, "bf16-resident": 2500.0, "int8": 5000.0}
+MFMA_PEAK_TFLOPS = {"bf16": 2500.0, "bf16-1pass": 2500.0, "bf16-2pass": 2500.0, "bf16-resident": 2500.0, "int8": 5000.0}
 
 D, FFN, QD, KVD, VOCAB, LAYERS = 2560, 9728, 4096, 1024, 151936, 36
 
@@ -315,11 +315,14 @@ def workload_c3(args, dev):
     flops = 2.0 * rows * cols * T
     tm = Timer(dev)
     bf16_path = args.path.startswith("bf16")
-    if args.path in ("bf16-2pass", "bf16-resident"):
+    path = args.path
+    if path == "bf16":                           # the faster way from the quantized matrix: two passes pay from about a thousand tokens on
+        path = "bf16-2pass" if T >= 1024 else "bf16-1pass"
+    if path in ("bf16-2pass", "bf16-resident"):
         # the matrix dequantized to a bf16 copy (inside every step, or once beforehand and kept), then the plain bf16 product
         xb = hip.hip_alloc(dev, dense.slabs_bytes(T, cols), zero=False)
         wb = dense.dequant_bf16(dev, m)
-        resident = args.path == "bf16-resident"
+        resident = path == "bf16-resident"
 
         def step(_):
             tm.launch("cvt", 0, lambda: dense.cvt_bf16_slabs(dev, xf, T, cols, xb))
@@ -327,7 +330,7 @@ def workload_c3(args, dev):
                 tm.launch("dequant", 0, lambda: dense.dequant_bf16(dev, m, wb))
             tm.launch("mm", flops, lambda: dense.mat_mul_bf16(dev, wb, rows, cols, xb, y, T))
         names = {"mm": "gemm_bf16_plain_kernel (both operands bf16 through LDS, v_mfma_f32_32x32x16_bf16)"}
-    elif args.path == "bf16":
+    elif path == "bf16-1pass":
         xb = hip.hip_alloc(dev, 2 * T * cols, zero=False)
 
         def step(_):
@@ -344,8 +347,8 @@ def workload_c3(args, dev):
     ms, dev_ms, per = tm.run(step, args.steps, args.warmup)
     roof = roofline_of({k: v for k, v in per.items() if k == "mm"}, "mfma", MFMA_PEAK_TFLOPS[args.path], "TFLOP/s" if bf16_path else "TOP/s", names)
     roof["unit"] = "TFLOP/s"
-    if args.path == "bf16" and T == 4096 and not args.transpose:
-        roof["traffic"] = traffic_of("c3", per)
+    if path in TRAFFIC["c3"] and T == 4096 and not args.transpose:
+        roof["traffic"] = TRAFFIC["c3"][path]
     tf = flops / (ms * 1e-3) / 1e12
 
     def cpu():
@@ -364,7 +367,7 @@ def workload_c3(args, dev):
     return {"value": round(tf, 1), "unit": "TFLOP/s", "ms_per_step": ms, "device_ms_per_step": dev_ms, "enqueue_ms": tm.enqueue_ms,
             "dtype": "bf16 x bf16, fp32 accumulate" if bf16_path else "int8 block dots, fp32 combine",
             "metric": "prefill product TFLOP/s (% of dense MFMA peak)",
-            "config": {"workload": f"c3: Q6_K prefill product {rows}x{cols} on {T} tokens, {args.path} path "
+            "config": {"workload": f"c3: Q6_K prefill product {rows}x{cols} on {T} tokens, {path} path "
                                    f"(activation conversion inside the step)", "flops_per_step": flops, "tokens": T},
             "extra": {"pct_of_mfma_peak": round(100 * tf / MFMA_PEAK_TFLOPS[args.path], 2)}, "roofline": roof, "cpu": cpu}
 
@@ -532,9 +535,9 @@ def main():
     ap.add_argument("--layers", type=int, default=LAYERS, help=argparse.SUPPRESS)
     ap.add_argument("--tokens", type=int, default=4096, help="c3, c5: tokens per step")
     ap.add_argument("--transpose", action="store_true", help="c3: the 5120x17408 matrix")
-    ap.add_argument("--path", default="bf16", choices=["bf16", "bf16-2pass", "bf16-resident", "int8"],
-                    help="c3, c5: which matrix-core path; c3 only: bf16-2pass = the matrix dequantized to a bf16 copy inside the step, then the plain "
-                         "bf16 product; bf16-resident = the copy made beforehand and kept")
+    ap.add_argument("--path", default="bf16", choices=["bf16", "bf16-1pass", "bf16-2pass", "bf16-resident", "int8"],
+                    help="c3, c5: which matrix-core path.  c3: bf16 = 2pass from 1024 tokens on, else 1pass; bf16-1pass = the matrix dequantized inside the product's loop; "
+                         "bf16-2pass = the matrix dequantized to a bf16 copy inside the step, then the plain bf16 product; bf16-resident = that copy made beforehand and kept")
     ap.add_argument("--norm", action="store_true", help="c2: include each layer's two norms and the output norm (inside the product launches in fused mode)")
     ap.add_argument("--mode", default="fused", choices=["fused", "fused-q", "single", "device"],
                     help="c4: fused = 5 launches a step, single = the reference's sequence of 12 (both with the routing done beforehand on the host, as the "

@@ -496,6 +496,7 @@ int ilt_dequant_bf16(uint64_t stream, int gguf_type, const void* w, uint16_t* wb
   ILT_REQUIRE(fmt && rows >= 0 && cols > 0 && cols % 256 == 0);
   if (rows == 0) return ILT_OK;
   ILT_REQUIRE(w && wb && ((uintptr_t)w & 1) == 0 && ((uintptr_t)wb & 15) == 0);
+  ILT_REQUIRE((long long)cols / 256 * block_bytes(fmt) * rows < 0xFFFFFFF0LL);
   return (int)ilt_k_dequant_bf16(fmt, (const uint8_t*)w, (long long)cols / 256 * block_bytes(fmt), rows, cols, wb, S(stream));
 }
 

@@ -239,13 +239,12 @@ __device__ __forceinline__ void store_tile(const v16f (&acc)[NA][NB], const BfPa
 }
 
 // TM rows x TN tokens per workgroup; wave w: rows 32*NB*(w/2).., tokens (TN/2)*(w%2)..: NA x NB
-// patches of 32x32.  NB = 2: 2*TM threads, two per row; NB = 4: TM threads, one per row, a
-// wave alone on its SIMD with 128x128 results in 256 accumulator registers.
+// patches of 32x32.  NB = 2: 2*TM threads, two per row.
 template <int TM, int NB> constexpr int bf16_threads() { return 64 * 2 * (TM / (32 * NB)); }
 
 template <int FMT, int TM, int TN, int NB>
 __global__ __launch_bounds__((bf16_threads<TM, NB>()), (TM == 256 ? 1 : TN == 256 ? 2 : 3)) void gemm_bf16_kernel(BfParams p) {
-  __shared__ Smem<TM, TN, (NB == 4 ? 4 : 3), (NB == 4 ? 3 : 2)> S;
+  __shared__ Smem<TM, TN, 3, 2> S;
   constexpr int THREADS = bf16_threads<TM, NB>();
   constexpr int NE = 2 * TM / THREADS;   // 16-column units of a row a thread dequantizes per step: 1 or 2
   constexpr int NA = TN / 64;            // 32-token patches per wave
@@ -354,79 +353,7 @@ __global__ __launch_bounds__((bf16_threads<TM, NB>()), (TM == 256 ? 1 : TN == 25
     for (int u = 0; u < NE; u++) load_w<FMT>(raw[u], rw, wrowoff, hb, e0 + u);
   };
 
-  if constexpr (NB == 4) {
-    // One wave per SIMD, 128x128 per wave: everything is one step deeper so that nothing waits
-    // after the barrier.  Step ks dequantizes step ks+2's weights (three weight slabs) and
-    // sends off step ks+3's x loads (four x slabs); the MFMA fragments are loaded half a step
-    // ahead: while the first 16 columns' MFMAs run, the second 16 columns' fragments are read,
-    // and under those MFMAs the next step's first fragments (its slabs were published by the
-    // barrier at the start of this step).
-    WRaw<FMT> rawa[NE], rawb[NE];
-    load_raw(rawa, 0);
-    issue_x(0, 0);
-    load_raw(rawb, 1);
-    issue_x(1, 1);
-    issue_x(2, 2);
-    dequant_to(rawa, 0, 0, 0);
-    dequant_to(rawa, 1, 0, 1);
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    ilt_barrier_lds();
-    int x0 = 0, x1 = 1, x2 = 2, x3 = 3;      // x ring: the step's slab, the next step's, ..., the one being filled
-    int w0 = 0, w1 = 1, w2 = 2;              // weight ring: the step's, the next step's, the one being written
-    v8bf fa[NA], fb[NB], ga[NA], gb[NB];
-#pragma unroll
-    for (int a = 0; a < NA; a++) fa[a] = *(const v8bf*)(S.xs[0] + aoff[a]);
-#pragma unroll
-    for (int b = 0; b < NB; b++) fb[b] = *(const v8bf*)(S.ws[0] + boff[b]);
-    auto step = [&](int ks, auto Jc) {
-      constexpr int J = decltype(Jc)::value;
-      constexpr int J2 = (J + 2) & 7;        // the step whose weights are dequantized now: 0..3 from rawa, 4..7 from rawb
-      if (J == 2) load_raw(rawa, min((ks >> 2) + 2, nh - 1));   // rawa's last use was during step 1
-      if (J == 6) load_raw(rawb, min((ks >> 2) + 2, nh - 1));
-      issue_x(x3, min(ks + 3, nk - 1));
-      __builtin_amdgcn_sched_barrier(0);
-      u8* wnew = S.ws[w2];
-      const WRaw<FMT>* rawn = J2 < 4 ? rawa : rawb;
-      // Each half step in four pieces the compiler may not mix: two fragment reads for the
-      // next half step, a quarter of a 16-weight unit's dequantization, four MFMAs.
-      auto half = [&](const u8* xs_next, const u8* ws_next, u32 flip, v8bf* ua, v8bf* ub, v8bf* na, v8bf* nb, int u) {
-        float o[16];
-#pragma unroll
-        for (int q = 0; q < 4; q++) {
-          na[q] = *(const v8bf*)(xs_next + (aoff[q] ^ flip));
-          nb[q] = *(const v8bf*)(ws_next + (boff[q] ^ flip));
-          dequant16<FMT>(rawn[u], J2 & 3, J2 >> 2, e0 + u, S.grid, o, q, q + 1);
-#pragma unroll
-          for (int b = 0; b < NB; b++) acc[q][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ua[q], ub[b], acc[q][b], 0, 0, 0);
-          __builtin_amdgcn_sched_barrier(0);
-        }
-        u32 pk[8];
-#pragma unroll
-        for (int i = 0; i < 8; i++) pk[i] = pack_bf16(o[2 * i], o[2 * i + 1]);
-        ilt_lds_st16_untracked(wnew + (wdst ^ (32 * u)), pk[0], pk[1], pk[2], pk[3]);
-        ilt_lds_st16_untracked(wnew + (wdst ^ (32 * u) ^ 16), pk[4], pk[5], pk[6], pk[7]);
-      };
-      half(S.xs[x0], S.ws[w0], 32, fa, fb, ga, gb, 0);     // columns 0..15: fa, fb; reads this step's columns 16..31
-      half(S.xs[x1], S.ws[w1], 0, ga, gb, fa, fb, 1);      // columns 16..31: ga, gb; reads the next step's columns 0..15
-      { const int t_ = x0; x0 = x1; x1 = x2; x2 = x3; x3 = t_; }
-      { const int t_ = w0; w0 = w1; w1 = w2; w2 = t_; }
-      // every load older than this step's has landed: this wave's share of x slab ks+2, which
-      // the next step reads; the barrier publishes it and the weight slab written just now
-      constexpr int mine = NI + ((J == 2 || J == 6) ? WL : 0);
-      asm volatile("s_waitcnt vmcnt(%0)" :: "n"(mine) : "memory");
-      ilt_barrier_lds();
-    };
-    for (int ks = 0; ks < nk; ks += 8) {
-      step(ks + 0, std::integral_constant<int, 0>{});
-      step(ks + 1, std::integral_constant<int, 1>{});
-      step(ks + 2, std::integral_constant<int, 2>{});
-      step(ks + 3, std::integral_constant<int, 3>{});
-      step(ks + 4, std::integral_constant<int, 4>{});
-      step(ks + 5, std::integral_constant<int, 5>{});
-      step(ks + 6, std::integral_constant<int, 6>{});
-      step(ks + 7, std::integral_constant<int, 7>{});
-    }
-  } else {
+  {
   // Two register sets of raw weights, each a half super-block (4 steps): rawa holds half 0
   // of a super-block, rawb half 1.  Step ks multiplies slab ks while it dequantizes step
   // ks+1's weights into the other weight slab; a set is reloaded, with the half two ahead,
@@ -506,31 +433,46 @@ __device__ __forceinline__ long long slab_addr(long long row, int ks, int nk) { 
   return ((row / SLAB_ROWS) * nk + ks) * SLAB_BYTES + (row % SLAB_ROWS) * (KS * 2);
 }
 
-// A workgroup: half super-block hb of a group of 128 rows; thread (row, e) dequantizes the 4 x 16
-// weights that kernel thread (row, e) dequantizes there, and writes 32 bytes into each of four slabs.
+// A workgroup: one super-block (256 columns, eight slabs) of a group of 128 rows, so that every
+// line of the quantized rows it touches is used up by it; thread (row, e) dequantizes the 2 x 4 x 16
+// weights that kernel thread (row, e) dequantizes there and writes 32 bytes into each slab.
+// Every eighth workgroup id is one XCD: an XCD takes a run of consecutive super-blocks, whose
+// rows' shared lines then meet in its L2.
 template <int FMT>
-__global__ __launch_bounds__(256) void dequant_bf16_kernel(const u8* __restrict__ w, long long row_bytes, int rows, int cols, u8* __restrict__ out) {
+__global__ __launch_bounds__(256) void dequant_bf16_kernel(const u8* __restrict__ w, long long row_bytes, int rows, int cols, u8* __restrict__ out,
+                                                           int total) {
   __shared__ u64 grid[256];
   if (FMT == ILT_IQ2_XXS) { grid[threadIdx.x] = bf_grid_dev[threadIdx.x]; __syncthreads(); }
-  const int nh = cols / 128, nk = cols / KS;
+  const int nsb = cols / 256, nk = cols / KS;
+  const int per = (total + 7) / 8, unit = (blockIdx.x & 7) * per + (blockIdx.x >> 3);
+  if ((int)(blockIdx.x >> 3) >= per || unit >= total) return;
   const int e = threadIdx.x & 1, rl = threadIdx.x >> 1;
-  const int hb = blockIdx.x % nh;
-  const long long row = (long long)(blockIdx.x / nh) * SLAB_ROWS + rl;
+  const int sb = unit % nsb;
+  const long long row = (long long)(unit / nsb) * SLAB_ROWS + rl;
   const bool live = row < rows;
-  WRaw<FMT> raw;
-  if (live) load_w<FMT>(raw, ilt_rsrc(w + row * row_bytes, (u32)row_bytes), 0u, hb, e);
+  WRaw<FMT> raw[2];
+  if (live) {
+    // one descriptor for the whole matrix (less than 4 GiB, checked by the host), the row in the lane's offset
+    const __amdgpu_buffer_rsrc_t rw = ilt_rsrc(w, (u32)min((long long)rows * row_bytes, 0xFFFFFFF0LL));
+    const u32 rowoff = (u32)(row * row_bytes);
+    load_w<FMT>(raw[0], rw, rowoff, 2 * sb, e);
+    load_w<FMT>(raw[1], rw, rowoff, 2 * sb + 1, e);
+  }
 #pragma unroll
-  for (int j = 0; j < 4; j++) {
-    u32 pk[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-    if (live) {
-      float o[16];
-      dequant16<FMT>(raw, j, hb & 1, e, grid, o);
+  for (int c = 0; c < 2; c++) {
 #pragma unroll
-      for (int k = 0; k < 8; k++) pk[k] = pack_bf16(o[2 * k], o[2 * k + 1]);
+    for (int j = 0; j < 4; j++) {
+      u32 pk[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+      if (live) {
+        float o[16];
+        dequant16<FMT>(raw[c], j, c, e, grid, o);
+#pragma unroll
+        for (int k = 0; k < 8; k++) pk[k] = pack_bf16(o[2 * k], o[2 * k + 1]);
+      }
+      u8* dst = out + slab_addr(row, 8 * sb + 4 * c + j, nk) + 32 * e;
+      *(int4*)dst = make_int4((int)pk[0], (int)pk[1], (int)pk[2], (int)pk[3]);
+      *(int4*)(dst + 16) = make_int4((int)pk[4], (int)pk[5], (int)pk[6], (int)pk[7]);
     }
-    u8* dst = out + slab_addr(row, 4 * hb + j, nk) + 32 * e;
-    *(int4*)dst = make_int4((int)pk[0], (int)pk[1], (int)pk[2], (int)pk[3]);
-    *(int4*)(dst + 16) = make_int4((int)pk[4], (int)pk[5], (int)pk[6], (int)pk[7]);
   }
 }
 
@@ -693,15 +635,14 @@ hipError_t ilt_k_gemm_bf16(int fmt, const uint8_t* w, long long row_bytes, int r
   // workgroups idle.  Cost of a variant: rounds over the 256 CUs x tile area / its measured
   // relative rate (128x128 0.85, 128x256 1.0, 256x256 1.1).
   const long long t128 = (ntok + 127) / 128, t256 = (ntok + 255) / 256, r256 = (rows + 255) / 256, r128 = (rows + 127) / 128;
-  const char* force = getenv("ILT_BF16_TILE");     // "1".."4": that variant whatever the shape (tests)
+  const char* force = getenv("ILT_BF16_TILE");     // "1".."3": that variant whatever the shape (tests)
   int tile = force ? atoi(force) : 0;
-  if (tile < 1 || tile > 4) {
+  if (tile < 1 || tile > 3) {
     const double c1 = (double)((t128 * r128 + 255) / 256) * 1.0 / 0.85;
     const double c2 = (double)((t256 * r128 + 255) / 256) * 2.0 / 1.0;
     const double c3 = (double)((t256 * r256 + 255) / 256) * 4.0 / 1.1;
     tile = c3 <= c2 && c3 <= c1 ? 3 : c2 <= c1 ? 2 : 1;
   }
-  if (tile == 4) return dispatch_bf16<256, 256, 4>(fmt, p, t256, st);
   if (tile == 3) return dispatch_bf16<256, 256, 2>(fmt, p, t256, st);
   if (tile == 2) return dispatch_bf16<128, 256, 2>(fmt, p, t256, st);
   return dispatch_bf16<128, 128, 2>(fmt, p, t128, st);
@@ -730,12 +671,15 @@ hipError_t ilt_k_dequant_bf16(int fmt, const uint8_t* w, long long row_bytes, in
   if (rows <= 0) return hipSuccess;
   u8* out = (u8*)outp;
   const long long groups = (rows + 255LL) / 256 * 2;                    // of 128 rows, the padding included
-  const dim3 grid((unsigned)(groups * (cols / 128)));
+  const long long units = groups * (cols / 256);
+  if (units > 0x7FFFFFF0LL) return hipErrorInvalidValue;
+  const int total = (int)units;
+  const dim3 grid((unsigned)((units + 7) / 8 * 8));
   switch (fmt) {
-    case ILT_Q4_K: hipLaunchKernelGGL(dequant_bf16_kernel<ILT_Q4_K>, grid, dim3(256), 0, st, w, row_bytes, rows, cols, out); break;
-    case ILT_Q6_K: hipLaunchKernelGGL(dequant_bf16_kernel<ILT_Q6_K>, grid, dim3(256), 0, st, w, row_bytes, rows, cols, out); break;
-    case ILT_Q2_K: hipLaunchKernelGGL(dequant_bf16_kernel<ILT_Q2_K>, grid, dim3(256), 0, st, w, row_bytes, rows, cols, out); break;
-    case ILT_IQ2_XXS: hipLaunchKernelGGL(dequant_bf16_kernel<ILT_IQ2_XXS>, grid, dim3(256), 0, st, w, row_bytes, rows, cols, out); break;
+    case ILT_Q4_K: hipLaunchKernelGGL(dequant_bf16_kernel<ILT_Q4_K>, grid, dim3(256), 0, st, w, row_bytes, rows, cols, out, total); break;
+    case ILT_Q6_K: hipLaunchKernelGGL(dequant_bf16_kernel<ILT_Q6_K>, grid, dim3(256), 0, st, w, row_bytes, rows, cols, out, total); break;
+    case ILT_Q2_K: hipLaunchKernelGGL(dequant_bf16_kernel<ILT_Q2_K>, grid, dim3(256), 0, st, w, row_bytes, rows, cols, out, total); break;
+    case ILT_IQ2_XXS: hipLaunchKernelGGL(dequant_bf16_kernel<ILT_IQ2_XXS>, grid, dim3(256), 0, st, w, row_bytes, rows, cols, out, total); break;
     default: return hipErrorInvalidValue;
   }
   return hipGetLastError();

@@ -44,7 +44,7 @@ def upload(dev, qtype, rows, cols, w):
 FORMATS = [synth.Q4_K, synth.Q6_K, synth.Q2_K, synth.IQ2_XXS]
 
 
-@pytest.mark.parametrize("tile", [1, 2, 3, 4])       # the 128x128, 128x256, 256x256 (8 waves) and 256x256 (4 waves) tiles
+@pytest.mark.parametrize("tile", [1, 2, 3])       # the 128x128, 128x256 and 256x256 tiles
 @pytest.mark.parametrize("qtype", FORMATS)
 @pytest.mark.parametrize("rows,cols", [(130, 512), (300, 256)])
 def test_one_hot_tokens_read_back_the_dequantized_matrix(dev, monkeypatch, qtype, rows, cols, tile):
@@ -72,7 +72,7 @@ def test_one_hot_tokens_read_back_the_dequantized_matrix(dev, monkeypatch, qtype
     (synth.IQ2_XXS, 256, 4096, 64),
     (synth.Q6_K, 8200, 512, 4000),       # enough tiles that the largest tile is chosen by itself; ragged both ways
 ])
-@pytest.mark.parametrize("tile", [0, 2, 3, 4])       # 0: chosen by shape; others: that tile forced
+@pytest.mark.parametrize("tile", [0, 1, 2, 3])       # 0: chosen by shape; others: that tile forced
 def test_dense_bf16_product_within_tolerance(dev, monkeypatch, qtype, rows, cols, n, tile):
     from illatio_amd import dense, hip
     if tile:
