@@ -97,10 +97,9 @@ __device__ __forceinline__ u32 word_of(const int4& v, int i) { return (u32)(i ==
 // scale times a 2- or 4-bit integer), and Q6_K's s*(q-32) is one rounding of an exact value;
 // so a fused multiply-add gives the same bits in half the instructions.
 // j: the step within the half super-block (a constant after unrolling); c: which half.
-// Words i0..i1-1 of the four (a word = 4 weights) are computed, so that a caller can spread the work.
-template <int FMT> __device__ __forceinline__ void dequant16(const WRaw<FMT>& r, int j, int c, int e, const u64* grid, float* o, int i0 = 0, int i1 = 4);
+template <int FMT> __device__ __forceinline__ void dequant16(const WRaw<FMT>& r, int j, int c, int e, float* o);
 
-template <> __device__ __forceinline__ void dequant16<ILT_Q4_K>(const WRaw<ILT_Q4_K>& r, int j, int c, int e, const u64*, float* o, int i0, int i1) {
+template <> __device__ __forceinline__ void dequant16<ILT_Q4_K>(const WRaw<ILT_Q4_K>& r, int j, int c, int e, float* o) {
   const int sh = 8 * j, hl = j & 1;              // group g = 4c + j of the super-block
   const u32 x0 = ((u32)r.hdr.y >> sh) & 0xFF, x1 = ((u32)r.hdr.z >> sh) & 0xFF, x2 = ((u32)r.hdr.w >> sh) & 0xFF;
   const u32 sc = c == 0 ? (x0 & 63) : ((x2 & 0xF) | ((x0 >> 6) << 4));
@@ -109,54 +108,81 @@ template <> __device__ __forceinline__ void dequant16<ILT_Q4_K>(const WRaw<ILT_Q
   const int4& q = r.q[j >> 1];
 #pragma unroll
   for (int i = 0; i < 4; i++) {
-    if (i < i0 || i >= i1) continue;
     const u32 v = (word_of(q, i) >> (4 * hl)) & 0x0F0F0F0F;
 #pragma unroll
     for (int k = 0; k < 4; k++) o[4 * i + k] = __builtin_fmaf(d1, (float)((v >> (8 * k)) & 0xFF), -m1);   // d1*q is exact in fp32
   }
 }
 
-template <> __device__ __forceinline__ void dequant16<ILT_Q6_K>(const WRaw<ILT_Q6_K>& r, int j, int c, int e, const u64*, float* o, int i0, int i1) {
+template <> __device__ __forceinline__ void dequant16<ILT_Q6_K>(const WRaw<ILT_Q6_K>& r, int j, int c, int e, float* o) {
   const int h = j >> 1;                          // 32-weight part j of the half: ql[j&1]'s nibble h, qh's bit pair j
   const u32 scw = (u32)(j < 2 ? r.sc.x : r.sc.y) >> (16 * (j & 1) + 8 * e);
   const float s = ilt_h2f((u16)r.d) * (float)(i8)(scw & 0xFF), s32 = -32.0f * s;
   const int4& ql = r.ql[j & 1];
 #pragma unroll
   for (int i = 0; i < 4; i++) {
-    if (i < i0 || i >= i1) continue;
     const u32 v = ((word_of(ql, i) >> (4 * h)) & 0x0F0F0F0F) | (((word_of(r.qh, i) >> (2 * j)) & 0x03030303) << 4);
 #pragma unroll
     for (int k = 0; k < 4; k++) o[4 * i + k] = __builtin_fmaf(s, (float)((v >> (8 * k)) & 0xFF), s32);   // = RN(s*(q-32)): one rounding either way
   }
 }
 
-template <> __device__ __forceinline__ void dequant16<ILT_Q2_K>(const WRaw<ILT_Q2_K>& r, int j, int c, int e, const u64*, float* o, int i0, int i1) {
+template <> __device__ __forceinline__ void dequant16<ILT_Q2_K>(const WRaw<ILT_Q2_K>& r, int j, int c, int e, float* o) {
   const u32 scw = ((u32)(j < 2 ? r.sc.x : r.sc.y) >> (16 * (j & 1) + 8 * e)) & 0xFF;
   const float dl = ilt_h2f((u16)(r.dd & 0xFFFF)) * (float)(scw & 15), ml = ilt_h2f((u16)(r.dd >> 16)) * (float)(scw >> 4);
 #pragma unroll
   for (int i = 0; i < 4; i++) {
-    if (i < i0 || i >= i1) continue;
     const u32 v = (word_of(r.q, i) >> (2 * j)) & 0x03030303;
 #pragma unroll
     for (int k = 0; k < 4; k++) o[4 * i + k] = __builtin_fmaf(dl, (float)((v >> (8 * k)) & 0xFF), -ml);   // dl*q is exact in fp32
   }
 }
 
-template <> __device__ __forceinline__ void dequant16<ILT_IQ2_XXS>(const WRaw<ILT_IQ2_XXS>& r, int j, int c, int e, const u64* grid, float* o, int i0, int i1) {
+// IQ2_XXS has three magnitudes (its codebook's bytes are 0x08, 0x19 and 0x2b), so a unit of 16
+// weights takes three products db*8, db*25, db*43 -- each the CPU's (db * mag), rounded to bf16
+// -- and every weight is one of those with its sign: a byte permute picks the pair of bf16 for
+// two weights, an xor sets their signs.  The permute selectors of a codebook entry and the sign
+// masks of a 7-bit sign index (+ parity) come ready-made from two tables in LDS.
+struct Iq2Tables {
+  u32 sel[256][4];       // entry g: selector for weights (2k, 2k+1) of codebook entry g, k = 0..3
+  u32 sgn[128][4];       // entry s: 0x8000 where weight 2k is negative | 0x80000000 where weight 2k+1 is
+};
+__device__ __forceinline__ void iq2_tables_fill(Iq2Tables& T, int t) {    // threads t = 0..255 of a workgroup; a barrier follows
+  const u64 g = bf_grid_dev[t & 255];
+#pragma unroll
+  for (int k = 0; k < 4; k++) {
+    const u32 t0 = ((u32)(g >> (16 * k + 3))) & 6, t1 = ((u32)(g >> (16 * k + 11))) & 6;    // 2 * (byte >> 4): 0, 2, 4
+    if (t < 256) T.sel[t][k] = t0 | ((t0 + 1) << 8) | (t1 << 16) | ((t1 + 1) << 24);
+  }
+  if (t < 128) {
+    const u32 sb = (u32)t | ((__popc(t) & 1) << 7);
+#pragma unroll
+    for (int k = 0; k < 4; k++) T.sgn[t][k] = (((sb >> (2 * k)) & 1) << 15) | (((sb >> (2 * k + 1)) & 1) << 31);
+  }
+}
+
+// 16 weights as 8 words of two bf16, in column order.
+template <int FMT>
+__device__ __forceinline__ void dequant16_pk(const WRaw<FMT>& r, int j, int c, int e, const Iq2Tables*, u32* pk) {
+  float o[16];
+  dequant16<FMT>(r, j, c, e, o);
+#pragma unroll
+  for (int i = 0; i < 8; i++) pk[i] = pack_bf16(o[2 * i], o[2 * i + 1]);
+}
+template <>
+__device__ __forceinline__ void dequant16_pk<ILT_IQ2_XXS>(const WRaw<ILT_IQ2_XXS>& r, int j, int c, int e, const Iq2Tables* T, u32* pk) {
   const int4& q = r.q[j >> 1];                   // the half's 32-weight group j: 8 bytes
   const u32 g = word_of(q, 2 * (j & 1)) >> (16 * e), aux = word_of(q, 2 * (j & 1) + 1);
   const float db = (ilt_h2f((u16)r.d) * (0.5f + (float)(aux >> 28))) * 0.25f;
+  const u32 t01 = pack_bf16(db * 8.0f, db * 25.0f), t2 = pack_bf16(db * 43.0f, 0.0f);
 #pragma unroll
   for (int l = 0; l < 2; l++) {
-    if (2 * l < i0 || 2 * l >= i1) continue;             // a codebook entry is two words
-    const int2 mag = ilt_lds_ld8(grid + ((g >> (8 * l)) & 0xFF));
-    u32 s = (aux >> (7 * (2 * e + l))) & 127;
-    s |= (__popc(s) & 1) << 7;
-#pragma unroll
-    for (int k = 0; k < 8; k++) {
-      const u32 m = ((k < 4 ? (u32)mag.x : (u32)mag.y) >> (8 * (k & 3))) & 0xFF;
-      o[8 * l + k] = (db * (float)m) * (((s >> k) & 1) ? -1.0f : 1.0f);
-    }
+    const int4 sel = ilt_lds_ld16(T->sel[(g >> (8 * l)) & 0xFF]);
+    const int4 sg = ilt_lds_ld16(T->sgn[(aux >> (7 * (2 * e + l))) & 127]);
+    pk[4 * l + 0] = __builtin_amdgcn_perm(t2, t01, (u32)sel.x) ^ (u32)sg.x;
+    pk[4 * l + 1] = __builtin_amdgcn_perm(t2, t01, (u32)sel.y) ^ (u32)sg.y;
+    pk[4 * l + 2] = __builtin_amdgcn_perm(t2, t01, (u32)sel.z) ^ (u32)sg.z;
+    pk[4 * l + 3] = __builtin_amdgcn_perm(t2, t01, (u32)sel.w) ^ (u32)sg.w;
   }
 }
 
@@ -174,7 +200,7 @@ struct BfParams {
 template <int TM, int TN, int NXS, int NWS> struct Smem {
   __align__(16) u8 xs[NXS][TN * KS * 2];
   __align__(16) u8 ws[NWS][TM * KS * 2];
-  u64 grid[256];
+  Iq2Tables iq2;
   u32 scan[256];
   int tile_z, tile_t0, tile_n;
 };
@@ -239,11 +265,12 @@ __device__ __forceinline__ void store_tile(const v16f (&acc)[NA][NB], const BfPa
 }
 
 // TM rows x TN tokens per workgroup; wave w: rows 32*NB*(w/2).., tokens (TN/2)*(w%2)..: NA x NB
-// patches of 32x32.  NB = 2: 2*TM threads, two per row.
+// patches of 32x32.  NB = 2: 2*TM threads, two per row (a thread dequantizes 16 weights a step);
+// NB = 4: TM threads, one per row (32 weights a step).
 template <int TM, int NB> constexpr int bf16_threads() { return 64 * 2 * (TM / (32 * NB)); }
 
 template <int FMT, int TM, int TN, int NB>
-__global__ __launch_bounds__((bf16_threads<TM, NB>()), (TM == 256 ? 1 : TN == 256 ? 2 : 3)) void gemm_bf16_kernel(BfParams p) {
+__global__ __launch_bounds__((bf16_threads<TM, NB>()), (TM * TN == 65536 ? 1 : TM * TN == 32768 ? 2 : 3)) void gemm_bf16_kernel(BfParams p) {
   __shared__ Smem<TM, TN, 3, 2> S;
   constexpr int THREADS = bf16_threads<TM, NB>();
   constexpr int NE = 2 * TM / THREADS;   // 16-column units of a row a thread dequantizes per step: 1 or 2
@@ -296,7 +323,7 @@ __global__ __launch_bounds__((bf16_threads<TM, NB>()), (TM == 256 ? 1 : TN == 25
   }
   const int r0 = rt * TM;
   if (FMT == ILT_IQ2_XXS) {
-    if (t < 256) S.grid[t] = bf_grid_dev[t];
+    if (t < 256) iq2_tables_fill(S.iq2, t);
     __syncthreads();
   }
 
@@ -336,11 +363,8 @@ __global__ __launch_bounds__((bf16_threads<TM, NB>()), (TM == 256 ? 1 : TN == 25
     for (int i = 0; i < NI; i++) ilt_g2lds16(xbase + ks * (KS * 2) + xoff[i], S.xs[stage] + (wave * NI + i) * 1024);
   };
   auto dequant_unit = [&](const WRaw<FMT>& raw, int u, int j, int c, u8* ws) {   // 16 weights of step j of a half into a slab
-    float o[16];
-    dequant16<FMT>(raw, j, c, e0 + u, S.grid, o);
     u32 pk[8];
-#pragma unroll
-    for (int i = 0; i < 8; i++) pk[i] = pack_bf16(o[2 * i], o[2 * i + 1]);
+    dequant16_pk<FMT>(raw, j, c, e0 + u, &S.iq2, pk);
     ilt_lds_st16_untracked(ws + (wdst ^ (32 * u)), pk[0], pk[1], pk[2], pk[3]);
     ilt_lds_st16_untracked(ws + (wdst ^ (32 * u) ^ 16), pk[4], pk[5], pk[6], pk[7]);
   };
@@ -441,8 +465,8 @@ __device__ __forceinline__ long long slab_addr(long long row, int ks, int nk) { 
 template <int FMT>
 __global__ __launch_bounds__(256) void dequant_bf16_kernel(const u8* __restrict__ w, long long row_bytes, int rows, int cols, u8* __restrict__ out,
                                                            int total) {
-  __shared__ u64 grid[256];
-  if (FMT == ILT_IQ2_XXS) { grid[threadIdx.x] = bf_grid_dev[threadIdx.x]; __syncthreads(); }
+  __shared__ Iq2Tables iq2;
+  if (FMT == ILT_IQ2_XXS) { iq2_tables_fill(iq2, threadIdx.x); __syncthreads(); }
   const int nsb = cols / 256, nk = cols / KS;
   const int per = (total + 7) / 8, unit = (blockIdx.x & 7) * per + (blockIdx.x >> 3);
   if ((int)(blockIdx.x >> 3) >= per || unit >= total) return;
@@ -463,12 +487,7 @@ __global__ __launch_bounds__(256) void dequant_bf16_kernel(const u8* __restrict_
 #pragma unroll
     for (int j = 0; j < 4; j++) {
       u32 pk[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-      if (live) {
-        float o[16];
-        dequant16<FMT>(raw[c], j, c, e, grid, o);
-#pragma unroll
-        for (int k = 0; k < 8; k++) pk[k] = pack_bf16(o[2 * k], o[2 * k + 1]);
-      }
+      if (live) dequant16_pk<FMT>(raw[c], j, c, e, &iq2, pk);
       u8* dst = out + slab_addr(row, 8 * sb + 4 * c + j, nk) + 32 * e;
       *(int4*)dst = make_int4((int)pk[0], (int)pk[1], (int)pk[2], (int)pk[3]);
       *(int4*)(dst + 16) = make_int4((int)pk[4], (int)pk[5], (int)pk[6], (int)pk[7]);
@@ -657,6 +676,14 @@ hipError_t ilt_k_gemm_bf16_id(int fmt, const uint64_t* ptrs, long long add, cons
   p.ptrs = ptrs; p.add = add; p.counts = counts; p.bases = bases; p.ne = ne;
   p.rows = rows; p.cols = cols; p.row_bytes = row_bytes; p.x = xb; p.rmap = rmap; p.y = y; p.ntok = (int)total_rows;
   p.ldy = rows;
+  // 256 rows x 128 tokens a workgroup (a wave: 128 x 64) when the matrices have the rows for it:
+  // an expert seldom has more than 128 rows of tokens in a chunk, and the taller tile reads a
+  // quarter less from LDS per MFMA than 128 x 128.  "1" in ILT_BF16_ID_TILE: 128 x 128 always (tests).
+  const char* force = getenv("ILT_BF16_ID_TILE");
+  if (rows % 256 == 0 && !(force && atoi(force) == 1)) {      // the expert formats (Q4_K / Q6_K raw sets would not fit the registers)
+    if (fmt == ILT_IQ2_XXS) return launch_bf16<ILT_IQ2_XXS, 256, 128, 4>(p, total_rows / 128 + ne, st);
+    if (fmt == ILT_Q2_K) return launch_bf16<ILT_Q2_K, 256, 128, 4>(p, total_rows / 128 + ne, st);
+  }
   return dispatch_bf16<128, 128, 2>(fmt, p, total_rows / 128 + ne, st);
 }
 

@@ -120,7 +120,8 @@ def exact_chunk(G, U, Dn, sel, ww, norms, clamp):
 
 @pytest.mark.parametrize("ne,d,ff,nu,n,clamp", [(8, 512, 256, 3, 37, 0.0), (16, 1024, 512, 4, 300, 0.6),
                                                  (12, 4096, 2048, 6, 96, 0.0)])
-def test_moe_prefill_chunk_bf16_within_tolerance(dev, ne, d, ff, nu, n, clamp):
+@pytest.mark.parametrize("id_tile", [None, "1"])       # 256 x 128 tiles where the rows allow (the default), 128 x 128 always
+def test_moe_prefill_chunk_bf16_within_tolerance(dev, monkeypatch, ne, d, ff, nu, n, clamp, id_tile):
     """The prefill chunk of test_gpu_gemm.py with the three grouped products on the bf16
     matrix cores.  Routing, counts and weights stay equal to the CPU path's.  Each grouped
     product is within 2e-2 of the CPU product (quantized activations, integer block dots)
@@ -128,6 +129,10 @@ def test_moe_prefill_chunk_bf16_within_tolerance(dev, ne, d, ff, nu, n, clamp):
     is the larger error (2-7% of the largest output at these shapes, against an exact
     double-precision chain), so the chain is held to this: the bf16 chunk is no farther
     from the exact chain than the CPU path's chunk is."""
+    if id_tile is None:
+        monkeypatch.delenv("ILT_BF16_ID_TILE", raising=False)
+    else:
+        monkeypatch.setenv("ILT_BF16_ID_TILE", id_tile)
     from illatio_amd import ds4f, hip
     rng = synth.make_rng(ne + d + n)
     gate = synth.weights(synth.IQ2_XXS, ne * ff, d, rng)
