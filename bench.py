@@ -49,12 +49,14 @@ def _t(fetch_kib, write_kib):
     return int((2 * fetch_kib + write_kib) * 1024)
 
 
-TRAFFIC = {"c1": {"up": _t(2407.5, 22.0), "down": _t(2347.5, 7.0)},
-           "c2": {"qkv": _t(4862.4, 33.3), "wo": _t(3041.5, 12.0), "glu": _t(13843.7, 48.0), "down": _t(10239.8, 12.0),
-                  "head": _t(176130.8, 638.9)},
-           "c3": {"bf16-1pass": _t(519278.8, 282880.0)},
-           "c4": {"d4_mv_iq2_xxs": _t(13388.0, 96.4), "d4_mv_q2_k": _t(8223.3, 96.4), "d4_mvq8": _t(4430.6, 10.7)},
-           "c5": {"d4_mm_id_bf16": _t((2 * 366921.8 + 388488.5) / 3, (2 * 196608.0 + 393216.0) / 3)}}
+TRAFFIC = {"c1": {"up": _t(2358.0, 22.0), "down": _t(2418.0, 7.0)},
+           "c2": {"qkv": _t(4879.9, 33.3), "wo": _t(3066.0, 12.0), "glu": _t(13872.2, 48.0), "down": _t(10383.6, 12.0),
+                  "head": _t(175754.1, 634.8)},
+           # one product: two-pass = the 256-tile launch plus the 128-tile launch for the rows left over
+           "c3": {"bf16-1pass": _t(519803.0, 278528.0), "bf16-2pass": _t(491863.8 + 61498.0, 262144.0 + 16384.0),
+                  "bf16-resident": _t(491863.8 + 61498.0, 262144.0 + 16384.0)},
+           "c4": {"d4_mv_glu_iq2_xxs": _t(12952.9, 63.8), "d4_mv_q2_k_f32": _t(8381.6, 96.4), "d4_mvq8_glu": _t(8860.1, 16.0)},
+           "c5": {"d4_mm_id_bf16": _t((2 * 305779.3 + 367082.0) / 3, (2 * 196608.0 + 393216.0) / 3)}}
 
 
 def traffic_of(workload, per):
@@ -440,7 +442,7 @@ def workload_c4(args, dev):
                         "d4_mvq8": "gemv_kernel<8> (shared expert, Q8_0)", "d4_mvq8_glu": "gemv_kernel<8> (shared expert gate, up, gated activation)"})
     roof["launch_us_all"] = {k: round(v[0] / v[2] * 1e3, 2) for k, v in per.items()}
     dom = max((k for k in per if per[k][1]), key=lambda k: per[k][0])
-    roof["traffic"] = TRAFFIC["c4"].get({"d4_mv_glu_iq2_xxs": "d4_mv_iq2_xxs", "d4_mv_q2_k_f32": "d4_mv_q2_k"}.get(dom, dom))
+    roof["traffic"] = TRAFFIC["c4"].get(dom)
     gbs = step_bytes / (ms * 1e-3) / 1e9
 
     def cpu():
