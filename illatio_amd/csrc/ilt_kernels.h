@@ -54,6 +54,7 @@ struct IltGemvParams {
   int nbatches;              // batches of rows in the launch (per group, per grid y; set at launch)
   int wgs_per_group;         // grouped rows: workgroups sharing one group (set at launch)
   int batch;                 // rows a wave takes through phase A at a time (set at launch)
+  int region;                // streamed variant: bytes of LDS per wave for its rows (set at launch)
   uint32_t s_magic;          // ceil(2^32 / blocks per row)
 };
 

@@ -308,9 +308,10 @@ __device__ __forceinline__ int ilt_or16(int v) {
 }
 
 // This lane's 16 values of the block its 16-lane row takes in pass PASS (zeros past the end).
+template <int NW = kWaves>
 __device__ __forceinline__ void load_q8k_pass(const float* __restrict__ x, int nblk, int pass, float4* t) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, g = lane >> 4, l = lane & 15;
-  const int b = 4 * wave + 4 * kWaves * pass + g;
+  const int b = 4 * wave + 4 * NW * pass + g;
 #pragma unroll
   for (int i = 0; i < 4; i++) t[i] = b < nblk ? *(const float4*)(x + b * 256 + 4 * (l + 16 * i)) : make_float4(0.f, 0.f, 0.f, 0.f);
 }
@@ -319,22 +320,23 @@ __device__ __forceinline__ void load_q8k_pass(const float* __restrict__ x, int n
 // NW: x is weighted first as rmsnorm! weights it, (x * nscale) * nw (model.lisp:215-216), NFIRST
 // being nw's first pass; H: those floats are stored as well.  PITCH: bytes from one block's
 // quants to the next's at LXQ.
-template <int PITCH>
+// NPRE: FIRST holds the first NPRE passes' values (four float4 each), the caller's loads.
+template <int PITCH, int NPRE = 1, int NW = kWaves>
 __device__ __forceinline__ void stage_q8k_from_f32(const float* __restrict__ x, int nblk, i8* lxq, float* lxs, int* lbs, const float4* first,
                                                    const float* __restrict__ nw = nullptr, const float4* nfirst = nullptr,
                                                    float nscale = 1.0f, float* __restrict__ h = nullptr) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, g = lane >> 4, l = lane & 15;
-  int pass = 0;
-  for (int b0 = 4 * wave; b0 < nblk; b0 += 4 * kWaves, pass++) {
-    const int b = b0 + g;
+  const int npass = (nblk + 4 * NW - 1) / (4 * NW);
+  auto one_pass = [&](int pass, const float4* pre) {
+    const int b = 4 * wave + 4 * NW * pass + g;
     const bool live = b < nblk;
     float4 t4[4];
-    if (pass == 0) { t4[0] = first[0]; t4[1] = first[1]; t4[2] = first[2]; t4[3] = first[3]; }
-    else load_q8k_pass(x, nblk, pass, t4);
+    if (pre) { t4[0] = pre[0]; t4[1] = pre[1]; t4[2] = pre[2]; t4[3] = pre[3]; }
+    else load_q8k_pass<NW>(x, nblk, pass, t4);
     if (nw) {
       float4 n4[4];
-      if (pass == 0) { n4[0] = nfirst[0]; n4[1] = nfirst[1]; n4[2] = nfirst[2]; n4[3] = nfirst[3]; }
-      else load_q8k_pass(nw, nblk, pass, n4);
+      if (pass == 0 && nfirst) { n4[0] = nfirst[0]; n4[1] = nfirst[1]; n4[2] = nfirst[2]; n4[3] = nfirst[3]; }
+      else load_q8k_pass<NW>(nw, nblk, pass, n4);
 #pragma unroll
       for (int i = 0; i < 4; i++) {
         t4[i] = make_float4((t4[i].x * nscale) * n4[i].x, (t4[i].y * nscale) * n4[i].y, (t4[i].z * nscale) * n4[i].z, (t4[i].w * nscale) * n4[i].w);
@@ -357,8 +359,8 @@ __device__ __forceinline__ void stage_q8k_from_f32(const float* __restrict__ x, 
       idx = hit ? 4 * (l + 16 * (k >> 2)) + (k & 3) : idx;
       val = hit ? v[k] : val;
     }
-    const int first = ilt_min16(idx);
-    const float mx = __int_as_float(ilt_or16(idx == first ? __float_as_int(val) : 0));
+    const int firstpos = ilt_min16(idx);
+    const float mx = __int_as_float(ilt_or16(idx == firstpos ? __float_as_int(val) : 0));
     const bool nz = amax != 0.0f;
     const float iscale = nz ? -127.0f / mx : 0.0f;
     const float d = nz ? 1.0f / iscale : 0.0f;
@@ -375,7 +377,11 @@ __device__ __forceinline__ void stage_q8k_from_f32(const float* __restrict__ x, 
       }
     }
     if (live && l == 0) lxs[b] = d;
-  }
+  };
+#pragma unroll
+  for (int pass = 0; pass < NPRE; pass++)
+    if (pass < npass) one_pass(pass, first + 4 * pass);
+  for (int pass = NPRE; pass < npass; pass++) one_pass(pass, nullptr);
 }
 
 // Q8_0 (quantize-q8!, tensor.lisp:245-262): 8 lanes a block of 32.  XSUM: each block's sum of
@@ -629,6 +635,165 @@ __global__ __launch_bounds__(kThreads) void gemv_kernel(IltGemvParams p) {
   asm volatile("" :: "v"(warm[0]), "v"(warm[1]), "v"(warm[2]), "v"(warm[3]));
 }
 
+// ---- the streamed variant: Q4_K / Q6_K matrices of up to ~100 KB per CU ----------------------------
+// A mid-size product (6-28 MB) is over before its loop's load -> use -> load chain has made a few
+// round trips to memory: its time is latency, not bytes.  Here every wave asks for its whole
+// share of the rows at once, as direct loads from global memory into its own piece of LDS,
+// before anything else but the activations' loads (which must go first: loads return in the
+// order they were issued); the matrix streams in at the memory's rate while the activations
+// are quantized, and the blocks' terms are then formed from LDS.  One workgroup a CU, one
+// batch of rows a wave.
+template <int FMT> struct LdsBlk;      // a block in LDS: LB bytes, PPB pieces of 16 bytes
+template <> struct LdsBlk<ILT_Q4_K> { static constexpr int LB = 144, PPB = 9; };
+// Q6_K's 212 bytes are spread to 224 so that every piece stays 16-byte aligned in LDS; the last
+// piece is bytes 196..211 of the block (not 208..223, which would read past a matrix's end):
+// the scale d lands at 220.
+template <> struct LdsBlk<ILT_Q6_K> { static constexpr int LB = 224, PPB = 14; };
+
+// Returns the number of load instructions issued (the same in every lane).
+template <int FMT>
+__device__ __forceinline__ int stream_run(const u8* w, long row0, int nrows, int S, long row_bytes, u8* lds_run, int lane) {
+  const u8* src = (const u8*)ilt_uniform_ptr(w + row0 * row_bytes);
+  const int npieces = __builtin_amdgcn_readfirstlane(nrows * S * LdsBlk<FMT>::PPB);
+  const int nfull = npieces >> 6, tail = npieces & 63;
+  // this lane's piece of the first instruction; each further instruction is 64 pieces on
+  u32 blk = ((u32)lane * 9363u) >> 17, pc = (u32)lane - 14 * blk;        // Q6_K: lane / 14, lane % 14
+  u32 off = (u32)lane * 16;                                              // Q4_K: the run as it is
+  for (int i = 0; i < nfull; i++) {
+    if (FMT == ILT_Q6_K) off = blk * ILT_Q6K_STRIDE + (pc == 13 ? 196u : 16 * pc);
+    ilt_g2lds16(src + off, lds_run + i * 1024);
+    if (FMT == ILT_Q6_K) { pc += 8; blk += 4; if (pc >= 14) { pc -= 14; blk += 1; } }      // 64 = 4 * 14 + 8
+    else off += 1024;
+  }
+  if (tail) {
+    if (FMT == ILT_Q6_K) off = blk * ILT_Q6K_STRIDE + (pc == 13 ? 196u : 16 * pc);
+    if (lane < tail) ilt_g2lds16(src + off, lds_run + nfull * 1024);     // the lanes past the end load nothing
+  }
+  return nfull + (tail ? 1 : 0);
+}
+
+template <int FMT> __device__ __forceinline__ void load_raw_lds(Raw<FMT>& r, const u8* run, u32 f, int j);
+template <> __device__ __forceinline__ void load_raw_lds<ILT_Q4_K>(Raw<ILT_Q4_K>& r, const u8* run, u32 f, int j) {
+  const u8* b = run + f * LdsBlk<ILT_Q4_K>::LB;
+  r.hdr = ilt_lds_ld16(b);
+  r.qa = ilt_lds_ld16(b + 16 + 32 * j);
+  r.qb = ilt_lds_ld16(b + 32 + 32 * j);
+}
+template <> __device__ __forceinline__ void load_raw_lds<ILT_Q6_K>(Raw<ILT_Q6_K>& r, const u8* run, u32 f, int j) {
+  const u8* b = run + f * LdsBlk<ILT_Q6_K>::LB;
+  const int c = j >> 1, pp = j & 1;
+  r.ql0 = ilt_lds_ld16(b + 64 * c + 32 * pp);
+  r.ql1 = ilt_lds_ld16(b + 64 * c + 32 * pp + 16);
+  r.qh0 = ilt_lds_ld16(b + 128 + 32 * c);
+  r.qh1 = ilt_lds_ld16(b + 128 + 32 * c + 16);
+  r.sc = ilt_lds_ld16(b + 192);
+  r.d = *(const ILT_LDS u16*)(b + 220);
+}
+
+// A wave's run of nrows*S blocks, in LDS: terms into t.
+template <int FMT>
+__device__ __forceinline__ void wave_rows_lds(const u8* run, int nrows, int S, u32 s_magic, const Lds& L, float* t, int lane) {
+  using F = Fmt<FMT>;
+  constexpr int GPW = ILT_WAVE / F::LPB;
+  const int j = lane % F::LPB, gl = lane / F::LPB;
+  const int nblk = nrows * S;
+  for (int f = gl; f < nblk; f += GPW) {
+    Raw<FMT> r;
+    load_raw_lds<FMT>(r, run, f, j);
+    const int s_ = S > 1 ? f - (int)__umulhi((u32)f, s_magic) * S : 0;
+    block_terms<FMT>(r, s_, j, L, t + (long)f * F::TERMS);
+  }
+}
+
+// 16 waves a workgroup (four a SIMD): a wave's share is a row or a few, the activations are
+// quantized in one pass (a 16-lane row a block: 64 blocks, cols <= 16384), and the waves' chains
+// of dependent instructions hide one another.
+constexpr int kStreamWaves = 16, kStreamThreads = 64 * kStreamWaves;
+
+// FSET: ILT_Q4_K, ILT_Q6_K or 0 (mixed).  p.batch = the most rows a wave takes; p.region = bytes of LDS
+// per wave for its rows (both matrices' when glu).
+template <int FSET>
+__global__ __launch_bounds__(kStreamThreads) void gemv_stream_kernel(IltGemvParams p) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  const int S = p.cols / 256;
+  i8* lxq = (i8*)smem;
+  int* lbs = (int*)(smem + S * XP);
+  float* lxs = (float*)(lbs + p.cols / 16);
+  float* terms = (float*)(((uintptr_t)(lxs + S) + 15) & ~(uintptr_t)15);
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);     // the same in every lane, said so
+  const int tpr = S * 2, nglu = p.glu ? 2 : 1;
+  float* tw = terms + (long)wave * p.batch * tpr * nglu;
+  u8* region = (u8*)(terms + (long)kStreamWaves * p.batch * tpr * nglu) + (long)wave * p.region;
+  const int wid = wave * gridDim.x + blockIdx.x;        // consecutive batches on different CUs
+
+  // 1. the activations' loads
+  float4 xall[4];
+  if (p.xf) load_q8k_pass<kStreamWaves>(p.xf, S, 0, xall);
+  // 2. this wave's rows, all of them
+  int mi = 0, nrows = 0; long row0 = 0;
+  const bool live = wid < p.nbatches;
+  if (live) {
+    if (!p.glu) while (mi + 1 < p.nmat && wid >= p.mat[mi + 1].batch0) mi++;
+    const int bl = wid - p.mat[mi].batch0, rq = p.mat[mi].rq, rr = p.mat[mi].rr;
+    row0 = (long)bl * rq + min(bl, rr);
+    nrows = rq + (bl < rr ? 1 : 0);
+  }
+  const IltGemvMat& m = p.mat[mi];
+  const int fmt = FSET != 0 ? FSET : m.fmt;
+  const int ufmt = FSET != 0 ? FSET : p.mat[1].fmt;
+  u8* region_up = region + p.region / 2;
+  int nup = 0;              // load instructions of the up matrix's rows: the last ones issued
+  if (live) {
+    if (fmt == ILT_Q4_K) stream_run<ILT_Q4_K>(m.w, row0, nrows, S, m.row_bytes, region, lane);
+    else stream_run<ILT_Q6_K>(m.w, row0, nrows, S, m.row_bytes, region, lane);
+    if (p.glu) {
+      if (ufmt == ILT_Q4_K) nup = stream_run<ILT_Q4_K>(p.mat[1].w, row0, nrows, S, p.mat[1].row_bytes, region_up, lane);
+      else nup = stream_run<ILT_Q6_K>(p.mat[1].w, row0, nrows, S, p.mat[1].row_bytes, region_up, lane);
+    }
+  }
+  // 3. the activations into LDS
+  if (p.xf) {
+    stage_q8k_from_f32<XP, 1, kStreamWaves>(p.xf, S, lxq, lxs, lbs, xall);
+  } else {
+    for (int i = threadIdx.x; i < S * 16; i += kStreamThreads)
+      *(int4*)(lxq + (i >> 4) * XP + 16 * (i & 15)) = *(const int4*)(p.xq + 16 * i);
+    for (int i = threadIdx.x; i < S; i += kStreamThreads) lxs[i] = p.xs[i];
+    for (int i = threadIdx.x; i < p.cols / 16; i += kStreamThreads) lbs[i] = p.bsums[i];
+  }
+  // The gate's rows (or the only matrix's) have landed when at most the up matrix's loads are
+  // still on their way: they return in the order they were issued.
+  if (nup == 0 || nup > 12) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  else if (nup <= 4) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+  else if (nup <= 8) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+  else asm volatile("s_waitcnt vmcnt(12)" ::: "memory");
+  ilt_barrier_lds();        // the activations are staged (no fence: the up matrix's loads stay in flight)
+  if (!live) return;
+
+  const Lds L = { lxq, lxs, lbs, nullptr };
+  if (fmt == ILT_Q4_K) wave_rows_lds<ILT_Q4_K>(region, nrows, S, p.s_magic, L, tw, lane);
+  else wave_rows_lds<ILT_Q6_K>(region, nrows, S, p.s_magic, L, tw, lane);
+  if (p.glu) {
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    if (ufmt == ILT_Q4_K) wave_rows_lds<ILT_Q4_K>(region_up, nrows, S, p.s_magic, L, tw + (long)p.batch * tpr, lane);
+    else wave_rows_lds<ILT_Q6_K>(region_up, nrows, S, p.s_magic, L, tw + (long)p.batch * tpr, lane);
+  }
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  if (lane < nrows) {
+    float v = sum_any(fmt, tw + (long)lane * S * (fmt == ILT_Q4_K ? 2 : 1), S);
+    const long r = row0 + lane;
+    if (p.glu) {
+      const float uv = sum_any(ufmt, tw + (long)p.batch * tpr + (long)lane * S * (ufmt == ILT_Q4_K ? 2 : 1), S);
+      m.y[r] = dense_glu(v, uv);
+    } else {
+      if (m.bias) v = v + m.bias[r];
+      if (p.acc) v = m.y[r] + v;
+      m.y[r] = v;
+    }
+  }
+}
+
 // rmsnorm! and the quantizer in one launch, a workgroup a row of DIM floats (the reference's
 // rmsnorm_q8, cuda/dense.cu:144-160): H (unless null) gets the floats, XQ / XS the quants and
 // scales -- Q8_0 blocks with XSUM (unless null) their sums, or with K set Q8_K blocks with
@@ -687,9 +852,77 @@ int resident_per_cu(int fset, size_t smem) {
 
 }  // namespace
 
+// The streamed variant's launch, when the product qualifies: dense Q4_K / Q6_K matrices, one
+// activation vector, at most 16 rows a wave over the 4096 waves of one workgroup per CU, and
+// everything within a CU's LDS.  Returns hipErrorNotSupported when it does not qualify.
+static hipError_t gemv_stream_launch(IltGemvParams& p, int fset, hipStream_t st) {
+  const char* force = getenv("ILT_GEMV_STREAM");          // "0": never (tests)
+  if (force && atoi(force) == 0) return hipErrorNotSupported;
+  if (!(fset == 0 || fset == ILT_Q4_K || fset == ILT_Q6_K) || p.ptrs || p.group_rows > 0 || p.glu > 1 || p.norm_w)
+    return hipErrorNotSupported;
+  const int S = p.cols / 256;
+  if (p.xf && S > 4 * kStreamWaves) return hipErrorNotSupported;
+  const int nm = p.glu ? 1 : p.nmat;
+  long total_rows = 0, bytes = 0;
+  for (int i = 0; i < nm; i++) { total_rows += p.mat[i].rows; bytes += (long)p.mat[i].rows * p.mat[i].row_bytes; }
+  constexpr int kWavesAll = 256 * kStreamWaves;
+  if (total_rows > 16L * kWavesAll || bytes * (p.glu ? 2 : 1) < (2L << 20)) return hipErrorNotSupported;
+  // every wave one batch: the waves are shared out over the matrices by rows, never more than there are
+  const int nb_total = (int)min((long)kWavesAll, total_rows);
+  int nb = 0, batch = 1, given = 0;
+  for (int i = 0; i < nm; i++) {
+    int nbi = (int)((long)nb_total * p.mat[i].rows / total_rows);
+    if (nbi < 1) nbi = 1;
+    p.mat[i].nbat = nbi; given += nbi;
+  }
+  for (int i = 0; given < nb_total; i = (i + 1) % nm)          // the rounding's leftovers, where rows allow
+    if (p.mat[i].nbat < p.mat[i].rows) { p.mat[i].nbat++; given++; }
+  if (given > kWavesAll) return hipErrorNotSupported;
+  for (int i = 0; i < p.nmat; i++) {
+    if (i >= nm) { p.mat[i].batch0 = 0; p.mat[i].nbat = p.mat[0].nbat; p.mat[i].rq = p.mat[0].rq; p.mat[i].rr = p.mat[0].rr; continue; }
+    p.mat[i].batch0 = nb;
+    p.mat[i].rq = p.mat[i].rows / p.mat[i].nbat;
+    p.mat[i].rr = p.mat[i].rows % p.mat[i].nbat;
+    batch = max(batch, p.mat[i].rq + (p.mat[i].rr ? 1 : 0));
+    nb += p.mat[i].nbat;
+  }
+  if (batch > 16) return hipErrorNotSupported;
+  p.nbatches = nb;
+  p.batch = batch;
+  const int nglu = p.glu ? 2 : 1;
+  const int lb = fset == ILT_Q4_K ? 144 : 224;                        // Q6_K's spread blocks at worst
+  const long one = (long)batch * S * lb;                              // a wave's rows of one matrix
+  p.region = (int)(one * nglu);
+  const size_t smem = (size_t)S * XP + (size_t)p.cols / 16 * 4 + (size_t)S * 4 + 16 + (size_t)kStreamWaves * batch * S * 2 * 4 * nglu +
+                      (size_t)kStreamWaves * p.region;
+  if (smem > 156 * 1024) return hipErrorNotSupported;
+  p.s_magic = (uint32_t)(0x100000000ULL / (uint64_t)S) + 1;
+  static bool attr_set[8] = {};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 8) dev = 0;
+  if (!attr_set[dev]) {            // more dynamic LDS than the default 64 KB: asked for once per device
+    hipError_t e = hipFuncSetAttribute((const void*)gemv_stream_kernel<0>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+    if (e == hipSuccess) e = hipFuncSetAttribute((const void*)gemv_stream_kernel<ILT_Q4_K>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+    if (e == hipSuccess) e = hipFuncSetAttribute((const void*)gemv_stream_kernel<ILT_Q6_K>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+    if (e != hipSuccess) { (void)hipGetLastError(); return hipErrorNotSupported; }
+    attr_set[dev] = true;
+  }
+  const dim3 grid(min(256, nb));                                      // wave w of workgroup g takes batch w * grid + g
+  switch (fset) {
+    case 0: hipLaunchKernelGGL(gemv_stream_kernel<0>, grid, dim3(kStreamThreads), smem, st, p); break;
+    case ILT_Q4_K: hipLaunchKernelGGL(gemv_stream_kernel<ILT_Q4_K>, grid, dim3(kStreamThreads), smem, st, p); break;
+    default: hipLaunchKernelGGL(gemv_stream_kernel<ILT_Q6_K>, grid, dim3(kStreamThreads), smem, st, p); break;
+  }
+  return hipGetLastError();
+}
+
 hipError_t ilt_gemv_launch(IltGemvParams& p, int nz, hipStream_t st) {
   int fset = p.mat[0].fmt;
   for (int i = 1; i < p.nmat; i++) if (p.mat[i].fmt != fset) fset = 0;
+  if (nz == 1) {
+    const hipError_t e = gemv_stream_launch(p, fset, st);
+    if (e != hipErrorNotSupported) return e;
+  }
   const bool q8 = fset == ILT_Q8_0;
   const int S = q8 ? p.cols / 32 : p.cols / 256;
   const int nm = p.glu ? 1 : p.nmat;

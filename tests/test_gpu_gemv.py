@@ -376,3 +376,57 @@ def test_norm_inside_the_product_bit_exact(dev, kind):
         hip.hip_free(nwb)
         for m in ms:
             m.free()
+
+
+# ---- the streamed variant of the decode product (mid-size Q4_K / Q6_K matrices) -----------------
+
+@pytest.mark.parametrize("stream", ["1", "0"])        # chosen by shape (these shapes qualify) / never
+def test_streamed_products_bit_exact(dev, monkeypatch, stream):
+    """Products of 2 MB and more over one activation vector take the variant that streams every
+    wave's rows into LDS; with it and without it the bits are the oracle's: float and
+    quantized activations, one matrix, Q/K/V (Q4_K and Q6_K mixed), gate/up, bias and acc,
+    ragged row counts, few and many rows per wave."""
+    from illatio_amd import dense, hip
+    if stream == "0":
+        monkeypatch.setenv("ILT_GEMV_STREAM", "0")
+    else:
+        monkeypatch.delenv("ILT_GEMV_STREAM", raising=False)
+    rng = synth.make_rng(4242)
+    for qtype, rows, cols in ((synth.Q4_K, 2560, 4096), (synth.Q6_K, 2560, 9728), (synth.Q6_K, 1030, 2560),
+                              (synth.Q4_K, 16384, 1024), (synth.Q4_K, 3000, 12288), (synth.Q6_K, 9000, 256)):
+        w = synth.weights(qtype, rows, cols, rng)
+        x = special_activations(cols, rng)
+        bias = synth.activations(rows, rng)
+        m = upload(dev, qtype, rows, cols, w)
+        xb, bb, y = hip.hip_upload_new(dev, x), hip.hip_upload_new(dev, bias), hip.hip_alloc(dev, 4 * rows)
+        want = orc.matmul(qtype, w, rows, cols, x)
+        dense.mv_multi(dev, [(m, y, None)], xf=xb)
+        assert np.array_equal(bits(hip.hip_floats(y, rows)), bits(want)), (qtype, rows, cols, "float x")
+        act = dense.QAct(dev, 1, cols, ("q8k",))
+        dense.quantize_act(dev, xb, act)
+        dense.mv_multi(dev, [(m, y, bb)], act, acc=True)
+        assert np.array_equal(bits(hip.hip_floats(y, rows)), bits(want + (want + bias))), (qtype, rows, cols, "quantized x, bias, acc")
+        for b in (xb, bb, y):
+            hip.hip_free(b)
+        act.free(); m.free()
+    # Q/K/V of a layer (two Q4_K and a Q6_K matrix in one launch) and its gate/up with the gated activation
+    cols = 2560
+    shape = [(synth.Q4_K, 4096), (synth.Q4_K, 1024), (synth.Q6_K, 1024)]
+    ws = [synth.weights(t, r, cols, rng) for t, r in shape]
+    ms = [upload(dev, t, r, cols, w) for (t, r), w in zip(shape, ws)]
+    x = synth.activations(cols, rng)
+    xb = hip.hip_upload_new(dev, x)
+    ys = [hip.hip_alloc(dev, 4 * r) for _, r in shape]
+    dense.mv_multi(dev, [(m, y, None) for m, y in zip(ms, ys)], xf=xb)
+    for (t, r), w, y in zip(shape, ws, ys):
+        assert np.array_equal(bits(hip.hip_floats(y, r)), bits(orc.matmul(t, w, r, cols, x))), ("qkv", t)
+    gw, uw = synth.weights(synth.Q4_K, 9728, cols, rng), synth.weights(synth.Q6_K, 9728, cols, rng)
+    gm, um = upload(dev, synth.Q4_K, 9728, cols, gw), upload(dev, synth.Q6_K, 9728, cols, uw)
+    fa = hip.hip_alloc(dev, 4 * 9728)
+    dense.glu_mul(dev, gm, um, None, fa, xf=xb)
+    want = orc.swiglu(orc.matmul(synth.Q4_K, gw, 9728, cols, x), orc.matmul(synth.Q6_K, uw, 9728, cols, x))
+    assert np.array_equal(bits(hip.hip_floats(fa, 9728)), bits(want)), "glu"
+    for b in [xb, fa] + ys:
+        hip.hip_free(b)
+    for m in ms + [gm, um]:
+        m.free()
