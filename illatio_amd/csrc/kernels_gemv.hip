@@ -316,6 +316,17 @@ __device__ __forceinline__ void load_q8k_pass(const float* __restrict__ x, int n
   for (int i = 0; i < 4; i++) t[i] = b < nblk ? *(const float4*)(x + b * 256 + 4 * (l + 16 * i)) : make_float4(0.f, 0.f, 0.f, 0.f);
 }
 
+// The same without the branch: a lane whose block does not exist reads the last block's values
+// instead (the quantizer stores nothing for such a lane).  A conditional load makes the compiler
+// wait for it at the join, before whatever the caller wanted to issue next.
+template <int NW = kWaves>
+__device__ __forceinline__ void load_q8k_pass_clamped(const float* __restrict__ x, int nblk, int pass, float4* t) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, g = lane >> 4, l = lane & 15;
+  const int b = min(4 * wave + 4 * NW * pass + g, nblk - 1);
+#pragma unroll
+  for (int i = 0; i < 4; i++) t[i] = *(const float4*)(x + b * 256 + 4 * (l + 16 * i));
+}
+
 // FIRST: the first pass's values, loaded by the caller ahead of time (load_q8k_pass(.., 0, ..)).
 // NW: x is weighted first as rmsnorm! weights it, (x * nscale) * nw (model.lisp:215-216), NFIRST
 // being nw's first pass; H: those floats are stored as well.  PITCH: bytes from one block's
@@ -325,9 +336,10 @@ template <int PITCH, int NPRE = 1, int NW = kWaves>
 __device__ __forceinline__ void stage_q8k_from_f32(const float* __restrict__ x, int nblk, i8* lxq, float* lxs, int* lbs, const float4* first,
                                                    const float* __restrict__ nw = nullptr, const float4* nfirst = nullptr,
                                                    float nscale = 1.0f, float* __restrict__ h = nullptr) {
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, g = lane >> 4, l = lane & 15;
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), g = lane >> 4, l = lane & 15;
   const int npass = (nblk + 4 * NW - 1) / (4 * NW);
   auto one_pass = [&](int pass, const float4* pre) {
+    if (4 * wave + 4 * NW * pass >= nblk) return;        // none of this wave's four blocks exists
     const int b = 4 * wave + 4 * NW * pass + g;
     const bool live = b < nblk;
     float4 t4[4];
@@ -705,10 +717,12 @@ __device__ __forceinline__ void wave_rows_lds(const u8* run, int nrows, int S, u
   }
 }
 
-// 16 waves a workgroup (four a SIMD): a wave's share is a row or a few, the activations are
-// quantized in one pass (a 16-lane row a block: 64 blocks, cols <= 16384), and the waves' chains
-// of dependent instructions hide one another.
-constexpr int kStreamWaves = 16, kStreamThreads = 64 * kStreamWaves;
+// 16 waves a workgroup (four a SIMD), in two roles.  Waves 0-3 load and quantize the activations
+// and have no rows; waves 4-15 send off the loads of their rows at once and wait.  So the
+// quantizer's chain of dependent instructions runs while the matrix streams in, and no wave
+// has activation loads queued ahead of matrix loads (loads return in the order issued: waiting
+// for the first would mean counting the second, whose number is not known at compile time).
+constexpr int kStreamWaves = 16, kStreamThreads = 64 * kStreamWaves, kStagers = 4, kRowWaves = kStreamWaves - kStagers;
 
 // FSET: ILT_Q4_K, ILT_Q6_K or 0 (mixed).  p.batch = the most rows a wave takes; p.region = bytes of LDS
 // per wave for its rows (both matrices' when glu).
@@ -722,13 +736,27 @@ __global__ __launch_bounds__(kStreamThreads) void gemv_stream_kernel(IltGemvPara
   float* terms = (float*)(((uintptr_t)(lxs + S) + 15) & ~(uintptr_t)15);
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);     // the same in every lane, said so
   const int tpr = S * 2, nglu = p.glu ? 2 : 1;
-  float* tw = terms + (long)wave * p.batch * tpr * nglu;
-  u8* region = (u8*)(terms + (long)kStreamWaves * p.batch * tpr * nglu) + (long)wave * p.region;
-  const int wid = wave * gridDim.x + blockIdx.x;        // consecutive batches on different CUs
 
-  // 1. the activations' loads
-  float4 xall[4];
-  if (p.xf) load_q8k_pass<kStreamWaves>(p.xf, S, 0, xall);
+  // 1. the activations into LDS, by the first four waves
+  if (wave < kStagers) {
+    if (p.xf) {
+      float4 xall[4];
+      load_q8k_pass_clamped<kStagers>(p.xf, S, 0, xall);
+      stage_q8k_from_f32<XP, 1, kStagers>(p.xf, S, lxq, lxs, lbs, xall);
+    } else {
+      for (int i = threadIdx.x; i < S * 16; i += 64 * kStagers)
+        *(int4*)(lxq + (i >> 4) * XP + 16 * (i & 15)) = *(const int4*)(p.xq + 16 * i);
+      for (int i = threadIdx.x; i < S; i += 64 * kStagers) lxs[i] = p.xs[i];
+      for (int i = threadIdx.x; i < p.cols / 16; i += 64 * kStagers) lbs[i] = p.bsums[i];
+    }
+    ilt_barrier_lds();
+    return;
+  }
+  const int rw = wave - kStagers;
+  float* tw = terms + (long)rw * p.batch * tpr * nglu;
+  u8* region = (u8*)(terms + (long)kRowWaves * p.batch * tpr * nglu) + (long)rw * p.region;
+  const int wid = rw * gridDim.x + blockIdx.x;          // consecutive batches on different CUs
+
   // 2. this wave's rows, all of them
   int mi = 0, nrows = 0; long row0 = 0;
   const bool live = wid < p.nbatches;
@@ -751,23 +779,17 @@ __global__ __launch_bounds__(kStreamThreads) void gemv_stream_kernel(IltGemvPara
       else nup = stream_run<ILT_Q6_K>(p.mat[1].w, row0, nrows, S, p.mat[1].row_bytes, region_up, lane);
     }
   }
-  // 3. the activations into LDS
-  if (p.xf) {
-    stage_q8k_from_f32<XP, 1, kStreamWaves>(p.xf, S, lxq, lxs, lbs, xall);
-  } else {
-    for (int i = threadIdx.x; i < S * 16; i += kStreamThreads)
-      *(int4*)(lxq + (i >> 4) * XP + 16 * (i & 15)) = *(const int4*)(p.xq + 16 * i);
-    for (int i = threadIdx.x; i < S; i += kStreamThreads) lxs[i] = p.xs[i];
-    for (int i = threadIdx.x; i < p.cols / 16; i += kStreamThreads) lbs[i] = p.bsums[i];
-  }
+  // The barrier is for the activations only, so it comes before this wave waits for its rows (no
+  // fence: the loads stay in flight): a wave whose rows land early starts on them while the
+  // other waves' rows are still streaming in.
+  ilt_barrier_lds();
+  if (!live) return;
   // The gate's rows (or the only matrix's) have landed when at most the up matrix's loads are
   // still on their way: they return in the order they were issued.
   if (nup == 0 || nup > 12) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   else if (nup <= 4) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
   else if (nup <= 8) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
   else asm volatile("s_waitcnt vmcnt(12)" ::: "memory");
-  ilt_barrier_lds();        // the activations are staged (no fence: the up matrix's loads stay in flight)
-  if (!live) return;
 
   const Lds L = { lxq, lxs, lbs, nullptr };
   if (fmt == ILT_Q4_K) wave_rows_lds<ILT_Q4_K>(region, nrows, S, p.s_magic, L, tw, lane);
@@ -853,7 +875,7 @@ int resident_per_cu(int fset, size_t smem) {
 }  // namespace
 
 // The streamed variant's launch, when the product qualifies: dense Q4_K / Q6_K matrices, one
-// activation vector, at most 16 rows a wave over the 4096 waves of one workgroup per CU, and
+// activation vector, at most 16 rows a wave over the 3072 row waves of one workgroup per CU, and
 // everything within a CU's LDS.  Returns hipErrorNotSupported when it does not qualify.
 static hipError_t gemv_stream_launch(IltGemvParams& p, int fset, hipStream_t st) {
   const char* force = getenv("ILT_GEMV_STREAM");          // "0": never (tests)
@@ -861,11 +883,11 @@ static hipError_t gemv_stream_launch(IltGemvParams& p, int fset, hipStream_t st)
   if (!(fset == 0 || fset == ILT_Q4_K || fset == ILT_Q6_K) || p.ptrs || p.group_rows > 0 || p.glu > 1 || p.norm_w)
     return hipErrorNotSupported;
   const int S = p.cols / 256;
-  if (p.xf && S > 4 * kStreamWaves) return hipErrorNotSupported;
+  if (S > 64) return hipErrorNotSupported;
   const int nm = p.glu ? 1 : p.nmat;
   long total_rows = 0, bytes = 0;
   for (int i = 0; i < nm; i++) { total_rows += p.mat[i].rows; bytes += (long)p.mat[i].rows * p.mat[i].row_bytes; }
-  constexpr int kWavesAll = 256 * kStreamWaves;
+  constexpr int kWavesAll = 256 * kRowWaves;
   if (total_rows > 16L * kWavesAll || bytes * (p.glu ? 2 : 1) < (2L << 20)) return hipErrorNotSupported;
   // every wave one batch: the waves are shared out over the matrices by rows, never more than there are
   const int nb_total = (int)min((long)kWavesAll, total_rows);
@@ -893,8 +915,8 @@ static hipError_t gemv_stream_launch(IltGemvParams& p, int fset, hipStream_t st)
   const int lb = fset == ILT_Q4_K ? 144 : 224;                        // Q6_K's spread blocks at worst
   const long one = (long)batch * S * lb;                              // a wave's rows of one matrix
   p.region = (int)(one * nglu);
-  const size_t smem = (size_t)S * XP + (size_t)p.cols / 16 * 4 + (size_t)S * 4 + 16 + (size_t)kStreamWaves * batch * S * 2 * 4 * nglu +
-                      (size_t)kStreamWaves * p.region;
+  const size_t smem = (size_t)S * XP + (size_t)p.cols / 16 * 4 + (size_t)S * 4 + 16 + (size_t)kRowWaves * batch * S * 2 * 4 * nglu +
+                      (size_t)kRowWaves * p.region;
   if (smem > 156 * 1024) return hipErrorNotSupported;
   p.s_magic = (uint32_t)(0x100000000ULL / (uint64_t)S) + 1;
   static bool attr_set[8] = {};
