@@ -255,6 +255,8 @@ int ilt_mv_multi(uint64_t stream, int nmat, const ilt_mv_desc* descs, int cols, 
   return gemv_multi(stream, nmat, fmts, ws, wds, ys, bs, rows, cols, xq, xs, bsums, xf, f16_scale, acc, glu, 0);
 }
 
+uint64_t ilt_streamed_launches(void) { return (uint64_t)ilt_k_streamed_launches(); }
+
 int ilt_mv_multi_norm(uint64_t stream, int nmat, const ilt_mv_desc* descs, int cols, const float* x, const float* norm_w,
                       float eps, int exact_order, int f16_scale, int glu) {
   ILT_REQUIRE(descs && nmat >= 1 && nmat <= 4 && x && norm_w);

@@ -61,6 +61,8 @@ struct IltGemvParams {
 // The kernel is chosen by the matrices' formats (mat[i].fmt): one format, or Q4_K and Q6_K mixed.
 hipError_t ilt_gemv_launch(IltGemvParams& p, int nz, hipStream_t st);
 
+unsigned long long ilt_k_streamed_launches();      // decode products launched as the streamed variant so far (diagnostic)
+
 hipError_t ilt_k_quant_q8(const float* x, int8_t* xq, float* xs, int* xsum, long long nblocks, int f16_scale, hipStream_t st);
 hipError_t ilt_k_quant_q8k(const float* x, int8_t* xq, float* xd, int* bsums, long long nblocks, hipStream_t st);
 // rmsnorm! then quantize-q8! (k 0; xsum may be null) or quantize-q8k! (k 1), a row of DIM floats a workgroup

@@ -724,6 +724,32 @@ __device__ __forceinline__ void wave_rows_lds(const u8* run, int nrows, int S, u
 // for the first would mean counting the second, whose number is not known at compile time).
 constexpr int kStreamWaves = 16, kStreamThreads = 64 * kStreamWaves, kStagers = 4, kRowWaves = kStreamWaves - kStagers;
 
+// rmsnorm!'s scale (see norm_scale) in the streamed kernel: the first kStagers waves hold the
+// squares, the other waves only keep step through the three barriers (always three, whether
+// or not the sum is taken again in the CPU's order, so that they need not know).
+__device__ __forceinline__ float norm_scale_stagers(double part, const float* __restrict__ x, int n, float eps, int seq) {
+  __shared__ double red[kStagers];
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) part += __shfl_xor(part, off);
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = part;
+  ilt_barrier_lds();
+  double sum = red[0];
+#pragma unroll
+  for (int w = 1; w < kStagers; w++) sum += red[w];
+  double v = sum / (double)n + (double)eps;
+  const double slack = v * ((double)(n + 8) * 0x1p-51);
+  const bool again = seq || (float)(v - slack) != (float)(v + slack);       // the same for every thread
+  ilt_barrier_lds();
+  if (again && threadIdx.x == 0) {
+    double s = 0.0;
+    for (int i = 0; i < n; i++) { const float xi = x[i]; s += (double)(xi * xi); }
+    red[0] = s;
+  }
+  ilt_barrier_lds();
+  if (again) v = red[0] / (double)n + (double)eps;
+  return 1.0f / sqrtf((float)v);
+}
+
 // FSET: ILT_Q4_K, ILT_Q6_K or 0 (mixed).  p.batch = the most rows a wave takes; p.region = bytes of LDS
 // per wave for its rows (both matrices' when glu).
 template <int FSET>
@@ -739,7 +765,20 @@ __global__ __launch_bounds__(kStreamThreads) void gemv_stream_kernel(IltGemvPara
 
   // 1. the activations into LDS, by the first four waves
   if (wave < kStagers) {
-    if (p.xf) {
+    if (p.xf && p.norm_w) {
+      float4 xall[4], nall[4];
+      load_q8k_pass<kStagers>(p.xf, S, 0, xall);           // zeros where there is no block: they are squared
+      load_q8k_pass_clamped<kStagers>(p.norm_w, S, 0, nall);
+      double sq = 0.0;
+      for (int pass = 1; pass * 4 * kStagers < S; pass++) {
+        float4 t[4];
+        load_q8k_pass<kStagers>(p.xf, S, pass, t);
+        sq += (sq4(t[0]) + sq4(t[1])) + (sq4(t[2]) + sq4(t[3]));
+      }
+      sq += (sq4(xall[0]) + sq4(xall[1])) + (sq4(xall[2]) + sq4(xall[3]));
+      const float nscale = norm_scale_stagers(sq, p.xf, p.cols, p.eps, p.norm_seq);
+      stage_q8k_from_f32<XP, 1, kStagers>(p.xf, S, lxq, lxs, lbs, xall, p.norm_w, nall, nscale);
+    } else if (p.xf) {
       float4 xall[4];
       load_q8k_pass_clamped<kStagers>(p.xf, S, 0, xall);
       stage_q8k_from_f32<XP, 1, kStagers>(p.xf, S, lxq, lxs, lbs, xall);
@@ -779,6 +818,7 @@ __global__ __launch_bounds__(kStreamThreads) void gemv_stream_kernel(IltGemvPara
       else nup = stream_run<ILT_Q6_K>(p.mat[1].w, row0, nrows, S, p.mat[1].row_bytes, region_up, lane);
     }
   }
+  if (p.norm_w) { ilt_barrier_lds(); ilt_barrier_lds(); ilt_barrier_lds(); }      // in step with norm_scale_stagers
   // The barrier is for the activations only, so it comes before this wave waits for its rows (no
   // fence: the loads stay in flight): a wave whose rows land early starts on them while the
   // other waves' rows are still streaming in.
@@ -877,10 +917,13 @@ int resident_per_cu(int fset, size_t smem) {
 // The streamed variant's launch, when the product qualifies: dense Q4_K / Q6_K matrices, one
 // activation vector, at most 16 rows a wave over the 3072 row waves of one workgroup per CU, and
 // everything within a CU's LDS.  Returns hipErrorNotSupported when it does not qualify.
+static unsigned long long g_streamed_launches = 0;
+unsigned long long ilt_k_streamed_launches() { return g_streamed_launches; }
+
 static hipError_t gemv_stream_launch(IltGemvParams& p, int fset, hipStream_t st) {
   const char* force = getenv("ILT_GEMV_STREAM");          // "0": never (tests)
   if (force && atoi(force) == 0) return hipErrorNotSupported;
-  if (!(fset == 0 || fset == ILT_Q4_K || fset == ILT_Q6_K) || p.ptrs || p.group_rows > 0 || p.glu > 1 || p.norm_w)
+  if (!(fset == 0 || fset == ILT_Q4_K || fset == ILT_Q6_K) || p.ptrs || p.group_rows > 0 || p.glu > 1)
     return hipErrorNotSupported;
   const int S = p.cols / 256;
   if (S > 64) return hipErrorNotSupported;
@@ -923,9 +966,9 @@ static hipError_t gemv_stream_launch(IltGemvParams& p, int fset, hipStream_t st)
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 8) dev = 0;
   if (!attr_set[dev]) {            // more dynamic LDS than the default 64 KB: asked for once per device
-    hipError_t e = hipFuncSetAttribute((const void*)gemv_stream_kernel<0>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-    if (e == hipSuccess) e = hipFuncSetAttribute((const void*)gemv_stream_kernel<ILT_Q4_K>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-    if (e == hipSuccess) e = hipFuncSetAttribute((const void*)gemv_stream_kernel<ILT_Q6_K>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+    hipError_t e = hipFuncSetAttribute((const void*)gemv_stream_kernel<0>, hipFuncAttributeMaxDynamicSharedMemorySize, 158 * 1024);
+    if (e == hipSuccess) e = hipFuncSetAttribute((const void*)gemv_stream_kernel<ILT_Q4_K>, hipFuncAttributeMaxDynamicSharedMemorySize, 158 * 1024);
+    if (e == hipSuccess) e = hipFuncSetAttribute((const void*)gemv_stream_kernel<ILT_Q6_K>, hipFuncAttributeMaxDynamicSharedMemorySize, 158 * 1024);
     if (e != hipSuccess) { (void)hipGetLastError(); return hipErrorNotSupported; }
     attr_set[dev] = true;
   }
@@ -935,6 +978,7 @@ static hipError_t gemv_stream_launch(IltGemvParams& p, int fset, hipStream_t st)
     case ILT_Q4_K: hipLaunchKernelGGL(gemv_stream_kernel<ILT_Q4_K>, grid, dim3(kStreamThreads), smem, st, p); break;
     default: hipLaunchKernelGGL(gemv_stream_kernel<ILT_Q6_K>, grid, dim3(kStreamThreads), smem, st, p); break;
   }
+  g_streamed_launches++;
   return hipGetLastError();
 }
 

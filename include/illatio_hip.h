@@ -170,6 +170,11 @@ int ilt_rmsnorm_q8k(uint64_t stream, const float* x, const float* w, float* h, i
 int ilt_mv_multi_norm(uint64_t stream, int nmat, const ilt_mv_desc* descs, int cols, const float* x, const float* norm_w,
                       float eps, int exact_order, int f16_scale, int glu);
 
+/* Diagnostic: how many decode products this process has launched as the streamed variant (the
+   one that sends every wave's rows to LDS at once; chosen by shape for Q4_K / Q6_K products of
+   2 MB and more whose share fits a CU's LDS).  No counterpart in the reference. */
+uint64_t ilt_streamed_launches(void);
+
 /* The indexed expert products (ds4f.cu:769, 837; CPU: iq2xxs-row-dot, q2k-row-dot,
    iquant.lisp:126-215).  For each z < nz: W = the nrows x ncols matrix at ptrs[z] + add
    (row_bytes apart), x = the Q8_K activations at element z*x_stride, y = dst + z*y_stride.

@@ -387,10 +387,14 @@ def test_streamed_products_bit_exact(dev, monkeypatch, stream):
     quantized activations, one matrix, Q/K/V (Q4_K and Q6_K mixed), gate/up, bias and acc,
     ragged row counts, few and many rows per wave."""
     from illatio_amd import dense, hip
+    import ctypes as C
     if stream == "0":
         monkeypatch.setenv("ILT_GEMV_STREAM", "0")
     else:
         monkeypatch.delenv("ILT_GEMV_STREAM", raising=False)
+    count = hip.lib().ilt_streamed_launches
+    count.restype = C.c_uint64
+    before = count()
     rng = synth.make_rng(4242)
     for qtype, rows, cols in ((synth.Q4_K, 2560, 4096), (synth.Q6_K, 2560, 9728), (synth.Q6_K, 1030, 2560),
                               (synth.Q4_K, 16384, 1024), (synth.Q4_K, 3000, 12288), (synth.Q6_K, 9000, 256)):
@@ -426,7 +430,24 @@ def test_streamed_products_bit_exact(dev, monkeypatch, stream):
     dense.glu_mul(dev, gm, um, None, fa, xf=xb)
     want = orc.swiglu(orc.matmul(synth.Q4_K, gw, 9728, cols, x), orc.matmul(synth.Q6_K, uw, 9728, cols, x))
     assert np.array_equal(bits(hip.hip_floats(fa, 9728)), bits(want)), "glu"
-    for b in [xb, fa] + ys:
+    # the same two launches with rmsnorm! inside: a random row, a row on a rounding tie (the sum is
+    # taken again in the CPU's order), and that order forced
+    nw = (synth.activations(cols, rng) * 0.3 + 1.0).astype(np.float32)
+    nwb = hip.hip_upload_new(dev, nw)
+    for xr, exact_order in ((x, False), (tie_row(cols), False), (x, True)):
+        h = orc.rmsnorm(xr, nw, 1e-6)
+        xrb = hip.hip_upload_new(dev, xr)
+        dense.mv_multi(dev, [(m, y, None) for m, y in zip(ms, ys)], xf=xrb, norm=(nwb, 1e-6), exact_order=exact_order)
+        for (t, r), w, y in zip(shape, ws, ys):
+            assert np.array_equal(bits(hip.hip_floats(y, r)), bits(orc.matmul(t, w, r, cols, h))), ("qkv with norm", t, exact_order)
+        dense.mv_multi(dev, [(gm, fa, None), (um, fa, None)], xf=xrb, norm=(nwb, 1e-6), glu=True, exact_order=exact_order)
+        want = orc.swiglu(orc.matmul(synth.Q4_K, gw, 9728, cols, h), orc.matmul(synth.Q6_K, uw, 9728, cols, h))
+        assert np.array_equal(bits(hip.hip_floats(fa, 9728)), bits(want)), ("glu with norm", exact_order)
+        hip.hip_free(xrb)
+    for b in [xb, fa, nwb] + ys:
         hip.hip_free(b)
     for m in ms + [gm, um]:
         m.free()
+    # 5 shapes x 2 launches + Q/K/V + 3 x Q/K/V with the norm took the streamed variant (9000 x 256 is
+    # under 2 MB; a Q4_K gate with a Q6_K up of 9728 rows does not fit a CU's LDS)
+    assert count() - before == (14 if stream == "1" else 0)
