@@ -331,69 +331,73 @@ __device__ __forceinline__ void load_q8k_pass_clamped(const float* __restrict__ 
 // NW: x is weighted first as rmsnorm! weights it, (x * nscale) * nw (model.lisp:215-216), NFIRST
 // being nw's first pass; H: those floats are stored as well.  PITCH: bytes from one block's
 // quants to the next's at LXQ.
-// NPRE: FIRST holds the first NPRE passes' values (four float4 each), the caller's loads.
-template <int PITCH, int NPRE = 1, int NW = kWaves>
+// One pass: this wave's four blocks 4*wave + 4*NW*pass + (0..3).  PRE: the pass's values, loaded by
+// the caller ahead of time (load_q8k_pass), or null to load them here; NPRE likewise for nw.
+template <int PITCH, int NW>
+__device__ __forceinline__ void q8k_pass(const float* __restrict__ x, int nblk, int pass, const float4* pre, i8* lxq, float* lxs, int* lbs,
+                                         const float* __restrict__ nw, const float4* npre, float nscale, float* __restrict__ h) {
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), g = lane >> 4, l = lane & 15;
+  if (4 * wave + 4 * NW * pass >= nblk) return;        // none of this wave's four blocks exists
+  const int b = 4 * wave + 4 * NW * pass + g;
+  const bool live = b < nblk;
+  float4 t4[4];
+  if (pre) { t4[0] = pre[0]; t4[1] = pre[1]; t4[2] = pre[2]; t4[3] = pre[3]; }
+  else load_q8k_pass<NW>(x, nblk, pass, t4);
+  if (nw) {
+    float4 n4[4];
+    if (npre) { n4[0] = npre[0]; n4[1] = npre[1]; n4[2] = npre[2]; n4[3] = npre[3]; }
+    else load_q8k_pass<NW>(nw, nblk, pass, n4);
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      t4[i] = make_float4((t4[i].x * nscale) * n4[i].x, (t4[i].y * nscale) * n4[i].y, (t4[i].z * nscale) * n4[i].z, (t4[i].w * nscale) * n4[i].w);
+      if (h && live) *(float4*)(h + b * 256 + 4 * (l + 16 * i)) = t4[i];
+    }
+  }
+  float v[16];
+#pragma unroll
+  for (int i = 0; i < 4; i++) { v[4 * i] = t4[i].x; v[4 * i + 1] = t4[i].y; v[4 * i + 2] = t4[i].z; v[4 * i + 3] = t4[i].w; }
+  float a8[8];
+#pragma unroll
+  for (int k = 0; k < 8; k++) a8[k] = fmaxf(fabsf(v[2 * k]), fabsf(v[2 * k + 1]));
+  const float am = fmaxf(fmaxf(fmaxf(a8[0], a8[1]), fmaxf(a8[2], a8[3])), fmaxf(fmaxf(a8[4], a8[5]), fmaxf(a8[6], a8[7])));
+  const float amax = ilt_max16(am);
+  // this lane's first position holding the maximum (its values are in rising position order), and the value there
+  int idx = 1 << 20;
+  float val = 0.0f;
+#pragma unroll
+  for (int k = 15; k >= 0; k--) {
+    const bool hit = fabsf(v[k]) == amax;
+    idx = hit ? 4 * (l + 16 * (k >> 2)) + (k & 3) : idx;
+    val = hit ? v[k] : val;
+  }
+  const int firstpos = ilt_min16(idx);
+  const float mx = __int_as_float(ilt_or16(idx == firstpos ? __float_as_int(val) : 0));
+  const bool nz = amax != 0.0f;
+  const float iscale = nz ? -127.0f / mx : 0.0f;
+  const float d = nz ? 1.0f / iscale : 0.0f;
+  int q[16];
+#pragma unroll
+  for (int k = 0; k < 16; k++) q[k] = nz ? min(127, (int)rintf(iscale * v[k])) : 0;
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+    const int s = ilt_sum4(q[4 * i] + q[4 * i + 1] + q[4 * i + 2] + q[4 * i + 3]);
+    if (live) {
+      *(int*)(lxq + b * PITCH + 4 * (l + 16 * i)) =
+          (q[4 * i] & 0xFF) | ((q[4 * i + 1] & 0xFF) << 8) | ((q[4 * i + 2] & 0xFF) << 16) | ((q[4 * i + 3] & 0xFF) << 24);
+      if (lbs && (l & 3) == 0) lbs[b * 16 + (l >> 2) + 4 * i] = s;     // IQ2_XXS takes no 16-sums: none staged
+    }
+  }
+  if (live && l == 0) lxs[b] = d;
+}
+
+// All passes; FIRST / NFIRST: the first pass's values (x's, the norm weights'), loaded by the caller.
+template <int PITCH, int NW = kWaves>
 __device__ __forceinline__ void stage_q8k_from_f32(const float* __restrict__ x, int nblk, i8* lxq, float* lxs, int* lbs, const float4* first,
                                                    const float* __restrict__ nw = nullptr, const float4* nfirst = nullptr,
                                                    float nscale = 1.0f, float* __restrict__ h = nullptr) {
-  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), g = lane >> 4, l = lane & 15;
   const int npass = (nblk + 4 * NW - 1) / (4 * NW);
-  auto one_pass = [&](int pass, const float4* pre) {
-    if (4 * wave + 4 * NW * pass >= nblk) return;        // none of this wave's four blocks exists
-    const int b = 4 * wave + 4 * NW * pass + g;
-    const bool live = b < nblk;
-    float4 t4[4];
-    if (pre) { t4[0] = pre[0]; t4[1] = pre[1]; t4[2] = pre[2]; t4[3] = pre[3]; }
-    else load_q8k_pass<NW>(x, nblk, pass, t4);
-    if (nw) {
-      float4 n4[4];
-      if (pass == 0 && nfirst) { n4[0] = nfirst[0]; n4[1] = nfirst[1]; n4[2] = nfirst[2]; n4[3] = nfirst[3]; }
-      else load_q8k_pass<NW>(nw, nblk, pass, n4);
-#pragma unroll
-      for (int i = 0; i < 4; i++) {
-        t4[i] = make_float4((t4[i].x * nscale) * n4[i].x, (t4[i].y * nscale) * n4[i].y, (t4[i].z * nscale) * n4[i].z, (t4[i].w * nscale) * n4[i].w);
-        if (h && live) *(float4*)(h + b * 256 + 4 * (l + 16 * i)) = t4[i];
-      }
-    }
-    float v[16];
-#pragma unroll
-    for (int i = 0; i < 4; i++) { v[4 * i] = t4[i].x; v[4 * i + 1] = t4[i].y; v[4 * i + 2] = t4[i].z; v[4 * i + 3] = t4[i].w; }
-    float am = 0.0f;
-#pragma unroll
-    for (int k = 0; k < 16; k++) am = fmaxf(am, fabsf(v[k]));
-    const float amax = ilt_max16(am);
-    // this lane's first position holding the maximum (its values are in rising position order), and the value there
-    int idx = 1 << 20;
-    float val = 0.0f;
-#pragma unroll
-    for (int k = 15; k >= 0; k--) {
-      const bool hit = fabsf(v[k]) == amax;
-      idx = hit ? 4 * (l + 16 * (k >> 2)) + (k & 3) : idx;
-      val = hit ? v[k] : val;
-    }
-    const int firstpos = ilt_min16(idx);
-    const float mx = __int_as_float(ilt_or16(idx == firstpos ? __float_as_int(val) : 0));
-    const bool nz = amax != 0.0f;
-    const float iscale = nz ? -127.0f / mx : 0.0f;
-    const float d = nz ? 1.0f / iscale : 0.0f;
-    int q[16];
-#pragma unroll
-    for (int k = 0; k < 16; k++) q[k] = nz ? min(127, (int)rintf(iscale * v[k])) : 0;
-#pragma unroll
-    for (int i = 0; i < 4; i++) {
-      const int s = ilt_sum4(q[4 * i] + q[4 * i + 1] + q[4 * i + 2] + q[4 * i + 3]);
-      if (live) {
-        *(int*)(lxq + b * PITCH + 4 * (l + 16 * i)) =
-            (q[4 * i] & 0xFF) | ((q[4 * i + 1] & 0xFF) << 8) | ((q[4 * i + 2] & 0xFF) << 16) | ((q[4 * i + 3] & 0xFF) << 24);
-        if (lbs && (l & 3) == 0) lbs[b * 16 + (l >> 2) + 4 * i] = s;     // IQ2_XXS takes no 16-sums: none staged
-      }
-    }
-    if (live && l == 0) lxs[b] = d;
-  };
-#pragma unroll
-  for (int pass = 0; pass < NPRE; pass++)
-    if (pass < npass) one_pass(pass, first + 4 * pass);
-  for (int pass = NPRE; pass < npass; pass++) one_pass(pass, nullptr);
+  q8k_pass<PITCH, NW>(x, nblk, 0, first, lxq, lxs, lbs, nw, nfirst, nscale, h);
+  for (int pass = 1; pass < npass; pass++) q8k_pass<PITCH, NW>(x, nblk, pass, nullptr, lxq, lxs, lbs, nw, nullptr, nscale, h);
 }
 
 // Q8_0 (quantize-q8!, tensor.lisp:245-262): 8 lanes a block of 32.  XSUM: each block's sum of
@@ -777,11 +781,23 @@ __global__ __launch_bounds__(kStreamThreads) void gemv_stream_kernel(IltGemvPara
       }
       sq += (sq4(xall[0]) + sq4(xall[1])) + (sq4(xall[2]) + sq4(xall[3]));
       const float nscale = norm_scale_stagers(sq, p.xf, p.cols, p.eps, p.norm_seq);
-      stage_q8k_from_f32<XP, 1, kStagers>(p.xf, S, lxq, lxs, lbs, xall, p.norm_w, nall, nscale);
+      stage_q8k_from_f32<XP, kStagers>(p.xf, S, lxq, lxs, lbs, xall, p.norm_w, nall, nscale);
+    } else if (p.xf && S > 4 * kStagers) {
+      // up to three passes (cols <= 12288): all their loads first, then the three passes' chains
+      // of dependent instructions, which are independent of one another and interleave
+      float4 x0[4], x1[4], x2[4];
+      load_q8k_pass_clamped<kStagers>(p.xf, S, 0, x0);
+      load_q8k_pass_clamped<kStagers>(p.xf, S, 1, x1);
+      load_q8k_pass_clamped<kStagers>(p.xf, S, 2, x2);
+      q8k_pass<XP, kStagers>(p.xf, S, 0, x0, lxq, lxs, lbs, nullptr, nullptr, 1.0f, nullptr);
+      q8k_pass<XP, kStagers>(p.xf, S, 1, x1, lxq, lxs, lbs, nullptr, nullptr, 1.0f, nullptr);
+      q8k_pass<XP, kStagers>(p.xf, S, 2, x2, lxq, lxs, lbs, nullptr, nullptr, 1.0f, nullptr);
+      for (int pass = 3; pass * 4 * kStagers < S; pass++)
+        q8k_pass<XP, kStagers>(p.xf, S, pass, nullptr, lxq, lxs, lbs, nullptr, nullptr, 1.0f, nullptr);
     } else if (p.xf) {
       float4 xall[4];
       load_q8k_pass_clamped<kStagers>(p.xf, S, 0, xall);
-      stage_q8k_from_f32<XP, 1, kStagers>(p.xf, S, lxq, lxs, lbs, xall);
+      stage_q8k_from_f32<XP, kStagers>(p.xf, S, lxq, lxs, lbs, xall);
     } else {
       for (int i = threadIdx.x; i < S * 16; i += 64 * kStagers)
         *(int4*)(lxq + (i >> 4) * XP + 16 * (i & 15)) = *(const int4*)(p.xq + 16 * i);
@@ -826,10 +842,11 @@ __global__ __launch_bounds__(kStreamThreads) void gemv_stream_kernel(IltGemvPara
   if (!live) return;
   // The gate's rows (or the only matrix's) have landed when at most the up matrix's loads are
   // still on their way: they return in the order they were issued.
-  if (nup == 0 || nup > 12) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-  else if (nup <= 4) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
-  else if (nup <= 8) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
-  else asm volatile("s_waitcnt vmcnt(12)" ::: "memory");
+  // (the count in the instruction is a constant: the largest of 12, 8, 4, 0 that is not above nup)
+  if (nup >= 12) asm volatile("s_waitcnt vmcnt(12)" ::: "memory");
+  else if (nup >= 8) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+  else if (nup >= 4) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+  else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 
   const Lds L = { lxq, lxs, lbs, nullptr };
   if (fmt == ILT_Q4_K) wave_rows_lds<ILT_Q4_K>(region, nrows, S, p.s_magic, L, tw, lane);
