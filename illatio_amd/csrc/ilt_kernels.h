@@ -55,6 +55,7 @@ struct IltGemvParams {
   int wgs_per_group;         // grouped rows: workgroups sharing one group (set at launch)
   int batch;                 // rows a wave takes through phase A at a time (set at launch)
   int region;                // streamed variant: bytes of LDS per wave for its rows (set at launch)
+  int nz;                    // streamed variant: experts taking part (set at launch)
   uint32_t s_magic;          // ceil(2^32 / blocks per row)
 };
 

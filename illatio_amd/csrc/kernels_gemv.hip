@@ -18,6 +18,7 @@
 #include "ilt_device.h"
 #include "ilt_iq2xxs_tables.h"
 #include "ilt_kernels.h"
+#include <type_traits>
 
 namespace {
 
@@ -39,7 +40,7 @@ struct Lds {
   const i8* xq;        // Q8_0: cols bytes; Q8_K: XP bytes per block of 256
   const float* xs;     // one scale per activation block
   const int* bsums;    // Q8_K: sums of 16 quants
-  const u64* grid;     // IQ2_XXS codebook
+  const u64* grid;     // IQ2_XXS codebook (256 entries), then its sign masks (128 entries, see iq2_sign_mask)
 };
 
 __device__ __forceinline__ int4 and4(const int4& v, int m) { return make_int4(v.x & m, v.y & m, v.z & m, v.w & m); }
@@ -96,18 +97,24 @@ template <> __device__ __forceinline__ void load_raw<ILT_IQ2_XXS>(Raw<ILT_IQ2_XX
 // One IQ2_XXS sub-block (32 weights): its integer dot with 32 activations.  The sign of
 // weight i of an 8-group is bit i of the 7-bit pattern, bit 7 their parity; with m the
 // bytes to negate, sum(sign*mag*x) = sum(mag*x) - 2*sum((mag&m)*x).
+// The byte masks (0xFF where the weight is negative) of the 128 sign patterns come from a table
+// in LDS behind the codebook: building them in registers takes four 32-bit multiplies a pattern,
+// which run at a quarter of the rate of the rest.
+__device__ __forceinline__ u64 iq2_sign_mask(u32 s7) {      // table entry s7 (0..127)
+  const u32 s = s7 | ((__popc(s7) & 1) << 7);
+  const u32 mlo = (((s & 0xF) * 0x00204081u) & 0x01010101u) * 0xFFu;
+  const u32 mhi = (((s >> 4) * 0x00204081u) & 0x01010101u) * 0xFFu;
+  return ((u64)mhi << 32) | mlo;
+}
 __device__ __forceinline__ int iq2xxs_sub_dot(u32 g, u32 aux, const i8* xb, const u64* grid) {
   int pos = 0, neg = 0;
 #pragma unroll
   for (int l = 0; l < 4; l++) {
     const int2 mag = ilt_lds_ld8(grid + ((g >> (8 * l)) & 0xFF));
-    u32 s = (aux >> (7 * l)) & 127;
-    s |= (__popc(s) & 1) << 7;
-    const u32 mlo = (((s & 0xF) * 0x00204081u) & 0x01010101u) * 0xFFu;
-    const u32 mhi = (((s >> 4) * 0x00204081u) & 0x01010101u) * 0xFFu;
+    const int2 m = ilt_lds_ld8(grid + 256 + ((aux >> (7 * l)) & 127));
     const int2 x = ilt_lds_ld8(xb + 8 * l);
     pos = ilt_dot4((int)mag.y, x.y, ilt_dot4((int)mag.x, x.x, pos));
-    neg = ilt_dot4((int)((u32)mag.y & mhi), x.y, ilt_dot4((int)((u32)mag.x & mlo), x.x, neg));
+    neg = ilt_dot4((int)(mag.y & m.y), x.y, ilt_dot4((int)(mag.x & m.x), x.x, neg));
   }
   return pos - 2 * neg;
 }
@@ -521,7 +528,7 @@ __global__ __launch_bounds__(kThreads) void gemv_kernel(IltGemvParams p) {
   const int nbs = (q8 || FSET == ILT_IQ2_XXS) ? 0 : p.cols / 16;
   float* lxs = (float*)(lbs + nbs);
   u64* lgrid = (u64*)(((uintptr_t)(lxs + S) + 7) & ~(uintptr_t)7);
-  float* terms = (float*)(lgrid + (FSET == ILT_IQ2_XXS ? 256 : 0));
+  float* terms = (float*)(lgrid + (FSET == ILT_IQ2_XXS ? 384 : 0));
 
   // grouped rows (d4_mvq8): wgs_per_group workgroups share one group's rows and activations
   const int group = p.group_rows > 0 ? blockIdx.x / p.wgs_per_group : 0;
@@ -604,7 +611,10 @@ __global__ __launch_bounds__(kThreads) void gemv_kernel(IltGemvParams p) {
       for (int i = threadIdx.x; i < nbs; i += kThreads) lbs[i] = p.bsums[xoff / 16 + i];
     }
   }
-  if (FSET == ILT_IQ2_XXS) lgrid[threadIdx.x] = ilt_iq2xxs_grid_dev[threadIdx.x];
+  if (FSET == ILT_IQ2_XXS) {
+    lgrid[threadIdx.x] = ilt_iq2xxs_grid_dev[threadIdx.x];
+    if (threadIdx.x < 128) lgrid[256 + threadIdx.x] = iq2_sign_mask(threadIdx.x);
+  }
   __syncthreads();
 
   const Lds L = { lxq, lxs, lbs, lgrid };
@@ -659,32 +669,47 @@ __global__ __launch_bounds__(kThreads) void gemv_kernel(IltGemvParams p) {
 // order they were issued); the matrix streams in at the memory's rate while the activations
 // are quantized, and the blocks' terms are then formed from LDS.  One workgroup a CU, one
 // batch of rows a wave.
-template <int FMT> struct LdsBlk;      // a block in LDS: LB bytes, PPB pieces of 16 bytes
-template <> struct LdsBlk<ILT_Q4_K> { static constexpr int LB = 144, PPB = 9; };
-// Q6_K's 212 bytes are spread to 224 so that every piece stays 16-byte aligned in LDS; the last
-// piece is bytes 196..211 of the block (not 208..223, which would read past a matrix's end):
-// the scale d lands at 220.
-template <> struct LdsBlk<ILT_Q6_K> { static constexpr int LB = 224, PPB = 14; };
+// A block in LDS: LB bytes as PPB pieces of 16 bytes, every piece 16-byte aligned there whatever the
+// block's size in memory (BB); goff(pc) = where piece pc comes from within the block.  No piece
+// reaches past its block's end (the last block of a matrix may be the last bytes of an allocation).
+template <int FMT> struct LdsBlk;
+template <> struct LdsBlk<ILT_Q4_K> {
+  static constexpr int LB = 144, PPB = 9, BB = 144;
+  static __device__ __forceinline__ u32 goff(u32 pc) { return 16 * pc; }
+};
+// Q6_K: 212 bytes spread to 224; the last piece is bytes 196..211, so the scale d lands at 220.
+template <> struct LdsBlk<ILT_Q6_K> {
+  static constexpr int LB = 224, PPB = 14, BB = ILT_Q6K_STRIDE;
+  static __device__ __forceinline__ u32 goff(u32 pc) { return pc == 13 ? 196u : 16 * pc; }
+};
+// IQ2_XXS: 66 bytes (d, then 8 sub-blocks of 8 bytes) as the four 16-byte pairs of sub-blocks, then
+// the block's first 16 bytes, whose first two are d: d lands at 64.
+template <> struct LdsBlk<ILT_IQ2_XXS> {
+  static constexpr int LB = 80, PPB = 5, BB = 66;
+  static __device__ __forceinline__ u32 goff(u32 pc) { return pc == 4 ? 0u : 2 + 16 * pc; }
+};
+// Q2_K: 84 bytes (16 scale bytes, 64 of quants, d and dmin) as those five pieces and bytes 68..83,
+// whose last four are d and dmin: they land at 92.
+template <> struct LdsBlk<ILT_Q2_K> {
+  static constexpr int LB = 96, PPB = 6, BB = 84;
+  static __device__ __forceinline__ u32 goff(u32 pc) { return pc == 5 ? 68u : 16 * pc; }
+};
 
 // Returns the number of load instructions issued (the same in every lane).
 template <int FMT>
 __device__ __forceinline__ int stream_run(const u8* w, long row0, int nrows, int S, long row_bytes, u8* lds_run, int lane) {
+  using B = LdsBlk<FMT>;
   const u8* src = (const u8*)ilt_uniform_ptr(w + row0 * row_bytes);
-  const int npieces = __builtin_amdgcn_readfirstlane(nrows * S * LdsBlk<FMT>::PPB);
+  const int npieces = __builtin_amdgcn_readfirstlane(nrows * S * B::PPB);
   const int nfull = npieces >> 6, tail = npieces & 63;
   // this lane's piece of the first instruction; each further instruction is 64 pieces on
-  u32 blk = ((u32)lane * 9363u) >> 17, pc = (u32)lane - 14 * blk;        // Q6_K: lane / 14, lane % 14
-  u32 off = (u32)lane * 16;                                              // Q4_K: the run as it is
+  u32 blk = (u32)lane / B::PPB, pc = (u32)lane % B::PPB;
   for (int i = 0; i < nfull; i++) {
-    if (FMT == ILT_Q6_K) off = blk * ILT_Q6K_STRIDE + (pc == 13 ? 196u : 16 * pc);
-    ilt_g2lds16(src + off, lds_run + i * 1024);
-    if (FMT == ILT_Q6_K) { pc += 8; blk += 4; if (pc >= 14) { pc -= 14; blk += 1; } }      // 64 = 4 * 14 + 8
-    else off += 1024;
+    ilt_g2lds16(src + blk * B::BB + B::goff(pc), lds_run + i * 1024);
+    blk += 64 / B::PPB; pc += 64 % B::PPB;
+    if (pc >= B::PPB) { pc -= B::PPB; blk += 1; }
   }
-  if (tail) {
-    if (FMT == ILT_Q6_K) off = blk * ILT_Q6K_STRIDE + (pc == 13 ? 196u : 16 * pc);
-    if (lane < tail) ilt_g2lds16(src + off, lds_run + nfull * 1024);     // the lanes past the end load nothing
-  }
+  if (tail && lane < tail) ilt_g2lds16(src + blk * B::BB + B::goff(pc), lds_run + nfull * 1024);   // the lanes past the end load nothing
   return nfull + (tail ? 1 : 0);
 }
 
@@ -704,6 +729,17 @@ template <> __device__ __forceinline__ void load_raw_lds<ILT_Q6_K>(Raw<ILT_Q6_K>
   r.qh1 = ilt_lds_ld16(b + 128 + 32 * c + 16);
   r.sc = ilt_lds_ld16(b + 192);
   r.d = *(const ILT_LDS u16*)(b + 220);
+}
+template <> __device__ __forceinline__ void load_raw_lds<ILT_IQ2_XXS>(Raw<ILT_IQ2_XXS>& r, const u8* run, u32 f, int j) {
+  const u8* b = run + f * LdsBlk<ILT_IQ2_XXS>::LB;
+  r.q = ilt_lds_ld16(b + 16 * j);
+  r.d = *(const ILT_LDS u16*)(b + 64);
+}
+template <> __device__ __forceinline__ void load_raw_lds<ILT_Q2_K>(Raw<ILT_Q2_K>& r, const u8* run, u32 f, int j) {
+  const u8* b = run + f * LdsBlk<ILT_Q2_K>::LB;
+  r.q = ilt_lds_ld16(b + 16 + 16 * j);
+  r.sb = ilt_lds_ld16(b);
+  r.dd = *(const ILT_LDS u32*)(b + 92);
 }
 
 // A wave's run of nrows*S blocks, in LDS: terms into t.
@@ -754,21 +790,43 @@ __device__ __forceinline__ float norm_scale_stagers(double part, const float* __
   return 1.0f / sqrtf((float)v);
 }
 
-// FSET: ILT_Q4_K, ILT_Q6_K or 0 (mixed).  p.batch = the most rows a wave takes; p.region = bytes of LDS
-// per wave for its rows (both matrices' when glu).
+// Calls f(integral_constant<int, FMT>) for the format FMT of a matrix.
+template <int FSET, typename F>
+__device__ __forceinline__ void with_format(int fmt, F&& f) {
+  if constexpr (FSET != 0) f(std::integral_constant<int, FSET>{});
+  else if (fmt == ILT_Q4_K) f(std::integral_constant<int, ILT_Q4_K>{});
+  else f(std::integral_constant<int, ILT_Q6_K>{});
+}
+__device__ __forceinline__ int lds_block_bytes(int fmt) {
+  return fmt == ILT_Q4_K ? 144 : fmt == ILT_Q6_K ? 224 : fmt == ILT_Q2_K ? 96 : 80;
+}
+
+// FSET: ILT_Q4_K, ILT_Q6_K, 0 (those two mixed), or the expert formats ILT_IQ2_XXS, ILT_Q2_K (then
+// p.ptrs gives the experts' slots and p.nz how many take part: a batch is rows of one expert,
+// batches per expert = p.mat[0].nbat).  p.batch = the most rows a wave takes; p.region = bytes
+// of LDS per wave for its rows (both matrices' when glu).
 template <int FSET>
 __global__ __launch_bounds__(kStreamThreads) void gemv_stream_kernel(IltGemvParams p) {
   extern __shared__ __align__(16) unsigned char smem[];
+  constexpr bool iq2 = FSET == ILT_IQ2_XXS;
   const int S = p.cols / 256;
+  const int nx = p.x_stride ? p.nz : 1;                  // activation vectors staged (one per expert, or one for all)
+  const int SX = S * nx;
   i8* lxq = (i8*)smem;
-  int* lbs = (int*)(smem + S * XP);
-  float* lxs = (float*)(lbs + p.cols / 16);
-  float* terms = (float*)(((uintptr_t)(lxs + S) + 15) & ~(uintptr_t)15);
+  int* lbs = (int*)(smem + SX * XP);
+  float* lxs = (float*)(lbs + (iq2 ? 0 : SX * 16));
+  u64* lgrid = (u64*)(((uintptr_t)(lxs + SX) + 15) & ~(uintptr_t)15);
+  float* terms = (float*)(lgrid + (iq2 ? 384 : 0));
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);     // the same in every lane, said so
   const int tpr = S * 2, nglu = p.glu ? 2 : 1;
 
   // 1. the activations into LDS, by the first four waves
   if (wave < kStagers) {
+    if (iq2) {
+      lgrid[threadIdx.x] = ilt_iq2xxs_grid_dev[threadIdx.x];
+      if (threadIdx.x < 128) lgrid[256 + threadIdx.x] = iq2_sign_mask(threadIdx.x);
+    }
+    int* sbs = iq2 ? nullptr : lbs;
     if (p.xf && p.norm_w) {
       float4 xall[4], nall[4];
       load_q8k_pass<kStagers>(p.xf, S, 0, xall);           // zeros where there is no block: they are squared
@@ -781,28 +839,28 @@ __global__ __launch_bounds__(kStreamThreads) void gemv_stream_kernel(IltGemvPara
       }
       sq += (sq4(xall[0]) + sq4(xall[1])) + (sq4(xall[2]) + sq4(xall[3]));
       const float nscale = norm_scale_stagers(sq, p.xf, p.cols, p.eps, p.norm_seq);
-      stage_q8k_from_f32<XP, kStagers>(p.xf, S, lxq, lxs, lbs, xall, p.norm_w, nall, nscale);
-    } else if (p.xf && S > 4 * kStagers) {
-      // up to three passes (cols <= 12288): all their loads first, then the three passes' chains
+      stage_q8k_from_f32<XP, kStagers>(p.xf, S, lxq, lxs, sbs, xall, p.norm_w, nall, nscale);
+    } else if (p.xf && SX > 4 * kStagers) {
+      // up to three passes (12288 activations): all their loads first, then the three passes' chains
       // of dependent instructions, which are independent of one another and interleave
       float4 x0[4], x1[4], x2[4];
-      load_q8k_pass_clamped<kStagers>(p.xf, S, 0, x0);
-      load_q8k_pass_clamped<kStagers>(p.xf, S, 1, x1);
-      load_q8k_pass_clamped<kStagers>(p.xf, S, 2, x2);
-      q8k_pass<XP, kStagers>(p.xf, S, 0, x0, lxq, lxs, lbs, nullptr, nullptr, 1.0f, nullptr);
-      q8k_pass<XP, kStagers>(p.xf, S, 1, x1, lxq, lxs, lbs, nullptr, nullptr, 1.0f, nullptr);
-      q8k_pass<XP, kStagers>(p.xf, S, 2, x2, lxq, lxs, lbs, nullptr, nullptr, 1.0f, nullptr);
-      for (int pass = 3; pass * 4 * kStagers < S; pass++)
-        q8k_pass<XP, kStagers>(p.xf, S, pass, nullptr, lxq, lxs, lbs, nullptr, nullptr, 1.0f, nullptr);
+      load_q8k_pass_clamped<kStagers>(p.xf, SX, 0, x0);
+      load_q8k_pass_clamped<kStagers>(p.xf, SX, 1, x1);
+      load_q8k_pass_clamped<kStagers>(p.xf, SX, 2, x2);
+      q8k_pass<XP, kStagers>(p.xf, SX, 0, x0, lxq, lxs, sbs, nullptr, nullptr, 1.0f, nullptr);
+      q8k_pass<XP, kStagers>(p.xf, SX, 1, x1, lxq, lxs, sbs, nullptr, nullptr, 1.0f, nullptr);
+      q8k_pass<XP, kStagers>(p.xf, SX, 2, x2, lxq, lxs, sbs, nullptr, nullptr, 1.0f, nullptr);
+      for (int pass = 3; pass * 4 * kStagers < SX; pass++)
+        q8k_pass<XP, kStagers>(p.xf, SX, pass, nullptr, lxq, lxs, sbs, nullptr, nullptr, 1.0f, nullptr);
     } else if (p.xf) {
       float4 xall[4];
-      load_q8k_pass_clamped<kStagers>(p.xf, S, 0, xall);
-      stage_q8k_from_f32<XP, kStagers>(p.xf, S, lxq, lxs, lbs, xall);
+      load_q8k_pass_clamped<kStagers>(p.xf, SX, 0, xall);
+      stage_q8k_from_f32<XP, kStagers>(p.xf, SX, lxq, lxs, sbs, xall);
     } else {
-      for (int i = threadIdx.x; i < S * 16; i += 64 * kStagers)
+      for (int i = threadIdx.x; i < SX * 16; i += 64 * kStagers)
         *(int4*)(lxq + (i >> 4) * XP + 16 * (i & 15)) = *(const int4*)(p.xq + 16 * i);
-      for (int i = threadIdx.x; i < S; i += 64 * kStagers) lxs[i] = p.xs[i];
-      for (int i = threadIdx.x; i < p.cols / 16; i += 64 * kStagers) lbs[i] = p.bsums[i];
+      for (int i = threadIdx.x; i < SX; i += 64 * kStagers) lxs[i] = p.xs[i];
+      if (!iq2) for (int i = threadIdx.x; i < SX * 16; i += 64 * kStagers) lbs[i] = p.bsums[i];
     }
     ilt_barrier_lds();
     return;
@@ -813,26 +871,27 @@ __global__ __launch_bounds__(kStreamThreads) void gemv_stream_kernel(IltGemvPara
   const int wid = rw * gridDim.x + blockIdx.x;          // consecutive batches on different CUs
 
   // 2. this wave's rows, all of them
-  int mi = 0, nrows = 0; long row0 = 0;
+  int mi = 0, nrows = 0, z = 0; long row0 = 0;
   const bool live = wid < p.nbatches;
+  int bl = wid;
   if (live) {
-    if (!p.glu) while (mi + 1 < p.nmat && wid >= p.mat[mi + 1].batch0) mi++;
-    const int bl = wid - p.mat[mi].batch0, rq = p.mat[mi].rq, rr = p.mat[mi].rr;
+    if (p.ptrs) { z = wid / p.mat[0].nbat; bl = wid - z * p.mat[0].nbat; }
+    else if (!p.glu) { while (mi + 1 < p.nmat && wid >= p.mat[mi + 1].batch0) mi++; bl = wid - p.mat[mi].batch0; }
+    const int rq = p.mat[mi].rq, rr = p.mat[mi].rr;
     row0 = (long)bl * rq + min(bl, rr);
     nrows = rq + (bl < rr ? 1 : 0);
   }
   const IltGemvMat& m = p.mat[mi];
   const int fmt = FSET != 0 ? FSET : m.fmt;
   const int ufmt = FSET != 0 ? FSET : p.mat[1].fmt;
+  const u8* slot = (live && p.ptrs) ? (const u8*)p.ptrs[p.sel ? p.sel[z] : z] : nullptr;
+  const u8* wg = p.ptrs ? slot + m.add : m.w;
+  const u8* wu = p.ptrs ? slot + p.mat[1].add : p.mat[1].w;
   u8* region_up = region + p.region / 2;
   int nup = 0;              // load instructions of the up matrix's rows: the last ones issued
   if (live) {
-    if (fmt == ILT_Q4_K) stream_run<ILT_Q4_K>(m.w, row0, nrows, S, m.row_bytes, region, lane);
-    else stream_run<ILT_Q6_K>(m.w, row0, nrows, S, m.row_bytes, region, lane);
-    if (p.glu) {
-      if (ufmt == ILT_Q4_K) nup = stream_run<ILT_Q4_K>(p.mat[1].w, row0, nrows, S, p.mat[1].row_bytes, region_up, lane);
-      else nup = stream_run<ILT_Q6_K>(p.mat[1].w, row0, nrows, S, p.mat[1].row_bytes, region_up, lane);
-    }
+    with_format<FSET>(fmt, [&](auto F) { stream_run<decltype(F)::value>(wg, row0, nrows, S, m.row_bytes, region, lane); });
+    if (p.glu) with_format<FSET>(ufmt, [&](auto F) { nup = stream_run<decltype(F)::value>(wu, row0, nrows, S, p.mat[1].row_bytes, region_up, lane); });
   }
   if (p.norm_w) { ilt_barrier_lds(); ilt_barrier_lds(); ilt_barrier_lds(); }      // in step with norm_scale_stagers
   // The barrier is for the activations only, so it comes before this wave waits for its rows (no
@@ -848,27 +907,36 @@ __global__ __launch_bounds__(kStreamThreads) void gemv_stream_kernel(IltGemvPara
   else if (nup >= 4) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
   else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 
-  const Lds L = { lxq, lxs, lbs, nullptr };
-  if (fmt == ILT_Q4_K) wave_rows_lds<ILT_Q4_K>(region, nrows, S, p.s_magic, L, tw, lane);
-  else wave_rows_lds<ILT_Q6_K>(region, nrows, S, p.s_magic, L, tw, lane);
+  const int zx = p.x_stride ? z : 0;
+  const Lds L = { lxq + (long)zx * S * XP, lxs + zx * S, lbs + zx * S * 16, lgrid };
+  with_format<FSET>(fmt, [&](auto F) { wave_rows_lds<decltype(F)::value>(region, nrows, S, p.s_magic, L, tw, lane); });
   if (p.glu) {
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    if (ufmt == ILT_Q4_K) wave_rows_lds<ILT_Q4_K>(region_up, nrows, S, p.s_magic, L, tw + (long)p.batch * tpr, lane);
-    else wave_rows_lds<ILT_Q6_K>(region_up, nrows, S, p.s_magic, L, tw + (long)p.batch * tpr, lane);
+    with_format<FSET>(ufmt, [&](auto F) { wave_rows_lds<decltype(F)::value>(region_up, nrows, S, p.s_magic, L, tw + (long)p.batch * tpr, lane); });
   }
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
   __builtin_amdgcn_wave_barrier();
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
   if (lane < nrows) {
-    float v = sum_any(fmt, tw + (long)lane * S * (fmt == ILT_Q4_K ? 2 : 1), S);
+    const int tper = (fmt == ILT_Q4_K || fmt == ILT_Q2_K) ? 2 : 1, uper = (ufmt == ILT_Q4_K || ufmt == ILT_Q2_K) ? 2 : 1;
+    float v = sum_any(fmt, tw + (long)lane * S * tper, S);
     const long r = row0 + lane;
+    float* y = m.y + (long)z * p.y_stride;
     if (p.glu) {
-      const float uv = sum_any(ufmt, tw + (long)p.batch * tpr + (long)lane * S * (ufmt == ILT_Q4_K ? 2 : 1), S);
-      m.y[r] = dense_glu(v, uv);
+      const float uv = sum_any(ufmt, tw + (long)p.batch * tpr + (long)lane * S * uper, S);
+      if (p.glu == 1) {
+        y[r] = dense_glu(v, uv);
+      } else {        // the experts' gated activation, as d4_swiglu_w computes it
+        float gv = v, uu = uv;
+        if (p.clamp > 1e-6f) { gv = fminf(gv, p.clamp); uu = fmaxf(-p.clamp, fminf(uu, p.clamp)); }
+        float o = ilt_silu(gv) * uu;
+        if (p.wts) o = o * p.wts[z];
+        y[r] = o;
+      }
     } else {
       if (m.bias) v = v + m.bias[r];
-      if (p.acc) v = m.y[r] + v;
-      m.y[r] = v;
+      if (p.acc) v = y[r] + v;
+      y[r] = v;
     }
   }
 }
@@ -901,7 +969,7 @@ size_t gemv_smem(int fset, const IltGemvParams& p) {
   size_t b = q8 ? (size_t)p.cols : (size_t)S * XP;
   b += (q8 || fset == ILT_IQ2_XXS) ? 0 : (size_t)p.cols / 16 * 4;
   b += 4 * (size_t)S + 8;
-  if (fset == ILT_IQ2_XXS) b += 2048;
+  if (fset == ILT_IQ2_XXS) b += 3072;
   return b + (size_t)kWaves * p.batch * S * (q8 ? 1 : 2) * 4 * (p.glu ? 2 : 1);
 }
 
@@ -931,69 +999,92 @@ int resident_per_cu(int fset, size_t smem) {
 
 }  // namespace
 
-// The streamed variant's launch, when the product qualifies: dense Q4_K / Q6_K matrices, one
-// activation vector, at most 16 rows a wave over the 3072 row waves of one workgroup per CU, and
-// everything within a CU's LDS.  Returns hipErrorNotSupported when it does not qualify.
+// The streamed variant's launch, when the product qualifies: Q4_K / Q6_K matrices on one
+// activation vector, or IQ2_XXS / Q2_K experts (nz of them, each on its own vector right after
+// the previous one's, or all on one); at most 16 rows a wave over the 3072 row waves of one
+// workgroup per CU; everything within a CU's LDS.  Returns hipErrorNotSupported otherwise.
 static unsigned long long g_streamed_launches = 0;
 unsigned long long ilt_k_streamed_launches() { return g_streamed_launches; }
 
-static hipError_t gemv_stream_launch(IltGemvParams& p, int fset, hipStream_t st) {
+static hipError_t gemv_stream_launch(IltGemvParams& p, int fset, int nz, hipStream_t st) {
   const char* force = getenv("ILT_GEMV_STREAM");          // "0": never (tests)
   if (force && atoi(force) == 0) return hipErrorNotSupported;
-  if (!(fset == 0 || fset == ILT_Q4_K || fset == ILT_Q6_K) || p.ptrs || p.group_rows > 0 || p.glu > 1)
+  const bool experts = p.ptrs != nullptr;
+  if (experts ? !(fset == ILT_IQ2_XXS || fset == ILT_Q2_K) : !(fset == 0 || fset == ILT_Q4_K || fset == ILT_Q6_K)) return hipErrorNotSupported;
+  if (p.group_rows > 0 || (!experts && (nz != 1 || p.glu > 1)) || (experts && (p.norm_w || !(p.x_stride == 0 || p.x_stride == p.cols))))
     return hipErrorNotSupported;
   const int S = p.cols / 256;
-  if (S > 64) return hipErrorNotSupported;
-  const int nm = p.glu ? 1 : p.nmat;
+  const int nx = p.x_stride ? nz : 1;
+  if (p.xf && p.norm_w ? S > 64 : (long)S * nx > 64 * 3) return hipErrorNotSupported;
+  const int nm = (p.glu || experts) ? 1 : p.nmat;
   long total_rows = 0, bytes = 0;
   for (int i = 0; i < nm; i++) { total_rows += p.mat[i].rows; bytes += (long)p.mat[i].rows * p.mat[i].row_bytes; }
   constexpr int kWavesAll = 256 * kRowWaves;
-  if (total_rows > 16L * kWavesAll || bytes * (p.glu ? 2 : 1) < (2L << 20)) return hipErrorNotSupported;
-  // every wave one batch: the waves are shared out over the matrices by rows, never more than there are
-  const int nb_total = (int)min((long)kWavesAll, total_rows);
-  int nb = 0, batch = 1, given = 0;
-  for (int i = 0; i < nm; i++) {
-    int nbi = (int)((long)nb_total * p.mat[i].rows / total_rows);
-    if (nbi < 1) nbi = 1;
-    p.mat[i].nbat = nbi; given += nbi;
-  }
-  for (int i = 0; given < nb_total; i = (i + 1) % nm)          // the rounding's leftovers, where rows allow
-    if (p.mat[i].nbat < p.mat[i].rows) { p.mat[i].nbat++; given++; }
-  if (given > kWavesAll) return hipErrorNotSupported;
-  for (int i = 0; i < p.nmat; i++) {
-    if (i >= nm) { p.mat[i].batch0 = 0; p.mat[i].nbat = p.mat[0].nbat; p.mat[i].rq = p.mat[0].rq; p.mat[i].rr = p.mat[0].rr; continue; }
-    p.mat[i].batch0 = nb;
-    p.mat[i].rq = p.mat[i].rows / p.mat[i].nbat;
-    p.mat[i].rr = p.mat[i].rows % p.mat[i].nbat;
-    batch = max(batch, p.mat[i].rq + (p.mat[i].rr ? 1 : 0));
-    nb += p.mat[i].nbat;
+  if (total_rows * nz > 16L * kWavesAll || bytes * nz * (p.glu ? 2 : 1) < (2L << 20)) return hipErrorNotSupported;
+  int nb = 0, batch = 1;
+  if (experts) {
+    // the waves are shared out evenly over the experts; a batch is rows of one expert
+    int nbz = kWavesAll / nz;
+    if (nbz < 1) return hipErrorNotSupported;
+    if (nbz > p.mat[0].rows) nbz = p.mat[0].rows;
+    for (int i = 0; i < p.nmat; i++) {
+      p.mat[i].batch0 = 0; p.mat[i].nbat = nbz; p.mat[i].rq = p.mat[0].rows / nbz; p.mat[i].rr = p.mat[0].rows % nbz;
+    }
+    batch = p.mat[0].rq + (p.mat[0].rr ? 1 : 0);
+    nb = nbz * nz;
+  } else {
+    // every wave one batch: the waves are shared out over the matrices by rows, never more than there are
+    const int nb_total = (int)min((long)kWavesAll, total_rows);
+    int given = 0;
+    for (int i = 0; i < nm; i++) {
+      int nbi = (int)((long)nb_total * p.mat[i].rows / total_rows);
+      if (nbi < 1) nbi = 1;
+      p.mat[i].nbat = nbi; given += nbi;
+    }
+    for (int i = 0; given < nb_total; i = (i + 1) % nm)          // the rounding's leftovers, where rows allow
+      if (p.mat[i].nbat < p.mat[i].rows) { p.mat[i].nbat++; given++; }
+    if (given > kWavesAll) return hipErrorNotSupported;
+    for (int i = 0; i < p.nmat; i++) {
+      if (i >= nm) { p.mat[i].batch0 = 0; p.mat[i].nbat = p.mat[0].nbat; p.mat[i].rq = p.mat[0].rq; p.mat[i].rr = p.mat[0].rr; continue; }
+      p.mat[i].batch0 = nb;
+      p.mat[i].rq = p.mat[i].rows / p.mat[i].nbat;
+      p.mat[i].rr = p.mat[i].rows % p.mat[i].nbat;
+      batch = max(batch, p.mat[i].rq + (p.mat[i].rr ? 1 : 0));
+      nb += p.mat[i].nbat;
+    }
   }
   if (batch > 16) return hipErrorNotSupported;
   p.nbatches = nb;
   p.batch = batch;
+  p.nz = nz;
   const int nglu = p.glu ? 2 : 1;
-  const int lb = fset == ILT_Q4_K ? 144 : 224;                        // Q6_K's spread blocks at worst
+  const int lb = fset == ILT_Q4_K ? 144 : fset == ILT_IQ2_XXS ? 80 : fset == ILT_Q2_K ? 96 : 224;      // Q6_K's spread blocks at worst
   const long one = (long)batch * S * lb;                              // a wave's rows of one matrix
   p.region = (int)(one * nglu);
-  const size_t smem = (size_t)S * XP + (size_t)p.cols / 16 * 4 + (size_t)S * 4 + 16 + (size_t)kRowWaves * batch * S * 2 * 4 * nglu +
-                      (size_t)kRowWaves * p.region;
+  const size_t smem = (size_t)S * nx * XP + (fset == ILT_IQ2_XXS ? 3072 : (size_t)S * nx * 16 * 4) + (size_t)S * nx * 4 + 16 +
+                      (size_t)kRowWaves * batch * S * 2 * 4 * nglu + (size_t)kRowWaves * p.region;
   if (smem > 156 * 1024) return hipErrorNotSupported;
   p.s_magic = (uint32_t)(0x100000000ULL / (uint64_t)S) + 1;
   static bool attr_set[8] = {};
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 8) dev = 0;
   if (!attr_set[dev]) {            // more dynamic LDS than the default 64 KB: asked for once per device
-    hipError_t e = hipFuncSetAttribute((const void*)gemv_stream_kernel<0>, hipFuncAttributeMaxDynamicSharedMemorySize, 158 * 1024);
-    if (e == hipSuccess) e = hipFuncSetAttribute((const void*)gemv_stream_kernel<ILT_Q4_K>, hipFuncAttributeMaxDynamicSharedMemorySize, 158 * 1024);
-    if (e == hipSuccess) e = hipFuncSetAttribute((const void*)gemv_stream_kernel<ILT_Q6_K>, hipFuncAttributeMaxDynamicSharedMemorySize, 158 * 1024);
-    if (e != hipSuccess) { (void)hipGetLastError(); return hipErrorNotSupported; }
+    const void* kernels[5] = { (const void*)gemv_stream_kernel<0>, (const void*)gemv_stream_kernel<ILT_Q4_K>, (const void*)gemv_stream_kernel<ILT_Q6_K>,
+                               (const void*)gemv_stream_kernel<ILT_IQ2_XXS>, (const void*)gemv_stream_kernel<ILT_Q2_K> };
+    for (int i = 0; i < 5; i++)
+      if (hipFuncSetAttribute(kernels[i], hipFuncAttributeMaxDynamicSharedMemorySize, 158 * 1024) != hipSuccess) {
+        (void)hipGetLastError();
+        return hipErrorNotSupported;
+      }
     attr_set[dev] = true;
   }
   const dim3 grid(min(256, nb));                                      // wave w of workgroup g takes batch w * grid + g
   switch (fset) {
     case 0: hipLaunchKernelGGL(gemv_stream_kernel<0>, grid, dim3(kStreamThreads), smem, st, p); break;
     case ILT_Q4_K: hipLaunchKernelGGL(gemv_stream_kernel<ILT_Q4_K>, grid, dim3(kStreamThreads), smem, st, p); break;
-    default: hipLaunchKernelGGL(gemv_stream_kernel<ILT_Q6_K>, grid, dim3(kStreamThreads), smem, st, p); break;
+    case ILT_Q6_K: hipLaunchKernelGGL(gemv_stream_kernel<ILT_Q6_K>, grid, dim3(kStreamThreads), smem, st, p); break;
+    case ILT_IQ2_XXS: hipLaunchKernelGGL(gemv_stream_kernel<ILT_IQ2_XXS>, grid, dim3(kStreamThreads), smem, st, p); break;
+    default: hipLaunchKernelGGL(gemv_stream_kernel<ILT_Q2_K>, grid, dim3(kStreamThreads), smem, st, p); break;
   }
   g_streamed_launches++;
   return hipGetLastError();
@@ -1002,8 +1093,8 @@ static hipError_t gemv_stream_launch(IltGemvParams& p, int fset, hipStream_t st)
 hipError_t ilt_gemv_launch(IltGemvParams& p, int nz, hipStream_t st) {
   int fset = p.mat[0].fmt;
   for (int i = 1; i < p.nmat; i++) if (p.mat[i].fmt != fset) fset = 0;
-  if (nz == 1) {
-    const hipError_t e = gemv_stream_launch(p, fset, st);
+  {
+    const hipError_t e = gemv_stream_launch(p, fset, nz, st);
     if (e != hipErrorNotSupported) return e;
   }
   const bool q8 = fset == ILT_Q8_0;
