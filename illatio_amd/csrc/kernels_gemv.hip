@@ -695,6 +695,24 @@ template <> struct LdsBlk<ILT_Q2_K> {
   static __device__ __forceinline__ u32 goff(u32 pc) { return pc == 5 ? 68u : 16 * pc; }
 };
 
+// Q8_0 (split at upload): the quants as they are, two pieces a block; the f16 scales are a second
+// run, copied four bytes a lane (stream_scales) behind the quants' room.
+template <> struct LdsBlk<ILT_Q8_0> {
+  static constexpr int LB = 32, PPB = 2, BB = 32;
+  static __device__ __forceinline__ u32 goff(u32 pc) { return 16 * pc; }
+};
+
+// NBYTES (a multiple of 4) from src to LDS, four bytes a lane.  Returns the number of instructions.
+__device__ __forceinline__ int stream_scales(const u8* src_, int nbytes, u8* lds, int lane) {
+  const u8* src = (const u8*)ilt_uniform_ptr(src_);
+  const int n4 = __builtin_amdgcn_readfirstlane(nbytes >> 2), nfull = n4 >> 6, tail = n4 & 63;
+  for (int i = 0; i < nfull; i++)
+    __builtin_amdgcn_global_load_lds((const ILT_GLOBAL void*)(src + (i * 64 + lane) * 4), (ILT_LDS void*)(lds + i * 256), 4, 0, 0);
+  if (tail && lane < tail)
+    __builtin_amdgcn_global_load_lds((const ILT_GLOBAL void*)(src + (nfull * 64 + lane) * 4), (ILT_LDS void*)(lds + nfull * 256), 4, 0, 0);
+  return nfull + (tail ? 1 : 0);
+}
+
 // Returns the number of load instructions issued (the same in every lane).
 template <int FMT>
 __device__ __forceinline__ int stream_run(const u8* w, long row0, int nrows, int S, long row_bytes, u8* lds_run, int lane) {
@@ -713,14 +731,19 @@ __device__ __forceinline__ int stream_run(const u8* w, long row0, int nrows, int
   return nfull + (tail ? 1 : 0);
 }
 
-template <int FMT> __device__ __forceinline__ void load_raw_lds(Raw<FMT>& r, const u8* run, u32 f, int j);
-template <> __device__ __forceinline__ void load_raw_lds<ILT_Q4_K>(Raw<ILT_Q4_K>& r, const u8* run, u32 f, int j) {
+// run2: Q8_0's scales (unused by the rest)
+template <int FMT> __device__ __forceinline__ void load_raw_lds(Raw<FMT>& r, const u8* run, const u8* run2, u32 f, int j);
+template <> __device__ __forceinline__ void load_raw_lds<ILT_Q8_0>(Raw<ILT_Q8_0>& r, const u8* run, const u8* run2, u32 f, int j) {
+  r.q = ilt_lds_ld16(run + f * LdsBlk<ILT_Q8_0>::LB + 16 * j);
+  r.d = *(const ILT_LDS u16*)(run2 + 2 * f);
+}
+template <> __device__ __forceinline__ void load_raw_lds<ILT_Q4_K>(Raw<ILT_Q4_K>& r, const u8* run, const u8*, u32 f, int j) {
   const u8* b = run + f * LdsBlk<ILT_Q4_K>::LB;
   r.hdr = ilt_lds_ld16(b);
   r.qa = ilt_lds_ld16(b + 16 + 32 * j);
   r.qb = ilt_lds_ld16(b + 32 + 32 * j);
 }
-template <> __device__ __forceinline__ void load_raw_lds<ILT_Q6_K>(Raw<ILT_Q6_K>& r, const u8* run, u32 f, int j) {
+template <> __device__ __forceinline__ void load_raw_lds<ILT_Q6_K>(Raw<ILT_Q6_K>& r, const u8* run, const u8*, u32 f, int j) {
   const u8* b = run + f * LdsBlk<ILT_Q6_K>::LB;
   const int c = j >> 1, pp = j & 1;
   r.ql0 = ilt_lds_ld16(b + 64 * c + 32 * pp);
@@ -730,12 +753,12 @@ template <> __device__ __forceinline__ void load_raw_lds<ILT_Q6_K>(Raw<ILT_Q6_K>
   r.sc = ilt_lds_ld16(b + 192);
   r.d = *(const ILT_LDS u16*)(b + 220);
 }
-template <> __device__ __forceinline__ void load_raw_lds<ILT_IQ2_XXS>(Raw<ILT_IQ2_XXS>& r, const u8* run, u32 f, int j) {
+template <> __device__ __forceinline__ void load_raw_lds<ILT_IQ2_XXS>(Raw<ILT_IQ2_XXS>& r, const u8* run, const u8*, u32 f, int j) {
   const u8* b = run + f * LdsBlk<ILT_IQ2_XXS>::LB;
   r.q = ilt_lds_ld16(b + 16 * j);
   r.d = *(const ILT_LDS u16*)(b + 64);
 }
-template <> __device__ __forceinline__ void load_raw_lds<ILT_Q2_K>(Raw<ILT_Q2_K>& r, const u8* run, u32 f, int j) {
+template <> __device__ __forceinline__ void load_raw_lds<ILT_Q2_K>(Raw<ILT_Q2_K>& r, const u8* run, const u8*, u32 f, int j) {
   const u8* b = run + f * LdsBlk<ILT_Q2_K>::LB;
   r.q = ilt_lds_ld16(b + 16 + 16 * j);
   r.sb = ilt_lds_ld16(b);
@@ -744,14 +767,14 @@ template <> __device__ __forceinline__ void load_raw_lds<ILT_Q2_K>(Raw<ILT_Q2_K>
 
 // A wave's run of nrows*S blocks, in LDS: terms into t.
 template <int FMT>
-__device__ __forceinline__ void wave_rows_lds(const u8* run, int nrows, int S, u32 s_magic, const Lds& L, float* t, int lane) {
+__device__ __forceinline__ void wave_rows_lds(const u8* run, const u8* run2, int nrows, int S, u32 s_magic, const Lds& L, float* t, int lane) {
   using F = Fmt<FMT>;
   constexpr int GPW = ILT_WAVE / F::LPB;
   const int j = lane % F::LPB, gl = lane / F::LPB;
   const int nblk = nrows * S;
   for (int f = gl; f < nblk; f += GPW) {
     Raw<FMT> r;
-    load_raw_lds<FMT>(r, run, f, j);
+    load_raw_lds<FMT>(r, run, run2, f, j);
     const int s_ = S > 1 ? f - (int)__umulhi((u32)f, s_magic) * S : 0;
     block_terms<FMT>(r, s_, j, L, t + (long)f * F::TERMS);
   }
@@ -798,7 +821,7 @@ __device__ __forceinline__ void with_format(int fmt, F&& f) {
   else f(std::integral_constant<int, ILT_Q6_K>{});
 }
 __device__ __forceinline__ int lds_block_bytes(int fmt) {
-  return fmt == ILT_Q4_K ? 144 : fmt == ILT_Q6_K ? 224 : fmt == ILT_Q2_K ? 96 : 80;
+  return fmt == ILT_Q4_K ? 144 : fmt == ILT_Q6_K ? 224 : fmt == ILT_Q2_K ? 96 : fmt == ILT_Q8_0 ? 32 : 80;
 }
 
 // FSET: ILT_Q4_K, ILT_Q6_K, 0 (those two mixed), or the expert formats ILT_IQ2_XXS, ILT_Q2_K (then
@@ -808,19 +831,28 @@ __device__ __forceinline__ int lds_block_bytes(int fmt) {
 template <int FSET>
 __global__ __launch_bounds__(kStreamThreads) void gemv_stream_kernel(IltGemvParams p) {
   extern __shared__ __align__(16) unsigned char smem[];
-  constexpr bool iq2 = FSET == ILT_IQ2_XXS;
-  const int S = p.cols / 256;
+  constexpr bool iq2 = FSET == ILT_IQ2_XXS, q8 = FSET == ILT_Q8_0;
+  const int S = q8 ? p.cols / 32 : p.cols / 256;
   const int nx = p.x_stride ? p.nz : 1;                  // activation vectors staged (one per expert, or one for all)
   const int SX = S * nx;
   i8* lxq = (i8*)smem;
-  int* lbs = (int*)(smem + SX * XP);
-  float* lxs = (float*)(lbs + (iq2 ? 0 : SX * 16));
+  int* lbs = (int*)(smem + (q8 ? p.cols : SX * XP));
+  float* lxs = (float*)(lbs + ((iq2 || q8) ? 0 : SX * 16));
   u64* lgrid = (u64*)(((uintptr_t)(lxs + SX) + 15) & ~(uintptr_t)15);
   float* terms = (float*)(lgrid + (iq2 ? 384 : 0));
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);     // the same in every lane, said so
-  const int tpr = S * 2, nglu = p.glu ? 2 : 1;
+  const int tpr = q8 ? S : S * 2, nglu = p.glu ? 2 : 1;
 
   // 1. the activations into LDS, by the first four waves
+  if (wave < kStagers && q8) {
+    if (p.xf) stage_q8_from_f32(p.xf, S, p.f16_scale, lxq, lxs);       // (its loop strides by the stagers' 256 threads)
+    else {
+      for (int i = threadIdx.x * 16; i < p.cols; i += 64 * kStagers * 16) *(int4*)(lxq + i) = *(const int4*)(p.xq + i);
+      for (int i = threadIdx.x; i < S; i += 64 * kStagers) lxs[i] = p.xs[i];
+    }
+    ilt_barrier_lds();
+    return;
+  }
   if (wave < kStagers) {
     if (iq2) {
       lgrid[threadIdx.x] = ilt_iq2xxs_grid_dev[threadIdx.x];
@@ -888,10 +920,17 @@ __global__ __launch_bounds__(kStreamThreads) void gemv_stream_kernel(IltGemvPara
   const u8* wg = p.ptrs ? slot + m.add : m.w;
   const u8* wu = p.ptrs ? slot + p.mat[1].add : p.mat[1].w;
   u8* region_up = region + p.region / 2;
+  // Q8_0: the scales' room behind the quants'
+  const u8* scales = region + (long)p.batch * p.cols;
+  const u8* scales_up = region_up + (long)p.batch * p.cols;
   int nup = 0;              // load instructions of the up matrix's rows: the last ones issued
   if (live) {
     with_format<FSET>(fmt, [&](auto F) { stream_run<decltype(F)::value>(wg, row0, nrows, S, m.row_bytes, region, lane); });
-    if (p.glu) with_format<FSET>(ufmt, [&](auto F) { nup = stream_run<decltype(F)::value>(wu, row0, nrows, S, p.mat[1].row_bytes, region_up, lane); });
+    if (q8) stream_scales((const u8*)(m.wd + row0 * S), nrows * S * 2, (u8*)scales, lane);
+    if (p.glu) {
+      with_format<FSET>(ufmt, [&](auto F) { nup = stream_run<decltype(F)::value>(wu, row0, nrows, S, p.mat[1].row_bytes, region_up, lane); });
+      if (q8) nup += stream_scales((const u8*)(p.mat[1].wd + row0 * S), nrows * S * 2, (u8*)scales_up, lane);
+    }
   }
   if (p.norm_w) { ilt_barrier_lds(); ilt_barrier_lds(); ilt_barrier_lds(); }      // in step with norm_scale_stagers
   // The barrier is for the activations only, so it comes before this wave waits for its rows (no
@@ -908,17 +947,17 @@ __global__ __launch_bounds__(kStreamThreads) void gemv_stream_kernel(IltGemvPara
   else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 
   const int zx = p.x_stride ? z : 0;
-  const Lds L = { lxq + (long)zx * S * XP, lxs + zx * S, lbs + zx * S * 16, lgrid };
-  with_format<FSET>(fmt, [&](auto F) { wave_rows_lds<decltype(F)::value>(region, nrows, S, p.s_magic, L, tw, lane); });
+  const Lds L = { q8 ? lxq : lxq + (long)zx * S * XP, lxs + zx * S, lbs + zx * S * 16, lgrid };
+  with_format<FSET>(fmt, [&](auto F) { wave_rows_lds<decltype(F)::value>(region, scales, nrows, S, p.s_magic, L, tw, lane); });
   if (p.glu) {
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    with_format<FSET>(ufmt, [&](auto F) { wave_rows_lds<decltype(F)::value>(region_up, nrows, S, p.s_magic, L, tw + (long)p.batch * tpr, lane); });
+    with_format<FSET>(ufmt, [&](auto F) { wave_rows_lds<decltype(F)::value>(region_up, scales_up, nrows, S, p.s_magic, L, tw + (long)p.batch * tpr, lane); });
   }
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
   __builtin_amdgcn_wave_barrier();
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
   if (lane < nrows) {
-    const int tper = (fmt == ILT_Q4_K || fmt == ILT_Q2_K) ? 2 : 1, uper = (ufmt == ILT_Q4_K || ufmt == ILT_Q2_K) ? 2 : 1;
+    const int tper = (fmt == ILT_Q4_K || fmt == ILT_Q2_K) ? 2 : 1, uper = (ufmt == ILT_Q4_K || ufmt == ILT_Q2_K) ? 2 : 1;      // floats a block
     float v = sum_any(fmt, tw + (long)lane * S * tper, S);
     const long r = row0 + lane;
     float* y = m.y + (long)z * p.y_stride;
@@ -1010,12 +1049,14 @@ static hipError_t gemv_stream_launch(IltGemvParams& p, int fset, int nz, hipStre
   const char* force = getenv("ILT_GEMV_STREAM");          // "0": never (tests)
   if (force && atoi(force) == 0) return hipErrorNotSupported;
   const bool experts = p.ptrs != nullptr;
-  if (experts ? !(fset == ILT_IQ2_XXS || fset == ILT_Q2_K) : !(fset == 0 || fset == ILT_Q4_K || fset == ILT_Q6_K)) return hipErrorNotSupported;
-  if (p.group_rows > 0 || (!experts && (nz != 1 || p.glu > 1)) || (experts && (p.norm_w || !(p.x_stride == 0 || p.x_stride == p.cols))))
+  const bool q8 = fset == ILT_Q8_0;
+  if (experts ? !(fset == ILT_IQ2_XXS || fset == ILT_Q2_K) : !(fset == 0 || fset == ILT_Q4_K || fset == ILT_Q6_K || q8)) return hipErrorNotSupported;
+  if (p.group_rows > 0 || (!experts && nz != 1) || (!experts && !q8 && p.glu > 1) || (experts && (p.norm_w || !(p.x_stride == 0 || p.x_stride == p.cols))))
     return hipErrorNotSupported;
-  const int S = p.cols / 256;
+  if (q8 && (p.norm_w || (p.cols / 32) % 2 != 0)) return hipErrorNotSupported;      // the scales go four bytes at a time
+  const int S = q8 ? p.cols / 32 : p.cols / 256;
   const int nx = p.x_stride ? nz : 1;
-  if (p.xf && p.norm_w ? S > 64 : (long)S * nx > 64 * 3) return hipErrorNotSupported;
+  if (!q8 && (p.xf && p.norm_w ? S > 64 : (long)S * nx > 64 * 3)) return hipErrorNotSupported;
   const int nm = (p.glu || experts) ? 1 : p.nmat;
   long total_rows = 0, bytes = 0;
   for (int i = 0; i < nm; i++) { total_rows += p.mat[i].rows; bytes += (long)p.mat[i].rows * p.mat[i].row_bytes; }
@@ -1059,19 +1100,22 @@ static hipError_t gemv_stream_launch(IltGemvParams& p, int fset, int nz, hipStre
   p.nz = nz;
   const int nglu = p.glu ? 2 : 1;
   const int lb = fset == ILT_Q4_K ? 144 : fset == ILT_IQ2_XXS ? 80 : fset == ILT_Q2_K ? 96 : 224;      // Q6_K's spread blocks at worst
-  const long one = (long)batch * S * lb;                              // a wave's rows of one matrix
+  // a wave's rows of one matrix (Q8_0: the quants, then the scales, rounded to 16 bytes)
+  const long one = q8 ? ((long)batch * (p.cols + 2 * S) + 15) / 16 * 16 : (long)batch * S * lb;
   p.region = (int)(one * nglu);
-  const size_t smem = (size_t)S * nx * XP + (fset == ILT_IQ2_XXS ? 3072 : (size_t)S * nx * 16 * 4) + (size_t)S * nx * 4 + 16 +
-                      (size_t)kRowWaves * batch * S * 2 * 4 * nglu + (size_t)kRowWaves * p.region;
+  const size_t xbytes = q8 ? (size_t)p.cols + (size_t)S * 4
+                           : (size_t)S * nx * XP + (fset == ILT_IQ2_XXS ? 3072 : (size_t)S * nx * 16 * 4) + (size_t)S * nx * 4;
+  const size_t smem = xbytes + 16 + (size_t)kRowWaves * batch * S * (q8 ? 1 : 2) * 4 * nglu + (size_t)kRowWaves * p.region;
   if (smem > 156 * 1024) return hipErrorNotSupported;
   p.s_magic = (uint32_t)(0x100000000ULL / (uint64_t)S) + 1;
   static bool attr_set[8] = {};
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 8) dev = 0;
   if (!attr_set[dev]) {            // more dynamic LDS than the default 64 KB: asked for once per device
-    const void* kernels[5] = { (const void*)gemv_stream_kernel<0>, (const void*)gemv_stream_kernel<ILT_Q4_K>, (const void*)gemv_stream_kernel<ILT_Q6_K>,
-                               (const void*)gemv_stream_kernel<ILT_IQ2_XXS>, (const void*)gemv_stream_kernel<ILT_Q2_K> };
-    for (int i = 0; i < 5; i++)
+    const void* kernels[6] = { (const void*)gemv_stream_kernel<0>, (const void*)gemv_stream_kernel<ILT_Q4_K>, (const void*)gemv_stream_kernel<ILT_Q6_K>,
+                               (const void*)gemv_stream_kernel<ILT_IQ2_XXS>, (const void*)gemv_stream_kernel<ILT_Q2_K>,
+                               (const void*)gemv_stream_kernel<ILT_Q8_0> };
+    for (int i = 0; i < 6; i++)
       if (hipFuncSetAttribute(kernels[i], hipFuncAttributeMaxDynamicSharedMemorySize, 158 * 1024) != hipSuccess) {
         (void)hipGetLastError();
         return hipErrorNotSupported;
@@ -1084,6 +1128,7 @@ static hipError_t gemv_stream_launch(IltGemvParams& p, int fset, int nz, hipStre
     case ILT_Q4_K: hipLaunchKernelGGL(gemv_stream_kernel<ILT_Q4_K>, grid, dim3(kStreamThreads), smem, st, p); break;
     case ILT_Q6_K: hipLaunchKernelGGL(gemv_stream_kernel<ILT_Q6_K>, grid, dim3(kStreamThreads), smem, st, p); break;
     case ILT_IQ2_XXS: hipLaunchKernelGGL(gemv_stream_kernel<ILT_IQ2_XXS>, grid, dim3(kStreamThreads), smem, st, p); break;
+    case ILT_Q8_0: hipLaunchKernelGGL(gemv_stream_kernel<ILT_Q8_0>, grid, dim3(kStreamThreads), smem, st, p); break;
     default: hipLaunchKernelGGL(gemv_stream_kernel<ILT_Q2_K>, grid, dim3(kStreamThreads), smem, st, p); break;
   }
   g_streamed_launches++;

@@ -397,7 +397,8 @@ def test_streamed_products_bit_exact(dev, monkeypatch, stream):
     before = count()
     rng = synth.make_rng(4242)
     for qtype, rows, cols in ((synth.Q4_K, 2560, 4096), (synth.Q6_K, 2560, 9728), (synth.Q6_K, 1030, 2560),
-                              (synth.Q4_K, 16384, 1024), (synth.Q4_K, 3000, 12288), (synth.Q6_K, 9000, 256)):
+                              (synth.Q4_K, 16384, 1024), (synth.Q4_K, 3000, 12288), (synth.Q6_K, 9000, 256),
+                              (synth.Q8_0, 4864, 896), (synth.Q8_0, 896, 4864)):
         w = synth.weights(qtype, rows, cols, rng)
         x = special_activations(cols, rng)
         bias = synth.activations(rows, rng)
@@ -406,7 +407,7 @@ def test_streamed_products_bit_exact(dev, monkeypatch, stream):
         want = orc.matmul(qtype, w, rows, cols, x)
         dense.mv_multi(dev, [(m, y, None)], xf=xb)
         assert np.array_equal(bits(hip.hip_floats(y, rows)), bits(want)), (qtype, rows, cols, "float x")
-        act = dense.QAct(dev, 1, cols, ("q8k",))
+        act = dense.QAct(dev, 1, cols, ("q8",) if qtype == synth.Q8_0 else ("q8k",))
         dense.quantize_act(dev, xb, act)
         dense.mv_multi(dev, [(m, y, bb)], act, acc=True)
         assert np.array_equal(bits(hip.hip_floats(y, rows)), bits(want + (want + bias))), (qtype, rows, cols, "quantized x, bias, acc")
@@ -448,6 +449,6 @@ def test_streamed_products_bit_exact(dev, monkeypatch, stream):
         hip.hip_free(b)
     for m in ms + [gm, um]:
         m.free()
-    # 5 shapes x 2 launches + Q/K/V + 3 x Q/K/V with the norm took the streamed variant (9000 x 256 is
+    # 7 shapes x 2 launches + Q/K/V + 3 x Q/K/V with the norm took the streamed variant (9000 x 256 is
     # under 2 MB; a Q4_K gate with a Q6_K up of 9728 rows does not fit a CU's LDS)
-    assert count() - before == (14 if stream == "1" else 0)
+    assert count() - before == (18 if stream == "1" else 0)
