@@ -49,13 +49,13 @@ def _t(fetch_kib, write_kib):
     return int((2 * fetch_kib + write_kib) * 1024)
 
 
-TRAFFIC = {"c1": {"up": _t(2358.0, 22.0), "down": _t(2418.0, 7.0)},
-           "c2": {"qkv": _t(4879.9, 33.3), "wo": _t(3066.0, 12.0), "glu": _t(13872.2, 48.0), "down": _t(10383.6, 12.0),
-                  "head": _t(175754.1, 634.8)},
+TRAFFIC = {"c1": {"up": _t(2507.3, 96.0), "down": _t(2443.0, 28.0)},
+           "c2": {"qkv": _t(4935.6, 96.0), "wo": _t(3043.9, 80.0), "glu": _t(14065.8, 116.0), "down": _t(10506.2, 80.0),
+                  "head": _t(175546.1, 636.4)},
            # one product: two-pass = the 256-tile launch plus the 128-tile launch for the rows left over
            "c3": {"bf16-1pass": _t(519803.0, 278528.0), "bf16-2pass": _t(491863.8 + 61498.0, 262144.0 + 16384.0),
                   "bf16-resident": _t(491863.8 + 61498.0, 262144.0 + 16384.0)},
-           "c4": {"d4_mv_glu_iq2_xxs": _t(12952.9, 63.8), "d4_mv_q2_k_f32": _t(8381.6, 96.4), "d4_mvq8_glu": _t(8860.1, 16.0)},
+           "c4": {"d4_mv_glu_iq2_xxs": _t(12854.8, 96.0), "d4_mv_q2_k_f32": _t(8394.5, 96.0), "d4_mvq8_glu": _t(8833.8, 96.0)},
            "c5": {"d4_mm_id_bf16": _t((2 * 305779.3 + 367082.0) / 3, (2 * 196608.0 + 393216.0) / 3)}}
 
 

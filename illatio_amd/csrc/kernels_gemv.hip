@@ -15,6 +15,10 @@
 //      the result has the CPU path's bits.
 // One launch may cover several matrices that share x (Q, K, V; gate and up), and may end
 // in silu(gate)*up (swiglu!, model.lisp:364-378).
+// Two kernels share those phases: gemv_kernel walks its rows with loads two steps ahead (any
+// size; the 300 MB output head), gemv_stream_kernel has every wave ask for all of its rows at
+// once as direct loads into LDS (products of 2 MB and more whose share fits a CU's LDS).  The
+// host chooses (ilt_gemv_launch).
 #include "ilt_device.h"
 #include "ilt_iq2xxs_tables.h"
 #include "ilt_kernels.h"
@@ -661,14 +665,12 @@ __global__ __launch_bounds__(kThreads) void gemv_kernel(IltGemvParams p) {
   asm volatile("" :: "v"(warm[0]), "v"(warm[1]), "v"(warm[2]), "v"(warm[3]));
 }
 
-// ---- the streamed variant: Q4_K / Q6_K matrices of up to ~100 KB per CU ----------------------------
+// ---- the streamed variant: matrices of up to ~100 KB per CU, every format ---------------------------
 // A mid-size product (6-28 MB) is over before its loop's load -> use -> load chain has made a few
-// round trips to memory: its time is latency, not bytes.  Here every wave asks for its whole
-// share of the rows at once, as direct loads from global memory into its own piece of LDS,
-// before anything else but the activations' loads (which must go first: loads return in the
-// order they were issued); the matrix streams in at the memory's rate while the activations
-// are quantized, and the blocks' terms are then formed from LDS.  One workgroup a CU, one
-// batch of rows a wave.
+// round trips to memory: its time is latency, not bytes.  Here every row wave asks for its whole
+// share of the rows at once, as direct loads from global memory into its own piece of LDS; the
+// matrix streams in at the memory's rate while other waves quantize the activations, and the
+// blocks' terms are then formed from LDS.  One workgroup a CU, one batch of rows a wave.
 // A block in LDS: LB bytes as PPB pieces of 16 bytes, every piece 16-byte aligned there whatever the
 // block's size in memory (BB); goff(pc) = where piece pc comes from within the block.  No piece
 // reaches past its block's end (the last block of a matrix may be the last bytes of an allocation).
