@@ -264,6 +264,54 @@ __device__ __forceinline__ void store_tile(const v16f (&acc)[NA][NB], const BfPa
   }
 }
 
+// Which tile a workgroup takes: row tile rt, tokens tok0 .. tok0+ntok-1 (of expert z's group,
+// with w its matrix, when grouped).  Tiles are numbered so that the eight XCDs' workgroups (the
+// hardware deals them round-robin) each walk a contiguous run, GR row tiles of one token tile
+// after another.  False: none (the grid is rounded up).  S: scan[256], tile_z, tile_t0, tile_n.
+template <int TM, int TN, typename SM>
+__device__ __forceinline__ bool pick_tile(const BfParams& p, SM& S, long& tok0, int& ntok, int& rt, const u8*& w) {
+  const int t = threadIdx.x;
+  const int NR = (p.rows + TM - 1) / TM;
+  int NT;
+  if (p.ptrs) {
+    if (t < 256) S.scan[t] = t < p.ne ? (p.counts[t] + TN - 1) / TN : 0;
+    __syncthreads();
+    for (int off = 1; off < 256; off <<= 1) {
+      const u32 v = (t < 256 && t >= off) ? S.scan[t - off] : 0;
+      __syncthreads();
+      if (t < 256) S.scan[t] += v;
+      __syncthreads();
+    }
+    NT = (int)S.scan[255];
+  } else {
+    NT = (p.ntok + TN - 1) / TN;
+  }
+  const int total = NT * NR, per = (total + 7) / 8;
+  const int L = blockIdx.x, j = L >> 3;
+  const int s = (L & 7) * per + j;
+  if (j >= per || s >= total) return false;
+  const int rg = s / (GR * NT), rem = s - rg * GR * NT, nr = min(GR, NR - rg * GR);
+  const int tt = rem / nr;
+  rt = rg * GR + (rem - tt * nr);
+  if (p.ptrs) {
+    if (t < p.ne) {
+      const u32 incl = S.scan[t], tiles = (p.counts[t] + TN - 1) / TN, excl = incl - tiles;
+      if ((u32)tt >= excl && (u32)tt < incl) {
+        S.tile_z = t;
+        S.tile_t0 = (int)(p.bases[t] + ((u32)tt - excl) * TN);
+        S.tile_n = (int)min((u32)TN, p.counts[t] - ((u32)tt - excl) * TN);
+      }
+    }
+    __syncthreads();
+    tok0 = S.tile_t0; ntok = S.tile_n;
+    w = (const u8*)(p.ptrs[S.tile_z] + p.add);
+  } else {
+    tok0 = (long)tt * TN;
+    ntok = min(TN, p.ntok - (int)tok0);
+  }
+  return true;
+}
+
 // TM rows x TN tokens per workgroup; wave w: rows 32*NB*(w/2).., tokens (TN/2)*(w%2)..: NA x NB
 // patches of 32x32.  NB = 2: 2*TM threads, two per row (a thread dequantizes 16 weights a step);
 // NB = 4: TM threads, one per row (32 weights a step).
@@ -278,49 +326,9 @@ __global__ __launch_bounds__((bf16_threads<TM, NB>()), (TM * TN == 65536 ? 1 : T
   constexpr int NI = 4 * TN / THREADS;   // direct-load instructions per wave and step
   constexpr int WL = WRaw<FMT>::LOADS * NE;
   const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
-  const int NR = (p.rows + TM - 1) / TM;
 
-  // ---- which tile ----
   long tok0; int ntok, rt; const u8* w = p.w;
-  {
-    int NT;
-    if (p.ptrs) {
-      if (t < 256) S.scan[t] = t < p.ne ? (p.counts[t] + TN - 1) / TN : 0;
-      __syncthreads();
-      for (int off = 1; off < 256; off <<= 1) {
-        const u32 v = (t < 256 && t >= off) ? S.scan[t - off] : 0;
-        __syncthreads();
-        if (t < 256) S.scan[t] += v;
-        __syncthreads();
-      }
-      NT = (int)S.scan[255];
-    } else {
-      NT = (p.ntok + TN - 1) / TN;
-    }
-    const int total = NT * NR, per = (total + 7) / 8;
-    const int L = blockIdx.x, j = L >> 3;
-    const int s = (L & 7) * per + j;
-    if (j >= per || s >= total) return;
-    const int rg = s / (GR * NT), rem = s - rg * GR * NT, nr = min(GR, NR - rg * GR);
-    const int tt = rem / nr;
-    rt = rg * GR + (rem - tt * nr);
-    if (p.ptrs) {
-      if (t < p.ne) {
-        const u32 incl = S.scan[t], tiles = (p.counts[t] + TN - 1) / TN, excl = incl - tiles;
-        if ((u32)tt >= excl && (u32)tt < incl) {
-          S.tile_z = t;
-          S.tile_t0 = (int)(p.bases[t] + ((u32)tt - excl) * TN);
-          S.tile_n = (int)min((u32)TN, p.counts[t] - ((u32)tt - excl) * TN);
-        }
-      }
-      __syncthreads();
-      tok0 = S.tile_t0; ntok = S.tile_n;
-      w = (const u8*)(p.ptrs[S.tile_z] + p.add);
-    } else {
-      tok0 = (long)tt * TN;
-      ntok = min(TN, p.ntok - (int)tok0);
-    }
-  }
+  if (!pick_tile<TM, TN>(p, S, tok0, ntok, rt, w)) return;
   const int r0 = rt * TM;
   if (FMT == ILT_IQ2_XXS) {
     if (t < 256) iq2_tables_fill(S.iq2, t);
@@ -437,6 +445,216 @@ __global__ __launch_bounds__((bf16_threads<TM, NB>()), (TM * TN == 65536 ? 1 : T
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // the tail's redundant loads: nothing may land in LDS after the workgroup ends
 
   store_tile<NA, NB>(acc, p, tok0, ntok, r0, wt0, wr0, l32, lh);
+}
+
+// ---- the grouped product with the weights dequantized into MFMA operands ------------------------
+// An expert's group of a prefill chunk is a hundred rows of tokens or so: one token tile, so
+// every weight is dequantized once whichever way, and the kernel above then spends more of the
+// LDS's bandwidth on weights (the slab written, then read by two waves as fragments) than on
+// anything else.  Here a wave keeps 64 rows of W to itself, over all of the tile's 128 tokens:
+// lane (l32, lh) dequantizes the 8 weights of a row that make up its share of an MFMA's B
+// operand -- columns 16*kk + 8*lh .. + 7 of the step, of row 32*b + l32 -- straight into
+// registers, and only the activations go through LDS.  The token patches past the group's last
+// row are skipped (a group of 40 rows takes half the MFMAs of one of 128).
+template <int FMT> struct RegB;
+
+// IQ2_XXS: a lane's raw set covers two steps (a quarter of a super-block: two groups of 32
+// weights, 8 bytes each) of a row.
+template <> struct RegB<ILT_IQ2_XXS> {
+  static constexpr int P = 2, LOADS = 2;               // steps a set covers, load instructions a set
+  struct Raw { int4 q; u32 d; };
+  struct Prep { u32 g, sg, t01, t2; };
+  static __device__ __forceinline__ void load(Raw& r, __amdgpu_buffer_rsrc_t rw, u32 rowoff, int unit, int lh) {
+    const u32 b = rowoff + (u32)(unit >> 2) * 66;
+    r.q = ilt_bld16(rw, b + 2 + 16 * (unit & 3));
+    r.d = ilt_bld2(rw, b);
+  }
+  // j: the step within the set.  The three magnitudes as dequant16_pk makes them.
+  static __device__ __forceinline__ Prep prep(const Raw& r, int j, int lh) {
+    const u32 aux = word_of(r.q, 2 * j + 1);
+    const float db = (ilt_h2f((u16)r.d) * (0.5f + (float)(aux >> 28))) * 0.25f;
+    return { word_of(r.q, 2 * j) >> (8 * lh), aux >> (7 * lh), pack_bf16(db * 8.0f, db * 25.0f), pack_bf16(db * 43.0f, 0.0f) };
+  }
+  // the lane's 8 weights of unit kk of the step
+  static __device__ __forceinline__ v8bf frag(const Raw&, const Prep& pr, int j, int kk, int lh, const Iq2Tables* T) {
+    const int4 sel = ilt_lds_ld16(T->sel[(pr.g >> (16 * kk)) & 0xFF]);
+    const int4 sm = ilt_lds_ld16(T->sgn[(pr.sg >> (14 * kk)) & 127]);
+    u32 pk[4];
+    pk[0] = __builtin_amdgcn_perm(pr.t2, pr.t01, (u32)sel.x) ^ (u32)sm.x;
+    pk[1] = __builtin_amdgcn_perm(pr.t2, pr.t01, (u32)sel.y) ^ (u32)sm.y;
+    pk[2] = __builtin_amdgcn_perm(pr.t2, pr.t01, (u32)sel.z) ^ (u32)sm.z;
+    pk[3] = __builtin_amdgcn_perm(pr.t2, pr.t01, (u32)sel.w) ^ (u32)sm.w;
+    v8bf out; __builtin_memcpy(&out, pk, 16); return out;
+  }
+};
+
+// Q2_K: a set covers four steps (half a super-block: its 128 weights share 32 bytes of quants,
+// of which the lane needs 8 for each of the two units, and 8 scale bytes).
+template <> struct RegB<ILT_Q2_K> {
+  static constexpr int P = 4, LOADS = 4;
+  struct Raw { int2 qa, qb, sc; u32 dd; };
+  struct Prep {};
+  static __device__ __forceinline__ void load(Raw& r, __amdgpu_buffer_rsrc_t rw, u32 rowoff, int unit, int lh) {
+    const u32 b = rowoff + (u32)(unit >> 1) * 84;
+    r.qa = ilt_bld8(rw, b + 16 + 32 * (unit & 1) + 8 * lh);
+    r.qb = ilt_bld8(rw, b + 32 + 32 * (unit & 1) + 8 * lh);
+    r.sc = ilt_bld8(rw, b + 8 * (unit & 1));
+    r.dd = ilt_bld4(rw, b + 80);
+  }
+  static __device__ __forceinline__ Prep prep(const Raw& r, int j, int lh) {
+    return {};
+  }
+  static __device__ __forceinline__ v8bf frag(const Raw& r, const Prep& pr, int j, int kk, int lh, const Iq2Tables*) {
+    const u32 scw = ((u32)(j < 2 ? r.sc.x : r.sc.y) >> (16 * (j & 1) + 8 * kk)) & 0xFF;
+    const float dl = ilt_h2f((u16)(r.dd & 0xFFFF)) * (float)(scw & 15), ml = ilt_h2f((u16)(r.dd >> 16)) * (float)(scw >> 4);
+    const int2 qq = kk ? r.qb : r.qa;
+    u32 pk[4];
+#pragma unroll
+    for (int i = 0; i < 2; i++) {
+      const u32 v = ((u32)(i ? qq.y : qq.x) >> (2 * j)) & 0x03030303;
+      float o[4];
+#pragma unroll
+      for (int k = 0; k < 4; k++) o[k] = __builtin_fmaf(dl, (float)((v >> (8 * k)) & 0xFF), -ml);   // dl*q is exact in fp32
+      pk[2 * i] = pack_bf16(o[0], o[1]);
+      pk[2 * i + 1] = pack_bf16(o[2], o[3]);
+    }
+    v8bf out; __builtin_memcpy(&out, pk, 16); return out;
+  }
+};
+
+struct RegbSmem {
+  __align__(16) u8 xs[3][128 * KS * 2];
+  Iq2Tables iq2;
+  u32 scan[256];
+  int tile_z, tile_t0, tile_n;
+};
+
+template <int FMT>
+__global__ __launch_bounds__(256, 2) void gemm_bf16_regb_kernel(BfParams p) {
+  constexpr int TM = 256, TN = 128, NA = 4, NB = 2, NI = 2;
+  typedef RegB<FMT> R;
+  constexpr int P = R::P, WL = R::LOADS * NB;
+  typedef typename R::Raw Raw;
+  typedef typename R::Prep Prep;
+  __shared__ RegbSmem S;
+  const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+
+  long tok0; int ntok, rt; const u8* w = p.w;
+  if (!pick_tile<TM, TN>(p, S, tok0, ntok, rt, w)) return;
+  const int r0 = rt * TM;
+  if (FMT == ILT_IQ2_XXS) {
+    iq2_tables_fill(S.iq2, t);
+    __syncthreads();
+  }
+
+  const int l32 = lane & 31, lh = lane >> 5, wr0 = 64 * wave;
+  const __amdgpu_buffer_rsrc_t rw = ilt_rsrc(ilt_uniform_ptr(w), (u32)min((long long)p.rows * p.row_bytes, 0xFFFFFFF0LL));
+  u32 wrowoff[NB];
+#pragma unroll
+  for (int b = 0; b < NB; b++) wrowoff[b] = (u32)((long long)min(r0 + wr0 + 32 * b + l32, p.rows - 1) * p.row_bytes);
+  const u8* xbase = (const u8*)ilt_uniform_ptr(p.rmap ? p.x : p.x + tok0 * (long)p.cols);
+  u32 xoff[NI];
+#pragma unroll
+  for (int i = 0; i < NI; i++) {
+    const int P_ = (wave * NI + i) * 64 + lane, tok = P_ >> 2, kp = (P_ & 3) ^ (int)slab_swz(tok);
+    const int tk = min(tok, ntok - 1);
+    xoff[i] = (p.rmap ? p.rmap[tok0 + tk] : (u32)tk) * (u32)p.cols * 2 + 16 * kp;
+  }
+
+  v16f acc[NA][NB];
+#pragma unroll
+  for (int a = 0; a < NA; a++)
+#pragma unroll
+    for (int b = 0; b < NB; b++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) acc[a][b][r] = 0.0f;
+  u32 aoff[NA];
+#pragma unroll
+  for (int a = 0; a < NA; a++) aoff[a] = slab_off(32 * a + l32, lh);
+
+  const int nk = p.cols / KS, nu = nk / P;                 // steps, raw sets a row
+  auto issue_x = [&](int stage, int ks) {
+#pragma unroll
+    for (int i = 0; i < NI; i++) ilt_g2lds16(xbase + ks * (KS * 2) + xoff[i], S.xs[stage] + (wave * NI + i) * 1024);
+  };
+  auto load_raw = [&](Raw* raw, int unit) {
+#pragma unroll
+    for (int b = 0; b < NB; b++) R::load(raw[b], rw, wrowoff[b], unit, lh);
+  };
+
+  // Raw sets A and B take turns, P steps each.  Half-step (ks, kk) multiplies with bq[kk] and
+  // makes the operands of the half-step after it: (ks, 1) during (ks, 0), (ks+1, 0) during
+  // (ks, 1).  So set A is last read in the first half of the step that ends its turn, and the
+  // step after that one loads it again, 2P-1 steps before its next turn starts.
+  Raw rawa[NB], rawb[NB];
+  Prep pr[NB];
+  v8bf bq[2][NB];
+  load_raw(rawa, 0);
+  issue_x(0, 0);
+  issue_x(1, 1);
+#pragma unroll
+  for (int b = 0; b < NB; b++) { pr[b] = R::prep(rawa[b], 0, lh); bq[0][b] = R::frag(rawa[b], pr[b], 0, 0, lh, &S.iq2); }
+
+  auto run = [&](auto NALc) {
+    constexpr int NAL = decltype(NALc)::value;               // token patches that hold rows
+    int st0 = 0, st1 = 1, st2 = 2;
+    auto step = [&](int ks, auto Jc) {
+      constexpr int J = decltype(Jc)::value;                 // the step's place in a round of both sets
+      // All loads but the previous step's have landed: this step's x slab has (sent two steps ago).
+      constexpr int prev = NI + (J % P == 1 ? WL : 0);
+      asm volatile("s_waitcnt vmcnt(%0)" :: "n"(prev) : "memory");
+      ilt_barrier_lds();                                     // no fence: later steps' loads stay in flight
+      if (J == 0) load_raw(rawb, min(ks / P + 1, nu - 1));
+      if (J == P) load_raw(rawa, min(ks / P + 1, nu - 1));
+      issue_x(st2, min(ks + 2, nk - 1));
+      __builtin_amdgcn_sched_barrier(0);
+      const u8* xs = S.xs[st0];
+      constexpr int J1 = (J + 1) % (2 * P);
+#pragma unroll
+      for (int kk = 0; kk < 2; kk++) {
+        v8bf af[NAL];
+#pragma unroll
+        for (int a = 0; a < NAL; a++) af[a] = *(const v8bf*)(xs + (aoff[a] ^ (32 * kk)));
+        if (kk == 0) {
+#pragma unroll
+          for (int b = 0; b < NB; b++) bq[1][b] = R::frag(J < P ? rawa[b] : rawb[b], pr[b], J % P, 1, lh, &S.iq2);
+        }
+#pragma unroll
+        for (int a = 0; a < NAL; a++)
+#pragma unroll
+          for (int b = 0; b < NB; b++) acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[a], bq[kk][b], acc[a][b], 0, 0, 0);
+        if (kk == 1) {       // (past the last step: operands nobody multiplies with)
+#pragma unroll
+          for (int b = 0; b < NB; b++) {
+            pr[b] = R::prep(J1 < P ? rawa[b] : rawb[b], J1 % P, lh);
+            bq[0][b] = R::frag(J1 < P ? rawa[b] : rawb[b], pr[b], J1 % P, 0, lh, &S.iq2);
+          }
+        }
+      }
+      const int s = st0; st0 = st1; st1 = st2; st2 = s;
+    };
+    for (int ks = 0; ks < nk; ks += 2 * P) {
+      step(ks + 0, std::integral_constant<int, 0>{});
+      step(ks + 1, std::integral_constant<int, 1>{});
+      step(ks + 2, std::integral_constant<int, 2>{});
+      step(ks + 3, std::integral_constant<int, 3>{});
+      if constexpr (P == 4) {
+        step(ks + 4, std::integral_constant<int, 4>{});
+        step(ks + 5, std::integral_constant<int, 5>{});
+        step(ks + 6, std::integral_constant<int, 6>{});
+        step(ks + 7, std::integral_constant<int, 7>{});
+      }
+    }
+  };
+  switch ((ntok + 31) >> 5) {
+    case 1: run(std::integral_constant<int, 1>{}); break;
+    case 2: run(std::integral_constant<int, 2>{}); break;
+    case 3: run(std::integral_constant<int, 3>{}); break;
+    default: run(std::integral_constant<int, 4>{}); break;
+  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // the tail's redundant loads: nothing may land in LDS after the workgroup ends
+
+  store_tile<NA, NB>(acc, p, tok0, ntok, r0, 0, wr0, l32, lh);
 }
 
 // ---- the two-pass product: W as plain bf16 ------------------------------------------------------
@@ -680,7 +898,15 @@ hipError_t ilt_k_gemm_bf16_id(int fmt, const uint64_t* ptrs, long long add, cons
   // an expert seldom has more than 128 rows of tokens in a chunk, and the taller tile reads a
   // quarter less from LDS per MFMA than 128 x 128.  "1" in ILT_BF16_ID_TILE: 128 x 128 always (tests).
   const char* force = getenv("ILT_BF16_ID_TILE");
-  if (rows % 256 == 0 && !(force && atoi(force) == 1)) {      // the expert formats (Q4_K / Q6_K raw sets would not fit the registers)
+  const int forced = force ? atoi(force) : 0;
+  if (rows % 256 == 0 && forced == 0 && (fmt == ILT_IQ2_XXS || fmt == ILT_Q2_K)) {      // weights straight into MFMA operands
+    const long long total = (total_rows / 128 + ne) * (rows / 256), per = (total + 7) / 8;
+    if (per * 8 > 0x7FFFFFFFLL) return hipErrorInvalidValue;
+    if (fmt == ILT_IQ2_XXS) hipLaunchKernelGGL(gemm_bf16_regb_kernel<ILT_IQ2_XXS>, dim3((unsigned)(per * 8)), dim3(256), 0, st, p);
+    else hipLaunchKernelGGL(gemm_bf16_regb_kernel<ILT_Q2_K>, dim3((unsigned)(per * 8)), dim3(256), 0, st, p);
+    return hipGetLastError();
+  }
+  if (rows % 256 == 0 && forced != 1) {      // the expert formats (Q4_K / Q6_K raw sets would not fit the registers)
     if (fmt == ILT_IQ2_XXS) return launch_bf16<ILT_IQ2_XXS, 256, 128, 4>(p, total_rows / 128 + ne, st);
     if (fmt == ILT_Q2_K) return launch_bf16<ILT_Q2_K, 256, 128, 4>(p, total_rows / 128 + ne, st);
   }

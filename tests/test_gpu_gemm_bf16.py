@@ -120,7 +120,9 @@ def exact_chunk(G, U, Dn, sel, ww, norms, clamp):
 
 @pytest.mark.parametrize("ne,d,ff,nu,n,clamp", [(8, 512, 256, 3, 37, 0.0), (16, 1024, 512, 4, 300, 0.6),
                                                  (12, 4096, 2048, 6, 96, 0.0)])
-@pytest.mark.parametrize("id_tile", [None, "1"])       # 256 x 128 tiles where the rows allow (the default), 128 x 128 always
+# the default (256 x 128 tiles with the weights dequantized into registers where the rows allow), 128 x 128 always,
+# 256 x 128 through LDS
+@pytest.mark.parametrize("id_tile", [None, "1", "2"])
 def test_moe_prefill_chunk_bf16_within_tolerance(dev, monkeypatch, ne, d, ff, nu, n, clamp, id_tile):
     """The prefill chunk of test_gpu_gemm.py with the three grouped products on the bf16
     matrix cores.  Routing, counts and weights stay equal to the CPU path's.  Each grouped
@@ -229,3 +231,44 @@ def test_two_pass_bf16_product(dev, monkeypatch, qtype, rows, cols, n, split):
     for b in (xf, xb, xs, bb, y1, y2, wb):
         hip.hip_free(b)
     m.free()
+
+
+@pytest.mark.parametrize("ne,d,ff,nu,n", [(8, 512, 256, 3, 37), (16, 1024, 512, 4, 300), (4, 1024, 256, 2, 333)])
+def test_grouped_product_variants_agree_bitwise(dev, monkeypatch, ne, d, ff, nu, n):
+    """The grouped product's variants make the same bf16 operands and add the same MFMA results
+    in the same order, so their outputs are equal bit for bit: groups of a few rows (token
+    patches skipped), of more than one tile of 128, and empty ones."""
+    from illatio_amd import ds4f, hip
+    rng = synth.make_rng(7 * ne + d + n)
+    gate = synth.weights(synth.IQ2_XXS, ne * ff, d, rng)
+    up = synth.weights(synth.IQ2_XXS, ne * ff, d, rng)
+    down = synth.weights(synth.Q2_K, ne * d, ff, rng)
+    norms = synth.activations((n, d), rng)
+    logits = synth.zipf_router_logits(n, ne, rng)
+    logits[:, ne - 1] = -30.0                             # an expert nobody picks
+    shared = synth.activations((n, d), rng)
+    pool = ds4f.ExpertPool(dev, ne, d, ff, gate, up, down)
+    lb, nb, sb = (hip.hip_upload_new(dev, a) for a in (logits, norms, shared))
+    res = {}
+    for tile in (None, "1", "2"):
+        if tile is None:
+            monkeypatch.delenv("ILT_BF16_ID_TILE", raising=False)
+        else:
+            monkeypatch.setenv("ILT_BF16_ID_TILE", tile)
+        keep = {}
+        moe = ds4f.ffn_routed_chunk_bf16(dev, pool, lb, nb, sb, n, ne, nu, 1.5, 0.0, keep=keep)
+        keep["out"] = hip.hip_floats(moe, n * d)
+        hip.hip_free(moe)
+        # a group's rows in the order of their tokens (the scatter's order within a group varies from run to run)
+        order = np.concatenate([int(b) + np.argsort(keep["rmap"][int(b):int(b) + int(c)], kind="stable")
+                                for b, c in zip(keep["bases"], keep["counts"])])
+        for k in ("gate", "up", "down"):
+            keep[k] = keep[k][order]
+        res[tile] = keep
+    assert int(res[None]["counts"][ne - 1]) == 0 and int(res[None]["counts"].max()) > (128 if n >= 300 else 0)
+    for tile in ("1", "2"):
+        for k in ("gate", "up", "down", "out"):
+            assert np.array_equal(res[None][k].view(np.uint32), res[tile][k].view(np.uint32)), (tile, k)
+    for b in (lb, nb, sb):
+        hip.hip_free(b)
+    pool.free()
