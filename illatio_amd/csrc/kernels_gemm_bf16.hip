@@ -451,23 +451,32 @@ __global__ __launch_bounds__((bf16_threads<TM, NB>()), (TM * TN == 65536 ? 1 : T
 // An expert's group of a prefill chunk is a hundred rows of tokens or so: one token tile, so
 // every weight is dequantized once whichever way, and the kernel above then spends more of the
 // LDS's bandwidth on weights (the slab written, then read by two waves as fragments) than on
-// anything else.  Here a wave keeps 64 rows of W to itself, over all of the tile's 128 tokens:
-// lane (l32, lh) dequantizes the 8 weights of a row that make up its share of an MFMA's B
-// operand -- columns 16*kk + 8*lh .. + 7 of the step, of row 32*b + l32 -- straight into
-// registers, and only the activations go through LDS.  The token patches past the group's last
-// row are skipped (a group of 40 rows takes half the MFMAs of one of 128).
+// anything else, and its per-lane loads of 16 or 32 bytes from as many rows as lanes ask the
+// memory pipeline for a whole line each.  Here
+//  - the quantized blocks go to LDS as they are, by direct loads of 16 bytes a lane from
+//    consecutive addresses (5 or 6 pieces a block, see RegB), a super-block (8 steps) of the
+//    tile's 256 rows at a time into one of two buffers, one load a wave and step;
+//  - a wave keeps 64 rows of W to itself, over all of the tile's 128 tokens: lane (l32, lh)
+//    dequantizes the 8 weights of a row that make up its share of an MFMA's B operand --
+//    columns 16*kk + 8*lh .. + 7 of the step, of row 32*b + l32 -- from the block in LDS straight
+//    into registers, and only the activations go through LDS as bf16;
+//  - the token patches past the group's last row are skipped (a group of 40 rows takes half
+//    the MFMAs of one of 128).
 template <int FMT> struct RegB;
 
-// IQ2_XXS: a lane's raw set covers two steps (a quarter of a super-block: two groups of 32
-// weights, 8 bytes each) of a row.
+// IQ2_XXS in LDS: 80 bytes a block, the 64 bytes of the eight groups first (four pieces from
+// byte 2 of the block on), then the block's first 16 bytes, which start with d.  A lane's raw
+// set covers two steps (a quarter of a super-block: two groups of 32 weights, 8 bytes each).
 template <> struct RegB<ILT_IQ2_XXS> {
-  static constexpr int P = 2, LOADS = 2;               // steps a set covers, load instructions a set
+  static constexpr int PPB = 5, LB = 80, BB = 66;
+  static constexpr int P = 2;                          // steps a set covers
+  static __device__ __forceinline__ u32 goff(u32 pc) { return pc == 4 ? 0u : 2 + 16 * pc; }
   struct Raw { int4 q; u32 d; };
   struct Prep { u32 g, sg, t01, t2; };
-  static __device__ __forceinline__ void load(Raw& r, __amdgpu_buffer_rsrc_t rw, u32 rowoff, int unit, int lh) {
-    const u32 b = rowoff + (u32)(unit >> 2) * 66;
-    r.q = ilt_bld16(rw, b + 2 + 16 * (unit & 3));
-    r.d = ilt_bld2(rw, b);
+  // u: the set's place in the super-block
+  static __device__ __forceinline__ void load(Raw& r, const u8* blk, int u, int lh) {
+    r.q = ilt_lds_ld16(blk + 16 * u);
+    r.d = *(const ILT_LDS u16*)(blk + 64);
   }
   // j: the step within the set.  The three magnitudes as dequant16_pk makes them.
   static __device__ __forceinline__ Prep prep(const Raw& r, int j, int lh) {
@@ -488,23 +497,24 @@ template <> struct RegB<ILT_IQ2_XXS> {
   }
 };
 
-// Q2_K: a set covers four steps (half a super-block: its 128 weights share 32 bytes of quants,
-// of which the lane needs 8 for each of the two units, and 8 scale bytes).
+// Q2_K in LDS: 96 bytes a block, its first 80 bytes (16 scale bytes, 64 of quants) as five
+// pieces, then bytes 68..83, whose last four are d and dmin: they land at 92.  A set covers
+// four steps (half a super-block: its 128 weights share 32 bytes of quants, of which the lane
+// needs 8 for each of the two units, and 8 scale bytes).
 template <> struct RegB<ILT_Q2_K> {
-  static constexpr int P = 4, LOADS = 4;
+  static constexpr int PPB = 6, LB = 96, BB = 84;
+  static constexpr int P = 4;
+  static __device__ __forceinline__ u32 goff(u32 pc) { return pc == 5 ? 68u : 16 * pc; }
   struct Raw { int2 qa, qb, sc; u32 dd; };
   struct Prep {};
-  static __device__ __forceinline__ void load(Raw& r, __amdgpu_buffer_rsrc_t rw, u32 rowoff, int unit, int lh) {
-    const u32 b = rowoff + (u32)(unit >> 1) * 84;
-    r.qa = ilt_bld8(rw, b + 16 + 32 * (unit & 1) + 8 * lh);
-    r.qb = ilt_bld8(rw, b + 32 + 32 * (unit & 1) + 8 * lh);
-    r.sc = ilt_bld8(rw, b + 8 * (unit & 1));
-    r.dd = ilt_bld4(rw, b + 80);
+  static __device__ __forceinline__ void load(Raw& r, const u8* blk, int u, int lh) {
+    r.qa = ilt_lds_ld8(blk + 16 + 32 * u + 8 * lh);
+    r.qb = ilt_lds_ld8(blk + 32 + 32 * u + 8 * lh);
+    r.sc = ilt_lds_ld8(blk + 8 * u);
+    r.dd = *(const ILT_LDS u32*)(blk + 92);
   }
-  static __device__ __forceinline__ Prep prep(const Raw& r, int j, int lh) {
-    return {};
-  }
-  static __device__ __forceinline__ v8bf frag(const Raw& r, const Prep& pr, int j, int kk, int lh, const Iq2Tables*) {
+  static __device__ __forceinline__ Prep prep(const Raw&, int j, int lh) { return {}; }
+  static __device__ __forceinline__ v8bf frag(const Raw& r, const Prep&, int j, int kk, int lh, const Iq2Tables*) {
     const u32 scw = ((u32)(j < 2 ? r.sc.x : r.sc.y) >> (16 * (j & 1) + 8 * kk)) & 0xFF;
     const float dl = ilt_h2f((u16)(r.dd & 0xFFFF)) * (float)(scw & 15), ml = ilt_h2f((u16)(r.dd >> 16)) * (float)(scw >> 4);
     const int2 qq = kk ? r.qb : r.qa;
@@ -522,36 +532,41 @@ template <> struct RegB<ILT_Q2_K> {
   }
 };
 
-struct RegbSmem {
-  __align__(16) u8 xs[3][128 * KS * 2];
-  Iq2Tables iq2;
-  u32 scan[256];
-  int tile_z, tile_t0, tile_n;
-};
+struct TileSel { u32 scan[256]; int tile_z, tile_t0, tile_n, pad; };
+
+// dynamic LDS: the x ring, the two buffers of blocks, the tile choice's scratch, IQ2_XXS's tables
+template <int FMT> constexpr size_t regb_smem() {
+  return 3 * 128 * KS * 2 + 2 * 256 * RegB<FMT>::LB + sizeof(TileSel) + (FMT == ILT_IQ2_XXS ? sizeof(Iq2Tables) : 0);
+}
 
 template <int FMT>
 __global__ __launch_bounds__(256, 2) void gemm_bf16_regb_kernel(BfParams p) {
   constexpr int TM = 256, TN = 128, NA = 4, NB = 2, NI = 2;
   typedef RegB<FMT> R;
-  constexpr int P = R::P, WL = R::LOADS * NB;
+  constexpr int P = R::P, UPS = 8 / P;                       // steps a raw set covers, sets a super-block
+  constexpr int NWW = TM * R::PPB / 64 / 4;                  // block loads a wave and super-block: 5 or 6
+  constexpr int WPS = P == 4 ? 2 : 1;                        // of which it sends this many a step, from step 0 on
+  constexpr int WSTEPS = (NWW + WPS - 1) / WPS;
+  constexpr int XS = TN * KS * 2, WS = TM * R::LB;
   typedef typename R::Raw Raw;
   typedef typename R::Prep Prep;
-  __shared__ RegbSmem S;
+  extern __shared__ __align__(16) u8 regb_lds[];
+  u8* const xsl = regb_lds;                                  // [3][XS]
+  u8* const wsl = regb_lds + 3 * XS;                         // [2][WS]
+  TileSel& S = *(TileSel*)(regb_lds + 3 * XS + 2 * WS);
+  const Iq2Tables* T = (const Iq2Tables*)(regb_lds + 3 * XS + 2 * WS + sizeof(TileSel));
   const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
 
   long tok0; int ntok, rt; const u8* w = p.w;
   if (!pick_tile<TM, TN>(p, S, tok0, ntok, rt, w)) return;
   const int r0 = rt * TM;
-  if (FMT == ILT_IQ2_XXS) {
-    iq2_tables_fill(S.iq2, t);
-    __syncthreads();
-  }
+  if (FMT == ILT_IQ2_XXS) iq2_tables_fill(*(Iq2Tables*)T, t);     // (a barrier follows, before the first operands are made)
 
   const int l32 = lane & 31, lh = lane >> 5, wr0 = 64 * wave;
-  const __amdgpu_buffer_rsrc_t rw = ilt_rsrc(ilt_uniform_ptr(w), (u32)min((long long)p.rows * p.row_bytes, 0xFFFFFFF0LL));
-  u32 wrowoff[NB];
-#pragma unroll
-  for (int b = 0; b < NB; b++) wrowoff[b] = (u32)((long long)min(r0 + wr0 + 32 * b + l32, p.rows - 1) * p.row_bytes);
+  // the pieces this lane sends to LDS for a super-block: piece 64*(wave + 4*i) + lane of the tile's 256 * PPB
+  const u8* wbase = (const u8*)ilt_uniform_ptr(w);
+  // (the addresses are made anew for every load: registers are scarcer than instruction slots)
+  const u32 wq0 = 64 * wave + lane, wrow_bytes = (u32)p.row_bytes, wlast = (u32)(p.rows - 1 - r0);
   const u8* xbase = (const u8*)ilt_uniform_ptr(p.rmap ? p.x : p.x + tok0 * (long)p.cols);
   u32 xoff[NI];
 #pragma unroll
@@ -568,56 +583,72 @@ __global__ __launch_bounds__(256, 2) void gemm_bf16_regb_kernel(BfParams p) {
     for (int b = 0; b < NB; b++)
 #pragma unroll
       for (int r = 0; r < 16; r++) acc[a][b][r] = 0.0f;
-  u32 aoff[NA];
-#pragma unroll
-  for (int a = 0; a < NA; a++) aoff[a] = slab_off(32 * a + l32, lh);
+  const u32 aoff0 = slab_off(l32, lh);                        // token 32a + l32: 2048a on (its swizzle is the same)
+  const u32 blk0 = (u32)(wr0 + l32) * R::LB;                  // this lane's first row's block in a buffer; the second 32 blocks on
 
-  const int nk = p.cols / KS, nu = nk / P;                 // steps, raw sets a row
+  const int nk = p.cols / KS, nsb = nk / 8;
   auto issue_x = [&](int stage, int ks) {
 #pragma unroll
-    for (int i = 0; i < NI; i++) ilt_g2lds16(xbase + ks * (KS * 2) + xoff[i], S.xs[stage] + (wave * NI + i) * 1024);
+    for (int i = 0; i < NI; i++) ilt_g2lds16(xbase + ks * (KS * 2) + xoff[i], xsl + stage * XS + (wave * NI + i) * 1024);
   };
-  auto load_raw = [&](Raw* raw, int unit) {
+  auto issue_w = [&](int i, int sb, int buf) {               // load i of super-block sb's blocks
+    const u32 q = wq0 + 256 * i, row = __umulhi(q, 0xFFFFFFFFu / R::PPB + 1), pc = q - row * R::PPB;
+    const u32 off = __umul24(r0 + min(row, wlast), wrow_bytes) + R::goff(pc);
+    ilt_g2lds16(wbase + (u32)sb * R::BB + off, wsl + buf * WS + (wave + 4 * i) * 1024);
+  };
+  auto load_raw = [&](Raw* raw, int unit) {                  // set number unit of the row, out of LDS
+    const int sb = unit / UPS;
 #pragma unroll
-    for (int b = 0; b < NB; b++) R::load(raw[b], rw, wrowoff[b], unit, lh);
+    for (int b = 0; b < NB; b++) R::load(raw[b], wsl + (sb & 1) * WS + blk0 + b * 32 * R::LB, unit - sb * UPS, lh);
   };
 
-  // Raw sets A and B take turns, P steps each.  Half-step (ks, kk) multiplies with bq[kk] and
-  // makes the operands of the half-step after it: (ks, 1) during (ks, 0), (ks+1, 0) during
-  // (ks, 1).  So set A is last read in the first half of the step that ends its turn, and the
-  // step after that one loads it again, 2P-1 steps before its next turn starts.
+  // Raw sets A and B take turns, P steps each, and are read out of LDS P steps (B) or 2P-1..P
+  // (A) before their turn.  Half-step (ks, kk) multiplies with bq[kk] and makes the operands of
+  // the half-step after it: (ks, 1) during (ks, 0), (ks+1, 0) during (ks, 1).  Super-block
+  // sb+1's blocks are sent for during the first steps of super-block sb, into the buffer that
+  // was last read early in super-block sb-1, and have landed when the first set is read from
+  // them (step 8-P of sb).
   Raw rawa[NB], rawb[NB];
   Prep pr[NB];
   v8bf bq[2][NB];
-  load_raw(rawa, 0);
+#pragma unroll
+  for (int i = 0; i < NWW; i++) issue_w(i, 0, 0);
   issue_x(0, 0);
   issue_x(1, 1);
+  asm volatile("s_waitcnt vmcnt(%0)" :: "n"(2 * NI) : "memory");
+  __syncthreads();
+  load_raw(rawa, 0);
 #pragma unroll
-  for (int b = 0; b < NB; b++) { pr[b] = R::prep(rawa[b], 0, lh); bq[0][b] = R::frag(rawa[b], pr[b], 0, 0, lh, &S.iq2); }
+  for (int b = 0; b < NB; b++) { pr[b] = R::prep(rawa[b], 0, lh); bq[0][b] = R::frag(rawa[b], pr[b], 0, 0, lh, T); }
 
   auto run = [&](auto NALc) {
     constexpr int NAL = decltype(NALc)::value;               // token patches that hold rows
     int st0 = 0, st1 = 1, st2 = 2;
     auto step = [&](int ks, auto Jc) {
-      constexpr int J = decltype(Jc)::value;                 // the step's place in a round of both sets
+      constexpr int J = decltype(Jc)::value;                 // the step's place in its super-block
+      constexpr int JJ = J % (2 * P);                        // and in a round of both sets
+      const int sb = ks >> 3;
       // All loads but the previous step's have landed: this step's x slab has (sent two steps ago).
-      constexpr int prev = NI + (J % P == 1 ? WL : 0);
+      constexpr int sent = (J >= 1 && J <= WSTEPS) ? (NWW - (J - 1) * WPS < WPS ? NWW - (J - 1) * WPS : WPS) : 0;   // block loads of the previous step
+      constexpr int prev = NI + sent;
       asm volatile("s_waitcnt vmcnt(%0)" :: "n"(prev) : "memory");
       ilt_barrier_lds();                                     // no fence: later steps' loads stay in flight
-      if (J == 0) load_raw(rawb, min(ks / P + 1, nu - 1));
-      if (J == P) load_raw(rawa, min(ks / P + 1, nu - 1));
+      if (JJ == 0) load_raw(rawb, min(ks / P + 1, nk / P - 1));
+      if (JJ == P) load_raw(rawa, min(ks / P + 1, nk / P - 1));
+#pragma unroll
+      for (int i = J * WPS; i < ((J + 1) * WPS < NWW ? (J + 1) * WPS : NWW); i++) issue_w(i, min(sb + 1, nsb - 1), (sb + 1) & 1);
       issue_x(st2, min(ks + 2, nk - 1));
       __builtin_amdgcn_sched_barrier(0);
-      const u8* xs = S.xs[st0];
-      constexpr int J1 = (J + 1) % (2 * P);
+      const u8* xs = xsl + st0 * XS;
+      constexpr int J1 = (JJ + 1) % (2 * P);
 #pragma unroll
       for (int kk = 0; kk < 2; kk++) {
         v8bf af[NAL];
 #pragma unroll
-        for (int a = 0; a < NAL; a++) af[a] = *(const v8bf*)(xs + (aoff[a] ^ (32 * kk)));
+        for (int a = 0; a < NAL; a++) af[a] = *(const v8bf*)(xs + (aoff0 ^ (32 * kk)) + 2048 * a);
         if (kk == 0) {
 #pragma unroll
-          for (int b = 0; b < NB; b++) bq[1][b] = R::frag(J < P ? rawa[b] : rawb[b], pr[b], J % P, 1, lh, &S.iq2);
+          for (int b = 0; b < NB; b++) bq[1][b] = R::frag(JJ < P ? rawa[b] : rawb[b], pr[b], JJ % P, 1, lh, T);
         }
 #pragma unroll
         for (int a = 0; a < NAL; a++)
@@ -627,23 +658,21 @@ __global__ __launch_bounds__(256, 2) void gemm_bf16_regb_kernel(BfParams p) {
 #pragma unroll
           for (int b = 0; b < NB; b++) {
             pr[b] = R::prep(J1 < P ? rawa[b] : rawb[b], J1 % P, lh);
-            bq[0][b] = R::frag(J1 < P ? rawa[b] : rawb[b], pr[b], J1 % P, 0, lh, &S.iq2);
+            bq[0][b] = R::frag(J1 < P ? rawa[b] : rawb[b], pr[b], J1 % P, 0, lh, T);
           }
         }
       }
       const int s = st0; st0 = st1; st1 = st2; st2 = s;
     };
-    for (int ks = 0; ks < nk; ks += 2 * P) {
+    for (int ks = 0; ks < nk; ks += 8) {
       step(ks + 0, std::integral_constant<int, 0>{});
       step(ks + 1, std::integral_constant<int, 1>{});
       step(ks + 2, std::integral_constant<int, 2>{});
       step(ks + 3, std::integral_constant<int, 3>{});
-      if constexpr (P == 4) {
-        step(ks + 4, std::integral_constant<int, 4>{});
-        step(ks + 5, std::integral_constant<int, 5>{});
-        step(ks + 6, std::integral_constant<int, 6>{});
-        step(ks + 7, std::integral_constant<int, 7>{});
-      }
+      step(ks + 4, std::integral_constant<int, 4>{});
+      step(ks + 5, std::integral_constant<int, 5>{});
+      step(ks + 6, std::integral_constant<int, 6>{});
+      step(ks + 7, std::integral_constant<int, 7>{});
     }
   };
   switch ((ntok + 31) >> 5) {
@@ -655,6 +684,22 @@ __global__ __launch_bounds__(256, 2) void gemm_bf16_regb_kernel(BfParams p) {
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // the tail's redundant loads: nothing may land in LDS after the workgroup ends
 
   store_tile<NA, NB>(acc, p, tok0, ntok, r0, 0, wr0, l32, lh);
+}
+
+template <int FMT>
+hipError_t launch_regb(const BfParams& p, long long token_tiles, hipStream_t st) {
+  const long long total = token_tiles * (p.rows / 256), per = (total + 7) / 8;
+  if (per * 8 > 0x7FFFFFFFLL) return hipErrorInvalidValue;
+  static bool attr_set[8] = {};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 8) dev = 0;
+  if (!attr_set[dev]) {            // more dynamic LDS than the default 64 KB: asked for once per device
+    const hipError_t e = hipFuncSetAttribute((const void*)gemm_bf16_regb_kernel<FMT>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)regb_smem<FMT>());
+    if (e != hipSuccess) return e;
+    attr_set[dev] = true;
+  }
+  hipLaunchKernelGGL(gemm_bf16_regb_kernel<FMT>, dim3((unsigned)(per * 8)), dim3(256), regb_smem<FMT>(), st, p);
+  return hipGetLastError();
 }
 
 // ---- the two-pass product: W as plain bf16 ------------------------------------------------------
@@ -900,11 +945,8 @@ hipError_t ilt_k_gemm_bf16_id(int fmt, const uint64_t* ptrs, long long add, cons
   const char* force = getenv("ILT_BF16_ID_TILE");
   const int forced = force ? atoi(force) : 0;
   if (rows % 256 == 0 && forced == 0 && (fmt == ILT_IQ2_XXS || fmt == ILT_Q2_K)) {      // weights straight into MFMA operands
-    const long long total = (total_rows / 128 + ne) * (rows / 256), per = (total + 7) / 8;
-    if (per * 8 > 0x7FFFFFFFLL) return hipErrorInvalidValue;
-    if (fmt == ILT_IQ2_XXS) hipLaunchKernelGGL(gemm_bf16_regb_kernel<ILT_IQ2_XXS>, dim3((unsigned)(per * 8)), dim3(256), 0, st, p);
-    else hipLaunchKernelGGL(gemm_bf16_regb_kernel<ILT_Q2_K>, dim3((unsigned)(per * 8)), dim3(256), 0, st, p);
-    return hipGetLastError();
+    if ((long long)rows * row_bytes >= 0x7FFFFFFFLL || row_bytes >= (1 << 24)) return hipErrorInvalidValue;      // the kernel's 32- and 24-bit address arithmetic
+    return fmt == ILT_IQ2_XXS ? launch_regb<ILT_IQ2_XXS>(p, total_rows / 128 + ne, st) : launch_regb<ILT_Q2_K>(p, total_rows / 128 + ne, st);
   }
   if (rows % 256 == 0 && forced != 1) {      // the expert formats (Q4_K / Q6_K raw sets would not fit the registers)
     if (fmt == ILT_IQ2_XXS) return launch_bf16<ILT_IQ2_XXS, 256, 128, 4>(p, total_rows / 128 + ne, st);
