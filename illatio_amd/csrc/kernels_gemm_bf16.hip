@@ -498,37 +498,49 @@ template <> struct RegB<ILT_IQ2_XXS> {
 };
 
 // Q2_K in LDS: 96 bytes a block, its first 80 bytes (16 scale bytes, 64 of quants) as five
-// pieces, then bytes 68..83, whose last four are d and dmin: they land at 92.  A set covers
-// four steps (half a super-block: its 128 weights share 32 bytes of quants, of which the lane
-// needs 8 for each of the two units, and 8 scale bytes).
+// pieces, then bytes 68..83, whose last four are d and dmin: they land at 92.
+// A 16-weight unit has one scale and one minimum, so its weights take four values,
+// fma(dl, q, -ml) for q = 0..3 as the CPU forms them: the lane makes those once for a whole
+// unit -- unit lh of the step, both halves of it -- and picks each weight's bf16 with byte
+// permutes that take the 2-bit codes as selectors.  Lane (l32, 0) then holds columns 0..15 of
+// the step and lane (l32, 1) columns 16..31, where the MFMA wants columns 16*kk + 8*lh ..:
+// one swap of the second half of the low lanes with the first half of the high lanes
+// (v_permlane32_swap) gives both operands.
 template <> struct RegB<ILT_Q2_K> {
   static constexpr int PPB = 6, LB = 96, BB = 84;
   static constexpr int P = 4;
   static __device__ __forceinline__ u32 goff(u32 pc) { return pc == 5 ? 68u : 16 * pc; }
-  struct Raw { int2 qa, qb, sc; u32 dd; };
+  struct Raw { int4 q; u32 sc, dd; };                  // of a step: the unit's 16 bytes of quants, its scale byte, d and dmin
   struct Prep {};
-  static __device__ __forceinline__ void load(Raw& r, const u8* blk, int u, int lh) {
-    r.qa = ilt_lds_ld8(blk + 16 + 32 * u + 8 * lh);
-    r.qb = ilt_lds_ld8(blk + 32 + 32 * u + 8 * lh);
-    r.sc = ilt_lds_ld8(blk + 8 * u);
+  // J: the step within the super-block
+  static __device__ __forceinline__ void read(Raw& r, const u8* blk, int J, int lh) {
+    r.q = ilt_lds_ld16(blk + 16 + 32 * (J >> 2) + 16 * lh);
+    r.sc = *(const ILT_LDS u8*)(blk + 2 * J + lh);
     r.dd = *(const ILT_LDS u32*)(blk + 92);
   }
-  static __device__ __forceinline__ Prep prep(const Raw&, int j, int lh) { return {}; }
-  static __device__ __forceinline__ v8bf frag(const Raw& r, const Prep&, int j, int kk, int lh, const Iq2Tables*) {
-    const u32 scw = ((u32)(j < 2 ? r.sc.x : r.sc.y) >> (16 * (j & 1) + 8 * kk)) & 0xFF;
-    const float dl = ilt_h2f((u16)(r.dd & 0xFFFF)) * (float)(scw & 15), ml = ilt_h2f((u16)(r.dd >> 16)) * (float)(scw >> 4);
-    const int2 qq = kk ? r.qb : r.qa;
-    u32 pk[4];
+  static __device__ __forceinline__ void make(const Raw& r, int J, v8bf& f0, v8bf& f1) {
+    const float dl = ilt_h2f((u16)(r.dd & 0xFFFF)) * (float)(r.sc & 15), ml = ilt_h2f((u16)(r.dd >> 16)) * (float)(r.sc >> 4);
+    // (q = 0 and 1 as fma too: -ml and dl - ml but for the sign of a zero)
+    const u32 p01 = pack_bf16(__builtin_fmaf(dl, 0.0f, -ml), __builtin_fmaf(dl, 1.0f, -ml));
+    const u32 p23 = pack_bf16(__builtin_fmaf(dl, 2.0f, -ml), __builtin_fmaf(dl, 3.0f, -ml));
+    const u32 lo4 = __builtin_amdgcn_perm(p23, p01, 0x06040200u), hi4 = __builtin_amdgcn_perm(p23, p01, 0x07050301u);   // the four low bytes, the four high bytes
+    u32 pk[8];
 #pragma unroll
-    for (int i = 0; i < 2; i++) {
-      const u32 v = ((u32)(i ? qq.y : qq.x) >> (2 * j)) & 0x03030303;
-      float o[4];
-#pragma unroll
-      for (int k = 0; k < 4; k++) o[k] = __builtin_fmaf(dl, (float)((v >> (8 * k)) & 0xFF), -ml);   // dl*q is exact in fp32
-      pk[2 * i] = pack_bf16(o[0], o[1]);
-      pk[2 * i + 1] = pack_bf16(o[2], o[3]);
+    for (int i = 0; i < 4; i++) {
+      const u32 v = (word_of(r.q, i) >> (2 * (J & 3))) & 0x03030303;       // weights 4i .. 4i+3 of the unit
+      const u32 lo = __builtin_amdgcn_perm(lo4, lo4, v), hi = __builtin_amdgcn_perm(hi4, hi4, v);
+      pk[2 * i] = __builtin_amdgcn_perm(hi, lo, 0x05010400u);
+      pk[2 * i + 1] = __builtin_amdgcn_perm(hi, lo, 0x07030602u);
     }
-    v8bf out; __builtin_memcpy(&out, pk, 16); return out;
+    u32 o0[4], o1[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      // lanes 32..63 of the first (columns 16..23) <-> lanes 0..31 of the second (columns 8..15)
+      const auto sw = __builtin_amdgcn_permlane32_swap(pk[i], pk[4 + i], false, false);
+      o0[i] = sw[0]; o1[i] = sw[1];
+    }
+    __builtin_memcpy(&f0, o0, 16);
+    __builtin_memcpy(&f1, o1, 16);
   }
 };
 
@@ -548,8 +560,6 @@ __global__ __launch_bounds__(256, 2) void gemm_bf16_regb_kernel(BfParams p) {
   constexpr int WPS = P == 4 ? 2 : 1;                        // of which it sends this many a step, from step 0 on
   constexpr int WSTEPS = (NWW + WPS - 1) / WPS;
   constexpr int XS = TN * KS * 2, WS = TM * R::LB;
-  typedef typename R::Raw Raw;
-  typedef typename R::Prep Prep;
   extern __shared__ __align__(16) u8 regb_lds[];
   u8* const xsl = regb_lds;                                  // [3][XS]
   u8* const wsl = regb_lds + 3 * XS;                         // [2][WS]
@@ -596,74 +606,26 @@ __global__ __launch_bounds__(256, 2) void gemm_bf16_regb_kernel(BfParams p) {
     const u32 off = __umul24(r0 + min(row, wlast), wrow_bytes) + R::goff(pc);
     ilt_g2lds16(wbase + (u32)sb * R::BB + off, wsl + buf * WS + (wave + 4 * i) * 1024);
   };
-  auto load_raw = [&](Raw* raw, int unit) {                  // set number unit of the row, out of LDS
-    const int sb = unit / UPS;
-#pragma unroll
-    for (int b = 0; b < NB; b++) R::load(raw[b], wsl + (sb & 1) * WS + blk0 + b * 32 * R::LB, unit - sb * UPS, lh);
-  };
-
-  // Raw sets A and B take turns, P steps each, and are read out of LDS P steps (B) or 2P-1..P
-  // (A) before their turn.  Half-step (ks, kk) multiplies with bq[kk] and makes the operands of
-  // the half-step after it: (ks, 1) during (ks, 0), (ks+1, 0) during (ks, 1).  Super-block
-  // sb+1's blocks are sent for during the first steps of super-block sb, into the buffer that
-  // was last read early in super-block sb-1, and have landed when the first set is read from
-  // them (step 8-P of sb).
-  Raw rawa[NB], rawb[NB];
-  Prep pr[NB];
-  v8bf bq[2][NB];
 #pragma unroll
   for (int i = 0; i < NWW; i++) issue_w(i, 0, 0);
   issue_x(0, 0);
   issue_x(1, 1);
   asm volatile("s_waitcnt vmcnt(%0)" :: "n"(2 * NI) : "memory");
   __syncthreads();
-  load_raw(rawa, 0);
-#pragma unroll
-  for (int b = 0; b < NB; b++) { pr[b] = R::prep(rawa[b], 0, lh); bq[0][b] = R::frag(rawa[b], pr[b], 0, 0, lh, T); }
 
-  auto run = [&](auto NALc) {
-    constexpr int NAL = decltype(NALc)::value;               // token patches that hold rows
-    int st0 = 0, st1 = 1, st2 = 2;
-    auto step = [&](int ks, auto Jc) {
-      constexpr int J = decltype(Jc)::value;                 // the step's place in its super-block
-      constexpr int JJ = J % (2 * P);                        // and in a round of both sets
-      const int sb = ks >> 3;
-      // All loads but the previous step's have landed: this step's x slab has (sent two steps ago).
-      constexpr int sent = (J >= 1 && J <= WSTEPS) ? (NWW - (J - 1) * WPS < WPS ? NWW - (J - 1) * WPS : WPS) : 0;   // block loads of the previous step
-      constexpr int prev = NI + sent;
-      asm volatile("s_waitcnt vmcnt(%0)" :: "n"(prev) : "memory");
-      ilt_barrier_lds();                                     // no fence: later steps' loads stay in flight
-      if (JJ == 0) load_raw(rawb, min(ks / P + 1, nk / P - 1));
-      if (JJ == P) load_raw(rawa, min(ks / P + 1, nk / P - 1));
+  // what every step starts with: the waits, the barrier, the loads it sends off
+  auto step_head = [&](int ks, auto Jc, int st2) {
+    constexpr int J = decltype(Jc)::value;                   // the step's place in its super-block
+    const int sb = ks >> 3;
+    // All loads but the previous step's have landed: this step's x slab has (sent two steps ago).
+    constexpr int sent = (J >= 1 && J <= WSTEPS) ? (NWW - (J - 1) * WPS < WPS ? NWW - (J - 1) * WPS : WPS) : 0;   // block loads of the previous step
+    asm volatile("s_waitcnt vmcnt(%0)" :: "n"(NI + sent) : "memory");
+    ilt_barrier_lds();                                       // no fence: later steps' loads stay in flight
 #pragma unroll
-      for (int i = J * WPS; i < ((J + 1) * WPS < NWW ? (J + 1) * WPS : NWW); i++) issue_w(i, min(sb + 1, nsb - 1), (sb + 1) & 1);
-      issue_x(st2, min(ks + 2, nk - 1));
-      __builtin_amdgcn_sched_barrier(0);
-      const u8* xs = xsl + st0 * XS;
-      constexpr int J1 = (JJ + 1) % (2 * P);
-#pragma unroll
-      for (int kk = 0; kk < 2; kk++) {
-        v8bf af[NAL];
-#pragma unroll
-        for (int a = 0; a < NAL; a++) af[a] = *(const v8bf*)(xs + (aoff0 ^ (32 * kk)) + 2048 * a);
-        if (kk == 0) {
-#pragma unroll
-          for (int b = 0; b < NB; b++) bq[1][b] = R::frag(JJ < P ? rawa[b] : rawb[b], pr[b], JJ % P, 1, lh, T);
-        }
-#pragma unroll
-        for (int a = 0; a < NAL; a++)
-#pragma unroll
-          for (int b = 0; b < NB; b++) acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[a], bq[kk][b], acc[a][b], 0, 0, 0);
-        if (kk == 1) {       // (past the last step: operands nobody multiplies with)
-#pragma unroll
-          for (int b = 0; b < NB; b++) {
-            pr[b] = R::prep(J1 < P ? rawa[b] : rawb[b], J1 % P, lh);
-            bq[0][b] = R::frag(J1 < P ? rawa[b] : rawb[b], pr[b], J1 % P, 0, lh, T);
-          }
-        }
-      }
-      const int s = st0; st0 = st1; st1 = st2; st2 = s;
-    };
+    for (int i = J * WPS; i < ((J + 1) * WPS < NWW ? (J + 1) * WPS : NWW); i++) issue_w(i, min(sb + 1, nsb - 1), (sb + 1) & 1);
+    issue_x(st2, min(ks + 2, nk - 1));
+  };
+  auto eight_steps = [&](auto& step) {
     for (int ks = 0; ks < nk; ks += 8) {
       step(ks + 0, std::integral_constant<int, 0>{});
       step(ks + 1, std::integral_constant<int, 1>{});
@@ -675,11 +637,117 @@ __global__ __launch_bounds__(256, 2) void gemm_bf16_regb_kernel(BfParams p) {
       step(ks + 7, std::integral_constant<int, 7>{});
     }
   };
-  switch ((ntok + 31) >> 5) {
-    case 1: run(std::integral_constant<int, 1>{}); break;
-    case 2: run(std::integral_constant<int, 2>{}); break;
-    case 3: run(std::integral_constant<int, 3>{}); break;
-    default: run(std::integral_constant<int, 4>{}); break;
+
+  if constexpr (FMT == ILT_Q2_K) {
+    // Step ks multiplies with the operands made during step ks-1 and makes step ks+1's: its
+    // first half row patch 0's (both units), its second half row patch 1's, from raw bytes read
+    // out of LDS at the step's start.
+    typedef typename R::Raw Raw;
+    v8bf bq[2][2][NB];                                       // [step parity][unit][row patch]
+    {
+      Raw r0_[NB];
+#pragma unroll
+      for (int b = 0; b < NB; b++) R::read(r0_[b], wsl + blk0 + b * 32 * R::LB, 0, lh);
+#pragma unroll
+      for (int b = 0; b < NB; b++) R::make(r0_[b], 0, bq[0][0][b], bq[0][1][b]);
+    }
+    auto run = [&](auto NALc) {
+      constexpr int NAL = decltype(NALc)::value;             // token patches that hold rows
+      int st0 = 0, st1 = 1, st2 = 2;
+      auto step = [&](int ks, auto Jc) {
+        constexpr int J = decltype(Jc)::value, J1 = (J + 1) & 7;
+        step_head(ks, Jc, st2);
+        Raw rn[NB];                                          // (past the last step: the last super-block's again)
+        const u8* wnext = wsl + (((ks >> 3) + (J == 7 ? 1 : 0)) & 1) * WS + blk0;
+#pragma unroll
+        for (int b = 0; b < NB; b++) R::read(rn[b], wnext + b * 32 * R::LB, J1, lh);
+        __builtin_amdgcn_sched_barrier(0);
+        const u8* xs = xsl + st0 * XS;
+#pragma unroll
+        for (int kk = 0; kk < 2; kk++) {
+          v8bf af[NAL];
+#pragma unroll
+          for (int a = 0; a < NAL; a++) af[a] = *(const v8bf*)(xs + (aoff0 ^ (32 * kk)) + 2048 * a);
+#pragma unroll
+          for (int a = 0; a < NAL; a++)
+#pragma unroll
+            for (int b = 0; b < NB; b++) acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[a], bq[J & 1][kk][b], acc[a][b], 0, 0, 0);
+          R::make(rn[kk], J1, bq[J1 & 1][0][kk], bq[J1 & 1][1][kk]);      // row patch kk of the next step
+        }
+        const int s_ = st0; st0 = st1; st1 = st2; st2 = s_;
+      };
+      eight_steps(step);
+    };
+    switch ((ntok + 31) >> 5) {
+      case 1: run(std::integral_constant<int, 1>{}); break;
+      case 2: run(std::integral_constant<int, 2>{}); break;
+      case 3: run(std::integral_constant<int, 3>{}); break;
+      default: run(std::integral_constant<int, 4>{}); break;
+    }
+  } else {
+    // Raw sets A and B take turns, P steps each, and are read out of LDS P steps (B) or 2P-1..P
+    // (A) before their turn.  Half-step (ks, kk) multiplies with bq[kk] and makes the operands of
+    // the half-step after it: (ks, 1) during (ks, 0), (ks+1, 0) during (ks, 1).  Super-block
+    // sb+1's blocks are sent for during the first steps of super-block sb, into the buffer that
+    // was last read early in super-block sb-1, and have landed when the first set is read from
+    // them (step 8-P of sb).
+    typedef typename R::Raw Raw;
+    typedef typename R::Prep Prep;
+    Raw rawa[NB], rawb[NB];
+    Prep pr[NB];
+    v8bf bq[2][NB];
+    auto load_raw = [&](Raw* raw, int unit) {                  // set number unit of the row, out of LDS
+      const int sb = unit / UPS;
+#pragma unroll
+      for (int b = 0; b < NB; b++) R::load(raw[b], wsl + (sb & 1) * WS + blk0 + b * 32 * R::LB, unit - sb * UPS, lh);
+    };
+    load_raw(rawa, 0);
+#pragma unroll
+    for (int b = 0; b < NB; b++) { pr[b] = R::prep(rawa[b], 0, lh); bq[0][b] = R::frag(rawa[b], pr[b], 0, 0, lh, T); }
+
+    auto run = [&](auto NALc) {
+      constexpr int NAL = decltype(NALc)::value;               // token patches that hold rows
+      int st0 = 0, st1 = 1, st2 = 2;
+      auto step = [&](int ks, auto Jc) {
+        constexpr int J = decltype(Jc)::value;                 // the step's place in its super-block
+        constexpr int JJ = J % (2 * P);                        // and in a round of both sets
+        step_head(ks, Jc, st2);
+        if (JJ == 0) load_raw(rawb, min(ks / P + 1, nk / P - 1));
+        if (JJ == P) load_raw(rawa, min(ks / P + 1, nk / P - 1));
+        __builtin_amdgcn_sched_barrier(0);
+        const u8* xs = xsl + st0 * XS;
+        constexpr int J1 = (JJ + 1) % (2 * P);
+#pragma unroll
+        for (int kk = 0; kk < 2; kk++) {
+          v8bf af[NAL];
+#pragma unroll
+          for (int a = 0; a < NAL; a++) af[a] = *(const v8bf*)(xs + (aoff0 ^ (32 * kk)) + 2048 * a);
+          if (kk == 0) {
+#pragma unroll
+            for (int b = 0; b < NB; b++) bq[1][b] = R::frag(JJ < P ? rawa[b] : rawb[b], pr[b], JJ % P, 1, lh, T);
+          }
+#pragma unroll
+          for (int a = 0; a < NAL; a++)
+#pragma unroll
+            for (int b = 0; b < NB; b++) acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[a], bq[kk][b], acc[a][b], 0, 0, 0);
+          if (kk == 1) {       // (past the last step: operands nobody multiplies with)
+#pragma unroll
+            for (int b = 0; b < NB; b++) {
+              pr[b] = R::prep(J1 < P ? rawa[b] : rawb[b], J1 % P, lh);
+              bq[0][b] = R::frag(J1 < P ? rawa[b] : rawb[b], pr[b], J1 % P, 0, lh, T);
+            }
+          }
+        }
+        const int s = st0; st0 = st1; st1 = st2; st2 = s;
+      };
+      eight_steps(step);
+    };
+    switch ((ntok + 31) >> 5) {
+      case 1: run(std::integral_constant<int, 1>{}); break;
+      case 2: run(std::integral_constant<int, 2>{}); break;
+      case 3: run(std::integral_constant<int, 3>{}); break;
+      default: run(std::integral_constant<int, 4>{}); break;
+    }
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // the tail's redundant loads: nothing may land in LDS after the workgroup ends
 
