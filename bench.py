@@ -489,16 +489,18 @@ def workload_c5(args, dev):
     def work_of(kernel, a):
         if kernel == "d4_mm_id_bf16":
             return 2.0 * rows * a[1] * a[2]
+        if kernel == "d4_mm_id_glu_bf16":            # gate and up
+            return 2 * 2.0 * rows * a[1] * a[2]
         if kernel in ("d4_mm_id_iq2_xxs", "d4_mm_id_q2_k"):
             return 2.0 * rows * a[0] * a[1]
         return 0
 
     ms, dev_ms, per = tm.run(step, args.steps, args.warmup, probe_steps=2, work_of=work_of)
-    # one grouped-product kernel template, three launches (gate, up: IQ2_XXS; down: Q2_K)
+    # the grouped products: gate + up (IQ2_XXS; one launch with the gated activation on the bf16 path) and down (Q2_K)
     mm = [k for k in per if per[k][1]]
     allmm = [sum(per[k][0] for k in mm), sum(per[k][1] for k in mm), sum(per[k][2] for k in mm)]
     roof = roofline_of({"mm_id": allmm}, "mfma", MFMA_PEAK_TFLOPS[args.path], "TFLOP/s",
-                       {"mm_id": "gemm_bf16_kernel<16|10, 128, 128, 2> grouped (d4_mm_id_bf16: gate, up, down)" if args.path == "bf16"
+                       {"mm_id": "gemm_bf16_regb_kernel<16, true> (d4_mm_id_glu_bf16: gate, up, activation) + <10, false> (d4_mm_id_bf16: down)" if args.path == "bf16"
                         else "gemm_i8_kernel grouped (d4_mm_id_iq2_xxs x2, d4_mm_id_q2_k), bit-exact"})
     roof["launch_us_all"] = {k: round(v[0] / v[2] * 1e3, 2) for k, v in per.items()}
     if args.path == "bf16" and n == 4096:

@@ -522,6 +522,19 @@ int ilt_d4_mm_id_bf16(uint64_t stream, int gguf_type, int ncols, int nrows, int 
   return (int)ilt_k_gemm_bf16_id(fmt, ptrs, add, counts, bases, ne, row_bytes, nrows, ncols, xb, rmap, total_rows, y, S(stream));
 }
 
+int ilt_d4_mm_id_glu_bf16(uint64_t stream, int gguf_type, int ncols, int nrows, int row_bytes, int64_t add_gate, int64_t add_up,
+                          const uint64_t* ptrs, const uint32_t* counts, const uint32_t* bases, int ne, int64_t total_rows,
+                          const uint16_t* xb, const uint32_t* rmap, float clamp, const float* wrow, uint16_t* mid) {
+  const int fmt = bf16_type(gguf_type);
+  ILT_REQUIRE(fmt == ILT_IQ2_XXS && ncols > 0 && ncols % 256 == 0 && nrows >= 0 && nrows % 128 == 0 && ne >= 0 && ne <= 256 && total_rows >= 0);
+  ILT_REQUIRE(row_bytes == ncols / 256 * block_bytes(fmt) && add_gate >= 0 && (add_gate & 1) == 0 && add_up >= add_gate && (add_up & 1) == 0);
+  if (nrows == 0 || ne == 0 || total_rows == 0) return ILT_OK;
+  ILT_REQUIRE(ptrs && counts && bases && xb && wrow && mid && ((uintptr_t)xb & 15) == 0 && ((uintptr_t)mid & 1) == 0 && total_rows < (1LL << 31));
+  ILT_REQUIRE((long long)row_bytes * nrows + (add_up - add_gate) < 0x7FFFFFFFLL && nrows < (1 << 21));
+  return (int)ilt_k_gemm_bf16_id_glu(fmt, ptrs, add_gate, add_up, counts, bases, ne, row_bytes, nrows, ncols, xb, rmap, total_rows, clamp,
+                                     wrow, mid, S(stream));
+}
+
 // ---- launch by name ---------------------------------------------------------------------------
 int ilt_launch(const char* kernel, unsigned gx, unsigned gy, unsigned gz, unsigned bx, unsigned by, unsigned bz,
                unsigned shared_bytes, uint64_t stream, void** params) {
@@ -562,6 +575,9 @@ int ilt_launch(const char* kernel, unsigned gx, unsigned gy, unsigned gz, unsign
   K("d4_mm_id_bf16")
     return ilt_d4_mm_id_bf16(stream, a.i32(0), a.i32(1), a.i32(2), a.i32(3), a.i64(4), a.ptr<const uint64_t*>(5), a.ptr<cu32>(6),
                              a.ptr<cu32>(7), a.i32(8), a.i64(9), a.ptr<cu16>(10), a.ptr<cu32>(11), a.ptr<float*>(12));
+  K("d4_mm_id_glu_bf16")
+    return ilt_d4_mm_id_glu_bf16(stream, a.i32(0), a.i32(1), a.i32(2), a.i32(3), a.i64(4), a.i64(5), a.ptr<const uint64_t*>(6), a.ptr<cu32>(7),
+                                 a.ptr<cu32>(8), a.i32(9), a.i64(10), a.ptr<cu16>(11), a.ptr<cu32>(12), a.f32(13), a.ptr<cf>(14), a.ptr<uint16_t*>(15));
   K("d4_swiglu_w_bf16") return ilt_d4_swiglu_w_bf16(stream, a.i32(0), a.i32(1), a.f32(2), a.ptr<cf>(3), a.ptr<cf>(4), a.ptr<cf>(5), a.ptr<uint16_t*>(6));
   K("d4_mm_id_iq2_xxs")
     return ilt_d4_mm_id_iq2_xxs(stream, a.i32(0), a.i32(1), a.i32(2), a.i64(5), a.ptr<const uint64_t*>(6), a.ptr<cu32>(7),

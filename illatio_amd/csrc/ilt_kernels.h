@@ -105,6 +105,10 @@ hipError_t ilt_k_gemm_bf16(int fmt, const uint8_t* w, long long row_bytes, int r
 hipError_t ilt_k_gemm_bf16_id(int fmt, const uint64_t* ptrs, long long add, const uint32_t* counts, const uint32_t* bases,
                               int ne, long long row_bytes, int rows, int cols, const uint16_t* xb, const uint32_t* rmap,
                               long long total_rows, float* y, hipStream_t st);
+hipError_t ilt_k_gemm_bf16_id_glu(int fmt, const uint64_t* ptrs, long long add_gate, long long add_up, const uint32_t* counts,
+                                  const uint32_t* bases, int ne, long long row_bytes, int rows, int cols, const uint16_t* xb,
+                                  const uint32_t* rmap, long long total_rows, float clamp, const float* wrow, uint16_t* mid,
+                                  hipStream_t st);
 // The two-pass product for many tokens: the matrix dequantized once to bf16, then a plain bf16
 // product (cols a multiple of 128).  Both operands in slabs (32 columns of 128 rows are 8 KB in
 // one piece), rows and tokens padded to a multiple of 256: 2 * cols * ceil(n / 256) * 256 bytes.

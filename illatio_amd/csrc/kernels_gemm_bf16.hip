@@ -195,6 +195,9 @@ struct BfParams {
   const u32* rmap;                           // grouped: row i of the groups is x's row rmap[i] (null: row i)
   float* y; const float* bias; int acc; int ntok;
   long long ldy;                             // floats from a token's results to the next token's in y (rows, unless p covers a part of the rows)
+  // the grouped gate and up products with the gated activation (gemm_bf16_regb_kernel<FMT, true>): rows = the width of
+  // each; up's matrix at ptrs[z] + add + up_delta; mid[i][r] = bf16((silu(gate) * up) * wrow[i]), clamped as d4_swiglu_w does
+  unsigned up_delta; const float* wrow; float clamp; u16* mid;
 };
 
 template <int TM, int TN, int NXS, int NWS> struct Smem {
@@ -551,9 +554,13 @@ template <int FMT> constexpr size_t regb_smem() {
   return 3 * 128 * KS * 2 + 2 * 256 * RegB<FMT>::LB + sizeof(TileSel) + (FMT == ILT_IQ2_XXS ? sizeof(Iq2Tables) : 0);
 }
 
-template <int FMT>
+// GLU: the tile's 256 rows are 128 rows of the gate matrix and the same 128 of the up matrix,
+// a wave's row patch 0 gate rows and patch 1 the up rows of the same numbers, so that a lane
+// holds both products of a (token, row) and the epilogue writes the gated activation.
+template <int FMT, bool GLU>
 __global__ __launch_bounds__(256, 2) void gemm_bf16_regb_kernel(BfParams p) {
   constexpr int TM = 256, TN = 128, NA = 4, NB = 2, NI = 2;
+  constexpr int TR = GLU ? 128 : 256;                        // rows of a matrix a tile covers
   typedef RegB<FMT> R;
   constexpr int P = R::P, UPS = 8 / P;                       // steps a raw set covers, sets a super-block
   constexpr int NWW = TM * R::PPB / 64 / 4;                  // block loads a wave and super-block: 5 or 6
@@ -568,8 +575,8 @@ __global__ __launch_bounds__(256, 2) void gemm_bf16_regb_kernel(BfParams p) {
   const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
 
   long tok0; int ntok, rt; const u8* w = p.w;
-  if (!pick_tile<TM, TN>(p, S, tok0, ntok, rt, w)) return;
-  const int r0 = rt * TM;
+  if (!pick_tile<TR, TN>(p, S, tok0, ntok, rt, w)) return;
+  const int r0 = rt * TR;
   if (FMT == ILT_IQ2_XXS) iq2_tables_fill(*(Iq2Tables*)T, t);     // (a barrier follows, before the first operands are made)
 
   const int l32 = lane & 31, lh = lane >> 5, wr0 = 64 * wave;
@@ -603,7 +610,9 @@ __global__ __launch_bounds__(256, 2) void gemm_bf16_regb_kernel(BfParams p) {
   };
   auto issue_w = [&](int i, int sb, int buf) {               // load i of super-block sb's blocks
     const u32 q = wq0 + 256 * i, row = __umulhi(q, 0xFFFFFFFFu / R::PPB + 1), pc = q - row * R::PPB;
-    const u32 off = __umul24(r0 + min(row, wlast), wrow_bytes) + R::goff(pc);
+    // GLU: tile row 64w + 32b + l is row 32w + l of the gate (b = 0) or up (b = 1) matrix's 128
+    const u32 mrow = GLU ? ((row >> 6) << 5) | (row & 31) : row;
+    const u32 off = __umul24(r0 + min(mrow, wlast), wrow_bytes) + R::goff(pc) + (GLU && (row & 32) ? p.up_delta : 0u);
     ilt_g2lds16(wbase + (u32)sb * R::BB + off, wsl + buf * WS + (wave + 4 * i) * 1024);
   };
 #pragma unroll
@@ -751,22 +760,46 @@ __global__ __launch_bounds__(256, 2) void gemm_bf16_regb_kernel(BfParams p) {
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // the tail's redundant loads: nothing may land in LDS after the workgroup ends
 
-  store_tile<NA, NB>(acc, p, tok0, ntok, r0, 0, wr0, l32, lh);
+  if constexpr (GLU) {
+    // register r of patch a: token 32a + 8*(r/4) + 4*lh + r%4 of the tile, row r0 + 32*wave + l32.
+    // Through descriptors that end with the tile's last token: a load past it gives 0, a store is dropped.
+    const int row = r0 + 32 * wave + l32;
+    const u32 nt = (u32)__builtin_amdgcn_readfirstlane(ntok);
+    const __amdgpu_buffer_rsrc_t rwt = ilt_rsrc(ilt_uniform_ptr(p.wrow + tok0), nt * 4);
+    const __amdgpu_buffer_rsrc_t rm = ilt_rsrc(ilt_uniform_ptr(p.mid + tok0 * (long)p.rows), (nt - 1) * (u32)p.rows * 2 + (u32)p.rows * 2);
+    const u32 base = row < p.rows ? (u32)row * 2 : 0x80000000u;
+#pragma unroll
+    for (int a = 0; a < NA; a++) {
+      if (32 * a < ntok) {
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+          const u32 tk = (u32)(32 * a + 8 * (r >> 2) + 4 * lh + (r & 3));
+          const float wv = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rwt, tk * 4, 0, 0));
+          float g = acc[a][0][r], u = acc[a][1][r];
+          if (p.clamp > 1e-6f) { g = fminf(g, p.clamp); u = fmaxf(-p.clamp, fminf(u, p.clamp)); }
+          const float o = (ilt_silu(g) * u) * wv;
+          __builtin_amdgcn_raw_buffer_store_b16((u16)(pack_bf16(o, 0.0f) & 0xFFFF), rm, base + tk * (u32)p.rows * 2, 0, 0);
+        }
+      }
+    }
+  } else {
+    store_tile<NA, NB>(acc, p, tok0, ntok, r0, 0, wr0, l32, lh);
+  }
 }
 
-template <int FMT>
+template <int FMT, bool GLU>
 hipError_t launch_regb(const BfParams& p, long long token_tiles, hipStream_t st) {
-  const long long total = token_tiles * (p.rows / 256), per = (total + 7) / 8;
+  const long long total = token_tiles * (p.rows / (GLU ? 128 : 256)), per = (total + 7) / 8;
   if (per * 8 > 0x7FFFFFFFLL) return hipErrorInvalidValue;
   static bool attr_set[8] = {};
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 8) dev = 0;
   if (!attr_set[dev]) {            // more dynamic LDS than the default 64 KB: asked for once per device
-    const hipError_t e = hipFuncSetAttribute((const void*)gemm_bf16_regb_kernel<FMT>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)regb_smem<FMT>());
+    const hipError_t e = hipFuncSetAttribute((const void*)gemm_bf16_regb_kernel<FMT, GLU>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)regb_smem<FMT>());
     if (e != hipSuccess) return e;
     attr_set[dev] = true;
   }
-  hipLaunchKernelGGL(gemm_bf16_regb_kernel<FMT>, dim3((unsigned)(per * 8)), dim3(256), regb_smem<FMT>(), st, p);
+  hipLaunchKernelGGL((gemm_bf16_regb_kernel<FMT, GLU>), dim3((unsigned)(per * 8)), dim3(256), regb_smem<FMT>(), st, p);
   return hipGetLastError();
 }
 
@@ -1014,13 +1047,29 @@ hipError_t ilt_k_gemm_bf16_id(int fmt, const uint64_t* ptrs, long long add, cons
   const int forced = force ? atoi(force) : 0;
   if (rows % 256 == 0 && forced == 0 && (fmt == ILT_IQ2_XXS || fmt == ILT_Q2_K)) {      // weights straight into MFMA operands
     if ((long long)rows * row_bytes >= 0x7FFFFFFFLL || row_bytes >= (1 << 24)) return hipErrorInvalidValue;      // the kernel's 32- and 24-bit address arithmetic
-    return fmt == ILT_IQ2_XXS ? launch_regb<ILT_IQ2_XXS>(p, total_rows / 128 + ne, st) : launch_regb<ILT_Q2_K>(p, total_rows / 128 + ne, st);
+    return fmt == ILT_IQ2_XXS ? launch_regb<ILT_IQ2_XXS, false>(p, total_rows / 128 + ne, st) : launch_regb<ILT_Q2_K, false>(p, total_rows / 128 + ne, st);
   }
   if (rows % 256 == 0 && forced != 1) {      // the expert formats (Q4_K / Q6_K raw sets would not fit the registers)
     if (fmt == ILT_IQ2_XXS) return launch_bf16<ILT_IQ2_XXS, 256, 128, 4>(p, total_rows / 128 + ne, st);
     if (fmt == ILT_Q2_K) return launch_bf16<ILT_Q2_K, 256, 128, 4>(p, total_rows / 128 + ne, st);
   }
   return dispatch_bf16<128, 128, 2>(fmt, p, total_rows / 128 + ne, st);
+}
+
+hipError_t ilt_k_gemm_bf16_id_glu(int fmt, const uint64_t* ptrs, long long add_gate, long long add_up, const uint32_t* counts,
+                                  const uint32_t* bases, int ne, long long row_bytes, int rows, int cols, const uint16_t* xb,
+                                  const uint32_t* rmap, long long total_rows, float clamp, const float* wrow, uint16_t* mid,
+                                  hipStream_t st) {
+  if (total_rows <= 0 || rows <= 0 || ne <= 0) return hipSuccess;
+  if (ne > 256 || fmt != ILT_IQ2_XXS || rows % 128 != 0 || add_up < add_gate) return hipErrorInvalidValue;
+  // the kernel's 32- and 24-bit address arithmetic
+  if ((long long)rows * row_bytes + (add_up - add_gate) >= 0x7FFFFFFFLL || row_bytes >= (1 << 24) || rows >= (1 << 21))
+    return hipErrorInvalidValue;
+  BfParams p = {};
+  p.ptrs = ptrs; p.add = add_gate; p.up_delta = (unsigned)(add_up - add_gate); p.counts = counts; p.bases = bases; p.ne = ne;
+  p.rows = rows; p.cols = cols; p.row_bytes = row_bytes; p.x = xb; p.rmap = rmap; p.ntok = (int)total_rows;
+  p.wrow = wrow; p.clamp = clamp; p.mid = mid;
+  return launch_regb<ILT_IQ2_XXS, true>(p, total_rows / 128 + ne, st);
 }
 
 hipError_t ilt_k_cvt_bf16_slabs(const float* x, uint16_t* out, int n, int cols, hipStream_t st) {

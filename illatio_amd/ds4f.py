@@ -209,13 +209,17 @@ def group_rows(dev, sel, w, n, ne, nu, alloc=hip.hip_alloc):
     return g
 
 
-def ffn_routed_chunk_bf16(dev, pool, logits, norm2, sout, n, ne, nu, scale, clamp, bias=None, keep=None, ws=None):
+def ffn_routed_chunk_bf16(dev, pool, logits, norm2, sout, n, ne, nu, scale, clamp, bias=None, keep=None, ws=None, fused=None):
     """FFN-ROUTED-CHUNK with the three grouped products on the bf16 matrix cores: the same
     routing, grouping, gated activation and slot-ordered sum, no activation quantizers and no
     gathered copy (the gate and up products read the tokens' rows through the row map).
     Within 2e-2 of the CPU path's chunk; the routing and grouping stay exact.  With a
-    Workspace WS nothing is allocated, freed or waited for."""
+    Workspace WS nothing is allocated, freed or waited for.  FUSED: gate, up and the gated
+    activation in one launch (the same bits; needs ff a multiple of 128); None = whenever
+    nobody asks to KEEP the two products."""
     d, ff = pool.d, pool.ff
+    if fused is None:
+        fused = keep is None and ff % 128 == 0
     rows = n * nu
     gb = pool.gate_bytes
     A = ws.alloc if ws else hip.hip_alloc
@@ -223,7 +227,7 @@ def ffn_routed_chunk_bf16(dev, pool, logits, norm2, sout, n, ne, nu, scale, clam
     g = group_rows(dev, sel, w, n, ne, nu, A)
     ptrs = pool.ptrs
     xb = dense.cvt_bf16(dev, norm2, n * d, A(dev, 2 * n * d))
-    gg, gu = (A(dev, 4 * rows * ff) for _ in range(2))
+    gg, gu = (A(dev, 4 * rows * ff) for _ in range(2)) if not fused else (None, None)
     mb = A(dev, 2 * rows * ff)
     down, moe = A(dev, 4 * rows * d), A(dev, 4 * n * d)
 
@@ -231,9 +235,14 @@ def ffn_routed_chunk_bf16(dev, pool, logits, norm2, sout, n, ne, nu, scale, clam
         hip.launch(dev, "d4_mm_id_bf16", (rows // 128 + ne, (nrows + 127) // 128), 256,
                    [qtype, ncols, nrows, rb, hip.I64(add), ptrs, g["counts"], g["bases"], ne, hip.I64(rows), xin, rmap, yout])
 
-    mm_id(IQ2_XXS, d, ff, pool.grb, 0, xb, g["rmap"], gg)
-    mm_id(IQ2_XXS, d, ff, pool.grb, gb, xb, g["rmap"], gu)
-    hip.launch(dev, "d4_swiglu_w_bf16", (rows * ff // 8 + 255) // 256, 256, [rows, ff, float(clamp), gg, gu, g["wrow"], mb])
+    if fused:
+        hip.launch(dev, "d4_mm_id_glu_bf16", (rows // 128 + ne, ff // 128), 256,
+                   [IQ2_XXS, d, ff, pool.grb, hip.I64(0), hip.I64(gb), ptrs, g["counts"], g["bases"], ne, hip.I64(rows), xb, g["rmap"],
+                    float(clamp), g["wrow"], mb])
+    else:
+        mm_id(IQ2_XXS, d, ff, pool.grb, 0, xb, g["rmap"], gg)
+        mm_id(IQ2_XXS, d, ff, pool.grb, gb, xb, g["rmap"], gu)
+        hip.launch(dev, "d4_swiglu_w_bf16", (rows * ff // 8 + 255) // 256, 256, [rows, ff, float(clamp), gg, gu, g["wrow"], mb])
     mm_id(Q2_K, ff, d, pool.drb, 2 * gb, mb, None, down)
     hip.launch(dev, "d4_moe_sum_rows", (n * d + 255) // 256, 256, [d, nu, n, down, g["smap"], sout, moe])
     if ws:
@@ -246,9 +255,10 @@ def ffn_routed_chunk_bf16(dev, pool, logits, norm2, sout, n, ne, nu, scale, clam
         keep["bases"] = hip.hip_download(g["bases"], np.uint32, ne)
         keep["rmap"] = hip.hip_download(g["rmap"], np.uint32, rows)
         keep["mid"] = (hip.hip_download(mb, np.uint16, rows * ff).astype(np.uint32) << 16).view(np.float32).reshape(rows, ff)
-        keep["gate"], keep["up"] = (hip.hip_floats(b, rows * ff).reshape(rows, ff) for b in (gg, gu))
+        if not fused:
+            keep["gate"], keep["up"] = (hip.hip_floats(b, rows * ff).reshape(rows, ff) for b in (gg, gu))
         keep["down"] = hip.hip_floats(down, rows * d).reshape(rows, d)
-    for b in [sel, w, xb, mb, gg, gu, down] + list(g.values()):
+    for b in [sel, w, xb, mb, down] + ([] if fused else [gg, gu]) + list(g.values()):
         hip.hip_free(b)
     return moe
 

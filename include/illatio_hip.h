@@ -280,7 +280,10 @@ int ilt_d4_mm_id_q2_k(uint64_t stream, int ncols, int nrows, int row_bytes, int6
      arguments as d4_mm_id_*.  Row i of the groups multiplies xb's row rmap[i] (d4_group_scatter's
      row -> token map: the tokens' activations are read in place, no gathered copy), or row i
      itself when rmap is null.
-   d4_swiglu_w_bf16: d4_swiglu_w's gated activation rounded to bf16 (ff a multiple of 8). */
+   d4_swiglu_w_bf16: d4_swiglu_w's gated activation rounded to bf16 (ff a multiple of 8).
+   d4_mm_id_glu_bf16: the gate and up products of d4_mm_id_bf16 (IQ2_XXS; up's matrix at
+     ptrs[z] + add_up, add_up >= add_gate) and d4_swiglu_w_bf16 in one launch: mid[i][r] for the
+     groups' row i and r < nrows (a multiple of 128), the bits the three launches give. */
 int ilt_cvt_bf16(uint64_t stream, const float* x, uint16_t* xb, int64_t n);
 int ilt_mm_k_bf16(uint64_t stream, int gguf_type, const void* w, const uint16_t* xb, float* y, const float* bias,
                   int rows, int cols, int n, int acc);
@@ -293,6 +296,9 @@ int ilt_d4_mm_id_bf16(uint64_t stream, int gguf_type, int ncols, int nrows, int 
                       const uint16_t* xb, const uint32_t* rmap, float* y);
 int ilt_d4_swiglu_w_bf16(uint64_t stream, int n, int ff, float clamp, const float* g, const float* u, const float* w,
                          uint16_t* mid);
+int ilt_d4_mm_id_glu_bf16(uint64_t stream, int gguf_type, int ncols, int nrows, int row_bytes, int64_t add_gate, int64_t add_up,
+                          const uint64_t* ptrs, const uint32_t* counts, const uint32_t* bases, int ne, int64_t total_rows,
+                          const uint16_t* xb, const uint32_t* rmap, float clamp, const float* wrow, uint16_t* mid);
 
 /* ---- 3. launch by name (src/cuda.lisp:323-352) -------------------------------------------
  * params[i] points at argument i's 8-byte slot: a pointer as 64 bits, an int in the low

@@ -233,8 +233,8 @@ def test_two_pass_bf16_product(dev, monkeypatch, qtype, rows, cols, n, split):
     m.free()
 
 
-@pytest.mark.parametrize("ne,d,ff,nu,n", [(8, 512, 256, 3, 37), (16, 1024, 512, 4, 300), (4, 1024, 256, 2, 333)])
-def test_grouped_product_variants_agree_bitwise(dev, monkeypatch, ne, d, ff, nu, n):
+@pytest.mark.parametrize("ne,d,ff,nu,n,clamp", [(8, 512, 256, 3, 37, 0.0), (16, 1024, 512, 4, 300, 0.6), (4, 1024, 256, 2, 333, 0.0)])
+def test_grouped_product_variants_agree_bitwise(dev, monkeypatch, ne, d, ff, nu, n, clamp):
     """The grouped product's variants make the same bf16 operands and add the same MFMA results
     in the same order, so their outputs are equal bit for bit: groups of a few rows (token
     patches skipped), of more than one tile of 128, and empty ones."""
@@ -256,7 +256,7 @@ def test_grouped_product_variants_agree_bitwise(dev, monkeypatch, ne, d, ff, nu,
         else:
             monkeypatch.setenv("ILT_BF16_ID_TILE", tile)
         keep = {}
-        moe = ds4f.ffn_routed_chunk_bf16(dev, pool, lb, nb, sb, n, ne, nu, 1.5, 0.0, keep=keep)
+        moe = ds4f.ffn_routed_chunk_bf16(dev, pool, lb, nb, sb, n, ne, nu, 1.5, clamp, keep=keep)
         keep["out"] = hip.hip_floats(moe, n * d)
         hip.hip_free(moe)
         # a group's rows in the order of their tokens (the scatter's order within a group varies from run to run)
@@ -269,6 +269,20 @@ def test_grouped_product_variants_agree_bitwise(dev, monkeypatch, ne, d, ff, nu,
     for tile in ("1", "2"):
         for k in ("gate", "up", "down", "out"):
             assert np.array_equal(res[None][k].view(np.uint32), res[tile][k].view(np.uint32)), (tile, k)
+    # gate, up and the gated activation in one launch: the same bits again
+    monkeypatch.delenv("ILT_BF16_ID_TILE", raising=False)
+    keep = {}
+    moe = ds4f.ffn_routed_chunk_bf16(dev, pool, lb, nb, sb, n, ne, nu, 1.5, clamp, keep=keep, fused=True)
+    out = hip.hip_floats(moe, n * d)
+    hip.hip_free(moe)
+    assert "gate" not in keep
+    order = np.concatenate([int(b) + np.argsort(keep["rmap"][int(b):int(b) + int(c)], kind="stable")
+                            for b, c in zip(keep["bases"], keep["counts"])])
+    order0 = np.concatenate([int(b) + np.argsort(res[None]["rmap"][int(b):int(b) + int(c)], kind="stable")
+                             for b, c in zip(res[None]["bases"], res[None]["counts"])])
+    assert np.array_equal(keep["mid"][order].view(np.uint32), res[None]["mid"][order0].view(np.uint32))
+    assert np.array_equal(keep["down"][order].view(np.uint32), res[None]["down"].view(np.uint32))
+    assert np.array_equal(out.view(np.uint32), res[None]["out"].view(np.uint32))
     for b in (lb, nb, sb):
         hip.hip_free(b)
     pool.free()
