@@ -25,7 +25,9 @@
 // Tiles are numbered so that the workgroups resident on one XCD (every eighth workgroup id)
 // form a block of 8 row tiles x several token tiles and share W and x slabs through that
 // XCD's L2.  The grouped expert product (d4_mm_id_*) walks the token tiles of every
-// expert's rows in turn.
+// expert's rows in turn; for the experts' own formats, IQ2_XXS and Q2_K, it has a kernel of
+// its own that dequantizes into the MFMA operands without a detour of the weights through LDS
+// as bf16 (gemm_bf16_regb_kernel).
 #include "ilt_device.h"
 #include "ilt_iq2xxs_tables.h"
 #include "ilt_kernels.h"
@@ -514,7 +516,6 @@ template <> struct RegB<ILT_Q2_K> {
   static constexpr int P = 4;
   static __device__ __forceinline__ u32 goff(u32 pc) { return pc == 5 ? 68u : 16 * pc; }
   struct Raw { int4 q; u32 sc, dd; };                  // of a step: the unit's 16 bytes of quants, its scale byte, d and dmin
-  struct Prep {};
   // J: the step within the super-block
   static __device__ __forceinline__ void read(Raw& r, const u8* blk, int J, int lh) {
     r.q = ilt_lds_ld16(blk + 16 + 32 * (J >> 2) + 16 * lh);
@@ -1040,9 +1041,10 @@ hipError_t ilt_k_gemm_bf16_id(int fmt, const uint64_t* ptrs, long long add, cons
   p.ptrs = ptrs; p.add = add; p.counts = counts; p.bases = bases; p.ne = ne;
   p.rows = rows; p.cols = cols; p.row_bytes = row_bytes; p.x = xb; p.rmap = rmap; p.y = y; p.ntok = (int)total_rows;
   p.ldy = rows;
-  // 256 rows x 128 tokens a workgroup (a wave: 128 x 64) when the matrices have the rows for it:
-  // an expert seldom has more than 128 rows of tokens in a chunk, and the taller tile reads a
-  // quarter less from LDS per MFMA than 128 x 128.  "1" in ILT_BF16_ID_TILE: 128 x 128 always (tests).
+  // 256 rows x 128 tokens a workgroup when the matrices have the rows for it: an expert seldom has
+  // more than 128 rows of tokens in a chunk.  The experts' formats go to gemm_bf16_regb_kernel;
+  // ILT_BF16_ID_TILE (tests): "2" = that tile in gemm_bf16_kernel (a wave: 128 x 64, a quarter less read
+  // from LDS per MFMA than 128 x 128), "1" = 128 x 128 always.
   const char* force = getenv("ILT_BF16_ID_TILE");
   const int forced = force ? atoi(force) : 0;
   if (rows % 256 == 0 && forced == 0 && (fmt == ILT_IQ2_XXS || fmt == ILT_Q2_K)) {      // weights straight into MFMA operands
