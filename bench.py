@@ -56,7 +56,8 @@ TRAFFIC = {"c1": {"up": _t(2507.3, 96.0), "down": _t(2443.0, 28.0)},
            "c3": {"bf16-1pass": _t(519803.0, 278528.0), "bf16-2pass": _t(491863.8 + 61498.0, 262144.0 + 16384.0),
                   "bf16-resident": _t(491863.8 + 61498.0, 262144.0 + 16384.0)},
            "c4": {"d4_mv_glu_iq2_xxs": _t(12854.8, 96.0), "d4_mv_q2_k_f32": _t(8394.5, 96.0), "d4_mvq8_glu": _t(8833.8, 96.0)},
-           "c5": {"d4_mm_id_bf16": _t((2 * 305779.3 + 367082.0) / 3, (2 * 196608.0 + 393216.0) / 3)}}
+           # per launch, over the step's two grouped launches (gate + up + activation; down)
+           "c5": {"mm_id": _t((569198.8 + 334480.4) / 2, (98304.6 + 393216.0) / 2)}}
 
 
 def traffic_of(workload, per):
@@ -504,7 +505,7 @@ def workload_c5(args, dev):
                         else "gemm_i8_kernel grouped (d4_mm_id_iq2_xxs x2, d4_mm_id_q2_k), bit-exact"})
     roof["launch_us_all"] = {k: round(v[0] / v[2] * 1e3, 2) for k, v in per.items()}
     if args.path == "bf16" and n == 4096:
-        roof["traffic"] = TRAFFIC["c5"]["d4_mm_id_bf16"]
+        roof["traffic"] = TRAFFIC["c5"]["mm_id"]
     tf = flops / (ms * 1e-3) / 1e12
 
     def cpu():
