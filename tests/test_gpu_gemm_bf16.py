@@ -233,7 +233,8 @@ def test_two_pass_bf16_product(dev, monkeypatch, qtype, rows, cols, n, split):
     m.free()
 
 
-@pytest.mark.parametrize("ne,d,ff,nu,n,clamp", [(8, 512, 256, 3, 37, 0.0), (16, 1024, 512, 4, 300, 0.6), (4, 1024, 256, 2, 333, 0.0)])
+@pytest.mark.parametrize("ne,d,ff,nu,n,clamp", [(8, 512, 256, 3, 37, 0.0), (16, 1024, 512, 4, 300, 0.6), (4, 1024, 256, 2, 333, 0.0),
+                                                 (6, 768, 256, 2, 70, 0.0)])      # the last: three super-blocks, three row tiles
 def test_grouped_product_variants_agree_bitwise(dev, monkeypatch, ne, d, ff, nu, n, clamp):
     """The grouped product's variants make the same bf16 operands and add the same MFMA results
     in the same order, so their outputs are equal bit for bit: groups of a few rows (token
