@@ -200,6 +200,8 @@ struct BfParams {
   // the grouped gate and up products with the gated activation (gemm_bf16_regb_kernel<FMT, true>): rows = the width of
   // each; up's matrix at ptrs[z] + add + up_delta; mid[i][r] = bf16((silu(gate) * up) * wrow[i]), clamped as d4_swiglu_w does
   unsigned up_delta; const float* wrow; float clamp; u16* mid;
+  // the exact product (gemm_i8p_kernel): x = the tokens' Q8_K quants (a byte a column), with their block scales and sums of 16
+  const float* xd; const int* bsums;
 };
 
 template <int TM, int TN, int NXS, int NWS> struct Smem {
@@ -804,6 +806,192 @@ hipError_t launch_regb(const BfParams& p, long long token_tiles, hipStream_t st)
   return hipGetLastError();
 }
 
+// ---- the exact product on the same pipeline: Q6_K as two int8 planes ----------------------------
+// Bit for bit the CPU path's MATMUL! (and gemm_i8_kernel's) result: per super-block the integer
+// isum = sum over its 256 columns of sc*(q-32)*xq, then sum += (d*yd) * float(isum), block after
+// block (kquant.lisp:205-236).  Any exact way to the integer will do, so the 13-bit products
+// P = sc*(q-32) go to the int8 matrix cores as two planes: T = P + 4128 (64 .. 8065) = 64*hi + lo
+// with hi 1..126 and lo 0..63, and isum = 64*(hi.xq) + (lo.xq) - 4128*(sum of the block's xq),
+// the last from the activations' sums of 16.  v_mfma_i32_32x32x32_i8 accumulates both planes
+// over the super-block's four steps of 64 columns; the lanes then combine them once per block.
+// Four weights are made at a time: the even and the odd bytes of a word as two 16-bit fields,
+// one signed 24-bit multiply-add (q*sc + C, C = 4128 - 32*sc, in both fields at once: each
+// field's total is within 0..65535, so borrows between them cancel).
+typedef int v4i_ __attribute__((ext_vector_type(4)));
+typedef int v16i_ __attribute__((ext_vector_type(16)));
+
+struct I8pRaw { int4 ql, qh; int2 sc; u32 d; };            // thread (row, q4), half c of a super-block: 16 weights of its parts q4/2 and 2 + q4/2
+
+struct I8pSmem {
+  __align__(16) u8 xs[3][128 * 64];       // the tokens' quants, 64 columns a step
+  __align__(16) u8 wh[2][128 * 64];       // the rows' hi plane, the step's and the next step's
+  __align__(16) u8 wl[2][128 * 64];       // lo plane
+  float wd[128];                          // of the super-block: d of the rows,
+  float xd[128];                          //   the tokens' scales
+  int cx[128];                            //   and 4128 * the sum of their quants
+  u32 scan[256];
+  int tile_z, tile_t0, tile_n;
+};
+
+__device__ __forceinline__ void ilt_lds_st4_untracked(void* p, u32 v) {
+  asm volatile("ds_write_b32 %0, %1" :: "v"((u32)(uintptr_t)(ILT_LDS void*)p), "v"(v) : "memory");
+}
+
+// 128 rows x 128 tokens a workgroup of eight waves (one workgroup a CU, two waves a SIMD: a
+// wave's two planes of integer sums, its float sums and the raw bytes leave no room for more);
+// wave w: rows 32*(w/2).., tokens 64*(w%2)...  Thread (row, q4) makes columns 16*q4.. of its row
+// in every step.
+__global__ __launch_bounds__(512, 1) void gemm_i8p_kernel(BfParams p) {
+  constexpr int TM = 128, TN = 128, NA = 2, NI = 1;
+  constexpr int WL = 4, XL = 5;                              // loads of a raw set, of a token's constants
+  constexpr int KW = 64;                                     // columns a step
+  __shared__ I8pSmem S;
+  const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+
+  long tok0; int ntok, rt; const u8* w = p.w;
+  if (!pick_tile<TM, TN>(p, S, tok0, ntok, rt, w)) return;
+  const int r0 = rt * TM;
+
+  const int wrow = t >> 2, q4 = t & 3;
+  const __amdgpu_buffer_rsrc_t rw = ilt_rsrc(ilt_uniform_ptr(w), (u32)min((long long)p.rows * p.row_bytes, 0xFFFFFFF0LL));
+  const u32 wrowoff = (u32)((long long)min(r0 + wrow, p.rows - 1) * p.row_bytes);
+  const u32 wdst = slab_off(wrow, q4);
+  const u8* xbase = (const u8*)ilt_uniform_ptr((const i8*)p.x + tok0 * (long)p.cols);
+  const u32 xoff = (u32)min(t >> 2, ntok - 1) * (u32)p.cols + 16 * ((t & 3) ^ (int)slab_swz(t >> 2));   // piece t of a slab
+  const int nk = p.cols / KW, nsb = p.cols / 256;
+  // a token's constants for a super-block, by thread t & 127 (every wave loads, so that all count the same loads)
+  const long ctok = tok0 + min(t & 127, ntok - 1);
+  const float* xdp = p.xd + ctok * nsb;
+  const int4* bsp = (const int4*)(p.bsums + ctok * (p.cols / 16));
+  float c_yd; int4 c_bs[4];
+  auto load_consts = [&](int sb) {
+    c_yd = xdp[sb];
+#pragma unroll
+    for (int i = 0; i < 4; i++) c_bs[i] = bsp[4 * sb + i];
+  };
+  auto store_consts = [&](const I8pRaw& ra) {                // after a barrier that ends the last block's reads
+    if (t < 128) {
+      int sx = 0;
+#pragma unroll
+      for (int i = 0; i < 4; i++) sx += c_bs[i].x + c_bs[i].y + c_bs[i].z + c_bs[i].w;
+      ilt_lds_st4_untracked(&S.xd[t], __builtin_bit_cast(u32, c_yd));
+      ilt_lds_st4_untracked(&S.cx[t], (u32)(4128 * sx));
+    }
+    if (q4 == 0) ilt_lds_st4_untracked(&S.wd[wrow], __builtin_bit_cast(u32, ilt_h2f((u16)ra.d)));
+  };
+  auto load_raw = [&](I8pRaw& r, int hb) {                   // half super-block hb of the thread's row
+    const u32 b = wrowoff + (u32)(hb >> 1) * ILT_Q6K_STRIDE;
+    const int c = hb & 1;
+    r.ql = ilt_bld16(rw, b + 64 * c + 16 * q4);              // ql[64c + 32*(part & 1) + l], part & 1 = q4 / 2, l = 16*(q4 & 1)..
+    r.qh = ilt_bld16(rw, b + 128 + 32 * c + 16 * (q4 & 1));
+    r.sc = ilt_bld8(rw, b + 192 + 8 * c);
+    r.d = ilt_bld2(rw, b + 208);
+  };
+  auto issue_x = [&](int stage, int ks) { ilt_g2lds16(xbase + ks * KW + xoff, S.xs[stage] + wave * 1024); };
+  // 16 weights of part 2*jj + q4/2 of the half in r, as the two planes, into a pair of slabs
+  auto dequant_to = [&](const I8pRaw& r, int jj, int slab) {
+    const int sc = (int)(i8)(((u32)(jj ? r.sc.y : r.sc.x) >> (8 * q4)) & 0xFF);      // scale 8c + 2*part + (q4 & 1)
+    const int cpair = (4128 - 32 * sc) * 0x10001;
+    int hi[4], lo[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      const u32 v = ((word_of(r.ql, i) >> (4 * jj)) & 0x0F0F0F0F) | (((word_of(r.qh, i) >> (4 * jj + 2 * (q4 >> 1))) & 0x03030303) << 4);
+      const u32 te = (u32)(__mul24((int)(v & 0x00FF00FF), sc) + cpair), to = (u32)(__mul24((int)((v >> 8) & 0x00FF00FF), sc) + cpair);
+      hi[i] = (int)(((te >> 6) & 0x007F007F) | (((to >> 6) & 0x007F007F) << 8));
+      lo[i] = (int)((te & 0x003F003F) | ((to & 0x003F003F) << 8));
+    }
+    ilt_lds_st16_untracked(S.wh[slab] + wdst, hi[0], hi[1], hi[2], hi[3]);
+    ilt_lds_st16_untracked(S.wl[slab] + wdst, lo[0], lo[1], lo[2], lo[3]);
+  };
+
+  v16f sum[NA][1];
+  v16i_ ah[NA], al[NA];
+#pragma unroll
+  for (int a = 0; a < NA; a++)
+#pragma unroll
+    for (int r = 0; r < 16; r++) { sum[a][0][r] = 0.0f; ah[a][r] = 0; al[a][r] = 0; }
+
+  const int wt0 = 64 * (wave & 1), wr0 = 32 * (wave >> 1);  // this wave's tokens and rows in the tile
+  const int l32 = lane & 31, lh = lane >> 5;
+  u32 aoff[NA];                                              // fragment offsets of the step's first 32 columns (piece lh); the second 32 at ^ 32
+#pragma unroll
+  for (int a = 0; a < NA; a++) aoff[a] = slab_off(wt0 + 32 * a + l32, lh);
+  const u32 boff = slab_off(wr0 + l32, lh);
+
+  // Raw set A holds half 0 of a super-block and B half 1, two steps each; step ks multiplies
+  // slab ks while it makes step ks+1's planes, so A is free after step 0 and loaded again (the
+  // next block's) in step 1, B after step 2 and loaded in step 3.  The next block's token
+  // constants are loaded in step 2 and stored in the next step 0.
+  I8pRaw rawa, rawb;
+  load_raw(rawa, 0);
+  load_consts(0);
+  issue_x(0, 0);
+  load_raw(rawb, 1);
+  issue_x(1, 1);
+  int st0 = 0, st1 = 1, st2 = 2;
+  dequant_to(rawa, 0, 0);
+  store_consts(rawa);
+
+  auto step = [&](int ks, auto Jc) {
+    constexpr int J = decltype(Jc)::value;                   // the step's place in its super-block
+    // All loads but the previous step's have landed: this step's x slab has (sent two steps ago).
+    constexpr int prev = NI + ((J == 0 || J == 2) ? WL : J == 3 ? XL : 0);
+    asm volatile("s_waitcnt vmcnt(%0)" :: "n"(prev) : "memory");
+    ilt_barrier_lds();                                       // no fence: later steps' loads stay in flight
+    const int sb = ks >> 2;
+    if (J == 0 && ks > 0) store_consts(rawa);                // (the first block's were stored before the loop)
+    if (J == 1) load_raw(rawa, min(2 * sb + 2, 2 * nsb - 1));
+    if (J == 2) load_consts(min(sb + 1, nsb - 1));
+    if (J == 3) load_raw(rawb, min(2 * sb + 3, 2 * nsb - 1));
+    issue_x(st2, min(ks + 2, nk - 1));
+    __builtin_amdgcn_sched_barrier(0);
+    const u8* xs = S.xs[st0];
+    const u8* whs = S.wh[J & 1];
+    const u8* wls = S.wl[J & 1];
+#pragma unroll
+    for (int kk = 0; kk < 2; kk++) {
+      v4i_ af[NA];
+#pragma unroll
+      for (int a = 0; a < NA; a++) af[a] = *(const v4i_*)(xs + (aoff[a] ^ (32 * kk)));
+      const v4i_ bh = *(const v4i_*)(whs + (boff ^ (32 * kk))), bl = *(const v4i_*)(wls + (boff ^ (32 * kk)));
+      if (kk == 0) {       // step ks+1's planes: J+1 = 1 from A, 2 and 3 from B, 4 = the next block's 0 from A (past the last step: planes nobody reads)
+        if (J == 0) dequant_to(rawa, 1, 1);
+        if (J == 1) dequant_to(rawb, 0, 0);
+        if (J == 2) dequant_to(rawb, 1, 1);
+        if (J == 3) dequant_to(rawa, 0, 0);
+      }
+#pragma unroll
+      for (int a = 0; a < NA; a++) {
+        ah[a] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[a], bh, ah[a], 0, 0, 0);
+        al[a] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[a], bl, al[a], 0, 0, 0);
+      }
+    }
+    if (J == 3) {          // the super-block is complete: sum += (d * yd) * float(isum), as the CPU path adds it
+      const float d = S.wd[wr0 + l32];
+#pragma unroll
+      for (int a = 0; a < NA; a++) {
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+          const int tk = wt0 + 32 * a + 8 * (r >> 2) + 4 * lh + (r & 3);
+          const int isum = 64 * ah[a][r] + al[a][r] - S.cx[tk];
+          sum[a][0][r] = sum[a][0][r] + (d * S.xd[tk]) * (float)isum;
+          ah[a][r] = 0; al[a][r] = 0;
+        }
+      }
+    }
+    const int s_ = st0; st0 = st1; st1 = st2; st2 = s_;
+  };
+  for (int ks = 0; ks < nk; ks += 4) {     // one super-block of 256 columns
+    step(ks + 0, std::integral_constant<int, 0>{});
+    step(ks + 1, std::integral_constant<int, 1>{});
+    step(ks + 2, std::integral_constant<int, 2>{});
+    step(ks + 3, std::integral_constant<int, 3>{});
+  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // the tail's redundant loads: nothing may land in LDS after the workgroup ends
+
+  store_tile<NA, 1>(sum, p, tok0, ntok, r0, wt0, wr0, l32, lh);
+}
+
 // ---- the two-pass product: W as plain bf16 ------------------------------------------------------
 // With thousands of tokens the in-loop dequantization above is repeated for every tile of 256
 // tokens and its VALU work competes with the MFMAs for issue slots.  With HBM to spare the
@@ -1072,6 +1260,19 @@ hipError_t ilt_k_gemm_bf16_id_glu(int fmt, const uint64_t* ptrs, long long add_g
   p.rows = rows; p.cols = cols; p.row_bytes = row_bytes; p.x = xb; p.rmap = rmap; p.ntok = (int)total_rows;
   p.wrow = wrow; p.clamp = clamp; p.mid = mid;
   return launch_regb<ILT_IQ2_XXS, true>(p, total_rows / 128 + ne, st);
+}
+
+hipError_t ilt_k_gemm_i8_planes(int fmt, const uint8_t* w, long long row_bytes, int rows, int cols, const int8_t* xq, const float* xd,
+                                const int* bsums, int ntok, float* y, const float* bias, int acc, hipStream_t st) {
+  if (ntok <= 0 || rows <= 0) return hipSuccess;
+  if (fmt != ILT_Q6_K || cols % 256 != 0 || (long long)rows * 1024 >= 0x7FFFFFFFLL) return hipErrorInvalidValue;
+  BfParams p = {};
+  p.w = w; p.rows = rows; p.cols = cols; p.row_bytes = row_bytes; p.x = (const u16*)xq; p.xd = xd; p.bsums = bsums;
+  p.y = y; p.bias = bias; p.acc = acc; p.ntok = ntok; p.ldy = rows;
+  const long long total = (long long)((ntok + 127) / 128) * ((rows + 127) / 128), per = (total + 7) / 8;
+  if (per * 8 > 0x7FFFFFFFLL) return hipErrorInvalidValue;
+  hipLaunchKernelGGL(gemm_i8p_kernel, dim3((unsigned)(per * 8)), dim3(512), 0, st, p);
+  return hipGetLastError();
 }
 
 hipError_t ilt_k_cvt_bf16_slabs(const float* x, uint16_t* out, int n, int cols, hipStream_t st) {
