@@ -810,9 +810,9 @@ hipError_t launch_regb(const BfParams& p, long long token_tiles, hipStream_t st)
 // Bit for bit the CPU path's MATMUL! (and gemm_i8_kernel's) result: per super-block the integer
 // isum = sum over its 256 columns of sc*(q-32)*xq, then sum += (d*yd) * float(isum), block after
 // block (kquant.lisp:205-236).  Any exact way to the integer will do, so the 13-bit products
-// P = sc*(q-32) go to the int8 matrix cores as two planes: T = P + 4128 (64 .. 8065) = 64*hi + lo
-// with hi 1..126 and lo 0..63, and isum = 64*(hi.xq) + (lo.xq) - 4128*(sum of the block's xq),
-// the last from the activations' sums of 16.  v_mfma_i32_32x32x32_i8 accumulates both planes
+// P = sc*(q-32) go to the int8 matrix cores as two planes, the bytes of T = P + 4128 (64 .. 8065):
+// hi = T >> 8 (0..31) and lo = (T & 255) - 128, so isum = 256*(hi.xq) + (lo.xq) - 4000*(sum of the
+// block's xq), the last from the activations' sums of 16.  v_mfma_i32_32x32x32_i8 accumulates both planes
 // over the super-block's four steps of 64 columns; the lanes then combine them once per block.
 // Four weights are made at a time: the even and the odd bytes of a word as two 16-bit fields,
 // one signed 24-bit multiply-add (q*sc + C, C = 4128 - 32*sc, in both fields at once: each
@@ -828,7 +828,7 @@ struct I8pSmem {
   __align__(16) u8 wl[2][128 * 64];       // lo plane
   float wd[128];                          // of the super-block: d of the rows,
   float xd[128];                          //   the tokens' scales
-  int cx[128];                            //   and 4128 * the sum of their quants
+  int cx[128];                            //   and 4000 * the sum of their quants
   u32 scan[256];
   int tile_z, tile_t0, tile_n;
 };
@@ -875,7 +875,7 @@ __global__ __launch_bounds__(512, 1) void gemm_i8p_kernel(BfParams p) {
 #pragma unroll
       for (int i = 0; i < 4; i++) sx += c_bs[i].x + c_bs[i].y + c_bs[i].z + c_bs[i].w;
       ilt_lds_st4_untracked(&S.xd[t], __builtin_bit_cast(u32, c_yd));
-      ilt_lds_st4_untracked(&S.cx[t], (u32)(4128 * sx));
+      ilt_lds_st4_untracked(&S.cx[t], (u32)(4000 * sx));
     }
     if (q4 == 0) ilt_lds_st4_untracked(&S.wd[wrow], __builtin_bit_cast(u32, ilt_h2f((u16)ra.d)));
   };
@@ -897,8 +897,8 @@ __global__ __launch_bounds__(512, 1) void gemm_i8p_kernel(BfParams p) {
     for (int i = 0; i < 4; i++) {
       const u32 v = ((word_of(r.ql, i) >> (4 * jj)) & 0x0F0F0F0F) | (((word_of(r.qh, i) >> (4 * jj + 2 * (q4 >> 1))) & 0x03030303) << 4);
       const u32 te = (u32)(__mul24((int)(v & 0x00FF00FF), sc) + cpair), to = (u32)(__mul24((int)((v >> 8) & 0x00FF00FF), sc) + cpair);
-      hi[i] = (int)(((te >> 6) & 0x007F007F) | (((to >> 6) & 0x007F007F) << 8));
-      lo[i] = (int)((te & 0x003F003F) | ((to & 0x003F003F) << 8));
+      hi[i] = (int)__builtin_amdgcn_perm(to, te, 0x07030501u);                  // the fields' high bytes, in the weights' order
+      lo[i] = (int)(__builtin_amdgcn_perm(to, te, 0x06020400u) ^ 0x80808080u);   // their low bytes - 128
     }
     ilt_lds_st16_untracked(S.wh[slab] + wdst, hi[0], hi[1], hi[2], hi[3]);
     ilt_lds_st16_untracked(S.wl[slab] + wdst, lo[0], lo[1], lo[2], lo[3]);
@@ -909,7 +909,7 @@ __global__ __launch_bounds__(512, 1) void gemm_i8p_kernel(BfParams p) {
 #pragma unroll
   for (int a = 0; a < NA; a++)
 #pragma unroll
-    for (int r = 0; r < 16; r++) { sum[a][0][r] = 0.0f; ah[a][r] = 0; al[a][r] = 0; }
+    for (int r = 0; r < 16; r++) sum[a][0][r] = 0.0f;
 
   const int wt0 = 64 * (wave & 1), wr0 = 32 * (wave >> 1);  // this wave's tokens and rows in the tile
   const int l32 = lane & 31, lh = lane >> 5;
@@ -962,8 +962,9 @@ __global__ __launch_bounds__(512, 1) void gemm_i8p_kernel(BfParams p) {
       }
 #pragma unroll
       for (int a = 0; a < NA; a++) {
-        ah[a] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[a], bh, ah[a], 0, 0, 0);
-        al[a] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[a], bl, al[a], 0, 0, 0);
+        const v16i_ zero = {};                                 // a super-block's first products start its integer sums
+        ah[a] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[a], bh, (J == 0 && kk == 0) ? zero : ah[a], 0, 0, 0);
+        al[a] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[a], bl, (J == 0 && kk == 0) ? zero : al[a], 0, 0, 0);
       }
     }
     if (J == 3) {          // the super-block is complete: sum += (d * yd) * float(isum), as the CPU path adds it
@@ -973,9 +974,8 @@ __global__ __launch_bounds__(512, 1) void gemm_i8p_kernel(BfParams p) {
 #pragma unroll
         for (int r = 0; r < 16; r++) {
           const int tk = wt0 + 32 * a + 8 * (r >> 2) + 4 * lh + (r & 3);
-          const int isum = 64 * ah[a][r] + al[a][r] - S.cx[tk];
+          const int isum = 256 * ah[a][r] + al[a][r] - S.cx[tk];
           sum[a][0][r] = sum[a][0][r] + (d * S.xd[tk]) * (float)isum;
-          ah[a][r] = 0; al[a][r] = 0;
         }
       }
     }
