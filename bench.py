@@ -324,8 +324,9 @@ def workload_c3(args, dev):
     from illatio_amd import dense, hip, synth
     rng = synth.make_rng(33)
     rows, cols, T = (17408, 5120, args.tokens) if not args.transpose else (5120, 17408, args.tokens)
-    w = np.tile(synth.weights(synth.Q6_K, 256, cols, rng, dscale=0.01), (rows // 256, 1))
-    m = dense.upload_gmat(dev, "w", synth.Q6_K, rows, cols, w)
+    qt = synth.Q4_K if args.qtype == "q4_k" else synth.Q6_K        # BASELINE's config 3 is Q6_K; --qtype q4_k: the same shape in the other dense format
+    w = np.tile(synth.weights(qt, 256, cols, rng, dscale=0.01), (rows // 256, 1))
+    m = dense.upload_gmat(dev, "w", qt, rows, cols, w)
     x = synth.activations((T, cols), rng)
     xf = hip.hip_upload_new(dev, x)
     y = hip.hip_alloc(dev, 4 * T * rows, zero=False)
@@ -360,7 +361,8 @@ def workload_c3(args, dev):
         def step(_):
             tm.launch("quant", 0, lambda: dense.quantize_act(dev, xf, act))
             tm.launch("mm", flops, lambda: dense.cmat_mul(dev, m, act, y, n=T))
-        names = {"mm": "gemm_i8_kernel (Q6_K unpacked to int8 in LDS, v_mfma_i32_16x16x64_i8, bit-exact with the CPU path)"}
+        names = {"mm": "gemm_i8p_kernel (scale * quant as two int8 planes in LDS, v_mfma_i32_32x32x32_i8, one float combine per super-block: "
+                       "bit-exact with the CPU path)"}
     ms, dev_ms, per = tm.run(step, args.steps, args.warmup)
     roof = roofline_of({k: v for k, v in per.items() if k == "mm"}, "mfma", MFMA_PEAK_TFLOPS[args.path], "TFLOP/s" if bf16_path else "TOP/s", names)
     roof["unit"] = "TFLOP/s"
@@ -375,7 +377,7 @@ def workload_c3(args, dev):
         t1 = time.perf_counter()
         reps = 0
         while time.perf_counter() - t1 < 10.0:
-            orc.matmul(synth.Q6_K, w, rows, cols, x[:ts], nthreads=cores)
+            orc.matmul(qt, w, rows, cols, x[:ts], nthreads=cores)
             reps += 1
         t_cpu = time.perf_counter() - t1
         return {"value": round(2.0 * rows * cols * ts * reps / t_cpu / 1e12, 4), "unit": "TFLOP/s", "cores": cores, "kind": "port",
@@ -384,7 +386,7 @@ def workload_c3(args, dev):
     return {"value": round(tf, 1), "unit": "TFLOP/s", "ms_per_step": ms, "device_ms_per_step": dev_ms, "enqueue_ms": tm.enqueue_ms,
             "dtype": "bf16 x bf16, fp32 accumulate" if bf16_path else "int8 block dots, fp32 combine",
             "metric": "prefill product TFLOP/s (% of dense MFMA peak)",
-            "config": {"workload": f"c3: Q6_K prefill product {rows}x{cols} on {T} tokens, {path} path "
+            "config": {"workload": f"c3: {args.qtype.upper()} prefill product {rows}x{cols} on {T} tokens, {path} path "
                                    f"(activation conversion inside the step)", "flops_per_step": flops, "tokens": T},
             "extra": {"pct_of_mfma_peak": round(100 * tf / MFMA_PEAK_TFLOPS[args.path], 2)}, "roofline": roof, "cpu": cpu}
 
@@ -554,6 +556,7 @@ def main():
     ap.add_argument("--layers", type=int, default=LAYERS, help=argparse.SUPPRESS)
     ap.add_argument("--tokens", type=int, default=4096, help="c3, c5: tokens per step")
     ap.add_argument("--transpose", action="store_true", help="c3: the 5120x17408 matrix")
+    ap.add_argument("--qtype", default="q6_k", choices=["q6_k", "q4_k"], help="c3: the matrix's format (BASELINE: q6_k)")
     ap.add_argument("--path", default="bf16", choices=["bf16", "bf16-1pass", "bf16-2pass", "bf16-resident", "int8"],
                     help="c3, c5: which matrix-core path.  c3: bf16 = 2pass from 1024 tokens on, else 1pass; bf16-1pass = the matrix dequantized inside the product's loop; "
                          "bf16-2pass = the matrix dequantized to a bf16 copy inside the step, then the plain bf16 product; bf16-resident = that copy made beforehand and kept")

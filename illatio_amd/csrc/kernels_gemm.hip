@@ -427,11 +427,11 @@ hipError_t ilt_k_gemm_i8(int fmt, const uint8_t* w, const uint16_t* wd, long lon
                          const int8_t* xq, const float* xs, const int* bsums, int ntok, float* y, const float* bias,
                          int acc, hipStream_t st) {
   if (ntok <= 0 || rows <= 0) return hipSuccess;
-  // Q6_K with enough tokens and rows to fill 128 x 128 tiles: the pipelined kernel with the weights as
+  // Q6_K and Q4_K with enough tokens and rows to fill 128 x 128 tiles: the pipelined kernel with the weights as
   // two int8 planes, the same bits.  ILT_I8_PLANES (tests): "0" never, "1" whenever the format allows.
   const char* force = getenv("ILT_I8_PLANES");
   const int forced = force ? atoi(force) : -1;
-  if (fmt == ILT_Q6_K && cols % 256 == 0 && forced != 0 && (forced == 1 || (ntok >= 96 && rows >= 128)))
+  if ((fmt == ILT_Q6_K || fmt == ILT_Q4_K) && cols % 256 == 0 && forced != 0 && (forced == 1 || (ntok >= 96 && rows >= 128)))
     return ilt_k_gemm_i8_planes(fmt, w, row_bytes, rows, cols, xq, xs, bsums, ntok, y, bias, acc, st);
   GemmParams p = {};
   p.w = w; p.wdq = wd; p.rows = rows; p.cols = cols; p.row_bytes = row_bytes;

@@ -806,29 +806,102 @@ hipError_t launch_regb(const BfParams& p, long long token_tiles, hipStream_t st)
   return hipGetLastError();
 }
 
-// ---- the exact product on the same pipeline: Q6_K as two int8 planes ----------------------------
-// Bit for bit the CPU path's MATMUL! (and gemm_i8_kernel's) result: per super-block the integer
-// isum = sum over its 256 columns of sc*(q-32)*xq, then sum += (d*yd) * float(isum), block after
-// block (kquant.lisp:205-236).  Any exact way to the integer will do, so the 13-bit products
-// P = sc*(q-32) go to the int8 matrix cores as two planes, the bytes of T = P + 4128 (64 .. 8065):
-// hi = T >> 8 (0..31) and lo = (T & 255) - 128, so isum = 256*(hi.xq) + (lo.xq) - 4000*(sum of the
-// block's xq), the last from the activations' sums of 16.  v_mfma_i32_32x32x32_i8 accumulates both planes
+// ---- the exact product on the same pipeline: Q6_K and Q4_K as two int8 planes -------------------
+// Bit for bit the CPU path's MATMUL! (and gemm_i8_kernel's) result: per super-block an integer
+// isum = sum over its 256 columns of (scale * quant) * xq, then sum += (d*yd) * float(isum) (and
+// Q4_K's term of the minimums before it), block after block (kquant.lisp:180-236).  Any exact
+// way to the integer will do, so the products P = sc*(q-32) (Q6_K, 13 bits) or sc*q (Q4_K, 10
+// bits) go to the int8 matrix cores as two planes, the bytes of T = P + C0 >= 0 (C0 = 4128 or
+// 0): hi = T >> 8 (0..31) and lo = (T & 255) - 128, so
+//   isum = 256*(hi.xq) + (lo.xq) + (128 - C0)*(sum of the block's xq),
+// the last from the activations' sums of 16.  v_mfma_i32_32x32x32_i8 accumulates both planes
 // over the super-block's four steps of 64 columns; the lanes then combine them once per block.
-// Four weights are made at a time: the even and the odd bytes of a word as two 16-bit fields,
-// one signed 24-bit multiply-add (q*sc + C, C = 4128 - 32*sc, in both fields at once: each
-// field's total is within 0..65535, so borrows between them cancel).
+// Four weights are made at a time: the even and the odd bytes of a word as two 16-bit fields
+// and one 24-bit multiply(-add) for both fields (each field's total is within 0..65535, so
+// borrows between them cancel).  Q4_K's sum of minimum * (sum of 32 quants) over the eight
+// groups is one more pair of small products per super-block, the sums of 32 split into planes
+// the same way.
 typedef int v4i_ __attribute__((ext_vector_type(4)));
 typedef int v16i_ __attribute__((ext_vector_type(16)));
+typedef int v3i_ __attribute__((ext_vector_type(3)));
 
-struct I8pRaw { int4 ql, qh; int2 sc; u32 d; };            // thread (row, q4), half c of a super-block: 16 weights of its parts q4/2 and 2 + q4/2
+template <int FMT> struct I8p;
+
+// Thread (row, q4) makes columns 16*q4.. of its row in every step of 64 columns: part
+// 2*jj + q4/2 of half c (jj = the step within the half), weights 16*(q4 & 1).. of the part.
+template <> struct I8p<ILT_Q6_K> {
+  static constexpr int KCX = 4000;                           // isum = 256*hi + lo - KCX * (sum of xq)
+  struct Raw { int4 ql, qh; int2 sc; u32 d; };               // a half super-block's share
+  static __device__ __forceinline__ void load(Raw& r, __amdgpu_buffer_rsrc_t rw, u32 rowoff, int hb, int q4) {
+    const u32 b = rowoff + (u32)(hb >> 1) * ILT_Q6K_STRIDE;
+    const int c = hb & 1;
+    r.ql = ilt_bld16(rw, b + 64 * c + 16 * q4);              // ql[64c + 32*(part & 1) + l], part & 1 = q4 / 2, l = 16*(q4 & 1)..
+    r.qh = ilt_bld16(rw, b + 128 + 32 * c + 16 * (q4 & 1));
+    r.sc = ilt_bld8(rw, b + 192 + 8 * c);
+    r.d = ilt_bld2(rw, b + 208);
+  }
+  static __device__ __forceinline__ float d_of(const Raw& r) { return ilt_h2f((u16)r.d); }
+  // J: the step within the super-block
+  static __device__ __forceinline__ void planes(const Raw& r, int J, int q4, int* hi, int* lo) {
+    const int jj = J & 1;
+    const int sc = (int)(i8)(((u32)(jj ? r.sc.y : r.sc.x) >> (8 * q4)) & 0xFF);      // scale 8c + 2*part + (q4 & 1)
+    const int cpair = (4128 - 32 * sc) * 0x10001;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      const u32 v = ((word_of(r.ql, i) >> (4 * jj)) & 0x0F0F0F0F) | (((word_of(r.qh, i) >> (4 * jj + 2 * (q4 >> 1))) & 0x03030303) << 4);
+      const u32 te = (u32)(__mul24((int)(v & 0x00FF00FF), sc) + cpair), to = (u32)(__mul24((int)((v >> 8) & 0x00FF00FF), sc) + cpair);
+      hi[i] = (int)__builtin_amdgcn_perm(to, te, 0x07030501u);                  // the fields' high bytes, in the weights' order
+      lo[i] = (int)(__builtin_amdgcn_perm(to, te, 0x06020400u) ^ 0x80808080u);   // their low bytes - 128
+    }
+  }
+};
+
+// Q4_K: step J of a super-block is groups 2J (low nibbles) and 2J+1 (high nibbles) of qs[32J..32J+31].
+template <> struct I8p<ILT_Q4_K> {
+  static constexpr int KCX = -128;
+  struct Raw { int4 q[2]; v3i_ s; u32 dd; };                 // a half's two steps of quants (the thread's 16 bytes), the block's 12 scale bytes, d and dmin
+  static __device__ __forceinline__ void load(Raw& r, __amdgpu_buffer_rsrc_t rw, u32 rowoff, int hb, int q4) {
+    const u32 b = rowoff + (u32)(hb >> 1) * 144;
+    r.q[0] = ilt_bld16(rw, b + 16 + 64 * (hb & 1) + 16 * (q4 & 1));
+    r.q[1] = ilt_bld16(rw, b + 48 + 64 * (hb & 1) + 16 * (q4 & 1));
+    r.s = __builtin_amdgcn_raw_buffer_load_b96(rw, b + 4, 0, 0);
+    r.dd = ilt_bld4(rw, b);
+  }
+  static __device__ __forceinline__ float d_of(const Raw& r) { return ilt_h2f((u16)(r.dd & 0xFFFF)); }
+  static __device__ __forceinline__ float dmin_of(const Raw& r) { return ilt_h2f((u16)(r.dd >> 16)); }
+  static __device__ __forceinline__ u32 sbyte(const Raw& r, int i) { return ((u32)(i < 4 ? r.s.x : i < 8 ? r.s.y : r.s.z) >> (8 * (i & 3))) & 0xFF; }
+  // scale-min-k4 (kquant.lisp:64-72), g a constant
+  static __device__ __forceinline__ u32 scale_of(const Raw& r, int g) {
+    return g < 4 ? (sbyte(r, g) & 63) : ((sbyte(r, g + 4) & 15) | ((sbyte(r, g - 4) >> 6) << 4));
+  }
+  static __device__ __forceinline__ u32 min_of(const Raw& r, int g) {
+    return g < 4 ? (sbyte(r, g + 4) & 63) : ((sbyte(r, g + 4) >> 4) | ((sbyte(r, g) >> 6) << 4));
+  }
+  static __device__ __forceinline__ void planes(const Raw& r, int J, int q4, int* hi, int* lo) {
+    const int jp = q4 >> 1;                                  // group 2J + jp
+    const int sc = (int)(jp ? scale_of(r, 2 * J + 1) : scale_of(r, 2 * J));
+    const int4& q = r.q[J & 1];
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      const u32 v = (word_of(q, i) >> (4 * jp)) & 0x0F0F0F0F;
+      const u32 te = (u32)__mul24((int)(v & 0x00FF00FF), sc), to = (u32)__mul24((int)((v >> 8) & 0x00FF00FF), sc);
+      hi[i] = (int)__builtin_amdgcn_perm(to, te, 0x07030501u);
+      lo[i] = (int)(__builtin_amdgcn_perm(to, te, 0x06020400u) ^ 0x80808080u);
+    }
+  }
+};
 
 struct I8pSmem {
   __align__(16) u8 xs[3][128 * 64];       // the tokens' quants, 64 columns a step
   __align__(16) u8 wh[2][128 * 64];       // the rows' hi plane, the step's and the next step's
   __align__(16) u8 wl[2][128 * 64];       // lo plane
-  float wd[128];                          // of the super-block: d of the rows,
+  float wd[128], wdm[128];                // of the super-block: d (and Q4_K's dmin) of the rows,
   float xd[128];                          //   the tokens' scales
-  int cx[128];                            //   and 4000 * the sum of their quants
+  int cx[128];                            //   and KCX * the sum of their quants
+  // Q4_K's minimums: the rows' eight minimums and their sum; the tokens' eight sums of 32 as planes
+  // (U = sum + 4096: U >> 8, and (U & 255) - 128)
+  int2 wmn[128]; int wms[128];
+  int2 bh[128], bl[128];
   u32 scan[256];
   int tile_z, tile_t0, tile_n;
 };
@@ -836,12 +909,18 @@ struct I8pSmem {
 __device__ __forceinline__ void ilt_lds_st4_untracked(void* p, u32 v) {
   asm volatile("ds_write_b32 %0, %1" :: "v"((u32)(uintptr_t)(ILT_LDS void*)p), "v"(v) : "memory");
 }
+__device__ __forceinline__ void ilt_lds_st8_untracked(void* p, u32 a, u32 b) {
+  const uint2 v = {a, b};
+  asm volatile("ds_write_b64 %0, %1" :: "v"((u32)(uintptr_t)(ILT_LDS void*)p), "v"(v) : "memory");
+}
 
 // 128 rows x 128 tokens a workgroup of eight waves (one workgroup a CU, two waves a SIMD: a
 // wave's two planes of integer sums, its float sums and the raw bytes leave no room for more);
-// wave w: rows 32*(w/2).., tokens 64*(w%2)...  Thread (row, q4) makes columns 16*q4.. of its row
-// in every step.
+// wave w: rows 32*(w/2).., tokens 64*(w%2)...
+template <int FMT>
 __global__ __launch_bounds__(512, 1) void gemm_i8p_kernel(BfParams p) {
+  typedef I8p<FMT> F;
+  typedef typename F::Raw Raw;
   constexpr int TM = 128, TN = 128, NA = 2, NI = 1;
   constexpr int WL = 4, XL = 5;                              // loads of a raw set, of a token's constants
   constexpr int KW = 64;                                     // columns a step
@@ -869,37 +948,44 @@ __global__ __launch_bounds__(512, 1) void gemm_i8p_kernel(BfParams p) {
 #pragma unroll
     for (int i = 0; i < 4; i++) c_bs[i] = bsp[4 * sb + i];
   };
-  auto store_consts = [&](const I8pRaw& ra) {                // after a barrier that ends the last block's reads
+  auto store_consts = [&](const Raw& ra) {                   // after a barrier that ends the last block's reads
     if (t < 128) {
       int sx = 0;
 #pragma unroll
       for (int i = 0; i < 4; i++) sx += c_bs[i].x + c_bs[i].y + c_bs[i].z + c_bs[i].w;
       ilt_lds_st4_untracked(&S.xd[t], __builtin_bit_cast(u32, c_yd));
-      ilt_lds_st4_untracked(&S.cx[t], (u32)(4000 * sx));
-    }
-    if (q4 == 0) ilt_lds_st4_untracked(&S.wd[wrow], __builtin_bit_cast(u32, ilt_h2f((u16)ra.d)));
-  };
-  auto load_raw = [&](I8pRaw& r, int hb) {                   // half super-block hb of the thread's row
-    const u32 b = wrowoff + (u32)(hb >> 1) * ILT_Q6K_STRIDE;
-    const int c = hb & 1;
-    r.ql = ilt_bld16(rw, b + 64 * c + 16 * q4);              // ql[64c + 32*(part & 1) + l], part & 1 = q4 / 2, l = 16*(q4 & 1)..
-    r.qh = ilt_bld16(rw, b + 128 + 32 * c + 16 * (q4 & 1));
-    r.sc = ilt_bld8(rw, b + 192 + 8 * c);
-    r.d = ilt_bld2(rw, b + 208);
-  };
-  auto issue_x = [&](int stage, int ks) { ilt_g2lds16(xbase + ks * KW + xoff, S.xs[stage] + wave * 1024); };
-  // 16 weights of part 2*jj + q4/2 of the half in r, as the two planes, into a pair of slabs
-  auto dequant_to = [&](const I8pRaw& r, int jj, int slab) {
-    const int sc = (int)(i8)(((u32)(jj ? r.sc.y : r.sc.x) >> (8 * q4)) & 0xFF);      // scale 8c + 2*part + (q4 & 1)
-    const int cpair = (4128 - 32 * sc) * 0x10001;
-    int hi[4], lo[4];
+      ilt_lds_st4_untracked(&S.cx[t], (u32)(F::KCX * sx));
+      if constexpr (FMT == ILT_Q4_K) {
+        u32 h[2] = {0, 0}, l[2] = {0, 0};
 #pragma unroll
-    for (int i = 0; i < 4; i++) {
-      const u32 v = ((word_of(r.ql, i) >> (4 * jj)) & 0x0F0F0F0F) | (((word_of(r.qh, i) >> (4 * jj + 2 * (q4 >> 1))) & 0x03030303) << 4);
-      const u32 te = (u32)(__mul24((int)(v & 0x00FF00FF), sc) + cpair), to = (u32)(__mul24((int)((v >> 8) & 0x00FF00FF), sc) + cpair);
-      hi[i] = (int)__builtin_amdgcn_perm(to, te, 0x07030501u);                  // the fields' high bytes, in the weights' order
-      lo[i] = (int)(__builtin_amdgcn_perm(to, te, 0x06020400u) ^ 0x80808080u);   // their low bytes - 128
+        for (int g = 0; g < 8; g++) {                        // the sum of group g's 32 quants
+          const int4& bs = c_bs[g >> 1];
+          const u32 u = (u32)(((g & 1) ? bs.z + bs.w : bs.x + bs.y) + 4096);
+          h[g >> 2] |= (u >> 8) << (8 * (g & 3));
+          l[g >> 2] |= ((u & 255) ^ 128) << (8 * (g & 3));
+        }
+        ilt_lds_st8_untracked(&S.bh[t], h[0], h[1]);
+        ilt_lds_st8_untracked(&S.bl[t], l[0], l[1]);
+      }
     }
+    if (q4 == 0) {
+      ilt_lds_st4_untracked(&S.wd[wrow], __builtin_bit_cast(u32, F::d_of(ra)));
+      if constexpr (FMT == ILT_Q4_K) {
+        ilt_lds_st4_untracked(&S.wdm[wrow], __builtin_bit_cast(u32, F::dmin_of(ra)));
+        u32 m[2] = {0, 0}, ms = 0;
+#pragma unroll
+        for (int g = 0; g < 8; g++) { const u32 mn = F::min_of(ra, g); m[g >> 2] |= mn << (8 * (g & 3)); ms += mn; }
+        ilt_lds_st8_untracked(&S.wmn[wrow], m[0], m[1]);
+        ilt_lds_st4_untracked(&S.wms[wrow], ms);
+      }
+    }
+  };
+  auto load_raw = [&](Raw& r, int hb) { F::load(r, rw, wrowoff, hb, q4); };       // half super-block hb of the thread's row
+  auto issue_x = [&](int stage, int ks) { ilt_g2lds16(xbase + ks * KW + xoff, S.xs[stage] + wave * 1024); };
+  // the thread's 16 weights of step J of a super-block, out of the set that holds its half, into a pair of slabs
+  auto dequant_to = [&](const Raw& r, int J, int slab) {
+    int hi[4], lo[4];
+    F::planes(r, J, q4, hi, lo);
     ilt_lds_st16_untracked(S.wh[slab] + wdst, hi[0], hi[1], hi[2], hi[3]);
     ilt_lds_st16_untracked(S.wl[slab] + wdst, lo[0], lo[1], lo[2], lo[3]);
   };
@@ -922,7 +1008,7 @@ __global__ __launch_bounds__(512, 1) void gemm_i8p_kernel(BfParams p) {
   // slab ks while it makes step ks+1's planes, so A is free after step 0 and loaded again (the
   // next block's) in step 1, B after step 2 and loaded in step 3.  The next block's token
   // constants are loaded in step 2 and stored in the next step 0.
-  I8pRaw rawa, rawb;
+  Raw rawa, rawb;
   load_raw(rawa, 0);
   load_consts(0);
   issue_x(0, 0);
@@ -948,6 +1034,7 @@ __global__ __launch_bounds__(512, 1) void gemm_i8p_kernel(BfParams p) {
     const u8* xs = S.xs[st0];
     const u8* whs = S.wh[J & 1];
     const u8* wls = S.wl[J & 1];
+    const v16i_ zero = {};
 #pragma unroll
     for (int kk = 0; kk < 2; kk++) {
       v4i_ af[NA];
@@ -956,26 +1043,50 @@ __global__ __launch_bounds__(512, 1) void gemm_i8p_kernel(BfParams p) {
       const v4i_ bh = *(const v4i_*)(whs + (boff ^ (32 * kk))), bl = *(const v4i_*)(wls + (boff ^ (32 * kk)));
       if (kk == 0) {       // step ks+1's planes: J+1 = 1 from A, 2 and 3 from B, 4 = the next block's 0 from A (past the last step: planes nobody reads)
         if (J == 0) dequant_to(rawa, 1, 1);
-        if (J == 1) dequant_to(rawb, 0, 0);
-        if (J == 2) dequant_to(rawb, 1, 1);
+        if (J == 1) dequant_to(rawb, 2, 0);
+        if (J == 2) dequant_to(rawb, 3, 1);
         if (J == 3) dequant_to(rawa, 0, 0);
       }
 #pragma unroll
-      for (int a = 0; a < NA; a++) {
-        const v16i_ zero = {};                                 // a super-block's first products start its integer sums
+      for (int a = 0; a < NA; a++) {                         // a super-block's first products start its integer sums
         ah[a] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[a], bh, (J == 0 && kk == 0) ? zero : ah[a], 0, 0, 0);
         al[a] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[a], bl, (J == 0 && kk == 0) ? zero : al[a], 0, 0, 0);
       }
     }
-    if (J == 3) {          // the super-block is complete: sum += (d * yd) * float(isum), as the CPU path adds it
-      const float d = S.wd[wr0 + l32];
+    if (J == 3) {          // the super-block is complete: its terms, as the CPU path adds them
+      const int row = wr0 + l32;
+      const float d = S.wd[row];
+      if constexpr (FMT == ILT_Q4_K) {
+        // im = sum over the groups of minimum * (sum of 32 quants) = 256*(mn.hi) + (mn.lo) - 3968*(sum of mn)
+        const float dm = S.wdm[row];
+        const int ms = 3968 * S.wms[row];
+        const int2 mnb = S.wmn[row];
+        const v4i_ bm = { lh ? 0 : mnb.x, lh ? 0 : mnb.y, 0, 0 };
 #pragma unroll
-      for (int a = 0; a < NA; a++) {
+        for (int a = 0; a < NA; a++) {
+          const int2 th = S.bh[wt0 + 32 * a + l32], tl = S.bl[wt0 + 32 * a + l32];
+          const v4i_ fh = { lh ? 0 : th.x, lh ? 0 : th.y, 0, 0 }, fl = { lh ? 0 : tl.x, lh ? 0 : tl.y, 0, 0 };
+          const v16i_ mh = __builtin_amdgcn_mfma_i32_32x32x32_i8(fh, bm, zero, 0, 0, 0);
+          const v16i_ ml = __builtin_amdgcn_mfma_i32_32x32x32_i8(fl, bm, zero, 0, 0, 0);
 #pragma unroll
-        for (int r = 0; r < 16; r++) {
-          const int tk = wt0 + 32 * a + 8 * (r >> 2) + 4 * lh + (r & 3);
-          const int isum = 256 * ah[a][r] + al[a][r] - S.cx[tk];
-          sum[a][0][r] = sum[a][0][r] + (d * S.xd[tk]) * (float)isum;
+          for (int r = 0; r < 16; r++) {
+            const int tk = wt0 + 32 * a + 8 * (r >> 2) + 4 * lh + (r & 3);
+            const float yd = S.xd[tk];
+            const int im = 256 * mh[r] + ml[r] - ms;
+            const int isum = 256 * ah[a][r] + al[a][r] - S.cx[tk];
+            sum[a][0][r] = sum[a][0][r] - (yd * dm) * (float)im;
+            sum[a][0][r] = sum[a][0][r] + (yd * d) * (float)isum;
+          }
+        }
+      } else {
+#pragma unroll
+        for (int a = 0; a < NA; a++) {
+#pragma unroll
+          for (int r = 0; r < 16; r++) {
+            const int tk = wt0 + 32 * a + 8 * (r >> 2) + 4 * lh + (r & 3);
+            const int isum = 256 * ah[a][r] + al[a][r] - S.cx[tk];
+            sum[a][0][r] = sum[a][0][r] + (d * S.xd[tk]) * (float)isum;
+          }
         }
       }
     }
@@ -1265,13 +1376,14 @@ hipError_t ilt_k_gemm_bf16_id_glu(int fmt, const uint64_t* ptrs, long long add_g
 hipError_t ilt_k_gemm_i8_planes(int fmt, const uint8_t* w, long long row_bytes, int rows, int cols, const int8_t* xq, const float* xd,
                                 const int* bsums, int ntok, float* y, const float* bias, int acc, hipStream_t st) {
   if (ntok <= 0 || rows <= 0) return hipSuccess;
-  if (fmt != ILT_Q6_K || cols % 256 != 0 || (long long)rows * 1024 >= 0x7FFFFFFFLL) return hipErrorInvalidValue;
+  if ((fmt != ILT_Q6_K && fmt != ILT_Q4_K) || cols % 256 != 0 || (long long)rows * 1024 >= 0x7FFFFFFFLL) return hipErrorInvalidValue;
   BfParams p = {};
   p.w = w; p.rows = rows; p.cols = cols; p.row_bytes = row_bytes; p.x = (const u16*)xq; p.xd = xd; p.bsums = bsums;
   p.y = y; p.bias = bias; p.acc = acc; p.ntok = ntok; p.ldy = rows;
   const long long total = (long long)((ntok + 127) / 128) * ((rows + 127) / 128), per = (total + 7) / 8;
   if (per * 8 > 0x7FFFFFFFLL) return hipErrorInvalidValue;
-  hipLaunchKernelGGL(gemm_i8p_kernel, dim3((unsigned)(per * 8)), dim3(512), 0, st, p);
+  if (fmt == ILT_Q6_K) hipLaunchKernelGGL(gemm_i8p_kernel<ILT_Q6_K>, dim3((unsigned)(per * 8)), dim3(512), 0, st, p);
+  else hipLaunchKernelGGL(gemm_i8p_kernel<ILT_Q4_K>, dim3((unsigned)(per * 8)), dim3(512), 0, st, p);
   return hipGetLastError();
 }
 
