@@ -54,7 +54,7 @@ TRAFFIC = {"c1": {"up": _t(2507.3, 96.0), "down": _t(2443.0, 28.0)},
                   "head": _t(175546.1, 636.4)},
            # one product: two-pass = the 256-tile launch plus the 128-tile launch for the rows left over
            "c3": {"bf16-1pass": _t(519803.0, 278528.0), "bf16-2pass": _t(491863.8 + 61498.0, 262144.0 + 16384.0),
-                  "bf16-resident": _t(491863.8 + 61498.0, 262144.0 + 16384.0)},
+                  "bf16-resident": _t(491863.8 + 61498.0, 262144.0 + 16384.0), "int8": _t(510205.6, 278528.0)},
            "c4": {"d4_mv_glu_iq2_xxs": _t(12854.8, 96.0), "d4_mv_q2_k_f32": _t(8394.5, 96.0), "d4_mvq8_glu": _t(8833.8, 96.0)},
            # per launch, over the step's two grouped launches (gate + up + activation; down)
            "c5": {"mm_id": _t((569198.8 + 334480.4) / 2, (98304.6 + 393216.0) / 2)}}
