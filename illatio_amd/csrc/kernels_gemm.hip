@@ -427,11 +427,11 @@ hipError_t ilt_k_gemm_i8(int fmt, const uint8_t* w, const uint16_t* wd, long lon
                          const int8_t* xq, const float* xs, const int* bsums, int ntok, float* y, const float* bias,
                          int acc, hipStream_t st) {
   if (ntok <= 0 || rows <= 0) return hipSuccess;
-  // Q6_K and Q4_K with enough tokens and rows to fill 128 x 128 tiles: the pipelined kernel with the weights as
-  // two int8 planes, the same bits.  ILT_I8_PLANES (tests): "0" never, "1" whenever the format allows.
+  // Q6_K, Q4_K and Q2_K with enough tokens and rows to fill 128 x 128 tiles: the pipelined kernel with scale * quant
+  // as int8 planes, the same bits.  ILT_I8_PLANES (tests): "0" never, "1" whenever the format allows.
   const char* force = getenv("ILT_I8_PLANES");
   const int forced = force ? atoi(force) : -1;
-  if ((fmt == ILT_Q6_K || fmt == ILT_Q4_K) && cols % 256 == 0 && forced != 0 && (forced == 1 || (ntok >= 96 && rows >= 128)))
+  if ((fmt == ILT_Q6_K || fmt == ILT_Q4_K || fmt == ILT_Q2_K) && cols % 256 == 0 && forced != 0 && (forced == 1 || (ntok >= 96 && rows >= 128)))
     return ilt_k_gemm_i8_planes(fmt, w, row_bytes, rows, cols, xq, xs, bsums, ntok, y, bias, acc, st);
   GemmParams p = {};
   p.w = w; p.wdq = wd; p.rows = rows; p.cols = cols; p.row_bytes = row_bytes;
@@ -444,6 +444,14 @@ hipError_t ilt_k_gemm_i8_id(int fmt, const uint64_t* ptrs, long long add, const 
                             const int* bsums, long long total_rows, float* y, hipStream_t st) {
   if (total_rows <= 0 || rows <= 0 || ne <= 0) return hipSuccess;
   if (ne > 256) return hipErrorInvalidValue;
+  {
+    // the experts' Q2_K (and Q4_K / Q6_K) matrices on the planes kernel when the groups average at least half a tile of 128 rows
+    const char* force = getenv("ILT_I8_PLANES");
+    const int forced = force ? atoi(force) : -1;
+    if ((fmt == ILT_Q6_K || fmt == ILT_Q4_K || fmt == ILT_Q2_K) && cols % 256 == 0 && forced != 0 &&
+        (forced == 1 || (total_rows >= 64LL * ne && rows >= 128)))
+      return ilt_k_gemm_i8_planes_id(fmt, ptrs, add, counts, bases, ne, row_bytes, rows, cols, xq, xs, bsums, total_rows, y, st);
+  }
   GemmParams p = {};
   p.ptrs = ptrs; p.add = add; p.counts = counts; p.bases = bases; p.ne = ne;
   p.rows = rows; p.cols = cols; p.row_bytes = row_bytes;

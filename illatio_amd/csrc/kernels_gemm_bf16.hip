@@ -831,6 +831,7 @@ template <int FMT> struct I8p;
 // 2*jj + q4/2 of half c (jj = the step within the half), weights 16*(q4 & 1).. of the part.
 template <> struct I8p<ILT_Q6_K> {
   static constexpr int KCX = 4000;                           // isum = 256*hi + lo - KCX * (sum of xq)
+  static constexpr int PLANES = 2, WL = 4;                   // planes; loads of a raw set
   struct Raw { int4 ql, qh; int2 sc; u32 d; };               // a half super-block's share
   static __device__ __forceinline__ void load(Raw& r, __amdgpu_buffer_rsrc_t rw, u32 rowoff, int hb, int q4) {
     const u32 b = rowoff + (u32)(hb >> 1) * ILT_Q6K_STRIDE;
@@ -859,6 +860,7 @@ template <> struct I8p<ILT_Q6_K> {
 // Q4_K: step J of a super-block is groups 2J (low nibbles) and 2J+1 (high nibbles) of qs[32J..32J+31].
 template <> struct I8p<ILT_Q4_K> {
   static constexpr int KCX = -128;
+  static constexpr int PLANES = 2, WL = 4;
   struct Raw { int4 q[2]; v3i_ s; u32 dd; };                 // a half's two steps of quants (the thread's 16 bytes), the block's 12 scale bytes, d and dmin
   static __device__ __forceinline__ void load(Raw& r, __amdgpu_buffer_rsrc_t rw, u32 rowoff, int hb, int q4) {
     const u32 b = rowoff + (u32)(hb >> 1) * 144;
@@ -887,6 +889,31 @@ template <> struct I8p<ILT_Q4_K> {
       const u32 te = (u32)__mul24((int)(v & 0x00FF00FF), sc), to = (u32)__mul24((int)((v >> 8) & 0x00FF00FF), sc);
       hi[i] = (int)__builtin_amdgcn_perm(to, te, 0x07030501u);
       lo[i] = (int)(__builtin_amdgcn_perm(to, te, 0x06020400u) ^ 0x80808080u);
+    }
+  }
+};
+
+// Q2_K: sc*q is at most 45, one plane.  Step J of a super-block is parts 2*(J&1) and 2*(J&1)+1 of half J/2, all four
+// parts of a half in the same 32 bytes of quants, two bits each; the minimums' term over the sixteen groups of 16.
+template <> struct I8p<ILT_Q2_K> {
+  static constexpr int KCX = 0;
+  static constexpr int PLANES = 1, WL = 3;
+  struct Raw { int4 q, s; u32 dd; };                         // the thread's 16 bytes of the half's quants, the block's 16 scale bytes, d and dmin
+  static __device__ __forceinline__ void load(Raw& r, __amdgpu_buffer_rsrc_t rw, u32 rowoff, int hb, int q4) {
+    const u32 b = rowoff + (u32)(hb >> 1) * 84;
+    r.q = ilt_bld16(rw, b + 16 + 32 * (hb & 1) + 16 * (q4 & 1));
+    r.s = ilt_bld16(rw, b);
+    r.dd = ilt_bld4(rw, b + 80);
+  }
+  static __device__ __forceinline__ float d_of(const Raw& r) { return ilt_h2f((u16)(r.dd & 0xFFFF)); }
+  static __device__ __forceinline__ float dmin_of(const Raw& r) { return ilt_h2f((u16)(r.dd >> 16)); }
+  static __device__ __forceinline__ void planes(const Raw& r, int J, int q4, int*, int* lo) {
+    const int c = J >> 1, jj = J & 1;
+    const u32 sc = (word_of(r.s, 2 * c + jj) >> (8 * q4)) & 15;             // scale 8c + 2*part + (q4 & 1), part = 2jj + q4/2
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      const u32 v = (word_of(r.q, i) >> (4 * jj + 2 * (q4 >> 1))) & 0x03030303;
+      lo[i] = (int)(v * sc);                                  // four products of at most 45: no carries between the bytes
     }
   }
 };
@@ -922,9 +949,14 @@ __global__ __launch_bounds__(512, 1) void gemm_i8p_kernel(BfParams p) {
   typedef I8p<FMT> F;
   typedef typename F::Raw Raw;
   constexpr int TM = 128, TN = 128, NA = 2, NI = 1;
-  constexpr int WL = 4, XL = 5;                              // loads of a raw set, of a token's constants
+  constexpr int WL = F::WL, XL = 5;                          // loads of a raw set, of a token's constants
+  constexpr bool TWO = F::PLANES == 2;
   constexpr int KW = 64;                                     // columns a step
   __shared__ I8pSmem S;
+  // Q2_K has no hi plane: its room holds the minimums' operands (sixteen groups: 16 bytes a row or token)
+  int4* const q2_wmn = (int4*)S.wh[0];
+  int4* const q2_bh = q2_wmn + 128;
+  int4* const q2_bl = q2_bh + 128;
   const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
 
   long tok0; int ntok, rt; const u8* w = p.w;
@@ -967,6 +999,17 @@ __global__ __launch_bounds__(512, 1) void gemm_i8p_kernel(BfParams p) {
         ilt_lds_st8_untracked(&S.bh[t], h[0], h[1]);
         ilt_lds_st8_untracked(&S.bl[t], l[0], l[1]);
       }
+      if constexpr (FMT == ILT_Q2_K) {
+        u32 h[4] = {0, 0, 0, 0}, l[4] = {0, 0, 0, 0};
+#pragma unroll
+        for (int g = 0; g < 16; g++) {                       // the sum of group g's 16 quants + 2048, as planes
+          const u32 u = (u32)(word_of(c_bs[g >> 2], g & 3) + 2048);
+          h[g >> 2] |= (u >> 8) << (8 * (g & 3));
+          l[g >> 2] |= ((u & 255) ^ 128) << (8 * (g & 3));
+        }
+        ilt_lds_st16_untracked(&q2_bh[t], (int)h[0], (int)h[1], (int)h[2], (int)h[3]);
+        ilt_lds_st16_untracked(&q2_bl[t], (int)l[0], (int)l[1], (int)l[2], (int)l[3]);
+      }
     }
     if (q4 == 0) {
       ilt_lds_st4_untracked(&S.wd[wrow], __builtin_bit_cast(u32, F::d_of(ra)));
@@ -978,6 +1021,17 @@ __global__ __launch_bounds__(512, 1) void gemm_i8p_kernel(BfParams p) {
         ilt_lds_st8_untracked(&S.wmn[wrow], m[0], m[1]);
         ilt_lds_st4_untracked(&S.wms[wrow], ms);
       }
+      if constexpr (FMT == ILT_Q2_K) {
+        ilt_lds_st4_untracked(&S.wdm[wrow], __builtin_bit_cast(u32, F::dmin_of(ra)));
+        u32 m[4], ms = 0;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {                        // the minimums: the scale bytes' high nibbles
+          m[i] = (word_of(ra.s, i) >> 4) & 0x0F0F0F0F;
+          ms += (m[i] & 0xFF) + ((m[i] >> 8) & 0xFF) + ((m[i] >> 16) & 0xFF) + (m[i] >> 24);
+        }
+        ilt_lds_st16_untracked(&q2_wmn[wrow], (int)m[0], (int)m[1], (int)m[2], (int)m[3]);
+        ilt_lds_st4_untracked(&S.wms[wrow], ms);
+      }
     }
   };
   auto load_raw = [&](Raw& r, int hb) { F::load(r, rw, wrowoff, hb, q4); };       // half super-block hb of the thread's row
@@ -986,7 +1040,7 @@ __global__ __launch_bounds__(512, 1) void gemm_i8p_kernel(BfParams p) {
   auto dequant_to = [&](const Raw& r, int J, int slab) {
     int hi[4], lo[4];
     F::planes(r, J, q4, hi, lo);
-    ilt_lds_st16_untracked(S.wh[slab] + wdst, hi[0], hi[1], hi[2], hi[3]);
+    if constexpr (TWO) ilt_lds_st16_untracked(S.wh[slab] + wdst, hi[0], hi[1], hi[2], hi[3]);
     ilt_lds_st16_untracked(S.wl[slab] + wdst, lo[0], lo[1], lo[2], lo[3]);
   };
 
@@ -1040,7 +1094,9 @@ __global__ __launch_bounds__(512, 1) void gemm_i8p_kernel(BfParams p) {
       v4i_ af[NA];
 #pragma unroll
       for (int a = 0; a < NA; a++) af[a] = *(const v4i_*)(xs + (aoff[a] ^ (32 * kk)));
-      const v4i_ bh = *(const v4i_*)(whs + (boff ^ (32 * kk))), bl = *(const v4i_*)(wls + (boff ^ (32 * kk)));
+      v4i_ bh = {};
+      if constexpr (TWO) bh = *(const v4i_*)(whs + (boff ^ (32 * kk)));
+      const v4i_ bl = *(const v4i_*)(wls + (boff ^ (32 * kk)));
       if (kk == 0) {       // step ks+1's planes: J+1 = 1 from A, 2 and 3 from B, 4 = the next block's 0 from A (past the last step: planes nobody reads)
         if (J == 0) dequant_to(rawa, 1, 1);
         if (J == 1) dequant_to(rawb, 2, 0);
@@ -1049,7 +1105,7 @@ __global__ __launch_bounds__(512, 1) void gemm_i8p_kernel(BfParams p) {
       }
 #pragma unroll
       for (int a = 0; a < NA; a++) {                         // a super-block's first products start its integer sums
-        ah[a] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[a], bh, (J == 0 && kk == 0) ? zero : ah[a], 0, 0, 0);
+        if constexpr (TWO) ah[a] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[a], bh, (J == 0 && kk == 0) ? zero : ah[a], 0, 0, 0);
         al[a] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[a], bl, (J == 0 && kk == 0) ? zero : al[a], 0, 0, 0);
       }
     }
@@ -1076,6 +1132,28 @@ __global__ __launch_bounds__(512, 1) void gemm_i8p_kernel(BfParams p) {
             const int isum = 256 * ah[a][r] + al[a][r] - S.cx[tk];
             sum[a][0][r] = sum[a][0][r] - (yd * dm) * (float)im;
             sum[a][0][r] = sum[a][0][r] + (yd * d) * (float)isum;
+          }
+        }
+      } else if constexpr (FMT == ILT_Q2_K) {
+        // im = sum over the sixteen groups of minimum * (sum of 16 quants) = 256*(mn.hi) + (mn.lo) - 1920*(sum of mn)
+        const float dm = S.wdm[row];
+        const int ms = 1920 * S.wms[row];
+        const int4 mnb = q2_wmn[row];
+        const v4i_ bm = { lh ? 0 : mnb.x, lh ? 0 : mnb.y, lh ? 0 : mnb.z, lh ? 0 : mnb.w };
+#pragma unroll
+        for (int a = 0; a < NA; a++) {
+          const int4 th = q2_bh[wt0 + 32 * a + l32], tl = q2_bl[wt0 + 32 * a + l32];
+          const v4i_ fh = { lh ? 0 : th.x, lh ? 0 : th.y, lh ? 0 : th.z, lh ? 0 : th.w };
+          const v4i_ fl = { lh ? 0 : tl.x, lh ? 0 : tl.y, lh ? 0 : tl.z, lh ? 0 : tl.w };
+          const v16i_ mh = __builtin_amdgcn_mfma_i32_32x32x32_i8(fh, bm, zero, 0, 0, 0);
+          const v16i_ ml = __builtin_amdgcn_mfma_i32_32x32x32_i8(fl, bm, zero, 0, 0, 0);
+#pragma unroll
+          for (int r = 0; r < 16; r++) {
+            const int tk = wt0 + 32 * a + 8 * (r >> 2) + 4 * lh + (r & 3);
+            const float yd = S.xd[tk];
+            const int im = 256 * mh[r] + ml[r] - ms;
+            sum[a][0][r] = sum[a][0][r] + ((-yd) * dm) * (float)im;
+            sum[a][0][r] = sum[a][0][r] + (yd * d) * (float)al[a][r];
           }
         }
       } else {
@@ -1373,18 +1451,37 @@ hipError_t ilt_k_gemm_bf16_id_glu(int fmt, const uint64_t* ptrs, long long add_g
   return launch_regb<ILT_IQ2_XXS, true>(p, total_rows / 128 + ne, st);
 }
 
+static hipError_t launch_i8p(int fmt, const BfParams& p, long long token_tiles, hipStream_t st) {
+  if ((fmt != ILT_Q6_K && fmt != ILT_Q4_K && fmt != ILT_Q2_K) || p.cols % 256 != 0 || (long long)p.rows * 1024 >= 0x7FFFFFFFLL)
+    return hipErrorInvalidValue;
+  const long long total = token_tiles * ((p.rows + 127) / 128), per = (total + 7) / 8;
+  if (per * 8 > 0x7FFFFFFFLL) return hipErrorInvalidValue;
+  const dim3 grid((unsigned)(per * 8));
+  if (fmt == ILT_Q6_K) hipLaunchKernelGGL(gemm_i8p_kernel<ILT_Q6_K>, grid, dim3(512), 0, st, p);
+  else if (fmt == ILT_Q4_K) hipLaunchKernelGGL(gemm_i8p_kernel<ILT_Q4_K>, grid, dim3(512), 0, st, p);
+  else hipLaunchKernelGGL(gemm_i8p_kernel<ILT_Q2_K>, grid, dim3(512), 0, st, p);
+  return hipGetLastError();
+}
+
 hipError_t ilt_k_gemm_i8_planes(int fmt, const uint8_t* w, long long row_bytes, int rows, int cols, const int8_t* xq, const float* xd,
                                 const int* bsums, int ntok, float* y, const float* bias, int acc, hipStream_t st) {
   if (ntok <= 0 || rows <= 0) return hipSuccess;
-  if ((fmt != ILT_Q6_K && fmt != ILT_Q4_K) || cols % 256 != 0 || (long long)rows * 1024 >= 0x7FFFFFFFLL) return hipErrorInvalidValue;
   BfParams p = {};
   p.w = w; p.rows = rows; p.cols = cols; p.row_bytes = row_bytes; p.x = (const u16*)xq; p.xd = xd; p.bsums = bsums;
   p.y = y; p.bias = bias; p.acc = acc; p.ntok = ntok; p.ldy = rows;
-  const long long total = (long long)((ntok + 127) / 128) * ((rows + 127) / 128), per = (total + 7) / 8;
-  if (per * 8 > 0x7FFFFFFFLL) return hipErrorInvalidValue;
-  if (fmt == ILT_Q6_K) hipLaunchKernelGGL(gemm_i8p_kernel<ILT_Q6_K>, dim3((unsigned)(per * 8)), dim3(512), 0, st, p);
-  else hipLaunchKernelGGL(gemm_i8p_kernel<ILT_Q4_K>, dim3((unsigned)(per * 8)), dim3(512), 0, st, p);
-  return hipGetLastError();
+  return launch_i8p(fmt, p, (ntok + 127) / 128, st);
+}
+
+hipError_t ilt_k_gemm_i8_planes_id(int fmt, const uint64_t* ptrs, long long add, const uint32_t* counts, const uint32_t* bases, int ne,
+                                   long long row_bytes, int rows, int cols, const int8_t* xq, const float* xd, const int* bsums,
+                                   long long total_rows, float* y, hipStream_t st) {
+  if (total_rows <= 0 || rows <= 0 || ne <= 0) return hipSuccess;
+  if (ne > 256) return hipErrorInvalidValue;
+  BfParams p = {};
+  p.ptrs = ptrs; p.add = add; p.counts = counts; p.bases = bases; p.ne = ne;
+  p.rows = rows; p.cols = cols; p.row_bytes = row_bytes; p.x = (const u16*)xq; p.xd = xd; p.bsums = bsums;
+  p.y = y; p.ntok = (int)total_rows; p.ldy = rows;
+  return launch_i8p(fmt, p, total_rows / 128 + ne, st);
 }
 
 hipError_t ilt_k_cvt_bf16_slabs(const float* x, uint16_t* out, int n, int cols, hipStream_t st) {

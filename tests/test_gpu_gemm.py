@@ -75,11 +75,16 @@ def test_dense_prefill_equals_cpu_matmul_bit_for_bit(dev, monkeypatch, qtype, ro
 
 @pytest.mark.parametrize("ne,d,ff,nu,n,clamp", [(8, 512, 256, 3, 37, 0.0), (16, 1024, 512, 4, 150, 0.6),
                                                  (12, 4096, 2048, 6, 96, 0.0)])
-def test_moe_prefill_chunk_bit_exact(dev, ne, d, ff, nu, n, clamp):
+@pytest.mark.parametrize("planes", [None, "0", "1"])        # the down product (Q2_K) on the 64 x 64 kernel / on the planes kernel
+def test_moe_prefill_chunk_bit_exact(dev, monkeypatch, ne, d, ff, nu, n, clamp, planes):
     """BASELINE config 5's sequence (route -> group -> gather -> grouped gate, up -> gated
     activation -> grouped down -> slot-ordered sum + shared) at reduced expert and token
     counts, Zipf-skewed routing, against the CPU path's chunk (ds4f.lisp:1169-1239)."""
     from illatio_amd import ds4f, hip
+    if planes is None:
+        monkeypatch.delenv("ILT_I8_PLANES", raising=False)
+    else:
+        monkeypatch.setenv("ILT_I8_PLANES", planes)
     rng = synth.make_rng(ne + d + n)
     gate = synth.weights(synth.IQ2_XXS, ne * ff, d, rng)
     up = synth.weights(synth.IQ2_XXS, ne * ff, d, rng)
