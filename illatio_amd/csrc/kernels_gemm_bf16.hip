@@ -843,7 +843,7 @@ template <> struct I8p<ILT_Q6_K> {
   }
   static __device__ __forceinline__ float d_of(const Raw& r) { return ilt_h2f((u16)r.d); }
   // J: the step within the super-block
-  static __device__ __forceinline__ void planes(const Raw& r, int J, int q4, int* hi, int* lo) {
+  template <typename SM> static __device__ __forceinline__ void planes(const Raw& r, int J, int q4, int* hi, int* lo, const SM&) {
     const int jj = J & 1;
     const int sc = (int)(i8)(((u32)(jj ? r.sc.y : r.sc.x) >> (8 * q4)) & 0xFF);      // scale 8c + 2*part + (q4 & 1)
     const int cpair = (4128 - 32 * sc) * 0x10001;
@@ -879,7 +879,7 @@ template <> struct I8p<ILT_Q4_K> {
   static __device__ __forceinline__ u32 min_of(const Raw& r, int g) {
     return g < 4 ? (sbyte(r, g + 4) & 63) : ((sbyte(r, g + 4) >> 4) | ((sbyte(r, g) >> 6) << 4));
   }
-  static __device__ __forceinline__ void planes(const Raw& r, int J, int q4, int* hi, int* lo) {
+  template <typename SM> static __device__ __forceinline__ void planes(const Raw& r, int J, int q4, int* hi, int* lo, const SM&) {
     const int jp = q4 >> 1;                                  // group 2J + jp
     const int sc = (int)(jp ? scale_of(r, 2 * J + 1) : scale_of(r, 2 * J));
     const int4& q = r.q[J & 1];
@@ -907,7 +907,7 @@ template <> struct I8p<ILT_Q2_K> {
   }
   static __device__ __forceinline__ float d_of(const Raw& r) { return ilt_h2f((u16)(r.dd & 0xFFFF)); }
   static __device__ __forceinline__ float dmin_of(const Raw& r) { return ilt_h2f((u16)(r.dd >> 16)); }
-  static __device__ __forceinline__ void planes(const Raw& r, int J, int q4, int*, int* lo) {
+  template <typename SM> static __device__ __forceinline__ void planes(const Raw& r, int J, int q4, int*, int* lo, const SM&) {
     const int c = J >> 1, jj = J & 1;
     const u32 sc = (word_of(r.s, 2 * c + jj) >> (8 * q4)) & 15;             // scale 8c + 2*part + (q4 & 1), part = 2jj + q4/2
 #pragma unroll
@@ -925,12 +925,55 @@ struct I8pSmem {
   float wd[128], wdm[128];                // of the super-block: d (and Q4_K's dmin) of the rows,
   float xd[128];                          //   the tokens' scales
   int cx[128];                            //   and KCX * the sum of their quants
-  // Q4_K's minimums: the rows' eight minimums and their sum; the tokens' eight sums of 32 as planes
-  // (U = sum + 4096: U >> 8, and (U & 255) - 128)
-  int2 wmn[128]; int wms[128];
-  int2 bh[128], bl[128];
+  union {
+    // Q4_K's minimums: the rows' eight minimums and their sum; the tokens' eight sums of 32 as planes
+    // (U = sum + 4096: U >> 8, and (U & 255) - 128)
+    struct { int2 wmn[128]; int wms[128]; int2 bh[128], bl[128]; };
+    // IQ2_XXS: the codebook, and for each 7-bit sign index (+ parity) 0xFF in the bytes of the negative weights
+    struct { u64 grid[256]; u64 smask[128]; };
+  };
   u32 scan[256];
   int tile_z, tile_t0, tile_n;
+};
+
+// IQ2_XXS: a block's eight groups of 32 weights add (float(sumi) * (0.5 + scale)) alternately to two sums,
+// fa (even groups) and fb (odd), then sum += (d*yd) * (fa + fb) (iquant.lisp:161-215).  Every term is a
+// multiple of 1/2 below 2^23 and so are the first three partial sums of a sum of four, so fa is the
+// float nearest to an integer / 2, one rounding at most, the same as float(S) * 0.5 for the integer
+// S = sum over the even groups of (2*scale + 1) * sumi.  So the weights go in as (2*scale + 1) * (signed
+// magnitude), at most 1333 in absolute value, + 1408 as two planes, and a step's first 32 columns (an even
+// group) and second 32 (an odd one) have integer sums of their own.
+template <> struct I8p<ILT_IQ2_XXS> {
+  static constexpr int KCX = 1280;
+  static constexpr int PLANES = 2, WL = 3;
+  struct Raw { int2 g[2]; u32 d; };                          // the thread's group of each of the half's two steps (8 bytes: four codebook indices, signs and scale), d
+  static __device__ __forceinline__ void load(Raw& r, __amdgpu_buffer_rsrc_t rw, u32 rowoff, int hb, int q4) {
+    const u32 b = rowoff + (u32)(hb >> 1) * 66 + 2 + 8 * (4 * (hb & 1) + (q4 >> 1));
+    r.g[0] = ilt_bld8(rw, b);
+    r.g[1] = ilt_bld8(rw, b + 16);
+    r.d = ilt_bld2(rw, rowoff + (u32)(hb >> 1) * 66);
+  }
+  static __device__ __forceinline__ float d_of(const Raw& r) { return ilt_h2f((u16)r.d); }
+  static __device__ __forceinline__ void planes(const Raw& r, int J, int q4, int* hi, int* lo, const I8pSmem& S) {
+    const u32 idx = (u32)r.g[J & 1].x, aux = (u32)r.g[J & 1].y;
+    const int mult = 2 * (int)(aux >> 28) + 1;
+    const u32 c0 = 1408u * 0x10001u;
+#pragma unroll
+    for (int l2 = 0; l2 < 2; l2++) {
+      const int l = 2 * (q4 & 1) + l2;                       // the group's l-th run of 8 weights
+      const int2 mag = ilt_lds_ld8(&S.grid[(idx >> (8 * l)) & 0xFF]);
+      const int2 neg = ilt_lds_ld8(&S.smask[(aux >> (7 * l)) & 127]);
+#pragma unroll
+      for (int h = 0; h < 2; h++) {
+        const u32 m = (u32)(h ? mag.y : mag.x), nb = (u32)(h ? neg.y : neg.x);
+        const u32 pe = (u32)__mul24((int)(m & 0x00FF00FF), mult), po = (u32)__mul24((int)((m >> 8) & 0x00FF00FF), mult);
+        const u32 me = __builtin_amdgcn_perm(nb, nb, 0x02020000u), mo = __builtin_amdgcn_perm(nb, nb, 0x03030101u);   // the fields of the negative weights
+        const u32 te = (pe ^ me) + (c0 - me), to = (po ^ mo) + (c0 - mo);       // 1408 +- the product, in both fields
+        hi[2 * l2 + h] = (int)__builtin_amdgcn_perm(to, te, 0x07030501u);
+        lo[2 * l2 + h] = (int)(__builtin_amdgcn_perm(to, te, 0x06020400u) ^ 0x80808080u);
+      }
+    }
+  }
 };
 
 __device__ __forceinline__ void ilt_lds_st4_untracked(void* p, u32 v) {
@@ -949,8 +992,9 @@ __global__ __launch_bounds__(512, 1) void gemm_i8p_kernel(BfParams p) {
   typedef I8p<FMT> F;
   typedef typename F::Raw Raw;
   constexpr int TM = 128, TN = 128, NA = 2, NI = 1;
-  constexpr int WL = F::WL, XL = 5;                          // loads of a raw set, of a token's constants
+  constexpr int WL = F::WL, XL = FMT == ILT_IQ2_XXS ? 1 : 5;  // loads of a raw set, of a token's constants (IQ2_XXS comes without the sums of 16: d4_mm_id_iq2_xxs has no such argument)
   constexpr bool TWO = F::PLANES == 2;
+  constexpr bool SPLIT = FMT == ILT_IQ2_XXS;                 // the first and the second 32 columns of a step have sums of their own
   constexpr int KW = 64;                                     // columns a step
   __shared__ I8pSmem S;
   // Q2_K has no hi plane: its room holds the minimums' operands (sixteen groups: 16 bytes a row or token)
@@ -962,6 +1006,18 @@ __global__ __launch_bounds__(512, 1) void gemm_i8p_kernel(BfParams p) {
   long tok0; int ntok, rt; const u8* w = p.w;
   if (!pick_tile<TM, TN>(p, S, tok0, ntok, rt, w)) return;
   const int r0 = rt * TM;
+  int* const cxo = (int*)S.wdm;                              // IQ2_XXS: cx for the even groups, this for the odd ones
+  if constexpr (FMT == ILT_IQ2_XXS) {
+    if (t < 256) S.grid[t] = bf_grid_dev[t];
+    if (t < 128) {
+      const u32 sb = (u32)t | ((__popc(t) & 1) << 7);
+      u32 m[2] = {0, 0};
+#pragma unroll
+      for (int j = 0; j < 8; j++) m[j >> 2] |= ((sb >> j) & 1) ? 0xFFu << (8 * (j & 3)) : 0u;
+      S.smask[t] = (u64)m[0] | ((u64)m[1] << 32);
+    }
+    __syncthreads();
+  }
 
   const int wrow = t >> 2, q4 = t & 3;
   const __amdgpu_buffer_rsrc_t rw = ilt_rsrc(ilt_uniform_ptr(w), (u32)min((long long)p.rows * p.row_bytes, 0xFFFFFFF0LL));
@@ -973,20 +1029,24 @@ __global__ __launch_bounds__(512, 1) void gemm_i8p_kernel(BfParams p) {
   // a token's constants for a super-block, by thread t & 127 (every wave loads, so that all count the same loads)
   const long ctok = tok0 + min(t & 127, ntok - 1);
   const float* xdp = p.xd + ctok * nsb;
-  const int4* bsp = (const int4*)(p.bsums + ctok * (p.cols / 16));
+  const int4* bsp = (const int4*)(p.bsums + ctok * (p.cols / 16));      // (IQ2_XXS: not read)
   float c_yd; int4 c_bs[4];
   auto load_consts = [&](int sb) {
     c_yd = xdp[sb];
+    if constexpr (!SPLIT) {
 #pragma unroll
-    for (int i = 0; i < 4; i++) c_bs[i] = bsp[4 * sb + i];
+      for (int i = 0; i < 4; i++) c_bs[i] = bsp[4 * sb + i];
+    }
   };
   auto store_consts = [&](const Raw& ra) {                   // after a barrier that ends the last block's reads
     if (t < 128) {
       int sx = 0;
+      if constexpr (!SPLIT) {
 #pragma unroll
-      for (int i = 0; i < 4; i++) sx += c_bs[i].x + c_bs[i].y + c_bs[i].z + c_bs[i].w;
+        for (int i = 0; i < 4; i++) sx += c_bs[i].x + c_bs[i].y + c_bs[i].z + c_bs[i].w;
+      }
       ilt_lds_st4_untracked(&S.xd[t], __builtin_bit_cast(u32, c_yd));
-      ilt_lds_st4_untracked(&S.cx[t], (u32)(F::KCX * sx));
+      if constexpr (!SPLIT) ilt_lds_st4_untracked(&S.cx[t], (u32)(F::KCX * sx));
       if constexpr (FMT == ILT_Q4_K) {
         u32 h[2] = {0, 0}, l[2] = {0, 0};
 #pragma unroll
@@ -1039,13 +1099,14 @@ __global__ __launch_bounds__(512, 1) void gemm_i8p_kernel(BfParams p) {
   // the thread's 16 weights of step J of a super-block, out of the set that holds its half, into a pair of slabs
   auto dequant_to = [&](const Raw& r, int J, int slab) {
     int hi[4], lo[4];
-    F::planes(r, J, q4, hi, lo);
+    F::planes(r, J, q4, hi, lo, S);
     if constexpr (TWO) ilt_lds_st16_untracked(S.wh[slab] + wdst, hi[0], hi[1], hi[2], hi[3]);
     ilt_lds_st16_untracked(S.wl[slab] + wdst, lo[0], lo[1], lo[2], lo[3]);
   };
 
   v16f sum[NA][1];
-  v16i_ ah[NA], al[NA];
+  v16i_ ah[SPLIT ? 2 : 1][NA], al[SPLIT ? 2 : 1][NA];
+  int xsum = 0;                                              // IQ2_XXS: see the step
 #pragma unroll
   for (int a = 0; a < NA; a++)
 #pragma unroll
@@ -1089,6 +1150,17 @@ __global__ __launch_bounds__(512, 1) void gemm_i8p_kernel(BfParams p) {
     const u8* whs = S.wh[J & 1];
     const u8* wls = S.wl[J & 1];
     const v16i_ zero = {};
+    if constexpr (SPLIT) {
+      // the sums of the tokens' quants over the block's even and odd groups, from the slabs: thread t adds piece t & 3
+      // of token t / 4; pieces 0 and 1 are the step's even group, 2 and 3 its odd one
+      const int4 xv = ilt_lds_ld16(xs + slab_off(t >> 2, t & 3));
+      int sp = __builtin_amdgcn_sdot4(xv.x, 0x01010101, 0, false);
+      sp = __builtin_amdgcn_sdot4(xv.y, 0x01010101, sp, false);
+      sp = __builtin_amdgcn_sdot4(xv.z, 0x01010101, sp, false);
+      sp = __builtin_amdgcn_sdot4(xv.w, 0x01010101, sp, false);
+      sp += __shfl_xor(sp, 1);
+      xsum = J == 0 ? sp : xsum + sp;
+    }
 #pragma unroll
     for (int kk = 0; kk < 2; kk++) {
       v4i_ af[NA];
@@ -1105,8 +1177,11 @@ __global__ __launch_bounds__(512, 1) void gemm_i8p_kernel(BfParams p) {
       }
 #pragma unroll
       for (int a = 0; a < NA; a++) {                         // a super-block's first products start its integer sums
-        if constexpr (TWO) ah[a] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[a], bh, (J == 0 && kk == 0) ? zero : ah[a], 0, 0, 0);
-        al[a] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[a], bl, (J == 0 && kk == 0) ? zero : al[a], 0, 0, 0);
+        constexpr int ps = 0;
+        const int pk = SPLIT ? kk : ps;
+        const bool first = J == 0 && (SPLIT || kk == 0);
+        if constexpr (TWO) ah[pk][a] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[a], bh, first ? zero : ah[pk][a], 0, 0, 0);
+        al[pk][a] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[a], bl, first ? zero : al[pk][a], 0, 0, 0);
       }
     }
     if (J == 3) {          // the super-block is complete: its terms, as the CPU path adds them
@@ -1129,9 +1204,23 @@ __global__ __launch_bounds__(512, 1) void gemm_i8p_kernel(BfParams p) {
             const int tk = wt0 + 32 * a + 8 * (r >> 2) + 4 * lh + (r & 3);
             const float yd = S.xd[tk];
             const int im = 256 * mh[r] + ml[r] - ms;
-            const int isum = 256 * ah[a][r] + al[a][r] - S.cx[tk];
+            const int isum = 256 * ah[0][a][r] + al[0][a][r] - S.cx[tk];
             sum[a][0][r] = sum[a][0][r] - (yd * dm) * (float)im;
             sum[a][0][r] = sum[a][0][r] + (yd * d) * (float)isum;
+          }
+        }
+      } else if constexpr (FMT == ILT_IQ2_XXS) {
+        if ((t & 3) == 0) ilt_lds_st4_untracked(&S.cx[t >> 2], (u32)(F::KCX * xsum));
+        if ((t & 3) == 2) ilt_lds_st4_untracked(&cxo[t >> 2], (u32)(F::KCX * xsum));
+        ilt_barrier_lds();
+#pragma unroll
+        for (int a = 0; a < NA; a++) {
+#pragma unroll
+          for (int r = 0; r < 16; r++) {
+            const int tk = wt0 + 32 * a + 8 * (r >> 2) + 4 * lh + (r & 3);
+            const float fa = (float)(256 * ah[0][a][r] + al[0][a][r] - S.cx[tk]) * 0.5f;
+            const float fb = (float)(256 * ah[1][a][r] + al[1][a][r] - cxo[tk]) * 0.5f;
+            sum[a][0][r] = sum[a][0][r] + (d * S.xd[tk]) * (fa + fb);
           }
         }
       } else if constexpr (FMT == ILT_Q2_K) {
@@ -1153,7 +1242,7 @@ __global__ __launch_bounds__(512, 1) void gemm_i8p_kernel(BfParams p) {
             const float yd = S.xd[tk];
             const int im = 256 * mh[r] + ml[r] - ms;
             sum[a][0][r] = sum[a][0][r] + ((-yd) * dm) * (float)im;
-            sum[a][0][r] = sum[a][0][r] + (yd * d) * (float)al[a][r];
+            sum[a][0][r] = sum[a][0][r] + (yd * d) * (float)al[0][a][r];
           }
         }
       } else {
@@ -1162,7 +1251,7 @@ __global__ __launch_bounds__(512, 1) void gemm_i8p_kernel(BfParams p) {
 #pragma unroll
           for (int r = 0; r < 16; r++) {
             const int tk = wt0 + 32 * a + 8 * (r >> 2) + 4 * lh + (r & 3);
-            const int isum = 256 * ah[a][r] + al[a][r] - S.cx[tk];
+            const int isum = 256 * ah[0][a][r] + al[0][a][r] - S.cx[tk];
             sum[a][0][r] = sum[a][0][r] + (d * S.xd[tk]) * (float)isum;
           }
         }
@@ -1178,6 +1267,12 @@ __global__ __launch_bounds__(512, 1) void gemm_i8p_kernel(BfParams p) {
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // the tail's redundant loads: nothing may land in LDS after the workgroup ends
 
+  if constexpr (FMT == ILT_IQ2_XXS) {
+#pragma unroll
+    for (int a = 0; a < NA; a++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) sum[a][0][r] = 0.25f * sum[a][0][r];
+  }
   store_tile<NA, 1>(sum, p, tok0, ntok, r0, wt0, wr0, l32, lh);
 }
 
@@ -1452,14 +1547,15 @@ hipError_t ilt_k_gemm_bf16_id_glu(int fmt, const uint64_t* ptrs, long long add_g
 }
 
 static hipError_t launch_i8p(int fmt, const BfParams& p, long long token_tiles, hipStream_t st) {
-  if ((fmt != ILT_Q6_K && fmt != ILT_Q4_K && fmt != ILT_Q2_K) || p.cols % 256 != 0 || (long long)p.rows * 1024 >= 0x7FFFFFFFLL)
+  if ((fmt != ILT_Q6_K && fmt != ILT_Q4_K && fmt != ILT_Q2_K && fmt != ILT_IQ2_XXS) || p.cols % 256 != 0 || (long long)p.rows * 1024 >= 0x7FFFFFFFLL)
     return hipErrorInvalidValue;
   const long long total = token_tiles * ((p.rows + 127) / 128), per = (total + 7) / 8;
   if (per * 8 > 0x7FFFFFFFLL) return hipErrorInvalidValue;
   const dim3 grid((unsigned)(per * 8));
   if (fmt == ILT_Q6_K) hipLaunchKernelGGL(gemm_i8p_kernel<ILT_Q6_K>, grid, dim3(512), 0, st, p);
   else if (fmt == ILT_Q4_K) hipLaunchKernelGGL(gemm_i8p_kernel<ILT_Q4_K>, grid, dim3(512), 0, st, p);
-  else hipLaunchKernelGGL(gemm_i8p_kernel<ILT_Q2_K>, grid, dim3(512), 0, st, p);
+  else if (fmt == ILT_Q2_K) hipLaunchKernelGGL(gemm_i8p_kernel<ILT_Q2_K>, grid, dim3(512), 0, st, p);
+  else hipLaunchKernelGGL(gemm_i8p_kernel<ILT_IQ2_XXS>, grid, dim3(512), 0, st, p);
   return hipGetLastError();
 }
 
