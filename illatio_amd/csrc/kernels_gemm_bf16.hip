@@ -938,9 +938,10 @@ struct I8pSmem {
 
 // IQ2_XXS: a block's eight groups of 32 weights add (float(sumi) * (0.5 + scale)) alternately to two sums,
 // fa (even groups) and fb (odd), then sum += (d*yd) * (fa + fb) (iquant.lisp:161-215).  Every term is a
-// multiple of 1/2 below 2^23 and so are the first three partial sums of a sum of four, so fa is the
-// float nearest to an integer / 2, one rounding at most, the same as float(S) * 0.5 for the integer
-// S = sum over the even groups of (2*scale + 1) * sumi.  So the weights go in as (2*scale + 1) * (signed
+// multiple of 1/2, and with the codebook's entries (byte sums of at most 203) twice a sum of four of them
+// stays below 2^24 (at most 4 * 31 * 4 * 128 * 203 = 12,888,064): none of those float additions rounds, and
+// fa = float(S) * 0.5 for the integer S = sum over the even groups of (2*scale + 1) * sumi.  (Were the
+// last addition to round, it would round the exact sum once, as the conversion of S does.)  So the weights go in as (2*scale + 1) * (signed
 // magnitude), at most 1333 in absolute value, + 1408 as two planes, and a step's first 32 columns (an even
 // group) and second 32 (an odd one) have integer sums of their own.
 template <> struct I8p<ILT_IQ2_XXS> {

@@ -436,3 +436,17 @@ def test_rmsnorm_closed_form_and_misreadings():
             if not np.array_equal(v[k].astype(f32).view(np.uint32), got.view(np.uint32)):
                 told.add(k)
     assert told == {"exact squares", "float sum", "weight folded"}, told
+
+
+def test_iq2xxs_even_and_odd_group_sums_are_exact_in_float():
+    """The CPU path adds a block's four even (and four odd) group terms float(sumi) * (0.5 + scale)
+    in single precision (iquant.lisp:161-215).  With the real codebook every such partial sum
+    is a multiple of 1/2 below 2^23, so none of these additions rounds: the exact prefill kernel
+    may form the integer sum of (2*scale + 1) * sumi and convert once.  The bound: four groups,
+    2*15 + 1, four codebook entries a group, |quant| <= 128, the largest entry's byte sum."""
+    import json, os
+    tables = json.load(open(os.path.join(os.path.dirname(__file__), "golden", "iq2xxs_tables.json")))
+    grid = [int(v, 16) if isinstance(v, str) else int(v) for v in tables["iq2xxs_grid"]]
+    assert len(grid) == 256 and {(g >> (8 * i)) & 0xFF for g in grid for i in range(8)} == {0x08, 0x19, 0x2B}
+    largest = max(sum((g >> (8 * i)) & 0xFF for i in range(8)) for g in grid)
+    assert 4 * 31 * 4 * 128 * largest < 2 ** 24          # twice the largest |partial sum|, as an integer
