@@ -518,7 +518,7 @@ def workload_c5(args, dev):
     allmm = [sum(per[k][0] for k in mm), sum(per[k][1] for k in mm), sum(per[k][2] for k in mm)]
     roof = roofline_of({"mm_id": allmm}, "mfma", MFMA_PEAK_TFLOPS[args.path], "TFLOP/s",
                        {"mm_id": "gemm_bf16_regb_kernel<16, true> (d4_mm_id_glu_bf16: gate, up, activation) + <10, false> (d4_mm_id_bf16: down)" if args.path == "bf16"
-                        else "gemm_i8_kernel grouped (d4_mm_id_iq2_xxs x2, d4_mm_id_q2_k), bit-exact"})
+                        else "gemm_i8p_kernel<16> (d4_mm_id_iq2_xxs x2) + <10> (d4_mm_id_q2_k): scale * quant as int8 planes, grouped, bit-exact with the CPU path"})
     roof["launch_us_all"] = {k: round(v[0] / v[2] * 1e3, 2) for k, v in per.items()}
     if args.path == "bf16" and n == 4096:
         roof["traffic"] = TRAFFIC["c5"]["mm_id"]
