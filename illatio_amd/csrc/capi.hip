@@ -163,6 +163,7 @@ int ilt_d4_quant(uint64_t stream, const float* x, int8_t* xq, float* xs, int nbl
 
 int ilt_quant_q8k(uint64_t stream, const float* x, int8_t* xq, float* xd, int32_t* bsums, int64_t nblocks) {
   ILT_REQUIRE(nblocks >= 0 && (nblocks == 0 || (x && xq && xd && bsums)));
+  ILT_REQUIRE(((uintptr_t)x & 15) == 0 && ((uintptr_t)xq & 3) == 0);      // 16-byte loads, 4-byte stores
   return (int)ilt_k_quant_q8k(x, xq, xd, bsums, nblocks, S(stream));
 }
 

@@ -34,42 +34,48 @@ __global__ __launch_bounds__(256) void quant_q8_kernel(const float* __restrict__
   }
 }
 
-// Q8_K activations (quantize-q8k!): a block of 256 per workgroup.  The
-// largest-magnitude value, the first of equals, sets iscale = -127/max;
-// q = min(127, round-half-even(iscale*x)); d = 1/iscale; sums of each 16 quants.
+// Q8_K activations (quantize-q8k!): a block of 256 per wave, four consecutive values a lane
+// (a 16-byte load, a 4-byte store; no LDS, no barrier).  The largest-magnitude value, the
+// first of equals, sets iscale = -127/max; q = min(127, round-half-even(iscale*x));
+// d = 1/iscale; sums of each 16 quants.
 __global__ __launch_bounds__(256) void quant_q8k_kernel(const float* __restrict__ x, i8* __restrict__ xq,
-                                                        float* __restrict__ xd, int* __restrict__ bsums) {
-  __shared__ u64 wkey[4];
-  __shared__ float smx;
-  const long long b = blockIdx.x;
-  const int t = threadIdx.x;
-  const float v = x[b * 256 + t];
+                                                        float* __restrict__ xd, int* __restrict__ bsums, long long nblocks) {
+  const int lane = threadIdx.x & 63;
+  const long long b = (long long)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (b >= nblocks) return;
+  const float4 v4 = ((const float4*)(x + b * 256))[lane];
+  const float v[4] = {v4.x, v4.y, v4.z, v4.w};
   // |v|'s bits order as |v| does; the low word prefers the earlier index
-  u64 key = ((u64)__float_as_uint(fabsf(v)) << 32) | (u32)(255 - t);
+  u64 key = 0;
+#pragma unroll
+  for (int k = 0; k < 4; k++) {
+    const u64 kk = ((u64)__float_as_uint(fabsf(v[k])) << 32) | (u32)(255 - (4 * lane + k));
+    key = kk > key ? kk : key;
+  }
 #pragma unroll
   for (int off = 32; off > 0; off >>= 1) {
     const u32 hi = __shfl_xor((u32)(key >> 32), off), lo = __shfl_xor((u32)key, off);
     const u64 o = ((u64)hi << 32) | lo;
     key = o > key ? o : key;
   }
-  if ((t & 63) == 0) wkey[t >> 6] = key;
-  __syncthreads();
-  u64 best = wkey[0];
-#pragma unroll
-  for (int w = 1; w < 4; w++) best = wkey[w] > best ? wkey[w] : best;
-  if (t == 255 - (int)(best & 0xFFFFFFFFu)) smx = v;
-  __syncthreads();
-  const float mx = smx;
-  int q = 0;
+  const int idx = 255 - (int)(key & 0xFFFFFFFFu);             // the same in every lane
+  const int ik = idx & 3;
+  const float mine = ik == 0 ? v[0] : ik == 1 ? v[1] : ik == 2 ? v[2] : v[3];
+  const float mx = __shfl(mine, idx >> 2);
+  int q[4] = {0, 0, 0, 0};
   float iscale = 0.0f;
-  if ((best >> 32) != 0) {
+  const bool any = (key >> 32) != 0;
+  if (any) {
     iscale = -127.0f / mx;
-    q = min(127, (int)rintf(iscale * v));
+#pragma unroll
+    for (int k = 0; k < 4; k++) q[k] = min(127, (int)rintf(iscale * v[k]));
   }
-  xq[b * 256 + t] = (i8)q;
-  const int s = ilt_sum16(q);
-  if ((t & 15) == 0) bsums[b * 16 + (t >> 4)] = s;
-  if (t == 0) xd[b] = (best >> 32) != 0 ? 1.0f / iscale : 0.0f;
+  ((u32*)(xq + b * 256))[lane] = (u32)(q[0] & 0xFF) | ((u32)(q[1] & 0xFF) << 8) | ((u32)(q[2] & 0xFF) << 16) | ((u32)(q[3] & 0xFF) << 24);
+  int s = (q[0] + q[1]) + (q[2] + q[3]);
+  s += __shfl_xor(s, 1);
+  s += __shfl_xor(s, 2);
+  if ((lane & 3) == 0) bsums[b * 16 + (lane >> 2)] = s;
+  if (lane == 0) xd[b] = any ? 1.0f / iscale : 0.0f;
 }
 
 // GGUF Q8_0 blocks (f16 d, 32 int8) split into an int8 array and an f16 scale array.
@@ -170,7 +176,7 @@ hipError_t ilt_k_quant_q8(const float* x, int8_t* xq, float* xs, int* xsum, long
 
 hipError_t ilt_k_quant_q8k(const float* x, int8_t* xq, float* xd, int* bsums, long long nblocks, hipStream_t st) {
   if (nblocks <= 0) return hipSuccess;
-  hipLaunchKernelGGL(quant_q8k_kernel, dim3((unsigned)nblocks), dim3(256), 0, st, x, xq, xd, bsums);
+  hipLaunchKernelGGL(quant_q8k_kernel, dim3((unsigned)((nblocks + 3) / 4)), dim3(256), 0, st, x, xq, xd, bsums, nblocks);
   return hipGetLastError();
 }
 
