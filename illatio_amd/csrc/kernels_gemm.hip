@@ -445,11 +445,11 @@ hipError_t ilt_k_gemm_i8_id(int fmt, const uint64_t* ptrs, long long add, const 
   if (total_rows <= 0 || rows <= 0 || ne <= 0) return hipSuccess;
   if (ne > 256) return hipErrorInvalidValue;
   {
-    // the experts' IQ2_XXS and Q2_K (and Q4_K / Q6_K) matrices on the planes kernel when the groups average at least half a tile of 128 rows
+    // the experts' IQ2_XXS and Q2_K (and Q4_K / Q6_K) matrices on the planes kernel when the groups average at least a quarter of a tile of 128 rows
     const char* force = getenv("ILT_I8_PLANES");
     const int forced = force ? atoi(force) : -1;
     if ((fmt == ILT_Q6_K || fmt == ILT_Q4_K || fmt == ILT_Q2_K || fmt == ILT_IQ2_XXS) && cols % 256 == 0 && forced != 0 &&
-        (forced == 1 || (total_rows >= 64LL * ne && rows >= 128)))
+        (forced == 1 || (total_rows >= 32LL * ne && rows >= 128)))
       return ilt_k_gemm_i8_planes_id(fmt, ptrs, add, counts, bases, ne, row_bytes, rows, cols, xq, xs, bsums, total_rows, y, st);
   }
   GemmParams p = {};

@@ -1113,7 +1113,10 @@ __global__ __launch_bounds__(512, 1) void gemm_i8p_kernel(BfParams p) {
 #pragma unroll
     for (int r = 0; r < 16; r++) sum[a][0][r] = 0.0f;
 
-  const int wt0 = 64 * (wave & 1), wr0 = 32 * (wave >> 1);  // this wave's tokens and rows in the tile
+  // this wave's tokens and rows in the tile: waves 0-3 the first 64 tokens, 4-7 the second, one of each on every SIMD.
+  // A wave whose tokens the group does not have (a group of up to 64 rows) only makes planes.
+  const int wt0 = 64 * (wave >> 2), wr0 = 32 * (wave & 3);
+  const bool work = __builtin_amdgcn_readfirstlane(wt0) < ntok;
   const int l32 = lane & 31, lh = lane >> 5;
   u32 aoff[NA];                                              // fragment offsets of the step's first 32 columns (piece lh); the second 32 at ^ 32
 #pragma unroll
@@ -1164,28 +1167,38 @@ __global__ __launch_bounds__(512, 1) void gemm_i8p_kernel(BfParams p) {
     }
 #pragma unroll
     for (int kk = 0; kk < 2; kk++) {
-      v4i_ af[NA];
+      v4i_ af[NA] = {}, bh = {}, bl = {};
+      if (work) {
 #pragma unroll
-      for (int a = 0; a < NA; a++) af[a] = *(const v4i_*)(xs + (aoff[a] ^ (32 * kk)));
-      v4i_ bh = {};
-      if constexpr (TWO) bh = *(const v4i_*)(whs + (boff ^ (32 * kk)));
-      const v4i_ bl = *(const v4i_*)(wls + (boff ^ (32 * kk)));
+        for (int a = 0; a < NA; a++) af[a] = *(const v4i_*)(xs + (aoff[a] ^ (32 * kk)));
+        if constexpr (TWO) bh = *(const v4i_*)(whs + (boff ^ (32 * kk)));
+        bl = *(const v4i_*)(wls + (boff ^ (32 * kk)));
+      }
       if (kk == 0) {       // step ks+1's planes: J+1 = 1 from A, 2 and 3 from B, 4 = the next block's 0 from A (past the last step: planes nobody reads)
         if (J == 0) dequant_to(rawa, 1, 1);
         if (J == 1) dequant_to(rawb, 2, 0);
         if (J == 2) dequant_to(rawb, 3, 1);
         if (J == 3) dequant_to(rawa, 0, 0);
       }
+      if (work) {
 #pragma unroll
-      for (int a = 0; a < NA; a++) {                         // a super-block's first products start its integer sums
-        constexpr int ps = 0;
-        const int pk = SPLIT ? kk : ps;
-        const bool first = J == 0 && (SPLIT || kk == 0);
-        if constexpr (TWO) ah[pk][a] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[a], bh, first ? zero : ah[pk][a], 0, 0, 0);
-        al[pk][a] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[a], bl, first ? zero : al[pk][a], 0, 0, 0);
+        for (int a = 0; a < NA; a++) {                       // a super-block's first products start its integer sums
+          constexpr int ps = 0;
+          const int pk = SPLIT ? kk : ps;
+          const bool first = J == 0 && (SPLIT || kk == 0);
+          if constexpr (TWO) ah[pk][a] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[a], bh, first ? zero : ah[pk][a], 0, 0, 0);
+          al[pk][a] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[a], bl, first ? zero : al[pk][a], 0, 0, 0);
+        }
       }
     }
-    if (J == 3) {          // the super-block is complete: its terms, as the CPU path adds them
+    if constexpr (FMT == ILT_IQ2_XXS) {
+      if (J == 3) {        // the block's sums of quants, for everyone's terms below
+        if ((t & 3) == 0) ilt_lds_st4_untracked(&S.cx[t >> 2], (u32)(F::KCX * xsum));
+        if ((t & 3) == 2) ilt_lds_st4_untracked(&cxo[t >> 2], (u32)(F::KCX * xsum));
+        ilt_barrier_lds();
+      }
+    }
+    if (J == 3 && work) {  // the super-block is complete: its terms, as the CPU path adds them
       const int row = wr0 + l32;
       const float d = S.wd[row];
       if constexpr (FMT == ILT_Q4_K) {
@@ -1211,9 +1224,6 @@ __global__ __launch_bounds__(512, 1) void gemm_i8p_kernel(BfParams p) {
           }
         }
       } else if constexpr (FMT == ILT_IQ2_XXS) {
-        if ((t & 3) == 0) ilt_lds_st4_untracked(&S.cx[t >> 2], (u32)(F::KCX * xsum));
-        if ((t & 3) == 2) ilt_lds_st4_untracked(&cxo[t >> 2], (u32)(F::KCX * xsum));
-        ilt_barrier_lds();
 #pragma unroll
         for (int a = 0; a < NA; a++) {
 #pragma unroll
