@@ -988,7 +988,7 @@ __device__ __forceinline__ void ilt_lds_st8_untracked(void* p, u32 a, u32 b) {
 // 128 rows x 128 tokens a workgroup of eight waves (one workgroup a CU, two waves a SIMD: a
 // wave's two planes of integer sums, its float sums and the raw bytes leave no room for more);
 // wave w: rows 32*(w/2).., tokens 64*(w%2)...
-template <int FMT>
+template <int FMT, bool GROUPED>
 __global__ __launch_bounds__(512, 1) void gemm_i8p_kernel(BfParams p) {
   typedef I8p<FMT> F;
   typedef typename F::Raw Raw;
@@ -1113,10 +1113,10 @@ __global__ __launch_bounds__(512, 1) void gemm_i8p_kernel(BfParams p) {
 #pragma unroll
     for (int r = 0; r < 16; r++) sum[a][0][r] = 0.0f;
 
-  // this wave's tokens and rows in the tile: waves 0-3 the first 64 tokens, 4-7 the second, one of each on every SIMD.
-  // A wave whose tokens the group does not have (a group of up to 64 rows) only makes planes.
-  const int wt0 = 64 * (wave >> 2), wr0 = 32 * (wave & 3);
-  const bool work = __builtin_amdgcn_readfirstlane(wt0) < ntok;
+  // this wave's tokens and rows in the tile.  Grouped: waves 0-3 the first 64 tokens, 4-7 the second, one of each on
+  // every SIMD, and a wave whose tokens the group does not have (a group of up to 64 rows) only makes planes.
+  const int wt0 = GROUPED ? 64 * (wave >> 2) : 64 * (wave & 1), wr0 = GROUPED ? 32 * (wave & 3) : 32 * (wave >> 1);
+  const bool work = !GROUPED || __builtin_amdgcn_readfirstlane(wt0) < ntok;
   const int l32 = lane & 31, lh = lane >> 5;
   u32 aoff[NA];                                              // fragment offsets of the step's first 32 columns (piece lh); the second 32 at ^ 32
 #pragma unroll
@@ -1557,16 +1557,17 @@ hipError_t ilt_k_gemm_bf16_id_glu(int fmt, const uint64_t* ptrs, long long add_g
   return launch_regb<ILT_IQ2_XXS, true>(p, total_rows / 128 + ne, st);
 }
 
+template <bool GROUPED>
 static hipError_t launch_i8p(int fmt, const BfParams& p, long long token_tiles, hipStream_t st) {
   if ((fmt != ILT_Q6_K && fmt != ILT_Q4_K && fmt != ILT_Q2_K && fmt != ILT_IQ2_XXS) || p.cols % 256 != 0 || (long long)p.rows * 1024 >= 0x7FFFFFFFLL)
     return hipErrorInvalidValue;
   const long long total = token_tiles * ((p.rows + 127) / 128), per = (total + 7) / 8;
   if (per * 8 > 0x7FFFFFFFLL) return hipErrorInvalidValue;
   const dim3 grid((unsigned)(per * 8));
-  if (fmt == ILT_Q6_K) hipLaunchKernelGGL(gemm_i8p_kernel<ILT_Q6_K>, grid, dim3(512), 0, st, p);
-  else if (fmt == ILT_Q4_K) hipLaunchKernelGGL(gemm_i8p_kernel<ILT_Q4_K>, grid, dim3(512), 0, st, p);
-  else if (fmt == ILT_Q2_K) hipLaunchKernelGGL(gemm_i8p_kernel<ILT_Q2_K>, grid, dim3(512), 0, st, p);
-  else hipLaunchKernelGGL(gemm_i8p_kernel<ILT_IQ2_XXS>, grid, dim3(512), 0, st, p);
+  if (fmt == ILT_Q6_K) hipLaunchKernelGGL((gemm_i8p_kernel<ILT_Q6_K, GROUPED>), grid, dim3(512), 0, st, p);
+  else if (fmt == ILT_Q4_K) hipLaunchKernelGGL((gemm_i8p_kernel<ILT_Q4_K, GROUPED>), grid, dim3(512), 0, st, p);
+  else if (fmt == ILT_Q2_K) hipLaunchKernelGGL((gemm_i8p_kernel<ILT_Q2_K, GROUPED>), grid, dim3(512), 0, st, p);
+  else hipLaunchKernelGGL((gemm_i8p_kernel<ILT_IQ2_XXS, GROUPED>), grid, dim3(512), 0, st, p);
   return hipGetLastError();
 }
 
@@ -1576,7 +1577,7 @@ hipError_t ilt_k_gemm_i8_planes(int fmt, const uint8_t* w, long long row_bytes, 
   BfParams p = {};
   p.w = w; p.rows = rows; p.cols = cols; p.row_bytes = row_bytes; p.x = (const u16*)xq; p.xd = xd; p.bsums = bsums;
   p.y = y; p.bias = bias; p.acc = acc; p.ntok = ntok; p.ldy = rows;
-  return launch_i8p(fmt, p, (ntok + 127) / 128, st);
+  return launch_i8p<false>(fmt, p, (ntok + 127) / 128, st);
 }
 
 hipError_t ilt_k_gemm_i8_planes_id(int fmt, const uint64_t* ptrs, long long add, const uint32_t* counts, const uint32_t* bases, int ne,
@@ -1588,7 +1589,7 @@ hipError_t ilt_k_gemm_i8_planes_id(int fmt, const uint64_t* ptrs, long long add,
   p.ptrs = ptrs; p.add = add; p.counts = counts; p.bases = bases; p.ne = ne;
   p.rows = rows; p.cols = cols; p.row_bytes = row_bytes; p.x = (const u16*)xq; p.xd = xd; p.bsums = bsums;
   p.y = y; p.ntok = (int)total_rows; p.ldy = rows;
-  return launch_i8p(fmt, p, total_rows / 128 + ne, st);
+  return launch_i8p<true>(fmt, p, total_rows / 128 + ne, st);
 }
 
 hipError_t ilt_k_cvt_bf16_slabs(const float* x, uint16_t* out, int n, int cols, hipStream_t st) {
