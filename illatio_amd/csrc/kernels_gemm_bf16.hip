@@ -28,6 +28,8 @@
 // expert's rows in turn; for the experts' own formats, IQ2_XXS and Q2_K, it has a kernel of
 // its own that dequantizes into the MFMA operands without a detour of the weights through LDS
 // as bf16 (gemm_bf16_regb_kernel).
+// The same pipeline also carries the exact product (gemm_i8p_kernel, further down): scale * quant
+// as int8 planes on v_mfma_i32_32x32x32_i8, the bits of the CPU path's MATMUL!.
 #include "ilt_device.h"
 #include "ilt_iq2xxs_tables.h"
 #include "ilt_kernels.h"
