@@ -324,7 +324,10 @@ def workload_c3(args, dev):
     from illatio_amd import dense, hip, synth
     rng = synth.make_rng(33)
     rows, cols, T = (17408, 5120, args.tokens) if not args.transpose else (5120, 17408, args.tokens)
-    qt = synth.Q4_K if args.qtype == "q4_k" else synth.Q6_K        # BASELINE's config 3 is Q6_K; --qtype q4_k: the same shape in the other dense format
+    # BASELINE's config 3 is Q6_K; --qtype: the same shape in the other dense formats (q8_0: the exact path only)
+    qt = {"q4_k": synth.Q4_K, "q6_k": synth.Q6_K, "q8_0": synth.Q8_0}[args.qtype]
+    if qt == synth.Q8_0 and args.path != "int8":
+        raise SystemExit("bench.py: --qtype q8_0 goes with --path int8 (the bf16 product multiplies the K-quants)")
     w = np.tile(synth.weights(qt, 256, cols, rng, dscale=0.01), (rows // 256, 1))
     m = dense.upload_gmat(dev, "w", qt, rows, cols, w)
     x = synth.activations((T, cols), rng)
@@ -356,7 +359,7 @@ def workload_c3(args, dev):
             tm.launch("mm", flops, lambda: dense.cmat_mul_bf16(dev, m, xb, y, T))
         names = {"mm": "gemm_bf16_kernel<14, TM, TN, NB> (Q6_K dequantized to bf16 in LDS, v_mfma_f32_32x32x16_bf16)"}
     else:
-        act = dense.QAct(dev, T, cols, ("q8k",))
+        act = dense.QAct(dev, T, cols, ("q8",) if qt == synth.Q8_0 else ("q8k",))
 
         def step(_):
             tm.launch("quant", 0, lambda: dense.quantize_act(dev, xf, act))
@@ -556,7 +559,7 @@ def main():
     ap.add_argument("--layers", type=int, default=LAYERS, help=argparse.SUPPRESS)
     ap.add_argument("--tokens", type=int, default=4096, help="c3, c5: tokens per step")
     ap.add_argument("--transpose", action="store_true", help="c3: the 5120x17408 matrix")
-    ap.add_argument("--qtype", default="q6_k", choices=["q6_k", "q4_k"], help="c3: the matrix's format (BASELINE: q6_k)")
+    ap.add_argument("--qtype", default="q6_k", choices=["q6_k", "q4_k", "q8_0"], help="c3: the matrix's format (BASELINE: q6_k)")
     ap.add_argument("--path", default="bf16", choices=["bf16", "bf16-1pass", "bf16-2pass", "bf16-resident", "int8"],
                     help="c3, c5: which matrix-core path.  c3: bf16 = 2pass from 1024 tokens on, else 1pass; bf16-1pass = the matrix dequantized inside the product's loop; "
                          "bf16-2pass = the matrix dequantized to a bf16 copy inside the step, then the plain bf16 product; bf16-resident = that copy made beforehand and kept")

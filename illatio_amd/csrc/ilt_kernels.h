@@ -95,6 +95,9 @@ hipError_t ilt_k_gemm_i8(int fmt, const uint8_t* w, const uint16_t* wd, long lon
 // Q6_K, Q4_K and Q2_K, exact, on the pipelined kernel (kernels_gemm_bf16.hip): scale * quant as int8 planes
 hipError_t ilt_k_gemm_i8_planes(int fmt, const uint8_t* w, long long row_bytes, int rows, int cols, const int8_t* xq, const float* xd,
                                 const int* bsums, int ntok, float* y, const float* bias, int acc, hipStream_t st);
+// Q8_0, exact, on the pipelined kernel (cols a multiple of 64)
+hipError_t ilt_k_gemm_i8_q8(const uint8_t* wq, const uint16_t* wd, int rows, int cols, const int8_t* xq, const float* xs, int ntok,
+                            float* y, const float* bias, int acc, hipStream_t st);
 hipError_t ilt_k_gemm_i8_planes_id(int fmt, const uint64_t* ptrs, long long add, const uint32_t* counts, const uint32_t* bases, int ne,
                                    long long row_bytes, int rows, int cols, const int8_t* xq, const float* xd, const int* bsums,
                                    long long total_rows, float* y, hipStream_t st);

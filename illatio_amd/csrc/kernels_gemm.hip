@@ -433,6 +433,8 @@ hipError_t ilt_k_gemm_i8(int fmt, const uint8_t* w, const uint16_t* wd, long lon
   const int forced = force ? atoi(force) : -1;
   if ((fmt == ILT_Q6_K || fmt == ILT_Q4_K || fmt == ILT_Q2_K) && cols % 256 == 0 && forced != 0 && (forced == 1 || (ntok >= 96 && rows >= 128)))
     return ilt_k_gemm_i8_planes(fmt, w, row_bytes, rows, cols, xq, xs, bsums, ntok, y, bias, acc, st);
+  if (fmt == ILT_Q8_0 && cols % 64 == 0 && forced != 0 && (forced == 1 || (ntok >= 96 && rows >= 128)))
+    return ilt_k_gemm_i8_q8(w, wd, rows, cols, xq, xs, ntok, y, bias, acc, st);
   GemmParams p = {};
   p.w = w; p.wdq = wd; p.rows = rows; p.cols = cols; p.row_bytes = row_bytes;
   p.xq = xq; p.xs = xs; p.bsums = bsums; p.y = y; p.bias = bias; p.acc = acc; p.ntok = ntok;

@@ -204,6 +204,8 @@ struct BfParams {
   unsigned up_delta; const float* wrow; float clamp; u16* mid;
   // the exact product (gemm_i8p_kernel): x = the tokens' Q8_K quants (a byte a column), with their block scales and sums of 16
   const float* xd; const int* bsums;
+  // Q8_0 (gemm_i8q_kernel): w = the quants (a byte a weight, rows of cols bytes), wdq their f16 scales, xd the tokens' scales (one per 32)
+  const u16* wdq;
 };
 
 template <int TM, int TN, int NXS, int NWS> struct Smem {
@@ -1289,6 +1291,103 @@ __global__ __launch_bounds__(512, 1) void gemm_i8p_kernel(BfParams p) {
   store_tile<NA, 1>(sum, p, tok0, ntok, r0, wt0, wr0, l32, lh);
 }
 
+// ---- the exact Q8_0 product on the same pipeline -------------------------------------------------
+// Q8_0 scales every block of 32 in float on either side: sum += float(isum) * (dw * dx), block
+// after block (tensor.lisp:329-336), so there is nothing to fold into integers; but the quants
+// are int8 as they lie in memory and a v_mfma_i32_32x32x32_i8 is exactly one block deep.  Both
+// operands' slabs (64 columns = two blocks a step) come by direct loads, three steps in
+// flight; the two scales a row and a token have per step go through registers a step ahead.
+struct I8qSmem {
+  __align__(16) u8 xs[3][128 * 64];
+  __align__(16) u8 ws[3][128 * 64];
+  float dw[2][2][128];                    // [step parity][block of the step][row]
+  float dx[2][2][128];                    // [step parity][block of the step][token]
+  u32 scan[256];
+  int tile_z, tile_t0, tile_n;
+};
+
+__global__ __launch_bounds__(512, 2) void gemm_i8q_kernel(BfParams p) {
+  constexpr int TM = 128, TN = 128, NA = 2, KW = 64;
+  __shared__ I8qSmem S;
+  const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+
+  long tok0; int ntok, rt; const u8* w = p.w;
+  if (!pick_tile<TM, TN>(p, S, tok0, ntok, rt, w)) return;
+  const int r0 = rt * TM;
+  const int nk = p.cols / KW, nb = p.cols / 32;
+
+  // piece t of a slab, of the tokens' and of the rows' quants
+  const int prow = t >> 2, pk = (t & 3) ^ (int)slab_swz(prow);
+  const u8* xbase = (const u8*)ilt_uniform_ptr((const i8*)p.x + tok0 * (long)p.cols);
+  const u8* wbase = (const u8*)ilt_uniform_ptr(w + (long)r0 * p.cols);
+  const u32 xoff = (u32)min(prow, ntok - 1) * (u32)p.cols + 16 * pk;
+  const u32 woff = (u32)min(prow, p.rows - 1 - r0) * (u32)p.cols + 16 * pk;
+  // a scale a thread and step: threads 0..255 a row's (row t/2, block t%2 of the step), 256..511 a token's
+  const int sidx = (t & 255) >> 1, sblk = t & 1;
+  const bool srow = t < 256;
+  const u16* dwp = p.wdq + (long)min(r0 + sidx, p.rows - 1) * nb + sblk;
+  const float* dxp = p.xd + (tok0 + min(sidx, ntok - 1)) * nb + sblk;
+  auto load_scale = [&](int ks) { return srow ? ilt_h2f(dwp[2 * ks]) : dxp[2 * ks]; };
+  auto store_scale = [&](float v, int ks) {
+    float* dst = srow ? &S.dw[ks & 1][sblk][sidx] : &S.dx[ks & 1][sblk][sidx];
+    asm volatile("ds_write_b32 %0, %1" :: "v"((u32)(uintptr_t)(ILT_LDS void*)dst), "v"(v) : "memory");
+  };
+  auto issue = [&](int stage, int ks) {
+    ilt_g2lds16(xbase + ks * KW + xoff, S.xs[stage] + wave * 1024);
+    ilt_g2lds16(wbase + ks * KW + woff, S.ws[stage] + wave * 1024);
+  };
+
+  v16f sum[NA][1];
+#pragma unroll
+  for (int a = 0; a < NA; a++)
+#pragma unroll
+    for (int r = 0; r < 16; r++) sum[a][0][r] = 0.0f;
+  const int wt0 = 64 * (wave & 1), wr0 = 32 * (wave >> 1);  // this wave's tokens and rows in the tile
+  const int l32 = lane & 31, lh = lane >> 5;
+  u32 aoff[NA];
+#pragma unroll
+  for (int a = 0; a < NA; a++) aoff[a] = slab_off(wt0 + 32 * a + l32, lh);
+  const u32 boff = slab_off(wr0 + l32, lh);
+
+  // Step ks waits for its slabs (sent two steps ago), stores the scales of step ks+1 (loaded a step
+  // ago), loads those of step ks+2 and sends for step ks+2's slabs.
+  // (in this order: step 0 waits for all but the last three loads)
+  store_scale(load_scale(0), 0);
+  issue(0, 0);
+  float sc_next = load_scale(min(1, nk - 1));
+  issue(1, min(1, nk - 1));
+  int st0 = 0, st1 = 1, st2 = 2;
+  const v16i_ zero = {};
+  for (int ks = 0; ks < nk; ks++) {
+    asm volatile("s_waitcnt vmcnt(3)" ::: "memory");         // all loads but the previous step's three (its scale and two slabs)
+    ilt_barrier_lds();                                       // no fence: later steps' loads stay in flight
+    store_scale(sc_next, ks + 1);
+    sc_next = load_scale(min(ks + 2, nk - 1));
+    issue(st2, min(ks + 2, nk - 1));
+    __builtin_amdgcn_sched_barrier(0);
+    const u8* xs = S.xs[st0];
+    const u8* ws = S.ws[st0];
+#pragma unroll
+    for (int kk = 0; kk < 2; kk++) {                         // block 2*ks + kk
+      const v4i_ bw = *(const v4i_*)(ws + (boff ^ (32 * kk)));
+      const float dw = S.dw[ks & 1][kk][wr0 + l32];
+#pragma unroll
+      for (int a = 0; a < NA; a++) {
+        const v4i_ af = *(const v4i_*)(xs + (aoff[a] ^ (32 * kk)));
+        const v16i_ d = __builtin_amdgcn_mfma_i32_32x32x32_i8(af, bw, zero, 0, 0, 0);
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+          const float dx = S.dx[ks & 1][kk][wt0 + 32 * a + 8 * (r >> 2) + 4 * lh + (r & 3)];
+          sum[a][0][r] = sum[a][0][r] + (float)d[r] * (dw * dx);
+        }
+      }
+    }
+    const int s_ = st0; st0 = st1; st1 = st2; st2 = s_;
+  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // the tail's redundant loads: nothing may land in LDS after the workgroup ends
+  store_tile<NA, 1>(sum, p, tok0, ntok, r0, wt0, wr0, l32, lh);
+}
+
 // ---- the two-pass product: W as plain bf16 ------------------------------------------------------
 // With thousands of tokens the in-loop dequantization above is repeated for every tile of 256
 // tokens and its VALU work competes with the MFMAs for issue slots.  With HBM to spare the
@@ -1580,6 +1679,19 @@ hipError_t ilt_k_gemm_i8_planes(int fmt, const uint8_t* w, long long row_bytes, 
   p.w = w; p.rows = rows; p.cols = cols; p.row_bytes = row_bytes; p.x = (const u16*)xq; p.xd = xd; p.bsums = bsums;
   p.y = y; p.bias = bias; p.acc = acc; p.ntok = ntok; p.ldy = rows;
   return launch_i8p<false>(fmt, p, (ntok + 127) / 128, st);
+}
+
+hipError_t ilt_k_gemm_i8_q8(const uint8_t* wq, const uint16_t* wd, int rows, int cols, const int8_t* xq, const float* xs, int ntok,
+                            float* y, const float* bias, int acc, hipStream_t st) {
+  if (ntok <= 0 || rows <= 0) return hipSuccess;
+  if (cols % 64 != 0 || (long long)rows * 1024 >= 0x7FFFFFFFLL || (long long)128 * cols >= 0x7FFFFFFFLL) return hipErrorInvalidValue;
+  BfParams p = {};
+  p.w = wq; p.wdq = wd; p.rows = rows; p.cols = cols; p.row_bytes = cols; p.x = (const u16*)xq; p.xd = xs;
+  p.y = y; p.bias = bias; p.acc = acc; p.ntok = ntok; p.ldy = rows;
+  const long long total = (long long)((ntok + 127) / 128) * ((rows + 127) / 128), per = (total + 7) / 8;
+  if (per * 8 > 0x7FFFFFFFLL) return hipErrorInvalidValue;
+  hipLaunchKernelGGL(gemm_i8q_kernel, dim3((unsigned)(per * 8)), dim3(512), 0, st, p);
+  return hipGetLastError();
 }
 
 hipError_t ilt_k_gemm_i8_planes_id(int fmt, const uint64_t* ptrs, long long add, const uint32_t* counts, const uint32_t* bases, int ne,

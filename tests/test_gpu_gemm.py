@@ -31,20 +31,21 @@ CASES = [
     (synth.Q6_K, 65, 256, 65),
     (synth.Q6_K, 300, 1024, 333),       # three row tiles and three token tiles of 128, the last of each ragged
     (synth.Q6_K, 256, 768, 128),        # an odd number of super-blocks
+    (synth.Q8_0, 300, 1024, 333),
     (synth.Q4_K, 300, 1024, 333),
     (synth.Q4_K, 256, 768, 128),
 ]
 
 
-# ILT_I8_PLANES: "0" = the 64 x 64 kernel always, "1" = Q6_K and Q4_K always on the pipelined kernel with the weights as two int8
-# planes (else only with enough tokens and rows to fill its 128 x 128 tiles)
+# ILT_I8_PLANES: "0" = the 64 x 64 kernel always, "1" = always the pipelined kernels (Q6_K and Q4_K as two int8 planes, Q8_0
+# a block per MFMA), else only with enough tokens and rows to fill their 128 x 128 tiles
 @pytest.mark.parametrize("planes", [None, "0", "1"])
 @pytest.mark.parametrize("qtype,rows,cols,n", CASES)
 def test_dense_prefill_equals_cpu_matmul_bit_for_bit(dev, monkeypatch, qtype, rows, cols, n, planes):
     from illatio_amd import dense, hip
     if planes is None:
         monkeypatch.delenv("ILT_I8_PLANES", raising=False)
-    elif qtype not in (synth.Q6_K, synth.Q4_K):
+    elif cols % 64:
         pytest.skip("one kernel for this format")
     else:
         monkeypatch.setenv("ILT_I8_PLANES", planes)
