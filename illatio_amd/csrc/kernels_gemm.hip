@@ -431,9 +431,10 @@ hipError_t ilt_k_gemm_i8(int fmt, const uint8_t* w, const uint16_t* wd, long lon
   // as int8 planes, the same bits.  ILT_I8_PLANES (tests): "0" never, "1" whenever the format allows.
   const char* force = getenv("ILT_I8_PLANES");
   const int forced = force ? atoi(force) : -1;
-  if ((fmt == ILT_Q6_K || fmt == ILT_Q4_K || fmt == ILT_Q2_K) && cols % 256 == 0 && forced != 0 && (forced == 1 || (ntok >= 96 && rows >= 128)))
+  const bool fits = rows < (1 << 21) && (long long)rows * row_bytes < 0x7FFFFFFFLL;      // the pipelined kernels' 32-bit offsets
+  if (fits && (fmt == ILT_Q6_K || fmt == ILT_Q4_K || fmt == ILT_Q2_K) && cols % 256 == 0 && forced != 0 && (forced == 1 || (ntok >= 96 && rows >= 128)))
     return ilt_k_gemm_i8_planes(fmt, w, row_bytes, rows, cols, xq, xs, bsums, ntok, y, bias, acc, st);
-  if (fmt == ILT_Q8_0 && cols % 64 == 0 && forced != 0 && (forced == 1 || (ntok >= 96 && rows >= 128)))
+  if (fits && fmt == ILT_Q8_0 && cols % 64 == 0 && forced != 0 && (forced == 1 || (ntok >= 96 && rows >= 128)))
     return ilt_k_gemm_i8_q8(w, wd, rows, cols, xq, xs, ntok, y, bias, acc, st);
   GemmParams p = {};
   p.w = w; p.wdq = wd; p.rows = rows; p.cols = cols; p.row_bytes = row_bytes;
@@ -450,7 +451,8 @@ hipError_t ilt_k_gemm_i8_id(int fmt, const uint64_t* ptrs, long long add, const 
     // the experts' IQ2_XXS and Q2_K (and Q4_K / Q6_K) matrices on the planes kernel when the groups average at least a quarter of a tile of 128 rows
     const char* force = getenv("ILT_I8_PLANES");
     const int forced = force ? atoi(force) : -1;
-    if ((fmt == ILT_Q6_K || fmt == ILT_Q4_K || fmt == ILT_Q2_K || fmt == ILT_IQ2_XXS) && cols % 256 == 0 && forced != 0 &&
+    if (rows < (1 << 21) && (long long)rows * row_bytes < 0x7FFFFFFFLL &&
+        (fmt == ILT_Q6_K || fmt == ILT_Q4_K || fmt == ILT_Q2_K || fmt == ILT_IQ2_XXS) && cols % 256 == 0 && forced != 0 &&
         (forced == 1 || (total_rows >= 32LL * ne && rows >= 128)))
       return ilt_k_gemm_i8_planes_id(fmt, ptrs, add, counts, bases, ne, row_bytes, rows, cols, xq, xs, bsums, total_rows, y, st);
   }
