@@ -68,7 +68,8 @@ def traffic_of(workload, per):
 
 
 HBM_PEAK_GBS = 8000.0
-MFMA_PEAK_TFLOPS = {"bf16": 2500.0, "bf16-1pass": 2500.0, "bf16-2pass": 2500.0, "bf16-resident": 2500.0, "int8": 5000.0}
+MFMA_PEAK_TFLOPS = {"bf16": 2500.0, "bf16-1pass": 2500.0, "bf16-2pass": 2500.0, "bf16-resident": 2500.0, "int8": 5000.0, "int8-2pass": 5000.0,
+                    "int8-resident": 5000.0}
 
 D, FFN, QD, KVD, VOCAB, LAYERS = 2560, 9728, 4096, 1024, 151936, 36
 
@@ -358,6 +359,19 @@ def workload_c3(args, dev):
             tm.launch("cvt", 0, lambda: dense.cvt_bf16(dev, xf, T * cols, xb))
             tm.launch("mm", flops, lambda: dense.cmat_mul_bf16(dev, m, xb, y, T))
         names = {"mm": "gemm_bf16_kernel<14, TM, TN, NB> (Q6_K dequantized to bf16 in LDS, v_mfma_f32_32x32x16_bf16)"}
+    elif path in ("int8-2pass", "int8-resident"):
+        # the exact product from the two int8 planes of the matrix, written inside every step or once beforehand and kept
+        act = dense.QAct(dev, T, cols, ("q8k",))
+        planes = dense.planes_i8(dev, m)
+        resident = path == "int8-resident"
+
+        def step(_):
+            tm.launch("quant", 0, lambda: dense.quantize_act(dev, xf, act))
+            if not resident:
+                tm.launch("planes", 0, lambda: dense.planes_i8(dev, m, planes))
+            tm.launch("mm", flops, lambda: dense.mat_mul_i8_planes(dev, planes, rows, cols, act, y, T))
+        names = {"mm": "gemm_i8pp_kernel (the two int8 planes of scale * (quant - 32) read as they were written beforehand, v_mfma_i32_32x32x32_i8, "
+                       "one float combine per super-block: bit-exact with the CPU path)"}
     else:
         act = dense.QAct(dev, T, cols, ("q8",) if qt == synth.Q8_0 else ("q8k",))
 
@@ -560,7 +574,7 @@ def main():
     ap.add_argument("--tokens", type=int, default=4096, help="c3, c5: tokens per step")
     ap.add_argument("--transpose", action="store_true", help="c3: the 5120x17408 matrix")
     ap.add_argument("--qtype", default="q6_k", choices=["q6_k", "q4_k", "q8_0"], help="c3: the matrix's format (BASELINE: q6_k)")
-    ap.add_argument("--path", default="bf16", choices=["bf16", "bf16-1pass", "bf16-2pass", "bf16-resident", "int8"],
+    ap.add_argument("--path", default="bf16", choices=["bf16", "bf16-1pass", "bf16-2pass", "bf16-resident", "int8", "int8-2pass", "int8-resident"],
                     help="c3, c5: which matrix-core path.  c3: bf16 = 2pass from 1024 tokens on, else 1pass; bf16-1pass = the matrix dequantized inside the product's loop; "
                          "bf16-2pass = the matrix dequantized to a bf16 copy inside the step, then the plain bf16 product; bf16-resident = that copy made beforehand and kept")
     ap.add_argument("--norm", action="store_true", help="c2: include each layer's two norms and the output norm (inside the product launches in fused mode)")

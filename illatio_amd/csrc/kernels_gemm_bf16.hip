@@ -206,6 +206,8 @@ struct BfParams {
   const float* xd; const int* bsums;
   // Q8_0 (gemm_i8q_kernel): w = the quants (a byte a weight, rows of cols bytes), wdq their f16 scales, xd the tokens' scales (one per 32)
   const u16* wdq;
+  // the planes made beforehand (gemm_i8pp_kernel): w = the hi plane, wlo the lo plane (a byte a weight, rows of cols bytes), wdf = d per row and super-block
+  const u8* wlo; const float* wdf;
 };
 
 template <int TM, int TN, int NXS, int NWS> struct Smem {
@@ -1388,6 +1390,168 @@ __global__ __launch_bounds__(512, 2) void gemm_i8q_kernel(BfParams p) {
   store_tile<NA, 1>(sum, p, tok0, ntok, r0, wt0, wr0, l32, lh);
 }
 
+// ---- the exact product in two passes: the planes once, then a loop without dequantization -------
+// As for bf16: with thousands of tokens (or a matrix multiplied again and again) the two planes
+// of a Q6_K matrix are worth writing out once -- a byte a weight each, in slabs of 128 rows x 64
+// columns (the row count padded to a multiple of 128), and d per row and super-block as floats -- so that the product's loop holds only direct loads of
+// three slabs, fragment reads, MFMAs and the combine per super-block.  The same integers, the
+// same float expression per block: the same bits as gemm_i8p_kernel and the CPU path.
+template <int FMT>
+__global__ __launch_bounds__(256) void planes_i8_kernel(const u8* __restrict__ w, long long row_bytes, int rows, int cols,
+                                                        u8* __restrict__ wh, u8* __restrict__ wl, float* __restrict__ wdf) {
+  typedef I8p<FMT> F;
+  const int nsb = cols / 256;
+  const long long u = (long long)blockIdx.x * 256 + threadIdx.x;       // 16 weights: unit q4 of step J of a super-block of a row
+  if (u >= (long long)rows * nsb * 16) return;
+  const int q4 = (int)(u & 3), J = (int)((u >> 2) & 3);
+  const long long sr = u >> 4;
+  const int sb = (int)(sr % nsb);
+  const long long row = sr / nsb;
+  const __amdgpu_buffer_rsrc_t rw = ilt_rsrc(ilt_uniform_ptr(w), (u32)min((long long)rows * row_bytes, 0xFFFFFFF0LL));
+  typename F::Raw r;
+  F::load(r, rw, (u32)(row * row_bytes), 2 * sb + (J >> 1), q4);
+  int hi[4], lo[4];
+  const int dummy = 0;
+  switch (J) {            // (the step is a constant inside planes)
+    case 0: F::planes(r, 0, q4, hi, lo, dummy); break;
+    case 1: F::planes(r, 1, q4, hi, lo, dummy); break;
+    case 2: F::planes(r, 2, q4, hi, lo, dummy); break;
+    default: F::planes(r, 3, q4, hi, lo, dummy); break;
+  }
+  // slab order: the 64 columns of a step for 128 consecutive rows are 8 KB in one piece (row r of the group at 64*r),
+  // the groups' slabs for step 0, 1, ... one after another, so that the product's direct loads read whole lines
+  const long long o = ((row >> 7) * (cols / 64) + sb * 4 + J) * 8192 + (row & 127) * 64 + 16 * q4;
+  *(int4*)(wh + o) = make_int4(hi[0], hi[1], hi[2], hi[3]);
+  *(int4*)(wl + o) = make_int4(lo[0], lo[1], lo[2], lo[3]);
+  if (J == 0 && q4 == 0) wdf[row * nsb + sb] = F::d_of(r);
+}
+
+constexpr int I8PP_RING = 5;             // slabs in flight + 1: the planes come from HBM, four steps ahead
+struct I8ppSmem {
+  __align__(16) u8 xs[I8PP_RING][128 * 64];
+  __align__(16) u8 wh[I8PP_RING][128 * 64];
+  __align__(16) u8 wl[I8PP_RING][128 * 64];
+  float wd[128], xd[128];                 // of the super-block: d of the rows, the tokens' scales
+  int cx[128];                            //   and 4000 * the sum of their quants
+  u32 scan[256];
+  int tile_z, tile_t0, tile_n, pad;
+};
+
+__global__ __launch_bounds__(512, 2) void gemm_i8pp_kernel(BfParams p) {
+  constexpr int TM = 128, TN = 128, NA = 2, KW = 64;
+  constexpr int NL = 3, XL = 6;                              // loads a step (three slabs), of a super-block's constants
+  extern __shared__ __align__(16) u8 i8pp_lds[];
+  I8ppSmem& S = *(I8ppSmem*)i8pp_lds;
+  const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+
+  long tok0; int ntok, rt; const u8* w = p.w;
+  if (!pick_tile<TM, TN>(p, S, tok0, ntok, rt, w)) return;
+  const int r0 = rt * TM;
+  const int nk = p.cols / KW, nsb = p.cols / 256;
+
+  const int prow = t >> 2, pk = (t & 3) ^ (int)slab_swz(prow);          // piece t of a slab
+  const u8* xbase = (const u8*)ilt_uniform_ptr((const i8*)p.x + tok0 * (long)p.cols);
+  const u8* hbase = (const u8*)ilt_uniform_ptr(p.w + (long)rt * nk * 8192);       // the row tile's slabs, one a step
+  const u8* lbase = (const u8*)ilt_uniform_ptr(p.wlo + (long)rt * nk * 8192);
+  const u32 xoff = (u32)min(prow, ntok - 1) * (u32)p.cols + 16 * pk;
+  const u32 woff = (u32)prow * 64 + 16 * pk;
+  auto issue = [&](int stage, int ks) {
+    ilt_g2lds16(xbase + ks * KW + xoff, S.xs[stage] + wave * 1024);
+    ilt_g2lds16(hbase + (long)ks * 8192 + woff, S.wh[stage] + wave * 1024);
+    ilt_g2lds16(lbase + (long)ks * 8192 + woff, S.wl[stage] + wave * 1024);
+  };
+  // a super-block's constants, by thread t & 127 (every wave loads, so that all count the same loads)
+  const long ctok = tok0 + min(t & 127, ntok - 1);
+  const float* xdp = p.xd + ctok * nsb;
+  const int4* bsp = (const int4*)(p.bsums + ctok * (p.cols / 16));
+  const float* wdp = p.wdf + (long)min(r0 + (t & 127), p.rows - 1) * nsb;
+  float c_yd, c_d; int4 c_bs[4];
+  auto load_consts = [&](int sb) {
+    c_yd = xdp[sb];
+    c_d = wdp[sb];
+#pragma unroll
+    for (int i = 0; i < 4; i++) c_bs[i] = bsp[4 * sb + i];
+  };
+  auto store_consts = [&]() {                                // after a barrier that ends the last block's reads
+    if (t < 128) {
+      int sx = 0;
+#pragma unroll
+      for (int i = 0; i < 4; i++) sx += c_bs[i].x + c_bs[i].y + c_bs[i].z + c_bs[i].w;
+      ilt_lds_st4_untracked(&S.xd[t], __builtin_bit_cast(u32, c_yd));
+      ilt_lds_st4_untracked(&S.cx[t], (u32)(4000 * sx));
+      ilt_lds_st4_untracked(&S.wd[t], __builtin_bit_cast(u32, c_d));
+    }
+  };
+
+  v16f sum[NA][1];
+  v16i_ ah[NA], al[NA];
+#pragma unroll
+  for (int a = 0; a < NA; a++)
+#pragma unroll
+    for (int r = 0; r < 16; r++) sum[a][0][r] = 0.0f;
+  const int wt0 = 64 * (wave & 1), wr0 = 32 * (wave >> 1);  // this wave's tokens and rows in the tile
+  const int l32 = lane & 31, lh = lane >> 5;
+  u32 aoff[NA];
+#pragma unroll
+  for (int a = 0; a < NA; a++) aoff[a] = slab_off(wt0 + 32 * a + l32, lh);
+  const u32 boff = slab_off(wr0 + l32, lh);
+
+  constexpr int D = I8PP_RING;
+  load_consts(0);
+  store_consts();
+#pragma unroll
+  for (int i = 0; i < D - 1; i++) issue(i, min(i, nk - 1));
+  int cur = 0;                                               // the step's slabs' place in the rings
+  const v16i_ zero = {};
+  auto step = [&](int ks, auto Jc) {
+    constexpr int J = decltype(Jc)::value;                   // the step's place in its super-block
+    // This step's slabs were sent D-1 steps ago: all loads but those of the D-2 steps since have landed
+    // (the constants' loads of step 2 of a super-block among them, unless this is step 2 itself).
+    constexpr int prev = (D - 2) * NL + (J != 2 ? XL : 0);
+    if (ks < D - 1) asm volatile("s_waitcnt vmcnt(%0)" :: "n"((D - 2) * NL) : "memory");     // (no constants' loads before the first super-block's slabs)
+    else asm volatile("s_waitcnt vmcnt(%0)" :: "n"(prev) : "memory");
+    ilt_barrier_lds();                                       // no fence: later steps' loads stay in flight
+    const int sb = ks >> 2;
+    if (J == 0 && ks > 0) store_consts();                    // (the first block's were stored before the loop)
+    if (J == 2) load_consts(min(sb + 1, nsb - 1));
+    issue(cur == 0 ? D - 1 : cur - 1, min(ks + D - 1, nk - 1));         // into the slabs the step before read
+    __builtin_amdgcn_sched_barrier(0);
+    const u8* xs = S.xs[cur];
+    const u8* whs = S.wh[cur];
+    const u8* wls = S.wl[cur];
+#pragma unroll
+    for (int kk = 0; kk < 2; kk++) {
+      const v4i_ bh = *(const v4i_*)(whs + (boff ^ (32 * kk))), bl = *(const v4i_*)(wls + (boff ^ (32 * kk)));
+#pragma unroll
+      for (int a = 0; a < NA; a++) {                         // a super-block's first products start its integer sums
+        const v4i_ af = *(const v4i_*)(xs + (aoff[a] ^ (32 * kk)));
+        ah[a] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af, bh, (J == 0 && kk == 0) ? zero : ah[a], 0, 0, 0);
+        al[a] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af, bl, (J == 0 && kk == 0) ? zero : al[a], 0, 0, 0);
+      }
+    }
+    if (J == 3) {          // the super-block is complete: sum += (d * yd) * float(isum), as the CPU path adds it
+      const float d = S.wd[wr0 + l32];
+#pragma unroll
+      for (int a = 0; a < NA; a++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+          const int tk = wt0 + 32 * a + 8 * (r >> 2) + 4 * lh + (r & 3);
+          const int isum = 256 * ah[a][r] + al[a][r] - S.cx[tk];
+          sum[a][0][r] = sum[a][0][r] + (d * S.xd[tk]) * (float)isum;
+        }
+    }
+    cur = cur == D - 1 ? 0 : cur + 1;
+  };
+  for (int ks = 0; ks < nk; ks += 4) {
+    step(ks + 0, std::integral_constant<int, 0>{});
+    step(ks + 1, std::integral_constant<int, 1>{});
+    step(ks + 2, std::integral_constant<int, 2>{});
+    step(ks + 3, std::integral_constant<int, 3>{});
+  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // the tail's redundant loads: nothing may land in LDS after the workgroup ends
+  store_tile<NA, 1>(sum, p, tok0, ntok, r0, wt0, wr0, l32, lh);
+}
+
 // ---- the two-pass product: W as plain bf16 ------------------------------------------------------
 // With thousands of tokens the in-loop dequantization above is repeated for every tile of 256
 // tokens and its VALU work competes with the MFMAs for issue slots.  With HBM to spare the
@@ -1679,6 +1843,37 @@ hipError_t ilt_k_gemm_i8_planes(int fmt, const uint8_t* w, long long row_bytes, 
   p.w = w; p.rows = rows; p.cols = cols; p.row_bytes = row_bytes; p.x = (const u16*)xq; p.xd = xd; p.bsums = bsums;
   p.y = y; p.bias = bias; p.acc = acc; p.ntok = ntok; p.ldy = rows;
   return launch_i8p<false>(fmt, p, (ntok + 127) / 128, st);
+}
+
+hipError_t ilt_k_planes_i8(int fmt, const uint8_t* w, long long row_bytes, int rows, int cols, uint8_t* wh, uint8_t* wl, float* wdf,
+                           hipStream_t st) {
+  if (rows <= 0) return hipSuccess;
+  if (fmt != ILT_Q6_K || cols % 256 != 0 || (long long)rows * row_bytes >= 0xFFFFFFF0LL) return hipErrorInvalidValue;
+  const long long units = (long long)rows * (cols / 256) * 16;
+  if ((units + 255) / 256 > 0x7FFFFFFFLL) return hipErrorInvalidValue;
+  hipLaunchKernelGGL(planes_i8_kernel<ILT_Q6_K>, dim3((unsigned)((units + 255) / 256)), dim3(256), 0, st, w, row_bytes, rows, cols, wh, wl, wdf);
+  return hipGetLastError();
+}
+
+hipError_t ilt_k_gemm_i8_pp(const uint8_t* wh, const uint8_t* wl, const float* wdf, int rows, int cols, const int8_t* xq, const float* xd,
+                            const int* bsums, int ntok, float* y, const float* bias, int acc, hipStream_t st) {
+  if (ntok <= 0 || rows <= 0) return hipSuccess;
+  if (cols % 256 != 0 || (long long)rows * 1024 >= 0x7FFFFFFFLL || (long long)128 * cols >= 0x7FFFFFFFLL) return hipErrorInvalidValue;
+  BfParams p = {};
+  p.w = wh; p.wlo = wl; p.wdf = wdf; p.rows = rows; p.cols = cols; p.row_bytes = cols; p.x = (const u16*)xq; p.xd = xd; p.bsums = bsums;
+  p.y = y; p.bias = bias; p.acc = acc; p.ntok = ntok; p.ldy = rows;
+  const long long total = (long long)((ntok + 127) / 128) * ((rows + 127) / 128), per = (total + 7) / 8;
+  if (per * 8 > 0x7FFFFFFFLL) return hipErrorInvalidValue;
+  static bool attr_set[8] = {};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 8) dev = 0;
+  if (!attr_set[dev]) {            // more dynamic LDS than the default 64 KB: asked for once per device
+    const hipError_t e = hipFuncSetAttribute((const void*)gemm_i8pp_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)sizeof(I8ppSmem));
+    if (e != hipSuccess) return e;
+    attr_set[dev] = true;
+  }
+  hipLaunchKernelGGL(gemm_i8pp_kernel, dim3((unsigned)(per * 8)), dim3(512), sizeof(I8ppSmem), st, p);
+  return hipGetLastError();
 }
 
 hipError_t ilt_k_gemm_i8_q8(const uint8_t* wq, const uint16_t* wd, int rows, int cols, const int8_t* xq, const float* xs, int ntok,

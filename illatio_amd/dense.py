@@ -169,6 +169,37 @@ def dequant_bf16(dev, w, out=None):
     return out
 
 
+def planes_bytes(rows, cols):
+    """Bytes of one int8 plane of a ROWS x COLS matrix (slabs of 128 rows x 64 columns; the rows padded to a multiple of 128)."""
+    return (rows + 127) // 128 * 128 * cols
+
+
+def planes_to_rows(a, rows, cols):
+    """A plane downloaded as bytes (64 columns of 128 rows in one piece) as ROWS x COLS."""
+    return a.reshape(-1, cols // 64, 128, 64).transpose(0, 2, 1, 3).reshape(-1, cols)[:rows]
+
+
+def planes_i8(dev, w, out=None):
+    """The Q6_K matrix W as the exact product's two int8 planes and its d per row and
+    super-block: (WH, WL, WDF), DBufs of PLANES-BYTES, PLANES-BYTES and 4*rows*cols/256 bytes
+    (OUT or new ones).  The first pass of the two-pass exact product."""
+    if w.type != Q6_K:
+        raise ValueError(f"the planes are made of Q6_K matrices; {w.name} is type {w.type}")
+    nb = planes_bytes(w.rows, w.cols)
+    wh, wl, wdf = out if out is not None else (hip.hip_alloc(dev, nb), hip.hip_alloc(dev, nb), hip.hip_alloc(dev, 4 * w.rows * (w.cols // 256), zero=False))
+    hip.launch(dev, "planes_i8", (w.rows * (w.cols // 256) * 16 + 255) // 256, 256, [w.type, w.qs, wh, wl, wdf, w.rows, w.cols])
+    return wh, wl, wdf
+
+
+def mat_mul_i8_planes(dev, planes, rows, cols, act, y, n, bias=None, acc=False):
+    """Y = W X for N tokens from PLANES (PLANES-I8's result) and the Q8_K activations in ACT:
+    CMAT-MUL's bits without dequantizing W again."""
+    wh, wl, wdf = planes
+    hip.launch(dev, "mm_i8_planes", ((n + 127) // 128, (rows + 127) // 128), 512,
+               [wh, wl, wdf, act.kq, act.kd, act.ksum, y, bias, rows, cols, n, 1 if acc else 0])
+    return y
+
+
 def cvt_bf16_slabs(dev, x, n, cols, out=None):
     """N tokens of COLS floats (a DBuf) rounded to bf16 in slabs, into OUT or a new DBuf of SLABS-BYTES."""
     out = out if out is not None else hip.hip_alloc(dev, slabs_bytes(n, cols), zero=False)

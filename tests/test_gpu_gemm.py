@@ -74,6 +74,42 @@ def test_dense_prefill_equals_cpu_matmul_bit_for_bit(dev, monkeypatch, qtype, ro
     act.free(); m.free()
 
 
+@pytest.mark.parametrize("rows,cols,n", [(640, 5120, 96), (65, 256, 65), (300, 1024, 333), (256, 768, 128)])
+def test_two_pass_exact_product_bit_for_bit(dev, rows, cols, n):
+    """The Q6_K product from planes written beforehand (planes_i8, mm_i8_planes): the planes hold
+    scale * (quant - 32) + 4128 split into bytes, and the product is the CPU's, bias and
+    accumulation included."""
+    from illatio_amd import dense, hip
+    rng = synth.make_rng(rows + cols + n)
+    w = synth.weights(synth.Q6_K, rows, cols, rng)
+    x = synth.activations((n, cols), rng)
+    x[0, :256] = 0.0
+    bias = synth.activations(rows, rng)
+    m = dense.upload_gmat(dev, "w", synth.Q6_K, rows, cols, w)
+    act = dense.QAct(dev, n, cols, ("q8k",))
+    xb, bb = hip.hip_upload_new(dev, x), hip.hip_upload_new(dev, bias)
+    y = hip.hip_alloc(dev, 4 * n * rows)
+    dense.quantize_act(dev, xb, act)
+    planes = dense.planes_i8(dev, m)
+    # every weight back from its planes: 256 * hi + (lo - 128 as a signed byte ... + 128) - 4128 = sc * (q - 32)
+    nbytes = dense.planes_bytes(rows, cols)
+    wh = dense.planes_to_rows(hip.hip_download(planes[0], np.uint8, nbytes), rows, cols).astype(np.int64).reshape(-1)
+    wl = dense.planes_to_rows(hip.hip_download(planes[1], np.int8, nbytes), rows, cols).astype(np.int64).reshape(-1)
+    deq = orc.dequant_rows(synth.Q6_K, w, cols).reshape(rows, cols // 256, 256)
+    d = hip.hip_floats(planes[2], rows * (cols // 256)).reshape(rows, cols // 256)
+    back = d[:, :, None] * (256 * wh + wl + 128 - 4128).reshape(rows, cols // 256, 256).astype(np.float32)
+    assert np.array_equal(back, deq), (np.abs(back - deq).max(), np.argwhere(back != deq)[:5])      # (as numbers: a zero's sign may differ)
+    dense.mat_mul_i8_planes(dev, planes, rows, cols, act, y, n)
+    want = orc.matmul(synth.Q6_K, w, rows, cols, x, nthreads=8)
+    got = hip.hip_floats(y, n * rows).reshape(n, rows)
+    assert np.array_equal(bits(got), bits(want)), (np.abs(got - want).max(), np.argwhere(bits(got) != bits(want))[:5])
+    dense.mat_mul_i8_planes(dev, planes, rows, cols, act, y, n, bias=bb, acc=True)
+    assert np.array_equal(bits(hip.hip_floats(y, n * rows).reshape(n, rows)), bits(want + (want + bias[None, :])))
+    for b in (xb, bb, y) + tuple(planes):
+        hip.hip_free(b)
+    act.free(); m.free()
+
+
 @pytest.mark.parametrize("ne,d,ff,nu,n,clamp", [(8, 512, 256, 3, 37, 0.0), (16, 1024, 512, 4, 150, 0.6),
                                                  (12, 4096, 2048, 6, 96, 0.0)])
 @pytest.mark.parametrize("planes", [None, "0", "1"])        # the down product (Q2_K) on the 64 x 64 kernel / on the planes kernel
