@@ -1426,22 +1426,27 @@ __global__ __launch_bounds__(256) void planes_i8_kernel(const u8* __restrict__ w
   if (J == 0 && q4 == 0) wdf[row * nsb + sb] = F::d_of(r);
 }
 
-constexpr int I8PP_RING = 5;             // slabs in flight + 1: the planes come from HBM, four steps ahead
-struct I8ppSmem {
-  __align__(16) u8 xs[I8PP_RING][128 * 64];
-  __align__(16) u8 wh[I8PP_RING][128 * 64];
-  __align__(16) u8 wl[I8PP_RING][128 * 64];
+// NB row patches a wave: 1 = eight waves of 32 rows x 64 tokens (one workgroup a CU, slabs four steps ahead).
+// (2 = four waves of 64 x 64, two workgroups a CU, reads a quarter less from LDS per MFMA but does not fit the
+// registers: 27 spilled, 486 against 590 TFLOP/s.)
+template <int NB> struct I8ppSmem {
+  static constexpr int RING = NB == 1 ? 5 : 3;
+  __align__(16) u8 xs[RING][128 * 64];
+  __align__(16) u8 wh[RING][128 * 64];
+  __align__(16) u8 wl[RING][128 * 64];
   float wd[128], xd[128];                 // of the super-block: d of the rows, the tokens' scales
   int cx[128];                            //   and 4000 * the sum of their quants
   u32 scan[256];
   int tile_z, tile_t0, tile_n, pad;
 };
 
-__global__ __launch_bounds__(512, 2) void gemm_i8pp_kernel(BfParams p) {
+template <int NB>
+__global__ __launch_bounds__(512 / NB, 2) void gemm_i8pp_kernel(BfParams p) {
   constexpr int TM = 128, TN = 128, NA = 2, KW = 64;
-  constexpr int NL = 3, XL = 6;                              // loads a step (three slabs), of a super-block's constants
+  constexpr int THREADS = 512 / NB, NWAVES = THREADS / 64, NP = 512 / THREADS;      // NP: pieces of a slab a thread sends for
+  constexpr int NL = 3 * NP, XL = 2;                         // loads a step (three slabs), of a super-block's constants
   extern __shared__ __align__(16) u8 i8pp_lds[];
-  I8ppSmem& S = *(I8ppSmem*)i8pp_lds;
+  I8ppSmem<NB>& S = *(I8ppSmem<NB>*)i8pp_lds;
   const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
 
   long tok0; int ntok, rt; const u8* w = p.w;
@@ -1449,54 +1454,60 @@ __global__ __launch_bounds__(512, 2) void gemm_i8pp_kernel(BfParams p) {
   const int r0 = rt * TM;
   const int nk = p.cols / KW, nsb = p.cols / 256;
 
-  const int prow = t >> 2, pk = (t & 3) ^ (int)slab_swz(prow);          // piece t of a slab
   const u8* xbase = (const u8*)ilt_uniform_ptr((const i8*)p.x + tok0 * (long)p.cols);
   const u8* hbase = (const u8*)ilt_uniform_ptr(p.w + (long)rt * nk * 8192);       // the row tile's slabs, one a step
   const u8* lbase = (const u8*)ilt_uniform_ptr(p.wlo + (long)rt * nk * 8192);
-  const u32 xoff = (u32)min(prow, ntok - 1) * (u32)p.cols + 16 * pk;
-  const u32 woff = (u32)prow * 64 + 16 * pk;
+  u32 xoff[NP], woff[NP];                                    // piece i * THREADS + t of a slab
+#pragma unroll
+  for (int i = 0; i < NP; i++) {
+    const int P_ = i * THREADS + t, prow = P_ >> 2, pk = (P_ & 3) ^ (int)slab_swz(prow);
+    xoff[i] = (u32)min(prow, ntok - 1) * (u32)p.cols + 16 * pk;
+    woff[i] = (u32)prow * 64 + 16 * pk;
+  }
   auto issue = [&](int stage, int ks) {
-    ilt_g2lds16(xbase + ks * KW + xoff, S.xs[stage] + wave * 1024);
-    ilt_g2lds16(hbase + (long)ks * 8192 + woff, S.wh[stage] + wave * 1024);
-    ilt_g2lds16(lbase + (long)ks * 8192 + woff, S.wl[stage] + wave * 1024);
+#pragma unroll
+    for (int i = 0; i < NP; i++) {
+      ilt_g2lds16(xbase + ks * KW + xoff[i], S.xs[stage] + (i * NWAVES + wave) * 1024);
+      ilt_g2lds16(hbase + (long)ks * 8192 + woff[i], S.wh[stage] + (i * NWAVES + wave) * 1024);
+      ilt_g2lds16(lbase + (long)ks * 8192 + woff[i], S.wl[stage] + (i * NWAVES + wave) * 1024);
+    }
   };
   // a super-block's constants, by thread t & 127 (every wave loads, so that all count the same loads)
   const long ctok = tok0 + min(t & 127, ntok - 1);
+  // (the sums of the tokens' quants over a super-block are taken from the slabs in LDS, see the step: the
+  // activations' sums of 16 would be 16 more registers held across two steps)
   const float* xdp = p.xd + ctok * nsb;
-  const int4* bsp = (const int4*)(p.bsums + ctok * (p.cols / 16));
   const float* wdp = p.wdf + (long)min(r0 + (t & 127), p.rows - 1) * nsb;
-  float c_yd, c_d; int4 c_bs[4];
+  float c_yd, c_d;
   auto load_consts = [&](int sb) {
     c_yd = xdp[sb];
     c_d = wdp[sb];
-#pragma unroll
-    for (int i = 0; i < 4; i++) c_bs[i] = bsp[4 * sb + i];
   };
   auto store_consts = [&]() {                                // after a barrier that ends the last block's reads
     if (t < 128) {
-      int sx = 0;
-#pragma unroll
-      for (int i = 0; i < 4; i++) sx += c_bs[i].x + c_bs[i].y + c_bs[i].z + c_bs[i].w;
       ilt_lds_st4_untracked(&S.xd[t], __builtin_bit_cast(u32, c_yd));
-      ilt_lds_st4_untracked(&S.cx[t], (u32)(4000 * sx));
       ilt_lds_st4_untracked(&S.wd[t], __builtin_bit_cast(u32, c_d));
     }
   };
+  int xsum[NP] = {};
 
-  v16f sum[NA][1];
-  v16i_ ah[NA], al[NA];
+  v16f sum[NA][NB];
+  v16i_ ah[NA][NB], al[NA][NB];
 #pragma unroll
   for (int a = 0; a < NA; a++)
 #pragma unroll
-    for (int r = 0; r < 16; r++) sum[a][0][r] = 0.0f;
-  const int wt0 = 64 * (wave & 1), wr0 = 32 * (wave >> 1);  // this wave's tokens and rows in the tile
+    for (int b = 0; b < NB; b++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) sum[a][b][r] = 0.0f;
+  const int wt0 = 64 * (wave & 1), wr0 = 32 * NB * (wave >> 1);       // this wave's tokens and rows in the tile
   const int l32 = lane & 31, lh = lane >> 5;
-  u32 aoff[NA];
+  u32 aoff[NA], boff[NB];
 #pragma unroll
   for (int a = 0; a < NA; a++) aoff[a] = slab_off(wt0 + 32 * a + l32, lh);
-  const u32 boff = slab_off(wr0 + l32, lh);
+#pragma unroll
+  for (int b = 0; b < NB; b++) boff[b] = slab_off(wr0 + 32 * b + l32, lh);
 
-  constexpr int D = I8PP_RING;
+  constexpr int D = I8ppSmem<NB>::RING;
   load_consts(0);
   store_consts();
 #pragma unroll
@@ -1506,8 +1517,9 @@ __global__ __launch_bounds__(512, 2) void gemm_i8pp_kernel(BfParams p) {
   auto step = [&](int ks, auto Jc) {
     constexpr int J = decltype(Jc)::value;                   // the step's place in its super-block
     // This step's slabs were sent D-1 steps ago: all loads but those of the D-2 steps since have landed
-    // (the constants' loads of step 2 of a super-block among them, unless this is step 2 itself).
-    constexpr int prev = (D - 2) * NL + (J != 2 ? XL : 0);
+    // (the constants' loads of step 2 of a super-block among them, if that step is one of those).
+    constexpr bool consts_since = D == 5 ? J != 2 : J == 3;
+    constexpr int prev = (D - 2) * NL + (consts_since ? XL : 0);
     if (ks < D - 1) asm volatile("s_waitcnt vmcnt(%0)" :: "n"((D - 2) * NL) : "memory");     // (no constants' loads before the first super-block's slabs)
     else asm volatile("s_waitcnt vmcnt(%0)" :: "n"(prev) : "memory");
     ilt_barrier_lds();                                       // no fence: later steps' loads stay in flight
@@ -1520,24 +1532,57 @@ __global__ __launch_bounds__(512, 2) void gemm_i8pp_kernel(BfParams p) {
     const u8* whs = S.wh[cur];
     const u8* wls = S.wl[cur];
 #pragma unroll
-    for (int kk = 0; kk < 2; kk++) {
-      const v4i_ bh = *(const v4i_*)(whs + (boff ^ (32 * kk))), bl = *(const v4i_*)(wls + (boff ^ (32 * kk)));
-#pragma unroll
-      for (int a = 0; a < NA; a++) {                         // a super-block's first products start its integer sums
-        const v4i_ af = *(const v4i_*)(xs + (aoff[a] ^ (32 * kk)));
-        ah[a] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af, bh, (J == 0 && kk == 0) ? zero : ah[a], 0, 0, 0);
-        al[a] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af, bl, (J == 0 && kk == 0) ? zero : al[a], 0, 0, 0);
-      }
+    for (int i = 0; i < NP; i++) {                           // the sum of the step's 64 quants of token (i * THREADS + t) / 4, in its four lanes
+      const int4 xv = ilt_lds_ld16(xs + slab_off((i * THREADS + t) >> 2, t & 3));
+      int sp = __builtin_amdgcn_sdot4(xv.x, 0x01010101, 0, false);
+      sp = __builtin_amdgcn_sdot4(xv.y, 0x01010101, sp, false);
+      sp = __builtin_amdgcn_sdot4(xv.z, 0x01010101, sp, false);
+      sp = __builtin_amdgcn_sdot4(xv.w, 0x01010101, sp, false);
+      sp += __shfl_xor(sp, 1);
+      sp += __shfl_xor(sp, 2);
+      xsum[i] = J == 0 ? sp : xsum[i] + sp;
     }
-    if (J == 3) {          // the super-block is complete: sum += (d * yd) * float(isum), as the CPU path adds it
-      const float d = S.wd[wr0 + l32];
+#pragma unroll
+    for (int kk = 0; kk < 2; kk++) {
+      v4i_ af[NA], bh[NB], bl[NB];
+#pragma unroll
+      for (int a = 0; a < NA; a++) af[a] = *(const v4i_*)(xs + (aoff[a] ^ (32 * kk)));
+#pragma unroll
+      for (int b = 0; b < NB; b++) { bh[b] = *(const v4i_*)(whs + (boff[b] ^ (32 * kk))); bl[b] = *(const v4i_*)(wls + (boff[b] ^ (32 * kk))); }
 #pragma unroll
       for (int a = 0; a < NA; a++)
 #pragma unroll
-        for (int r = 0; r < 16; r++) {
-          const int tk = wt0 + 32 * a + 8 * (r >> 2) + 4 * lh + (r & 3);
-          const int isum = 256 * ah[a][r] + al[a][r] - S.cx[tk];
-          sum[a][0][r] = sum[a][0][r] + (d * S.xd[tk]) * (float)isum;
+        for (int b = 0; b < NB; b++) {                       // a super-block's first products start its integer sums
+          ah[a][b] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[a], bh[b], (J == 0 && kk == 0) ? zero : ah[a][b], 0, 0, 0);
+          al[a][b] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[a], bl[b], (J == 0 && kk == 0) ? zero : al[a][b], 0, 0, 0);
+        }
+    }
+    if (J == 3) {          // the super-block is complete: sum += (d * yd) * float(isum), as the CPU path adds it
+#pragma unroll
+      for (int i = 0; i < NP; i++)
+        if ((t & 3) == 0) ilt_lds_st4_untracked(&S.cx[(i * THREADS + t) >> 2], (u32)(4000 * xsum[i]));
+      ilt_barrier_lds();
+      float d[NB];
+#pragma unroll
+      for (int b = 0; b < NB; b++) d[b] = S.wd[wr0 + 32 * b + l32];
+#pragma unroll
+      for (int a = 0; a < NA; a++)
+#pragma unroll
+        for (int r4 = 0; r4 < 4; r4++) {                     // four consecutive tokens' constants at a time
+          const int tk = wt0 + 32 * a + 8 * r4 + 4 * lh;
+          const float4 yd = *(const float4*)&S.xd[tk];
+          const int4 cx = *(const int4*)&S.cx[tk];
+          const float ydv[4] = {yd.x, yd.y, yd.z, yd.w};
+          const int cxv[4] = {cx.x, cx.y, cx.z, cx.w};
+#pragma unroll
+          for (int k = 0; k < 4; k++)
+#pragma unroll
+            for (int b = 0; b < NB; b++) {
+              const int r = 4 * r4 + k;
+              const int isum = 256 * ah[a][b][r] + al[a][b][r] - cxv[k];
+              sum[a][b][r] = sum[a][b][r] + (d[b] * ydv[k]) * (float)isum;
+            }
+          __builtin_amdgcn_sched_barrier(0);
         }
     }
     cur = cur == D - 1 ? 0 : cur + 1;
@@ -1549,7 +1594,7 @@ __global__ __launch_bounds__(512, 2) void gemm_i8pp_kernel(BfParams p) {
     step(ks + 3, std::integral_constant<int, 3>{});
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // the tail's redundant loads: nothing may land in LDS after the workgroup ends
-  store_tile<NA, 1>(sum, p, tok0, ntok, r0, wt0, wr0, l32, lh);
+  store_tile<NA, NB>(sum, p, tok0, ntok, r0, wt0, wr0, l32, lh);
 }
 
 // ---- the two-pass product: W as plain bf16 ------------------------------------------------------
@@ -1868,11 +1913,11 @@ hipError_t ilt_k_gemm_i8_pp(const uint8_t* wh, const uint8_t* wl, const float* w
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 8) dev = 0;
   if (!attr_set[dev]) {            // more dynamic LDS than the default 64 KB: asked for once per device
-    const hipError_t e = hipFuncSetAttribute((const void*)gemm_i8pp_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)sizeof(I8ppSmem));
+    const hipError_t e = hipFuncSetAttribute((const void*)gemm_i8pp_kernel<1>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)sizeof(I8ppSmem<1>));
     if (e != hipSuccess) return e;
     attr_set[dev] = true;
   }
-  hipLaunchKernelGGL(gemm_i8pp_kernel, dim3((unsigned)(per * 8)), dim3(512), sizeof(I8ppSmem), st, p);
+  hipLaunchKernelGGL(gemm_i8pp_kernel<1>, dim3((unsigned)(per * 8)), dim3(512), sizeof(I8ppSmem<1>), st, p);
   return hipGetLastError();
 }
 
