@@ -513,12 +513,11 @@ int ilt_planes_i8(uint64_t stream, int gguf_type, const void* w, int8_t* wh, int
 }
 
 int ilt_mm_i8_planes(uint64_t stream, const int8_t* wh, const int8_t* wl, const float* wdf, const int8_t* xq, const float* xd,
-                     const int32_t* bsums, float* y, const float* bias, int rows, int cols, int n, int acc) {
+                     float* y, const float* bias, int rows, int cols, int n, int acc) {
   ILT_REQUIRE(rows >= 0 && n >= 0 && cols > 0 && cols % 256 == 0 && cols < (1 << 22) && rows < (1 << 21));
   if (rows == 0 || n == 0) return ILT_OK;
-  ILT_REQUIRE(wh && wl && wdf && xq && xd && bsums && y && ((uintptr_t)wh & 15) == 0 && ((uintptr_t)wl & 15) == 0 && ((uintptr_t)xq & 15) == 0 &&
-              ((uintptr_t)bsums & 15) == 0);
-  return (int)ilt_k_gemm_i8_pp((const uint8_t*)wh, (const uint8_t*)wl, wdf, rows, cols, xq, xd, bsums, n, y, bias, acc, S(stream));
+  ILT_REQUIRE(wh && wl && wdf && xq && xd && y && ((uintptr_t)wh & 15) == 0 && ((uintptr_t)wl & 15) == 0 && ((uintptr_t)xq & 15) == 0);
+  return (int)ilt_k_gemm_i8_pp((const uint8_t*)wh, (const uint8_t*)wl, wdf, rows, cols, xq, xd, n, y, bias, acc, S(stream));
 }
 
 int ilt_mm_bf16(uint64_t stream, const uint16_t* wb, const uint16_t* xb, float* y, const float* bias, int rows, int cols, int n,
@@ -591,8 +590,8 @@ int ilt_launch(const char* kernel, unsigned gx, unsigned gy, unsigned gz, unsign
   K("cvt_bf16_slabs") return ilt_cvt_bf16_slabs(stream, a.ptr<cf>(0), a.ptr<uint16_t*>(1), a.i32(2), a.i32(3));
   K("planes_i8") return ilt_planes_i8(stream, a.i32(0), a.ptr<const void*>(1), a.ptr<int8_t*>(2), a.ptr<int8_t*>(3), a.ptr<float*>(4), a.i32(5), a.i32(6));
   K("mm_i8_planes")
-    return ilt_mm_i8_planes(stream, a.ptr<ci8>(0), a.ptr<ci8>(1), a.ptr<cf>(2), a.ptr<ci8>(3), a.ptr<cf>(4), a.ptr<const int32_t*>(5), a.ptr<float*>(6),
-                            a.ptr<cf>(7), a.i32(8), a.i32(9), a.i32(10), a.i32(11));
+    return ilt_mm_i8_planes(stream, a.ptr<ci8>(0), a.ptr<ci8>(1), a.ptr<cf>(2), a.ptr<ci8>(3), a.ptr<cf>(4), a.ptr<float*>(5),
+                            a.ptr<cf>(6), a.i32(7), a.i32(8), a.i32(9), a.i32(10));
   K("dequant_bf16") return ilt_dequant_bf16(stream, a.i32(0), a.ptr<const void*>(1), a.ptr<uint16_t*>(2), a.i32(3), a.i32(4));
   K("mm_bf16") return ilt_mm_bf16(stream, a.ptr<cu16>(0), a.ptr<cu16>(1), a.ptr<float*>(2), a.ptr<cf>(3), a.i32(4), a.i32(5), a.i32(6), a.i32(7));
   K("d4_mm_id_bf16")

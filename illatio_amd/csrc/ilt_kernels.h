@@ -99,7 +99,7 @@ hipError_t ilt_k_gemm_i8_planes(int fmt, const uint8_t* w, long long row_bytes, 
 hipError_t ilt_k_planes_i8(int fmt, const uint8_t* w, long long row_bytes, int rows, int cols, uint8_t* wh, uint8_t* wl, float* wdf,
                            hipStream_t st);
 hipError_t ilt_k_gemm_i8_pp(const uint8_t* wh, const uint8_t* wl, const float* wdf, int rows, int cols, const int8_t* xq, const float* xd,
-                            const int* bsums, int ntok, float* y, const float* bias, int acc, hipStream_t st);
+                            int ntok, float* y, const float* bias, int acc, hipStream_t st);
 // Q8_0, exact, on the pipelined kernel (cols a multiple of 64)
 hipError_t ilt_k_gemm_i8_q8(const uint8_t* wq, const uint16_t* wd, int rows, int cols, const int8_t* xq, const float* xs, int ntok,
                             float* y, const float* bias, int acc, hipStream_t st);

@@ -999,7 +999,10 @@ __global__ __launch_bounds__(512, 1) void gemm_i8p_kernel(BfParams p) {
   typedef I8p<FMT> F;
   typedef typename F::Raw Raw;
   constexpr int TM = 128, TN = 128, NA = 2, NI = 1;
-  constexpr int WL = F::WL, XL = FMT == ILT_IQ2_XXS ? 1 : 5;  // loads of a raw set, of a token's constants (IQ2_XXS comes without the sums of 16: d4_mm_id_iq2_xxs has no such argument)
+  // Q6_K needs the quants' sum over a block and IQ2_XXS over its even and odd groups (d4_mm_id_iq2_xxs has no argument for
+  // the sums of 16 anyway): both are added up from the slabs in LDS, which saves four 16-byte loads a thread and block.
+  constexpr bool XSLAB = FMT == ILT_IQ2_XXS || FMT == ILT_Q6_K;
+  constexpr int WL = F::WL, XL = XSLAB ? 1 : 5;               // loads of a raw set, of a token's constants
   constexpr bool TWO = F::PLANES == 2;
   constexpr bool SPLIT = FMT == ILT_IQ2_XXS;                 // the first and the second 32 columns of a step have sums of their own
   constexpr int KW = 64;                                     // columns a step
@@ -1040,7 +1043,7 @@ __global__ __launch_bounds__(512, 1) void gemm_i8p_kernel(BfParams p) {
   float c_yd; int4 c_bs[4];
   auto load_consts = [&](int sb) {
     c_yd = xdp[sb];
-    if constexpr (!SPLIT) {
+    if constexpr (!XSLAB) {
 #pragma unroll
       for (int i = 0; i < 4; i++) c_bs[i] = bsp[4 * sb + i];
     }
@@ -1048,12 +1051,12 @@ __global__ __launch_bounds__(512, 1) void gemm_i8p_kernel(BfParams p) {
   auto store_consts = [&](const Raw& ra) {                   // after a barrier that ends the last block's reads
     if (t < 128) {
       int sx = 0;
-      if constexpr (!SPLIT) {
+      if constexpr (!XSLAB) {
 #pragma unroll
         for (int i = 0; i < 4; i++) sx += c_bs[i].x + c_bs[i].y + c_bs[i].z + c_bs[i].w;
       }
       ilt_lds_st4_untracked(&S.xd[t], __builtin_bit_cast(u32, c_yd));
-      if constexpr (!SPLIT) ilt_lds_st4_untracked(&S.cx[t], (u32)(F::KCX * sx));
+      if constexpr (!XSLAB) ilt_lds_st4_untracked(&S.cx[t], (u32)(F::KCX * sx));
       if constexpr (FMT == ILT_Q4_K) {
         u32 h[2] = {0, 0}, l[2] = {0, 0};
 #pragma unroll
@@ -1113,7 +1116,7 @@ __global__ __launch_bounds__(512, 1) void gemm_i8p_kernel(BfParams p) {
 
   v16f sum[NA][1];
   v16i_ ah[SPLIT ? 2 : 1][NA], al[SPLIT ? 2 : 1][NA];
-  int xsum = 0;                                              // IQ2_XXS: see the step
+  int xsum = 0;                                              // IQ2_XXS, Q6_K: see the step
 #pragma unroll
   for (int a = 0; a < NA; a++)
 #pragma unroll
@@ -1160,15 +1163,16 @@ __global__ __launch_bounds__(512, 1) void gemm_i8p_kernel(BfParams p) {
     const u8* whs = S.wh[J & 1];
     const u8* wls = S.wl[J & 1];
     const v16i_ zero = {};
-    if constexpr (SPLIT) {
-      // the sums of the tokens' quants over the block's even and odd groups, from the slabs: thread t adds piece t & 3
-      // of token t / 4; pieces 0 and 1 are the step's even group, 2 and 3 its odd one
+    if constexpr (XSLAB) {
+      // the sums of the tokens' quants over the block (IQ2_XXS: over its even and its odd groups), from the slabs: thread t
+      // adds piece t & 3 of token t / 4; pieces 0 and 1 are the step's even group, 2 and 3 its odd one
       const int4 xv = ilt_lds_ld16(xs + slab_off(t >> 2, t & 3));
       int sp = __builtin_amdgcn_sdot4(xv.x, 0x01010101, 0, false);
       sp = __builtin_amdgcn_sdot4(xv.y, 0x01010101, sp, false);
       sp = __builtin_amdgcn_sdot4(xv.z, 0x01010101, sp, false);
       sp = __builtin_amdgcn_sdot4(xv.w, 0x01010101, sp, false);
       sp += __shfl_xor(sp, 1);
+      if constexpr (!SPLIT) sp += __shfl_xor(sp, 2);
       xsum = J == 0 ? sp : xsum + sp;
     }
 #pragma unroll
@@ -1197,10 +1201,10 @@ __global__ __launch_bounds__(512, 1) void gemm_i8p_kernel(BfParams p) {
         }
       }
     }
-    if constexpr (FMT == ILT_IQ2_XXS) {
+    if constexpr (XSLAB) {
       if (J == 3) {        // the block's sums of quants, for everyone's terms below
         if ((t & 3) == 0) ilt_lds_st4_untracked(&S.cx[t >> 2], (u32)(F::KCX * xsum));
-        if ((t & 3) == 2) ilt_lds_st4_untracked(&cxo[t >> 2], (u32)(F::KCX * xsum));
+        if (SPLIT && (t & 3) == 2) ilt_lds_st4_untracked(&cxo[t >> 2], (u32)(F::KCX * xsum));
         ilt_barrier_lds();
       }
     }
@@ -1901,11 +1905,11 @@ hipError_t ilt_k_planes_i8(int fmt, const uint8_t* w, long long row_bytes, int r
 }
 
 hipError_t ilt_k_gemm_i8_pp(const uint8_t* wh, const uint8_t* wl, const float* wdf, int rows, int cols, const int8_t* xq, const float* xd,
-                            const int* bsums, int ntok, float* y, const float* bias, int acc, hipStream_t st) {
+                            int ntok, float* y, const float* bias, int acc, hipStream_t st) {
   if (ntok <= 0 || rows <= 0) return hipSuccess;
   if (cols % 256 != 0 || (long long)rows * 1024 >= 0x7FFFFFFFLL || (long long)128 * cols >= 0x7FFFFFFFLL) return hipErrorInvalidValue;
   BfParams p = {};
-  p.w = wh; p.wlo = wl; p.wdf = wdf; p.rows = rows; p.cols = cols; p.row_bytes = cols; p.x = (const u16*)xq; p.xd = xd; p.bsums = bsums;
+  p.w = wh; p.wlo = wl; p.wdf = wdf; p.rows = rows; p.cols = cols; p.row_bytes = cols; p.x = (const u16*)xq; p.xd = xd;
   p.y = y; p.bias = bias; p.acc = acc; p.ntok = ntok; p.ldy = rows;
   const long long total = (long long)((ntok + 127) / 128) * ((rows + 127) / 128), per = (total + 7) / 8;
   if (per * 8 > 0x7FFFFFFFLL) return hipErrorInvalidValue;

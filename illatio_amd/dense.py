@@ -196,7 +196,7 @@ def mat_mul_i8_planes(dev, planes, rows, cols, act, y, n, bias=None, acc=False):
     CMAT-MUL's bits without dequantizing W again."""
     wh, wl, wdf = planes
     hip.launch(dev, "mm_i8_planes", ((n + 127) // 128, (rows + 127) // 128), 512,
-               [wh, wl, wdf, act.kq, act.kd, act.ksum, y, bias, rows, cols, n, 1 if acc else 0])
+               [wh, wl, wdf, act.kq, act.kd, y, bias, rows, cols, n, 1 if acc else 0])
     return y
 
 

@@ -294,10 +294,10 @@ int ilt_mm_bf16(uint64_t stream, const uint16_t* wb, const uint16_t* xb, float* 
 /* The exact product in two passes (no counterpart in the reference: its GPU prefill does not have the CPU
    path's bits): planes_i8 writes a Q6_K matrix as the two int8 planes of scale * (quant - 32) (slabs of 128
    rows x 64 columns: ceil(rows/128)*128*cols bytes each) and d per row and super-block as floats (rows * cols / 256); mm_i8_planes is mm_k from
-   those, bit for bit, for a matrix multiplied again and again or by thousands of tokens. */
+   those and the Q8_K quants and scales (it adds the quants up itself: no sums of 16), bit for bit, for a matrix multiplied again and again or by thousands of tokens. */
 int ilt_planes_i8(uint64_t stream, int gguf_type, const void* w, int8_t* wh, int8_t* wl, float* wdf, int rows, int cols);
 int ilt_mm_i8_planes(uint64_t stream, const int8_t* wh, const int8_t* wl, const float* wdf, const int8_t* xq, const float* xd,
-                     const int32_t* bsums, float* y, const float* bias, int rows, int cols, int n, int acc);
+                     float* y, const float* bias, int rows, int cols, int n, int acc);
 int ilt_d4_mm_id_bf16(uint64_t stream, int gguf_type, int ncols, int nrows, int row_bytes, int64_t add, const uint64_t* ptrs,
                       const uint32_t* counts, const uint32_t* bases, int ne, int64_t total_rows,
                       const uint16_t* xb, const uint32_t* rmap, float* y);
