@@ -102,6 +102,44 @@ def test_dense_bf16_product_within_tolerance(dev, monkeypatch, qtype, rows, cols
     m.free()
 
 
+@pytest.mark.parametrize("two_pass", [False, True])
+def test_output_head_keeps_the_cpu_paths_top_token(dev, two_pass):
+    """128 positions through an output head (Q6_K, config 2's width, 8192 of its rows): the
+    bf16 product picks the CPU path's token at every position, except where the CPU path's
+    own two best logits lie closer than 5 % of the position's logit spread -- the near-tie
+    rule of the reference's consistency checks (cuda-consistency-test.lisp:20-22,
+    vectors-test.lisp:26-27); the two paths' difference between two logits has an rms of
+    1.6 % of the spread, most of it the CPU path's quantized activations -- and at 90 % of
+    the positions at least (ds4f-vectors-test.lisp:30-32)."""
+    from illatio_amd import dense, hip
+    rows, cols, n = 8192, 2560, 128
+    rng = synth.make_rng(4242)
+    w = synth.weights(synth.Q6_K, rows, cols, rng)
+    x = synth.activations((n, cols), rng)
+    m = upload(dev, synth.Q6_K, rows, cols, w)
+    xf, y = hip.hip_upload_new(dev, x), hip.hip_alloc(dev, 4 * n * rows)
+    if two_pass:
+        wb = dense.dequant_bf16(dev, m)
+        xs = dense.cvt_bf16_slabs(dev, xf, n, cols)
+        dense.mat_mul_bf16(dev, wb, rows, cols, xs, y, n)
+        tmp = (wb, xs)
+    else:
+        xb = dense.cvt_bf16(dev, xf, x.size)
+        dense.cmat_mul_bf16(dev, m, xb, y, n)
+        tmp = (xb,)
+    got = hip.hip_floats(y, n * rows).reshape(n, rows)
+    cpu = orc.matmul(synth.Q6_K, w, rows, cols, x, nthreads=16)
+    top, mine = cpu.argmax(1), got.argmax(1)
+    best2 = np.sort(cpu, axis=1)[:, -2:]
+    near_tie = (best2[:, 1] - best2[:, 0]) < 0.05 * cpu.std(axis=1)
+    differ = top != mine
+    assert not np.any(differ & ~near_tie), (np.argwhere(differ & ~near_tie).ravel(), near_tie.sum())
+    assert differ.sum() <= n // 10, differ.sum()
+    for b in (xf, y) + tmp:
+        hip.hip_free(b)
+    m.free()
+
+
 def exact_chunk(G, U, Dn, sel, ww, norms, clamp):
     """The routed experts of a chunk in double precision from the dequantized weights and
     the float activations (no activation quantization, no bf16): what both paths approximate."""
