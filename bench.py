@@ -41,7 +41,7 @@ sys.path.insert(0, ROOT)
 sys.path.insert(0, os.path.join(ROOT, "tests"))
 
 # HBM bytes per launch of the product kernels, from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE
-# (KiB per dispatch; profiles/traffic_*.txt): FETCH_SIZE reads 0.500 of what a plain streaming
+# (KiB per dispatch; the tables at the end of each file under profiles/): FETCH_SIZE reads 0.500 of what a plain streaming
 # kernel of known size fetches (cvt_bf16: 83,886,080 bytes read, counter 40,971 KiB), WRITE_SIZE
 # reads 1.000 (same kernel: 41,943,040 bytes written, counter 40,960 KiB); so bytes =
 # (2 * FETCH_SIZE + WRITE_SIZE) * 1024.
@@ -54,10 +54,11 @@ TRAFFIC = {"c1": {"up": _t(2507.3, 96.0), "down": _t(2443.0, 28.0)},
                   "head": _t(175546.1, 636.4)},
            # one product: two-pass = the 256-tile launch plus the 128-tile launch for the rows left over
            "c3": {"bf16-1pass": _t(519803.0, 278528.0), "bf16-2pass": _t(491863.8 + 61498.0, 262144.0 + 16384.0),
-                  "bf16-resident": _t(491863.8 + 61498.0, 262144.0 + 16384.0), "int8": _t(510205.6, 278528.0)},
+                  "bf16-resident": _t(491863.8 + 61498.0, 262144.0 + 16384.0), "int8": _t(466661.6, 278528.0),
+                  "int8-2pass": _t(941922.8, 278528.0), "int8-resident": _t(941922.8, 278528.0)},
            "c4": {"d4_mv_glu_iq2_xxs": _t(12854.8, 96.0), "d4_mv_q2_k_f32": _t(8394.5, 96.0), "d4_mvq8_glu": _t(8833.8, 96.0)},
            # per launch, over the step's two grouped launches (gate + up + activation; down)
-           "c5": {"mm_id": _t((569198.8 + 334480.4) / 2, (98304.6 + 393216.0) / 2)}}
+           "c5": {"mm_id": _t((578091.8 + 335996.1) / 2, (98304.6 + 393216.0) / 2)}}
 
 
 def traffic_of(workload, per):
@@ -383,7 +384,7 @@ def workload_c3(args, dev):
     ms, dev_ms, per = tm.run(step, args.steps, args.warmup)
     roof = roofline_of({k: v for k, v in per.items() if k == "mm"}, "mfma", MFMA_PEAK_TFLOPS[args.path], "TFLOP/s" if bf16_path else "TOP/s", names)
     roof["unit"] = "TFLOP/s"
-    if path in TRAFFIC["c3"] and T == 4096 and not args.transpose:
+    if path in TRAFFIC["c3"] and T == 4096 and not args.transpose and args.qtype == "q6_k":
         roof["traffic"] = TRAFFIC["c3"][path]
     tf = flops / (ms * 1e-3) / 1e12
 
@@ -586,7 +587,7 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU; --gpus N with N above 1 is not supported "
-              "(the path shards by rows / by experts, see DESIGN.md)", file=sys.stderr)
+              "(the path would shard by rows of a matrix and by experts; nothing here uses a second GPU)", file=sys.stderr)
         return 2
 
     from illatio_amd import hip

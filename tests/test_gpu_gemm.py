@@ -110,6 +110,33 @@ def test_two_pass_exact_product_bit_for_bit(dev, rows, cols, n):
     act.free(); m.free()
 
 
+def test_products_of_no_tokens_write_nothing(dev):
+    """No tokens (an empty chunk): every prefill product returns without touching y."""
+    from illatio_amd import dense, hip
+    rows, cols = 256, 512
+    rng = synth.make_rng(5)
+    mark = synth.activations(4 * rows, rng)
+    y = hip.hip_upload_new(dev, mark)
+    for qtype in (synth.Q8_0, synth.Q4_K, synth.Q6_K):
+        m = dense.upload_gmat(dev, "w", qtype, rows, cols, synth.weights(qtype, rows, cols, rng))
+        act = dense.QAct(dev, 4, cols, ("q8",) if qtype == synth.Q8_0 else ("q8k",))
+        dense.cmat_mul(dev, m, act, y, n=0)
+        if qtype != synth.Q8_0:
+            xb = hip.hip_alloc(dev, 2 * 4 * cols)
+            dense.cmat_mul_bf16(dev, m, xb, y, 0)
+            wb = dense.dequant_bf16(dev, m)
+            dense.mat_mul_bf16(dev, wb, rows, cols, xb, y, 0)
+            hip.hip_free(xb); hip.hip_free(wb)
+        if qtype == synth.Q6_K:
+            planes = dense.planes_i8(dev, m)
+            dense.mat_mul_i8_planes(dev, planes, rows, cols, act, y, 0)
+            for b in planes:
+                hip.hip_free(b)
+        act.free(); m.free()
+    assert np.array_equal(bits(hip.hip_floats(y, 4 * rows)), bits(mark))
+    hip.hip_free(y)
+
+
 @pytest.mark.parametrize("ne,d,ff,nu,n,clamp", [(8, 512, 256, 3, 37, 0.0), (16, 1024, 512, 4, 150, 0.6),
                                                  (12, 4096, 2048, 6, 96, 0.0)])
 @pytest.mark.parametrize("planes", [None, "0", "1"])        # the down product (Q2_K) on the 64 x 64 kernel / on the planes kernel
