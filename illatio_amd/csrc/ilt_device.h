@@ -57,6 +57,16 @@ __device__ __forceinline__ int ilt_dot16(const int4& a, const int4& b, int c) {
   c = ilt_dot4(a.x, b.x, c); c = ilt_dot4(a.y, b.y, c); c = ilt_dot4(a.z, b.z, c); return ilt_dot4(a.w, b.w, c);
 }
 
+// a * b and a * b + c for a and b that fit 24 bits (signed), at the full rate; a 32-bit multiply takes
+// four times as long.  The operands' sign extension from bit 23 is written out: it shows the compiler
+// that v_mul_i32_i24 / v_mad_i32_i24 will do, and it goes away where the range is known (known within the
+// basic block: an operand that comes out of a branch has lost its range, and the multiply is a 32-bit one
+// again).  Not inline assembly: the compiler puts the wait states that a dot instruction's result needs
+// before its own instructions only.
+__device__ __forceinline__ int ilt_s24(int a) { return (a << 8) >> 8; }
+__device__ __forceinline__ int ilt_mul24(int a, int b) { return ilt_s24(a) * ilt_s24(b); }
+__device__ __forceinline__ int ilt_mad24(int a, int b, int c) { return ilt_s24(a) * ilt_s24(b) + c; }
+
 // Address spaces spelled out.  A pointer rebuilt from an integer (an expert's slot
 // address), or carried through a struct, is "generic" to the compiler; generic loads are
 // FLAT instructions, which count against the LDS counter as well as the memory counter and
@@ -68,15 +78,19 @@ __device__ __forceinline__ int ilt_dot16(const int4& a, const int4& b, int c) {
 typedef int ilt_v4i __attribute__((ext_vector_type(4)));
 typedef int ilt_v2i __attribute__((ext_vector_type(2)));
 typedef float ilt_v2f __attribute__((ext_vector_type(2)));
+// (The pointer goes through its low 32 bits -- a generic pointer into LDS holds the LDS address there --
+// because a cast from generic to LDS proper first compares the pointer with null: two more
+// instructions on 64-bit values per address, in loops that are bound by their instruction count.)
+#define ILT_LDS_PTR(T, p) ((ILT_LDS T*)(unsigned long long)(unsigned)(unsigned long long)(p))
 __device__ __forceinline__ int4 ilt_lds_ld16(const void* p) {
-  const ilt_v4i v = *(const ILT_LDS ilt_v4i*)p; return make_int4(v.x, v.y, v.z, v.w);
+  const ilt_v4i v = *ILT_LDS_PTR(const ilt_v4i, p); return make_int4(v.x, v.y, v.z, v.w);
 }
 __device__ __forceinline__ int2 ilt_lds_ld8(const void* p) {
-  const ilt_v2i v = *(const ILT_LDS ilt_v2i*)p; return make_int2(v.x, v.y);
+  const ilt_v2i v = *ILT_LDS_PTR(const ilt_v2i, p); return make_int2(v.x, v.y);
 }
-__device__ __forceinline__ float ilt_lds_ldf(const void* p) { return *(const ILT_LDS float*)p; }
-__device__ __forceinline__ void ilt_lds_stf(void* p, float v) { *(ILT_LDS float*)p = v; }
-__device__ __forceinline__ void ilt_lds_stf2(void* p, float a, float b) { ilt_v2f v = {a, b}; *(ILT_LDS ilt_v2f*)p = v; }
+__device__ __forceinline__ float ilt_lds_ldf(const void* p) { return *ILT_LDS_PTR(const float, p); }
+__device__ __forceinline__ void ilt_lds_stf(void* p, float v) { *ILT_LDS_PTR(float, p) = v; }
+__device__ __forceinline__ void ilt_lds_stf2(void* p, float a, float b) { ilt_v2f v = {a, b}; *ILT_LDS_PTR(ilt_v2f, p) = v; }
 
 // Global loads that may be only 2-byte aligned (GGUF blocks of 34, 66, 84 and 210 bytes are
 // not 16-byte multiples); gfx950 performs them in hardware.

@@ -133,23 +133,24 @@ template <> __device__ __forceinline__ void block_terms<ILT_Q8_0>(const Raw<ILT_
 }
 
 template <> __device__ __forceinline__ void block_terms<ILT_Q4_K>(const Raw<ILT_Q4_K>& r, int s, int j, const Lds& L, float* t) {
-  const i8* xb = L.xq + s * XP + 64 * j;
+  const i8* xb = L.xq + ilt_mul24(s, XP) + 64 * j;
   int lo = ilt_dot16(and4(r.qa, 0x0F0F0F0F), ilt_lds_ld16(xb), 0);
   lo = ilt_dot16(and4(r.qb, 0x0F0F0F0F), ilt_lds_ld16(xb + 16), lo);
   int hi = ilt_dot16(and4(shr4(r.qa, 4), 0x0F0F0F0F), ilt_lds_ld16(xb + 32), 0);
   hi = ilt_dot16(and4(shr4(r.qb, 4), 0x0F0F0F0F), ilt_lds_ld16(xb + 48), hi);
-  // get_scale_min_k4 for groups 2j and 2j+1 at once, on 16-bit fields of the 12 scale bytes
+  // get_scale_min_k4 for groups 2j and 2j+1 at once, on the two bytes of a 16-bit field of the 12 scale
+  // bytes, without a branch: groups 0..3 take six bits of a byte, groups 4..7 a nibble and two top bits
   const int sh = 16 * (j & 1);
-  const u32 a = ((u32)r.hdr.y >> sh) & 0xFFFF, b = ((u32)r.hdr.z >> sh) & 0xFFFF, c = ((u32)r.hdr.w >> sh) & 0xFFFF;
-  int sc0, sc1, m0, m1;
-  if (j < 2) { sc0 = a & 63; sc1 = (a >> 8) & 63; m0 = b & 63; m1 = (b >> 8) & 63; }
-  else {
-    sc0 = (c & 0xF) | (((a >> 6) & 3) << 4); sc1 = ((c >> 8) & 0xF) | (((a >> 14) & 3) << 4);
-    m0 = ((c >> 4) & 0xF) | (((b >> 6) & 3) << 4); m1 = ((c >> 12) & 0xF) | (((b >> 14) & 3) << 4);
-  }
+  const u32 a = (u32)r.hdr.y >> sh, b = (u32)r.hdr.z >> sh, c = (u32)r.hdr.w >> sh;
+  // (both forms computed and one taken by a mask: a branch here would hide the values' ranges from the
+  // multiplies below, which then would not be the 24-bit ones)
+  const u32 upper = j < 2 ? 0u : 0xFFFFFFFFu;
+  const u32 sc = ((a & 0x3F3F) & ~upper) | (((c & 0x0F0F) | ((a >> 2) & 0x3030)) & upper);
+  const u32 mn = ((b & 0x3F3F) & ~upper) | ((((c >> 4) & 0x0F0F) | ((b >> 2) & 0x3030)) & upper);
   const int4 bs = ilt_lds_ld16(L.bsums + s * 16 + 4 * j);
-  const int isum = ilt_sum4(lo * sc0 + hi * sc1);
-  const int imin = ilt_sum4(m0 * (bs.x + bs.y) + m1 * (bs.z + bs.w));
+  // 24-bit multiplies (full rate): a group's dot is at most 32 * 15 * 128, two sums of 16 at most 32 * 127
+  const int isum = ilt_sum4(ilt_mad24(lo, (int)(sc & 0xFF), ilt_mul24(hi, (int)(sc >> 8))));
+  const int imin = ilt_sum4(ilt_mad24((int)(mn & 0xFF), bs.x + bs.y, ilt_mul24((int)(mn >> 8), bs.z + bs.w)));
   if (j == 0) {
     const float ydi = ilt_lds_ldf(L.xs + s);
     const float d = ydi * ilt_h2f((u16)(r.hdr.x & 0xFFFF)), dmin = ydi * ilt_h2f((u16)((u32)r.hdr.x >> 16));
@@ -159,7 +160,7 @@ template <> __device__ __forceinline__ void block_terms<ILT_Q4_K>(const Raw<ILT_
 
 template <> __device__ __forceinline__ void block_terms<ILT_Q6_K>(const Raw<ILT_Q6_K>& r, int s, int j, const Lds& L, float* t) {
   const int c = j >> 1, pp = j & 1;
-  const i8* xb = L.xq + s * XP + 128 * c + 32 * pp;
+  const i8* xb = L.xq + ilt_mul24(s, XP) + 128 * c + 32 * pp;
   const int s0 = 2 * pp, s1 = 2 * pp + 4;
   // low nibbles: weights 128c + 32pp + l; high nibbles: the same + 64 (l = 0..31)
   const int4 lo0 = or_shl4(and4(r.ql0, 0x0F0F0F0F), shr4(r.qh0, s0), 0x03030303, 4);
@@ -170,12 +171,13 @@ template <> __device__ __forceinline__ void block_terms<ILT_Q6_K>(const Raw<ILT_
   const int dh0 = ilt_dot16(hi0, ilt_lds_ld16(xb + 64), 0), dh1 = ilt_dot16(hi1, ilt_lds_ld16(xb + 80), 0);
   // int8 scales: groups 8c+2pp+{0,1} for the low nibbles, 8c+4+2pp+{0,1} for the high
   const u32 wl = (u32)(c ? r.sc.z : r.sc.x) >> (16 * pp), wh = (u32)(c ? r.sc.w : r.sc.y) >> (16 * pp);
-  int isum = dl0 * (int)(i8)(wl & 0xFF) + dl1 * (int)(i8)((wl >> 8) & 0xFF);
-  isum += dh0 * (int)(i8)(wh & 0xFF) + dh1 * (int)(i8)((wh >> 8) & 0xFF);
+  // (24-bit multiplies, full rate: a dot of 16 is at most 16 * 63 * 128, a sum of 16 at most 16 * 128)
+  int isum = ilt_mad24(dl0, (int)(i8)(wl & 0xFF), ilt_mul24(dl1, (int)(i8)((wl >> 8) & 0xFF)));
+  isum = ilt_mad24(dh0, (int)(i8)(wh & 0xFF), ilt_mad24(dh1, (int)(i8)((wh >> 8) & 0xFF), isum));
   const u32 wj = (u32)sel4(r.sc, j);
   const int4 bs = ilt_lds_ld16(L.bsums + s * 16 + 4 * j);
-  int imins = bs.x * (int)(i8)(wj & 0xFF) + bs.y * (int)(i8)((wj >> 8) & 0xFF);
-  imins += bs.z * (int)(i8)((wj >> 16) & 0xFF) + bs.w * (int)(i8)(wj >> 24);
+  int imins = ilt_mad24(bs.x, (int)(i8)(wj & 0xFF), ilt_mul24(bs.y, (int)(i8)((wj >> 8) & 0xFF)));
+  imins = ilt_mad24(bs.z, (int)(i8)((wj >> 16) & 0xFF), ilt_mad24(bs.w, (int)(i8)(wj >> 24), imins));
   isum = ilt_sum4(isum);
   imins = ilt_sum4(imins);
   if (j == 0) ilt_lds_stf(t, (ilt_h2f(r.d) * ilt_lds_ldf(L.xs + s)) * (float)(isum - 32 * imins));
@@ -183,19 +185,19 @@ template <> __device__ __forceinline__ void block_terms<ILT_Q6_K>(const Raw<ILT_
 
 template <> __device__ __forceinline__ void block_terms<ILT_Q2_K>(const Raw<ILT_Q2_K>& r, int s, int j, const Lds& L, float* t) {
   const int h = j >> 1, half = j & 1;
-  const i8* xb = L.xq + s * XP + 128 * h + 16 * half;
+  const i8* xb = L.xq + ilt_mul24(s, XP) + 128 * h + 16 * half;
   const u32 wa = (u32)(h ? r.sb.z : r.sb.x) >> (8 * half), wb = (u32)(h ? r.sb.w : r.sb.y) >> (8 * half);
   int isum = 0;
 #pragma unroll
   for (int k = 0; k < 4; k++) {
     const int dot = ilt_dot16(and4(shr4(r.q, 2 * k), 0x03030303), ilt_lds_ld16(xb + 32 * k), 0);
     const u32 sw = ((k < 2 ? wa : wb) >> (16 * (k & 1))) & 0xF;
-    isum += (int)sw * dot;
+    isum = ilt_mad24((int)sw, dot, isum);
   }
   const u32 wj = (u32)sel4(r.sb, j);
   const int4 bs = ilt_lds_ld16(L.bsums + s * 16 + 4 * j);
-  int mins = (int)((wj >> 4) & 0xF) * bs.x + (int)((wj >> 12) & 0xF) * bs.y;
-  mins += (int)((wj >> 20) & 0xF) * bs.z + (int)(wj >> 28) * bs.w;
+  int mins = ilt_mad24((int)((wj >> 4) & 0xF), bs.x, ilt_mul24((int)((wj >> 12) & 0xF), bs.y));
+  mins = ilt_mad24((int)((wj >> 20) & 0xF), bs.z, ilt_mad24((int)(wj >> 28), bs.w, mins));
   isum = ilt_sum4(isum);
   mins = ilt_sum4(mins);
   if (j == 0) {
@@ -206,7 +208,7 @@ template <> __device__ __forceinline__ void block_terms<ILT_Q2_K>(const Raw<ILT_
 }
 
 template <> __device__ __forceinline__ void block_terms<ILT_IQ2_XXS>(const Raw<ILT_IQ2_XXS>& r, int s, int j, const Lds& L, float* t) {
-  const i8* xb = L.xq + s * XP + 64 * j;
+  const i8* xb = L.xq + ilt_mul24(s, XP) + 64 * j;
   const u32 aux0 = (u32)r.q.y, aux1 = (u32)r.q.w;
   const float te = (float)iq2xxs_sub_dot((u32)r.q.x, aux0, xb, L.grid) * (0.5f + (float)(aux0 >> 28));
   const float to = (float)iq2xxs_sub_dot((u32)r.q.z, aux1, xb + 32, L.grid) * (0.5f + (float)(aux1 >> 28));
@@ -774,11 +776,16 @@ __device__ __forceinline__ void wave_rows_lds(const u8* run, const u8* run2, int
   constexpr int GPW = ILT_WAVE / F::LPB;
   const int j = lane % F::LPB, gl = lane / F::LPB;
   const int nblk = nrows * S;
+  // the block's place in its row, f mod S, kept by addition (a division by multiplication takes two
+  // quarter-rate instructions a step)
+  const int step = S > 1 ? GPW - (int)__umulhi((u32)GPW, s_magic) * S : 0;      // GPW mod S
+  int s_ = S > 1 ? gl - (int)__umulhi((u32)gl, s_magic) * S : 0;
   for (int f = gl; f < nblk; f += GPW) {
     Raw<FMT> r;
     load_raw_lds<FMT>(r, run, run2, f, j);
-    const int s_ = S > 1 ? f - (int)__umulhi((u32)f, s_magic) * S : 0;
     block_terms<FMT>(r, s_, j, L, t + (long)f * F::TERMS);
+    s_ += step;
+    if (s_ >= S) s_ -= S;
   }
 }
 
