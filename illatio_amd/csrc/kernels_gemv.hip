@@ -51,10 +51,17 @@ __device__ __forceinline__ int4 and4(const int4& v, int m) { return make_int4(v.
 __device__ __forceinline__ int4 shr4(const int4& v, int n) {
   return make_int4((u32)v.x >> n, (u32)v.y >> n, (u32)v.z >> n, (u32)v.w >> n);
 }
-__device__ __forceinline__ int4 or_shl4(const int4& a, const int4& b, int m, int n) {   // a | ((b & m) << n)
-  return make_int4(a.x | ((b.x & m) << n), a.y | ((b.y & m) << n), a.z | ((b.z & m) << n), a.w | ((b.w & m) << n));
+// (two levels of selects, no chain of comparisons: that one becomes branches)
+__device__ __forceinline__ int sel4(const int4& v, int i) {
+  const int even = (i & 2) ? v.z : v.x, odd = (i & 2) ? v.w : v.y;
+  return (i & 1) ? odd : even;
 }
-__device__ __forceinline__ int sel4(const int4& v, int i) { return i == 0 ? v.x : i == 1 ? v.y : i == 2 ? v.z : v.w; }
+__device__ __forceinline__ int4 shl4(const int4& v, int n) {
+  return make_int4((int)((u32)v.x << n), (int)((u32)v.y << n), (int)((u32)v.z << n), (int)((u32)v.w << n));
+}
+__device__ __forceinline__ int4 or_and4(const int4& a, const int4& b, int m) {           // a | (b & m)
+  return make_int4(a.x | (b.x & m), a.y | (b.y & m), a.z | (b.z & m), a.w | (b.w & m));
+}
 
 // ---- the raw bytes a lane needs for one block (issued early, consumed a step later) ------------
 template <int FMT> struct Raw;
@@ -111,14 +118,19 @@ __device__ __forceinline__ u64 iq2_sign_mask(u32 s7) {      // table entry s7 (0
   return ((u64)mhi << 32) | mlo;
 }
 __device__ __forceinline__ int iq2xxs_sub_dot(u32 g, u32 aux, const i8* xb, const u64* grid) {
+  // the eight table reads first, then the dots: read one by one, each dot waits out an LDS round trip
+  int2 mag[4], m[4];
+#pragma unroll
+  for (int l = 0; l < 4; l++) {
+    mag[l] = ilt_lds_ld8(grid + ((g >> (8 * l)) & 0xFF));
+    m[l] = ilt_lds_ld8(grid + 256 + ((aux >> (7 * l)) & 127));
+  }
   int pos = 0, neg = 0;
 #pragma unroll
   for (int l = 0; l < 4; l++) {
-    const int2 mag = ilt_lds_ld8(grid + ((g >> (8 * l)) & 0xFF));
-    const int2 m = ilt_lds_ld8(grid + 256 + ((aux >> (7 * l)) & 127));
     const int2 x = ilt_lds_ld8(xb + 8 * l);
-    pos = ilt_dot4((int)mag.y, x.y, ilt_dot4((int)mag.x, x.x, pos));
-    neg = ilt_dot4((int)(mag.y & m.y), x.y, ilt_dot4((int)(mag.x & m.x), x.x, neg));
+    pos = ilt_dot4((int)mag[l].y, x.y, ilt_dot4((int)mag[l].x, x.x, pos));
+    neg = ilt_dot4((int)(mag[l].y & m[l].y), x.y, ilt_dot4((int)(mag[l].x & m[l].x), x.x, neg));
   }
   return pos - 2 * neg;
 }
@@ -161,12 +173,15 @@ template <> __device__ __forceinline__ void block_terms<ILT_Q4_K>(const Raw<ILT_
 template <> __device__ __forceinline__ void block_terms<ILT_Q6_K>(const Raw<ILT_Q6_K>& r, int s, int j, const Lds& L, float* t) {
   const int c = j >> 1, pp = j & 1;
   const i8* xb = L.xq + ilt_mul24(s, XP) + 128 * c + 32 * pp;
-  const int s0 = 2 * pp, s1 = 2 * pp + 4;
+  const int s0 = 2 * pp;                  // (and s1 = s0 + 4)
   // low nibbles: weights 128c + 32pp + l; high nibbles: the same + 64 (l = 0..31)
-  const int4 lo0 = or_shl4(and4(r.ql0, 0x0F0F0F0F), shr4(r.qh0, s0), 0x03030303, 4);
-  const int4 lo1 = or_shl4(and4(r.ql1, 0x0F0F0F0F), shr4(r.qh1, s0), 0x03030303, 4);
-  const int4 hi0 = or_shl4(and4(shr4(r.ql0, 4), 0x0F0F0F0F), shr4(r.qh0, s1), 0x03030303, 4);
-  const int4 hi1 = or_shl4(and4(shr4(r.ql1, 4), 0x0F0F0F0F), shr4(r.qh1, s1), 0x03030303, 4);
+  // the two top bits of a quant are bits s0, s0 + 1 (low nibbles) and s1, s1 + 1 (high) of its qh byte: one shift
+  // by 4 - s0 to the left, or by s1 - 4 = s0 to the right, brings them to bits 4 and 5 (what crosses into a
+  // neighbouring byte lands outside the mask)
+  const int4 lo0 = or_and4(and4(r.ql0, 0x0F0F0F0F), shl4(r.qh0, 4 - s0), 0x30303030);
+  const int4 lo1 = or_and4(and4(r.ql1, 0x0F0F0F0F), shl4(r.qh1, 4 - s0), 0x30303030);
+  const int4 hi0 = or_and4(and4(shr4(r.ql0, 4), 0x0F0F0F0F), shr4(r.qh0, s0), 0x30303030);
+  const int4 hi1 = or_and4(and4(shr4(r.ql1, 4), 0x0F0F0F0F), shr4(r.qh1, s0), 0x30303030);
   const int dl0 = ilt_dot16(lo0, ilt_lds_ld16(xb), 0), dl1 = ilt_dot16(lo1, ilt_lds_ld16(xb + 16), 0);
   const int dh0 = ilt_dot16(hi0, ilt_lds_ld16(xb + 64), 0), dh1 = ilt_dot16(hi1, ilt_lds_ld16(xb + 80), 0);
   // int8 scales: groups 8c+2pp+{0,1} for the low nibbles, 8c+4+2pp+{0,1} for the high
@@ -739,7 +754,7 @@ __device__ __forceinline__ int stream_run(const u8* w, long row0, int nrows, int
 template <int FMT> __device__ __forceinline__ void load_raw_lds(Raw<FMT>& r, const u8* run, const u8* run2, u32 f, int j);
 template <> __device__ __forceinline__ void load_raw_lds<ILT_Q8_0>(Raw<ILT_Q8_0>& r, const u8* run, const u8* run2, u32 f, int j) {
   r.q = ilt_lds_ld16(run + f * LdsBlk<ILT_Q8_0>::LB + 16 * j);
-  r.d = *(const ILT_LDS u16*)(run2 + 2 * f);
+  r.d = *ILT_LDS_PTR(const u16, run2 + 2 * f);
 }
 template <> __device__ __forceinline__ void load_raw_lds<ILT_Q4_K>(Raw<ILT_Q4_K>& r, const u8* run, const u8*, u32 f, int j) {
   const u8* b = run + f * LdsBlk<ILT_Q4_K>::LB;
@@ -755,18 +770,18 @@ template <> __device__ __forceinline__ void load_raw_lds<ILT_Q6_K>(Raw<ILT_Q6_K>
   r.qh0 = ilt_lds_ld16(b + 128 + 32 * c);
   r.qh1 = ilt_lds_ld16(b + 128 + 32 * c + 16);
   r.sc = ilt_lds_ld16(b + 192);
-  r.d = *(const ILT_LDS u16*)(b + 220);
+  r.d = *ILT_LDS_PTR(const u16, b + 220);
 }
 template <> __device__ __forceinline__ void load_raw_lds<ILT_IQ2_XXS>(Raw<ILT_IQ2_XXS>& r, const u8* run, const u8*, u32 f, int j) {
   const u8* b = run + f * LdsBlk<ILT_IQ2_XXS>::LB;
   r.q = ilt_lds_ld16(b + 16 * j);
-  r.d = *(const ILT_LDS u16*)(b + 64);
+  r.d = *ILT_LDS_PTR(const u16, b + 64);
 }
 template <> __device__ __forceinline__ void load_raw_lds<ILT_Q2_K>(Raw<ILT_Q2_K>& r, const u8* run, const u8*, u32 f, int j) {
   const u8* b = run + f * LdsBlk<ILT_Q2_K>::LB;
   r.q = ilt_lds_ld16(b + 16 + 16 * j);
   r.sb = ilt_lds_ld16(b);
-  r.dd = *(const ILT_LDS u32*)(b + 92);
+  r.dd = *ILT_LDS_PTR(const u32, b + 92);
 }
 
 // A wave's run of nrows*S blocks, in LDS: terms into t.
