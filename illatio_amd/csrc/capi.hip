@@ -435,6 +435,32 @@ int ilt_mm_q8(uint64_t stream, const int8_t* wq, const uint16_t* wd, const int8_
   return (int)ilt_k_gemm_i8(ILT_Q8_0, (const uint8_t*)wq, wd, cols, rows, cols, xq, xs, nullptr, n, y, bias, acc, S(stream));
 }
 
+int ilt_mm_q8_mma2(uint64_t stream, const int8_t* w0, const uint16_t* d0, float* y0, const float* b0, int rows0, const int8_t* w1,
+                   const uint16_t* d1, float* y1, const float* b1, int rows1, const int8_t* w2, const uint16_t* d2, float* y2,
+                   const float* b2, int rows2, const int8_t* xq, const float* xs, int cols, int n, int acc) {
+  // a matrix of no rows (or a null one) takes no part, as in the reference's grid
+  const int8_t* ws[3] = {w0, w1, w2}; const uint16_t* ds[3] = {d0, d1, d2}; float* ys[3] = {y0, y1, y2};
+  const float* bs[3] = {b0, b1, b2}; const int rows[3] = {rows0, rows1, rows2};
+  for (int i = 0; i < 3; i++) {
+    ILT_REQUIRE(rows[i] >= 0);
+    if (rows[i] == 0 || !ws[i]) continue;
+    const int e = ilt_mm_q8(stream, ws[i], ds[i], xq, xs, ys[i], bs[i], rows[i], cols, n, acc);
+    if (e != ILT_OK) return e;
+  }
+  return ILT_OK;
+}
+
+int ilt_d4_mvq8n(uint64_t stream, int rows, int cols, int group_rows, int ntok, int x_tstride, int y_tstride, const int8_t* wq,
+                 const uint16_t* wd, const int8_t* xq, const float* xs, float* y) {
+  ILT_REQUIRE(ntok >= 0 && ntok <= 9 && x_tstride >= 0 && x_tstride % 32 == 0 && y_tstride >= 0 && cols > 0 && cols % 32 == 0);
+  for (int t = 0; t < ntok; t++) {
+    const int e = ilt_d4_mvq8(stream, rows, cols, group_rows, wq, wd, xq + (long long)t * x_tstride, xs + (long long)t * x_tstride / 32,
+                              y + (long long)t * y_tstride);
+    if (e != ILT_OK) return e;
+  }
+  return ILT_OK;
+}
+
 int ilt_mm_k(uint64_t stream, int type, const void* w, const int8_t* xq, const float* xd, const int32_t* bsums, float* y,
              const float* bias, int rows, int cols, int n, int acc) {
   const int fmt = kquant_type(type);
@@ -579,6 +605,12 @@ int ilt_launch(const char* kernel, unsigned gx, unsigned gy, unsigned gz, unsign
   if (!strcmp(kernel, "mm_q8") || !strcmp(kernel, "mm_q8_mma"))
     return ilt_mm_q8(stream, a.ptr<ci8>(0), a.ptr<cu16>(1), a.ptr<ci8>(2), a.ptr<cf>(3), a.ptr<float*>(4), a.ptr<cf>(5),
                      a.i32(6), a.i32(7), a.i32(8), a.i32(9));
+  K("mm_q8_mma2")
+    return ilt_mm_q8_mma2(stream, a.ptr<ci8>(0), a.ptr<cu16>(1), a.ptr<float*>(2), a.ptr<cf>(3), a.i32(4), a.ptr<ci8>(5), a.ptr<cu16>(6),
+                          a.ptr<float*>(7), a.ptr<cf>(8), a.i32(9), a.ptr<ci8>(10), a.ptr<cu16>(11), a.ptr<float*>(12), a.ptr<cf>(13),
+                          a.i32(14), a.ptr<ci8>(15), a.ptr<cf>(16), a.i32(17), a.i32(18), a.i32(19));
+  K("d4_mvq8n") return ilt_d4_mvq8n(stream, a.i32(0), a.i32(1), a.i32(2), a.i32(3), a.i32(4), a.i32(5), a.ptr<ci8>(6), a.ptr<cu16>(7),
+                                    a.ptr<ci8>(8), a.ptr<cf>(9), a.ptr<float*>(10));
   K("mm_k") return ilt_mm_k(stream, a.i32(0), a.ptr<const void*>(1), a.ptr<ci8>(2), a.ptr<cf>(3), a.ptr<const int32_t*>(4),
                             a.ptr<float*>(5), a.ptr<cf>(6), a.i32(7), a.i32(8), a.i32(9), a.i32(10));
   if (!strcmp(kernel, "mm_q4k_mma") || !strcmp(kernel, "mm_q6k_mma"))

@@ -123,6 +123,12 @@ int ilt_mv_k(uint64_t stream, int type, const void* w, const int8_t* xq, const f
              const float* bias, int rows, int cols, int acc);
 int ilt_d4_mvq8(uint64_t stream, int rows, int cols, int group_rows, const int8_t* wq, const uint16_t* wd,
                 const int8_t* xq, const float* xs, float* y);
+/* d4_mvq8n (ds4f.cu:66; cuda-ds4f-prefill.lisp:89): d4_mvq8 for ntok <= 9 tokens (a speculative
+   step's): token t's quantized input at xq + t*x_tstride (its scales at xs + t*x_tstride/32, the
+   row's group g at + g*cols within it), its output at y + t*y_tstride; each token's sums are
+   decode's. */
+int ilt_d4_mvq8n(uint64_t stream, int rows, int cols, int group_rows, int ntok, int x_tstride, int y_tstride, const int8_t* wq,
+                 const uint16_t* wd, const int8_t* xq, const float* xs, float* y);
 
 /* Gate and up in one launch ending in swiglu! (model.lisp:364-378): out[r] =
    (g / (1 + exp(-g))) * u with g = gate[r].x, u = up[r].x, each the decode product's bits.
@@ -249,6 +255,12 @@ int ilt_mm_q8(uint64_t stream, const int8_t* wq, const uint16_t* wd, const int8_
               const float* bias, int rows, int cols, int n, int acc);
 int ilt_mm_k(uint64_t stream, int type, const void* w, const int8_t* xq, const float* xd, const int32_t* bsums, float* y,
              const float* bias, int rows, int cols, int n, int acc);
+/* mm_q8_mma2 (dense.cu:884; cuda-dense.lisp:215, 255-258): up to three Q8_0 matrices on the same
+   quantized tokens (Q, K, V of a prefill chunk) in one call; a matrix of no rows takes no part.
+   Each is ilt_mm_q8's product. */
+int ilt_mm_q8_mma2(uint64_t stream, const int8_t* w0, const uint16_t* d0, float* y0, const float* b0, int rows0, const int8_t* w1,
+                   const uint16_t* d1, float* y1, const float* b1, int rows1, const int8_t* w2, const uint16_t* d2, float* y2,
+                   const float* b2, int rows2, const int8_t* xq, const float* xs, int cols, int n, int acc);
 int ilt_d4_mm_id_iq2_xxs(uint64_t stream, int ncols, int nrows, int row_bytes, int64_t add, const uint64_t* ptrs,
                          const uint32_t* counts, const uint32_t* bases, int ne, int64_t total_rows,
                          const int8_t* xq, const float* xd, float* y);

@@ -110,6 +110,43 @@ def test_two_pass_exact_product_bit_for_bit(dev, rows, cols, n):
     act.free(); m.free()
 
 
+def test_mm_q8_mma2_three_matrices_on_the_same_tokens(dev):
+    """mm_q8_mma2 (dense.cu:884): Q, K and V of a prefill chunk in one call, each with mm_q8's (the
+    CPU matmul!'s) bits; a matrix of no rows takes no part."""
+    from illatio_amd import dense, hip
+    rng = synth.make_rng(515)
+    cols, n = 896, 70
+    shape = [896, 128, 136]
+    ws = [synth.weights(synth.Q8_0, r, cols, rng) for r in shape]
+    ms = [dense.upload_gmat(dev, f"w{i}", synth.Q8_0, r, cols, w) for i, (r, w) in enumerate(zip(shape, ws))]
+    x = synth.activations((n, cols), rng)
+    xb = hip.hip_upload_new(dev, x)
+    act = dense.QAct(dev, n, cols, ("q8",))
+    dense.quantize_act(dev, xb, act, n=n)
+    bias = [synth.activations(r, rng) for r in shape]
+    bbs = [hip.hip_upload_new(dev, b) for b in bias]
+    ys = [hip.hip_alloc(dev, 4 * n * r) for r in shape]
+    grid = ((n + 63) // 64, sum((r + 127) // 128 for r in shape))
+    hip.launch(dev, "mm_q8_mma2", grid, 256, [ms[0].qs, ms[0].d, ys[0], bbs[0], shape[0], ms[1].qs, ms[1].d, ys[1], None, shape[1],
+                                              ms[2].qs, ms[2].d, ys[2], bbs[2], shape[2], act.xq, act.xs, cols, n, 0])
+    want = [np.stack([orc.matmul(synth.Q8_0, w, r, cols, x[t]) for t in range(n)]) for w, r in zip(ws, shape)]
+    want[0] = want[0] + bias[0]; want[2] = want[2] + bias[2]
+    for i, r in enumerate(shape):
+        assert np.array_equal(bits(hip.hip_floats(ys[i], n * r)), bits(want[i].reshape(-1))), i
+    # the middle matrix absent, the others accumulated onto what is there
+    hip.launch(dev, "mm_q8_mma2", grid, 256, [ms[0].qs, ms[0].d, ys[0], None, shape[0], None, None, None, None, 0,
+                                              ms[2].qs, ms[2].d, ys[2], None, shape[2], act.xq, act.xs, cols, n, 1])
+    plain = [np.stack([orc.matmul(synth.Q8_0, w, r, cols, x[t]) for t in range(n)]) for w, r in zip(ws, shape)]
+    assert np.array_equal(bits(hip.hip_floats(ys[0], n * shape[0])), bits((want[0] + plain[0]).reshape(-1)))
+    assert np.array_equal(bits(hip.hip_floats(ys[1], n * shape[1])), bits(want[1].reshape(-1)))
+    assert np.array_equal(bits(hip.hip_floats(ys[2], n * shape[2])), bits((want[2] + plain[2]).reshape(-1)))
+    for b in [xb] + bbs + ys:
+        hip.hip_free(b)
+    act.free()
+    for m in ms:
+        m.free()
+
+
 def test_products_of_no_tokens_write_nothing(dev):
     """No tokens (an empty chunk): every prefill product returns without touching y."""
     from illatio_amd import dense, hip

@@ -198,6 +198,39 @@ def test_indexed_expert_gemv_bit_for_bit(dev, qtype, rows, cols):
     hip.hip_free(pool); hip.hip_free(ptrs)
 
 
+def test_d4_mvq8n_tokens_of_a_speculative_step(dev):
+    """d4_mvq8n (ds4f.cu:66-107): up to nine tokens through the grouped Q8_0 product, token t's
+    input x_tstride and output y_tstride apart, each token's sums decode's; no tokens write nothing."""
+    from illatio_amd import hip
+    rng = synth.make_rng(79)
+    rows, cols, groups, ntok = 192, 512, 2, 9
+    xts, yts = groups * cols + 64, rows + 5                      # strides wider than a token's data
+    w = synth.weights(synth.Q8_0, rows, cols, rng)
+    x = np.zeros((ntok, xts), np.float32)
+    x[:, :groups * cols] = synth.activations((ntok, groups * cols), rng)
+    m = upload(dev, synth.Q8_0, rows, cols, w)
+    xb = hip.hip_upload_new(dev, x)
+    q, s = hip.hip_alloc(dev, ntok * xts), hip.hip_alloc(dev, 4 * ntok * xts // 32)
+    y = hip.hip_upload_new(dev, np.full(ntok * yts, 7.0, np.float32))
+    hip.launch(dev, "d4_quant", (ntok * xts + 255) // 256, 256, [xb, q, s, ntok * xts // 32])
+    hip.launch(dev, "d4_mvq8n", (rows + 3) // 4, 128, [rows, cols, rows // groups, 0, xts, yts, m.qs, m.d, q, s, y])
+    assert np.all(hip.hip_floats(y, ntok * yts) == 7.0)
+    for nt in (1, ntok):
+        hip.launch(dev, "d4_mvq8n", (rows + 3) // 4, 128, [rows, cols, rows // groups, nt, xts, yts, m.qs, m.d, q, s, y])
+        got = hip.hip_floats(y, ntok * yts).reshape(ntok, yts)
+        gr = rows // groups
+        for t in range(nt):
+            for g in range(groups):
+                want = orc.matmul(synth.Q8_0, w[g * gr:(g + 1) * gr], gr, cols, x[t, g * cols:(g + 1) * cols], f16_scale=False)
+                assert np.array_equal(bits(got[t, g * gr:(g + 1) * gr]), bits(want)), (nt, t, g)
+        assert np.all(got[:, rows:] == 7.0) and np.all(got[nt:] == 7.0)
+    with pytest.raises(hip.HipError):
+        hip.launch(dev, "d4_mvq8n", (rows + 3) // 4, 128, [rows, cols, rows // groups, 10, xts, yts, m.qs, m.d, q, s, y])
+    for b in (xb, q, s, y):
+        hip.hip_free(b)
+    m.free()
+
+
 def test_invalid_arguments_are_errors_not_faults(dev):
     from illatio_amd import hip
     b = hip.hip_alloc(dev, 4096)
