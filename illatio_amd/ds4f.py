@@ -187,6 +187,46 @@ def ffn_step_device(dev, pool, sh, logits, norm2, ne, nu, scale, clamp, bias=Non
     return moe
 
 
+def ffn_small(dev, pool, sh, logits, norm2, n, ne, nu, scale, clamp, bias=None):
+    """The FFN past the router for a short pass's N <= 9 tokens (DK-FFN-SMALL,
+    cuda-ds4f-spec.lisp:30-100: a speculative step's verification), every token with decode's
+    bits.  The reference routes on the CPU and hands each expert its tokens' rows through
+    counts/bases; here d4_route leaves sel and the weights on the device and the expert
+    kernels take one slot per (token, slot) row, row t*nu + j on expert sel[t*nu + j]: the
+    gathered rows, gate+up+gated activation of all rows in one launch, their downs in one, the
+    sums in slot order with the shared expert's (d4_mvq8n for its three products).  Returns
+    MOE (N x d)."""
+    d, ff = pool.d, pool.ff
+    rows = n * nu
+    gb = pool.gate_bytes
+    A = hip.hip_alloc
+    # the shared expert on the N tokens
+    qn_q, qn_s = A(dev, n * d), A(dev, 4 * n * d // 32)
+    sg, su, smid = (A(dev, 4 * n * ff) for _ in range(3))
+    qm_q, qm_s = A(dev, n * ff), A(dev, 4 * n * ff // 32)
+    sout = A(dev, 4 * n * d)
+    one = hip.hip_upload_new(dev, np.ones(n, np.float32))
+    hip.launch(dev, "d4_quant", (n * d + 255) // 256, 256, [norm2, qn_q, qn_s, n * d // 32])
+    hip.launch(dev, "d4_mvq8n", (ff + 3) // 4, 128, [ff, d, ff, n, d, ff, sh.gate.qs, sh.gate.d, qn_q, qn_s, sg])
+    hip.launch(dev, "d4_mvq8n", (ff + 3) // 4, 128, [ff, d, ff, n, d, ff, sh.up.qs, sh.up.d, qn_q, qn_s, su])
+    hip.launch(dev, "d4_swiglu_w", (n * ff + 255) // 256, 256, [n, ff, float(clamp), sg, su, one, smid, qm_q, qm_s])
+    hip.launch(dev, "d4_mvq8n", (d + 3) // 4, 128, [d, ff, d, n, ff, d, sh.down.qs, sh.down.d, qm_q, qm_s, sout])
+    # the routed experts: row r = (token r / nu, slot r % nu)
+    sel, w = route(dev, logits, n, ne, nu, scale, bias)
+    rmap = hip.hip_upload_new(dev, (np.arange(rows) // nu).astype(np.uint32))
+    smap = hip.hip_upload_new(dev, np.arange(rows, dtype=np.uint32))
+    x, bm, bd, moe = A(dev, 4 * rows * d), A(dev, 4 * rows * ff), A(dev, 4 * rows * d), A(dev, 4 * n * d)
+    hip.launch(dev, "d4_gather_rows", (rows * d + 255) // 256, 256, [d, rows, norm2, rmap, x])
+    hip.launch(dev, "d4_mv_glu_iq2_xxs", ((ff + 7) // 8, 1, rows), 64,
+               [d, ff, pool.grb, hip.I64(0), hip.I64(gb), d, ff, pool.ptrs, sel, x, w, float(clamp), bm])
+    hip.launch(dev, "d4_mv_q2_k_f32", ((d + 7) // 8, 1, rows), 64, [ff, d, pool.drb, hip.I64(2 * gb), ff, d, pool.ptrs, sel, bm, bd])
+    hip.launch(dev, "d4_moe_sum_rows", (n * d + 255) // 256, 256, [d, nu, n, bd, smap, sout, moe])
+    hip.hip_sync(dev)
+    for b in (qn_q, qn_s, sg, su, smid, qm_q, qm_s, sout, one, sel, w, rmap, smap, x, bm, bd):
+        hip.hip_free(b)
+    return moe
+
+
 def route(dev, logits, n, ne, nu, scale, bias=None, alloc=hip.hip_alloc):
     """D4_ROUTE for N tokens' LOGITS (a DBuf): returns (sel, w) DBufs of N x NU."""
     sel, w = alloc(dev, 4 * n * nu), alloc(dev, 4 * n * nu)

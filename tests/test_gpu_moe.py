@@ -161,3 +161,27 @@ def test_moe_decode_step_bit_exact(dev, ne, d, ff, nu, clamp):
         for b in (lb, nb, sel, w, sout, moe, fused, ondev):
             hip.hip_free(b)
     pool.free(); sh.free()
+
+
+@pytest.mark.parametrize("ne,d,ff,nu,n,clamp", [(8, 512, 256, 3, 9, 0.05), (12, 4096, 2048, 6, 4, 0.0)])
+def test_moe_short_pass_of_a_few_tokens_bit_exact(dev, ne, d, ff, nu, n, clamp):
+    """A speculative step's verification (cuda-ds4f-spec.lisp:30-100): the FFN of up to nine tokens
+    at once, experts shared between tokens, every token with the bits of its own decode step."""
+    from illatio_amd import ds4f, hip
+    rng = synth.make_rng(ne * 77 + n)
+    gate, up, down, sg, su, sd = _moe_weights(rng, ne, d, ff)
+    pool = ds4f.ExpertPool(dev, ne, d, ff, gate, up, down)
+    sh = ds4f.SharedExpert(dev, d, ff, sg, su, sd)
+    norm = synth.activations((n, d), rng)
+    logits = synth.activations((n, ne), rng)
+    logits[1] = logits[0]                     # two tokens on the same experts
+    lb, nb = hip.hip_upload_new(dev, logits), hip.hip_upload_new(dev, norm)
+    moe = ds4f.ffn_small(dev, pool, sh, lb, nb, n, ne, nu, 1.5, clamp)
+    got = hip.hip_floats(moe, n * d).reshape(n, d)
+    for t in range(n):
+        want, _, _ = orc.moe_token(gate, up, down, sg, su, sd, d, ff, ne, nu, 1.5, clamp, logits[t], norm[t])
+        assert np.array_equal(bits(got[t]), bits(want)), (t, np.abs(got[t] - want).max())
+    for b in (lb, nb, moe):
+        hip.hip_free(b)
+    pool.free(); sh.free()
+
