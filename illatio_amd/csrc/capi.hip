@@ -131,13 +131,15 @@ int ilt_host_alloc(uint64_t* hptr, uint64_t bytes, unsigned flags) {
   return ILT_OK;
 }
 int ilt_host_free(uint64_t hptr) { return (int)hipHostFree((void*)(uintptr_t)hptr); }
+// Pinning memory that already exists is not offered: the hosts this library is deployed on refuse
+// hipHostRegister, and the error it leaves is reported by whichever GPU call comes next.  The caller
+// (the reference pins mmap'd expert files, cuda.lisp:359-366) takes pinned memory from ilt_host_alloc
+// and reads the file into it; with every expert resident in HBM nothing needs read-through.
 int ilt_host_register(void* p, uint64_t bytes, unsigned flags) {
-  unsigned f = 0;
-  if (flags & 1) f |= hipHostRegisterPortable;
-  if (flags & 2) f |= hipHostRegisterMapped;
-  return (int)hipHostRegister(p, bytes, f);
+  (void)p; (void)bytes; (void)flags;
+  return (int)hipErrorNotSupported;
 }
-int ilt_host_unregister(void* p) { return (int)hipHostUnregister(p); }
+int ilt_host_unregister(void* p) { (void)p; return (int)hipErrorNotSupported; }
 
 // ---- kernels ----------------------------------------------------------------------------------
 

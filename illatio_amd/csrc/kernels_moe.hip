@@ -14,65 +14,116 @@ __device__ __forceinline__ float softplus(float x) {
   return ilt_logf_via_double(1.0f + ilt_expf_via_double(x));
 }
 
-// d4-route: a workgroup a token, a thread an expert.  p = sqrt(softplus(logit)); the top
-// NU of p (+ bias), the earlier expert first of equal ones; weights p/sum(p)*scale with
-// the sum taken in slot order and floored at 2^-14.  hash 1: the experts come from
-// tid2eid[token].
-__global__ void route_kernel(int ne, int nu, int hash, float scale, int has_bias, const float* __restrict__ logits,
-                             const float* __restrict__ bias, const int* __restrict__ tid2eid,
-                             const u32* __restrict__ tokens, u32* __restrict__ sel, float* __restrict__ wout) {
-  extern __shared__ float sh[];
-  float* probs = sh;                    // ne
-  float* sv = sh + ne;                  // ne
-  u64* wbest = (u64*)(sh + 2 * ne);     // up to 16 waves
-  u32* picked = (u32*)(wbest + 16);     // nu
-  const int t = blockIdx.x, e = threadIdx.x;
-  if (e < ne) {
-    const float p = sqrtf(softplus(logits[(long long)t * ne + e]));
-    probs[e] = p;
-    sv[e] = has_bias ? p + bias[(has_bias == 2 ? (long long)t * ne : 0) + e] : p;
-  }
-  __syncthreads();
+// d4-route (ds4f.lisp:950-978): p = sqrt(softplus(logit)); the top NU of p (+ bias), the
+// earlier expert first of equal ones; weights p/sum(p)*scale with the sum taken in slot order
+// and floored at 2^-14.  hash 1: the experts come from tid2eid[token].
+//
+// A wave a token, K experts a lane (expert k*64 + lane), everything in registers.  A round
+// picks one expert: each lane's best remaining score as an order-preserving integer key
+// (0 = nothing left), the wave's largest key, then the smallest expert index among the lanes
+// that hold it; the winning lane strikes its expert off a bit mask.  Lane j keeps slot j.
+// Scores that are NaN (an overflow upstream) compare false both ways in the CPU's insertion,
+// whose result then depends on the order of the insertions: such a token takes the slow
+// branch, one lane doing the CPU's insertion as it is written, so that sel always holds NU
+// different experts below NE, which the kernels downstream index tables with.
+#define ROUTE_WAVES 4
+
+__device__ __forceinline__ u32 wave_max_u32(u32 v) {
+  v = max(v, (u32)ilt_dpp<ILT_DPP_XOR1>((int)v));
+  v = max(v, (u32)ilt_dpp<ILT_DPP_XOR2>((int)v));
+  v = max(v, (u32)ilt_dpp<ILT_DPP_HALF_MIRROR>((int)v));
+  v = max(v, (u32)ilt_dpp<ILT_DPP_ROW_MIRROR>((int)v));
+  const u32 a = __builtin_amdgcn_readlane(v, 0), b = __builtin_amdgcn_readlane(v, 16);
+  const u32 c = __builtin_amdgcn_readlane(v, 32), d = __builtin_amdgcn_readlane(v, 48);
+  return max(max(a, b), max(c, d));
+}
+
+__device__ __forceinline__ float route_prob(float logit) { return sqrtf(softplus(logit)); }
+
+template <int K>
+__global__ __launch_bounds__(64 * ROUTE_WAVES) void route_kernel(int ntok, int ne, int nu, int hash, float scale, int has_bias,
+                                                                 const float* __restrict__ logits, const float* __restrict__ bias,
+                                                                 const int* __restrict__ tid2eid, const u32* __restrict__ tokens,
+                                                                 u32* __restrict__ sel, float* __restrict__ wout) {
+  __shared__ u32 s_idx[ROUTE_WAVES][64];
+  __shared__ float s_sc[ROUTE_WAVES][64];
+  const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+  const int t = blockIdx.x * ROUTE_WAVES + wv;
+  if (t >= ntok) return;                                      // whole waves leave; no barrier below
+  const float* lg = logits + (long long)t * ne;
+  const float* bs = has_bias ? bias + (has_bias == 2 ? (long long)t * ne : 0) : nullptr;
+  u32 my_sel = 0;
+  float my_p = 0.0f;
   if (hash == 1) {
-    if (e < nu) picked[e] = (u32)tid2eid[(long long)tokens[t] * nu + e];
+    if (lane < nu) {
+      const u32 e = min((u32)tid2eid[(long long)tokens[t] * nu + lane], (u32)(ne - 1));
+      my_sel = e;
+      my_p = route_prob(lg[e]);
+    }
   } else {
-    for (int k = 0; k < nu; k++) {
-      // order-preserving key of a float, then the complement of the index: the largest key
-      // is the largest score, the earliest expert among equals
-      u64 key = 0;
-      if (e < ne) {
-        const u32 b = __float_as_uint(sv[e]);
-        const u32 ord = (b & 0x80000000u) ? ~b : (b | 0x80000000u);
-        key = ((u64)ord << 32) | (u32)(0x7FFFFFFF - e);
-        if (sv[e] != sv[e]) key = 0;    // a NaN never wins
-      }
+    float p[K], sc[K];
+    u32 left = 0;                                             // bit k: expert k*64 + lane can still be picked
+    bool nan = false;
 #pragma unroll
-      for (int off = 32; off > 0; off >>= 1) {
-        const u32 hi = __shfl_xor((u32)(key >> 32), off), lo = __shfl_xor((u32)key, off);
-        const u64 o = ((u64)hi << 32) | lo;
-        key = o > key ? o : key;
+    for (int k = 0; k < K; k++) {
+      const int e = k * 64 + lane;
+      p[k] = 0.0f; sc[k] = 0.0f;
+      if (e < ne) {
+        p[k] = route_prob(lg[e]);
+        sc[k] = (bs ? p[k] + bs[e] : p[k]) + 0.0f;            // + 0: no minus zero, which the integer key would rank below zero
+        left |= 1u << k;
+        nan |= sc[k] != sc[k];
       }
-      if ((e & 63) == 0) wbest[e >> 6] = key;
-      __syncthreads();
-      if (e == 0) {
-        u64 best = wbest[0];
-        for (int w = 1; w < (int)(blockDim.x + 63) / 64; w++) best = wbest[w] > best ? wbest[w] : best;
-        const u32 bi = 0x7FFFFFFF - (u32)(best & 0xFFFFFFFFu);
-        picked[k] = bi;
-        sv[bi] = -INFINITY;
+    }
+    if (__builtin_amdgcn_ballot_w64(nan) == 0) {
+      for (int j = 0; j < nu; j++) {
+        u32 key = 0; int bk = 0;
+#pragma unroll
+        for (int k = 0; k < K; k++) {
+          const u32 b = __float_as_uint(sc[k]);
+          const u32 ord = (b & 0x80000000u) ? ~b : (b | 0x80000000u);      // > 0 for every number, -inf included
+          if (((left >> k) & 1u) && ord > key) { key = ord; bk = k; }      // strict: the lane's earliest expert of equal ones
+        }
+        const u32 top = wave_max_u32(key);
+        const u32 cand = (key == top && key != 0) ? (u32)(bk * 64 + lane) : 0xFFFFFFFFu;
+        const u32 e = ~wave_max_u32(~cand);                                // the smallest index holding the top score
+        const int wl = (int)(e & 63u);
+        float pe = 0.0f;
+#pragma unroll
+        for (int k = 0; k < K; k++) if ((int)(e >> 6) == k) pe = p[k];
+        pe = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, pe), wl));
+        if (lane == wl) left &= ~(1u << (e >> 6));
+        if (lane == j) { my_sel = e; my_p = pe; }
       }
-      __syncthreads();
+    } else {
+      // the CPU's insertion, verbatim, by one lane (slots fill from the left, so "empty" is j >= cnt)
+      if (lane == 0) {
+        int cnt = 0;
+        for (int i = 0; i < ne; i++) {
+          const float pi = route_prob(lg[i]);
+          const float si = bs ? pi + bs[i] : pi;
+          for (int j = 0; j < nu; j++) {
+            if (j >= cnt || si > s_sc[wv][j]) {
+              for (int k = min(cnt, nu - 1); k > j; k--) { s_sc[wv][k] = s_sc[wv][k - 1]; s_idx[wv][k] = s_idx[wv][k - 1]; }
+              s_sc[wv][j] = si; s_idx[wv][j] = (u32)i;
+              if (cnt < nu) cnt++;
+              break;
+            }
+          }
+        }
+      }
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+      if (lane < nu) { my_sel = s_idx[wv][lane]; my_p = route_prob(lg[my_sel]); }
     }
   }
-  __syncthreads();
-  if (e == 0) {
-    float sum = 0.0f;
-    for (int i = 0; i < nu; i++) sum = sum + probs[picked[i]];
-    if (sum < 6.103515625e-5f) sum = 6.103515625e-5f;
-    for (int i = 0; i < nu; i++) {
-      sel[(long long)t * nu + i] = picked[i];
-      wout[(long long)t * nu + i] = (probs[picked[i]] / sum) * scale;
-    }
+  float sum = 0.0f;
+  for (int j = 0; j < nu; j++) sum = sum + __shfl(my_p, j);   // in slot order, as the CPU adds them
+  if (sum < 6.103515625e-5f) sum = 6.103515625e-5f;
+  if (lane < nu) {
+    sel[(long long)t * nu + lane] = my_sel;
+    wout[(long long)t * nu + lane] = (my_p / sum) * scale;
   }
 }
 
@@ -227,11 +278,15 @@ __global__ __launch_bounds__(256) void moe_sum_rows_kernel(int d, int nu, int nt
 hipError_t ilt_k_route(int ne, int nu, int hash, float scale, int has_bias, const float* logits, const float* bias,
                        const int* tid2eid, const uint32_t* tokens, uint32_t* sel, float* wout, int ntok, hipStream_t st) {
   if (ntok <= 0) return hipSuccess;
-  if (ne < 1 || ne > 1024 || nu < 1 || nu > ne || hash < 0 || hash > 1) return hipErrorInvalidValue;
-  const int threads = (ne + 63) / 64 * 64;
-  const size_t smem = 4 * (size_t)(2 * ne) + 8 * 16 + 4 * (size_t)nu;
-  hipLaunchKernelGGL(route_kernel, dim3(ntok), dim3(threads), smem, st, ne, nu, hash, scale, has_bias, logits, bias,
-                     tid2eid, tokens, sel, wout);
+  if (ne < 1 || ne > 1024 || nu < 1 || nu > ne || nu > 64 || hash < 0 || hash > 1) return hipErrorInvalidValue;
+  if (hash == 1 && (!tid2eid || !tokens)) return hipErrorInvalidValue;
+  const dim3 grid((ntok + ROUTE_WAVES - 1) / ROUTE_WAVES), block(64 * ROUTE_WAVES);
+#define ROUTE_LAUNCH(K) hipLaunchKernelGGL(route_kernel<K>, grid, block, 0, st, ntok, ne, nu, hash, scale, has_bias, logits, bias, \
+                                           tid2eid, tokens, sel, wout)
+  const int k = (ne + 63) / 64;
+  if (k <= 1) ROUTE_LAUNCH(1); else if (k <= 2) ROUTE_LAUNCH(2); else if (k <= 4) ROUTE_LAUNCH(4);
+  else if (k <= 8) ROUTE_LAUNCH(8); else ROUTE_LAUNCH(16);
+#undef ROUTE_LAUNCH
   return hipGetLastError();
 }
 

@@ -80,8 +80,10 @@ int ilt_memcpy_dtoh_async(void* dst, uint64_t src, uint64_t bytes, uint64_t stre
 int ilt_memcpy_dtod_async(uint64_t dst, uint64_t src, uint64_t bytes, uint64_t stream);    /* :423-428 */
 int ilt_host_alloc(uint64_t* hptr, uint64_t bytes, unsigned flags); /* cuMemHostAlloc, :371-378; flags 1 portable, 2 mapped */
 int ilt_host_free(uint64_t hptr);                       /* cuMemFreeHost, :380 */
-int ilt_host_register(void* p, uint64_t bytes, unsigned flags); /* cuMemHostRegister, :359-366 */
-int ilt_host_unregister(void* p);                       /* cuMemHostUnregister, :368-369 */
+/* cuMemHostRegister / cuMemHostUnregister, :359-369: always hipErrorNotSupported (801) and no runtime call.
+   Memory that already exists is not pinned here; take pinned memory from ilt_host_alloc instead. */
+int ilt_host_register(void* p, uint64_t bytes, unsigned flags);
+int ilt_host_unregister(void* p);
 
 /* ---- 2. the kernels --------------------------------------------------------------------
  * Pointers are device addresses.  "|0" marks an argument that may be null.             */

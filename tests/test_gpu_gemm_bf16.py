@@ -18,7 +18,7 @@ pytestmark = pytest.mark.gpu
 
 TOL_VS_CPU = 2e-2      # max |gpu - cpu| / max |cpu|
 TOL_RMS_VS_EXACT = 5e-3
-TOL_CHAIN_VS_EXACT = 3e-2   # three products and a clamped gate compounded, against the exact chain
+TOL_CHAIN_VS_EXACT = 2e-2   # the whole chain (three products, a clamped gate) against the exact double-precision chain
 
 
 @pytest.fixture(scope="module")

@@ -193,6 +193,17 @@ def test_indexed_expert_gemv_bit_for_bit(dev, qtype, rows, cols):
         for z, e in enumerate(chosen):
             want = orc.matmul(qtype, w[e].reshape(rows, rb), rows, cols, x[z if x_stride else 0])
             assert np.array_equal(bits(got[z]), bits(want)), (qtype, z, np.abs(got[z] - want).max())
+            # the x86 float order of the same integer sums (avx2.lisp:77-150), which the reference's CPUs
+            # take when they compute an expert: other roundings, within 1e-5 of the largest output and of
+            # each row's sum of |terms| (the yardstick of inspect/iquant-test.lisp:50-53)
+            xz = x[z if x_stride else 0]
+            hq, hd, hs = orc.quantize_q8k(xz)
+            wrows = w[e].reshape(rows, rb)
+            avx = np.array([orc.row_dot(qtype, wrows[r], cols, hq, hd, hs, order="avx2") for r in range(rows)], np.float32)
+            terms = np.abs(orc.dequant_rows(qtype, wrows, cols).astype(np.float64)) @ np.abs(
+                hq.astype(np.float64) * np.repeat(hd.astype(np.float64), 256))
+            assert np.abs(got[z] - avx).max() <= 1e-5 * np.abs(avx).max(), (qtype, z)
+            assert (np.abs(got[z].astype(np.float64) - avx) <= 1e-5 * np.maximum(terms, 1e-30)).all(), (qtype, z)
         for b in (xb, kq, kd, ks, y):
             hip.hip_free(b)
     hip.hip_free(pool); hip.hip_free(ptrs)

@@ -44,6 +44,45 @@ def test_route_indices_and_weights_bit_exact(dev, ne, nu, n):
             hip.hip_free(b)
 
 
+def test_route_with_nan_and_masked_scores(dev):
+    """Scores that are NaN (an overflow upstream) and experts masked by a bias of minus infinity: the
+    CPU's insertion (ds4f.lisp:966-972) compares NaNs false both ways, so its result depends on the
+    insertion order; the kernel gives the same indices (NU different experts below NE in every
+    case, which the kernels downstream index tables with) and the same weights, NaN where the CPU's
+    are NaN."""
+    from illatio_amd import ds4f, hip
+    rng = synth.make_rng(99)
+    ne, nu, n = 256, 6, 12
+    logits = synth.activations((n, ne), rng)
+    logits[0, :] = np.nan                                  # every score NaN: the first nu experts, in order
+    logits[1, 3] = np.nan                                  # one NaN among the first nu inserted
+    logits[2, 100] = np.nan                                # one NaN later on: never inserted
+    logits[3, ::2] = np.nan
+    logits[4, :ne - 3] = np.nan                            # fewer numbers than slots
+    logits[5, [0, 1, 2, 3, 4, 5]] = [np.nan, 9.0, np.nan, 8.0, 7.0, np.nan]
+    logits[6, 7] = np.inf
+    logits[7, :] = -200.0                                  # softplus underflows to zero: all tied at 0, the sum floored
+    bias = np.zeros(ne, np.float32)
+    bias[10:200] = -np.inf                                 # masked experts
+    for b in (None, bias):
+        lb = hip.hip_upload_new(dev, logits)
+        bb = None if b is None else hip.hip_upload_new(dev, b)
+        sel, w = ds4f.route(dev, lb, n, ne, nu, 1.5, bb)
+        gs = hip.hip_download(sel, np.uint32, n * nu).reshape(n, nu)
+        gw = hip.hip_floats(w, n * nu).reshape(n, nu)
+        for t in range(n):
+            ws, ww = orc.route(logits[t], nu, 1.5, b)
+            assert gs[t].tolist() == ws.tolist(), (t, gs[t], ws)
+            assert len(set(gs[t].tolist())) == nu and int(gs[t].max()) < ne
+            assert np.array_equal(np.isnan(gw[t]), np.isnan(ww)), t
+            ok = ~np.isnan(ww)
+            assert np.array_equal(bits(gw[t][ok]), bits(ww[ok])), t
+        if b is None:
+            assert gs[0].tolist() == list(range(nu)) and gs[7].tolist() == list(range(nu))
+        for x in (lb, bb, sel, w):
+            hip.hip_free(x)
+
+
 def test_group_rows_invariants_and_gather(dev):
     from illatio_amd import ds4f, hip
     rng = synth.make_rng(5)

@@ -306,6 +306,39 @@ def test_activation_functions_correctly_rounded():
         assert np.float32(orc.softplus(x)) == sp
 
 
+# ---- swiglu! (model.lisp:364-378): x / (1 + e^-x) * b, every rounding explicit ---------------------
+def test_swiglu_against_explicit_roundings_and_misreadings():
+    """Each step of (* (/ x (+ 1f0 (exp (- x)))) b) rounded to single by hand from a long-double
+    evaluation: exp to single (SBCL widens, calls libm, rounds back), the sum, the quotient, the
+    product.  A gate below about -88.7 overflows e^-x to infinity, and the quotient is -0.0
+    (model.lisp:365-368).  The d4-silu form x * sigmoid(x) (ds4f.lisp:248-251) and a product
+    (x*b)/(1+e) are told apart on the same inputs."""
+    f32, ld = np.float32, np.longdouble
+    rng = synth.make_rng(21)
+    gs = np.concatenate([rng.standard_normal(3000).astype(f32) * 5,
+                         np.array([0.0, -0.0, 1.0, -1.0, 20.0, -20.0, 60.0, -60.0, 88.0, -88.0, -88.7, -88.8,
+                                   -89.0, -100.0, -1000.0, 90.0, 1000.0], f32)])
+    us = np.concatenate([rng.standard_normal(3000).astype(f32) * 3, rng.standard_normal(17).astype(f32)])
+    got = orc.swiglu(gs, us)
+    told = set()
+    with np.errstate(over="ignore"):
+        for x, b, y in zip(gs, us, got):
+            e = f32(np.exp(ld(-x)))                              # inf past single's range
+            want = f32(f32(x / f32(f32(1) + e)) * b)
+            assert want.view(np.uint32) == y.view(np.uint32), (x, b)
+            sig = (f32(1) / f32(f32(1) + e)) if x >= 0 else f32(np.exp(ld(x))) / f32(f32(1) + f32(np.exp(ld(x))))
+            if f32(f32(x * sig) * b).view(np.uint32) != y.view(np.uint32):
+                told.add("x*sigmoid")
+            if f32(f32(x * b) / f32(f32(1) + e)).view(np.uint32) != y.view(np.uint32):
+                told.add("(x*b)/(1+e)")
+    assert told == {"x*sigmoid", "(x*b)/(1+e)"}
+    # the overflow case: the quotient is minus zero, the product keeps its sign rule
+    for x in (-88.8, -89.0, -100.0, -1000.0):
+        for b in (2.0, -2.0):
+            y = orc.swiglu([x], [b])[0]
+            assert y == 0 and np.signbit(y) == (b > 0)
+
+
 # ---- routing -------------------------------------------------------------------------------------
 def test_route_against_stable_sort():
     rng = synth.make_rng(7)
@@ -381,6 +414,42 @@ def test_moe_chunk_equals_token_at_a_time():
         one, s1, w1 = orc.moe_token(gate, up, down, sg, su, sd, d, ff, ne, nu, 1.5, 0.0, logits[t], norms[t])
         assert s1.tolist() == sel[t].tolist() and np.array_equal(w1, w[t])
         assert np.array_equal(one.view(np.uint32), out[t].view(np.uint32))
+
+
+def test_moe_shared_composed_from_pinned_pieces():
+    """d4-shared! (ds4f.lisp:1039-1048) put together by hand from functions other tests pin:
+    quantize-q8! with the scale kept as a float (ds4f.lisp:1052-1053: *q8-f16-scale* NIL), the
+    Q8_0 row dot, d4-silu.  The same composition with an f16-rounded scale, or with swiglu!'s
+    x/(1+e^-x) in place of d4-silu, must give other bits somewhere, or the case pins nothing."""
+    f32 = np.float32
+    rng = synth.make_rng(22)
+    d, ff = 256, 128
+    sg = synth.weights(synth.Q8_0, ff, d, rng); su = synth.weights(synth.Q8_0, ff, d, rng)
+    sd = synth.weights(synth.Q8_0, d, ff, rng, dscale=0.5)
+    norm = synth.activations(d, rng) * f32(3)
+
+    def compose(clamp, f16_scale, silu):
+        xq, xs = orc.quantize_q8(norm, f16_scale)
+        mid = np.empty(ff, f32)
+        for r in range(ff):
+            g = f32(orc.row_dot(synth.Q8_0, sg[r], d, xq, xs))
+            u = f32(orc.row_dot(synth.Q8_0, su[r], d, xq, xs))
+            if clamp > 1e-6:
+                g = min(g, f32(clamp)); u = max(f32(-clamp), min(u, f32(clamp)))
+            mid[r] = f32(silu(g) * u)
+        mq, ms = orc.quantize_q8(mid, f16_scale)
+        return np.array([orc.row_dot(synth.Q8_0, sd[r], ff, mq, ms) for r in range(d)], f32)
+
+    d4 = lambda g: f32(orc.silu(g))
+    for clamp in (0.0, 0.3):
+        got = orc.moe_shared(sg, su, sd, d, ff, clamp, norm)
+        want = compose(clamp, False, d4)
+        assert np.array_equal(got.view(np.uint32), want.view(np.uint32)), clamp
+        assert not np.array_equal(got.view(np.uint32), compose(clamp, True, d4).view(np.uint32))
+        assert np.array_equal(got.view(np.uint32),
+                              orc.moe_shared(sg, su, sd, d, ff, clamp, norm, nthreads=3).view(np.uint32))
+    # the clamp changes the result on this input (it is exercised), and it is one-sided for the gate
+    assert not np.array_equal(orc.moe_shared(sg, su, sd, d, ff, 0.0, norm), orc.moe_shared(sg, su, sd, d, ff, 0.3, norm))
 
 
 # ---- rmsnorm! (model.lisp:205-216) -----------------------------------------------------------
