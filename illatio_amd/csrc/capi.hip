@@ -429,6 +429,59 @@ int ilt_d4_moe_sum_rows(uint64_t stream, int d, int nu, int ntok, const float* d
   return (int)ilt_k_moe_sum_rows(d, nu, ntok, down, map, shared_, moe, S(stream));
 }
 
+// ---- one token's FFN past the router in one call ------------------------------------------------
+// The step's intermediate results, 256-byte aligned pieces of one buffer.
+namespace {
+struct StepLayout { uint64_t sel, w, smid, sout, bm, bd, total; };
+inline uint64_t up256(uint64_t v) { return (v + 255) / 256 * 256; }
+StepLayout step_layout(int nu, int d, int ff) {
+  StepLayout l; uint64_t o = 0;
+  l.sel = o; o += up256(4ull * nu);
+  l.w = o; o += up256(4ull * nu);
+  l.smid = o; o += up256(4ull * ff);
+  l.sout = o; o += up256(4ull * d);
+  l.bm = o; o += up256(4ull * nu * ff);
+  l.bd = o; o += up256(4ull * nu * d);
+  l.total = o;
+  return l;
+}
+int step_args_ok(int ne, int nu, int d, int ff, const ilt_ffn_step_weights* wt, const float* logits, const float* x, float* moe) {
+  ILT_REQUIRE(wt && logits && x && moe && ne >= 1 && ne <= 1024 && nu >= 1 && nu <= 64 && nu <= ne);
+  ILT_REQUIRE(d > 0 && ff > 0 && d % 256 == 0 && ff % 256 == 0 && d <= (1 << 20) && ff <= (1 << 20));
+  ILT_REQUIRE(wt->slots && wt->gate_bytes == (int64_t)ff * (d / 256 * 66) && wt->sgate_q && wt->sgate_d && wt->sup_q && wt->sup_d &&
+              wt->sdown_q && wt->sdown_d);
+  return ILT_OK;
+}
+// Six launches on STREAM, nothing allocated, freed or waited for; ws holds step_layout's bytes.
+int step_run(uint64_t stream, uint8_t* ws, int ne, int nu, int d, int ff, float scale, float clamp, const ilt_ffn_step_weights* wt,
+             const float* logits, const float* bias, const float* x, float* moe) {
+  const StepLayout l = step_layout(nu, d, ff);
+  uint32_t* sel = (uint32_t*)(ws + l.sel);
+  float *w = (float*)(ws + l.w), *smid = (float*)(ws + l.smid), *sout = (float*)(ws + l.sout);
+  float *bm = (float*)(ws + l.bm), *bd = (float*)(ws + l.bd);
+  const int grb = d / 256 * 66, drb = ff / 256 * 84;
+  ILT_TRY((hipError_t)ilt_d4_route(stream, ne, nu, 0, scale, bias ? 1 : 0, logits, bias, nullptr, nullptr, sel, w, 1));
+  ILT_TRY((hipError_t)ilt_d4_mvq8_glu(stream, ff, d, wt->sgate_q, wt->sgate_d, wt->sup_q, wt->sup_d, x, clamp, smid));
+  ilt_mv_desc down = {ILT_Q8_0, d, wt->sdown_q, wt->sdown_d, sout, nullptr};
+  ILT_TRY((hipError_t)ilt_mv_multi(stream, 1, &down, ff, nullptr, nullptr, nullptr, smid, 0, 0, 0));
+  ILT_TRY((hipError_t)ilt_d4_mv_glu_iq2_xxs(stream, d, ff, grb, 0, wt->gate_bytes, 0, ff, wt->slots, sel, nu, x, w, clamp, bm));
+  ILT_TRY((hipError_t)ilt_d4_mv_q2_k_f32(stream, ff, d, drb, 2 * wt->gate_bytes, ff, d, wt->slots, sel, nu, bm, bd));
+  return ilt_d4_moe_sum(stream, d, nu, bd, sout, moe, nullptr);
+}
+}  // namespace
+
+uint64_t ilt_d4_ffn_step_workspace(int nu, int d, int ff) {
+  if (nu < 1 || d < 1 || ff < 1 || nu > 64 || d > (1 << 20) || ff > (1 << 20)) return 0;
+  return step_layout(nu, d, ff).total;
+}
+
+int ilt_d4_ffn_step(uint64_t stream, void* ws, uint64_t ws_bytes, int ne, int nu, int d, int ff, float scale, float clamp,
+                    const ilt_ffn_step_weights* wt, const float* logits, const float* bias, const float* x, float* moe) {
+  ILT_TRY((hipError_t)step_args_ok(ne, nu, d, ff, wt, logits, x, moe));
+  ILT_REQUIRE(ws && ((uintptr_t)ws & 255) == 0 && ws_bytes >= step_layout(nu, d, ff).total);
+  return step_run(stream, (uint8_t*)ws, ne, nu, d, ff, scale, clamp, wt, logits, bias, x, moe);
+}
+
 int ilt_mm_q8(uint64_t stream, const int8_t* wq, const uint16_t* wd, const int8_t* xq, const float* xs, float* y,
               const float* bias, int rows, int cols, int n, int acc) {
   ILT_REQUIRE(rows >= 0 && n >= 0 && cols > 0 && cols % 32 == 0);

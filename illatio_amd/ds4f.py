@@ -11,6 +11,8 @@ Activations are quantized as the reference's CPU path quantizes them (Q8_K for t
 experts, D4-ROUTED!, ds4f.lisp:994-1037; Q8_0 with a float scale for the shared expert,
 D4-SHARED!, :1039-1048), not left as floats as its CUDA kernels take them.
 """
+import ctypes as C
+
 import numpy as np
 
 from . import dense, hip
@@ -184,6 +186,42 @@ def ffn_step_device(dev, pool, sh, logits, norm2, ne, nu, scale, clamp, bias=Non
     moe = ffn_step_fused(dev, pool, sh, nu, None, norm2, clamp, ws=ws, routed=(sel, w))
     if not ws:
         hip.hip_free(sel); hip.hip_free(w)
+    return moe
+
+
+class FfnStepWeights(C.Structure):
+    """ilt_ffn_step_weights: the slot table and the shared expert's repacked matrices."""
+    _fields_ = [("slots", C.c_uint64), ("gate_bytes", C.c_int64),
+                ("sgate_q", C.c_uint64), ("sgate_d", C.c_uint64), ("sup_q", C.c_uint64), ("sup_d", C.c_uint64),
+                ("sdown_q", C.c_uint64), ("sdown_d", C.c_uint64)]
+
+
+def step_weights(pool, sh):
+    return FfnStepWeights(pool.ptrs.ptr, pool.gate_bytes, sh.gate.qs.ptr, sh.gate.d.ptr, sh.up.qs.ptr, sh.up.d.ptr,
+                          sh.down.qs.ptr, sh.down.d.ptr)
+
+
+def step_workspace_bytes(nu, d, ff):
+    f = hip.lib().ilt_d4_ffn_step_workspace
+    f.restype = C.c_uint64
+    return int(f(C.c_int(nu), C.c_int(d), C.c_int(ff)))
+
+
+def ffn_step_call(dev, pool, sh, logits, norm2, moe, ne, nu, scale, clamp, bias=None, wsbuf=None):
+    """ffn_step_device's six launches queued by one call into the library (ilt_d4_ffn_step): the
+    host crosses the boundary once a layer instead of once a launch.  WSBUF: a DBuf of
+    step_workspace_bytes for the intermediate results (one is made and freed if None);
+    MOE: the output DBuf (d floats)."""
+    own = wsbuf is None
+    if own:
+        wsbuf = hip.hip_alloc(dev, step_workspace_bytes(nu, pool.d, pool.ff), zero=False)
+    wt = step_weights(pool, sh)
+    hip.call("ilt_d4_ffn_step", C.c_uint64(dev.stream), C.c_uint64(wsbuf.ptr), C.c_uint64(wsbuf.bytes), C.c_int(ne), C.c_int(nu),
+             C.c_int(pool.d), C.c_int(pool.ff), C.c_float(scale), C.c_float(clamp), C.byref(wt), C.c_uint64(logits.ptr),
+             C.c_uint64(bias.ptr if bias is not None else 0), C.c_uint64(norm2.ptr), C.c_uint64(moe.ptr))
+    if own:
+        hip.hip_sync(dev)
+        hip.hip_free(wsbuf)
     return moe
 
 

@@ -216,6 +216,30 @@ int ilt_d4_mv_q2_k_f32(uint64_t stream, int ncols, int nrows, int row_bytes, int
 int ilt_d4_mvq8_glu(uint64_t stream, int rows, int cols, const int8_t* gq, const uint16_t* gd, const int8_t* uq,
                     const uint16_t* ud, const float* x, float clamp, float* mid);
 
+/* One token's FFN past the router in one call: DK-FFN-HEAD's shared expert and DK-FFN-TAIL
+   (cuda-ds4f.lisp:883-956) with the routing left on the device (the reference copies the
+   logits out, waits and routes on the CPU in every layer, :991-999).  Six launches on stream:
+   d4_route, d4_mvq8_glu, the shared expert's down, d4_mv_glu_iq2_xxs and d4_mv_q2_k_f32 indexed
+   by d4_route's sel, d4_moe_sum; moe[d] = the nu routed experts' rows in slot order + the shared
+   expert's, with the CPU path's bits (d4-ffn without HC, ds4f.lisp:980-992).  Nothing is
+   allocated, freed or waited for.  The intermediate results (sel, weights, the two gated
+   activations, the shared expert's row, one down row per slot) live in ws, 256-byte aligned,
+   ilt_d4_ffn_step_workspace(nu, d, ff) bytes of device memory that the caller owns (0 for
+   sizes the step does not take: nu <= 64, ne <= 1024, d and ff multiples of 256).
+   slots: the table of all ne expert slots, each gate | up | down with gate_bytes =
+   ff * (d/256) * 66; the shared expert's three Q8_0 matrices repacked by ilt_repack_q8.
+   bias may be null.  Calls on one stream that share ws run one after another. */
+typedef struct ilt_ffn_step_weights {
+  const uint64_t* slots;
+  int64_t gate_bytes;
+  const int8_t* sgate_q; const uint16_t* sgate_d;
+  const int8_t* sup_q; const uint16_t* sup_d;
+  const int8_t* sdown_q; const uint16_t* sdown_d;
+} ilt_ffn_step_weights;
+uint64_t ilt_d4_ffn_step_workspace(int nu, int d, int ff);
+int ilt_d4_ffn_step(uint64_t stream, void* ws, uint64_t ws_bytes, int ne, int nu, int d, int ff, float scale, float clamp,
+                    const ilt_ffn_step_weights* wt, const float* logits, const float* bias, const float* x, float* moe);
+
 /* Rows as floats (dense.cu:53 embed_q8, kquant.cu:202 embed_k; CPU: q8mat-row!, kmat-row!,
    iq2xxs-row-floats!, q2k-row-floats!): out[n] = row tokens[n] (row n when tokens is null)
    of W, bit-exact.  ilt_dequant_rows takes a GGUF type (any of the five; Q8_0 repacked,

@@ -197,8 +197,28 @@ def test_moe_decode_step_bit_exact(dev, ne, d, ff, nu, clamp):
         ondev = ds4f.ffn_step_device(dev, pool, sh, lb, nb, ne, nu, 1.5, clamp)
         got = hip.hip_floats(ondev, d)
         assert np.array_equal(bits(got), bits(want)), np.abs(got - want).max()
-        for b in (lb, nb, sel, w, sout, moe, fused, ondev):
+        # the same six launches queued by one call into the library, its intermediates in a caller's workspace
+        out = hip.hip_alloc(dev, 4 * d)
+        ds4f.ffn_step_call(dev, pool, sh, lb, nb, out, ne, nu, 1.5, clamp)
+        got = hip.hip_floats(out, d)
+        assert np.array_equal(bits(got), bits(want)), np.abs(got - want).max()
+        for b in (lb, nb, sel, w, sout, moe, fused, ondev, out):
             hip.hip_free(b)
+    # a bias on the scores, a workspace used twice, and one that is too small
+    bias = (rng.standard_normal(ne) * 0.5).astype(np.float32)
+    norm, logits = synth.activations(d, rng), synth.activations(ne, rng)
+    want, wsel, _ = orc.moe_token(gate, up, down, sg, su, sd, d, ff, ne, nu, 1.5, clamp, logits, norm, bias=bias)
+    assert wsel.tolist() != orc.route(logits, nu, 1.5)[0].tolist()          # the bias changes the choice
+    lb, nb, bb, out = hip.hip_upload_new(dev, logits), hip.hip_upload_new(dev, norm), hip.hip_upload_new(dev, bias), hip.hip_alloc(dev, 4 * d)
+    ws = hip.hip_alloc(dev, ds4f.step_workspace_bytes(nu, d, ff), zero=False)
+    for _ in range(2):
+        ds4f.ffn_step_call(dev, pool, sh, lb, nb, out, ne, nu, 1.5, clamp, bias=bb, wsbuf=ws)
+        assert np.array_equal(bits(hip.hip_floats(out, d)), bits(want))
+    small = hip.DBuf(ws.ptr, ws.bytes - 256, dev)
+    with pytest.raises(hip.HipError):
+        ds4f.ffn_step_call(dev, pool, sh, lb, nb, out, ne, nu, 1.5, clamp, wsbuf=small)
+    for b in (lb, nb, bb, out, ws):
+        hip.hip_free(b)
     pool.free(); sh.free()
 
 
