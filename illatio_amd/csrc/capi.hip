@@ -482,6 +482,44 @@ int ilt_d4_ffn_step(uint64_t stream, void* ws, uint64_t ws_bytes, int ne, int nu
   return step_run(stream, (uint8_t*)ws, ne, nu, d, ff, scale, clamp, wt, logits, bias, x, moe);
 }
 
+// ilt_d4_ffn_step for callers that cannot allocate or pass a workspace: the step's intermediate
+// results in a device array that is part of the library's code object.  Each GPU the library runs
+// on holds its own copy, at its own address, until the process ends.
+#define ILT_STEP_SCRATCH_BYTES (1u << 20)
+static __device__ __align__(256) __attribute__((used)) unsigned char scratch[ILT_STEP_SCRATCH_BYTES];
+// The array's address on each device, asked of the runtime once per device with that device
+// current.  In host code the name `scratch` is a stand-in for the symbol, not a device address:
+// only these pointers go to kernels.
+#define ILT_MAX_DEVICES 64
+static void* g_scratch_ptr[ILT_MAX_DEVICES];
+
+static int step_scratch(uint8_t** out) {
+  int dev = -1;
+  ILT_TRY(hipGetDevice(&dev));
+  ILT_REQUIRE(dev >= 0 && dev < ILT_MAX_DEVICES);
+  void* p = __atomic_load_n(&g_scratch_ptr[dev], __ATOMIC_ACQUIRE);
+  if (!p) {
+    ILT_TRY(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+    ILT_REQUIRE(p && ((uintptr_t)p & 255) == 0);
+    __atomic_store_n(&g_scratch_ptr[dev], p, __ATOMIC_RELEASE);       // two threads racing store the same address
+  }
+  *out = (uint8_t*)p;
+  return ILT_OK;
+}
+
+uint64_t ilt_d4_ffn_step_noalloc_max_bytes(void) { return ILT_STEP_SCRATCH_BYTES; }
+
+int ilt_d4_ffn_step_noalloc(uint64_t stream, int ne, int nu, int d, int ff, float scale, float clamp,
+                            const ilt_ffn_step_weights* wt, const float* logits, const float* bias, const float* x, float* moe) {
+  ILT_TRY((hipError_t)step_args_ok(ne, nu, d, ff, wt, logits, x, moe));
+  if (step_layout(nu, d, ff).total > ILT_STEP_SCRATCH_BYTES) return (int)hipErrorInvalidValue;    // beyond the array: say so, touch nothing
+  uint8_t* ws = nullptr;
+  ILT_TRY((hipError_t)step_scratch(&ws));
+  // Every piece of the layout is written in full by the launch that produces it before a later
+  // launch reads it, so nothing of the previous call's contents has to be cleared.
+  return step_run(stream, ws, ne, nu, d, ff, scale, clamp, wt, logits, bias, x, moe);
+}
+
 int ilt_mm_q8(uint64_t stream, const int8_t* wq, const uint16_t* wd, const int8_t* xq, const float* xs, float* y,
               const float* bias, int rows, int cols, int n, int acc) {
   ILT_REQUIRE(rows >= 0 && n >= 0 && cols > 0 && cols % 32 == 0);

@@ -225,6 +225,17 @@ def ffn_step_call(dev, pool, sh, logits, norm2, moe, ne, nu, scale, clamp, bias=
     return moe
 
 
+def ffn_step_noalloc(dev, pool, sh, logits, norm2, moe, ne, nu, scale, clamp, bias=None):
+    """ffn_step_call with the intermediate results in the library's own device array
+    (ilt_d4_ffn_step_noalloc): no workspace, no allocation; steps of more than 1 MiB of
+    intermediates raise.  Calls that overlap on one GPU race on the array."""
+    wt = step_weights(pool, sh)
+    hip.call("ilt_d4_ffn_step_noalloc", C.c_uint64(dev.stream), C.c_int(ne), C.c_int(nu), C.c_int(pool.d), C.c_int(pool.ff),
+             C.c_float(scale), C.c_float(clamp), C.byref(wt), C.c_uint64(logits.ptr),
+             C.c_uint64(bias.ptr if bias is not None else 0), C.c_uint64(norm2.ptr), C.c_uint64(moe.ptr))
+    return moe
+
+
 def ffn_small(dev, pool, sh, logits, norm2, n, ne, nu, scale, clamp, bias=None):
     """The FFN past the router for a short pass's N <= 9 tokens (DK-FFN-SMALL,
     cuda-ds4f-spec.lisp:30-100: a speculative step's verification), every token with decode's

@@ -240,6 +240,20 @@ uint64_t ilt_d4_ffn_step_workspace(int nu, int d, int ff);
 int ilt_d4_ffn_step(uint64_t stream, void* ws, uint64_t ws_bytes, int ne, int nu, int d, int ff, float scale, float clamp,
                     const ilt_ffn_step_weights* wt, const float* logits, const float* bias, const float* x, float* moe);
 
+/* ilt_d4_ffn_step without a workspace and without any allocation.  No counterpart in the
+   reference: it is for callers that cannot allocate device memory or keep a workspace alive --
+   code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  The
+   intermediate results live in a device array inside the library, ilt_d4_ffn_step_noalloc_max_bytes()
+   = 1 MiB per GPU, held until the process ends; a step whose ilt_d4_ffn_step_workspace(nu, d, ff)
+   is larger returns hipErrorInvalidValue (1) and does nothing (config 4's step, nu 6, d 4096,
+   ff 2048, takes 172,544 bytes).  The call makes no hipMalloc, hipFree or other allocating call;
+   the array's address is asked of the runtime on the first call on each device.  Every call on a
+   GPU shares that GPU's array: calls on one stream run one after another and are safe; calls that
+   overlap on one GPU (two streams, two threads) race on it.  Same results as ilt_d4_ffn_step. */
+uint64_t ilt_d4_ffn_step_noalloc_max_bytes(void);
+int ilt_d4_ffn_step_noalloc(uint64_t stream, int ne, int nu, int d, int ff, float scale, float clamp,
+                            const ilt_ffn_step_weights* wt, const float* logits, const float* bias, const float* x, float* moe);
+
 /* Rows as floats (dense.cu:53 embed_q8, kquant.cu:202 embed_k; CPU: q8mat-row!, kmat-row!,
    iq2xxs-row-floats!, q2k-row-floats!): out[n] = row tokens[n] (row n when tokens is null)
    of W, bit-exact.  ilt_dequant_rows takes a GGUF type (any of the five; Q8_0 repacked,
