@@ -260,19 +260,6 @@ int ilt_mv_multi(uint64_t stream, int nmat, const ilt_mv_desc* descs, int cols, 
 
 uint64_t ilt_streamed_launches(void) { return (uint64_t)ilt_k_streamed_launches(); }
 
-int ilt_chain_create(uint64_t* chain, const ilt_chain_stage* stages, int nstages) {
-  ILT_REQUIRE(chain);
-  IltChain* c = nullptr;
-  ILT_TRY(ilt_k_chain_create(stages, nstages, &c));
-  *chain = (uint64_t)(uintptr_t)c;
-  return ILT_OK;
-}
-int ilt_chain_run(uint64_t stream, uint64_t chain) { return (int)ilt_k_chain_run((IltChain*)(uintptr_t)chain, S(stream)); }
-int ilt_chain_status(uint64_t stream, uint64_t chain, uint32_t* flags) {
-  return (int)ilt_k_chain_status((IltChain*)(uintptr_t)chain, S(stream), flags);
-}
-int ilt_chain_destroy(uint64_t chain) { return (int)ilt_k_chain_destroy((IltChain*)(uintptr_t)chain); }
-
 int ilt_mv_multi_norm(uint64_t stream, int nmat, const ilt_mv_desc* descs, int cols, const float* x, const float* norm_w,
                       float eps, int exact_order, int f16_scale, int glu) {
   ILT_REQUIRE(descs && nmat >= 1 && nmat <= 4 && x && norm_w);

@@ -62,16 +62,7 @@ struct IltGemvParams {
 // The kernel is chosen by the matrices' formats (mat[i].fmt): one format, or Q4_K and Q6_K mixed.
 hipError_t ilt_gemv_launch(IltGemvParams& p, int nz, hipStream_t st);
 
-unsigned long long ilt_k_streamed_launches();
-
-// A chain of dependent decode products in one launch (kernels_gemv.hip); ilt_chain_stage is the public struct.
-struct ilt_chain_stage;
-struct IltChain;
-hipError_t ilt_k_chain_create(const ilt_chain_stage* stages, int n, IltChain** out);
-hipError_t ilt_k_chain_run(IltChain* c, hipStream_t stream);
-hipError_t ilt_k_chain_status(IltChain* c, hipStream_t stream, uint32_t* flags);
-hipError_t ilt_k_chain_destroy(IltChain* c);
-      // decode products launched as the streamed variant so far (diagnostic)
+unsigned long long ilt_k_streamed_launches();      // decode products launched as the streamed variant so far (diagnostic)
 
 hipError_t ilt_k_quant_q8(const float* x, int8_t* xq, float* xs, int* xsum, long long nblocks, int f16_scale, hipStream_t st);
 hipError_t ilt_k_quant_q8k(const float* x, int8_t* xq, float* xd, int* bsums, long long nblocks, hipStream_t st);

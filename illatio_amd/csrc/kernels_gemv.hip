@@ -22,10 +22,7 @@
 #include "ilt_device.h"
 #include "ilt_iq2xxs_tables.h"
 #include "ilt_kernels.h"
-#include "../../include/illatio_hip.h"
-#include <string.h>
 #include <type_traits>
-#include <vector>
 
 namespace {
 
@@ -1029,295 +1026,6 @@ __global__ __launch_bounds__(kThreads) void rmsnorm_quant_kernel(const float* __
   }
 }
 
-// ---- a chain of dependent products in one launch ---------------------------------------------------
-// One decoded token's products depend on one another (a layer's wo on its Q, its gate and up on the
-// residual stream after wo, its down on their gated activation, the next layer's Q/K/V on the stream after
-// down), and at batch one each is short: as launches of its own a product costs about 3 us before its first
-// instruction and its matrix only starts to stream then.  Here a grid of one workgroup per CU stays resident
-// and walks a table of stages.  A stage's input vector is exchanged between the workgroups through memory,
-// each float in an 8-byte word beside the tag of the stage that made it (one store publishes both, one load
-// sees both: no flag, no fence, no counter; the readers poll the data); the CU's share of the next stage's
-// matrix is already streaming into LDS while that exchange is under way.
-//
-// Roles, as in the streamed kernel: waves 0-3 poll the input, take rmsnorm!'s scale where the stage has one,
-// and quantize into LDS; waves 4-15 send off the loads of the CU's rows (each wave a run of consecutive
-// blocks, so it waits for its own loads only), form the blocks' terms, and after a barrier add each row's
-// terms in the CPU's order.  Two workgroup barriers a stage: A = the activations are staged; B = every
-// block's terms are written and the matrix's room in LDS is free for the next stage's.
-// All waits on other workgroups are bounded: a wave that gives up sets *err and goes on (with wrong
-// numbers), so every wave reaches every barrier and the grid always drains.
-struct ChainMat {
-  const u8* w; float* y; const float* bias; u64* y_ll;
-  long long row_bytes; int rows; int fmt;
-};
-struct ChainStage {
-  ChainMat mat[3];                       // one to three matrices on the same input; glu: gate, up
-  const u64* x_ll; const float* x_plain; // the input: exchanged words of an earlier stage, or plain floats (made before the launch)
-  const float* norm_w;                   // rmsnorm! by these weights before quantizing, or null
-  const u64* r_ll; const float* r_plain; // y = residual + W x (mat[0] only): exchanged words, or plain floats, or neither
-  float eps; int norm_seq;
-  int nmat, glu, cols;
-  u32 x_tag, r_tag, out_tag;             // added to the launch's base tag
-  u32 s_magic;
-};
-constexpr int kChainSpin = 1 << 17;
-
-__device__ __forceinline__ u64 ll_load(const u64* p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
-__device__ __forceinline__ u32 ll_flag(const u32* p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
-__device__ __forceinline__ void ll_store(u64* p, u32 tag, float v) {
-  __hip_atomic_store(p, ((u64)tag << 32) | (u64)__float_as_uint(v), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-
-// nblocks consecutive blocks from src into LDS, 64 pieces of 16 bytes an instruction.
-template <int FMT>
-__device__ __forceinline__ void stream_blocks(const u8* src_, int nblocks, u8* lds_run, int lane) {
-  using B = LdsBlk<FMT>;
-  const u8* src = (const u8*)ilt_uniform_ptr(src_);
-  const int npieces = __builtin_amdgcn_readfirstlane(nblocks * B::PPB);
-  const int nfull = npieces >> 6, tail = npieces & 63;
-  u32 blk = (u32)lane / B::PPB, pc = (u32)lane % B::PPB;
-  for (int i = 0; i < nfull; i++) {
-    ilt_g2lds16(src + blk * B::BB + B::goff(pc), lds_run + i * 1024);
-    blk += 64 / B::PPB; pc += 64 % B::PPB;
-    if (pc >= B::PPB) { pc -= B::PPB; blk += 1; }
-  }
-  if (tail && lane < tail) ilt_g2lds16(src + blk * B::BB + B::goff(pc), lds_run + nfull * 1024);
-}
-
-// Blocks f0 .. f1-1 of a run in LDS (block f is block f mod S of its row): terms into t + f * TERMS.
-template <int FMT>
-__device__ __forceinline__ void wave_blocks_lds(const u8* run, int f0, int f1, int S, u32 s_magic, const Lds& L, float* t, int lane) {
-  using F = Fmt<FMT>;
-  constexpr int GPW = ILT_WAVE / F::LPB;
-  const int j = lane % F::LPB, gl = lane / F::LPB;
-  const int step = S > 1 ? GPW - (int)__umulhi((u32)GPW, s_magic) * S : 0;
-  const int first = f0 + gl;
-  int s_ = S > 1 ? first - (int)__umulhi((u32)first, s_magic) * S : 0;
-  for (int f = first; f < f1; f += GPW) {
-    Raw<FMT> r;
-    load_raw_lds<FMT>(r, run, nullptr, f, j);
-    block_terms<FMT>(r, s_, j, L, t + (long)f * F::TERMS);
-    s_ += step;
-    if (s_ >= S) s_ -= S;
-  }
-}
-
-// rmsnorm!'s scale from the stagers' partial sums of squares (see norm_scale); XF = the vector as floats in
-// LDS, for the rare case that the squares have to be added again in the CPU's order.  Three barriers, which
-// the other waves keep step with.
-__device__ __forceinline__ float norm_scale_chain(double part, const float* xf, int n, float eps, int seq, double* red) {
-#pragma unroll
-  for (int off = 32; off > 0; off >>= 1) part += __shfl_xor(part, off);
-  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = part;
-  ilt_barrier_lds();
-  double sum = red[0];
-#pragma unroll
-  for (int w = 1; w < kStagers; w++) sum += red[w];
-  double v = sum / (double)n + (double)eps;
-  const double slack = v * ((double)(n + 8) * 0x1p-51);
-  const bool again = seq || (float)(v - slack) != (float)(v + slack);
-  ilt_barrier_lds();
-  if (again && threadIdx.x == 0) {
-    double s = 0.0;
-    for (int i = 0; i < n; i++) { const float xi = ilt_lds_ldf(xf + i); s += (double)(xi * xi); }
-    red[0] = s;
-  }
-  ilt_barrier_lds();
-  if (again) v = red[0] / (double)n + (double)eps;
-  return 1.0f / sqrtf((float)v);
-}
-
-__device__ __forceinline__ int chain_lds_block(int fmt) { return fmt == ILT_Q4_K ? 144 : 224; }
-__device__ __forceinline__ int chain_mem_block(int fmt) { return fmt == ILT_Q4_K ? 144 : ILT_Q6K_STRIDE; }
-
-// LDS: xq | bsums | xs | xf (norm stages) | red | terms | the matrices' blocks
-__global__ __launch_bounds__(kStreamThreads) void gemv_chain_kernel(const ChainStage* __restrict__ stages, int nstages, u32 base, int smax,
-                                                                   int tmax, int xfmax, u32* err) {
-  extern __shared__ __align__(16) unsigned char smem[];
-  i8* lxq = (i8*)smem;
-  int* lbs = (int*)(smem + (long)smax * XP);
-  float* lxs = (float*)(lbs + smax * 16);
-  float* xf = lxs + ((smax + 3) & ~3);
-  double* red = (double*)(xf + xfmax);
-  float* terms = (float*)(red + kStagers);
-  u8* wroom = (u8*)(terms + tmax);
-  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int G = gridDim.x, g = blockIdx.x;
-  const bool stager = wave < kStagers;
-  const int rw = wave - kStagers;
-  bool failed = false;
-
-  // what the row waves need of a stage: the CU's rows of each matrix, their blocks' place in LDS
-  struct Plan { int lo[3], nb[3], woff[3], toff[3], total, up_off; };
-  auto plan_of = [&](const ChainStage& st, Plan& pl) {
-    const int S = st.cols >> 8;
-    int off = 0, t = 0, tot = 0;
-    const int nm = st.glu ? 1 : st.nmat;
-#pragma unroll
-    for (int m = 0; m < 3; m++) {
-      pl.lo[m] = pl.nb[m] = pl.woff[m] = pl.toff[m] = 0;
-      if (m >= nm) continue;
-      const long rows = st.mat[m].rows;
-      const int lo = (int)((rows * g) / G), hi = (int)((rows * (g + 1)) / G);
-      pl.lo[m] = lo; pl.nb[m] = (hi - lo) * S; pl.woff[m] = off; pl.toff[m] = t;
-      off += pl.nb[m] * chain_lds_block(st.mat[m].fmt); t += pl.nb[m] * 2; tot += pl.nb[m];
-    }
-    pl.total = tot;
-    pl.up_off = off;                   // glu: the up matrix's blocks behind the gate's; its terms behind the gate's
-  };
-  // this wave's run of the stage's blocks (the matrices' blocks one after another), cut at the matrices' ends
-  auto for_segments = [&](const Plan& pl, auto&& f) {
-    const int a = (int)(((long)pl.total * rw) / kRowWaves), b = (int)(((long)pl.total * (rw + 1)) / kRowWaves);
-    int start = 0;
-#pragma unroll
-    for (int m = 0; m < 3; m++) {
-      const int lo = max(a, start) - start, hi = min(b, start + pl.nb[m]) - start;
-      if (lo < hi) f(m, lo, hi);
-      start += pl.nb[m];
-    }
-  };
-  auto prefetch = [&](const ChainStage& st, const Plan& pl) {
-    for_segments(pl, [&](int m, int lo, int hi) {
-      const int fmt = st.mat[m].fmt;
-      const long at = (long)pl.lo[m] * st.mat[m].row_bytes + (long)lo * chain_mem_block(fmt);
-      u8* dst = wroom + pl.woff[m] + lo * chain_lds_block(fmt);
-      with_format<0>(fmt, [&](auto F) { stream_blocks<decltype(F)::value>(st.mat[m].w + at, hi - lo, dst, lane); });
-      if (st.glu) {
-        const int ufmt = st.mat[1].fmt;
-        const long uat = (long)pl.lo[m] * st.mat[1].row_bytes + (long)lo * chain_mem_block(ufmt);
-        u8* udst = wroom + pl.up_off + lo * chain_lds_block(ufmt);
-        with_format<0>(ufmt, [&](auto F) { stream_blocks<decltype(F)::value>(st.mat[1].w + uat, hi - lo, udst, lane); });
-      }
-    });
-  };
-  // phase B of a stage: a row a lane, spread over the row waves; the epilogue; the results stored and published
-  auto finish = [&](const ChainStage& st, const Plan& pl) {
-    const int S = st.cols >> 8;
-    const int item = lane * kRowWaves + rw;
-    int start = 0;
-    const int nm = st.glu ? 1 : st.nmat;
-#pragma unroll
-    for (int m = 0; m < 3; m++) {
-      if (m >= nm) continue;
-      const int nrows = pl.nb[m] / S;
-      const int i = item - start;
-      start += nrows;
-      if (i < 0 || i >= nrows) continue;
-      const ChainMat& M = st.mat[m];
-      const int tper = M.fmt == ILT_Q4_K ? 2 : 1;
-      float v = sum_any(M.fmt, terms + pl.toff[m] + (long)i * S * tper, S);
-      const long r = pl.lo[m] + i;
-      if (st.glu) {
-        const int uper = st.mat[1].fmt == ILT_Q4_K ? 2 : 1;
-        const float uv = sum_any(st.mat[1].fmt, terms + pl.total * 2 + (long)i * S * uper, S);
-        v = dense_glu(v, uv);
-      } else {
-        if (M.bias) v = v + M.bias[r];
-        if (m == 0 && st.r_ll) {
-          const u32 want = base + st.r_tag;
-          u64 wv = ll_load(st.r_ll + r);
-          for (int spins = 1; (u32)(wv >> 32) != want && !failed; wv = ll_load(st.r_ll + r), spins++)
-            if ((spins & 1023) == 0 && (spins > kChainSpin || ll_flag(err))) { failed = true; atomicOr(err, 2u); }
-          v = __uint_as_float((u32)wv) + v;
-        } else if (m == 0 && st.r_plain) {
-          v = st.r_plain[r] + v;
-        }
-      }
-      if (M.y) M.y[r] = v;
-      if (M.y_ll) ll_store(M.y_ll + r, base + st.out_tag, v);
-    }
-  };
-
-  Plan cur;
-  if (!stager) {
-    plan_of(stages[0], cur);
-    prefetch(stages[0], cur);
-  }
-  for (int si = 0; si < nstages; si++) {
-    const ChainStage& st = stages[si];
-    const int S = st.cols >> 8;
-    if (stager) {
-      // ---- the input: polled (or loaded), normalized, quantized ----
-      const int gq = lane >> 4, l = lane & 15;
-      const u32 want = base + st.x_tag;
-      const int npass = (S + 4 * kStagers - 1) / (4 * kStagers);
-      double sq = 0.0;                                  // a norm stage: this lane's squares (one pass: S <= 16)
-      for (int pass = 0; pass < npass; pass++) {
-        const int b = 4 * wave + 4 * kStagers * pass + gq;
-        const bool live = b < S;
-        float4 t4[4];
-#pragma unroll
-        for (int i = 0; i < 4; i++) t4[i] = make_float4(0.f, 0.f, 0.f, 0.f);
-        if (live && st.x_plain) {
-#pragma unroll
-          for (int i = 0; i < 4; i++) t4[i] = *(const float4*)(st.x_plain + b * 256 + 4 * (l + 16 * i));
-        } else if (live) {
-          const u64* src = st.x_ll + b * 256 + 4 * l;
-          u64 wv[16];
-          bool ok = false;
-          for (int spins = 0; !ok; spins++) {
-#pragma unroll
-            for (int i = 0; i < 4; i++)
-#pragma unroll
-              for (int c = 0; c < 4; c++) wv[4 * i + c] = ll_load(src + 64 * i + c);
-            ok = true;
-#pragma unroll
-            for (int k = 0; k < 16; k++) ok = ok && (u32)(wv[k] >> 32) == want;
-            // gives up at the limit, or soon after any wave anywhere has
-            if (!ok && (failed || ((spins & 1023) == 1023 && (spins > kChainSpin || ll_flag(err))))) { atomicOr(err, 1u); failed = true; ok = true; }
-          }
-#pragma unroll
-          for (int i = 0; i < 4; i++)
-            t4[i] = make_float4(__uint_as_float((u32)wv[4 * i]), __uint_as_float((u32)wv[4 * i + 1]), __uint_as_float((u32)wv[4 * i + 2]),
-                                __uint_as_float((u32)wv[4 * i + 3]));
-        }
-        if (st.norm_w) {
-          sq += (sq4(t4[0]) + sq4(t4[1])) + (sq4(t4[2]) + sq4(t4[3]));
-          if (live) {
-#pragma unroll
-            for (int i = 0; i < 4; i++) *(float4*)(xf + b * 256 + 4 * (l + 16 * i)) = t4[i];
-          }
-        } else {
-          q8k_pass<XP, kStagers>(nullptr, S, pass, t4, lxq, lxs, lbs, nullptr, nullptr, 1.0f, nullptr);
-        }
-      }
-      if (st.norm_w) {
-        const float nscale = norm_scale_chain(sq, xf, st.cols, st.eps, st.norm_seq, red);
-        const int b = 4 * wave + gq;
-        float4 t4[4];
-#pragma unroll
-        for (int i = 0; i < 4; i++) t4[i] = b < S ? *(const float4*)(xf + b * 256 + 4 * (l + 16 * i)) : make_float4(0.f, 0.f, 0.f, 0.f);
-        q8k_pass<XP, kStagers>(nullptr, S, 0, t4, lxq, lxs, lbs, st.norm_w, nullptr, nscale, nullptr);
-      }
-      ilt_barrier_lds();                                // A
-      ilt_barrier_lds();                                // B
-    } else {
-      if (st.norm_w) { ilt_barrier_lds(); ilt_barrier_lds(); ilt_barrier_lds(); }      // in step with norm_scale_chain
-      ilt_barrier_lds();                                // A: the activations are staged
-      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's blocks have landed
-      const Lds L = { lxq, lxs, lbs, nullptr };
-      for_segments(cur, [&](int m, int lo, int hi) {
-        const int fmt = st.mat[m].fmt;
-        with_format<0>(fmt, [&](auto F) {
-          wave_blocks_lds<decltype(F)::value>(wroom + cur.woff[m], lo, hi, S, st.s_magic, L, terms + cur.toff[m], lane);
-        });
-        if (st.glu) {
-          const int ufmt = st.mat[1].fmt;
-          with_format<0>(ufmt, [&](auto F) {
-            wave_blocks_lds<decltype(F)::value>(wroom + cur.up_off, lo, hi, S, st.s_magic, L, terms + cur.total * 2, lane);
-          });
-        }
-      });
-      ilt_barrier_lds();                                // B: the terms are written, the blocks' room is free
-      finish(st, cur);
-      if (si + 1 < nstages) {
-        plan_of(stages[si + 1], cur);
-        prefetch(stages[si + 1], cur);
-      }
-    }
-  }
-}
-
 size_t gemv_smem(int fset, const IltGemvParams& p) {
   const bool q8 = fset == ILT_Q8_0;
   const int S = q8 ? p.cols / 32 : p.cols / 256;
@@ -1449,131 +1157,6 @@ static hipError_t gemv_stream_launch(IltGemvParams& p, int fset, int nz, hipStre
   }
   g_streamed_launches++;
   return hipGetLastError();
-}
-
-// ---- the chain's host side ------------------------------------------------------------------------------
-struct IltChain {
-  ChainStage* d_stages = nullptr;
-  u64* d_words = nullptr;               // every exchanged output, one 8-byte word a row
-  u32* d_err = nullptr;
-  size_t words = 0;
-  int nstages = 0, smax = 0, tmax = 0, xfmax = 0, grid = 0;
-  size_t smem = 0;
-  u32 next_base = 0;
-};
-
-hipError_t ilt_k_chain_destroy(IltChain* c) {
-  if (!c) return hipSuccess;
-  (void)hipFree(c->d_stages); (void)hipFree(c->d_words); (void)hipFree(c->d_err);
-  delete c;
-  return hipSuccess;
-}
-
-hipError_t ilt_k_chain_create(const ilt_chain_stage* in, int n, IltChain** out) {
-  if (!in || !out || n < 1 || n > 4096) return hipErrorInvalidValue;
-  int dev = 0, cus = 0;
-  hipError_t e = hipGetDevice(&dev);
-  if (e != hipSuccess) return e;
-  e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
-  if (e != hipSuccess) return e;
-  const int G = cus < 256 ? cus : 256;
-  if (G < 1) return hipErrorInvalidValue;
-  std::vector<ChainStage> st(n);
-  std::vector<size_t> word_off((size_t)n * 3, (size_t)-1);      // where output (stage, mat) is exchanged, if anybody reads it
-  size_t words = 0;
-  auto need = [&](int s, int m) { size_t& o = word_off[(size_t)s * 3 + m]; if (o == (size_t)-1) { o = words; words += (size_t)in[s].mat[in[s].glu ? 0 : m].rows; } };
-  for (int i = 0; i < n; i++) {
-    const ilt_chain_stage& a = in[i];
-    if (a.nmat < 1 || a.nmat > 3 || a.cols < 256 || a.cols % 256 || (a.glu && a.nmat != 2)) return hipErrorInvalidValue;
-    const int S = a.cols / 256;
-    if (S > 48 || (a.norm_w && S > 4 * kStagers)) return hipErrorInvalidValue;
-    for (int m = 0; m < a.nmat; m++) {
-      const ilt_mv_desc& d = a.mat[m];
-      if ((d.gguf_type != ILT_Q4_K && d.gguf_type != ILT_Q6_K) || d.rows < 1 || !d.w || ((uintptr_t)d.w & 15)) return hipErrorInvalidValue;
-      if (a.glu && d.rows != a.mat[0].rows) return hipErrorInvalidValue;
-    }
-    const int nout = a.glu ? 1 : a.nmat;
-    if (a.x_stage >= i || a.x_stage < -1 || (a.x_stage >= 0 && (a.x_mat < 0 || a.x_mat >= (in[a.x_stage].glu ? 1 : in[a.x_stage].nmat)))) return hipErrorInvalidValue;
-    if (a.x_stage < 0 ? (!a.x_in || ((uintptr_t)a.x_in & 15)) : in[a.x_stage].mat[a.x_mat].rows != a.cols) return hipErrorInvalidValue;
-    if (a.r_stage >= i || a.r_stage < -2 || (a.glu && a.r_stage != -1)) return hipErrorInvalidValue;
-    if (a.r_stage >= 0 && (a.r_mat < 0 || a.r_mat >= (in[a.r_stage].glu ? 1 : in[a.r_stage].nmat) || in[a.r_stage].mat[a.r_mat].rows != a.mat[0].rows)) return hipErrorInvalidValue;
-    if (a.r_stage == -2 && !a.r_in) return hipErrorInvalidValue;
-    if (a.norm_w && ((uintptr_t)a.norm_w & 15)) return hipErrorInvalidValue;
-    if (a.x_stage >= 0) need(a.x_stage, a.x_mat);
-    if (a.r_stage >= 0) need(a.r_stage, a.r_mat);
-    (void)nout;
-  }
-  IltChain* c = new IltChain;
-  c->nstages = n; c->grid = G; c->words = words;
-  e = hipMalloc((void**)&c->d_stages, sizeof(ChainStage) * n);
-  if (e == hipSuccess) e = hipMalloc((void**)&c->d_words, 8 * (words ? words : 1));
-  if (e == hipSuccess) e = hipMalloc((void**)&c->d_err, 256);
-  if (e == hipSuccess) e = hipMemset(c->d_words, 0, 8 * (words ? words : 1));
-  if (e == hipSuccess) e = hipMemset(c->d_err, 0, 256);
-  if (e != hipSuccess) { (void)ilt_k_chain_destroy(c); return e; }
-  size_t wmax = 0;
-  for (int i = 0; i < n; i++) {
-    const ilt_chain_stage& a = in[i];
-    ChainStage& s = st[i];
-    memset(&s, 0, sizeof(s));
-    const int S = a.cols / 256;
-    size_t wbytes = 0; int tfl = 0;
-    for (int m = 0; m < a.nmat; m++) {
-      const ilt_mv_desc& d = a.mat[m];
-      ChainMat& M = s.mat[m];
-      M.w = (const u8*)d.w; M.y = d.y; M.bias = d.bias; M.rows = d.rows; M.fmt = d.gguf_type;
-      M.row_bytes = (long long)S * (d.gguf_type == ILT_Q4_K ? 144 : ILT_Q6K_STRIDE);
-      const size_t o = word_off[(size_t)i * 3 + (a.glu ? 0 : m)];
-      M.y_ll = (o == (size_t)-1 || (a.glu && m)) ? nullptr : c->d_words + o;
-      const int per_cu = (d.rows + G - 1) / G;
-      wbytes += (size_t)per_cu * S * (d.gguf_type == ILT_Q4_K ? 144 : 224);
-      tfl += per_cu * S * 2;
-    }
-    if (wbytes > wmax) wmax = wbytes;
-    if (tfl > c->tmax) c->tmax = tfl;
-    if (S > c->smax) c->smax = S;
-    if (a.norm_w && a.cols > c->xfmax) c->xfmax = a.cols;
-    s.nmat = a.nmat; s.glu = a.glu; s.cols = a.cols; s.norm_w = a.norm_w; s.eps = a.eps; s.norm_seq = a.exact_order ? 1 : 0;
-    if (a.x_stage < 0) s.x_plain = a.x_in; else { s.x_ll = c->d_words + word_off[(size_t)a.x_stage * 3 + a.x_mat]; s.x_tag = (u32)a.x_stage + 1; }
-    if (a.r_stage >= 0) { s.r_ll = c->d_words + word_off[(size_t)a.r_stage * 3 + a.r_mat]; s.r_tag = (u32)a.r_stage + 1; }
-    else if (a.r_stage == -2) s.r_plain = a.r_in;
-    s.out_tag = (u32)i + 1;
-    s.s_magic = (uint32_t)(0x100000000ULL / (uint64_t)S) + 1;
-  }
-  c->tmax = (c->tmax + 3) & ~3;
-  c->smem = (size_t)c->smax * XP + (size_t)c->smax * 64 + (size_t)((c->smax + 3) & ~3) * 4 + (size_t)c->xfmax * 4 + 8 * kStagers +
-            (size_t)c->tmax * 4 + wmax;
-  if (c->smem > 156 * 1024) { (void)ilt_k_chain_destroy(c); return hipErrorInvalidValue; }      // a stage's share of its matrices does not fit a CU's LDS
-  e = hipFuncSetAttribute((const void*)gemv_chain_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 158 * 1024);
-  if (e == hipSuccess) e = hipMemcpy(c->d_stages, st.data(), sizeof(ChainStage) * n, hipMemcpyHostToDevice);
-  if (e != hipSuccess) { (void)ilt_k_chain_destroy(c); return e; }
-  *out = c;
-  return hipSuccess;
-}
-
-hipError_t ilt_k_chain_run(IltChain* c, hipStream_t stream) {
-  if (!c) return hipErrorInvalidValue;
-  if (c->next_base > 0xF0000000u) {            // the tags would wrap: start over from cleared words
-    const hipError_t e = hipMemsetAsync(c->d_words, 0, 8 * (c->words ? c->words : 1), stream);
-    if (e != hipSuccess) return e;
-    c->next_base = 0;
-  }
-  u32 base = c->next_base;
-  c->next_base += (u32)c->nstages + 1;
-  const ChainStage* stages = c->d_stages;
-  int n = c->nstages, smax = c->smax, tmax = c->tmax, xfmax = c->xfmax;
-  u32* err = c->d_err;
-  void* args[] = { &stages, &n, &base, &smax, &tmax, &xfmax, &err };
-  // a cooperative launch: the runtime refuses it unless every workgroup can be resident at once, which the
-  // exchange between the workgroups needs
-  return hipLaunchCooperativeKernel((const void*)gemv_chain_kernel, dim3(c->grid), dim3(kStreamThreads), args, c->smem, stream);
-}
-
-hipError_t ilt_k_chain_status(IltChain* c, hipStream_t stream, uint32_t* flags) {
-  if (!c || !flags) return hipErrorInvalidValue;
-  hipError_t e = hipMemcpyAsync(flags, c->d_err, 4, hipMemcpyDeviceToHost, stream);
-  if (e == hipSuccess) e = hipStreamSynchronize(stream);
-  return e;
 }
 
 hipError_t ilt_gemv_launch(IltGemvParams& p, int nz, hipStream_t st) {

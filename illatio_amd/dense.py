@@ -270,64 +270,3 @@ def embed(dev, emb, tokens, x, n, d):
     else:
         hip.launch(dev, "embed_q8", n, 256, [emb.qs, emb.d, tokens, x, d])
     return x
-
-
-# ---- a chain of dependent decode products in one launch (ilt_chain_*) ---------------------------------
-class ChainStageC(C.Structure):
-    _fields_ = [("nmat", C.c_int), ("glu", C.c_int), ("cols", C.c_int), ("mat", MvDesc * 3), ("x_stage", C.c_int), ("x_mat", C.c_int),
-                ("x_in", C.c_uint64), ("norm_w", C.c_uint64), ("eps", C.c_float), ("exact_order", C.c_int), ("r_stage", C.c_int),
-                ("r_mat", C.c_int), ("r_in", C.c_uint64)]
-
-
-def chain_stage(mats, x, glu=False, norm=None, resid=None, exact_order=False):
-    """One stage of a Chain.  MATS: up to three (W Y BIAS) on the same input (Y, BIAS may be None); with GLU
-    the pair gate, up, the gated activation into the first Y.  X: a DBuf of floats written before the run, or
-    (stage index, output index) of an earlier stage.  NORM = (weights DBuf, eps): rmsnorm! before the
-    quantizer.  RESID: None, a DBuf of floats, or (stage index, output index): the first matrix's result is
-    added to it (CMAT-MUL's acc)."""
-    s = ChainStageC()
-    s.nmat, s.glu, s.cols = len(mats), 1 if glu else 0, mats[0][0].cols
-    for i, (w, y, bias) in enumerate(mats):
-        if w.cols != s.cols:
-            raise ValueError("a stage's matrices share their input")
-        s.mat[i] = MvDesc(w.type, w.rows, w.qs.ptr, 0, y.ptr if y is not None else 0, bias.ptr if bias is not None else 0)
-    if isinstance(x, tuple):
-        s.x_stage, s.x_mat, s.x_in = x[0], x[1], 0
-    else:
-        s.x_stage, s.x_mat, s.x_in = -1, 0, x.ptr
-    if norm is not None:
-        s.norm_w, s.eps = norm[0].ptr, norm[1]
-    s.exact_order = 1 if exact_order else 0
-    if resid is None:
-        s.r_stage, s.r_mat, s.r_in = -1, 0, 0
-    elif isinstance(resid, tuple):
-        s.r_stage, s.r_mat, s.r_in = resid[0], resid[1], 0
-    else:
-        s.r_stage, s.r_mat, s.r_in = -2, 0, resid.ptr
-    return s
-
-
-class Chain:
-    """A table of stages made once (ilt_chain_create); run() queues one launch that walks it."""
-
-    def __init__(self, dev, stages):
-        self.dev, self.n = dev, len(stages)
-        arr = (ChainStageC * self.n)(*stages)
-        h = C.c_uint64(0)
-        hip.hip_current(dev)
-        hip.call("ilt_chain_create", C.byref(h), arr, C.c_int(self.n))
-        self.handle = h.value
-
-    def run(self):
-        hip.call("ilt_chain_run", C.c_uint64(self.dev.stream), C.c_uint64(self.handle))
-
-    def status(self):
-        """Waits for the stream; 0 unless a workgroup gave up waiting for another."""
-        f = C.c_uint32(0)
-        hip.call("ilt_chain_status", C.c_uint64(self.dev.stream), C.c_uint64(self.handle), C.byref(f))
-        return f.value
-
-    def free(self):
-        if self.handle:
-            hip.call("ilt_chain_destroy", C.c_uint64(self.handle))
-            self.handle = 0

@@ -178,40 +178,6 @@ int ilt_rmsnorm_q8k(uint64_t stream, const float* x, const float* w, float* h, i
 int ilt_mv_multi_norm(uint64_t stream, int nmat, const ilt_mv_desc* descs, int cols, const float* x, const float* norm_w,
                       float eps, int exact_order, int f16_scale, int glu);
 
-/* A chain of dependent decode products in one launch.  One token's products at batch one feed one
-   another (cuda-forward-n, cuda-dense.lisp:380-432: Q/K/V -> attention -> wo with acc -> norm ->
-   glu -> down with acc -> the next layer), and as launches of their own each costs about 3 us
-   before its first instruction.  A chain is a table of stages, made once; running it is one launch of
-   a grid that stays resident, exchanges each stage's output between its workgroups through memory
-   and streams the next stage's matrix into LDS meanwhile.  No counterpart in the reference.
-   A stage = up to three Q4_K / Q6_K matrices on the same input of cols floats (mat[i].y may be null
-   when only later stages read the result), or with glu the pair gate, up ending in swiglu!
-   (model.lisp:364-378) into mat[0].y.  Its input is output x_mat of the earlier stage x_stage, or
-   with x_stage -1 the floats x_in (written before the launch); with norm_w it goes through rmsnorm!
-   (model.lisp:205-216; exact_order as in ilt_mv_multi_norm) before quantize-q8k!.  r_stage >= 0:
-   mat[0]'s result is added to output r_mat of stage r_stage (cmat-mul's acc: the residual
-   stream); -2: to the floats r_in; -1: nothing.  Every product has the decode kernels' bits.
-   cols <= 12288 (4096 with a norm); each stage's share of its matrices must fit a CU's LDS
-   (rows * row bytes / 256 CUs below about 110 KB), else create returns hipErrorInvalidValue.
-   ilt_chain_run queues the launch on stream and returns; runs of one chain must not overlap.
-   ilt_chain_status waits for stream and returns 0 in *flags, or non-zero if a workgroup gave up
-   waiting for another (the results are then wrong; never seen unless the GPU is shared). */
-typedef struct ilt_chain_stage {
-  int nmat, glu, cols;
-  ilt_mv_desc mat[3];
-  int x_stage, x_mat;
-  const float* x_in;
-  const float* norm_w;
-  float eps;
-  int exact_order;
-  int r_stage, r_mat;
-  const float* r_in;
-} ilt_chain_stage;
-int ilt_chain_create(uint64_t* chain, const ilt_chain_stage* stages, int nstages);
-int ilt_chain_run(uint64_t stream, uint64_t chain);
-int ilt_chain_status(uint64_t stream, uint64_t chain, uint32_t* flags);
-int ilt_chain_destroy(uint64_t chain);
-
 /* Diagnostic: how many decode products this process has launched as the streamed variant (the
    one that sends every wave's rows to LDS at once; chosen by shape for Q4_K / Q6_K products of
    2 MB and more whose share fits a CU's LDS).  No counterpart in the reference. */
