@@ -420,7 +420,6 @@ def moe_weights(rng, ne_unique, ne, d, ff):
 
 def workload_c4(args, dev):
     from illatio_amd import ds4f, hip, synth
-    import oracle_lib as orc
     rng = synth.make_rng(44)
     ne, nu, d, ff, nlayers = 256, 6, 4096, 2048, 3
     gate, up, down = moe_weights(rng, 32, ne, d, ff)
@@ -436,11 +435,16 @@ def workload_c4(args, dev):
     logits = []
     for i in range(nsteps):                      # the reference routes on the CPU (cuda-ds4f.lisp:991-999); tables made beforehand
         lg = synth.activations(ne, rng)
-        sel, w = orc.route(lg, nu, 1.5)
-        routes.append((sel, w))
+        lgb = hip.hip_upload_new(dev, lg)
         if ondev:                                # device mode: only the router's logits are resident; d4_route runs in the step
-            logits.append(hip.hip_upload_new(dev, lg))
-        else:
+            logits.append(lgb)
+            routes.append(None)
+        else:                                    # the tables of the host-routed modes, made by d4_route ahead of the timed steps
+            dsel, dw = ds4f.route(dev, lgb, 1, ne, nu, 1.5)
+            sel, w = hip.hip_download(dsel, np.uint32, nu).astype(np.int32), hip.hip_floats(dw, nu)
+            for b in (lgb, dsel, dw):
+                hip.hip_free(b)
+            routes.append((sel, w))
             tables.append((ds4f.fused_tables if fused else ds4f.tail_tables)(dev, pools[i % nlayers], sel, w))
     ws = hip.Workspace(dev, 8 << 20)
     iq, q2, q8 = synth.row_bytes(synth.IQ2_XXS, d), synth.row_bytes(synth.Q2_K, ff), 34
@@ -450,7 +454,7 @@ def workload_c4(args, dev):
     def step(i):
         ws.reset()
         L = i % nlayers
-        sel, w = routes[i]
+        sel, w = routes[i] if routes[i] else (None, None)
         if ondev:
             ds4f.ffn_step_device(dev, pools[L], shared[L], logits[i], xb, ne, nu, 1.5, 0.0, ws=ws)
         elif fused:
@@ -481,10 +485,12 @@ def workload_c4(args, dev):
     gbs = step_bytes / (ms * 1e-3) / 1e9
 
     def cpu():
+        import oracle_lib as orc
         cores = host_cores()
+        crng = synth.make_rng(45)
         t1, reps = time.perf_counter(), 0
         while time.perf_counter() - t1 < 10.0:
-            sel, w = routes[reps % len(routes)]
+            sel, w = orc.route(synth.activations(ne, crng), nu, 1.5)
             orc.moe_routed(gate, up, down, d, ff, sel, w, 0.0, x, nthreads=cores)
             orc.moe_shared(sg, su, sd, d, ff, 0.0, x, nthreads=cores)
             reps += 1
@@ -502,7 +508,6 @@ def workload_c4(args, dev):
 
 def workload_c5(args, dev):
     from illatio_amd import ds4f, hip, synth
-    import oracle_lib as orc
     rng = synth.make_rng(55)
     ne, nu, d, ff, n = 256, 6, 4096, 2048, args.tokens
     gate, up, down = moe_weights(rng, 32, ne, d, ff)
@@ -543,6 +548,7 @@ def workload_c5(args, dev):
     tf = flops / (ms * 1e-3) / 1e12
 
     def cpu():
+        import oracle_lib as orc
         cores = host_cores()
         ts = 8
         t1, reps = time.perf_counter(), 0
@@ -569,7 +575,8 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="c2", choices=sorted(WORKLOADS))
+    ap.add_argument("--workload", default=None, choices=sorted(WORKLOADS),
+                    help="one workload only; default: c2 (the line's value) and then c1, c3, c4, c5 under \"configs\"")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--layers", type=int, default=LAYERS, help=argparse.SUPPRESS)
     ap.add_argument("--tokens", type=int, default=4096, help="c3, c5: tokens per step")
@@ -592,6 +599,9 @@ def main():
 
     from illatio_amd import hip
     dev = hip.open_hip(0)
+    everything = args.workload is None
+    if everything:
+        args.workload = "c2"
     r = WORKLOADS[args.workload](args, dev)
     out = {"metric": r.get("metric", "Q-matvec achieved HBM GB/s (% of 8 TB/s); decode tok/s at Qwen3-4B shape"),
            "value": r["value"], "unit": r["unit"], "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -602,6 +612,28 @@ def main():
     out["host_enqueue_ms_per_step"] = round(r["enqueue_ms"], 4)
     out["roofline"] = r["roofline"]
     out["cpu_baseline"] = None if args.no_cpu else r["cpu"]()
+    if everything:
+        # BASELINE's other configurations on the same clock (no CPU leg): c4 with the routing on the device, c3 and
+        # c5 on the bf16 matrix cores at 4096 tokens and, as a second entry each, on the bit-exact int8 path
+        import copy
+        import gc
+        out["configs"] = {}
+        extras = [("c1", {}), ("c3", {"path": "bf16", "tokens": 4096}), ("c3_exact", {"path": "int8", "tokens": 4096}),
+                  ("c4", {"mode": "device"}), ("c5", {"path": "bf16", "tokens": 4096}), ("c5_exact", {"path": "int8", "tokens": 4096})]
+        for name, over in extras:
+            a = copy.copy(args)
+            a.workload, a.steps, a.warmup = name[:2], min(args.steps, 10), min(args.warmup, 3)
+            for k, v in over.items():
+                setattr(a, k, v)
+            del r
+            gc.collect()
+            r = WORKLOADS[a.workload](a, dev)
+            roof = r["roofline"]
+            out["configs"][name] = {
+                "workload": r["config"]["workload"], "value": r["value"], "unit": r["unit"], "ms_per_step": round(r["ms_per_step"], 4),
+                "steps": a.steps, "warmup": a.warmup, "dtype": r["dtype"],
+                "roofline": {k: roof.get(k) for k in ("bound", "achieved", "peak", "unit", "frac", "traffic", "kernel", "launches", "avg_launch_us",
+                                                      "launch_us_all", "other_kernels")}}
     print(json.dumps(out))
     return 0
 
