@@ -10,6 +10,7 @@
 #include "ilt_kernels.h"
 
 #define ILT_TRY(expr) do { hipError_t e_ = (expr); if (e_ != hipSuccess) return (int)e_; } while (0)
+#define ILT_MAX_DEVICES 64
 #define ILT_REQUIRE(cond) do { if (!(cond)) return (int)hipErrorInvalidValue; } while (0)
 
 static inline hipStream_t S(uint64_t s) { return (hipStream_t)(uintptr_t)s; }
@@ -490,7 +491,6 @@ static __device__ __align__(256) __attribute__((used)) unsigned char scratch[ILT
 // The array's address on each device, asked of the runtime once per device with that device
 // current.  In host code the name `scratch` is a stand-in for the symbol, not a device address:
 // only these pointers go to kernels.
-#define ILT_MAX_DEVICES 64
 static void* g_scratch_ptr[ILT_MAX_DEVICES];
 
 static int step_scratch(uint8_t** out) {
@@ -584,6 +584,73 @@ int ilt_d4_mm_id_q2_k(uint64_t stream, int ncols, int nrows, int row_bytes, int6
                       const uint32_t* counts, const uint32_t* bases, int ne, int64_t total_rows,
                       const int8_t* xq, const float* xd, const int32_t* bsums, float* y) {
   return mm_id(stream, ILT_Q2_K, ncols, nrows, row_bytes, add, ptrs, counts, bases, ne, total_rows, xq, xd, bsums, y);
+}
+
+// ---- d4_mm_<format>: one matrix on a chunk of tokens' float activations (ds4f_mm.cu:252-255) ----------
+// The reference's kernels round weights and activations to halves; these quantize the activations as the CPU
+// path does and run the exact products, so the quantized activations need room: a buffer per device that only
+// ever grows, kept until the process ends.  Calls that overlap on one GPU (two streams) would share it: the
+// reference's host issues these on one stream.
+namespace {
+struct QRoom { void* p; size_t bytes; };
+QRoom g_qroom[ILT_MAX_DEVICES];
+int qroom(size_t bytes, uint8_t** out) {
+  int dev = -1;
+  ILT_TRY(hipGetDevice(&dev));
+  ILT_REQUIRE(dev >= 0 && dev < ILT_MAX_DEVICES);
+  QRoom& q = g_qroom[dev];
+  if (q.bytes < bytes) {
+    if (q.p) ILT_TRY(hipFree(q.p));                      // (waits for the work that still reads it)
+    q.p = nullptr; q.bytes = 0;
+    const size_t want = bytes + bytes / 4 + (1 << 20);
+    ILT_TRY(hipMalloc(&q.p, want));
+    q.bytes = want;
+  }
+  *out = (uint8_t*)q.p;
+  return ILT_OK;
+}
+int d4_mm_quantized(uint64_t stream, int fmt, int ncols, int nrows, int ntok, int row_bytes, int x_stride, int y_stride, const void* w,
+                    const uint16_t* wd, const float* x, float* y) {
+  const int bw = block_weights(fmt);
+  ILT_REQUIRE(ncols > 0 && ncols % bw == 0 && nrows >= 0 && ntok >= 0);
+  if (nrows == 0 || ntok == 0) return ILT_OK;
+  ILT_REQUIRE(w && x && y && ((uintptr_t)w & 15) == 0 && ((uintptr_t)x & 15) == 0);
+  if (x_stride != ncols || y_stride != nrows) return (int)hipErrorNotSupported;       // tokens' rows one after another only
+  const size_t n = (size_t)ntok * ncols;
+  const size_t qb = (n + 255) / 256 * 256, sb = (n / bw * 4 + 255) / 256 * 256, bb = fmt == ILT_Q8_0 ? 0 : (n / 16 * 4 + 255) / 256 * 256;
+  uint8_t* room = nullptr;
+  ILT_TRY((hipError_t)qroom(qb + sb + bb, &room));
+  int8_t* xq = (int8_t*)room; float* xs = (float*)(room + qb); int32_t* bs = (int32_t*)(room + qb + sb);
+  if (fmt == ILT_Q8_0) {
+    // d4-shared!'s and the attention projections' activations: quantize-q8! with the scale kept a float (ds4f.lisp:1052-1053)
+    ILT_REQUIRE(wd && (row_bytes == 0 || row_bytes == ncols));
+    ILT_TRY(ilt_k_quant_q8(x, xq, xs, nullptr, (long long)(n / 32), 0, S(stream)));
+    return (int)ilt_k_gemm_i8(ILT_Q8_0, (const uint8_t*)w, wd, ncols, nrows, ncols, xq, xs, nullptr, ntok, y, nullptr, 0, S(stream));
+  }
+  ILT_REQUIRE(row_bytes == ncols / 256 * block_bytes(fmt));
+  ILT_TRY(ilt_k_quant_q8k(x, xq, xs, bs, (long long)(n / 256), S(stream)));
+  return (int)ilt_k_gemm_i8(fmt, (const uint8_t*)w, nullptr, row_bytes, nrows, ncols, xq, xs, bs, ntok, y, nullptr, 0, S(stream));
+}
+}  // namespace
+
+int ilt_d4_mm_q8_0(uint64_t stream, int ncols, int nrows, int ntok, int row_bytes, int x_stride, int y_stride, const int8_t* w,
+                   const uint16_t* wd, const float* x, float* y) {
+  return d4_mm_quantized(stream, ILT_Q8_0, ncols, nrows, ntok, row_bytes, x_stride, y_stride, w, wd, x, y);
+}
+int ilt_d4_mm_q2_k(uint64_t stream, int ncols, int nrows, int ntok, int row_bytes, int x_stride, int y_stride, const void* w,
+                   const float* x, float* y) {
+  return d4_mm_quantized(stream, ILT_Q2_K, ncols, nrows, ntok, row_bytes, x_stride, y_stride, w, nullptr, x, y);
+}
+int ilt_d4_mm_iq2_xxs(uint64_t stream, int ncols, int nrows, int ntok, int row_bytes, int x_stride, int y_stride, const void* w,
+                      const float* x, float* y) {
+  return d4_mm_quantized(stream, ILT_IQ2_XXS, ncols, nrows, ntok, row_bytes, x_stride, y_stride, w, nullptr, x, y);
+}
+int ilt_d4_mm_f16(uint64_t stream, int ncols, int nrows, int ntok, int row_bytes, int x_stride, int y_stride, const uint16_t* w,
+                  const float* x, float* y) {
+  ILT_REQUIRE(ncols > 0 && ncols % 16 == 0 && nrows >= 0 && ntok >= 0 && row_bytes >= 2 * ncols && row_bytes % 2 == 0);
+  if (nrows == 0 || ntok == 0) return ILT_OK;
+  ILT_REQUIRE(w && x && y && x_stride >= ncols && y_stride >= nrows);
+  return (int)ilt_k_mm_f16(ncols, nrows, ntok, row_bytes / 2, x_stride, y_stride, w, x, y, S(stream));
 }
 
 static int bf16_type(int t) { return (t == ILT_Q2_K || t == ILT_Q4_K || t == ILT_Q6_K || t == ILT_IQ2_XXS) ? t : 0; }
@@ -726,6 +793,10 @@ int ilt_launch(const char* kernel, unsigned gx, unsigned gy, unsigned gz, unsign
     return ilt_d4_mm_id_glu_bf16(stream, a.i32(0), a.i32(1), a.i32(2), a.i32(3), a.i64(4), a.i64(5), a.ptr<const uint64_t*>(6), a.ptr<cu32>(7),
                                  a.ptr<cu32>(8), a.i32(9), a.i64(10), a.ptr<cu16>(11), a.ptr<cu32>(12), a.f32(13), a.ptr<cf>(14), a.ptr<uint16_t*>(15));
   K("d4_swiglu_w_bf16") return ilt_d4_swiglu_w_bf16(stream, a.i32(0), a.i32(1), a.f32(2), a.ptr<cf>(3), a.ptr<cf>(4), a.ptr<cf>(5), a.ptr<uint16_t*>(6));
+  K("d4_mm_q8_0") return ilt_d4_mm_q8_0(stream, a.i32(0), a.i32(1), a.i32(2), a.i32(3), a.i32(4), a.i32(5), a.ptr<ci8>(6), a.ptr<cu16>(7), a.ptr<cf>(8), a.ptr<float*>(9));
+  K("d4_mm_f16") return ilt_d4_mm_f16(stream, a.i32(0), a.i32(1), a.i32(2), a.i32(3), a.i32(4), a.i32(5), a.ptr<cu16>(6), a.ptr<cf>(8), a.ptr<float*>(9));
+  K("d4_mm_q2_k") return ilt_d4_mm_q2_k(stream, a.i32(0), a.i32(1), a.i32(2), a.i32(3), a.i32(4), a.i32(5), a.ptr<const void*>(6), a.ptr<cf>(8), a.ptr<float*>(9));
+  K("d4_mm_iq2_xxs") return ilt_d4_mm_iq2_xxs(stream, a.i32(0), a.i32(1), a.i32(2), a.i32(3), a.i32(4), a.i32(5), a.ptr<const void*>(6), a.ptr<cf>(8), a.ptr<float*>(9));
   K("d4_mm_id_iq2_xxs")
     return ilt_d4_mm_id_iq2_xxs(stream, a.i32(0), a.i32(1), a.i32(2), a.i64(5), a.ptr<const uint64_t*>(6), a.ptr<cu32>(7),
                                 a.ptr<cu32>(8), (int)gz, a.i64(13), a.ptr<ci8>(9), a.ptr<cf>(11), a.ptr<float*>(10));

@@ -69,6 +69,8 @@ hipError_t ilt_k_quant_q8k(const float* x, int8_t* xq, float* xd, int* bsums, lo
 // rmsnorm! then quantize-q8! (k 0; xsum may be null) or quantize-q8k! (k 1), a row of DIM floats a workgroup
 hipError_t ilt_k_rmsnorm_quant(int k, const float* x, const float* w, float* h, int8_t* xq, float* xs, int* xsum, int dim,
                                float eps, int f16_scale, int seq, int nrows, hipStream_t st);
+hipError_t ilt_k_mm_f16(int ncols, int nrows, int ntok, long long row_halfs, int x_stride, int y_stride, const uint16_t* w, const float* x,
+                        float* y, hipStream_t st);
 hipError_t ilt_k_repack_q8(const uint8_t* raw, int8_t* qs, uint16_t* d, long long nblocks, hipStream_t st);
 hipError_t ilt_k_repack_q6k(const uint8_t* raw, uint8_t* out, long long nblocks, hipStream_t st);
 hipError_t ilt_k_copy_bytes(const uint8_t* src, uint8_t* dst, long long bytes, hipStream_t st);

@@ -166,6 +166,47 @@ __global__ __launch_bounds__(256) void dequant_rows_kernel(int fmt, const u8* __
     out[n * cols + col] = dequant_one(fmt, wrow, wdrow, col);
 }
 
+
+// y[t*y_stride + r] = W[r] . x[t*x_stride ..] for an F16 matrix and float activations (the router's product,
+// ds4f_mm.cu:253; CPU: f32mm!, ds4f.lisp:278-293).  Each dot is F32-DOT16's (tensor.lisp:370-378): column i's
+// product, rounded to a float, is added to partial sum i mod 16; the sixteen sums meet as
+// c(j) = (s[j] + s[4+j]) + (s[8+j] + s[12+j]), (c(0) + c(1)) + (c(2) + c(3)) -- the CPU's bits.
+// 16 lanes a row (lane l = partial sum l), 16 rows a workgroup, 16 tokens a workgroup whose activations go
+// through LDS 256 columns at a time; a thread keeps its 16 tokens' partial sums.
+__global__ __launch_bounds__(256) void mm_f16_dot16_kernel(int ncols, int nrows, int ntok, long long row_halfs, int x_stride, int y_stride,
+                                                           const u16* __restrict__ w, const float* __restrict__ x, float* __restrict__ y) {
+  __shared__ float xs[16][256];
+  const int l = threadIdx.x & 15, rl = threadIdx.x >> 4;
+  const int r = blockIdx.y * 16 + rl, t0 = blockIdx.x * 16;
+  const u16* wr = w + (long long)min(r, nrows - 1) * row_halfs;
+  float acc[16];
+#pragma unroll
+  for (int tt = 0; tt < 16; tt++) acc[tt] = 0.0f;
+  for (int c0 = 0; c0 < ncols; c0 += 256) {
+    const int nc = min(256, ncols - c0);                   // a multiple of 16
+    __syncthreads();
+    for (int i = threadIdx.x; i < 16 * 256; i += 256) {
+      const int tt = i >> 8, c = i & 255;
+      xs[tt][c] = (t0 + tt < ntok && c < nc) ? x[(long long)(t0 + tt) * x_stride + c0 + c] : 0.0f;
+    }
+    __syncthreads();
+    for (int jj = 0; jj < nc; jj += 16) {
+      const float wv = ilt_h2f(wr[c0 + jj + l]);
+#pragma unroll
+      for (int tt = 0; tt < 16; tt++) acc[tt] = acc[tt] + wv * xs[tt][jj + l];
+    }
+  }
+#pragma unroll
+  for (int tt = 0; tt < 16; tt++) {
+    float a = acc[tt];
+    a = a + ilt_dppf<ILT_DPP_SHL(4)>(a);                   // lanes 0-3 and 8-11: s[l] + s[l+4]
+    a = a + ilt_dppf<ILT_DPP_SHL(8)>(a);                   // lanes 0-3: c(l)
+    a = a + ilt_dppf<ILT_DPP_SHL(1)>(a);                   // lanes 0, 2: c(0)+c(1), c(2)+c(3)
+    a = a + ilt_dppf<ILT_DPP_SHL(2)>(a);                   // lane 0: the dot
+    if (l == 0 && r < nrows && t0 + tt < ntok) y[(long long)(t0 + tt) * y_stride + r] = a;
+  }
+}
+
 }  // namespace
 
 hipError_t ilt_k_quant_q8(const float* x, int8_t* xq, float* xs, int* xsum, long long nblocks, int f16_scale, hipStream_t st) {
@@ -209,5 +250,14 @@ hipError_t ilt_k_dequant_rows(int fmt, const uint8_t* w, const uint16_t* wd, con
                        rows_idx ? rows_idx + n0 : nullptr, cols, row_bytes, out + n0 * cols);
     if (!rows_idx) w += 65535 * row_bytes, wd = wd ? wd + 65535LL * (cols >> 5) : nullptr;
   }
+  return hipGetLastError();
+}
+
+hipError_t ilt_k_mm_f16(int ncols, int nrows, int ntok, long long row_halfs, int x_stride, int y_stride, const uint16_t* w, const float* x,
+                        float* y, hipStream_t st) {
+  if (nrows <= 0 || ntok <= 0) return hipSuccess;
+  if (ncols <= 0 || ncols % 16) return hipErrorInvalidValue;
+  hipLaunchKernelGGL(mm_f16_dot16_kernel, dim3((ntok + 15) / 16, (nrows + 15) / 16), dim3(256), 0, st, ncols, nrows, ntok, row_halfs, x_stride,
+                     y_stride, w, x, y);
   return hipGetLastError();
 }

@@ -98,6 +98,33 @@ def ffn_shared(dev, sh, norm2, clamp, n=1, ws=None):
     return sout
 
 
+def dk_mm(dev, kernel, w, wd, rbytes, rows, cols, x, y, n, x_stride=None, y_stride=None):
+    """Y (N rows, Y-STRIDE apart) = W X (N rows, X-STRIDE apart): D4_MM_<format> (DK-MM, cuda-ds4f-prefill.lisp:65-68)."""
+    hip.launch(dev, kernel, ((n + 63) // 64, (rows + 63) // 64), 128,
+               [cols, rows, n, rbytes, cols if x_stride is None else x_stride, rows if y_stride is None else y_stride, w, wd, x, y])
+
+
+def ffn_shared_chunk(dev, sh, norm2, n, clamp, ws=None):
+    """The shared expert of a chunk of N tokens (DK-FFN-HEAD-CHUNK's second half, cuda-ds4f-prefill.lisp:294-298):
+    gate and up through D4_MM_Q8_0 on the float rows, the gated activation, down through D4_MM_Q8_0.  Each token's
+    row has d4-shared!'s bits.  Returns SOUT (N x d)."""
+    d, ff = sh.d, sh.ff
+    A = ws.alloc if ws else hip.hip_alloc
+    sg, su, smid, sout = A(dev, 4 * n * ff), A(dev, 4 * n * ff), A(dev, 4 * n * ff), A(dev, 4 * n * d)
+    if getattr(sh, "ones", None) is None or sh.ones.bytes < 4 * n:
+        sh.ones = hip.hip_upload_new(dev, np.ones(n, np.float32))
+    dk_mm(dev, "d4_mm_q8_0", sh.gate.qs, sh.gate.d, 0, ff, d, norm2, sg, n)
+    dk_mm(dev, "d4_mm_q8_0", sh.up.qs, sh.up.d, 0, ff, d, norm2, su, n)
+    hip.launch(dev, "d4_swiglu_w", (n * ff + 255) // 256, 256, [n, ff, float(clamp), sg, su, sh.ones, smid, None, None])
+    dk_mm(dev, "d4_mm_q8_0", sh.down.qs, sh.down.d, 0, d, ff, smid, sout, n)
+    if ws:
+        return sout
+    hip.hip_sync(dev)
+    for b in (sg, su, smid):
+        hip.hip_free(b)
+    return sout
+
+
 def tail_tables(dev, pool, sel, w):
     """The device tables DK-FFN-TAIL's kernels take for one token: the 2k matrix addresses
     (the selected experts' gates, then their ups) and the k weights."""

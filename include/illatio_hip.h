@@ -295,6 +295,27 @@ int ilt_mm_q8(uint64_t stream, const int8_t* wq, const uint16_t* wd, const int8_
               const float* bias, int rows, int cols, int n, int acc);
 int ilt_mm_k(uint64_t stream, int type, const void* w, const int8_t* xq, const float* xd, const int32_t* bsums, float* y,
              const float* bias, int rows, int cols, int n, int acc);
+/* d4_mm_<format> (ds4f_mm.cu:252-255; dk-mm, cuda-ds4f-prefill.lisp:65-68): one matrix on a chunk of
+   ntok tokens' FLOAT activations, y[t*y_stride + r] = W[r] . x[t*x_stride ..].  The reference's kernels
+   round weights and activations to halves; these give the CPU path's results:
+   q8_0 (the shared expert and the attention projections of a chunk; w, wd as ilt_repack_q8 leaves them,
+     row_bytes 0 or ncols): every token quantized by quantize-q8! with the scale kept a float, then
+     ilt_mm_q8's exact product -- q8mv!'s bits per token (ds4f.lisp:294-297, 1039-1048);
+   q2_k, iq2_xxs: quantize-q8k!, then the exact product (the row dots of iquant.lisp:126-215);
+   f16 (the router, ds4f.lisp:1175 f32mm!): floats, every dot added up in F32-DOT16's order
+     (tensor.lisp:370-378), bit for bit; ncols a multiple of 16.
+   The quantized formats take x_stride = ncols and y_stride = nrows only (hipErrorNotSupported, 801,
+   otherwise) and keep their quantized activations in a buffer inside the library that grows to the largest
+   chunk seen (per GPU, until the process ends; calls that overlap on one GPU share it). */
+int ilt_d4_mm_q8_0(uint64_t stream, int ncols, int nrows, int ntok, int row_bytes, int x_stride, int y_stride, const int8_t* w,
+                   const uint16_t* wd, const float* x, float* y);
+int ilt_d4_mm_f16(uint64_t stream, int ncols, int nrows, int ntok, int row_bytes, int x_stride, int y_stride, const uint16_t* w,
+                  const float* x, float* y);
+int ilt_d4_mm_q2_k(uint64_t stream, int ncols, int nrows, int ntok, int row_bytes, int x_stride, int y_stride, const void* w,
+                   const float* x, float* y);
+int ilt_d4_mm_iq2_xxs(uint64_t stream, int ncols, int nrows, int ntok, int row_bytes, int x_stride, int y_stride, const void* w,
+                      const float* x, float* y);
+
 /* mm_q8_mma2 (dense.cu:884; cuda-dense.lisp:215, 255-258): up to three Q8_0 matrices on the same
    quantized tokens (Q, K, V of a prefill chunk) in one call; a matrix of no rows takes no part.
    Each is ilt_mm_q8's product. */

@@ -470,6 +470,27 @@ void orc_matmul_q(int type, const uint8_t* w, int64_t rows, int64_t cols, const 
   orc_pool_run(nthreads, orc_mm_job, &a);
 }
 
+/* ---- f32-dot16 (src/tensor.lisp:370-378): column i's product into partial sum i mod 16; the sixteen sums
+        combined as c(j) = (s[j] + s[4+j]) + (s[8+j] + s[12+j]), (c(0) + c(1)) + (c(2) + c(3)) ------------------ */
+float orc_f32_dot16(const float* a, const float* b, int64_t n) {
+  float s[16];
+  for (int l = 0; l < 16; l++) s[l] = 0.0f;
+  for (int64_t i = 0; i < n; i++) { volatile float p = a[i] * b[i]; s[i & 15] = s[i & 15] + p; }
+  float c[4];
+  for (int j = 0; j < 4; j++) { volatile float u = s[j] + s[4 + j], v = s[8 + j] + s[12 + j]; c[j] = u + v; }
+  volatile float u = c[0] + c[1], v = c[2] + c[3];
+  return u + v;
+}
+/* f32mm! (src/ds4f.lisp:278-293) for a matrix held as halves (widening is exact): out[t*rows + r] */
+void orc_f16mm(const uint16_t* w, int64_t rows, int64_t cols, const float* x, int64_t ntok, float* out) {
+  float* wr = (float*)malloc(sizeof(float) * cols);
+  for (int64_t r = 0; r < rows; r++) {
+    for (int64_t c = 0; c < cols; c++) wr[c] = orc_half_to_single(w[r * cols + c]);
+    for (int64_t t = 0; t < ntok; t++) out[t * rows + r] = orc_f32_dot16(wr, x + t * cols, cols);
+  }
+  free(wr);
+}
+
 /* ---- src/ds4f.lisp:248-254 ------------------------------------------------------------------------ */
 static inline float sb_exp(float x) { return (float)exp((double)x); }
 static inline float sb_log(float x) { return (float)log((double)x); }

@@ -151,6 +151,23 @@ def matmul_q(qtype, w, rows, cols, xq, xs, bsums, ntok, nthreads=1):
     return out
 
 
+def f32_dot16(a, b):
+    """F32-DOT16 (tensor.lisp:370-378) of two float vectors."""
+    a, b = _c(a, np.float32).ravel(), _c(b, np.float32).ravel()
+    f = lib().orc_f32_dot16
+    f.restype = C.c_float
+    return np.float32(f(_p(a), _p(b), C.c_int64(a.size)))
+
+
+def f16mm(w_bits, rows, cols, x):
+    """out[t, r] = F32-DOT16(W[r], x[t]) for W given as f16 bit patterns (f32mm!, ds4f.lisp:278-293)."""
+    w_bits, x = _c(w_bits, np.uint16), _c(x, np.float32)
+    ntok = 1 if x.ndim == 1 else x.shape[0]
+    out = np.empty((ntok, rows), np.float32)
+    lib().orc_f16mm(_p(w_bits), C.c_int64(rows), C.c_int64(cols), _p(x), C.c_int64(ntok), _p(out))
+    return out[0] if x.ndim == 1 else out
+
+
 def silu(x):
     return lib().orc_silu(float(np.float32(x)))
 

@@ -206,3 +206,62 @@ def test_moe_prefill_chunk_bit_exact(dev, monkeypatch, ne, d, ff, nu, n, clamp, 
     for b in (lb, nb, sb, moe):
         hip.hip_free(b)
     pool.free()
+
+
+@pytest.mark.parametrize("rows,cols,n", [(256, 4096, 70), (37, 48, 5), (300, 1024, 129)])
+def test_d4_mm_f16_router_product_bit_exact(dev, rows, cols, n):
+    """d4_mm_f16 (ds4f_mm.cu:253): an F16 matrix on float rows, every dot in F32-DOT16's order (the CPU's f32mm!,
+    ds4f.lisp:278-293; the router's logits of a chunk), with the tokens' rows and the outputs strided."""
+    from illatio_amd import ds4f, hip
+    rng = synth.make_rng(rows + cols + n)
+    w = (rng.standard_normal((rows, cols)) * 0.05).astype(np.float16)
+    x = synth.activations((n, cols), rng)
+    want = orc.f16mm(w.view(np.uint16), rows, cols, x)
+    wb, xb = hip.hip_upload_new(dev, w.view(np.uint16)), hip.hip_upload_new(dev, x)
+    y = hip.hip_alloc(dev, 4 * n * rows)
+    ds4f.dk_mm(dev, "d4_mm_f16", wb, None, 2 * cols, rows, cols, xb, y, n)
+    got = hip.hip_floats(y, n * rows).reshape(n, rows)
+    assert np.array_equal(bits(got), bits(want)), np.abs(got - want).max()
+    # strides: the tokens' rows and the outputs farther apart (cuda-ds4f-prefill.lisp:154 writes 32 apart)
+    xs, ys = cols + 16, rows + 7
+    xpad = np.zeros((n, xs), np.float32); xpad[:, :cols] = x
+    xb2, y2 = hip.hip_upload_new(dev, xpad), hip.hip_alloc(dev, 4 * n * ys)
+    ds4f.dk_mm(dev, "d4_mm_f16", wb, None, 2 * cols, rows, cols, xb2, y2, n, x_stride=xs, y_stride=ys)
+    got2 = hip.hip_floats(y2, n * ys).reshape(n, ys)
+    assert np.array_equal(bits(got2[:, :rows]), bits(want)) and not got2[:, rows:].any()
+    for b in (wb, xb, y, xb2, y2):
+        hip.hip_free(b)
+
+
+@pytest.mark.parametrize("qtype,rows,cols,n", [(synth.Q8_0, 2048, 4096, 130), (synth.Q8_0, 100, 96, 7), (synth.Q2_K, 512, 2048, 200),
+                                               (synth.IQ2_XXS, 300, 1024, 33), (synth.Q8_0, 4096, 2048, 1)])
+def test_d4_mm_on_float_rows_bit_exact(dev, qtype, rows, cols, n):
+    """d4_mm_q8_0 / d4_mm_q2_k / d4_mm_iq2_xxs (ds4f_mm.cu:252-255) take float rows; each token's result is the CPU
+    path's: quantize-q8! with a float scale and the Q8_0 row dot (q8mv!, ds4f.lisp:294-297), or quantize-q8k! and
+    the expert formats' row dots.  Two calls of different sizes in a row (the library's room for the quantized rows
+    grows), and the strides the quantized formats do not take are refused."""
+    from illatio_amd import dense, ds4f, hip
+    rng = synth.make_rng(qtype * 13 + rows + n)
+    w = synth.weights(qtype, rows, cols, rng)
+    name = {synth.Q8_0: "d4_mm_q8_0", synth.Q2_K: "d4_mm_q2_k", synth.IQ2_XXS: "d4_mm_iq2_xxs"}[qtype]
+    if qtype == synth.Q8_0:
+        m = dense.upload_gmat(dev, "w", qtype, rows, cols, w)
+        wq, wd, rb = m.qs, m.d, 0
+    else:
+        wq, wd, rb = hip.hip_upload_new(dev, w), None, synth.row_bytes(qtype, cols)
+    for ntok in (n, max(1, n // 3), n):
+        x = synth.activations((ntok, cols), rng)
+        x[0, :32] = 0.0
+        xb, y = hip.hip_upload_new(dev, x), hip.hip_alloc(dev, 4 * ntok * rows)
+        ds4f.dk_mm(dev, name, wq, wd, rb, rows, cols, xb, y, ntok)
+        got = hip.hip_floats(y, ntok * rows).reshape(ntok, rows)
+        want = orc.matmul(qtype, w, rows, cols, x, f16_scale=False, nthreads=8).reshape(ntok, rows)
+        assert np.array_equal(bits(got), bits(want)), (ntok, np.abs(got - want).max())
+        if ntok == n:
+            with pytest.raises(hip.HipError):
+                ds4f.dk_mm(dev, name, wq, wd, rb, rows, cols, xb, y, ntok, y_stride=rows + 8)
+        hip.hip_free(xb); hip.hip_free(y)
+    if qtype == synth.Q8_0:
+        m.free()
+    else:
+        hip.hip_free(wq)

@@ -244,3 +244,33 @@ def test_moe_short_pass_of_a_few_tokens_bit_exact(dev, ne, d, ff, nu, n, clamp):
         hip.hip_free(b)
     pool.free(); sh.free()
 
+
+
+@pytest.mark.parametrize("d,ff,n,clamp", [(512, 256, 37, 0.05), (4096, 2048, 130, 0.0)])
+def test_shared_expert_over_a_chunk_bit_exact(dev, d, ff, n, clamp):
+    """The shared expert of a chunk through d4_mm_q8_0 (DK-FFN-HEAD-CHUNK, cuda-ds4f-prefill.lisp:294-298): every
+    token's row has d4-shared!'s bits (ds4f.lisp:1039-1048), and the chunk's routed experts summed with it give
+    each token its own decode step."""
+    from illatio_amd import ds4f, hip
+    rng = synth.make_rng(d + n)
+    ne, nu = 8, 3
+    gate, up, down, sg, su, sd = _moe_weights(rng, ne, d, ff)
+    pool = ds4f.ExpertPool(dev, ne, d, ff, gate, up, down)
+    sh = ds4f.SharedExpert(dev, d, ff, sg, su, sd)
+    norms = synth.activations((n, d), rng)
+    logits = synth.zipf_router_logits(n, ne, rng)
+    lb, nb = hip.hip_upload_new(dev, logits), hip.hip_upload_new(dev, norms)
+    sout = ds4f.ffn_shared_chunk(dev, sh, nb, n, clamp)
+    got = hip.hip_floats(sout, n * d).reshape(n, d)
+    sample = sorted({0, 1, n // 2, n - 1})
+    for t in sample:
+        want = orc.moe_shared(sg, su, sd, d, ff, clamp, norms[t], nthreads=8)
+        assert np.array_equal(bits(got[t]), bits(want)), (t, np.abs(got[t] - want).max())
+    moe = ds4f.ffn_routed_chunk(dev, pool, lb, nb, sout, n, ne, nu, 1.5, clamp)
+    out = hip.hip_floats(moe, n * d).reshape(n, d)
+    for t in sample:
+        want, _, _ = orc.moe_token(gate, up, down, sg, su, sd, d, ff, ne, nu, 1.5, clamp, logits[t], norms[t], nthreads=8)
+        assert np.array_equal(bits(out[t]), bits(want)), (t, np.abs(out[t] - want).max())
+    for b in (lb, nb, sout, moe):
+        hip.hip_free(b)
+    pool.free(); sh.free()

@@ -339,6 +339,52 @@ def test_swiglu_against_explicit_roundings_and_misreadings():
             assert y == 0 and np.signbit(y) == (b > 0)
 
 
+# ---- f32-dot16 (tensor.lisp:370-378): the router's and the attention's dot ---------------------------
+def test_f32_dot16_order_against_numpy_and_misreadings():
+    """Sixteen partial sums (column i into sum i mod 16, products rounded to single first), combined
+    as c(j) = (s[j] + s[4+j]) + (s[8+j] + s[12+j]), (c0 + c1) + (c2 + c3): numpy's single-precision
+    operations, each correctly rounded, in that order.  A plain running sum, a pairwise tree over the
+    sixteen, and products kept exact (a fused multiply-add) must give other bits on some input."""
+    f32 = np.float32
+    rng = synth.make_rng(23)
+    told = set()
+    for trial in range(200):
+        n = int(rng.choice([16, 32, 128, 4096]))
+        a = (rng.standard_normal(n) * rng.choice([1.0, 100.0])).astype(f32)
+        b = rng.standard_normal(n).astype(f32)
+        s = np.zeros(16, f32)
+        for j in range(0, n, 16):
+            s = (s + (a[j:j + 16] * b[j:j + 16]).astype(f32)).astype(f32)
+        c = [f32(f32(s[j] + s[4 + j]) + f32(s[8 + j] + s[12 + j])) for j in range(4)]
+        want = f32(f32(c[0] + c[1]) + f32(c[2] + c[3]))
+        got = orc.f32_dot16(a, b)
+        assert got.view(np.uint32) == want.view(np.uint32), trial
+        run = f32(0)
+        for v in (a * b).astype(f32):
+            run = f32(run + v)
+        tree = s.copy()
+        while tree.size > 1:
+            tree = (tree[0::2] + tree[1::2]).astype(f32)
+        sx = np.zeros(16, np.float64)                       # products not rounded to single before the add
+        for j in range(0, n, 16):
+            sx = (sx + a[j:j + 16].astype(np.float64) * b[j:j + 16].astype(np.float64)).astype(f32).astype(np.float64)
+        cx = [f32(f32(f32(sx[j]) + f32(sx[4 + j])) + f32(f32(sx[8 + j]) + f32(sx[12 + j]))) for j in range(4)]
+        fused = f32(f32(cx[0] + cx[1]) + f32(cx[2] + cx[3]))
+        for name, v in (("running sum", run), ("pairwise tree", tree[0]), ("fused products", fused)):
+            if v.view(np.uint32) != got.view(np.uint32):
+                told.add(name)
+    assert told == {"running sum", "pairwise tree", "fused products"}, told
+    # sixteen columns: the tree alone, on values whose sums are exact
+    a = np.arange(1, 17, dtype=f32); b = np.ones(16, f32)
+    assert orc.f32_dot16(a, b) == 136.0
+    w = rng.standard_normal((5, 64)).astype(np.float16)
+    x = rng.standard_normal((3, 64)).astype(f32)
+    out = orc.f16mm(w.view(np.uint16), 5, 64, x)
+    for t in range(3):
+        for r in range(5):
+            assert out[t, r] == orc.f32_dot16(w[r].astype(f32), x[t])
+
+
 # ---- routing -------------------------------------------------------------------------------------
 def test_route_against_stable_sort():
     rng = synth.make_rng(7)
