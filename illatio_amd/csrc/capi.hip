@@ -406,6 +406,10 @@ int ilt_d4_group_scatter(uint64_t stream, int n, int ne, int nu, const uint32_t*
   ILT_REQUIRE(n >= 0 && nu > 0 && (n == 0 || (sel && rank && bases && w && rmap && smap && wrow)));
   return (int)ilt_k_group_scatter(n, ne, nu, sel, rank, bases, w, rmap, smap, wrow, S(stream));
 }
+int ilt_d4_rows_expert(uint64_t stream, int n, const uint32_t* sel, const uint32_t* smap, uint32_t* rexp) {
+  ILT_REQUIRE(n >= 0 && (n == 0 || (sel && smap && rexp)));
+  return (int)ilt_k_rows_expert(n, sel, smap, rexp, S(stream));
+}
 int ilt_d4_gather_rows(uint64_t stream, int d, int nrows, const float* src, const uint32_t* map, float* x) {
   ILT_REQUIRE(d > 0 && nrows >= 0 && (nrows == 0 || (src && map && x)));
   return (int)ilt_k_gather_rows(d, nrows, src, map, x, S(stream));
@@ -793,6 +797,7 @@ int ilt_launch(const char* kernel, unsigned gx, unsigned gy, unsigned gz, unsign
     return ilt_d4_mm_id_glu_bf16(stream, a.i32(0), a.i32(1), a.i32(2), a.i32(3), a.i64(4), a.i64(5), a.ptr<const uint64_t*>(6), a.ptr<cu32>(7),
                                  a.ptr<cu32>(8), a.i32(9), a.i64(10), a.ptr<cu16>(11), a.ptr<cu32>(12), a.f32(13), a.ptr<cf>(14), a.ptr<uint16_t*>(15));
   K("d4_swiglu_w_bf16") return ilt_d4_swiglu_w_bf16(stream, a.i32(0), a.i32(1), a.f32(2), a.ptr<cf>(3), a.ptr<cf>(4), a.ptr<cf>(5), a.ptr<uint16_t*>(6));
+  K("d4_rows_expert") return ilt_d4_rows_expert(stream, a.i32(0), a.ptr<cu32>(1), a.ptr<cu32>(2), a.ptr<uint32_t*>(3));
   K("d4_mm_q8_0") return ilt_d4_mm_q8_0(stream, a.i32(0), a.i32(1), a.i32(2), a.i32(3), a.i32(4), a.i32(5), a.ptr<ci8>(6), a.ptr<cu16>(7), a.ptr<cf>(8), a.ptr<float*>(9));
   K("d4_mm_f16") return ilt_d4_mm_f16(stream, a.i32(0), a.i32(1), a.i32(2), a.i32(3), a.i32(4), a.i32(5), a.ptr<cu16>(6), a.ptr<cf>(8), a.ptr<float*>(9));
   K("d4_mm_q2_k") return ilt_d4_mm_q2_k(stream, a.i32(0), a.i32(1), a.i32(2), a.i32(3), a.i32(4), a.i32(5), a.ptr<const void*>(6), a.ptr<cf>(8), a.ptr<float*>(9));

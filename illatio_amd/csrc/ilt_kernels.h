@@ -84,6 +84,7 @@ hipError_t ilt_k_group_count(int n, int ne, int nu, const uint32_t* sel, uint32_
 hipError_t ilt_k_group_scan(int n, int ne, int nu, const uint32_t* counts, uint32_t* bases, hipStream_t st);
 hipError_t ilt_k_group_scatter(int n, int ne, int nu, const uint32_t* sel, const uint32_t* rank, const uint32_t* bases,
                                const float* w, uint32_t* rmap, uint32_t* smap, float* wrow, hipStream_t st);
+hipError_t ilt_k_rows_expert(int n, const uint32_t* sel, const uint32_t* smap, uint32_t* rexp, hipStream_t st);
 hipError_t ilt_k_gather_rows(int d, int nrows, const float* src, const uint32_t* map, float* x, hipStream_t st);
 hipError_t ilt_k_swiglu_w(int n, int ff, float clamp, const float* g, const float* u, const float* w, float* mid,
                           int8_t* xq, float* xs, hipStream_t st);

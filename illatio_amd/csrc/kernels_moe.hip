@@ -177,6 +177,12 @@ __global__ void group_scatter_kernel(int n, int nu, const u32* __restrict__ sel,
   rmap[row] = gid / nu; smap[gid] = row; wrow[row] = w[gid];
 }
 
+// rexp[row] = the expert of grouped row `row` (row smap[i] is (token, slot) i's)
+__global__ void rows_expert_kernel(int n, const u32* __restrict__ sel, const u32* __restrict__ smap, u32* __restrict__ rexp) {
+  const int gid = blockIdx.x * blockDim.x + threadIdx.x;
+  if (gid < n) rexp[smap[gid]] = sel[gid];
+}
+
 __global__ void gather_rows_kernel(int d, int nrows, const float* __restrict__ src, const u32* __restrict__ map,
                                    float* __restrict__ x) {
   const long long gid = ((long long)blockIdx.x * blockDim.x + threadIdx.x) * 4;
@@ -312,6 +318,12 @@ hipError_t ilt_k_group_scatter(int n, int ne, int nu, const uint32_t* sel, const
                                const float* w, uint32_t* rmap, uint32_t* smap, float* wrow, hipStream_t st) {
   if (n <= 0) return hipSuccess;
   hipLaunchKernelGGL(group_scatter_kernel, dim3((n + 255) / 256), dim3(256), 0, st, n, nu, sel, rank, bases, w, rmap, smap, wrow);
+  return hipGetLastError();
+}
+
+hipError_t ilt_k_rows_expert(int n, const uint32_t* sel, const uint32_t* smap, uint32_t* rexp, hipStream_t st) {
+  if (n <= 0) return hipSuccess;
+  hipLaunchKernelGGL(rows_expert_kernel, dim3((n + 255) / 256), dim3(256), 0, st, n, sel, smap, rexp);
   return hipGetLastError();
 }
 

@@ -263,7 +263,7 @@ def ffn_step_noalloc(dev, pool, sh, logits, norm2, moe, ne, nu, scale, clamp, bi
     return moe
 
 
-def ffn_small(dev, pool, sh, logits, norm2, n, ne, nu, scale, clamp, bias=None):
+def ffn_small(dev, pool, sh, logits, norm2, n, ne, nu, scale, clamp, bias=None, grouped=False):
     """The FFN past the router for a short pass's N <= 9 tokens (DK-FFN-SMALL,
     cuda-ds4f-spec.lisp:30-100: a speculative step's verification), every token with decode's
     bits.  The reference routes on the CPU and hands each expert its tokens' rows through
@@ -289,16 +289,27 @@ def ffn_small(dev, pool, sh, logits, norm2, n, ne, nu, scale, clamp, bias=None):
     hip.launch(dev, "d4_mvq8n", (d + 3) // 4, 128, [d, ff, d, n, ff, d, sh.down.qs, sh.down.d, qm_q, qm_s, sout])
     # the routed experts: row r = (token r / nu, slot r % nu)
     sel, w = route(dev, logits, n, ne, nu, scale, bias)
-    rmap = hip.hip_upload_new(dev, (np.arange(rows) // nu).astype(np.uint32))
-    smap = hip.hip_upload_new(dev, np.arange(rows, dtype=np.uint32))
+    extra = []
+    if grouped:
+        # GROUPED: the rows grouped by expert on the device (d4_group_*), an expert's rows one after another, so its
+        # matrices come from memory once for all its tokens: what the reference's counts / bases arguments give
+        g = group_rows(dev, sel, w, n, ne, nu)
+        rmap, smap, wrow = g["rmap"], g["smap"], g["wrow"]
+        rexp = A(dev, 4 * rows)
+        hip.launch(dev, "d4_rows_expert", (rows + 255) // 256, 256, [rows, sel, smap, rexp])
+        extra = [rexp] + [v for k, v in g.items() if k not in ("rmap", "smap")]
+    else:
+        rmap = hip.hip_upload_new(dev, (np.arange(rows) // nu).astype(np.uint32))
+        smap = hip.hip_upload_new(dev, np.arange(rows, dtype=np.uint32))
+        rexp, wrow = sel, w
     x, bm, bd, moe = A(dev, 4 * rows * d), A(dev, 4 * rows * ff), A(dev, 4 * rows * d), A(dev, 4 * n * d)
     hip.launch(dev, "d4_gather_rows", (rows * d + 255) // 256, 256, [d, rows, norm2, rmap, x])
     hip.launch(dev, "d4_mv_glu_iq2_xxs", ((ff + 7) // 8, 1, rows), 64,
-               [d, ff, pool.grb, hip.I64(0), hip.I64(gb), d, ff, pool.ptrs, sel, x, w, float(clamp), bm])
-    hip.launch(dev, "d4_mv_q2_k_f32", ((d + 7) // 8, 1, rows), 64, [ff, d, pool.drb, hip.I64(2 * gb), ff, d, pool.ptrs, sel, bm, bd])
+               [d, ff, pool.grb, hip.I64(0), hip.I64(gb), d, ff, pool.ptrs, rexp, x, wrow, float(clamp), bm])
+    hip.launch(dev, "d4_mv_q2_k_f32", ((d + 7) // 8, 1, rows), 64, [ff, d, pool.drb, hip.I64(2 * gb), ff, d, pool.ptrs, rexp, bm, bd])
     hip.launch(dev, "d4_moe_sum_rows", (n * d + 255) // 256, 256, [d, nu, n, bd, smap, sout, moe])
     hip.hip_sync(dev)
-    for b in (qn_q, qn_s, sg, su, smid, qm_q, qm_s, sout, one, sel, w, rmap, smap, x, bm, bd):
+    for b in [qn_q, qn_s, sg, su, smid, qm_q, qm_s, sout, one, sel, w, rmap, smap, x, bm, bd] + extra:
         hip.hip_free(b)
     return moe
 

@@ -150,3 +150,44 @@ def upload_tensor(dev, g, name):
         raise GgufError(f"{name}: {len(ti.dims)} dimensions, a matrix has two")
     cols, rows = ti.dims
     return dense.upload_gmat(dev, name, ti.type, rows, cols, tensor_bytes(g, ti))
+
+
+def expert_tensor(g, name):
+    """(TensorInfo, bytes a row, rows an expert, cols, experts) of the 3-D expert tensor NAME, dims
+    [cols, rows, experts] (EXPERT-TENSOR, ds4f.lisp:95-100): expert e's rows start e * rows * row bytes in."""
+    ti = gguf_tensor(g, name)
+    if len(ti.dims) != 3:
+        raise GgufError(f"{name}: {len(ti.dims)} dimensions, an expert tensor has three")
+    cols, rows, ne = ti.dims
+    return ti, ti.nbytes() // (rows * ne), rows, cols, ne
+
+
+def upload_experts(dev, g, layer):
+    """Layer LAYER's routed experts of G as an ExpertPool on DEV: blk.<layer>.ffn_gate_exps / ffn_up_exps
+    (IQ2_XXS) and ffn_down_exps (Q2_K), each expert into its slot as gate | up | down (the slots D4-FILL
+    makes, cuda-ds4f.lisp:162-166, 190-202; with all experts resident slot e is expert e)."""
+    from . import ds4f
+    from .synth import IQ2_XXS, Q2_K
+    (gt, grb, ff, d, ne), (ut, urb, uff, ud, une), (dt, drb, dd, dff, dne) = (
+        expert_tensor(g, f"blk.{layer}.ffn_{n}_exps.weight") for n in ("gate", "up", "down"))
+    if (gt.type, ut.type, dt.type) != (IQ2_XXS, IQ2_XXS, Q2_K):
+        raise GgufError(f"blk.{layer}: the expert products take IQ2_XXS gate/up and Q2_K down, not "
+                        f"{gt.type_name}/{ut.type_name}/{dt.type_name}")
+    if (uff, ud, une) != (ff, d, ne) or (dd, dff, dne) != (d, ff, ne):
+        raise GgufError(f"blk.{layer}: the experts' gate, up and down do not fit one another")
+    return ds4f.ExpertPool(dev, ne, d, ff, tensor_bytes(g, gt), tensor_bytes(g, ut), tensor_bytes(g, dt))
+
+
+def upload_shared_expert(dev, g, layer):
+    """Layer LAYER's shared expert (ffn_gate_shexp / ffn_up_shexp / ffn_down_shexp, Q8_0) repacked on DEV
+    (D4-UPLOAD-WEIGHTS, cuda-ds4f.lisp:244-290)."""
+    from . import ds4f
+    from .synth import Q8_0
+    tis = [gguf_tensor(g, f"blk.{layer}.ffn_{n}_shexp.weight") for n in ("gate", "up", "down")]
+    for ti in tis:
+        if ti.type != Q8_0 or len(ti.dims) != 2:
+            raise GgufError(f"{ti.name}: the shared expert's matrices are 2-D Q8_0")
+    d, ff = tis[0].dims
+    if tuple(tis[1].dims) != (d, ff) or tuple(tis[2].dims) != (ff, d):
+        raise GgufError(f"blk.{layer}: the shared expert's gate, up and down do not fit one another")
+    return ds4f.SharedExpert(dev, d, ff, *(tensor_bytes(g, ti) for ti in tis))

@@ -274,6 +274,12 @@ int ilt_d4_group_scan(uint64_t stream, int n, int ne, int nu, const uint32_t* co
 int ilt_d4_group_scatter(uint64_t stream, int n, int ne, int nu, const uint32_t* sel, const uint32_t* rank,
                          const uint32_t* bases, const float* w, uint32_t* rmap, uint32_t* smap, float* wrow);
 int ilt_d4_gather_rows(uint64_t stream, int d, int nrows, const float* src, const uint32_t* map, float* x);
+/* The expert of every grouped row: rexp[smap[i]] = sel[i] for the n (token, slot) pairs.  With it the indexed
+   expert kernels (sel = rexp over the table of all slots, one launch slot a grouped row) take an expert's rows
+   one after another, so its matrices come from memory once for all its tokens and from the cache after -- what
+   the counts / bases arguments of the reference's d4_mv_* give a short pass (ds4f.cu:762-772,
+   cuda-ds4f-spec.lisp:83-88), with the routing and the grouping left on the device. */
+int ilt_d4_rows_expert(uint64_t stream, int n, const uint32_t* sel, const uint32_t* smap, uint32_t* rexp);
 int ilt_d4_swiglu_w(uint64_t stream, int n, int ff, float clamp, const float* g, const float* u, const float* w,
                     float* mid, int8_t* xq, float* xs);
 int ilt_d4_moe_sum(uint64_t stream, int d, int k, const float* down, const float* shared_, float* moe, const uint32_t* perm);

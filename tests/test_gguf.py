@@ -102,3 +102,59 @@ def test_tensors_of_a_file_multiply_with_the_oracles_bits(tmp_path):
         m.free()
     with pytest.raises(gguf.GgufError):
         gguf.upload_tensor(dev, g, "output_norm.weight")
+
+
+def _moe_file(tmp_path, rng, ne, d, ff):
+    gate = synth.weights(synth.IQ2_XXS, ne * ff, d, rng)
+    up = synth.weights(synth.IQ2_XXS, ne * ff, d, rng)
+    down = synth.weights(synth.Q2_K, ne * d, ff, rng)
+    sg, su, sd = synth.weights(synth.Q8_0, ff, d, rng), synth.weights(synth.Q8_0, ff, d, rng), synth.weights(synth.Q8_0, d, ff, rng)
+    p = tmp_path / "moe.gguf"
+    write_gguf(p, {"general.architecture": "deepseek4"}, [
+        ("blk.3.ffn_gate_exps.weight", (d, ff, ne), synth.IQ2_XXS, gate), ("blk.3.ffn_up_exps.weight", (d, ff, ne), synth.IQ2_XXS, up),
+        ("blk.3.ffn_down_exps.weight", (ff, d, ne), synth.Q2_K, down),
+        ("blk.3.ffn_gate_shexp.weight", (d, ff), synth.Q8_0, sg), ("blk.3.ffn_up_shexp.weight", (d, ff), synth.Q8_0, su),
+        ("blk.3.ffn_down_shexp.weight", (ff, d), synth.Q8_0, sd),
+        ("blk.4.ffn_gate_exps.weight", (d, ff, ne), synth.Q4_K, synth.weights(synth.Q4_K, ne * ff, d, rng)),
+        ("blk.4.ffn_up_exps.weight", (d, ff, ne), synth.IQ2_XXS, up), ("blk.4.ffn_down_exps.weight", (ff, d, ne), synth.Q2_K, down)])
+    return p, (gate, up, down, sg, su, sd)
+
+
+def test_expert_tensor_directory(tmp_path):
+    """A 3-D expert tensor [cols, rows, experts]: bytes a row, rows an expert (EXPERT-TENSOR, ds4f.lisp:95-100)."""
+    ne, d, ff = 5, 512, 256
+    p, w = _moe_file(tmp_path, synth.make_rng(3), ne, d, ff)
+    g = gguf.read_gguf(str(p))
+    ti, rb, rows, cols, n = gguf.expert_tensor(g, "blk.3.ffn_gate_exps.weight")
+    assert (rb, rows, cols, n) == (synth.row_bytes(synth.IQ2_XXS, d), ff, d, ne)
+    ti, rb, rows, cols, n = gguf.expert_tensor(g, "blk.3.ffn_down_exps.weight")
+    assert (rb, rows, cols, n) == (synth.row_bytes(synth.Q2_K, ff), d, ff, ne)
+    raw = gguf.tensor_bytes(g, ti).reshape(ne, d * rb)
+    assert np.array_equal(raw[4], w[2].reshape(ne, d * rb)[4])            # expert 4's rows start 4 * rows * row bytes in
+    with pytest.raises(gguf.GgufError):
+        gguf.expert_tensor(g, "blk.3.ffn_gate_shexp.weight")
+
+
+@pytest.mark.gpu
+def test_experts_of_a_file_take_a_decode_step_with_the_oracles_bits(tmp_path):
+    """The routed experts (3-D tensors) and the shared expert of a written file, uploaded into slots and repacked
+    (d4-upload-weights, cuda-ds4f.lisp:244-290), run one token's FFN with the CPU path's bits."""
+    import oracle_lib as orc
+    from illatio_amd import ds4f, hip
+    dev = hip.open_hip(0)
+    rng = synth.make_rng(12)
+    ne, d, ff, nu = 6, 512, 256, 3
+    p, (gate, up, down, sg, su, sd) = _moe_file(tmp_path, rng, ne, d, ff)
+    g = gguf.read_gguf(str(p))
+    pool, sh = gguf.upload_experts(dev, g, 3), gguf.upload_shared_expert(dev, g, 3)
+    assert (pool.ne, pool.d, pool.ff, sh.d, sh.ff) == (ne, d, ff, d, ff)
+    logits, norm = synth.activations(ne, rng), synth.activations(d, rng)
+    want, _, _ = orc.moe_token(gate, up, down, sg, su, sd, d, ff, ne, nu, 1.5, 0.0, logits, norm)
+    lb, nb, out = hip.hip_upload_new(dev, logits), hip.hip_upload_new(dev, norm), hip.hip_alloc(dev, 4 * d)
+    ds4f.ffn_step_call(dev, pool, sh, lb, nb, out, ne, nu, 1.5, 0.0)
+    assert np.array_equal(hip.hip_floats(out, d).view(np.uint32), want.view(np.uint32))
+    with pytest.raises(gguf.GgufError, match="IQ2_XXS gate/up"):
+        gguf.upload_experts(dev, g, 4)                                    # a Q4_K gate: not what the expert products take
+    for b in (lb, nb, out):
+        hip.hip_free(b)
+    pool.free(); sh.free()

@@ -235,12 +235,14 @@ def test_moe_short_pass_of_a_few_tokens_bit_exact(dev, ne, d, ff, nu, n, clamp):
     logits = synth.activations((n, ne), rng)
     logits[1] = logits[0]                     # two tokens on the same experts
     lb, nb = hip.hip_upload_new(dev, logits), hip.hip_upload_new(dev, norm)
-    moe = ds4f.ffn_small(dev, pool, sh, lb, nb, n, ne, nu, 1.5, clamp)
-    got = hip.hip_floats(moe, n * d).reshape(n, d)
-    for t in range(n):
-        want, _, _ = orc.moe_token(gate, up, down, sg, su, sd, d, ff, ne, nu, 1.5, clamp, logits[t], norm[t])
-        assert np.array_equal(bits(got[t]), bits(want)), (t, np.abs(got[t] - want).max())
-    for b in (lb, nb, moe):
+    for grouped in (False, True):             # a launch slot per (token, slot) row in token order; the rows grouped by expert
+        moe = ds4f.ffn_small(dev, pool, sh, lb, nb, n, ne, nu, 1.5, clamp, grouped=grouped)
+        got = hip.hip_floats(moe, n * d).reshape(n, d)
+        for t in range(n):
+            want, _, _ = orc.moe_token(gate, up, down, sg, su, sd, d, ff, ne, nu, 1.5, clamp, logits[t], norm[t])
+            assert np.array_equal(bits(got[t]), bits(want)), (grouped, t, np.abs(got[t] - want).max())
+        hip.hip_free(moe)
+    for b in (lb, nb):
         hip.hip_free(b)
     pool.free(); sh.free()
 
