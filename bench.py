@@ -76,12 +76,39 @@ D, FFN, QD, KVD, VOCAB, LAYERS = 2560, 9728, 4096, 1024, 151936, 36
 
 
 def host_cores():
-    cores = min(os.cpu_count() or 1, 64)
+    """Physical cores this process may run on (hyperthreads counted once), at most the 16 of a one-GPU box's share."""
     try:
-        cores = min(cores, len(os.sched_getaffinity(0)))
+        allowed = set(os.sched_getaffinity(0))
     except AttributeError:
+        allowed = set(range(os.cpu_count() or 1))
+    cores = set()
+    try:
+        cpu = phys = core = None
+        for line in open("/proc/cpuinfo"):
+            k, _, v = line.partition(":")
+            k, v = k.strip(), v.strip()
+            if k == "processor":
+                cpu, phys, core = int(v), None, None
+            elif k == "physical id":
+                phys = v
+            elif k == "core id":
+                core = v
+            if cpu is not None and phys is not None and core is not None:
+                if cpu in allowed:
+                    cores.add((phys, core))
+                cpu = None
+    except OSError:
         pass
-    return cores
+    n = len(cores) if cores else len(allowed)
+    return max(1, min(n, 16))
+
+
+def one_thread_figure(work_fn, seconds=3.0):
+    """WORK_FN(nthreads) -> units of work done; its rate on one thread over about SECONDS."""
+    t1, done = time.perf_counter(), 0.0
+    while time.perf_counter() - t1 < seconds:
+        done += work_fn(1)
+    return done / (time.perf_counter() - t1)
 
 
 class Timer:
@@ -260,9 +287,14 @@ def workload_c2(args, dev):
                 t_cpu += time.perf_counter() - t1
                 nbytes += host[name].size
             reps += 1
+        def one(nt):
+            name, qt, rows, cols, src = specs[4]             # the gate matrix, 9728 x 2560 Q4_K
+            orc.matmul(qt, host[name], rows, cols, xs[src], nthreads=nt)
+            return host[name].size
         return {"value": round(nbytes / t_cpu / 1e9, 3), "unit": "GB/s", "cores": cores, "kind": "port",
                 "sample": f"{reps} x one layer's seven products (activation quantization included), {nbytes} weight bytes, {t_cpu:.1f} s",
-                "tok_per_s_equiv": round(nbytes / t_cpu / step_bytes, 3)}
+                "tok_per_s_equiv": round(nbytes / t_cpu / step_bytes, 3),
+                "one_thread": {"value": round(one_thread_figure(one) / 1e9, 3), "unit": "GB/s", "sample": "the 9728 x 2560 Q4_K product, about 3 s"}}
 
     return {"value": round(gbs, 1), "unit": "GB/s", "ms_per_step": ms, "device_ms_per_step": dev_ms, "enqueue_ms": tm.enqueue_ms,
             "dtype": "int8 block dots, fp32 combine",

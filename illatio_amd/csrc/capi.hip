@@ -1,7 +1,9 @@
 // The C ABI of libillatio_hip.so (declared in include/illatio_hip.h): the driver calls the
 // reference's src/cuda.lisp makes, typed entry points for the kernels, and launch by name.
-// Host code only validates shapes and picks launch geometry; it does no arithmetic on data.
+// Host code only validates shapes and picks launch geometry; it does no arithmetic on data (ilt_rope_table, a
+// model's constants, aside).
 #include <hip/hip_runtime.h>
+#include <math.h>
 #include <stdint.h>
 #include <stdio.h>
 #include <string.h>
@@ -744,6 +746,41 @@ int ilt_d4_mm_id_glu_bf16(uint64_t stream, int gguf_type, int ncols, int nrows, 
 }
 
 // ---- launch by name ---------------------------------------------------------------------------
+// ---- between the products of a dense layer (the forward harness) ----------------------------------
+int ilt_qk_rope(uint64_t stream, float* q, float* k, const float* v, const float* qn, const float* kn, const float* rope, float* kc,
+                float* vc, int nh, int nkv, int hd, int rd, int pos0, float eps, int neox, int ntok) {
+  ILT_REQUIRE(ntok >= 0 && (ntok == 0 || (q && k && v && rope && kc && vc)) && pos0 >= 0);
+  return (int)ilt_k_qk_rope(q, k, v, qn, kn, rope, kc, vc, nh, nkv, hd, rd, pos0, eps, neox, ntok, S(stream));
+}
+// rope-table (model.lisp:218-231) for positions pos0 .. pos0 + n - 1, on the host: a position's head_dim/2 cosines
+// then head_dim/2 sines, theta advanced by repeated single-float multiplication, theta-scale, cos and sin through
+// double and rounded to single as SBCL evaluates them.  The only float arithmetic this file does: model constants,
+// made once and uploaded by the caller; nothing here can overflow or trap.
+int ilt_rope_table(int head_dim, int pos0, int n, float base, float* out) {
+  ILT_REQUIRE(out && head_dim >= 2 && head_dim % 2 == 0 && pos0 >= 0 && n >= 0 && base > 0.0f);
+  const int half = head_dim / 2;
+  const float e = -2.0f / (float)head_dim;
+  const float theta_scale = (float)pow((double)base, (double)e);
+  for (int p = 0; p < n; p++) {
+    float theta = (float)(pos0 + p);
+    float* row = out + (size_t)p * head_dim;
+    for (int i = 0; i < half; i++) {
+      row[i] = (float)cos((double)theta); row[half + i] = (float)sin((double)theta);
+      const volatile float next = theta * theta_scale;
+      theta = next;
+    }
+  }
+  return ILT_OK;
+}
+int ilt_attn_rows(uint64_t stream, const float* q, const float* kc, const float* vc, float* out, int nh, int nkv, int hd, int pos0, int ntok) {
+  ILT_REQUIRE(ntok >= 0 && (ntok == 0 || (q && kc && vc && out)) && nh > 0 && nkv > 0);
+  return (int)ilt_k_attn_rows(q, kc, vc, out, nh, nkv, hd, pos0, ntok, S(stream));
+}
+int ilt_swiglu(uint64_t stream, float* a, const float* b, int64_t n) {
+  ILT_REQUIRE(n >= 0 && (n == 0 || (a && b)));
+  return (int)ilt_k_swiglu_rows(a, b, n, S(stream));
+}
+
 int ilt_launch(const char* kernel, unsigned gx, unsigned gy, unsigned gz, unsigned bx, unsigned by, unsigned bz,
                unsigned shared_bytes, uint64_t stream, void** params) {
   ILT_REQUIRE(kernel && params);
@@ -797,6 +834,10 @@ int ilt_launch(const char* kernel, unsigned gx, unsigned gy, unsigned gz, unsign
     return ilt_d4_mm_id_glu_bf16(stream, a.i32(0), a.i32(1), a.i32(2), a.i32(3), a.i64(4), a.i64(5), a.ptr<const uint64_t*>(6), a.ptr<cu32>(7),
                                  a.ptr<cu32>(8), a.i32(9), a.i64(10), a.ptr<cu16>(11), a.ptr<cu32>(12), a.f32(13), a.ptr<cf>(14), a.ptr<uint16_t*>(15));
   K("d4_swiglu_w_bf16") return ilt_d4_swiglu_w_bf16(stream, a.i32(0), a.i32(1), a.f32(2), a.ptr<cf>(3), a.ptr<cf>(4), a.ptr<cf>(5), a.ptr<uint16_t*>(6));
+  K("qk_rope") return ilt_qk_rope(stream, a.ptr<float*>(0), a.ptr<float*>(1), a.ptr<cf>(2), a.ptr<cf>(3), a.ptr<cf>(4), a.ptr<cf>(5), a.ptr<float*>(6),
+                                  a.ptr<float*>(7), a.i32(8), a.i32(9), a.i32(10), a.i32(11), a.i32(12), a.f32(13), a.i32(14), (int)gy);
+  K("swiglu") return ilt_swiglu(stream, a.ptr<float*>(0), a.ptr<cf>(1), a.i64(2));
+  K("attn_rows") return ilt_attn_rows(stream, a.ptr<cf>(0), a.ptr<cf>(1), a.ptr<cf>(2), a.ptr<float*>(3), a.i32(4), a.i32(5), a.i32(6), a.i32(7), (int)gy);
   K("d4_rows_expert") return ilt_d4_rows_expert(stream, a.i32(0), a.ptr<cu32>(1), a.ptr<cu32>(2), a.ptr<uint32_t*>(3));
   K("d4_mm_q8_0") return ilt_d4_mm_q8_0(stream, a.i32(0), a.i32(1), a.i32(2), a.i32(3), a.i32(4), a.i32(5), a.ptr<ci8>(6), a.ptr<cu16>(7), a.ptr<cf>(8), a.ptr<float*>(9));
   K("d4_mm_f16") return ilt_d4_mm_f16(stream, a.i32(0), a.i32(1), a.i32(2), a.i32(3), a.i32(4), a.i32(5), a.ptr<cu16>(6), a.ptr<cf>(8), a.ptr<float*>(9));

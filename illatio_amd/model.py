@@ -1,0 +1,133 @@
+"""A dense decoder on the device: the host side of the reference's CUDA-FORWARD-N (src/cuda-dense.lisp:380-432)
+for the K-quant models of the benchmark's config 2 -- embedding, and per layer: norm, Q/K/V, head norms + RoPE +
+cache update, attention, wo added to the stream, norm, gate/up with swiglu!, down added to the stream; then the
+output norm and head.  One token runs the decode products (matrix-vector kernels that take the norm and the
+quantizer inside); several tokens run the prefill products (EVAL-TOKENS, batch.lisp:289-307).  Either way a
+token's logits have the CPU path's bits (FORWARD-1, model.lisp:396-462): the products are bit-exact and the
+kernels between them add in the CPU's order.
+
+synth_model makes the random-init model the benchmark and the tests run (there are no model files here):
+Q4_K for most matrices, Q6_K for V, down and the tied embedding / output head, as Q4_K_M files have them.
+"""
+import ctypes as C
+
+import numpy as np
+
+from . import dense, hip, synth
+from .synth import Q4_K, Q6_K
+
+
+def synth_model(seed, d=2560, ffn=9728, nh=32, nkv=8, hd=128, nl=36, vocab=151936, eps=1e-6, rope_base=1e6, head_scale=8.0):
+    """A seeded random-init dense decoder as numpy arrays: {"config", "embd", "output", "output_norm", "layers"}; a
+    matrix is (GGUF type, uint8 rows).  HEAD_SCALE spreads the output head's logits so that the greedy token is not
+    decided in the last bits (random weights give nearly flat logits)."""
+    rng = synth.make_rng(seed)
+    qd, kvd = nh * hd, nkv * hd
+    norm = lambda n: (synth.activations(n, rng) * 0.1 + 1.0).astype(np.float32)
+    layers = []
+    for _ in range(nl):
+        layers.append({"wq": (Q4_K, synth.weights(Q4_K, qd, d, rng)), "wk": (Q4_K, synth.weights(Q4_K, kvd, d, rng)),
+                       "wv": (Q6_K, synth.weights(Q6_K, kvd, d, rng)), "wo": (Q4_K, synth.weights(Q4_K, d, qd, rng, dscale=0.0002)),
+                       "gate": (Q4_K, synth.weights(Q4_K, ffn, d, rng)), "up": (Q4_K, synth.weights(Q4_K, ffn, d, rng)),
+                       "down": (Q6_K, synth.weights(Q6_K, d, ffn, rng, dscale=0.002)),
+                       "attn_norm": norm(d), "ffn_norm": norm(d), "q_norm": norm(hd), "k_norm": norm(hd)})
+    embd = (Q6_K, synth.weights(Q6_K, vocab, d, rng, dscale=0.01 * head_scale))
+    return {"config": {"d": d, "ffn": ffn, "nh": nh, "nkv": nkv, "hd": hd, "nl": nl, "vocab": vocab, "eps": eps, "rope_base": rope_base,
+                       "neox": True},
+            "embd": embd, "output": embd, "output_norm": norm(d), "layers": layers}
+
+
+class DenseModel:
+    """HOST (synth_model's dict, or the same made from a file's tensors) on DEV, with caches for NCTX positions."""
+
+    def __init__(self, dev, host, nctx, chunk=512):
+        c = host["config"]
+        self.dev, self.c, self.nctx, self.chunk, self.pos = dev, c, nctx, chunk, 0
+        d, ffn, hd = c["d"], c["ffn"], c["hd"]
+        self.qd, self.kvd = c["nh"] * hd, c["nkv"] * hd
+        up = lambda name, m, rows, cols: dense.upload_gmat(dev, name, m[0], rows, cols, m[1])
+        fl = lambda a: None if a is None else hip.hip_upload_new(dev, np.ascontiguousarray(a, np.float32))
+        self.layers = []
+        for li, L in enumerate(host["layers"]):
+            self.layers.append({"wq": up(f"blk.{li}.attn_q", L["wq"], self.qd, d), "wk": up(f"blk.{li}.attn_k", L["wk"], self.kvd, d),
+                                "wv": up(f"blk.{li}.attn_v", L["wv"], self.kvd, d), "wo": up(f"blk.{li}.attn_output", L["wo"], d, self.qd),
+                                "gate": up(f"blk.{li}.ffn_gate", L["gate"], ffn, d), "up": up(f"blk.{li}.ffn_up", L["up"], ffn, d),
+                                "down": up(f"blk.{li}.ffn_down", L["down"], d, ffn),
+                                "attn_norm": fl(L["attn_norm"]), "ffn_norm": fl(L["ffn_norm"]), "q_norm": fl(L.get("q_norm")),
+                                "k_norm": fl(L.get("k_norm")),
+                                "kc": hip.hip_alloc(dev, 4 * nctx * self.kvd), "vc": hip.hip_alloc(dev, 4 * nctx * self.kvd)})
+        self.embd = up("token_embd", host["embd"], c["vocab"], d)
+        self.output = self.embd if host["output"] is host["embd"] else up("output", host["output"], c["vocab"], d)
+        self.output_norm = fl(host["output_norm"])
+        rope = np.empty((nctx, hd), np.float32)
+        hip.call("ilt_rope_table", C.c_int(hd), C.c_int(0), C.c_int(nctx), C.c_float(c["rope_base"]), rope.ctypes.data_as(C.c_void_p))
+        self.rope = hip.hip_upload_new(dev, rope)
+        n = chunk
+        A = lambda nbytes: hip.hip_alloc(dev, nbytes)
+        self.x, self.q, self.k, self.v = A(4 * n * d), A(4 * n * self.qd), A(4 * n * self.kvd), A(4 * n * self.kvd)
+        self.att, self.fa, self.fb = A(4 * n * self.qd), A(4 * n * ffn), A(4 * n * ffn)
+        self.tokens = A(4 * n)
+        self.logits = A(4 * c["vocab"])
+        self.acts = {cols: dense.QAct(dev, n, cols, ("q8k",)) for cols in {d, self.qd, ffn}}
+
+    def forward_n(self, tokens, logits=True):
+        """TOKENS at the next positions (CUDA-FORWARD-N); the last one's logits, if LOGITS, into self.logits."""
+        dev, c, n = self.dev, self.c, len(tokens)
+        d, ffn, hd, nh, nkv, eps = c["d"], c["ffn"], c["hd"], c["nh"], c["nkv"], c["eps"]
+        if n < 1 or n > self.chunk or self.pos + n > self.nctx:
+            raise ValueError(f"{n} tokens at position {self.pos}: the chunk holds {self.chunk}, the context {self.nctx}")
+        S = C.c_uint64(dev.stream)
+        P = lambda b, off=0: C.c_uint64(b.ptr + off if b is not None else 0)
+        hip.hip_upload_vector(self.tokens, np.asarray(tokens, np.int32))
+        dense.embed(dev, self.embd, self.tokens, self.x, n, d)
+        for L in self.layers:
+            if n == 1:
+                dense.qkv_mul(dev, L["wq"], L["wk"], L["wv"], None, self.q, self.k, self.v, xf=self.x, norm=(L["attn_norm"], eps))
+            else:
+                a = dense.rmsnorm_q8(dev, self.x, L["attn_norm"], self.acts[d], d, eps, n=n)
+                for w, y in ((L["wq"], self.q), (L["wk"], self.k), (L["wv"], self.v)):
+                    dense.cmat_mul(dev, w, a, y, n=n)
+            hip.call("ilt_qk_rope", S, P(self.q), P(self.k), P(self.v), P(L["q_norm"]), P(L["k_norm"]), P(self.rope), P(L["kc"]), P(L["vc"]),
+                     C.c_int(nh), C.c_int(nkv), C.c_int(hd), C.c_int(hd), C.c_int(self.pos), C.c_float(eps), C.c_int(1 if c["neox"] else 0),
+                     C.c_int(n))
+            hip.call("ilt_attn_rows", S, P(self.q), P(L["kc"]), P(L["vc"]), P(self.att), C.c_int(nh), C.c_int(nkv), C.c_int(hd),
+                     C.c_int(self.pos), C.c_int(n))
+            if n == 1:
+                dense.mv_multi(dev, [(L["wo"], self.x, None)], xf=self.att, acc=True)
+                dense.glu_mul(dev, L["gate"], L["up"], None, self.fa, xf=self.x, norm=(L["ffn_norm"], eps))
+                dense.mv_multi(dev, [(L["down"], self.x, None)], xf=self.fa, acc=True)
+            else:
+                dense.cmat_mul(dev, L["wo"], dense.quantize_act(dev, self.att, self.acts[self.qd], n=n), self.x, n=n, acc=True)
+                a = dense.rmsnorm_q8(dev, self.x, L["ffn_norm"], self.acts[d], d, eps, n=n)
+                dense.cmat_mul(dev, L["gate"], a, self.fa, n=n)
+                dense.cmat_mul(dev, L["up"], a, self.fb, n=n)
+                hip.call("ilt_swiglu", S, P(self.fa), P(self.fb), C.c_int64(n * ffn))
+                dense.cmat_mul(dev, L["down"], dense.quantize_act(dev, self.fa, self.acts[ffn], n=n), self.x, n=n, acc=True)
+        self.pos += n
+        if logits:
+            last = hip.DBuf(self.x.ptr + 4 * (n - 1) * d, 4 * d, dev)
+            dense.mv_multi(dev, [(self.output, self.logits, None)], xf=last, norm=(self.output_norm, eps))
+        return self.logits
+
+    def eval_tokens(self, tokens, logits=True):
+        """The prompt in chunks (CUDA-EVAL, cuda-dense.lisp:295-305); the logits of the last token only."""
+        tokens = list(tokens)
+        for i in range(0, len(tokens), self.chunk):
+            part = tokens[i:i + self.chunk]
+            self.forward_n(part, logits=logits and i + len(part) >= len(tokens))
+
+    def argmax(self):
+        """The greedy token of self.logits (ARGMAX, model.lisp:464-468: the first of equal ones)."""
+        return int(np.argmax(hip.hip_floats(self.logits, self.c["vocab"])))
+
+    def free(self):
+        for L in self.layers:
+            for v in L.values():
+                (v.free if hasattr(v, "free") else lambda: hip.hip_free(v))()
+        if self.output is not self.embd:
+            self.output.free()
+        self.embd.free()
+        for b in (self.output_norm, self.rope, self.x, self.q, self.k, self.v, self.att, self.fa, self.fb, self.tokens, self.logits):
+            hip.hip_free(b)
+        for a in self.acts.values():
+            a.free()

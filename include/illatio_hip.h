@@ -286,6 +286,24 @@ int ilt_d4_moe_sum(uint64_t stream, int d, int k, const float* down, const float
 int ilt_d4_moe_sum_rows(uint64_t stream, int d, int nu, int ntok, const float* down, const uint32_t* map,
                         const float* shared_, float* moe);
 
+/* Between the products of a dense decoder layer: what the forward harness (illatio_amd/model.py, the
+   reference's cuda-forward-n, cuda-dense.lisp:380-432) runs besides them.  The floats are the CPU path's
+   (model.lisp:205-334, 364-378), sum for sum, so a token's logits have the CPU path's bits.
+   qk_rope (dense.cu:318-362, the same arguments; tokens = grid y): the head norms where qn / kn are given,
+     RoPE from rope (a position's rd/2 cosines then rd/2 sines; rope-table, model.lisp:218-231, made by the
+     host), K and V of token t into the caches at position pos0 + t.
+   attn_rows: attend-head! for every query head of ntok tokens, token t over positions 0 .. pos0 + t; scores
+     in F32-DOT16's order, the softmax's sum in double, the values added position after position.  It stands
+     where the reference launches attn_decode + attn_merge / attn_prefill (dense.cu:376-727), whose partial
+     sums meet in another order.
+   swiglu (dense.cu:307): swiglu! on n values, a = (a / (1 + e^-a)) * b, the exponential through double. */
+/* The table qk_rope takes, for positions pos0 .. pos0 + n - 1, written to host memory (n * head_dim floats). */
+int ilt_rope_table(int head_dim, int pos0, int n, float base, float* out);
+int ilt_qk_rope(uint64_t stream, float* q, float* k, const float* v, const float* qn, const float* kn, const float* rope, float* kc,
+                float* vc, int nh, int nkv, int hd, int rd, int pos0, float eps, int neox, int ntok);
+int ilt_attn_rows(uint64_t stream, const float* q, const float* kc, const float* vc, float* out, int nh, int nkv, int hd, int pos0, int ntok);
+int ilt_swiglu(uint64_t stream, float* a, const float* b, int64_t n);
+
 /* Prefill products on the int8 matrix cores, y[t*rows + r] = W[r].x_t (+ bias[r]) for n
    tokens, each (row, token) with the decode kernel's bits (CPU: MATMUL!, batch.lisp:128-205,
    "bit-identical to feeding the tokens one at a time", :10-12).

@@ -26,6 +26,7 @@
  * correctly rounded value, which SBCL's libm call yields except where the
  * double result falls within ~2^-29 of a single-precision rounding boundary.
  */
+#include <float.h>
 #include <math.h>
 #include <pthread.h>
 #include <stdint.h>
@@ -365,20 +366,78 @@ void orc_dequant_row(int type, const uint8_t* wrow, int64_t cols, float* out) {
   }
 }
 
-/* ---- a thread pool's share: src/pool.lisp:162-165 ------------------------------------------------- */
+/* ---- the thread pool: src/pool.lisp:120-178.  Workers that stay: a worker spins on the pool's generation
+        for a while after a job, then parks on a condition variable; pool-run publishes the job, wakes
+        sleepers if there are any, runs share 0 itself and spins until the others are done.  One pool,
+        remade when another size is asked for. ------------------------------------------------------------ */
 typedef void (*orc_job_fn)(void* arg, int index, int count);
-typedef struct { orc_job_fn fn; void* arg; int index, count; } orc_job;
-static void* orc_job_main(void* p) { orc_job* j = (orc_job*)p; j->fn(j->arg, j->index, j->count); return NULL; }
+typedef struct {
+  int size, stop;
+  pthread_t* th;
+  orc_job_fn fn; void* arg;
+  unsigned generation; int pending, sleepers;
+  pthread_mutex_t lock; pthread_cond_t wake;
+} orc_pool;
+typedef struct { orc_pool* p; int index; } orc_worker_arg;
+static orc_pool* g_pool = NULL;
+static pthread_mutex_t g_pool_lock = PTHREAD_MUTEX_INITIALIZER;
+#define ORC_SPINS 200000
+
+static void* orc_worker(void* va) {
+  orc_worker_arg* wa = (orc_worker_arg*)va;
+  orc_pool* p = wa->p; const int index = wa->index;
+  free(wa);
+  unsigned seen = 0;
+  for (;;) {
+    int spins = 0;
+    while (__atomic_load_n(&p->generation, __ATOMIC_ACQUIRE) == seen && !__atomic_load_n(&p->stop, __ATOMIC_ACQUIRE)) {
+      if (++spins < ORC_SPINS) { __builtin_ia32_pause(); continue; }
+      pthread_mutex_lock(&p->lock);
+      __atomic_fetch_add(&p->sleepers, 1, __ATOMIC_SEQ_CST);
+      while (__atomic_load_n(&p->generation, __ATOMIC_ACQUIRE) == seen && !p->stop) pthread_cond_wait(&p->wake, &p->lock);
+      __atomic_fetch_sub(&p->sleepers, 1, __ATOMIC_SEQ_CST);
+      pthread_mutex_unlock(&p->lock);
+    }
+    if (__atomic_load_n(&p->stop, __ATOMIC_ACQUIRE)) return NULL;
+    seen = __atomic_load_n(&p->generation, __ATOMIC_ACQUIRE);
+    p->fn(p->arg, index, p->size);
+    __atomic_fetch_sub(&p->pending, 1, __ATOMIC_RELEASE);
+  }
+}
+static void orc_pool_free(orc_pool* p) {
+  pthread_mutex_lock(&p->lock);
+  __atomic_store_n(&p->stop, 1, __ATOMIC_RELEASE);
+  pthread_cond_broadcast(&p->wake);
+  pthread_mutex_unlock(&p->lock);
+  for (int i = 1; i < p->size; i++) pthread_join(p->th[i], NULL);
+  free(p->th); free(p);
+}
+static orc_pool* orc_pool_of(int size) {
+  if (g_pool && g_pool->size == size) return g_pool;
+  if (g_pool) { orc_pool_free(g_pool); g_pool = NULL; }
+  orc_pool* p = (orc_pool*)calloc(1, sizeof(orc_pool));
+  p->size = size; p->th = (pthread_t*)calloc(size, sizeof(pthread_t));
+  pthread_mutex_init(&p->lock, NULL); pthread_cond_init(&p->wake, NULL);
+  for (int i = 1; i < size; i++) {
+    orc_worker_arg* wa = (orc_worker_arg*)malloc(sizeof(orc_worker_arg));
+    wa->p = p; wa->index = i;
+    pthread_create(&p->th[i], NULL, orc_worker, wa);
+  }
+  return g_pool = p;
+}
 static void orc_pool_run(int nthreads, orc_job_fn fn, void* arg) {
   if (nthreads <= 1) { fn(arg, 0, 1); return; }
-  pthread_t* th = (pthread_t*)malloc(sizeof(pthread_t) * nthreads);
-  orc_job* jobs = (orc_job*)malloc(sizeof(orc_job) * nthreads);
-  for (int i = 0; i < nthreads; i++) {
-    jobs[i].fn = fn; jobs[i].arg = arg; jobs[i].index = i; jobs[i].count = nthreads;
-    pthread_create(&th[i], NULL, orc_job_main, &jobs[i]);
+  pthread_mutex_lock(&g_pool_lock);                   /* one caller at a time */
+  orc_pool* p = orc_pool_of(nthreads);
+  p->fn = fn; p->arg = arg;
+  __atomic_store_n(&p->pending, p->size - 1, __ATOMIC_RELEASE);
+  __atomic_fetch_add(&p->generation, 1, __ATOMIC_SEQ_CST);
+  if (__atomic_load_n(&p->sleepers, __ATOMIC_SEQ_CST) > 0) {
+    pthread_mutex_lock(&p->lock); pthread_cond_broadcast(&p->wake); pthread_mutex_unlock(&p->lock);
   }
-  for (int i = 0; i < nthreads; i++) pthread_join(th[i], NULL);
-  free(th); free(jobs);
+  fn(arg, 0, p->size);
+  while (__atomic_load_n(&p->pending, __ATOMIC_ACQUIRE) != 0) __builtin_ia32_pause();
+  pthread_mutex_unlock(&g_pool_lock);
 }
 static inline void share(int64_t n, int index, int count, int64_t* s, int64_t* e) {
   *s = n * index / count; *e = n * (index + 1) / count;
@@ -718,4 +777,119 @@ void orc_moe_chunk(const uint8_t* gate, const uint8_t* up, const uint8_t* down, 
   if (counts_out) memcpy(counts_out, counts, sizeof(int32_t) * ne);
   free(sels); free(ws); free(counts); free(experts); free(ubase); free(ebase); free(users); free(fill);
   free(xq); free(xd); free(xbs); free(mid); free(mq); free(md); free(mbs); free(downs);
+}
+
+/* ---- the dense decoder, one token: src/model.lisp:205-462 (forward-1 and what it calls) ------------------ */
+/* rope-table (model.lisp:218-231): theta advanced by repeated single-float multiplication from pos;
+   theta-scale = expt(base, -2/hd), which SBCL evaluates through double pow and rounds to single; cos and sin of
+   a single float likewise through double. */
+void orc_rope_table(int head_dim, int pos, float base, float* cosv, float* sinv) {
+  const int half = head_dim / 2;
+  const float e = -2.0f / (float)head_dim;
+  const float theta_scale = (float)pow((double)base, (double)e);
+  float theta = (float)pos;
+  for (int i = 0; i < half; i++) {
+    cosv[i] = (float)cos((double)theta); sinv[i] = (float)sin((double)theta);
+    theta = theta * theta_scale;
+  }
+}
+/* rope-head! (model.lisp:233-244): pairs (i, i + half) when neox, else (2i, 2i + 1) */
+void orc_rope_head(float* x, int head_dim, int neox, const float* cosv, const float* sinv) {
+  const int half = head_dim / 2;
+  for (int i = 0; i < half; i++) {
+    const int a = neox ? i : 2 * i, b = neox ? i + half : 2 * i + 1;
+    const float x0 = x[a], x1 = x[b], c = cosv[i], s = sinv[i];
+    volatile float p0 = x0 * c, p1 = x1 * s, p2 = x0 * s, p3 = x1 * c;
+    x[a] = p0 - p1; x[b] = p2 + p3;
+  }
+}
+/* attend-head! (model.lisp:298-334): scores in f32-dot16's order times 1/sqrt(hd); softmax with exp in single
+   (through double, as SBCL evaluates it), the sum in double, scaled by single(1/sum); then out += score * V row,
+   position after position.  kc, vc: the layer's caches, kvd floats a position; ko: the KV head's offset. */
+void orc_attend_head(const float* kc, const float* vc, const float* q, float* out, int n, int hd, int kvd, int ko, float* scores) {
+  const float scale = 1.0f / sqrtf((float)hd);
+  float mx = -FLT_MAX;
+  for (int p = 0; p < n; p++) {
+    const float s = orc_f32_dot16(kc + (int64_t)p * kvd + ko, q, hd) * scale;
+    scores[p] = s;
+    if (s > mx) mx = s;
+  }
+  double sum = 0.0;
+  for (int p = 0; p < n; p++) { const float e = sb_exp(scores[p] - mx); scores[p] = e; sum += (double)e; }
+  const float inv = (float)(1.0 / sum);
+  for (int p = 0; p < n; p++) scores[p] = scores[p] * inv;
+  for (int i = 0; i < hd; i++) out[i] = 0.0f;
+  for (int p = 0; p < n; p++) {
+    const float w = scores[p]; const float* v = vc + (int64_t)p * kvd + ko;
+    for (int i = 0; i < hd; i++) { volatile float t = w * v[i]; out[i] = out[i] + t; }
+  }
+}
+
+typedef struct {
+  const uint8_t *wq, *wk, *wv, *wo, *wgate, *wup, *wdown;
+  int tq, tk, tv, to, tg, tu, td;                       /* GGUF type codes */
+  const float *attn_norm, *ffn_norm, *q_norm, *k_norm;  /* q_norm, k_norm: null for a model without head norms */
+  const float *bq, *bk, *bv;                            /* or null */
+} orc_layer;
+typedef struct {
+  int d, ffn, nh, nkv, hd, nl, vocab, neox;
+  float eps, rope_base;
+  const uint8_t *embd, *output; int embd_type, output_type;
+  const float* output_norm;
+  const orc_layer* layers;
+} orc_model;
+
+static void orc_qmv(int type, const uint8_t* w, int64_t rows, int64_t cols, const float* x, const float* bias, float* out, int nt) {
+  orc_matmul(type, w, rows, cols, x, 1, 1, out, nt);   /* quantize-act! (Q8_0 scales through f16) + qmatvec! */
+  if (bias) for (int64_t r = 0; r < rows; r++) out[r] = out[r] + bias[r];
+}
+typedef struct { const orc_model* m; const float *kc, *vc, *q; float* att; int n; float* scores; } orc_att_args;
+static void orc_att_job(void* p, int index, int count) {
+  orc_att_args* a = (orc_att_args*)p;
+  const orc_model* m = a->m;
+  int64_t s, e; share(m->nh, index, count, &s, &e);
+  const int group = m->nh / m->nkv, kvd = m->nkv * m->hd;
+  for (int64_t h = s; h < e; h++)
+    orc_attend_head(a->kc, a->vc, a->q + h * m->hd, a->att + h * m->hd, a->n, m->hd, kvd, (int)(h / group) * m->hd, a->scores + h * a->n);
+}
+/* forward-1 (model.lisp:396-462) at position pos; kcache/vcache: nl x nctx x kvd floats.  logits may be null. */
+void orc_forward(const orc_model* m, int token, int pos, float* kcache, float* vcache, int nctx, float* logits, float* x_out, int nthreads) {
+  const int d = m->d, hd = m->hd, kvd = m->nkv * m->hd, qd = m->nh * m->hd;
+  float* x = (float*)malloc(sizeof(float) * d); float* h = (float*)malloc(sizeof(float) * d);
+  float* q = (float*)malloc(sizeof(float) * qd); float* k = (float*)malloc(sizeof(float) * kvd); float* v = (float*)malloc(sizeof(float) * kvd);
+  float* att = (float*)malloc(sizeof(float) * qd);
+  float* fa = (float*)malloc(sizeof(float) * m->ffn); float* fb = (float*)malloc(sizeof(float) * m->ffn);
+  float* cosv = (float*)malloc(sizeof(float) * hd); float* sinv = cosv + hd / 2;
+  float* scores = (float*)malloc(sizeof(float) * (size_t)m->nh * (pos + 1));
+  const int64_t erb = m->d / (m->embd_type == ORC_Q8_0 ? 32 : QK_K) * orc_block_bytes(m->embd_type);
+  orc_dequant_row(m->embd_type, m->embd + (int64_t)token * erb, d, x);
+  orc_rope_table(hd, pos, m->rope_base, cosv, sinv);
+  for (int li = 0; li < m->nl; li++) {
+    const orc_layer* l = &m->layers[li];
+    float* kc = kcache + (int64_t)li * nctx * kvd; float* vc = vcache + (int64_t)li * nctx * kvd;
+    orc_rmsnorm(x, l->attn_norm, h, m->eps, d);
+    orc_qmv(l->tq, l->wq, qd, d, h, l->bq, q, nthreads);
+    orc_qmv(l->tk, l->wk, kvd, d, h, l->bk, k, nthreads);
+    orc_qmv(l->tv, l->wv, kvd, d, h, l->bv, v, nthreads);
+    for (int u = 0; u < m->nh; u++) { if (l->q_norm) orc_rmsnorm(q + u * hd, l->q_norm, q + u * hd, m->eps, hd); orc_rope_head(q + u * hd, hd, m->neox, cosv, sinv); }
+    for (int u = 0; u < m->nkv; u++) { if (l->k_norm) orc_rmsnorm(k + u * hd, l->k_norm, k + u * hd, m->eps, hd); orc_rope_head(k + u * hd, hd, m->neox, cosv, sinv); }
+    memcpy(kc + (int64_t)pos * kvd, k, sizeof(float) * kvd);
+    memcpy(vc + (int64_t)pos * kvd, v, sizeof(float) * kvd);
+    orc_att_args aa = { m, kc, vc, q, att, pos + 1, scores };
+    orc_pool_run(nthreads, orc_att_job, &aa);
+    orc_qmv(l->to, l->wo, d, qd, att, NULL, h, nthreads);
+    for (int i = 0; i < d; i++) x[i] = x[i] + h[i];
+    orc_rmsnorm(x, l->ffn_norm, h, m->eps, d);
+    orc_qmv(l->tg, l->wgate, m->ffn, d, h, NULL, fa, nthreads);
+    orc_qmv(l->tu, l->wup, m->ffn, d, h, NULL, fb, nthreads);
+    for (int i = 0; i < m->ffn; i++) fa[i] = orc_swiglu(fa[i], fb[i]);
+    orc_qmv(l->td, l->wdown, d, m->ffn, fa, NULL, h, nthreads);
+    for (int i = 0; i < d; i++) x[i] = x[i] + h[i];
+  }
+  if (x_out) memcpy(x_out, x, sizeof(float) * d);
+  if (logits) {
+    orc_rmsnorm(x, m->output_norm, h, m->eps, d);
+    orc_qmv(m->output_type, m->output, m->vocab, d, h, NULL, logits, nthreads);
+  }
+  free(x); free(h); free(q); free(k); free(v); free(att); free(fa); free(fb); free(cosv); free(scores);
 }

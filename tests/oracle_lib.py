@@ -250,3 +250,71 @@ def moe_chunk(gate, up, down, d, ff, ne, nu, scale, clamp, logits, norms, shared
                         C.c_int(ne), C.c_int(nu), C.c_float(scale), C.c_float(clamp), C.c_int(n), _p(logits), _p(b),
                         _p(norms), _p(sh), _p(out), _p(sel), _p(w), _p(counts), C.c_int(nthreads))
     return out, sel, w, counts
+
+
+# ---- the dense decoder (model.lisp:205-462) ---------------------------------------------------------
+def rope_table(head_dim, pos, base):
+    c, s = np.empty(head_dim // 2, np.float32), np.empty(head_dim // 2, np.float32)
+    lib().orc_rope_table(C.c_int(head_dim), C.c_int(pos), C.c_float(base), _p(c), _p(s))
+    return c, s
+
+
+def rope_head(x, neox, cosv, sinv):
+    x = np.array(x, np.float32)
+    lib().orc_rope_head(_p(x), C.c_int(x.size), C.c_int(1 if neox else 0), _p(_c(cosv, np.float32)), _p(_c(sinv, np.float32)))
+    return x
+
+
+def attend_head(kc, vc, q, n, hd, kvd, ko):
+    out, scores = np.empty(hd, np.float32), np.empty(n, np.float32)
+    lib().orc_attend_head(_p(_c(kc, np.float32)), _p(_c(vc, np.float32)), _p(_c(q, np.float32)), _p(out), C.c_int(n), C.c_int(hd),
+                          C.c_int(kvd), C.c_int(ko), _p(scores))
+    return out, scores
+
+
+class _Layer(C.Structure):
+    _fields_ = [(n, C.c_void_p) for n in ("wq", "wk", "wv", "wo", "wgate", "wup", "wdown")] + \
+               [(n, C.c_int) for n in ("tq", "tk", "tv", "to", "tg", "tu", "td")] + \
+               [(n, C.c_void_p) for n in ("attn_norm", "ffn_norm", "q_norm", "k_norm", "bq", "bk", "bv")]
+
+
+class _Model(C.Structure):
+    _fields_ = [(n, C.c_int) for n in ("d", "ffn", "nh", "nkv", "hd", "nl", "vocab", "neox")] + [("eps", C.c_float), ("rope_base", C.c_float),
+               ("embd", C.c_void_p), ("output", C.c_void_p), ("embd_type", C.c_int), ("output_type", C.c_int), ("output_norm", C.c_void_p),
+               ("layers", C.POINTER(_Layer))]
+
+
+class DenseModel:
+    """The CPU side of a dense decoder: HOST = a dict as illatio_amd.model.synth_model makes it (numpy arrays)."""
+
+    def __init__(self, host, nctx):
+        self.h, self.nctx = host, nctx
+        c = host["config"]
+        self.keep = []
+
+        def ptr(a):
+            if a is None:
+                return None
+            self.keep.append(a)
+            return a.ctypes.data
+        self.layers = (_Layer * c["nl"])()
+        for i, L in enumerate(host["layers"]):
+            self.layers[i] = _Layer(*[ptr(L[n][1]) for n in ("wq", "wk", "wv", "wo", "gate", "up", "down")],
+                                    *[L[n][0] for n in ("wq", "wk", "wv", "wo", "gate", "up", "down")],
+                                    ptr(L["attn_norm"]), ptr(L["ffn_norm"]), ptr(L.get("q_norm")), ptr(L.get("k_norm")),
+                                    ptr(L.get("bq")), ptr(L.get("bk")), ptr(L.get("bv")))
+        self.m = _Model(c["d"], c["ffn"], c["nh"], c["nkv"], c["hd"], c["nl"], c["vocab"], 1 if c["neox"] else 0, c["eps"], c["rope_base"],
+                        ptr(host["embd"][1]), ptr(host["output"][1]), host["embd"][0], host["output"][0], ptr(host["output_norm"]), self.layers)
+        kvd = c["nkv"] * c["hd"]
+        self.kc = np.zeros((c["nl"], nctx, kvd), np.float32)
+        self.vc = np.zeros((c["nl"], nctx, kvd), np.float32)
+        self.pos = 0
+
+    def forward(self, token, logits=True, nthreads=8):
+        c = self.h["config"]
+        lg = np.empty(c["vocab"], np.float32) if logits else None
+        x = np.empty(c["d"], np.float32)
+        lib().orc_forward(C.byref(self.m), C.c_int(int(token)), C.c_int(self.pos), _p(self.kc), _p(self.vc), C.c_int(self.nctx), _p(lg), _p(x),
+                          C.c_int(nthreads))
+        self.pos += 1
+        return lg, x

@@ -565,3 +565,112 @@ def test_iq2xxs_even_and_odd_group_sums_are_exact_in_float():
     assert len(grid) == 256 and {(g >> (8 * i)) & 0xFF for g in grid for i in range(8)} == {0x08, 0x19, 0x2B}
     largest = max(sum((g >> (8 * i)) & 0xFF for i in range(8)) for g in grid)
     assert 4 * 31 * 4 * 128 * largest < 2 ** 24          # twice the largest |partial sum|, as an integer
+
+
+# ---- the dense decoder's pieces (model.lisp:205-462) ---------------------------------------------------
+def test_rope_table_and_rope_head():
+    """rope-table (model.lisp:218-231): theta advanced by repeated single multiplication from pos, theta-scale
+    through double pow, cos and sin through double; against numpy with each rounding explicit.  A fresh power per
+    pair (the misreading the reference's docstring warns of) gives other bits somewhere.  rope-head!: the pairs
+    (i, i + half) when neox, (2i, 2i + 1) else, rotated by the table."""
+    f32, f64 = np.float32, np.float64
+    told = False
+    for hd, base in ((128, 1e6), (64, 10000.0)):
+        ts = f32(np.power(f64(f32(base)), f64(f32(-2.0) / f32(hd))))
+        for pos in (0, 1, 7, 511, 4000):
+            c, s = orc.rope_table(hd, pos, base)
+            theta = f32(pos)
+            for i in range(hd // 2):
+                assert c[i] == f32(np.cos(f64(theta))) and s[i] == f32(np.sin(f64(theta))), (hd, pos, i)
+                fresh = f32(f32(pos) * f32(np.power(f64(f32(base)), f64(f32(-2.0 * i) / f32(hd)))))
+                told = told or (pos > 0 and f32(np.cos(f64(fresh))) != c[i])
+                theta = f32(theta * ts)
+            if pos == 0:
+                assert np.all(c == 1) and np.all(s == 0)
+    assert told
+    x = np.arange(1, 9, dtype=f32)
+    quarter = (np.zeros(4, f32), np.ones(4, f32))                   # cos 0, sin 1: (x0, x1) -> (-x1, x0)
+    assert orc.rope_head(x, True, *quarter).tolist() == [-5, -6, -7, -8, 1, 2, 3, 4]
+    assert orc.rope_head(x, False, *quarter).tolist() == [-2, 1, -4, 3, -6, 5, -8, 7]
+    rng = synth.make_rng(31)
+    v = rng.standard_normal(128).astype(f32)
+    c, s = orc.rope_table(128, 77, 1e6)
+    got = orc.rope_head(v, True, c, s)
+    want = v.copy()
+    want[:64] = (v[:64] * c).astype(f32) - (v[64:] * s).astype(f32)
+    want[64:] = (v[:64] * s).astype(f32) + (v[64:] * c).astype(f32)
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+    assert abs(float(np.dot(got, got)) - float(np.dot(v, v))) < 1e-3 * float(np.dot(v, v))      # a rotation
+
+
+def test_attend_head_against_explicit_evaluation():
+    """attend-head! (model.lisp:298-334): scores = f32-dot16 * 1/sqrt(hd); exp of a single (through double); the sum
+    in double, position after position; every score times single(1/sum); out += score * V row, position after
+    position.  Against numpy with each rounding explicit; a float sum or products kept exact in the output give
+    other bits.  Equal keys: the mean of the values."""
+    f32, f64 = np.float32, np.float64
+    rng = synth.make_rng(32)
+    told = set()
+    for n, hd, nkv in ((1, 64, 1), (5, 64, 2), (130, 128, 2), (300, 128, 8)):
+        kvd = nkv * hd
+        ko = (nkv - 1) * hd
+        kc, vc = rng.standard_normal((n, kvd)).astype(f32), rng.standard_normal((n, kvd)).astype(f32)
+        q = (rng.standard_normal(hd) * 2).astype(f32)
+        out, scores = orc.attend_head(kc, vc, q, n, hd, kvd, ko)
+        scale = f32(1) / np.sqrt(f32(hd))
+        sc = np.array([f32(orc.f32_dot16(kc[p, ko:ko + hd], q) * scale) for p in range(n)], f32)
+        e = np.exp((sc - sc.max()).astype(f32).astype(f64)).astype(f32)
+        tot, ftot = f64(0), f32(0)
+        for v in e:
+            tot += f64(v); ftot = f32(ftot + v)
+        w = (e * f32(f64(1) / tot)).astype(f32)
+        assert np.array_equal(scores.view(np.uint32), w.view(np.uint32)), n
+        acc, exact = np.zeros(hd, f32), np.zeros(hd, f64)
+        for p in range(n):
+            acc = (acc + (w[p] * vc[p, ko:ko + hd]).astype(f32)).astype(f32)
+            exact = (exact + f64(w[p]) * vc[p, ko:ko + hd].astype(f64)).astype(f32).astype(f64)
+        assert np.array_equal(out.view(np.uint32), acc.view(np.uint32)), n
+        if not np.array_equal((e * f32(f32(1) / ftot)).astype(f32).view(np.uint32), w.view(np.uint32)):
+            told.add("float sum")
+        if not np.array_equal(exact.astype(f32).view(np.uint32), out.view(np.uint32)):
+            told.add("fused output")
+    assert told == {"float sum", "fused output"}, told
+    kc = np.tile(rng.standard_normal(64).astype(f32), (8, 1)); vc = rng.standard_normal((8, 64)).astype(f32)
+    out, scores = orc.attend_head(kc, vc, rng.standard_normal(64).astype(f32), 8, 64, 64, 0)
+    assert np.all(scores == f32(0.125)) and np.allclose(out, vc.mean(axis=0), atol=1e-6)
+
+
+def test_forward_is_its_pieces_in_order():
+    """forward-1 (model.lisp:396-462) on a tiny model, three tokens: put together by hand from the functions the
+    tests above pin (rmsnorm!, the quantized products, rope, attend-head!, swiglu!), the caches included."""
+    from illatio_amd import model
+    f32 = np.float32
+    host = model.synth_model(5, d=256, ffn=512, nh=4, nkv=2, hd=64, nl=2, vocab=300)
+    c = host["config"]
+    d, ffn, nh, nkv, hd = c["d"], c["ffn"], c["nh"], c["nkv"], c["hd"]
+    qd, kvd = nh * hd, nkv * hd
+    cpu = orc.DenseModel(host, nctx=8)
+    kc, vc = np.zeros((c["nl"], 8, kvd), f32), np.zeros((c["nl"], 8, kvd), f32)
+    for pos, tok in enumerate((17, 299, 0)):
+        logits, xout = cpu.forward(tok, nthreads=2)
+        x = orc.dequant_rows(host["embd"][0], host["embd"][1][tok:tok + 1], d)[0]
+        cs, sn = orc.rope_table(hd, pos, c["rope_base"])
+        for li, L in enumerate(host["layers"]):
+            h = orc.rmsnorm(x, L["attn_norm"], c["eps"])
+            q = orc.matmul(L["wq"][0], L["wq"][1], qd, d, h); k = orc.matmul(L["wk"][0], L["wk"][1], kvd, d, h)
+            v = orc.matmul(L["wv"][0], L["wv"][1], kvd, d, h)
+            for u in range(nh):
+                q[u * hd:(u + 1) * hd] = orc.rope_head(orc.rmsnorm(q[u * hd:(u + 1) * hd], L["q_norm"], c["eps"]), True, cs, sn)
+            for u in range(nkv):
+                k[u * hd:(u + 1) * hd] = orc.rope_head(orc.rmsnorm(k[u * hd:(u + 1) * hd], L["k_norm"], c["eps"]), True, cs, sn)
+            kc[li, pos], vc[li, pos] = k, v
+            att = np.concatenate([orc.attend_head(kc[li], vc[li], q[u * hd:(u + 1) * hd], pos + 1, hd, kvd, (u // (nh // nkv)) * hd)[0]
+                                  for u in range(nh)])
+            x = (x + orc.matmul(L["wo"][0], L["wo"][1], d, qd, att)).astype(f32)
+            h = orc.rmsnorm(x, L["ffn_norm"], c["eps"])
+            mid = orc.swiglu(orc.matmul(L["gate"][0], L["gate"][1], ffn, d, h), orc.matmul(L["up"][0], L["up"][1], ffn, d, h))
+            x = (x + orc.matmul(L["down"][0], L["down"][1], d, ffn, mid)).astype(f32)
+        assert np.array_equal(xout.view(np.uint32), x.view(np.uint32)), pos
+        want = orc.matmul(host["output"][0], host["output"][1], c["vocab"], d, orc.rmsnorm(x, host["output_norm"], c["eps"]))
+        assert np.array_equal(logits.view(np.uint32), want.view(np.uint32)), pos
+        assert np.array_equal(cpu.kc[:, :pos + 1], kc[:, :pos + 1]) and np.array_equal(cpu.vc[:, :pos + 1], vc[:, :pos + 1])
