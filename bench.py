@@ -599,7 +599,52 @@ def workload_c5(args, dev):
             "extra": {"pct_of_mfma_peak": round(100 * tf / MFMA_PEAK_TFLOPS[args.path], 2)}, "roofline": roof, "cpu": cpu}
 
 
-WORKLOADS = {"c1": workload_c1, "c2": workload_c2, "c3": workload_c3, "c4": workload_c4, "c5": workload_c5}
+def workload_c2d(args, dev):
+    """Config 2 as it is stated: the whole dense decoder at the Qwen3-4B shape (36 layers, head norms, RoPE,
+    grouped-query attention over an fp32 KV cache, Q4_K / Q6_K weights), random-init: a 512-token prompt through the
+    prefill products, then a 256-token greedy decode at batch 1.  A step is one decoded token, logits downloaded and
+    the next token picked on the host (as the reference's loop does, cuda-dense.lisp:428-430)."""
+    from illatio_amd import hip, model, synth
+    nl, nprompt, ndecode = args.layers, 512, 256
+    host = model.synth_model(2, nl=nl)
+    c = host["config"]
+    m = model.DenseModel(dev, host, nctx=nprompt + ndecode + args.warmup + 8, chunk=512)
+    rng = synth.make_rng(3)
+    prompt = rng.integers(0, c["vocab"], nprompt).tolist()
+    hip.hip_sync(dev)
+    t0 = time.perf_counter()
+    m.eval_tokens(prompt)
+    hip.hip_sync(dev)
+    prefill_s = time.perf_counter() - t0
+    tok = m.argmax()
+    for _ in range(args.warmup):
+        m.forward_n([tok]); tok = m.argmax()
+    hip.hip_sync(dev)
+    t0 = time.perf_counter()
+    toks = []
+    for _ in range(ndecode):
+        m.forward_n([tok])
+        tok = m.argmax()
+        toks.append(tok)
+    decode_s = time.perf_counter() - t0
+    wbytes = sum(a[1].size for L in host["layers"] for k, a in L.items() if isinstance(a, tuple)) + host["output"][1].size
+    ms = decode_s * 1e3 / ndecode
+    m.free()
+    return {"value": round(ndecode / decode_s, 1), "unit": "tok/s", "ms_per_step": ms, "device_ms_per_step": ms, "enqueue_ms": 0.0,
+            "dtype": "int8 block dots, fp32 combine; fp32 attention",
+            "metric": "decode tok/s at Qwen3-4B shape",
+            "config": {"workload": f"c2 decode: qwen3-4b-shape dense decoder, {nl} layers, random-init Q4_K/Q6_K, {nprompt}-token prompt then "
+                                   f"{ndecode}-token greedy decode at batch 1", "weight_bytes_per_token": int(wbytes)},
+            "extra": {"prefill_tok_per_s": round(nprompt / prefill_s, 1), "distinct_tokens_decoded": len(set(toks)),
+                      "weights_GBps_in_decode": round(wbytes / (ms * 1e-3) / 1e9, 1)},
+            "roofline": {"bound": "hbm", "achieved": round(wbytes / (ms * 1e-3) / 1e9, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                         "frac": round(wbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4), "traffic": None,
+                         "kernel": "whole token: 6 launches a layer (Q/K/V, qk_rope, attn_rows, wo, gate+up, down) + embedding + head, logits to the host",
+                         "launches": 6 * nl + 2, "avg_launch_us": round(ms * 1e3 / (6 * nl + 2), 2)},
+            "cpu": lambda: None}
+
+
+WORKLOADS = {"c1": workload_c1, "c2": workload_c2, "c2d": workload_c2d, "c3": workload_c3, "c4": workload_c4, "c5": workload_c5}
 
 
 def main():
@@ -650,20 +695,24 @@ def main():
         import copy
         import gc
         out["configs"] = {}
-        extras = [("c1", {}), ("c3", {"path": "bf16", "tokens": 4096}), ("c3_exact", {"path": "int8", "tokens": 4096}),
+        extras = [("c2_decode", {}), ("c1", {}), ("c3", {"path": "bf16", "tokens": 4096}), ("c3_exact", {"path": "int8", "tokens": 4096}),
                   ("c4", {"mode": "device"}), ("c5", {"path": "bf16", "tokens": 4096}), ("c5_exact", {"path": "int8", "tokens": 4096})]
         for name, over in extras:
             a = copy.copy(args)
-            a.workload, a.steps, a.warmup = name[:2], min(args.steps, 10), min(args.warmup, 3)
+            a.workload, a.steps, a.warmup = ("c2d" if name == "c2_decode" else name[:2]), min(args.steps, 10), min(args.warmup, 3)
             for k, v in over.items():
                 setattr(a, k, v)
             del r
             gc.collect()
             r = WORKLOADS[a.workload](a, dev)
             roof = r["roofline"]
+            if name == "c2_decode":
+                out["decode_tok_per_s"] = r["value"]
+                out["decode_ms_per_token"] = round(r["ms_per_step"], 4)
+                out["prefill_tok_per_s"] = r["extra"]["prefill_tok_per_s"]
             out["configs"][name] = {
                 "workload": r["config"]["workload"], "value": r["value"], "unit": r["unit"], "ms_per_step": round(r["ms_per_step"], 4),
-                "steps": a.steps, "warmup": a.warmup, "dtype": r["dtype"],
+                "steps": a.steps, "warmup": a.warmup, "dtype": r["dtype"], "extra": r["extra"],
                 "roofline": {k: roof.get(k) for k in ("bound", "achieved", "peak", "unit", "frac", "traffic", "kernel", "launches", "avg_launch_us",
                                                       "launch_us_all", "other_kernels")}}
     print(json.dumps(out))

@@ -772,9 +772,10 @@ int ilt_rope_table(int head_dim, int pos0, int n, float base, float* out) {
   }
   return ILT_OK;
 }
-int ilt_attn_rows(uint64_t stream, const float* q, const float* kc, const float* vc, float* out, int nh, int nkv, int hd, int pos0, int ntok) {
+int ilt_attn_rows(uint64_t stream, const float* q, const float* kc, const float* vc, float* out, int nh, int nkv, int hd, int pos0, int ntok,
+                  float* scratch) {
   ILT_REQUIRE(ntok >= 0 && (ntok == 0 || (q && kc && vc && out)) && nh > 0 && nkv > 0);
-  return (int)ilt_k_attn_rows(q, kc, vc, out, nh, nkv, hd, pos0, ntok, S(stream));
+  return (int)ilt_k_attn_rows(q, kc, vc, out, nh, nkv, hd, pos0, ntok, scratch, S(stream));
 }
 int ilt_swiglu(uint64_t stream, float* a, const float* b, int64_t n) {
   ILT_REQUIRE(n >= 0 && (n == 0 || (a && b)));
@@ -837,7 +838,7 @@ int ilt_launch(const char* kernel, unsigned gx, unsigned gy, unsigned gz, unsign
   K("qk_rope") return ilt_qk_rope(stream, a.ptr<float*>(0), a.ptr<float*>(1), a.ptr<cf>(2), a.ptr<cf>(3), a.ptr<cf>(4), a.ptr<cf>(5), a.ptr<float*>(6),
                                   a.ptr<float*>(7), a.i32(8), a.i32(9), a.i32(10), a.i32(11), a.i32(12), a.f32(13), a.i32(14), (int)gy);
   K("swiglu") return ilt_swiglu(stream, a.ptr<float*>(0), a.ptr<cf>(1), a.i64(2));
-  K("attn_rows") return ilt_attn_rows(stream, a.ptr<cf>(0), a.ptr<cf>(1), a.ptr<cf>(2), a.ptr<float*>(3), a.i32(4), a.i32(5), a.i32(6), a.i32(7), (int)gy);
+  K("attn_rows") return ilt_attn_rows(stream, a.ptr<cf>(0), a.ptr<cf>(1), a.ptr<cf>(2), a.ptr<float*>(3), a.i32(4), a.i32(5), a.i32(6), a.i32(7), (int)gy, a.ptr<float*>(8));
   K("d4_rows_expert") return ilt_d4_rows_expert(stream, a.i32(0), a.ptr<cu32>(1), a.ptr<cu32>(2), a.ptr<uint32_t*>(3));
   K("d4_mm_q8_0") return ilt_d4_mm_q8_0(stream, a.i32(0), a.i32(1), a.i32(2), a.i32(3), a.i32(4), a.i32(5), a.ptr<ci8>(6), a.ptr<cu16>(7), a.ptr<cf>(8), a.ptr<float*>(9));
   K("d4_mm_f16") return ilt_d4_mm_f16(stream, a.i32(0), a.i32(1), a.i32(2), a.i32(3), a.i32(4), a.i32(5), a.ptr<cu16>(6), a.ptr<cf>(8), a.ptr<float*>(9));

@@ -61,46 +61,65 @@ __global__ __launch_bounds__(64) void qk_rope_kernel(float* __restrict__ q, floa
 // 0 .. pos0 + t.  Scores: F32-DOT16 (tensor.lisp:370-378; 16 lanes a position, lane l the partial sum l)
 // times 1/sqrt(hd).  Softmax: exp of a single through double; the sum of the exps in double -- added in
 // parallel here and, where that order could change the single 1/sum is rounded to, once more one after
-// another as the CPU adds them; then out += score * V row, position after position, an output column a thread.
-__global__ __launch_bounds__(256) void attn_rows_kernel(const float* __restrict__ q, const float* __restrict__ kc, const float* __restrict__ vc,
-                                                        float* __restrict__ out, int nh, int nkv, int hd, int pos0, float scale) {
-  extern __shared__ float scores[];                // npos floats
-  __shared__ float redf[4];
-  __shared__ double redd[4];
+// another as the CPU adds them.  Then out += score * V row, position after position: the adds of a column are a
+// chain, so a column is one thread's; the value rows come through LDS in tiles of 64 positions that all sixteen
+// waves load (two tiles in flight), so the chain never waits for memory.
+constexpr int kAttnThreads = 1024, kAttnTile = 64;
+__global__ __launch_bounds__(kAttnThreads) void attn_rows_kernel(const float* __restrict__ q, const float* __restrict__ kc,
+                                                                 const float* __restrict__ vc, float* __restrict__ out, int nh, int nkv, int hd,
+                                                                 int pos0, float scale, int smax) {
+  extern __shared__ __align__(16) float dyn[];
+  float* scores = dyn;                             // smax floats (a multiple of 4)
+  float* vt = dyn + smax;                          // two tiles of kAttnTile x hd floats
+  __shared__ float redf[16];
+  __shared__ double redd[16];
   const int h = blockIdx.x, t = blockIdx.y, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int npos = pos0 + t + 1;
   const int group = nh / nkv, kvd = nkv * hd, ko = (h / group) * hd;
   const float* qh = q + ((long long)t * nh + h) * hd;
-  const int l = tid & 15, pg = tid >> 4;           // 16 positions at a time
+  const int l = tid & 15, pg = tid >> 4;           // 64 positions at a time
   const int nj = hd >> 4;                          // terms a partial sum (hd <= 256: at most 16)
   float qv[16];
 #pragma unroll
   for (int j = 0; j < 16; j++) qv[j] = j < nj ? qh[l + 16 * j] : 0.0f;
   float mx = -3.402823466e38f;
-  for (int p0 = 0; p0 < npos; p0 += 16) {
-    const int p = p0 + pg;
-    const float* kr = kc + (long long)min(p, npos - 1) * kvd + ko;
-    float s = 0.0f;
+  for (int p0 = 0; p0 < npos; p0 += 128) {         // two passes' loads before either is used
+    float kv[2][16];
 #pragma unroll
-    for (int j = 0; j < 16; j++) if (j < nj) s = s + kr[l + 16 * j] * qv[j];
-    s = s + ilt_dppf<ILT_DPP_SHL(4)>(s);
-    s = s + ilt_dppf<ILT_DPP_SHL(8)>(s);
-    s = s + ilt_dppf<ILT_DPP_SHL(1)>(s);
-    s = s + ilt_dppf<ILT_DPP_SHL(2)>(s);
-    if (l == 0 && p < npos) { const float sv = s * scale; scores[p] = sv; mx = fmaxf(mx, sv); }
+    for (int u = 0; u < 2; u++) {
+      const float* kr = kc + (long long)min(p0 + 64 * u + pg, npos - 1) * kvd + ko;
+#pragma unroll
+      for (int j = 0; j < 16; j++) kv[u][j] = j < nj ? kr[l + 16 * j] : 0.0f;
+    }
+#pragma unroll
+    for (int u = 0; u < 2; u++) {
+      const int p = p0 + 64 * u + pg;
+      float s = 0.0f;
+#pragma unroll
+      for (int j = 0; j < 16; j++) if (j < nj) s = s + kv[u][j] * qv[j];
+      s = s + ilt_dppf<ILT_DPP_SHL(4)>(s);
+      s = s + ilt_dppf<ILT_DPP_SHL(8)>(s);
+      s = s + ilt_dppf<ILT_DPP_SHL(1)>(s);
+      s = s + ilt_dppf<ILT_DPP_SHL(2)>(s);
+      if (l == 0 && p < npos) { const float sv = s * scale; scores[p] = sv; mx = fmaxf(mx, sv); }
+    }
   }
 #pragma unroll
   for (int off = 32; off > 0; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off));
   if (lane == 0) redf[wave] = mx;
   __syncthreads();
-  mx = fmaxf(fmaxf(redf[0], redf[1]), fmaxf(redf[2], redf[3]));
+  mx = redf[0];
+#pragma unroll
+  for (int w = 1; w < 16; w++) mx = fmaxf(mx, redf[w]);
   double part = 0.0;
-  for (int p = tid; p < npos; p += 256) { const float e = ilt_expf_via_double(scores[p] - mx); scores[p] = e; part += (double)e; }
+  for (int p = tid; p < npos; p += kAttnThreads) { const float e = ilt_expf_via_double(scores[p] - mx); scores[p] = e; part += (double)e; }
 #pragma unroll
   for (int off = 32; off > 0; off >>= 1) part += __shfl_xor(part, off);
   if (lane == 0) redd[wave] = part;
   __syncthreads();
-  double sum = (redd[0] + redd[1]) + (redd[2] + redd[3]);
+  double sum = 0.0;
+#pragma unroll
+  for (int w = 0; w < 16; w++) sum += redd[w];
   const double slack = sum * ((double)(npos + 8) * 0x1p-51);
   if ((float)(1.0 / (sum - slack)) != (float)(1.0 / (sum + slack))) {      // the same in every thread
     __syncthreads();
@@ -110,21 +129,214 @@ __global__ __launch_bounds__(256) void attn_rows_kernel(const float* __restrict_
   }
   const float inv = (float)(1.0 / sum);
   __syncthreads();
-  for (int p = tid; p < npos; p += 256) scores[p] = scores[p] * inv;
-  __syncthreads();
-  if (tid < hd) {
-    const float* vr = vc + ko + tid;
+  for (int p = tid; p < npos; p += kAttnThreads) scores[p] = scores[p] * inv;
+  // the values: tile i of 64 positions into buffer i & 1, loaded a tile ahead of the adds
+  const int ntile = (npos + kAttnTile - 1) / kAttnTile;
+  const int per = kAttnTile * hd / 4;              // float4 pieces a tile
+  auto load_tile = [&](int ti) {
+    float* dst = vt + (ti & 1) * kAttnTile * hd;
+    for (int i = tid; i < per; i += kAttnThreads) {
+      const int pp = i / (hd / 4), c4 = i - pp * (hd / 4);
+      const int p = min(ti * kAttnTile + pp, npos - 1);
+      *(float4*)(dst + pp * hd + 4 * c4) = *(const float4*)(vc + (long long)p * kvd + ko + 4 * c4);
+    }
+  };
+  load_tile(0);
+  float o = 0.0f;
+  for (int ti = 0; ti < ntile; ti++) {
+    __syncthreads();                               // tile ti is in LDS (and the scores are scaled); buffer (ti + 1) & 1 is free
+    if (ti + 1 < ntile) load_tile(ti + 1);
+    if (tid < hd) {
+      const float* col = vt + (ti & 1) * kAttnTile * hd + tid;
+      const int np = min(kAttnTile, npos - ti * kAttnTile);
+      const float* sc = scores + ti * kAttnTile;
+      int pp = 0;
+      for (; pp + 8 <= np; pp += 8) {
+        float pr[8];
+#pragma unroll
+        for (int u = 0; u < 8; u++) pr[u] = sc[pp + u] * col[(pp + u) * hd];
+#pragma unroll
+        for (int u = 0; u < 8; u++) o = o + pr[u];
+      }
+      for (; pp < np; pp++) o = o + sc[pp] * col[pp * hd];
+    }
+  }
+  if (tid < hd) out[((long long)t * nh + h) * hd + tid] = o;
+}
+
+// The same attention as two launches, for contexts whose scores and value slice fit LDS (2048 positions): the
+// scores of all positions at once over many workgroups (nothing in them depends on anything else), then the
+// softmax and the ordered sums, a workgroup taking a query head's 16-column slice of the values for a group of
+// TG tokens: the whole slice is asked for at once (one trip to memory), and 16 threads a token then run the
+// chains from LDS.  A group's tokens share the keys (registers) and the value slice (LDS), so a prompt's chunk
+// reads them once for 16 tokens.  The numbers are attn_rows_kernel's: the same operations in the same order.
+// raw[(t*nh + h)*spitch + p] = F32-DOT16(K[p], q) * scale
+template <int TG>
+__global__ __launch_bounds__(1024) void attn_scores_kernel(const float* __restrict__ q, const float* __restrict__ kc, float* __restrict__ raw,
+                                                           int nh, int nkv, int hd, int pos0, int ntok, float scale, int spitch) {
+  __shared__ float qs[TG > 1 ? TG * 256 : 1];
+  const int h = blockIdx.x, t0 = blockIdx.z * TG, tid = threadIdx.x;
+  const int tn = min(TG, ntok - t0), nposmax = pos0 + t0 + tn, pbase = blockIdx.y * 256;
+  if (pbase >= nposmax) return;                    // the same in every thread
+  const int group = nh / nkv, kvd = nkv * hd, ko = (h / group) * hd;
+  const int l = tid & 15, pg = tid >> 4, nj = hd >> 4;
+  float kv[4][16];
+#pragma unroll
+  for (int u = 0; u < 4; u++) {
+    const float* kr = kc + (long long)min(pbase + 64 * u + pg, nposmax - 1) * kvd + ko;
+#pragma unroll
+    for (int j = 0; j < 16; j++) kv[u][j] = j < nj ? kr[l + 16 * j] : 0.0f;
+  }
+  if (TG > 1) {
+    for (int i = tid; i < tn * hd; i += 1024) { const int tt = i / hd, c = i - tt * hd; qs[tt * 256 + c] = q[((long long)(t0 + tt) * nh + h) * hd + c]; }
+    __syncthreads();
+  }
+  for (int tt = 0; tt < tn; tt++) {
+    const int npos = pos0 + t0 + tt + 1;
+    if (pbase >= npos) continue;
+    const float* qh = q + ((long long)(t0 + tt) * nh + h) * hd;
+    float qv[16];
+#pragma unroll
+    for (int j = 0; j < 16; j++) qv[j] = j < nj ? (TG > 1 ? qs[tt * 256 + l + 16 * j] : qh[l + 16 * j]) : 0.0f;
+#pragma unroll
+    for (int u = 0; u < 4; u++) {
+      const int p = pbase + 64 * u + pg;
+      float sacc = 0.0f;
+#pragma unroll
+      for (int j = 0; j < 16; j++) if (j < nj) sacc = sacc + kv[u][j] * qv[j];
+      sacc = sacc + ilt_dppf<ILT_DPP_SHL(4)>(sacc);
+      sacc = sacc + ilt_dppf<ILT_DPP_SHL(8)>(sacc);
+      sacc = sacc + ilt_dppf<ILT_DPP_SHL(1)>(sacc);
+      sacc = sacc + ilt_dppf<ILT_DPP_SHL(2)>(sacc);
+      if (l == 0 && p < npos) raw[((long long)(t0 + tt) * nh + h) * spitch + p] = sacc * scale;
+    }
+  }
+}
+
+// softmax of one token's raw scores into sc (LDS) by the NT threads that call it (me = 0..NT-1): NT = 64, one
+// wave, or the whole workgroup of 256 with red/redd for the waves to meet.  PRE: the thread's raw scores
+// (positions me, me + NT, ..) are in pre already, at most eight of them.
+template <int NT, bool PRE>
+__device__ __forceinline__ void attn_softmax(const float* __restrict__ rw, const float* pre, float* sc, int npos, int me, float* redf, double* redd) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  float mx = -3.402823466e38f;
+  if (PRE) {
+#pragma unroll
+    for (int u = 0; u < 8; u++) if (me + NT * u < npos) { sc[me + NT * u] = pre[u]; mx = fmaxf(mx, pre[u]); }
+  } else {
+    for (int p = me; p < npos; p += NT) { const float sv = rw[p]; sc[p] = sv; mx = fmaxf(mx, sv); }
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off));
+  if (NT > 64) {
+    if (lane == 0) redf[wave] = mx;
+    __syncthreads();
+    mx = fmaxf(fmaxf(redf[0], redf[1]), fmaxf(redf[2], redf[3]));
+  }
+  double part = 0.0;
+  for (int p = me; p < npos; p += NT) { const float e = ilt_expf_via_double(sc[p] - mx); sc[p] = e; part += (double)e; }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) part += __shfl_xor(part, off);
+  double sum = part;
+  if (NT > 64) {
+    if (lane == 0) redd[wave] = part;
+    __syncthreads();
+    sum = (redd[0] + redd[1]) + (redd[2] + redd[3]);
+  }
+  // the CPU adds the terms one after another: take its sum where the order could show in the rounded reciprocal
+  const double slack = sum * ((double)(npos + 8) * 0x1p-51);
+  if ((float)(1.0 / (sum - slack)) != (float)(1.0 / (sum + slack))) {      // the same in all NT threads
+    if (NT > 64) __syncthreads();
+    if (me == 0) { double s2 = 0.0; for (int p = 0; p < npos; p++) s2 += (double)sc[p]; redd[NT > 64 ? 0 : 4 + wave] = s2; }
+    if (NT > 64) __syncthreads();
+    sum = redd[NT > 64 ? 0 : 4 + wave];
+  }
+  const float inv = (float)(1.0 / sum);
+  for (int p = me; p < npos; p += NT) sc[p] = sc[p] * inv;
+}
+
+// grid x = head * (hd/16) + column slice; grid y = token group.  LDS: TG rows of spitch scores, then the value
+// slice with the positions along a row, vt[c * vpitch + p] (vpitch = 4 mod 64: sixteen threads' 16-byte reads
+// of sixteen rows fall on different banks).  NB: the slice is at most NB * 2048 16-byte pieces (512 NB positions).
+// With one token a workgroup the slice is stored times that token's scores, by all threads, and the chains add.
+template <int TG, int NB>
+__global__ __launch_bounds__(256) void attn_values_kernel(const float* __restrict__ raw, const float* __restrict__ vc, float* __restrict__ out,
+                                                          int nh, int nkv, int hd, int pos0, int ntok, int spitch, int vpitch) {
+  extern __shared__ __align__(16) float dyn[];
+  __shared__ float redf[4];
+  __shared__ double redd[8];
+  const int ns = hd >> 4, h = blockIdx.x / ns, cs = blockIdx.x - h * ns, t0 = blockIdx.y * TG, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tn = min(TG, ntok - t0), nposmax = pos0 + t0 + tn;
+  const int group = nh / nkv, kvd = nkv * hd, ko = (h / group) * hd + 16 * cs;
+  float* scores = dyn;
+  float* vt = dyn + TG * spitch;
+  // every load is asked for before anything waits, the scores first: no branch around a load, so that the
+  // softmax waits for the scores alone and the value slice arrives meanwhile
+  float pre[8];
+  if (TG == 1) {
+    const float* rw = raw + ((long long)t0 * nh + h) * spitch;
+#pragma unroll
+    for (int u = 0; u < 2 * NB; u++) pre[u] = rw[min(tid + 256 * u, nposmax - 1)];
+  }
+  float4 r[8 * NB];
+  const int total = nposmax * 4;                   // 16-byte pieces
+#pragma unroll
+  for (int u = 0; u < 8 * NB; u++) {
+    const int i = min(tid + 256 * u, total - 1);
+    r[u] = *(const float4*)(vc + (long long)(i >> 2) * kvd + ko + 4 * (i & 3));
+  }
+  if (TG == 1) {
+#pragma unroll
+    for (int u = 2 * NB; u < 8; u++) pre[u] = 0.0f;
+    attn_softmax<256, true>(nullptr, pre, scores, nposmax, tid, redf, redd);
+    __syncthreads();                               // every thread's scaled scores, for the products below
+  } else {
+    for (int tt = wave; tt < tn; tt += 4)
+      attn_softmax<64, false>(raw + ((long long)(t0 + tt) * nh + h) * spitch, nullptr, scores + tt * spitch, pos0 + t0 + tt + 1, lane, redf, redd);
+  }
+#pragma unroll
+  for (int u = 0; u < 8 * NB; u++) {
+    const int i = tid + 256 * u;
+    if (i < total) {
+      float* dst = vt + (4 * (i & 3)) * vpitch + (i >> 2);
+      if (TG == 1) {
+        const float sp = scores[i >> 2];
+        dst[0] = sp * r[u].x; dst[vpitch] = sp * r[u].y; dst[2 * vpitch] = sp * r[u].z; dst[3 * vpitch] = sp * r[u].w;
+      } else {
+        dst[0] = r[u].x; dst[vpitch] = r[u].y; dst[2 * vpitch] = r[u].z; dst[3 * vpitch] = r[u].w;
+      }
+    }
+  }
+  __syncthreads();                                 // the scores are scaled, the slice is in place
+  if (tid < tn * 16) {
+    const int tt = tid >> 4, c = tid & 15, npos = pos0 + t0 + tt + 1;
+    const float* sc = scores + tt * spitch;
+    const float* col = vt + c * vpitch;
     float o = 0.0f;
     int p = 0;
-    for (; p + 8 <= npos; p += 8) {
-      float vv[8];
+    if (TG == 1) {
+      for (; p + 32 <= npos; p += 32) {
+        float4 v4[8];
 #pragma unroll
-      for (int u = 0; u < 8; u++) vv[u] = vr[(long long)(p + u) * kvd];
+        for (int u = 0; u < 8; u++) v4[u] = *(const float4*)(col + p + 4 * u);
 #pragma unroll
-      for (int u = 0; u < 8; u++) o = o + scores[p + u] * vv[u];
+        for (int u = 0; u < 8; u++) { o = o + v4[u].x; o = o + v4[u].y; o = o + v4[u].z; o = o + v4[u].w; }
+      }
+      for (; p < npos; p++) o = o + col[p];
+    } else {
+      for (; p + 16 <= npos; p += 16) {
+        float4 s4[4], v4[4];
+#pragma unroll
+        for (int u = 0; u < 4; u++) { s4[u] = *(const float4*)(sc + p + 4 * u); v4[u] = *(const float4*)(col + p + 4 * u); }
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+          const float a0 = s4[u].x * v4[u].x, a1 = s4[u].y * v4[u].y, a2 = s4[u].z * v4[u].z, a3 = s4[u].w * v4[u].w;
+          o = o + a0; o = o + a1; o = o + a2; o = o + a3;
+        }
+      }
+      for (; p < npos; p++) o = o + sc[p] * col[p];
     }
-    for (; p < npos; p++) o = o + scores[p] * vr[(long long)p * kvd];
-    out[((long long)t * nh + h) * hd + tid] = o;
+    out[((long long)(t0 + tt) * nh + h) * hd + 16 * cs + c] = o;
   }
 }
 
@@ -144,12 +356,51 @@ hipError_t ilt_k_qk_rope(float* q, float* k, const float* v, const float* qn, co
   return hipGetLastError();
 }
 
+// scratch: ntok * nh * ((pos0 + ntok + 3) & ~3) floats for the two-launch variant (contexts up to 2048 positions),
+// or null: one launch
 hipError_t ilt_k_attn_rows(const float* q, const float* kc, const float* vc, float* out, int nh, int nkv, int hd, int pos0, int ntok,
-                           hipStream_t st) {
+                           float* scratch, hipStream_t st) {
   if (ntok <= 0) return hipSuccess;
-  if (hd % 16 || hd > 256 || nh % nkv || pos0 < 0 || pos0 + ntok > 15000) return hipErrorInvalidValue;      // the scores of a query sit in LDS
+  if (hd % 16 || hd > 256 || nh % nkv || pos0 < 0) return hipErrorInvalidValue;
+  const int smax = (pos0 + ntok + 3) & ~3;
   const float scale = 1.0f / sqrtf((float)hd);
-  hipLaunchKernelGGL(attn_rows_kernel, dim3(nh, ntok), dim3(256), sizeof(float) * (size_t)(pos0 + ntok), st, q, kc, vc, out, nh, nkv, hd, pos0, scale);
+  static bool attr_set[64] = {};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) dev = 0;
+  if (scratch && pos0 + ntok <= 2048) {
+    const int ctx = pos0 + ntok, vpitch = ((ctx + 63) & ~63) + 4;
+    // tokens a workgroup: as many as leave their scores and the value slice room in LDS (150 KB)
+    auto bytes = [&](int tg) { return sizeof(float) * ((size_t)tg * smax + 16 * (size_t)vpitch); };
+    const int tg = ntok == 1 ? 1 : bytes(16) <= 150 * 1024 ? 16 : bytes(4) <= 150 * 1024 ? 4 : 1;
+    const int nb = (ctx + 511) / 512;
+    const dim3 gs(nh, (ctx + 255) / 256, (ntok + tg - 1) / tg), gv(nh * (hd / 16), (ntok + tg - 1) / tg);
+    hipError_t e = hipErrorInvalidValue;
+#define ILT_ATTN(TG, NB)                                                                                                                       \
+  if (tg == TG && nb == NB) {                                                                                                                  \
+    static bool set[64] = {};                                                                                                                  \
+    e = set[dev] ? hipSuccess                                                                                                                  \
+                 : hipFuncSetAttribute((const void*)attn_values_kernel<TG, NB>, hipFuncAttributeMaxDynamicSharedMemorySize, 152 * 1024);       \
+    if (e == hipSuccess) {                                                                                                                     \
+      set[dev] = true;                                                                                                                         \
+      hipLaunchKernelGGL(attn_scores_kernel<TG>, gs, dim3(1024), 0, st, q, kc, scratch, nh, nkv, hd, pos0, ntok, scale, smax);                 \
+      hipLaunchKernelGGL((attn_values_kernel<TG, NB>), gv, dim3(256), bytes(TG), st, scratch, vc, out, nh, nkv, hd, pos0, ntok, smax, vpitch); \
+      e = hipGetLastError();                                                                                                                   \
+    }                                                                                                                                          \
+  }
+    ILT_ATTN(1, 1) ILT_ATTN(1, 2) ILT_ATTN(1, 3) ILT_ATTN(1, 4)
+    ILT_ATTN(4, 3) ILT_ATTN(4, 4)
+    ILT_ATTN(16, 1) ILT_ATTN(16, 2) ILT_ATTN(16, 3)
+#undef ILT_ATTN
+    return e;
+  }
+  if (!attr_set[dev]) {
+    const hipError_t e = hipFuncSetAttribute((const void*)attn_rows_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 152 * 1024);
+    if (e != hipSuccess) return e;
+    attr_set[dev] = true;
+  }
+  const size_t smem = sizeof(float) * ((size_t)smax + 2 * (size_t)kAttnTile * hd);
+  if (smem > 150 * 1024) return hipErrorInvalidValue;      // a query's scores sit in LDS: about 20,000 positions at hd 128
+  hipLaunchKernelGGL(attn_rows_kernel, dim3(nh, ntok), dim3(kAttnThreads), smem, st, q, kc, vc, out, nh, nkv, hd, pos0, scale, smax);
   return hipGetLastError();
 }
 

@@ -67,6 +67,7 @@ class DenseModel:
         self.x, self.q, self.k, self.v = A(4 * n * d), A(4 * n * self.qd), A(4 * n * self.kvd), A(4 * n * self.kvd)
         self.att, self.fa, self.fb = A(4 * n * self.qd), A(4 * n * ffn), A(4 * n * ffn)
         self.tokens = A(4 * n)
+        self.scores = A(4 * n * c["nh"] * ((nctx + 3) // 4 * 4)) if nctx <= 2048 else None      # the attention's raw scores
         self.logits = A(4 * c["vocab"])
         self.acts = {cols: dense.QAct(dev, n, cols, ("q8k",)) for cols in {d, self.qd, ffn}}
 
@@ -91,7 +92,7 @@ class DenseModel:
                      C.c_int(nh), C.c_int(nkv), C.c_int(hd), C.c_int(hd), C.c_int(self.pos), C.c_float(eps), C.c_int(1 if c["neox"] else 0),
                      C.c_int(n))
             hip.call("ilt_attn_rows", S, P(self.q), P(L["kc"]), P(L["vc"]), P(self.att), C.c_int(nh), C.c_int(nkv), C.c_int(hd),
-                     C.c_int(self.pos), C.c_int(n))
+                     C.c_int(self.pos), C.c_int(n), P(self.scores))
             if n == 1:
                 dense.mv_multi(dev, [(L["wo"], self.x, None)], xf=self.att, acc=True)
                 dense.glu_mul(dev, L["gate"], L["up"], None, self.fa, xf=self.x, norm=(L["ffn_norm"], eps))
@@ -127,7 +128,7 @@ class DenseModel:
         if self.output is not self.embd:
             self.output.free()
         self.embd.free()
-        for b in (self.output_norm, self.rope, self.x, self.q, self.k, self.v, self.att, self.fa, self.fb, self.tokens, self.logits):
+        for b in (self.output_norm, self.rope, self.x, self.q, self.k, self.v, self.att, self.fa, self.fb, self.tokens, self.logits, self.scores):
             hip.hip_free(b)
         for a in self.acts.values():
             a.free()

@@ -295,13 +295,16 @@ int ilt_d4_moe_sum_rows(uint64_t stream, int d, int nu, int ntok, const float* d
    attn_rows: attend-head! for every query head of ntok tokens, token t over positions 0 .. pos0 + t; scores
      in F32-DOT16's order, the softmax's sum in double, the values added position after position.  It stands
      where the reference launches attn_decode + attn_merge / attn_prefill (dense.cu:376-727), whose partial
-     sums meet in another order.
+     sums meet in another order.  scratch: ntok * nh * ((pos0 + ntok + 3) & ~3) floats of the caller's for the raw
+     scores (two launches, for contexts up to 2048 positions: the scores over many workgroups, then a 16-column
+     slice of the values a workgroup), or null (one launch, a workgroup a head, any context that fits LDS).
    swiglu (dense.cu:307): swiglu! on n values, a = (a / (1 + e^-a)) * b, the exponential through double. */
 /* The table qk_rope takes, for positions pos0 .. pos0 + n - 1, written to host memory (n * head_dim floats). */
 int ilt_rope_table(int head_dim, int pos0, int n, float base, float* out);
 int ilt_qk_rope(uint64_t stream, float* q, float* k, const float* v, const float* qn, const float* kn, const float* rope, float* kc,
                 float* vc, int nh, int nkv, int hd, int rd, int pos0, float eps, int neox, int ntok);
-int ilt_attn_rows(uint64_t stream, const float* q, const float* kc, const float* vc, float* out, int nh, int nkv, int hd, int pos0, int ntok);
+int ilt_attn_rows(uint64_t stream, const float* q, const float* kc, const float* vc, float* out, int nh, int nkv, int hd, int pos0, int ntok,
+                  float* scratch);
 int ilt_swiglu(uint64_t stream, float* a, const float* b, int64_t n);
 
 /* Prefill products on the int8 matrix cores, y[t*rows + r] = W[r].x_t (+ bias[r]) for n

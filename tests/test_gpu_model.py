@@ -67,6 +67,17 @@ def test_small_decoder_prefill_chunks_and_decode(dev):
     run_greedy(dev, host, nprompt=9, ndecode=2, chunk=64, nctx=16, seed=3)
 
 
+def test_small_decoder_long_contexts(dev):
+    """Contexts past one workgroup's 256 positions of scores: the two-launch attention with 16 tokens, 4 tokens and one
+    token a workgroup as the context grows towards 2048 positions, and past that the single launch with its value tiles."""
+    from illatio_amd import model
+    host = model.synth_model(6, d=256, ffn=512, nh=4, nkv=2, hd=64, nl=2, vocab=500)
+    same, _ = run_greedy(dev, host, nprompt=2030, ndecode=6, chunk=512, nctx=2040, seed=6)
+    assert same == 6
+    same, _ = run_greedy(dev, host, nprompt=2060, ndecode=4, chunk=512, nctx=2100, seed=7)
+    assert same == 4
+
+
 def test_config_2_width_four_layers_128_greedy_tokens(dev):
     """Config 2's layer at its full width (hidden 2560, intermediate 9728, 32 query and 8 KV heads of 128, vocabulary
     151936), four layers: a 64-token prompt through the prefill products, then 128 greedy tokens, each step's logits
