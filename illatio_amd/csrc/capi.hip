@@ -752,6 +752,13 @@ int ilt_qk_rope(uint64_t stream, float* q, float* k, const float* v, const float
   ILT_REQUIRE(ntok >= 0 && (ntok == 0 || (q && k && v && rope && kc && vc)) && pos0 >= 0);
   return (int)ilt_k_qk_rope(q, k, v, qn, kn, rope, kc, vc, nh, nkv, hd, rd, pos0, eps, neox, ntok, S(stream));
 }
+// ilt_qk_rope and ilt_attn_rows for one token at position pos, as two launches instead of three (the first one
+// norms and turns the heads where it needs them and writes the caches' rows); q and k are left as they came
+int ilt_attn_step(uint64_t stream, const float* q, const float* k, const float* v, const float* qn, const float* kn, const float* rope, float* kc,
+                  float* vc, float* out, int nh, int nkv, int hd, int rd, int pos, float eps, int neox, float* scratch) {
+  ILT_REQUIRE(q && k && v && rope && kc && vc && out && scratch && nh > 0 && nkv > 0 && pos >= 0 && pos < 2048);
+  return (int)ilt_k_attn_step(q, k, v, qn, kn, rope, kc, vc, out, nh, nkv, hd, rd, pos, eps, neox, scratch, S(stream));
+}
 // rope-table (model.lisp:218-231) for positions pos0 .. pos0 + n - 1, on the host: a position's head_dim/2 cosines
 // then head_dim/2 sines, theta advanced by repeated single-float multiplication, theta-scale, cos and sin through
 // double and rounded to single as SBCL evaluates them.  The only float arithmetic this file does: model constants,
@@ -839,6 +846,9 @@ int ilt_launch(const char* kernel, unsigned gx, unsigned gy, unsigned gz, unsign
                                   a.ptr<float*>(7), a.i32(8), a.i32(9), a.i32(10), a.i32(11), a.i32(12), a.f32(13), a.i32(14), (int)gy);
   K("swiglu") return ilt_swiglu(stream, a.ptr<float*>(0), a.ptr<cf>(1), a.i64(2));
   K("attn_rows") return ilt_attn_rows(stream, a.ptr<cf>(0), a.ptr<cf>(1), a.ptr<cf>(2), a.ptr<float*>(3), a.i32(4), a.i32(5), a.i32(6), a.i32(7), (int)gy, a.ptr<float*>(8));
+  K("attn_step") return ilt_attn_step(stream, a.ptr<cf>(0), a.ptr<cf>(1), a.ptr<cf>(2), a.ptr<cf>(3), a.ptr<cf>(4), a.ptr<cf>(5), a.ptr<float*>(6),
+                                      a.ptr<float*>(7), a.ptr<float*>(8), a.i32(9), a.i32(10), a.i32(11), a.i32(12), a.i32(13), a.f32(14), a.i32(15),
+                                      a.ptr<float*>(16));
   K("d4_rows_expert") return ilt_d4_rows_expert(stream, a.i32(0), a.ptr<cu32>(1), a.ptr<cu32>(2), a.ptr<uint32_t*>(3));
   K("d4_mm_q8_0") return ilt_d4_mm_q8_0(stream, a.i32(0), a.i32(1), a.i32(2), a.i32(3), a.i32(4), a.i32(5), a.ptr<ci8>(6), a.ptr<cu16>(7), a.ptr<cf>(8), a.ptr<float*>(9));
   K("d4_mm_f16") return ilt_d4_mm_f16(stream, a.i32(0), a.i32(1), a.i32(2), a.i32(3), a.i32(4), a.i32(5), a.ptr<cu16>(6), a.ptr<cf>(8), a.ptr<float*>(9));

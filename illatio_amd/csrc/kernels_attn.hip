@@ -10,42 +10,55 @@
 
 namespace {
 
-// qk_rope: a workgroup (one wave) a head of a token.  rmsnorm! of the head when its weights are given
-// (model.lisp:205-216: the squares, rounded to floats, added in double one after another), rope-head!
-// from the position's table (cos, then sin, rd/2 each), K and V into the caches at pos0 + t.
+// What one lane of a wave stored in LDS, for the other lanes of that wave: the hardware keeps a wave's LDS
+// accesses in program order; this keeps the compiler from moving them across.
+__device__ __forceinline__ void wave_lds_sync() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+// One head by one wave: x (hd floats) into xs (LDS): rmsnorm! of the head when its weights are given
+// (model.lisp:205-216: the squares, rounded to floats, added in double one after another), then rope-head!
+// from the position's table cs (cos, then sin, rd/2 each).  Only this wave touches xs and sc.
+__device__ __forceinline__ void rope_head_wave(const float* __restrict__ x, const float* __restrict__ nw, const float* __restrict__ cs,
+                                               float* xs, float* sc, int hd, int rd, float eps, int neox, int i) {
+  const int half = rd >> 1;
+  for (int j = i; j < hd; j += 64) xs[j] = x[j];
+  wave_lds_sync();
+  if (nw) {
+    if (i == 0) {
+      double s = 0.0;
+      for (int j = 0; j < hd; j++) { const float sq = xs[j] * xs[j]; s += (double)sq; }
+      *sc = 1.0f / sqrtf((float)(s / (double)hd + (double)eps));
+    }
+    wave_lds_sync();
+    const float scale = *sc;
+    for (int j = i; j < hd; j += 64) xs[j] = (xs[j] * scale) * nw[j];
+    wave_lds_sync();
+  }
+  for (int p = i; p < half; p += 64) {
+    const int a = neox ? p : 2 * p, b = neox ? p + half : 2 * p + 1;
+    const float x0 = xs[a], x1 = xs[b], c = cs[p], sn = cs[half + p];
+    xs[a] = x0 * c - x1 * sn;                      // (no contraction: each product rounds on its own)
+    xs[b] = x0 * sn + x1 * c;
+  }
+  wave_lds_sync();
+}
+
+// qk_rope: a workgroup (one wave) a head of a token; K and V into the caches at pos0 + t.
 __global__ __launch_bounds__(64) void qk_rope_kernel(float* __restrict__ q, float* __restrict__ k, const float* __restrict__ v,
                                                      const float* __restrict__ qn, const float* __restrict__ kn,
                                                      const float* __restrict__ rope, float* __restrict__ kc, float* __restrict__ vc,
                                                      int nh, int nkv, int hd, int rd, int pos0, float eps, int neox) {
   __shared__ float xs[512];
   __shared__ float sc;
-  const int head = blockIdx.x, t = blockIdx.y, i = threadIdx.x, half = rd >> 1;
+  const int head = blockIdx.x, t = blockIdx.y, i = threadIdx.x;
   const int pos = pos0 + t;
   const int qd = nh * hd, kvd = nkv * hd;
   const bool isq = head < nh;
   float* x = isq ? q + (long long)t * qd + head * hd : k + (long long)t * kvd + (head - nh) * hd;
-  const float* nw = isq ? qn : kn;
-  for (int j = i; j < hd; j += 64) xs[j] = x[j];
-  __syncthreads();
-  if (nw) {
-    if (i == 0) {
-      double s = 0.0;
-      for (int j = 0; j < hd; j++) { const float sq = xs[j] * xs[j]; s += (double)sq; }
-      sc = 1.0f / sqrtf((float)(s / (double)hd + (double)eps));
-    }
-    __syncthreads();
-    const float scale = sc;
-    for (int j = i; j < hd; j += 64) xs[j] = (xs[j] * scale) * nw[j];
-    __syncthreads();
-  }
-  const float* cs = rope + (long long)pos * rd;
-  for (int p = i; p < half; p += 64) {
-    const int a = neox ? p : 2 * p, b = neox ? p + half : 2 * p + 1;
-    const float x0 = xs[a], x1 = xs[b], c = cs[p], s = cs[half + p];
-    xs[a] = x0 * c - x1 * s;                       // (no contraction: each product rounds on its own)
-    xs[b] = x0 * s + x1 * c;
-  }
-  __syncthreads();
+  rope_head_wave(x, isq ? qn : kn, rope + (long long)pos * rd, xs, &sc, hd, rd, eps, neox, i);
   for (int j = i; j < hd; j += 64) x[j] = xs[j];
   if (!isq) {
     const int kh = head - nh;
@@ -210,6 +223,59 @@ __global__ __launch_bounds__(1024) void attn_scores_kernel(const float* __restri
       sacc = sacc + ilt_dppf<ILT_DPP_SHL(2)>(sacc);
       if (l == 0 && p < npos) raw[((long long)(t0 + tt) * nh + h) * spitch + p] = sacc * scale;
     }
+  }
+}
+
+// One token's qk_rope and scores in one launch: every workgroup of a query head norms and turns that head
+// itself (wave 0; a sixteenth of a microsecond of arithmetic against a launch), the workgroup whose 256
+// positions hold the token's own does the same for its KV head's key (wave 1) and takes that key from LDS,
+// and the group's first query head there writes the key and the value into the caches, for the launch with
+// the values.  q and k are left as they came.
+__global__ __launch_bounds__(1024) void attn_step_scores_kernel(const float* __restrict__ q, const float* __restrict__ k, const float* __restrict__ v,
+                                                                const float* __restrict__ qn, const float* __restrict__ kn,
+                                                                const float* __restrict__ rope, float* __restrict__ kc, float* __restrict__ vc,
+                                                                float* __restrict__ raw, int nh, int nkv, int hd, int rd, int pos, float eps,
+                                                                int neox, float scale, int spitch) {
+  __shared__ float qsh[256], ksh[256];
+  __shared__ float scs[2];
+  const int h = blockIdx.x, tid = threadIdx.x, npos = pos + 1, pbase = blockIdx.y * 256;
+  if (pbase >= npos) return;
+  const int group = nh / nkv, kvd = nkv * hd, kh = h / group, ko = kh * hd;
+  const int l = tid & 15, pg = tid >> 4, nj = hd >> 4, wave = tid >> 6;
+  const bool own = pos < pbase + 256;              // this workgroup's positions hold the token's own
+  float kv[4][16];
+#pragma unroll
+  for (int u = 0; u < 4; u++) {
+    const float* kr = kc + (long long)min(pbase + 64 * u + pg, max(pos - 1, 0)) * kvd + ko;      // rows before the token's own
+#pragma unroll
+    for (int j = 0; j < 16; j++) kv[u][j] = j < nj ? kr[l + 16 * j] : 0.0f;
+  }
+  const float* cs = rope + (long long)pos * rd;
+  if (wave == 0) rope_head_wave(q + h * hd, qn, cs, qsh, &scs[0], hd, rd, eps, neox, tid & 63);
+  if (wave == 1 && own) rope_head_wave(k + ko, kn, cs, ksh, &scs[1], hd, rd, eps, neox, tid & 63);
+  __syncthreads();
+  if (own && h == kh * group && tid < hd) {
+    kc[(long long)pos * kvd + ko + tid] = ksh[tid];
+    vc[(long long)pos * kvd + ko + tid] = v[ko + tid];
+  }
+  float qv[16];
+#pragma unroll
+  for (int j = 0; j < 16; j++) qv[j] = j < nj ? qsh[l + 16 * j] : 0.0f;
+#pragma unroll
+  for (int u = 0; u < 4; u++) {
+    const int p = pbase + 64 * u + pg;
+    if (p == pos) {
+#pragma unroll
+      for (int j = 0; j < 16; j++) kv[u][j] = j < nj ? ksh[l + 16 * j] : 0.0f;
+    }
+    float sacc = 0.0f;
+#pragma unroll
+    for (int j = 0; j < 16; j++) if (j < nj) sacc = sacc + kv[u][j] * qv[j];
+    sacc = sacc + ilt_dppf<ILT_DPP_SHL(4)>(sacc);
+    sacc = sacc + ilt_dppf<ILT_DPP_SHL(8)>(sacc);
+    sacc = sacc + ilt_dppf<ILT_DPP_SHL(1)>(sacc);
+    sacc = sacc + ilt_dppf<ILT_DPP_SHL(2)>(sacc);
+    if (l == 0 && p < npos) raw[(long long)h * spitch + p] = sacc * scale;
   }
 }
 
@@ -402,6 +468,35 @@ hipError_t ilt_k_attn_rows(const float* q, const float* kc, const float* vc, flo
   if (smem > 150 * 1024) return hipErrorInvalidValue;      // a query's scores sit in LDS: about 20,000 positions at hd 128
   hipLaunchKernelGGL(attn_rows_kernel, dim3(nh, ntok), dim3(kAttnThreads), smem, st, q, kc, vc, out, nh, nkv, hd, pos0, scale, smax);
   return hipGetLastError();
+}
+
+// One token at position pos: qk_rope and attention in two launches instead of three
+hipError_t ilt_k_attn_step(const float* q, const float* k, const float* v, const float* qn, const float* kn, const float* rope, float* kc,
+                           float* vc, float* out, int nh, int nkv, int hd, int rd, int pos, float eps, int neox, float* scratch, hipStream_t st) {
+  if (hd % 16 || hd > 256 || rd > hd || (rd & 1) || nh % nkv || pos < 0 || pos >= 2048 || !scratch) return hipErrorInvalidValue;
+  const int ctx = pos + 1, smax = (ctx + 3) & ~3, vpitch = ((ctx + 63) & ~63) + 4, nb = (ctx + 511) / 512;
+  const float scale = 1.0f / sqrtf((float)hd);
+  const size_t smem = sizeof(float) * ((size_t)smax + 16 * (size_t)vpitch);
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) dev = 0;
+  hipLaunchKernelGGL(attn_step_scores_kernel, dim3(nh, (ctx + 255) / 256), dim3(1024), 0, st, q, k, v, qn, kn, rope, kc, vc, scratch, nh, nkv, hd, rd,
+                     pos, eps, neox, scale, smax);
+  hipError_t e = hipErrorInvalidValue;
+#define ILT_ATTN1(NB)                                                                                                                         \
+  if (nb == NB) {                                                                                                                             \
+    static bool set[64] = {};                                                                                                                 \
+    e = set[dev] ? hipSuccess                                                                                                                 \
+                 : hipFuncSetAttribute((const void*)attn_values_kernel<1, NB>, hipFuncAttributeMaxDynamicSharedMemorySize, 152 * 1024);       \
+    if (e == hipSuccess) {                                                                                                                    \
+      set[dev] = true;                                                                                                                        \
+      hipLaunchKernelGGL((attn_values_kernel<1, NB>), dim3(nh * (hd / 16), 1), dim3(256), smem, st, scratch, vc, out, nh, nkv, hd, pos, 1,    \
+                         smax, vpitch);                                                                                                       \
+      e = hipGetLastError();                                                                                                                  \
+    }                                                                                                                                         \
+  }
+  ILT_ATTN1(1) ILT_ATTN1(2) ILT_ATTN1(3) ILT_ATTN1(4)
+#undef ILT_ATTN1
+  return e;
 }
 
 hipError_t ilt_k_swiglu_rows(float* a, const float* b, long long n, hipStream_t st) {

@@ -88,11 +88,16 @@ class DenseModel:
                 a = dense.rmsnorm_q8(dev, self.x, L["attn_norm"], self.acts[d], d, eps, n=n)
                 for w, y in ((L["wq"], self.q), (L["wk"], self.k), (L["wv"], self.v)):
                     dense.cmat_mul(dev, w, a, y, n=n)
-            hip.call("ilt_qk_rope", S, P(self.q), P(self.k), P(self.v), P(L["q_norm"]), P(L["k_norm"]), P(self.rope), P(L["kc"]), P(L["vc"]),
-                     C.c_int(nh), C.c_int(nkv), C.c_int(hd), C.c_int(hd), C.c_int(self.pos), C.c_float(eps), C.c_int(1 if c["neox"] else 0),
-                     C.c_int(n))
-            hip.call("ilt_attn_rows", S, P(self.q), P(L["kc"]), P(L["vc"]), P(self.att), C.c_int(nh), C.c_int(nkv), C.c_int(hd),
-                     C.c_int(self.pos), C.c_int(n), P(self.scores))
+            if n == 1 and self.scores is not None:
+                hip.call("ilt_attn_step", S, P(self.q), P(self.k), P(self.v), P(L["q_norm"]), P(L["k_norm"]), P(self.rope), P(L["kc"]), P(L["vc"]),
+                         P(self.att), C.c_int(nh), C.c_int(nkv), C.c_int(hd), C.c_int(hd), C.c_int(self.pos), C.c_float(eps),
+                         C.c_int(1 if c["neox"] else 0), P(self.scores))
+            else:
+                hip.call("ilt_qk_rope", S, P(self.q), P(self.k), P(self.v), P(L["q_norm"]), P(L["k_norm"]), P(self.rope), P(L["kc"]), P(L["vc"]),
+                         C.c_int(nh), C.c_int(nkv), C.c_int(hd), C.c_int(hd), C.c_int(self.pos), C.c_float(eps), C.c_int(1 if c["neox"] else 0),
+                         C.c_int(n))
+                hip.call("ilt_attn_rows", S, P(self.q), P(L["kc"]), P(L["vc"]), P(self.att), C.c_int(nh), C.c_int(nkv), C.c_int(hd),
+                         C.c_int(self.pos), C.c_int(n), P(self.scores))
             if n == 1:
                 dense.mv_multi(dev, [(L["wo"], self.x, None)], xf=self.att, acc=True)
                 dense.glu_mul(dev, L["gate"], L["up"], None, self.fa, xf=self.x, norm=(L["ffn_norm"], eps))

@@ -67,6 +67,46 @@ def test_small_decoder_prefill_chunks_and_decode(dev):
     run_greedy(dev, host, nprompt=9, ndecode=2, chunk=64, nctx=16, seed=3)
 
 
+@pytest.mark.parametrize("norms", [True, False])
+def test_attn_step_is_qk_rope_then_attn_rows(dev, norms):
+    """One token's attention as two launches (ilt_attn_step) against the three it stands for, at positions in the
+    first and in later blocks of 256 scores and on a block's edges: the output and the caches' rows bit for bit,
+    q and k untouched."""
+    import ctypes as C
+    from illatio_amd import hip
+    nh, nkv, hd, nctx, eps = 8, 2, 64, 600, 1e-6
+    rng = synth.make_rng(11)
+    f = lambda *sh: (rng.standard_normal(sh) * 1.5).astype(np.float32)
+    up = lambda a: (lambda b: (hip.hip_upload_vector(b, a), b)[1])(hip.hip_alloc(dev, a.nbytes))
+    P = lambda b: C.c_uint64(b.ptr if b is not None else 0)
+    S = C.c_uint64(0)
+    table = np.zeros((nctx, hd), np.float32)
+    assert hip.lib().ilt_rope_table(C.c_int(hd), C.c_int(0), C.c_int(nctx), C.c_float(1e6), table.ctypes.data_as(C.c_void_p)) == 0
+    rope, qn, kn = up(table), (up(f(hd)) if norms else None), (up(f(hd)) if norms else None)
+    kc0, vc0 = f(nctx, nkv * hd), f(nctx, nkv * hd)
+    scratch = hip.hip_alloc(dev, 4 * nh * nctx)
+    for pos in (0, 1, 255, 256, 257, 511, 599):
+        q, k, v = f(nh * hd), f(nkv * hd), f(nkv * hd)
+        res = []
+        for fused in (False, True):
+            dq, dk, dv, kc, vc, out = up(q), up(k), up(v), up(kc0), up(vc0), hip.hip_alloc(dev, 4 * nh * hd)
+            ints = (C.c_int(nh), C.c_int(nkv), C.c_int(hd), C.c_int(hd), C.c_int(pos), C.c_float(eps), C.c_int(1))
+            if fused:
+                hip.call("ilt_attn_step", S, P(dq), P(dk), P(dv), P(qn), P(kn), P(rope), P(kc), P(vc), P(out), *ints, P(scratch))
+                assert np.array_equal(bits(hip.hip_floats(dq, nh * hd)), bits(q)) and np.array_equal(bits(hip.hip_floats(dk, nkv * hd)), bits(k))
+            else:
+                hip.call("ilt_qk_rope", S, P(dq), P(dk), P(dv), P(qn), P(kn), P(rope), P(kc), P(vc), *ints, C.c_int(1))
+                hip.call("ilt_attn_rows", S, P(dq), P(kc), P(vc), P(out), C.c_int(nh), C.c_int(nkv), C.c_int(hd), C.c_int(pos), C.c_int(1), P(None))
+            res.append([hip.hip_floats(b, n) for b, n in ((out, nh * hd), (kc, nctx * nkv * hd), (vc, nctx * nkv * hd))])
+            for b in (dq, dk, dv, kc, vc, out):
+                hip.hip_free(b)
+        for a, b, what in zip(res[0], res[1], ("out", "kc", "vc")):
+            assert np.array_equal(bits(a), bits(b)), (pos, what)
+        assert not np.array_equal(res[0][1], kc0.ravel())         # the key's row was written
+    for b in (rope, qn, kn, scratch):
+        hip.hip_free(b)
+
+
 def test_small_decoder_long_contexts(dev):
     """Contexts past one workgroup's 256 positions of scores: the two-launch attention with 16 tokens, 4 tokens and one
     token a workgroup as the context grows towards 2048 positions, and past that the single launch with its value tiles."""
