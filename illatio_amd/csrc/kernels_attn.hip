@@ -20,20 +20,30 @@ __device__ __forceinline__ void wave_lds_sync() {
 
 // One head by one wave: x (hd floats) into xs (LDS): rmsnorm! of the head when its weights are given
 // (model.lisp:205-216: the squares, rounded to floats, added in double one after another), then rope-head!
-// from the position's table cs (cos, then sin, rd/2 each).  Only this wave touches xs and sc.
+// from the position's table cs (cos, then sin, rd/2 each).  Only this wave touches xs and sd.  The lanes add
+// the squares in parallel; where the order of the adds could show in the single the mean is rounded to, one
+// lane adds them again one after another, as the CPU does.
 __device__ __forceinline__ void rope_head_wave(const float* __restrict__ x, const float* __restrict__ nw, const float* __restrict__ cs,
-                                               float* xs, float* sc, int hd, int rd, float eps, int neox, int i) {
+                                               float* xs, double* sd, int hd, int rd, float eps, int neox, int i) {
   const int half = rd >> 1;
   for (int j = i; j < hd; j += 64) xs[j] = x[j];
   wave_lds_sync();
   if (nw) {
-    if (i == 0) {
-      double s = 0.0;
-      for (int j = 0; j < hd; j++) { const float sq = xs[j] * xs[j]; s += (double)sq; }
-      *sc = 1.0f / sqrtf((float)(s / (double)hd + (double)eps));
+    double s = 0.0;
+    for (int j = i; j < hd; j += 64) { const float sq = xs[j] * xs[j]; s += (double)sq; }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) s += __shfl_xor(s, off);
+    const double slack = s * ((double)(hd + 8) * 0x1p-51);
+    if ((float)((s - slack) / (double)hd + (double)eps) != (float)((s + slack) / (double)hd + (double)eps)) {      // the same in every lane
+      if (i == 0) {
+        double s2 = 0.0;
+        for (int j = 0; j < hd; j++) { const float sq = xs[j] * xs[j]; s2 += (double)sq; }
+        *sd = s2;
+      }
+      wave_lds_sync();
+      s = *sd;
     }
-    wave_lds_sync();
-    const float scale = *sc;
+    const float scale = 1.0f / sqrtf((float)(s / (double)hd + (double)eps));
     for (int j = i; j < hd; j += 64) xs[j] = (xs[j] * scale) * nw[j];
     wave_lds_sync();
   }
@@ -52,7 +62,7 @@ __global__ __launch_bounds__(64) void qk_rope_kernel(float* __restrict__ q, floa
                                                      const float* __restrict__ rope, float* __restrict__ kc, float* __restrict__ vc,
                                                      int nh, int nkv, int hd, int rd, int pos0, float eps, int neox) {
   __shared__ float xs[512];
-  __shared__ float sc;
+  __shared__ double sc;
   const int head = blockIdx.x, t = blockIdx.y, i = threadIdx.x;
   const int pos = pos0 + t;
   const int qd = nh * hd, kvd = nkv * hd;
@@ -237,7 +247,7 @@ __global__ __launch_bounds__(1024) void attn_step_scores_kernel(const float* __r
                                                                 float* __restrict__ raw, int nh, int nkv, int hd, int rd, int pos, float eps,
                                                                 int neox, float scale, int spitch) {
   __shared__ float qsh[256], ksh[256];
-  __shared__ float scs[2];
+  __shared__ double scs[2];
   const int h = blockIdx.x, tid = threadIdx.x, npos = pos + 1, pbase = blockIdx.y * 256;
   if (pbase >= npos) return;
   const int group = nh / nkv, kvd = nkv * hd, kh = h / group, ko = kh * hd;
