@@ -18,13 +18,17 @@
  * the quantizers' special cases; row dots against a double-precision dot of
  * dequantized values (the reference's own criterion, inspect/iquant-test.lisp:
  * 45-53); d4-route against a stable sort; the IQ2_XXS tables against the
- * reference's three copies.
+ * reference's three copies; swiglu!, f32-dot16, rope-table, rope-head!,
+ * attend-head! against explicit evaluations in numpy (with the plausible
+ * misreadings shown to give other bits), forward-1 as those pieces in order.
  *
  * Parity unpinned (last-bit only): orc_silu / orc_softplus / orc_sigmoid use
  * (float)exp((double)x) and (float)log((double)x) as SBCL does for
  * single-float arguments (ds4f.lisp:248-254); they are checked against the
  * correctly rounded value, which SBCL's libm call yields except where the
- * double result falls within ~2^-29 of a single-precision rounding boundary.
+ * double result falls within ~2^-29 of a single-precision rounding boundary;
+ * orc_rope_table's cos and sin likewise.  Parity unpinned: orc_rmsnorm (no
+ * vector of the reference's covers it; see its comment).
  */
 #include <float.h>
 #include <math.h>
