@@ -10,7 +10,15 @@ streamed from HBM per step, every matrix its own allocation, so the working set 
 is far beyond the 256 MB MALL.  No attention, norm or RoPE runs in a step: those belong to
 the dense-forward harness, not to this path.
 
+Without --workload the line is c2's, and the other configurations run after it on the same clock
+and are reported under "configs" (c2_decode, c1, c3 and c5 on the bf16 matrix cores and on the exact
+int8 path, c4 with the routing on the device); c2_decode's figures are also the line's
+decode_tok_per_s, decode_ms_per_token and prefill_tok_per_s.
+
 Other workloads (--workload), each BASELINE.json's config of the same number:
+  c2d the whole dense decoder at config 2's shape (36 layers, head norms, RoPE, attention over an
+      fp32 KV cache): a 512-token prompt through the prefill products, then 256 greedy tokens,
+      every token's logits downloaded and the next token picked on the host
   c1  Q8_0 decode GEMV 4864x896 and 896x4864, rotating over 64 copies (593 MB)
   c3  Q6_K prefill product 17408x5120 on T tokens (--tokens, default 4096): bf16 matrix
       cores (--path bf16, the float activations rounded to bf16 inside the step) or the
@@ -630,6 +638,23 @@ def workload_c2d(args, dev):
     wbytes = sum(a[1].size for L in host["layers"] for k, a in L.items() if isinstance(a, tuple)) + host["output"][1].size
     ms = decode_s * 1e3 / ndecode
     m.free()
+
+    def cpu():
+        import oracle_lib as orc
+        cores = host_cores()
+        cm = orc.DenseModel(host, 64)
+        t_tok = prompt[0]
+        cm.forward(t_tok, nthreads=cores)                     # the pool's threads started, the weights touched
+        t1 = time.perf_counter()
+        n = 0
+        while time.perf_counter() - t1 < 10.0 and n < 60:
+            logits, _ = cm.forward(t_tok, nthreads=cores)
+            t_tok = int(np.argmax(logits))
+            n += 1
+        t_cpu = time.perf_counter() - t1
+        return {"value": round(n / t_cpu, 3), "unit": "tok/s", "cores": cores, "kind": "port",
+                "sample": f"{n} greedy tokens of the same model from an empty context (attention over at most {n + 1} positions), {t_cpu:.1f} s"}
+
     return {"value": round(ndecode / decode_s, 1), "unit": "tok/s", "ms_per_step": ms, "device_ms_per_step": ms, "enqueue_ms": 0.0,
             "dtype": "int8 block dots, fp32 combine; fp32 attention",
             "metric": "decode tok/s at Qwen3-4B shape",
@@ -639,9 +664,10 @@ def workload_c2d(args, dev):
                       "weights_GBps_in_decode": round(wbytes / (ms * 1e-3) / 1e9, 1)},
             "roofline": {"bound": "hbm", "achieved": round(wbytes / (ms * 1e-3) / 1e9, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                          "frac": round(wbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4), "traffic": None,
-                         "kernel": "whole token: 6 launches a layer (Q/K/V, qk_rope, attn_rows, wo, gate+up, down) + embedding + head, logits to the host",
+                         "kernel": "whole token: 6 launches a layer (Q/K/V, head norms + RoPE + attention scores, softmax + values, wo, gate+up, "
+                                   "down) + embedding + head, logits to the host",
                          "launches": 6 * nl + 2, "avg_launch_us": round(ms * 1e3 / (6 * nl + 2), 2)},
-            "cpu": lambda: None}
+            "cpu": cpu}
 
 
 WORKLOADS = {"c1": workload_c1, "c2": workload_c2, "c2d": workload_c2d, "c3": workload_c3, "c4": workload_c4, "c5": workload_c5}
