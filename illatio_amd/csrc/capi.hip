@@ -759,6 +759,35 @@ int ilt_attn_step(uint64_t stream, const float* q, const float* k, const float* 
   ILT_REQUIRE(q && k && v && rope && kc && vc && out && scratch && nh > 0 && nkv > 0 && pos >= 0 && pos < 2048);
   return (int)ilt_k_attn_step(q, k, v, qn, kn, rope, kc, vc, out, nh, nkv, hd, rd, pos, eps, neox, scratch, S(stream));
 }
+// ---- one token through the dense decoder: the launches of the single calls, queued in one ----------
+static ilt_mv_desc mv_of(const ilt_dense_mat& w, float* y) { return {w.gguf_type, w.rows, w.w, w.wd, y, nullptr}; }
+int ilt_dense_decode(uint64_t stream, const ilt_dense_model* m, const int32_t* token, int pos, int want_logits) {
+  ILT_REQUIRE(m && token && m->layers && m->nl > 0 && pos >= 0 && pos < 2048);
+  ILT_REQUIRE(m->x && m->q && m->k && m->v && m->att && m->fa && m->scores && m->rope && (!want_logits || (m->logits && m->output_norm)));
+  int e;
+  if (m->embd.gguf_type == ILT_TYPE_Q8_0) e = ilt_embed_q8(stream, (const int8_t*)m->embd.w, m->embd.wd, token, m->x, m->d, 1);
+  else e = ilt_embed_k(stream, m->embd.gguf_type == ILT_TYPE_Q4_K ? 0 : m->embd.gguf_type == ILT_TYPE_Q6_K ? 2 : -1, m->embd.w, token, m->x, m->d, 1);
+  if (e) return e;
+  for (int l = 0; l < m->nl; l++) {
+    const ilt_dense_layer& L = m->layers[l];
+    const ilt_mv_desc qkv[3] = {mv_of(L.wq, m->q), mv_of(L.wk, m->k), mv_of(L.wv, m->v)};
+    if ((e = ilt_mv_multi_norm(stream, 3, qkv, m->d, m->x, L.attn_norm, m->eps, 0, 1, 0))) return e;
+    if ((e = ilt_attn_step(stream, m->q, m->k, m->v, L.q_norm, L.k_norm, m->rope, L.kc, L.vc, m->att, m->nh, m->nkv, m->hd, m->rd, pos, m->eps,
+                           m->neox, m->scores))) return e;
+    const ilt_mv_desc wo = mv_of(L.wo, m->x);
+    if ((e = ilt_mv_multi(stream, 1, &wo, L.wo.cols, nullptr, nullptr, nullptr, m->att, 1, 1, 0))) return e;
+    const ilt_mv_desc glu[2] = {mv_of(L.gate, m->fa), mv_of(L.up, m->fa)};
+    if ((e = ilt_mv_multi_norm(stream, 2, glu, m->d, m->x, L.ffn_norm, m->eps, 0, 1, 1))) return e;
+    const ilt_mv_desc down = mv_of(L.down, m->x);
+    if ((e = ilt_mv_multi(stream, 1, &down, L.down.cols, nullptr, nullptr, nullptr, m->fa, 1, 1, 0))) return e;
+  }
+  if (want_logits) {
+    const ilt_mv_desc head = mv_of(m->output, m->logits);
+    if ((e = ilt_mv_multi_norm(stream, 1, &head, m->d, m->x, m->output_norm, m->eps, 0, 1, 0))) return e;
+  }
+  return ILT_OK;
+}
+
 // rope-table (model.lisp:218-231) for positions pos0 .. pos0 + n - 1, on the host: a position's head_dim/2 cosines
 // then head_dim/2 sines, theta advanced by repeated single-float multiplication, theta-scale, cos and sin through
 // double and rounded to single as SBCL evaluates them.  The only float arithmetic this file does: model constants,

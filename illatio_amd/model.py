@@ -37,6 +37,25 @@ def synth_model(seed, d=2560, ffn=9728, nh=32, nkv=8, hd=128, nl=36, vocab=15193
             "embd": embd, "output": embd, "output_norm": norm(d), "layers": layers}
 
 
+class _Mat(C.Structure):
+    _fields_ = [("gguf_type", C.c_int), ("rows", C.c_int), ("cols", C.c_int), ("w", C.c_uint64), ("wd", C.c_uint64)]
+
+
+class _Layer(C.Structure):
+    _fields_ = [("attn_norm", C.c_uint64), ("q_norm", C.c_uint64), ("k_norm", C.c_uint64), ("ffn_norm", C.c_uint64)] + \
+               [(n, _Mat) for n in ("wq", "wk", "wv", "wo", "gate", "up", "down")] + [("kc", C.c_uint64), ("vc", C.c_uint64)]
+
+
+class _Model(C.Structure):
+    _fields_ = [(n, C.c_int) for n in ("nl", "d", "ffn", "nh", "nkv", "hd", "rd", "neox")] + [("eps", C.c_float), ("embd", _Mat), ("output", _Mat),
+               ("output_norm", C.c_uint64), ("rope", C.c_uint64), ("layers", C.POINTER(_Layer))] + \
+               [(n, C.c_uint64) for n in ("x", "q", "k", "v", "att", "fa", "scores", "logits")]
+
+
+def _mat(w):
+    return _Mat(w.type, w.rows, w.cols, w.qs.ptr, w.d.ptr if w.d else 0)
+
+
 class DenseModel:
     """HOST (synth_model's dict, or the same made from a file's tensors) on DEV, with caches for NCTX positions."""
 
@@ -70,6 +89,16 @@ class DenseModel:
         self.scores = A(4 * n * c["nh"] * ((nctx + 3) // 4 * 4)) if nctx <= 2048 else None      # the attention's raw scores
         self.logits = A(4 * c["vocab"])
         self.acts = {cols: dense.QAct(dev, n, cols, ("q8k",)) for cols in {d, self.qd, ffn}}
+        # the model as ilt_dense_decode reads it: a token's launches queued by one call
+        ptr = lambda b: b.ptr if b is not None else 0
+        self._clayers = (_Layer * len(self.layers))()
+        for i, L in enumerate(self.layers):
+            self._clayers[i] = _Layer(ptr(L["attn_norm"]), ptr(L["q_norm"]), ptr(L["k_norm"]), ptr(L["ffn_norm"]),
+                                      *[_mat(L[n]) for n in ("wq", "wk", "wv", "wo", "gate", "up", "down")], L["kc"].ptr, L["vc"].ptr)
+        self._cmodel = _Model(len(self.layers), d, ffn, c["nh"], c["nkv"], hd, hd, 1 if c["neox"] else 0, c["eps"], _mat(self.embd), _mat(self.output),
+                              self.output_norm.ptr, self.rope.ptr, self._clayers, self.x.ptr, self.q.ptr, self.k.ptr, self.v.ptr, self.att.ptr,
+                              self.fa.ptr, ptr(self.scores), self.logits.ptr)
+        self.one_call = self.scores is not None       # False: a token's launches one by one from here (the same launches)
 
     def forward_n(self, tokens, logits=True):
         """TOKENS at the next positions (CUDA-FORWARD-N); the last one's logits, if LOGITS, into self.logits."""
@@ -80,6 +109,10 @@ class DenseModel:
         S = C.c_uint64(dev.stream)
         P = lambda b, off=0: C.c_uint64(b.ptr + off if b is not None else 0)
         hip.hip_upload_vector(self.tokens, np.asarray(tokens, np.int32))
+        if n == 1 and self.one_call:
+            hip.call("ilt_dense_decode", S, C.byref(self._cmodel), P(self.tokens), C.c_int(self.pos), C.c_int(1 if logits else 0))
+            self.pos += 1
+            return self.logits
         dense.embed(dev, self.embd, self.tokens, self.x, n, d)
         for L in self.layers:
             if n == 1:

@@ -311,6 +311,30 @@ int ilt_attn_rows(uint64_t stream, const float* q, const float* kc, const float*
    scratch: nh * ((pos + 4) & ~3) floats. */
 int ilt_attn_step(uint64_t stream, const float* q, const float* k, const float* v, const float* qn, const float* kn, const float* rope, float* kc,
                   float* vc, float* out, int nh, int nkv, int hd, int rd, int pos, float eps, int neox, float* scratch);
+
+/* One token through the whole dense decoder in one call: what the host loop of cuda-forward-n queues for one
+   token (cuda-dense.lisp:380-432; the CPU's forward-1, model.lisp:396-462) -- embedding row, then per layer the
+   Q/K/V products with the norm inside, ilt_attn_step, wo onto the residual, gate/up with the norm and the gated
+   activation inside, down onto the residual, and (want_logits) the output norm and head: 6 launches a layer + 2.
+   The structs are read on the host during the call; every pointer in them is device memory but `layers`.
+   Matrices as dense uploads hold them (Q8_0 split into quants and scales, Q6_K in 212-byte blocks).  pos < 2048
+   (the attention's scratch), the caches hold at least pos + 1 positions, rope at least (pos + 1) * rd floats.
+   token: one id, on the device.  The results are those of the single calls, bit for bit. */
+typedef struct ilt_dense_mat { int gguf_type, rows, cols; const void* w; const uint16_t* wd; } ilt_dense_mat;
+typedef struct ilt_dense_layer {
+  const float *attn_norm, *q_norm, *k_norm, *ffn_norm;        /* q_norm, k_norm: null when the model has no head norms */
+  ilt_dense_mat wq, wk, wv, wo, gate, up, down;
+  float *kc, *vc;                                             /* this layer's caches, nkv * hd floats a position */
+} ilt_dense_layer;
+typedef struct ilt_dense_model {
+  int nl, d, ffn, nh, nkv, hd, rd, neox;
+  float eps;
+  ilt_dense_mat embd, output;
+  const float *output_norm, *rope;
+  const ilt_dense_layer* layers;                              /* nl of them, host memory */
+  float *x, *q, *k, *v, *att, *fa, *scores, *logits;          /* d, nh*hd, nkv*hd, nkv*hd, nh*hd, ffn, nh*((pos+4)&~3), vocab floats */
+} ilt_dense_model;
+int ilt_dense_decode(uint64_t stream, const ilt_dense_model* m, const int32_t* token, int pos, int want_logits);
 int ilt_swiglu(uint64_t stream, float* a, const float* b, int64_t n);
 
 /* Prefill products on the int8 matrix cores, y[t*rows + r] = W[r].x_t (+ bias[r]) for n

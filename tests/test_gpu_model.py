@@ -23,7 +23,7 @@ def bits(a):
     return np.ascontiguousarray(a, np.float32).view(np.uint32)
 
 
-def run_greedy(dev, host, nprompt, ndecode, chunk, nctx, seed, check_cache=False):
+def run_greedy(dev, host, nprompt, ndecode, chunk, nctx, seed, check_cache=False, one_call=True):
     from illatio_amd import hip, model
     c = host["config"]
     rng = synth.make_rng(seed)
@@ -33,6 +33,7 @@ def run_greedy(dev, host, nprompt, ndecode, chunk, nctx, seed, check_cache=False
         cpu.forward(t, logits=False, nthreads=16)
     want, _ = cpu.forward(prompt[-1], nthreads=16)
     gpu = model.DenseModel(dev, host, nctx, chunk=chunk)
+    gpu.one_call = gpu.one_call and one_call                  # a token by ilt_dense_decode, or launch by launch from Python
     gpu.eval_tokens(prompt)                                   # the prompt through the prefill products, chunk by chunk
     got = hip.hip_floats(gpu.logits, c["vocab"])
     assert np.array_equal(bits(got), bits(want)), ("prompt", np.abs(got - want).max())
@@ -61,6 +62,8 @@ def test_small_decoder_prefill_chunks_and_decode(dev):
     from illatio_amd import model
     host = model.synth_model(3, d=512, ffn=1024, nh=8, nkv=2, hd=64, nl=3, vocab=1000)
     same, _ = run_greedy(dev, host, nprompt=40, ndecode=24, chunk=16, nctx=80, seed=1, check_cache=True)
+    assert same == 24
+    same, _ = run_greedy(dev, host, nprompt=40, ndecode=24, chunk=16, nctx=80, seed=1, one_call=False)
     assert same == 24
     # a prompt of one token, and a chunk larger than the prompt
     run_greedy(dev, host, nprompt=1, ndecode=3, chunk=16, nctx=8, seed=2)
