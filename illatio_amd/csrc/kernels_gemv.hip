@@ -947,6 +947,13 @@ __global__ __launch_bounds__(kStreamThreads) void gemv_stream_kernel(IltGemvPara
   // Q8_0: the scales' room behind the quants'
   const u8* scales = region + (long)p.batch * p.cols;
   const u8* scales_up = region_up + (long)p.batch * p.cols;
+  // What the sum is added to (acc) and the bias, asked for before the rows: they are there when the sums are, instead
+  // of a trip to memory after them.  No branch around the loads (a conditional load is waited for at the join): a
+  // launch without them reads y, whose value it does not use.
+  float* const ydst = m.y + (long)z * p.y_stride;
+  const long rmine = row0 + min(lane, max(nrows - 1, 0));
+  const float* const bsrc = m.bias ? m.bias : ydst;
+  const float yold = ydst[rmine], bval = bsrc[rmine];
   int nup = 0;              // load instructions of the up matrix's rows: the last ones issued
   if (live) {
     with_format<FSET>(fmt, [&](auto F) { stream_run<decltype(F)::value>(wg, row0, nrows, S, m.row_bytes, region, lane); });
@@ -997,8 +1004,8 @@ __global__ __launch_bounds__(kStreamThreads) void gemv_stream_kernel(IltGemvPara
         y[r] = o;
       }
     } else {
-      if (m.bias) v = v + m.bias[r];
-      if (p.acc) v = y[r] + v;
+      if (m.bias) v = v + bval;
+      if (p.acc) v = yold + v;
       y[r] = v;
     }
   }
