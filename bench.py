@@ -717,11 +717,14 @@ def main():
     out["cpu_baseline"] = None if args.no_cpu else r["cpu"]()
     if everything:
         # BASELINE's other configurations on the same clock (no CPU leg): c4 with the routing on the device, c3 and
-        # c5 on the bf16 matrix cores at 4096 tokens and, as a second entry each, on the bit-exact int8 path
+        # c5 on the bf16 matrix cores at 4096 tokens and, as a second entry each, on the bit-exact int8 path; c3 also at
+        # its other two token counts and with the matrix's bf16 copy made once and kept (2 bytes a weight of the 288 GB)
         import copy
         import gc
         out["configs"] = {}
-        extras = [("c2_decode", {}), ("c1", {}), ("c3", {"path": "bf16", "tokens": 4096}), ("c3_exact", {"path": "int8", "tokens": 4096}),
+        extras = [("c2_decode", {}), ("c1", {}), ("c3", {"path": "bf16", "tokens": 4096}), ("c3_t2048", {"path": "bf16", "tokens": 2048}),
+                  ("c3_t512", {"path": "bf16", "tokens": 512}), ("c3_resident", {"path": "bf16-resident", "tokens": 4096}),
+                  ("c3_exact", {"path": "int8", "tokens": 4096}),
                   ("c4", {"mode": "device"}), ("c5", {"path": "bf16", "tokens": 4096}), ("c5_exact", {"path": "int8", "tokens": 4096})]
         for name, over in extras:
             a = copy.copy(args)

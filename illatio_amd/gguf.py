@@ -191,3 +191,71 @@ def upload_shared_expert(dev, g, layer):
     if tuple(tis[1].dims) != (d, ff) or tuple(tis[2].dims) != (ff, d):
         raise GgufError(f"blk.{layer}: the shared expert's gate, up and down do not fit one another")
     return ds4f.SharedExpert(dev, d, ff, *(tensor_bytes(g, ti) for ti in tis))
+
+
+DENSE_ARCHS = {"qwen2": True, "qwen3": True, "qwen3vl": True, "llama": False}       # architecture -> NEOX RoPE (model.lisp:94-96)
+
+
+def dense_model(g):
+    """The dense decoder in the GGUF file G as the dict illatio_amd.model.DenseModel takes (LOAD-MODEL-1,
+    model.lisp:66-138): the architecture's keys into "config", every matrix as (GGUF type, its rows' bytes, memory-
+    mapped), the norms as floats; without an output.weight the head is the embedding.  Q4_K / Q6_K matrices and
+    layers without attention biases (the decoder here multiplies those); anything else raises."""
+    from .synth import Q4_K, Q6_K, row_bytes
+    arch = g.meta("general.architecture")
+    if arch not in DENSE_ARCHS:
+        raise GgufError(f"architecture {arch!r} is not a dense decoder this loader reads ({', '.join(DENSE_ARCHS)} are)")
+    key = lambda k, default=None: g.meta(f"{arch}.{k}", default)
+
+    def need(k):
+        v = key(k)
+        if v is None:
+            raise GgufError(f"GGUF: no {arch}.{k}")
+        return v
+
+    nl, d, nh = int(need("block_count")), int(need("embedding_length")), int(need("attention.head_count"))
+    nkv = int(key("attention.head_count_kv", nh))
+    hd = int(key("attention.key_length", d // nh))
+    rd = int(key("rope.dimension_count", hd))
+    if rd != hd:
+        raise GgufError(f"RoPE over {rd} of a head's {hd} dimensions is not supported")
+
+    def mat(name, rows, cols):
+        ti = gguf_tensor(g, name)
+        if ti.type not in (Q4_K, Q6_K):
+            raise GgufError(f"{name}: type {ti.type_name}; the decoder here multiplies Q4_K and Q6_K matrices")
+        if tuple(ti.dims) != (cols, rows):
+            raise GgufError(f"{name}: dimensions {list(ti.dims)}, expected [{cols}, {rows}]")
+        return ti.type, tensor_bytes(g, ti).reshape(rows, row_bytes(ti.type, cols))
+
+    def f32(name, n, optional=False):
+        ti = gguf_tensor(g, name, errorp=not optional)
+        if ti is None:
+            return None
+        if GGML_TYPES[ti.type][0] != "f32" or ti.elements() != n:
+            raise GgufError(f"{name}: expected {n} F32 values")
+        return np.frombuffer(tensor_bytes(g, ti), np.float32).copy()
+
+    ffn = int(need("feed_forward_length"))
+    embd_ti = gguf_tensor(g, "token_embd.weight")
+    vocab = int(embd_ti.dims[1])
+    embd = mat("token_embd.weight", vocab, d)
+    layers = []
+    for i in range(nl):
+        n = lambda t: f"blk.{i}.{t}"
+        for b in ("attn_q.bias", "attn_k.bias", "attn_v.bias"):
+            if gguf_tensor(g, n(b), errorp=False) is not None:
+                raise GgufError(f"{n(b)}: attention biases are not supported")
+        ffn_norm = f32(n("ffn_norm.weight"), d, optional=True)
+        layers.append({"attn_norm": f32(n("attn_norm.weight"), d), "wq": mat(n("attn_q.weight"), nh * hd, d),
+                       "wk": mat(n("attn_k.weight"), nkv * hd, d), "wv": mat(n("attn_v.weight"), nkv * hd, d),
+                       "wo": mat(n("attn_output.weight"), d, nh * hd),
+                       "q_norm": f32(n("attn_q_norm.weight"), hd, optional=True), "k_norm": f32(n("attn_k_norm.weight"), hd, optional=True),
+                       "ffn_norm": ffn_norm if ffn_norm is not None else f32(n("post_attention_norm.weight"), d),
+                       "gate": mat(n("ffn_gate.weight"), ffn, d), "up": mat(n("ffn_up.weight"), ffn, d),
+                       "down": mat(n("ffn_down.weight"), d, ffn)})
+    output = mat("output.weight", vocab, d) if gguf_tensor(g, "output.weight", errorp=False) is not None else embd
+    return {"config": {"d": d, "ffn": ffn, "nh": nh, "nkv": nkv, "hd": hd, "nl": nl, "vocab": vocab,
+                       "eps": float(np.float32(need("attention.layer_norm_rms_epsilon"))), "rope_base": float(np.float32(key("rope.freq_base", 10000.0))),
+                       "neox": DENSE_ARCHS[arch]},
+            "embd": embd, "output": output, "output_norm": f32("output_norm.weight", d), "layers": layers}

@@ -158,3 +158,82 @@ def test_experts_of_a_file_take_a_decode_step_with_the_oracles_bits(tmp_path):
     for b in (lb, nb, out):
         hip.hip_free(b)
     pool.free(); sh.free()
+
+
+def _dense_file(tmp_path, host, arch="qwen3", tied=True):
+    """HOST (model.synth_model's dict) as a GGUF file of architecture ARCH, as llama.cpp's converter names things."""
+    c = host["config"]
+    qd, kvd = c["nh"] * c["hd"], c["nkv"] * c["hd"]
+    F32 = 0
+    meta = {"general.architecture": arch, f"{arch}.block_count": c["nl"], f"{arch}.embedding_length": c["d"],
+            f"{arch}.feed_forward_length": c["ffn"], f"{arch}.attention.head_count": c["nh"],
+            f"{arch}.attention.head_count_kv": c["nkv"], f"{arch}.attention.key_length": c["hd"],
+            f"{arch}.attention.layer_norm_rms_epsilon": float(c["eps"]), f"{arch}.rope.freq_base": float(c["rope_base"])}
+    fb = lambda a: np.ascontiguousarray(a, np.float32).view(np.uint8)
+    tensors = [("token_embd.weight", (c["d"], c["vocab"]), host["embd"][0], host["embd"][1]),
+               ("output_norm.weight", (c["d"],), F32, fb(host["output_norm"]))]
+    if not tied:
+        tensors.append(("output.weight", (c["d"], c["vocab"]), host["output"][0], host["output"][1]))
+    shapes = {"wq": ("attn_q", c["d"], qd), "wk": ("attn_k", c["d"], kvd), "wv": ("attn_v", c["d"], kvd), "wo": ("attn_output", qd, c["d"]),
+              "gate": ("ffn_gate", c["d"], c["ffn"]), "up": ("ffn_up", c["d"], c["ffn"]), "down": ("ffn_down", c["ffn"], c["d"])}
+    for i, L in enumerate(host["layers"]):
+        for k, (name, cols, rows) in shapes.items():
+            tensors.append((f"blk.{i}.{name}.weight", (cols, rows), L[k][0], L[k][1]))
+        for k, name in (("attn_norm", "attn_norm"), ("ffn_norm", "ffn_norm"), ("q_norm", "attn_q_norm"), ("k_norm", "attn_k_norm")):
+            tensors.append((f"blk.{i}.{name}.weight", (len(L[k]),), F32, fb(L[k])))
+    p = tmp_path / f"{arch}.gguf"
+    write_gguf(p, meta, tensors)
+    return p
+
+
+def test_dense_model_of_a_file(tmp_path):
+    """gguf.dense_model (load-model-1, model.lisp:66-138): the architecture's keys, every matrix and norm of a written
+    qwen3-style file, the head tied to the embedding when the file has no output.weight; files it does not read raise."""
+    from illatio_amd import model
+    host = model.synth_model(21, d=256, ffn=512, nh=4, nkv=2, hd=64, nl=2, vocab=300)
+    g = gguf.read_gguf(str(_dense_file(tmp_path, host)))
+    got = gguf.dense_model(g)
+    f32 = lambda c: {k: (float(np.float32(v)) if isinstance(v, float) else v) for k, v in c.items()}      # the file holds singles
+    assert f32(got["config"]) == f32(host["config"])
+    assert got["output"] is got["embd"]
+    assert got["embd"][0] == host["embd"][0] and np.array_equal(got["embd"][1], host["embd"][1])
+    assert np.array_equal(got["output_norm"], host["output_norm"])
+    for a, b in zip(got["layers"], host["layers"]):
+        assert set(a) == set(b)
+        for k in b:
+            if isinstance(b[k], tuple):
+                assert a[k][0] == b[k][0] and np.array_equal(a[k][1], b[k][1]), k
+            else:
+                assert np.array_equal(a[k], b[k]), k
+    host2 = dict(host, output=(host["embd"][0], host["embd"][1][::-1].copy()))
+    got2 = gguf.dense_model(gguf.read_gguf(str(_dense_file(tmp_path, host2, arch="llama", tied=False))))
+    assert got2["config"]["neox"] is False and got2["output"] is not got2["embd"]
+    assert np.array_equal(got2["output"][1], host2["output"][1])
+    with pytest.raises(gguf.GgufError):
+        gguf.dense_model(gguf.read_gguf(str(_dense_file(tmp_path, host, arch="deepseek4"))))
+    bad = dict(host, layers=[dict(L, wq=(synth.Q8_0, synth.weights(synth.Q8_0, 256, 256, synth.make_rng(1)))) for L in host["layers"]])
+    with pytest.raises(gguf.GgufError):
+        gguf.dense_model(gguf.read_gguf(str(_dense_file(tmp_path, bad))))
+
+
+@pytest.mark.gpu
+def test_decoder_of_a_file_decodes_with_the_oracles_bits(tmp_path):
+    """A written qwen3-style file read back, uploaded and run: prompt and greedy tokens with the CPU oracle's logits."""
+    import oracle_lib as orc
+    from illatio_amd import hip, model
+    dev = hip.open_hip(0)
+    host = model.synth_model(22, d=256, ffn=512, nh=4, nkv=2, hd=64, nl=2, vocab=300)
+    got = gguf.dense_model(gguf.read_gguf(str(_dense_file(tmp_path, host))))
+    cpu, gpu = orc.DenseModel(host, 24), model.DenseModel(dev, got, 24, chunk=8)
+    prompt = [5, 17, 255, 3, 99, 100, 1, 42, 7, 8, 9]
+    for t in prompt[:-1]:
+        cpu.forward(t, logits=False, nthreads=4)
+    want, _ = cpu.forward(prompt[-1], nthreads=4)
+    gpu.eval_tokens(prompt)
+    for _ in range(6):
+        have = hip.hip_floats(gpu.logits, 300)
+        assert np.array_equal(have.view(np.uint32), want.view(np.uint32))
+        tok = int(np.argmax(want))
+        want, _ = cpu.forward(tok, nthreads=4)
+        gpu.forward_n([tok])
+    gpu.free()
