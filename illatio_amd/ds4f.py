@@ -20,9 +20,12 @@ from .synth import IQ2_XXS, Q2_K, Q8_0, row_bytes
 
 
 class ExpertPool:
-    """NE experts on DEV, slot e = gate | up | down of expert e, 256-byte aligned."""
+    """NE experts on DEV, slot e = gate | up | down of expert e, 256-byte aligned.  The experts in HOST_EXPERTS stay
+    in pinned host memory instead and are read through from there by the same kernels, their table entries pointing
+    at it (what the reference's srcs[z] gives an expert without a slot, ds4f.cu:742-760): for a pool larger than the
+    device's memory; with 288 GB every expert of a layer set fits and the default keeps all of them in HBM."""
 
-    def __init__(self, dev, ne, d, ff, gate, up, down):
+    def __init__(self, dev, ne, d, ff, gate, up, down, host_experts=()):
         self.dev, self.ne, self.d, self.ff = dev, ne, d, ff
         self.grb, self.drb = row_bytes(IQ2_XXS, d), row_bytes(Q2_K, ff)
         self.gate_bytes, self.down_bytes = ff * self.grb, d * self.drb
@@ -32,14 +35,31 @@ class ExpertPool:
         host[:, self.gate_bytes:2 * self.gate_bytes] = np.asarray(up, np.uint8).reshape(ne, self.gate_bytes)
         host[:, 2 * self.gate_bytes:2 * self.gate_bytes + self.down_bytes] = np.asarray(down, np.uint8).reshape(ne, self.down_bytes)
         self.pool = hip.hip_upload_new(dev, host)
+        self.host_experts = sorted(set(int(e) for e in host_experts))
+        self.host_buf = 0
+        if self.host_experts:
+            import ctypes
+            self.host_buf = hip.hip_host_alloc(dev, len(self.host_experts) * self.slot_bytes)
+            for i, e in enumerate(self.host_experts):
+                ctypes.memmove(self.host_buf + i * self.slot_bytes, host[e].ctypes.data, self.slot_bytes)
+                hip.hip_zero(hip.DBuf(self.slot_ptr_device(e), self.slot_bytes, dev))      # the device slot plays no part
         self.ptrs = hip.hip_upload_new(dev, np.array([self.slot_ptr(e) for e in range(ne)], np.uint64))
 
-    def slot_ptr(self, e):
+    def slot_ptr_device(self, e):
         return self.pool.ptr + int(e) * self.slot_bytes
 
+    def slot_ptr(self, e):
+        if int(e) in self.host_experts:
+            return self.host_buf + self.host_experts.index(int(e)) * self.slot_bytes
+        return self.slot_ptr_device(e)
+
     def free(self):
+        hip.hip_sync(self.dev)
         hip.hip_free(self.pool)
         hip.hip_free(self.ptrs)
+        if self.host_buf:
+            hip.hip_host_free(self.host_buf)
+            self.host_buf = 0
 
 
 class SharedExpert:

@@ -204,6 +204,19 @@ def hip_floats(b, n, start=0):
     return hip_download(b, np.float32, n, 4 * start)
 
 
+def hip_host_alloc(dev, nbytes, mapped=True):
+    """NBYTES of pinned host memory (CUDA-HOST-ALLOC, cuda.lisp:359-366); MAPPED: kernels on DEV may read it at the
+    same address (an expert's matrices read through from host memory).  Returns the address."""
+    hip_current(dev)
+    p = C.c_uint64(0)
+    call("ilt_host_alloc", C.byref(p), C.c_uint64(nbytes), C.c_uint(1 | (2 if mapped else 0)))
+    return p.value
+
+
+def hip_host_free(addr):
+    call("ilt_host_free", C.c_uint64(addr))
+
+
 def hip_event_create(dev, timing=False):
     hip_current(dev)
     e = C.c_uint64(0)

@@ -222,6 +222,27 @@ def test_moe_decode_step_bit_exact(dev, ne, d, ff, nu, clamp):
     pool.free(); sh.free()
 
 
+def test_experts_read_through_from_pinned_host_memory(dev):
+    """Experts without a place in HBM: their matrices stay in pinned, mapped host memory and the table of slots points
+    there (the reference's read-through, ds4f.cu:742-760, cuda-ds4f.lisp:553-640); their device slots are zeroed, so the
+    decode step's bits -- equal to the all-resident pool's and the oracle's -- can only come from host memory."""
+    from illatio_amd import ds4f, hip
+    ne, d, ff, nu, clamp = 8, 512, 256, 3, 0.05
+    rng = synth.make_rng(77)
+    gate, up, down, sg, su, sd = _moe_weights(rng, ne, d, ff)
+    sh = ds4f.SharedExpert(dev, d, ff, sg, su, sd)
+    norm, logits = synth.activations(d, rng), synth.activations(ne, rng)
+    want, wsel, _ = orc.moe_token(gate, up, down, sg, su, sd, d, ff, ne, nu, 1.5, clamp, logits, norm)
+    on_host = [int(wsel[0]), int(wsel[2]), int(next(e for e in range(ne) if e not in wsel.tolist()))]      # two that are chosen, one that is not
+    pool = ds4f.ExpertPool(dev, ne, d, ff, gate, up, down, host_experts=on_host)
+    lb, nb, out = hip.hip_upload_new(dev, logits), hip.hip_upload_new(dev, norm), hip.hip_alloc(dev, 4 * d)
+    ds4f.ffn_step_call(dev, pool, sh, lb, nb, out, ne, nu, 1.5, clamp)
+    assert np.array_equal(bits(hip.hip_floats(out, d)), bits(want))
+    for b in (lb, nb, out):
+        hip.hip_free(b)
+    pool.free(); sh.free()
+
+
 @pytest.mark.parametrize("ne,d,ff,nu,n,clamp", [(8, 512, 256, 3, 9, 0.05), (12, 4096, 2048, 6, 4, 0.0)])
 def test_moe_short_pass_of_a_few_tokens_bit_exact(dev, ne, d, ff, nu, n, clamp):
     """A speculative step's verification (cuda-ds4f-spec.lisp:30-100): the FFN of up to nine tokens
