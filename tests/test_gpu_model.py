@@ -110,6 +110,22 @@ def test_attn_step_is_qk_rope_then_attn_rows(dev, norms):
         hip.hip_free(b)
 
 
+def test_llama_style_decoder(dev):
+    """No head norms, RoPE on adjacent pairs (2i, 2i + 1), heads of 96 (six partial sums of sixteen a score), one KV
+    head for all query heads; then heads of 256, the widest the attention takes."""
+    from illatio_amd import model
+    host = model.synth_model(8, d=512, ffn=768, nh=8, nkv=1, hd=96, nl=2, vocab=400)
+    host["config"]["neox"] = False
+    for L in host["layers"]:
+        L["q_norm"] = L["k_norm"] = None
+    for one_call in (True, False):
+        same, _ = run_greedy(dev, host, nprompt=21, ndecode=8, chunk=8, nctx=40, seed=8, check_cache=True, one_call=one_call)
+        assert same == 8
+    host = model.synth_model(9, d=512, ffn=768, nh=2, nkv=2, hd=256, nl=1, vocab=400)
+    same, _ = run_greedy(dev, host, nprompt=300, ndecode=4, chunk=64, nctx=320, seed=9)
+    assert same == 4
+
+
 def test_small_decoder_long_contexts(dev):
     """Contexts past one workgroup's 256 positions of scores: the two-launch attention with 16 tokens, 4 tokens and one
     token a workgroup as the context grows towards 2048 positions, and past that the single launch with its value tiles."""
