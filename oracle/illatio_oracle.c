@@ -22,13 +22,16 @@
  * attend-head! against explicit evaluations in numpy (with the plausible
  * misreadings shown to give other bits), forward-1 as those pieces in order.
  *
- * Parity unpinned (last-bit only): orc_silu / orc_softplus / orc_sigmoid use
- * (float)exp((double)x) and (float)log((double)x) as SBCL does for
- * single-float arguments (ds4f.lisp:248-254); they are checked against the
- * correctly rounded value, which SBCL's libm call yields except where the
- * double result falls within ~2^-29 of a single-precision rounding boundary;
- * orc_rope_table's cos and sin likewise.  Parity unpinned: orc_rmsnorm (no
- * vector of the reference's covers it; see its comment).
+ * No function here is unpinned.  Notes on three pins: orc_silu / orc_softplus /
+ * orc_sigmoid use (float)f((double)x) as SBCL does for single-float arguments
+ * (ds4f.lisp:248-254); they are checked against the correctly rounded value from
+ * an independent extended-precision evaluation, which SBCL's libm call yields
+ * except where the double result falls within ~2^-29 of a single-precision
+ * rounding boundary (no test input does).  orc_rope_table's cos and sin are the
+ * C library's double routines rounded to single, likewise; its theta sequence
+ * and roundings are pinned against numpy with each rounding explicit.
+ * orc_rmsnorm has no vector of the reference's: it is pinned by what its text
+ * fixes, on inputs where each misreading gives other bits (see its comment).
  */
 #include <float.h>
 #include <math.h>
@@ -559,8 +562,9 @@ static inline float sb_exp(float x) { return (float)exp((double)x); }
 static inline float sb_log(float x) { return (float)log((double)x); }
 /* rmsnorm! (model.lisp:205-216): the squares are single-float products, added one after
    another in double; scale = 1 / sqrt(float(sum/n + eps)); out = (x * scale) * w.
-   Parity unpinned: the reference holds no vector for it; tests pin it against what the
-   formula fixes (closed forms, the float-rounded squares, the order of the two products). */
+   The reference holds no vector for it; tests pin it against what the formula fixes (closed
+   forms, the float-rounded squares, the order of the two products), on inputs where each
+   misreading gives other bits. */
 void orc_rmsnorm(const float* x, const float* w, float* out, float eps, int64_t n) {
   double sum = 0.0;
   for (int64_t i = 0; i < n; i++) { volatile float sq = x[i] * x[i]; sum += (double)sq; }
