@@ -148,6 +148,10 @@ class DenseModel:
             dense.mv_multi(dev, [(self.output, self.logits, None)], xf=last, norm=(self.output_norm, eps))
         return self.logits
 
+    def reset(self):
+        """Forget the tokens seen: the next one is at position 0 (the caches' rows are overwritten as positions are reached)."""
+        self.pos = 0
+
     def eval_tokens(self, tokens, logits=True):
         """The prompt in chunks (CUDA-EVAL, cuda-dense.lisp:295-305); the logits of the last token only."""
         tokens = list(tokens)

@@ -110,6 +110,32 @@ def test_attn_step_is_qk_rope_then_attn_rows(dev, norms):
         hip.hip_free(b)
 
 
+def test_reused_context_is_a_fresh_one(dev):
+    """A context used for one sequence, reset and used for another gives the second the logits a fresh context gives
+    (the reference's consistency-test.lisp:52-61): nothing of the first sequence's caches or buffers shows."""
+    from illatio_amd import hip, model
+    host = model.synth_model(10, d=512, ffn=1024, nh=8, nkv=2, hd=64, nl=2, vocab=600)
+    rng = synth.make_rng(10)
+    first, second = rng.integers(0, 600, 50).tolist(), rng.integers(0, 600, 23).tolist()
+    gpu = model.DenseModel(dev, host, 64, chunk=16)
+    gpu.eval_tokens(first)
+    for _ in range(5):
+        gpu.forward_n([gpu.argmax()])
+    gpu.reset()
+    gpu.eval_tokens(second)
+    reused = hip.hip_floats(gpu.logits, 600).copy()
+    gpu.free()
+    fresh = model.DenseModel(dev, host, 64, chunk=16)
+    fresh.eval_tokens(second)
+    assert np.array_equal(bits(reused), bits(hip.hip_floats(fresh.logits, 600)))
+    cpu = orc.DenseModel(host, 64)
+    for t in second[:-1]:
+        cpu.forward(t, logits=False, nthreads=8)
+    want, _ = cpu.forward(second[-1], nthreads=8)
+    assert np.array_equal(bits(reused), bits(want))
+    fresh.free()
+
+
 def test_llama_style_decoder(dev):
     """No head norms, RoPE on adjacent pairs (2i, 2i + 1), heads of 96 (six partial sums of sixteen a score), one KV
     head for all query heads; then heads of 256, the widest the attention takes."""
