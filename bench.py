@@ -353,8 +353,15 @@ def workload_c1(args, dev):
                 t_cpu += time.perf_counter() - t1
                 nb += host[n].size
             reps += 1
+        def one(nt):
+            done = 0
+            for n, r, c in shapes:
+                orc.matmul(synth.Q8_0, host[n], r, c, xs[n], nthreads=nt)
+                done += host[n].size
+            return done
         return {"value": round(nb / t_cpu / 1e9, 3), "unit": "GB/s", "cores": cores, "kind": "port",
-                "sample": f"{reps} x both products (quantization included), {nb} weight bytes, {t_cpu:.1f} s"}
+                "sample": f"{reps} x both products (quantization included), {nb} weight bytes, {t_cpu:.1f} s",
+                "one_thread": {"value": round(one_thread_figure(one) / 1e9, 3), "unit": "GB/s", "sample": "both products, about 3 s"}}
 
     return {"value": round(gbs, 1), "unit": "GB/s", "ms_per_step": ms, "device_ms_per_step": dev_ms, "enqueue_ms": tm.enqueue_ms, "dtype": "int8 block dots, fp32 combine",
             "config": {"workload": "c1: Q8_0 decode GEMV 4864x896 and 896x4864 (Qwen2-0.5B MLP), batch 1, rotating over 64 copies",
@@ -438,8 +445,12 @@ def workload_c3(args, dev):
             orc.matmul(qt, w, rows, cols, x[:ts], nthreads=cores)
             reps += 1
         t_cpu = time.perf_counter() - t1
+        def one(nt):
+            orc.matmul(qt, w, rows, cols, x[:1], nthreads=nt)
+            return 2.0 * rows * cols
         return {"value": round(2.0 * rows * cols * ts * reps / t_cpu / 1e12, 4), "unit": "TFLOP/s", "cores": cores, "kind": "port",
-                "sample": f"{reps} x the same matrix on {ts} tokens (quantization included), {t_cpu:.1f} s"}
+                "sample": f"{reps} x the same matrix on {ts} tokens (quantization included), {t_cpu:.1f} s",
+                "one_thread": {"value": round(one_thread_figure(one) / 1e12, 5), "unit": "TFLOP/s", "sample": "the same matrix on one token, about 3 s"}}
 
     return {"value": round(tf, 1), "unit": "TFLOP/s", "ms_per_step": ms, "device_ms_per_step": dev_ms, "enqueue_ms": tm.enqueue_ms,
             "dtype": "bf16 x bf16, fp32 accumulate" if bf16_path else "int8 block dots, fp32 combine",
@@ -535,8 +546,14 @@ def workload_c4(args, dev):
             orc.moe_shared(sg, su, sd, d, ff, 0.0, x, nthreads=cores)
             reps += 1
         t_cpu = time.perf_counter() - t1
+        def one(nt):
+            sel, w = orc.route(synth.activations(ne, crng), nu, 1.5)
+            orc.moe_routed(gate, up, down, d, ff, sel, w, 0.0, x, nthreads=nt)
+            orc.moe_shared(sg, su, sd, d, ff, 0.0, x, nthreads=nt)
+            return step_bytes
         return {"value": round(step_bytes * reps / t_cpu / 1e9, 3), "unit": "GB/s", "cores": cores, "kind": "port",
-                "sample": f"{reps} decode steps (6 routed experts + shared expert), {t_cpu:.1f} s"}
+                "sample": f"{reps} decode steps (6 routed experts + shared expert), {t_cpu:.1f} s",
+                "one_thread": {"value": round(one_thread_figure(one) / 1e9, 3), "unit": "GB/s", "sample": "the same steps, about 3 s"}}
 
     return {"value": round(gbs, 1), "unit": "GB/s", "ms_per_step": ms, "device_ms_per_step": dev_ms, "enqueue_ms": tm.enqueue_ms, "dtype": "int8 block dots, fp32 combine",
             "metric": "MoE decode step achieved HBM GB/s (% of 8 TB/s)",
@@ -596,8 +613,12 @@ def workload_c5(args, dev):
             orc.moe_chunk(gate, up, down, d, ff, ne, nu, 1.5, 0.0, logits[:ts], norms[:ts], None, nthreads=cores)
             reps += 1
         t_cpu = time.perf_counter() - t1
+        def one(nt):
+            orc.moe_chunk(gate, up, down, d, ff, ne, nu, 1.5, 0.0, logits[:1], norms[:1], None, nthreads=nt)
+            return 2.0 * nu * 3 * ff * d
         return {"value": round(2.0 * ts * nu * 3 * ff * d * reps / t_cpu / 1e12, 4), "unit": "TFLOP/s", "cores": cores, "kind": "port",
-                "sample": f"{reps} chunks of {ts} tokens (48 rows each), {t_cpu:.1f} s"}
+                "sample": f"{reps} chunks of {ts} tokens (48 rows each), {t_cpu:.1f} s",
+                "one_thread": {"value": round(one_thread_figure(one) / 1e12, 5), "unit": "TFLOP/s", "sample": "one token's six experts, about 3 s"}}
 
     return {"value": round(tf, 1), "unit": "TFLOP/s", "ms_per_step": ms, "device_ms_per_step": dev_ms, "enqueue_ms": tm.enqueue_ms,
             "dtype": "bf16 x bf16, fp32 accumulate" if args.path == "bf16" else "int8 block dots, fp32 combine",
@@ -652,8 +673,12 @@ def workload_c2d(args, dev):
             t_tok = int(np.argmax(logits))
             n += 1
         t_cpu = time.perf_counter() - t1
+        t2 = time.perf_counter()
+        cm.forward(t_tok, nthreads=1)
+        one = 1.0 / (time.perf_counter() - t2)
         return {"value": round(n / t_cpu, 3), "unit": "tok/s", "cores": cores, "kind": "port",
-                "sample": f"{n} greedy tokens of the same model from an empty context (attention over at most {n + 1} positions), {t_cpu:.1f} s"}
+                "sample": f"{n} greedy tokens of the same model from an empty context (attention over at most {n + 1} positions), {t_cpu:.1f} s",
+                "one_thread": {"value": round(one, 3), "unit": "tok/s", "sample": "one more token on one thread"}}
 
     return {"value": round(ndecode / decode_s, 1), "unit": "tok/s", "ms_per_step": ms, "device_ms_per_step": ms, "enqueue_ms": 0.0,
             "dtype": "int8 block dots, fp32 combine; fp32 attention",
