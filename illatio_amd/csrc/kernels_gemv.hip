@@ -852,7 +852,8 @@ __device__ __forceinline__ int lds_block_bytes(int fmt) {
 // p.ptrs gives the experts' slots and p.nz how many take part: a batch is rows of one expert,
 // batches per expert = p.mat[0].nbat).  p.batch = the most rows a wave takes; p.region = bytes
 // of LDS per wave for its rows (both matrices' when glu).
-template <int FSET>
+// EARLY: the launch adds to y or has a bias (never a gate/up pair): those values are asked for behind the rows.
+template <int FSET, bool EARLY = false>
 __global__ __launch_bounds__(kStreamThreads) void gemv_stream_kernel(IltGemvParams p) {
   extern __shared__ __align__(16) unsigned char smem[];
   constexpr bool iq2 = FSET == ILT_IQ2_XXS, q8 = FSET == ILT_Q8_0;
@@ -947,13 +948,13 @@ __global__ __launch_bounds__(kStreamThreads) void gemv_stream_kernel(IltGemvPara
   // Q8_0: the scales' room behind the quants'
   const u8* scales = region + (long)p.batch * p.cols;
   const u8* scales_up = region_up + (long)p.batch * p.cols;
-  // What the sum is added to (acc) and the bias, asked for before the rows: they are there when the sums are, instead
-  // of a trip to memory after them.  No branch around the loads (a conditional load is waited for at the join): a
-  // launch without them reads y, whose value it does not use.
+  // What the sum is added to (acc) and the bias are asked for ahead of the rows: they are there when the sums are,
+  // instead of a trip to memory after them (asked for behind the rows they come in last and gain nothing).
   float* const ydst = m.y + (long)z * p.y_stride;
   const long rmine = row0 + min(lane, max(nrows - 1, 0));
   const float* const bsrc = m.bias ? m.bias : ydst;
-  const float yold = ydst[rmine], bval = bsrc[rmine];
+  float yold = 0.0f, bval = 0.0f;
+  if constexpr (EARLY) { yold = ydst[rmine]; bval = bsrc[rmine]; }
   int nup = 0;              // load instructions of the up matrix's rows: the last ones issued
   if (live) {
     with_format<FSET>(fmt, [&](auto F) { stream_run<decltype(F)::value>(wg, row0, nrows, S, m.row_bytes, region, lane); });
@@ -963,6 +964,8 @@ __global__ __launch_bounds__(kStreamThreads) void gemv_stream_kernel(IltGemvPara
       if (q8) nup += stream_scales((const u8*)(p.mat[1].wd + row0 * S), nrows * S * 2, (u8*)scales_up, lane);
     }
   }
+  // (no branch around the loads, which the compiler would wait out at the join: a launch that has neither runs the
+  // kernel built without them; one that has only one of them reads y twice)
   if (p.norm_w) { ilt_barrier_lds(); ilt_barrier_lds(); ilt_barrier_lds(); }      // in step with norm_scale_stagers
   // The barrier is for the activations only, so it comes before this wave waits for its rows (no
   // fence: the loads stay in flight): a wave whose rows land early starts on them while the
@@ -1004,8 +1007,8 @@ __global__ __launch_bounds__(kStreamThreads) void gemv_stream_kernel(IltGemvPara
         y[r] = o;
       }
     } else {
-      if (m.bias) v = v + bval;
-      if (p.acc) v = yold + v;
+      if (m.bias) v = v + (EARLY ? bval : m.bias[r]);
+      if (p.acc) v = (EARLY ? yold : y[r]) + v;
       y[r] = v;
     }
   }
@@ -1143,10 +1146,12 @@ static hipError_t gemv_stream_launch(IltGemvParams& p, int fset, int nz, hipStre
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 8) dev = 0;
   if (!attr_set[dev]) {            // more dynamic LDS than the default 64 KB: asked for once per device
-    const void* kernels[6] = { (const void*)gemv_stream_kernel<0>, (const void*)gemv_stream_kernel<ILT_Q4_K>, (const void*)gemv_stream_kernel<ILT_Q6_K>,
-                               (const void*)gemv_stream_kernel<ILT_IQ2_XXS>, (const void*)gemv_stream_kernel<ILT_Q2_K>,
-                               (const void*)gemv_stream_kernel<ILT_Q8_0> };
-    for (int i = 0; i < 6; i++)
+    const void* kernels[10] = { (const void*)gemv_stream_kernel<0>, (const void*)gemv_stream_kernel<ILT_Q4_K>, (const void*)gemv_stream_kernel<ILT_Q6_K>,
+                                (const void*)gemv_stream_kernel<ILT_IQ2_XXS>, (const void*)gemv_stream_kernel<ILT_Q2_K>,
+                                (const void*)gemv_stream_kernel<ILT_Q8_0>, (const void*)gemv_stream_kernel<0, true>,
+                                (const void*)gemv_stream_kernel<ILT_Q4_K, true>, (const void*)gemv_stream_kernel<ILT_Q6_K, true>,
+                                (const void*)gemv_stream_kernel<ILT_Q8_0, true> };
+    for (int i = 0; i < 10; i++)
       if (hipFuncSetAttribute(kernels[i], hipFuncAttributeMaxDynamicSharedMemorySize, 158 * 1024) != hipSuccess) {
         (void)hipGetLastError();
         return hipErrorNotSupported;
@@ -1154,6 +1159,19 @@ static hipError_t gemv_stream_launch(IltGemvParams& p, int fset, int nz, hipStre
     attr_set[dev] = true;
   }
   const dim3 grid(min(256, nb));                                      // wave w of workgroup g takes batch w * grid + g
+  bool early = p.acc != 0;
+  for (int i = 0; i < p.nmat; i++) early = early || p.mat[i].bias != nullptr;
+  early = early && !p.glu && !p.ptrs;
+  if (early) {
+    switch (fset) {
+      case 0: hipLaunchKernelGGL((gemv_stream_kernel<0, true>), grid, dim3(kStreamThreads), smem, st, p); break;
+      case ILT_Q4_K: hipLaunchKernelGGL((gemv_stream_kernel<ILT_Q4_K, true>), grid, dim3(kStreamThreads), smem, st, p); break;
+      case ILT_Q6_K: hipLaunchKernelGGL((gemv_stream_kernel<ILT_Q6_K, true>), grid, dim3(kStreamThreads), smem, st, p); break;
+      case ILT_Q8_0: hipLaunchKernelGGL((gemv_stream_kernel<ILT_Q8_0, true>), grid, dim3(kStreamThreads), smem, st, p); break;
+      default: early = false; break;
+    }
+    if (early) { g_streamed_launches++; return hipGetLastError(); }
+  }
   switch (fset) {
     case 0: hipLaunchKernelGGL(gemv_stream_kernel<0>, grid, dim3(kStreamThreads), smem, st, p); break;
     case ILT_Q4_K: hipLaunchKernelGGL(gemv_stream_kernel<ILT_Q4_K>, grid, dim3(kStreamThreads), smem, st, p); break;
