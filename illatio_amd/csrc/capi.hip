@@ -570,6 +570,32 @@ int ilt_mm_k(uint64_t stream, int type, const void* w, const int8_t* xq, const f
                             bsums, n, y, bias, acc, S(stream));
 }
 
+// Up to three K-quant matrices of one type on the same tokens (what mm_q8_mma2 is for Q8_0, cuda-dense.lisp:250-258):
+// one launch when the shapes allow it, else one after another; a matrix of no rows (or a null one) takes no part.
+int ilt_mm_k_n(uint64_t stream, int type, const void* w0, float* y0, const float* b0, int rows0, const void* w1, float* y1, const float* b1,
+               int rows1, const void* w2, float* y2, const float* b2, int rows2, const int8_t* xq, const float* xd, const int32_t* bsums,
+               int cols, int n, int acc) {
+  const int fmt = kquant_type(type);
+  ILT_REQUIRE(fmt && n >= 0 && cols > 0 && cols % 256 == 0 && rows0 >= 0 && rows1 >= 0 && rows2 >= 0);
+  const void* wsrc[3] = {w0, w1, w2}; float* ysrc[3] = {y0, y1, y2}; const float* bsrc[3] = {b0, b1, b2}; const int rsrc[3] = {rows0, rows1, rows2};
+  const uint8_t* ws[3]; float* ys[3]; const float* bs[3]; int rows[3], nm = 0;
+  for (int i = 0; i < 3; i++) {
+    if (rsrc[i] == 0 || !wsrc[i]) continue;
+    ILT_REQUIRE(ysrc[i] && ((uintptr_t)wsrc[i] & 15) == 0);
+    ws[nm] = (const uint8_t*)wsrc[i]; ys[nm] = ysrc[i]; bs[nm] = bsrc[i]; rows[nm] = rsrc[i]; nm++;
+  }
+  if (nm == 0 || n == 0) return ILT_OK;
+  ILT_REQUIRE(xq && xd && bsums && ((uintptr_t)xq & 15) == 0);
+  const long long row_bytes = (long long)cols / 256 * block_bytes(fmt);
+  const hipError_t e = ilt_k_gemm_i8_planes_n(fmt, nm, ws, rows, ys, bs, row_bytes, cols, xq, xd, bsums, n, acc, S(stream));
+  if (e != hipErrorNotSupported) return (int)e;
+  for (int i = 0; i < nm; i++) {
+    const int r = ilt_mm_k(stream, type, ws[i], xq, xd, bsums, ys[i], bs[i], rows[i], cols, n, acc);
+    if (r != ILT_OK) return r;
+  }
+  return ILT_OK;
+}
+
 static int mm_id(uint64_t stream, int fmt, int ncols, int nrows, int row_bytes, int64_t add, const uint64_t* ptrs,
                  const uint32_t* counts, const uint32_t* bases, int ne, int64_t total_rows, const int8_t* xq,
                  const float* xd, const int32_t* bsums, float* y) {
@@ -849,6 +875,10 @@ int ilt_launch(const char* kernel, unsigned gx, unsigned gy, unsigned gz, unsign
                           a.i32(14), a.ptr<ci8>(15), a.ptr<cf>(16), a.i32(17), a.i32(18), a.i32(19));
   K("d4_mvq8n") return ilt_d4_mvq8n(stream, a.i32(0), a.i32(1), a.i32(2), a.i32(3), a.i32(4), a.i32(5), a.ptr<ci8>(6), a.ptr<cu16>(7),
                                     a.ptr<ci8>(8), a.ptr<cf>(9), a.ptr<float*>(10));
+  K("mm_k_n")
+    return ilt_mm_k_n(stream, a.i32(0), a.ptr<const void*>(1), a.ptr<float*>(2), a.ptr<cf>(3), a.i32(4), a.ptr<const void*>(5), a.ptr<float*>(6),
+                      a.ptr<cf>(7), a.i32(8), a.ptr<const void*>(9), a.ptr<float*>(10), a.ptr<cf>(11), a.i32(12), a.ptr<ci8>(13), a.ptr<cf>(14),
+                      a.ptr<const int32_t*>(15), a.i32(16), a.i32(17), a.i32(18));
   K("mm_k") return ilt_mm_k(stream, a.i32(0), a.ptr<const void*>(1), a.ptr<ci8>(2), a.ptr<cf>(3), a.ptr<const int32_t*>(4),
                             a.ptr<float*>(5), a.ptr<cf>(6), a.i32(7), a.i32(8), a.i32(9), a.i32(10));
   if (!strcmp(kernel, "mm_q4k_mma") || !strcmp(kernel, "mm_q6k_mma"))

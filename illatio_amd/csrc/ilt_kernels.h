@@ -98,6 +98,9 @@ hipError_t ilt_k_gemm_i8(int fmt, const uint8_t* w, const uint16_t* wd, long lon
 // Q6_K, Q4_K and Q2_K, exact, on the pipelined kernel (kernels_gemm_bf16.hip): scale * quant as int8 planes
 hipError_t ilt_k_gemm_i8_planes(int fmt, const uint8_t* w, long long row_bytes, int rows, int cols, const int8_t* xq, const float* xd,
                                 const int* bsums, int ntok, float* y, const float* bias, int acc, hipStream_t st);
+hipError_t ilt_k_gemm_i8_planes_n(int fmt, int nmat, const uint8_t* const* ws, const int* rows, float* const* ys, const float* const* biases,
+                                  long long row_bytes, int cols, const int8_t* xq, const float* xd, const int* bsums, int ntok, int acc,
+                                  hipStream_t st);
 // The exact product in two passes (Q6_K): the two int8 planes and d per row and super-block once, then the product from them
 hipError_t ilt_k_planes_i8(int fmt, const uint8_t* w, long long row_bytes, int rows, int cols, uint8_t* wh, uint8_t* wl, float* wdf,
                            hipStream_t st);

@@ -199,6 +199,9 @@ struct BfParams {
   const u32* rmap;                           // grouped: row i of the groups is x's row rmap[i] (null: row i)
   float* y; const float* bias; int acc; int ntok;
   long long ldy;                             // floats from a token's results to the next token's in y (rows, unless p covers a part of the rows)
+  // several matrices of one format on the same tokens in one launch (gemm_i8p_kernel, dense): matrix m's row tiles follow
+  // matrix m-1's; rows = the tiles of all of them together times 128 until the workgroup has found its matrix
+  int nmulti; const u8* mw[3]; int mrows[3]; float* my[3]; const float* mbias[3];
   // the grouped gate and up products with the gated activation (gemm_bf16_regb_kernel<FMT, true>): rows = the width of
   // each; up's matrix at ptrs[z] + add + up_delta; mid[i][r] = bf16((silu(gate) * up) * wrow[i]), clamped as d4_swiglu_w does
   unsigned up_delta; const float* wrow; float clamp; u16* mid;
@@ -1015,6 +1018,18 @@ __global__ __launch_bounds__(512, 1) void gemm_i8p_kernel(BfParams p) {
 
   long tok0; int ntok, rt; const u8* w = p.w;
   if (!pick_tile<TM, TN>(p, S, tok0, ntok, rt, w)) return;
+  if constexpr (!GROUPED) {
+    if (p.nmulti > 1) {                                      // which of the launch's matrices the row tile belongs to
+      const int n0 = (p.mrows[0] + TM - 1) / TM, n1 = n0 + (p.mrows[1] + TM - 1) / TM;
+      const int m = rt < n0 ? 0 : rt < n1 ? 1 : 2;
+      rt -= m == 0 ? 0 : m == 1 ? n0 : n1;
+      w = m == 0 ? p.mw[0] : m == 1 ? p.mw[1] : p.mw[2];
+      p.rows = m == 0 ? p.mrows[0] : m == 1 ? p.mrows[1] : p.mrows[2];
+      p.y = m == 0 ? p.my[0] : m == 1 ? p.my[1] : p.my[2];
+      p.bias = m == 0 ? p.mbias[0] : m == 1 ? p.mbias[1] : p.mbias[2];
+      p.ldy = p.rows;
+    }
+  }
   const int r0 = rt * TM;
   int* const cxo = (int*)S.wdm;                              // IQ2_XXS: cx for the even groups, this for the odd ones
   if constexpr (FMT == ILT_IQ2_XXS) {
@@ -1891,6 +1906,27 @@ hipError_t ilt_k_gemm_i8_planes(int fmt, const uint8_t* w, long long row_bytes, 
   BfParams p = {};
   p.w = w; p.rows = rows; p.cols = cols; p.row_bytes = row_bytes; p.x = (const u16*)xq; p.xd = xd; p.bsums = bsums;
   p.y = y; p.bias = bias; p.acc = acc; p.ntok = ntok; p.ldy = rows;
+  return launch_i8p<false>(fmt, p, (ntok + 127) / 128, st);
+}
+
+// Up to three matrices of one format (Q6_K, Q4_K, Q2_K) on the same tokens in one launch: their row tiles one after
+// another, so that matrices too small to fill the chip on their own share it (Q/K/V, gate and up of a prompt's chunk).
+// hipErrorNotSupported: the caller launches them one by one.
+hipError_t ilt_k_gemm_i8_planes_n(int fmt, int nmat, const uint8_t* const* ws, const int* rows, float* const* ys, const float* const* biases,
+                                  long long row_bytes, int cols, const int8_t* xq, const float* xd, const int* bsums, int ntok, int acc,
+                                  hipStream_t st) {
+  if (nmat < 2 || nmat > 3 || ntok < 96 || (fmt != ILT_Q6_K && fmt != ILT_Q4_K && fmt != ILT_Q2_K) || cols % 256 != 0) return hipErrorNotSupported;
+  BfParams p = {};
+  long long tiles = 0;
+  for (int m = 0; m < nmat; m++) {
+    if (rows[m] < 128 || rows[m] >= (1 << 21) || (long long)rows[m] * row_bytes >= 0x7FFFFFFFLL) return hipErrorNotSupported;
+    p.mw[m] = ws[m]; p.mrows[m] = rows[m]; p.my[m] = ys[m]; p.mbias[m] = biases ? biases[m] : nullptr;
+    tiles += (rows[m] + 127) / 128;
+  }
+  if (tiles * 128 >= (1 << 21)) return hipErrorNotSupported;
+  p.nmulti = nmat;
+  p.w = ws[0]; p.rows = (int)(tiles * 128); p.cols = cols; p.row_bytes = row_bytes; p.x = (const u16*)xq; p.xd = xd; p.bsums = bsums;
+  p.y = ys[0]; p.acc = acc; p.ntok = ntok; p.ldy = rows[0];
   return launch_i8p<false>(fmt, p, (ntok + 127) / 128, st);
 }
 

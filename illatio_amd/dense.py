@@ -130,6 +130,26 @@ def cmat_mul(dev, w, act, y, n=1, bias=None, acc=False):
     return y
 
 
+def cmat_mul_n(dev, parts, act, n, acc=False):
+    """PARTS, (W Y BIAS) sharing X, for N tokens (CMAT-MUL-N, cuda-dense.lisp:250-258): the K-quant matrices of one
+    type, up to three at a time, in one launch of mm_k_n; whatever is left one by one."""
+    todo = list(parts)
+    while todo:
+        w0 = todo[0][0]
+        same = [pt for pt in todo if pt[0].kquant_p() and pt[0].type == w0.type and pt[0].cols == w0.cols][:3] if w0.kquant_p() and n > 1 else []
+        if len(same) >= 2:
+            args = [KQUANT_CODE[w0.type]]
+            for k in range(3):
+                w, y, bias = same[k] if k < len(same) else (None, None, None)
+                args += [w.qs if w else None, y, bias, w.rows if w else 0]
+            hip.launch(dev, "mm_k_n", ((n + 127) // 128, sum((w.rows + 127) // 128 for w, _, _ in same)), 512,
+                       args + [act.kq, act.kd, act.ksum, w0.cols, n, 1 if acc else 0])
+            todo = [pt for pt in todo if not any(pt is q for q in same)]
+        else:
+            w, y, bias = todo.pop(0)
+            cmat_mul(dev, w, act, y, n=n, bias=bias, acc=acc)
+
+
 def cvt_bf16(dev, x, n_elems, out=None):
     """N_ELEMS floats of X (a DBuf) rounded to bf16, into OUT or a new DBuf: the bf16
     product's counterpart of QUANTIZE-ACT!."""

@@ -119,8 +119,7 @@ class DenseModel:
                 dense.qkv_mul(dev, L["wq"], L["wk"], L["wv"], None, self.q, self.k, self.v, xf=self.x, norm=(L["attn_norm"], eps))
             else:
                 a = dense.rmsnorm_q8(dev, self.x, L["attn_norm"], self.acts[d], d, eps, n=n)
-                for w, y in ((L["wq"], self.q), (L["wk"], self.k), (L["wv"], self.v)):
-                    dense.cmat_mul(dev, w, a, y, n=n)
+                dense.cmat_mul_n(dev, [(L["wq"], self.q, None), (L["wk"], self.k, None), (L["wv"], self.v, None)], a, n)
             if n == 1 and self.scores is not None:
                 hip.call("ilt_attn_step", S, P(self.q), P(self.k), P(self.v), P(L["q_norm"]), P(L["k_norm"]), P(self.rope), P(L["kc"]), P(L["vc"]),
                          P(self.att), C.c_int(nh), C.c_int(nkv), C.c_int(hd), C.c_int(hd), C.c_int(self.pos), C.c_float(eps),
@@ -138,8 +137,7 @@ class DenseModel:
             else:
                 dense.cmat_mul(dev, L["wo"], dense.quantize_act(dev, self.att, self.acts[self.qd], n=n), self.x, n=n, acc=True)
                 a = dense.rmsnorm_q8(dev, self.x, L["ffn_norm"], self.acts[d], d, eps, n=n)
-                dense.cmat_mul(dev, L["gate"], a, self.fa, n=n)
-                dense.cmat_mul(dev, L["up"], a, self.fb, n=n)
+                dense.cmat_mul_n(dev, [(L["gate"], self.fa, None), (L["up"], self.fb, None)], a, n)
                 hip.call("ilt_swiglu", S, P(self.fa), P(self.fb), C.c_int64(n * ffn))
                 dense.cmat_mul(dev, L["down"], dense.quantize_act(dev, self.fa, self.acts[ffn], n=n), self.x, n=n, acc=True)
         self.pos += n

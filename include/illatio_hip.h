@@ -352,6 +352,14 @@ int ilt_mm_q8(uint64_t stream, const int8_t* wq, const uint16_t* wd, const int8_
               const float* bias, int rows, int cols, int n, int acc);
 int ilt_mm_k(uint64_t stream, int type, const void* w, const int8_t* xq, const float* xd, const int32_t* bsums, float* y,
              const float* bias, int rows, int cols, int n, int acc);
+/* Up to three K-quant matrices of one type on the same tokens in one launch -- for Q4_K / Q6_K what mm_q8_mma2 is
+   for Q8_0 (cuda-dense.lisp:250-258: cmat-mul-n; same argument pattern: (w, y, bias, rows) three times, then the
+   activations): the row tiles of matrices too small to fill the chip on their own share a launch (Q/K/V, gate and
+   up of a prompt's chunk).  type: the reference's kquant code (0 Q4_K, 2 Q6_K).  A matrix of no rows or a null one
+   takes no part.  The results are ilt_mm_k's, bit for bit. */
+int ilt_mm_k_n(uint64_t stream, int type, const void* w0, float* y0, const float* b0, int rows0, const void* w1, float* y1, const float* b1,
+               int rows1, const void* w2, float* y2, const float* b2, int rows2, const int8_t* xq, const float* xd, const int32_t* bsums,
+               int cols, int n, int acc);
 /* d4_mm_<format> (ds4f_mm.cu:252-255; dk-mm, cuda-ds4f-prefill.lisp:65-68): one matrix on a chunk of
    ntok tokens' FLOAT activations, y[t*y_stride + r] = W[r] . x[t*x_stride ..].  The reference's kernels
    round weights and activations to halves; these give the CPU path's results:

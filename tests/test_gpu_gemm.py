@@ -147,6 +147,55 @@ def test_mm_q8_mma2_three_matrices_on_the_same_tokens(dev):
         m.free()
 
 
+@pytest.mark.parametrize("qtype,n", [(synth.Q4_K, 200), (synth.Q6_K, 130), (synth.Q4_K, 40)])
+def test_mm_k_n_matrices_on_the_same_tokens(dev, qtype, n):
+    """mm_k_n: up to three K-quant matrices of one type on the same tokens, their row tiles in one launch (ragged row
+    counts, one with a bias, the middle one absent, accumulation) -- each with the CPU matmul!'s bits, which are
+    mm_k's; 40 tokens: too few for the shared launch, the call falls back on one product after another."""
+    from illatio_amd import dense, hip
+    rng = synth.make_rng(616 + n)
+    cols = 512
+    shape = [300, 128, 520]
+    ws = [synth.weights(qtype, r, cols, rng) for r in shape]
+    ms = [dense.upload_gmat(dev, f"w{i}", qtype, r, cols, w) for i, (r, w) in enumerate(zip(shape, ws))]
+    x = synth.activations((n, cols), rng)
+    xb = hip.hip_upload_new(dev, x)
+    act = dense.QAct(dev, n, cols, ("q8k",))
+    dense.quantize_act(dev, xb, act, n=n)
+    bias = synth.activations(shape[2], rng)
+    bb = hip.hip_upload_new(dev, bias)
+    ys = [hip.hip_alloc(dev, 4 * n * r) for r in shape]
+    code = dense.KQUANT_CODE[qtype]
+    grid = ((n + 127) // 128, sum((r + 127) // 128 for r in shape))
+    tail = [act.kq, act.kd, act.ksum, cols, n]
+    hip.launch(dev, "mm_k_n", grid, 512, [code, ms[0].qs, ys[0], None, shape[0], ms[1].qs, ys[1], None, shape[1],
+                                          ms[2].qs, ys[2], bb, shape[2]] + tail + [0])
+    plain = [orc.matmul(qtype, w, r, cols, x, nthreads=8).reshape(n, r) for w, r in zip(ws, shape)]
+    want = [plain[0], plain[1], plain[2] + bias]
+    for i, r in enumerate(shape):
+        assert np.array_equal(bits(hip.hip_floats(ys[i], n * r)), bits(want[i].reshape(-1))), i
+    # the middle matrix absent, the others accumulated onto what is there
+    hip.launch(dev, "mm_k_n", grid, 512, [code, ms[0].qs, ys[0], None, shape[0], None, None, None, 0,
+                                          ms[2].qs, ys[2], None, shape[2]] + tail + [1])
+    assert np.array_equal(bits(hip.hip_floats(ys[0], n * shape[0])), bits((want[0] + plain[0]).reshape(-1)))
+    assert np.array_equal(bits(hip.hip_floats(ys[1], n * shape[1])), bits(want[1].reshape(-1)))
+    assert np.array_equal(bits(hip.hip_floats(ys[2], n * shape[2])), bits((want[2] + plain[2]).reshape(-1)))
+    # the host's grouping: matrices of another type or width go on their own
+    otype = synth.Q6_K if qtype == synth.Q4_K else synth.Q4_K
+    ow = synth.weights(otype, 256, cols, rng)
+    other = dense.upload_gmat(dev, "o", otype, 256, cols, ow)
+    yo = hip.hip_alloc(dev, 4 * n * 256)
+    dense.cmat_mul_n(dev, [(ms[0], ys[0], None), (other, yo, None), (ms[1], ys[1], None), (ms[2], ys[2], bb)], act, n)
+    for i, r in enumerate(shape):
+        assert np.array_equal(bits(hip.hip_floats(ys[i], n * r)), bits(want[i].reshape(-1))), i
+    assert np.array_equal(bits(hip.hip_floats(yo, n * 256)), bits(orc.matmul(otype, ow, 256, cols, x, nthreads=8).reshape(-1)))
+    for b in [xb, bb, yo] + ys:
+        hip.hip_free(b)
+    act.free()
+    for m in ms + [other]:
+        m.free()
+
+
 def test_products_of_no_tokens_write_nothing(dev):
     """No tokens (an empty chunk): every prefill product returns without touching y."""
     from illatio_amd import dense, hip
