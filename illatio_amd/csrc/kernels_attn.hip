@@ -335,7 +335,21 @@ __device__ __forceinline__ void attn_softmax(const float* __restrict__ rw, const
 // slice with the positions along a row, vt[c * vpitch + p] (vpitch = 4 mod 64: sixteen threads' 16-byte reads
 // of sixteen rows fall on different banks).  NB: the slice is at most NB * 2048 16-byte pieces (512 NB positions).
 // With one token a workgroup the slice is stored times that token's scores, by all threads, and the chains add.
-template <int TG, int NB>
+// A prompt chunk's softmax, once a (head, token) instead of once in each of the head's hd/16 workgroups of
+// attn_values_kernel (the exps go through double: eight times over they were most of that kernel): the raw scores of
+// row (t, h) become the scaled scores, in place.
+__global__ __launch_bounds__(256) void attn_softmax_kernel(float* __restrict__ raw, int nh, int pos0, int spitch) {
+  extern __shared__ __align__(16) float dyn[];
+  __shared__ float redf[4];
+  __shared__ double redd[8];
+  const int h = blockIdx.x, t = blockIdx.y, npos = pos0 + t + 1;
+  float* rw = raw + ((long long)t * nh + h) * spitch;
+  attn_softmax<256, false>(rw, nullptr, dyn, npos, threadIdx.x, redf, redd);
+  for (int p = threadIdx.x; p < npos; p += 256) rw[p] = dyn[p];       // (each thread the entries it scaled itself)
+}
+
+// PROB: raw holds the scaled scores already (attn_softmax_kernel ran).
+template <int TG, int NB, bool PROB = false>
 __global__ __launch_bounds__(256) void attn_values_kernel(const float* __restrict__ raw, const float* __restrict__ vc, float* __restrict__ out,
                                                           int nh, int nkv, int hd, int pos0, int ntok, int spitch, int vpitch) {
   extern __shared__ __align__(16) float dyn[];
@@ -366,6 +380,11 @@ __global__ __launch_bounds__(256) void attn_values_kernel(const float* __restric
     for (int u = 2 * NB; u < 8; u++) pre[u] = 0.0f;
     attn_softmax<256, true>(nullptr, pre, scores, nposmax, tid, redf, redd);
     __syncthreads();                               // every thread's scaled scores, for the products below
+  } else if (PROB) {
+    for (int tt = 0; tt < tn; tt++) {
+      const float* rw = raw + ((long long)(t0 + tt) * nh + h) * spitch;
+      for (int p = tid; p < pos0 + t0 + tt + 1; p += 256) scores[tt * spitch + p] = rw[p];
+    }
   } else {
     for (int tt = wave; tt < tn; tt += 4)
       attn_softmax<64, false>(raw + ((long long)(t0 + tt) * nh + h) * spitch, nullptr, scores + tt * spitch, pos0 + t0 + tt + 1, lane, redf, redd);
@@ -455,11 +474,14 @@ hipError_t ilt_k_attn_rows(const float* q, const float* kc, const float* vc, flo
   if (tg == TG && nb == NB) {                                                                                                                  \
     static bool set[64] = {};                                                                                                                  \
     e = set[dev] ? hipSuccess                                                                                                                  \
-                 : hipFuncSetAttribute((const void*)attn_values_kernel<TG, NB>, hipFuncAttributeMaxDynamicSharedMemorySize, 152 * 1024);       \
+                 : hipFuncSetAttribute((const void*)attn_values_kernel<TG, NB, (TG > 1)>, hipFuncAttributeMaxDynamicSharedMemorySize,          \
+                                       152 * 1024);                                                                                            \
     if (e == hipSuccess) {                                                                                                                     \
       set[dev] = true;                                                                                                                         \
       hipLaunchKernelGGL(attn_scores_kernel<TG>, gs, dim3(1024), 0, st, q, kc, scratch, nh, nkv, hd, pos0, ntok, scale, smax);                 \
-      hipLaunchKernelGGL((attn_values_kernel<TG, NB>), gv, dim3(256), bytes(TG), st, scratch, vc, out, nh, nkv, hd, pos0, ntok, smax, vpitch); \
+      if (TG > 1) hipLaunchKernelGGL(attn_softmax_kernel, dim3(nh, ntok), dim3(256), sizeof(float) * smax, st, scratch, nh, pos0, smax);        \
+      hipLaunchKernelGGL((attn_values_kernel<TG, NB, (TG > 1)>), gv, dim3(256), bytes(TG), st, scratch, vc, out, nh, nkv, hd, pos0, ntok,      \
+                         smax, vpitch);                                                                                                        \
       e = hipGetLastError();                                                                                                                   \
     }                                                                                                                                          \
   }
