@@ -224,6 +224,7 @@ __global__ __launch_bounds__(1024) void attn_scores_kernel(const float* __restri
 #pragma unroll
     for (int u = 0; u < 4; u++) {
       const int p = pbase + 64 * u + pg;
+      if (pbase + 64 * u >= npos) continue;        // none of the pass's 64 positions is the token's to see (the same in every thread)
       float sacc = 0.0f;
 #pragma unroll
       for (int j = 0; j < 16; j++) if (j < nj) sacc = sacc + kv[u][j] * qv[j];
@@ -359,7 +360,10 @@ __global__ __launch_bounds__(256) void attn_values_kernel(const float* __restric
   const int tn = min(TG, ntok - t0), nposmax = pos0 + t0 + tn;
   const int group = nh / nkv, kvd = nkv * hd, ko = (h / group) * hd + 16 * cs;
   float* scores = dyn;
-  float* vt = dyn + TG * spitch;
+  // a token's scores 4 floats further on in LDS than a multiple of 64: the 16-byte reads of a wave's four tokens fall on
+  // different banks (at a multiple they all want the same four)
+  const int lp = TG > 1 ? spitch + 4 : spitch;
+  float* vt = dyn + TG * lp;
   // every load is asked for before anything waits, the scores first: no branch around a load, so that the
   // softmax waits for the scores alone and the value slice arrives meanwhile
   float pre[8];
@@ -381,13 +385,27 @@ __global__ __launch_bounds__(256) void attn_values_kernel(const float* __restric
     attn_softmax<256, true>(nullptr, pre, scores, nposmax, tid, redf, redd);
     __syncthreads();                               // every thread's scaled scores, for the products below
   } else if (PROB) {
-    for (int tt = 0; tt < tn; tt++) {
-      const float* rw = raw + ((long long)(t0 + tt) * nh + h) * spitch;
-      for (int p = tid; p < pos0 + t0 + tt + 1; p += 256) scores[tt * spitch + p] = rw[p];
+    // the group's rows of scaled scores, 16 bytes a thread, eight loads in flight before the first is stored (a load
+    // and its store one pair after another would be a trip to memory each); what lies past a token's own positions in
+    // its row is carried along and never read
+    const int q4 = spitch >> 2, totalq = tn * q4;
+    const float* rbase = raw + ((long long)t0 * nh + h) * spitch;
+    for (int base = 0; base < totalq; base += 256 * 8) {
+      float4 tmp[8];
+#pragma unroll
+      for (int u = 0; u < 8; u++) {
+        const int i = min(base + tid + 256 * u, totalq - 1), tt = i / q4, j = i - tt * q4;
+        tmp[u] = *(const float4*)(rbase + (long long)tt * nh * spitch + 4 * j);
+      }
+#pragma unroll
+      for (int u = 0; u < 8; u++) {
+        const int i = base + tid + 256 * u, tt = i / q4, j = i - tt * q4;
+        if (i < totalq) *(float4*)(scores + tt * lp + 4 * j) = tmp[u];
+      }
     }
   } else {
     for (int tt = wave; tt < tn; tt += 4)
-      attn_softmax<64, false>(raw + ((long long)(t0 + tt) * nh + h) * spitch, nullptr, scores + tt * spitch, pos0 + t0 + tt + 1, lane, redf, redd);
+      attn_softmax<64, false>(raw + ((long long)(t0 + tt) * nh + h) * spitch, nullptr, scores + tt * lp, pos0 + t0 + tt + 1, lane, redf, redd);
   }
 #pragma unroll
   for (int u = 0; u < 8 * NB; u++) {
@@ -405,7 +423,7 @@ __global__ __launch_bounds__(256) void attn_values_kernel(const float* __restric
   __syncthreads();                                 // the scores are scaled, the slice is in place
   if (tid < tn * 16) {
     const int tt = tid >> 4, c = tid & 15, npos = pos0 + t0 + tt + 1;
-    const float* sc = scores + tt * spitch;
+    const float* sc = scores + tt * lp;
     const float* col = vt + c * vpitch;
     float o = 0.0f;
     int p = 0;
@@ -465,7 +483,7 @@ hipError_t ilt_k_attn_rows(const float* q, const float* kc, const float* vc, flo
   if (scratch && pos0 + ntok <= 2048) {
     const int ctx = pos0 + ntok, vpitch = ((ctx + 63) & ~63) + 4;
     // tokens a workgroup: as many as leave their scores and the value slice room in LDS (150 KB)
-    auto bytes = [&](int tg) { return sizeof(float) * ((size_t)tg * smax + 16 * (size_t)vpitch); };
+    auto bytes = [&](int tg) { return sizeof(float) * ((size_t)tg * (smax + (tg > 1 ? 4 : 0)) + 16 * (size_t)vpitch); };
     const int tg = ntok == 1 ? 1 : bytes(16) <= 150 * 1024 ? 16 : bytes(4) <= 150 * 1024 ? 4 : 1;
     const int nb = (ctx + 511) / 512;
     const dim3 gs(nh, (ctx + 255) / 256, (ntok + tg - 1) / tg), gv(nh * (hd / 16), (ntok + tg - 1) / tg);
