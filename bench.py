@@ -747,10 +747,10 @@ def main():
         import copy
         import gc
         out["configs"] = {}
-        extras = [("c2_decode", {}), ("c1", {}), ("c3", {"path": "bf16", "tokens": 4096}), ("c3_t2048", {"path": "bf16", "tokens": 2048}),
+        extras = [("c2_decode", {}), ("c1", {"steps": 200, "warmup": 20}), ("c3", {"path": "bf16", "tokens": 4096}), ("c3_t2048", {"path": "bf16", "tokens": 2048}),
                   ("c3_t512", {"path": "bf16", "tokens": 512}), ("c3_resident", {"path": "bf16-resident", "tokens": 4096}),
                   ("c3_exact", {"path": "int8", "tokens": 4096}),
-                  ("c4", {"mode": "device"}), ("c5", {"path": "bf16", "tokens": 4096}), ("c5_exact", {"path": "int8", "tokens": 4096})]
+                  ("c4", {"mode": "device", "steps": 50, "warmup": 5}), ("c5", {"path": "bf16", "tokens": 4096}), ("c5_exact", {"path": "int8", "tokens": 4096})]
         for name, over in extras:
             a = copy.copy(args)
             a.workload, a.steps, a.warmup = ("c2d" if name == "c2_decode" else name[:2]), min(args.steps, 10), min(args.warmup, 3)
