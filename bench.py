@@ -2,7 +2,7 @@
 """bench.py -- the quantized matrix-product path on one MI355X.
 
 The default workload (c2) is the one the metric is quoted on: a step is one decoded token's
-worth of quantized products at the Qwen3-4B shape (BASELINE.json configs[1]) -- for each of
+worth of quantized products at the Qwen3-4B shape (the benchmark's configuration 2) -- for each of
 36 layers the activation quantizations (inside the product kernels) and the seven matrix-vector products (Q4_K wq
 4096x2560, wk 1024x2560, wo 2560x4096, gate and up 9728x2560; Q6_K wv 1024x2560, down
 2560x9728), then the Q6_K output head 151936x2560: 2,618,273,280 bytes of GGUF blocks
@@ -15,7 +15,7 @@ and are reported under "configs" (c2_decode, c1, c3 and c5 on the bf16 matrix co
 int8 path, c4 with the routing on the device); c2_decode's figures are also the line's
 decode_tok_per_s, decode_ms_per_token and prefill_tok_per_s.
 
-Other workloads (--workload), each BASELINE.json's config of the same number:
+Other workloads (--workload), each the benchmark configuration of the same number:
   c2d the whole dense decoder at config 2's shape (36 layers, head norms, RoPE, attention over an
       fp32 KV cache): a 512-token prompt through the prefill products, then 256 greedy tokens,
       every token's logits downloaded and the next token picked on the host
@@ -373,7 +373,7 @@ def workload_c3(args, dev):
     from illatio_amd import dense, hip, synth
     rng = synth.make_rng(33)
     rows, cols, T = (17408, 5120, args.tokens) if not args.transpose else (5120, 17408, args.tokens)
-    # BASELINE's config 3 is Q6_K; --qtype: the same shape in the other dense formats (q8_0: the exact path only)
+    # the benchmark's configuration 3 is Q6_K; --qtype: the same shape in the other dense formats (q8_0: the exact path only)
     qt = {"q4_k": synth.Q4_K, "q6_k": synth.Q6_K, "q8_0": synth.Q8_0}[args.qtype]
     if qt == synth.Q8_0 and args.path != "int8":
         raise SystemExit("bench.py: --qtype q8_0 goes with --path int8 (the bf16 product multiplies the K-quants)")
@@ -709,7 +709,7 @@ def main():
     ap.add_argument("--layers", type=int, default=LAYERS, help=argparse.SUPPRESS)
     ap.add_argument("--tokens", type=int, default=4096, help="c3, c5: tokens per step")
     ap.add_argument("--transpose", action="store_true", help="c3: the 5120x17408 matrix")
-    ap.add_argument("--qtype", default="q6_k", choices=["q6_k", "q4_k", "q8_0"], help="c3: the matrix's format (BASELINE: q6_k)")
+    ap.add_argument("--qtype", default="q6_k", choices=["q6_k", "q4_k", "q8_0"], help="c3: the matrix's format (the benchmark's: q6_k)")
     ap.add_argument("--path", default="bf16", choices=["bf16", "bf16-1pass", "bf16-2pass", "bf16-resident", "int8", "int8-2pass", "int8-resident"],
                     help="c3, c5: which matrix-core path.  c3: bf16 = 2pass from 1024 tokens on, else 1pass; bf16-1pass = the matrix dequantized inside the product's loop; "
                          "bf16-2pass = the matrix dequantized to a bf16 copy inside the step, then the plain bf16 product; bf16-resident = that copy made beforehand and kept")
@@ -741,7 +741,7 @@ def main():
     out["roofline"] = r["roofline"]
     out["cpu_baseline"] = None if args.no_cpu else r["cpu"]()
     if everything:
-        # BASELINE's other configurations on the same clock (no CPU leg): c4 with the routing on the device, c3 and
+        # the benchmark's other configurations on the same clock (no CPU leg): c4 with the routing on the device, c3 and
         # c5 on the bf16 matrix cores at 4096 tokens and, as a second entry each, on the bit-exact int8 path; c3 also at
         # its other two token counts and with the matrix's bf16 copy made once and kept (2 bytes a weight of the 288 GB)
         import copy

@@ -22,12 +22,12 @@ def bits(a):
 
 
 CASES = [
-    (synth.Q8_0, 4864, 896, 70),        # BASELINE config 1's matrices, a ragged token count
+    (synth.Q8_0, 4864, 896, 70),        # the benchmark's config 1's matrices, a ragged token count
     (synth.Q8_0, 896, 4864, 5),
     (synth.Q8_0, 100, 64, 129),         # rows and columns that fill no tile
     (synth.Q4_K, 1024, 2560, 64),
     (synth.Q4_K, 200, 512, 3),
-    (synth.Q6_K, 640, 5120, 96),        # BASELINE config 3's format and width, fewer rows
+    (synth.Q6_K, 640, 5120, 96),        # the benchmark's config 3's format and width, fewer rows
     (synth.Q6_K, 65, 256, 65),
     (synth.Q6_K, 300, 1024, 333),       # three row tiles and three token tiles of 128, the last of each ragged
     (synth.Q6_K, 256, 768, 128),        # an odd number of super-blocks
@@ -227,7 +227,7 @@ def test_products_of_no_tokens_write_nothing(dev):
                                                  (12, 4096, 2048, 6, 96, 0.0)])
 @pytest.mark.parametrize("planes", [None, "0", "1"])        # the down product (Q2_K) on the 64 x 64 kernel / on the planes kernel
 def test_moe_prefill_chunk_bit_exact(dev, monkeypatch, ne, d, ff, nu, n, clamp, planes):
-    """BASELINE config 5's sequence (route -> group -> gather -> grouped gate, up -> gated
+    """the benchmark's config 5's sequence (route -> group -> gather -> grouped gate, up -> gated
     activation -> grouped down -> slot-ordered sum + shared) at reduced expert and token
     counts, Zipf-skewed routing, against the CPU path's chunk (ds4f.lisp:1169-1239)."""
     from illatio_amd import ds4f, hip

@@ -65,7 +65,7 @@ def test_one_hot_tokens_read_back_the_dequantized_matrix(dev, monkeypatch, qtype
 
 
 @pytest.mark.parametrize("qtype,rows,cols,n", [
-    (synth.Q6_K, 640, 5120, 200),        # BASELINE config 3's format and width, fewer rows, ragged tokens
+    (synth.Q6_K, 640, 5120, 200),        # the benchmark's config 3's format and width, fewer rows, ragged tokens
     (synth.Q6_K, 1000, 1024, 128),
     (synth.Q4_K, 1024, 2560, 77),
     (synth.Q2_K, 300, 2048, 129),
