@@ -1,4 +1,4 @@
-"""Seeded synthetic GGUF-layout weights and activations for the BASELINE configs.
+"""Seeded synthetic GGUF-layout weights and activations for the benchmark configurations.
 
 Nothing here reads a model file: every block is built from a counter-based
 generator (numpy's Philox) in the GGUF byte order the kernels read

@@ -107,7 +107,7 @@ def test_dequant_rows_bit_exact(dev, qtype):
 
 
 DENSE_SHAPES = {
-    synth.Q8_0: [(4864, 896), (896, 4864), (36, 64), (1, 32)],       # BASELINE config 1, then ragged
+    synth.Q8_0: [(4864, 896), (896, 4864), (36, 64), (1, 32)],       # the benchmark's config 1, then ragged
     synth.Q4_K: [(4096, 2560), (2560, 4096), (1024, 2560), (100, 9728), (3, 256)],
     synth.Q6_K: [(1024, 2560), (2560, 9728), (64, 5120), (37, 512)],
 }
