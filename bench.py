@@ -18,7 +18,8 @@ decode_tok_per_s, decode_ms_per_token and prefill_tok_per_s.
 Other workloads (--workload), each the benchmark configuration of the same number:
   c2d the whole dense decoder at config 2's shape (36 layers, head norms, RoPE, attention over an
       fp32 KV cache): a 512-token prompt through the prefill products, then 256 greedy tokens,
-      every token's logits downloaded and the next token picked on the host
+      each picked on the device and fed on from device memory (--host-argmax: every token's
+      logits downloaded and the next token picked on the host)
   c1  Q8_0 decode GEMV 4864x896 and 896x4864, rotating over 64 copies (593 MB)
   c3  Q6_K prefill product 17408x5120 on T tokens (--tokens, default 4096): bf16 matrix
       cores (--path bf16, the float activations rounded to bf16 inside the step) or the
@@ -631,8 +632,9 @@ def workload_c5(args, dev):
 def workload_c2d(args, dev):
     """Config 2 as it is stated: the whole dense decoder at the Qwen3-4B shape (36 layers, head norms, RoPE,
     grouped-query attention over an fp32 KV cache, Q4_K / Q6_K weights), random-init: a 512-token prompt through the
-    prefill products, then a 256-token greedy decode at batch 1.  A step is one decoded token, logits downloaded and
-    the next token picked on the host (as the reference's loop does, cuda-dense.lisp:428-430)."""
+    prefill products, then a 256-token greedy decode at batch 1.  A step is one decoded token: its whole forward pass to
+    the logits and the greedy pick -- on the device, the ids read back after the last token (--host-argmax: logits
+    downloaded and the token picked on the host every step, as the reference's loop does, cuda-dense.lisp:428-430)."""
     from illatio_amd import hip, model, synth
     nl, nprompt, ndecode = args.layers, 512, 256
     host = model.synth_model(2, nl=nl)
@@ -650,11 +652,15 @@ def workload_c2d(args, dev):
         m.forward_n([tok]); tok = m.argmax()
     hip.hip_sync(dev)
     t0 = time.perf_counter()
-    toks = []
-    for _ in range(ndecode):
-        m.forward_n([tok])
-        tok = m.argmax()
-        toks.append(tok)
+    if args.host_argmax:                                     # the reference's loop: logits to the host, the token picked there
+        toks = []
+        for _ in range(ndecode):
+            m.forward_n([tok])
+            tok = m.argmax()
+            toks.append(tok)
+    else:                                                    # the token picked on the device and fed on from device memory
+        toks = m.decode_greedy(ndecode)
+    hip.hip_sync(dev)
     decode_s = time.perf_counter() - t0
     wbytes = sum(a[1].size for L in host["layers"] for k, a in L.items() if isinstance(a, tuple)) + host["output"][1].size
     ms = decode_s * 1e3 / ndecode
@@ -690,8 +696,8 @@ def workload_c2d(args, dev):
             "roofline": {"bound": "hbm", "achieved": round(wbytes / (ms * 1e-3) / 1e9, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                          "frac": round(wbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4), "traffic": None,
                          "kernel": "whole token: 6 launches a layer (Q/K/V, head norms + RoPE + attention scores, softmax + values, wo, gate+up, "
-                                   "down) + embedding + head, logits to the host",
-                         "launches": 6 * nl + 2, "avg_launch_us": round(ms * 1e3 / (6 * nl + 2), 2)},
+                                   "down) + embedding + head + the greedy pick",
+                         "launches": 6 * nl + 3, "avg_launch_us": round(ms * 1e3 / (6 * nl + 3), 2)},
             "cpu": cpu}
 
 
@@ -709,6 +715,7 @@ def main():
     ap.add_argument("--layers", type=int, default=LAYERS, help=argparse.SUPPRESS)
     ap.add_argument("--tokens", type=int, default=4096, help="c3, c5: tokens per step")
     ap.add_argument("--transpose", action="store_true", help="c3: the 5120x17408 matrix")
+    ap.add_argument("--host-argmax", action="store_true", help="c2d: every token's logits to the host and the next token picked there")
     ap.add_argument("--qtype", default="q6_k", choices=["q6_k", "q4_k", "q8_0"], help="c3: the matrix's format (the benchmark's: q6_k)")
     ap.add_argument("--path", default="bf16", choices=["bf16", "bf16-1pass", "bf16-2pass", "bf16-resident", "int8", "int8-2pass", "int8-resident"],
                     help="c3, c5: which matrix-core path.  c3: bf16 = 2pass from 1024 tokens on, else 1pass; bf16-1pass = the matrix dequantized inside the product's loop; "

@@ -785,6 +785,13 @@ int ilt_attn_step(uint64_t stream, const float* q, const float* k, const float* 
   ILT_REQUIRE(q && k && v && rope && kc && vc && out && scratch && nh > 0 && nkv > 0 && pos >= 0 && pos < 2048);
   return (int)ilt_k_attn_step(q, k, v, qn, kn, rope, kc, vc, out, nh, nkv, hd, rd, pos, eps, neox, scratch, S(stream));
 }
+// ARGMAX (model.lisp:464-468) of n floats on the device: the index into out[0] (device memory), so that a greedy
+// decode can go on without the logits' trip to the host (the reference picks the token on the host, cuda-dense.lisp:428-430)
+int ilt_argmax(uint64_t stream, const float* v, int n, int32_t* out) {
+  ILT_REQUIRE(v && out && n > 0 && ((uintptr_t)v & 15) == 0);
+  return (int)ilt_k_argmax(v, n, out, S(stream));
+}
+
 // ---- one token through the dense decoder: the launches of the single calls, queued in one ----------
 static ilt_mv_desc mv_of(const ilt_dense_mat& w, float* y) { return {w.gguf_type, w.rows, w.w, w.wd, y, nullptr}; }
 int ilt_dense_decode(uint64_t stream, const ilt_dense_model* m, const int32_t* token, int pos, int want_logits) {
@@ -905,6 +912,7 @@ int ilt_launch(const char* kernel, unsigned gx, unsigned gy, unsigned gz, unsign
                                   a.ptr<float*>(7), a.i32(8), a.i32(9), a.i32(10), a.i32(11), a.i32(12), a.f32(13), a.i32(14), (int)gy);
   K("swiglu") return ilt_swiglu(stream, a.ptr<float*>(0), a.ptr<cf>(1), a.i64(2));
   K("attn_rows") return ilt_attn_rows(stream, a.ptr<cf>(0), a.ptr<cf>(1), a.ptr<cf>(2), a.ptr<float*>(3), a.i32(4), a.i32(5), a.i32(6), a.i32(7), (int)gy, a.ptr<float*>(8));
+  K("argmax") return ilt_argmax(stream, a.ptr<cf>(0), a.i32(1), a.ptr<int32_t*>(2));
   K("attn_step") return ilt_attn_step(stream, a.ptr<cf>(0), a.ptr<cf>(1), a.ptr<cf>(2), a.ptr<cf>(3), a.ptr<cf>(4), a.ptr<cf>(5), a.ptr<float*>(6),
                                       a.ptr<float*>(7), a.ptr<float*>(8), a.i32(9), a.i32(10), a.i32(11), a.i32(12), a.i32(13), a.f32(14), a.i32(15),
                                       a.ptr<float*>(16));

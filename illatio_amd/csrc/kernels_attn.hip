@@ -454,6 +454,39 @@ __global__ __launch_bounds__(256) void attn_values_kernel(const float* __restric
 }
 
 // swiglu! (model.lisp:364-378) on n values: a = (a / (1 + e^-a)) * b, the exponential through double
+// ARGMAX (model.lisp:464-468): best = 0; an element replaces the best when it is greater -- so the first of equal
+// maxima, a NaN never (and if v[0] is a NaN nothing replaces it).  One workgroup: every thread the best of its own
+// elements (16 bytes a load, many in flight), then the best of those, a smaller index winning among equals.
+__global__ __launch_bounds__(1024) void argmax_kernel(const float* __restrict__ v, int n, int* __restrict__ out) {
+  __shared__ float bv[16];
+  __shared__ int bi[16];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  float best = -__builtin_inff();
+  int at = 0x7FFFFFFF;
+  auto take = [&](float x, int i) { if (x > best || (x == best && i < at)) { best = x; at = i; } };
+  const int n4 = n >> 2;
+  for (int i = tid; i < n4; i += 1024) {
+    const float4 x = *(const float4*)(v + 4 * i);
+    take(x.x, 4 * i); take(x.y, 4 * i + 1); take(x.z, 4 * i + 2); take(x.w, 4 * i + 3);
+  }
+  for (int i = 4 * n4 + tid; i < n; i += 1024) take(v[i], i);
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) {
+    const float ob = __shfl_xor(best, off);
+    const int oa = __shfl_xor(at, off);
+    if (ob > best || (ob == best && oa < at)) { best = ob; at = oa; }
+  }
+  if (lane == 0) { bv[wave] = best; bi[wave] = at; }
+  __syncthreads();
+  if (tid == 0) {
+    for (int w = 1; w < 16; w++)
+      if (bv[w] > best || (bv[w] == best && bi[w] < at)) { best = bv[w]; at = bi[w]; }
+    // a NaN in front (nothing is greater than a NaN) or nothing but NaNs: the scan never leaves index 0
+    const float v0 = v[0];
+    out[0] = (v0 != v0 || at == 0x7FFFFFFF) ? 0 : at;
+  }
+}
+
 __global__ __launch_bounds__(256) void swiglu_rows_kernel(float* __restrict__ a, const float* __restrict__ b, long long n) {
   const long long i = (long long)blockIdx.x * 256 + threadIdx.x;
   if (i < n) { const float g = a[i]; a[i] = (g / (1.0f + ilt_expf_via_double(-g))) * b[i]; }
@@ -547,6 +580,12 @@ hipError_t ilt_k_attn_step(const float* q, const float* k, const float* v, const
   ILT_ATTN1(1) ILT_ATTN1(2) ILT_ATTN1(3) ILT_ATTN1(4)
 #undef ILT_ATTN1
   return e;
+}
+
+hipError_t ilt_k_argmax(const float* v, int n, int* out, hipStream_t st) {
+  if (n <= 0) return hipErrorInvalidValue;
+  hipLaunchKernelGGL(argmax_kernel, dim3(1), dim3(1024), 0, st, v, n, out);
+  return hipGetLastError();
 }
 
 hipError_t ilt_k_swiglu_rows(float* a, const float* b, long long n, hipStream_t st) {

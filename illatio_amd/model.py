@@ -146,6 +146,25 @@ class DenseModel:
             dense.mv_multi(dev, [(self.output, self.logits, None)], xf=last, norm=(self.output_norm, eps))
         return self.logits
 
+    def decode_greedy(self, ntokens):
+        """NTOKENS greedy tokens after what the context holds, the first one picked from self.logits: every token picked
+        on the device (ilt_argmax) and fed to the next step from device memory, nothing waited for until the ids are
+        read back at the end.  Returns the ids; self.logits holds the logits after the last of them."""
+        if not self.one_call:
+            raise ValueError("the device-side loop runs over ilt_dense_decode (contexts up to 2048 positions)")
+        if self.pos + ntokens > self.nctx:
+            raise ValueError(f"{ntokens} more tokens at position {self.pos}: the context holds {self.nctx}")
+        dev, vocab = self.dev, self.c["vocab"]
+        S = C.c_uint64(dev.stream)
+        ids = hip.hip_alloc(dev, 4 * ntokens)
+        for i in range(ntokens):
+            hip.call("ilt_argmax", S, C.c_uint64(self.logits.ptr), C.c_int(vocab), C.c_uint64(ids.ptr + 4 * i))
+            hip.call("ilt_dense_decode", S, C.byref(self._cmodel), C.c_uint64(ids.ptr + 4 * i), C.c_int(self.pos), C.c_int(1))
+            self.pos += 1
+        out = hip.hip_download(ids, np.int32, ntokens).tolist()
+        hip.hip_free(ids)
+        return out
+
     def reset(self):
         """Forget the tokens seen: the next one is at position 0 (the caches' rows are overwritten as positions are reached)."""
         self.pos = 0

@@ -110,6 +110,65 @@ def test_attn_step_is_qk_rope_then_attn_rows(dev, norms):
         hip.hip_free(b)
 
 
+def test_argmax_on_the_device(dev):
+    """ilt_argmax against ARGMAX's scan (model.lisp:464-468): the first of equal maxima, -0 and +0 equal, a NaN never
+    greater, a NaN in front staying the best, nothing but -inf or NaN leaving index 0; lengths that are and are not
+    multiples of four."""
+    import ctypes as C
+    from illatio_amd import hip
+    def scan(v):
+        best = 0
+        for i in range(len(v)):
+            if v[i] > v[best]:
+                best = i
+        return best
+    rng = synth.make_rng(99)
+    out = hip.hip_alloc(dev, 4)
+    cases = []
+    for n in (1, 3, 4, 1000, 4099, 151936):
+        v = rng.standard_normal(n).astype(np.float32)
+        cases.append(v)
+        w = v.copy(); w[n // 2:] = v.max(); cases.append(w)                      # many equal maxima: the first
+        w = v.copy(); w[-1] = np.inf; cases.append(w)
+        w = v.copy(); w[::3] = np.nan; cases.append(w)                           # a NaN in front
+        if n > 4:
+            w = v.copy(); w[1::3] = np.nan; w[5] = 100.0; cases.append(w)        # NaNs elsewhere
+    cases += [np.full(70, -np.inf, np.float32), np.full(9, np.nan, np.float32), np.array([-0.0, 0.0, -0.0], np.float32),
+              np.array([-np.inf, -np.inf, 1.0, 1.0], np.float32), np.array([2.0, np.nan, 2.0, 3.0, np.nan, 3.0], np.float32)]
+    for v in cases:
+        b = hip.hip_upload_new(dev, v)
+        hip.call("ilt_argmax", C.c_uint64(dev.stream), C.c_uint64(b.ptr), C.c_int(len(v)), C.c_uint64(out.ptr))
+        got = int(hip.hip_download(out, np.int32, 1)[0])
+        with np.errstate(invalid="ignore"):
+            assert got == scan(v), (len(v), got, scan(v))
+        hip.hip_free(b)
+    hip.hip_free(out)
+
+
+def test_greedy_decode_on_the_device(dev):
+    """decode_greedy: the tokens picked on the device and fed on from device memory are the tokens the oracle's greedy
+    decode picks, and the logits after the last of them have the oracle's bits."""
+    from illatio_amd import hip, model
+    host = model.synth_model(12, d=512, ffn=1024, nh=8, nkv=2, hd=64, nl=2, vocab=777)
+    rng = synth.make_rng(12)
+    prompt = rng.integers(0, 777, 19).tolist()
+    cpu = orc.DenseModel(host, 64)
+    for t in prompt[:-1]:
+        cpu.forward(t, logits=False, nthreads=8)
+    want, _ = cpu.forward(prompt[-1], nthreads=8)
+    gpu = model.DenseModel(dev, host, 64, chunk=8)
+    gpu.eval_tokens(prompt)
+    ids = gpu.decode_greedy(30)
+    expect = []
+    for _ in range(30):
+        tok = int(np.argmax(want))
+        expect.append(tok)
+        want, _ = cpu.forward(tok, nthreads=8)
+    assert ids == expect
+    assert np.array_equal(bits(hip.hip_floats(gpu.logits, 777)), bits(want))
+    gpu.free()
+
+
 def test_reused_context_is_a_fresh_one(dev):
     """A context used for one sequence, reset and used for another gives the second the logits a fresh context gives
     (the reference's consistency-test.lisp:52-61): nothing of the first sequence's caches or buffers shows."""
