@@ -787,9 +787,9 @@ int ilt_attn_step(uint64_t stream, const float* q, const float* k, const float* 
 }
 // ARGMAX (model.lisp:464-468) of n floats on the device: the index into out[0] (device memory), so that a greedy
 // decode can go on without the logits' trip to the host (the reference picks the token on the host, cuda-dense.lisp:428-430)
-int ilt_argmax(uint64_t stream, const float* v, int n, int32_t* out) {
-  ILT_REQUIRE(v && out && n > 0 && ((uintptr_t)v & 15) == 0);
-  return (int)ilt_k_argmax(v, n, out, S(stream));
+int ilt_argmax(uint64_t stream, const float* v, int n, int32_t* out, void* scratch) {
+  ILT_REQUIRE(v && out && n > 0 && ((uintptr_t)v & 15) == 0 && ((uintptr_t)scratch & 7) == 0);
+  return (int)ilt_k_argmax(v, n, out, scratch, S(stream));
 }
 
 // ---- one token through the dense decoder: the launches of the single calls, queued in one ----------
@@ -912,7 +912,7 @@ int ilt_launch(const char* kernel, unsigned gx, unsigned gy, unsigned gz, unsign
                                   a.ptr<float*>(7), a.i32(8), a.i32(9), a.i32(10), a.i32(11), a.i32(12), a.f32(13), a.i32(14), (int)gy);
   K("swiglu") return ilt_swiglu(stream, a.ptr<float*>(0), a.ptr<cf>(1), a.i64(2));
   K("attn_rows") return ilt_attn_rows(stream, a.ptr<cf>(0), a.ptr<cf>(1), a.ptr<cf>(2), a.ptr<float*>(3), a.i32(4), a.i32(5), a.i32(6), a.i32(7), (int)gy, a.ptr<float*>(8));
-  K("argmax") return ilt_argmax(stream, a.ptr<cf>(0), a.i32(1), a.ptr<int32_t*>(2));
+  K("argmax") return ilt_argmax(stream, a.ptr<cf>(0), a.i32(1), a.ptr<int32_t*>(2), a.ptr<void*>(3));
   K("attn_step") return ilt_attn_step(stream, a.ptr<cf>(0), a.ptr<cf>(1), a.ptr<cf>(2), a.ptr<cf>(3), a.ptr<cf>(4), a.ptr<cf>(5), a.ptr<float*>(6),
                                       a.ptr<float*>(7), a.ptr<float*>(8), a.i32(9), a.i32(10), a.i32(11), a.i32(12), a.i32(13), a.f32(14), a.i32(15),
                                       a.ptr<float*>(16));

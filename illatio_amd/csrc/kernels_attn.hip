@@ -455,36 +455,51 @@ __global__ __launch_bounds__(256) void attn_values_kernel(const float* __restric
 
 // swiglu! (model.lisp:364-378) on n values: a = (a / (1 + e^-a)) * b, the exponential through double
 // ARGMAX (model.lisp:464-468): best = 0; an element replaces the best when it is greater -- so the first of equal
-// maxima, a NaN never (and if v[0] is a NaN nothing replaces it).  One workgroup: every thread the best of its own
-// elements (16 bytes a load, many in flight), then the best of those, a smaller index winning among equals.
-__global__ __launch_bounds__(1024) void argmax_kernel(const float* __restrict__ v, int n, int* __restrict__ out) {
+// maxima, a NaN never (and if v[0] is a NaN nothing replaces it).  Two steps: each workgroup the best of its
+// stretch (every thread's own elements first, eight 16-byte loads in flight, then the threads', a smaller index
+// winning among equals) into part[blockIdx]; then one workgroup the best of those.  With no room for the parts
+// (part null) one workgroup does it all.
+struct ArgBest { float v; int i; };
+__device__ __forceinline__ void arg_take(ArgBest& b, float x, int i) { if (x > b.v || (x == b.v && i < b.i)) { b.v = x; b.i = i; } }
+__device__ __forceinline__ ArgBest arg_block(ArgBest b) {      // the workgroup's best, in thread 0
   __shared__ float bv[16];
   __shared__ int bi[16];
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  float best = -__builtin_inff();
-  int at = 0x7FFFFFFF;
-  auto take = [&](float x, int i) { if (x > best || (x == best && i < at)) { best = x; at = i; } };
-  const int n4 = n >> 2;
-  for (int i = tid; i < n4; i += 1024) {
-    const float4 x = *(const float4*)(v + 4 * i);
-    take(x.x, 4 * i); take(x.y, 4 * i + 1); take(x.z, 4 * i + 2); take(x.w, 4 * i + 3);
-  }
-  for (int i = 4 * n4 + tid; i < n; i += 1024) take(v[i], i);
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, nw = blockDim.x >> 6;
 #pragma unroll
-  for (int off = 32; off > 0; off >>= 1) {
-    const float ob = __shfl_xor(best, off);
-    const int oa = __shfl_xor(at, off);
-    if (ob > best || (ob == best && oa < at)) { best = ob; at = oa; }
-  }
-  if (lane == 0) { bv[wave] = best; bi[wave] = at; }
+  for (int off = 32; off > 0; off >>= 1) arg_take(b, __shfl_xor(b.v, off), __shfl_xor(b.i, off));
+  if (lane == 0) { bv[wave] = b.v; bi[wave] = b.i; }
   __syncthreads();
-  if (tid == 0) {
-    for (int w = 1; w < 16; w++)
-      if (bv[w] > best || (bv[w] == best && bi[w] < at)) { best = bv[w]; at = bi[w]; }
-    // a NaN in front (nothing is greater than a NaN) or nothing but NaNs: the scan never leaves index 0
-    const float v0 = v[0];
-    out[0] = (v0 != v0 || at == 0x7FFFFFFF) ? 0 : at;
+  if (tid == 0) for (int w = 1; w < nw; w++) arg_take(b, bv[w], bi[w]);
+  return b;
+}
+__global__ __launch_bounds__(1024) void argmax_part_kernel(const float* __restrict__ v, int n, ArgBest* __restrict__ part, int* __restrict__ out) {
+  const int tid = threadIdx.x, nt = blockDim.x, n4 = n >> 2;
+  const int per = (n4 + gridDim.x - 1) / gridDim.x, lo = blockIdx.x * per, hi = min(n4, lo + per);      // this workgroup's 16-byte pieces
+  ArgBest b = { -__builtin_inff(), 0x7FFFFFFF };
+  for (int base = lo; base < hi; base += 8 * nt) {
+    float4 x[8];
+#pragma unroll
+    for (int u = 0; u < 8; u++) x[u] = *(const float4*)(v + 4 * min(base + tid + nt * u, hi - 1));       // (past the end: the last piece again)
+#pragma unroll
+    for (int u = 0; u < 8; u++) {
+      const int i = 4 * min(base + tid + nt * u, hi - 1);
+      arg_take(b, x[u].x, i); arg_take(b, x[u].y, i + 1); arg_take(b, x[u].z, i + 2); arg_take(b, x[u].w, i + 3);
+    }
   }
+  if (blockIdx.x == gridDim.x - 1)
+    for (int i = 4 * n4 + tid; i < n; i += nt) arg_take(b, v[i], i);
+  b = arg_block(b);
+  if (tid == 0) {
+    if (part) part[blockIdx.x] = b;
+    else { const float v0 = v[0]; out[0] = (v0 != v0 || b.i == 0x7FFFFFFF) ? 0 : b.i; }
+  }
+}
+__global__ __launch_bounds__(256) void argmax_last_kernel(const float* __restrict__ v, const ArgBest* __restrict__ part, int nparts, int* __restrict__ out) {
+  ArgBest b = { -__builtin_inff(), 0x7FFFFFFF };
+  for (int i = threadIdx.x; i < nparts; i += 256) arg_take(b, part[i].v, part[i].i);
+  b = arg_block(b);
+  // a NaN in front (nothing is greater than a NaN) or nothing but NaNs: the scan never leaves index 0
+  if (threadIdx.x == 0) { const float v0 = v[0]; out[0] = (v0 != v0 || b.i == 0x7FFFFFFF) ? 0 : b.i; }
 }
 
 __global__ __launch_bounds__(256) void swiglu_rows_kernel(float* __restrict__ a, const float* __restrict__ b, long long n) {
@@ -582,9 +597,16 @@ hipError_t ilt_k_attn_step(const float* q, const float* k, const float* v, const
   return e;
 }
 
-hipError_t ilt_k_argmax(const float* v, int n, int* out, hipStream_t st) {
+// scratch: 2048 bytes of the caller's for the workgroups' bests, or null (one workgroup then reads everything)
+hipError_t ilt_k_argmax(const float* v, int n, int* out, void* scratch, hipStream_t st) {
   if (n <= 0) return hipErrorInvalidValue;
-  hipLaunchKernelGGL(argmax_kernel, dim3(1), dim3(1024), 0, st, v, n, out);
+  const int nparts = scratch && n >= (1 << 15) ? 128 : 1;
+  if (nparts == 1) {
+    hipLaunchKernelGGL(argmax_part_kernel, dim3(1), dim3(1024), 0, st, v, n, (ArgBest*)nullptr, out);
+  } else {
+    hipLaunchKernelGGL(argmax_part_kernel, dim3(nparts), dim3(256), 0, st, v, n, (ArgBest*)scratch, out);
+    hipLaunchKernelGGL(argmax_last_kernel, dim3(1), dim3(256), 0, st, v, (const ArgBest*)scratch, nparts, out);
+  }
   return hipGetLastError();
 }
 

@@ -156,13 +156,14 @@ class DenseModel:
             raise ValueError(f"{ntokens} more tokens at position {self.pos}: the context holds {self.nctx}")
         dev, vocab = self.dev, self.c["vocab"]
         S = C.c_uint64(dev.stream)
-        ids = hip.hip_alloc(dev, 4 * ntokens)
+        ids, scratch = hip.hip_alloc(dev, 4 * ntokens), hip.hip_alloc(dev, 2048)
         for i in range(ntokens):
-            hip.call("ilt_argmax", S, C.c_uint64(self.logits.ptr), C.c_int(vocab), C.c_uint64(ids.ptr + 4 * i))
+            hip.call("ilt_argmax", S, C.c_uint64(self.logits.ptr), C.c_int(vocab), C.c_uint64(ids.ptr + 4 * i), C.c_uint64(scratch.ptr))
             hip.call("ilt_dense_decode", S, C.byref(self._cmodel), C.c_uint64(ids.ptr + 4 * i), C.c_int(self.pos), C.c_int(1))
             self.pos += 1
         out = hip.hip_download(ids, np.int32, ntokens).tolist()
         hip.hip_free(ids)
+        hip.hip_free(scratch)
         return out
 
     def reset(self):

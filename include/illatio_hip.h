@@ -323,8 +323,10 @@ int ilt_attn_step(uint64_t stream, const float* q, const float* k, const float* 
 /* ARGMAX (model.lisp:464-468) on the device: out[0] = the index of the first of the greatest of v's n floats (a NaN
    is never greater; a NaN in front stays the best, as in the reference's scan).  No counterpart among the
    reference's kernels: its host picks the token (cuda-dense.lisp:428-430); with this a greedy decode queues token
-   after token without the logits' trip to the host (ilt_dense_decode takes its token from device memory). */
-int ilt_argmax(uint64_t stream, const float* v, int n, int32_t* out);
+   after token without the logits' trip to the host (ilt_dense_decode takes its token from device memory).  scratch:
+   2048 bytes of the caller's, 8-byte aligned (128 workgroups leave their bests there for a second launch), or null
+   (one workgroup reads everything: several times slower on a vocabulary's logits). */
+int ilt_argmax(uint64_t stream, const float* v, int n, int32_t* out, void* scratch);
 typedef struct ilt_dense_mat { int gguf_type, rows, cols; const void* w; const uint16_t* wd; } ilt_dense_mat;
 typedef struct ilt_dense_layer {
   const float *attn_norm, *q_norm, *k_norm, *ffn_norm;        /* q_norm, k_norm: null when the model has no head norms */

@@ -123,7 +123,7 @@ def test_argmax_on_the_device(dev):
                 best = i
         return best
     rng = synth.make_rng(99)
-    out = hip.hip_alloc(dev, 4)
+    out, scratch = hip.hip_alloc(dev, 4), hip.hip_alloc(dev, 2048)
     cases = []
     for n in (1, 3, 4, 1000, 4099, 151936):
         v = rng.standard_normal(n).astype(np.float32)
@@ -137,12 +137,14 @@ def test_argmax_on_the_device(dev):
               np.array([-np.inf, -np.inf, 1.0, 1.0], np.float32), np.array([2.0, np.nan, 2.0, 3.0, np.nan, 3.0], np.float32)]
     for v in cases:
         b = hip.hip_upload_new(dev, v)
-        hip.call("ilt_argmax", C.c_uint64(dev.stream), C.c_uint64(b.ptr), C.c_int(len(v)), C.c_uint64(out.ptr))
-        got = int(hip.hip_download(out, np.int32, 1)[0])
-        with np.errstate(invalid="ignore"):
-            assert got == scan(v), (len(v), got, scan(v))
+        for sc in (0, scratch.ptr):                                              # one workgroup; 128 and a second launch
+            hip.call("ilt_argmax", C.c_uint64(dev.stream), C.c_uint64(b.ptr), C.c_int(len(v)), C.c_uint64(out.ptr), C.c_uint64(sc))
+            got = int(hip.hip_download(out, np.int32, 1)[0])
+            with np.errstate(invalid="ignore"):
+                assert got == scan(v), (len(v), got, scan(v), sc != 0)
         hip.hip_free(b)
     hip.hip_free(out)
+    hip.hip_free(scratch)
 
 
 def test_greedy_decode_on_the_device(dev):
