@@ -782,7 +782,7 @@ int ilt_qk_rope(uint64_t stream, float* q, float* k, const float* v, const float
 // norms and turns the heads where it needs them and writes the caches' rows); q and k are left as they came
 int ilt_attn_step(uint64_t stream, const float* q, const float* k, const float* v, const float* qn, const float* kn, const float* rope, float* kc,
                   float* vc, float* out, int nh, int nkv, int hd, int rd, int pos, float eps, int neox, float* scratch) {
-  ILT_REQUIRE(q && k && v && rope && kc && vc && out && scratch && nh > 0 && nkv > 0 && pos >= 0 && pos < 2048);
+  ILT_REQUIRE(q && k && v && rope && kc && vc && out && scratch && nh > 0 && nkv > 0 && pos >= 0 && pos < 8192);
   return (int)ilt_k_attn_step(q, k, v, qn, kn, rope, kc, vc, out, nh, nkv, hd, rd, pos, eps, neox, scratch, S(stream));
 }
 // ARGMAX (model.lisp:464-468) of n floats on the device: the index into out[0] (device memory), so that a greedy
@@ -795,7 +795,7 @@ int ilt_argmax(uint64_t stream, const float* v, int n, int32_t* out, void* scrat
 // ---- one token through the dense decoder: the launches of the single calls, queued in one ----------
 static ilt_mv_desc mv_of(const ilt_dense_mat& w, float* y) { return {w.gguf_type, w.rows, w.w, w.wd, y, nullptr}; }
 int ilt_dense_decode(uint64_t stream, const ilt_dense_model* m, const int32_t* token, int pos, int want_logits) {
-  ILT_REQUIRE(m && token && m->layers && m->nl > 0 && pos >= 0 && pos < 2048);
+  ILT_REQUIRE(m && token && m->layers && m->nl > 0 && pos >= 0 && pos < 8192);
   ILT_REQUIRE(m->x && m->q && m->k && m->v && m->att && m->fa && m->scores && m->rope && (!want_logits || (m->logits && m->output_norm)));
   int e;
   if (m->embd.gguf_type == ILT_TYPE_Q8_0) e = ilt_embed_q8(stream, (const int8_t*)m->embd.w, m->embd.wd, token, m->x, m->d, 1);

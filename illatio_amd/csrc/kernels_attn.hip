@@ -454,6 +454,100 @@ __global__ __launch_bounds__(256) void attn_values_kernel(const float* __restric
 }
 
 // swiglu! (model.lisp:364-378) on n values: a = (a / (1 + e^-a)) * b, the exponential through double
+// The same for contexts whose value slice no longer fits LDS (2,049 to 8,192 positions): the slice comes through
+// LDS in tiles of kValTile positions, and a chain carries its sum from tile to tile -- position after position all
+// the same.  TG 1: the token's scores are taken and scaled here and stay in LDS.  TG 16 (a prompt's chunk): the
+// scores come scaled from attn_softmax_kernel and go through LDS tile by tile like the values.
+constexpr int kValTile = 1024, kValPitch = kValTile + 4;
+template <int TG>
+__global__ __launch_bounds__(256) void attn_values_tiled_kernel(const float* __restrict__ raw, const float* __restrict__ vc, float* __restrict__ out,
+                                                                int nh, int nkv, int hd, int pos0, int ntok, int spitch) {
+  extern __shared__ __align__(16) float dyn[];
+  __shared__ float redf[4];
+  __shared__ double redd[8];
+  const int ns = hd >> 4, h = blockIdx.x / ns, cs = blockIdx.x - h * ns, t0 = blockIdx.y * TG, tid = threadIdx.x;
+  const int tn = min(TG, ntok - t0), nposmax = pos0 + t0 + tn;
+  const int group = nh / nkv, kvd = nkv * hd, ko = (h / group) * hd + 16 * cs;
+  const int lp = TG > 1 ? kValPitch : spitch;        // TG > 1: a token's scores of the tile; TG 1: all of the token's
+  float* scores = dyn;
+  float* vt = dyn + TG * lp;
+  const float* rbase = raw + ((long long)t0 * nh + h) * spitch;
+  if (TG == 1) attn_softmax<256, false>(rbase, nullptr, scores, nposmax, tid, redf, redd);
+  const int tt = tid >> 4, c = tid & 15, npos = pos0 + t0 + tt + 1;       // a chain's token and column (tid < tn * 16)
+  const float* sc = scores + tt * lp;
+  const float* col = vt + c * kValPitch;
+  float o = 0.0f;
+  for (int p0 = 0; p0 < nposmax; p0 += kValTile) {
+    const int npt = min(kValTile, nposmax - p0), total = npt * 4;       // the tile's positions, its 16-byte pieces of values
+    float4 r[16];
+#pragma unroll
+    for (int u = 0; u < 16; u++) {
+      const int i = min(tid + 256 * u, total - 1);
+      r[u] = *(const float4*)(vc + (long long)(p0 + (i >> 2)) * kvd + ko + 4 * (i & 3));
+    }
+    __syncthreads();                                 // the scores are there (TG 1, first tile); the chains are through with the tile before
+    if (TG > 1) {
+      // the group's scores of the tile's positions: 256 pieces a row at most (what lies past a token's own positions is
+      // carried along and never read; past the row's end nothing is loaded)
+      const int q4 = (npt + 3) >> 2, totalq = tn * q4;
+      for (int base = 0; base < totalq; base += 256 * 8) {
+        float4 tmp[8];
+#pragma unroll
+        for (int u = 0; u < 8; u++) {
+          const int i = min(base + tid + 256 * u, totalq - 1), rt = i / q4, j = i - rt * q4;
+          tmp[u] = *(const float4*)(rbase + (long long)rt * nh * spitch + p0 + 4 * j);
+        }
+#pragma unroll
+        for (int u = 0; u < 8; u++) {
+          const int i = base + tid + 256 * u, rt = i / q4, j = i - rt * q4;
+          if (i < totalq) *(float4*)(scores + rt * lp + 4 * j) = tmp[u];
+        }
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < 16; u++) {
+      const int i = tid + 256 * u;
+      if (i < total) {
+        float* dst = vt + (4 * (i & 3)) * kValPitch + (i >> 2);
+        if (TG == 1) {
+          const float sp = scores[p0 + (i >> 2)];
+          dst[0] = sp * r[u].x; dst[kValPitch] = sp * r[u].y; dst[2 * kValPitch] = sp * r[u].z; dst[3 * kValPitch] = sp * r[u].w;
+        } else {
+          dst[0] = r[u].x; dst[kValPitch] = r[u].y; dst[2 * kValPitch] = r[u].z; dst[3 * kValPitch] = r[u].w;
+        }
+      }
+    }
+    __syncthreads();
+    if (tid < tn * 16) {
+      const int np = min(kValTile, npos - p0);       // of the tile's positions, the token's own (may be none)
+      int p = 0;
+      if (TG == 1) {
+        for (; p + 32 <= np; p += 32) {
+          float4 v4[8];
+#pragma unroll
+          for (int u = 0; u < 8; u++) v4[u] = *(const float4*)(col + p + 4 * u);
+#pragma unroll
+          for (int u = 0; u < 8; u++) { o = o + v4[u].x; o = o + v4[u].y; o = o + v4[u].z; o = o + v4[u].w; }
+        }
+        for (; p < np; p++) o = o + col[p];
+      } else {
+        for (; p + 16 <= np; p += 16) {
+          float4 s4[4], v4[4];
+#pragma unroll
+          for (int u = 0; u < 4; u++) { s4[u] = *(const float4*)(sc + p + 4 * u); v4[u] = *(const float4*)(col + p + 4 * u); }
+#pragma unroll
+          for (int u = 0; u < 4; u++) {
+            const float a0 = s4[u].x * v4[u].x, a1 = s4[u].y * v4[u].y, a2 = s4[u].z * v4[u].z, a3 = s4[u].w * v4[u].w;
+            o = o + a0; o = o + a1; o = o + a2; o = o + a3;
+          }
+        }
+        for (; p < np; p++) o = o + sc[p] * col[p];
+      }
+    }
+  }
+  if (tid < tn * 16) out[((long long)(t0 + tt) * nh + h) * hd + 16 * cs + c] = o;
+}
+
 // ARGMAX (model.lisp:464-468): best = 0; an element replaces the best when it is greater -- so the first of equal
 // maxima, a NaN never (and if v[0] is a NaN nothing replaces it).  Two steps: each workgroup the best of its
 // stretch (every thread's own elements first, eight 16-byte loads in flight, then the threads', a smaller index
@@ -517,8 +611,8 @@ hipError_t ilt_k_qk_rope(float* q, float* k, const float* v, const float* qn, co
   return hipGetLastError();
 }
 
-// scratch: ntok * nh * ((pos0 + ntok + 3) & ~3) floats for the two-launch variant (contexts up to 2048 positions),
-// or null: one launch
+// scratch: ntok * nh * ((pos0 + ntok + 3) & ~3) floats for the variants of two or three launches (contexts up to 8192
+// positions), or null: one launch
 hipError_t ilt_k_attn_rows(const float* q, const float* kc, const float* vc, float* out, int nh, int nkv, int hd, int pos0, int ntok,
                            float* scratch, hipStream_t st) {
   if (ntok <= 0) return hipSuccess;
@@ -557,6 +651,27 @@ hipError_t ilt_k_attn_rows(const float* q, const float* kc, const float* vc, flo
 #undef ILT_ATTN
     return e;
   }
+  if (scratch && pos0 + ntok <= 8192) {              // the value slice through LDS in tiles
+    const int ctx = pos0 + ntok, tg = ntok > 1 ? 16 : 1;
+    const size_t smem = sizeof(float) * ((tg > 1 ? (size_t)tg * kValPitch : (size_t)smax) + 16 * (size_t)kValPitch);
+    const dim3 gs(nh, (ctx + 255) / 256, (ntok + tg - 1) / tg), gv(nh * (hd / 16), (ntok + tg - 1) / tg);
+    static bool set[64] = {};
+    if (!set[dev]) {
+      hipError_t e = hipFuncSetAttribute((const void*)attn_values_tiled_kernel<1>, hipFuncAttributeMaxDynamicSharedMemorySize, 152 * 1024);
+      if (e == hipSuccess) e = hipFuncSetAttribute((const void*)attn_values_tiled_kernel<16>, hipFuncAttributeMaxDynamicSharedMemorySize, 152 * 1024);
+      if (e != hipSuccess) return e;
+      set[dev] = true;
+    }
+    if (tg == 16) {
+      hipLaunchKernelGGL(attn_scores_kernel<16>, gs, dim3(1024), 0, st, q, kc, scratch, nh, nkv, hd, pos0, ntok, scale, smax);
+      hipLaunchKernelGGL(attn_softmax_kernel, dim3(nh, ntok), dim3(256), sizeof(float) * smax, st, scratch, nh, pos0, smax);
+      hipLaunchKernelGGL(attn_values_tiled_kernel<16>, gv, dim3(256), smem, st, scratch, vc, out, nh, nkv, hd, pos0, ntok, smax);
+    } else {
+      hipLaunchKernelGGL(attn_scores_kernel<1>, gs, dim3(1024), 0, st, q, kc, scratch, nh, nkv, hd, pos0, ntok, scale, smax);
+      hipLaunchKernelGGL(attn_values_tiled_kernel<1>, gv, dim3(256), smem, st, scratch, vc, out, nh, nkv, hd, pos0, ntok, smax);
+    }
+    return hipGetLastError();
+  }
   if (!attr_set[dev]) {
     const hipError_t e = hipFuncSetAttribute((const void*)attn_rows_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 152 * 1024);
     if (e != hipSuccess) return e;
@@ -571,7 +686,7 @@ hipError_t ilt_k_attn_rows(const float* q, const float* kc, const float* vc, flo
 // One token at position pos: qk_rope and attention in two launches instead of three
 hipError_t ilt_k_attn_step(const float* q, const float* k, const float* v, const float* qn, const float* kn, const float* rope, float* kc,
                            float* vc, float* out, int nh, int nkv, int hd, int rd, int pos, float eps, int neox, float* scratch, hipStream_t st) {
-  if (hd % 16 || hd > 256 || rd > hd || (rd & 1) || nh % nkv || pos < 0 || pos >= 2048 || !scratch) return hipErrorInvalidValue;
+  if (hd % 16 || hd > 256 || rd > hd || (rd & 1) || nh % nkv || pos < 0 || pos >= 8192 || !scratch) return hipErrorInvalidValue;
   const int ctx = pos + 1, smax = (ctx + 3) & ~3, vpitch = ((ctx + 63) & ~63) + 4, nb = (ctx + 511) / 512;
   const float scale = 1.0f / sqrtf((float)hd);
   const size_t smem = sizeof(float) * ((size_t)smax + 16 * (size_t)vpitch);
@@ -579,6 +694,17 @@ hipError_t ilt_k_attn_step(const float* q, const float* k, const float* v, const
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) dev = 0;
   hipLaunchKernelGGL(attn_step_scores_kernel, dim3(nh, (ctx + 255) / 256), dim3(1024), 0, st, q, k, v, qn, kn, rope, kc, vc, scratch, nh, nkv, hd, rd,
                      pos, eps, neox, scale, smax);
+  if (ctx > 2048) {
+    static bool set[64] = {};
+    if (!set[dev]) {
+      const hipError_t e = hipFuncSetAttribute((const void*)attn_values_tiled_kernel<1>, hipFuncAttributeMaxDynamicSharedMemorySize, 152 * 1024);
+      if (e != hipSuccess) return e;
+      set[dev] = true;
+    }
+    hipLaunchKernelGGL(attn_values_tiled_kernel<1>, dim3(nh * (hd / 16), 1), dim3(256), sizeof(float) * ((size_t)smax + 16 * (size_t)kValPitch), st,
+                       scratch, vc, out, nh, nkv, hd, pos, 1, smax);
+    return hipGetLastError();
+  }
   hipError_t e = hipErrorInvalidValue;
 #define ILT_ATTN1(NB)                                                                                                                         \
   if (nb == NB) {                                                                                                                             \

@@ -86,7 +86,7 @@ class DenseModel:
         self.x, self.q, self.k, self.v = A(4 * n * d), A(4 * n * self.qd), A(4 * n * self.kvd), A(4 * n * self.kvd)
         self.att, self.fa, self.fb = A(4 * n * self.qd), A(4 * n * ffn), A(4 * n * ffn)
         self.tokens = A(4 * n)
-        self.scores = A(4 * n * c["nh"] * ((nctx + 3) // 4 * 4)) if nctx <= 2048 else None      # the attention's raw scores
+        self.scores = A(4 * n * c["nh"] * ((nctx + 3) // 4 * 4)) if nctx <= 8192 else None      # the attention's raw scores
         self.logits = A(4 * c["vocab"])
         self.acts = {cols: dense.QAct(dev, n, cols, ("q8k",)) for cols in {d, self.qd, ffn}}
         # the model as ilt_dense_decode reads it: a token's launches queued by one call
@@ -151,7 +151,7 @@ class DenseModel:
         on the device (ilt_argmax) and fed to the next step from device memory, nothing waited for until the ids are
         read back at the end.  Returns the ids; self.logits holds the logits after the last of them."""
         if not self.one_call:
-            raise ValueError("the device-side loop runs over ilt_dense_decode (contexts up to 2048 positions)")
+            raise ValueError("the device-side loop runs over ilt_dense_decode (contexts up to 8192 positions)")
         if self.pos + ntokens > self.nctx:
             raise ValueError(f"{ntokens} more tokens at position {self.pos}: the context holds {self.nctx}")
         dev, vocab = self.dev, self.c["vocab"]

@@ -296,7 +296,7 @@ int ilt_d4_moe_sum_rows(uint64_t stream, int d, int nu, int ntok, const float* d
      in F32-DOT16's order, the softmax's sum in double, the values added position after position.  It stands
      where the reference launches attn_decode + attn_merge / attn_prefill (dense.cu:376-727), whose partial
      sums meet in another order.  scratch: ntok * nh * ((pos0 + ntok + 3) & ~3) floats of the caller's for the raw
-     scores (two launches, for contexts up to 2048 positions: the scores over many workgroups, then a 16-column
+     scores (two launches, for contexts up to 2048 positions, the value slice in tiles up to 8192: the scores over many workgroups, then a 16-column
      slice of the values a workgroup), or null (one launch, a workgroup a head, any context that fits LDS).
    swiglu (dense.cu:307): swiglu! on n values, a = (a / (1 + e^-a)) * b, the exponential through double. */
 /* The table qk_rope takes, for positions pos0 .. pos0 + n - 1, written to host memory (n * head_dim floats). */
@@ -305,7 +305,7 @@ int ilt_qk_rope(uint64_t stream, float* q, float* k, const float* v, const float
                 float* vc, int nh, int nkv, int hd, int rd, int pos0, float eps, int neox, int ntok);
 int ilt_attn_rows(uint64_t stream, const float* q, const float* kc, const float* vc, float* out, int nh, int nkv, int hd, int pos0, int ntok,
                   float* scratch);
-/* ilt_qk_rope and ilt_attn_rows of one token at position pos (< 2048) with one launch fewer: the launch that takes
+/* ilt_qk_rope and ilt_attn_rows of one token at position pos (< 8192) with one launch fewer: the launch that takes
    the scores norms and turns the query heads and the token's key itself and writes the caches' rows at pos.  out is
    what ilt_attn_rows gives after ilt_qk_rope, bit for bit; q and k are left as they came (not normed, not turned).
    scratch: nh * ((pos + 4) & ~3) floats. */
@@ -317,7 +317,7 @@ int ilt_attn_step(uint64_t stream, const float* q, const float* k, const float* 
    Q/K/V products with the norm inside, ilt_attn_step, wo onto the residual, gate/up with the norm and the gated
    activation inside, down onto the residual, and (want_logits) the output norm and head: 6 launches a layer + 2.
    The structs are read on the host during the call; every pointer in them is device memory but `layers`.
-   Matrices as dense uploads hold them (Q8_0 split into quants and scales, Q6_K in 212-byte blocks).  pos < 2048
+   Matrices as dense uploads hold them (Q8_0 split into quants and scales, Q6_K in 212-byte blocks).  pos < 8192
    (the attention's scratch), the caches hold at least pos + 1 positions, rope at least (pos + 1) * rd floats.
    token: one id, on the device.  The results are those of the single calls, bit for bit. */
 /* ARGMAX (model.lisp:464-468) on the device: out[0] = the index of the first of the greatest of v's n floats (a NaN

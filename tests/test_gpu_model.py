@@ -215,13 +215,19 @@ def test_llama_style_decoder(dev):
 
 def test_small_decoder_long_contexts(dev):
     """Contexts past one workgroup's 256 positions of scores: the two-launch attention with 16 tokens, 4 tokens and one
-    token a workgroup as the context grows towards 2048 positions, and past that the single launch with its value tiles."""
+    token a workgroup as the context grows towards 2048 positions, and past that the value slice in tiles."""
     from illatio_amd import model
     host = model.synth_model(6, d=256, ffn=512, nh=4, nkv=2, hd=64, nl=2, vocab=500)
     same, _ = run_greedy(dev, host, nprompt=2030, ndecode=6, chunk=512, nctx=2040, seed=6)
     assert same == 6
     same, _ = run_greedy(dev, host, nprompt=2060, ndecode=4, chunk=512, nctx=2100, seed=7)
     assert same == 4
+    # past 2048 positions the value slice goes through LDS in tiles of 1024 positions: four tokens a workgroup up to
+    # 4096 positions, one beyond; the decode steps cross a tile's edge (4096 -> 4097)
+    same, _ = run_greedy(dev, host, nprompt=4094, ndecode=6, chunk=512, nctx=4110, seed=13)
+    assert same == 6
+    same, _ = run_greedy(dev, host, nprompt=4400, ndecode=3, chunk=512, nctx=4410, seed=14, one_call=False)
+    assert same == 3
 
 
 def test_config_2_width_four_layers_128_greedy_tokens(dev):
