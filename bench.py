@@ -697,9 +697,9 @@ def workload_c2d(args, dev):
                       "weights_GBps_in_decode": round(wbytes / (ms * 1e-3) / 1e9, 1)},
             "roofline": {"bound": "hbm", "achieved": round(wbytes / (ms * 1e-3) / 1e9, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                          "frac": round(wbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4), "traffic": None,
-                         "kernel": "whole token: 6 launches a layer (Q/K/V, head norms + RoPE + attention scores, softmax + values, wo, gate+up, "
-                                   "down) + embedding + head + the greedy pick",
-                         "launches": 6 * nl + 3, "avg_launch_us": round(ms * 1e3 / (6 * nl + 3), 2)},
+                         "kernel": "whole token: 5 launches a layer (Q/K/V, attention, wo, gate+up, down) + embedding + head + the "
+                                   "greedy pick's two",
+                         "launches": 5 * nl + 4, "avg_launch_us": round(ms * 1e3 / (5 * nl + 4), 2)},
             "cpu": cpu}
 
 

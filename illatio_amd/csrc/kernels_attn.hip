@@ -7,6 +7,7 @@
 // partial sums meet in its own order, dense.cu:364-373).
 #include "ilt_device.h"
 #include "ilt_kernels.h"
+#include <stdlib.h>
 
 namespace {
 
@@ -18,21 +19,64 @@ __device__ __forceinline__ void wave_lds_sync() {
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
+// A wave's maximum and a wave's sum of doubles, the same in every lane: butterflies over a row's 16 lanes through DPP,
+// the four rows through readlane -- a tenth of the trips through LDS that __shfl_xor's permutes make.  All 64 lanes
+// must be active.  (The order of the adds is not the CPU's: callers check whether that could show.)
+template <int CTRL> __device__ __forceinline__ double dpp_double(double v) {
+  return __hiloint2double(ilt_dpp<CTRL>(__double2hiint(v)), ilt_dpp<CTRL>(__double2loint(v)));
+}
+__device__ __forceinline__ double readlane_double(double v, int lane) {
+  return __hiloint2double(__builtin_amdgcn_readlane(__double2hiint(v), lane), __builtin_amdgcn_readlane(__double2loint(v), lane));
+}
+__device__ __forceinline__ double wave_sum_double(double v) {
+  v += dpp_double<ILT_DPP_XOR1>(v);
+  v += dpp_double<ILT_DPP_XOR2>(v);
+  v += dpp_double<ILT_DPP_HALF_MIRROR>(v);
+  v += dpp_double<ILT_DPP_ROW_MIRROR>(v);
+  return (readlane_double(v, 0) + readlane_double(v, 16)) + (readlane_double(v, 32) + readlane_double(v, 48));
+}
+__device__ __forceinline__ float wave_max_float(float v) {
+  v = ilt_max16(v);
+  const int b = __float_as_int(v);
+  return fmaxf(fmaxf(__int_as_float(__builtin_amdgcn_readlane(b, 0)), __int_as_float(__builtin_amdgcn_readlane(b, 16))),
+               fmaxf(__int_as_float(__builtin_amdgcn_readlane(b, 32)), __int_as_float(__builtin_amdgcn_readlane(b, 48))));
+}
+
 // One head by one wave: x (hd floats) into xs (LDS): rmsnorm! of the head when its weights are given
 // (model.lisp:205-216: the squares, rounded to floats, added in double one after another), then rope-head!
 // from the position's table cs (cos, then sin, rd/2 each).  Only this wave touches xs and sd.  The lanes add
 // the squares in parallel; where the order of the adds could show in the single the mean is rounded to, one
 // lane adds them again one after another, as the CPU does.
-__device__ __forceinline__ void rope_head_wave(const float* __restrict__ x, const float* __restrict__ nw, const float* __restrict__ cs,
-                                               float* xs, double* sd, int hd, int rd, float eps, int neox, int i) {
+// In two steps, so that a kernel can ask for the head, its norm weights and the table's row before the loads it
+// makes for other things, and wait for these alone: lane i's share of the three (NT floats of the head: hd <= 64 NT).
+template <int NT> struct RopeIn { float x[NT], w[NT], c[(NT + 1) / 2], s[(NT + 1) / 2]; };
+template <int NT>
+__device__ __forceinline__ void rope_head_load(RopeIn<NT>& r, const float* __restrict__ x, const float* __restrict__ nw, const float* __restrict__ cs,
+                                               int hd, int rd, int i) {
   const int half = rd >> 1;
-  for (int j = i; j < hd; j += 64) xs[j] = x[j];
-  wave_lds_sync();
-  if (nw) {
-    double s = 0.0;
-    for (int j = i; j < hd; j += 64) { const float sq = xs[j] * xs[j]; s += (double)sq; }
 #pragma unroll
-    for (int off = 32; off > 0; off >>= 1) s += __shfl_xor(s, off);
+  for (int t = 0; t < NT; t++) {
+    const int j = min(i + 64 * t, hd - 1);
+    r.x[t] = x[j];
+    r.w[t] = nw ? nw[j] : 0.0f;
+  }
+#pragma unroll
+  for (int t = 0; t < (NT + 1) / 2; t++) {
+    const int p = min(i + 64 * t, max(half - 1, 0));
+    r.c[t] = half > 0 ? cs[p] : 0.0f; r.s[t] = half > 0 ? cs[half + p] : 0.0f;
+  }
+}
+template <int NT>
+__device__ __forceinline__ void rope_head_turn(const RopeIn<NT>& r, bool norm, float* xs, double* sd, int hd, int rd, float eps, int neox, int i) {
+  const int half = rd >> 1;
+#pragma unroll
+  for (int t = 0; t < NT; t++) if (i + 64 * t < hd) xs[i + 64 * t] = r.x[t];
+  wave_lds_sync();
+  if (norm) {
+    double s = 0.0;
+#pragma unroll
+    for (int t = 0; t < NT; t++) if (i + 64 * t < hd) { const float sq = r.x[t] * r.x[t]; s += (double)sq; }
+    s = wave_sum_double(s);
     const double slack = s * ((double)(hd + 8) * 0x1p-51);
     if ((float)((s - slack) / (double)hd + (double)eps) != (float)((s + slack) / (double)hd + (double)eps)) {      // the same in every lane
       if (i == 0) {
@@ -44,16 +88,27 @@ __device__ __forceinline__ void rope_head_wave(const float* __restrict__ x, cons
       s = *sd;
     }
     const float scale = 1.0f / sqrtf((float)(s / (double)hd + (double)eps));
-    for (int j = i; j < hd; j += 64) xs[j] = (xs[j] * scale) * nw[j];
+#pragma unroll
+    for (int t = 0; t < NT; t++) if (i + 64 * t < hd) xs[i + 64 * t] = (r.x[t] * scale) * r.w[t];
     wave_lds_sync();
   }
-  for (int p = i; p < half; p += 64) {
-    const int a = neox ? p : 2 * p, b = neox ? p + half : 2 * p + 1;
-    const float x0 = xs[a], x1 = xs[b], c = cs[p], sn = cs[half + p];
-    xs[a] = x0 * c - x1 * sn;                      // (no contraction: each product rounds on its own)
-    xs[b] = x0 * sn + x1 * c;
+#pragma unroll
+  for (int t = 0; t < (NT + 1) / 2; t++) {
+    const int p = i + 64 * t;
+    if (p < half) {
+      const int a = neox ? p : 2 * p, b = neox ? p + half : 2 * p + 1;
+      const float x0 = xs[a], x1 = xs[b], c = r.c[t], sn = r.s[t];
+      xs[a] = x0 * c - x1 * sn;                    // (no contraction: each product rounds on its own)
+      xs[b] = x0 * sn + x1 * c;
+    }
   }
   wave_lds_sync();
+}
+__device__ __forceinline__ void rope_head_wave(const float* __restrict__ x, const float* __restrict__ nw, const float* __restrict__ cs,
+                                               float* xs, double* sd, int hd, int rd, float eps, int neox, int i) {
+  RopeIn<8> r;                                     // hd <= 512
+  rope_head_load(r, x, nw, cs, hd, rd, i);
+  rope_head_turn(r, nw != nullptr, xs, sd, hd, rd, eps, neox, i);
 }
 
 // qk_rope: a workgroup (one wave) a head of a token; K and V into the caches at pos0 + t.
@@ -127,8 +182,7 @@ __global__ __launch_bounds__(kAttnThreads) void attn_rows_kernel(const float* __
       if (l == 0 && p < npos) { const float sv = s * scale; scores[p] = sv; mx = fmaxf(mx, sv); }
     }
   }
-#pragma unroll
-  for (int off = 32; off > 0; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off));
+  mx = wave_max_float(mx);
   if (lane == 0) redf[wave] = mx;
   __syncthreads();
   mx = redf[0];
@@ -136,8 +190,7 @@ __global__ __launch_bounds__(kAttnThreads) void attn_rows_kernel(const float* __
   for (int w = 1; w < 16; w++) mx = fmaxf(mx, redf[w]);
   double part = 0.0;
   for (int p = tid; p < npos; p += kAttnThreads) { const float e = ilt_expf_via_double(scores[p] - mx); scores[p] = e; part += (double)e; }
-#pragma unroll
-  for (int off = 32; off > 0; off >>= 1) part += __shfl_xor(part, off);
+  part = wave_sum_double(part);
   if (lane == 0) redd[wave] = part;
   __syncthreads();
   double sum = 0.0;
@@ -254,6 +307,11 @@ __global__ __launch_bounds__(1024) void attn_step_scores_kernel(const float* __r
   const int group = nh / nkv, kvd = nkv * hd, kh = h / group, ko = kh * hd;
   const int l = tid & 15, pg = tid >> 4, nj = hd >> 4, wave = tid >> 6;
   const bool own = pos < pbase + 256;              // this workgroup's positions hold the token's own
+  // the head's own loads first (waves 0 and 1), the keys' after: the norms and the turn wait for the first alone
+  const float* cs = rope + (long long)pos * rd;
+  RopeIn<4> rin;
+  const bool turns = wave == 0 || (wave == 1 && own);
+  if (turns) rope_head_load(rin, wave == 0 ? q + h * hd : k + ko, wave == 0 ? qn : kn, cs, hd, rd, tid & 63);
   float kv[4][16];
 #pragma unroll
   for (int u = 0; u < 4; u++) {
@@ -261,9 +319,7 @@ __global__ __launch_bounds__(1024) void attn_step_scores_kernel(const float* __r
 #pragma unroll
     for (int j = 0; j < 16; j++) kv[u][j] = j < nj ? kr[l + 16 * j] : 0.0f;
   }
-  const float* cs = rope + (long long)pos * rd;
-  if (wave == 0) rope_head_wave(q + h * hd, qn, cs, qsh, &scs[0], hd, rd, eps, neox, tid & 63);
-  if (wave == 1 && own) rope_head_wave(k + ko, kn, cs, ksh, &scs[1], hd, rd, eps, neox, tid & 63);
+  if (turns) rope_head_turn(rin, (wave == 0 ? qn : kn) != nullptr, wave == 0 ? qsh : ksh, &scs[wave], hd, rd, eps, neox, tid & 63);
   __syncthreads();
   if (own && h == kh * group && tid < hd) {
     kc[(long long)pos * kvd + ko + tid] = ksh[tid];
@@ -290,6 +346,51 @@ __global__ __launch_bounds__(1024) void attn_step_scores_kernel(const float* __r
   }
 }
 
+// Eight 16-byte LDS reads (32 floats from P on) into A##0 .. A##7 that the compiler does not wait for, and the wait
+// that hands those registers over once at most LEFT LDS reads asked for after them are still on their way (LDS
+// answers in order).  Between a read and its wait the program may ask LDS for nothing else but more of these reads.
+#define ILT_LDS_READ32_AHEAD(A, P)                                                                                                          \
+  asm volatile("ds_read_b128 %0, %8\n\tds_read_b128 %1, %8 offset:16\n\tds_read_b128 %2, %8 offset:32\n\tds_read_b128 %3, %8 offset:48\n\t" \
+               "ds_read_b128 %4, %8 offset:64\n\tds_read_b128 %5, %8 offset:80\n\tds_read_b128 %6, %8 offset:96\n\tds_read_b128 %7, %8 offset:112" \
+               : "=&v"(A##0), "=&v"(A##1), "=&v"(A##2), "=&v"(A##3), "=&v"(A##4), "=&v"(A##5), "=&v"(A##6), "=&v"(A##7)                   \
+               : "v"((u32)(uintptr_t)(ILT_LDS const void*)(P)) : "memory")
+#define ILT_LDS_READ32_WAIT(A, LEFT)                                                                                                        \
+  asm volatile("s_waitcnt lgkmcnt(" #LEFT ")" : "+v"(A##0), "+v"(A##1), "+v"(A##2), "+v"(A##3), "+v"(A##4), "+v"(A##5), "+v"(A##6), "+v"(A##7) :: "memory")
+#define ILT_CHAIN_ADD32(O, A)                                                                                                               \
+  do {                                                                                                                                      \
+    O = O + (A##0).x; O = O + (A##0).y; O = O + (A##0).z; O = O + (A##0).w; O = O + (A##1).x; O = O + (A##1).y; O = O + (A##1).z; O = O + (A##1).w;          \
+    O = O + (A##2).x; O = O + (A##2).y; O = O + (A##2).z; O = O + (A##2).w; O = O + (A##3).x; O = O + (A##3).y; O = O + (A##3).z; O = O + (A##3).w;          \
+    O = O + (A##4).x; O = O + (A##4).y; O = O + (A##4).z; O = O + (A##4).w; O = O + (A##5).x; O = O + (A##5).y; O = O + (A##5).z; O = O + (A##5).w;          \
+    O = O + (A##6).x; O = O + (A##6).y; O = O + (A##6).z; O = O + (A##6).w; O = O + (A##7).x; O = O + (A##7).y; O = O + (A##7).z; O = O + (A##7).w;          \
+  } while (0)
+
+// The chain of one column: o = ((0 + col[0]) + col[1]) + .. over npos floats of a row in LDS; last_read: the last
+// float of the row from which 32 can be read (the row is padded past npos).  The reads of 32 positions are on their
+// way while the 32 before them are added: left to itself the compiler moves every read down to its use, and a chain
+// of adds then waits for LDS once every 32 positions.
+__device__ __forceinline__ float chain_add_row(const float* col, int npos, int last_read) {
+  float o = 0.0f;
+  int p = 0;
+  typedef float f4v __attribute__((ext_vector_type(4)));
+  f4v v0, v1, v2, v3, v4, v5, v6, v7, w0, w1, w2, w3, w4, w5, w6, w7;
+  ILT_LDS_READ32_AHEAD(v, col);
+  for (; p + 64 <= npos; p += 64) {
+    ILT_LDS_READ32_AHEAD(w, col + p + 32);
+    ILT_LDS_READ32_WAIT(v, 8);
+    ILT_CHAIN_ADD32(o, v);
+    ILT_LDS_READ32_AHEAD(v, col + min(p + 64, last_read));
+    ILT_LDS_READ32_WAIT(w, 8);
+    ILT_CHAIN_ADD32(o, w);
+  }
+  ILT_LDS_READ32_WAIT(v, 0);
+  if (p + 32 <= npos) {                            // v holds positions p .. p+31
+    ILT_CHAIN_ADD32(o, v);
+    p += 32;
+  }
+  for (; p < npos; p++) o = o + col[p];
+  return o;
+}
+
 // softmax of one token's raw scores into sc (LDS) by the NT threads that call it (me = 0..NT-1): NT = 64, one
 // wave, or the whole workgroup of 256 with red/redd for the waves to meet.  PRE: the thread's raw scores
 // (positions me, me + NT, ..) are in pre already, at most eight of them.
@@ -303,8 +404,7 @@ __device__ __forceinline__ void attn_softmax(const float* __restrict__ rw, const
   } else {
     for (int p = me; p < npos; p += NT) { const float sv = rw[p]; sc[p] = sv; mx = fmaxf(mx, sv); }
   }
-#pragma unroll
-  for (int off = 32; off > 0; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off));
+  mx = wave_max_float(mx);
   if (NT > 64) {
     if (lane == 0) redf[wave] = mx;
     __syncthreads();
@@ -312,8 +412,7 @@ __device__ __forceinline__ void attn_softmax(const float* __restrict__ rw, const
   }
   double part = 0.0;
   for (int p = me; p < npos; p += NT) { const float e = ilt_expf_via_double(sc[p] - mx); sc[p] = e; part += (double)e; }
-#pragma unroll
-  for (int off = 32; off > 0; off >>= 1) part += __shfl_xor(part, off);
+  part = wave_sum_double(part);
   double sum = part;
   if (NT > 64) {
     if (lane == 0) redd[wave] = part;
@@ -428,14 +527,7 @@ __global__ __launch_bounds__(256) void attn_values_kernel(const float* __restric
     float o = 0.0f;
     int p = 0;
     if (TG == 1) {
-      for (; p + 32 <= npos; p += 32) {
-        float4 v4[8];
-#pragma unroll
-        for (int u = 0; u < 8; u++) v4[u] = *(const float4*)(col + p + 4 * u);
-#pragma unroll
-        for (int u = 0; u < 8; u++) { o = o + v4[u].x; o = o + v4[u].y; o = o + v4[u].z; o = o + v4[u].w; }
-      }
-      for (; p < npos; p++) o = o + col[p];
+      o = chain_add_row(col, npos, vpitch - 36);
     } else {
       for (; p + 16 <= npos; p += 16) {
         float4 s4[4], v4[4];
@@ -453,7 +545,137 @@ __global__ __launch_bounds__(256) void attn_values_kernel(const float* __restric
   }
 }
 
-// swiglu! (model.lisp:364-378) on n values: a = (a / (1 + e^-a)) * b, the exponential through double
+// One token's whole attention in one launch, for contexts of up to 1,024 positions: a workgroup of 1,024 threads a
+// (query head, CS columns of the values).  Each norms and turns its query head and its KV head's key itself
+// (waves 0 and 1), takes the head's scores for every position (attn_step_scores_kernel's sums; the keys of a head
+// come from L2 once for each of its hd/CS workgroups, which is what bounds the context), scales them, and adds its
+// CS columns as attn_values_kernel<1> does.  The group's first query head's first workgroup writes the key and the
+// value into the caches; the token's own key and value are taken from k and v, never from the caches.  NJ = hd/16.
+template <int NJ, int CS>
+__global__ __launch_bounds__(1024) void attn_step_fused_kernel(const float* __restrict__ q, const float* __restrict__ k, const float* __restrict__ v,
+                                                               const float* __restrict__ qn, const float* __restrict__ kn,
+                                                               const float* __restrict__ rope, float* __restrict__ kc, float* __restrict__ vc,
+                                                               float* __restrict__ out, int nh, int nkv, int rd, int pos, float eps, int neox,
+                                                               float scale, int vpitch) {
+  extern __shared__ __align__(16) float dyn[];
+  __shared__ float qsh[16 * NJ], ksh[16 * NJ], redf[16];
+  __shared__ double scs[2], redd[17];
+  constexpr int hd = 16 * NJ;
+  // the hardware deals consecutive workgroups to the eight dies in turn: die x takes the workgroups of consecutive heads
+  // (with 32 query heads on 8 KV heads, one KV head's), so a head's keys and values come from memory into one L2 only
+  const int nwg = gridDim.x, wg = (nwg & 7) ? (int)blockIdx.x : (int)(blockIdx.x & 7) * (nwg >> 3) + (int)(blockIdx.x >> 3);
+  const int ns = hd / CS, h = wg / ns, cs = wg - h * ns, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, npos = pos + 1;
+  const int group = nh / nkv, kvd = nkv * hd, kh = h / group, ko = kh * hd, vo = ko + CS * cs;
+  const int l = tid & 15, pg = tid >> 4, last = max(pos - 1, 0);
+  float* sc = dyn;                                 // 1,024 scores
+  float* vt = dyn + 1024;                          // the slice times the scores, a column a row of vpitch
+  // the keys of positions 256 b .. 256 b + 255 for this thread's four passes (rows before the token's own)
+  auto load_keys = [&](float (&kv)[4][NJ], int b) {
+#pragma unroll
+    for (int u = 0; u < 4; u++) {
+      const float* kr = kc + (long long)min(256 * b + 64 * u + pg, last) * kvd + ko;
+#pragma unroll
+      for (int j = 0; j < NJ; j++) kv[u][j] = kr[l + 16 * j];
+    }
+  };
+  // the head's own loads first (waves 0 and 1): the norms and the turn then wait for these alone
+  const float* cst = rope + (long long)pos * rd;
+  RopeIn<(NJ + 3) / 4> rin;
+  if (wave < 2) rope_head_load(rin, wave == 0 ? q + h * hd : k + ko, wave == 0 ? qn : kn, cst, hd, rd, lane);
+  float ka[4][NJ], kb[4][NJ];
+  load_keys(ka, 0);
+  // (the rest of the loads after the heads are turned: sixteen waves' loads take as long to ask for as the turn takes,
+  // and the workgroup would wait for the slowest wave's)
+  if (wave < 2) rope_head_turn(rin, (wave == 0 ? qn : kn) != nullptr, wave == 0 ? qsh : ksh, &scs[wave], hd, rd, eps, neox, lane);
+  __syncthreads();
+  load_keys(kb, 1);
+  // the slice: 16-byte piece i = position i / PP, part i % PP; the token's own row from v
+  constexpr int PP = CS / 4;
+  float4 r[PP];
+  const int total = npos * PP;
+#pragma unroll
+  for (int u = 0; u < PP; u++) {
+    const int i = min(tid + 1024 * u, total - 1), p = i / PP;
+    const float* src = p == pos ? v + vo : vc + (long long)p * kvd + vo;
+    r[u] = *(const float4*)(src + 4 * (i % PP));
+  }
+  if (h == kh * group && cs == 0 && tid < hd) {
+    kc[(long long)pos * kvd + ko + tid] = ksh[tid];
+    vc[(long long)pos * kvd + ko + tid] = v[ko + tid];
+  }
+  float qv[NJ];
+#pragma unroll
+  for (int j = 0; j < NJ; j++) qv[j] = qsh[l + 16 * j];
+  auto take_scores = [&](float (&kv)[4][NJ], int b) {
+#pragma unroll
+    for (int u = 0; u < 4; u++) {
+      const int p = 256 * b + 64 * u + pg;
+      if (p == pos) {
+#pragma unroll
+        for (int j = 0; j < NJ; j++) kv[u][j] = ksh[l + 16 * j];
+      }
+      float sacc = 0.0f;
+#pragma unroll
+      for (int j = 0; j < NJ; j++) sacc = sacc + kv[u][j] * qv[j];
+      sacc = sacc + ilt_dppf<ILT_DPP_SHL(4)>(sacc);
+      sacc = sacc + ilt_dppf<ILT_DPP_SHL(8)>(sacc);
+      sacc = sacc + ilt_dppf<ILT_DPP_SHL(1)>(sacc);
+      sacc = sacc + ilt_dppf<ILT_DPP_SHL(2)>(sacc);
+      if (l == 0 && p < npos) sc[p] = sacc * scale;
+    }
+  };
+  const int nb = (npos + 255) >> 8;                // 1 .. 4
+  take_scores(ka, 0);
+  if (nb > 2) load_keys(ka, 2);
+  if (nb > 1) take_scores(kb, 1);
+  if (nb > 3) load_keys(kb, 3);
+  if (nb > 2) take_scores(ka, 2);
+  if (nb > 3) take_scores(kb, 3);
+  __syncthreads();
+  // softmax (attn_softmax's steps with a position a thread)
+  const bool mine = tid < npos;
+  float mx = mine ? sc[tid] : -3.402823466e38f;
+  const float sv = mx;
+  mx = wave_max_float(mx);
+  if (lane == 0) redf[wave] = mx;
+  __syncthreads();
+  mx = redf[0];
+#pragma unroll
+  for (int w = 1; w < 16; w++) mx = fmaxf(mx, redf[w]);
+  const float e = mine ? ilt_expf_via_double(sv - mx) : 0.0f;
+  const double part = wave_sum_double((double)e);
+  if (lane == 0) redd[wave] = part;
+  if (mine) sc[tid] = e;
+  __syncthreads();
+  double sum = redd[0];
+#pragma unroll
+  for (int w = 1; w < 16; w++) sum += redd[w];
+  // the CPU adds the terms one after another: take its sum where the order could show in the rounded reciprocal
+  const double slack = sum * ((double)(npos + 8) * 0x1p-51);
+  if ((float)(1.0 / (sum - slack)) != (float)(1.0 / (sum + slack))) {      // the same in every thread
+    if (tid == 0) { double s2 = 0.0; for (int p = 0; p < npos; p++) s2 += (double)sc[p]; redd[16] = s2; }
+    __syncthreads();
+    sum = redd[16];
+  }
+  const float inv = (float)(1.0 / sum);
+  if (mine) sc[tid] = e * inv;
+  __syncthreads();
+#pragma unroll
+  for (int u = 0; u < PP; u++) {
+    const int i = tid + 1024 * u;
+    if (i < total) {
+      float* dst = vt + (4 * (i % PP)) * vpitch + i / PP;
+      const float sp = sc[i / PP];
+      dst[0] = sp * r[u].x; dst[vpitch] = sp * r[u].y; dst[2 * vpitch] = sp * r[u].z; dst[3 * vpitch] = sp * r[u].w;
+    }
+  }
+  __syncthreads();
+  if (tid < CS) {
+    const float* col = vt + tid * vpitch;
+    out[h * hd + CS * cs + tid] = chain_add_row(col, npos, vpitch - 36);
+  }
+}
+
 // The same for contexts whose value slice no longer fits LDS (2,049 to 8,192 positions): the slice comes through
 // LDS in tiles of kValTile positions, and a chain carries its sum from tile to tile -- position after position all
 // the same.  TG 1: the token's scores are taken and scaled here and stay in LDS.  TG 16 (a prompt's chunk): the
@@ -596,6 +818,7 @@ __global__ __launch_bounds__(256) void argmax_last_kernel(const float* __restric
   if (threadIdx.x == 0) { const float v0 = v[0]; out[0] = (v0 != v0 || b.i == 0x7FFFFFFF) ? 0 : b.i; }
 }
 
+// swiglu! (model.lisp:364-378) on n values: a = (a / (1 + e^-a)) * b, the exponential through double
 __global__ __launch_bounds__(256) void swiglu_rows_kernel(float* __restrict__ a, const float* __restrict__ b, long long n) {
   const long long i = (long long)blockIdx.x * 256 + threadIdx.x;
   if (i < n) { const float g = a[i]; a[i] = (g / (1.0f + ilt_expf_via_double(-g))) * b[i]; }
@@ -692,6 +915,27 @@ hipError_t ilt_k_attn_step(const float* q, const float* k, const float* v, const
   const size_t smem = sizeof(float) * ((size_t)smax + 16 * (size_t)vpitch);
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) dev = 0;
+  // up to 1,024 positions, heads of 64 or 128: one launch ("ILT_ATTN_FUSED=0": the two launches below, for tests)
+  static const bool fused_ok = []{ const char* f = getenv("ILT_ATTN_FUSED"); return !(f && f[0] == '0'); }();
+  if (fused_ok && ctx <= 1024 && (hd == 64 || hd == 128)) {
+    // 16 columns a workgroup: with 32, half as many workgroups read a head's keys, and the launch is no faster (each
+    // workgroup takes as long over them: 9,000 cycles for 640 positions, its own loads and sums, not L2's bandwidth)
+    static bool set[64] = {};
+    if (!set[dev]) {
+      hipError_t e = hipFuncSetAttribute((const void*)attn_step_fused_kernel<4, 16>, hipFuncAttributeMaxDynamicSharedMemorySize, 80 * 1024);
+      if (e == hipSuccess) e = hipFuncSetAttribute((const void*)attn_step_fused_kernel<8, 16>, hipFuncAttributeMaxDynamicSharedMemorySize, 80 * 1024);
+      if (e != hipSuccess) return e;
+      set[dev] = true;
+    }
+    const size_t fsmem = sizeof(float) * (1024 + 16 * (size_t)vpitch);
+    if (hd == 64)
+      hipLaunchKernelGGL((attn_step_fused_kernel<4, 16>), dim3(nh * 4), dim3(1024), fsmem, st, q, k, v, qn, kn, rope, kc, vc, out, nh, nkv, rd, pos, eps,
+                         neox, scale, vpitch);
+    else
+      hipLaunchKernelGGL((attn_step_fused_kernel<8, 16>), dim3(nh * 8), dim3(1024), fsmem, st, q, k, v, qn, kn, rope, kc, vc, out, nh, nkv, rd, pos, eps,
+                         neox, scale, vpitch);
+    return hipGetLastError();
+  }
   hipLaunchKernelGGL(attn_step_scores_kernel, dim3(nh, (ctx + 255) / 256), dim3(1024), 0, st, q, k, v, qn, kn, rope, kc, vc, scratch, nh, nkv, hd, rd,
                      pos, eps, neox, scale, smax);
   if (ctx > 2048) {

@@ -305,10 +305,12 @@ int ilt_qk_rope(uint64_t stream, float* q, float* k, const float* v, const float
                 float* vc, int nh, int nkv, int hd, int rd, int pos0, float eps, int neox, int ntok);
 int ilt_attn_rows(uint64_t stream, const float* q, const float* kc, const float* vc, float* out, int nh, int nkv, int hd, int pos0, int ntok,
                   float* scratch);
-/* ilt_qk_rope and ilt_attn_rows of one token at position pos (< 8192) with one launch fewer: the launch that takes
-   the scores norms and turns the query heads and the token's key itself and writes the caches' rows at pos.  out is
-   what ilt_attn_rows gives after ilt_qk_rope, bit for bit; q and k are left as they came (not normed, not turned).
-   scratch: nh * ((pos + 4) & ~3) floats. */
+/* ilt_qk_rope and ilt_attn_rows of one token at position pos (< 8192) in fewer launches.  Up to position 1023 with
+   heads of 64 or 128: one launch, a workgroup a (query head, 16 columns of the values), each norming and turning its
+   head and the token's key itself and taking all of the head's scores (scratch is not touched).  Otherwise two: the
+   launch that takes the scores norms and turns the query heads and the token's key and writes the caches' rows at
+   pos.  Either way out is what ilt_attn_rows gives after ilt_qk_rope, bit for bit; q and k are left as they came
+   (not normed, not turned).  scratch: nh * ((pos + 4) & ~3) floats. */
 int ilt_attn_step(uint64_t stream, const float* q, const float* k, const float* v, const float* qn, const float* kn, const float* rope, float* kc,
                   float* vc, float* out, int nh, int nkv, int hd, int rd, int pos, float eps, int neox, float* scratch);
 

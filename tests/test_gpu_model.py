@@ -230,6 +230,18 @@ def test_small_decoder_long_contexts(dev):
     assert same == 3
 
 
+def test_one_launch_attention_up_to_1024_positions(dev):
+    """A token's attention in one launch (contexts of up to 1,024 positions, heads of 64 and of 128): decode steps in
+    every one of its four blocks of 256 positions, on the blocks' edges, and across position 1023 -> 1024, where the
+    two launches take over."""
+    from illatio_amd import model
+    for seed, hd, nh, nkv in ((21, 64, 4, 2), (22, 128, 4, 1)):
+        host = model.synth_model(seed, d=256, ffn=512, nh=nh, nkv=nkv, hd=hd, nl=2, vocab=500)
+        for nprompt, ndecode in ((250, 10), (508, 8), (764, 8), (1018, 10)):
+            same, _ = run_greedy(dev, host, nprompt=nprompt, ndecode=ndecode, chunk=512, nctx=nprompt + ndecode + 2, seed=seed + nprompt)
+            assert same == ndecode
+
+
 def test_config_2_width_four_layers_128_greedy_tokens(dev):
     """Config 2's layer at its full width (hidden 2560, intermediate 9728, 32 query and 8 KV heads of 128, vocabulary
     151936), four layers: a 64-token prompt through the prefill products, then 128 greedy tokens, each step's logits
