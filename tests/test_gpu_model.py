@@ -70,14 +70,14 @@ def test_small_decoder_prefill_chunks_and_decode(dev):
     run_greedy(dev, host, nprompt=9, ndecode=2, chunk=64, nctx=16, seed=3)
 
 
-@pytest.mark.parametrize("norms", [True, False])
-def test_attn_step_is_qk_rope_then_attn_rows(dev, norms):
-    """One token's attention as two launches (ilt_attn_step) against the three it stands for, at positions in the
-    first and in later blocks of 256 scores and on a block's edges: the output and the caches' rows bit for bit,
-    q and k untouched."""
+@pytest.mark.parametrize("norms,nh,nkv,hd", [(True, 8, 2, 64), (False, 8, 2, 64), (True, 3, 1, 64), (True, 4, 2, 32)])
+def test_attn_step_is_qk_rope_then_attn_rows(dev, norms, nh, nkv, hd):
+    """One token's attention as one launch (heads of 64) or two (heads of 32) (ilt_attn_step) against the three it
+    stands for, at positions in the first and in later blocks of 256 scores and on a block's edges: the output and the
+    caches' rows bit for bit, q and k untouched."""
     import ctypes as C
     from illatio_amd import hip
-    nh, nkv, hd, nctx, eps = 8, 2, 64, 600, 1e-6
+    nctx, eps = 600, 1e-6                             # (3 heads: 12 workgroups, not a multiple of the eight dies)
     rng = synth.make_rng(11)
     f = lambda *sh: (rng.standard_normal(sh) * 1.5).astype(np.float32)
     up = lambda a: (lambda b: (hip.hip_upload_vector(b, a), b)[1])(hip.hip_alloc(dev, a.nbytes))
