@@ -364,6 +364,22 @@ __global__ __launch_bounds__(1024) void attn_step_scores_kernel(const float* __r
     O = O + (A##6).x; O = O + (A##6).y; O = O + (A##6).z; O = O + (A##6).w; O = O + (A##7).x; O = O + (A##7).y; O = O + (A##7).z; O = O + (A##7).w;          \
   } while (0)
 
+// The same for a chain of products: 16 scores from PS into S##0 .. S##3 and 16 values from PV into V##0 .. V##3.
+#define ILT_LDS_READ16X2_AHEAD(S, V, PS, PV)                                                                                                \
+  asm volatile("ds_read_b128 %0, %8\n\tds_read_b128 %1, %8 offset:16\n\tds_read_b128 %2, %8 offset:32\n\tds_read_b128 %3, %8 offset:48\n\t" \
+               "ds_read_b128 %4, %9\n\tds_read_b128 %5, %9 offset:16\n\tds_read_b128 %6, %9 offset:32\n\tds_read_b128 %7, %9 offset:48"   \
+               : "=&v"(S##0), "=&v"(S##1), "=&v"(S##2), "=&v"(S##3), "=&v"(V##0), "=&v"(V##1), "=&v"(V##2), "=&v"(V##3)                   \
+               : "v"((u32)(uintptr_t)(ILT_LDS const void*)(PS)), "v"((u32)(uintptr_t)(ILT_LDS const void*)(PV)) : "memory")
+#define ILT_LDS_READ16X2_WAIT(S, V, LEFT)                                                                                                   \
+  asm volatile("s_waitcnt lgkmcnt(" #LEFT ")" : "+v"(S##0), "+v"(S##1), "+v"(S##2), "+v"(S##3), "+v"(V##0), "+v"(V##1), "+v"(V##2), "+v"(V##3) :: "memory")
+#define ILT_CHAIN_MULADD4(O, S, V)                                                                                                          \
+  do {                                                                                                                                      \
+    const float a0_ = (S).x * (V).x, a1_ = (S).y * (V).y, a2_ = (S).z * (V).z, a3_ = (S).w * (V).w;                                         \
+    O = O + a0_; O = O + a1_; O = O + a2_; O = O + a3_;                                                                                     \
+  } while (0)
+#define ILT_CHAIN_MULADD16(O, S, V)                                                                                                         \
+  do { ILT_CHAIN_MULADD4(O, S##0, V##0); ILT_CHAIN_MULADD4(O, S##1, V##1); ILT_CHAIN_MULADD4(O, S##2, V##2); ILT_CHAIN_MULADD4(O, S##3, V##3); } while (0)
+
 // The chain of one column: o = ((0 + col[0]) + col[1]) + .. over npos floats of a row in LDS; last_read: the last
 // float of the row from which 32 can be read (the row is padded past npos).  The reads of 32 positions are on their
 // way while the 32 before them are added: left to itself the compiler moves every read down to its use, and a chain
@@ -388,6 +404,32 @@ __device__ __forceinline__ float chain_add_row(const float* col, int npos, int l
     p += 32;
   }
   for (; p < npos; p++) o = o + col[p];
+  return o;
+}
+
+// The chain of one column with the products made on the way: o = ((0 + sc[0] col[0]) + sc[1] col[1]) + ..; the reads
+// of 16 positions on their way while the 16 before them are multiplied and added.  last_read: the last float of col's
+// row from which 16 can be read; sc's row may be read 16 floats past npos.
+__device__ __forceinline__ float chain_muladd_row(const float* sc, const float* col, int npos, int last_read) {
+  typedef float f4v __attribute__((ext_vector_type(4)));
+  float o = 0.0f;
+  int p = 0;
+  f4v s0, s1, s2, s3, v0, v1, v2, v3, t0, t1, t2, t3, w0, w1, w2, w3;
+  ILT_LDS_READ16X2_AHEAD(s, v, sc, col);
+  for (; p + 32 <= npos; p += 32) {
+    ILT_LDS_READ16X2_AHEAD(t, w, sc + p + 16, col + p + 16);
+    ILT_LDS_READ16X2_WAIT(s, v, 8);
+    ILT_CHAIN_MULADD16(o, s, v);
+    ILT_LDS_READ16X2_AHEAD(s, v, sc + p + 32, col + min(p + 32, last_read));
+    ILT_LDS_READ16X2_WAIT(t, w, 8);
+    ILT_CHAIN_MULADD16(o, t, w);
+  }
+  ILT_LDS_READ16X2_WAIT(s, v, 0);
+  if (p + 16 <= npos) {                            // s, v hold positions p .. p+15
+    ILT_CHAIN_MULADD16(o, s, v);
+    p += 16;
+  }
+  for (; p < npos; p++) o = o + sc[p] * col[p];
   return o;
 }
 
@@ -524,24 +566,7 @@ __global__ __launch_bounds__(256) void attn_values_kernel(const float* __restric
     const int tt = tid >> 4, c = tid & 15, npos = pos0 + t0 + tt + 1;
     const float* sc = scores + tt * lp;
     const float* col = vt + c * vpitch;
-    float o = 0.0f;
-    int p = 0;
-    if (TG == 1) {
-      o = chain_add_row(col, npos, vpitch - 36);
-    } else {
-      for (; p + 16 <= npos; p += 16) {
-        float4 s4[4], v4[4];
-#pragma unroll
-        for (int u = 0; u < 4; u++) { s4[u] = *(const float4*)(sc + p + 4 * u); v4[u] = *(const float4*)(col + p + 4 * u); }
-#pragma unroll
-        for (int u = 0; u < 4; u++) {
-          const float a0 = s4[u].x * v4[u].x, a1 = s4[u].y * v4[u].y, a2 = s4[u].z * v4[u].z, a3 = s4[u].w * v4[u].w;
-          o = o + a0; o = o + a1; o = o + a2; o = o + a3;
-        }
-      }
-      for (; p < npos; p++) o = o + sc[p] * col[p];
-    }
-    out[((long long)(t0 + tt) * nh + h) * hd + 16 * cs + c] = o;
+    out[((long long)(t0 + tt) * nh + h) * hd + 16 * cs + c] = TG == 1 ? chain_add_row(col, npos, vpitch - 36) : chain_muladd_row(sc, col, npos, vpitch - 16);
   }
 }
 
