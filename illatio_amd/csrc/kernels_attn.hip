@@ -19,29 +19,6 @@ __device__ __forceinline__ void wave_lds_sync() {
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
-// A wave's maximum and a wave's sum of doubles, the same in every lane: butterflies over a row's 16 lanes through DPP,
-// the four rows through readlane -- a tenth of the trips through LDS that __shfl_xor's permutes make.  All 64 lanes
-// must be active.  (The order of the adds is not the CPU's: callers check whether that could show.)
-template <int CTRL> __device__ __forceinline__ double dpp_double(double v) {
-  return __hiloint2double(ilt_dpp<CTRL>(__double2hiint(v)), ilt_dpp<CTRL>(__double2loint(v)));
-}
-__device__ __forceinline__ double readlane_double(double v, int lane) {
-  return __hiloint2double(__builtin_amdgcn_readlane(__double2hiint(v), lane), __builtin_amdgcn_readlane(__double2loint(v), lane));
-}
-__device__ __forceinline__ double wave_sum_double(double v) {
-  v += dpp_double<ILT_DPP_XOR1>(v);
-  v += dpp_double<ILT_DPP_XOR2>(v);
-  v += dpp_double<ILT_DPP_HALF_MIRROR>(v);
-  v += dpp_double<ILT_DPP_ROW_MIRROR>(v);
-  return (readlane_double(v, 0) + readlane_double(v, 16)) + (readlane_double(v, 32) + readlane_double(v, 48));
-}
-__device__ __forceinline__ float wave_max_float(float v) {
-  v = ilt_max16(v);
-  const int b = __float_as_int(v);
-  return fmaxf(fmaxf(__int_as_float(__builtin_amdgcn_readlane(b, 0)), __int_as_float(__builtin_amdgcn_readlane(b, 16))),
-               fmaxf(__int_as_float(__builtin_amdgcn_readlane(b, 32)), __int_as_float(__builtin_amdgcn_readlane(b, 48))));
-}
-
 // One head by one wave: x (hd floats) into xs (LDS): rmsnorm! of the head when its weights are given
 // (model.lisp:205-216: the squares, rounded to floats, added in double one after another), then rope-head!
 // from the position's table cs (cos, then sin, rd/2 each).  Only this wave touches xs and sd.  The lanes add

@@ -480,8 +480,7 @@ __device__ __forceinline__ double norm_partial(const float* __restrict__ x, int 
 // PART: this thread's part of the sum; all threads of the workgroup call this.
 __device__ __forceinline__ float norm_scale(double part, const float* __restrict__ x, int n, float eps, int seq) {
   __shared__ double red[kWaves];
-#pragma unroll
-  for (int off = 32; off > 0; off >>= 1) part += __shfl_xor(part, off);
+  part = wave_sum_double(part);
   if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = part;
   __syncthreads();
   double sum = red[0];
@@ -816,8 +815,7 @@ constexpr int kStreamWaves = 16, kStreamThreads = 64 * kStreamWaves, kStagers = 
 // or not the sum is taken again in the CPU's order, so that they need not know).
 __device__ __forceinline__ float norm_scale_stagers(double part, const float* __restrict__ x, int n, float eps, int seq) {
   __shared__ double red[kStagers];
-#pragma unroll
-  for (int off = 32; off > 0; off >>= 1) part += __shfl_xor(part, off);
+  part = wave_sum_double(part);
   if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = part;
   ilt_barrier_lds();
   double sum = red[0];
