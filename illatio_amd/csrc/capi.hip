@@ -350,8 +350,9 @@ int ilt_d4_mv_q2_k_f32(uint64_t stream, int ncols, int nrows, int row_bytes, int
                       nullptr, x, nullptr, 0.0f, dst, sel);
 }
 
-int ilt_d4_mvq8_glu(uint64_t stream, int rows, int cols, const int8_t* gq, const uint16_t* gd, const int8_t* uq,
-                    const uint16_t* ud, const float* x, float clamp, float* mid) {
+// route: a token's routing for the launch to carry along, or null; its done says whether the launch did
+static int mvq8_glu(uint64_t stream, int rows, int cols, const int8_t* gq, const uint16_t* gd, const int8_t* uq,
+                    const uint16_t* ud, const float* x, float clamp, float* mid, IltRouteAlong* route) {
   ILT_REQUIRE(rows >= 0 && cols > 0 && cols % 32 == 0);
   if (rows == 0) return ILT_OK;
   ILT_REQUIRE(gq && gd && uq && ud && x && mid && ((uintptr_t)gq & 15) == 0 && ((uintptr_t)uq & 15) == 0 && ((uintptr_t)x & 15) == 0);
@@ -362,7 +363,15 @@ int ilt_d4_mvq8_glu(uint64_t stream, int rows, int cols, const int8_t* gq, const
     p.mat[i].rows = rows; p.mat[i].fmt = ILT_Q8_0; p.mat[i].row_bytes = cols;
   }
   p.cols = cols; p.xf = x; p.f16_scale = 0; p.glu = 2; p.clamp = clamp;
-  return (int)ilt_gemv_launch(p, 1, S(stream));
+  if (route) { p.route = *route; p.route.done = 0; }
+  const int e = (int)ilt_gemv_launch(p, 1, S(stream));
+  if (route) route->done = e == ILT_OK ? p.route.done : 0;
+  return e;
+}
+
+int ilt_d4_mvq8_glu(uint64_t stream, int rows, int cols, const int8_t* gq, const uint16_t* gd, const int8_t* uq,
+                    const uint16_t* ud, const float* x, float clamp, float* mid) {
+  return mvq8_glu(stream, rows, cols, gq, gd, uq, ud, x, clamp, mid, nullptr);
 }
 
 int ilt_dequant_rows(uint64_t stream, int gguf_type, const void* w, const uint16_t* wd, const int32_t* rows_idx,
@@ -467,8 +476,11 @@ int step_run(uint64_t stream, uint8_t* ws, int ne, int nu, int d, int ff, float 
   float *w = (float*)(ws + l.w), *smid = (float*)(ws + l.smid), *sout = (float*)(ws + l.sout);
   float *bm = (float*)(ws + l.bm), *bd = (float*)(ws + l.bd);
   const int grb = d / 256 * 66, drb = ff / 256 * 84;
-  ILT_TRY((hipError_t)ilt_d4_route(stream, ne, nu, 0, scale, bias ? 1 : 0, logits, bias, nullptr, nullptr, sel, w, 1));
-  ILT_TRY((hipError_t)ilt_d4_mvq8_glu(stream, ff, d, wt->sgate_q, wt->sgate_d, wt->sup_q, wt->sup_d, x, clamp, smid));
+  // the routing rides along with the shared expert's gate/up launch (one of its waves routes while the rows stream
+  // in); where that launch cannot take it, a launch of its own
+  IltRouteAlong route = {logits, bias, sel, w, ne, nu, scale, 0};
+  ILT_TRY((hipError_t)mvq8_glu(stream, ff, d, wt->sgate_q, wt->sgate_d, wt->sup_q, wt->sup_d, x, clamp, smid, &route));
+  if (!route.done) ILT_TRY((hipError_t)ilt_d4_route(stream, ne, nu, 0, scale, bias ? 1 : 0, logits, bias, nullptr, nullptr, sel, w, 1));
   ilt_mv_desc down = {ILT_Q8_0, d, wt->sdown_q, wt->sdown_d, sout, nullptr};
   ILT_TRY((hipError_t)ilt_mv_multi(stream, 1, &down, ff, nullptr, nullptr, nullptr, smid, 0, 0, 0));
   ILT_TRY((hipError_t)ilt_d4_mv_glu_iq2_xxs(stream, d, ff, grb, 0, wt->gate_bytes, 0, ff, wt->slots, sel, nu, x, w, clamp, bm));

@@ -29,7 +29,18 @@ struct IltGemvMat {
   int rq, rr;                // rows / nbat and rows % nbat: batch i is rq rows, one more for the first rr (set at launch)
 };
 
+// A token's d4-route carried along by a product launch (the streamed variant, Q8_0): one of the activation waves of the
+// first workgroup routes once its own work is done, while the rows stream in.  logits null: none.  done: set by
+// ilt_gemv_launch when the launch it made takes the routing along (otherwise the caller launches d4_route itself).
+struct IltRouteAlong {
+  const float* logits; const float* bias;    // ne logits; ne biases or null
+  uint32_t* sel; float* wout;                // nu slots each
+  int ne, nu; float scale;
+  int done;
+};
+
 struct IltGemvParams {
+  IltRouteAlong route;
   IltGemvMat mat[4];         // up to four matrices sharing the activations
   int nmat;
   const uint64_t* ptrs;      // experts: grid y's matrices are at ptrs[y] + mat[i].add,

@@ -22,6 +22,7 @@
 #include "ilt_device.h"
 #include "ilt_iq2xxs_tables.h"
 #include "ilt_kernels.h"
+#include "ilt_route.h"
 #include <type_traits>
 
 namespace {
@@ -874,6 +875,14 @@ __global__ __launch_bounds__(kStreamThreads) void gemv_stream_kernel(IltGemvPara
       for (int i = threadIdx.x; i < S; i += 64 * kStagers) lxs[i] = p.xs[i];
     }
     ilt_barrier_lds();
+    if constexpr (q8 && !EARLY) {
+      // a token's routing carried along: this wave has nothing left to do while the rows stream in
+      if (p.route.logits && blockIdx.x == 0 && wave == 0) {
+        __shared__ u32 r_idx[64];
+        __shared__ float r_sc[64];
+        route_token<4>(lane, p.route.ne, p.route.nu, p.route.scale, p.route.logits, p.route.bias, nullptr, p.route.sel, p.route.wout, r_idx, r_sc);
+      }
+    }
     return;
   }
   if (wave < kStagers) {
@@ -1170,6 +1179,9 @@ static hipError_t gemv_stream_launch(IltGemvParams& p, int fset, int nz, hipStre
     }
     if (early) { g_streamed_launches++; return hipGetLastError(); }
   }
+  // a routing to carry along goes with the Q8_0 kernel only, for up to 256 experts (four a lane)
+  if (p.route.logits) p.route.done = fset == ILT_Q8_0 && p.route.ne <= 256 && p.route.nu <= 64 && p.route.nu <= p.route.ne ? 1 : 0;
+  if (p.route.logits && !p.route.done) p.route.logits = nullptr;
   switch (fset) {
     case 0: hipLaunchKernelGGL(gemv_stream_kernel<0>, grid, dim3(kStreamThreads), smem, st, p); break;
     case ILT_Q4_K: hipLaunchKernelGGL(gemv_stream_kernel<ILT_Q4_K>, grid, dim3(kStreamThreads), smem, st, p); break;

@@ -158,10 +158,12 @@ def test_moe_decode_step_of_config_4_with_256_experts(dev, clamp):
         moe = ds4f.ffn_tail(dev, pool, hsel, hw, nb, sout, clamp)
         fused = ds4f.ffn_step_fused(dev, pool, sh, hsel, hw, nb, clamp)
         ondev = ds4f.ffn_step_device(dev, pool, sh, lb, nb, ne, nu, 1.5, clamp)
-        for name, b in (("12 launches", moe), ("5 launches", fused), ("routing on the device", ondev)):
+        call = hip.hip_alloc(dev, 4 * d)                        # one call into the library: the routing over all 256 experts
+        ds4f.ffn_step_call(dev, pool, sh, lb, nb, call, ne, nu, 1.5, clamp)      # carried along by the shared expert's gate/up launch
+        for name, b in (("12 launches", moe), ("5 launches", fused), ("routing on the device", ondev), ("one call", call)):
             got = hip.hip_floats(b, d)
             assert np.array_equal(bits(got), bits(want)), (name, trial, np.abs(got - want).max())
-        for b in (lb, nb, sel, w, sout, moe, fused, ondev):
+        for b in (lb, nb, sel, w, sout, moe, fused, ondev, call):
             hip.hip_free(b)
     assert {0, 128, 255} <= seen and len(seen) > 12
     pool.free(); sh.free()

@@ -217,6 +217,17 @@ def test_moe_decode_step_bit_exact(dev, ne, d, ff, nu, clamp):
     small = hip.DBuf(ws.ptr, ws.bytes - 256, dev)
     with pytest.raises(hip.HipError):
         ds4f.ffn_step_call(dev, pool, sh, lb, nb, out, ne, nu, 1.5, clamp, wsbuf=small)
+    # scores that are NaN (the routing's slow branch, here inside the launch that carries the routing along at the
+    # large shape): the step ends normally, NaN where the CPU path's result is NaN and its bits elsewhere
+    for where in ([1], list(range(0, ne, 2)), list(range(ne))):
+        lg = logits.copy(); lg[where] = np.nan
+        want, _, _ = orc.moe_token(gate, up, down, sg, su, sd, d, ff, ne, nu, 1.5, clamp, lg, norm)
+        hip.hip_upload_vector(lb, lg)
+        ds4f.ffn_step_call(dev, pool, sh, lb, nb, out, ne, nu, 1.5, clamp, wsbuf=ws)
+        got = hip.hip_floats(out, d)
+        assert np.array_equal(np.isnan(got), np.isnan(want)), where
+        ok = ~np.isnan(want)
+        assert np.array_equal(bits(got[ok]), bits(want[ok])), where
     for b in (lb, nb, bb, out, ws):
         hip.hip_free(b)
     pool.free(); sh.free()
