@@ -27,7 +27,7 @@ Other workloads (--workload), each the benchmark configuration of the same numbe
   c4  MoE decode step: 256 resident experts (IQ2_XXS gate/up, Q2_K down), top-6, the Q8_0
       shared expert, rotating over 3 layers' pools (5.4 GB); routing tables made beforehand;
       --mode fused (default): 5 launches a step; --mode single: the reference's 12;
-      --mode device: routing on the device inside the step (6 launches, no host tables)
+      --mode device: routing on the device inside the step, one call into the library (5 launches, no host tables)
   c5  MoE prefill chunk: 4096 tokens, Zipf(1.1)-skewed top-6 routing, route -> group ->
       gather -> grouped gate, up -> gated activation -> grouped down -> ordered sum
 Weights and activations are synthetic and seeded (illatio_amd/synth.py); inputs are resident
@@ -729,7 +729,7 @@ def main():
     ap.add_argument("--norm", action="store_true", help="c2: include each layer's two norms and the output norm (inside the product launches in fused mode)")
     ap.add_argument("--mode", default="fused", choices=["fused", "fused-q", "single", "device"],
                     help="c4: fused = 5 launches a step, single = the reference's sequence of 12 (both with the routing done beforehand on the host, as the "
-                         "reference routes on the CPU), device = the routing kernel inside the step and the expert kernels indexing the slot table by its result (6 launches).  c2: fused = Q/K/V in one launch, gate+up in one, activations quantized inside the product "
+                         "reference routes on the CPU), device = the routing inside the step (carried along by the shared expert's gate/up launch), the expert kernels indexing the slot table by its result, one call into the library (5 launches).  c2: fused = Q/K/V in one launch, gate+up in one, activations quantized inside the product "
                          "kernels; fused-q = the same launches after separate quantizer launches; "
                          "single = one launch per matrix after separate quantizer launches")
     args = ap.parse_args()

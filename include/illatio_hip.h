@@ -218,9 +218,10 @@ int ilt_d4_mvq8_glu(uint64_t stream, int rows, int cols, const int8_t* gq, const
 
 /* One token's FFN past the router in one call: DK-FFN-HEAD's shared expert and DK-FFN-TAIL
    (cuda-ds4f.lisp:883-956) with the routing left on the device (the reference copies the
-   logits out, waits and routes on the CPU in every layer, :991-999).  Six launches on stream:
-   d4_route, d4_mvq8_glu, the shared expert's down, d4_mv_glu_iq2_xxs and d4_mv_q2_k_f32 indexed
-   by d4_route's sel, d4_moe_sum; moe[d] = the nu routed experts' rows in slot order + the shared
+   logits out, waits and routes on the CPU in every layer, :991-999).  Five launches on stream:
+   d4_mvq8_glu (one of whose waves does d4_route's work while the rows stream in: up to 256 experts and a
+   shared expert large enough for the streamed product, else d4_route is a sixth launch), the shared
+   expert's down, d4_mv_glu_iq2_xxs and d4_mv_q2_k_f32 indexed by the routing's sel, d4_moe_sum; moe[d] = the nu routed experts' rows in slot order + the shared
    expert's, with the CPU path's bits (d4-ffn without HC, ds4f.lisp:980-992).  Nothing is
    allocated, freed or waited for.  The intermediate results (sel, weights, the two gated
    activations, the shared expert's row, one down row per slot) live in ws, 256-byte aligned,
@@ -317,7 +318,8 @@ int ilt_attn_step(uint64_t stream, const float* q, const float* k, const float* 
 /* One token through the whole dense decoder in one call: what the host loop of cuda-forward-n queues for one
    token (cuda-dense.lisp:380-432; the CPU's forward-1, model.lisp:396-462) -- embedding row, then per layer the
    Q/K/V products with the norm inside, ilt_attn_step, wo onto the residual, gate/up with the norm and the gated
-   activation inside, down onto the residual, and (want_logits) the output norm and head: 6 launches a layer + 2.
+   activation inside, down onto the residual, and (want_logits) the output norm and head: 5 launches a layer + 2 while
+   the context is at most 1,024 positions, 6 beyond.
    The structs are read on the host during the call; every pointer in them is device memory but `layers`.
    Matrices as dense uploads hold them (Q8_0 split into quants and scales, Q6_K in 212-byte blocks).  pos < 8192
    (the attention's scratch), the caches hold at least pos + 1 positions, rope at least (pos + 1) * rd floats.

@@ -197,7 +197,8 @@ def test_moe_decode_step_bit_exact(dev, ne, d, ff, nu, clamp):
         ondev = ds4f.ffn_step_device(dev, pool, sh, lb, nb, ne, nu, 1.5, clamp)
         got = hip.hip_floats(ondev, d)
         assert np.array_equal(bits(got), bits(want)), np.abs(got - want).max()
-        # the same six launches queued by one call into the library, its intermediates in a caller's workspace
+        # the same step queued by one call into the library (the routing carried along by the shared expert's gate/up
+        # launch at the large shape), its intermediates in a caller's workspace
         out = hip.hip_alloc(dev, 4 * d)
         ds4f.ffn_step_call(dev, pool, sh, lb, nb, out, ne, nu, 1.5, clamp)
         got = hip.hip_floats(out, d)

@@ -1,5 +1,5 @@
 """ilt_d4_ffn_step_noalloc, the entry point that allocates nothing: its output against
-ilt_d4_ffn_step's (the same six launches with the intermediates in a caller's workspace), bit
+ilt_d4_ffn_step's (the same launches with the intermediates in a caller's workspace), bit
 for bit, on two calls in a row of which the second is the smaller one -- the library's array
 still holds the first call's contents then."""
 import ctypes as C
