@@ -805,7 +805,17 @@ int ilt_argmax(uint64_t stream, const float* v, int n, int32_t* out, void* scrat
 }
 
 // ---- one token through the dense decoder: the launches of the single calls, queued in one ----------
-static ilt_mv_desc mv_of(const ilt_dense_mat& w, float* y) { return {w.gguf_type, w.rows, w.w, w.wd, y, nullptr}; }
+static ilt_mv_desc mv_of(const ilt_dense_mat& w, float* y, const float* bias = nullptr) { return {w.gguf_type, w.rows, w.w, w.wd, y, bias}; }
+// Q/K/V with the norm inside: one launch where the three share an activation format (all Q8_0, or K-quants), else one each
+static int qkv_norm(uint64_t stream, const ilt_mv_desc (&qkv)[3], int d, const float* x, const float* norm, float eps) {
+  const bool q8[3] = {qkv[0].gguf_type == ILT_TYPE_Q8_0, qkv[1].gguf_type == ILT_TYPE_Q8_0, qkv[2].gguf_type == ILT_TYPE_Q8_0};
+  if (q8[0] == q8[1] && q8[1] == q8[2]) return ilt_mv_multi_norm(stream, 3, qkv, d, x, norm, eps, 0, 1, 0);
+  for (int i = 0; i < 3; i++) {
+    const int e = ilt_mv_multi_norm(stream, 1, &qkv[i], d, x, norm, eps, 0, 1, 0);
+    if (e) return e;
+  }
+  return ILT_OK;
+}
 int ilt_dense_decode(uint64_t stream, const ilt_dense_model* m, const int32_t* token, int pos, int want_logits) {
   ILT_REQUIRE(m && token && m->layers && m->nl > 0 && pos >= 0 && pos < 8192);
   ILT_REQUIRE(m->x && m->q && m->k && m->v && m->att && m->fa && m->scores && m->rope && (!want_logits || (m->logits && m->output_norm)));
@@ -815,8 +825,8 @@ int ilt_dense_decode(uint64_t stream, const ilt_dense_model* m, const int32_t* t
   if (e) return e;
   for (int l = 0; l < m->nl; l++) {
     const ilt_dense_layer& L = m->layers[l];
-    const ilt_mv_desc qkv[3] = {mv_of(L.wq, m->q), mv_of(L.wk, m->k), mv_of(L.wv, m->v)};
-    if ((e = ilt_mv_multi_norm(stream, 3, qkv, m->d, m->x, L.attn_norm, m->eps, 0, 1, 0))) return e;
+    const ilt_mv_desc qkv[3] = {mv_of(L.wq, m->q, L.bq), mv_of(L.wk, m->k, L.bk), mv_of(L.wv, m->v, L.bv)};
+    if ((e = qkv_norm(stream, qkv, m->d, m->x, L.attn_norm, m->eps))) return e;
     if ((e = ilt_attn_step(stream, m->q, m->k, m->v, L.q_norm, L.k_norm, m->rope, L.kc, L.vc, m->att, m->nh, m->nkv, m->hd, m->rd, pos, m->eps,
                            m->neox, m->scores))) return e;
     const ilt_mv_desc wo = mv_of(L.wo, m->x);

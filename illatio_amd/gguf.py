@@ -199,9 +199,9 @@ DENSE_ARCHS = {"qwen2": True, "qwen3": True, "qwen3vl": True, "llama": False}   
 def dense_model(g):
     """The dense decoder in the GGUF file G as the dict illatio_amd.model.DenseModel takes (LOAD-MODEL-1,
     model.lisp:66-138): the architecture's keys into "config", every matrix as (GGUF type, its rows' bytes, memory-
-    mapped), the norms as floats; without an output.weight the head is the embedding.  Q4_K / Q6_K matrices and
-    layers without attention biases (the decoder here multiplies those); anything else raises."""
-    from .synth import Q4_K, Q6_K, row_bytes
+    mapped), the norms and the attention biases (qwen2) as floats; without an output.weight the head is the embedding.
+    Q8_0, Q4_K and Q6_K matrices (the decoder here multiplies those); anything else raises."""
+    from .synth import Q4_K, Q6_K, Q8_0, row_bytes
     arch = g.meta("general.architecture")
     if arch not in DENSE_ARCHS:
         raise GgufError(f"architecture {arch!r} is not a dense decoder this loader reads ({', '.join(DENSE_ARCHS)} are)")
@@ -222,8 +222,8 @@ def dense_model(g):
 
     def mat(name, rows, cols):
         ti = gguf_tensor(g, name)
-        if ti.type not in (Q4_K, Q6_K):
-            raise GgufError(f"{name}: type {ti.type_name}; the decoder here multiplies Q4_K and Q6_K matrices")
+        if ti.type not in (Q8_0, Q4_K, Q6_K):
+            raise GgufError(f"{name}: type {ti.type_name}; the decoder here multiplies Q8_0, Q4_K and Q6_K matrices")
         if tuple(ti.dims) != (cols, rows):
             raise GgufError(f"{name}: dimensions {list(ti.dims)}, expected [{cols}, {rows}]")
         return ti.type, tensor_bytes(g, ti).reshape(rows, row_bytes(ti.type, cols))
@@ -243,13 +243,12 @@ def dense_model(g):
     layers = []
     for i in range(nl):
         n = lambda t: f"blk.{i}.{t}"
-        for b in ("attn_q.bias", "attn_k.bias", "attn_v.bias"):
-            if gguf_tensor(g, n(b), errorp=False) is not None:
-                raise GgufError(f"{n(b)}: attention biases are not supported")
         ffn_norm = f32(n("ffn_norm.weight"), d, optional=True)
         layers.append({"attn_norm": f32(n("attn_norm.weight"), d), "wq": mat(n("attn_q.weight"), nh * hd, d),
                        "wk": mat(n("attn_k.weight"), nkv * hd, d), "wv": mat(n("attn_v.weight"), nkv * hd, d),
                        "wo": mat(n("attn_output.weight"), d, nh * hd),
+                       "bq": f32(n("attn_q.bias"), nh * hd, optional=True), "bk": f32(n("attn_k.bias"), nkv * hd, optional=True),
+                       "bv": f32(n("attn_v.bias"), nkv * hd, optional=True),
                        "q_norm": f32(n("attn_q_norm.weight"), hd, optional=True), "k_norm": f32(n("attn_k_norm.weight"), hd, optional=True),
                        "ffn_norm": ffn_norm if ffn_norm is not None else f32(n("post_attention_norm.weight"), d),
                        "gate": mat(n("ffn_gate.weight"), ffn, d), "up": mat(n("ffn_up.weight"), ffn, d),

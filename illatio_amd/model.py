@@ -1,5 +1,6 @@
 """A dense decoder on the device: the host side of the reference's CUDA-FORWARD-N (src/cuda-dense.lisp:380-432)
-for the K-quant models of the benchmark's config 2 -- embedding, and per layer: norm, Q/K/V, head norms + RoPE +
+for the K-quant models of the benchmark's config 2 and the Q8_0 ones of config 1 (qwen2: biases on Q, K and V, no head
+norms) -- embedding, and per layer: norm, Q/K/V, head norms + RoPE +
 cache update, attention, wo added to the stream, norm, gate/up with swiglu!, down added to the stream; then the
 output norm and head.  One token runs the decode products (matrix-vector kernels that take the norm and the
 quantizer inside); several tokens run the prefill products (EVAL-TOKENS, batch.lisp:289-307).  Either way a
@@ -14,7 +15,7 @@ import ctypes as C
 import numpy as np
 
 from . import dense, hip, synth
-from .synth import Q4_K, Q6_K
+from .synth import Q4_K, Q6_K, Q8_0
 
 
 def synth_model(seed, d=2560, ffn=9728, nh=32, nkv=8, hd=128, nl=36, vocab=151936, eps=1e-6, rope_base=1e6, head_scale=8.0):
@@ -37,13 +38,31 @@ def synth_model(seed, d=2560, ffn=9728, nh=32, nkv=8, hd=128, nl=36, vocab=15193
             "embd": embd, "output": embd, "output_norm": norm(d), "layers": layers}
 
 
+def synth_model_q8(seed, d=896, ffn=4864, nh=14, nkv=2, hd=64, nl=24, vocab=151936, eps=1e-6, rope_base=1e6, head_scale=8.0):
+    """The same for the benchmark's config 1 family (Qwen2.5-0.5B in Q8_0): every matrix Q8_0, biases on Q, K and V,
+    no head norms, the head tied to the embedding."""
+    rng = synth.make_rng(seed)
+    qd, kvd = nh * hd, nkv * hd
+    norm = lambda n: (synth.activations(n, rng) * 0.1 + 1.0).astype(np.float32)
+    bias = lambda n: (synth.activations(n, rng) * 0.5).astype(np.float32)
+    q8 = lambda rows, cols: (Q8_0, synth.weights(Q8_0, rows, cols, rng))
+    layers = [{"wq": q8(qd, d), "wk": q8(kvd, d), "wv": q8(kvd, d), "wo": q8(d, qd), "gate": q8(ffn, d), "up": q8(ffn, d), "down": q8(d, ffn),
+               "bq": bias(qd), "bk": bias(kvd), "bv": bias(kvd), "attn_norm": norm(d), "ffn_norm": norm(d), "q_norm": None, "k_norm": None}
+              for _ in range(nl)]
+    embd = q8(vocab, d)
+    return {"config": {"d": d, "ffn": ffn, "nh": nh, "nkv": nkv, "hd": hd, "nl": nl, "vocab": vocab, "eps": eps, "rope_base": rope_base,
+                       "neox": True},
+            "embd": embd, "output": embd, "output_norm": norm(d), "layers": layers}
+
+
 class _Mat(C.Structure):
     _fields_ = [("gguf_type", C.c_int), ("rows", C.c_int), ("cols", C.c_int), ("w", C.c_uint64), ("wd", C.c_uint64)]
 
 
 class _Layer(C.Structure):
     _fields_ = [("attn_norm", C.c_uint64), ("q_norm", C.c_uint64), ("k_norm", C.c_uint64), ("ffn_norm", C.c_uint64)] + \
-               [(n, _Mat) for n in ("wq", "wk", "wv", "wo", "gate", "up", "down")] + [("kc", C.c_uint64), ("vc", C.c_uint64)]
+               [(n, _Mat) for n in ("wq", "wk", "wv", "wo", "gate", "up", "down")] + [("kc", C.c_uint64), ("vc", C.c_uint64)] + \
+               [(n, C.c_uint64) for n in ("bq", "bk", "bv")]
 
 
 class _Model(C.Structure):
@@ -73,7 +92,7 @@ class DenseModel:
                                 "gate": up(f"blk.{li}.ffn_gate", L["gate"], ffn, d), "up": up(f"blk.{li}.ffn_up", L["up"], ffn, d),
                                 "down": up(f"blk.{li}.ffn_down", L["down"], d, ffn),
                                 "attn_norm": fl(L["attn_norm"]), "ffn_norm": fl(L["ffn_norm"]), "q_norm": fl(L.get("q_norm")),
-                                "k_norm": fl(L.get("k_norm")),
+                                "k_norm": fl(L.get("k_norm")), "bq": fl(L.get("bq")), "bk": fl(L.get("bk")), "bv": fl(L.get("bv")),
                                 "kc": hip.hip_alloc(dev, 4 * nctx * self.kvd), "vc": hip.hip_alloc(dev, 4 * nctx * self.kvd)})
         self.embd = up("token_embd", host["embd"], c["vocab"], d)
         self.output = self.embd if host["output"] is host["embd"] else up("output", host["output"], c["vocab"], d)
@@ -88,13 +107,22 @@ class DenseModel:
         self.tokens = A(4 * n)
         self.scores = A(4 * n * c["nh"] * ((nctx + 3) // 4 * 4)) if nctx <= 8192 else None      # the attention's raw scores
         self.logits = A(4 * c["vocab"])
-        self.acts = {cols: dense.QAct(dev, n, cols, ("q8k",)) for cols in {d, self.qd, ffn}}
+        # a chunk's quantized activations per width, in the formats the matrices that read that width take
+        # (Q8_0 blocks for Q8_0 matrices, Q8_K blocks for K-quants, as the CPU path makes them)
+        reads = {d: ("wq", "wk", "wv", "gate", "up"), self.qd: ("wo",), ffn: ("down",)}
+        kinds = {}
+        for cols, names in reads.items():
+            for L in self.layers:
+                for nm in names:
+                    kinds.setdefault(cols, set()).add("q8k" if L[nm].kquant_p() else "q8")
+        self.acts = {cols: dense.QAct(dev, n, cols, tuple(sorted(k))) for cols, k in kinds.items()}
         # the model as ilt_dense_decode reads it: a token's launches queued by one call
         ptr = lambda b: b.ptr if b is not None else 0
         self._clayers = (_Layer * len(self.layers))()
         for i, L in enumerate(self.layers):
             self._clayers[i] = _Layer(ptr(L["attn_norm"]), ptr(L["q_norm"]), ptr(L["k_norm"]), ptr(L["ffn_norm"]),
-                                      *[_mat(L[n]) for n in ("wq", "wk", "wv", "wo", "gate", "up", "down")], L["kc"].ptr, L["vc"].ptr)
+                                      *[_mat(L[n]) for n in ("wq", "wk", "wv", "wo", "gate", "up", "down")], L["kc"].ptr, L["vc"].ptr,
+                                      ptr(L["bq"]), ptr(L["bk"]), ptr(L["bv"]))
         self._cmodel = _Model(len(self.layers), d, ffn, c["nh"], c["nkv"], hd, hd, 1 if c["neox"] else 0, c["eps"], _mat(self.embd), _mat(self.output),
                               self.output_norm.ptr, self.rope.ptr, self._clayers, self.x.ptr, self.q.ptr, self.k.ptr, self.v.ptr, self.att.ptr,
                               self.fa.ptr, ptr(self.scores), self.logits.ptr)
@@ -116,10 +144,11 @@ class DenseModel:
         dense.embed(dev, self.embd, self.tokens, self.x, n, d)
         for L in self.layers:
             if n == 1:
-                dense.qkv_mul(dev, L["wq"], L["wk"], L["wv"], None, self.q, self.k, self.v, xf=self.x, norm=(L["attn_norm"], eps))
+                dense.qkv_mul(dev, L["wq"], L["wk"], L["wv"], None, self.q, self.k, self.v, L["bq"], L["bk"], L["bv"], xf=self.x,
+                              norm=(L["attn_norm"], eps))
             else:
                 a = dense.rmsnorm_q8(dev, self.x, L["attn_norm"], self.acts[d], d, eps, n=n)
-                dense.cmat_mul_n(dev, [(L["wq"], self.q, None), (L["wk"], self.k, None), (L["wv"], self.v, None)], a, n)
+                dense.cmat_mul_n(dev, [(L["wq"], self.q, L["bq"]), (L["wk"], self.k, L["bk"]), (L["wv"], self.v, L["bv"])], a, n)
             if n == 1 and self.scores is not None:
                 hip.call("ilt_attn_step", S, P(self.q), P(self.k), P(self.v), P(L["q_norm"]), P(L["k_norm"]), P(self.rope), P(L["kc"]), P(L["vc"]),
                          P(self.att), C.c_int(nh), C.c_int(nkv), C.c_int(hd), C.c_int(hd), C.c_int(self.pos), C.c_float(eps),

@@ -336,6 +336,7 @@ typedef struct ilt_dense_layer {
   const float *attn_norm, *q_norm, *k_norm, *ffn_norm;        /* q_norm, k_norm: null when the model has no head norms */
   ilt_dense_mat wq, wk, wv, wo, gate, up, down;
   float *kc, *vc;                                             /* this layer's caches, nkv * hd floats a position */
+  const float *bq, *bk, *bv;                                  /* Q, K and V's biases, or null (qwen2 has them) */
 } ilt_dense_layer;
 typedef struct ilt_dense_model {
   int nl, d, ffn, nh, nkv, hd, rd, neox;

@@ -179,8 +179,10 @@ def _dense_file(tmp_path, host, arch="qwen3", tied=True):
     for i, L in enumerate(host["layers"]):
         for k, (name, cols, rows) in shapes.items():
             tensors.append((f"blk.{i}.{name}.weight", (cols, rows), L[k][0], L[k][1]))
-        for k, name in (("attn_norm", "attn_norm"), ("ffn_norm", "ffn_norm"), ("q_norm", "attn_q_norm"), ("k_norm", "attn_k_norm")):
-            tensors.append((f"blk.{i}.{name}.weight", (len(L[k]),), F32, fb(L[k])))
+        for k, name in (("attn_norm", "attn_norm.weight"), ("ffn_norm", "ffn_norm.weight"), ("q_norm", "attn_q_norm.weight"),
+                        ("k_norm", "attn_k_norm.weight"), ("bq", "attn_q.bias"), ("bk", "attn_k.bias"), ("bv", "attn_v.bias")):
+            if L.get(k) is not None:
+                tensors.append((f"blk.{i}.{name}", (len(L[k]),), F32, fb(L[k])))
     p = tmp_path / f"{arch}.gguf"
     write_gguf(p, meta, tensors)
     return p
@@ -198,32 +200,42 @@ def test_dense_model_of_a_file(tmp_path):
     assert got["output"] is got["embd"]
     assert got["embd"][0] == host["embd"][0] and np.array_equal(got["embd"][1], host["embd"][1])
     assert np.array_equal(got["output_norm"], host["output_norm"])
-    for a, b in zip(got["layers"], host["layers"]):
-        assert set(a) == set(b)
-        for k in b:
-            if isinstance(b[k], tuple):
-                assert a[k][0] == b[k][0] and np.array_equal(a[k][1], b[k][1]), k
-            else:
-                assert np.array_equal(a[k], b[k]), k
+    def same_layers(got, host):
+        for a, b in zip(got["layers"], host["layers"]):
+            assert {k for k in a if a[k] is not None} == {k for k in b if b[k] is not None}
+            for k in b:
+                if isinstance(b[k], tuple):
+                    assert a[k][0] == b[k][0] and np.array_equal(a[k][1], b[k][1]), k
+                elif b[k] is not None:
+                    assert np.array_equal(a[k], b[k]), k
+    same_layers(got, host)
+    # a qwen2-style file: Q8_0 matrices, biases on Q, K and V, no head norms
+    hostq = model.synth_model_q8(23, d=256, ffn=512, nh=4, nkv=2, hd=64, nl=2, vocab=300)
+    gotq = gguf.dense_model(gguf.read_gguf(str(_dense_file(tmp_path, hostq, arch="qwen2"))))
+    assert gotq["layers"][0]["q_norm"] is None and gotq["layers"][0]["bq"] is not None and gotq["embd"][0] == synth.Q8_0
+    same_layers(gotq, hostq)
     host2 = dict(host, output=(host["embd"][0], host["embd"][1][::-1].copy()))
     got2 = gguf.dense_model(gguf.read_gguf(str(_dense_file(tmp_path, host2, arch="llama", tied=False))))
     assert got2["config"]["neox"] is False and got2["output"] is not got2["embd"]
     assert np.array_equal(got2["output"][1], host2["output"][1])
     with pytest.raises(gguf.GgufError):
         gguf.dense_model(gguf.read_gguf(str(_dense_file(tmp_path, host, arch="deepseek4"))))
-    bad = dict(host, layers=[dict(L, wq=(synth.Q8_0, synth.weights(synth.Q8_0, 256, 256, synth.make_rng(1)))) for L in host["layers"]])
+    bad = dict(host, layers=[dict(L, wq=(synth.Q2_K, synth.weights(synth.Q2_K, 256, 256, synth.make_rng(1)))) for L in host["layers"]])
     with pytest.raises(gguf.GgufError):
         gguf.dense_model(gguf.read_gguf(str(_dense_file(tmp_path, bad))))
 
 
 @pytest.mark.gpu
-def test_decoder_of_a_file_decodes_with_the_oracles_bits(tmp_path):
-    """A written qwen3-style file read back, uploaded and run: prompt and greedy tokens with the CPU oracle's logits."""
+@pytest.mark.parametrize("arch", ["qwen3", "qwen2"])
+def test_decoder_of_a_file_decodes_with_the_oracles_bits(tmp_path, arch):
+    """A written qwen3-style file (K-quants, head norms) and a qwen2-style one (Q8_0, biases) read back, uploaded and
+    run: prompt and greedy tokens with the CPU oracle's logits."""
     import oracle_lib as orc
     from illatio_amd import hip, model
     dev = hip.open_hip(0)
-    host = model.synth_model(22, d=256, ffn=512, nh=4, nkv=2, hd=64, nl=2, vocab=300)
-    got = gguf.dense_model(gguf.read_gguf(str(_dense_file(tmp_path, host))))
+    make = model.synth_model if arch == "qwen3" else model.synth_model_q8
+    host = make(22, d=256, ffn=512, nh=4, nkv=2, hd=64, nl=2, vocab=300)
+    got = gguf.dense_model(gguf.read_gguf(str(_dense_file(tmp_path, host, arch=arch))))
     cpu, gpu = orc.DenseModel(host, 24), model.DenseModel(dev, got, 24, chunk=8)
     prompt = [5, 17, 255, 3, 99, 100, 1, 42, 7, 8, 9]
     for t in prompt[:-1]:

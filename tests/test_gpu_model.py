@@ -213,6 +213,22 @@ def test_llama_style_decoder(dev):
     assert same == 4
 
 
+def test_qwen2_style_q8_decoder(dev):
+    """The config 1 family: every matrix Q8_0 (activations in Q8_0 blocks with the scale through fp16), biases on Q, K
+    and V, no head norms -- a small model with the prompt in chunks and both ways of queueing a token, then config 1's
+    own widths (896 / 4864, 14 query heads on 2 KV heads of 64, the full vocabulary), two layers."""
+    from illatio_amd import model
+    host = model.synth_model_q8(31, d=512, ffn=1024, nh=8, nkv=2, hd=64, nl=2, vocab=600)
+    assert host["layers"][0]["bq"] is not None and host["layers"][0]["q_norm"] is None
+    same, _ = run_greedy(dev, host, nprompt=20, ndecode=12, chunk=8, nctx=40, seed=31, check_cache=True)
+    assert same == 12
+    same, _ = run_greedy(dev, host, nprompt=20, ndecode=6, chunk=8, nctx=40, seed=32, one_call=False)
+    assert same == 6
+    host = model.synth_model_q8(33, nl=2)
+    same, margins = run_greedy(dev, host, nprompt=40, ndecode=24, chunk=32, nctx=70, seed=33)
+    assert same == 24 and min(margins) > 0
+
+
 def test_small_decoder_long_contexts(dev):
     """Contexts past one workgroup's 256 positions of scores: the two-launch attention with 16 tokens, 4 tokens and one
     token a workgroup as the context grows towards 2048 positions, and past that the value slice in tiles."""
