@@ -11,7 +11,7 @@ is far beyond the 256 MB MALL.  No attention, norm or RoPE runs in a step: those
 the dense-forward harness, not to this path.
 
 Without --workload the line is c2's, and the other configurations run after it on the same clock
-and are reported under "configs" (c2_decode, c1, c3 and c5 on the bf16 matrix cores and on the exact
+and are reported under "configs" (c2_decode, c1, c1_decode, c3 and c5 on the bf16 matrix cores and on the exact
 int8 path, c4 with the routing on the device); c2_decode's figures are also the line's
 decode_tok_per_s, decode_ms_per_token and prefill_tok_per_s.
 
@@ -640,8 +640,10 @@ def workload_c2d(args, dev):
     the logits and the greedy pick -- on the device, the ids read back after the last token (--host-argmax: logits
     downloaded and the token picked on the host every step, as the reference's loop does, cuda-dense.lisp:428-430)."""
     from illatio_amd import hip, model, synth
-    nl, nprompt, ndecode = args.layers, 512, 256
-    host = model.synth_model(2, nl=nl)
+    q8 = getattr(args, "q8_model", False)                    # c1d: config 1's family (Qwen2.5-0.5B's shape, Q8_0, 24 layers)
+    nl, nprompt, ndecode = (min(args.layers, 24) if q8 else args.layers), 512, 256
+    host = model.synth_model_q8(2, nl=nl) if q8 else model.synth_model(2, nl=nl)
+    shape = "qwen2.5-0.5b" if q8 else "qwen3-4b"
     c = host["config"]
     m = model.DenseModel(dev, host, nctx=nprompt + ndecode + args.warmup + 8, chunk=512)
     rng = synth.make_rng(3)
@@ -694,8 +696,8 @@ def workload_c2d(args, dev):
 
     return {"value": round(ndecode / decode_s, 1), "unit": "tok/s", "ms_per_step": ms, "device_ms_per_step": ms, "enqueue_ms": 0.0,
             "dtype": "int8 block dots, fp32 combine; fp32 attention",
-            "metric": "decode tok/s at Qwen3-4B shape",
-            "config": {"workload": f"c2 decode: qwen3-4b-shape dense decoder, {nl} layers, random-init Q4_K/Q6_K, {nprompt}-token prompt then "
+            "metric": "decode tok/s at Qwen2.5-0.5B shape" if q8 else "decode tok/s at Qwen3-4B shape",
+            "config": {"workload": f"{'c1' if q8 else 'c2'} decode: {shape}-shape dense decoder, {nl} layers, random-init {'Q8_0' if q8 else 'Q4_K/Q6_K'}, {nprompt}-token prompt then "
                                    f"{ndecode}-token greedy decode at batch 1", "weight_bytes_per_token": int(wbytes)},
             "extra": {"prefill_tok_per_s": round(nprompt / prefill_s, 1), "distinct_tokens_decoded": len(set(toks)),
                       "weights_GBps_in_decode": round(wbytes / (ms * 1e-3) / 1e9, 1)},
@@ -707,7 +709,16 @@ def workload_c2d(args, dev):
             "cpu": cpu}
 
 
-WORKLOADS = {"c1": workload_c1, "c2": workload_c2, "c2d": workload_c2d, "c3": workload_c3, "c4": workload_c4, "c5": workload_c5}
+def workload_c1d(args, dev):
+    """Config 1's family as a whole decoder: the Qwen2.5-0.5B shape in Q8_0 (24 layers, hidden 896, intermediate 4864, 14
+    query heads on 2 KV heads of 64, biases on Q, K and V), random-init: a 512-token prompt, then 256 greedy tokens."""
+    import copy
+    a = copy.copy(args)
+    a.q8_model = True
+    return workload_c2d(a, dev)
+
+
+WORKLOADS = {"c1": workload_c1, "c1d": workload_c1d, "c2": workload_c2, "c2d": workload_c2d, "c3": workload_c3, "c4": workload_c4, "c5": workload_c5}
 
 
 def main():
@@ -760,13 +771,13 @@ def main():
         import copy
         import gc
         out["configs"] = {}
-        extras = [("c2_decode", {}), ("c1", {"steps": 200, "warmup": 20}), ("c3", {"path": "bf16", "tokens": 4096}), ("c3_t2048", {"path": "bf16", "tokens": 2048}),
+        extras = [("c2_decode", {}), ("c1", {"steps": 200, "warmup": 20}), ("c1_decode", {}), ("c3", {"path": "bf16", "tokens": 4096}), ("c3_t2048", {"path": "bf16", "tokens": 2048}),
                   ("c3_t512", {"path": "bf16", "tokens": 512}), ("c3_resident", {"path": "bf16-resident", "tokens": 4096}),
                   ("c3_exact", {"path": "int8", "tokens": 4096}),
                   ("c4", {"mode": "device", "steps": 50, "warmup": 5}), ("c5", {"path": "bf16", "tokens": 4096}), ("c5_exact", {"path": "int8", "tokens": 4096})]
         for name, over in extras:
             a = copy.copy(args)
-            a.workload, a.steps, a.warmup = ("c2d" if name == "c2_decode" else name[:2]), min(args.steps, 10), min(args.warmup, 3)
+            a.workload, a.steps, a.warmup = {"c2_decode": "c2d", "c1_decode": "c1d"}.get(name, name[:2]), min(args.steps, 10), min(args.warmup, 3)
             for k, v in over.items():
                 setattr(a, k, v)
             del r
