@@ -177,7 +177,7 @@ int ilt_quant_q8k(uint64_t stream, const float* x, int8_t* xq, float* xd, int32_
 static int gemv_multi(uint64_t stream, int nmat, const int* fmts, const void* const* ws, const uint16_t* const* wds,
                       float* const* ys, const float* const* biases, const int* rows, int cols, const int8_t* xq,
                       const float* xs, const int32_t* bsums, const float* xf, int f16_scale, int acc, int glu,
-                      int group_rows, const float* norm_w = nullptr, float eps = 0.0f, int norm_seq = 0) {
+                      int group_rows, const float* norm_w = nullptr, float eps = 0.0f, int norm_seq = 0, const IltCacheAhead* ahead = nullptr) {
   ILT_REQUIRE(nmat >= 1 && nmat <= 4 && cols > 0);
   const bool q8 = fmts[0] == ILT_Q8_0;
   IltGemvParams p = {};
@@ -204,6 +204,7 @@ static int gemv_multi(uint64_t stream, int nmat, const int* fmts, const void* co
     ILT_REQUIRE(live == 1 && p.mat[0].rows % group_rows == 0);
     p.group_rows = group_rows;
   }
+  if (ahead) p.ahead = *ahead;
   return (int)ilt_gemv_launch(p, 1, S(stream));
 }
 
@@ -807,9 +808,16 @@ int ilt_argmax(uint64_t stream, const float* v, int n, int32_t* out, void* scrat
 // ---- one token through the dense decoder: the launches of the single calls, queued in one ----------
 static ilt_mv_desc mv_of(const ilt_dense_mat& w, float* y, const float* bias = nullptr) { return {w.gguf_type, w.rows, w.w, w.wd, y, bias}; }
 // Q/K/V with the norm inside: one launch where the three share an activation format (all Q8_0, or K-quants), else one each
-static int qkv_norm(uint64_t stream, const ilt_mv_desc (&qkv)[3], int d, const float* x, const float* norm, float eps) {
+static int qkv_norm(uint64_t stream, const ilt_mv_desc (&qkv)[3], int d, const float* x, const float* norm, float eps, const IltCacheAhead* ahead) {
   const bool q8[3] = {qkv[0].gguf_type == ILT_TYPE_Q8_0, qkv[1].gguf_type == ILT_TYPE_Q8_0, qkv[2].gguf_type == ILT_TYPE_Q8_0};
-  if (q8[0] == q8[1] && q8[1] == q8[2]) return ilt_mv_multi_norm(stream, 3, qkv, d, x, norm, eps, 0, 1, 0);
+  if (q8[0] == q8[1] && q8[1] == q8[2]) {
+    int fmts[3], rows[3]; const void* ws[3]; const uint16_t* wds[3]; float* ys[3]; const float* bs[3];
+    for (int i = 0; i < 3; i++) {
+      fmts[i] = qkv[i].gguf_type; rows[i] = qkv[i].rows; ws[i] = qkv[i].w; wds[i] = qkv[i].wd; ys[i] = qkv[i].y; bs[i] = qkv[i].bias;
+    }
+    ILT_REQUIRE(x && norm);
+    return gemv_multi(stream, 3, fmts, ws, wds, ys, bs, rows, d, nullptr, nullptr, nullptr, x, 1, 0, 0, 0, norm, eps, 0, ahead);
+  }
   for (int i = 0; i < 3; i++) {
     const int e = ilt_mv_multi_norm(stream, 1, &qkv[i], d, x, norm, eps, 0, 1, 0);
     if (e) return e;
@@ -826,7 +834,23 @@ int ilt_dense_decode(uint64_t stream, const ilt_dense_model* m, const int32_t* t
   for (int l = 0; l < m->nl; l++) {
     const ilt_dense_layer& L = m->layers[l];
     const ilt_mv_desc qkv[3] = {mv_of(L.wq, m->q, L.bq), mv_of(L.wk, m->k, L.bk), mv_of(L.wv, m->v, L.bv)};
-    if ((e = qkv_norm(stream, qkv, m->d, m->x, L.attn_norm, m->eps))) return e;
+    // the attention's keys and values read ahead into the L2 of the die whose workgroups will want them (the one-launch
+    // attention deals a die consecutive heads: attn_step_fused_kernel's mapping), with the table's row and the head norms
+    IltCacheAhead ahead = {};
+    static const bool ahead_on = []{ const char* f = getenv("ILT_CACHE_AHEAD"); return !(f && f[0] == '0'); }();
+    const int nwg = m->nh * (m->hd / 16);
+    if (ahead_on && pos > 0 && pos < 1024 && (m->hd == 64 || m->hd == 128) && nwg % 8 == 0 && m->nkv > 0 && m->nh % m->nkv == 0) {
+      const int ns = m->hd / 16, group = m->nh / m->nkv;
+      ahead.a = L.kc; ahead.b = L.vc; ahead.stride = m->nkv * m->hd; ahead.nrows = pos;
+      for (int x = 0; x < 8; x++) {
+        const int h0 = x * (nwg / 8) / ns, h1 = ((x + 1) * (nwg / 8) - 1) / ns, k0 = h0 / group, k1 = h1 / group;
+        ahead.off[x] = k0 * m->hd; ahead.width[x] = (k1 - k0 + 1) * m->hd;
+      }
+      ahead.small[0] = m->rope + (long long)pos * m->rd; ahead.nsmall[0] = m->rd;
+      ahead.small[1] = L.q_norm; ahead.nsmall[1] = m->hd;
+      ahead.small[2] = L.k_norm; ahead.nsmall[2] = m->hd;
+    }
+    if ((e = qkv_norm(stream, qkv, m->d, m->x, L.attn_norm, m->eps, ahead.a ? &ahead : nullptr))) return e;
     if ((e = ilt_attn_step(stream, m->q, m->k, m->v, L.q_norm, L.k_norm, m->rope, L.kc, L.vc, m->att, m->nh, m->nkv, m->hd, m->rd, pos, m->eps,
                            m->neox, m->scores))) return e;
     const ilt_mv_desc wo = mv_of(L.wo, m->x);

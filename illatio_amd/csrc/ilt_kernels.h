@@ -39,8 +39,20 @@ struct IltRouteAlong {
   int done;
 };
 
+// KV cache rows read ahead by a product launch's activation waves once their own work is done (the streamed variant):
+// the launch after it -- one token's attention -- then finds its keys and values in the L2 of the die that wants them.
+// Workgroup g runs on die g % 8; die x reads floats off[x] .. off[x] + width[x] - 1 of each of the nrows rows of a and
+// of b (stride floats apart), and every die the three small vectors.  a null: nothing.
+struct IltCacheAhead {
+  const float* a; const float* b;
+  int stride, nrows;
+  int off[8], width[8];
+  const float* small[3]; int nsmall[3];
+};
+
 struct IltGemvParams {
   IltRouteAlong route;
+  IltCacheAhead ahead;
   IltGemvMat mat[4];         // up to four matrices sharing the activations
   int nmat;
   const uint64_t* ptrs;      // experts: grid y's matrices are at ptrs[y] + mat[i].add,

@@ -847,6 +847,37 @@ __device__ __forceinline__ int lds_block_bytes(int fmt) {
   return fmt == ILT_Q4_K ? 144 : fmt == ILT_Q6_K ? 224 : fmt == ILT_Q2_K ? 96 : fmt == ILT_Q8_0 ? 32 : 80;
 }
 
+// What the activation waves (256 threads a workgroup) read ahead for the next launch; the values go nowhere, the
+// lines stay in this die's L2.  The loads queue behind the row waves' (all asked for at the kernel's start), so they
+// take memory's time when the rows have arrived.
+__device__ __forceinline__ void cache_ahead(const IltCacheAhead& h, float* sink) {
+  const int die = blockIdx.x & 7, w4 = h.width[die] >> 2;
+  const int me = (int)(blockIdx.x >> 3) * (64 * kStagers) + (int)threadIdx.x, all = (int)((gridDim.x + 7) >> 3) * (64 * kStagers);
+  float keep = 0.0f;
+  if (w4 > 0) {
+    // four pieces of each array a thread at a time, all asked for before any is looked at (a piece a trip to memory
+    // otherwise); past the end the last piece again
+    const int total = h.nrows * w4;
+    for (int i0 = me; i0 < total; i0 += 4 * all) {
+      float4 x[4], y[4];
+#pragma unroll
+      for (int u = 0; u < 4; u++) {
+        const int i = min(i0 + u * all, total - 1), row = i / w4, c = i - row * w4;
+        const long long o = (long long)row * h.stride + h.off[die] + 4 * c;
+        x[u] = *(const float4*)(h.a + o); y[u] = *(const float4*)(h.b + o);
+      }
+#pragma unroll
+      for (int u = 0; u < 4; u++) keep += (x[u].x + x[u].y + x[u].z + x[u].w) + (y[u].x + y[u].y + y[u].z + y[u].w);
+    }
+  }
+  if ((blockIdx.x >> 3) == 0) {
+#pragma unroll
+    for (int r = 0; r < 3; r++)
+      if (h.small[r]) for (int i = threadIdx.x; i < h.nsmall[r]; i += 64 * kStagers) keep += h.small[r][i];
+  }
+  if (keep == 1.2345678e38f) *sink = keep;               // (never: the loads must not be dropped)
+}
+
 // FSET: ILT_Q4_K, ILT_Q6_K, 0 (those two mixed), or the expert formats ILT_IQ2_XXS, ILT_Q2_K (then
 // p.ptrs gives the experts' slots and p.nz how many take part: a batch is rows of one expert,
 // batches per expert = p.mat[0].nbat).  p.batch = the most rows a wave takes; p.region = bytes
@@ -875,6 +906,7 @@ __global__ __launch_bounds__(kStreamThreads) void gemv_stream_kernel(IltGemvPara
       for (int i = threadIdx.x; i < S; i += 64 * kStagers) lxs[i] = p.xs[i];
     }
     ilt_barrier_lds();
+    if (p.ahead.a) cache_ahead(p.ahead, p.mat[0].y);
     if constexpr (q8 && !EARLY) {
       // a token's routing carried along: this wave has nothing left to do while the rows stream in
       if (p.route.logits && blockIdx.x == 0 && wave == 0) {
@@ -927,6 +959,7 @@ __global__ __launch_bounds__(kStreamThreads) void gemv_stream_kernel(IltGemvPara
       if (!iq2) for (int i = threadIdx.x; i < SX * 16; i += 64 * kStagers) lbs[i] = p.bsums[i];
     }
     ilt_barrier_lds();
+    if (p.ahead.a) cache_ahead(p.ahead, p.mat[0].y);
     return;
   }
   const int rw = wave - kStagers;
@@ -1195,6 +1228,7 @@ static hipError_t gemv_stream_launch(IltGemvParams& p, int fset, int nz, hipStre
 }
 
 hipError_t ilt_gemv_launch(IltGemvParams& p, int nz, hipStream_t st) {
+  if (p.ahead.a && (p.ahead.nrows <= 0 || (p.ahead.stride & 3))) p.ahead.a = nullptr;
   int fset = p.mat[0].fmt;
   for (int i = 1; i < p.nmat; i++) if (p.mat[i].fmt != fset) fset = 0;
   {
