@@ -50,9 +50,18 @@ struct IltCacheAhead {
   const float* small[3]; int nsmall[3];
 };
 
+// The next streamed product's rows, read ahead the same way: that launch's plan (ilt_gemv_plan) says which rows its
+// workgroup g -- die g % 8 -- will stream, and this launch's idle waves on that die touch their cache lines, so that
+// the next launch streams from L2 instead of HBM.  nm 0: nothing.
+struct IltRowsAhead {
+  int nm;                                                                       // matrices (a gate/up pair: two, with the same batches)
+  struct M { const uint8_t* w; long long row_bytes; int rq, rr, batch0, nbat; } m[4];
+};
+
 struct IltGemvParams {
   IltRouteAlong route;
   IltCacheAhead ahead;
+  IltRowsAhead rows_ahead;
   IltGemvMat mat[4];         // up to four matrices sharing the activations
   int nmat;
   const uint64_t* ptrs;      // experts: grid y's matrices are at ptrs[y] + mat[i].add,
@@ -84,6 +93,11 @@ struct IltGemvParams {
 
 // The kernel is chosen by the matrices' formats (mat[i].fmt): one format, or Q4_K and Q6_K mixed.
 hipError_t ilt_gemv_launch(IltGemvParams& p, int nz, hipStream_t st);
+// The streamed variant's plan for p without launching (the batches of each matrix): hipSuccess when ilt_gemv_launch
+// would take the streamed variant with a grid of 256 workgroups, hipErrorNotSupported otherwise.
+hipError_t ilt_gemv_plan(IltGemvParams& p, int nz);
+// out = the rows p's launch will stream, for another launch's rows_ahead (p planned by ilt_gemv_plan)
+void ilt_gemv_rows_of(const IltGemvParams& p, IltRowsAhead& out);
 
 unsigned long long ilt_k_streamed_launches();      // decode products launched as the streamed variant so far (diagnostic)
 

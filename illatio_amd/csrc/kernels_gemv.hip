@@ -878,6 +878,35 @@ __device__ __forceinline__ void cache_ahead(const IltCacheAhead& h, float* sink)
   if (keep == 1.2345678e38f) *sink = keep;               // (never: the loads must not be dropped)
 }
 
+// The next product's rows for this die, a 128-byte line a lane (one dword of a line brings the line into L2).  Batch b of
+// the next launch goes to its workgroup b % 256, die b % 8: this die's batches of matrix i are bl = r0, r0 + 8, ...
+__device__ __forceinline__ void rows_ahead(const IltRowsAhead& h, float* sink) {
+  const int die = blockIdx.x & 7;
+  const int me = (int)(blockIdx.x >> 3) * (64 * kStagers) + (int)threadIdx.x, all = (int)((gridDim.x + 7) >> 3) * (64 * kStagers);
+  u32 keep = 0;
+  for (int i = 0; i < h.nm; i++) {
+    const IltRowsAhead::M& m = h.m[i];
+    const int r0 = (((die - m.batch0) % 8) + 8) % 8;
+    if (r0 >= m.nbat) continue;
+    const int K = (m.nbat - r0 + 7) >> 3;
+    const int maxl = (int)(((long long)(m.rq + 1) * m.row_bytes + 127) >> 7) + 1;      // lines a batch, at most
+    const int total = K * maxl;
+    for (int i0 = me; i0 < total; i0 += 4 * all) {
+      u32 v[4];
+#pragma unroll
+      for (int u = 0; u < 4; u++) {
+        const int j = min(i0 + u * all, total - 1), k = j / maxl, ll = j - k * maxl, bl = r0 + 8 * k;
+        const long long row0 = (long long)bl * m.rq + min(bl, m.rr), nrows = m.rq + (bl < m.rr ? 1 : 0);
+        const long long start = row0 * m.row_bytes, end = start + nrows * m.row_bytes;
+        const long long a = min((start & ~127LL) + 128LL * ll, (end - 1) & ~127LL);       // past the batch's end: its last line again
+        v[u] = *(const u32*)(m.w + a);
+      }
+      keep ^= (v[0] ^ v[1]) ^ (v[2] ^ v[3]);
+    }
+  }
+  if (keep == 0x9E3779B9u && h.nm < 0) *sink = 0.0f;       // (never: the loads must not be dropped)
+}
+
 // FSET: ILT_Q4_K, ILT_Q6_K, 0 (those two mixed), or the expert formats ILT_IQ2_XXS, ILT_Q2_K (then
 // p.ptrs gives the experts' slots and p.nz how many take part: a batch is rows of one expert,
 // batches per expert = p.mat[0].nbat).  p.batch = the most rows a wave takes; p.region = bytes
@@ -907,6 +936,7 @@ __global__ __launch_bounds__(kStreamThreads) void gemv_stream_kernel(IltGemvPara
     }
     ilt_barrier_lds();
     if (p.ahead.a) cache_ahead(p.ahead, p.mat[0].y);
+    if (p.rows_ahead.nm) rows_ahead(p.rows_ahead, p.mat[0].y);
     if constexpr (q8 && !EARLY) {
       // a token's routing carried along: this wave has nothing left to do while the rows stream in
       if (p.route.logits && blockIdx.x == 0 && wave == 0) {
@@ -960,6 +990,7 @@ __global__ __launch_bounds__(kStreamThreads) void gemv_stream_kernel(IltGemvPara
     }
     ilt_barrier_lds();
     if (p.ahead.a) cache_ahead(p.ahead, p.mat[0].y);
+    if (p.rows_ahead.nm) rows_ahead(p.rows_ahead, p.mat[0].y);
     return;
   }
   const int rw = wave - kStagers;
@@ -1119,7 +1150,7 @@ int resident_per_cu(int fset, size_t smem) {
 static unsigned long long g_streamed_launches = 0;
 unsigned long long ilt_k_streamed_launches() { return g_streamed_launches; }
 
-static hipError_t gemv_stream_launch(IltGemvParams& p, int fset, int nz, hipStream_t st) {
+static hipError_t gemv_stream_launch(IltGemvParams& p, int fset, int nz, hipStream_t st, bool plan_only = false) {
   const char* force = getenv("ILT_GEMV_STREAM");          // "0": never (tests)
   if (force && atoi(force) == 0) return hipErrorNotSupported;
   const bool experts = p.ptrs != nullptr;
@@ -1182,6 +1213,7 @@ static hipError_t gemv_stream_launch(IltGemvParams& p, int fset, int nz, hipStre
   const size_t smem = xbytes + 16 + (size_t)kRowWaves * batch * S * (q8 ? 1 : 2) * 4 * nglu + (size_t)kRowWaves * p.region;
   if (smem > 156 * 1024) return hipErrorNotSupported;
   p.s_magic = (uint32_t)(0x100000000ULL / (uint64_t)S) + 1;
+  if (plan_only) return nb >= 256 ? hipSuccess : hipErrorNotSupported;
   static bool attr_set[8] = {};
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 8) dev = 0;
@@ -1225,6 +1257,21 @@ static hipError_t gemv_stream_launch(IltGemvParams& p, int fset, int nz, hipStre
   }
   g_streamed_launches++;
   return hipGetLastError();
+}
+
+hipError_t ilt_gemv_plan(IltGemvParams& p, int nz) {
+  int fset = p.mat[0].fmt;
+  for (int i = 1; i < p.nmat; i++) if (p.mat[i].fmt != fset) fset = 0;
+  return gemv_stream_launch(p, fset, nz, nullptr, true);
+}
+
+void ilt_gemv_rows_of(const IltGemvParams& p, IltRowsAhead& out) {
+  out.nm = 0;
+  if (p.ptrs) return;
+  for (int i = 0; i < p.nmat && i < 4; i++) {
+    const IltGemvMat& m = p.mat[i];
+    out.m[out.nm++] = {m.w, m.row_bytes, m.rq, m.rr, m.batch0, m.nbat};
+  }
 }
 
 hipError_t ilt_gemv_launch(IltGemvParams& p, int nz, hipStream_t st) {
