@@ -897,9 +897,9 @@ __device__ __forceinline__ void rows_ahead(const IltRowsAhead& h, float* sink) {
       for (int u = 0; u < 4; u++) {
         const int j = min(i0 + u * all, total - 1), k = j / maxl, ll = j - k * maxl, bl = r0 + 8 * k;
         const long long row0 = (long long)bl * m.rq + min(bl, m.rr), nrows = m.rq + (bl < m.rr ? 1 : 0);
-        const long long start = row0 * m.row_bytes, end = start + nrows * m.row_bytes;
-        const long long a = min((start & ~127LL) + 128LL * ll, (end - 1) & ~127LL);       // past the batch's end: its last line again
-        v[u] = *(const u32*)(m.w + a);
+        const u64 start = (u64)(uintptr_t)m.w + (u64)(row0 * m.row_bytes), end = start + (u64)(nrows * m.row_bytes);
+        const u64 a = min((start & ~127ULL) + 128ULL * (u64)ll, (end - 1) & ~127ULL);     // past the batch's end: its last line again
+        v[u] = *(const u32*)(uintptr_t)max(a, start & ~3ULL);                            // (never before the batch's first dword)
       }
       keep ^= (v[0] ^ v[1]) ^ (v[2] ^ v[3]);
     }
