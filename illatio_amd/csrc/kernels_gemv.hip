@@ -1275,7 +1275,8 @@ void ilt_gemv_rows_of(const IltGemvParams& p, IltRowsAhead& out) {
 }
 
 hipError_t ilt_gemv_launch(IltGemvParams& p, int nz, hipStream_t st) {
-  if (p.ahead.a && (p.ahead.nrows <= 0 || (p.ahead.stride & 3))) p.ahead.a = nullptr;
+  if (p.ahead.a && (p.ahead.nrows <= 0 || (p.ahead.stride & 3) || !p.ahead.b || (((uintptr_t)p.ahead.a | (uintptr_t)p.ahead.b) & 15)))
+    p.ahead.a = nullptr;                                   // (rows that 16-byte loads cannot take: no reading ahead)
   int fset = p.mat[0].fmt;
   for (int i = 1; i < p.nmat; i++) if (p.mat[i].fmt != fset) fset = 0;
   {
