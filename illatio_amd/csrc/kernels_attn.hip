@@ -19,6 +19,17 @@ __device__ __forceinline__ void wave_lds_sync() {
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
+// The softmax's 1/sum as the CPU rounds it to a single, from a sum of n exps added in another order than the CPU's
+// (within sum * (n + 8) * 2^-51 of the CPU's): one division, then whether every sum that near has the same single for
+// its reciprocal -- the reciprocals of all of them lie within inv * (1 -+ d), d a little more than twice that slack
+// plus the division's own rounding, and rounding to single keeps their order.  False: the caller adds the exps again
+// in the CPU's order.
+__device__ __forceinline__ bool recip_settled(double sum, int n, float* inv) {
+  const double r = 1.0 / sum, d = (double)(n + 8) * 0x1p-50 + 0x1p-50;
+  *inv = (float)r;
+  return (float)(r - r * d) == (float)(r + r * d);
+}
+
 // One head by one wave: x (hd floats) into xs (LDS): rmsnorm! of the head when its weights are given
 // (model.lisp:205-216: the squares, rounded to floats, added in double one after another), then rope-head!
 // from the position's table cs (cos, then sin, rd/2 each).  Only this wave touches xs and sd.  The lanes add
@@ -173,14 +184,13 @@ __global__ __launch_bounds__(kAttnThreads) void attn_rows_kernel(const float* __
   double sum = 0.0;
 #pragma unroll
   for (int w = 0; w < 16; w++) sum += redd[w];
-  const double slack = sum * ((double)(npos + 8) * 0x1p-51);
-  if ((float)(1.0 / (sum - slack)) != (float)(1.0 / (sum + slack))) {      // the same in every thread
+  float inv;
+  if (!recip_settled(sum, npos, &inv)) {           // the same in every thread
     __syncthreads();
     if (tid == 0) { double s2 = 0.0; for (int p = 0; p < npos; p++) s2 += (double)scores[p]; redd[0] = s2; }
     __syncthreads();
-    sum = redd[0];
+    inv = (float)(1.0 / redd[0]);
   }
-  const float inv = (float)(1.0 / sum);
   __syncthreads();
   for (int p = tid; p < npos; p += kAttnThreads) scores[p] = scores[p] * inv;
   // the values: tile i of 64 positions into buffer i & 1, loaded a tile ahead of the adds
@@ -439,14 +449,13 @@ __device__ __forceinline__ void attn_softmax(const float* __restrict__ rw, const
     sum = (redd[0] + redd[1]) + (redd[2] + redd[3]);
   }
   // the CPU adds the terms one after another: take its sum where the order could show in the rounded reciprocal
-  const double slack = sum * ((double)(npos + 8) * 0x1p-51);
-  if ((float)(1.0 / (sum - slack)) != (float)(1.0 / (sum + slack))) {      // the same in all NT threads
+  float inv;
+  if (!recip_settled(sum, npos, &inv)) {           // the same in all NT threads
     if (NT > 64) __syncthreads();
     if (me == 0) { double s2 = 0.0; for (int p = 0; p < npos; p++) s2 += (double)sc[p]; redd[NT > 64 ? 0 : 4 + wave] = s2; }
     if (NT > 64) __syncthreads();
-    sum = redd[NT > 64 ? 0 : 4 + wave];
+    inv = (float)(1.0 / redd[NT > 64 ? 0 : 4 + wave]);
   }
-  const float inv = (float)(1.0 / sum);
   for (int p = me; p < npos; p += NT) sc[p] = sc[p] * inv;
 }
 
@@ -653,13 +662,12 @@ __global__ __launch_bounds__(1024) void attn_step_fused_kernel(const float* __re
 #pragma unroll
   for (int w = 1; w < 16; w++) sum += redd[w];
   // the CPU adds the terms one after another: take its sum where the order could show in the rounded reciprocal
-  const double slack = sum * ((double)(npos + 8) * 0x1p-51);
-  if ((float)(1.0 / (sum - slack)) != (float)(1.0 / (sum + slack))) {      // the same in every thread
+  float inv;
+  if (!recip_settled(sum, npos, &inv)) {           // the same in every thread
     if (tid == 0) { double s2 = 0.0; for (int p = 0; p < npos; p++) s2 += (double)sc[p]; redd[16] = s2; }
     __syncthreads();
-    sum = redd[16];
+    inv = (float)(1.0 / redd[16]);
   }
-  const float inv = (float)(1.0 / sum);
   if (mine) sc[tid] = e * inv;
   __syncthreads();
 #pragma unroll
