@@ -17,7 +17,7 @@
 // in silu(gate)*up (swiglu!, model.lisp:364-378).
 // Two kernels share those phases: gemv_kernel walks its rows with loads two steps ahead (any
 // size; the 300 MB output head), gemv_stream_kernel has every wave ask for all of its rows at
-// once as direct loads into LDS (products of 2 MB and more whose share fits a CU's LDS).  The
+// once as direct loads into LDS (products of half a megabyte and more whose share fits a CU's LDS).  The
 // host chooses (ilt_gemv_launch).
 #include "ilt_device.h"
 #include "ilt_iq2xxs_tables.h"
@@ -1166,7 +1166,8 @@ static hipError_t gemv_stream_launch(IltGemvParams& p, int fset, int nz, hipStre
   long total_rows = 0, bytes = 0;
   for (int i = 0; i < nm; i++) { total_rows += p.mat[i].rows; bytes += (long)p.mat[i].rows * p.mat[i].row_bytes; }
   constexpr int kWavesAll = 256 * kRowWaves;
-  if (total_rows * nz > 16L * kWavesAll || bytes * nz * (p.glu ? 2 : 1) < (2L << 20)) return hipErrorNotSupported;
+  // (from half a megabyte on: below that the looping variant's smaller workgroups are as fast)
+  if (total_rows * nz > 16L * kWavesAll || bytes * nz * (p.glu ? 2 : 1) < (512L << 10)) return hipErrorNotSupported;
   int nb = 0, batch = 1;
   if (experts) {
     // the waves are shared out evenly over the experts; a batch is rows of one expert
