@@ -248,8 +248,10 @@ def workload_c2(args, dev):
                           lambda: dense.mv_multi(dev, [(L["wo"], ybuf["wo"], None)], acts["att"], xf=xbuf["att"] if inq else None))
                 if not inq:
                     quantize_x()
+                # (the gate/up launch reads the rows of the down product after it ahead, as the decoder does)
+                nxt = ([(L["down"], ybuf["down"], None)], False) if inq else None
                 tm.launch("glu", wbytes["gate"] + wbytes["up"] + D + 4 * FFN,
-                          lambda: dense.glu_mul(dev, L["gate"], L["up"], acts["x"], ybuf["gate"], xf=xf, norm=norm))
+                          lambda: dense.glu_mul(dev, L["gate"], L["up"], acts["x"], ybuf["gate"], xf=xf, norm=norm, ahead=nxt))
                 if inq:
                     tm.launch("down", wbytes["down"] + FFN + 4 * D, lambda: dense.mv_multi(dev, [(L["down"], ybuf["down"], None)], xf=xbuf["mid"]))
                 else:

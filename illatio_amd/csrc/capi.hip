@@ -275,6 +275,29 @@ int ilt_mv_multi(uint64_t stream, int nmat, const ilt_mv_desc* descs, int cols, 
   return gemv_multi(stream, nmat, fmts, ws, wds, ys, bs, rows, cols, xq, xs, bsums, xf, f16_scale, acc, glu, 0);
 }
 
+// ilt_mv_multi / ilt_mv_multi_norm on float activations, reading the rows of the caller's next product ahead while it
+// runs (norm_w null: no norm).  The next product is described, not launched; where either of the two does not take
+// the streamed variant the call is the plain one.
+int ilt_mv_multi_ahead(uint64_t stream, int nmat, const ilt_mv_desc* descs, int cols, const float* xf, const float* norm_w, float eps,
+                       int f16_scale, int acc, int glu, int next_nmat, const ilt_mv_desc* next_descs, int next_cols, int next_glu) {
+  ILT_REQUIRE(descs && nmat >= 1 && nmat <= 4 && xf && (!next_nmat || (next_descs && next_nmat >= 1 && next_nmat <= 4 && next_cols > 0)));
+  auto build = [&](IltGemvParams& p, int* live, int n, const ilt_mv_desc* d, int c, const float* x, const float* nw, int a, int g) -> int {
+    int fmts[4], rows[4]; const void* ws[4]; const uint16_t* wds[4]; float* ys[4]; const float* bs[4];
+    for (int i = 0; i < n; i++) { fmts[i] = d[i].gguf_type; rows[i] = d[i].rows; ws[i] = d[i].w; wds[i] = d[i].wd; ys[i] = d[i].y; bs[i] = d[i].bias; }
+    return gemv_multi_build(p, live, n, fmts, ws, wds, ys, bs, rows, c, nullptr, nullptr, nullptr, x, f16_scale, a, g, 0, nw, eps, 0);
+  };
+  IltGemvParams p, pn;
+  int live = 0, live_n = 0;
+  const int e = build(p, &live, nmat, descs, cols, xf, norm_w, acc, glu);
+  if (e != ILT_OK || live == 0) return e;
+  // (the next product's activations do not matter to its plan: this call's stand in for them)
+  static const bool rows_on = []{ const char* f = getenv("ILT_ROWS_AHEAD"); return !(f && f[0] == '0'); }();      // ("0": never, for tests)
+  if (rows_on && next_nmat && build(pn, &live_n, next_nmat, next_descs, next_cols, xf, nullptr, 0, next_glu) == ILT_OK && live_n &&
+      ilt_gemv_plan(p, 1) == hipSuccess && ilt_gemv_plan(pn, 1) == hipSuccess)
+    ilt_gemv_rows_of(pn, p.rows_ahead);
+  return (int)ilt_gemv_launch(p, 1, S(stream));
+}
+
 uint64_t ilt_streamed_launches(void) { return (uint64_t)ilt_k_streamed_launches(); }
 
 int ilt_mv_multi_norm(uint64_t stream, int nmat, const ilt_mv_desc* descs, int cols, const float* x, const float* norm_w,

@@ -239,15 +239,28 @@ class MvDesc(C.Structure):
                 ("y", C.c_uint64), ("bias", C.c_uint64)]
 
 
-def mv_multi(dev, parts, act=None, xf=None, f16_scale=True, acc=False, glu=False, norm=None, exact_order=False):
-    """PARTS, up to four (W Y BIAS) sharing X, in one launch (CMAT-MUL-N's idea, for one
-    token): X quantized in ACT, or the floats XF, which the kernel then quantizes itself --
-    after RMSNORM! by NORM = (weights DBuf, eps) when given: norm, quantizer and products in
-    one launch."""
+def _descs(parts):
     descs = (MvDesc * len(parts))()
     for i, (w, y, bias) in enumerate(parts):
         descs[i] = MvDesc(w.type, w.rows, w.qs.ptr, w.d.ptr if w.d else 0, y.ptr, bias.ptr if bias else 0)
+    return descs
+
+
+def mv_multi(dev, parts, act=None, xf=None, f16_scale=True, acc=False, glu=False, norm=None, exact_order=False, ahead=None):
+    """PARTS, up to four (W Y BIAS) sharing X, in one launch (CMAT-MUL-N's idea, for one
+    token): X quantized in ACT, or the floats XF, which the kernel then quantizes itself --
+    after RMSNORM! by NORM = (weights DBuf, eps) when given: norm, quantizer and products in
+    one launch.  AHEAD = (parts of the caller's next product, its glu flag): with float activations the launch reads
+    that product's rows ahead into L2 while it runs (ilt_mv_multi_ahead)."""
+    descs = _descs(parts)
     w0 = parts[0][0]
+    if ahead is not None and xf is not None and not exact_order:
+        nparts, nglu = ahead
+        hip.call("ilt_mv_multi_ahead", C.c_uint64(dev.stream), C.c_int(len(parts)), descs, C.c_int(w0.cols), C.c_uint64(xf.ptr),
+                 C.c_uint64(norm[0].ptr if norm is not None else 0), C.c_float(norm[1] if norm is not None else 0.0),
+                 C.c_int(1 if f16_scale else 0), C.c_int(1 if acc else 0), C.c_int(1 if glu else 0),
+                 C.c_int(len(nparts)), _descs(nparts), C.c_int(nparts[0][0].cols), C.c_int(1 if nglu else 0))
+        return
     if norm is not None:
         if xf is None or acc:
             raise ValueError("a norm takes float activations and no accumulation")
@@ -271,10 +284,10 @@ def qkv_mul(dev, wq, wk, wv, act, q, k, v, bq=None, bk=None, bv=None, xf=None, n
     mv_multi(dev, [(wq, q, bq), (wk, k, bk), (wv, v, bv)], act, xf, norm=norm)
 
 
-def glu_mul(dev, g, u, act, fa, xf=None, norm=None):
-    """silu(G x) * (U x) into FA for one token (GLU-MUL, cuda-dense.lisp:326-339)."""
+def glu_mul(dev, g, u, act, fa, xf=None, norm=None, ahead=None):
+    """silu(G x) * (U x) into FA for one token (GLU-MUL, cuda-dense.lisp:326-339).  AHEAD: see mv_multi."""
     if xf is not None:
-        return mv_multi(dev, [(g, fa, None), (u, fa, None)], None, xf, glu=True, norm=norm)
+        return mv_multi(dev, [(g, fa, None), (u, fa, None)], None, xf, glu=True, norm=norm, ahead=ahead)
     f, d = g.rows, g.cols
     if g.kquant_p():
         hip.launch(dev, "mv_k_glu", (f + 3) // 4, 128,

@@ -424,6 +424,37 @@ def test_norm_inside_the_product_bit_exact(dev, kind):
 
 # ---- the streamed variant of the decode product (mid-size Q4_K / Q6_K matrices) -----------------
 
+def test_product_reading_the_next_products_rows_ahead(dev):
+    """ilt_mv_multi_ahead: a layer's gate/up launch told of the down product after it (its idle waves read down's rows
+    ahead into L2), Q/K/V told of wo, and a next product too small for the streamed variant: every result the plain
+    call's, which is the oracle's, and the product read ahead for is right afterwards."""
+    from illatio_amd import dense, hip
+    rng = synth.make_rng(777)
+    d, ffn = 2560, 9728
+    gw, uw, dw = synth.weights(synth.Q4_K, ffn, d, rng), synth.weights(synth.Q4_K, ffn, d, rng), synth.weights(synth.Q6_K, d, ffn, rng)
+    sw = synth.weights(synth.Q6_K, 64, ffn, rng)
+    gm, um, dm, sm = (dense.upload_gmat(dev, n, t, r, c, w) for n, t, r, c, w in
+                      (("g", synth.Q4_K, ffn, d, gw), ("u", synth.Q4_K, ffn, d, uw), ("d", synth.Q6_K, d, ffn, dw), ("s", synth.Q6_K, 64, ffn, sw)))
+    x, nw = special_activations(d, rng), (synth.activations(d, rng) * 0.2 + 1.0).astype(np.float32)
+    xb, nwb = hip.hip_upload_new(dev, x), hip.hip_upload_new(dev, nw)
+    fa, y, ys = hip.hip_alloc(dev, 4 * ffn), hip.hip_alloc(dev, 4 * d), hip.hip_alloc(dev, 4 * 64)
+    h = orc.rmsnorm(x, nw, 1e-6)
+    want_fa = orc.swiglu(orc.matmul(synth.Q4_K, gw, ffn, d, h), orc.matmul(synth.Q4_K, uw, ffn, d, h))
+    for nxt in (([(dm, y, None)], False), ([(sm, ys, None)], False)):
+        dense.glu_mul(dev, gm, um, None, fa, xf=xb, norm=(nwb, 1e-6), ahead=nxt)
+        assert np.array_equal(bits(hip.hip_floats(fa, ffn)), bits(want_fa))
+        dense.mv_multi(dev, [(dm, y, None)], xf=fa)
+        assert np.array_equal(bits(hip.hip_floats(y, d)), bits(orc.matmul(synth.Q6_K, dw, d, ffn, want_fa)))
+    # without a norm, onto what y holds, and told of a gate/up pair
+    before = hip.hip_floats(y, d)
+    dense.mv_multi(dev, [(dm, y, None)], xf=fa, acc=True, ahead=([(gm, fa, None), (um, fa, None)], True))
+    assert np.array_equal(bits(hip.hip_floats(y, d)), bits(before + orc.matmul(synth.Q6_K, dw, d, ffn, want_fa)))
+    for b in (xb, nwb, fa, y, ys):
+        hip.hip_free(b)
+    for m in (gm, um, dm, sm):
+        m.free()
+
+
 @pytest.mark.parametrize("stream", ["1", "0"])        # chosen by shape (these shapes qualify) / never
 def test_streamed_products_bit_exact(dev, monkeypatch, stream):
     """Products of half a megabyte and more over one activation vector take the variant that streams every
