@@ -483,7 +483,9 @@ __global__ __launch_bounds__(256) void attn_values_kernel(const float* __restric
   extern __shared__ __align__(16) float dyn[];
   __shared__ float redf[4];
   __shared__ double redd[8];
-  const int ns = hd >> 4, h = blockIdx.x / ns, cs = blockIdx.x - h * ns, t0 = blockIdx.y * TG, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  // (a head's hd/16 workgroups on one die, as in attn_step_fused_kernel: the head's score rows come into one L2)
+  const int gx = gridDim.x, bx = (gx & 7) ? (int)blockIdx.x : (int)(blockIdx.x & 7) * (gx >> 3) + (int)(blockIdx.x >> 3);
+  const int ns = hd >> 4, h = bx / ns, cs = bx - h * ns, t0 = blockIdx.y * TG, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int tn = min(TG, ntok - t0), nposmax = pos0 + t0 + tn;
   const int group = nh / nkv, kvd = nkv * hd, ko = (h / group) * hd + 16 * cs;
   float* scores = dyn;
