@@ -118,7 +118,9 @@ __device__ __forceinline__ u64 iq2_sign_mask(u32 s7) {      // table entry s7 (0
   const u32 mhi = (((s >> 4) * 0x00204081u) & 0x01010101u) * 0xFFu;
   return ((u64)mhi << 32) | mlo;
 }
-__device__ __forceinline__ int iq2xxs_sub_dot(u32 g, u32 aux, const i8* xb, const u64* grid) {
+// XR: the 32 activations come from registers (xr) instead of LDS (xb).
+template <bool XR = false>
+__device__ __forceinline__ int iq2xxs_sub_dot(u32 g, u32 aux, const i8* xb, const u64* grid, const int2* xr = nullptr) {
   // the eight table reads first, then the dots: read one by one, each dot waits out an LDS round trip
   int2 mag[4], m[4];
 #pragma unroll
@@ -129,7 +131,8 @@ __device__ __forceinline__ int iq2xxs_sub_dot(u32 g, u32 aux, const i8* xb, cons
   int pos = 0, neg = 0;
 #pragma unroll
   for (int l = 0; l < 4; l++) {
-    const int2 x = ilt_lds_ld8(xb + 8 * l);
+    int2 x;
+    if constexpr (XR) x = xr[l]; else x = ilt_lds_ld8(xb + 8 * l);
     pos = ilt_dot4((int)mag[l].y, x.y, ilt_dot4((int)mag[l].x, x.x, pos));
     neg = ilt_dot4((int)(mag[l].y & m[l].y), x.y, ilt_dot4((int)(mag[l].x & m[l].x), x.x, neg));
   }
@@ -199,41 +202,73 @@ template <> __device__ __forceinline__ void block_terms<ILT_Q6_K>(const Raw<ILT_
   if (j == 0) ilt_lds_stf(t, (ilt_h2f(r.d) * ilt_lds_ldf(L.xs + s)) * (float)(isum - 32 * imins));
 }
 
-template <> __device__ __forceinline__ void block_terms<ILT_Q2_K>(const Raw<ILT_Q2_K>& r, int s, int j, const Lds& L, float* t) {
+// A lane's share of one block's activations (and lane 0's: the block's scale), kept in registers
+// over a run of blocks that all sit at the same place in their rows (wave_rows_lds).
+template <int FMT> struct XRegs {};
+template <> struct XRegs<ILT_IQ2_XXS> { int2 x[8]; float xs; };
+template <> struct XRegs<ILT_Q2_K> { int4 x[4]; int4 bs; float xs; };
+template <int FMT> __device__ __forceinline__ void load_xregs(XRegs<FMT>& X, int s, int j, const Lds& L);
+template <> __device__ __forceinline__ void load_xregs<ILT_IQ2_XXS>(XRegs<ILT_IQ2_XXS>& X, int s, int j, const Lds& L) {
+  const i8* xb = L.xq + ilt_mul24(s, XP) + 64 * j;
+#pragma unroll
+  for (int l = 0; l < 8; l++) X.x[l] = ilt_lds_ld8(xb + 8 * l);
+  X.xs = ilt_lds_ldf(L.xs + s);
+}
+template <> __device__ __forceinline__ void load_xregs<ILT_Q2_K>(XRegs<ILT_Q2_K>& X, int s, int j, const Lds& L) {
+  const i8* xb = L.xq + ilt_mul24(s, XP) + 128 * (j >> 1) + 16 * (j & 1);
+#pragma unroll
+  for (int k = 0; k < 4; k++) X.x[k] = ilt_lds_ld16(xb + 32 * k);
+  X.bs = ilt_lds_ld16(L.bsums + s * 16 + 4 * j);
+  X.xs = ilt_lds_ldf(L.xs + s);
+}
+
+template <bool XR>
+__device__ __forceinline__ void block_terms_q2k(const Raw<ILT_Q2_K>& r, int s, int j, const Lds& L, float* t, const XRegs<ILT_Q2_K>* X) {
   const int h = j >> 1, half = j & 1;
-  const i8* xb = L.xq + ilt_mul24(s, XP) + 128 * h + 16 * half;
+  const i8* xb = XR ? nullptr : L.xq + ilt_mul24(s, XP) + 128 * h + 16 * half;
   const u32 wa = (u32)(h ? r.sb.z : r.sb.x) >> (8 * half), wb = (u32)(h ? r.sb.w : r.sb.y) >> (8 * half);
   int isum = 0;
 #pragma unroll
   for (int k = 0; k < 4; k++) {
-    const int dot = ilt_dot16(and4(shr4(r.q, 2 * k), 0x03030303), ilt_lds_ld16(xb + 32 * k), 0);
+    int4 xk;
+    if constexpr (XR) xk = X->x[k]; else xk = ilt_lds_ld16(xb + 32 * k);
+    const int dot = ilt_dot16(and4(shr4(r.q, 2 * k), 0x03030303), xk, 0);
     const u32 sw = ((k < 2 ? wa : wb) >> (16 * (k & 1))) & 0xF;
     isum = ilt_mad24((int)sw, dot, isum);
   }
   const u32 wj = (u32)sel4(r.sb, j);
-  const int4 bs = ilt_lds_ld16(L.bsums + s * 16 + 4 * j);
+  int4 bs;
+  if constexpr (XR) bs = X->bs; else bs = ilt_lds_ld16(L.bsums + s * 16 + 4 * j);
   int mins = ilt_mad24((int)((wj >> 4) & 0xF), bs.x, ilt_mul24((int)((wj >> 12) & 0xF), bs.y));
   mins = ilt_mad24((int)((wj >> 20) & 0xF), bs.z, ilt_mad24((int)(wj >> 28), bs.w, mins));
   isum = ilt_sum4(isum);
   mins = ilt_sum4(mins);
   if (j == 0) {
-    const float ydb = ilt_lds_ldf(L.xs + s);
+    float ydb;
+    if constexpr (XR) ydb = X->xs; else ydb = ilt_lds_ldf(L.xs + s);
     const float d = ydb * ilt_h2f((u16)(r.dd & 0xFFFF)), dmin = (-ydb) * ilt_h2f((u16)(r.dd >> 16));
     ilt_lds_stf2(t, dmin * (float)mins, d * (float)isum);
   }
 }
+template <> __device__ __forceinline__ void block_terms<ILT_Q2_K>(const Raw<ILT_Q2_K>& r, int s, int j, const Lds& L, float* t) {
+  block_terms_q2k<false>(r, s, j, L, t, nullptr);
+}
 
-template <> __device__ __forceinline__ void block_terms<ILT_IQ2_XXS>(const Raw<ILT_IQ2_XXS>& r, int s, int j, const Lds& L, float* t) {
-  const i8* xb = L.xq + ilt_mul24(s, XP) + 64 * j;
+template <bool XR>
+__device__ __forceinline__ void block_terms_iq2xxs(const Raw<ILT_IQ2_XXS>& r, int s, int j, const Lds& L, float* t, const XRegs<ILT_IQ2_XXS>* X) {
+  const i8* xb = XR ? nullptr : L.xq + ilt_mul24(s, XP) + 64 * j;
   const u32 aux0 = (u32)r.q.y, aux1 = (u32)r.q.w;
-  const float te = (float)iq2xxs_sub_dot((u32)r.q.x, aux0, xb, L.grid) * (0.5f + (float)(aux0 >> 28));
-  const float to = (float)iq2xxs_sub_dot((u32)r.q.z, aux1, xb + 32, L.grid) * (0.5f + (float)(aux1 >> 28));
+  const float te = (float)iq2xxs_sub_dot<XR>((u32)r.q.x, aux0, xb, L.grid, XR ? X->x : nullptr) * (0.5f + (float)(aux0 >> 28));
+  const float to = (float)iq2xxs_sub_dot<XR>((u32)r.q.z, aux1, xb + 32, L.grid, XR ? X->x + 4 : nullptr) * (0.5f + (float)(aux1 >> 28));
   // lane 0 adds the even sub-blocks' terms in order, then the odd ones' (ds4's order)
   float a = 0.0f + te, b = 0.0f + to;
   a = a + ilt_dppf<ILT_DPP_SHL(1)>(te); b = b + ilt_dppf<ILT_DPP_SHL(1)>(to);
   a = a + ilt_dppf<ILT_DPP_SHL(2)>(te); b = b + ilt_dppf<ILT_DPP_SHL(2)>(to);
   a = a + ilt_dppf<ILT_DPP_SHL(3)>(te); b = b + ilt_dppf<ILT_DPP_SHL(3)>(to);
-  if (j == 0) ilt_lds_stf(t, (ilt_h2f(r.d) * ilt_lds_ldf(L.xs + s)) * (a + b));
+  if (j == 0) ilt_lds_stf(t, (ilt_h2f(r.d) * (XR ? X->xs : ilt_lds_ldf(L.xs + s))) * (a + b));
+}
+template <> __device__ __forceinline__ void block_terms<ILT_IQ2_XXS>(const Raw<ILT_IQ2_XXS>& r, int s, int j, const Lds& L, float* t) {
+  block_terms_iq2xxs<false>(r, s, j, L, t, nullptr);
 }
 
 // ---- phase B: a row's terms in block order -------------------------------------------------
@@ -795,6 +830,21 @@ __device__ __forceinline__ void wave_rows_lds(const u8* run, const u8* run2, int
   // quarter-rate instructions a step)
   const int step = S > 1 ? GPW - (int)__umulhi((u32)GPW, s_magic) * S : 0;      // GPW mod S
   int s_ = S > 1 ? gl - (int)__umulhi((u32)gl, s_magic) * S : 0;
+  if constexpr (FMT == ILT_IQ2_XXS || FMT == ILT_Q2_K) {
+    // the experts' widths (4096, 2048 columns: S = 16, 8) divide the 16 blocks of a step: a lane's blocks all sit
+    // at one place in their rows, so its share of the activations is read from LDS once, not once a row
+    if (step == 0 && nblk > GPW) {
+      XRegs<FMT> X;
+      load_xregs<FMT>(X, s_, j, L);
+      for (int f = gl; f < nblk; f += GPW) {
+        Raw<FMT> r;
+        load_raw_lds<FMT>(r, run, run2, f, j);
+        if constexpr (FMT == ILT_IQ2_XXS) block_terms_iq2xxs<true>(r, s_, j, L, t + (long)f * F::TERMS, &X);
+        else block_terms_q2k<true>(r, s_, j, L, t + (long)f * F::TERMS, &X);
+      }
+      return;
+    }
+  }
   for (int f = gl; f < nblk; f += GPW) {
     Raw<FMT> r;
     load_raw_lds<FMT>(r, run, run2, f, j);
