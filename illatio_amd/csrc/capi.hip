@@ -505,7 +505,20 @@ int step_args_ok(int ne, int nu, int d, int ff, const ilt_ffn_step_weights* wt, 
               wt->sdown_q && wt->sdown_d);
   return ILT_OK;
 }
-// Six launches on STREAM, nothing allocated, freed or waited for; ws holds step_layout's bytes.
+// The shared expert's down product as the step's last launch, the step's sum carried along (IltSumAlong): MOE gets
+// ((0 + bd[0]) + ... + bd[nu-1]) + W.smid.  hipErrorNotSupported (nothing launched) where the launch cannot take it.
+int shared_down_sum(uint64_t stream, int d, int ff, const int8_t* wq, const uint16_t* wd, const float* smid, const float* bd, int nu,
+                    float* moe) {
+  IltGemvParams p;
+  int live = 0, fmt = ILT_Q8_0, rows = d;
+  const void* w = wq; const float* nobias = nullptr;
+  const int e = gemv_multi_build(p, &live, 1, &fmt, &w, &wd, &moe, &nobias, &rows, ff, nullptr, nullptr, nullptr, smid, 0, 0, 0, 0, nullptr, 0.0f, 0);
+  if (e != ILT_OK) return e;
+  if (live == 0) return (int)hipErrorNotSupported;
+  p.sum = {bd, (long long)d, nu};
+  return (int)ilt_gemv_launch(p, 1, S(stream));
+}
+// Five launches on STREAM, nothing allocated, freed or waited for; ws holds step_layout's bytes.
 int step_run(uint64_t stream, uint8_t* ws, int ne, int nu, int d, int ff, float scale, float clamp, const ilt_ffn_step_weights* wt,
              const float* logits, const float* bias, const float* x, float* moe) {
   const StepLayout l = step_layout(nu, d, ff);
@@ -518,10 +531,14 @@ int step_run(uint64_t stream, uint8_t* ws, int ne, int nu, int d, int ff, float 
   IltRouteAlong route = {logits, bias, sel, w, ne, nu, scale, 0};
   ILT_TRY((hipError_t)mvq8_glu(stream, ff, d, wt->sgate_q, wt->sgate_d, wt->sup_q, wt->sup_d, x, clamp, smid, &route));
   if (!route.done) ILT_TRY((hipError_t)ilt_d4_route(stream, ne, nu, 0, scale, bias ? 1 : 0, logits, bias, nullptr, nullptr, sel, w, 1));
-  ilt_mv_desc down = {ILT_Q8_0, d, wt->sdown_q, wt->sdown_d, sout, nullptr};
-  ILT_TRY((hipError_t)ilt_mv_multi(stream, 1, &down, ff, nullptr, nullptr, nullptr, smid, 0, 0, 0));
   ILT_TRY((hipError_t)ilt_d4_mv_glu_iq2_xxs(stream, d, ff, grb, 0, wt->gate_bytes, 0, ff, wt->slots, sel, nu, x, w, clamp, bm));
   ILT_TRY((hipError_t)ilt_d4_mv_q2_k_f32(stream, ff, d, drb, 2 * wt->gate_bytes, ff, d, wt->slots, sel, nu, bm, bd));
+  // the shared expert's down product last, adding the routed experts' rows and its own as it stores them; where
+  // that launch cannot (more than eight slots, a matrix too small for the streamed variant): the product, then the sum
+  const int e = shared_down_sum(stream, d, ff, wt->sdown_q, wt->sdown_d, smid, bd, nu, moe);
+  if (e != (int)hipErrorNotSupported) return e;
+  ilt_mv_desc down = {ILT_Q8_0, d, wt->sdown_q, wt->sdown_d, sout, nullptr};
+  ILT_TRY((hipError_t)ilt_mv_multi(stream, 1, &down, ff, nullptr, nullptr, nullptr, smid, 0, 0, 0));
   return ilt_d4_moe_sum(stream, d, nu, bd, sout, moe, nullptr);
 }
 }  // namespace

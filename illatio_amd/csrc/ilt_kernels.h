@@ -58,6 +58,17 @@ struct IltRowsAhead {
   struct M { const uint8_t* w; long long row_bytes; int rq, rr, batch0, nbat; } m[4];
 };
 
+// The MoE step's sum carried along by its last product (the shared expert's down launch): y[r] becomes
+// ((0 + rows[0][r]) + rows[1][r] + ...) + (the product's row r) -- the routed experts' down rows added in order, then
+// the shared expert's, as d4-routed! and its caller add them (moe_sum's arithmetic) -- instead of a launch for the
+// sum.  rows null: nothing.  Streamed Q8_0 launches without bias or acc only, k <= 8; ilt_gemv_launch returns
+// hipErrorNotSupported where the launch cannot take it, and has launched nothing then.
+struct IltSumAlong {
+  const float* rows;
+  long long stride;          // floats from one row to the next
+  int k;
+};
+
 struct IltGemvParams {
   IltRouteAlong route;
   IltCacheAhead ahead;
@@ -89,6 +100,7 @@ struct IltGemvParams {
   int region;                // streamed variant: bytes of LDS per wave for its rows (set at launch)
   int nz;                    // streamed variant: experts taking part (set at launch)
   uint32_t s_magic;          // ceil(2^32 / blocks per row)
+  IltSumAlong sum;
 };
 
 // The kernel is chosen by the matrices' formats (mat[i].fmt): one format, or Q4_K and Q6_K mixed.

@@ -961,8 +961,9 @@ __device__ __forceinline__ void rows_ahead(const IltRowsAhead& h, float* sink) {
 // p.ptrs gives the experts' slots and p.nz how many take part: a batch is rows of one expert,
 // batches per expert = p.mat[0].nbat).  p.batch = the most rows a wave takes; p.region = bytes
 // of LDS per wave for its rows (both matrices' when glu).
-// EARLY: the launch adds to y or has a bias (never a gate/up pair): those values are asked for behind the rows.
-template <int FSET, bool EARLY = false>
+// EARLY 1: the launch adds to y or has a bias (never a gate/up pair): those values are asked for behind the rows.
+// EARLY 2: the launch adds its rows to an ordered sum of up to eight vectors (IltSumAlong), asked for likewise.
+template <int FSET, int EARLY = 0>
 __global__ __launch_bounds__(kStreamThreads) void gemv_stream_kernel(IltGemvParams p) {
   extern __shared__ __align__(16) unsigned char smem[];
   constexpr bool iq2 = FSET == ILT_IQ2_XXS, q8 = FSET == ILT_Q8_0;
@@ -1075,7 +1076,12 @@ __global__ __launch_bounds__(kStreamThreads) void gemv_stream_kernel(IltGemvPara
   const long rmine = row0 + min(lane, max(nrows - 1, 0));
   const float* const bsrc = m.bias ? m.bias : ydst;
   float yold = 0.0f, bval = 0.0f;
-  if constexpr (EARLY) { yold = ydst[rmine]; bval = bsrc[rmine]; }
+  float srow[8];
+  if constexpr (EARLY == 1) { yold = ydst[rmine]; bval = bsrc[rmine]; }
+  if constexpr (EARLY == 2) {
+#pragma unroll
+    for (int i = 0; i < 8; i++) srow[i] = p.sum.rows[(long)min(i, p.sum.k - 1) * p.sum.stride + rmine];
+  }
   int nup = 0;              // load instructions of the up matrix's rows: the last ones issued
   if (live) {
     with_format<FSET>(fmt, [&](auto F) { stream_run<decltype(F)::value>(wg, row0, nrows, S, m.row_bytes, region, lane); });
@@ -1128,8 +1134,15 @@ __global__ __launch_bounds__(kStreamThreads) void gemv_stream_kernel(IltGemvPara
         y[r] = o;
       }
     } else {
-      if (m.bias) v = v + (EARLY ? bval : m.bias[r]);
-      if (p.acc) v = (EARLY ? yold : y[r]) + v;
+      if constexpr (EARLY == 2) {
+        float a = 0.0f;
+#pragma unroll
+        for (int i = 0; i < 8; i++) a = i < p.sum.k ? a + srow[i] : a;
+        v = a + v;
+      } else {
+        if (m.bias) v = v + (EARLY ? bval : m.bias[r]);
+        if (p.acc) v = (EARLY ? yold : y[r]) + v;
+      }
       y[r] = v;
     }
   }
@@ -1269,12 +1282,12 @@ static hipError_t gemv_stream_launch(IltGemvParams& p, int fset, int nz, hipStre
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 8) dev = 0;
   if (!attr_set[dev]) {            // more dynamic LDS than the default 64 KB: asked for once per device
-    const void* kernels[10] = { (const void*)gemv_stream_kernel<0>, (const void*)gemv_stream_kernel<ILT_Q4_K>, (const void*)gemv_stream_kernel<ILT_Q6_K>,
+    const void* kernels[11] = { (const void*)gemv_stream_kernel<0>, (const void*)gemv_stream_kernel<ILT_Q4_K>, (const void*)gemv_stream_kernel<ILT_Q6_K>,
                                 (const void*)gemv_stream_kernel<ILT_IQ2_XXS>, (const void*)gemv_stream_kernel<ILT_Q2_K>,
                                 (const void*)gemv_stream_kernel<ILT_Q8_0>, (const void*)gemv_stream_kernel<0, true>,
                                 (const void*)gemv_stream_kernel<ILT_Q4_K, true>, (const void*)gemv_stream_kernel<ILT_Q6_K, true>,
-                                (const void*)gemv_stream_kernel<ILT_Q8_0, true> };
-    for (int i = 0; i < 10; i++)
+                                (const void*)gemv_stream_kernel<ILT_Q8_0, true>, (const void*)gemv_stream_kernel<ILT_Q8_0, 2> };
+    for (int i = 0; i < 11; i++)
       if (hipFuncSetAttribute(kernels[i], hipFuncAttributeMaxDynamicSharedMemorySize, 158 * 1024) != hipSuccess) {
         (void)hipGetLastError();
         return hipErrorNotSupported;
@@ -1284,6 +1297,11 @@ static hipError_t gemv_stream_launch(IltGemvParams& p, int fset, int nz, hipStre
   const dim3 grid(min(256, nb));                                      // wave w of workgroup g takes batch w * grid + g
   bool early = p.acc != 0;
   for (int i = 0; i < p.nmat; i++) early = early || p.mat[i].bias != nullptr;
+  if (p.sum.rows) {                 // (its conditions were checked before the plan was made)
+    hipLaunchKernelGGL((gemv_stream_kernel<ILT_Q8_0, 2>), grid, dim3(kStreamThreads), smem, st, p);
+    g_streamed_launches++;
+    return hipGetLastError();
+  }
   early = early && !p.glu && !p.ptrs;
   if (early) {
     switch (fset) {
@@ -1330,9 +1348,14 @@ hipError_t ilt_gemv_launch(IltGemvParams& p, int nz, hipStream_t st) {
     p.ahead.a = nullptr;                                   // (rows that 16-byte loads cannot take: no reading ahead)
   int fset = p.mat[0].fmt;
   for (int i = 1; i < p.nmat; i++) if (p.mat[i].fmt != fset) fset = 0;
+  if (p.sum.rows) {               // a sum carried along: the streamed Q8_0 launch of one matrix takes it, nothing else does
+    bool ok = fset == ILT_Q8_0 && p.nmat == 1 && !p.acc && !p.mat[0].bias && !p.glu && !p.ptrs && p.group_rows == 0 && nz == 1 &&
+              p.sum.k >= 1 && p.sum.k <= 8 && p.sum.stride >= p.mat[0].rows;
+    if (!ok) return hipErrorNotSupported;
+  }
   {
     const hipError_t e = gemv_stream_launch(p, fset, nz, st);
-    if (e != hipErrorNotSupported) return e;
+    if (e != hipErrorNotSupported || p.sum.rows) return e;
   }
   const bool q8 = fset == ILT_Q8_0;
   const int S = q8 ? p.cols / 32 : p.cols / 256;

@@ -163,11 +163,13 @@ def _moe_weights(rng, ne, d, ff):
     return gate, up, down, sg, su, sd
 
 
-@pytest.mark.parametrize("ne,d,ff,nu,clamp", [(8, 512, 256, 3, 0.0), (8, 512, 256, 3, 0.05), (12, 4096, 2048, 6, 0.0)])
+@pytest.mark.parametrize("ne,d,ff,nu,clamp", [(8, 512, 256, 3, 0.0), (8, 512, 256, 3, 0.05), (12, 4096, 2048, 6, 0.0),
+                                                (12, 2048, 1024, 9, 0.0)])      # (nine slots: the sum as a launch of its own)
 def test_moe_decode_step_bit_exact(dev, ne, d, ff, nu, clamp):
     """the benchmark's config 4's sequence at a reduced expert count (12 resident experts of the
     full 4096 x 2048 shape), and a small shape with the clamp on: route -> gate/up -> gated
-    activation -> per-slot Q8_K -> down -> ordered sum + shared expert."""
+    activation -> per-slot Q8_K -> down -> ordered sum + shared expert.  In the one-call step the sum rides on the
+    shared expert's down launch at the large shape; the small one and the one with nine slots launch it."""
     from illatio_amd import ds4f, hip
     rng = synth.make_rng(ne * 1000 + d)
     gate, up, down, sg, su, sd = _moe_weights(rng, ne, d, ff)
