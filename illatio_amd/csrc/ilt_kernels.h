@@ -70,9 +70,6 @@ struct IltSumAlong {
 };
 
 struct IltGemvParams {
-  IltRouteAlong route;
-  IltCacheAhead ahead;
-  IltRowsAhead rows_ahead;
   IltGemvMat mat[4];         // up to four matrices sharing the activations
   int nmat;
   const uint64_t* ptrs;      // experts: grid y's matrices are at ptrs[y] + mat[i].add,
@@ -100,7 +97,12 @@ struct IltGemvParams {
   int region;                // streamed variant: bytes of LDS per wave for its rows (set at launch)
   int nz;                    // streamed variant: experts taking part (set at launch)
   uint32_t s_magic;          // ceil(2^32 / blocks per row)
+  // (what only some waves read, and late, comes last: the fields every wave needs for its first loads then sit in the
+  // kernel arguments' first cache lines, where a few scalar loads bring them in)
   IltSumAlong sum;
+  IltRouteAlong route;
+  IltCacheAhead ahead;
+  IltRowsAhead rows_ahead;
 };
 
 // The kernel is chosen by the matrices' formats (mat[i].fmt): one format, or Q4_K and Q6_K mixed.
