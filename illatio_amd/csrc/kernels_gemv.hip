@@ -1047,31 +1047,47 @@ __global__ __launch_bounds__(kStreamThreads) void gemv_stream_kernel(IltGemvPara
     return;
   }
   const int rw = wave - kStagers;
-  float* tw = terms + (long)rw * p.batch * tpr * nglu;
-  u8* region = (u8*)(terms + (long)kRowWaves * p.batch * tpr * nglu) + (long)rw * p.region;
   const int wid = rw * gridDim.x + blockIdx.x;          // consecutive batches on different CUs
+  // What a row wave must know before its first loads, read from the arguments in two goes -- the launch's numbers and
+  // the matrices' first batches; then this wave's matrix, whole.  (Argument loads left where the values are used
+  // come one after another, each behind a branch on the one before: a dozen round trips to the scalar cache.)
+  const int a_nbatches = p.nbatches, a_nmat = p.nmat, a_glu = p.glu, a_batch = p.batch, a_region = p.region, a_cols = p.cols;
+  const int b1 = p.mat[1].batch0, b2 = p.mat[2].batch0, b3 = p.mat[3].batch0;
+  const uint64_t* const a_ptrs = p.ptrs;
+  const uint32_t* const a_sel = p.sel;
+  const u8* const u_w = p.mat[1].w;
+  const u16* const u_wd = p.mat[1].wd;
+  const long long u_row_bytes = p.mat[1].row_bytes, u_add = p.mat[1].add;
+  const int u_fmt = p.mat[1].fmt;
+  asm volatile("" ::"s"(a_nbatches), "s"(a_nmat), "s"(a_glu), "s"(a_batch), "s"(a_region), "s"(a_cols), "s"(b1), "s"(b2), "s"(b3), "s"(a_ptrs),
+               "s"(a_sel), "s"(u_w), "s"(u_wd), "s"(u_row_bytes), "s"(u_add), "s"(u_fmt));
+  float* tw = terms + (long)rw * a_batch * tpr * nglu;
+  u8* region = (u8*)(terms + (long)kRowWaves * a_batch * tpr * nglu) + (long)rw * a_region;
 
   // 2. this wave's rows, all of them
   int mi = 0, nrows = 0, z = 0; long row0 = 0;
-  const bool live = wid < p.nbatches;
+  const bool live = wid < a_nbatches;
+  // (the matrices' first batches rise: the matrix of batch wid is the last one that starts at or before it)
+  if (!a_ptrs && !a_glu) mi = (a_nmat > 1 && wid >= b1 ? 1 : 0) + (a_nmat > 2 && wid >= b2 ? 1 : 0) + (a_nmat > 3 && wid >= b3 ? 1 : 0);
+  const IltGemvMat m = p.mat[mi];
+  asm volatile("" ::"s"(m.w), "s"(m.wd), "s"(m.y), "s"(m.bias), "s"(m.row_bytes), "s"(m.add), "s"(m.rows), "s"(m.fmt), "s"(m.batch0),
+               "s"(m.nbat), "s"(m.rq), "s"(m.rr));
   int bl = wid;
   if (live) {
-    if (p.ptrs) { z = wid / p.mat[0].nbat; bl = wid - z * p.mat[0].nbat; }
-    else if (!p.glu) { while (mi + 1 < p.nmat && wid >= p.mat[mi + 1].batch0) mi++; bl = wid - p.mat[mi].batch0; }
-    const int rq = p.mat[mi].rq, rr = p.mat[mi].rr;
-    row0 = (long)bl * rq + min(bl, rr);
-    nrows = rq + (bl < rr ? 1 : 0);
+    if (a_ptrs) { z = wid / m.nbat; bl = wid - z * m.nbat; }
+    else if (!a_glu) bl = wid - m.batch0;
+    row0 = (long)bl * m.rq + min(bl, m.rr);
+    nrows = m.rq + (bl < m.rr ? 1 : 0);
   }
-  const IltGemvMat& m = p.mat[mi];
   const int fmt = FSET != 0 ? FSET : m.fmt;
-  const int ufmt = FSET != 0 ? FSET : p.mat[1].fmt;
-  const u8* slot = (live && p.ptrs) ? (const u8*)p.ptrs[p.sel ? p.sel[z] : z] : nullptr;
-  const u8* wg = p.ptrs ? slot + m.add : m.w;
-  const u8* wu = p.ptrs ? slot + p.mat[1].add : p.mat[1].w;
-  u8* region_up = region + p.region / 2;
+  const int ufmt = FSET != 0 ? FSET : u_fmt;
+  const u8* slot = (live && a_ptrs) ? (const u8*)a_ptrs[a_sel ? a_sel[z] : z] : nullptr;
+  const u8* wg = a_ptrs ? slot + m.add : m.w;
+  const u8* wu = a_ptrs ? slot + u_add : u_w;
+  u8* region_up = region + a_region / 2;
   // Q8_0: the scales' room behind the quants'
-  const u8* scales = region + (long)p.batch * p.cols;
-  const u8* scales_up = region_up + (long)p.batch * p.cols;
+  const u8* scales = region + (long)a_batch * a_cols;
+  const u8* scales_up = region_up + (long)a_batch * a_cols;
   // What the sum is added to (acc) and the bias are asked for ahead of the rows: they are there when the sums are,
   // instead of a trip to memory after them (asked for behind the rows they come in last and gain nothing).
   float* const ydst = m.y + (long)z * p.y_stride;
@@ -1088,9 +1104,9 @@ __global__ __launch_bounds__(kStreamThreads) void gemv_stream_kernel(IltGemvPara
   if (live) {
     with_format<FSET>(fmt, [&](auto F) { stream_run<decltype(F)::value>(wg, row0, nrows, S, m.row_bytes, region, lane); });
     if (q8) stream_scales((const u8*)(m.wd + row0 * S), nrows * S * 2, (u8*)scales, lane);
-    if (p.glu) {
-      with_format<FSET>(ufmt, [&](auto F) { nup = stream_run<decltype(F)::value>(wu, row0, nrows, S, p.mat[1].row_bytes, region_up, lane); });
-      if (q8) nup += stream_scales((const u8*)(p.mat[1].wd + row0 * S), nrows * S * 2, (u8*)scales_up, lane);
+    if (a_glu) {
+      with_format<FSET>(ufmt, [&](auto F) { nup = stream_run<decltype(F)::value>(wu, row0, nrows, S, u_row_bytes, region_up, lane); });
+      if (q8) nup += stream_scales((const u8*)(u_wd + row0 * S), nrows * S * 2, (u8*)scales_up, lane);
     }
   }
   // (no branch around the loads, which the compiler would wait out at the join: a launch that has neither runs the
