@@ -175,17 +175,17 @@ __device__ __forceinline__ void ilt_lds_st16_untracked(void* p, int a, int b, in
 // A kernel's arguments sit in device memory that nothing has read yet: the first scalar load from each of their
 // 64-byte lines is a trip to memory, and code that reads an argument, branches on it and reads the next makes those
 // trips one after another (a launch whose arguments were left in host memory took 3.8 us longer).  This asks for
-// one dword of each of the first 12 lines (768 bytes) at once and waits for them together; the loads that follow
-// find the lines in the scalar cache.  Loads only.
-__device__ __forceinline__ void ilt_kernarg_warm12() {
+// one dword of each of the first 7 lines (448 bytes: what every wave of the product kernels reads before its first
+// loads) at once and waits for them together; the loads that follow find the lines in the scalar cache.  (All 12
+// lines of those kernels' arguments: 0.25 % slower; the later ones are read by few waves, late.)  Loads only.
+__device__ __forceinline__ void ilt_kernarg_warm7() {
   const auto k = __builtin_amdgcn_kernarg_segment_ptr();
-  unsigned t0, t1, t2, t3, t4, t5, t6, t7, t8, t9, t10, t11;
+  unsigned t0, t1, t2, t3, t4, t5, t6;
   asm volatile(
-      "s_load_dword %0, %12, 0x0\n\ts_load_dword %1, %12, 0x40\n\ts_load_dword %2, %12, 0x80\n\ts_load_dword %3, %12, 0xc0\n\t"
-      "s_load_dword %4, %12, 0x100\n\ts_load_dword %5, %12, 0x140\n\ts_load_dword %6, %12, 0x180\n\ts_load_dword %7, %12, 0x1c0\n\t"
-      "s_load_dword %8, %12, 0x200\n\ts_load_dword %9, %12, 0x240\n\ts_load_dword %10, %12, 0x280\n\ts_load_dword %11, %12, 0x2c0\n\t"
+      "s_load_dword %0, %7, 0x0\n\ts_load_dword %1, %7, 0x40\n\ts_load_dword %2, %7, 0x80\n\ts_load_dword %3, %7, 0xc0\n\t"
+      "s_load_dword %4, %7, 0x100\n\ts_load_dword %5, %7, 0x140\n\ts_load_dword %6, %7, 0x180\n\t"
       "s_waitcnt lgkmcnt(0)"
-      : "=&s"(t0), "=&s"(t1), "=&s"(t2), "=&s"(t3), "=&s"(t4), "=&s"(t5), "=&s"(t6), "=&s"(t7), "=&s"(t8), "=&s"(t9), "=&s"(t10), "=&s"(t11)
+      : "=&s"(t0), "=&s"(t1), "=&s"(t2), "=&s"(t3), "=&s"(t4), "=&s"(t5), "=&s"(t6)
       : "s"(k)
       : "memory");
 }

@@ -965,8 +965,8 @@ __device__ __forceinline__ void rows_ahead(const IltRowsAhead& h, float* sink) {
 // EARLY 2: the launch adds its rows to an ordered sum of up to eight vectors (IltSumAlong), asked for likewise.
 template <int FSET, int EARLY = 0>
 __global__ __launch_bounds__(kStreamThreads) void gemv_stream_kernel(IltGemvParams p) {
-  static_assert(sizeof(IltGemvParams) <= 768, "ilt_kernarg_warm12 covers 768 bytes");
-  ilt_kernarg_warm12();
+  static_assert(offsetof(IltGemvParams, route) <= 456 && sizeof(IltGemvParams) >= 448, "ilt_kernarg_warm7 covers the arguments' first 448 bytes");
+  ilt_kernarg_warm7();
   extern __shared__ __align__(16) unsigned char smem[];
   constexpr bool iq2 = FSET == ILT_IQ2_XXS, q8 = FSET == ILT_Q8_0;
   const int S = q8 ? p.cols / 32 : p.cols / 256;
