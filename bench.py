@@ -27,7 +27,7 @@ Other workloads (--workload), each the benchmark configuration of the same numbe
   c4  MoE decode step: 256 resident experts (IQ2_XXS gate/up, Q2_K down), top-6, the Q8_0
       shared expert, rotating over 3 layers' pools (5.4 GB); routing tables made beforehand;
       --mode fused (default): 5 launches a step; --mode single: the reference's 12;
-      --mode device: routing on the device inside the step, one call into the library (5 launches, no host tables)
+      --mode device: routing on the device inside the step, one call into the library (4 launches, no host tables)
   c5  MoE prefill chunk: 4096 tokens, Zipf(1.1)-skewed top-6 routing, route -> group ->
       gather -> grouped gate, up -> gated activation -> grouped down -> ordered sum
 Weights and activations are synthetic and seeded (illatio_amd/synth.py); inputs are resident
@@ -519,7 +519,7 @@ def workload_c4(args, dev):
         ws.reset()
         L = i % nlayers
         sel, w = routes[i] if routes[i] else (None, None)
-        if ondev and not tm.probing:             # the step as one call into the library (the routing rides along with the shared expert's gate/up launch: 5 launches)
+        if ondev and not tm.probing:             # the step as one call into the library (the routing rides along with the shared expert's gate/up launch, the sum with its down launch: 4 launches)
             ds4f.ffn_step_call(dev, pools[L], shared[L], logits[i], xb, moe_out, ne, nu, 1.5, 0.0, wsbuf=step_ws)
         elif ondev:                              # the probing pass: the same kernels launched one by one (6 launches), an event pair around each
             ds4f.ffn_step_device(dev, pools[L], shared[L], logits[i], xb, ne, nu, 1.5, 0.0, ws=ws)
@@ -574,7 +574,7 @@ def workload_c4(args, dev):
             "metric": "MoE decode step achieved HBM GB/s (% of 8 TB/s)",
             "config": {"workload": f"c4: MoE decode step, 256 resident experts (IQ2_XXS gate/up, Q2_K down) top-6 + Q8_0 shared expert, "
                                    f"d 4096, ff 2048, batch 1, rotating over {nlayers} layers", "bytes_per_step": step_bytes},
-            "extra": {"pct_of_hbm_peak": round(100 * gbs / HBM_PEAK_GBS, 2), "launches_per_step": 6 if ondev else 5 if fused else 12,
+            "extra": {"pct_of_hbm_peak": round(100 * gbs / HBM_PEAK_GBS, 2), "launches_per_step": 4 if ondev else 5 if fused else 12,
                       "launch_mode": args.mode}, "roofline": roof, "cpu": cpu}
 
 

@@ -255,8 +255,9 @@ def step_workspace_bytes(nu, d, ff):
 
 
 def ffn_step_call(dev, pool, sh, logits, norm2, moe, ne, nu, scale, clamp, bias=None, wsbuf=None):
-    """ffn_step_device's step queued by one call into the library (ilt_d4_ffn_step; five launches, the routing carried
-    along by the shared expert's gate/up launch where that launch is the streamed one, else six): the
+    """ffn_step_device's step queued by one call into the library (ilt_d4_ffn_step; four launches, the routing carried
+    along by the shared expert's gate/up launch and the ordered sum by its down launch where those launches are the
+    streamed ones, else one launch more for each): the
     host crosses the boundary once a layer instead of once a launch.  WSBUF: a DBuf of
     step_workspace_bytes for the intermediate results (one is made and freed if None);
     MOE: the output DBuf (d floats)."""

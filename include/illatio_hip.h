@@ -228,10 +228,13 @@ int ilt_d4_mvq8_glu(uint64_t stream, int rows, int cols, const int8_t* gq, const
 
 /* One token's FFN past the router in one call: DK-FFN-HEAD's shared expert and DK-FFN-TAIL
    (cuda-ds4f.lisp:883-956) with the routing left on the device (the reference copies the
-   logits out, waits and routes on the CPU in every layer, :991-999).  Five launches on stream:
+   logits out, waits and routes on the CPU in every layer, :991-999).  Four launches on stream:
    d4_mvq8_glu (one of whose waves does d4_route's work while the rows stream in: up to 256 experts and a
-   shared expert large enough for the streamed product, else d4_route is a sixth launch), the shared
-   expert's down, d4_mv_glu_iq2_xxs and d4_mv_q2_k_f32 indexed by the routing's sel, d4_moe_sum; moe[d] = the nu routed experts' rows in slot order + the shared
+   shared expert large enough for the streamed product, else d4_route is a launch of its own),
+   d4_mv_glu_iq2_xxs and d4_mv_q2_k_f32 indexed by the routing's sel, and last the shared expert's down
+   product, which adds the routed experts' rows in slot order and then its own as it stores them (d4_moe_sum's
+   arithmetic; up to 8 slots and a matrix large enough for the streamed product, else the product and d4_moe_sum
+   are two launches); moe[d] = the nu routed experts' rows in slot order + the shared
    expert's, with the CPU path's bits (d4-ffn without HC, ds4f.lisp:980-992).  Nothing is
    allocated, freed or waited for.  The intermediate results (sel, weights, the two gated
    activations, the shared expert's row, one down row per slot) live in ws, 256-byte aligned,
