@@ -1262,7 +1262,18 @@ static hipError_t gemv_stream_launch(IltGemvParams& p, int fset, int nz, hipStre
     nb = nbz * nz;
   } else {
     // every wave one batch: the waves are shared out over the matrices by rows, never more than there are
-    const int nb_total = (int)min((long)kWavesAll, total_rows);
+    int nb_total = (int)min((long)kWavesAll, total_rows);
+    if (total_rows >= kWavesAll) {
+      // A wave forms its terms 16 blocks (Q8_0: 32) a step, so a wave with 20 blocks takes two steps as one with 30
+      // does: two row waves a SIMD with three rows each then take 4 steps a SIMD where three with two rows take 6.
+      // Two waves a SIMD where that saves a quarter of the steps and the rows still fit.
+      const int gpw = q8 ? 32 : 16;
+      auto steps = [&](int waves) { const long r = (total_rows + waves - 1) / waves; return (waves / 1024) * ((r * S + gpw - 1) / gpw); };
+      const long r2 = (total_rows + 2047) / 2048;
+      const long one2 = q8 ? (r2 * (p.cols + 2 * S) + 15) / 16 * 16 : r2 * S * 224;
+      const size_t smem2 = (size_t)S * nx * (XP + 16 * 4 + 4) + 3200 + (size_t)kRowWaves * r2 * S * 2 * 4 * (p.glu ? 2 : 1) + (size_t)kRowWaves * one2 * (p.glu ? 2 : 1);
+      if (steps(2048) * 4 <= steps(kWavesAll) * 3 && r2 <= 16 && smem2 <= 150 * 1024) nb_total = 2048;
+    }
     int given = 0;
     for (int i = 0; i < nm; i++) {
       int nbi = (int)((long)nb_total * p.mat[i].rows / total_rows);
