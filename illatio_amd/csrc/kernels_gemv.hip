@@ -170,7 +170,7 @@ template <> __device__ __forceinline__ void block_terms<ILT_Q4_K>(const Raw<ILT_
   if (j == 0) {
     const float ydi = ilt_lds_ldf(L.xs + s);
     const float d = ydi * ilt_h2f((u16)(r.hdr.x & 0xFFFF)), dmin = ydi * ilt_h2f((u16)((u32)r.hdr.x >> 16));
-    ilt_lds_stf2(t, dmin * (float)imin, d * (float)isum);
+    ilt_lds_stf2(t, -(dmin * (float)imin), d * (float)isum);        // (-A, B): the row's sum subtracts A (row_sum)
   }
 }
 
@@ -272,27 +272,58 @@ template <> __device__ __forceinline__ void block_terms<ILT_IQ2_XXS>(const Raw<I
 }
 
 // ---- phase B: a row's terms in block order -------------------------------------------------
-// The adds are a chain; the LDS reads are not, so they go eight blocks ahead of it.
-template <int FMT> __device__ __forceinline__ float row_sum(const float* t, int S) {
-  constexpr int TERMS = Fmt<FMT>::TERMS;
-  float sum = 0.0f;
-  int s = 0;
-  for (; s + 8 <= S; s += 8) {
-    float v[8 * TERMS];
-#pragma unroll
-    for (int k = 0; k < 8 * TERMS; k++) v[k] = ilt_lds_ldf(t + s * TERMS + k);
-#pragma unroll
-    for (int k = 0; k < 8; k++) {
-      if (FMT == ILT_Q4_K) { sum = sum - v[2 * k]; sum = sum + v[2 * k + 1]; }
-      else if (FMT == ILT_Q2_K) { sum = sum + v[2 * k]; sum = sum + v[2 * k + 1]; }
-      else sum = sum + v[k];
+// The adds are a chain (a dependent add issues every 8 cycles or so); the LDS reads are not, so 16 terms are on their
+// way while the 16 before them are added.  Left to itself the compiler moves every read down to its use and the
+// chain waits for LDS once a batch: the reads are inline asm with their own waits.  ds_read2_b32: the terms of a
+// row are 4-byte aligned, no more.  A read past the row's end starts again at its last 16 terms instead.
+typedef float ilt_f2v __attribute__((ext_vector_type(2)));
+#define ILT_TERMS16_AHEAD(A, P)                                                                                                            \
+  asm volatile("ds_read2_b32 %0, %8 offset1:1\n\tds_read2_b32 %1, %8 offset0:2 offset1:3\n\tds_read2_b32 %2, %8 offset0:4 offset1:5\n\t"   \
+               "ds_read2_b32 %3, %8 offset0:6 offset1:7\n\tds_read2_b32 %4, %8 offset0:8 offset1:9\n\tds_read2_b32 %5, %8 offset0:10 offset1:11\n\t" \
+               "ds_read2_b32 %6, %8 offset0:12 offset1:13\n\tds_read2_b32 %7, %8 offset0:14 offset1:15"                                    \
+               : "=&v"(A##0), "=&v"(A##1), "=&v"(A##2), "=&v"(A##3), "=&v"(A##4), "=&v"(A##5), "=&v"(A##6), "=&v"(A##7)                  \
+               : "v"((u32)(uintptr_t)(ILT_LDS const void*)(P)) : "memory")
+#define ILT_TERMS16_WAIT(A, LEFT)                                                                                                          \
+  asm volatile("s_waitcnt lgkmcnt(" #LEFT ")" : "+v"(A##0), "+v"(A##1), "+v"(A##2), "+v"(A##3), "+v"(A##4), "+v"(A##5), "+v"(A##6), "+v"(A##7) :: "memory")
+#define ILT_TERMS16_ADD(O, A)                                                                                                              \
+  do {                                                                                                                                     \
+    O = O + (A##0).x; O = O + (A##0).y; O = O + (A##1).x; O = O + (A##1).y; O = O + (A##2).x; O = O + (A##2).y; O = O + (A##3).x; O = O + (A##3).y;        \
+    O = O + (A##4).x; O = O + (A##4).y; O = O + (A##5).x; O = O + (A##5).y; O = O + (A##6).x; O = O + (A##6).y; O = O + (A##7).x; O = O + (A##7).y;        \
+  } while (0)
+__device__ __forceinline__ float chain_terms(const float* t, int n) {       // ((0 + t[0]) + t[1]) + ... + t[n-1]
+  float o = 0.0f;
+  int q = 0;
+  if (n >= 64) {                                // a long row (Q8_0: a term every 32 columns)
+    ilt_f2v a0, a1, a2, a3, a4, a5, a6, a7, b0, b1, b2, b3, b4, b5, b6, b7;
+    ILT_TERMS16_AHEAD(a, t);
+    for (; q + 32 <= n; q += 32) {
+      ILT_TERMS16_AHEAD(b, t + q + 16);
+      ILT_TERMS16_WAIT(a, 8);
+      ILT_TERMS16_ADD(o, a);
+      ILT_TERMS16_AHEAD(a, t + min(q + 32, n - 16));
+      ILT_TERMS16_WAIT(b, 8);
+      ILT_TERMS16_ADD(o, b);
+    }
+    ILT_TERMS16_WAIT(a, 0);
+    if (q + 16 <= n) {                          // a holds terms q .. q+15
+      ILT_TERMS16_ADD(o, a);
+      q += 16;
     }
   }
-  for (; s < S; s++) {
-    if (FMT == ILT_Q4_K) { sum = sum - ilt_lds_ldf(t + 2 * s); sum = sum + ilt_lds_ldf(t + 2 * s + 1); }
-    else if (FMT == ILT_Q2_K) { sum = sum + ilt_lds_ldf(t + 2 * s); sum = sum + ilt_lds_ldf(t + 2 * s + 1); }
-    else sum = sum + ilt_lds_ldf(t + s);
+  // a short row, or a long one's last terms: eight reads together, then their adds
+  for (; q + 8 <= n; q += 8) {
+    float v[8];
+#pragma unroll
+    for (int k = 0; k < 8; k++) v[k] = ilt_lds_ldf(t + q + k);
+#pragma unroll
+    for (int k = 0; k < 8; k++) o = o + v[k];
   }
+  for (; q < n; q++) o = o + ilt_lds_ldf(t + q);
+  return o;
+}
+// Q4_K's two terms a block are stored as -A and B: sum - A + B is sum + (-A) + B to the bit.
+template <int FMT> __device__ __forceinline__ float row_sum(const float* t, int S) {
+  float sum = chain_terms(t, S * Fmt<FMT>::TERMS);
   if (FMT == ILT_IQ2_XXS) sum = 0.25f * sum;
   return sum;
 }
@@ -1135,13 +1166,22 @@ __global__ __launch_bounds__(kStreamThreads) void gemv_stream_kernel(IltGemvPara
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
   __builtin_amdgcn_wave_barrier();
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  // A row's sum is one lane's chain of adds.  Of a gate/up pair the gate rows are summed by lanes 0.., the up rows by
+  // lanes 32.. at the same time (a wave has at most 16 rows), and a lane of the first half fetches its partner's sum.
+  const int tper = (fmt == ILT_Q4_K || fmt == ILT_Q2_K) ? 2 : 1, uper = (ufmt == ILT_Q4_K || ufmt == ILT_Q2_K) ? 2 : 1;      // floats a block
+  const int rl = lane & 31;
+  const bool up_lane = lane >= 32;
+  float v = 0.0f;
+  if (rl < nrows && (!up_lane || a_glu)) {        // (one call for both halves: two would run one after the other)
+    const int per = up_lane ? uper : tper;
+    v = chain_terms(up_lane ? tw + (long)a_batch * tpr + (long)rl * S * uper : tw + (long)rl * S * tper, S * per);
+    if ((up_lane ? ufmt : fmt) == ILT_IQ2_XXS) v = 0.25f * v;
+  }
+  const float uv = __int_as_float(__builtin_amdgcn_ds_bpermute(4 * (lane ^ 32), __float_as_int(v)));
   if (lane < nrows) {
-    const int tper = (fmt == ILT_Q4_K || fmt == ILT_Q2_K) ? 2 : 1, uper = (ufmt == ILT_Q4_K || ufmt == ILT_Q2_K) ? 2 : 1;      // floats a block
-    float v = sum_any(fmt, tw + (long)lane * S * tper, S);
     const long r = row0 + lane;
     float* y = m.y + (long)z * p.y_stride;
     if (p.glu) {
-      const float uv = sum_any(ufmt, tw + (long)p.batch * tpr + (long)lane * S * uper, S);
       if (p.glu == 1) {
         y[r] = dense_glu(v, uv);
       } else {        // the experts' gated activation, as d4_swiglu_w computes it
