@@ -497,25 +497,35 @@ __device__ __forceinline__ void stage_q8k_from_f32(const float* __restrict__ x, 
 
 // Q8_0 (quantize-q8!, tensor.lisp:245-262): 8 lanes a block of 32.  XSUM: each block's sum of
 // quants as well.  NW, NSCALE, H as for the Q8_K staging.
-__device__ __forceinline__ void stage_q8_from_f32(const float* __restrict__ x, int nblk, int f16_scale, i8* lxq, float* lxs,
-                                                  int* xsum = nullptr, const float* __restrict__ nw = nullptr, float nscale = 1.0f,
-                                                  float* __restrict__ h = nullptr) {
-  const int n8 = nblk * 8;
-  for (int c0 = 0; c0 < n8; c0 += kThreads) {
-    const int c = c0 + threadIdx.x;
-    float4 v = c < n8 ? *(const float4*)(x + 4 * c) : make_float4(0.f, 0.f, 0.f, 0.f);
+// NP passes of the workgroup's first 256 threads over the blocks' float4s from c0 on: every pass's loads are asked for
+// before the first is quantized (a pass a trip to memory otherwise), without a branch around any of them (past the
+// end: the last float4 again; nothing is stored for it).
+template <int NP>
+__device__ __forceinline__ void stage_q8_passes(const float* __restrict__ x, int n8, int c0, int f16_scale, i8* lxq, float* lxs, int* xsum,
+                                                const float* __restrict__ nw, float nscale, float* __restrict__ h) {
+  float4 v[NP], n[NP];
+  const float* const nwp = nw ? nw : x;
+#pragma unroll
+  for (int i = 0; i < NP; i++) {
+    const int cc = min(c0 + i * kThreads + (int)threadIdx.x, n8 - 1);
+    v[i] = *(const float4*)(x + 4 * cc);
+    n[i] = *(const float4*)(nwp + 4 * cc);
+  }
+#pragma unroll
+  for (int i = 0; i < NP; i++) {
+    const int c = c0 + i * kThreads + (int)threadIdx.x;
+    float4 w = v[i];
     if (nw) {
-      const float4 n = c < n8 ? *(const float4*)(nw + 4 * c) : make_float4(0.f, 0.f, 0.f, 0.f);
-      v = make_float4((v.x * nscale) * n.x, (v.y * nscale) * n.y, (v.z * nscale) * n.z, (v.w * nscale) * n.w);
-      if (h && c < n8) *(float4*)(h + 4 * c) = v;
+      w = make_float4((w.x * nscale) * n[i].x, (w.y * nscale) * n[i].y, (w.z * nscale) * n[i].z, (w.w * nscale) * n[i].w);
+      if (h && c < n8) *(float4*)(h + 4 * c) = w;
     }
-    float amax = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
+    float amax = fmaxf(fmaxf(fabsf(w.x), fabsf(w.y)), fmaxf(fabsf(w.z), fabsf(w.w)));
     amax = fmaxf(amax, ilt_dppf<ILT_DPP_XOR1>(amax));
     amax = fmaxf(amax, ilt_dppf<ILT_DPP_XOR2>(amax));
     amax = fmaxf(amax, ilt_dppf<ILT_DPP_HALF_MIRROR>(amax));
     const float d = amax / 127.0f;
     const float id = d == 0.0f ? 0.0f : 1.0f / d;
-    const int q0 = (int)rintf(v.x * id), q1 = (int)rintf(v.y * id), q2 = (int)rintf(v.z * id), q3 = (int)rintf(v.w * id);
+    const int q0 = (int)rintf(w.x * id), q1 = (int)rintf(w.y * id), q2 = (int)rintf(w.z * id), q3 = (int)rintf(w.w * id);
     const int qs = xsum ? ilt_sum8(q0 + q1 + q2 + q3) : 0;
     if (c < n8) {
       *(int*)(lxq + 4 * c) = (q0 & 0xFF) | ((q1 & 0xFF) << 8) | ((q2 & 0xFF) << 16) | ((q3 & 0xFF) << 24);
@@ -525,6 +535,16 @@ __device__ __forceinline__ void stage_q8_from_f32(const float* __restrict__ x, i
       }
     }
   }
+}
+__device__ __forceinline__ void stage_q8_from_f32(const float* __restrict__ x, int nblk, int f16_scale, i8* lxq, float* lxs,
+                                                  int* xsum = nullptr, const float* __restrict__ nw = nullptr, float nscale = 1.0f,
+                                                  float* __restrict__ h = nullptr) {
+  const int n8 = nblk * 8;
+  int c0 = 0;
+  for (; c0 + 3 * kThreads < n8; c0 += 4 * kThreads) stage_q8_passes<4>(x, n8, c0, f16_scale, lxq, lxs, xsum, nw, nscale, h);
+  if (c0 + 2 * kThreads < n8) stage_q8_passes<3>(x, n8, c0, f16_scale, lxq, lxs, xsum, nw, nscale, h);
+  else if (c0 + kThreads < n8) stage_q8_passes<2>(x, n8, c0, f16_scale, lxq, lxs, xsum, nw, nscale, h);
+  else if (c0 < n8) stage_q8_passes<1>(x, n8, c0, f16_scale, lxq, lxs, xsum, nw, nscale, h);
 }
 
 // ---- rmsnorm!'s scale (model.lisp:205-214) ----------------------------------------------------
