@@ -39,9 +39,11 @@ __device__ __forceinline__ float route_prob(float logit) { return sqrtf(softplus
 
 // One token by one wave (all 64 lanes active): lg its ne logits, bs its bias or null, eids its nu experts when they
 // come from a table (hash layers) or null; sel and wout its nu slots; s_idx and s_sc 64 entries of LDS of this wave's.
-template <int K>
+// PRE: the lane's K logits (expert k*64 + lane) and biases were read beforehand, into plg and pbs.
+template <int K, bool PRE = false>
 __device__ __forceinline__ void route_token(int lane, int ne, int nu, float scale, const float* __restrict__ lg, const float* __restrict__ bs,
-                                            const int* __restrict__ eids, u32* __restrict__ sel, float* __restrict__ wout, u32* s_idx, float* s_sc) {
+                                            const int* __restrict__ eids, u32* __restrict__ sel, float* __restrict__ wout, u32* s_idx, float* s_sc,
+                                            const float* plg = nullptr, const float* pbs = nullptr) {
   u32 my_sel = 0;
   float my_p = 0.0f;
   if (eids) {
@@ -59,8 +61,8 @@ __device__ __forceinline__ void route_token(int lane, int ne, int nu, float scal
       const int e = k * 64 + lane;
       p[k] = 0.0f; sc[k] = 0.0f;
       if (e < ne) {
-        p[k] = route_prob(lg[e]);
-        sc[k] = (bs ? p[k] + bs[e] : p[k]) + 0.0f;            // + 0: no minus zero, which the integer key would rank below zero
+        p[k] = route_prob(PRE ? plg[k] : lg[e]);
+        sc[k] = (bs ? p[k] + (PRE ? pbs[k] : bs[e]) : p[k]) + 0.0f;      // + 0: no minus zero, which the integer key would rank below zero
         left |= 1u << k;
         nan |= sc[k] != sc[k];
       }

@@ -502,18 +502,18 @@ __device__ __forceinline__ void stage_q8k_from_f32(const float* __restrict__ x, 
 // end: the last float4 again; nothing is stored for it).
 template <int NP>
 __device__ __forceinline__ void stage_q8_passes(const float* __restrict__ x, int n8, int c0, int f16_scale, i8* lxq, float* lxs, int* xsum,
-                                                const float* __restrict__ nw, float nscale, float* __restrict__ h) {
+                                                const float* __restrict__ nw, float nscale, float* __restrict__ h, int tid, int nthreads) {
   float4 v[NP], n[NP];
   const float* const nwp = nw ? nw : x;
 #pragma unroll
   for (int i = 0; i < NP; i++) {
-    const int cc = min(c0 + i * kThreads + (int)threadIdx.x, n8 - 1);
+    const int cc = min(c0 + i * nthreads + tid, n8 - 1);
     v[i] = *(const float4*)(x + 4 * cc);
     n[i] = *(const float4*)(nwp + 4 * cc);
   }
 #pragma unroll
   for (int i = 0; i < NP; i++) {
-    const int c = c0 + i * kThreads + (int)threadIdx.x;
+    const int c = c0 + i * nthreads + tid;
     float4 w = v[i];
     if (nw) {
       w = make_float4((w.x * nscale) * n[i].x, (w.y * nscale) * n[i].y, (w.z * nscale) * n[i].z, (w.w * nscale) * n[i].w);
@@ -536,15 +536,18 @@ __device__ __forceinline__ void stage_q8_passes(const float* __restrict__ x, int
     }
   }
 }
+// TID, NTHREADS: the threads that stage (a multiple of 8, eight lanes a block), numbered from 0: the workgroup's first
+// 256 unless said otherwise.
 __device__ __forceinline__ void stage_q8_from_f32(const float* __restrict__ x, int nblk, int f16_scale, i8* lxq, float* lxs,
                                                   int* xsum = nullptr, const float* __restrict__ nw = nullptr, float nscale = 1.0f,
-                                                  float* __restrict__ h = nullptr) {
+                                                  float* __restrict__ h = nullptr, int tid = -1, int nthreads = kThreads) {
+  if (tid < 0) tid = (int)threadIdx.x;
   const int n8 = nblk * 8;
   int c0 = 0;
-  for (; c0 + 3 * kThreads < n8; c0 += 4 * kThreads) stage_q8_passes<4>(x, n8, c0, f16_scale, lxq, lxs, xsum, nw, nscale, h);
-  if (c0 + 2 * kThreads < n8) stage_q8_passes<3>(x, n8, c0, f16_scale, lxq, lxs, xsum, nw, nscale, h);
-  else if (c0 + kThreads < n8) stage_q8_passes<2>(x, n8, c0, f16_scale, lxq, lxs, xsum, nw, nscale, h);
-  else if (c0 < n8) stage_q8_passes<1>(x, n8, c0, f16_scale, lxq, lxs, xsum, nw, nscale, h);
+  for (; c0 + 3 * nthreads < n8; c0 += 4 * nthreads) stage_q8_passes<4>(x, n8, c0, f16_scale, lxq, lxs, xsum, nw, nscale, h, tid, nthreads);
+  if (c0 + 2 * nthreads < n8) stage_q8_passes<3>(x, n8, c0, f16_scale, lxq, lxs, xsum, nw, nscale, h, tid, nthreads);
+  else if (c0 + nthreads < n8) stage_q8_passes<2>(x, n8, c0, f16_scale, lxq, lxs, xsum, nw, nscale, h, tid, nthreads);
+  else if (c0 < n8) stage_q8_passes<1>(x, n8, c0, f16_scale, lxq, lxs, xsum, nw, nscale, h, tid, nthreads);
 }
 
 // ---- rmsnorm!'s scale (model.lisp:205-214) ----------------------------------------------------
@@ -1033,20 +1036,35 @@ __global__ __launch_bounds__(kStreamThreads) void gemv_stream_kernel(IltGemvPara
 
   // 1. the activations into LDS, by the first four waves
   if (wave < kStagers && q8) {
-    if (p.xf) stage_q8_from_f32(p.xf, S, p.f16_scale, lxq, lxs);       // (its loop strides by the stagers' 256 threads)
-    else {
-      for (int i = threadIdx.x * 16; i < p.cols; i += 64 * kStagers * 16) *(int4*)(lxq + i) = *(const int4*)(p.xq + i);
-      for (int i = threadIdx.x; i < S; i += 64 * kStagers) lxs[i] = p.xs[i];
+    // A token's routing carried along (IltRouteAlong): the first workgroup's first wave does not stage -- its other
+    // three activation waves take its share -- but reads its logits at once, ahead of the row waves' loads (behind
+    // them they would come in when the whole matrix has), and routes when the barrier is behind it.
+    bool routing = false;
+    float r_lg[4] = {0.f, 0.f, 0.f, 0.f}, r_bs[4] = {0.f, 0.f, 0.f, 0.f};
+    if constexpr (!EARLY) routing = p.route.logits && blockIdx.x == 0;
+    if (routing && wave == 0) {
+#pragma unroll
+      for (int k = 0; k < 4; k++) {
+        const int e = k * 64 + lane;
+        if (e < p.route.ne) { r_lg[k] = p.route.logits[e]; if (p.route.bias) r_bs[k] = p.route.bias[e]; }
+      }
+    } else if (p.xf) {
+      if (routing) stage_q8_from_f32(p.xf, S, p.f16_scale, lxq, lxs, nullptr, nullptr, 1.0f, nullptr, (int)threadIdx.x - 64, 64 * (kStagers - 1));
+      else stage_q8_from_f32(p.xf, S, p.f16_scale, lxq, lxs);
+    } else {
+      const int tid = routing ? (int)threadIdx.x - 64 : (int)threadIdx.x, nt = routing ? 64 * (kStagers - 1) : 64 * kStagers;
+      for (int i = tid * 16; i < p.cols; i += nt * 16) *(int4*)(lxq + i) = *(const int4*)(p.xq + i);
+      for (int i = tid; i < S; i += nt) lxs[i] = p.xs[i];
     }
     ilt_barrier_lds();
     if (p.ahead.a) cache_ahead(p.ahead, p.mat[0].y);
     if (p.rows_ahead.nm) rows_ahead(p.rows_ahead, p.mat[0].y);
-    if constexpr (q8 && !EARLY) {
-      // a token's routing carried along: this wave has nothing left to do while the rows stream in
-      if (p.route.logits && blockIdx.x == 0 && wave == 0) {
+    if constexpr (!EARLY) {
+      if (routing && wave == 0) {
         __shared__ u32 r_idx[64];
         __shared__ float r_sc[64];
-        route_token<4>(lane, p.route.ne, p.route.nu, p.route.scale, p.route.logits, p.route.bias, nullptr, p.route.sel, p.route.wout, r_idx, r_sc);
+        route_token<4, true>(lane, p.route.ne, p.route.nu, p.route.scale, p.route.logits, p.route.bias, nullptr, p.route.sel, p.route.wout, r_idx,
+                             r_sc, r_lg, r_bs);
       }
     }
     return;
