@@ -428,11 +428,11 @@ __device__ __forceinline__ void load_q8k_pass_clamped(const float* __restrict__ 
 // quants to the next's at LXQ.
 // One pass: this wave's four blocks 4*wave + 4*NW*pass + (0..3).  PRE: the pass's values, loaded by
 // the caller ahead of time (load_q8k_pass), or null to load them here; NPRE likewise for nw.
-template <int PITCH, int NW>
-__device__ __forceinline__ void q8k_pass(const float* __restrict__ x, int nblk, int pass, const float4* pre, i8* lxq, float* lxs, int* lbs,
-                                         const float* __restrict__ nw, const float4* npre, float nscale, float* __restrict__ h) {
+template <int PITCH, int NW, bool SEARCH>
+__device__ __forceinline__ bool q8k_pass_impl(const float* __restrict__ x, int nblk, int pass, const float4* pre, i8* lxq, float* lxs, int* lbs,
+                                              const float* __restrict__ nw, const float4* npre, float nscale, float* __restrict__ h) {
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), g = lane >> 4, l = lane & 15;
-  if (4 * wave + 4 * NW * pass >= nblk) return;        // none of this wave's four blocks exists
+  if (4 * wave + 4 * NW * pass >= nblk) return false;  // none of this wave's four blocks exists
   const int b = 4 * wave + 4 * NW * pass + g;
   const bool live = b < nblk;
   float4 t4[4];
@@ -451,28 +451,53 @@ __device__ __forceinline__ void q8k_pass(const float* __restrict__ x, int nblk, 
   float v[16];
 #pragma unroll
   for (int i = 0; i < 4; i++) { v[4 * i] = t4[i].x; v[4 * i + 1] = t4[i].y; v[4 * i + 2] = t4[i].z; v[4 * i + 3] = t4[i].w; }
-  float a8[8];
+  // The block's scale comes from its first value of the largest magnitude, sign and all (quantize-q8k!).  The largest
+  // and the smallest value tell which it is unless they are equal in magnitude; the pass is then made again with
+  // SEARCH set, which looks for the first position (three instructions a value: a quarter of the pass, for one
+  // block in very many).  Without SEARCH there is no branch in here, so that a wave's passes interleave.
+  float amax, mx;
+  bool tie = false;
+  if constexpr (SEARCH) {
+    float sa, sm;
+    {
+      float a8[8];
 #pragma unroll
-  for (int k = 0; k < 8; k++) a8[k] = fmaxf(fabsf(v[2 * k]), fabsf(v[2 * k + 1]));
-  const float am = fmaxf(fmaxf(fmaxf(a8[0], a8[1]), fmaxf(a8[2], a8[3])), fmaxf(fmaxf(a8[4], a8[5]), fmaxf(a8[6], a8[7])));
-  const float amax = ilt_max16(am);
-  // this lane's first position holding the maximum (its values are in rising position order), and the value there
-  int idx = 1 << 20;
-  float val = 0.0f;
+      for (int k = 0; k < 8; k++) a8[k] = fmaxf(fabsf(v[2 * k]), fabsf(v[2 * k + 1]));
+      const float am = fmaxf(fmaxf(fmaxf(a8[0], a8[1]), fmaxf(a8[2], a8[3])), fmaxf(fmaxf(a8[4], a8[5]), fmaxf(a8[6], a8[7])));
+      const float amax_s = ilt_max16(am);
+      // this lane's first position holding the maximum (its values are in rising position order), and the value there
+      int idx = 1 << 20;
+      float val = 0.0f;
 #pragma unroll
-  for (int k = 15; k >= 0; k--) {
-    const bool hit = fabsf(v[k]) == amax;
-    idx = hit ? 4 * (l + 16 * (k >> 2)) + (k & 3) : idx;
-    val = hit ? v[k] : val;
+      for (int k = 15; k >= 0; k--) {
+        const bool hit = fabsf(v[k]) == amax_s;
+        idx = hit ? 4 * (l + 16 * (k >> 2)) + (k & 3) : idx;
+        val = hit ? v[k] : val;
+      }
+      const int firstpos = ilt_min16(idx);
+      const float mx_s = __int_as_float(ilt_or16(idx == firstpos ? __float_as_int(val) : 0));
+      sa = amax_s; sm = mx_s;
+    }
+    amax = sa; mx = sm;
+  } else {
+    float hi = fmaxf(fmaxf(fmaxf(v[0], v[1]), fmaxf(v[2], v[3])), fmaxf(fmaxf(v[4], v[5]), fmaxf(v[6], v[7])));
+    hi = fmaxf(hi, fmaxf(fmaxf(fmaxf(v[8], v[9]), fmaxf(v[10], v[11])), fmaxf(fmaxf(v[12], v[13]), fmaxf(v[14], v[15]))));
+    float lo = fminf(fminf(fminf(v[0], v[1]), fminf(v[2], v[3])), fminf(fminf(v[4], v[5]), fminf(v[6], v[7])));
+    lo = fminf(lo, fminf(fminf(fminf(v[8], v[9]), fminf(v[10], v[11])), fminf(fminf(v[12], v[13]), fminf(v[14], v[15]))));
+    hi = ilt_max16(hi);
+    lo = -ilt_max16(-lo);
+    amax = fmaxf(hi, -lo);
+    mx = hi >= -lo ? hi : lo;
+    if (amax != amax) mx = 0.0f;        // nothing but NaNs: no value is the largest (the CPU's comparisons all fail), the scale is 1 / (-127 / 0)
+    tie = hi == -lo && amax != 0.0f;
   }
-  const int firstpos = ilt_min16(idx);
-  const float mx = __int_as_float(ilt_or16(idx == firstpos ? __float_as_int(val) : 0));
   const bool nz = amax != 0.0f;
   const float iscale = nz ? -127.0f / mx : 0.0f;
   const float d = nz ? 1.0f / iscale : 0.0f;
   int q[16];
+  // (quantize-q8k!'s (min 127 ..) never takes effect: |iscale * v| <= 127 (1 + 2^-23), which rounds to 127)
 #pragma unroll
-  for (int k = 0; k < 16; k++) q[k] = nz ? min(127, (int)rintf(iscale * v[k])) : 0;
+  for (int k = 0; k < 16; k++) q[k] = nz ? (int)rintf(iscale * v[k]) : 0;
 #pragma unroll
   for (int i = 0; i < 4; i++) {
     const int s = ilt_sum4(q[4 * i] + q[4 * i + 1] + q[4 * i + 2] + q[4 * i + 3]);
@@ -483,6 +508,14 @@ __device__ __forceinline__ void q8k_pass(const float* __restrict__ x, int nblk, 
     }
   }
   if (live && l == 0) lxs[b] = d;
+  return tie;
+}
+// A pass, and where a block's largest magnitude comes with both signs (the lanes of that block only) once more.
+template <int PITCH, int NW>
+__device__ __forceinline__ void q8k_pass(const float* __restrict__ x, int nblk, int pass, const float4* pre, i8* lxq, float* lxs, int* lbs,
+                                         const float* __restrict__ nw, const float4* npre, float nscale, float* __restrict__ h) {
+  if (q8k_pass_impl<PITCH, NW, false>(x, nblk, pass, pre, lxq, lxs, lbs, nw, npre, nscale, h))
+    q8k_pass_impl<PITCH, NW, true>(x, nblk, pass, pre, lxq, lxs, lbs, nw, npre, nscale, h);
 }
 
 // All passes; FIRST / NFIRST: the first pass's values (x's, the norm weights'), loaded by the caller.
@@ -1095,9 +1128,12 @@ __global__ __launch_bounds__(kStreamThreads) void gemv_stream_kernel(IltGemvPara
       load_q8k_pass_clamped<kStagers>(p.xf, SX, 0, x0);
       load_q8k_pass_clamped<kStagers>(p.xf, SX, 1, x1);
       load_q8k_pass_clamped<kStagers>(p.xf, SX, 2, x2);
-      q8k_pass<XP, kStagers>(p.xf, SX, 0, x0, lxq, lxs, sbs, nullptr, nullptr, 1.0f, nullptr);
-      q8k_pass<XP, kStagers>(p.xf, SX, 1, x1, lxq, lxs, sbs, nullptr, nullptr, 1.0f, nullptr);
-      q8k_pass<XP, kStagers>(p.xf, SX, 2, x2, lxq, lxs, sbs, nullptr, nullptr, 1.0f, nullptr);
+      const bool t0 = q8k_pass_impl<XP, kStagers, false>(p.xf, SX, 0, x0, lxq, lxs, sbs, nullptr, nullptr, 1.0f, nullptr);
+      const bool t1 = q8k_pass_impl<XP, kStagers, false>(p.xf, SX, 1, x1, lxq, lxs, sbs, nullptr, nullptr, 1.0f, nullptr);
+      const bool t2 = q8k_pass_impl<XP, kStagers, false>(p.xf, SX, 2, x2, lxq, lxs, sbs, nullptr, nullptr, 1.0f, nullptr);
+      if (t0) q8k_pass_impl<XP, kStagers, true>(p.xf, SX, 0, x0, lxq, lxs, sbs, nullptr, nullptr, 1.0f, nullptr);
+      if (t1) q8k_pass_impl<XP, kStagers, true>(p.xf, SX, 1, x1, lxq, lxs, sbs, nullptr, nullptr, 1.0f, nullptr);
+      if (t2) q8k_pass_impl<XP, kStagers, true>(p.xf, SX, 2, x2, lxq, lxs, sbs, nullptr, nullptr, 1.0f, nullptr);
       for (int pass = 3; pass * 4 * kStagers < SX; pass++)
         q8k_pass<XP, kStagers>(p.xf, SX, pass, nullptr, lxq, lxs, sbs, nullptr, nullptr, 1.0f, nullptr);
     } else if (p.xf) {

@@ -30,6 +30,10 @@ def special_activations(cols, rng):
         x[256:512] = 0.0               # a zero Q8_K block
     x[40] = -7.5                       # block maximum on a negative value
     x[70] = 3.25; x[90] = -3.25        # equal magnitudes: the first wins
+    if cols >= 1280:                   # a Q8_K block's largest magnitude with both signs: the first one's sign is the scale's
+        x[512 + 5] = 9.0; x[512 + 200] = -9.0
+        x[768 + 3] = -8.0; x[768 + 100] = 8.0; x[768 + 101] = 8.0
+        x[1024 + 255] = -6.5; x[1024 + 254] = 6.5; x[1024 + 17] = 6.5
     return x
 
 
