@@ -1164,8 +1164,10 @@ __global__ __launch_bounds__(kStreamThreads) void gemv_stream_kernel(IltGemvPara
   const u16* const u_wd = p.mat[1].wd;
   const long long u_row_bytes = p.mat[1].row_bytes, u_add = p.mat[1].add;
   const int u_fmt = p.mat[1].fmt;
+  IltGemvMat m = p.mat[0];          // (the first matrix with them: the only one of most launches, no second go for those)
   asm volatile("" ::"s"(a_nbatches), "s"(a_nmat), "s"(a_glu), "s"(a_batch), "s"(a_region), "s"(a_cols), "s"(b1), "s"(b2), "s"(b3), "s"(a_ptrs),
-               "s"(a_sel), "s"(u_w), "s"(u_wd), "s"(u_row_bytes), "s"(u_add), "s"(u_fmt));
+               "s"(a_sel), "s"(u_w), "s"(u_wd), "s"(u_row_bytes), "s"(u_add), "s"(u_fmt), "s"(m.w), "s"(m.wd), "s"(m.y), "s"(m.bias),
+               "s"(m.row_bytes), "s"(m.add), "s"(m.rows), "s"(m.fmt), "s"(m.batch0), "s"(m.nbat), "s"(m.rq), "s"(m.rr));
   float* tw = terms + (long)rw * a_batch * tpr * nglu;
   u8* region = (u8*)(terms + (long)kRowWaves * a_batch * tpr * nglu) + (long)rw * a_region;
 
@@ -1174,9 +1176,11 @@ __global__ __launch_bounds__(kStreamThreads) void gemv_stream_kernel(IltGemvPara
   const bool live = wid < a_nbatches;
   // (the matrices' first batches rise: the matrix of batch wid is the last one that starts at or before it)
   if (!a_ptrs && !a_glu) mi = (a_nmat > 1 && wid >= b1 ? 1 : 0) + (a_nmat > 2 && wid >= b2 ? 1 : 0) + (a_nmat > 3 && wid >= b3 ? 1 : 0);
-  const IltGemvMat m = p.mat[mi];
-  asm volatile("" ::"s"(m.w), "s"(m.wd), "s"(m.y), "s"(m.bias), "s"(m.row_bytes), "s"(m.add), "s"(m.rows), "s"(m.fmt), "s"(m.batch0),
-               "s"(m.nbat), "s"(m.rq), "s"(m.rr));
+  if (mi != 0) {
+    m = p.mat[mi];
+    asm volatile("" ::"s"(m.w), "s"(m.wd), "s"(m.y), "s"(m.bias), "s"(m.row_bytes), "s"(m.add), "s"(m.rows), "s"(m.fmt), "s"(m.batch0),
+                 "s"(m.nbat), "s"(m.rq), "s"(m.rr));
+  }
   int bl = wid;
   if (live) {
     if (a_ptrs) { z = wid / m.nbat; bl = wid - z * m.nbat; }
