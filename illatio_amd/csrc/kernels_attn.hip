@@ -564,15 +564,26 @@ __global__ __launch_bounds__(256) void attn_values_kernel(const float* __restric
 // come from L2 once for each of its hd/CS workgroups, which is what bounds the context), scales them, and adds its
 // CS columns as attn_values_kernel<1> does.  The group's first query head's first workgroup writes the key and the
 // value into the caches; the token's own key and value are taken from k and v, never from the caches.  NJ = hd/16.
+// RAW set: the head's scores are shared out over its hd / CS workgroups -- each takes the passes of 64 positions
+// numbered its slice, its slice + hd / CS, .. and writes their scores to RAW (nh rows of smax floats), raises its flag,
+// waits for the others' and reads the whole row -- instead of each taking all of them (the keys of
+// 640 positions are 330 KB a workgroup, read by every one of the head's eight).  The launcher asks for this where
+// the head's workgroups run on one die: the exchange then goes through that die's L2 (1.2 us; through memory, with
+// device-scope stores, the scores alone took 3 us to write), and a workgroup reads the row only if the counter says
+// that all of them did run on its die.  One that finds them spread over dies, or has waited PATIENCE ticks of the
+// 100 MHz clock (its partners are not resident), takes all the scores itself, as without RAW.  The flags carry the head's generation, which the head's first workgroup advances as it
+// ends: nothing for the host to reset or to count, and a launch replayed from a graph works as the first one did.
+__device__ unsigned attn_gen[256], attn_flag[256 * 8];
 template <int NJ, int CS>
 __global__ __launch_bounds__(1024) void attn_step_fused_kernel(const float* __restrict__ q, const float* __restrict__ k, const float* __restrict__ v,
                                                                const float* __restrict__ qn, const float* __restrict__ kn,
                                                                const float* __restrict__ rope, float* __restrict__ kc, float* __restrict__ vc,
                                                                float* __restrict__ out, int nh, int nkv, int rd, int pos, float eps, int neox,
-                                                               float scale, int vpitch) {
+                                                               float scale, int vpitch, float* __restrict__ raw, int smax, int patience) {
   extern __shared__ __align__(16) float dyn[];
   __shared__ float qsh[16 * NJ], ksh[16 * NJ], redf[16];
   __shared__ double scs[2], redd[17];
+  __shared__ int got_all;
   constexpr int hd = 16 * NJ;
   // the hardware deals consecutive workgroups to the eight dies in turn: die x takes the workgroups of consecutive heads
   // (with 32 query heads on 8 KV heads, one KV head's), so a head's keys and values come from memory into one L2 only
@@ -596,22 +607,38 @@ __global__ __launch_bounds__(1024) void attn_step_fused_kernel(const float* __re
   RopeIn<(NJ + 3) / 4> rin;
   if (wave < 2) rope_head_load(rin, wave == 0 ? q + h * hd : k + ko, wave == 0 ? qn : kn, cst, hd, rd, lane);
   float ka[4][NJ], kb[4][NJ];
-  load_keys(ka, 0);
+  constexpr int NPASS = 16 / (hd / CS);            // passes of 64 positions a workgroup takes of a head's shared-out scores
+  float kx[NPASS][NJ];
+  const bool split = raw != nullptr;
+  // (the head's generation: the number its workgroups will write into their flags; read now, wanted after the scores)
+  unsigned gen = 0;
+  if (split && tid < ns) gen = __hip_atomic_load(&attn_gen[h], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + 1;
+  if (split) {
+#pragma unroll
+    for (int i = 0; i < NPASS; i++) {
+      const float* kr = kc + (long long)min(64 * (cs + ns * i) + pg, last) * kvd + ko;
+#pragma unroll
+      for (int j = 0; j < NJ; j++) kx[i][j] = kr[l + 16 * j];
+    }
+  } else load_keys(ka, 0);
   // (the rest of the loads after the heads are turned: sixteen waves' loads take as long to ask for as the turn takes,
   // and the workgroup would wait for the slowest wave's)
   if (wave < 2) rope_head_turn(rin, (wave == 0 ? qn : kn) != nullptr, wave == 0 ? qsh : ksh, &scs[wave], hd, rd, eps, neox, lane);
   __syncthreads();
-  load_keys(kb, 1);
+  if (!split) load_keys(kb, 1);
   // the slice: 16-byte piece i = position i / PP, part i % PP; the token's own row from v
   constexpr int PP = CS / 4;
   float4 r[PP];
   const int total = npos * PP;
+  auto load_slice = [&]() {
 #pragma unroll
-  for (int u = 0; u < PP; u++) {
-    const int i = min(tid + 1024 * u, total - 1), p = i / PP;
-    const float* src = p == pos ? v + vo : vc + (long long)p * kvd + vo;
-    r[u] = *(const float4*)(src + 4 * (i % PP));
-  }
+    for (int u = 0; u < PP; u++) {
+      const int i = min(tid + 1024 * u, total - 1), p = i / PP;
+      const float* src = p == pos ? v + vo : vc + (long long)p * kvd + vo;
+      r[u] = *(const float4*)(src + 4 * (i % PP));
+    }
+  };
+  if (!split) load_slice();          // (shared-out scores: asked for once the scores are written, whose stores would wait for these loads)
   if (h == kh * group && cs == 0 && tid < hd) {
     kc[(long long)pos * kvd + ko + tid] = ksh[tid];
     vc[(long long)pos * kvd + ko + tid] = v[ko + tid];
@@ -638,20 +665,72 @@ __global__ __launch_bounds__(1024) void attn_step_fused_kernel(const float* __re
     }
   };
   const int nb = (npos + 255) >> 8;                // 1 .. 4
-  take_scores(ka, 0);
-  if (nb > 2) load_keys(ka, 2);
-  if (nb > 1) take_scores(kb, 1);
-  if (nb > 3) load_keys(kb, 3);
-  if (nb > 2) take_scores(ka, 2);
-  if (nb > 3) take_scores(kb, 3);
-  __syncthreads();
+  bool shared = false;
+  if (split) {
+    float* const row = raw + (long long)h * smax;
+#pragma unroll
+    for (int i = 0; i < NPASS; i++) {
+      const int p = 64 * (cs + ns * i) + pg;
+      if (p == pos) {
+#pragma unroll
+        for (int j = 0; j < NJ; j++) kx[i][j] = ksh[l + 16 * j];
+      }
+      float sacc = 0.0f;
+#pragma unroll
+      for (int j = 0; j < NJ; j++) sacc = sacc + kx[i][j] * qv[j];
+      sacc = sacc + ilt_dppf<ILT_DPP_SHL(4)>(sacc);
+      sacc = sacc + ilt_dppf<ILT_DPP_SHL(8)>(sacc);
+      sacc = sacc + ilt_dppf<ILT_DPP_SHL(1)>(sacc);
+      sacc = sacc + ilt_dppf<ILT_DPP_SHL(2)>(sacc);
+      if (l == 0 && p < npos) row[p] = sacc * scale;
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");          // this wave's scores are written
+    ilt_barrier_lds();                                        // ... and every wave's
+    // The scores are plain stores: they are in this die's L2 (the wait above) and no further, so the row may only be
+    // read where every one of the head's workgroups ran on this die.  A workgroup's flag is the head's generation
+    // and its die (HW_REG_XCC_ID); lane j of the first wave waits for workgroup j's.  (A counter the workgroups add
+    // themselves to took 2.5 us to be seen by all: read-modify-writes of device scope are made in memory.)
+    if (tid < ns) {
+      const unsigned die = __builtin_amdgcn_s_getreg((4 - 1) << 11 | 20) & 15u;
+      if (tid == 0) __hip_atomic_store(&attn_flag[h * 8 + cs], gen << 4 | die, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      int ok = 0;
+      const long long t0 = wall_clock64();
+      for (;;) {
+        const unsigned f = __hip_atomic_load(&attn_flag[h * 8 + tid], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (f >> 4 == gen) { ok = (f & 15u) == die; break; }          // there; on this die?
+        if (wall_clock64() - t0 >= (long long)patience) break;        // not resident: alone
+        __builtin_amdgcn_s_sleep(1);
+      }
+      const int all = __builtin_amdgcn_ballot_w64(ok != 0) == (1ull << ns) - 1;
+      if (tid == 0) got_all = all;
+    }
+    ilt_barrier_lds();
+    shared = got_all != 0;
+    // (the row, then the slice: loads come back in the order asked for, and the row is wanted first.  From here to the
+    // products the barriers wait for LDS only -- __syncthreads waits for every load in flight, the slice's too)
+    float mine_raw = 0.0f;
+    if (shared && tid < npos) mine_raw = __builtin_nontemporal_load(row + tid);
+    load_slice();
+    if (shared && tid < npos) sc[tid] = mine_raw;
+    ilt_barrier_lds();                                        // the row is read, its values in LDS (or given up)
+  }
+  if (!shared) {
+    if (split) { load_keys(ka, 0); load_keys(kb, 1); }
+    take_scores(ka, 0);
+    if (nb > 2) load_keys(ka, 2);
+    if (nb > 1) take_scores(kb, 1);
+    if (nb > 3) load_keys(kb, 3);
+    if (nb > 2) take_scores(ka, 2);
+    if (nb > 3) take_scores(kb, 3);
+  }
+  ilt_barrier_lds();
   // softmax (attn_softmax's steps with a position a thread)
   const bool mine = tid < npos;
   float mx = mine ? sc[tid] : -3.402823466e38f;
   const float sv = mx;
   mx = wave_max_float(mx);
   if (lane == 0) redf[wave] = mx;
-  __syncthreads();
+  ilt_barrier_lds();
   mx = redf[0];
 #pragma unroll
   for (int w = 1; w < 16; w++) mx = fmaxf(mx, redf[w]);
@@ -659,7 +738,7 @@ __global__ __launch_bounds__(1024) void attn_step_fused_kernel(const float* __re
   const double part = wave_sum_double((double)e);
   if (lane == 0) redd[wave] = part;
   if (mine) sc[tid] = e;
-  __syncthreads();
+  ilt_barrier_lds();
   double sum = redd[0];
 #pragma unroll
   for (int w = 1; w < 16; w++) sum += redd[w];
@@ -667,11 +746,11 @@ __global__ __launch_bounds__(1024) void attn_step_fused_kernel(const float* __re
   float inv;
   if (!recip_settled(sum, npos, &inv)) {           // the same in every thread
     if (tid == 0) { double s2 = 0.0; for (int p = 0; p < npos; p++) s2 += (double)sc[p]; redd[16] = s2; }
-    __syncthreads();
+    ilt_barrier_lds();
     inv = (float)(1.0 / redd[16]);
   }
   if (mine) sc[tid] = e * inv;
-  __syncthreads();
+  ilt_barrier_lds();
 #pragma unroll
   for (int u = 0; u < PP; u++) {
     const int i = tid + 1024 * u;
@@ -681,11 +760,15 @@ __global__ __launch_bounds__(1024) void attn_step_fused_kernel(const float* __re
       dst[0] = sp * r[u].x; dst[vpitch] = sp * r[u].y; dst[2 * vpitch] = sp * r[u].z; dst[3 * vpitch] = sp * r[u].w;
     }
   }
-  __syncthreads();
+  ilt_barrier_lds();
   if (tid < CS) {
     const float* col = vt + tid * vpitch;
     out[h * hd + CS * cs + tid] = chain_add_row(col, npos, vpitch - 36);
   }
+  // The head's first workgroup advances the generation as it ends: every workgroup of this launch read it as it
+  // started, many microseconds ago (one that starts only now finds the new one, matches no flag and takes all the scores
+  // itself).  A store: a counter of readers would be a read-modify-write whose answer a workgroup waits 2 us for.
+  if (split && tid == 0 && cs == 0) __hip_atomic_store(&attn_gen[h], gen & 0x0FFFFFFFu, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 // The same for contexts whose value slice no longer fits LDS (2,049 to 8,192 positions): the slice comes through
@@ -940,12 +1023,20 @@ hipError_t ilt_k_attn_step(const float* q, const float* k, const float* v, const
       set[dev] = true;
     }
     const size_t fsmem = sizeof(float) * (1024 + 16 * (size_t)vpitch);
+    // A head's scores shared out over its workgroups where those run on one die: consecutive workgroups go to the
+    // eight dies in turn and the kernel renumbers them so that a die takes nwg / 8 consecutive (head, slice) pairs.
+    // "ILT_ATTN_SPLIT=0": never; "=2": every workgroup gives up waiting at once and takes all the scores (tests).
+    const int ns = hd / 16, nwg = nh * ns;
+    const char* sp = getenv("ILT_ATTN_SPLIT");
+    const bool split = !(sp && sp[0] == '0') && (nwg & 7) == 0 && ((nwg >> 3) % ns) == 0 && nh <= 256 && ctx >= 64;
+    float* const raw = split ? scratch : nullptr;
+    const int patience = sp && sp[0] == '2' ? 0 : 20000;       // 200 us
     if (hd == 64)
-      hipLaunchKernelGGL((attn_step_fused_kernel<4, 16>), dim3(nh * 4), dim3(1024), fsmem, st, q, k, v, qn, kn, rope, kc, vc, out, nh, nkv, rd, pos, eps,
-                         neox, scale, vpitch);
+      hipLaunchKernelGGL((attn_step_fused_kernel<4, 16>), dim3(nwg), dim3(1024), fsmem, st, q, k, v, qn, kn, rope, kc, vc, out, nh, nkv, rd, pos, eps,
+                         neox, scale, vpitch, raw, smax, patience);
     else
-      hipLaunchKernelGGL((attn_step_fused_kernel<8, 16>), dim3(nh * 8), dim3(1024), fsmem, st, q, k, v, qn, kn, rope, kc, vc, out, nh, nkv, rd, pos, eps,
-                         neox, scale, vpitch);
+      hipLaunchKernelGGL((attn_step_fused_kernel<8, 16>), dim3(nwg), dim3(1024), fsmem, st, q, k, v, qn, kn, rope, kc, vc, out, nh, nkv, rd, pos, eps,
+                         neox, scale, vpitch, raw, smax, patience);
     return hipGetLastError();
   }
   hipLaunchKernelGGL(attn_step_scores_kernel, dim3(nh, (ctx + 255) / 256), dim3(1024), 0, st, q, k, v, qn, kn, rope, kc, vc, scratch, nh, nkv, hd, rd,
