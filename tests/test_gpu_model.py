@@ -258,6 +258,23 @@ def test_one_launch_attention_up_to_1024_positions(dev):
             assert same == ndecode
 
 
+def test_one_launch_attention_scores_shared_out(dev, monkeypatch):
+    """The one-launch attention with a head's scores shared out over its workgroups (eight query heads: a head's
+    workgroups then run on one die and exchange their scores inside the launch), in each block of 256 positions; the same
+    with every workgroup giving up the wait at once and taking all the scores itself, and with the sharing switched off."""
+    from illatio_amd import model
+    for seed, hd, nkv in ((41, 64, 2), (42, 128, 4)):
+        host = model.synth_model(seed, d=256, ffn=512, nh=8, nkv=nkv, hd=hd, nl=2, vocab=500)
+        for mode in (None, "2", "0"):
+            if mode is None:
+                monkeypatch.delenv("ILT_ATTN_SPLIT", raising=False)
+            else:
+                monkeypatch.setenv("ILT_ATTN_SPLIT", mode)
+            for nprompt, ndecode in ((70, 6), (250, 10), (764, 6), (1018, 8)) if mode is None else ((250, 10), (1018, 8)):
+                same, _ = run_greedy(dev, host, nprompt=nprompt, ndecode=ndecode, chunk=512, nctx=nprompt + ndecode + 2, seed=seed + nprompt)
+                assert same == ndecode, (hd, mode, nprompt)
+
+
 def test_config_2_width_four_layers_128_greedy_tokens(dev):
     """Config 2's layer at its full width (hidden 2560, intermediate 9728, 32 query and 8 KV heads of 128, vocabulary
     151936), four layers: a 64-token prompt through the prefill products, then 128 greedy tokens, each step's logits
