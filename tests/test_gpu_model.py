@@ -110,6 +110,56 @@ def test_attn_step_is_qk_rope_then_attn_rows(dev, norms, nh, nkv, hd):
         hip.hip_free(b)
 
 
+def test_attn_step_replayed_from_a_graph(dev):
+    """The one-launch attention with the scores shared out keeps its flags' generation on the device: a launch captured
+    into a HIP graph and replayed (new q, k, v each time, the program's own copies and waits between the replays) gives
+    what the three launches it stands for give, every time."""
+    import ctypes as C
+    from illatio_amd import hip
+    rt = C.CDLL("libamdhip64.so")
+    nh, nkv, hd, nctx, pos, eps = 8, 2, 64, 400, 300, 1e-6
+    rng = synth.make_rng(12)
+    f = lambda *sh: (rng.standard_normal(sh) * 1.5).astype(np.float32)
+    up = lambda a: (lambda b: (hip.hip_upload_vector(b, a), b)[1])(hip.hip_alloc(dev, a.nbytes))
+    P = lambda b: C.c_uint64(b.ptr if b is not None else 0)
+    table = np.zeros((nctx, hd), np.float32)
+    assert hip.lib().ilt_rope_table(C.c_int(hd), C.c_int(0), C.c_int(nctx), C.c_float(1e6), table.ctypes.data_as(C.c_void_p)) == 0
+    rope, qn, kn = up(table), up(f(hd)), up(f(hd))
+    kc0, vc0 = f(nctx, nkv * hd), f(nctx, nkv * hd)
+    scratch = hip.hip_alloc(dev, 4 * nh * nctx)
+    q, k, v = f(nh * hd), f(nkv * hd), f(nkv * hd)
+    dq, dk, dv, kc, vc, out = up(q), up(k), up(v), up(kc0), up(vc0), hip.hip_alloc(dev, 4 * nh * hd)
+    ints = (C.c_int(nh), C.c_int(nkv), C.c_int(hd), C.c_int(hd), C.c_int(pos), C.c_float(eps), C.c_int(1))
+    S = C.c_uint64(dev.stream)
+    step = lambda: hip.call("ilt_attn_step", S, P(dq), P(dk), P(dv), P(qn), P(kn), P(rope), P(kc), P(vc), P(out), *ints, P(scratch))
+    step()                                             # once outside the graph: the kernel's attributes are set on its first launch
+    hip.hip_sync(dev)
+    graph, gexec = C.c_void_p(), C.c_void_p()
+    assert rt.hipStreamBeginCapture(C.c_void_p(dev.stream), C.c_int(0)) == 0
+    step()
+    assert rt.hipStreamEndCapture(C.c_void_p(dev.stream), C.byref(graph)) == 0
+    assert rt.hipGraphInstantiate(C.byref(gexec), graph, None, None, C.c_size_t(0)) == 0
+    for rep in range(4):
+        q, k, v = f(nh * hd), f(nkv * hd), f(nkv * hd)
+        for b, a in ((dq, q), (dk, k), (dv, v), (kc, kc0), (vc, vc0)):
+            hip.hip_upload_vector(b, a)
+        hip.hip_sync(dev)
+        assert rt.hipGraphLaunch(gexec, C.c_void_p(dev.stream)) == 0
+        hip.hip_sync(dev)
+        got = [hip.hip_floats(b, n) for b, n in ((out, nh * hd), (kc, nctx * nkv * hd))]
+        eq, ek, ev, ekc, evc, eout = up(q), up(k), up(v), up(kc0), up(vc0), hip.hip_alloc(dev, 4 * nh * hd)
+        hip.call("ilt_qk_rope", S, P(eq), P(ek), P(ev), P(qn), P(kn), P(rope), P(ekc), P(evc), *ints, C.c_int(1))
+        hip.call("ilt_attn_rows", S, P(eq), P(ekc), P(evc), P(eout), C.c_int(nh), C.c_int(nkv), C.c_int(hd), C.c_int(pos), C.c_int(1), P(None))
+        want = [hip.hip_floats(b, n) for b, n in ((eout, nh * hd), (ekc, nctx * nkv * hd))]
+        for a, b, what in zip(got, want, ("out", "kc")):
+            assert np.array_equal(bits(a), bits(b)), (rep, what)
+        for b in (eq, ek, ev, ekc, evc, eout):
+            hip.hip_free(b)
+    assert rt.hipGraphExecDestroy(gexec) == 0 and rt.hipGraphDestroy(graph) == 0
+    for b in (rope, qn, kn, scratch, dq, dk, dv, kc, vc, out):
+        hip.hip_free(b)
+
+
 def test_argmax_on_the_device(dev):
     """ilt_argmax against ARGMAX's scan (model.lisp:464-468): the first of equal maxima, -0 and +0 equal, a NaN never
     greater, a NaN in front staying the best, nothing but -inf or NaN leaving index 0; lengths that are and are not
