@@ -949,26 +949,40 @@ __device__ __forceinline__ void wave_rows_lds(const u8* run, const u8* run2, int
 constexpr int kStreamWaves = 16, kStreamThreads = 64 * kStreamWaves, kStagers = 4, kRowWaves = kStreamWaves - kStagers;
 
 // rmsnorm!'s scale (see norm_scale) in the streamed kernel: the first kStagers waves hold the
-// squares, the other waves only keep step through the three barriers (always three, whether
-// or not the sum is taken again in the CPU's order, so that they need not know).
-__device__ __forceinline__ float norm_scale_stagers(double part, const float* __restrict__ x, int n, float eps, int seq) {
+// squares; the other waves have no part in it.
+// The four activation waves meet three times on the way (partial sums written; read by all before one of them is
+// written again; the sum added again where that was needed).  They meet through counters in LDS, cleared at the
+// kernel's start: s_barrier would have to be reached by the row waves too, and those are held up while they send off
+// their loads (the memory pipeline takes a wave's loads at the rate the rows arrive: the last row wave of a 28 MB
+// launch reaches a barrier 4 us into the launch).  meet: this wave's LDS writes are done, it counts itself, and waits
+// until all four have; nothing that is waited for waits for anything itself, the polls are bounded all the same.
+__device__ __forceinline__ void stagers_meet(u32* slot) {
+  asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+  if ((threadIdx.x & 63) == 0) __hip_atomic_fetch_add(slot, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+  for (int polls = 0; polls < (1 << 22); polls++) {
+    if (__hip_atomic_load(slot, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) >= (u32)kStagers) break;
+    __builtin_amdgcn_s_sleep(1);
+  }
+  asm volatile("" ::: "memory");
+}
+__device__ __forceinline__ float norm_scale_stagers(double part, const float* __restrict__ x, int n, float eps, int seq, u32* meet) {
   __shared__ double red[kStagers];
   part = wave_sum_double(part);
   if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = part;
-  ilt_barrier_lds();
+  stagers_meet(meet);
   double sum = red[0];
 #pragma unroll
   for (int w = 1; w < kStagers; w++) sum += red[w];
   double v = sum / (double)n + (double)eps;
   const double slack = v * ((double)(n + 8) * 0x1p-51);
   const bool again = seq || (float)(v - slack) != (float)(v + slack);       // the same for every thread
-  ilt_barrier_lds();
+  stagers_meet(meet + 1);
   if (again && threadIdx.x == 0) {
     double s = 0.0;
     for (int i = 0; i < n; i++) { const float xi = x[i]; s += (double)(xi * xi); }
     red[0] = s;
   }
-  ilt_barrier_lds();
+  stagers_meet(meet + 2);
   if (again) v = red[0] / (double)n + (double)eps;
   return 1.0f / sqrtf((float)v);
 }
@@ -1054,6 +1068,12 @@ template <int FSET, int EARLY = 0>
 __global__ __launch_bounds__(kStreamThreads) void gemv_stream_kernel(IltGemvParams p) {
   static_assert(offsetof(IltGemvParams, route) <= 456 && sizeof(IltGemvParams) >= 448, "ilt_kernarg_warm7 covers the arguments' first 448 bytes");
   ilt_kernarg_warm7();
+  __shared__ u32 s_meet[4];            // the norm's three meetings of the activation waves (stagers_meet)
+  asm volatile("" ::"s"(p.norm_w), "s"(p.cols), "s"(p.x_stride), "s"(p.nz));      // (read together with what every wave reads first anyway)
+  if (p.norm_w) {                      // (the workgroup's waves start within a few cycles of one another: this barrier is cheap)
+    if (threadIdx.x < 4) s_meet[threadIdx.x] = 0;
+    ilt_barrier_lds();
+  }
   extern __shared__ __align__(16) unsigned char smem[];
   constexpr bool iq2 = FSET == ILT_IQ2_XXS, q8 = FSET == ILT_Q8_0;
   const int S = q8 ? p.cols / 32 : p.cols / 256;
@@ -1119,7 +1139,7 @@ __global__ __launch_bounds__(kStreamThreads) void gemv_stream_kernel(IltGemvPara
         sq += (sq4(t[0]) + sq4(t[1])) + (sq4(t[2]) + sq4(t[3]));
       }
       sq += (sq4(xall[0]) + sq4(xall[1])) + (sq4(xall[2]) + sq4(xall[3]));
-      const float nscale = norm_scale_stagers(sq, p.xf, p.cols, p.eps, p.norm_seq);
+      const float nscale = norm_scale_stagers(sq, p.xf, p.cols, p.eps, p.norm_seq, s_meet);
       stage_q8k_from_f32<XP, kStagers>(p.xf, S, lxq, lxs, sbs, xall, p.norm_w, nall, nscale);
     } else if (p.xf && SX > 4 * kStagers) {
       // up to three passes (12288 activations): all their loads first, then the three passes' chains
@@ -1220,7 +1240,6 @@ __global__ __launch_bounds__(kStreamThreads) void gemv_stream_kernel(IltGemvPara
   }
   // (no branch around the loads, which the compiler would wait out at the join: a launch that has neither runs the
   // kernel built without them; one that has only one of them reads y twice)
-  if (p.norm_w) { ilt_barrier_lds(); ilt_barrier_lds(); ilt_barrier_lds(); }      // in step with norm_scale_stagers
   // The barrier is for the activations only, so it comes before this wave waits for its rows (no
   // fence: the loads stay in flight): a wave whose rows land early starts on them while the
   // other waves' rows are still streaming in.
