@@ -6,6 +6,7 @@
 // not the point of these kernels (the reference's CUDA attention splits the keys and lets the
 // partial sums meet in its own order, dense.cu:364-373).
 #include "ilt_device.h"
+#include <atomic>
 #include "ilt_kernels.h"
 #include <stdlib.h>
 
@@ -564,26 +565,32 @@ __global__ __launch_bounds__(256) void attn_values_kernel(const float* __restric
 // come from L2 once for each of its hd/CS workgroups, which is what bounds the context), scales them, and adds its
 // CS columns as attn_values_kernel<1> does.  The group's first query head's first workgroup writes the key and the
 // value into the caches; the token's own key and value are taken from k and v, never from the caches.  NJ = hd/16.
-// RAW set: the head's scores are shared out over its hd / CS workgroups -- each takes the passes of 64 positions
-// numbered its slice, its slice + hd / CS, .. and writes their scores to RAW (nh rows of smax floats), raises its flag,
-// waits for the others' and reads the whole row -- instead of each taking all of them (the keys of
-// 640 positions are 330 KB a workgroup, read by every one of the head's eight).  The launcher asks for this where
-// the head's workgroups run on one die: the exchange then goes through that die's L2 (1.2 us; through memory, with
-// device-scope stores, the scores alone took 3 us to write), and a workgroup reads the row only if the counter says
-// that all of them did run on its die.  One that finds them spread over dies, or has waited PATIENCE ticks of the
-// 100 MHz clock (its partners are not resident), takes all the scores itself, as without RAW.  The flags carry the head's generation, which the head's first workgroup advances as it
-// ends: nothing for the host to reset or to count, and a launch replayed from a graph works as the first one did.
-__device__ unsigned attn_gen[256], attn_flag[256 * 8];
+// SHARE set: the head's scores are shared out over its hd / CS workgroups -- each takes the passes of 64 positions
+// numbered its slice, its slice + hd / CS, .. (at most two) -- instead of each taking all of them (the keys of 640
+// positions are 330 KB a workgroup, read by every one of the head's eight).  A score travels as eight bytes, its bits
+// and a tag (the head's generation on the device, the host's count of launches, the writer's die), written with one
+// plain store into attn_xrow, a buffer of the library's; the thread that wants position p reads that word until it
+// carries this launch's tag.  A plain store is seen in its die's L2 and no further within a launch, so the tag's die
+// must be the reader's own (HW_REG_XCC_ID): the launcher asks for SHARE where a head's workgroups run on one die, and
+// where the hardware puts them elsewhere -- or a partner is not resident and nothing arrives within PATIENCE ticks of
+// the 100 MHz clock -- the workgroup takes all the scores itself, as without SHARE.  The head's first workgroup
+// advances the generation as it ends (every workgroup read it as it started, microseconds earlier), so a launch
+// replayed from a graph finds new tags; the host's count tells apart launches that overlap on one GPU, which make each
+// other give up (they share the buffer) but do not read each other's scores.  (24 bits of generation: a word left in
+// the buffer could pass for a fresh one only if it was written exactly 2^24 launches of its head earlier.)
+__device__ unsigned attn_gen[256];
+__device__ unsigned long long attn_xrow[256 * 1024];
 template <int NJ, int CS>
 __global__ __launch_bounds__(1024) void attn_step_fused_kernel(const float* __restrict__ q, const float* __restrict__ k, const float* __restrict__ v,
                                                                const float* __restrict__ qn, const float* __restrict__ kn,
                                                                const float* __restrict__ rope, float* __restrict__ kc, float* __restrict__ vc,
                                                                float* __restrict__ out, int nh, int nkv, int rd, int pos, float eps, int neox,
-                                                               float scale, int vpitch, float* __restrict__ raw, int smax, int patience) {
+                                                               float scale, int vpitch, int share, unsigned epoch, int patience) {
   extern __shared__ __align__(16) float dyn[];
   __shared__ float qsh[16 * NJ], ksh[16 * NJ], redf[16];
   __shared__ double scs[2], redd[17];
   __shared__ int got_all;
+  __shared__ unsigned tag_sh;
   constexpr int hd = 16 * NJ;
   // the hardware deals consecutive workgroups to the eight dies in turn: die x takes the workgroups of consecutive heads
   // (with 32 query heads on 8 KV heads, one KV head's), so a head's keys and values come from memory into one L2 only
@@ -609,10 +616,13 @@ __global__ __launch_bounds__(1024) void attn_step_fused_kernel(const float* __re
   float ka[4][NJ], kb[4][NJ];
   constexpr int NPASS = 16 / (hd / CS);            // passes of 64 positions a workgroup takes of a head's shared-out scores
   float kx[NPASS][NJ];
-  const bool split = raw != nullptr;
-  // (the head's generation: the number its workgroups will write into their flags; read now, wanted after the scores)
-  unsigned gen = 0;
-  if (split && tid < ns) gen = __hip_atomic_load(&attn_gen[h], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + 1;
+  const bool split = share != 0;
+  // (the head's generation, read now and wanted after the heads are turned: the barrier there hands it round)
+  if (split && tid == 0) {
+    const unsigned gen = (__hip_atomic_load(&attn_gen[h], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + 1) & 0xFFFFFFu;
+    tag_sh = gen << 8 | (epoch & 15u) << 4;
+    got_all = 1;
+  }
   if (split) {
 #pragma unroll
     for (int i = 0; i < NPASS; i++) {
@@ -667,7 +677,8 @@ __global__ __launch_bounds__(1024) void attn_step_fused_kernel(const float* __re
   const int nb = (npos + 255) >> 8;                // 1 .. 4
   bool shared = false;
   if (split) {
-    float* const row = raw + (long long)h * smax;
+    const unsigned die = __builtin_amdgcn_s_getreg((4 - 1) << 11 | 20) & 15u, tag = tag_sh | die;
+    unsigned long long* const row = attn_xrow + (long long)h * 1024;
 #pragma unroll
     for (int i = 0; i < NPASS; i++) {
       const int p = 64 * (cs + ns * i) + pg;
@@ -682,37 +693,28 @@ __global__ __launch_bounds__(1024) void attn_step_fused_kernel(const float* __re
       sacc = sacc + ilt_dppf<ILT_DPP_SHL(8)>(sacc);
       sacc = sacc + ilt_dppf<ILT_DPP_SHL(1)>(sacc);
       sacc = sacc + ilt_dppf<ILT_DPP_SHL(2)>(sacc);
-      if (l == 0 && p < npos) row[p] = sacc * scale;
+      if (l == 0 && p < npos) row[p] = (unsigned long long)tag << 32 | __float_as_uint(sacc * scale);
     }
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");          // this wave's scores are written
-    ilt_barrier_lds();                                        // ... and every wave's
-    // The scores are plain stores: they are in this die's L2 (the wait above) and no further, so the row may only be
-    // read where every one of the head's workgroups ran on this die.  A workgroup's flag is the head's generation
-    // and its die (HW_REG_XCC_ID); lane j of the first wave waits for workgroup j's.  (A counter the workgroups add
-    // themselves to took 2.5 us to be seen by all: read-modify-writes of device scope are made in memory.)
-    if (tid < ns) {
-      const unsigned die = __builtin_amdgcn_s_getreg((4 - 1) << 11 | 20) & 15u;
-      if (tid == 0) __hip_atomic_store(&attn_flag[h * 8 + cs], gen << 4 | die, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      int ok = 0;
+    // position tid's score: its word until it carries the tag (any die's: this launch's, and then its die decides)
+    if (tid < npos) {
       const long long t0 = wall_clock64();
+      bool ok = false;
+      unsigned long long w = 0;
       for (;;) {
-        const unsigned f = __hip_atomic_load(&attn_flag[h * 8 + tid], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        if (f >> 4 == gen) { ok = (f & 15u) == die; break; }          // there; on this die?
-        if (wall_clock64() - t0 >= (long long)patience) break;        // not resident: alone
+        w = __hip_atomic_load(row + tid, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        const unsigned t = (unsigned)(w >> 32);
+        if ((t ^ tag) >> 4 == 0) { ok = (t & 15u) == die; break; }
+        if (wall_clock64() - t0 >= (long long)patience) break;
         __builtin_amdgcn_s_sleep(1);
       }
-      const int all = __builtin_amdgcn_ballot_w64(ok != 0) == (1ull << ns) - 1;
-      if (tid == 0) got_all = all;
+      if (ok) sc[tid] = __uint_as_float((unsigned)w);
+      else got_all = 0;
     }
+    // (the slice behind the row: loads come back in the order asked for, and the row is wanted first.  From here to
+    // the products the barriers wait for LDS only -- __syncthreads waits for every load in flight, the slice's too)
+    load_slice();
     ilt_barrier_lds();
     shared = got_all != 0;
-    // (the row, then the slice: loads come back in the order asked for, and the row is wanted first.  From here to the
-    // products the barriers wait for LDS only -- __syncthreads waits for every load in flight, the slice's too)
-    float mine_raw = 0.0f;
-    if (shared && tid < npos) mine_raw = __builtin_nontemporal_load(row + tid);
-    load_slice();
-    if (shared && tid < npos) sc[tid] = mine_raw;
-    ilt_barrier_lds();                                        // the row is read, its values in LDS (or given up)
   }
   if (!shared) {
     if (split) { load_keys(ka, 0); load_keys(kb, 1); }
@@ -768,7 +770,7 @@ __global__ __launch_bounds__(1024) void attn_step_fused_kernel(const float* __re
   // The head's first workgroup advances the generation as it ends: every workgroup of this launch read it as it
   // started, many microseconds ago (one that starts only now finds the new one, matches no flag and takes all the scores
   // itself).  A store: a counter of readers would be a read-modify-write whose answer a workgroup waits 2 us for.
-  if (split && tid == 0 && cs == 0) __hip_atomic_store(&attn_gen[h], gen & 0x0FFFFFFFu, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  if (split && tid == 0 && cs == 0) __hip_atomic_store(&attn_gen[h], tag_sh >> 8, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 // The same for contexts whose value slice no longer fits LDS (2,049 to 8,192 positions): the slice comes through
@@ -1029,14 +1031,15 @@ hipError_t ilt_k_attn_step(const float* q, const float* k, const float* v, const
     const int ns = hd / 16, nwg = nh * ns;
     const char* sp = getenv("ILT_ATTN_SPLIT");
     const bool split = !(sp && sp[0] == '0') && (nwg & 7) == 0 && ((nwg >> 3) % ns) == 0 && nh <= 256 && ctx >= 64;
-    float* const raw = split ? scratch : nullptr;
     const int patience = sp && sp[0] == '2' ? 0 : 20000;       // 200 us
+    static std::atomic<unsigned> launches{0};
+    const unsigned epoch = ++launches;
     if (hd == 64)
       hipLaunchKernelGGL((attn_step_fused_kernel<4, 16>), dim3(nwg), dim3(1024), fsmem, st, q, k, v, qn, kn, rope, kc, vc, out, nh, nkv, rd, pos, eps,
-                         neox, scale, vpitch, raw, smax, patience);
+                         neox, scale, vpitch, split ? 1 : 0, epoch, patience);
     else
       hipLaunchKernelGGL((attn_step_fused_kernel<8, 16>), dim3(nwg), dim3(1024), fsmem, st, q, k, v, qn, kn, rope, kc, vc, out, nh, nkv, rd, pos, eps,
-                         neox, scale, vpitch, raw, smax, patience);
+                         neox, scale, vpitch, split ? 1 : 0, epoch, patience);
     return hipGetLastError();
   }
   hipLaunchKernelGGL(attn_step_scores_kernel, dim3(nh, (ctx + 255) / 256), dim3(1024), 0, st, q, k, v, qn, kn, rope, kc, vc, scratch, nh, nkv, hd, rd,
