@@ -322,8 +322,9 @@ int ilt_attn_rows(uint64_t stream, const float* q, const float* kc, const float*
 /* ilt_qk_rope and ilt_attn_rows of one token at position pos (< 8192) in fewer launches.  Up to position 1023 with
    heads of 64 or 128: one launch, a workgroup a (query head, 16 columns of the values), each norming and turning its
    head and the token's key itself; where a head's workgroups run on one die (nh a multiple of 8) each takes an eighth
-   of the head's scores and they exchange them through scratch inside the launch, else each takes all of them.  Launches
-   of it that overlap on one GPU make each other give that exchange up (correct, slower).  Otherwise two: the
+   of the head's scores and they exchange them inside the launch through a buffer of the library's (scratch is not
+   touched), else each takes all of them.  Launches of it that overlap on one GPU make each other give that exchange up
+   (correct, slower).  Otherwise two: the
    launch that takes the scores norms and turns the query heads and the token's key and writes the caches' rows at
    pos.  Either way out is what ilt_attn_rows gives after ilt_qk_rope, bit for bit; q and k are left as they came
    (not normed, not turned).  scratch: nh * ((pos + 4) & ~3) floats. */
