@@ -751,14 +751,14 @@ __global__ __launch_bounds__(1024) void attn_step_fused_kernel(const float* __re
     ilt_barrier_lds();
     inv = (float)(1.0 / redd[16]);
   }
-  if (mine) sc[tid] = e * inv;
-  ilt_barrier_lds();
+  // (a position's probability, e * inv, is made by the threads that multiply with it: sc keeps the e's, which every
+  // thread may read since the barrier above, and the barrier that handing the products round would take is saved)
 #pragma unroll
   for (int u = 0; u < PP; u++) {
     const int i = tid + 1024 * u;
     if (i < total) {
       float* dst = vt + (4 * (i % PP)) * vpitch + i / PP;
-      const float sp = sc[i / PP];
+      const float sp = sc[i / PP] * inv;
       dst[0] = sp * r[u].x; dst[vpitch] = sp * r[u].y; dst[2 * vpitch] = sp * r[u].z; dst[3 * vpitch] = sp * r[u].w;
     }
   }
