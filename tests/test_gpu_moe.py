@@ -164,7 +164,8 @@ def _moe_weights(rng, ne, d, ff):
 
 
 @pytest.mark.parametrize("ne,d,ff,nu,clamp", [(8, 512, 256, 3, 0.0), (8, 512, 256, 3, 0.05), (12, 4096, 2048, 6, 0.0),
-                                                (12, 2048, 1024, 9, 0.0)])      # (nine slots: the sum as a launch of its own)
+                                                (12, 2048, 1024, 9, 0.0),       # (nine slots: the sum as a launch of its own)
+                                                (12, 2048, 1024, 8, 0.05)])     # (eight: the most the last product adds itself)
 def test_moe_decode_step_bit_exact(dev, ne, d, ff, nu, clamp):
     """the benchmark's config 4's sequence at a reduced expert count (12 resident experts of the
     full 4096 x 2048 shape), and a small shape with the clamp on: route -> gate/up -> gated
