@@ -712,8 +712,11 @@ int d4_mm_quantized(uint64_t stream, int fmt, int ncols, int nrows, int ntok, in
   const int bw = block_weights(fmt);
   ILT_REQUIRE(ncols > 0 && ncols % bw == 0 && nrows >= 0 && ntok >= 0);
   if (nrows == 0 || ntok == 0) return ILT_OK;
+  // a token's ncols floats start x_stride floats after the token before's, its nrows results y_stride floats after
+  // (the grouped attention output product reads a slice of each token's heads and writes a slice of its low rows,
+  // cuda-ds4f-prefill.lisp:277-281); the quantized activations are packed
   ILT_REQUIRE(w && x && y && ((uintptr_t)w & 15) == 0 && ((uintptr_t)x & 15) == 0);
-  if (x_stride != ncols || y_stride != nrows) return (int)hipErrorNotSupported;       // tokens' rows one after another only
+  ILT_REQUIRE(x_stride >= ncols && y_stride >= nrows && (fmt == ILT_Q8_0 || x_stride % 4 == 0));
   const size_t n = (size_t)ntok * ncols;
   const size_t qb = (n + 255) / 256 * 256, sb = (n / bw * 4 + 255) / 256 * 256, bb = fmt == ILT_Q8_0 ? 0 : (n / 16 * 4 + 255) / 256 * 256;
   uint8_t* room = nullptr;
@@ -722,12 +725,12 @@ int d4_mm_quantized(uint64_t stream, int fmt, int ncols, int nrows, int ntok, in
   if (fmt == ILT_Q8_0) {
     // d4-shared!'s and the attention projections' activations: quantize-q8! with the scale kept a float (ds4f.lisp:1052-1053)
     ILT_REQUIRE(wd && (row_bytes == 0 || row_bytes == ncols));
-    ILT_TRY(ilt_k_quant_q8(x, xq, xs, nullptr, (long long)(n / 32), 0, S(stream)));
-    return (int)ilt_k_gemm_i8(ILT_Q8_0, (const uint8_t*)w, wd, ncols, nrows, ncols, xq, xs, nullptr, ntok, y, nullptr, 0, S(stream));
+    ILT_TRY(ilt_k_quant_rows(0, x, xq, xs, nullptr, ntok, ncols, x_stride, 0, S(stream)));
+    return (int)ilt_k_gemm_i8(ILT_Q8_0, (const uint8_t*)w, wd, ncols, nrows, ncols, xq, xs, nullptr, ntok, y, nullptr, 0, S(stream), y_stride);
   }
   ILT_REQUIRE(row_bytes == ncols / 256 * block_bytes(fmt));
-  ILT_TRY(ilt_k_quant_q8k(x, xq, xs, bs, (long long)(n / 256), S(stream)));
-  return (int)ilt_k_gemm_i8(fmt, (const uint8_t*)w, nullptr, row_bytes, nrows, ncols, xq, xs, bs, ntok, y, nullptr, 0, S(stream));
+  ILT_TRY(ilt_k_quant_rows(1, x, xq, xs, bs, ntok, ncols, x_stride, 0, S(stream)));
+  return (int)ilt_k_gemm_i8(fmt, (const uint8_t*)w, nullptr, row_bytes, nrows, ncols, xq, xs, bs, ntok, y, nullptr, 0, S(stream), y_stride);
 }
 }  // namespace
 

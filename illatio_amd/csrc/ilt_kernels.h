@@ -117,6 +117,9 @@ unsigned long long ilt_k_streamed_launches();      // decode products launched a
 
 hipError_t ilt_k_quant_q8(const float* x, int8_t* xq, float* xs, int* xsum, long long nblocks, int f16_scale, hipStream_t st);
 hipError_t ilt_k_quant_q8k(const float* x, int8_t* xq, float* xd, int* bsums, long long nblocks, hipStream_t st);
+// ntok rows of cols floats, x_stride floats apart, quantized into packed rows: quantize-q8! (k 0) or quantize-q8k! (k 1)
+hipError_t ilt_k_quant_rows(int k, const float* x, int8_t* xq, float* xs, int* bsums, long long ntok, int cols, long long x_stride,
+                            int f16_scale, hipStream_t st);
 // rmsnorm! then quantize-q8! (k 0; xsum may be null) or quantize-q8k! (k 1), a row of DIM floats a workgroup
 hipError_t ilt_k_rmsnorm_quant(int k, const float* x, const float* w, float* h, int8_t* xq, float* xs, int* xsum, int dim,
                                float eps, int f16_scale, int seq, int nrows, hipStream_t st);
@@ -143,12 +146,13 @@ hipError_t ilt_k_moe_sum(int d, int k, const float* down, const float* shared_, 
 hipError_t ilt_k_moe_sum_rows(int d, int nu, int ntok, const float* down, const uint32_t* map, const float* shared_,
                               float* moe, hipStream_t st);
 
+// ldy: floats from one token's results to the next token's in y (0: rows)
 hipError_t ilt_k_gemm_i8(int fmt, const uint8_t* w, const uint16_t* wd, long long row_bytes, int rows, int cols,
                          const int8_t* xq, const float* xs, const int* bsums, int ntok, float* y, const float* bias,
-                         int acc, hipStream_t st);
+                         int acc, hipStream_t st, long long ldy = 0);
 // Q6_K, Q4_K and Q2_K, exact, on the pipelined kernel (kernels_gemm_bf16.hip): scale * quant as int8 planes
 hipError_t ilt_k_gemm_i8_planes(int fmt, const uint8_t* w, long long row_bytes, int rows, int cols, const int8_t* xq, const float* xd,
-                                const int* bsums, int ntok, float* y, const float* bias, int acc, hipStream_t st);
+                                const int* bsums, int ntok, float* y, const float* bias, int acc, hipStream_t st, long long ldy = 0);
 hipError_t ilt_k_gemm_i8_planes_n(int fmt, int nmat, const uint8_t* const* ws, const int* rows, float* const* ys, const float* const* biases,
                                   long long row_bytes, int cols, const int8_t* xq, const float* xd, const int* bsums, int ntok, int acc,
                                   hipStream_t st);
@@ -159,7 +163,7 @@ hipError_t ilt_k_gemm_i8_pp(const uint8_t* wh, const uint8_t* wl, const float* w
                             int ntok, float* y, const float* bias, int acc, hipStream_t st);
 // Q8_0, exact, on the pipelined kernel (cols a multiple of 64)
 hipError_t ilt_k_gemm_i8_q8(const uint8_t* wq, const uint16_t* wd, int rows, int cols, const int8_t* xq, const float* xs, int ntok,
-                            float* y, const float* bias, int acc, hipStream_t st);
+                            float* y, const float* bias, int acc, hipStream_t st, long long ldy = 0);
 hipError_t ilt_k_gemm_i8_planes_id(int fmt, const uint64_t* ptrs, long long add, const uint32_t* counts, const uint32_t* bases, int ne,
                                    long long row_bytes, int rows, int cols, const int8_t* xq, const float* xd, const int* bsums,
                                    long long total_rows, float* y, hipStream_t st);

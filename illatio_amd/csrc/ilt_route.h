@@ -48,6 +48,10 @@ __device__ __forceinline__ void route_token(int lane, int ne, int nu, float scal
   float my_p = 0.0f;
   if (eids) {
     if (lane < nu) {
+      // A table entry names an expert below ne in every model file; the reference's CPU path indexes probs with it
+      // unchecked (an array-bounds error in Lisp, whatever lies behind the array in its CUDA kernel).  Here an entry
+      // from outside is brought inside, so that neither this read nor a later launch's slot table is indexed out of
+      // bounds; entries below ne pass unchanged.
       const u32 e = min((u32)eids[lane], (u32)(ne - 1));
       my_sel = e;
       my_p = route_prob(lg[e]);

@@ -202,6 +202,7 @@ struct GemmParams {
   int rows, cols; long row_bytes;
   const i8* xq; const float* xs; const int* bsums;
   float* y; const float* bias; int acc; int ntok;
+  long ldy;                               // floats from one token's results to the next token's
 };
 
 template <int FMT>
@@ -389,7 +390,7 @@ __global__ __launch_bounds__(256) void gemm_i8_kernel(GemmParams p) {
     for (int b = 0; b < 2; b++) {
       const int tk = wt0 + 16 * b + li;
       if (tk >= ntok) continue;
-      float* yo = p.y + (tok0 + tk) * (long)p.rows + row;
+      float* yo = p.y + (tok0 + tk) * p.ldy + row;
 #pragma unroll
       for (int r = 0; r < 4; r++) {
         if (row + r >= p.rows) continue;
@@ -425,20 +426,22 @@ hipError_t dispatch(int fmt, const GemmParams& p, unsigned tiles_x, hipStream_t 
 
 hipError_t ilt_k_gemm_i8(int fmt, const uint8_t* w, const uint16_t* wd, long long row_bytes, int rows, int cols,
                          const int8_t* xq, const float* xs, const int* bsums, int ntok, float* y, const float* bias,
-                         int acc, hipStream_t st) {
+                         int acc, hipStream_t st, long long ldy) {
   if (ntok <= 0 || rows <= 0) return hipSuccess;
+  if (ldy == 0) ldy = rows;
+  if (ldy < rows) return hipErrorInvalidValue;
   // Q6_K, Q4_K and Q2_K with enough tokens and rows to fill 128 x 128 tiles: the pipelined kernel with scale * quant
   // as int8 planes, the same bits.  ILT_I8_PLANES (tests): "0" never, "1" whenever the format allows.
   const char* force = getenv("ILT_I8_PLANES");
   const int forced = force ? atoi(force) : -1;
-  const bool fits = rows < (1 << 21) && (long long)rows * row_bytes < 0x7FFFFFFFLL;      // the pipelined kernels' 32-bit offsets
+  const bool fits = rows < (1 << 21) && ldy < (1 << 21) && (long long)rows * row_bytes < 0x7FFFFFFFLL;      // the pipelined kernels' 32-bit offsets
   if (fits && (fmt == ILT_Q6_K || fmt == ILT_Q4_K || fmt == ILT_Q2_K) && cols % 256 == 0 && forced != 0 && (forced == 1 || (ntok >= 96 && rows >= 128)))
-    return ilt_k_gemm_i8_planes(fmt, w, row_bytes, rows, cols, xq, xs, bsums, ntok, y, bias, acc, st);
+    return ilt_k_gemm_i8_planes(fmt, w, row_bytes, rows, cols, xq, xs, bsums, ntok, y, bias, acc, st, ldy);
   if (fits && fmt == ILT_Q8_0 && cols % 64 == 0 && forced != 0 && (forced == 1 || (ntok >= 96 && rows >= 128)))
-    return ilt_k_gemm_i8_q8(w, wd, rows, cols, xq, xs, ntok, y, bias, acc, st);
+    return ilt_k_gemm_i8_q8(w, wd, rows, cols, xq, xs, ntok, y, bias, acc, st, ldy);
   GemmParams p = {};
   p.w = w; p.wdq = wd; p.rows = rows; p.cols = cols; p.row_bytes = row_bytes;
-  p.xq = xq; p.xs = xs; p.bsums = bsums; p.y = y; p.bias = bias; p.acc = acc; p.ntok = ntok;
+  p.xq = xq; p.xs = xs; p.bsums = bsums; p.y = y; p.bias = bias; p.acc = acc; p.ntok = ntok; p.ldy = (long)ldy;
   return dispatch(fmt, p, (unsigned)((ntok + TN - 1) / TN), st);
 }
 
@@ -459,7 +462,7 @@ hipError_t ilt_k_gemm_i8_id(int fmt, const uint64_t* ptrs, long long add, const 
   GemmParams p = {};
   p.ptrs = ptrs; p.add = add; p.counts = counts; p.bases = bases; p.ne = ne;
   p.rows = rows; p.cols = cols; p.row_bytes = row_bytes;
-  p.xq = xq; p.xs = xs; p.bsums = bsums; p.y = y; p.ntok = (int)total_rows;
+  p.xq = xq; p.xs = xs; p.bsums = bsums; p.y = y; p.ntok = (int)total_rows; p.ldy = rows;
   // sum over experts of ceil(count/64) <= total/64 + ne
   return dispatch(fmt, p, (unsigned)(total_rows / TN + ne), st);
 }

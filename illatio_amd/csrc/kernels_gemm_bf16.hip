@@ -1901,11 +1901,13 @@ static hipError_t launch_i8p(int fmt, const BfParams& p, long long token_tiles, 
 }
 
 hipError_t ilt_k_gemm_i8_planes(int fmt, const uint8_t* w, long long row_bytes, int rows, int cols, const int8_t* xq, const float* xd,
-                                const int* bsums, int ntok, float* y, const float* bias, int acc, hipStream_t st) {
+                                const int* bsums, int ntok, float* y, const float* bias, int acc, hipStream_t st, long long ldy) {
   if (ntok <= 0 || rows <= 0) return hipSuccess;
+  if (ldy == 0) ldy = rows;
+  if (ldy < rows || ldy * 1024 >= 0x7FFFFFFFLL) return hipErrorInvalidValue;
   BfParams p = {};
   p.w = w; p.rows = rows; p.cols = cols; p.row_bytes = row_bytes; p.x = (const u16*)xq; p.xd = xd; p.bsums = bsums;
-  p.y = y; p.bias = bias; p.acc = acc; p.ntok = ntok; p.ldy = rows;
+  p.y = y; p.bias = bias; p.acc = acc; p.ntok = ntok; p.ldy = ldy;
   return launch_i8p<false>(fmt, p, (ntok + 127) / 128, st);
 }
 
@@ -1962,12 +1964,13 @@ hipError_t ilt_k_gemm_i8_pp(const uint8_t* wh, const uint8_t* wl, const float* w
 }
 
 hipError_t ilt_k_gemm_i8_q8(const uint8_t* wq, const uint16_t* wd, int rows, int cols, const int8_t* xq, const float* xs, int ntok,
-                            float* y, const float* bias, int acc, hipStream_t st) {
+                            float* y, const float* bias, int acc, hipStream_t st, long long ldy) {
   if (ntok <= 0 || rows <= 0) return hipSuccess;
-  if (cols % 64 != 0 || (long long)rows * 1024 >= 0x7FFFFFFFLL || (long long)128 * cols >= 0x7FFFFFFFLL) return hipErrorInvalidValue;
+  if (ldy == 0) ldy = rows;
+  if (cols % 64 != 0 || ldy < rows || ldy * 1024 >= 0x7FFFFFFFLL || (long long)128 * cols >= 0x7FFFFFFFLL) return hipErrorInvalidValue;
   BfParams p = {};
   p.w = wq; p.wdq = wd; p.rows = rows; p.cols = cols; p.row_bytes = cols; p.x = (const u16*)xq; p.xd = xs;
-  p.y = y; p.bias = bias; p.acc = acc; p.ntok = ntok; p.ldy = rows;
+  p.y = y; p.bias = bias; p.acc = acc; p.ntok = ntok; p.ldy = ldy;
   const long long total = (long long)((ntok + 127) / 128) * ((rows + 127) / 128), per = (total + 7) / 8;
   if (per * 8 > 0x7FFFFFFFLL) return hipErrorInvalidValue;
   hipLaunchKernelGGL(gemm_i8q_kernel, dim3((unsigned)(per * 8)), dim3(512), 0, st, p);

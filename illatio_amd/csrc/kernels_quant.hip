@@ -14,11 +14,12 @@ __device__ const u64 q_grid_dev[256] = { ILT_IQ2XXS_GRID_VALUES };
 // unrounded d.  xsum (optional) gets the block's integer sum.
 __global__ __launch_bounds__(256) void quant_q8_kernel(const float* __restrict__ x, i8* __restrict__ xq,
                                                        float* __restrict__ xs, int* __restrict__ xsum,
-                                                       long long nblocks, int f16_scale) {
+                                                       long long nblocks, int f16_scale, long long bpr, long long x_stride) {
   const long long i = (long long)blockIdx.x * 256 + threadIdx.x;
   const long long b = i >> 5;
   const bool live = b < nblocks;
-  const float v = live ? x[i] : 0.0f;
+  // bpr > 0: rows of bpr blocks, x_stride floats from one row's start to the next's (the output stays packed)
+  const float v = live ? x[bpr > 0 ? (b / bpr) * x_stride + (b % bpr) * 32 + (i & 31) : i] : 0.0f;
   float amax = ilt_max16(fabsf(v));
   amax = fmaxf(amax, __shfl_xor(amax, 16));
   const float d = amax / 127.0f;
@@ -39,11 +40,13 @@ __global__ __launch_bounds__(256) void quant_q8_kernel(const float* __restrict__
 // first of equals, sets iscale = -127/max; q = min(127, round-half-even(iscale*x));
 // d = 1/iscale; sums of each 16 quants.
 __global__ __launch_bounds__(256) void quant_q8k_kernel(const float* __restrict__ x, i8* __restrict__ xq,
-                                                        float* __restrict__ xd, int* __restrict__ bsums, long long nblocks) {
+                                                        float* __restrict__ xd, int* __restrict__ bsums, long long nblocks,
+                                                        long long bpr, long long x_stride) {
   const int lane = threadIdx.x & 63;
   const long long b = (long long)blockIdx.x * 4 + (threadIdx.x >> 6);
   if (b >= nblocks) return;
-  const float4 v4 = ((const float4*)(x + b * 256))[lane];
+  // bpr > 0: rows of bpr blocks, x_stride floats (a multiple of 4) from one row's start to the next's
+  const float4 v4 = ((const float4*)(x + (bpr > 0 ? (b / bpr) * x_stride + (b % bpr) * 256 : b * 256)))[lane];
   const float v[4] = {v4.x, v4.y, v4.z, v4.w};
   // |v|'s bits order as |v| does; the low word prefers the earlier index
   u64 key = 0;
@@ -211,13 +214,26 @@ __global__ __launch_bounds__(256) void mm_f16_dot16_kernel(int ncols, int nrows,
 
 hipError_t ilt_k_quant_q8(const float* x, int8_t* xq, float* xs, int* xsum, long long nblocks, int f16_scale, hipStream_t st) {
   if (nblocks <= 0) return hipSuccess;
-  hipLaunchKernelGGL(quant_q8_kernel, dim3((unsigned)((nblocks * 32 + 255) / 256)), dim3(256), 0, st, x, xq, xs, xsum, nblocks, f16_scale);
+  hipLaunchKernelGGL(quant_q8_kernel, dim3((unsigned)((nblocks * 32 + 255) / 256)), dim3(256), 0, st, x, xq, xs, xsum, nblocks, f16_scale,
+                     0LL, 0LL);
   return hipGetLastError();
 }
 
 hipError_t ilt_k_quant_q8k(const float* x, int8_t* xq, float* xd, int* bsums, long long nblocks, hipStream_t st) {
   if (nblocks <= 0) return hipSuccess;
-  hipLaunchKernelGGL(quant_q8k_kernel, dim3((unsigned)((nblocks + 3) / 4)), dim3(256), 0, st, x, xq, xd, bsums, nblocks);
+  hipLaunchKernelGGL(quant_q8k_kernel, dim3((unsigned)((nblocks + 3) / 4)), dim3(256), 0, st, x, xq, xd, bsums, nblocks, 0LL, 0LL);
+  return hipGetLastError();
+}
+
+hipError_t ilt_k_quant_rows(int k, const float* x, int8_t* xq, float* xs, int* bsums, long long ntok, int cols, long long x_stride,
+                            int f16_scale, hipStream_t st) {
+  const int bw = k ? 256 : 32;
+  if (ntok <= 0) return hipSuccess;
+  if (cols <= 0 || cols % bw != 0 || x_stride < cols || (k && x_stride % 4 != 0)) return hipErrorInvalidValue;
+  const long long bpr = cols / bw, nblocks = ntok * bpr;
+  if (k) hipLaunchKernelGGL(quant_q8k_kernel, dim3((unsigned)((nblocks + 3) / 4)), dim3(256), 0, st, x, xq, xs, bsums, nblocks, bpr, x_stride);
+  else hipLaunchKernelGGL(quant_q8_kernel, dim3((unsigned)((nblocks * 32 + 255) / 256)), dim3(256), 0, st, x, xq, xs, (int*)nullptr, nblocks,
+                          f16_scale, bpr, x_stride);
   return hipGetLastError();
 }
 

@@ -225,11 +225,12 @@ def ffn_step_fused(dev, pool, sh, sel, w, norm2, clamp, ws=None, tables=None, ro
     return moe
 
 
-def ffn_step_device(dev, pool, sh, logits, norm2, ne, nu, scale, clamp, bias=None, ws=None):
+def ffn_step_device(dev, pool, sh, logits, norm2, ne, nu, scale, clamp, bias=None, ws=None, tid2eid=None, tokens=None):
     """A decode step with nothing going through the host: d4_route on the device, then
-    ffn_step_fused indexing the slot table by its result (six launches)."""
+    ffn_step_fused indexing the slot table by its result (six launches).  TID2EID, TOKENS:
+    a hash layer's table and the token's id on the device (see route)."""
     A = ws.alloc if ws else hip.hip_alloc
-    sel, w = route(dev, logits, 1, ne, nu, scale, bias, A)
+    sel, w = route(dev, logits, 1, ne, nu, scale, bias, A, tid2eid=tid2eid, tokens=tokens)
     moe = ffn_step_fused(dev, pool, sh, nu, None, norm2, clamp, ws=ws, routed=(sel, w))
     if not ws:
         hip.hip_free(sel); hip.hip_free(w)
@@ -336,10 +337,16 @@ def ffn_small(dev, pool, sh, logits, norm2, n, ne, nu, scale, clamp, bias=None, 
     return moe
 
 
-def route(dev, logits, n, ne, nu, scale, bias=None, alloc=hip.hip_alloc):
-    """D4_ROUTE for N tokens' LOGITS (a DBuf): returns (sel, w) DBufs of N x NU."""
+def route(dev, logits, n, ne, nu, scale, bias=None, alloc=hip.hip_alloc, tid2eid=None, tokens=None):
+    """D4_ROUTE for N tokens' LOGITS (a DBuf): returns (sel, w) DBufs of N x NU.  On a hash layer
+    (d4-route, ds4f.lisp:961-963; DK-FFN-ROUTED-CHUNK passes HASH 1, cuda-ds4f-prefill.lisp) TID2EID is
+    the layer's table on the device (int32, NU experts a vocabulary entry) and TOKENS the N token ids
+    (uint32): token t's experts are its row of the table as it stands, the weights from the logits."""
+    if (tid2eid is None) != (tokens is None):
+        raise ValueError("a hash layer's routing takes both the table and the token ids")
     sel, w = alloc(dev, 4 * n * nu), alloc(dev, 4 * n * nu)
-    hip.launch(dev, "d4_route", n, ne, [ne, nu, 0, float(scale), 1 if bias is not None else 0, logits, bias, None, None, sel, w],
+    hip.launch(dev, "d4_route", n, ne, [ne, nu, 0 if tid2eid is None else 1, float(scale), 1 if bias is not None else 0, logits, bias,
+                                        tid2eid, tokens, sel, w],
                shared=4 * (2 * ne + 64 + nu))
     return sel, w
 

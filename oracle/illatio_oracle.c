@@ -17,7 +17,9 @@
  * the GGUF layouts and hand-built blocks; integer block sums by brute force;
  * the quantizers' special cases; row dots against a double-precision dot of
  * dequantized values (the reference's own criterion, inspect/iquant-test.lisp:
- * 45-53); d4-route against a stable sort; the IQ2_XXS tables against the
+ * 45-53); d4-route against a stable sort (its hash-table branch against an
+ * explicit evaluation and against the other branch on a row that is the
+ * top choice); the IQ2_XXS tables against the
  * reference's three copies; swiglu!, f32-dot16, rope-table, rope-head!,
  * attend-head! against explicit evaluations in numpy (with the plausible
  * misreadings shown to give other bits), forward-1 as those pieces in order.
@@ -606,6 +608,21 @@ void orc_route(const float* logits, const float* bias, int ne, int nu, float sca
   if (sum < 6.103515625e-5f) sum = 6.103515625e-5f;
   for (int i = 0; i < nu; i++) w[i] = (w[i] / sum) * scale;
   free(probs); free(s);
+}
+
+/* ---- src/ds4f.lisp:961-963, 973-977 (d4-route), the hash-table branch ------------------------------- */
+/* The first layers of the model take a token's experts from a table: sel[i] = tid2eid[token*nu + i],
+   in the table's order (no sorting, duplicates and all); the weights are formed from the unbiased
+   probabilities exactly as in the top-N_USED branch (the bias plays no part: it only enters the
+   scores the other branch picks by). */
+void orc_route_table(const float* logits, const int32_t* tid2eid, int token, int ne, int nu, float scale,
+                     int32_t* sel, float* w) {
+  for (int i = 0; i < nu; i++) sel[i] = tid2eid[(int64_t)token * nu + i];
+  float sum = 0.0f;
+  for (int i = 0; i < nu; i++) { w[i] = sqrtf(orc_softplus(logits[sel[i]])); sum = sum + w[i]; }
+  if (sum < 6.103515625e-5f) sum = 6.103515625e-5f;
+  for (int i = 0; i < nu; i++) w[i] = (w[i] / sum) * scale;
+  (void)ne;
 }
 
 /* ---- the routed experts of one token: src/ds4f.lisp:994-1037 (d4-routed!) ------------------------ */

@@ -205,6 +205,17 @@ def route(logits, nu, scale, bias=None):
     return sel, w
 
 
+def route_table(logits, tid2eid, token, nu, scale):
+    """d4-route on a hash layer: TOKEN's row of the TID2EID table (ds4f.lisp:961-963)."""
+    logits = _c(logits, np.float32)
+    table = _c(tid2eid, np.int32)
+    sel = np.empty(nu, np.int32)
+    w = np.empty(nu, np.float32)
+    lib().orc_route_table(_p(logits), _p(table), C.c_int(int(token)), C.c_int(logits.size), C.c_int(nu), C.c_float(scale),
+                          _p(sel), _p(w))
+    return sel, w
+
+
 def moe_routed(gate, up, down, d, ff, sel, w, clamp, norm, avx2=False, nthreads=1):
     nu = len(sel)
     moe = np.empty(d, np.float32)

@@ -288,7 +288,7 @@ def test_d4_mm_on_float_rows_bit_exact(dev, qtype, rows, cols, n):
     """d4_mm_q8_0 / d4_mm_q2_k / d4_mm_iq2_xxs (ds4f_mm.cu:252-255) take float rows; each token's result is the CPU
     path's: quantize-q8! with a float scale and the Q8_0 row dot (q8mv!, ds4f.lisp:294-297), or quantize-q8k! and
     the expert formats' row dots.  Two calls of different sizes in a row (the library's room for the quantized rows
-    grows), and the strides the quantized formats do not take are refused."""
+    grows); strides shorter than a row are refused."""
     from illatio_amd import dense, ds4f, hip
     rng = synth.make_rng(qtype * 13 + rows + n)
     w = synth.weights(qtype, rows, cols, rng)
@@ -308,9 +308,62 @@ def test_d4_mm_on_float_rows_bit_exact(dev, qtype, rows, cols, n):
         assert np.array_equal(bits(got), bits(want)), (ntok, np.abs(got - want).max())
         if ntok == n:
             with pytest.raises(hip.HipError):
-                ds4f.dk_mm(dev, name, wq, wd, rb, rows, cols, xb, y, ntok, y_stride=rows + 8)
+                ds4f.dk_mm(dev, name, wq, wd, rb, rows, cols, xb, y, ntok, y_stride=rows - 1)
+            with pytest.raises(hip.HipError):
+                ds4f.dk_mm(dev, name, wq, wd, rb, rows, cols, xb, y, ntok, x_stride=cols - 4)
         hip.hip_free(xb); hip.hip_free(y)
     if qtype == synth.Q8_0:
         m.free()
     else:
         hip.hip_free(wq)
+
+
+@pytest.mark.parametrize("groups,rank,gdim,n", [(4, 128, 512, 130), (3, 48, 96, 9), (8, 256, 1024, 257)])
+def test_d4_mm_q8_0_grouped_attention_output_strided(dev, groups, rank, gdim, n):
+    """The reference's strided call of d4_mm_q8_0 (cuda-ds4f-prefill.lisp:277-281): the grouped attention output
+    product runs once a group on a slice of each token's heads (x_stride = nh*hd floats between tokens) with that
+    group's rows of the matrix (the quants and the scales at offsets into their arrays), into a slice of each
+    token's low row (y_stride = groups*rank).  Every (token, group) has the CPU path's bits: quantize-q8! with a
+    float scale on the group's slice, the Q8_0 row dots of the group's rows."""
+    from illatio_amd import dense, ds4f, hip
+    rng = synth.make_rng(groups * 1000 + n)
+    rows = groups * rank
+    w = synth.weights(synth.Q8_0, rows, gdim, rng)
+    m = dense.upload_gmat(dev, "attn_output_a", synth.Q8_0, rows, gdim, w)
+    heads = synth.activations((n, groups * gdim), rng)
+    hb = hip.hip_upload_new(dev, heads)
+    low = hip.hip_alloc(dev, 4 * n * rows)
+    hip.hip_zero(low)
+    for g in range(groups):
+        ds4f.dk_mm(dev, "d4_mm_q8_0", m.qs.at(g * rank * gdim), m.d.at(2 * g * rank * (gdim // 32)), 0, rank, gdim,
+                   hb.at(4 * g * gdim), low.at(4 * g * rank), n, x_stride=groups * gdim, y_stride=rows)
+    got = hip.hip_floats(low, n * rows).reshape(n, groups, rank)
+    rb = synth.row_bytes(synth.Q8_0, gdim)
+    for g in range(groups):
+        xg = np.ascontiguousarray(heads[:, g * gdim:(g + 1) * gdim])
+        wg = w[g * rank * rb:(g + 1) * rank * rb]
+        want = orc.matmul(synth.Q8_0, wg, rank, gdim, xg, f16_scale=False, nthreads=8).reshape(n, rank)
+        assert np.array_equal(bits(got[:, g]), bits(want)), (g, np.abs(got[:, g] - want).max())
+    hip.hip_free(hb); hip.hip_free(low); m.free()
+
+
+@pytest.mark.parametrize("qtype,rows,cols,n", [(synth.Q2_K, 256, 512, 140), (synth.IQ2_XXS, 70, 256, 5)])
+def test_d4_mm_k_formats_strided(dev, qtype, rows, cols, n):
+    """d4_mm_q2_k / d4_mm_iq2_xxs with the tokens' rows and results further apart than their widths: what lies between
+    is neither read nor written."""
+    from illatio_amd import ds4f, hip
+    rng = synth.make_rng(qtype + rows + n)
+    w = synth.weights(qtype, rows, cols, rng)
+    name = {synth.Q2_K: "d4_mm_q2_k", synth.IQ2_XXS: "d4_mm_iq2_xxs"}[qtype]
+    wb = hip.hip_upload_new(dev, w)
+    xs, ys = cols + 64, rows + 24
+    x = synth.activations((n, xs), rng)
+    x[:, cols:] = np.nan
+    xb, y = hip.hip_upload_new(dev, x), hip.hip_upload_new(dev, np.full((n, ys), 7.0, np.float32))
+    ds4f.dk_mm(dev, name, wb, None, synth.row_bytes(qtype, cols), rows, cols, xb, y, n, x_stride=xs, y_stride=ys)
+    got = hip.hip_floats(y, n * ys).reshape(n, ys)
+    want = orc.matmul(qtype, w, rows, cols, np.ascontiguousarray(x[:, :cols]), nthreads=8).reshape(n, rows)
+    assert np.array_equal(bits(got[:, :rows]), bits(want))
+    assert (got[:, rows:] == 7.0).all()
+    for b in (wb, xb, y):
+        hip.hip_free(b)

@@ -23,14 +23,16 @@ def bits(a):
     return np.ascontiguousarray(a, np.float32).view(np.uint32)
 
 
-def run_greedy(dev, host, nprompt, ndecode, chunk, nctx, seed, check_cache=False, one_call=True):
+def run_greedy(dev, host, nprompt, ndecode, chunk, nctx, seed, check_cache=False, one_call=True, say=None):
     from illatio_amd import hip, model
     c = host["config"]
     rng = synth.make_rng(seed)
     prompt = rng.integers(0, c["vocab"], nprompt).tolist()
     cpu = orc.DenseModel(host, nctx)
-    for t in prompt[:-1]:
+    for i, t in enumerate(prompt[:-1]):
         cpu.forward(t, logits=False, nthreads=16)
+        if say and i % 64 == 63:
+            say(f"oracle: prompt position {i + 1} of {nprompt}")
     want, _ = cpu.forward(prompt[-1], nthreads=16)
     gpu = model.DenseModel(dev, host, nctx, chunk=chunk)
     gpu.one_call = gpu.one_call and one_call                  # a token by ilt_dense_decode, or launch by launch from Python
@@ -54,6 +56,8 @@ def run_greedy(dev, host, nprompt, ndecode, chunk, nctx, seed, check_cache=False
         got = hip.hip_floats(gpu.logits, c["vocab"])
         assert np.array_equal(bits(got), bits(want)), (step, np.abs(got - want).max())
         same += 1
+        if say and step % 32 == 31:
+            say(f"greedy token {step + 1} of {ndecode}: logits bit for bit, smallest top-1 margin so far {min(margins):.4f}")
     gpu.free()
     return same, margins
 
@@ -342,3 +346,23 @@ def test_config_2_all_36_layers(dev):
     host = model.synth_model(36)
     same, _ = run_greedy(dev, host, nprompt=8, ndecode=12, chunk=8, nctx=24, seed=5)
     assert same == 12
+
+
+def test_config_2_as_stated_36_layers_512_token_prompt_128_greedy_tokens(dev, capsys):
+    """Config 2 at its stated size under the oracle: all 36 layers at full width, the seeded prompt of 512 random token
+    ids through the prefill products in chunks of 128, then 128 greedy tokens at contexts of 512 to 639 positions (the
+    one-launch attention with a head's scores shared out), every step's logits the CPU path's bit for bit -- hence the
+    same top-1 token at every step, without a near-tie allowance; the smallest margin between the two best logits is
+    printed and must be positive.  (The oracle's 640 positions take two to three minutes on the host's cores: a line is
+    printed every 64 positions.)"""
+    from illatio_amd import model
+
+    def say(msg):
+        with capsys.disabled():
+            print("  [config 2]", msg, flush=True)
+
+    host = model.synth_model(2)
+    same, margins = run_greedy(dev, host, nprompt=512, ndecode=128, chunk=128, nctx=640, seed=22, say=say)
+    assert same == 128
+    say(f"128 greedy tokens, smallest top-1 margin {min(margins):.4f}, median {float(np.median(margins)):.4f}")
+    assert min(margins) > 0

@@ -44,6 +44,70 @@ def test_route_indices_and_weights_bit_exact(dev, ne, nu, n):
             hip.hip_free(b)
 
 
+@pytest.mark.parametrize("ne,nu,n,vocab", [(256, 6, 70, 500), (16, 3, 5, 9), (64, 8, 33, 129280)])
+def test_route_from_the_hash_table_bit_exact(dev, ne, nu, n, vocab):
+    """A hash layer's routing (d4-route's tid2eid branch, ds4f.lisp:961-963; d4_route with hash = 1,
+    cuda/ds4f_chunk.cu:439-440): each token's experts are its row of the table as it stands -- unsorted, an expert
+    named twice staying twice, the bias ignored -- and the weights are the oracle's bit for bit."""
+    from illatio_amd import ds4f, hip
+    rng = synth.make_rng(ne + n + 5)
+    logits = synth.zipf_router_logits(n, ne, rng)
+    logits[1, :] = -40.0                                   # the sum of the probabilities under its floor
+    logits[2, :4] = [30.0, -30.0, 21.0, -21.0]             # softplus's outer branches
+    table = np.stack([rng.permutation(ne)[:nu] for _ in range(vocab)]).astype(np.int32)
+    table[vocab - 1, :] = ne - 1                           # one expert in every slot
+    table[0, :] = np.arange(nu)[::-1]
+    table[1, :4 if nu > 3 else nu] = [0, 1, 2, 3][:4 if nu > 3 else nu]
+    tokens = rng.integers(0, vocab, n).astype(np.uint32)
+    tokens[0], tokens[1], tokens[2] = vocab - 1, 0, 1
+    lb, tb, kb = hip.hip_upload_new(dev, logits), hip.hip_upload_new(dev, table), hip.hip_upload_new(dev, tokens)
+    bias = (rng.standard_normal(ne) * 0.5).astype(np.float32)
+    bb = hip.hip_upload_new(dev, bias)
+    for b in (None, bb):                                   # the bias plays no part on a hash layer
+        sel, w = ds4f.route(dev, lb, n, ne, nu, 1.5, b, tid2eid=tb, tokens=kb)
+        gs = hip.hip_download(sel, np.uint32, n * nu).reshape(n, nu)
+        gw = hip.hip_floats(w, n * nu).reshape(n, nu)
+        for t in range(n):
+            ws, ww = orc.route_table(logits[t], table, tokens[t], nu, 1.5)
+            assert gs[t].tolist() == ws.tolist() == table[tokens[t]].tolist(), (t, gs[t], ws)
+            assert np.array_equal(bits(gw[t]), bits(ww)), t
+        hip.hip_free(sel); hip.hip_free(w)
+    # the slot-block launch by the reference's name refuses a hash layer without its table
+    with pytest.raises(hip.HipError):
+        hip.launch(dev, "d4_route", n, ne, [ne, nu, 1, 1.5, 0, lb, None, None, None, lb, lb], shared=0)
+    with pytest.raises(ValueError):
+        ds4f.route(dev, lb, n, ne, nu, 1.5, tid2eid=tb)
+    for b in (lb, tb, kb, bb):
+        hip.hip_free(b)
+
+
+def test_hash_layer_decode_step_bit_exact(dev):
+    """One token's FFN on a hash layer with nothing going through the host: d4_route leaves the token's table row on
+    the device, the experts' launches index the slot table by it, and the step has the bits of d4-routed! +
+    d4-shared! on the oracle's table row."""
+    from illatio_amd import ds4f, hip
+    rng = synth.make_rng(77)
+    ne, nu, d, ff, clamp, vocab = 16, 3, 512, 256, 7.0, 40
+    gate, up, down, sg, su, sd = _moe_weights(rng, ne, d, ff)
+    pool = ds4f.ExpertPool(dev, ne, d, ff, gate, up, down)
+    sh = ds4f.SharedExpert(dev, d, ff, sg, su, sd)
+    logits, norm = synth.activations(ne, rng), synth.activations(d, rng)
+    table = np.stack([rng.permutation(ne)[:nu] for _ in range(vocab)]).astype(np.int32)
+    token = np.array([23], np.uint32)
+    lb, tb, kb, nb = (hip.hip_upload_new(dev, a) for a in (logits, table, token, norm))
+    wsel, ww = orc.route_table(logits, table, 23, nu, 1.5)
+    assert sorted(wsel.tolist()) != sorted(orc.route(logits, nu, 1.5)[0].tolist())
+    routed, _ = orc.moe_routed(gate, up, down, d, ff, wsel, ww, clamp, norm)
+    shared = orc.moe_shared(sg, su, sd, d, ff, clamp, norm)
+    want = (routed + shared).astype(np.float32)           # d4-ffn's last step (ds4f.lisp:980-992): the ordered sum, then the shared row
+    moe = ds4f.ffn_step_device(dev, pool, sh, lb, nb, ne, nu, 1.5, clamp, tid2eid=tb, tokens=kb)
+    got = hip.hip_floats(moe, d)
+    assert np.array_equal(bits(got), bits(want)), np.abs(got - want).max()
+    for b in (lb, tb, kb, nb, moe):
+        hip.hip_free(b)
+    pool.free(); sh.free()
+
+
 def test_route_with_nan_and_masked_scores(dev):
     """Scores that are NaN (an overflow upstream) and experts masked by a bias of minus infinity: the
     CPU's insertion (ds4f.lisp:966-972) compares NaNs false both ways, so its result depends on the

@@ -407,6 +407,48 @@ def test_route_against_stable_sort():
         assert abs(float(w.sum()) - 1.5) < 1e-5
 
 
+def test_route_from_the_hash_table():
+    """The hash layers' branch (ds4f.lisp:961-963): the token's row of tid2eid as it stands -- unsorted, the bias
+    ignored -- with the weights of the other branch.  Pinned three ways: an explicit numpy evaluation with every
+    rounding written out; a table row that IS the top-nu choice gives orc_route's output, which the stable sort
+    pins; and the misreadings (the row sorted by score, the biased scores in the weights) give other results."""
+    rng = synth.make_rng(17)
+    f32 = np.float32
+    for trial in range(40):
+        ne, nu = (256, 6) if trial % 2 else (16, 3)
+        ntok = 50
+        logits = rng.standard_normal(ne).astype(f32)
+        table = np.stack([rng.permutation(ne)[:nu] for _ in range(ntok)]).astype(np.int32)
+        token = int(rng.integers(0, ntok))
+        sel, w = orc.route_table(logits, table, token, nu, 1.5)
+        assert sel.tolist() == table[token].tolist()
+        p = np.array([np.sqrt(f32(orc.softplus(v))) for v in logits], f32)
+        tot = f32(0)
+        for i in table[token]:
+            tot = f32(tot + p[i])
+        tot = max(tot, f32(6.103515625e-5))
+        want = ((p[table[token]] / tot) * f32(1.5)).astype(f32)
+        assert np.array_equal(w.view(np.uint32), want.view(np.uint32))
+        # a row equal to the top-nu choice: the other branch's output, sum order included
+        tsel, tw = orc.route(logits, nu, 1.5)
+        table[token] = tsel
+        sel2, w2 = orc.route_table(logits, table, token, nu, 1.5)
+        assert sel2.tolist() == tsel.tolist() and np.array_equal(w2.view(np.uint32), tw.view(np.uint32))
+        # the row reversed: the same experts in the table's order, not by score
+        table[token] = tsel[::-1]
+        sel3, w3 = orc.route_table(logits, table, token, nu, 1.5)
+        assert sel3.tolist() == tsel[::-1].tolist()
+        assert np.allclose(w3[::-1], tw, rtol=1e-6)
+    # tiny probabilities: the sum is floored at 2^-14
+    logits = np.full(16, -40.0, f32)
+    sel, w = orc.route_table(logits, np.array([[3, 1, 2]], np.int32), 0, 3, 1.5)
+    p = np.sqrt(f32(orc.softplus(-40.0)))
+    assert np.array_equal(w, np.full(3, (p / f32(6.103515625e-5)) * f32(1.5), f32))
+    # an expert named twice stays twice (the table is taken as it stands)
+    sel, w = orc.route_table(rng.standard_normal(16).astype(f32), np.array([[5, 5, 2]], np.int32), 0, 3, 1.5)
+    assert sel.tolist() == [5, 5, 2] and w[0] == w[1]
+
+
 # ---- the experts ----------------------------------------------------------------------------------
 def _experts(rng, ne, d, ff):
     gate = synth.weights(synth.IQ2_XXS, ne * ff, d, rng)
