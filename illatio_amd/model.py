@@ -30,9 +30,9 @@ def synth_model(seed, d=2560, ffn=9728, nh=32, nkv=8, hd=128, nl=36, vocab=15193
         layers.append({"wq": (Q4_K, synth.weights(Q4_K, qd, d, rng)), "wk": (Q4_K, synth.weights(Q4_K, kvd, d, rng)),
                        "wv": (Q6_K, synth.weights(Q6_K, kvd, d, rng)), "wo": (Q4_K, synth.weights(Q4_K, d, qd, rng, dscale=0.0002)),
                        "gate": (Q4_K, synth.weights(Q4_K, ffn, d, rng)), "up": (Q4_K, synth.weights(Q4_K, ffn, d, rng)),
-                       "down": (Q6_K, synth.weights(Q6_K, d, ffn, rng, dscale=0.002)),
+                       "down": (Q6_K, synth.weights(Q6_K, d, ffn, rng, dscale=0.002 / 32.0)),
                        "attn_norm": norm(d), "ffn_norm": norm(d), "q_norm": norm(hd), "k_norm": norm(hd)})
-    embd = (Q6_K, synth.weights(Q6_K, vocab, d, rng, dscale=0.01 * head_scale))
+    embd = (Q6_K, synth.weights(Q6_K, vocab, d, rng, dscale=0.01 * head_scale / 32.0))
     return {"config": {"d": d, "ffn": ffn, "nh": nh, "nkv": nkv, "hd": hd, "nl": nl, "vocab": vocab, "eps": eps, "rope_base": rope_base,
                        "neox": True},
             "embd": embd, "output": embd, "output_norm": norm(d), "layers": layers}

@@ -338,10 +338,9 @@ def test_d4_mm_q8_0_grouped_attention_output_strided(dev, groups, rank, gdim, n)
         ds4f.dk_mm(dev, "d4_mm_q8_0", m.qs.at(g * rank * gdim), m.d.at(2 * g * rank * (gdim // 32)), 0, rank, gdim,
                    hb.at(4 * g * gdim), low.at(4 * g * rank), n, x_stride=groups * gdim, y_stride=rows)
     got = hip.hip_floats(low, n * rows).reshape(n, groups, rank)
-    rb = synth.row_bytes(synth.Q8_0, gdim)
     for g in range(groups):
         xg = np.ascontiguousarray(heads[:, g * gdim:(g + 1) * gdim])
-        wg = w[g * rank * rb:(g + 1) * rank * rb]
+        wg = np.ascontiguousarray(w[g * rank:(g + 1) * rank])
         want = orc.matmul(synth.Q8_0, wg, rank, gdim, xg, f16_scale=False, nthreads=8).reshape(n, rank)
         assert np.array_equal(bits(got[:, g]), bits(want)), (g, np.abs(got[:, g] - want).max())
     hip.hip_free(hb); hip.hip_free(low); m.free()
