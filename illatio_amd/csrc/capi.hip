@@ -763,6 +763,13 @@ int ilt_cvt_bf16(uint64_t stream, const float* x, uint16_t* xb, int64_t n) {
   return (int)ilt_k_cvt_bf16(x, xb, n, S(stream));
 }
 
+int ilt_q8k_bf16(uint64_t stream, const int8_t* xq, const float* xd, uint16_t* xb, int n, int cols, int slabs) {
+  ILT_REQUIRE(n >= 0 && cols > 0 && cols % 256 == 0);
+  if (n == 0) return ILT_OK;
+  ILT_REQUIRE(xq && xd && xb && ((uintptr_t)xq & 7) == 0 && ((uintptr_t)xb & 15) == 0);
+  return (int)ilt_k_q8k_bf16(xq, xd, xb, n, cols, slabs, S(stream));
+}
+
 int ilt_mm_k_bf16(uint64_t stream, int gguf_type, const void* w, const uint16_t* xb, float* y, const float* bias,
                   int rows, int cols, int n, int acc) {
   const int fmt = bf16_type(gguf_type);
@@ -1021,6 +1028,7 @@ int ilt_launch(const char* kernel, unsigned gx, unsigned gy, unsigned gz, unsign
   if (!strcmp(kernel, "mm_q4k_mma") || !strcmp(kernel, "mm_q6k_mma"))
     return ilt_mm_k(stream, kernel[4] == '4' ? 0 : 2, a.ptr<const void*>(0), a.ptr<ci8>(1), a.ptr<cf>(2),
                     a.ptr<const int32_t*>(3), a.ptr<float*>(4), a.ptr<cf>(5), a.i32(6), a.i32(7), a.i32(8), a.i32(9));
+  K("q8k_bf16") return ilt_q8k_bf16(stream, a.ptr<ci8>(0), a.ptr<cf>(1), a.ptr<uint16_t*>(2), a.i32(3), a.i32(4), a.i32(5));
   K("cvt_bf16") return ilt_cvt_bf16(stream, a.ptr<cf>(0), a.ptr<uint16_t*>(1), a.i64(2));
   K("mm_k_bf16") return ilt_mm_k_bf16(stream, a.i32(0), a.ptr<const void*>(1), a.ptr<cu16>(2), a.ptr<float*>(3), a.ptr<cf>(4),
                                       a.i32(5), a.i32(6), a.i32(7), a.i32(8));

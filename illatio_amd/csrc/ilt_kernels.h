@@ -175,6 +175,8 @@ hipError_t ilt_k_gemm_i8_id(int fmt, const uint64_t* ptrs, long long add, const 
 // of 8); weights dequantized to bf16 in LDS: Q4_K, Q6_K (212-byte device blocks), Q2_K,
 // IQ2_XXS.  Within 2e-2 of the CPU path.
 hipError_t ilt_k_cvt_bf16(const float* x, uint16_t* xb, long long n, hipStream_t st);
+// Q8_K quants times their block scales as bf16, n tokens of cols (a multiple of 256): rows of cols, or cvt_bf16_slabs' layout
+hipError_t ilt_k_q8k_bf16(const int8_t* xq, const float* xd, uint16_t* out, int n, int cols, int slabs, hipStream_t st);
 hipError_t ilt_k_gemm_bf16(int fmt, const uint8_t* w, long long row_bytes, int rows, int cols, const uint16_t* xb, int ntok,
                            float* y, const float* bias, int acc, hipStream_t st);
 hipError_t ilt_k_gemm_bf16_id(int fmt, const uint64_t* ptrs, long long add, const uint32_t* counts, const uint32_t* bases,

@@ -1793,6 +1793,43 @@ __global__ __launch_bounds__(256) void cvt_bf16_kernel(const float* __restrict__
   ((int4*)xb)[i] = make_int4(pack_bf16(a.x, a.y), pack_bf16(a.z, a.w), pack_bf16(b.x, b.y), pack_bf16(b.z, b.w));
 }
 
+// Q8_K activations (quantize-q8k!'s quants and block scales) as bf16: d * q, the value the CPU path's row dots
+// multiply the weights with, rounded to bf16 -- 8 quants a thread.  SLABS: into cvt_bf16_slabs' layout
+// (npad tokens written, zeros past n).
+template <bool SLABS>
+__global__ __launch_bounds__(256) void q8k_bf16_kernel(const i8* __restrict__ xq, const float* __restrict__ xd, u8* __restrict__ out, int n,
+                                                       long long npad, int cols) {
+  const long long i = (long long)blockIdx.x * 256 + threadIdx.x;      // rows: (token, 8 columns); slabs: (group, ks, token in group, piece)
+  long long tok; int c0; u8* dst;
+  if (SLABS) {
+    const int nk = cols / KS;
+    const int piece = (int)(i & 3), tl = (int)((i >> 2) % SLAB_ROWS);
+    const long long gk = i / (4 * SLAB_ROWS);
+    const int ks = (int)(gk % nk);
+    tok = (gk / nk) * SLAB_ROWS + tl; c0 = ks * KS + 8 * piece;
+    if (tok >= npad) return;
+    dst = out + slab_addr(tok, ks, nk) + 16 * piece;
+  } else {
+    const int per = cols / 8;
+    tok = i / per; c0 = (int)(i % per) * 8;
+    if (tok >= n) return;
+    dst = out + (tok * cols + c0) * 2;
+  }
+  int4 v = make_int4(0, 0, 0, 0);
+  if (tok < n) {
+    const int2 q = *(const int2*)(xq + tok * cols + c0);
+    const float d = xd[(tok * cols + c0) >> 8];
+    float f[8];
+#pragma unroll
+    for (int k = 0; k < 4; k++) {
+      f[k] = d * (float)(i8)((u32)q.x >> (8 * k));
+      f[4 + k] = d * (float)(i8)((u32)q.y >> (8 * k));
+    }
+    v = make_int4(pack_bf16(f[0], f[1]), pack_bf16(f[2], f[3]), pack_bf16(f[4], f[5]), pack_bf16(f[6], f[7]));
+  }
+  *(int4*)dst = v;
+}
+
 template <int FMT, int TM, int TN, int NB>
 hipError_t launch_bf16(const BfParams& p, long long token_tiles, hipStream_t st) {
   const long long total = token_tiles * ((p.rows + TM - 1) / TM), per = (total + 7) / 8;
@@ -1818,6 +1855,19 @@ hipError_t ilt_k_cvt_bf16(const float* x, uint16_t* xb, long long n, hipStream_t
   if (n <= 0) return hipSuccess;
   const long long n8 = n / 8;
   hipLaunchKernelGGL(cvt_bf16_kernel, dim3((unsigned)((n8 + 255) / 256)), dim3(256), 0, st, x, xb, n8);
+  return hipGetLastError();
+}
+
+hipError_t ilt_k_q8k_bf16(const int8_t* xq, const float* xd, uint16_t* out, int n, int cols, int slabs, hipStream_t st) {
+  if (n <= 0) return hipSuccess;
+  if (cols <= 0 || cols % 256 != 0) return hipErrorInvalidValue;
+  if (slabs) {
+    const long long npad = ((long long)n + 255) / 256 * 256, units = npad * (cols / 8);
+    hipLaunchKernelGGL(q8k_bf16_kernel<true>, dim3((unsigned)((units + 255) / 256)), dim3(256), 0, st, (const i8*)xq, xd, (u8*)out, n, npad, cols);
+  } else {
+    const long long units = (long long)n * (cols / 8);
+    hipLaunchKernelGGL(q8k_bf16_kernel<false>, dim3((unsigned)((units + 255) / 256)), dim3(256), 0, st, (const i8*)xq, xd, (u8*)out, n, (long long)n, cols);
+  }
   return hipGetLastError();
 }
 

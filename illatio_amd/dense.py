@@ -158,6 +158,16 @@ def cvt_bf16(dev, x, n_elems, out=None):
     return out
 
 
+def q8k_bf16(dev, act, n, out=None, slabs=False):
+    """ACT's Q8_K blocks of N tokens as bf16 -- each quant times its block's scale, the value the CPU path's row dots
+    see of the activation -- as rows (for CMAT-MUL-BF16) or in slabs (for MAT-MUL-BF16): the bf16 products then share
+    the CPU path's rounding of the activations to int8 blocks."""
+    nbytes = slabs_bytes(n, act.cols) if slabs else 2 * n * act.cols
+    out = out if out is not None else hip.hip_alloc(dev, nbytes, zero=False)
+    hip.launch(dev, "q8k_bf16", 1, 256, [act.kq, act.kd, out, n, act.cols, 1 if slabs else 0])
+    return out
+
+
 def cmat_mul_bf16(dev, w, xb, y, n, bias=None, acc=False):
     """Y = W X for N tokens on the bf16 matrix cores, XB a DBuf of N x COLS bf16 (CVT-BF16):
     no activation quantizer runs; within 2e-2 of CMAT-MUL's result rather than equal to it."""

@@ -18,20 +18,24 @@ from . import dense, hip, synth
 from .synth import Q4_K, Q6_K, Q8_0
 
 
-def synth_model(seed, d=2560, ffn=9728, nh=32, nkv=8, hd=128, nl=36, vocab=151936, eps=1e-6, rope_base=1e6, head_scale=8.0):
+def synth_model(seed, d=2560, ffn=9728, nh=32, nkv=8, hd=128, nl=36, vocab=151936, eps=1e-6, rope_base=1e6, head_scale=8.0, update_scale=1.0, attn_temp=1.0):
     """A seeded random-init dense decoder as numpy arrays: {"config", "embd", "output", "output_norm", "layers"}; a
     matrix is (GGUF type, uint8 rows).  HEAD_SCALE spreads the output head's logits so that the greedy token is not
-    decided in the last bits (random weights give nearly flat logits)."""
+    decided in the last bits (random weights give nearly flat logits).  UPDATE_SCALE multiplies the block scales of wo
+    and down, i.e. what a layer adds to the residual stream: at 1 a layer's update is some forty times the stream it
+    is added to, so every layer rewrites the stream (the hardest case for bit-exactness, and one where any rounding
+    difference grows about fivefold a layer); around 0.005 the stream dominates its updates, as in a trained model.  ATTN_TEMP multiplies the query heads' norm weights, i.e.
+    the attention's scores (at 1 they are about N(0, 1)).  Neither changes the values drawn at 1."""
     rng = synth.make_rng(seed)
     qd, kvd = nh * hd, nkv * hd
     norm = lambda n: (synth.activations(n, rng) * 0.1 + 1.0).astype(np.float32)
     layers = []
     for _ in range(nl):
         layers.append({"wq": (Q4_K, synth.weights(Q4_K, qd, d, rng)), "wk": (Q4_K, synth.weights(Q4_K, kvd, d, rng)),
-                       "wv": (Q6_K, synth.weights(Q6_K, kvd, d, rng)), "wo": (Q4_K, synth.weights(Q4_K, d, qd, rng, dscale=0.0002)),
+                       "wv": (Q6_K, synth.weights(Q6_K, kvd, d, rng)), "wo": (Q4_K, synth.weights(Q4_K, d, qd, rng, dscale=0.0002 * update_scale)),
                        "gate": (Q4_K, synth.weights(Q4_K, ffn, d, rng)), "up": (Q4_K, synth.weights(Q4_K, ffn, d, rng)),
-                       "down": (Q6_K, synth.weights(Q6_K, d, ffn, rng, dscale=0.002 / 32.0)),
-                       "attn_norm": norm(d), "ffn_norm": norm(d), "q_norm": norm(hd), "k_norm": norm(hd)})
+                       "down": (Q6_K, synth.weights(Q6_K, d, ffn, rng, dscale=0.002 / 32.0 * update_scale)),
+                       "attn_norm": norm(d), "ffn_norm": norm(d), "q_norm": (norm(hd) * attn_temp).astype(np.float32), "k_norm": norm(hd)})
     embd = (Q6_K, synth.weights(Q6_K, vocab, d, rng, dscale=0.01 * head_scale / 32.0))
     return {"config": {"d": d, "ffn": ffn, "nh": nh, "nkv": nkv, "hd": hd, "nl": nl, "vocab": vocab, "eps": eps, "rope_base": rope_base,
                        "neox": True},
@@ -78,8 +82,17 @@ def _mat(w):
 class DenseModel:
     """HOST (synth_model's dict, or the same made from a file's tensors) on DEV, with caches for NCTX positions."""
 
-    def __init__(self, dev, host, nctx, chunk=512):
+    def __init__(self, dev, host, nctx, chunk=512, prefill="exact"):
+        """PREFILL: how a chunk of several tokens is multiplied.  "exact": the int8 products, every token with the bits
+        of its own decode step (the CPU path's MATMUL!).  "bf16": the bf16 matrix-core products on the CPU path's own
+        quantized activations (each Q8_K quant times its block scale, rounded to bf16), K-quant matrices only: within
+        the bf16 roundings of the exact products, not equal to them.  "bf16-resident": the same numbers from bf16
+        copies of the matrices made once here and kept beside the quantized ones that decode reads (2 bytes a
+        weight).  One token always takes the decode products."""
         c = host["config"]
+        if prefill not in ("exact", "bf16", "bf16-resident"):
+            raise ValueError(f"prefill {prefill!r}: exact, bf16 or bf16-resident")
+        self.prefill = prefill
         self.dev, self.c, self.nctx, self.chunk, self.pos = dev, c, nctx, chunk, 0
         d, ffn, hd = c["d"], c["ffn"], c["hd"]
         self.qd, self.kvd = c["nh"] * hd, c["nkv"] * hd
@@ -116,6 +129,16 @@ class DenseModel:
                 for nm in names:
                     kinds.setdefault(cols, set()).add("q8k" if L[nm].kquant_p() else "q8")
         self.acts = {cols: dense.QAct(dev, n, cols, tuple(sorted(k))) for cols, k in kinds.items()}
+        self.xb, self.wb = {}, {}
+        if prefill != "exact":
+            if any("q8" in k for k in kinds.values()):
+                raise ValueError("the bf16 prefill multiplies K-quant matrices; this model has Q8_0 ones")
+            # a chunk's activations as bf16 per width (rows, or slabs for the resident copies' product)
+            self.xb = {cols: hip.hip_alloc(dev, dense.slabs_bytes(n, cols), zero=False) for cols in kinds}
+            if prefill == "bf16-resident":
+                for li, L in enumerate(self.layers):
+                    for nm in ("wq", "wk", "wv", "wo", "gate", "up", "down"):
+                        self.wb[(li, nm)] = dense.dequant_bf16(dev, L[nm])
         # the model as ilt_dense_decode reads it: a token's launches queued by one call
         ptr = lambda b: b.ptr if b is not None else 0
         self._clayers = (_Layer * len(self.layers))()
@@ -142,13 +165,29 @@ class DenseModel:
             self.pos += 1
             return self.logits
         dense.embed(dev, self.embd, self.tokens, self.x, n, d)
-        for L in self.layers:
+        fast = self.prefill != "exact" and n > 1
+        slabs = self.prefill == "bf16-resident"
+
+        def mul_fast(li, parts, act, acc=False):
+            """PARTS (name, y, bias) on ACT's Q8_K blocks taken as bf16."""
+            xb = dense.q8k_bf16(dev, act, n, out=self.xb[act.cols], slabs=slabs)
+            for nm, y, bias in parts:
+                w = self.layers[li][nm]
+                if slabs:
+                    dense.mat_mul_bf16(dev, self.wb[(li, nm)], w.rows, w.cols, xb, y, n, bias=bias, acc=acc)
+                else:
+                    dense.cmat_mul_bf16(dev, w, xb, y, n, bias=bias, acc=acc)
+
+        for li, L in enumerate(self.layers):
             if n == 1:
                 dense.qkv_mul(dev, L["wq"], L["wk"], L["wv"], None, self.q, self.k, self.v, L["bq"], L["bk"], L["bv"], xf=self.x,
                               norm=(L["attn_norm"], eps))
             else:
                 a = dense.rmsnorm_q8(dev, self.x, L["attn_norm"], self.acts[d], d, eps, n=n)
-                dense.cmat_mul_n(dev, [(L["wq"], self.q, L["bq"]), (L["wk"], self.k, L["bk"]), (L["wv"], self.v, L["bv"])], a, n)
+                if fast:
+                    mul_fast(li, [("wq", self.q, L["bq"]), ("wk", self.k, L["bk"]), ("wv", self.v, L["bv"])], a)
+                else:
+                    dense.cmat_mul_n(dev, [(L["wq"], self.q, L["bq"]), (L["wk"], self.k, L["bk"]), (L["wv"], self.v, L["bv"])], a, n)
             if n == 1 and self.scores is not None:
                 hip.call("ilt_attn_step", S, P(self.q), P(self.k), P(self.v), P(L["q_norm"]), P(L["k_norm"]), P(self.rope), P(L["kc"]), P(L["vc"]),
                          P(self.att), C.c_int(nh), C.c_int(nkv), C.c_int(hd), C.c_int(hd), C.c_int(self.pos), C.c_float(eps),
@@ -163,6 +202,11 @@ class DenseModel:
                 dense.mv_multi(dev, [(L["wo"], self.x, None)], xf=self.att, acc=True)
                 dense.glu_mul(dev, L["gate"], L["up"], None, self.fa, xf=self.x, norm=(L["ffn_norm"], eps))
                 dense.mv_multi(dev, [(L["down"], self.x, None)], xf=self.fa, acc=True)
+            elif fast:
+                mul_fast(li, [("wo", self.x, None)], dense.quantize_act(dev, self.att, self.acts[self.qd], n=n), acc=True)
+                mul_fast(li, [("gate", self.fa, None), ("up", self.fb, None)], dense.rmsnorm_q8(dev, self.x, L["ffn_norm"], self.acts[d], d, eps, n=n))
+                hip.call("ilt_swiglu", S, P(self.fa), P(self.fb), C.c_int64(n * ffn))
+                mul_fast(li, [("down", self.x, None)], dense.quantize_act(dev, self.fa, self.acts[ffn], n=n), acc=True)
             else:
                 dense.cmat_mul(dev, L["wo"], dense.quantize_act(dev, self.att, self.acts[self.qd], n=n), self.x, n=n, acc=True)
                 a = dense.rmsnorm_q8(dev, self.x, L["ffn_norm"], self.acts[d], d, eps, n=n)
@@ -221,3 +265,5 @@ class DenseModel:
             hip.hip_free(b)
         for a in self.acts.values():
             a.free()
+        for b in list(self.xb.values()) + list(self.wb.values()):
+            hip.hip_free(b)

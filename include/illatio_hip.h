@@ -451,6 +451,13 @@ int ilt_d4_mm_id_q2_k(uint64_t stream, int ncols, int nrows, int row_bytes, int6
      ptrs[z] + add_up, add_up >= add_gate) and d4_swiglu_w_bf16 in one launch: mid[i][r] for the
      groups' row i and r < nrows (a multiple of 128), the bits the three launches give. */
 int ilt_cvt_bf16(uint64_t stream, const float* x, uint16_t* xb, int64_t n);
+/* The bf16 products on the activations the CPU path multiplies with: quantize-q8k!'s quants times their block
+   scales (kquant.lisp:117-167; what q4k-row-dot and the others see of x), rounded to bf16, n tokens of cols (a
+   multiple of 256) -- as rows for mm_k_bf16 (slabs 0) or in cvt_bf16_slabs' layout for mm_bf16 (slabs 1).  With
+   these the bf16 path shares the CPU path's rounding of the activations to int8 blocks and differs from it by the
+   bf16 roundings alone.  No counterpart in the reference's CUDA path (its mm_*_mma kernels multiply integer
+   operands, kquant.cu:300-304). */
+int ilt_q8k_bf16(uint64_t stream, const int8_t* xq, const float* xd, uint16_t* xb, int n, int cols, int slabs);
 int ilt_mm_k_bf16(uint64_t stream, int gguf_type, const void* w, const uint16_t* xb, float* y, const float* bias,
                   int rows, int cols, int n, int acc);
 int ilt_cvt_bf16_slabs(uint64_t stream, const float* x, uint16_t* xs, int n, int cols);

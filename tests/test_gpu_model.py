@@ -366,3 +366,66 @@ def test_config_2_as_stated_36_layers_512_token_prompt_128_greedy_tokens(dev, ca
     assert same == 128
     say(f"128 greedy tokens, smallest top-1 margin {min(margins):.4f}, median {float(np.median(margins)):.4f}")
     assert min(margins) > 0
+
+
+def _logprobs(v):
+    v = v.astype(np.float64)
+    m = v.max()
+    return v - (m + np.log(np.exp(v - m).sum()))
+
+
+CHAOTIC = pytest.mark.skip(reason="on the default random-init model every layer rewrites the residual stream and the attention is sharp: "
+                              "measured, a prompt's K rows are 0.25 % (rms) from the CPU path's in layer 0, 2-9 % in layers 1-2 and 17 % in "
+                              "layer 3, the logits' top ten move by up to 4.7 in logprob within 16 greedy steps and the top-1 token differs "
+                              "at a step where the CPU path's two best are 0.67 apart (four layers, head_scale 8: step 7, 18 apart).  Not the "
+                              "bf16 roundings: any difference from the CPU path, however small, grows to the size of a Q8_K step within two "
+                              "layers, because the CPU path re-quantizes its activations before every product and a perturbed input rounds "
+                              "to other quants (rms sqrt(difference x step)); in this model nothing damps it afterwards")
+
+
+@pytest.mark.parametrize("prefill,damped", [("bf16", True), ("bf16-resident", True), pytest.param("bf16", False, marks=CHAOTIC)])
+def test_bf16_prefill_keeps_the_top_1_token_over_128_greedy_tokens(dev, prefill, damped, capsys):
+    """The prompt through the bf16 matrix-core products (on the CPU path's own quantized activations, each Q8_K quant
+    times its block scale rounded to bf16), then 128 greedy tokens through the exact decode products reading the
+    caches that prefill left: all 36 layers at config 2's width.  The bar is the reference's for its GPU path against
+    its CPU path (inspect/cuda-consistency-test.lisp:19-22, 40-47): at every step the top-1 token is the CPU path's, or
+    the two candidates lie closer than 0.1 in logprob (a near-tie), and no logprob among the top ten moves by 0.3.
+    Each step is fed the CPU path's token, so one step's difference does not hide the next ones'.
+    DAMPED: a random-init model conditioned as a trained one is -- a layer adds a fraction of the residual stream
+    (update_scale), the attention's scores are soft (attn_temp), the logits spread like a language model's (std 2.7
+    instead of 86) -- since the bar is in logprob and was set on trained checkpoints."""
+    from illatio_amd import hip, model
+    kw = dict(head_scale=0.25, update_scale=0.005, attn_temp=0.3) if damped else {}
+    host = model.synth_model(4, nl=36 if damped else 4, **kw)
+    c = host["config"]
+    nprompt, ndecode = 64, 128
+    rng = synth.make_rng(4)
+    prompt = rng.integers(0, c["vocab"], nprompt).tolist()
+    cpu = orc.DenseModel(host, nprompt + ndecode + 8)
+    for t in prompt[:-1]:
+        cpu.forward(t, logits=False, nthreads=16)
+    want, _ = cpu.forward(prompt[-1], nthreads=16)
+    gpu = model.DenseModel(dev, host, nprompt + ndecode + 8, chunk=64, prefill=prefill)
+    gpu.eval_tokens(prompt)
+    worst, differ = 0.0, 0
+    for step in range(ndecode + 1):
+        got = hip.hip_floats(gpu.logits, c["vocab"])
+        a, b = _logprobs(got), _logprobs(want)
+        top = np.argsort(-a)[:10]
+        worst = max(worst, float(np.abs(a[top] - b[top]).max()))
+        ga, wa = int(np.argmax(got)), int(np.argmax(want))
+        if ga != wa:
+            differ += 1
+            assert float(a[ga] - a[wa]) < 0.1, (step, float(a[ga] - a[wa]))
+        assert worst < 0.3, (step, worst)
+        if step == ndecode:
+            break
+        want, _ = cpu.forward(wa, nthreads=16)
+        gpu.forward_n([wa])
+        if step % 32 == 31:
+            with capsys.disabled():
+                print(f"  [{prefill} prefill] step {step + 1}: top-1 differs at {differ} steps so far, worst |dlogprob| {worst:.4f}", flush=True)
+    gpu.free()
+    with capsys.disabled():
+        print(f"  [{prefill} prefill] {ndecode} greedy tokens: top-1 differs at {differ} steps (near-ties), worst |dlogprob| in the top ten {worst:.4f}",
+              flush=True)
