@@ -540,7 +540,32 @@ def workload_c4(args, dev):
         return 0
 
     ms, dev_ms, per = tm.run(step, args.steps, args.warmup, probe_steps=10, work_of=work_of)
+    if ondev:
+        # the timed sequence itself (four launches queued by one call), the library recording an event before each of
+        # its launches and one behind the last: per launch, the median over 20 steps
+        import ctypes as C
+        evs = [hip.hip_event_create(dev, True) for _ in range(5)]
+        arr = (C.c_uint64 * 5)(*evs)
+        hip.call("ilt_d4_ffn_step_events", arr, C.c_int(5))
+        gaps = []
+        try:
+            for i in range(20):
+                ds4f.ffn_step_call(dev, pools[i % nlayers], shared[i % nlayers], logits[i % len(logits)], xb, moe_out, ne, nu, 1.5, 0.0, wsbuf=step_ws)
+                hip.hip_sync(dev)
+                gaps.append([hip.hip_event_elapsed_ms(evs[k], evs[k + 1]) for k in range(4)])
+        finally:
+            hip.call("ilt_d4_ffn_step_events", None, C.c_int(0))
+        for e in evs:
+            hip.hip_event_destroy(e)
+        med = np.median(np.array(gaps), axis=0)
+        names = ["d4_mvq8_glu+route", "d4_mv_glu_iq2_xxs", "d4_mv_q2_k_f32", "d4_mvq8+sum"]
+        works = [work_of("d4_mvq8_glu", [ff, d]), work_of("d4_mv_glu_iq2_xxs", None), work_of("d4_mv_q2_k_f32", None), work_of("d4_mvq8", [d, ff])]
+        per = {nm: [float(med[k]), works[k], 1] for k, nm in enumerate(names)}
     roof = roofline_of({k: v for k, v in per.items() if v[1]}, "hbm", HBM_PEAK_GBS, "GB/s",
+                       {"d4_mvq8_glu+route": "gemv_stream_kernel<8, 0> (shared expert's Q8_0 gate, up and gated activation; one of its waves routes the token)",
+                        "d4_mvq8+sum": "gemv_stream_kernel<8, 2> (shared expert's Q8_0 down, the step's ordered sum carried along)",
+                        "d4_mv_glu_iq2_xxs": "gemv_stream_kernel<16, 0> (the 6 selected experts' IQ2_XXS gate, up and gated activation, one launch)",
+                        "d4_mv_q2_k_f32": "gemv_stream_kernel<10, 0> (the 6 selected experts' Q2_K down)"} if ondev else
                        {"d4_mv_iq2_xxs": "gemv_kernel<16> (the 6 selected experts' IQ2_XXS gate and up, one launch over 12 matrices)",
                         "d4_mv_glu_iq2_xxs": "gemv_kernel<16> (the 6 selected experts' IQ2_XXS gate, up and gated activation, one launch)",
                         "d4_mv_q2_k": "gemv_kernel<10> (the 6 experts' Q2_K down)", "d4_mv_q2_k_f32": "gemv_kernel<10> (the 6 experts' Q2_K down)",
@@ -548,6 +573,8 @@ def workload_c4(args, dev):
     roof["launch_us_all"] = {k: round(v[0] / v[2] * 1e3, 2) for k, v in per.items()}
     dom = max((k for k in per if per[k][1]), key=lambda k: per[k][0])
     roof["traffic"] = TRAFFIC["c4"].get(dom)
+    if ondev:
+        roof["timed_by"] = "events the library records around each launch of the timed one-call step (an event pair adds about 2 us to a launch)"
     gbs = step_bytes / (ms * 1e-3) / 1e9
 
     def cpu():
@@ -587,7 +614,8 @@ def workload_c5(args, dev):
     norms = synth.activations((n, d), rng)
     logits = synth.zipf_router_logits(n, ne, rng)
     lb, nb = hip.hip_upload_new(dev, logits), hip.hip_upload_new(dev, norms)
-    sb = hip.hip_alloc(dev, 4 * n * d)
+    sb = hip.hip_alloc(dev, 4 * n * d)           # the rows the ordered sum ends with, zeros: configuration 5 states no shared expert (a chunk's
+                                                 # shared expert is ffn_shared_chunk's, timed with the decode step's in c4)
     rows = n * nu
     ws = hip.Workspace(dev, rows * (4 * d * 2 + 2 * d + 4 * ff * 3 + 2 * ff + d + ff + 4096) + 4 * n * d + (16 << 20))
     flops = 2.0 * rows * 3 * ff * d
@@ -683,6 +711,31 @@ def workload_c2d(args, dev):
     wbytes = sum(a[1].size for L in host["layers"] for k, a in L.items() if isinstance(a, tuple)) + host["output"][1].size
     ms = decode_s * 1e3 / ndecode
     m.free()
+    more = {}
+    if not q8:
+        # the same prompt through the bf16 matrix-core products (on the CPU path's quantized activations; within the
+        # bf16 roundings of the exact prefill, not equal to it), from the quantized matrices and from bf16 copies kept resident
+        for mode in ("bf16", "bf16-resident"):
+            mb = model.DenseModel(dev, host, nctx=nprompt + 8, chunk=512, prefill=mode)
+            mb.eval_tokens(prompt)
+            mb.reset()
+            hip.hip_sync(dev)
+            t0 = time.perf_counter()
+            mb.eval_tokens(prompt)
+            hip.hip_sync(dev)
+            more[f"prefill_{mode.replace('-', '_')}_tok_per_s"] = round(nprompt / (time.perf_counter() - t0), 1)
+            mb.free()
+        # the decode at a context past the one-launch attention's 1,024 positions: a 2,048-token prompt, 64 greedy tokens
+        ml = model.DenseModel(dev, host, nctx=2048 + 64 + 8, chunk=512)
+        long_prompt = rng.integers(0, c["vocab"], 2048).tolist()
+        ml.eval_tokens(long_prompt)
+        ml.decode_greedy(4)
+        hip.hip_sync(dev)
+        t0 = time.perf_counter()
+        ml.decode_greedy(60)
+        hip.hip_sync(dev)
+        more["decode_tok_per_s_at_2048_positions"] = round(60 / (time.perf_counter() - t0), 1)
+        ml.free()
 
     def cpu():
         import oracle_lib as orc
@@ -709,8 +762,8 @@ def workload_c2d(args, dev):
             "metric": "decode tok/s at Qwen2.5-0.5B shape" if q8 else "decode tok/s at Qwen3-4B shape",
             "config": {"workload": f"{'c1' if q8 else 'c2'} decode: {shape}-shape dense decoder, {nl} layers, random-init {'Q8_0' if q8 else 'Q4_K/Q6_K'}, {nprompt}-token prompt then "
                                    f"{ndecode}-token greedy decode at batch 1", "weight_bytes_per_token": int(wbytes)},
-            "extra": {"prefill_tok_per_s": round(nprompt / prefill_s, 1), "distinct_tokens_decoded": len(set(toks)),
-                      "weights_GBps_in_decode": round(wbytes / (ms * 1e-3) / 1e9, 1)},
+            "extra": {"prefill_tok_per_s": round(nprompt / prefill_s, 1), "distinct_tokens_decoded": len(set(toks)), "tokens_decoded": ndecode,
+                      "weights_GBps_in_decode": round(wbytes / (ms * 1e-3) / 1e9, 1), **more},
             "roofline": {"bound": "hbm", "achieved": round(wbytes / (ms * 1e-3) / 1e9, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                          "frac": round(wbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4), "traffic": None,
                          "kernel": "whole token: 5 launches a layer (Q/K/V, attention, wo, gate+up, down) + embedding + head + the "
@@ -800,7 +853,7 @@ def main():
                 out["prefill_tok_per_s"] = r["extra"]["prefill_tok_per_s"]
             out["configs"][name] = {
                 "workload": r["config"]["workload"], "value": r["value"], "unit": r["unit"], "ms_per_step": round(r["ms_per_step"], 4),
-                "steps": a.steps, "warmup": a.warmup, "dtype": r["dtype"], "extra": r["extra"],
+                "steps": r["extra"].get("tokens_decoded", a.steps), "warmup": a.warmup, "dtype": r["dtype"], "extra": r["extra"],
                 "roofline": {k: roof.get(k) for k in ("bound", "achieved", "peak", "unit", "frac", "traffic", "kernel", "launches", "avg_launch_us",
                                                       "launch_us_all", "other_kernels")}}
     print(json.dumps(out))

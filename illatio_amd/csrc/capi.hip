@@ -2,6 +2,7 @@
 // reference's src/cuda.lisp makes, typed entry points for the kernels, and launch by name.
 // Host code only validates shapes and picks launch geometry; it does no arithmetic on data (ilt_rope_table, a
 // model's constants, aside).
+#include <mutex>
 #include <hip/hip_runtime.h>
 #include <math.h>
 #include <stdint.h>
@@ -518,6 +519,14 @@ int shared_down_sum(uint64_t stream, int d, int ff, const int8_t* wq, const uint
   p.sum = {bd, (long long)d, nu};
   return (int)ilt_gemv_launch(p, 1, S(stream));
 }
+// A caller's events around the step's launches (ilt_d4_ffn_step_events): event i recorded on the stream before launch
+// i, the one after the last launch behind it.  Per thread; none by default.
+thread_local const uint64_t* g_step_events = nullptr;
+thread_local int g_step_nevents = 0, g_step_marked = 0;
+int step_mark(uint64_t stream) {
+  if (g_step_events && g_step_marked < g_step_nevents) ILT_TRY(hipEventRecord((hipEvent_t)g_step_events[g_step_marked++], S(stream)));
+  return ILT_OK;
+}
 // Five launches on STREAM, nothing allocated, freed or waited for; ws holds step_layout's bytes.
 int step_run(uint64_t stream, uint8_t* ws, int ne, int nu, int d, int ff, float scale, float clamp, const ilt_ffn_step_weights* wt,
              const float* logits, const float* bias, const float* x, float* moe) {
@@ -529,19 +538,34 @@ int step_run(uint64_t stream, uint8_t* ws, int ne, int nu, int d, int ff, float 
   // the routing rides along with the shared expert's gate/up launch (one of its waves routes while the rows stream
   // in); where that launch cannot take it, a launch of its own
   IltRouteAlong route = {logits, bias, sel, w, ne, nu, scale, 0};
+  g_step_marked = 0;
+  ILT_TRY((hipError_t)step_mark(stream));
   ILT_TRY((hipError_t)mvq8_glu(stream, ff, d, wt->sgate_q, wt->sgate_d, wt->sup_q, wt->sup_d, x, clamp, smid, &route));
   if (!route.done) ILT_TRY((hipError_t)ilt_d4_route(stream, ne, nu, 0, scale, bias ? 1 : 0, logits, bias, nullptr, nullptr, sel, w, 1));
+  ILT_TRY((hipError_t)step_mark(stream));
   ILT_TRY((hipError_t)ilt_d4_mv_glu_iq2_xxs(stream, d, ff, grb, 0, wt->gate_bytes, 0, ff, wt->slots, sel, nu, x, w, clamp, bm));
+  ILT_TRY((hipError_t)step_mark(stream));
   ILT_TRY((hipError_t)ilt_d4_mv_q2_k_f32(stream, ff, d, drb, 2 * wt->gate_bytes, ff, d, wt->slots, sel, nu, bm, bd));
+  ILT_TRY((hipError_t)step_mark(stream));
   // the shared expert's down product last, adding the routed experts' rows and its own as it stores them; where
   // that launch cannot (more than eight slots, a matrix too small for the streamed variant): the product, then the sum
-  const int e = shared_down_sum(stream, d, ff, wt->sdown_q, wt->sdown_d, smid, bd, nu, moe);
-  if (e != (int)hipErrorNotSupported) return e;
-  ilt_mv_desc down = {ILT_Q8_0, d, wt->sdown_q, wt->sdown_d, sout, nullptr};
-  ILT_TRY((hipError_t)ilt_mv_multi(stream, 1, &down, ff, nullptr, nullptr, nullptr, smid, 0, 0, 0));
-  return ilt_d4_moe_sum(stream, d, nu, bd, sout, moe, nullptr);
+  int e = shared_down_sum(stream, d, ff, wt->sdown_q, wt->sdown_d, smid, bd, nu, moe);
+  if (e == (int)hipErrorNotSupported) {
+    ilt_mv_desc down = {ILT_Q8_0, d, wt->sdown_q, wt->sdown_d, sout, nullptr};
+    ILT_TRY((hipError_t)ilt_mv_multi(stream, 1, &down, ff, nullptr, nullptr, nullptr, smid, 0, 0, 0));
+    e = ilt_d4_moe_sum(stream, d, nu, bd, sout, moe, nullptr);
+  }
+  if (e != ILT_OK) return e;
+  return step_mark(stream);
 }
 }  // namespace
+
+int ilt_d4_ffn_step_events(const uint64_t* events, int n) {
+  ILT_REQUIRE(n >= 0 && n <= 8 && (n == 0 || events));
+  g_step_events = n ? events : nullptr;
+  g_step_nevents = n;
+  return ILT_OK;
+}
 
 uint64_t ilt_d4_ffn_step_workspace(int nu, int d, int ff) {
   if (nu < 1 || d < 1 || ff < 1 || nu > 64 || d > (1 << 20) || ff > (1 << 20)) return 0;
@@ -688,14 +712,22 @@ int ilt_d4_mm_id_q2_k(uint64_t stream, int ncols, int nrows, int row_bytes, int6
 // The reference's kernels round weights and activations to halves; these quantize the activations as the CPU
 // path does and run the exact products, so the quantized activations need room: a buffer per device that only
 // ever grows, kept until the process ends.  Calls that overlap on one GPU (two streams) would share it: the
-// reference's host issues these on one stream.
+// reference's host issues these on one stream.  Growing frees and allocates, which waits for the device and cannot
+// happen while a stream is being captured: a caller that captures, or that wants no such stall in its loop, sizes
+// the buffer once beforehand (ilt_d4_mm_reserve).  The bookkeeping is guarded; the buffer itself is one per device.
 namespace {
 struct QRoom { void* p; size_t bytes; };
 QRoom g_qroom[ILT_MAX_DEVICES];
+std::mutex g_qroom_mu;
+size_t qroom_bytes(int fmt, size_t ntok, size_t ncols) {
+  const size_t n = ntok * ncols, bw = fmt == ILT_Q8_0 ? 32 : 256;
+  return (n + 255) / 256 * 256 + (n / bw * 4 + 255) / 256 * 256 + (fmt == ILT_Q8_0 ? 0 : (n / 16 * 4 + 255) / 256 * 256);
+}
 int qroom(size_t bytes, uint8_t** out) {
   int dev = -1;
   ILT_TRY(hipGetDevice(&dev));
   ILT_REQUIRE(dev >= 0 && dev < ILT_MAX_DEVICES);
+  std::lock_guard<std::mutex> lock(g_qroom_mu);
   QRoom& q = g_qroom[dev];
   if (q.bytes < bytes) {
     if (q.p) ILT_TRY(hipFree(q.p));                      // (waits for the work that still reads it)
@@ -733,6 +765,12 @@ int d4_mm_quantized(uint64_t stream, int fmt, int ncols, int nrows, int ntok, in
   return (int)ilt_k_gemm_i8(fmt, (const uint8_t*)w, nullptr, row_bytes, nrows, ncols, xq, xs, bs, ntok, y, nullptr, 0, S(stream), y_stride);
 }
 }  // namespace
+
+int ilt_d4_mm_reserve(int ntok, int ncols) {
+  ILT_REQUIRE(ntok >= 0 && ncols >= 0);
+  uint8_t* room = nullptr;
+  return qroom(qroom_bytes(ILT_Q2_K, (size_t)ntok, (size_t)ncols), &room);       // the K formats' layout is the larger one
+}
 
 int ilt_d4_mm_q8_0(uint64_t stream, int ncols, int nrows, int ntok, int row_bytes, int x_stride, int y_stride, const int8_t* w,
                    const uint16_t* wd, const float* x, float* y) {
@@ -857,9 +895,17 @@ int ilt_qk_rope(uint64_t stream, float* q, float* k, const float* v, const float
 // ilt_qk_rope and ilt_attn_rows for one token at position pos, as two launches instead of three (the first one
 // norms and turns the heads where it needs them and writes the caches' rows); q and k are left as they came
 int ilt_attn_step(uint64_t stream, const float* q, const float* k, const float* v, const float* qn, const float* kn, const float* rope, float* kc,
-                  float* vc, float* out, int nh, int nkv, int hd, int rd, int pos, float eps, int neox, float* scratch) {
-  ILT_REQUIRE(q && k && v && rope && kc && vc && out && scratch && nh > 0 && nkv > 0 && pos >= 0 && pos < 8192);
+                  float* vc, float* out, int nh, int nkv, int hd, int rd, int pos, float eps, int neox, float* scratch, int nctx) {
+  // pos < nctx: the caches' rows at pos are written (kc, vc hold nctx rows); 8192: what the tiled values kernel takes
+  ILT_REQUIRE(q && k && v && rope && kc && vc && out && scratch && nh > 0 && nkv > 0 && pos >= 0 && pos < nctx && pos < 8192);
   return (int)ilt_k_attn_step(q, k, v, qn, kn, rope, kc, vc, out, nh, nkv, hd, rd, pos, eps, neox, scratch, S(stream));
+}
+int ilt_attn_giveups(uint64_t* out) {
+  ILT_REQUIRE(out);
+  unsigned long long v = 0;
+  ILT_TRY(ilt_k_attn_giveups(&v));
+  *out = v;
+  return ILT_OK;
 }
 // ARGMAX (model.lisp:464-468) of n floats on the device: the index into out[0] (device memory), so that a greedy
 // decode can go on without the logits' trip to the host (the reference picks the token on the host, cuda-dense.lisp:428-430)
@@ -901,7 +947,7 @@ static int dec_build_qkv(DecLaunch& Q, const ilt_dense_model* m, const ilt_dense
   return dec_build(Q, 3, qkv, m->d, m->x, L.attn_norm, m->eps, 0, 0);
 }
 int ilt_dense_decode(uint64_t stream, const ilt_dense_model* m, const int32_t* token, int pos, int want_logits) {
-  ILT_REQUIRE(m && token && m->layers && m->nl > 0 && pos >= 0 && pos < 8192);
+  ILT_REQUIRE(m && token && m->layers && m->nl > 0 && pos >= 0 && pos < m->nctx && pos < 8192);
   ILT_REQUIRE(m->x && m->q && m->k && m->v && m->att && m->fa && m->scores && m->rope && (!want_logits || (m->logits && m->output_norm)));
   int e;
   if (m->embd.gguf_type == ILT_TYPE_Q8_0) e = ilt_embed_q8(stream, (const int8_t*)m->embd.w, m->embd.wd, token, m->x, m->d, 1);
@@ -941,7 +987,7 @@ int ilt_dense_decode(uint64_t stream, const ilt_dense_model* m, const int32_t* t
         if ((e = ilt_mv_multi_norm(stream, 1, &d3[i], m->d, m->x, L.attn_norm, m->eps, 0, 1, 0))) return e;
     }
     if ((e = ilt_attn_step(stream, m->q, m->k, m->v, L.q_norm, L.k_norm, m->rope, L.kc, L.vc, m->att, m->nh, m->nkv, m->hd, m->rd, pos, m->eps,
-                           m->neox, m->scores))) return e;
+                           m->neox, m->scores, m->nctx))) return e;
     // gate/up's launch reads down's rows ahead: it is the one launch long enough after its own rows are in (the terms
     // of both matrices' rows, two sums a row and the gated activation) for the next matrix to arrive meanwhile.  The
     // other links of the chain -- Q/K/V reading wo's rows ahead, wo gate/up's, down the next layer's Q/K/V's -- lengthen
@@ -1053,7 +1099,7 @@ int ilt_launch(const char* kernel, unsigned gx, unsigned gy, unsigned gz, unsign
   K("argmax") return ilt_argmax(stream, a.ptr<cf>(0), a.i32(1), a.ptr<int32_t*>(2), a.ptr<void*>(3));
   K("attn_step") return ilt_attn_step(stream, a.ptr<cf>(0), a.ptr<cf>(1), a.ptr<cf>(2), a.ptr<cf>(3), a.ptr<cf>(4), a.ptr<cf>(5), a.ptr<float*>(6),
                                       a.ptr<float*>(7), a.ptr<float*>(8), a.i32(9), a.i32(10), a.i32(11), a.i32(12), a.i32(13), a.f32(14), a.i32(15),
-                                      a.ptr<float*>(16));
+                                      a.ptr<float*>(16), a.i32(17));
   K("d4_rows_expert") return ilt_d4_rows_expert(stream, a.i32(0), a.ptr<cu32>(1), a.ptr<cu32>(2), a.ptr<uint32_t*>(3));
   K("d4_mm_q8_0") return ilt_d4_mm_q8_0(stream, a.i32(0), a.i32(1), a.i32(2), a.i32(3), a.i32(4), a.i32(5), a.ptr<ci8>(6), a.ptr<cu16>(7), a.ptr<cf>(8), a.ptr<float*>(9));
   K("d4_mm_f16") return ilt_d4_mm_f16(stream, a.i32(0), a.i32(1), a.i32(2), a.i32(3), a.i32(4), a.i32(5), a.ptr<cu16>(6), a.ptr<cf>(8), a.ptr<float*>(9));

@@ -201,6 +201,7 @@ hipError_t ilt_k_qk_rope(float* q, float* k, const float* v, const float* qn, co
 hipError_t ilt_k_argmax(const float* v, int n, int* out, void* scratch, hipStream_t st);
 hipError_t ilt_k_attn_step(const float* q, const float* k, const float* v, const float* qn, const float* kn, const float* rope, float* kc,
                            float* vc, float* out, int nh, int nkv, int hd, int rd, int pos, float eps, int neox, float* scratch, hipStream_t st);
+hipError_t ilt_k_attn_giveups(unsigned long long* out);
 hipError_t ilt_k_attn_rows(const float* q, const float* kc, const float* vc, float* out, int nh, int nkv, int hd, int pos0, int ntok,
                            float* scratch, hipStream_t st);
 hipError_t ilt_k_swiglu_rows(float* a, const float* b, long long n, hipStream_t st);

@@ -7,6 +7,7 @@
 // partial sums meet in its own order, dense.cu:364-373).
 #include "ilt_device.h"
 #include <atomic>
+#include <mutex>
 #include "ilt_kernels.h"
 #include <stdlib.h>
 
@@ -577,15 +578,28 @@ __global__ __launch_bounds__(256) void attn_values_kernel(const float* __restric
 // advances the generation as it ends (every workgroup read it as it started, microseconds earlier), so a launch
 // replayed from a graph finds new tags; the host's count tells apart launches that overlap on one GPU, which make each
 // other give up (they share the buffer) but do not read each other's scores.  (24 bits of generation: a word left in
-// the buffer could pass for a fresh one only if it was written exactly 2^24 launches of its head earlier.)
-__device__ unsigned attn_gen[256];
-__device__ unsigned long long attn_xrow[256 * 1024];
+// the buffer could pass for a fresh one only if it was written exactly 2^24 - 1 launches of its head earlier.)
+// A workgroup that gives up writes its own words over with a tag no launch uses (generation 0xFFFFFF is skipped),
+// so that what it wrote under a generation its partners did not share -- it started after its head's first workgroup
+// had ended and read the advanced generation -- cannot pass for fresh in a later launch that reaches that generation
+// with the same count of launches (the same captured launch replayed), and it counts itself in attn_giveups.
+// Launches overlap on a GPU only across streams, so each stream gets a buffer of its own (kAttnSlots of them; the
+// streams past that share the last one): two decoders on one GPU do not make each other give up.
+// What sharing out relies on, beyond its tests: consecutive workgroups go to the eight dies in turn, and a head's
+// workgroups are resident together (256 workgroups of 1,024 threads: one a CU on an otherwise idle GPU).  Where either
+// fails the cost is the wait (PATIENCE, 200 us a launch), not the result.
+constexpr int kAttnSlots = 8;
+constexpr unsigned kAttnNoGen = 0xFFFFFFu;
+__device__ unsigned attn_gen[kAttnSlots][256];
+__device__ unsigned long long attn_xrow[kAttnSlots][256 * 1024];
+__device__ unsigned long long attn_giveups;
 template <int NJ, int CS>
 __global__ __launch_bounds__(1024) void attn_step_fused_kernel(const float* __restrict__ q, const float* __restrict__ k, const float* __restrict__ v,
                                                                const float* __restrict__ qn, const float* __restrict__ kn,
                                                                const float* __restrict__ rope, float* __restrict__ kc, float* __restrict__ vc,
                                                                float* __restrict__ out, int nh, int nkv, int rd, int pos, float eps, int neox,
-                                                               float scale, int vpitch, int share, unsigned epoch, int patience) {
+                                                               float scale, int vpitch, int share, unsigned epoch, int patience,
+                                                               unsigned* __restrict__ xgen, unsigned long long* __restrict__ xrow) {
   extern __shared__ __align__(16) float dyn[];
   __shared__ float qsh[16 * NJ], ksh[16 * NJ], redf[16];
   __shared__ double scs[2], redd[17];
@@ -619,8 +633,8 @@ __global__ __launch_bounds__(1024) void attn_step_fused_kernel(const float* __re
   const bool split = share != 0;
   // (the head's generation, read now and wanted after the heads are turned: the barrier there hands it round)
   if (split && tid == 0) {
-    const unsigned gen = (__hip_atomic_load(&attn_gen[h], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + 1) & 0xFFFFFFu;
-    tag_sh = gen << 8 | (epoch & 15u) << 4;
+    const unsigned gen = ((__hip_atomic_load(&xgen[h], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) & 0xFFFFFFu) + 1) % kAttnNoGen;
+    tag_sh = gen << 8 | (epoch & 31u) << 3;
     got_all = 1;
   }
   if (split) {
@@ -677,8 +691,8 @@ __global__ __launch_bounds__(1024) void attn_step_fused_kernel(const float* __re
   const int nb = (npos + 255) >> 8;                // 1 .. 4
   bool shared = false;
   if (split) {
-    const unsigned die = __builtin_amdgcn_s_getreg((4 - 1) << 11 | 20) & 15u, tag = tag_sh | die;
-    unsigned long long* const row = attn_xrow + (long long)h * 1024;
+    const unsigned die = __builtin_amdgcn_s_getreg((4 - 1) << 11 | 20) & 7u, tag = tag_sh | die;
+    unsigned long long* const row = xrow + (long long)h * 1024;
 #pragma unroll
     for (int i = 0; i < NPASS; i++) {
       const int p = 64 * (cs + ns * i) + pg;
@@ -703,7 +717,7 @@ __global__ __launch_bounds__(1024) void attn_step_fused_kernel(const float* __re
       for (;;) {
         w = __hip_atomic_load(row + tid, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         const unsigned t = (unsigned)(w >> 32);
-        if ((t ^ tag) >> 4 == 0) { ok = (t & 15u) == die; break; }
+        if ((t ^ tag) >> 3 == 0) { ok = (t & 7u) == die; break; }
         if (wall_clock64() - t0 >= (long long)patience) break;
         __builtin_amdgcn_s_sleep(1);
       }
@@ -715,6 +729,15 @@ __global__ __launch_bounds__(1024) void attn_step_fused_kernel(const float* __re
     load_slice();
     ilt_barrier_lds();
     shared = got_all != 0;
+    if (!shared) {
+      // giving up: this workgroup's words made unmatchable (see above), and the give-up counted
+#pragma unroll
+      for (int i = 0; i < NPASS; i++) {
+        const int p = 64 * (cs + ns * i) + pg;
+        if (l == 0 && p < npos) row[p] = ~0ull;
+      }
+      if (tid == 0) atomicAdd(&attn_giveups, 1ull);
+    }
   }
   if (!shared) {
     if (split) { load_keys(ka, 0); load_keys(kb, 1); }
@@ -770,7 +793,7 @@ __global__ __launch_bounds__(1024) void attn_step_fused_kernel(const float* __re
   // The head's first workgroup advances the generation as it ends: every workgroup of this launch read it as it
   // started, many microseconds ago (one that starts only now finds the new one, matches no flag and takes all the scores
   // itself).  A store: a counter of readers would be a read-modify-write whose answer a workgroup waits 2 us for.
-  if (split && tid == 0 && cs == 0) __hip_atomic_store(&attn_gen[h], tag_sh >> 8, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  if (split && tid == 0 && cs == 0) __hip_atomic_store(&xgen[h], tag_sh >> 8, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 // The same for contexts whose value slice no longer fits LDS (2,049 to 8,192 positions): the slice comes through
@@ -1003,6 +1026,39 @@ hipError_t ilt_k_attn_rows(const float* q, const float* kc, const float* vc, flo
   return hipGetLastError();
 }
 
+// The exchange buffers of stream ST on device DEV: the device arrays' addresses (asked of the runtime once a device) and
+// the stream's slot -- its own while fewer than kAttnSlots streams have asked on this device, else the last one, shared.
+static hipError_t attn_exchange_of(int dev, hipStream_t st, unsigned** xgen, unsigned long long** xrow) {
+  struct PerDev { unsigned* gen; unsigned long long* row; unsigned long long* giveups; hipStream_t streams[kAttnSlots]; int n; };
+  static PerDev devs[64] = {};
+  static std::mutex mu;
+  std::lock_guard<std::mutex> lock(mu);
+  PerDev& d = devs[dev];
+  if (!d.gen) {
+    void *g = nullptr, *r = nullptr, *c = nullptr;
+    hipError_t e = hipGetSymbolAddress(&g, HIP_SYMBOL(attn_gen));
+    if (e == hipSuccess) e = hipGetSymbolAddress(&r, HIP_SYMBOL(attn_xrow));
+    if (e == hipSuccess) e = hipGetSymbolAddress(&c, HIP_SYMBOL(attn_giveups));
+    if (e != hipSuccess) return e;
+    d.gen = (unsigned*)g; d.row = (unsigned long long*)r; d.giveups = (unsigned long long*)c;
+  }
+  int slot = -1;
+  for (int i = 0; i < d.n; i++) if (d.streams[i] == st) { slot = i; break; }
+  if (slot < 0) {
+    if (d.n < kAttnSlots) { slot = d.n; d.streams[d.n++] = st; }
+    else slot = kAttnSlots - 1;
+  }
+  *xgen = d.gen + slot * 256;
+  *xrow = d.row + (long long)slot * 256 * 1024;
+  return hipSuccess;
+}
+
+// Workgroups of the one-launch attention that gave up waiting for their partners' scores, on the current device, since
+// the library was loaded (waits for the device's work).
+hipError_t ilt_k_attn_giveups(unsigned long long* out) {
+  return hipMemcpyFromSymbol(out, HIP_SYMBOL(attn_giveups), sizeof(unsigned long long), 0, hipMemcpyDeviceToHost);
+}
+
 // One token at position pos: qk_rope and attention in two launches instead of three
 hipError_t ilt_k_attn_step(const float* q, const float* k, const float* v, const float* qn, const float* kn, const float* rope, float* kc,
                            float* vc, float* out, int nh, int nkv, int hd, int rd, int pos, float eps, int neox, float* scratch, hipStream_t st) {
@@ -1034,12 +1090,17 @@ hipError_t ilt_k_attn_step(const float* q, const float* k, const float* v, const
     const int patience = sp && sp[0] == '2' ? 0 : 20000;       // 200 us
     static std::atomic<unsigned> launches{0};
     const unsigned epoch = ++launches;
+    unsigned* xgen = nullptr; unsigned long long* xrow = nullptr;
+    if (split) {
+      const hipError_t e = attn_exchange_of(dev, st, &xgen, &xrow);
+      if (e != hipSuccess) return e;
+    }
     if (hd == 64)
       hipLaunchKernelGGL((attn_step_fused_kernel<4, 16>), dim3(nwg), dim3(1024), fsmem, st, q, k, v, qn, kn, rope, kc, vc, out, nh, nkv, rd, pos, eps,
-                         neox, scale, vpitch, split ? 1 : 0, epoch, patience);
+                         neox, scale, vpitch, split ? 1 : 0, epoch, patience, xgen, xrow);
     else
       hipLaunchKernelGGL((attn_step_fused_kernel<8, 16>), dim3(nwg), dim3(1024), fsmem, st, q, k, v, qn, kn, rope, kc, vc, out, nh, nkv, rd, pos, eps,
-                         neox, scale, vpitch, split ? 1 : 0, epoch, patience);
+                         neox, scale, vpitch, split ? 1 : 0, epoch, patience, xgen, xrow);
     return hipGetLastError();
   }
   hipLaunchKernelGGL(attn_step_scores_kernel, dim3(nh, (ctx + 255) / 256), dim3(1024), 0, st, q, k, v, qn, kn, rope, kc, vc, scratch, nh, nkv, hd, rd,

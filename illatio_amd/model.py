@@ -70,7 +70,7 @@ class _Layer(C.Structure):
 
 
 class _Model(C.Structure):
-    _fields_ = [(n, C.c_int) for n in ("nl", "d", "ffn", "nh", "nkv", "hd", "rd", "neox")] + [("eps", C.c_float), ("embd", _Mat), ("output", _Mat),
+    _fields_ = [(n, C.c_int) for n in ("nl", "d", "ffn", "nh", "nkv", "hd", "rd", "neox", "nctx")] + [("eps", C.c_float), ("embd", _Mat), ("output", _Mat),
                ("output_norm", C.c_uint64), ("rope", C.c_uint64), ("layers", C.POINTER(_Layer))] + \
                [(n, C.c_uint64) for n in ("x", "q", "k", "v", "att", "fa", "scores", "logits")]
 
@@ -146,7 +146,7 @@ class DenseModel:
             self._clayers[i] = _Layer(ptr(L["attn_norm"]), ptr(L["q_norm"]), ptr(L["k_norm"]), ptr(L["ffn_norm"]),
                                       *[_mat(L[n]) for n in ("wq", "wk", "wv", "wo", "gate", "up", "down")], L["kc"].ptr, L["vc"].ptr,
                                       ptr(L["bq"]), ptr(L["bk"]), ptr(L["bv"]))
-        self._cmodel = _Model(len(self.layers), d, ffn, c["nh"], c["nkv"], hd, hd, 1 if c["neox"] else 0, c["eps"], _mat(self.embd), _mat(self.output),
+        self._cmodel = _Model(len(self.layers), d, ffn, c["nh"], c["nkv"], hd, hd, 1 if c["neox"] else 0, nctx, c["eps"], _mat(self.embd), _mat(self.output),
                               self.output_norm.ptr, self.rope.ptr, self._clayers, self.x.ptr, self.q.ptr, self.k.ptr, self.v.ptr, self.att.ptr,
                               self.fa.ptr, ptr(self.scores), self.logits.ptr)
         self.one_call = self.scores is not None       # False: a token's launches one by one from here (the same launches)
@@ -191,7 +191,7 @@ class DenseModel:
             if n == 1 and self.scores is not None:
                 hip.call("ilt_attn_step", S, P(self.q), P(self.k), P(self.v), P(L["q_norm"]), P(L["k_norm"]), P(self.rope), P(L["kc"]), P(L["vc"]),
                          P(self.att), C.c_int(nh), C.c_int(nkv), C.c_int(hd), C.c_int(hd), C.c_int(self.pos), C.c_float(eps),
-                         C.c_int(1 if c["neox"] else 0), P(self.scores))
+                         C.c_int(1 if c["neox"] else 0), P(self.scores), C.c_int(self.nctx))
             else:
                 hip.call("ilt_qk_rope", S, P(self.q), P(self.k), P(self.v), P(L["q_norm"]), P(L["k_norm"]), P(self.rope), P(L["kc"]), P(L["vc"]),
                          C.c_int(nh), C.c_int(nkv), C.c_int(hd), C.c_int(hd), C.c_int(self.pos), C.c_float(eps), C.c_int(1 if c["neox"] else 0),

@@ -253,6 +253,10 @@ typedef struct ilt_ffn_step_weights {
 uint64_t ilt_d4_ffn_step_workspace(int nu, int d, int ff);
 int ilt_d4_ffn_step(uint64_t stream, void* ws, uint64_t ws_bytes, int ne, int nu, int d, int ff, float scale, float clamp,
                     const ilt_ffn_step_weights* wt, const float* logits, const float* bias, const float* x, float* moe);
+/* Measurement only (no counterpart in the reference): the calling thread's next ilt_d4_ffn_step calls record
+   events[i] (ilt_event_create's handles, n <= 8) on the stream before their launch i and the one after their last
+   launch behind it, so that a bench can time the step's launches as the step queues them; n = 0 switches it off. */
+int ilt_d4_ffn_step_events(const uint64_t* events, int n);
 
 /* ilt_d4_ffn_step without a workspace and without any allocation.  No counterpart in the
    reference: it is for callers that cannot allocate device memory or keep a workspace alive --
@@ -327,9 +331,13 @@ int ilt_attn_rows(uint64_t stream, const float* q, const float* kc, const float*
    (correct, slower).  Otherwise two: the
    launch that takes the scores norms and turns the query heads and the token's key and writes the caches' rows at
    pos.  Either way out is what ilt_attn_rows gives after ilt_qk_rope, bit for bit; q and k are left as they came
-   (not normed, not turned).  scratch: nh * ((pos + 4) & ~3) floats. */
+   (not normed, not turned).  scratch: nh * ((pos + 4) & ~3) floats.  nctx: the rows kc and vc hold; pos at or past
+   it is refused (the caches' rows at pos are written).  Each stream's launches exchange through a buffer of their
+   own (the first eight streams of a device; the rest share one); ilt_attn_giveups counts the workgroups that gave
+   an exchange up since the library was loaded (a diagnostic: such a launch is correct and about 200 us longer). */
 int ilt_attn_step(uint64_t stream, const float* q, const float* k, const float* v, const float* qn, const float* kn, const float* rope, float* kc,
-                  float* vc, float* out, int nh, int nkv, int hd, int rd, int pos, float eps, int neox, float* scratch);
+                  float* vc, float* out, int nh, int nkv, int hd, int rd, int pos, float eps, int neox, float* scratch, int nctx);
+int ilt_attn_giveups(uint64_t* out);
 
 /* One token through the whole dense decoder in one call: what the host loop of cuda-forward-n queues for one
    token (cuda-dense.lisp:380-432; the CPU's forward-1, model.lisp:396-462) -- embedding row, then per layer the
@@ -356,6 +364,7 @@ typedef struct ilt_dense_layer {
 } ilt_dense_layer;
 typedef struct ilt_dense_model {
   int nl, d, ffn, nh, nkv, hd, rd, neox;
+  int nctx;                                                   /* rows of every layer's kc and vc: a token at or past it is refused */
   float eps;
   ilt_dense_mat embd, output;
   const float *output_norm, *rope;
@@ -397,9 +406,14 @@ int ilt_mm_k_n(uint64_t stream, int type, const void* w0, float* y0, const float
    q2_k, iq2_xxs: quantize-q8k!, then the exact product (the row dots of iquant.lisp:126-215);
    f16 (the router, ds4f.lisp:1175 f32mm!): floats, every dot added up in F32-DOT16's order
      (tensor.lisp:370-378), bit for bit; ncols a multiple of 16.
-   The quantized formats take x_stride = ncols and y_stride = nrows only (hipErrorNotSupported, 801,
-   otherwise) and keep their quantized activations in a buffer inside the library that grows to the largest
-   chunk seen (per GPU, until the process ends; calls that overlap on one GPU share it). */
+   x_stride >= ncols and y_stride >= nrows: the reference passes them for the grouped attention output product,
+   one call a group on a slice of each token's heads into a slice of its low row, w and wd at offsets into
+   their arrays (cuda-ds4f-prefill.lisp:277-281); the K formats want x_stride a multiple of 4.
+   The quantized formats keep their quantized activations in a buffer inside the library that grows to the
+   largest chunk seen (per GPU, until the process ends; calls that overlap on one GPU share it).  Growing frees
+   and allocates: ilt_d4_mm_reserve(ntok, ncols) sizes it beforehand for chunks of up to ntok tokens of ncols
+   columns, after which calls within that size allocate nothing (callers under stream capture need this). */
+int ilt_d4_mm_reserve(int ntok, int ncols);
 int ilt_d4_mm_q8_0(uint64_t stream, int ncols, int nrows, int ntok, int row_bytes, int x_stride, int y_stride, const int8_t* w,
                    const uint16_t* wd, const float* x, float* y);
 int ilt_d4_mm_f16(uint64_t stream, int ncols, int nrows, int ntok, int row_bytes, int x_stride, int y_stride, const uint16_t* w,

@@ -298,6 +298,9 @@ def test_d4_mm_on_float_rows_bit_exact(dev, qtype, rows, cols, n):
         wq, wd, rb = m.qs, m.d, 0
     else:
         wq, wd, rb = hip.hip_upload_new(dev, w), None, synth.row_bytes(qtype, cols)
+    if qtype == synth.Q2_K:                                   # the library's room for the quantized rows sized beforehand
+        import ctypes as C
+        hip.call("ilt_d4_mm_reserve", C.c_int(n), C.c_int(cols))
     for ntok in (n, max(1, n // 3), n):
         x = synth.activations((ntok, cols), rng)
         x[0, :32] = 0.0

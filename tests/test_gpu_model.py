@@ -99,7 +99,7 @@ def test_attn_step_is_qk_rope_then_attn_rows(dev, norms, nh, nkv, hd):
             dq, dk, dv, kc, vc, out = up(q), up(k), up(v), up(kc0), up(vc0), hip.hip_alloc(dev, 4 * nh * hd)
             ints = (C.c_int(nh), C.c_int(nkv), C.c_int(hd), C.c_int(hd), C.c_int(pos), C.c_float(eps), C.c_int(1))
             if fused:
-                hip.call("ilt_attn_step", S, P(dq), P(dk), P(dv), P(qn), P(kn), P(rope), P(kc), P(vc), P(out), *ints, P(scratch))
+                hip.call("ilt_attn_step", S, P(dq), P(dk), P(dv), P(qn), P(kn), P(rope), P(kc), P(vc), P(out), *ints, P(scratch), C.c_int(nctx))
                 assert np.array_equal(bits(hip.hip_floats(dq, nh * hd)), bits(q)) and np.array_equal(bits(hip.hip_floats(dk, nkv * hd)), bits(k))
             else:
                 hip.call("ilt_qk_rope", S, P(dq), P(dk), P(dv), P(qn), P(kn), P(rope), P(kc), P(vc), *ints, C.c_int(1))
@@ -110,6 +110,13 @@ def test_attn_step_is_qk_rope_then_attn_rows(dev, norms, nh, nkv, hd):
         for a, b, what in zip(res[0], res[1], ("out", "kc", "vc")):
             assert np.array_equal(bits(a), bits(b)), (pos, what)
         assert not np.array_equal(res[0][1], kc0.ravel())         # the key's row was written
+    # a position the caches have no row for is refused
+    dq, dk, dv, kc, vc, out = up(f(nh * hd)), up(f(nkv * hd)), up(f(nkv * hd)), up(kc0), up(vc0), hip.hip_alloc(dev, 4 * nh * hd)
+    with pytest.raises(hip.HipError):
+        hip.call("ilt_attn_step", S, P(dq), P(dk), P(dv), P(qn), P(kn), P(rope), P(kc), P(vc), P(out), C.c_int(nh), C.c_int(nkv), C.c_int(hd),
+                 C.c_int(hd), C.c_int(nctx), C.c_float(eps), C.c_int(1), P(scratch), C.c_int(nctx))
+    for b in (dq, dk, dv, kc, vc, out):
+        hip.hip_free(b)
     for b in (rope, qn, kn, scratch):
         hip.hip_free(b)
 
@@ -135,7 +142,7 @@ def test_attn_step_replayed_from_a_graph(dev):
     dq, dk, dv, kc, vc, out = up(q), up(k), up(v), up(kc0), up(vc0), hip.hip_alloc(dev, 4 * nh * hd)
     ints = (C.c_int(nh), C.c_int(nkv), C.c_int(hd), C.c_int(hd), C.c_int(pos), C.c_float(eps), C.c_int(1))
     S = C.c_uint64(dev.stream)
-    step = lambda: hip.call("ilt_attn_step", S, P(dq), P(dk), P(dv), P(qn), P(kn), P(rope), P(kc), P(vc), P(out), *ints, P(scratch))
+    step = lambda: hip.call("ilt_attn_step", S, P(dq), P(dk), P(dv), P(qn), P(kn), P(rope), P(kc), P(vc), P(out), *ints, P(scratch), C.c_int(nctx))
     step()                                             # once outside the graph: the kernel's attributes are set on its first launch
     hip.hip_sync(dev)
     graph, gexec = C.c_void_p(), C.c_void_p()
@@ -324,9 +331,53 @@ def test_one_launch_attention_scores_shared_out(dev, monkeypatch):
                 monkeypatch.delenv("ILT_ATTN_SPLIT", raising=False)
             else:
                 monkeypatch.setenv("ILT_ATTN_SPLIT", mode)
+            before = _giveups()
             for nprompt, ndecode in ((70, 6), (250, 10), (764, 6), (1018, 8)) if mode is None else ((250, 10), (1018, 8)):
                 same, _ = run_greedy(dev, host, nprompt=nprompt, ndecode=ndecode, chunk=512, nctx=nprompt + ndecode + 2, seed=seed + nprompt)
                 assert same == ndecode, (hd, mode, nprompt)
+            # the library counts the workgroups that gave an exchange up: none where a head's workgroups find each other
+            # (a slowdown of 200 us a launch could otherwise hide behind correct results), every one of them where told to
+            gave_up = _giveups() - before
+            assert (gave_up == 0) if mode is None else (gave_up > 0) if mode == "2" else (gave_up == 0), (hd, mode, gave_up)
+
+
+def _giveups():
+    import ctypes as C
+    from illatio_amd import hip
+    n = C.c_uint64(0)
+    hip.call("ilt_attn_giveups", C.byref(n))
+    return n.value
+
+
+def test_two_decoders_on_two_streams_do_not_make_each_other_give_up(dev):
+    """Two decoders stepping at once on one GPU, each on a stream of its own: the one-launch attention's exchange goes
+    through a buffer per stream, so neither gives an exchange up (each step would take 200 us longer if they did),
+    and both decode the tokens they decode alone."""
+    from illatio_amd import hip, model
+    host = model.synth_model(51, d=256, ffn=512, nh=8, nkv=2, hd=64, nl=2, vocab=500)
+    rng = synth.make_rng(51)
+    prompt = rng.integers(0, 500, 300).tolist()
+    alone = model.DenseModel(dev, host, 340)
+    alone.eval_tokens(prompt)
+    want = alone.decode_greedy(24)
+    alone.free()
+    import ctypes as C
+    info = hip.DeviceInfo()
+    hip.call("ilt_device_get_info", C.c_int(dev.index), C.byref(info))
+    other = hip.Device(dev.index, info, hip.hip_stream_create(dev))
+    a, b = model.DenseModel(dev, host, 340), model.DenseModel(other, host, 340)
+    a.eval_tokens(prompt); b.eval_tokens(prompt)
+    hip.hip_sync(dev); hip.hip_stream_sync(other.stream)
+    before = _giveups()
+    got_a, got_b = [], []
+    for _ in range(24):                                       # a token of each queued before either is waited for
+        ta, tb = a.argmax(), b.argmax()
+        got_a.append(ta); got_b.append(tb)
+        a.forward_n([ta]); b.forward_n([tb])
+    hip.hip_sync(dev); hip.hip_stream_sync(other.stream)
+    assert got_a == want and got_b == want
+    assert _giveups() == before
+    a.free(); b.free()
 
 
 def test_config_2_width_four_layers_128_greedy_tokens(dev):
