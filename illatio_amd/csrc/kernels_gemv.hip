@@ -722,14 +722,19 @@ __global__ __launch_bounds__(kThreads) void gemv_kernel(IltGemvParams p) {
     const u8* w0 = p.ptrs ? (const u8*)(p.ptrs[p.sel ? p.sel[z] : z] + m.add) : m.w;
     if (FSET != 0 || m.fmt == ILT_Q4_K) first_load<(FSET ? FSET : ILT_Q4_K)>(pre.a, w0, m.wd, row0, nrows, S, m.row_bytes, lane);
     else first_load<(FSET ? FSET : ILT_Q6_K)>(pre.b, w0, m.wd, row0, nrows, S, m.row_bytes, lane);
-    // and a touch of every 64-byte line of the batch's first 16 KB, so the later steps hit in L2
+    // and a touch of every 64-byte line of the batch's first 16 KB, so the later steps hit in L2 -- where the touched
+    // lines of all the grid's waves together fit the dies' L2s (32 MB): in a launch of thousands of waves (the output
+    // head: 64 MB touched at once) most are evicted again before their wave reads them, and the matrix is then
+    // fetched 1.12 times over
     const u8* wb = w0 + row0 * m.row_bytes;
     const long bytes = (long)nrows * m.row_bytes;
     // (the values are looked at only when the kernel ends: nothing waits for these loads here)
+    if ((long)nw * 16384 <= (24L << 20)) {
 #pragma unroll
-    for (int i = 0; i < 4; i++) {
-      const long o = 64L * lane + 4096L * i;
-      if (o < bytes) warm[i] = *(const int*)(wb + (o & ~3L));
+      for (int i = 0; i < 4; i++) {
+        const long o = 64L * lane + 4096L * i;
+        if (o < bytes) warm[i] = *(const int*)(wb + (o & ~3L));
+      }
     }
   }
 
