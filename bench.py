@@ -49,25 +49,36 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 sys.path.insert(0, os.path.join(ROOT, "tests"))
 
-# HBM bytes per launch of the product kernels, from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE
-# (KiB per dispatch; the tables at the end of each file under profiles/): FETCH_SIZE reads 0.500 of what a plain streaming
-# kernel of known size fetches (cvt_bf16: 83,886,080 bytes read, counter 40,971 KiB), WRITE_SIZE
-# reads 1.000 (same kernel: 41,943,040 bytes written, counter 40,960 KiB); so bytes =
-# (2 * FETCH_SIZE + WRITE_SIZE) * 1024.
+# HBM bytes per launch of the product kernels, from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE (KiB per dispatch), as
+# profiles/hbm_traffic_per_launch.md lists them (its header says how its rows were measured): FETCH_SIZE reads 0.500 of
+# what a plain streaming kernel of known size fetches (cvt_bf16: 83,886,080 bytes read, counter 40,971 KiB), WRITE_SIZE
+# reads 1.000 (same kernel: 41,943,040 bytes written, counter 40,960 KiB); so bytes = (2 * FETCH_SIZE + WRITE_SIZE) * 1024.
+# The counters sit between a die's L2 and the fabric: bytes that come from the memory-side cache count like bytes from HBM.
 def _t(fetch_kib, write_kib):
     return int((2 * fetch_kib + write_kib) * 1024)
 
 
-TRAFFIC = {"c1": {"up": _t(2507.3, 96.0), "down": _t(2443.0, 28.0)},
-           "c2": {"qkv": _t(4935.6, 96.0), "wo": _t(3043.9, 80.0), "glu": _t(14065.8, 116.0), "down": _t(10506.2, 80.0),
-                  "head": _t(175546.1, 636.4)},
-           # one product: two-pass = the 256-tile launch plus the 128-tile launch for the rows left over
-           "c3": {"bf16-1pass": _t(519803.0, 278528.0), "bf16-2pass": _t(491863.8 + 61498.0, 262144.0 + 16384.0),
-                  "bf16-resident": _t(491863.8 + 61498.0, 262144.0 + 16384.0), "int8": _t(466661.6, 278528.0),
-                  "int8-2pass": _t(941922.8, 278528.0), "int8-resident": _t(941922.8, 278528.0)},
-           "c4": {"d4_mv_glu_iq2_xxs": _t(12854.8, 96.0), "d4_mv_q2_k_f32": _t(8394.5, 96.0), "d4_mvq8_glu": _t(8833.8, 96.0)},
-           # per launch, over the step's two grouped launches (gate + up + activation; down)
-           "c5": {"mm_id": _t((578091.8 + 335996.1) / 2, (98304.6 + 393216.0) / 2)}}
+def load_traffic(path=os.path.join(ROOT, "profiles", "hbm_traffic_per_launch.md")):
+    """{workload: {launch: bytes}} from the table's rows `| workload | launch | kernel | FETCH_SIZE KiB | WRITE_SIZE KiB |`
+    (several kernels of one launch shape: their rows add up)."""
+    t = {}
+    try:
+        for line in open(path):
+            cells = [c.strip() for c in line.strip().strip("|").split("|")]
+            if len(cells) < 5 or cells[0] in ("workload", "") or set(cells[0]) <= set("-: "):
+                continue
+            try:
+                b = _t(float(cells[3]), float(cells[4]))
+            except ValueError:
+                continue
+            w = t.setdefault(cells[0], {})
+            w[cells[1]] = w.get(cells[1], 0) + b
+    except OSError:
+        pass
+    return t
+
+
+TRAFFIC = load_traffic()
 
 
 def traffic_of(workload, per):
@@ -442,7 +453,7 @@ def workload_c3(args, dev):
     ms, dev_ms, per = tm.run(step, args.steps, args.warmup)
     roof = roofline_of({k: v for k, v in per.items() if k == "mm"}, "mfma", MFMA_PEAK_TFLOPS[args.path], "TFLOP/s" if bf16_path else "TOP/s", names)
     roof["unit"] = "TFLOP/s"
-    if path in TRAFFIC["c3"] and T == 4096 and not args.transpose and args.qtype == "q6_k":
+    if path in TRAFFIC.get("c3", {}) and T == 4096 and not args.transpose and args.qtype == "q6_k":
         roof["traffic"] = TRAFFIC["c3"][path]
     tf = flops / (ms * 1e-3) / 1e12
 
@@ -572,7 +583,7 @@ def workload_c4(args, dev):
                         "d4_mvq8": "gemv_kernel<8> (shared expert, Q8_0)", "d4_mvq8_glu": "gemv_kernel<8> (shared expert gate, up, gated activation)"})
     roof["launch_us_all"] = {k: round(v[0] / v[2] * 1e3, 2) for k, v in per.items()}
     dom = max((k for k in per if per[k][1]), key=lambda k: per[k][0])
-    roof["traffic"] = TRAFFIC["c4"].get(dom)
+    roof["traffic"] = TRAFFIC.get("c4", {}).get(dom)
     if ondev:
         roof["timed_by"] = "events the library records around each launch of the timed one-call step (an event pair adds about 2 us to a launch)"
     gbs = step_bytes / (ms * 1e-3) / 1e9
@@ -644,7 +655,8 @@ def workload_c5(args, dev):
                         else "gemm_i8p_kernel<16> (d4_mm_id_iq2_xxs x2) + <10> (d4_mm_id_q2_k): scale * quant as int8 planes, grouped, bit-exact with the CPU path"})
     roof["launch_us_all"] = {k: round(v[0] / v[2] * 1e3, 2) for k, v in per.items()}
     if args.path == "bf16" and n == 4096:
-        roof["traffic"] = TRAFFIC["c5"]["mm_id"]
+        t5 = TRAFFIC.get("c5", {})
+        roof["traffic"] = int(sum(t5.values()) / len(t5)) if t5 else None       # per launch, over the step's two grouped launches
     tf = flops / (ms * 1e-3) / 1e12
 
     def cpu():
