@@ -1095,6 +1095,21 @@ int ilt_launch(const char* kernel, unsigned gx, unsigned gy, unsigned gz, unsign
   K("qk_rope") return ilt_qk_rope(stream, a.ptr<float*>(0), a.ptr<float*>(1), a.ptr<cf>(2), a.ptr<cf>(3), a.ptr<cf>(4), a.ptr<cf>(5), a.ptr<float*>(6),
                                   a.ptr<float*>(7), a.i32(8), a.i32(9), a.i32(10), a.i32(11), a.i32(12), a.f32(13), a.i32(14), (int)gy);
   K("swiglu") return ilt_swiglu(stream, a.ptr<float*>(0), a.ptr<cf>(1), a.i64(2));
+  // The reference's attention launches by their names and slots (cuda-dense.lisp:341-364; dense.cu:376, 482, 517, 727),
+  // computed in the CPU's float order: attn_decode leaves one token's finished heads in PART (its split of the keys and
+  // its partial sums have no counterpart here: chunk, nsplit and scale are read past), attn_merge moves them to ATT and
+  // quantizes them for a Q8_0 output projection when XQ is given; attn_prefill / attn_prefill2 are a chunk's attn_rows.
+  K("attn_decode") return ilt_attn_rows(stream, a.ptr<cf>(0), a.ptr<cf>(1), a.ptr<cf>(2), a.ptr<float*>(3), a.i32(4), a.i32(5), a.i32(6), a.i32(7), 1, nullptr);
+  K("attn_merge") {
+    const int nh = a.i32(5), hd = a.i32(6), ntok = gy ? (int)gy : 1;
+    ILT_REQUIRE(a.ptr<cf>(0) && a.ptr<float*>(1) && nh > 0 && hd > 0 && (long long)nh * hd % 32 == 0);
+    const uint64_t bytes = 4ull * nh * hd * ntok;
+    ILT_TRY((hipError_t)ilt_memcpy_dtod_async((uint64_t)(uintptr_t)a.ptr<float*>(1), (uint64_t)(uintptr_t)a.ptr<cf>(0), bytes, stream));
+    if (!a.ptr<int8_t*>(2)) return ILT_OK;
+    return ilt_quant_q8(stream, a.ptr<cf>(1), a.ptr<int8_t*>(2), a.ptr<float*>(3), a.ptr<int32_t*>(4), (int64_t)nh * hd * ntok / 32);
+  }
+  if (!strcmp(kernel, "attn_prefill") || !strcmp(kernel, "attn_prefill2"))
+    return ilt_attn_rows(stream, a.ptr<cf>(0), a.ptr<cf>(1), a.ptr<cf>(2), a.ptr<float*>(3), a.i32(4), a.i32(5), a.i32(6), a.i32(7), a.i32(8), nullptr);
   K("attn_rows") return ilt_attn_rows(stream, a.ptr<cf>(0), a.ptr<cf>(1), a.ptr<cf>(2), a.ptr<float*>(3), a.i32(4), a.i32(5), a.i32(6), a.i32(7), (int)gy, a.ptr<float*>(8));
   K("argmax") return ilt_argmax(stream, a.ptr<cf>(0), a.i32(1), a.ptr<int32_t*>(2), a.ptr<void*>(3));
   K("attn_step") return ilt_attn_step(stream, a.ptr<cf>(0), a.ptr<cf>(1), a.ptr<cf>(2), a.ptr<cf>(3), a.ptr<cf>(4), a.ptr<cf>(5), a.ptr<float*>(6),

@@ -121,6 +121,43 @@ def test_attn_step_is_qk_rope_then_attn_rows(dev, norms, nh, nkv, hd):
         hip.hip_free(b)
 
 
+def test_the_reference_attention_names_launch(dev):
+    """attn_decode + attn_merge and attn_prefill / attn_prefill2 by the reference's names and argument lists
+    (cuda-dense.lisp:341-364): the heads they leave are attn_rows' -- the CPU's float order -- and attn_merge's
+    quantized copy is quant_q8's of them."""
+    from illatio_amd import hip
+    nh, nkv, hd, nctx = 8, 2, 64, 300
+    rng = synth.make_rng(21)
+    f = lambda *sh: (rng.standard_normal(sh) * 1.5).astype(np.float32)
+    up = lambda a: hip.hip_upload_new(dev, a)
+    kc, vc = up(f(nctx, nkv * hd)), up(f(nctx, nkv * hd))
+    scale = float(1.0 / np.sqrt(hd))
+    # one token at position 200
+    q = up(f(nh * hd))
+    part, att, want = (hip.hip_alloc(dev, 4 * nh * (hd + 2) * 8) for _ in range(3))
+    xq, xs, xsum = hip.hip_alloc(dev, nh * hd), hip.hip_alloc(dev, 4 * nh * hd // 32), hip.hip_alloc(dev, 4 * nh * hd // 32)
+    hip.launch(dev, "attn_decode", (nkv, 4), 128, [q, kc, vc, part, nh, nkv, hd, 200, 64, 4, scale], shared=4096)
+    hip.launch(dev, "attn_merge", (nh, 1), 64, [part, att, xq, xs, xsum, nh, hd, 200, 64, 4])
+    hip.launch(dev, "attn_rows", (nh, 1), 256, [q, kc, vc, want, nh, nkv, hd, 200, None])
+    w = hip.hip_floats(want, nh * hd)
+    assert np.array_equal(bits(hip.hip_floats(att, nh * hd)), bits(w))
+    wq, ws_, wsum = hip.hip_alloc(dev, nh * hd), hip.hip_alloc(dev, 4 * nh * hd // 32), hip.hip_alloc(dev, 4 * nh * hd // 32)
+    hip.launch(dev, "quant_q8", 1, 256, [want, wq, ws_, wsum, hip.I64(nh * hd // 32)])
+    for got, ref, dt, n in ((xq, wq, np.int8, nh * hd), (xs, ws_, np.float32, nh * hd // 32), (xsum, wsum, np.int32, nh * hd // 32)):
+        assert np.array_equal(hip.hip_download(got, dt, n), hip.hip_download(ref, dt, n))
+    # a chunk of 37 tokens at positions 100..136, both names
+    n = 37
+    qn = up(f(n, nh * hd))
+    for name, extra in (("attn_prefill2", []), ("attn_prefill", [4])):
+        out, ref = hip.hip_alloc(dev, 4 * n * nh * hd), hip.hip_alloc(dev, 4 * n * nh * hd)
+        hip.launch(dev, name, (nh, 1), 256, [qn, kc, vc, out, nh, nkv, hd, 100, n, scale] + extra, shared=8192)
+        hip.launch(dev, "attn_rows", (nh, n), 256, [qn, kc, vc, ref, nh, nkv, hd, 100, None])
+        assert np.array_equal(bits(hip.hip_floats(out, n * nh * hd)), bits(hip.hip_floats(ref, n * nh * hd))), name
+        hip.hip_free(out); hip.hip_free(ref)
+    for b in (kc, vc, q, part, att, want, xq, xs, xsum, wq, ws_, wsum, qn):
+        hip.hip_free(b)
+
+
 def test_attn_step_replayed_from_a_graph(dev):
     """The one-launch attention with the scores shared out keeps its flags' generation on the device: a launch captured
     into a HIP graph and replayed (new q, k, v each time, the program's own copies and waits between the replays) gives
