@@ -118,7 +118,9 @@ class DenseModel:
         self.x, self.q, self.k, self.v = A(4 * n * d), A(4 * n * self.qd), A(4 * n * self.kvd), A(4 * n * self.kvd)
         self.att, self.fa, self.fb = A(4 * n * self.qd), A(4 * n * ffn), A(4 * n * ffn)
         self.tokens = A(4 * n)
-        self.scores = A(4 * n * c["nh"] * ((nctx + 3) // 4 * 4)) if nctx <= 8192 else None      # the attention's raw scores
+        # the attention's raw scores, for the positions the kernels that keep them in memory take (up to 8192); past
+        # those a token's attention runs as one launch with its scores in LDS
+        self.scores = A(4 * n * c["nh"] * ((min(nctx, 8192) + 3) // 4 * 4))
         self.logits = A(4 * c["vocab"])
         # a chunk's quantized activations per width, in the formats the matrices that read that width take
         # (Q8_0 blocks for Q8_0 matrices, Q8_K blocks for K-quants, as the CPU path makes them)
@@ -149,7 +151,7 @@ class DenseModel:
         self._cmodel = _Model(len(self.layers), d, ffn, c["nh"], c["nkv"], hd, hd, 1 if c["neox"] else 0, nctx, c["eps"], _mat(self.embd), _mat(self.output),
                               self.output_norm.ptr, self.rope.ptr, self._clayers, self.x.ptr, self.q.ptr, self.k.ptr, self.v.ptr, self.att.ptr,
                               self.fa.ptr, ptr(self.scores), self.logits.ptr)
-        self.one_call = self.scores is not None       # False: a token's launches one by one from here (the same launches)
+        self.one_call = True                          # False: a token's launches one by one from here (the same launches)
 
     def forward_n(self, tokens, logits=True):
         """TOKENS at the next positions (CUDA-FORWARD-N); the last one's logits, if LOGITS, into self.logits."""
@@ -160,7 +162,8 @@ class DenseModel:
         S = C.c_uint64(dev.stream)
         P = lambda b, off=0: C.c_uint64(b.ptr + off if b is not None else 0)
         hip.hip_upload_vector(self.tokens, np.asarray(tokens, np.int32))
-        if n == 1 and self.one_call:
+        scratch = self.scores if self.pos + n <= 8192 else None
+        if n == 1 and self.one_call and scratch is not None:
             hip.call("ilt_dense_decode", S, C.byref(self._cmodel), P(self.tokens), C.c_int(self.pos), C.c_int(1 if logits else 0))
             self.pos += 1
             return self.logits
@@ -188,7 +191,7 @@ class DenseModel:
                     mul_fast(li, [("wq", self.q, L["bq"]), ("wk", self.k, L["bk"]), ("wv", self.v, L["bv"])], a)
                 else:
                     dense.cmat_mul_n(dev, [(L["wq"], self.q, L["bq"]), (L["wk"], self.k, L["bk"]), (L["wv"], self.v, L["bv"])], a, n)
-            if n == 1 and self.scores is not None:
+            if n == 1 and scratch is not None:
                 hip.call("ilt_attn_step", S, P(self.q), P(self.k), P(self.v), P(L["q_norm"]), P(L["k_norm"]), P(self.rope), P(L["kc"]), P(L["vc"]),
                          P(self.att), C.c_int(nh), C.c_int(nkv), C.c_int(hd), C.c_int(hd), C.c_int(self.pos), C.c_float(eps),
                          C.c_int(1 if c["neox"] else 0), P(self.scores), C.c_int(self.nctx))
@@ -197,7 +200,7 @@ class DenseModel:
                          C.c_int(nh), C.c_int(nkv), C.c_int(hd), C.c_int(hd), C.c_int(self.pos), C.c_float(eps), C.c_int(1 if c["neox"] else 0),
                          C.c_int(n))
                 hip.call("ilt_attn_rows", S, P(self.q), P(L["kc"]), P(L["vc"]), P(self.att), C.c_int(nh), C.c_int(nkv), C.c_int(hd),
-                         C.c_int(self.pos), C.c_int(n), P(self.scores))
+                         C.c_int(self.pos), C.c_int(n), P(scratch))
             if n == 1:
                 dense.mv_multi(dev, [(L["wo"], self.x, None)], xf=self.att, acc=True)
                 dense.glu_mul(dev, L["gate"], L["up"], None, self.fa, xf=self.x, norm=(L["ffn_norm"], eps))
@@ -223,7 +226,7 @@ class DenseModel:
         """NTOKENS greedy tokens after what the context holds, the first one picked from self.logits: every token picked
         on the device (ilt_argmax) and fed to the next step from device memory, nothing waited for until the ids are
         read back at the end.  Returns the ids; self.logits holds the logits after the last of them."""
-        if not self.one_call:
+        if not self.one_call or self.pos + ntokens > 8192:
             raise ValueError("the device-side loop runs over ilt_dense_decode (contexts up to 8192 positions)")
         if self.pos + ntokens > self.nctx:
             raise ValueError(f"{ntokens} more tokens at position {self.pos}: the context holds {self.nctx}")

@@ -344,6 +344,50 @@ def test_small_decoder_long_contexts(dev):
     assert same == 3
 
 
+def test_decode_across_position_8192(dev):
+    """A context longer than the 8,192 positions the kernels with their scores in memory take: tokens at positions 8,190
+    and 8,191 go through ilt_dense_decode (tiled values), those at 8,192 and 8,193 through qk_rope + attn_rows with the
+    scores in LDS, all with the oracle's logits bit for bit.  The caches' first 8,190 rows are filled with the same
+    random keys and values on both sides instead of running a prompt that long through the oracle."""
+    from illatio_amd import hip, model
+    host = model.synth_model(61, d=256, ffn=512, nh=4, nkv=2, hd=64, nl=2, vocab=300)
+    c = host["config"]
+    nctx, pos0, kvd = 8200, 8190, c["nkv"] * c["hd"]
+    rng = synth.make_rng(61)
+    cpu = orc.DenseModel(host, nctx)
+    gpu = model.DenseModel(dev, host, nctx, chunk=16)
+    for li in range(c["nl"]):
+        k, v = synth.activations((pos0, kvd), rng), synth.activations((pos0, kvd), rng)
+        cpu.kc[li, :pos0], cpu.vc[li, :pos0] = k, v
+        hip.hip_upload_vector(gpu.layers[li]["kc"], k)
+        hip.hip_upload_vector(gpu.layers[li]["vc"], v)
+    cpu.pos = gpu.pos = pos0
+    tok = 17
+    for step in range(4):
+        want, _ = cpu.forward(tok, nthreads=16)
+        gpu.forward_n([tok])
+        got = hip.hip_floats(gpu.logits, c["vocab"])
+        assert np.array_equal(bits(got), bits(want)), (pos0 + step, np.abs(got - want).max())
+        tok = int(np.argmax(want))
+    assert gpu.pos == 8194
+    # a chunk that ends past 8,192 positions: the same fallback, the caches' rows as decode leaves them
+    cpu2, gpu2 = orc.DenseModel(host, nctx), model.DenseModel(dev, host, nctx, chunk=16)
+    for li in range(c["nl"]):
+        cpu2.kc[li, :pos0], cpu2.vc[li, :pos0] = cpu.kc[li, :pos0], cpu.vc[li, :pos0]
+        hip.hip_upload_vector(gpu2.layers[li]["kc"], cpu.kc[li, :pos0])
+        hip.hip_upload_vector(gpu2.layers[li]["vc"], cpu.vc[li, :pos0])
+    cpu2.pos = gpu2.pos = pos0
+    toks = [5, 6, 7, 8, 9]
+    for t in toks[:-1]:
+        cpu2.forward(t, logits=False, nthreads=16)
+    want, _ = cpu2.forward(toks[-1], nthreads=16)
+    gpu2.forward_n(toks)
+    assert np.array_equal(bits(hip.hip_floats(gpu2.logits, c["vocab"])), bits(want))
+    with pytest.raises(ValueError):
+        gpu2.forward_n([1] * 6)                                # past the context's 8,200 rows
+    gpu.free(); gpu2.free()
+
+
 def test_one_launch_attention_up_to_1024_positions(dev):
     """A token's attention in one launch (contexts of up to 1,024 positions, heads of 64 and of 128): decode steps in
     every one of its four blocks of 256 positions, on the blocks' edges, and across position 1023 -> 1024, where the
