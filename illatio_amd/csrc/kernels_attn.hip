@@ -970,6 +970,10 @@ hipError_t ilt_k_attn_rows(const float* q, const float* kc, const float* vc, flo
     // tokens a workgroup: as many as leave their scores and the value slice room in LDS (150 KB)
     auto bytes = [&](int tg) { return sizeof(float) * ((size_t)tg * (smax + (tg > 1 ? 4 : 0)) + 16 * (size_t)vpitch); };
     const int tg = ntok == 1 ? 1 : bytes(16) <= 150 * 1024 ? 16 : bytes(4) <= 150 * 1024 ? 4 : 1;
+    // (a chunk whose sixteen tokens' scores and slice no longer fit LDS together -- past about 1,100 positions --
+    // goes through the tiled kernels below, sixteen tokens a workgroup still: with four tokens a workgroup its values
+    // took 1.6 ms a layer at 1,536 positions, with one 6.1 ms at 2,048)
+    if (ntok == 1 || tg == 16) {
     const int nb = (ctx + 511) / 512;
     const dim3 gs(nh, (ctx + 255) / 256, (ntok + tg - 1) / tg), gv(nh * (hd / 16), (ntok + tg - 1) / tg);
     hipError_t e = hipErrorInvalidValue;
@@ -989,10 +993,10 @@ hipError_t ilt_k_attn_rows(const float* q, const float* kc, const float* vc, flo
     }                                                                                                                                          \
   }
     ILT_ATTN(1, 1) ILT_ATTN(1, 2) ILT_ATTN(1, 3) ILT_ATTN(1, 4)
-    ILT_ATTN(4, 3) ILT_ATTN(4, 4)
     ILT_ATTN(16, 1) ILT_ATTN(16, 2) ILT_ATTN(16, 3)
 #undef ILT_ATTN
     return e;
+    }
   }
   if (scratch && pos0 + ntok <= 8192) {              // the value slice through LDS in tiles
     const int ctx = pos0 + ntok, tg = ntok > 1 ? 16 : 1;
