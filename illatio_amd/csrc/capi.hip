@@ -343,10 +343,11 @@ int ilt_d4_mvq8(uint64_t stream, int rows, int cols, int group_rows, const int8_
 static int gemv_experts(uint64_t stream, int fmt, int ncols, int nrows, int row_bytes, int64_t add, int64_t add_up,
                         int x_stride, int y_stride, const uint64_t* ptrs, int nz, const int8_t* xq, const float* xd,
                         const int32_t* bsums, const float* xf, const float* wts, float clamp, float* dst,
-                        const uint32_t* sel = nullptr) {
+                        const uint32_t* sel = nullptr, const uint32_t* counts = nullptr, const uint32_t* bases = nullptr) {
   ILT_REQUIRE(nrows >= 0 && nz >= 0 && ncols > 0 && ncols % 256 == 0 && row_bytes == ncols / 256 * block_bytes(fmt));
   if (nrows == 0 || nz == 0) return ILT_OK;
   ILT_REQUIRE(ptrs && dst && add >= 0 && (add & 1) == 0 && (add_up < 0 || (add_up & 1) == 0) && x_stride % 256 == 0 && x_stride >= 0);
+  ILT_REQUIRE(!counts || (bases && xf && !sel && add_up < 0));
   if (xf) ILT_REQUIRE(((uintptr_t)xf & 15) == 0);
   else ILT_REQUIRE(xq && xd && (bsums || fmt == ILT_IQ2_XXS) && ((uintptr_t)xq & 15) == 0);
   ILT_REQUIRE(nz <= 65535);
@@ -358,7 +359,34 @@ static int gemv_experts(uint64_t stream, int fmt, int ncols, int nrows, int row_
   }
   p.ptrs = ptrs; p.sel = sel; p.cols = ncols;
   p.xq = xq; p.xs = xd; p.bsums = bsums; p.xf = xf; p.x_stride = x_stride; p.y_stride = y_stride;
+  p.counts = counts; p.bases = bases;
   return (int)ilt_gemv_launch(p, nz, S(stream));
+}
+
+// the reference's own arguments (ds4f.cu:762-772): srcs read through first, float rows quantized by the kernel
+static int mv_rows(uint64_t stream, int fmt, int ncols, int nrows, int row_bytes, int64_t add, int x_stride, int y_stride,
+                   const uint64_t* ptrs, const uint64_t* srcs, int nz, const float* x, float* y, const uint32_t* counts,
+                   const uint32_t* bases) {
+  ILT_REQUIRE(x && (counts == nullptr) == (bases == nullptr));
+  if (srcs && nrows > 0 && nz > 0) {
+    ILT_REQUIRE(ptrs && add >= 0 && (add & 1) == 0 && row_bytes > 0 && nz <= 65535);
+    ILT_TRY(ilt_k_read_through((const unsigned long long*)srcs, (const unsigned long long*)ptrs, nz, add, (long long)nrows * row_bytes,
+                               S(stream)));
+  }
+  return gemv_experts(stream, fmt, ncols, nrows, row_bytes, add, -1, x_stride, y_stride, ptrs, nz, nullptr, nullptr, nullptr, x,
+                      nullptr, 0.0f, y, nullptr, counts, bases);
+}
+
+int ilt_d4_mv_rows_iq2_xxs(uint64_t stream, int ncols, int nrows, int row_bytes, int64_t add, int x_stride, int y_stride,
+                           const uint64_t* ptrs, const uint64_t* srcs, int nz, const float* x, float* y,
+                           const uint32_t* counts, const uint32_t* bases) {
+  return mv_rows(stream, ILT_IQ2_XXS, ncols, nrows, row_bytes, add, x_stride, y_stride, ptrs, srcs, nz, x, y, counts, bases);
+}
+
+int ilt_d4_mv_rows_q2_k(uint64_t stream, int ncols, int nrows, int row_bytes, int64_t add, int x_stride, int y_stride,
+                        const uint64_t* ptrs, const uint64_t* srcs, int nz, const float* x, float* y,
+                        const uint32_t* counts, const uint32_t* bases) {
+  return mv_rows(stream, ILT_Q2_K, ncols, nrows, row_bytes, add, x_stride, y_stride, ptrs, srcs, nz, x, y, counts, bases);
 }
 
 int ilt_d4_mv_iq2_xxs(uint64_t stream, int ncols, int nrows, int row_bytes, int64_t add, int x_stride, int y_stride,
@@ -1141,16 +1169,20 @@ int ilt_launch(const char* kernel, unsigned gx, unsigned gy, unsigned gz, unsign
                                           a.ptr<cf>(6), a.f32(7), a.ptr<float*>(8));
   K("d4_mvq8") return ilt_d4_mvq8(stream, a.i32(0), a.i32(1), a.i32(2), a.ptr<ci8>(3), a.ptr<cu16>(4), a.ptr<ci8>(5),
                                   a.ptr<cf>(6), a.ptr<float*>(7));
-  K("d4_mv_iq2_xxs") {
-    ILT_REQUIRE(a.ptr<const void*>(7) == nullptr);
+  // d4_mv_iq2_xxs / d4_mv_q2_k: the reference's twelve slots (ds4f.cu:769-772, 837-840), float rows in
+  K("d4_mv_iq2_xxs")
+    return ilt_d4_mv_rows_iq2_xxs(stream, a.i32(0), a.i32(1), a.i32(2), a.i64(3), a.i32(4), a.i32(5), a.ptr<const uint64_t*>(6),
+                                  a.ptr<const uint64_t*>(7), (int)gz, a.ptr<cf>(8), a.ptr<float*>(9), a.ptr<cu32>(10), a.ptr<cu32>(11));
+  K("d4_mv_q2_k")
+    return ilt_d4_mv_rows_q2_k(stream, a.i32(0), a.i32(1), a.i32(2), a.i64(3), a.i32(4), a.i32(5), a.ptr<const uint64_t*>(6),
+                               a.ptr<const uint64_t*>(7), (int)gz, a.ptr<cf>(8), a.ptr<float*>(9), a.ptr<cu32>(10), a.ptr<cu32>(11));
+  // the same on activations quantized beforehand (quant_q8k): slot 7 unused, slots 8, 10, 11 = xq, xd, bsums
+  K("d4_mvq_iq2_xxs")
     return ilt_d4_mv_iq2_xxs(stream, a.i32(0), a.i32(1), a.i32(2), a.i64(3), a.i32(4), a.i32(5), a.ptr<const uint64_t*>(6),
                              (int)gz, a.ptr<ci8>(8), a.ptr<cf>(10), a.ptr<float*>(9));
-  }
-  K("d4_mv_q2_k") {
-    ILT_REQUIRE(a.ptr<const void*>(7) == nullptr);
+  K("d4_mvq_q2_k")
     return ilt_d4_mv_q2_k(stream, a.i32(0), a.i32(1), a.i32(2), a.i64(3), a.i32(4), a.i32(5), a.ptr<const uint64_t*>(6),
                           (int)gz, a.ptr<ci8>(8), a.ptr<cf>(10), a.ptr<const int32_t*>(11), a.ptr<float*>(9));
-  }
   K("embed_q8") return ilt_embed_q8(stream, a.ptr<ci8>(0), a.ptr<cu16>(1), a.ptr<const int32_t*>(2), a.ptr<float*>(3), a.i32(4), (int)gx);
   K("embed_k") return ilt_embed_k(stream, a.i32(0), a.ptr<const void*>(1), a.ptr<const int32_t*>(2), a.ptr<float*>(3), a.i32(4), (int)gx);
   K("d4_route") return ilt_d4_route(stream, a.i32(0), a.i32(1), a.i32(2), a.f32(3), a.i32(4), a.ptr<cf>(5), a.ptr<cf>(6),

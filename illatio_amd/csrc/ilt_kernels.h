@@ -103,6 +103,11 @@ struct IltGemvParams {
   IltRouteAlong route;
   IltCacheAhead ahead;
   IltRowsAhead rows_ahead;
+  // grid y's expert on several rows of activations (the looping variant only): rows bases[y] .. bases[y] + counts[y] - 1
+  // of the activations and of the output, x_stride / y_stride apart, its matrix read from memory once and from the
+  // cache for the rows after the first (the counts / bases of the reference's d4_mv_*, ds4f.cu:762-772); null = row y
+  const uint32_t* counts;
+  const uint32_t* bases;
 };
 
 // The kernel is chosen by the matrices' formats (mat[i].fmt): one format, or Q4_K and Q6_K mixed.
@@ -128,6 +133,9 @@ hipError_t ilt_k_mm_f16(int ncols, int nrows, int ntok, long long row_halfs, int
 hipError_t ilt_k_repack_q8(const uint8_t* raw, int8_t* qs, uint16_t* d, long long nblocks, hipStream_t st);
 hipError_t ilt_k_repack_q6k(const uint8_t* raw, uint8_t* out, long long nblocks, hipStream_t st);
 hipError_t ilt_k_copy_bytes(const uint8_t* src, uint8_t* dst, long long bytes, hipStream_t st);
+// for each of the nz experts with srcs[z] set: bytes from srcs[z] + add to ptrs[z] + add (d4_read_through, ds4f.cu:742-760)
+hipError_t ilt_k_read_through(const unsigned long long* srcs, const unsigned long long* ptrs, int nz, long long add, long long bytes,
+                              hipStream_t st);
 hipError_t ilt_k_dequant_rows(int fmt, const uint8_t* w, const uint16_t* wd, const int* rows_idx, long long nrows,
                               int cols, long long row_bytes, float* out, hipStream_t st);
 

@@ -658,10 +658,9 @@ __device__ __forceinline__ float sum_any(int fmt, const float* t, int S) {
 
 // FSET: the format of every matrix of the launch, or 0 when they mix Q4_K and Q6_K.  The
 // expert formats (IQ2_XXS, Q2_K) take grid y = expert.
+// (z: grid y, which chooses the expert; xy: the row of activations and of the output it works on)
 template <int FSET>
-__global__ __launch_bounds__(kThreads) void gemv_kernel(IltGemvParams p) {
-  extern __shared__ __align__(16) unsigned char smem[];
-  const int z = blockIdx.y;
+__device__ __forceinline__ void gemv_body(const IltGemvParams& p, const int z, const long xy, unsigned char* smem) {
   constexpr bool q8 = FSET == ILT_Q8_0;
   const int S = q8 ? p.cols / 32 : p.cols / 256;
   // LDS: xq | bsums | xs | (grid) | terms (per wave)
@@ -695,7 +694,7 @@ __global__ __launch_bounds__(kThreads) void gemv_kernel(IltGemvParams p) {
 
   // Float activations to quantize here: their first loads go out before any weight load, since
   // loads return in order and these (hot in L2) are needed first.
-  const long xoff = (long)z * p.x_stride + (long)group * p.cols;
+  const long xoff = xy * p.x_stride + (long)group * p.cols;
   float4 xfirst[4], nfirst[4];
   if (!q8 && p.xf) load_q8k_pass(p.xf + xoff, S, 0, xfirst);
   // ... and when they are normalized first: the norm's weights likewise, and now the squares
@@ -786,18 +785,18 @@ __global__ __launch_bounds__(kThreads) void gemv_kernel(IltGemvParams p) {
       if (p.glu) {
         const int ufmt = FSET != 0 ? FSET : p.mat[1].fmt;
         const float uv = sum_any(ufmt, tw + (long)RB * tpr + (long)lane * S * ((ufmt == ILT_Q4_K || ufmt == ILT_Q2_K) ? 2 : 1), S);
-        float* y = m.y + (long)z * p.y_stride;
+        float* y = m.y + xy * p.y_stride;
         if (p.glu == 1) {
           y[r] = dense_glu(v, uv);
         } else {        // the experts' gated activation, as d4_swiglu_w computes it
           float gv = v, uu = uv;
           if (p.clamp > 1e-6f) { gv = fminf(gv, p.clamp); uu = fmaxf(-p.clamp, fminf(uu, p.clamp)); }
           float o = ilt_silu(gv) * uu;
-          if (p.wts) o = o * p.wts[z];
+          if (p.wts) o = o * p.wts[xy];
           y[r] = o;
         }
       } else {
-        float* y = m.y + (long)z * p.y_stride;
+        float* y = m.y + xy * p.y_stride;
         if (m.bias) v = v + m.bias[r];
         if (p.acc) v = y[r] + v;
         y[r] = v;
@@ -807,6 +806,25 @@ __global__ __launch_bounds__(kThreads) void gemv_kernel(IltGemvParams p) {
     __builtin_amdgcn_wave_barrier();
   }
   asm volatile("" :: "v"(warm[0]), "v"(warm[1]), "v"(warm[2]), "v"(warm[3]));
+}
+
+template <int FSET>
+__global__ __launch_bounds__(kThreads) void gemv_kernel(IltGemvParams p) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  gemv_body<FSET>(p, blockIdx.y, blockIdx.y, smem);
+}
+
+// Grid y's expert on its counts[y] rows of activations, one after another: the rows after the first find the matrix
+// in the cache (ds4f.cu:762-772).  An expert with no rows ends at once.
+template <int FSET>
+__global__ __launch_bounds__(kThreads) void gemv_rows_kernel(IltGemvParams p) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  const int z = blockIdx.y, n = (int)p.counts[z];
+  const long t0 = p.bases[z];
+  for (int tk = 0; tk < n; tk++) {
+    if (tk) __syncthreads();                           // the row before is through with the staged activations
+    gemv_body<FSET>(p, z, t0 + tk, smem);
+  }
 }
 
 // ---- the streamed variant: matrices of up to ~100 KB per CU, every format ---------------------------
@@ -1524,7 +1542,11 @@ hipError_t ilt_gemv_launch(IltGemvParams& p, int nz, hipStream_t st) {
               p.sum.k >= 1 && p.sum.k <= 8 && p.sum.stride >= p.mat[0].rows;
     if (!ok) return hipErrorNotSupported;
   }
-  {
+  if (p.counts) {                 // an expert's several rows: the looping variant of the experts' formats, floats in
+    if (!p.bases || !p.ptrs || p.sel || !p.xf || p.glu || p.acc || p.norm_w || p.group_rows || p.nmat != 1 || p.mat[0].bias ||
+        !(fset == ILT_IQ2_XXS || fset == ILT_Q2_K))
+      return hipErrorNotSupported;
+  } else {
     const hipError_t e = gemv_stream_launch(p, fset, nz, st);
     if (e != hipErrorNotSupported || p.sum.rows) return e;
   }
@@ -1576,6 +1598,11 @@ hipError_t ilt_gemv_launch(IltGemvParams& p, int nz, hipStream_t st) {
   const int wgs = waves_each / kWaves;
   p.wgs_per_group = wgs;
   dim3 grid(wgs * ngroups, nz);
+  if (p.counts) {
+    if (fset == ILT_IQ2_XXS) hipLaunchKernelGGL(gemv_rows_kernel<ILT_IQ2_XXS>, grid, dim3(kThreads), smem, st, p);
+    else hipLaunchKernelGGL(gemv_rows_kernel<ILT_Q2_K>, grid, dim3(kThreads), smem, st, p);
+    return hipGetLastError();
+  }
   switch (fset) {
     case 0: hipLaunchKernelGGL(gemv_kernel<0>, grid, dim3(kThreads), smem, st, p); break;
     case ILT_Q8_0: hipLaunchKernelGGL(gemv_kernel<ILT_Q8_0>, grid, dim3(kThreads), smem, st, p); break;

@@ -108,6 +108,28 @@ __global__ __launch_bounds__(256) void copy_bytes_kernel(const u8* __restrict__ 
   else if (i < bytes) dst[i] = src[i];
 }
 
+// d4_read_through (ds4f.cu:742-760) as a launch in front of the product: the experts whose srcs entry is set have the
+// BYTES at srcs[z] + add (host memory the device can read) copied to ptrs[z] + add, their slot.  Grid y = the expert;
+// 16 bytes a lane where both addresses allow, else two.
+__global__ __launch_bounds__(256) void read_through_kernel(const unsigned long long* __restrict__ srcs, const unsigned long long* __restrict__ ptrs,
+                                                           long long add, long long bytes) {
+  const unsigned long long s0 = srcs[blockIdx.y];
+  if (!s0) return;
+  const u8* src = (const u8*)(s0 + add);
+  u8* dst = (u8*)(ptrs[blockIdx.y] + add);
+  const long long step = (long long)gridDim.x * 256, t = (long long)blockIdx.x * 256 + threadIdx.x;
+  if ((((unsigned long long)src | (unsigned long long)dst) & 15) == 0) {
+    const long long n16 = bytes >> 4;
+    for (long long i = t; i < n16; i += step) ((int4*)dst)[i] = ((const int4*)src)[i];
+    for (long long i = (n16 << 4) + t; i < bytes; i += step) dst[i] = src[i];
+  } else {
+    for (long long i = 2 * t; i < bytes; i += 2 * step) {
+      if (i + 1 < bytes) *(u16*)(dst + i) = *(const u16*)(src + i);
+      else dst[i] = src[i];
+    }
+  }
+}
+
 // ---- rows as floats (embed_q8 / embed_k; q8mat-row!, kmat-row!, *-row-floats!) ------------------
 __device__ __forceinline__ void scale_min_k4_bytes(int j, const u8* q, int& sc, int& m) {
   if (j < 4) { sc = q[j] & 63; m = q[j + 4] & 63; }
@@ -253,6 +275,15 @@ hipError_t ilt_k_repack_q6k(const uint8_t* raw, uint8_t* out, long long nblocks,
 hipError_t ilt_k_copy_bytes(const uint8_t* src, uint8_t* dst, long long bytes, hipStream_t st) {
   if (bytes <= 0) return hipSuccess;
   hipLaunchKernelGGL(copy_bytes_kernel, dim3((unsigned)((bytes / 2 + 256) / 256)), dim3(256), 0, st, src, dst, bytes);
+  return hipGetLastError();
+}
+
+hipError_t ilt_k_read_through(const unsigned long long* srcs, const unsigned long long* ptrs, int nz, long long add, long long bytes,
+                              hipStream_t st) {
+  if (bytes <= 0 || nz <= 0) return hipSuccess;
+  if (nz > 65535 || (add & 1)) return hipErrorInvalidValue;
+  const long long wgs = (bytes / 16 + 255) / 256;
+  hipLaunchKernelGGL(read_through_kernel, dim3((unsigned)(wgs < 1 ? 1 : wgs > 64 ? 64 : wgs), (unsigned)nz), dim3(256), 0, st, srcs, ptrs, add, bytes);
   return hipGetLastError();
 }
 

@@ -155,8 +155,9 @@ def tail_tables(dev, pool, sel, w):
 
 def ffn_tail(dev, pool, sel, w, norm2, sout, clamp, keep=None, ws=None, tables=None):
     """One token's routed experts SEL (weights W) on NORM2, summed in SEL's order with the
-    shared expert's SOUT (DK-FFN-TAIL): gate and up in one launch over 2k matrices, the
-    gated activation, each slot's Q8_K quantization, down, the ordered sum.  Returns MOE.
+    shared expert's SOUT (DK-FFN-TAIL, cuda-ds4f.lisp:908-956, its launches with its argument lists):
+    gate and up in one launch over 2k matrices, the gated activation, down, the ordered sum; the
+    expert kernels quantize their float rows themselves (Q8_K, as the CPU path does).  Returns MOE.
     With a Workspace WS nothing is allocated, freed or waited for; TABLES = tail_tables()
     made beforehand."""
     d, ff, k = pool.d, pool.ff, len(sel)
@@ -165,13 +166,11 @@ def ffn_tail(dev, pool, sel, w, norm2, sout, clamp, keep=None, ws=None, tables=N
     ptrs, bw = tables if tables else tail_tables(dev, pool, sel, w)
     bgu, bm = A(dev, 4 * 2 * k * ff), A(dev, 4 * k * ff)
     bd, moe = A(dev, 4 * k * d), A(dev, 4 * d)
-    xq, xd, xs = _q8k(dev, norm2, d, A)
     hip.launch(dev, "d4_mv_iq2_xxs", ((ff + 7) // 8, 1, 2 * k), 64,
-               [d, ff, pool.grb, hip.I64(0), 0, ff, ptrs, None, xq, bgu, xd, xs])
+               [d, ff, pool.grb, hip.I64(0), 0, ff, ptrs, None, norm2, bgu, None, None])
     hip.launch(dev, "d4_swiglu_w", (k * ff + 255) // 256, 256, [k, ff, float(clamp), bgu, bgu.at(4 * k * ff), bw, bm, None, None])
-    mq, md, ms = _q8k(dev, bm, k * ff, A)
     hip.launch(dev, "d4_mv_q2_k", ((d + 7) // 8, 1, k), 64,
-               [ff, d, pool.drb, hip.I64(2 * gb), ff, d, ptrs, None, mq, bd, md, ms])
+               [ff, d, pool.drb, hip.I64(2 * gb), ff, d, ptrs, None, bm, bd, None, None])
     hip.launch(dev, "d4_moe_sum", (d + 255) // 256, 256, [d, k, bd, sout, moe, None])
     if ws:
         return moe
@@ -180,7 +179,7 @@ def ffn_tail(dev, pool, sel, w, norm2, sout, clamp, keep=None, ws=None, tables=N
         keep["mid"] = hip.hip_floats(bm, k * ff).reshape(k, ff)
         keep["gu"] = hip.hip_floats(bgu, 2 * k * ff).reshape(2, k, ff)
         keep["down"] = hip.hip_floats(bd, k * d).reshape(k, d)
-    for b in (bgu, bm, bd, xq, xd, xs, mq, md, ms) + (() if tables else (ptrs, bw)):
+    for b in (bgu, bm, bd) + (() if tables else (ptrs, bw)):
         hip.hip_free(b)
     return moe
 
@@ -294,7 +293,10 @@ def ffn_small(dev, pool, sh, logits, norm2, n, ne, nu, scale, clamp, bias=None, 
     kernels take one slot per (token, slot) row, row t*nu + j on expert sel[t*nu + j]: the
     gathered rows, gate+up+gated activation of all rows in one launch, their downs in one, the
     sums in slot order with the shared expert's (d4_mvq8n for its three products).  Returns
-    MOE (N x d)."""
+    MOE (N x d).  GROUPED "counts": DK-FFN-SMALL's own launches with its argument lists
+    (cuda-ds4f-spec.lisp:82-88) -- d4_gather_rows, d4_mv_iq2_xxs for the gates and again for the ups,
+    d4_swiglu_w, d4_mv_q2_k, each expert kernel over all NE slots with the counts and bases that
+    d4_group_* left on the device (an expert nobody chose has a count of 0)."""
     d, ff = pool.d, pool.ff
     rows = n * nu
     gb = pool.gate_bytes
@@ -313,6 +315,23 @@ def ffn_small(dev, pool, sh, logits, norm2, n, ne, nu, scale, clamp, bias=None, 
     # the routed experts: row r = (token r / nu, slot r % nu)
     sel, w = route(dev, logits, n, ne, nu, scale, bias)
     extra = []
+    if grouped == "counts":
+        g = group_rows(dev, sel, w, n, ne, nu)
+        rmap, smap, wrow = g["rmap"], g["smap"], g["wrow"]
+        x, bg, bu = A(dev, 4 * rows * d), A(dev, 4 * rows * ff), A(dev, 4 * rows * ff)
+        bm, bd, moe = A(dev, 4 * rows * ff), A(dev, 4 * rows * d), A(dev, 4 * n * d)
+        hip.launch(dev, "d4_gather_rows", (rows * d + 255) // 256, 256, [d, rows, norm2, rmap, x])
+        for add, out in ((0, bg), (gb, bu)):
+            hip.launch(dev, "d4_mv_iq2_xxs", ((ff + 7) // 8, 1, ne), 64,
+                       [d, ff, pool.grb, hip.I64(add), d, ff, pool.ptrs, None, x, out, g["counts"], g["bases"]])
+        hip.launch(dev, "d4_swiglu_w", (rows * ff + 255) // 256, 256, [rows, ff, float(clamp), bg, bu, wrow, bm, None, None])
+        hip.launch(dev, "d4_mv_q2_k", ((d + 7) // 8, 1, ne), 64,
+                   [ff, d, pool.drb, hip.I64(2 * gb), ff, d, pool.ptrs, None, bm, bd, g["counts"], g["bases"]])
+        hip.launch(dev, "d4_moe_sum_rows", (n * d + 255) // 256, 256, [d, nu, n, bd, smap, sout, moe])
+        hip.hip_sync(dev)
+        for b in [qn_q, qn_s, sg, su, smid, qm_q, qm_s, sout, one, sel, w, x, bg, bu, bm, bd] + list(g.values()):
+            hip.hip_free(b)
+        return moe
     if grouped:
         # GROUPED: the rows grouped by expert on the device (d4_group_*), an expert's rows one after another, so its
         # matrices come from memory once for all its tokens: what the reference's counts / bases arguments give

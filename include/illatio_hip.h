@@ -201,6 +201,21 @@ int ilt_d4_mv_iq2_xxs(uint64_t stream, int ncols, int nrows, int row_bytes, int6
                       const uint64_t* ptrs, int nz, const int8_t* xq, const float* xd, float* dst);
 int ilt_d4_mv_q2_k(uint64_t stream, int ncols, int nrows, int row_bytes, int64_t add, int x_stride, int y_stride,
                    const uint64_t* ptrs, int nz, const int8_t* xq, const float* xd, const int32_t* bsums, float* dst);
+/* The same two with the reference kernels' own arguments (ds4f.cu:762-772, 837-840; callers: DK-FFN-TAIL,
+   cuda-ds4f.lisp:937-941, and DK-FFN-SMALL, cuda-ds4f-spec.lisp:83-88): x = rows of floats, which the kernel
+   quantizes as quantize-act! does (kquant.lisp:511-514), so y has the CPU path's bits.
+   srcs (or null): for each z with srcs[z] set, the matrix's nrows * row_bytes bytes are first copied from
+     srcs[z] + add (host memory the device can read) to ptrs[z] + add, the expert's slot (d4_read_through,
+     ds4f.cu:742-760), as a launch of its own in front of the product.
+   counts, bases (both or neither): expert z works on rows bases[z] .. bases[z] + counts[z] - 1 of x and y
+     (x_stride / y_stride floats apart), its matrix read from memory once and from the cache after; an expert
+     with a count of 0 does nothing.  Without them expert z works on row z (x_stride 0: all on row 0). */
+int ilt_d4_mv_rows_iq2_xxs(uint64_t stream, int ncols, int nrows, int row_bytes, int64_t add, int x_stride, int y_stride,
+                           const uint64_t* ptrs, const uint64_t* srcs, int nz, const float* x, float* y,
+                           const uint32_t* counts, const uint32_t* bases);
+int ilt_d4_mv_rows_q2_k(uint64_t stream, int ncols, int nrows, int row_bytes, int64_t add, int x_stride, int y_stride,
+                        const uint64_t* ptrs, const uint64_t* srcs, int nz, const float* x, float* y,
+                        const uint32_t* counts, const uint32_t* bases);
 
 /* The decode step of d4-routed! / d4-shared! (ds4f.lisp:994-1048; DK-FFN-TAIL, cuda-ds4f.lisp:
    908-956) in fewer launches, with the same bits: the activations come as floats and every
@@ -499,8 +514,9 @@ int ilt_d4_mm_id_glu_bf16(uint64_t stream, int gguf_type, int ncols, int nrows, 
  * 32 bits, a float in the low 32 bits, a long long as 64 bits.  Kernel names and argument
  * orders are the reference's (its src/cuda/ *.cu); the grid and block passed in are read
  * only where an argument count lives in them (d4_route: tokens = gx; d4_mv_*: experts =
- * gz).  For d4_mv_iq2_xxs / d4_mv_q2_k the slots "src1, counts, bases" carry the Q8_K
- * activations "xq, xd, bsums" and srcs must be null.  mm_q8, mm_q8_mma, mm_k, mm_q4k_mma and
+ * gz).  d4_mv_iq2_xxs / d4_mv_q2_k take the reference's twelve slots (ilt_d4_mv_rows_*); as
+ * d4_mvq_iq2_xxs / d4_mvq_q2_k the slots "src1, counts, bases" carry Q8_K activations made
+ * beforehand, "xq, xd, bsums", and srcs is not read (ilt_d4_mv_iq2_xxs / ilt_d4_mv_q2_k).  mm_q8, mm_q8_mma, mm_k, mm_q4k_mma and
  * mm_q6k_mma take the reference's lists.  d4_mm_id_iq2_xxs / d4_mm_id_q2_k take the
  * reference's eleven slots (ncols, nrows, row_bytes, x_stride, y_stride, add, ptrs, counts,
  * bases, x, y) with x = xq, followed by three more: xd, bsums, total_rows (long long);

@@ -190,7 +190,7 @@ def test_indexed_expert_gemv_bit_for_bit(dev, qtype, rows, cols):
         kq, kd, ks = hip.hip_alloc(dev, nz * cols), hip.hip_alloc(dev, 4 * nz * cols // 256), hip.hip_alloc(dev, 4 * nz * cols // 16)
         hip.launch(dev, "quant_q8k", nz * cols // 256, 256, [xb, kq, kd, ks, hip.I64(nz * cols // 256)])
         y = hip.hip_alloc(dev, 4 * nz * rows)
-        name = "d4_mv_iq2_xxs" if qtype == synth.IQ2_XXS else "d4_mv_q2_k"
+        name = "d4_mvq_iq2_xxs" if qtype == synth.IQ2_XXS else "d4_mvq_q2_k"     # (activations quantized beforehand)
         hip.launch(dev, name, ((rows + 7) // 8, 1, nz), 64,
                    [cols, rows, rb, hip.I64(pad), x_stride, rows, ptrs, None, kq, y, kd, ks])
         got = hip.hip_floats(y, nz * rows).reshape(nz, rows)
@@ -211,6 +211,83 @@ def test_indexed_expert_gemv_bit_for_bit(dev, qtype, rows, cols):
         for b in (xb, kq, kd, ks, y):
             hip.hip_free(b)
     hip.hip_free(pool); hip.hip_free(ptrs)
+
+
+@pytest.mark.parametrize("qtype,rows,cols", [(synth.IQ2_XXS, 2048, 4096), (synth.Q2_K, 4096, 2048),
+                                              (synth.IQ2_XXS, 50, 512), (synth.Q2_K, 9, 256)])
+def test_expert_gemv_with_the_reference_arguments(dev, qtype, rows, cols):
+    """d4_mv_iq2_xxs / d4_mv_q2_k launched with the reference kernels' twelve slots (ds4f.cu:769-772, 837-840):
+    float rows in (quantized by the kernel as the CPU path quantizes them), ptrs[z] + add, and
+    - neither counts nor bases: expert z on row z of x (DK-FFN-TAIL's launches, cuda-ds4f.lisp:937-941; x_stride 0 = all
+      on one row);
+    - counts and bases: expert z on rows bases[z] .. bases[z] + counts[z] - 1 (DK-FFN-SMALL's,
+      cuda-ds4f-spec.lisp:83-88), an expert with no rows writing nothing, strides wider than a row;
+    - srcs: an expert whose slot is empty has its matrix read through from pinned host memory into the slot first
+      (ds4f.cu:742-760), and the slot holds it afterwards."""
+    import ctypes
+    from illatio_amd import hip
+    rng = synth.make_rng(qtype * 11 + rows)
+    nexp = 5
+    rb = synth.row_bytes(qtype, cols)
+    pad = 512
+    slot = (pad + rows * rb + 255) // 256 * 256
+    w = synth.weights(qtype, nexp * rows, cols, rng).reshape(nexp, rows * rb)
+    host = np.zeros((nexp, slot), np.uint8)
+    host[:, pad:pad + rows * rb] = w
+    name = "d4_mv_iq2_xxs" if qtype == synth.IQ2_XXS else "d4_mv_q2_k"
+    chosen = [4, 0, 2]
+    # expert 0's slot on the device is empty; its bytes wait in pinned host memory
+    dev_host = host.copy()
+    dev_host[0] = 0
+    pool = hip.hip_upload_new(dev, dev_host)
+    pinned = hip.hip_host_alloc(dev, slot)
+    ctypes.memmove(pinned, host[0].ctypes.data, slot)
+    ptrs = hip.hip_upload_new(dev, np.array([pool.ptr + e * slot for e in chosen], np.uint64))
+    srcs = hip.hip_upload_new(dev, np.array([0, pinned, 0], np.uint64))
+
+    def want_row(e, xrow):
+        return orc.matmul(qtype, w[e].reshape(rows, rb), rows, cols, xrow)
+
+    # counts and bases: rows 0-1 for expert 4, rows 2-4 for expert 0 (read through), none for expert 2
+    counts, bases = [2, 3, 0], [0, 2, 5]
+    nrows_x = 5
+    xs, ys = cols + 256, rows + 8
+    x = np.zeros((nrows_x, xs), np.float32)
+    x[:, :cols] = special_activations(cols * nrows_x, rng).reshape(nrows_x, cols) if cols >= 512 else synth.activations((nrows_x, cols), rng)
+    xb = hip.hip_upload_new(dev, x)
+    y = hip.hip_upload_new(dev, np.full(nrows_x * ys, 7.0, np.float32))
+    cb, bb = hip.hip_upload_new(dev, np.array(counts, np.uint32)), hip.hip_upload_new(dev, np.array(bases, np.uint32))
+    hip.launch(dev, name, ((rows + 7) // 8, 1, 3), 64, [cols, rows, rb, hip.I64(pad), xs, ys, ptrs, srcs, xb, y, cb, bb])
+    got = hip.hip_floats(y, nrows_x * ys).reshape(nrows_x, ys)
+    assert np.all(got[:, rows:] == 7.0)
+    for z, e in enumerate(chosen):
+        for r in range(bases[z], bases[z] + counts[z]):
+            assert np.array_equal(bits(got[r, :rows]), bits(want_row(e, x[r, :cols]))), (qtype, z, r)
+    # the slot holds the matrix now (and nothing else of the pool changed)
+    back = hip.hip_download(pool, np.uint8, nexp * slot).reshape(nexp, slot)
+    assert np.array_equal(back[0, pad:pad + rows * rb], w[0])
+    assert np.array_equal(back[1:], host[1:])
+    # with the slot filled, no srcs are needed any more
+    y2 = hip.hip_upload_new(dev, np.full(nrows_x * ys, 7.0, np.float32))
+    hip.launch(dev, name, ((rows + 7) // 8, 1, 3), 64, [cols, rows, rb, hip.I64(pad), xs, ys, ptrs, None, xb, y2, cb, bb])
+    assert np.array_equal(bits(hip.hip_floats(y2, nrows_x * ys)), bits(got.reshape(-1)))
+    # no counts: expert z on row z, or all on row 0
+    for x_stride in (0, cols):
+        xz = np.ascontiguousarray(x[:3, :cols])
+        xzb = hip.hip_upload_new(dev, xz)
+        y3 = hip.hip_alloc(dev, 4 * 3 * rows)
+        hip.launch(dev, name, ((rows + 7) // 8, 1, 3), 64, [cols, rows, rb, hip.I64(pad), x_stride, rows, ptrs, None, xzb, y3, None, None])
+        got3 = hip.hip_floats(y3, 3 * rows).reshape(3, rows)
+        for z, e in enumerate(chosen):
+            assert np.array_equal(bits(got3[z]), bits(want_row(e, xz[z if x_stride else 0]))), (qtype, z, x_stride)
+        hip.hip_free(xzb); hip.hip_free(y3)
+    # one of counts / bases without the other is refused
+    with pytest.raises(hip.HipError):
+        hip.launch(dev, name, ((rows + 7) // 8, 1, 3), 64, [cols, rows, rb, hip.I64(pad), xs, ys, ptrs, None, xb, y2, cb, None])
+    hip.hip_sync(dev)
+    for b in (pool, ptrs, srcs, xb, y, y2, cb, bb):
+        hip.hip_free(b)
+    hip.hip_host_free(pinned)
 
 
 def test_d4_mvq8n_tokens_of_a_speculative_step(dev):

@@ -335,7 +335,9 @@ def test_moe_short_pass_of_a_few_tokens_bit_exact(dev, ne, d, ff, nu, n, clamp):
     logits = synth.activations((n, ne), rng)
     logits[1] = logits[0]                     # two tokens on the same experts
     lb, nb = hip.hip_upload_new(dev, logits), hip.hip_upload_new(dev, norm)
-    for grouped in (False, True):             # a launch slot per (token, slot) row in token order; the rows grouped by expert
+    # a launch slot per (token, slot) row in token order; the rows grouped by expert; the reference's own launches
+    # with counts and bases (cuda-ds4f-spec.lisp:82-88)
+    for grouped in (False, True, "counts"):
         moe = ds4f.ffn_small(dev, pool, sh, lb, nb, n, ne, nu, 1.5, clamp, grouped=grouped)
         got = hip.hip_floats(moe, n * d).reshape(n, d)
         for t in range(n):
