@@ -409,7 +409,7 @@ def workload_c3(args, dev):
     bf16_path = args.path.startswith("bf16")
     path = args.path
     if path == "bf16":                           # the faster way from the quantized matrix: two passes pay from about a thousand tokens on
-        path = "bf16-2pass" if T >= 1024 else "bf16-1pass"
+        path = "bf16-2pass" if T >= 1536 else "bf16-1pass"
     if path in ("bf16-2pass", "bf16-resident"):
         # the matrix dequantized to a bf16 copy (inside every step, or once beforehand and kept), then the plain bf16 product
         xb = hip.hip_alloc(dev, dense.slabs_bytes(T, cols), zero=False)
@@ -810,7 +810,7 @@ def main():
     ap.add_argument("--host-argmax", action="store_true", help="c2d: every token's logits to the host and the next token picked there")
     ap.add_argument("--qtype", default="q6_k", choices=["q6_k", "q4_k", "q8_0"], help="c3: the matrix's format (the benchmark's: q6_k)")
     ap.add_argument("--path", default="bf16", choices=["bf16", "bf16-1pass", "bf16-2pass", "bf16-resident", "int8", "int8-2pass", "int8-resident"],
-                    help="c3, c5: which matrix-core path.  c3: bf16 = 2pass from 1024 tokens on, else 1pass; bf16-1pass = the matrix dequantized inside the product's loop; "
+                    help="c3, c5: which matrix-core path.  c3: bf16 = 2pass from 1536 tokens on, else 1pass; bf16-1pass = the matrix dequantized inside the product's loop; "
                          "bf16-2pass = the matrix dequantized to a bf16 copy inside the step, then the plain bf16 product; bf16-resident = that copy made beforehand and kept")
     ap.add_argument("--norm", action="store_true", help="c2: include each layer's two norms and the output norm (inside the product launches in fused mode)")
     ap.add_argument("--mode", default="fused", choices=["fused", "fused-q", "single", "device"],

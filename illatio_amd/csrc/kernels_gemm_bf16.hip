@@ -34,6 +34,7 @@
 #include "ilt_iq2xxs_tables.h"
 #include "ilt_kernels.h"
 #include <stdlib.h>
+#include <mutex>
 #include <type_traits>
 
 namespace {
@@ -211,6 +212,10 @@ struct BfParams {
   const u16* wdq;
   // the planes made beforehand (gemm_i8pp_kernel): w = the hi plane, wlo the lo plane (a byte a weight, rows of cols bytes), wdf = d per row and super-block
   const u8* wlo; const float* wdf;
+  // the columns split over workgroups (gemm_bf16_kernel, dense): workgroups from split_from on take the tiles from
+  // split_from on, ksplit of them a tile, each a run of the super-blocks, and leave their sums in part (a tile of TM x TN
+  // floats each, token after token); bf16_split_sum_kernel adds a tile's parts in order and writes y.  ksplit 0: none
+  int ksplit, split_from; float* part;
 };
 
 template <int TM, int TN, int NXS, int NWS> struct Smem {
@@ -284,8 +289,16 @@ __device__ __forceinline__ void store_tile(const v16f (&acc)[NA][NB], const BfPa
 // with w its matrix, when grouped).  Tiles are numbered so that the eight XCDs' workgroups (the
 // hardware deals them round-robin) each walk a contiguous run, GR row tiles of one token tile
 // after another.  False: none (the grid is rounded up).  S: scan[256], tile_z, tile_t0, tile_n.
+// (dense) tile number s of the NT x NR: its row tile and its first token
+__device__ __forceinline__ void tile_place(int s, int NT, int NR, int& rt, int& tt) {
+  const int rg = s / (GR * NT), rem = s - rg * GR * NT, nr = min(GR, NR - rg * GR);
+  tt = rem / nr;
+  rt = rg * GR + (rem - tt * nr);
+}
+
+// LIMIT >= 0: only the tiles before it are dealt out (a multiple of 8; the workgroups from it on take parts of the rest)
 template <int TM, int TN, typename SM>
-__device__ __forceinline__ bool pick_tile(const BfParams& p, SM& S, long& tok0, int& ntok, int& rt, const u8*& w) {
+__device__ __forceinline__ bool pick_tile(const BfParams& p, SM& S, long& tok0, int& ntok, int& rt, const u8*& w, int limit = -1) {
   const int t = threadIdx.x;
   const int NR = (p.rows + TM - 1) / TM;
   int NT;
@@ -302,13 +315,12 @@ __device__ __forceinline__ bool pick_tile(const BfParams& p, SM& S, long& tok0, 
   } else {
     NT = (p.ntok + TN - 1) / TN;
   }
-  const int total = NT * NR, per = (total + 7) / 8;
+  const int total = limit >= 0 ? limit : NT * NR, per = (total + 7) / 8;
   const int L = blockIdx.x, j = L >> 3;
   const int s = (L & 7) * per + j;
   if (j >= per || s >= total) return false;
-  const int rg = s / (GR * NT), rem = s - rg * GR * NT, nr = min(GR, NR - rg * GR);
-  const int tt = rem / nr;
-  rt = rg * GR + (rem - tt * nr);
+  int tt;
+  tile_place(s, NT, NR, rt, tt);
   if (p.ptrs) {
     if (t < p.ne) {
       const u32 incl = S.scan[t], tiles = (p.counts[t] + TN - 1) / TN, excl = incl - tiles;
@@ -344,7 +356,19 @@ __global__ __launch_bounds__((bf16_threads<TM, NB>()), (TM * TN == 65536 ? 1 : T
   const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
 
   long tok0; int ntok, rt; const u8* w = p.w;
-  if (!pick_tile<TM, TN>(p, S, tok0, ntok, rt, w)) return;
+  int sb0 = 0, sb1 = p.cols / 256;                         // the super-blocks this workgroup multiplies
+  const bool part = p.ksplit > 1 && (int)blockIdx.x >= p.split_from;
+  if (part) {
+    const int q = (int)blockIdx.x - p.split_from, ti = q / p.ksplit, ky = q - ti * p.ksplit;
+    const int NT = (p.ntok + TN - 1) / TN, NR = (p.rows + TM - 1) / TM;
+    if (p.split_from + ti >= NT * NR) return;
+    int tt;
+    tile_place(p.split_from + ti, NT, NR, rt, tt);
+    tok0 = (long)tt * TN;
+    ntok = min(TN, p.ntok - (int)tok0);
+    sb0 = (int)((long)ky * sb1 / p.ksplit);
+    sb1 = (int)((long)(ky + 1) * sb1 / p.ksplit);
+  } else if (!pick_tile<TM, TN>(p, S, tok0, ntok, rt, w, p.ksplit > 1 ? p.split_from : -1)) return;
   const int r0 = rt * TM;
   if (FMT == ILT_IQ2_XXS) {
     if (t < 256) iq2_tables_fill(S.iq2, t);
@@ -407,10 +431,10 @@ __global__ __launch_bounds__((bf16_threads<TM, NB>()), (TM * TN == 65536 ? 1 : T
   // ks+1's weights into the other weight slab; a set is reloaded, with the half two ahead,
   // right after its last step is dequantized, four steps before it is needed again.
   WRaw<FMT> rawa[NE], rawb[NE];
-  load_raw(rawa, 0);
-  issue_x(0, 0);
-  load_raw(rawb, 1);
-  issue_x(1, 1);
+  load_raw(rawa, 2 * sb0);
+  issue_x(0, 8 * sb0);
+  load_raw(rawb, 2 * sb0 + 1);
+  issue_x(1, 8 * sb0 + 1);
   int st0 = 0, st1 = 1, st2 = 2;                           // ring: the step's slab, the next step's, the one after
   dequant_to(rawa, 0, 0, 0);
 
@@ -447,7 +471,7 @@ __global__ __launch_bounds__((bf16_threads<TM, NB>()), (TM * TN == 65536 ? 1 : T
     }
     const int s = st0; st0 = st1; st1 = st2; st2 = s;
   };
-  for (int ks = 0; ks < nk; ks += 8) {     // one super-block of 256 columns
+  for (int ks = 8 * sb0; ks < 8 * sb1; ks += 8) {     // one super-block of 256 columns
     step(ks + 0, std::integral_constant<int, 0>{});
     step(ks + 1, std::integral_constant<int, 1>{});
     step(ks + 2, std::integral_constant<int, 2>{});
@@ -460,7 +484,43 @@ __global__ __launch_bounds__((bf16_threads<TM, NB>()), (TM * TN == 65536 ? 1 : T
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // the tail's redundant loads: nothing may land in LDS after the workgroup ends
 
-  store_tile<NA, NB>(acc, p, tok0, ntok, r0, wt0, wr0, l32, lh);
+  if (part) {              // the sums of this run of columns, the whole tile (what lies past the matrix or the tokens: never read)
+    BfParams q = p;
+    q.y = p.part + (long)((int)blockIdx.x - p.split_from) * (TM * TN); q.ldy = TM; q.rows = TM; q.bias = nullptr; q.acc = 0;
+    store_tile<NA, NB>(acc, q, 0, TN, 0, wt0, wr0, l32, lh);
+  } else {
+    store_tile<NA, NB>(acc, p, tok0, ntok, r0, wt0, wr0, l32, lh);
+  }
+}
+
+// The split tiles' parts added up, part after part, and written to y as store_tile writes a tile (bias, acc).
+// Grid (TM * TN / 1024, tiles): a thread four rows of a token.
+template <int TM, int TN>
+__global__ __launch_bounds__(256) void bf16_split_sum_kernel(BfParams p) {
+  const int ti = blockIdx.y, e = ((int)blockIdx.x * 256 + (int)threadIdx.x) * 4, tok = e / TM, row = e - tok * TM;
+  const int NT = (p.ntok + TN - 1) / TN, NR = (p.rows + TM - 1) / TM;
+  int rt, tt;
+  tile_place(p.split_from + ti, NT, NR, rt, tt);
+  const long tk = (long)tt * TN + tok;
+  if (tk >= p.ntok) return;
+  const float* src = p.part + (long)ti * p.ksplit * (TM * TN) + e;
+  float4 s = *(const float4*)src;
+  for (int k = 1; k < p.ksplit; k++) {
+    const float4 v = *(const float4*)(src + (long)k * (TM * TN));
+    s.x = s.x + v.x; s.y = s.y + v.y; s.z = s.z + v.z; s.w = s.w + v.w;
+  }
+  const float o[4] = {s.x, s.y, s.z, s.w};
+  float* y = p.y + tk * p.ldy;
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+    const int r = rt * TM + row + i;
+    if (r < p.rows) {
+      float v = o[i];
+      if (p.bias) v = v + p.bias[r];
+      if (p.acc) v = y[r] + v;
+      y[r] = v;
+    }
+  }
 }
 
 // ---- the grouped product with the weights dequantized into MFMA operands ------------------------
@@ -1830,10 +1890,82 @@ __global__ __launch_bounds__(256) void q8k_bf16_kernel(const i8* __restrict__ xq
   *(int4*)dst = v;
 }
 
+// Room for the split tiles' parts: a buffer per (device, stream) -- launches on two streams may overlap, and each needs
+// its parts to itself -- grown when a launch needs more, never inside a stream capture; sixteen of them at most.  A
+// launch that gets no room (capturing with too little, the table full, no memory) goes unsplit.
+struct PartRoom { int dev; hipStream_t st; float* p; size_t bytes; };
+std::mutex g_part_mu;
+PartRoom g_part[16] = {};
+int g_nparts = 0;
+float* part_room(size_t bytes, hipStream_t st) {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return nullptr;
+  std::lock_guard<std::mutex> lock(g_part_mu);
+  PartRoom* r = nullptr;
+  for (int i = 0; i < g_nparts; i++) if (g_part[i].dev == dev && g_part[i].st == st) r = &g_part[i];
+  if (r && r->bytes >= bytes) return r->p;
+  hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(st, &cs) != hipSuccess || cs != hipStreamCaptureStatusNone) { (void)hipGetLastError(); return nullptr; }
+  if (!r) {
+    if (g_nparts == 16) return nullptr;
+    r = &g_part[g_nparts++];
+    *r = {dev, st, nullptr, 0};
+  }
+  if (r->p) {
+    if (hipStreamSynchronize(st) != hipSuccess) return nullptr;        // this stream's earlier launches may still use the old room
+    (void)hipFree(r->p);
+    r->p = nullptr; r->bytes = 0;
+  }
+  const size_t want = bytes + bytes / 4;
+  if (hipMalloc((void**)&r->p, want) != hipSuccess) { (void)hipGetLastError(); r->p = nullptr; return nullptr; }
+  r->bytes = want;
+  return r->p;
+}
+
+// The tiles past the last whole round over the 256 CUs would take a round of their own (272 tiles: two rounds, the second
+// one sixteenth full).  They are split instead: KSPLIT workgroups a tile, each a run of the columns' super-blocks, dealt
+// over all CUs beside the whole rounds' tiles, and a small kernel adds a tile's parts.  Chosen where the model -- rounds
+// of whole tiles plus rounds of parts (split_rounds) -- says it saves a twentieth or more.
+// ILT_BF16_SPLITK=0: never (tests).
+// (a part: its share of the columns and what every workgroup spends besides its columns, about two super-blocks' worth;
+// the parts' round as such -- they start when the whole tiles' last round ends, write their sums, and the adding kernel
+// reads them back -- about 0.3 of a tile's time, measured on 17408 x 5120 at 512 to 4096 tokens)
+inline double split_rounds(long long full, long long lo, int k, int nsb) {
+  return (double)(full / 256) + (double)((lo * k + 255) / 256) * (1.0 / k + 2.0 / nsb) + 0.3;
+}
+inline int choose_ksplit(long long total, int nsb, long long& split_from) {
+  const char* force = getenv("ILT_BF16_SPLITK");
+  if (force && atoi(force) == 0) return 0;
+  const long long full = total / 256 * 256, lo = total - full;
+  if (lo == 0 || nsb < 2) return 0;
+  const double plain = (double)((total + 255) / 256);
+  double best = plain; int bk = 0;
+  for (int k = 2; k <= nsb && k <= 32; k++) {
+    const double c = split_rounds(full, lo, k, nsb);
+    if (c < best - 1e-9) { best = c; bk = k; }
+  }
+  if (bk == 0 || best > plain * 0.95) return 0;
+  split_from = full;
+  return bk;
+}
+
 template <int FMT, int TM, int TN, int NB>
-hipError_t launch_bf16(const BfParams& p, long long token_tiles, hipStream_t st) {
+hipError_t launch_bf16(const BfParams& p0, long long token_tiles, hipStream_t st) {
+  BfParams p = p0;
   const long long total = token_tiles * ((p.rows + TM - 1) / TM), per = (total + 7) / 8;
   if (per * 8 > 0x7FFFFFFFLL) return hipErrorInvalidValue;
+  long long split_from = 0;
+  const int k = p.ptrs ? 0 : choose_ksplit(total, p.cols / 256, split_from);
+  if (k > 1) {
+    const long long lo = total - split_from;
+    float* room = (size_t)lo * k * TM * TN * 4 <= ((size_t)256 << 20) ? part_room((size_t)lo * k * TM * TN * 4, st) : nullptr;
+    if (room) {
+      p.ksplit = k; p.split_from = (int)split_from; p.part = room;
+      hipLaunchKernelGGL((gemm_bf16_kernel<FMT, TM, TN, NB>), dim3((unsigned)(split_from + lo * k)), dim3(bf16_threads<TM, NB>()), 0, st, p);
+      hipLaunchKernelGGL((bf16_split_sum_kernel<TM, TN>), dim3(TM * TN / 1024, (unsigned)lo), dim3(256), 0, st, p);
+      return hipGetLastError();
+    }
+  }
   hipLaunchKernelGGL((gemm_bf16_kernel<FMT, TM, TN, NB>), dim3((unsigned)(per * 8)), dim3(bf16_threads<TM, NB>()), 0, st, p);
   return hipGetLastError();
 }
@@ -1879,14 +2011,21 @@ hipError_t ilt_k_gemm_bf16(int fmt, const uint8_t* w, long long row_bytes, int r
   p.ldy = rows;
   // Larger tiles fetch and dequantize less per product but leave more of the last round of
   // workgroups idle.  Cost of a variant: rounds over the 256 CUs x tile area / its measured
-  // relative rate (128x128 0.85, 128x256 1.0, 256x256 1.1).
+  // relative rate (128x128 0.85, 128x256 1.0, 256x256 1.36: a CU's 58-63, 53.7 and 39.5 us for 128 rows x 128 tokens x
+  // 5120 columns of Q6_K, with as many workgroups on it as fit).
   const long long t128 = (ntok + 127) / 128, t256 = (ntok + 255) / 256, r256 = (rows + 255) / 256, r128 = (rows + 127) / 128;
   const char* force = getenv("ILT_BF16_TILE");     // "1".."3": that variant whatever the shape (tests)
   int tile = force ? atoi(force) : 0;
   if (tile < 1 || tile > 3) {
-    const double c1 = (double)((t128 * r128 + 255) / 256) * 1.0 / 0.85;
-    const double c2 = (double)((t256 * r128 + 255) / 256) * 2.0 / 1.0;
-    const double c3 = (double)((t256 * r256 + 255) / 256) * 4.0 / 1.1;
+    // (rounds: whole ones, and the parts' where the last round's tiles are split, see choose_ksplit)
+    auto rounds = [&](long long tiles) {
+      long long from = 0;
+      const int k = choose_ksplit(tiles, cols / 256, from);
+      return k > 1 ? split_rounds(from, tiles - from, k, cols / 256) : (double)((tiles + 255) / 256);
+    };
+    const double c1 = rounds(t128 * r128) * 1.0 / 0.85;
+    const double c2 = rounds(t256 * r128) * 2.0 / 1.0;
+    const double c3 = rounds(t256 * r256) * 4.0 / 1.36;
     tile = c3 <= c2 && c3 <= c1 ? 3 : c2 <= c1 ? 2 : 1;
   }
   if (tile == 3) return dispatch_bf16<256, 256, 2>(fmt, p, t256, st);

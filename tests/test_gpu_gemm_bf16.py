@@ -102,6 +102,55 @@ def test_dense_bf16_product_within_tolerance(dev, monkeypatch, qtype, rows, cols
     m.free()
 
 
+@pytest.mark.parametrize("qtype,rows,cols,n,tile", [
+    (synth.Q6_K, 8704, 2048, 512, 1),      # 272 tiles of 128 x 128: a whole round over the CUs, and 16 tiles split eight ways
+    (synth.Q6_K, 4352, 2048, 500, 2),      # 68 tiles of 128 x 256, all split; ragged tokens
+    (synth.Q4_K, 2560, 9728, 512, 0),      # a decoder's down product on a prompt's chunk: few tiles, many columns, 38 super-blocks split unevenly
+    (synth.Q2_K, 700, 2048, 130, 0),       # ragged rows and tokens
+])
+def test_tiles_split_over_the_columns(dev, monkeypatch, qtype, rows, cols, n, tile):
+    """Where a product's tiles do not fill a round over the CUs, the tiles of the last round are split over the columns'
+    super-blocks and their parts added by a second kernel: the same product as unsplit but for the order of fp32 sums
+    (within 1e-5 of the largest output), within the path's tolerance of the CPU path on a sample of the tokens, and
+    bias and accumulation as the unsplit store applies them."""
+    from illatio_amd import dense, hip
+    if tile:
+        monkeypatch.setenv("ILT_BF16_TILE", str(tile))
+    else:
+        monkeypatch.delenv("ILT_BF16_TILE", raising=False)
+    rng = synth.make_rng(qtype * 13 + rows + n)
+    w = synth.weights(qtype, rows, cols, rng)
+    x = synth.activations((n, cols), rng)
+    bias = synth.activations(rows, rng)
+    m = upload(dev, qtype, rows, cols, w)
+    xf, bb = hip.hip_upload_new(dev, x), hip.hip_upload_new(dev, bias)
+    xb = dense.cvt_bf16(dev, xf, x.size)
+    out = {}
+    for split in ("0", None):
+        if split is None:
+            monkeypatch.delenv("ILT_BF16_SPLITK", raising=False)
+        else:
+            monkeypatch.setenv("ILT_BF16_SPLITK", split)
+        y = hip.hip_upload_new(dev, np.full(n * rows + 64, 3.0, np.float32))
+        dense.cmat_mul_bf16(dev, m, xb, y, n)
+        a = hip.hip_floats(y, n * rows + 64)
+        assert np.all(a[n * rows:] == 3.0)                       # nothing past the last token's rows
+        dense.cmat_mul_bf16(dev, m, xb, y, n, bias=bb, acc=True)
+        b = hip.hip_floats(y, n * rows).reshape(n, rows)
+        a = a[:n * rows].reshape(n, rows)
+        assert np.array_equal(b, a + (a + bias[None, :]))
+        out[split] = a
+        hip.hip_free(y)
+    assert np.abs(out[None] - out["0"]).max() <= 1e-5 * np.abs(out["0"]).max()
+    assert not np.array_equal(out[None], out["0"])               # (the split was taken: the sums' order shows somewhere)
+    pick = np.unique(np.concatenate([np.arange(0, n, 37), [n - 1]]))
+    cpu = orc.matmul(qtype, w, rows, cols, x[pick], nthreads=16)
+    assert np.abs(out[None][pick] - cpu).max() <= TOL_VS_CPU * np.abs(cpu).max()
+    for b_ in (xf, xb, bb):
+        hip.hip_free(b_)
+    m.free()
+
+
 @pytest.mark.parametrize("two_pass", [False, True])
 def test_output_head_keeps_the_cpu_paths_top_token(dev, two_pass):
     """128 positions through an output head (Q6_K, config 2's width, 8192 of its rows): the
@@ -229,9 +278,11 @@ def test_moe_prefill_chunk_bf16_within_tolerance(dev, monkeypatch, ne, d, ff, nu
 @pytest.mark.parametrize("split", [None, "0", "128"])      # tiles chosen by shape (256-tiles + 128-tiles for the rows left over), 256 only, 128 only
 def test_two_pass_bf16_product(dev, monkeypatch, qtype, rows, cols, n, split):
     """dequant_bf16 writes each weight as the one-pass kernel rounds it; mm_bf16 on that copy adds
-    the same products in the same order, so it returns the one-pass kernel's numbers."""
+    the same products in the same order, so it returns the one-pass kernel's numbers (the one-pass kernel
+    with its tiles whole: split over the columns it adds a tile's parts in another order)."""
     from illatio_amd import dense, hip
     monkeypatch.delenv("ILT_BF16_TILE", raising=False)
+    monkeypatch.setenv("ILT_BF16_SPLITK", "0")
     if split is None:
         monkeypatch.delenv("ILT_BF16_PLAIN_SPLIT", raising=False)
     else:
