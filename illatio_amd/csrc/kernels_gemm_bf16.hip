@@ -987,10 +987,10 @@ template <> struct I8p<ILT_Q2_K> {
   }
 };
 
-struct I8pSmem {
+template <int TM> struct I8pSmemT {
   __align__(16) u8 xs[3][128 * 64];       // the tokens' quants, 64 columns a step
-  __align__(16) u8 wh[2][128 * 64];       // the rows' hi plane, the step's and the next step's
-  __align__(16) u8 wl[2][128 * 64];       // lo plane
+  __align__(16) u8 wh[2][TM * 64];        // the rows' hi plane, the step's and the next step's
+  __align__(16) u8 wl[2][TM * 64];        // lo plane
   float wd[128], wdm[128];                // of the super-block: d (and Q4_K's dmin) of the rows,
   float xd[128];                          //   the tokens' scales
   int cx[128];                            //   and KCX * the sum of their quants
@@ -1004,6 +1004,7 @@ struct I8pSmem {
   u32 scan[256];
   int tile_z, tile_t0, tile_n;
 };
+typedef I8pSmemT<128> I8pSmem;
 
 // IQ2_XXS: a block's eight groups of 32 weights add (float(sumi) * (0.5 + scale)) alternately to two sums,
 // fa (even groups) and fb (odd), then sum += (d*yd) * (fa + fb) (iquant.lisp:161-215).  Every term is a
@@ -1024,7 +1025,7 @@ template <> struct I8p<ILT_IQ2_XXS> {
     r.d = ilt_bld2(rw, rowoff + (u32)(hb >> 1) * 66);
   }
   static __device__ __forceinline__ float d_of(const Raw& r) { return ilt_h2f((u16)r.d); }
-  static __device__ __forceinline__ void planes(const Raw& r, int J, int q4, int* hi, int* lo, const I8pSmem& S) {
+  template <typename SM> static __device__ __forceinline__ void planes(const Raw& r, int J, int q4, int* hi, int* lo, const SM& S) {
     const u32 idx = (u32)r.g[J & 1].x, aux = (u32)r.g[J & 1].y;
     const int mult = 2 * (int)(aux >> 28) + 1;
     const u32 c0 = 1408u * 0x10001u;
@@ -1056,12 +1057,15 @@ __device__ __forceinline__ void ilt_lds_st8_untracked(void* p, u32 a, u32 b) {
 
 // 128 rows x 128 tokens a workgroup of eight waves (one workgroup a CU, two waves a SIMD: a
 // wave's two planes of integer sums, its float sums and the raw bytes leave no room for more);
-// wave w: rows 32*(w/2).., tokens 64*(w%2)...
-template <int FMT, bool GROUPED>
-__global__ __launch_bounds__(512, 1) void gemm_i8p_kernel(BfParams p) {
+// wave w: rows 32*(w/2).., tokens 64*(w%2)...  TM 64 (dense): 64 rows x 128 tokens a workgroup of four waves, two or
+// three workgroups a CU -- for products whose 128-row tiles are fewer than the CUs, or leave the last round over them
+// mostly empty (a prompt's chunk on a small model's matrices); the same sums in the same order.
+template <int FMT, bool GROUPED, int TM = 128>
+__global__ __launch_bounds__(4 * TM, TM == 128 ? 1 : 2) void gemm_i8p_kernel(BfParams p) {
   typedef I8p<FMT> F;
   typedef typename F::Raw Raw;
-  constexpr int TM = 128, TN = 128, NA = 2, NI = 1;
+  static_assert(TM == 128 || (TM == 64 && !GROUPED), "the grouped wave layout takes eight waves");
+  constexpr int TN = 128, NA = 2, THREADS = 4 * TM, NI = 512 / THREADS;
   // Q6_K needs the quants' sum over a block and IQ2_XXS over its even and odd groups (d4_mm_id_iq2_xxs has no argument for
   // the sums of 16 anyway): both are added up from the slabs in LDS, which saves four 16-byte loads a thread and block.
   constexpr bool XSLAB = FMT == ILT_IQ2_XXS || FMT == ILT_Q6_K;
@@ -1069,8 +1073,9 @@ __global__ __launch_bounds__(512, 1) void gemm_i8p_kernel(BfParams p) {
   constexpr bool TWO = F::PLANES == 2;
   constexpr bool SPLIT = FMT == ILT_IQ2_XXS;                 // the first and the second 32 columns of a step have sums of their own
   constexpr int KW = 64;                                     // columns a step
-  __shared__ I8pSmem S;
-  // Q2_K has no hi plane: its room holds the minimums' operands (sixteen groups: 16 bytes a row or token)
+  __shared__ I8pSmemT<TM> S;
+  // Q2_K has no hi plane: its room holds the minimums' operands (sixteen groups: 16 bytes a row or token; 6 KB of the
+  // hi plane's two slabs, 8 KB at 64 rows)
   int4* const q2_wmn = (int4*)S.wh[0];
   int4* const q2_bh = q2_wmn + 128;
   int4* const q2_bl = q2_bh + 128;
@@ -1109,7 +1114,12 @@ __global__ __launch_bounds__(512, 1) void gemm_i8p_kernel(BfParams p) {
   const u32 wrowoff = (u32)((long long)min(r0 + wrow, p.rows - 1) * p.row_bytes);
   const u32 wdst = slab_off(wrow, q4);
   const u8* xbase = (const u8*)ilt_uniform_ptr((const i8*)p.x + tok0 * (long)p.cols);
-  const u32 xoff = (u32)min(t >> 2, ntok - 1) * (u32)p.cols + 16 * ((t & 3) ^ (int)slab_swz(t >> 2));   // piece t of a slab
+  u32 xoff[NI];                                              // piece (wave * NI + i) * 64 + lane of a slab: token piece / 4, part piece % 4
+#pragma unroll
+  for (int i = 0; i < NI; i++) {
+    const int P = (wave * NI + i) * 64 + lane;
+    xoff[i] = (u32)min(P >> 2, ntok - 1) * (u32)p.cols + 16 * ((P & 3) ^ (int)slab_swz(P >> 2));
+  }
   const int nk = p.cols / KW, nsb = p.cols / 256;
   // a token's constants for a super-block, by thread t & 127 (every wave loads, so that all count the same loads)
   const long ctok = tok0 + min(t & 127, ntok - 1);
@@ -1180,7 +1190,10 @@ __global__ __launch_bounds__(512, 1) void gemm_i8p_kernel(BfParams p) {
     }
   };
   auto load_raw = [&](Raw& r, int hb) { F::load(r, rw, wrowoff, hb, q4); };       // half super-block hb of the thread's row
-  auto issue_x = [&](int stage, int ks) { ilt_g2lds16(xbase + ks * KW + xoff, S.xs[stage] + wave * 1024); };
+  auto issue_x = [&](int stage, int ks) {
+#pragma unroll
+    for (int i = 0; i < NI; i++) ilt_g2lds16(xbase + ks * KW + xoff[i], S.xs[stage] + (wave * NI + i) * 1024);
+  };
   // the thread's 16 weights of step J of a super-block, out of the set that holds its half, into a pair of slabs
   auto dequant_to = [&](const Raw& r, int J, int slab) {
     int hi[4], lo[4];
@@ -1191,7 +1204,7 @@ __global__ __launch_bounds__(512, 1) void gemm_i8p_kernel(BfParams p) {
 
   v16f sum[NA][1];
   v16i_ ah[SPLIT ? 2 : 1][NA], al[SPLIT ? 2 : 1][NA];
-  int xsum = 0;                                              // IQ2_XXS, Q6_K: see the step
+  int xsum[NI] = {};                                         // IQ2_XXS, Q6_K: see the step
 #pragma unroll
   for (int a = 0; a < NA; a++)
 #pragma unroll
@@ -1240,15 +1253,19 @@ __global__ __launch_bounds__(512, 1) void gemm_i8p_kernel(BfParams p) {
     const v16i_ zero = {};
     if constexpr (XSLAB) {
       // the sums of the tokens' quants over the block (IQ2_XXS: over its even and its odd groups), from the slabs: thread t
-      // adds piece t & 3 of token t / 4; pieces 0 and 1 are the step's even group, 2 and 3 its odd one
-      const int4 xv = ilt_lds_ld16(xs + slab_off(t >> 2, t & 3));
-      int sp = __builtin_amdgcn_sdot4(xv.x, 0x01010101, 0, false);
-      sp = __builtin_amdgcn_sdot4(xv.y, 0x01010101, sp, false);
-      sp = __builtin_amdgcn_sdot4(xv.z, 0x01010101, sp, false);
-      sp = __builtin_amdgcn_sdot4(xv.w, 0x01010101, sp, false);
-      sp += __shfl_xor(sp, 1);
-      if constexpr (!SPLIT) sp += __shfl_xor(sp, 2);
-      xsum = J == 0 ? sp : xsum + sp;
+      // adds piece t & 3 of token t / 4 (and of token t / 4 + 64 with four waves); pieces 0 and 1 are the step's even
+      // group, 2 and 3 its odd one
+#pragma unroll
+      for (int i = 0; i < NI; i++) {
+        const int4 xv = ilt_lds_ld16(xs + slab_off((t >> 2) + (THREADS / 4) * i, t & 3));
+        int sp = __builtin_amdgcn_sdot4(xv.x, 0x01010101, 0, false);
+        sp = __builtin_amdgcn_sdot4(xv.y, 0x01010101, sp, false);
+        sp = __builtin_amdgcn_sdot4(xv.z, 0x01010101, sp, false);
+        sp = __builtin_amdgcn_sdot4(xv.w, 0x01010101, sp, false);
+        sp += __shfl_xor(sp, 1);
+        if constexpr (!SPLIT) sp += __shfl_xor(sp, 2);
+        xsum[i] = J == 0 ? sp : xsum[i] + sp;
+      }
     }
 #pragma unroll
     for (int kk = 0; kk < 2; kk++) {
@@ -1278,8 +1295,11 @@ __global__ __launch_bounds__(512, 1) void gemm_i8p_kernel(BfParams p) {
     }
     if constexpr (XSLAB) {
       if (J == 3) {        // the block's sums of quants, for everyone's terms below
-        if ((t & 3) == 0) ilt_lds_st4_untracked(&S.cx[t >> 2], (u32)(F::KCX * xsum));
-        if (SPLIT && (t & 3) == 2) ilt_lds_st4_untracked(&cxo[t >> 2], (u32)(F::KCX * xsum));
+#pragma unroll
+        for (int i = 0; i < NI; i++) {
+          if ((t & 3) == 0) ilt_lds_st4_untracked(&S.cx[(t >> 2) + (THREADS / 4) * i], (u32)(F::KCX * xsum[i]));
+          if (SPLIT && (t & 3) == 2) ilt_lds_st4_untracked(&cxo[(t >> 2) + (THREADS / 4) * i], (u32)(F::KCX * xsum[i]));
+        }
         ilt_barrier_lds();
       }
     }
@@ -2075,13 +2095,31 @@ hipError_t ilt_k_gemm_bf16_id_glu(int fmt, const uint64_t* ptrs, long long add_g
   return launch_regb<ILT_IQ2_XXS, true>(p, total_rows / 128 + ne, st);
 }
 
+// 64-row tiles (dense) where the 128-row tiles would leave CUs idle: fewer tiles than one and a half rounds over the
+// 256 CUs, or a last round less than half full.  ILT_I8P_TM (tests): 64 or 128 whatever the shape.
+static int i8p_tile_rows(long long tiles128) {
+  const char* force = getenv("ILT_I8P_TM");
+  if (force && (atoi(force) == 64 || atoi(force) == 128)) return atoi(force);
+  const long long rem = tiles128 % 256;
+  return (tiles128 < 384 || (tiles128 < 1024 && rem != 0 && rem < 128)) ? 64 : 128;
+}
+
 template <bool GROUPED>
-static hipError_t launch_i8p(int fmt, const BfParams& p, long long token_tiles, hipStream_t st) {
+static hipError_t launch_i8p(int fmt, const BfParams& p, long long token_tiles, hipStream_t st, int tm = 128) {
   if ((fmt != ILT_Q6_K && fmt != ILT_Q4_K && fmt != ILT_Q2_K && fmt != ILT_IQ2_XXS) || p.cols % 256 != 0 || (long long)p.rows * 1024 >= 0x7FFFFFFFLL)
     return hipErrorInvalidValue;
-  const long long total = token_tiles * ((p.rows + 127) / 128), per = (total + 7) / 8;
+  const long long total = token_tiles * ((p.rows + tm - 1) / tm), per = (total + 7) / 8;
   if (per * 8 > 0x7FFFFFFFLL) return hipErrorInvalidValue;
   const dim3 grid((unsigned)(per * 8));
+  if constexpr (!GROUPED) {
+    if (tm == 64) {
+      if (fmt == ILT_Q6_K) hipLaunchKernelGGL((gemm_i8p_kernel<ILT_Q6_K, false, 64>), grid, dim3(256), 0, st, p);
+      else if (fmt == ILT_Q4_K) hipLaunchKernelGGL((gemm_i8p_kernel<ILT_Q4_K, false, 64>), grid, dim3(256), 0, st, p);
+      else if (fmt == ILT_Q2_K) hipLaunchKernelGGL((gemm_i8p_kernel<ILT_Q2_K, false, 64>), grid, dim3(256), 0, st, p);
+      else hipLaunchKernelGGL((gemm_i8p_kernel<ILT_IQ2_XXS, false, 64>), grid, dim3(256), 0, st, p);
+      return hipGetLastError();
+    }
+  }
   if (fmt == ILT_Q6_K) hipLaunchKernelGGL((gemm_i8p_kernel<ILT_Q6_K, GROUPED>), grid, dim3(512), 0, st, p);
   else if (fmt == ILT_Q4_K) hipLaunchKernelGGL((gemm_i8p_kernel<ILT_Q4_K, GROUPED>), grid, dim3(512), 0, st, p);
   else if (fmt == ILT_Q2_K) hipLaunchKernelGGL((gemm_i8p_kernel<ILT_Q2_K, GROUPED>), grid, dim3(512), 0, st, p);
@@ -2097,7 +2135,8 @@ hipError_t ilt_k_gemm_i8_planes(int fmt, const uint8_t* w, long long row_bytes, 
   BfParams p = {};
   p.w = w; p.rows = rows; p.cols = cols; p.row_bytes = row_bytes; p.x = (const u16*)xq; p.xd = xd; p.bsums = bsums;
   p.y = y; p.bias = bias; p.acc = acc; p.ntok = ntok; p.ldy = ldy;
-  return launch_i8p<false>(fmt, p, (ntok + 127) / 128, st);
+  const long long tt = (ntok + 127) / 128;
+  return launch_i8p<false>(fmt, p, tt, st, i8p_tile_rows(tt * ((rows + 127) / 128)));
 }
 
 // Up to three matrices of one format (Q6_K, Q4_K, Q2_K) on the same tokens in one launch: their row tiles one after
@@ -2108,17 +2147,20 @@ hipError_t ilt_k_gemm_i8_planes_n(int fmt, int nmat, const uint8_t* const* ws, c
                                   hipStream_t st) {
   if (nmat < 2 || nmat > 3 || ntok < 96 || (fmt != ILT_Q6_K && fmt != ILT_Q4_K && fmt != ILT_Q2_K) || cols % 256 != 0) return hipErrorNotSupported;
   BfParams p = {};
-  long long tiles = 0;
+  long long tiles128 = 0;
   for (int m = 0; m < nmat; m++) {
     if (rows[m] < 128 || rows[m] >= (1 << 21) || (long long)rows[m] * row_bytes >= 0x7FFFFFFFLL) return hipErrorNotSupported;
     p.mw[m] = ws[m]; p.mrows[m] = rows[m]; p.my[m] = ys[m]; p.mbias[m] = biases ? biases[m] : nullptr;
-    tiles += (rows[m] + 127) / 128;
+    tiles128 += (rows[m] + 127) / 128;
   }
-  if (tiles * 128 >= (1 << 21)) return hipErrorNotSupported;
+  if (tiles128 * 128 >= (1 << 21)) return hipErrorNotSupported;
+  const int tm = i8p_tile_rows(tiles128 * ((ntok + 127) / 128));
+  long long tiles = 0;
+  for (int m = 0; m < nmat; m++) tiles += (rows[m] + tm - 1) / tm;
   p.nmulti = nmat;
-  p.w = ws[0]; p.rows = (int)(tiles * 128); p.cols = cols; p.row_bytes = row_bytes; p.x = (const u16*)xq; p.xd = xd; p.bsums = bsums;
+  p.w = ws[0]; p.rows = (int)(tiles * tm); p.cols = cols; p.row_bytes = row_bytes; p.x = (const u16*)xq; p.xd = xd; p.bsums = bsums;
   p.y = ys[0]; p.acc = acc; p.ntok = ntok; p.ldy = rows[0];
-  return launch_i8p<false>(fmt, p, (ntok + 127) / 128, st);
+  return launch_i8p<false>(fmt, p, (ntok + 127) / 128, st, tm);
 }
 
 hipError_t ilt_k_planes_i8(int fmt, const uint8_t* w, long long row_bytes, int rows, int cols, uint8_t* wh, uint8_t* wl, float* wdf,

@@ -38,17 +38,22 @@ CASES = [
 
 
 # ILT_I8_PLANES: "0" = the 64 x 64 kernel always, "1" = always the pipelined kernels (Q6_K and Q4_K as two int8 planes, Q8_0
-# a block per MFMA), else only with enough tokens and rows to fill their 128 x 128 tiles
-@pytest.mark.parametrize("planes", [None, "0", "1"])
+# a block per MFMA), else only with enough tokens and rows to fill their 128 x 128 tiles.  The planes' kernel takes 64-row
+# tiles where 128-row tiles would leave most CUs idle -- every shape here -- and ILT_I8P_TM=128 holds it to the large tile
+# ("1/128").
+@pytest.mark.parametrize("planes", [None, "0", "1", "1/128"])
 @pytest.mark.parametrize("qtype,rows,cols,n", CASES)
 def test_dense_prefill_equals_cpu_matmul_bit_for_bit(dev, monkeypatch, qtype, rows, cols, n, planes):
     from illatio_amd import dense, hip
+    monkeypatch.delenv("ILT_I8P_TM", raising=False)
     if planes is None:
         monkeypatch.delenv("ILT_I8_PLANES", raising=False)
-    elif cols % 64:
+    elif cols % 64 or (planes == "1/128" and qtype == synth.Q8_0):
         pytest.skip("one kernel for this format")
     else:
-        monkeypatch.setenv("ILT_I8_PLANES", planes)
+        monkeypatch.setenv("ILT_I8_PLANES", planes[0])
+        if planes == "1/128":
+            monkeypatch.setenv("ILT_I8P_TM", "128")
     rng = synth.make_rng(qtype * 31 + rows + n)
     w = synth.weights(qtype, rows, cols, rng)
     x = synth.activations((n, cols), rng)
