@@ -373,8 +373,10 @@ __global__ __launch_bounds__(1024) void attn_step_scores_kernel(const float* __r
 // float of the row from which 32 can be read (the row is padded past npos).  The reads of 32 positions are on their
 // way while the 32 before them are added: left to itself the compiler moves every read down to its use, and a chain
 // of adds then waits for LDS once every 32 positions.
-__device__ __forceinline__ float chain_add_row(const float* col, int npos, int last_read) {
-  float o = 0.0f;
+__device__ __forceinline__ float chain_add_from(float o, const float* col, int npos, int last_read);
+__device__ __forceinline__ float chain_add_row(const float* col, int npos, int last_read) { return chain_add_from(0.0f, col, npos, last_read); }
+// (the same carried on from o: a column that comes in tiles)
+__device__ __forceinline__ float chain_add_from(float o, const float* col, int npos, int last_read) {
   int p = 0;
   typedef float f4v __attribute__((ext_vector_type(4)));
   f4v v0, v1, v2, v3, v4, v5, v6, v7, w0, w1, w2, w3, w4, w5, w6, w7;
@@ -890,6 +892,96 @@ __global__ __launch_bounds__(256) void attn_values_tiled_kernel(const float* __r
   if (tid < tn * 16) out[((long long)(t0 + tt) * nh + h) * hd + 16 * cs + c] = o;
 }
 
+// One token's values for contexts past the one-launch kernel's, with the slice's tiles arriving while the chains run:
+// a workgroup of sixteen waves a (query head, 16 columns); wave 0's first sixteen lanes do nothing but add -- a column
+// each, tile after tile -- and the other fifteen waves bring the tiles in: tile t+1 is multiplied by its positions'
+// scores and stored into the buffer tile t-1 has left while tile t is being added, and tile t+2's loads are on their way
+// from then on.  All sixteen waves take the softmax first (the scores come from attn_step_scores_kernel, raw).  The
+// numbers are attn_values_tiled_kernel<1>'s: every product and every sum the same, in the same order.
+constexpr int kStreamTile = 480, kStreamPitch = kStreamTile + 36;      // (a row: 32 floats of room past a tile for the reads ahead; 4 mod 64)
+__global__ __launch_bounds__(1024) void attn_values_stream_kernel(const float* __restrict__ raw, const float* __restrict__ vc, float* __restrict__ out,
+                                                                  int nh, int nkv, int hd, int pos, int spitch) {
+  extern __shared__ __align__(16) float dyn[];
+  __shared__ float redf[16];
+  __shared__ double redd[17];
+  const int gx = gridDim.x, bx = (gx & 7) ? (int)blockIdx.x : (int)(blockIdx.x & 7) * (gx >> 3) + (int)(blockIdx.x >> 3);
+  const int ns = hd >> 4, h = bx / ns, cs = bx - h * ns, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int npos = pos + 1, group = nh / nkv, kvd = nkv * hd, ko = (h / group) * hd + 16 * cs;
+  float* sc = dyn;                                 // the token's scores, all of them
+  float* vt = dyn + spitch;                        // two tiles of the slice times the scores, a column a row of kStreamPitch
+  const float* rw = raw + (long long)h * spitch;
+  const int ntiles = (npos + kStreamTile - 1) / kStreamTile, li = tid - 64;      // li: a loading thread's number, 0 .. 959
+  // tile's 16-byte pieces li and li + 960: position piece / 4, columns 4 * (piece % 4) ..
+  auto load_tile = [&](int tile, float4 (&r)[2]) {
+    const int p0 = tile * kStreamTile, total = min(kStreamTile, npos - p0) * 4;
+#pragma unroll
+    for (int u = 0; u < 2; u++) {
+      const int i = min(li + 960 * u, total - 1);
+      r[u] = *(const float4*)(vc + (long long)(p0 + (i >> 2)) * kvd + ko + 4 * (i & 3));
+    }
+  };
+  auto store_tile = [&](int tile, const float4 (&r)[2]) {
+    const int p0 = tile * kStreamTile, total = min(kStreamTile, npos - p0) * 4;
+    float* b = vt + (tile & 1) * (16 * kStreamPitch);
+#pragma unroll
+    for (int u = 0; u < 2; u++) {
+      const int i = li + 960 * u;
+      if (i < total) {
+        float* dst = b + (4 * (i & 3)) * kStreamPitch + (i >> 2);
+        const float sp = sc[p0 + (i >> 2)];
+        dst[0] = sp * r[u].x; dst[kStreamPitch] = sp * r[u].y; dst[2 * kStreamPitch] = sp * r[u].z; dst[3 * kStreamPitch] = sp * r[u].w;
+      }
+    }
+  };
+  float4 ra[2], rb[2];
+  if (wave > 0) {
+    load_tile(0, ra);
+    if (ntiles > 1) load_tile(1, rb);
+  }
+  // softmax (attn_softmax's steps over sixteen waves)
+  float mx = -3.402823466e38f;
+  for (int p = tid; p < npos; p += 1024) { const float sv = rw[p]; sc[p] = sv; mx = fmaxf(mx, sv); }
+  mx = wave_max_float(mx);
+  if (lane == 0) redf[wave] = mx;
+  __syncthreads();
+  mx = redf[0];
+#pragma unroll
+  for (int w = 1; w < 16; w++) mx = fmaxf(mx, redf[w]);
+  double part = 0.0;
+  for (int p = tid; p < npos; p += 1024) { const float e = ilt_expf_via_double(sc[p] - mx); sc[p] = e; part += (double)e; }
+  part = wave_sum_double(part);
+  if (lane == 0) redd[wave] = part;
+  __syncthreads();
+  double sum = redd[0];
+#pragma unroll
+  for (int w = 1; w < 16; w++) sum += redd[w];
+  float inv;
+  if (!recip_settled(sum, npos, &inv)) {           // the same in every thread
+    if (tid == 0) { double s2 = 0.0; for (int p = 0; p < npos; p++) s2 += (double)sc[p]; redd[16] = s2; }
+    __syncthreads();
+    inv = (float)(1.0 / redd[16]);
+  }
+  for (int p = tid; p < npos; p += 1024) sc[p] = sc[p] * inv;
+  __syncthreads();                                 // every position's scaled score, for the products
+  if (wave > 0) store_tile(0, ra);
+  float o = 0.0f;
+  const float* col = vt + lane * kStreamPitch;     // (lanes 0 .. 15 of wave 0)
+  auto step = [&](int t, float4 (&next)[2], float4 (&after)[2]) {      // next holds tile t+1; after: free, takes tile t+2
+    __syncthreads();                               // tile t is in place, and tile t-1's chains are through with the other buffer
+    if (wave == 0) {
+      if (lane < 16) o = chain_add_from(o, col + (t & 1) * (16 * kStreamPitch), min(kStreamTile, npos - t * kStreamTile), kStreamPitch - 36);
+    } else {
+      if (t + 1 < ntiles) store_tile(t + 1, next);
+      if (t + 2 < ntiles) load_tile(t + 2, after);
+    }
+  };
+  for (int t = 0; t < ntiles; t += 2) {
+    step(t, rb, ra);
+    if (t + 1 < ntiles) step(t + 1, ra, rb);
+  }
+  if (tid < 16) out[h * hd + 16 * cs + tid] = o;
+}
+
 // ARGMAX (model.lisp:464-468): best = 0; an element replaces the best when it is greater -- so the first of equal
 // maxima, a NaN never (and if v[0] is a NaN nothing replaces it).  Two steps: each workgroup the best of its
 // stretch (every thread's own elements first, eight 16-byte loads in flight, then the threads', a smaller index
@@ -942,6 +1034,21 @@ __global__ __launch_bounds__(256) void argmax_last_kernel(const float* __restric
 __global__ __launch_bounds__(256) void swiglu_rows_kernel(float* __restrict__ a, const float* __restrict__ b, long long n) {
   const long long i = (long long)blockIdx.x * 256 + threadIdx.x;
   if (i < n) { const float g = a[i]; a[i] = (g / (1.0f + ilt_expf_via_double(-g))) * b[i]; }
+}
+
+// one token's values past 2,048 positions (the scores: smax floats a head in scratch, raw)
+hipError_t launch_values_stream(int dev, const float* scratch, const float* vc, float* out, int nh, int nkv, int hd, int pos, int smax,
+                                hipStream_t st) {
+  static bool set[64] = {};
+  const size_t smem = sizeof(float) * ((size_t)smax + 2 * 16 * (size_t)kStreamPitch);
+  if (smem > 152 * 1024 || dev < 0 || dev >= 64) return hipErrorInvalidValue;
+  if (!set[dev]) {
+    const hipError_t e = hipFuncSetAttribute((const void*)attn_values_stream_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 152 * 1024);
+    if (e != hipSuccess) return e;
+    set[dev] = true;
+  }
+  hipLaunchKernelGGL(attn_values_stream_kernel, dim3(nh * (hd / 16)), dim3(1024), smem, st, scratch, vc, out, nh, nkv, hd, pos, smax);
+  return hipGetLastError();
 }
 
 }  // namespace
@@ -1015,7 +1122,8 @@ hipError_t ilt_k_attn_rows(const float* q, const float* kc, const float* vc, flo
       hipLaunchKernelGGL(attn_values_tiled_kernel<16>, gv, dim3(256), smem, st, scratch, vc, out, nh, nkv, hd, pos0, ntok, smax);
     } else {
       hipLaunchKernelGGL(attn_scores_kernel<1>, gs, dim3(1024), 0, st, q, kc, scratch, nh, nkv, hd, pos0, ntok, scale, smax);
-      hipLaunchKernelGGL(attn_values_tiled_kernel<1>, gv, dim3(256), smem, st, scratch, vc, out, nh, nkv, hd, pos0, ntok, smax);
+      const hipError_t e = launch_values_stream(dev, scratch, vc, out, nh, nkv, hd, pos0, smax, st);
+      if (e != hipSuccess) return e;
     }
     return hipGetLastError();
   }
@@ -1109,17 +1217,7 @@ hipError_t ilt_k_attn_step(const float* q, const float* k, const float* v, const
   }
   hipLaunchKernelGGL(attn_step_scores_kernel, dim3(nh, (ctx + 255) / 256), dim3(1024), 0, st, q, k, v, qn, kn, rope, kc, vc, scratch, nh, nkv, hd, rd,
                      pos, eps, neox, scale, smax);
-  if (ctx > 2048) {
-    static bool set[64] = {};
-    if (!set[dev]) {
-      const hipError_t e = hipFuncSetAttribute((const void*)attn_values_tiled_kernel<1>, hipFuncAttributeMaxDynamicSharedMemorySize, 152 * 1024);
-      if (e != hipSuccess) return e;
-      set[dev] = true;
-    }
-    hipLaunchKernelGGL(attn_values_tiled_kernel<1>, dim3(nh * (hd / 16), 1), dim3(256), sizeof(float) * ((size_t)smax + 16 * (size_t)kValPitch), st,
-                       scratch, vc, out, nh, nkv, hd, pos, 1, smax);
-    return hipGetLastError();
-  }
+  if (ctx > 2048) return launch_values_stream(dev, scratch, vc, out, nh, nkv, hd, pos, smax, st);
   hipError_t e = hipErrorInvalidValue;
 #define ILT_ATTN1(NB)                                                                                                                         \
   if (nb == NB) {                                                                                                                             \

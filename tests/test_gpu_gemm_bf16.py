@@ -151,6 +151,46 @@ def test_tiles_split_over_the_columns(dev, monkeypatch, qtype, rows, cols, n, ti
     m.free()
 
 
+def test_split_products_on_two_streams_keep_their_parts_apart(dev):
+    """Two split products queued on two streams of one GPU at once: each stream's launches keep their parts in a
+    buffer of that stream's, so both give what each gives alone."""
+    import ctypes as C
+    from illatio_amd import dense, hip
+    info = hip.DeviceInfo()
+    hip.call("ilt_device_get_info", C.c_int(dev.index), C.byref(info))
+    other = hip.Device(dev.index, info, hip.hip_stream_create(dev))
+    rng = synth.make_rng(97)
+    rows, cols, n = 2560, 9728, 512                           # 80 tiles of 128 x 128 or fewer of the larger: split either way
+    ms, xs, ys, alone = [], [], [], []
+    for d_ in (dev, other):
+        w = synth.weights(synth.Q4_K, rows, cols, rng)
+        x = synth.activations((n, cols), rng)
+        m = upload(d_, synth.Q4_K, rows, cols, w)
+        xf = hip.hip_upload_new(d_, x)
+        xb = dense.cvt_bf16(d_, xf, x.size)
+        y = hip.hip_alloc(d_, 4 * n * rows)
+        dense.cmat_mul_bf16(d_, m, xb, y, n)
+        alone.append(hip.hip_floats(y, n * rows))             # (waits for the stream)
+        hip.hip_free(xf)
+        ms.append(m); xs.append(xb); ys.append(y)
+    for _ in range(3):                                         # both streams busy with split products at the same time
+        for d_, m, xb, y in zip((dev, other), ms, xs, ys):
+            hip.hip_zero(y)
+            for _ in range(4):
+                dense.cmat_mul_bf16(d_, m, xb, y, n)
+        hip.hip_sync(dev); hip.hip_stream_sync(other.stream)
+        for y, a in zip(ys, alone):
+            assert np.array_equal(bits_of(hip.hip_floats(y, n * rows)), bits_of(a))
+    for b_ in xs + ys:
+        hip.hip_free(b_)
+    for m in ms:
+        m.free()
+
+
+def bits_of(a):
+    return np.ascontiguousarray(a, np.float32).view(np.uint32)
+
+
 @pytest.mark.parametrize("two_pass", [False, True])
 def test_output_head_keeps_the_cpu_paths_top_token(dev, two_pass):
     """128 positions through an output head (Q6_K, config 2's width, 8192 of its rows): the
