@@ -401,9 +401,14 @@ __device__ __forceinline__ float chain_add_from(float o, const float* col, int n
 // The chain of one column with the products made on the way: o = ((0 + sc[0] col[0]) + sc[1] col[1]) + ..; the reads
 // of 16 positions on their way while the 16 before them are multiplied and added.  last_read: the last float of col's
 // row from which 16 can be read; sc's row may be read 16 floats past npos.
+__device__ __forceinline__ float chain_muladd_from(float o, const float* sc, const float* col, int npos, int last_read);
 __device__ __forceinline__ float chain_muladd_row(const float* sc, const float* col, int npos, int last_read) {
+  return chain_muladd_from(0.0f, sc, col, npos, last_read);
+}
+// (carried on from o: scores and column that come in tiles.  sc's row too is read from min(.., last_read) here, so both
+// rows need 16 floats of room past last_read and no more)
+__device__ __forceinline__ float chain_muladd_from(float o, const float* sc, const float* col, int npos, int last_read) {
   typedef float f4v __attribute__((ext_vector_type(4)));
-  float o = 0.0f;
   int p = 0;
   f4v s0, s1, s2, s3, v0, v1, v2, v3, t0, t1, t2, t3, w0, w1, w2, w3;
   ILT_LDS_READ16X2_AHEAD(s, v, sc, col);
@@ -411,7 +416,7 @@ __device__ __forceinline__ float chain_muladd_row(const float* sc, const float* 
     ILT_LDS_READ16X2_AHEAD(t, w, sc + p + 16, col + p + 16);
     ILT_LDS_READ16X2_WAIT(s, v, 8);
     ILT_CHAIN_MULADD16(o, s, v);
-    ILT_LDS_READ16X2_AHEAD(s, v, sc + p + 32, col + min(p + 32, last_read));
+    ILT_LDS_READ16X2_AHEAD(s, v, sc + min(p + 32, last_read), col + min(p + 32, last_read));
     ILT_LDS_READ16X2_WAIT(t, w, 8);
     ILT_CHAIN_MULADD16(o, t, w);
   }
@@ -982,6 +987,65 @@ __global__ __launch_bounds__(1024) void attn_values_stream_kernel(const float* _
   if (tid < 16) out[h * hd + 16 * cs + tid] = o;
 }
 
+// A prompt chunk's values, 32 tokens x 32 columns of a query head a workgroup of 1,024 threads, a chain each: the scaled
+// scores (attn_softmax_kernel's) and the value slice come through LDS in tiles of 256 positions, each tile's loads on
+// their way while the tile before it is multiplied and added.  A tile of scores serves 32 columns and a tile of values
+// 32 tokens -- attn_values_kernel<16> and attn_values_tiled_kernel<16> bring a tile in for 16 of each, and what those
+// kernels wait for is the tiles, not the chains.  The numbers are theirs: the same products and sums in the same order.
+constexpr int kChunkTile = 256, kChunkPitch = kChunkTile + 4;      // (4 mod 64: sixteen rows' 16-byte reads on different banks)
+__global__ __launch_bounds__(1024) void attn_values_chunk_kernel(const float* __restrict__ raw, const float* __restrict__ vc, float* __restrict__ out,
+                                                                 int nh, int nkv, int hd, int pos0, int ntok, int spitch) {
+  extern __shared__ __align__(16) float dyn[];
+  float* const scs = dyn;                          // a row a token
+  float* const vts = dyn + 32 * kChunkPitch;       // a row a column
+  const int gx = gridDim.x, bx = (gx & 7) ? (int)blockIdx.x : (int)(blockIdx.x & 7) * (gx >> 3) + (int)(blockIdx.x >> 3);
+  const int ns = hd >> 5, h = bx / ns, cs = bx - h * ns, t0 = blockIdx.y * 32, tid = threadIdx.x;
+  const int tn = min(32, ntok - t0), nposmax = pos0 + t0 + tn;
+  const int group = nh / nkv, kvd = nkv * hd, ko = (h / group) * hd + 32 * cs;
+  const float* rbase = raw + ((long long)t0 * nh + h) * spitch;
+  const int tt = tid >> 5, c = tid & 31, npos = tt < tn ? pos0 + t0 + tt + 1 : 0;      // this thread's chain: token t0 + tt, column 32 cs + c
+  const int ntiles = (nposmax + kChunkTile - 1) / kChunkTile;
+  float4 rs[2], rv[2];
+  // a tile's 16-byte pieces: of the scores, q4 a token's row (what lies past a token's own positions is carried along and
+  // never read; past the rows' end nothing is loaded); of the values, eight a position
+  auto load_tile = [&](int tile) {
+    const int p0 = tile * kChunkTile, q4 = min(kChunkTile, spitch - p0) >> 2, totalq = tn * q4;
+    const int totalv = min(kChunkTile, nposmax - p0) * 8;
+#pragma unroll
+    for (int u = 0; u < 2; u++) {
+      const int i = min(tid + 1024 * u, totalq - 1), rt = i / q4, j = i - rt * q4;
+      rs[u] = *(const float4*)(rbase + (long long)rt * nh * spitch + p0 + 4 * j);
+      const int k = min(tid + 1024 * u, totalv - 1);
+      rv[u] = *(const float4*)(vc + (long long)(p0 + (k >> 3)) * kvd + ko + 4 * (k & 7));
+    }
+  };
+  auto store_tile = [&](int tile) {
+    const int p0 = tile * kChunkTile, q4 = min(kChunkTile, spitch - p0) >> 2, totalq = tn * q4;
+    const int totalv = min(kChunkTile, nposmax - p0) * 8;
+#pragma unroll
+    for (int u = 0; u < 2; u++) {
+      const int i = tid + 1024 * u, rt = i / q4, j = i - rt * q4;
+      if (i < totalq) *(float4*)(scs + rt * kChunkPitch + 4 * j) = rs[u];
+      const int k = tid + 1024 * u;
+      if (k < totalv) {
+        float* dst = vts + (4 * (k & 7)) * kChunkPitch + (k >> 3);
+        dst[0] = rv[u].x; dst[kChunkPitch] = rv[u].y; dst[2 * kChunkPitch] = rv[u].z; dst[3 * kChunkPitch] = rv[u].w;
+      }
+    }
+  };
+  load_tile(0);
+  float o = 0.0f;
+  for (int t = 0; t < ntiles; t++) {
+    if (t) __syncthreads();                        // the chains are through with the tile before
+    store_tile(t);
+    if (t + 1 < ntiles) load_tile(t + 1);          // on their way while this tile is added
+    __syncthreads();
+    const int np = min(kChunkTile, npos - t * kChunkTile);       // of the tile's positions, the token's own (may be none)
+    if (np > 0) o = chain_muladd_from(o, scs + tt * kChunkPitch, vts + c * kChunkPitch, np, kChunkPitch - 16);
+  }
+  if (tt < tn) out[((long long)(t0 + tt) * nh + h) * hd + 32 * cs + c] = o;
+}
+
 // ARGMAX (model.lisp:464-468): best = 0; an element replaces the best when it is greater -- so the first of equal
 // maxima, a NaN never (and if v[0] is a NaN nothing replaces it).  Two steps: each workgroup the best of its
 // stretch (every thread's own elements first, eight 16-byte loads in flight, then the threads', a smaller index
@@ -1072,6 +1136,27 @@ hipError_t ilt_k_attn_rows(const float* q, const float* kc, const float* vc, flo
   static bool attr_set[64] = {};
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) dev = 0;
+  // A chunk: scores, softmax, then 32 tokens x 32 columns a workgroup.  "ILT_ATTN_CHUNK=0": the kernels of 16 tokens x 16
+  // columns below instead (tests).
+  if (scratch && ntok > 1 && pos0 + ntok <= 8192 && hd % 32 == 0) {
+    const char* off = getenv("ILT_ATTN_CHUNK");
+    if (!(off && off[0] == '0')) {
+      static bool set[64] = {};
+      const size_t smem = sizeof(float) * 2 * 32 * (size_t)kChunkPitch;
+      if (!set[dev]) {
+        const hipError_t e = hipFuncSetAttribute((const void*)attn_values_chunk_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+        if (e != hipSuccess) return e;
+        set[dev] = true;
+      }
+      const int ctx = pos0 + ntok;
+      hipLaunchKernelGGL(attn_scores_kernel<16>, dim3(nh, (ctx + 255) / 256, (ntok + 15) / 16), dim3(1024), 0, st, q, kc, scratch, nh, nkv, hd, pos0, ntok,
+                         scale, smax);
+      hipLaunchKernelGGL(attn_softmax_kernel, dim3(nh, ntok), dim3(256), sizeof(float) * smax, st, scratch, nh, pos0, smax);
+      hipLaunchKernelGGL(attn_values_chunk_kernel, dim3(nh * (hd / 32), (ntok + 31) / 32), dim3(1024), smem, st, scratch, vc, out, nh, nkv, hd, pos0,
+                         ntok, smax);
+      return hipGetLastError();
+    }
+  }
   if (scratch && pos0 + ntok <= 2048) {
     const int ctx = pos0 + ntok, vpitch = ((ctx + 63) & ~63) + 4;
     // tokens a workgroup: as many as leave their scores and the value slice room in LDS (150 KB)
