@@ -236,21 +236,23 @@ __global__ __launch_bounds__(kAttnThreads) void attn_rows_kernel(const float* __
 // chains from LDS.  A group's tokens share the keys (registers) and the value slice (LDS), so a prompt's chunk
 // reads them once for 16 tokens.  The numbers are attn_rows_kernel's: the same operations in the same order.
 // raw[(t*nh + h)*spitch + p] = F32-DOT16(K[p], q) * scale
-template <int TG>
+// NJ: hd / 16 as a constant (heads of 64 and of 128), or 0: any head up to 256, the count read at run time
+template <int TG, int NJ = 0>
 __global__ __launch_bounds__(1024) void attn_scores_kernel(const float* __restrict__ q, const float* __restrict__ kc, float* __restrict__ raw,
                                                            int nh, int nkv, int hd, int pos0, int ntok, float scale, int spitch) {
+  constexpr int NJM = NJ ? NJ : 16;
   __shared__ float qs[TG > 1 ? TG * 256 : 1];
   const int h = blockIdx.x, t0 = blockIdx.z * TG, tid = threadIdx.x;
   const int tn = min(TG, ntok - t0), nposmax = pos0 + t0 + tn, pbase = blockIdx.y * 256;
   if (pbase >= nposmax) return;                    // the same in every thread
   const int group = nh / nkv, kvd = nkv * hd, ko = (h / group) * hd;
-  const int l = tid & 15, pg = tid >> 4, nj = hd >> 4;
-  float kv[4][16];
+  const int l = tid & 15, pg = tid >> 4, nj = NJ ? NJ : hd >> 4;
+  float kv[4][NJM];
 #pragma unroll
   for (int u = 0; u < 4; u++) {
     const float* kr = kc + (long long)min(pbase + 64 * u + pg, nposmax - 1) * kvd + ko;
 #pragma unroll
-    for (int j = 0; j < 16; j++) kv[u][j] = j < nj ? kr[l + 16 * j] : 0.0f;
+    for (int j = 0; j < NJM; j++) kv[u][j] = (NJ || j < nj) ? kr[l + 16 * j] : 0.0f;
   }
   if (TG > 1) {
     for (int i = tid; i < tn * hd; i += 1024) { const int tt = i / hd, c = i - tt * hd; qs[tt * 256 + c] = q[((long long)(t0 + tt) * nh + h) * hd + c]; }
@@ -260,16 +262,16 @@ __global__ __launch_bounds__(1024) void attn_scores_kernel(const float* __restri
     const int npos = pos0 + t0 + tt + 1;
     if (pbase >= npos) continue;
     const float* qh = q + ((long long)(t0 + tt) * nh + h) * hd;
-    float qv[16];
+    float qv[NJM];
 #pragma unroll
-    for (int j = 0; j < 16; j++) qv[j] = j < nj ? (TG > 1 ? qs[tt * 256 + l + 16 * j] : qh[l + 16 * j]) : 0.0f;
+    for (int j = 0; j < NJM; j++) qv[j] = (NJ || j < nj) ? (TG > 1 ? qs[tt * 256 + l + 16 * j] : qh[l + 16 * j]) : 0.0f;
 #pragma unroll
     for (int u = 0; u < 4; u++) {
       const int p = pbase + 64 * u + pg;
       if (pbase + 64 * u >= npos) continue;        // none of the pass's 64 positions is the token's to see (the same in every thread)
       float sacc = 0.0f;
 #pragma unroll
-      for (int j = 0; j < 16; j++) if (j < nj) sacc = sacc + kv[u][j] * qv[j];
+      for (int j = 0; j < NJM; j++) if (NJ || j < nj) sacc = sacc + kv[u][j] * qv[j];
       sacc = sacc + ilt_dppf<ILT_DPP_SHL(4)>(sacc);
       sacc = sacc + ilt_dppf<ILT_DPP_SHL(8)>(sacc);
       sacc = sacc + ilt_dppf<ILT_DPP_SHL(1)>(sacc);
@@ -1100,6 +1102,14 @@ __global__ __launch_bounds__(256) void swiglu_rows_kernel(float* __restrict__ a,
   if (i < n) { const float g = a[i]; a[i] = (g / (1.0f + ilt_expf_via_double(-g))) * b[i]; }
 }
 
+template <int TG>
+void launch_scores(dim3 grid, hipStream_t st, const float* q, const float* kc, float* raw, int nh, int nkv, int hd, int pos0, int ntok, float scale,
+                   int spitch) {
+  if (hd == 128) hipLaunchKernelGGL((attn_scores_kernel<TG, 8>), grid, dim3(1024), 0, st, q, kc, raw, nh, nkv, hd, pos0, ntok, scale, spitch);
+  else if (hd == 64) hipLaunchKernelGGL((attn_scores_kernel<TG, 4>), grid, dim3(1024), 0, st, q, kc, raw, nh, nkv, hd, pos0, ntok, scale, spitch);
+  else hipLaunchKernelGGL((attn_scores_kernel<TG, 0>), grid, dim3(1024), 0, st, q, kc, raw, nh, nkv, hd, pos0, ntok, scale, spitch);
+}
+
 // one token's values past 2,048 positions (the scores: smax floats a head in scratch, raw)
 hipError_t launch_values_stream(int dev, const float* scratch, const float* vc, float* out, int nh, int nkv, int hd, int pos, int smax,
                                 hipStream_t st) {
@@ -1149,8 +1159,7 @@ hipError_t ilt_k_attn_rows(const float* q, const float* kc, const float* vc, flo
         set[dev] = true;
       }
       const int ctx = pos0 + ntok;
-      hipLaunchKernelGGL(attn_scores_kernel<16>, dim3(nh, (ctx + 255) / 256, (ntok + 15) / 16), dim3(1024), 0, st, q, kc, scratch, nh, nkv, hd, pos0, ntok,
-                         scale, smax);
+      launch_scores<16>(dim3(nh, (ctx + 255) / 256, (ntok + 15) / 16), st, q, kc, scratch, nh, nkv, hd, pos0, ntok, scale, smax);
       hipLaunchKernelGGL(attn_softmax_kernel, dim3(nh, ntok), dim3(256), sizeof(float) * smax, st, scratch, nh, pos0, smax);
       hipLaunchKernelGGL(attn_values_chunk_kernel, dim3(nh * (hd / 32), (ntok + 31) / 32), dim3(1024), smem, st, scratch, vc, out, nh, nkv, hd, pos0,
                          ntok, smax);
@@ -1177,7 +1186,7 @@ hipError_t ilt_k_attn_rows(const float* q, const float* kc, const float* vc, flo
                                        152 * 1024);                                                                                            \
     if (e == hipSuccess) {                                                                                                                     \
       set[dev] = true;                                                                                                                         \
-      hipLaunchKernelGGL(attn_scores_kernel<TG>, gs, dim3(1024), 0, st, q, kc, scratch, nh, nkv, hd, pos0, ntok, scale, smax);                 \
+      launch_scores<TG>(gs, st, q, kc, scratch, nh, nkv, hd, pos0, ntok, scale, smax);                                                         \
       if (TG > 1) hipLaunchKernelGGL(attn_softmax_kernel, dim3(nh, ntok), dim3(256), sizeof(float) * smax, st, scratch, nh, pos0, smax);        \
       hipLaunchKernelGGL((attn_values_kernel<TG, NB, (TG > 1)>), gv, dim3(256), bytes(TG), st, scratch, vc, out, nh, nkv, hd, pos0, ntok,      \
                          smax, vpitch);                                                                                                        \
@@ -1202,11 +1211,11 @@ hipError_t ilt_k_attn_rows(const float* q, const float* kc, const float* vc, flo
       set[dev] = true;
     }
     if (tg == 16) {
-      hipLaunchKernelGGL(attn_scores_kernel<16>, gs, dim3(1024), 0, st, q, kc, scratch, nh, nkv, hd, pos0, ntok, scale, smax);
+      launch_scores<16>(gs, st, q, kc, scratch, nh, nkv, hd, pos0, ntok, scale, smax);
       hipLaunchKernelGGL(attn_softmax_kernel, dim3(nh, ntok), dim3(256), sizeof(float) * smax, st, scratch, nh, pos0, smax);
       hipLaunchKernelGGL(attn_values_tiled_kernel<16>, gv, dim3(256), smem, st, scratch, vc, out, nh, nkv, hd, pos0, ntok, smax);
     } else {
-      hipLaunchKernelGGL(attn_scores_kernel<1>, gs, dim3(1024), 0, st, q, kc, scratch, nh, nkv, hd, pos0, ntok, scale, smax);
+      launch_scores<1>(gs, st, q, kc, scratch, nh, nkv, hd, pos0, ntok, scale, smax);
       const hipError_t e = launch_values_stream(dev, scratch, vc, out, nh, nkv, hd, pos0, smax, st);
       if (e != hipSuccess) return e;
     }

@@ -28,6 +28,8 @@ def synth_model(seed, d=2560, ffn=9728, nh=32, nkv=8, hd=128, nl=36, vocab=15193
     the attention's scores (at 1 they are about N(0, 1)).  Neither changes the values drawn at 1."""
     rng = synth.make_rng(seed)
     qd, kvd = nh * hd, nkv * hd
+    if d % 256 or qd % 256 or ffn % 256:
+        raise ValueError("K-quant rows are whole super-blocks of 256 columns: d, nh * hd and ffn must be multiples of 256")
     norm = lambda n: (synth.activations(n, rng) * 0.1 + 1.0).astype(np.float32)
     layers = []
     for _ in range(nl):

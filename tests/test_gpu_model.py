@@ -350,6 +350,22 @@ def test_small_decoder_long_contexts(dev):
     assert same == 5
 
 
+def test_chunk_attention_on_the_kernels_of_16_tokens(dev, monkeypatch):
+    """The kernels a chunk's values went through before the 32 x 32 one, still taken by heads whose width is not a multiple
+    of 32 (and, with ILT_ATTN_CHUNK=0, by any): whole in LDS up to about 1,100 positions, in tiles past that; and heads of
+    48, whose score kernel reads the head's width at run time."""
+    from illatio_amd import model
+    host = model.synth_model(8, d=256, ffn=512, nh=16, nkv=4, hd=48, nl=2, vocab=400)      # (16 x 48 = 768 columns for wo: whole super-blocks)
+    same, _ = run_greedy(dev, host, nprompt=300, ndecode=3, chunk=128, nctx=310, seed=21)
+    assert same == 3
+    same, _ = run_greedy(dev, host, nprompt=1300, ndecode=2, chunk=256, nctx=1310, seed=22)
+    assert same == 2
+    monkeypatch.setenv("ILT_ATTN_CHUNK", "0")
+    host = model.synth_model(9, d=256, ffn=512, nh=4, nkv=2, hd=64, nl=2, vocab=400)
+    same, _ = run_greedy(dev, host, nprompt=1300, ndecode=2, chunk=256, nctx=1310, seed=23)
+    assert same == 2
+
+
 def test_decode_across_position_8192(dev):
     """A context longer than the 8,192 positions the kernels with their scores in memory take: tokens at positions 8,190
     and 8,191 go through ilt_dense_decode (tiled values), those at 8,192 and 8,193 through qk_rope + attn_rows with the
