@@ -286,6 +286,7 @@ __global__ __launch_bounds__(1024) void attn_scores_kernel(const float* __restri
 // positions hold the token's own does the same for its KV head's key (wave 1) and takes that key from LDS,
 // and the group's first query head there writes the key and the value into the caches, for the launch with
 // the values.  q and k are left as they came.
+template <int NJ>      // hd / 16 as a constant, or 0: read at run time (heads up to 256)
 __global__ __launch_bounds__(1024) void attn_step_scores_kernel(const float* __restrict__ q, const float* __restrict__ k, const float* __restrict__ v,
                                                                 const float* __restrict__ qn, const float* __restrict__ kn,
                                                                 const float* __restrict__ rope, float* __restrict__ kc, float* __restrict__ vc,
@@ -296,19 +297,20 @@ __global__ __launch_bounds__(1024) void attn_step_scores_kernel(const float* __r
   const int h = blockIdx.x, tid = threadIdx.x, npos = pos + 1, pbase = blockIdx.y * 256;
   if (pbase >= npos) return;
   const int group = nh / nkv, kvd = nkv * hd, kh = h / group, ko = kh * hd;
-  const int l = tid & 15, pg = tid >> 4, nj = hd >> 4, wave = tid >> 6;
+  constexpr int NJM = NJ ? NJ : 16;
+  const int l = tid & 15, pg = tid >> 4, nj = NJ ? NJ : hd >> 4, wave = tid >> 6;
   const bool own = pos < pbase + 256;              // this workgroup's positions hold the token's own
   // the head's own loads first (waves 0 and 1), the keys' after: the norms and the turn wait for the first alone
   const float* cs = rope + (long long)pos * rd;
   RopeIn<4> rin;
   const bool turns = wave == 0 || (wave == 1 && own);
   if (turns) rope_head_load(rin, wave == 0 ? q + h * hd : k + ko, wave == 0 ? qn : kn, cs, hd, rd, tid & 63);
-  float kv[4][16];
+  float kv[4][NJM];
 #pragma unroll
   for (int u = 0; u < 4; u++) {
     const float* kr = kc + (long long)min(pbase + 64 * u + pg, max(pos - 1, 0)) * kvd + ko;      // rows before the token's own
 #pragma unroll
-    for (int j = 0; j < 16; j++) kv[u][j] = j < nj ? kr[l + 16 * j] : 0.0f;
+    for (int j = 0; j < NJM; j++) kv[u][j] = (NJ || j < nj) ? kr[l + 16 * j] : 0.0f;
   }
   if (turns) rope_head_turn(rin, (wave == 0 ? qn : kn) != nullptr, wave == 0 ? qsh : ksh, &scs[wave], hd, rd, eps, neox, tid & 63);
   __syncthreads();
@@ -316,19 +318,19 @@ __global__ __launch_bounds__(1024) void attn_step_scores_kernel(const float* __r
     kc[(long long)pos * kvd + ko + tid] = ksh[tid];
     vc[(long long)pos * kvd + ko + tid] = v[ko + tid];
   }
-  float qv[16];
+  float qv[NJM];
 #pragma unroll
-  for (int j = 0; j < 16; j++) qv[j] = j < nj ? qsh[l + 16 * j] : 0.0f;
+  for (int j = 0; j < NJM; j++) qv[j] = (NJ || j < nj) ? qsh[l + 16 * j] : 0.0f;
 #pragma unroll
   for (int u = 0; u < 4; u++) {
     const int p = pbase + 64 * u + pg;
     if (p == pos) {
 #pragma unroll
-      for (int j = 0; j < 16; j++) kv[u][j] = j < nj ? ksh[l + 16 * j] : 0.0f;
+      for (int j = 0; j < NJM; j++) kv[u][j] = (NJ || j < nj) ? ksh[l + 16 * j] : 0.0f;
     }
     float sacc = 0.0f;
 #pragma unroll
-    for (int j = 0; j < 16; j++) if (j < nj) sacc = sacc + kv[u][j] * qv[j];
+    for (int j = 0; j < NJM; j++) if (NJ || j < nj) sacc = sacc + kv[u][j] * qv[j];
     sacc = sacc + ilt_dppf<ILT_DPP_SHL(4)>(sacc);
     sacc = sacc + ilt_dppf<ILT_DPP_SHL(8)>(sacc);
     sacc = sacc + ilt_dppf<ILT_DPP_SHL(1)>(sacc);
@@ -1309,8 +1311,15 @@ hipError_t ilt_k_attn_step(const float* q, const float* k, const float* v, const
                          neox, scale, vpitch, split ? 1 : 0, epoch, patience, xgen, xrow);
     return hipGetLastError();
   }
-  hipLaunchKernelGGL(attn_step_scores_kernel, dim3(nh, (ctx + 255) / 256), dim3(1024), 0, st, q, k, v, qn, kn, rope, kc, vc, scratch, nh, nkv, hd, rd,
-                     pos, eps, neox, scale, smax);
+  {
+    const dim3 gs(nh, (ctx + 255) / 256);
+    if (hd == 128)
+      hipLaunchKernelGGL(attn_step_scores_kernel<8>, gs, dim3(1024), 0, st, q, k, v, qn, kn, rope, kc, vc, scratch, nh, nkv, hd, rd, pos, eps, neox, scale, smax);
+    else if (hd == 64)
+      hipLaunchKernelGGL(attn_step_scores_kernel<4>, gs, dim3(1024), 0, st, q, k, v, qn, kn, rope, kc, vc, scratch, nh, nkv, hd, rd, pos, eps, neox, scale, smax);
+    else
+      hipLaunchKernelGGL(attn_step_scores_kernel<0>, gs, dim3(1024), 0, st, q, k, v, qn, kn, rope, kc, vc, scratch, nh, nkv, hd, rd, pos, eps, neox, scale, smax);
+  }
   if (ctx > 2048) return launch_values_stream(dev, scratch, vc, out, nh, nkv, hd, pos, smax, st);
   hipError_t e = hipErrorInvalidValue;
 #define ILT_ATTN1(NB)                                                                                                                         \
