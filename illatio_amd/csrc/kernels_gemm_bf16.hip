@@ -1911,8 +1911,8 @@ __global__ __launch_bounds__(256) void q8k_bf16_kernel(const i8* __restrict__ xq
 }
 
 // Room for the split tiles' parts: a buffer per (device, stream) -- launches on two streams may overlap, and each needs
-// its parts to itself -- grown when a launch needs more, never inside a stream capture; sixteen of them at most.  A
-// launch that gets no room (capturing with too little, the table full, no memory) goes unsplit.
+// its parts to itself -- grown when a launch needs more; sixteen of them at most.  A launch that gets no room (a stream
+// under capture, the table full, no memory) goes unsplit.
 struct PartRoom { int dev; hipStream_t st; float* p; size_t bytes; };
 std::mutex g_part_mu;
 PartRoom g_part[16] = {};
@@ -1920,12 +1920,14 @@ int g_nparts = 0;
 float* part_room(size_t bytes, hipStream_t st) {
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess) return nullptr;
+  // (a captured launch would keep the room's address while a later launch may grow the room and free it: under capture
+  // nothing is split)
+  hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(st, &cs) != hipSuccess || cs != hipStreamCaptureStatusNone) { (void)hipGetLastError(); return nullptr; }
   std::lock_guard<std::mutex> lock(g_part_mu);
   PartRoom* r = nullptr;
   for (int i = 0; i < g_nparts; i++) if (g_part[i].dev == dev && g_part[i].st == st) r = &g_part[i];
   if (r && r->bytes >= bytes) return r->p;
-  hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
-  if (hipStreamIsCapturing(st, &cs) != hipSuccess || cs != hipStreamCaptureStatusNone) { (void)hipGetLastError(); return nullptr; }
   if (!r) {
     if (g_nparts == 16) return nullptr;
     r = &g_part[g_nparts++];
