@@ -738,33 +738,56 @@ int ilt_d4_mm_id_q2_k(uint64_t stream, int ncols, int nrows, int row_bytes, int6
 
 // ---- d4_mm_<format>: one matrix on a chunk of tokens' float activations (ds4f_mm.cu:252-255) ----------
 // The reference's kernels round weights and activations to halves; these quantize the activations as the CPU
-// path does and run the exact products, so the quantized activations need room: a buffer per device that only
-// ever grows, kept until the process ends.  Calls that overlap on one GPU (two streams) would share it: the
-// reference's host issues these on one stream.  Growing frees and allocates, which waits for the device and cannot
-// happen while a stream is being captured: a caller that captures, or that wants no such stall in its loop, sizes
-// the buffer once beforehand (ilt_d4_mm_reserve).  The bookkeeping is guarded; the buffer itself is one per device.
+// path does and run the exact products, so the quantized activations need room: a buffer per (device, stream) that
+// only ever grows, kept until the process ends -- calls that overlap on one GPU are on different streams, and each
+// stream's calls have a buffer to themselves (sixteen of them at most; a seventeenth stream is refused).  Growing frees
+// and allocates, which waits for the stream and cannot happen while it is being captured (refused then): a caller that
+// captures, or that wants no such stall in its loop, sizes the buffers beforehand -- ilt_d4_mm_reserve for every buffer
+// made from then on and the ones there are, ilt_d4_mm_reserve_stream for one stream's at once.
 namespace {
-struct QRoom { void* p; size_t bytes; };
-QRoom g_qroom[ILT_MAX_DEVICES];
+struct QRoom { int dev; hipStream_t st; void* p; size_t bytes; };
+QRoom g_qroom[16];
+int g_nqrooms = 0;
+size_t g_qroom_min = 0;
 std::mutex g_qroom_mu;
 size_t qroom_bytes(int fmt, size_t ntok, size_t ncols) {
   const size_t n = ntok * ncols, bw = fmt == ILT_Q8_0 ? 32 : 256;
   return (n + 255) / 256 * 256 + (n / bw * 4 + 255) / 256 * 256 + (fmt == ILT_Q8_0 ? 0 : (n / 16 * 4 + 255) / 256 * 256);
 }
-int qroom(size_t bytes, uint8_t** out) {
+// (the lock held) the stream's buffer grown to BYTES
+int qroom_grow(QRoom& q, size_t bytes) {
+  if (q.bytes >= bytes) return ILT_OK;
+  hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
+  ILT_TRY(hipStreamIsCapturing(q.st, &cs));
+  if (cs != hipStreamCaptureStatusNone) return (int)hipErrorStreamCaptureUnsupported;
+  if (q.p) {
+    ILT_TRY(hipStreamSynchronize(q.st));                 // the stream's earlier calls may still read the old buffer
+    ILT_TRY(hipFree(q.p));
+  }
+  q.p = nullptr; q.bytes = 0;
+  const size_t want = bytes + bytes / 4 + (1 << 20);
+  ILT_TRY(hipMalloc(&q.p, want));
+  q.bytes = want;
+  return ILT_OK;
+}
+int qroom(uint64_t stream, size_t bytes, uint8_t** out) {
   int dev = -1;
   ILT_TRY(hipGetDevice(&dev));
-  ILT_REQUIRE(dev >= 0 && dev < ILT_MAX_DEVICES);
   std::lock_guard<std::mutex> lock(g_qroom_mu);
-  QRoom& q = g_qroom[dev];
-  if (q.bytes < bytes) {
-    if (q.p) ILT_TRY(hipFree(q.p));                      // (waits for the work that still reads it)
-    q.p = nullptr; q.bytes = 0;
-    const size_t want = bytes + bytes / 4 + (1 << 20);
-    ILT_TRY(hipMalloc(&q.p, want));
-    q.bytes = want;
+  QRoom* q = nullptr;
+  for (int i = 0; i < g_nqrooms; i++) if (g_qroom[i].dev == dev && g_qroom[i].st == S(stream)) q = &g_qroom[i];
+  if (!q) {
+    if (g_nqrooms == 16) return (int)hipErrorOutOfMemory;
+    q = &g_qroom[g_nqrooms];
+    *q = {dev, S(stream), nullptr, 0};
+    const int e = qroom_grow(*q, bytes > g_qroom_min ? bytes : g_qroom_min);
+    if (e != ILT_OK) return e;
+    g_nqrooms++;
+  } else {
+    const int e = qroom_grow(*q, bytes);
+    if (e != ILT_OK) return e;
   }
-  *out = (uint8_t*)q.p;
+  if (out) *out = (uint8_t*)q->p;
   return ILT_OK;
 }
 int d4_mm_quantized(uint64_t stream, int fmt, int ncols, int nrows, int ntok, int row_bytes, int x_stride, int y_stride, const void* w,
@@ -780,7 +803,7 @@ int d4_mm_quantized(uint64_t stream, int fmt, int ncols, int nrows, int ntok, in
   const size_t n = (size_t)ntok * ncols;
   const size_t qb = (n + 255) / 256 * 256, sb = (n / bw * 4 + 255) / 256 * 256, bb = fmt == ILT_Q8_0 ? 0 : (n / 16 * 4 + 255) / 256 * 256;
   uint8_t* room = nullptr;
-  ILT_TRY((hipError_t)qroom(qb + sb + bb, &room));
+  ILT_TRY((hipError_t)qroom(stream, qb + sb + bb, &room));
   int8_t* xq = (int8_t*)room; float* xs = (float*)(room + qb); int32_t* bs = (int32_t*)(room + qb + sb);
   if (fmt == ILT_Q8_0) {
     // d4-shared!'s and the attention projections' activations: quantize-q8! with the scale kept a float (ds4f.lisp:1052-1053)
@@ -796,8 +819,22 @@ int d4_mm_quantized(uint64_t stream, int fmt, int ncols, int nrows, int ntok, in
 
 int ilt_d4_mm_reserve(int ntok, int ncols) {
   ILT_REQUIRE(ntok >= 0 && ncols >= 0);
-  uint8_t* room = nullptr;
-  return qroom(qroom_bytes(ILT_Q2_K, (size_t)ntok, (size_t)ncols), &room);       // the K formats' layout is the larger one
+  const size_t bytes = qroom_bytes(ILT_Q2_K, (size_t)ntok, (size_t)ncols);       // the K formats' layout is the larger one
+  int dev = -1;
+  ILT_TRY(hipGetDevice(&dev));
+  std::lock_guard<std::mutex> lock(g_qroom_mu);
+  if (bytes > g_qroom_min) g_qroom_min = bytes;
+  for (int i = 0; i < g_nqrooms; i++)
+    if (g_qroom[i].dev == dev) {
+      const int e = qroom_grow(g_qroom[i], bytes);
+      if (e != ILT_OK) return e;
+    }
+  return ILT_OK;
+}
+
+int ilt_d4_mm_reserve_stream(uint64_t stream, int ntok, int ncols) {
+  ILT_REQUIRE(ntok >= 0 && ncols >= 0);
+  return qroom(stream, qroom_bytes(ILT_Q2_K, (size_t)ntok, (size_t)ncols), nullptr);
 }
 
 int ilt_d4_mm_q8_0(uint64_t stream, int ncols, int nrows, int ntok, int row_bytes, int x_stride, int y_stride, const int8_t* w,

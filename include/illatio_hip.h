@@ -424,11 +424,16 @@ int ilt_mm_k_n(uint64_t stream, int type, const void* w0, float* y0, const float
    x_stride >= ncols and y_stride >= nrows: the reference passes them for the grouped attention output product,
    one call a group on a slice of each token's heads into a slice of its low row, w and wd at offsets into
    their arrays (cuda-ds4f-prefill.lisp:277-281); the K formats want x_stride a multiple of 4.
-   The quantized formats keep their quantized activations in a buffer inside the library that grows to the
-   largest chunk seen (per GPU, until the process ends; calls that overlap on one GPU share it).  Growing frees
-   and allocates: ilt_d4_mm_reserve(ntok, ncols) sizes it beforehand for chunks of up to ntok tokens of ncols
-   columns, after which calls within that size allocate nothing (callers under stream capture need this). */
+   The quantized formats keep their quantized activations in a buffer inside the library, one per (GPU, stream), that
+   grows to the largest chunk seen and is kept until the process ends: calls that overlap on one GPU are on different
+   streams and do not share a buffer (sixteen buffers at most; a call on a seventeenth stream returns
+   hipErrorOutOfMemory).  Growing waits for the stream, frees and allocates, and is refused while the stream is being
+   captured (hipErrorStreamCaptureUnsupported): ilt_d4_mm_reserve(ntok, ncols) sizes the current GPU's buffers -- those
+   there are, and every one made later -- for chunks of up to ntok tokens of ncols columns, and
+   ilt_d4_mm_reserve_stream makes and sizes one stream's at once; calls within that size allocate nothing.  Neither has a
+   counterpart in the reference (its kernels take the float rows as they are). */
 int ilt_d4_mm_reserve(int ntok, int ncols);
+int ilt_d4_mm_reserve_stream(uint64_t stream, int ntok, int ncols);
 int ilt_d4_mm_q8_0(uint64_t stream, int ncols, int nrows, int ntok, int row_bytes, int x_stride, int y_stride, const int8_t* w,
                    const uint16_t* wd, const float* x, float* y);
 int ilt_d4_mm_f16(uint64_t stream, int ncols, int nrows, int ntok, int row_bytes, int x_stride, int y_stride, const uint16_t* w,

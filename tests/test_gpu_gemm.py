@@ -326,6 +326,38 @@ def test_d4_mm_on_float_rows_bit_exact(dev, qtype, rows, cols, n):
         hip.hip_free(wq)
 
 
+def test_d4_mm_on_two_streams_at_once(dev):
+    """d4_mm_* calls queued on two streams of one GPU at once: each stream's calls quantize their rows into a buffer of
+    that stream's (one sized beforehand through ilt_d4_mm_reserve_stream, the other grown by its first call), so both
+    give what each gives alone."""
+    import ctypes as C
+    from illatio_amd import ds4f, hip
+    info = hip.DeviceInfo()
+    hip.call("ilt_device_get_info", C.c_int(dev.index), C.byref(info))
+    other = hip.Device(dev.index, info, hip.hip_stream_create(dev))
+    rng = synth.make_rng(131)
+    rows, cols, n = 1024, 2048, 300
+    rb = synth.row_bytes(synth.Q2_K, cols)
+    hip.call("ilt_d4_mm_reserve_stream", C.c_uint64(other.stream), C.c_int(n), C.c_int(cols))
+    sets = []
+    for d_ in (dev, other):
+        w = synth.weights(synth.Q2_K, rows, cols, rng)
+        x = synth.activations((n, cols), rng)
+        sets.append((d_, hip.hip_upload_new(d_, w), hip.hip_upload_new(d_, x), hip.hip_alloc(d_, 4 * n * rows),
+                     orc.matmul(synth.Q2_K, w, rows, cols, x, nthreads=8).reshape(n, rows)))
+    for _ in range(3):
+        for d_, wq, xb, y, _w in sets:
+            hip.hip_zero(y)
+            for _ in range(6):
+                ds4f.dk_mm(d_, "d4_mm_q2_k", wq, None, rb, rows, cols, xb, y, n)
+        hip.hip_sync(dev); hip.hip_stream_sync(other.stream)
+        for d_, wq, xb, y, want in sets:
+            assert np.array_equal(bits(hip.hip_floats(y, n * rows).reshape(n, rows)), bits(want))
+    for d_, wq, xb, y, _w in sets:
+        for b in (wq, xb, y):
+            hip.hip_free(b)
+
+
 @pytest.mark.parametrize("groups,rank,gdim,n", [(4, 128, 512, 130), (3, 48, 96, 9), (8, 256, 1024, 257)])
 def test_d4_mm_q8_0_grouped_attention_output_strided(dev, groups, rank, gdim, n):
     """The reference's strided call of d4_mm_q8_0 (cuda-ds4f-prefill.lisp:277-281): the grouped attention output
