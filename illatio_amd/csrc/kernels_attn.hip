@@ -1320,7 +1320,11 @@ hipError_t ilt_k_attn_step(const float* q, const float* k, const float* v, const
     else
       hipLaunchKernelGGL(attn_step_scores_kernel<0>, gs, dim3(1024), 0, st, q, k, v, qn, kn, rope, kc, vc, scratch, nh, nkv, hd, rd, pos, eps, neox, scale, smax);
   }
-  if (ctx > 2048) return launch_values_stream(dev, scratch, vc, out, nh, nkv, hd, pos, smax, st);
+  // past the one-launch kernel's 1,024 positions the values come in tiles while the chains run (at 1,536 positions 523
+  // tok/s at the Qwen3-4B shape against 493 with the whole slice brought into LDS first, at 1,990 500 against 464);
+  // "ILT_ATTN_STREAM_FROM=2048": the whole slice first up to 2,048 positions (tests)
+  static const int stream_from = []{ const char* f = getenv("ILT_ATTN_STREAM_FROM"); return f ? atoi(f) : 1024; }();
+  if (ctx > stream_from || ctx > 2048) return launch_values_stream(dev, scratch, vc, out, nh, nkv, hd, pos, smax, st);
   hipError_t e = hipErrorInvalidValue;
 #define ILT_ATTN1(NB)                                                                                                                         \
   if (nb == NB) {                                                                                                                             \

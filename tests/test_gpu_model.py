@@ -348,6 +348,12 @@ def test_small_decoder_long_contexts(dev):
     assert same == 6
     same, _ = run_greedy(dev, host, nprompt=2878, ndecode=5, chunk=512, nctx=2890, seed=16)
     assert same == 5
+    # 1,025 to 2,048 positions: the same kernel by default (1,438 -> 1,441: a tile's edge); launch by launch from Python
+    # the values' whole slice goes into LDS first (attn_rows' kernels of one token)
+    same, _ = run_greedy(dev, host, nprompt=1436, ndecode=6, chunk=512, nctx=1450, seed=17)
+    assert same == 6
+    same, _ = run_greedy(dev, host, nprompt=1500, ndecode=3, chunk=512, nctx=1510, seed=18, one_call=False)
+    assert same == 3
 
 
 def test_chunk_attention_on_the_kernels_of_16_tokens(dev, monkeypatch):
