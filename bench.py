@@ -363,6 +363,10 @@ def workload_c1(args, dev):
     roof["by_launch_shape"] = {k: {"avg_launch_us": round(v[0] / v[2] * 1e3, 2), "bytes_per_launch": v[1] // v[2]} for k, v in per.items()}
     roof["traffic"] = traffic_of("c1", per)
     gbs = step_bytes / (ms * 1e-3) / 1e9
+    # the same two products on one copy of the matrices every step: 9 MB, in the memory-side cache (and mostly the L2s) after the first
+    tc = Timer(dev)
+    ms_cached, _, _ = tc.run(lambda i: [tc.launch(n, nbytes[n], lambda n=n: dense.mv_multi(dev, [(mats[0][n], ys[n], None)], xf=xb[n])) for n, r, c in shapes],
+                             args.steps, args.warmup, probe_steps=0)
 
     def cpu():
         import oracle_lib as orc
@@ -388,7 +392,8 @@ def workload_c1(args, dev):
     return {"value": round(gbs, 1), "unit": "GB/s", "ms_per_step": ms, "device_ms_per_step": dev_ms, "enqueue_ms": tm.enqueue_ms, "dtype": "int8 block dots, fp32 combine",
             "config": {"workload": "c1: Q8_0 decode GEMV 4864x896 and 896x4864 (Qwen2-0.5B MLP), batch 1, rotating over 64 copies",
                        "bytes_per_step": step_bytes},
-            "extra": {"pct_of_hbm_peak": round(100 * gbs / HBM_PEAK_GBS, 2)}, "roofline": roof, "cpu": cpu}
+            "extra": {"pct_of_hbm_peak": round(100 * gbs / HBM_PEAK_GBS, 2),
+                      "cached_GBps": round(step_bytes / (ms_cached * 1e-3) / 1e9, 1)}, "roofline": roof, "cpu": cpu}
 
 
 def workload_c3(args, dev):
@@ -479,7 +484,11 @@ def workload_c3(args, dev):
             "metric": "prefill product TFLOP/s (% of dense MFMA peak)",
             "config": {"workload": f"c3: {args.qtype.upper()} prefill product {rows}x{cols} on {T} tokens, {path} path "
                                    f"(activation conversion inside the step)", "flops_per_step": flops, "tokens": T},
-            "extra": {"pct_of_mfma_peak": round(100 * tf / MFMA_PEAK_TFLOPS[args.path], 2)}, "roofline": roof, "cpu": cpu}
+            "extra": {"pct_of_mfma_peak": round(100 * tf / MFMA_PEAK_TFLOPS[args.path], 2),
+                      # the step's algorithmic bytes (the quantized matrix once, the float activations, the float results) over its
+                      # time: far below 8,000 GB/s, i.e. not bound by memory at this token count
+                      "algorithmic_GBps": round((w.size + 4.0 * T * cols + 4.0 * T * rows) / (ms * 1e-3) / 1e9, 1)},
+            "roofline": roof, "cpu": cpu}
 
 
 def moe_weights(rng, ne_unique, ne, d, ff):
@@ -680,7 +689,11 @@ def workload_c5(args, dev):
             "metric": "MoE prefill grouped product TFLOP/s (% of dense MFMA peak)",
             "config": {"workload": f"c5: MoE prefill chunk, {n} tokens x top-6 of 256 experts (Zipf 1.1), IQ2_XXS gate/up, Q2_K down, "
                                    f"d 4096, ff 2048, {args.path} path, routing to ordered sum", "flops_per_step": flops, "tokens": n},
-            "extra": {"pct_of_mfma_peak": round(100 * tf / MFMA_PEAK_TFLOPS[args.path], 2)}, "roofline": roof, "cpu": cpu}
+            "extra": {"pct_of_mfma_peak": round(100 * tf / MFMA_PEAK_TFLOPS[args.path], 2),
+                      # the chunk's algorithmic bytes (every expert's matrices once, the tokens' rows in, the summed rows out)
+                      # over its time: not bound by memory
+                      "algorithmic_GBps": round((ne * (2.0 * pool.gate_bytes + pool.down_bytes) + 2 * 4.0 * n * d) / (ms * 1e-3) / 1e9, 1)},
+            "roofline": roof, "cpu": cpu}
 
 
 def workload_c2d(args, dev):
