@@ -1050,6 +1050,135 @@ __global__ __launch_bounds__(1024) void attn_values_chunk_kernel(const float* __
   if (tt < tn) out[((long long)(t0 + tt) * nh + h) * hd + 32 * cs + c] = o;
 }
 
+// The same values with sixteen chains a thread, four tokens by four columns: a workgroup of 256 threads takes a query
+// head's HD columns for 4096 / HD tokens (32 at HD = 128).  The kernel above reads LDS eight times (16 bytes each) per
+// chain and 16 positions, which is what it waits for; here the four scores of a token (16 bytes along the positions)
+// serve four columns and a position's four values (16 bytes along the columns, as the cache holds them: no transpose)
+// four tokens -- half a read per chain and 4 positions -- and what is left is the multiplies and adds.  Tiles of 32
+// positions, in two LDS buffers, loaded into registers a tile ahead of their store.  A tile that lies wholly below all
+// of a wave's tokens goes without a test; the one or two at the tokens' own positions leave a chain alone from its
+// token's last position on.  Every chain: the same products and sums in the
+// same order as above.
+template <int HD>
+__global__ __launch_bounds__(256) void attn_values_quad_kernel(const float* __restrict__ raw, const float* __restrict__ vc, float* __restrict__ out,
+                                                               int nh, int nkv, int pos0, int ntok, int spitch) {
+  constexpr int CQ = HD / 4, TQ = 256 / CQ, NTOK = 4 * TQ, P = 32, SP = P + 4;
+  constexpr int NV = P * CQ / 256;                 // 16-byte pieces of a tile a thread brings in: of the values,
+  constexpr int NS = NTOK * (P / 4) / 256;         // of the scores
+  static_assert((NV == 2 || NV == 4) && (NS == 1 || NS == 2) && 256 % CQ == 0, "HD 64 or 128");
+  __shared__ __align__(16) float scs[2][NTOK * SP];      // a row a token
+  __shared__ __align__(16) float vts[2][P * HD];         // a row a position
+  const int gx = gridDim.x, h = (gx & 7) ? (int)blockIdx.x : (int)(blockIdx.x & 7) * (gx >> 3) + (int)(blockIdx.x >> 3);
+  // (token tiles: the first half of the launch takes them from the last -- the longest -- downwards, the second half
+  // from the first upwards: workgroups half a launch apart tend to share a CU, and so a long one meets a short one)
+  const int ny = gridDim.y, yh = ny >> 1, by = blockIdx.y;
+  const int t0 = (by < yh ? ny - 1 - by : by - yh) * NTOK, tid = threadIdx.x;
+  const int tn = min(NTOK, ntok - t0), nposmax = pos0 + t0 + tn;
+  const int group = nh / nkv, kvd = nkv * HD, ko = (h / group) * HD;
+  const float* rbase = raw + ((long long)t0 * nh + h) * spitch;
+  const int tq = tid / CQ, cq = tid - tq * CQ;     // tokens t0 + 4 tq .. + 3, columns 4 cq .. + 3
+  const int wtq = (tid >> 6) * (64 / CQ);          // the wave's first tq
+  const int ntiles = (nposmax + P - 1) / P;
+  // (named registers: arrays indexed in these loops were left in private memory)
+  float4 rs0 = {}, rs1 = {}, rv0 = {}, rv1 = {}, rv2 = {}, rv3 = {};
+  // (past a token's own positions, past the rows' end and past the chunk's last token: a piece that exists, never used)
+  auto load_s = [&](int p0, int u) {
+    const int i = tid + 256 * u, rt = min(i >> 3, tn - 1), pc = min((p0 >> 2) + (i & 7), (spitch >> 2) - 1);
+    return *(const float4*)(rbase + (long long)rt * nh * spitch + 4 * pc);
+  };
+  auto load_v = [&](int p0, int u) {
+    const int k = tid + 256 * u, p = min(p0 + k / CQ, nposmax - 1);
+    return *(const float4*)(vc + (long long)p * kvd + ko + 4 * (k % CQ));
+  };
+  auto load_tile = [&](int tile) {
+    const int p0 = tile * P;
+    rs0 = load_s(p0, 0);
+    if (NS > 1) rs1 = load_s(p0, 1);
+    rv0 = load_v(p0, 0);
+    if (NV > 1) rv1 = load_v(p0, 1);
+    if (NV > 2) { rv2 = load_v(p0, 2); rv3 = load_v(p0, 3); }
+  };
+  auto store_s = [&](int buf, int u, const float4& r) {
+    const int i = tid + 256 * u;
+    *(float4*)(scs[buf] + (i >> 3) * SP + 4 * (i & 7)) = r;
+  };
+  auto store_tile = [&](int buf) {
+    store_s(buf, 0, rs0);
+    if (NS > 1) store_s(buf, 1, rs1);
+    *(float4*)(vts[buf] + 4 * tid) = rv0;
+    if (NV > 1) *(float4*)(vts[buf] + 4 * (tid + 256)) = rv1;
+    if (NV > 2) { *(float4*)(vts[buf] + 4 * (tid + 512)) = rv2; *(float4*)(vts[buf] + 4 * (tid + 768)) = rv3; }
+  };
+  float acc[4][4];
+#pragma unroll
+  for (int i = 0; i < 4; i++)
+#pragma unroll
+    for (int k = 0; k < 4; k++) acc[i][k] = 0.0f;
+  load_tile(0);
+  store_tile(0);
+  if (ntiles > 1) load_tile(1);
+  __syncthreads();
+  for (int t = 0; t < ntiles; t++) {
+    // tile t is in buffer t & 1; the registers hold tile t+1, and the other buffer's readers passed the last barrier
+    if (t + 1 < ntiles) store_tile((t + 1) & 1);
+    if (t + 2 < ntiles) load_tile(t + 2);
+    const float* S = scs[t & 1] + 4 * tq * SP;
+    const float* V = vts[t & 1] + 4 * cq;
+    // of the tile's positions, token 4 tq + i has the first np + i (all of them from 32 on, none up to 0)
+    const int np = pos0 + t0 + 4 * tq + 1 - t * P;
+    const int npw = pos0 + t0 + 4 * wtq + 1 - t * P;       // the wave's first tokens': its least
+    if (npw >= P) {
+#pragma unroll
+      for (int q = 0; q < P / 4; q++) {
+        float4 s[4], v[4];
+#pragma unroll
+        for (int i = 0; i < 4; i++) s[i] = *(const float4*)(S + i * SP + 4 * q);
+#pragma unroll
+        for (int j = 0; j < 4; j++) v[j] = *(const float4*)(V + (4 * q + j) * HD);
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+#pragma unroll
+          for (int i = 0; i < 4; i++) {
+            const float sv = j == 0 ? s[i].x : j == 1 ? s[i].y : j == 2 ? s[i].z : s[i].w;
+            acc[i][0] = acc[i][0] + sv * v[j].x;
+            acc[i][1] = acc[i][1] + sv * v[j].y;
+            acc[i][2] = acc[i][2] + sv * v[j].z;
+            acc[i][3] = acc[i][3] + sv * v[j].w;
+          }
+      }
+    } else if (npw + 4 * (64 / CQ) - 1 > 0) {              // some lane of the wave has positions here
+#pragma unroll 1
+      for (int q = 0; q < P / 4; q++) {
+        if (4 * q >= np + 3) break;
+        float4 s[4], v[4];
+#pragma unroll
+        for (int i = 0; i < 4; i++) s[i] = *(const float4*)(S + i * SP + 4 * q);
+#pragma unroll
+        for (int j = 0; j < 4; j++) v[j] = *(const float4*)(V + (4 * q + j) * HD);
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+#pragma unroll
+          for (int i = 0; i < 4; i++) {
+            const float sv = j == 0 ? s[i].x : j == 1 ? s[i].y : j == 2 ? s[i].z : s[i].w;
+            const bool own = 4 * q + j < np + i;
+            const float a0 = acc[i][0] + sv * v[j].x, a1 = acc[i][1] + sv * v[j].y;
+            const float a2 = acc[i][2] + sv * v[j].z, a3 = acc[i][3] + sv * v[j].w;
+            acc[i][0] = own ? a0 : acc[i][0];
+            acc[i][1] = own ? a1 : acc[i][1];
+            acc[i][2] = own ? a2 : acc[i][2];
+            acc[i][3] = own ? a3 : acc[i][3];
+          }
+      }
+    }
+    __syncthreads();
+  }
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+    const int tk = t0 + 4 * tq + i;
+    if (tk < ntok) *(float4*)(out + ((long long)tk * nh + h) * HD + 4 * cq) = make_float4(acc[i][0], acc[i][1], acc[i][2], acc[i][3]);
+  }
+}
+
 // ARGMAX (model.lisp:464-468): best = 0; an element replaces the best when it is greater -- so the first of equal
 // maxima, a NaN never (and if v[0] is a NaN nothing replaces it).  Two steps: each workgroup the best of its
 // stretch (every thread's own elements first, eight 16-byte loads in flight, then the threads', a smaller index
@@ -1163,6 +1292,17 @@ hipError_t ilt_k_attn_rows(const float* q, const float* kc, const float* vc, flo
       const int ctx = pos0 + ntok;
       launch_scores<16>(dim3(nh, (ctx + 255) / 256, (ntok + 15) / 16), st, q, kc, scratch, nh, nkv, hd, pos0, ntok, scale, smax);
       hipLaunchKernelGGL(attn_softmax_kernel, dim3(nh, ntok), dim3(256), sizeof(float) * smax, st, scratch, nh, pos0, smax);
+      // sixteen chains a thread for heads of 64 or 128 columns (16-byte loads and stores: of scratch, vc and out);
+      // "ILT_ATTN_QUAD=0": the kernel of one chain a thread (tests)
+      const char* quad = getenv("ILT_ATTN_QUAD");
+      const bool aligned = ((((uintptr_t)scratch) | ((uintptr_t)vc) | ((uintptr_t)out)) & 15) == 0;
+      if ((hd == 128 || hd == 64) && aligned && !(quad && quad[0] == '0')) {
+        if (hd == 128)
+          hipLaunchKernelGGL(attn_values_quad_kernel<128>, dim3(nh, (ntok + 31) / 32), dim3(256), 0, st, scratch, vc, out, nh, nkv, pos0, ntok, smax);
+        else
+          hipLaunchKernelGGL(attn_values_quad_kernel<64>, dim3(nh, (ntok + 63) / 64), dim3(256), 0, st, scratch, vc, out, nh, nkv, pos0, ntok, smax);
+        return hipGetLastError();
+      }
       hipLaunchKernelGGL(attn_values_chunk_kernel, dim3(nh * (hd / 32), (ntok + 31) / 32), dim3(1024), smem, st, scratch, vc, out, nh, nkv, hd, pos0,
                          ntok, smax);
       return hipGetLastError();

@@ -372,6 +372,38 @@ def test_chunk_attention_on_the_kernels_of_16_tokens(dev, monkeypatch):
     assert same == 2
 
 
+@pytest.mark.parametrize("nh,nkv,hd,pos0,ntok", [(8, 2, 128, 0, 100), (8, 2, 128, 300, 77), (3, 1, 128, 37, 33), (8, 2, 64, 0, 130),
+                                                 (6, 2, 64, 500, 65), (16, 4, 128, 1536, 512), (8, 8, 64, 31, 1)])
+def test_chunk_values_with_sixteen_chains_a_thread(dev, monkeypatch, nh, nkv, hd, pos0, ntok):
+    """A chunk's attention through scores, softmax and the values kernel of four tokens x four columns a thread (heads of
+    64 and 128) against attn_rows' one launch (a workgroup a head and token, the CPU's float order from end to end) and
+    against the values kernel of one chain a thread: bit for bit; chunks that end inside a token tile, that start at a
+    position that is no multiple of the position tile, heads that do not fill the eight dies, one token."""
+    import ctypes as C
+    from illatio_amd import hip
+    rng = synth.make_rng(1000 + nh + hd + pos0 + ntok)
+    f = lambda *sh: (rng.standard_normal(sh) * 1.5).astype(np.float32)
+    nctx = pos0 + ntok
+    q, kc, vc = (hip.hip_upload_new(dev, a) for a in (f(ntok, nh * hd), f(nctx, nkv * hd), f(nctx, nkv * hd)))
+    smax = (nctx + 3) & ~3
+    scratch = hip.hip_alloc(dev, 4 * ntok * nh * smax)
+    P = lambda b: C.c_uint64(b.ptr if b is not None else 0)
+    ints = (C.c_int(nh), C.c_int(nkv), C.c_int(hd), C.c_int(pos0), C.c_int(ntok))
+    outs = []
+    for scr, quad in ((None, None), (scratch, "1"), (scratch, "0")):
+        if quad is not None:
+            monkeypatch.setenv("ILT_ATTN_QUAD", quad)
+        out = hip.hip_upload_new(dev, np.full(ntok * nh * hd, np.nan, np.float32))
+        hip.call("ilt_attn_rows", C.c_uint64(0), P(q), P(kc), P(vc), P(out), *ints, P(scr))
+        outs.append(hip.hip_floats(out, ntok * nh * hd))
+        hip.hip_free(out)
+    assert not np.isnan(outs[0]).any()
+    assert np.array_equal(bits(outs[1]), bits(outs[0])), np.abs(outs[1] - outs[0]).max()
+    assert np.array_equal(bits(outs[2]), bits(outs[0]))
+    for b in (q, kc, vc, scratch):
+        hip.hip_free(b)
+
+
 def test_decode_across_position_8192(dev):
     """A context longer than the 8,192 positions the kernels with their scores in memory take: tokens at positions 8,190
     and 8,191 go through ilt_dense_decode (tiled values), those at 8,192 and 8,193 through qk_rope + attn_rows with the
