@@ -281,6 +281,117 @@ __global__ __launch_bounds__(1024) void attn_scores_kernel(const float* __restri
   }
 }
 
+// A prompt chunk's scores, sixteen of them a thread: a workgroup of 256 threads takes 64 tokens x 64 positions of a
+// query head, thread (tq, pq) the tokens tq + 16a and the positions pq + 16b.  F32-DOT16 keeps sixteen running sums,
+// sum l over the columns l, l + 16, ..., and adds them as ((s_l + s_l+4) + (s_l+8 + s_l+12)) = X_l for l = 0..3, then
+// (X_0 + X_1) + (X_2 + X_3).  The kernel above gives a score to sixteen lanes, a running sum each, and every lane
+// then goes through the four adds of the tree and the scaling for the sake of lane 0; here one thread keeps a score's
+// four sums l = e, e+4, e+8, e+12 for e = 0, 1, 2, 3 in turn, so that nothing is added that the score does not need, and
+// a 16-byte read of a token's or a position's row serves four scores.  For that the rows lie in LDS with every sixteen
+// columns transposed as 4 x 4 (place 4e + m holds column 4m + e): a thread that brings a row's sixteen columns in
+// stores them as four pieces of 16 bytes.  Row pitch HD + 4 floats: sixteen lanes' 16-byte reads of sixteen
+// consecutive rows fall on different banks.  The numbers are those of the kernel above.
+template <int NJ>      // HD / 16
+__global__ __launch_bounds__(256, 2) void attn_scores_quad_kernel(const float* __restrict__ q, const float* __restrict__ kc, float* __restrict__ raw,
+                                                               int nh, int nkv, int pos0, int ntok, float scale, int spitch) {
+  constexpr int HD = 16 * NJ, RP = HD + 4;
+  extern __shared__ __align__(16) float dyn[];     // 2 * 64 * RP floats
+  float* const qs = dyn;
+  float* const ks = dyn + 64 * RP;
+  const int h = blockIdx.x, p0 = blockIdx.y * 64, t0 = blockIdx.z * 64, tid = threadIdx.x;
+  const int tn = min(64, ntok - t0), nposmax = pos0 + t0 + tn;
+  if (p0 >= nposmax) return;                       // the same in every thread
+  const int group = nh / nkv, kvd = nkv * HD, ko = (h / group) * HD;
+  // rows 0..63: the tokens' q, 64..127: the positions' keys; 128 * NJ groups of sixteen columns, NJ / 2 a thread
+#pragma unroll
+  for (int u = 0; u < NJ / 2; u++) {
+    const int g = tid + 256 * u, row = g / NJ, j = g - row * NJ;
+    const float* src = row < 64 ? q + ((long long)(t0 + min(row, tn - 1)) * nh + h) * HD + 16 * j
+                                : kc + (long long)min(p0 + row - 64, nposmax - 1) * kvd + ko + 16 * j;
+    const float4 m0 = *(const float4*)src, m1 = *(const float4*)(src + 4), m2 = *(const float4*)(src + 8), m3 = *(const float4*)(src + 12);
+    float* dst = (row < 64 ? qs + row * RP : ks + (row - 64) * RP) + 16 * j;
+    *(float4*)dst = make_float4(m0.x, m1.x, m2.x, m3.x);
+    *(float4*)(dst + 4) = make_float4(m0.y, m1.y, m2.y, m3.y);
+    *(float4*)(dst + 8) = make_float4(m0.z, m1.z, m2.z, m3.z);
+    *(float4*)(dst + 12) = make_float4(m0.w, m1.w, m2.w, m3.w);
+  }
+  __syncthreads();
+  const int tq = tid >> 4, pq = tid & 15;
+  // none of the thread's positions is any of its tokens' to see (its first position, its last token)
+  if (p0 + pq >= pos0 + t0 + tq + 48 + 1) return;
+  const float* Q = qs + tq * RP;
+  const float* K = ks + pq * RP;
+  float y[4][4], z[4][4];
+  auto read_step = [&](float4 (&qr)[4], float4 (&kr)[4], const float* Qe, const float* Ke) {
+#pragma unroll
+    for (int a = 0; a < 4; a++) qr[a] = *(const float4*)(Qe + 16 * a * RP);
+#pragma unroll
+    for (int b = 0; b < 4; b++) kr[b] = *(const float4*)(Ke + 16 * b * RP);
+  };
+  // sums e, e+4, e+8, e+12 of the sixteen scores: two steps of sixteen columns a turn of the loop, each step's reads sent
+  // off before the step before it is multiplied (left to itself the compiler reads every step's rows first and spills)
+  auto sums = [&](auto Ec) {
+    constexpr int e = decltype(Ec)::value;
+    float4 acc[4][4], qa[4], ka[4], qb[4], kb[4];
+#pragma unroll
+    for (int a = 0; a < 4; a++)
+#pragma unroll
+      for (int b = 0; b < 4; b++) acc[a][b] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+    auto mac = [&](const float4 (&qr)[4], const float4 (&kr)[4]) {
+#pragma unroll
+      for (int a = 0; a < 4; a++)
+#pragma unroll
+        for (int b = 0; b < 4; b++) {
+          acc[a][b].x = acc[a][b].x + kr[b].x * qr[a].x;
+          acc[a][b].y = acc[a][b].y + kr[b].y * qr[a].y;
+          acc[a][b].z = acc[a][b].z + kr[b].z * qr[a].z;
+          acc[a][b].w = acc[a][b].w + kr[b].w * qr[a].w;
+        }
+    };
+    const float* Qe = Q + 4 * e;
+    const float* Ke = K + 4 * e;
+    read_step(qa, ka, Qe, Ke);
+#pragma unroll 1
+    for (int j = 0; j < NJ; j += 2) {
+      read_step(qb, kb, Qe + 16 * (j + 1), Ke + 16 * (j + 1));
+      mac(qa, ka);
+      asm volatile("" ::: "memory");
+      const int jn = min(j + 2, NJ - 2);           // (after the last step: rows read again, for nobody)
+      read_step(qa, ka, Qe + 16 * jn, Ke + 16 * jn);
+      mac(qb, kb);
+      asm volatile("" ::: "memory");
+    }
+#pragma unroll
+    for (int a = 0; a < 4; a++)
+#pragma unroll
+      for (int b = 0; b < 4; b++) {
+        float x = (acc[a][b].x + acc[a][b].y) + (acc[a][b].z + acc[a][b].w);      // X_e
+        asm volatile("" : "+v"(x));                // (added here, not where the score is stored: the four sums are not kept till then)
+        if (e == 0) y[a][b] = x;
+        if (e == 1) y[a][b] = y[a][b] + x;
+        if (e == 2) z[a][b] = x;
+        if (e == 3) z[a][b] = z[a][b] + x;
+      }
+    __builtin_amdgcn_sched_barrier(0);             // (one set of sums in registers at a time)
+  };
+  sums(std::integral_constant<int, 0>{});
+  sums(std::integral_constant<int, 1>{});
+  sums(std::integral_constant<int, 2>{});
+  sums(std::integral_constant<int, 3>{});
+#pragma unroll
+  for (int a = 0; a < 4; a++) {
+    const int tt = tq + 16 * a, npos = pos0 + t0 + tt + 1;
+    if (tt < tn) {
+      float* dst = raw + ((long long)(t0 + tt) * nh + h) * spitch;
+#pragma unroll
+      for (int b = 0; b < 4; b++) {
+        const int p = p0 + pq + 16 * b;
+        if (p < npos) dst[p] = (y[a][b] + z[a][b]) * scale;
+      }
+    }
+  }
+}
+
 // One token's qk_rope and scores in one launch: every workgroup of a query head norms and turns that head
 // itself (wave 0; a sixteenth of a microsecond of arithmetic against a launch), the workgroup whose 256
 // positions hold the token's own does the same for its KV head's key (wave 1) and takes that key from LDS,
@@ -1290,11 +1401,29 @@ hipError_t ilt_k_attn_rows(const float* q, const float* kc, const float* vc, flo
         set[dev] = true;
       }
       const int ctx = pos0 + ntok;
-      launch_scores<16>(dim3(nh, (ctx + 255) / 256, (ntok + 15) / 16), st, q, kc, scratch, nh, nkv, hd, pos0, ntok, scale, smax);
+      // sixteen scores a thread for heads of 64 or 128 columns (16-byte loads of q and kc); "ILT_ATTN_QUAD=0" or "=v": the
+      // kernel of sixteen lanes a score (tests)
+      const char* quad = getenv("ILT_ATTN_QUAD");
+      const bool qaligned = ((((uintptr_t)q) | ((uintptr_t)kc)) & 15) == 0;
+      if ((hd == 128 || hd == 64) && qaligned && !(quad && (quad[0] == '0' || quad[0] == 'v'))) {
+        static bool qset[64] = {};
+        const size_t qsmem = sizeof(float) * 2 * 64 * (size_t)(hd + 4);
+        if (!qset[dev]) {
+          hipError_t e = hipFuncSetAttribute((const void*)attn_scores_quad_kernel<8>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)(sizeof(float) * 2 * 64 * 132));
+          if (e == hipSuccess)
+            e = hipFuncSetAttribute((const void*)attn_scores_quad_kernel<4>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)(sizeof(float) * 2 * 64 * 68));
+          if (e != hipSuccess) return e;
+          qset[dev] = true;
+        }
+        const dim3 gq(nh, (ctx + 63) / 64, (ntok + 63) / 64);
+        if (hd == 128) hipLaunchKernelGGL(attn_scores_quad_kernel<8>, gq, dim3(256), qsmem, st, q, kc, scratch, nh, nkv, pos0, ntok, scale, smax);
+        else hipLaunchKernelGGL(attn_scores_quad_kernel<4>, gq, dim3(256), qsmem, st, q, kc, scratch, nh, nkv, pos0, ntok, scale, smax);
+      } else {
+        launch_scores<16>(dim3(nh, (ctx + 255) / 256, (ntok + 15) / 16), st, q, kc, scratch, nh, nkv, hd, pos0, ntok, scale, smax);
+      }
       hipLaunchKernelGGL(attn_softmax_kernel, dim3(nh, ntok), dim3(256), sizeof(float) * smax, st, scratch, nh, pos0, smax);
       // sixteen chains a thread for heads of 64 or 128 columns (16-byte loads and stores: of scratch, vc and out);
       // "ILT_ATTN_QUAD=0": the kernel of one chain a thread (tests)
-      const char* quad = getenv("ILT_ATTN_QUAD");
       const bool aligned = ((((uintptr_t)scratch) | ((uintptr_t)vc) | ((uintptr_t)out)) & 15) == 0;
       if ((hd == 128 || hd == 64) && aligned && !(quad && quad[0] == '0')) {
         if (hd == 128)

@@ -374,9 +374,9 @@ def test_chunk_attention_on_the_kernels_of_16_tokens(dev, monkeypatch):
 
 @pytest.mark.parametrize("nh,nkv,hd,pos0,ntok", [(8, 2, 128, 0, 100), (8, 2, 128, 300, 77), (3, 1, 128, 37, 33), (8, 2, 64, 0, 130),
                                                  (6, 2, 64, 500, 65), (16, 4, 128, 1536, 512), (8, 8, 64, 31, 1)])
-def test_chunk_values_with_sixteen_chains_a_thread(dev, monkeypatch, nh, nkv, hd, pos0, ntok):
-    """A chunk's attention through scores, softmax and the values kernel of four tokens x four columns a thread (heads of
-    64 and 128) against attn_rows' one launch (a workgroup a head and token, the CPU's float order from end to end) and
+def test_chunk_attention_with_sixteen_scores_and_chains_a_thread(dev, monkeypatch, nh, nkv, hd, pos0, ntok):
+    """A chunk's attention through the scores kernel of four tokens x four positions a thread, softmax and the values kernel
+    of four tokens x four columns a thread (heads of 64 and 128) against attn_rows' one launch (a workgroup a head and token, the CPU's float order from end to end) and
     against the values kernel of one chain a thread: bit for bit; chunks that end inside a token tile, that start at a
     position that is no multiple of the position tile, heads that do not fill the eight dies, one token."""
     import ctypes as C
@@ -390,7 +390,7 @@ def test_chunk_values_with_sixteen_chains_a_thread(dev, monkeypatch, nh, nkv, hd
     P = lambda b: C.c_uint64(b.ptr if b is not None else 0)
     ints = (C.c_int(nh), C.c_int(nkv), C.c_int(hd), C.c_int(pos0), C.c_int(ntok))
     outs = []
-    for scr, quad in ((None, None), (scratch, "1"), (scratch, "0")):
+    for scr, quad in ((None, None), (scratch, "1"), (scratch, "v"), (scratch, "0")):      # "v": only the values on the new kernel
         if quad is not None:
             monkeypatch.setenv("ILT_ATTN_QUAD", quad)
         out = hip.hip_upload_new(dev, np.full(ntok * nh * hd, np.nan, np.float32))
@@ -399,7 +399,7 @@ def test_chunk_values_with_sixteen_chains_a_thread(dev, monkeypatch, nh, nkv, hd
         hip.hip_free(out)
     assert not np.isnan(outs[0]).any()
     assert np.array_equal(bits(outs[1]), bits(outs[0])), np.abs(outs[1] - outs[0]).max()
-    assert np.array_equal(bits(outs[2]), bits(outs[0]))
+    assert np.array_equal(bits(outs[2]), bits(outs[0])) and np.array_equal(bits(outs[3]), bits(outs[0]))
     for b in (q, kc, vc, scratch):
         hip.hip_free(b)
 
