@@ -84,8 +84,11 @@ def _mat(w):
 class DenseModel:
     """HOST (synth_model's dict, or the same made from a file's tensors) on DEV, with caches for NCTX positions."""
 
-    def __init__(self, dev, host, nctx, chunk=512, prefill="exact"):
-        """PREFILL: how a chunk of several tokens is multiplied.  "exact": the int8 products, every token with the bits
+    def __init__(self, dev, host, nctx, chunk=2048, prefill="exact"):
+        """CHUNK: the tokens of a prompt that go through the layers together (*CUDA-CHUNK*, cuda-dense.lisp:29, is 512;
+        on 256 CUs a 512-token chunk's smaller products -- V, wo, down -- are 64 to 160 workgroups, and a 2,048-token
+        prompt takes 79.6 ms in one chunk against 99.1 ms in four; the results do not depend on it).
+        PREFILL: how a chunk of several tokens is multiplied.  "exact": the int8 products, every token with the bits
         of its own decode step (the CPU path's MATMUL!).  "bf16": the bf16 matrix-core products on the CPU path's own
         quantized activations (each Q8_K quant times its block scale, rounded to bf16), K-quant matrices only: within
         the bf16 roundings of the exact products, not equal to them.  "bf16-resident": the same numbers from bf16
@@ -95,6 +98,7 @@ class DenseModel:
         if prefill not in ("exact", "bf16", "bf16-resident"):
             raise ValueError(f"prefill {prefill!r}: exact, bf16 or bf16-resident")
         self.prefill = prefill
+        chunk = max(1, min(chunk, nctx))
         self.dev, self.c, self.nctx, self.chunk, self.pos = dev, c, nctx, chunk, 0
         d, ffn, hd = c["d"], c["ffn"], c["hd"]
         self.qd, self.kvd = c["nh"] * hd, c["nkv"] * hd

@@ -344,7 +344,7 @@ def test_small_decoder_long_contexts(dev):
     assert same == 3
     # one token's values past 2,048 positions come in tiles of 480 positions while the chains run: the decode steps cross
     # a tile's edge (2,400 -> 2,401), with an even and with an odd number of tiles
-    same, _ = run_greedy(dev, host, nprompt=2397, ndecode=6, chunk=512, nctx=2410, seed=15)
+    same, _ = run_greedy(dev, host, nprompt=2397, ndecode=6, chunk=2048, nctx=2410, seed=15)      # (a chunk of 2,048 tokens, then 349)
     assert same == 6
     same, _ = run_greedy(dev, host, nprompt=2878, ndecode=5, chunk=512, nctx=2890, seed=16)
     assert same == 5
