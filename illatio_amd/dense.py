@@ -130,24 +130,46 @@ def cmat_mul(dev, w, act, y, n=1, bias=None, acc=False):
     return y
 
 
+BESIDE = True      # False: cmat_mul_n's launches one after another on the device's stream
+
+
 def cmat_mul_n(dev, parts, act, n, acc=False):
     """PARTS, (W Y BIAS) sharing X, for N tokens (CMAT-MUL-N, cuda-dense.lisp:250-258): the K-quant matrices of one
     type, up to three at a time, in one launch of mm_k_n; whatever is left one by one."""
-    todo = list(parts)
+    todo, groups = list(parts), []
     while todo:
         w0 = todo[0][0]
         same = [pt for pt in todo if pt[0].kquant_p() and pt[0].type == w0.type and pt[0].cols == w0.cols][:3] if w0.kquant_p() and n > 1 else []
         if len(same) >= 2:
-            args = [KQUANT_CODE[w0.type]]
-            for k in range(3):
-                w, y, bias = same[k] if k < len(same) else (None, None, None)
-                args += [w.qs if w else None, y, bias, w.rows if w else 0]
-            hip.launch(dev, "mm_k_n", ((n + 127) // 128, sum((w.rows + 127) // 128 for w, _, _ in same)), 512,
-                       args + [act.kq, act.kd, act.ksum, w0.cols, n, 1 if acc else 0])
+            groups.append(same)
             todo = [pt for pt in todo if not any(pt is q for q in same)]
         else:
-            w, y, bias = todo.pop(0)
+            groups.append([todo.pop(0)])
+
+    def run(group):
+        if len(group) >= 2:
+            w0 = group[0][0]
+            args = [KQUANT_CODE[w0.type]]
+            for k in range(3):
+                w, y, bias = group[k] if k < len(group) else (None, None, None)
+                args += [w.qs if w else None, y, bias, w.rows if w else 0]
+            hip.launch(dev, "mm_k_n", ((n + 127) // 128, sum((w.rows + 127) // 128 for w, _, _ in group)), 512,
+                       args + [act.kq, act.kd, act.ksum, w0.cols, n, 1 if acc else 0])
+        else:
+            w, y, bias = group[0]
             cmat_mul(dev, w, act, y, n=n, bias=bias, acc=acc)
+
+    # A chunk's launches share X and write different Y: the ones after the first go to the device's second stream
+    # (Q+K is 320 workgroups at 512 tokens and V 64: side by side they take what Q+K takes).
+    if len(groups) > 1 and n > 1 and BESIDE:
+        with hip.beside(dev):
+            for g in groups[1:]:
+                run(g)
+        run(groups[0])
+        hip.rejoin(dev)
+    else:
+        for g in groups:
+            run(g)
 
 
 def cvt_bf16(dev, x, n_elems, out=None):

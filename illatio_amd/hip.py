@@ -262,6 +262,36 @@ def hip_stream_sync(stream):
     call("ilt_stream_sync", C.c_uint64(stream))
 
 
+class beside:
+    """with beside(dev): what is queued inside goes to DEV's second stream, which first waits for everything DEV's
+    stream holds so far; rejoin(dev) then makes DEV's stream wait for it.  For launches that do not depend on each
+    other and do not fill the GPU one by one (a prompt chunk's V product beside its Q and K product).  Both streams
+    at the default priority."""
+
+    def __init__(self, dev):
+        self.dev = dev
+
+    def __enter__(self):
+        dev = self.dev
+        if getattr(dev, "second", None) is None:
+            dev.second = hip_stream_create(dev)
+            dev.forked, dev.joined = hip_event_create(dev), hip_event_create(dev)
+        hip_event_record(dev.forked, dev.stream)
+        hip_stream_wait(dev.second, dev.forked)
+        self.main, dev.stream = dev.stream, dev.second
+        return self
+
+    def __exit__(self, *exc):
+        dev = self.dev
+        dev.stream = self.main
+        hip_event_record(dev.joined, dev.second)
+        return False
+
+
+def rejoin(dev):
+    hip_stream_wait(dev.stream, dev.joined)
+
+
 class I64:
     """(:i64 n): a long long argument for LAUNCH."""
 
