@@ -1098,6 +1098,11 @@ int ilt_swiglu(uint64_t stream, float* a, const float* b, int64_t n) {
   ILT_REQUIRE(n >= 0 && (n == 0 || (a && b)));
   return (int)ilt_k_swiglu_rows(a, b, n, S(stream));
 }
+int ilt_swiglu_quant_q8k(uint64_t stream, const float* gate, const float* up, int8_t* xq, float* xd, int32_t* bsums, int64_t nblocks) {
+  ILT_REQUIRE(nblocks >= 0 && (nblocks == 0 || (gate && up && xq && xd && bsums)));
+  ILT_REQUIRE(((((uintptr_t)gate) | ((uintptr_t)up)) & 15) == 0);
+  return (int)ilt_k_swiglu_quant_q8k(gate, up, xq, xd, bsums, nblocks, S(stream));
+}
 
 int ilt_launch(const char* kernel, unsigned gx, unsigned gy, unsigned gz, unsigned bx, unsigned by, unsigned bz,
                unsigned shared_bytes, uint64_t stream, void** params) {

@@ -122,6 +122,7 @@ unsigned long long ilt_k_streamed_launches();      // decode products launched a
 
 hipError_t ilt_k_quant_q8(const float* x, int8_t* xq, float* xs, int* xsum, long long nblocks, int f16_scale, hipStream_t st);
 hipError_t ilt_k_quant_q8k(const float* x, int8_t* xq, float* xd, int* bsums, long long nblocks, hipStream_t st);
+hipError_t ilt_k_swiglu_quant_q8k(const float* gate, const float* up, int8_t* xq, float* xd, int* bsums, long long nblocks, hipStream_t st);
 // ntok rows of cols floats, x_stride floats apart, quantized into packed rows: quantize-q8! (k 0) or quantize-q8k! (k 1)
 hipError_t ilt_k_quant_rows(int k, const float* x, int8_t* xq, float* xs, int* bsums, long long ntok, int cols, long long x_stride,
                             int f16_scale, hipStream_t st);

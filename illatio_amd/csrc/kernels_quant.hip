@@ -39,7 +39,11 @@ __global__ __launch_bounds__(256) void quant_q8_kernel(const float* __restrict__
 // (a 16-byte load, a 4-byte store; no LDS, no barrier).  The largest-magnitude value, the
 // first of equals, sets iscale = -127/max; q = min(127, round-half-even(iscale*x));
 // d = 1/iscale; sums of each 16 quants.
-__global__ __launch_bounds__(256) void quant_q8k_kernel(const float* __restrict__ x, i8* __restrict__ xq,
+// GLU: the values quantized are swiglu!'s (model.lisp:364-378) of x and up, (x / (1 + e^-x)) * up with the exponential
+// through double -- a prompt chunk's gated activations go straight into the blocks the down product reads, and the
+// floats are neither written nor read again.
+template <bool GLU>
+__global__ __launch_bounds__(256) void quant_q8k_kernel(const float* __restrict__ x, const float* __restrict__ up, i8* __restrict__ xq,
                                                         float* __restrict__ xd, int* __restrict__ bsums, long long nblocks,
                                                         long long bpr, long long x_stride) {
   const int lane = threadIdx.x & 63;
@@ -47,7 +51,13 @@ __global__ __launch_bounds__(256) void quant_q8k_kernel(const float* __restrict_
   if (b >= nblocks) return;
   // bpr > 0: rows of bpr blocks, x_stride floats (a multiple of 4) from one row's start to the next's
   const float4 v4 = ((const float4*)(x + (bpr > 0 ? (b / bpr) * x_stride + (b % bpr) * 256 : b * 256)))[lane];
-  const float v[4] = {v4.x, v4.y, v4.z, v4.w};
+  float v[4] = {v4.x, v4.y, v4.z, v4.w};
+  if (GLU) {
+    const float4 u4 = ((const float4*)(up + b * 256))[lane];
+    const float u[4] = {u4.x, u4.y, u4.z, u4.w};
+#pragma unroll
+    for (int k = 0; k < 4; k++) v[k] = (v[k] / (1.0f + ilt_expf_via_double(-v[k]))) * u[k];
+  }
   // |v|'s bits order as |v| does; the low word prefers the earlier index
   u64 key = 0;
 #pragma unroll
@@ -243,7 +253,13 @@ hipError_t ilt_k_quant_q8(const float* x, int8_t* xq, float* xs, int* xsum, long
 
 hipError_t ilt_k_quant_q8k(const float* x, int8_t* xq, float* xd, int* bsums, long long nblocks, hipStream_t st) {
   if (nblocks <= 0) return hipSuccess;
-  hipLaunchKernelGGL(quant_q8k_kernel, dim3((unsigned)((nblocks + 3) / 4)), dim3(256), 0, st, x, xq, xd, bsums, nblocks, 0LL, 0LL);
+  hipLaunchKernelGGL(quant_q8k_kernel<false>, dim3((unsigned)((nblocks + 3) / 4)), dim3(256), 0, st, x, (const float*)nullptr, xq, xd, bsums, nblocks, 0LL, 0LL);
+  return hipGetLastError();
+}
+
+hipError_t ilt_k_swiglu_quant_q8k(const float* gate, const float* up, int8_t* xq, float* xd, int* bsums, long long nblocks, hipStream_t st) {
+  if (nblocks <= 0) return hipSuccess;
+  hipLaunchKernelGGL(quant_q8k_kernel<true>, dim3((unsigned)((nblocks + 3) / 4)), dim3(256), 0, st, gate, up, xq, xd, bsums, nblocks, 0LL, 0LL);
   return hipGetLastError();
 }
 
@@ -253,7 +269,7 @@ hipError_t ilt_k_quant_rows(int k, const float* x, int8_t* xq, float* xs, int* b
   if (ntok <= 0) return hipSuccess;
   if (cols <= 0 || cols % bw != 0 || x_stride < cols || (k && x_stride % 4 != 0)) return hipErrorInvalidValue;
   const long long bpr = cols / bw, nblocks = ntok * bpr;
-  if (k) hipLaunchKernelGGL(quant_q8k_kernel, dim3((unsigned)((nblocks + 3) / 4)), dim3(256), 0, st, x, xq, xs, bsums, nblocks, bpr, x_stride);
+  if (k) hipLaunchKernelGGL(quant_q8k_kernel<false>, dim3((unsigned)((nblocks + 3) / 4)), dim3(256), 0, st, x, (const float*)nullptr, xq, xs, bsums, nblocks, bpr, x_stride);
   else hipLaunchKernelGGL(quant_q8_kernel, dim3((unsigned)((nblocks * 32 + 255) / 256)), dim3(256), 0, st, x, xq, xs, (int*)nullptr, nblocks,
                           f16_scale, bpr, x_stride);
   return hipGetLastError();

@@ -95,6 +95,18 @@ def quantize_act(dev, x, act, n=None, f16_scale=True):
     return act
 
 
+def swiglu_quantize_act(dev, gate, up, act, n):
+    """swiglu! of GATE and UP (N x COLS floats each) quantized into ACT's Q8_K blocks in one launch -- what the "swiglu"
+    launch and QUANTIZE-ACT! after it leave there, without the floats written and read again; None when ACT also
+    holds Q8_0 blocks (the caller then takes the two launches)."""
+    if act.xq is not None or act.kq is None:
+        return None
+    nb = n * act.cols // 256
+    hip.call("ilt_swiglu_quant_q8k", C.c_uint64(dev.stream), C.c_uint64(gate.ptr), C.c_uint64(up.ptr), C.c_uint64(act.kq.ptr),
+             C.c_uint64(act.kd.ptr), C.c_uint64(act.ksum.ptr), C.c_int64(nb))
+    return act
+
+
 def rmsnorm_q8(dev, x, w, act, d, eps, n=1, h=None, exact_order=False):
     """RMSNORM! of N rows of X (D wide) by W, quantized into ACT in each format it holds, the
     floats into H unless None (RMSNORM-Q8, cuda-dense.lisp:260-264; Q8_K blocks when ACT holds

@@ -200,6 +200,15 @@ class DenseModel:
                 for pt in parts:
                     run(*pt)
 
+        def gated():
+            """The chunk's gated activations as the down product reads them: swiglu and the quantizer in one launch, or
+            (a model with Q8_0 matrices) one after the other."""
+            a = dense.swiglu_quantize_act(dev, self.fa, self.fb, self.acts[ffn], n)
+            if a is None:
+                hip.call("ilt_swiglu", S, P(self.fa), P(self.fb), C.c_int64(n * ffn))
+                a = dense.quantize_act(dev, self.fa, self.acts[ffn], n=n)
+            return a
+
         for li, L in enumerate(self.layers):
             if n == 1:
                 dense.qkv_mul(dev, L["wq"], L["wk"], L["wv"], None, self.q, self.k, self.v, L["bq"], L["bk"], L["bv"], xf=self.x,
@@ -227,14 +236,12 @@ class DenseModel:
             elif fast:
                 mul_fast(li, [("wo", self.x, None)], dense.quantize_act(dev, self.att, self.acts[self.qd], n=n), acc=True)
                 mul_fast(li, [("gate", self.fa, None), ("up", self.fb, None)], dense.rmsnorm_q8(dev, self.x, L["ffn_norm"], self.acts[d], d, eps, n=n))
-                hip.call("ilt_swiglu", S, P(self.fa), P(self.fb), C.c_int64(n * ffn))
-                mul_fast(li, [("down", self.x, None)], dense.quantize_act(dev, self.fa, self.acts[ffn], n=n), acc=True)
+                mul_fast(li, [("down", self.x, None)], gated(), acc=True)
             else:
                 dense.cmat_mul(dev, L["wo"], dense.quantize_act(dev, self.att, self.acts[self.qd], n=n), self.x, n=n, acc=True)
                 a = dense.rmsnorm_q8(dev, self.x, L["ffn_norm"], self.acts[d], d, eps, n=n)
                 dense.cmat_mul_n(dev, [(L["gate"], self.fa, None), (L["up"], self.fb, None)], a, n)
-                hip.call("ilt_swiglu", S, P(self.fa), P(self.fb), C.c_int64(n * ffn))
-                dense.cmat_mul(dev, L["down"], dense.quantize_act(dev, self.fa, self.acts[ffn], n=n), self.x, n=n, acc=True)
+                dense.cmat_mul(dev, L["down"], gated(), self.x, n=n, acc=True)
         self.pos += n
         if logits:
             last = hip.DBuf(self.x.ptr + 4 * (n - 1) * d, 4 * d, dev)

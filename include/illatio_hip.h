@@ -388,6 +388,10 @@ typedef struct ilt_dense_model {
 } ilt_dense_model;
 int ilt_dense_decode(uint64_t stream, const ilt_dense_model* m, const int32_t* token, int pos, int want_logits);
 int ilt_swiglu(uint64_t stream, float* a, const float* b, int64_t n);
+/* ilt_swiglu followed by ilt_quant_q8k in one launch, for a prompt chunk whose gated activations only the down product
+   reads (GLU-MUL's "swiglu" launch, cuda-dense.lisp:338-339, and the quantizing launch that follows it in
+   CUDA-FORWARD-N, cuda-dense.lisp:417-418): the blocks are those the two leave, the floats are not written.  gate, up: nblocks * 256 floats, 16-byte aligned. */
+int ilt_swiglu_quant_q8k(uint64_t stream, const float* gate, const float* up, int8_t* xq, float* xd, int32_t* bsums, int64_t nblocks);
 
 /* Prefill products on the int8 matrix cores, y[t*rows + r] = W[r].x_t (+ bias[r]) for n
    tokens, each (row, token) with the decode kernel's bits (CPU: MATMUL!, batch.lisp:128-205,

@@ -75,6 +75,38 @@ def test_quant_q8k_bit_exact(dev, n):
         hip.hip_free(b)
 
 
+@pytest.mark.parametrize("n", [256, 9728, 256 * 96])
+def test_swiglu_quant_q8k_is_swiglu_then_quant_q8k(dev, n):
+    """The gated activations of a prompt chunk quantized in the launch that makes them: the blocks of "swiglu" followed
+    by "quant_q8k", which are the oracle's of its own swiglu (gates large enough for e^-x to overflow, zeros, a block
+    of zeros among them)."""
+    import ctypes as C
+    from illatio_amd import hip
+    rng = synth.make_rng(n + 7)
+    g, u = special_activations(n, rng) * 3.0, special_activations(n, rng)
+    g[:3] = (-200.0, 120.0, 0.0)
+    if n > 512:
+        u[256:512] = 0.0
+    gb, ub = hip.hip_upload_new(dev, g), hip.hip_upload_new(dev, u)
+    outs = []
+    for fused in (True, False):
+        q, d, bs = hip.hip_alloc(dev, n), hip.hip_alloc(dev, 4 * n // 256), hip.hip_alloc(dev, 4 * n // 16)
+        if fused:
+            hip.call("ilt_swiglu_quant_q8k", C.c_uint64(dev.stream), C.c_uint64(gb.ptr), C.c_uint64(ub.ptr), C.c_uint64(q.ptr), C.c_uint64(d.ptr),
+                     C.c_uint64(bs.ptr), C.c_int64(n // 256))
+            assert np.array_equal(bits(hip.hip_floats(gb, n)), bits(g))            # the gates are left as they came
+        else:
+            hip.launch(dev, "swiglu", (n + 255) // 256, 256, [gb, ub, hip.I64(n)])
+            hip.launch(dev, "quant_q8k", n // 256, 256, [gb, q, d, bs, hip.I64(n // 256)])
+        outs.append((hip.hip_download(q, np.int8, n), hip.hip_floats(d, n // 256), hip.hip_download(bs, np.int32, n // 16)))
+        for b in (q, d, bs):
+            hip.hip_free(b)
+    wq, wd, wbs = orc.quantize_q8k(orc.swiglu(g, u))
+    for got in outs:
+        assert np.array_equal(got[0], wq) and np.array_equal(bits(got[1]), bits(wd)) and np.array_equal(got[2], wbs)
+    hip.hip_free(gb); hip.hip_free(ub)
+
+
 def upload(dev, qtype, rows, cols, w):
     """The matrix as the kernels read it: Q8_0 repacked, the rest in GGUF blocks."""
     from illatio_amd import dense, hip
