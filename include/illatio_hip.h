@@ -329,8 +329,10 @@ int ilt_d4_moe_sum_rows(uint64_t stream, int d, int nu, int ntok, const float* d
      in F32-DOT16's order, the softmax's sum in double, the values added position after position.  It stands
      where the reference launches attn_decode + attn_merge / attn_prefill (dense.cu:376-727), whose partial
      sums meet in another order.  scratch: ntok * nh * ((pos0 + ntok + 3) & ~3) floats of the caller's for the raw
-     scores (two launches, for contexts up to 2048 positions, the value slice in tiles up to 8192: the scores over many workgroups, then a 16-column
-     slice of the values a workgroup), or null (one launch, a workgroup a head, any context that fits LDS).
+     scores (contexts up to 8192 positions: the scores over many workgroups, for several tokens their softmax, then
+     the values -- a chunk of tokens with heads of 64 or 128: 64 tokens x 64 positions of scores and 32 tokens x a
+     head of values a workgroup, sixteen results a thread; pointers 16-byte aligned for those), or null (one launch,
+     a workgroup a head, any context that fits LDS).
    swiglu (dense.cu:307): swiglu! on n values, a = (a / (1 + e^-a)) * b, the exponential through double. */
 /* The table qk_rope takes, for positions pos0 .. pos0 + n - 1, written to host memory (n * head_dim floats). */
 int ilt_rope_table(int head_dim, int pos0, int n, float base, float* out);
