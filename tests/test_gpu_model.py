@@ -404,6 +404,35 @@ def test_chunk_attention_with_sixteen_scores_and_chains_a_thread(dev, monkeypatc
         hip.hip_free(b)
 
 
+def test_chunk_attention_on_seeded_random_shapes(dev):
+    """The same comparison on a dozen seeded shapes: heads of 64 and 128, 1 to 12 query heads on 1 to 4 KV heads, chunks
+    of 2 to 300 tokens starting anywhere up to 3,000 positions, and one chunk that ends at position 8,192."""
+    import ctypes as C
+    from illatio_amd import hip
+    rng = synth.make_rng(4242)
+    shapes = []
+    for _ in range(11):
+        nkv = int(rng.integers(1, 5)); nh = nkv * int(rng.integers(1, 4)); hd = int(rng.choice([64, 128]))
+        shapes.append((nh, nkv, hd, int(rng.integers(0, 3000)), int(rng.integers(2, 301))))
+    shapes.append((2, 1, 128, 8192 - 70, 70))
+    P = lambda b: C.c_uint64(b.ptr if b is not None else 0)
+    for nh, nkv, hd, pos0, ntok in shapes:
+        f = lambda *sh: (rng.standard_normal(sh) * 1.5).astype(np.float32)
+        nctx = pos0 + ntok
+        q, kc, vc = (hip.hip_upload_new(dev, a) for a in (f(ntok, nh * hd), f(nctx, nkv * hd), f(nctx, nkv * hd)))
+        scratch = hip.hip_alloc(dev, 4 * ntok * nh * ((nctx + 3) & ~3))
+        ints = (C.c_int(nh), C.c_int(nkv), C.c_int(hd), C.c_int(pos0), C.c_int(ntok))
+        outs = []
+        for scr in (None, scratch):
+            out = hip.hip_upload_new(dev, np.full(ntok * nh * hd, np.nan, np.float32))
+            hip.call("ilt_attn_rows", C.c_uint64(0), P(q), P(kc), P(vc), P(out), *ints, P(scr))
+            outs.append(hip.hip_floats(out, ntok * nh * hd))
+            hip.hip_free(out)
+        assert np.array_equal(bits(outs[1]), bits(outs[0])), (nh, nkv, hd, pos0, ntok)
+        for b in (q, kc, vc, scratch):
+            hip.hip_free(b)
+
+
 def test_decode_across_position_8192(dev):
     """A context longer than the 8,192 positions the kernels with their scores in memory take: tokens at positions 8,190
     and 8,191 go through ilt_dense_decode (tiled values), those at 8,192 and 8,193 through qk_rope + attn_rows with the
