@@ -81,6 +81,13 @@ def _mat(w):
     return _Mat(w.type, w.rows, w.cols, w.qs.ptr, w.d.ptr if w.d else 0)
 
 
+HALVES_FROM, HALVES_UPTO = 256, 2048      # eval_tokens: chunks of so many tokens as two halves on two streams (0, -1: never)
+
+
+class _Work:
+    """A chunk's buffers and the device handle (its stream) their launches go to."""
+
+
 class DenseModel:
     """HOST (synth_model's dict, or the same made from a file's tensors) on DEV, with caches for NCTX positions."""
 
@@ -119,30 +126,25 @@ class DenseModel:
         rope = np.empty((nctx, hd), np.float32)
         hip.call("ilt_rope_table", C.c_int(hd), C.c_int(0), C.c_int(nctx), C.c_float(c["rope_base"]), rope.ctypes.data_as(C.c_void_p))
         self.rope = hip.hip_upload_new(dev, rope)
-        n = chunk
-        A = lambda nbytes: hip.hip_alloc(dev, nbytes)
-        self.x, self.q, self.k, self.v = A(4 * n * d), A(4 * n * self.qd), A(4 * n * self.kvd), A(4 * n * self.kvd)
-        self.att, self.fa, self.fb = A(4 * n * self.qd), A(4 * n * ffn), A(4 * n * ffn)
-        self.tokens = A(4 * n)
-        # the attention's raw scores, for the positions the kernels that keep them in memory take (up to 8192); past
-        # those a token's attention runs as one launch with its scores in LDS
-        self.scores = A(4 * n * c["nh"] * ((min(nctx, 8192) + 3) // 4 * 4))
-        self.logits = A(4 * c["vocab"])
+        self.logits = hip.hip_alloc(dev, 4 * c["vocab"])
         # a chunk's quantized activations per width, in the formats the matrices that read that width take
         # (Q8_0 blocks for Q8_0 matrices, Q8_K blocks for K-quants, as the CPU path makes them)
         reads = {d: ("wq", "wk", "wv", "gate", "up"), self.qd: ("wo",), ffn: ("down",)}
-        kinds = {}
+        self._kinds = {}
         for cols, names in reads.items():
             for L in self.layers:
                 for nm in names:
-                    kinds.setdefault(cols, set()).add("q8k" if L[nm].kquant_p() else "q8")
-        self.acts = {cols: dense.QAct(dev, n, cols, tuple(sorted(k))) for cols, k in kinds.items()}
-        self.xb, self.wb = {}, {}
+                    self._kinds.setdefault(cols, set()).add("q8k" if L[nm].kquant_p() else "q8")
+        if prefill != "exact" and any("q8" in k for k in self._kinds.values()):
+            raise ValueError("the bf16 prefill multiplies K-quant matrices; this model has Q8_0 ones")
+        # the buffers a chunk goes through the layers in (a second set, on a stream of its own, is made when two
+        # halves of a chunk first go side by side: eval_tokens)
+        self.work, self.work2 = self._work_set(dev, chunk), None
+        w = self.work
+        self.x, self.q, self.k, self.v, self.att, self.fa, self.fb = w.x, w.q, w.k, w.v, w.att, w.fa, w.fb
+        self.tokens, self.scores, self.acts, self.xb = w.tokens, w.scores, w.acts, w.xb
+        self.wb = {}
         if prefill != "exact":
-            if any("q8" in k for k in kinds.values()):
-                raise ValueError("the bf16 prefill multiplies K-quant matrices; this model has Q8_0 ones")
-            # a chunk's activations as bf16 per width (rows, or slabs for the resident copies' product)
-            self.xb = {cols: hip.hip_alloc(dev, dense.slabs_bytes(n, cols), zero=False) for cols in kinds}
             if prefill == "bf16-resident":
                 for li, L in enumerate(self.layers):
                     for nm in ("wq", "wk", "wv", "wo", "gate", "up", "down"):
@@ -159,27 +161,61 @@ class DenseModel:
                               self.fa.ptr, ptr(self.scores), self.logits.ptr)
         self.one_call = True                          # False: a token's launches one by one from here (the same launches)
 
+    def _work_set(self, dev, n):
+        """The buffers N tokens go through the layers in, their launches on DEV's stream."""
+        c = self.c
+        d, ffn = c["d"], c["ffn"]
+        A = lambda nbytes: hip.hip_alloc(dev, nbytes)
+        w = _Work()
+        w.dev, w.n = dev, n
+        w.x, w.q, w.k, w.v = A(4 * n * d), A(4 * n * self.qd), A(4 * n * self.kvd), A(4 * n * self.kvd)
+        w.att, w.fa, w.fb = A(4 * n * self.qd), A(4 * n * ffn), A(4 * n * ffn)
+        w.tokens = A(4 * n)
+        # the attention's raw scores, for the positions the kernels that keep them in memory take (up to 8192); past
+        # those a token's attention runs as one launch with its scores in LDS
+        w.scores = A(4 * n * c["nh"] * ((min(self.nctx, 8192) + 3) // 4 * 4))
+        w.acts = {cols: dense.QAct(dev, n, cols, tuple(sorted(k))) for cols, k in self._kinds.items()}
+        # a chunk's activations as bf16 per width (rows, or slabs for the resident copies' product)
+        w.xb = {} if self.prefill == "exact" else {cols: hip.hip_alloc(dev, dense.slabs_bytes(n, cols), zero=False) for cols in self._kinds}
+        return w
+
+    def _free_work(self, w):
+        for b in (w.x, w.q, w.k, w.v, w.att, w.fa, w.fb, w.tokens, w.scores):
+            hip.hip_free(b)
+        for a in w.acts.values():
+            a.free()
+        for b in w.xb.values():
+            hip.hip_free(b)
+
     def forward_n(self, tokens, logits=True):
         """TOKENS at the next positions (CUDA-FORWARD-N); the last one's logits, if LOGITS, into self.logits."""
-        dev, c, n = self.dev, self.c, len(tokens)
-        d, ffn, hd, nh, nkv, eps = c["d"], c["ffn"], c["hd"], c["nh"], c["nkv"], c["eps"]
+        n = len(tokens)
         if n < 1 or n > self.chunk or self.pos + n > self.nctx:
             raise ValueError(f"{n} tokens at position {self.pos}: the chunk holds {self.chunk}, the context {self.nctx}")
+        for _ in self._steps(tokens, self.pos, logits, self.work):
+            pass
+        self.pos += n
+        return self.logits
+
+    def _steps(self, tokens, pos, logits, W):
+        """forward_n's launches for TOKENS at positions POS.. in the work set W, as a generator: it yields ("keys", layer)
+        when a layer's keys and values are queued for the caches and ("layer", layer) when the layer is."""
+        dev, c, n = W.dev, self.c, len(tokens)
+        d, ffn, hd, nh, nkv, eps = c["d"], c["ffn"], c["hd"], c["nh"], c["nkv"], c["eps"]
         S = C.c_uint64(dev.stream)
         P = lambda b, off=0: C.c_uint64(b.ptr + off if b is not None else 0)
-        hip.hip_upload_vector(self.tokens, np.asarray(tokens, np.int32))
-        scratch = self.scores if self.pos + n <= 8192 else None
-        if n == 1 and self.one_call and scratch is not None:
-            hip.call("ilt_dense_decode", S, C.byref(self._cmodel), P(self.tokens), C.c_int(self.pos), C.c_int(1 if logits else 0))
-            self.pos += 1
-            return self.logits
-        dense.embed(dev, self.embd, self.tokens, self.x, n, d)
+        hip.hip_upload_vector(W.tokens, np.asarray(tokens, np.int32))
+        scratch = W.scores if pos + n <= 8192 else None
+        if n == 1 and self.one_call and scratch is not None and W is self.work:
+            hip.call("ilt_dense_decode", S, C.byref(self._cmodel), P(W.tokens), C.c_int(pos), C.c_int(1 if logits else 0))
+            return
+        dense.embed(dev, self.embd, W.tokens, W.x, n, d)
         fast = self.prefill != "exact" and n > 1
         slabs = self.prefill == "bf16-resident"
 
         def mul_fast(li, parts, act, acc=False):
             """PARTS (name, y, bias) on ACT's Q8_K blocks taken as bf16."""
-            xb = dense.q8k_bf16(dev, act, n, out=self.xb[act.cols], slabs=slabs)
+            xb = dense.q8k_bf16(dev, act, n, out=W.xb[act.cols], slabs=slabs)
 
             def run(nm, y, bias):
                 w = self.layers[li][nm]
@@ -203,50 +239,50 @@ class DenseModel:
         def gated():
             """The chunk's gated activations as the down product reads them: swiglu and the quantizer in one launch, or
             (a model with Q8_0 matrices) one after the other."""
-            a = dense.swiglu_quantize_act(dev, self.fa, self.fb, self.acts[ffn], n)
+            a = dense.swiglu_quantize_act(dev, W.fa, W.fb, W.acts[ffn], n)
             if a is None:
-                hip.call("ilt_swiglu", S, P(self.fa), P(self.fb), C.c_int64(n * ffn))
-                a = dense.quantize_act(dev, self.fa, self.acts[ffn], n=n)
+                hip.call("ilt_swiglu", S, P(W.fa), P(W.fb), C.c_int64(n * ffn))
+                a = dense.quantize_act(dev, W.fa, W.acts[ffn], n=n)
             return a
 
         for li, L in enumerate(self.layers):
             if n == 1:
-                dense.qkv_mul(dev, L["wq"], L["wk"], L["wv"], None, self.q, self.k, self.v, L["bq"], L["bk"], L["bv"], xf=self.x,
+                dense.qkv_mul(dev, L["wq"], L["wk"], L["wv"], None, W.q, W.k, W.v, L["bq"], L["bk"], L["bv"], xf=W.x,
                               norm=(L["attn_norm"], eps))
             else:
-                a = dense.rmsnorm_q8(dev, self.x, L["attn_norm"], self.acts[d], d, eps, n=n)
+                a = dense.rmsnorm_q8(dev, W.x, L["attn_norm"], W.acts[d], d, eps, n=n)
                 if fast:
-                    mul_fast(li, [("wq", self.q, L["bq"]), ("wk", self.k, L["bk"]), ("wv", self.v, L["bv"])], a)
+                    mul_fast(li, [("wq", W.q, L["bq"]), ("wk", W.k, L["bk"]), ("wv", W.v, L["bv"])], a)
                 else:
-                    dense.cmat_mul_n(dev, [(L["wq"], self.q, L["bq"]), (L["wk"], self.k, L["bk"]), (L["wv"], self.v, L["bv"])], a, n)
+                    dense.cmat_mul_n(dev, [(L["wq"], W.q, L["bq"]), (L["wk"], W.k, L["bk"]), (L["wv"], W.v, L["bv"])], a, n)
             if n == 1 and scratch is not None:
-                hip.call("ilt_attn_step", S, P(self.q), P(self.k), P(self.v), P(L["q_norm"]), P(L["k_norm"]), P(self.rope), P(L["kc"]), P(L["vc"]),
-                         P(self.att), C.c_int(nh), C.c_int(nkv), C.c_int(hd), C.c_int(hd), C.c_int(self.pos), C.c_float(eps),
-                         C.c_int(1 if c["neox"] else 0), P(self.scores), C.c_int(self.nctx))
+                hip.call("ilt_attn_step", S, P(W.q), P(W.k), P(W.v), P(L["q_norm"]), P(L["k_norm"]), P(self.rope), P(L["kc"]), P(L["vc"]),
+                         P(W.att), C.c_int(nh), C.c_int(nkv), C.c_int(hd), C.c_int(hd), C.c_int(pos), C.c_float(eps),
+                         C.c_int(1 if c["neox"] else 0), P(W.scores), C.c_int(self.nctx))
             else:
-                hip.call("ilt_qk_rope", S, P(self.q), P(self.k), P(self.v), P(L["q_norm"]), P(L["k_norm"]), P(self.rope), P(L["kc"]), P(L["vc"]),
-                         C.c_int(nh), C.c_int(nkv), C.c_int(hd), C.c_int(hd), C.c_int(self.pos), C.c_float(eps), C.c_int(1 if c["neox"] else 0),
+                hip.call("ilt_qk_rope", S, P(W.q), P(W.k), P(W.v), P(L["q_norm"]), P(L["k_norm"]), P(self.rope), P(L["kc"]), P(L["vc"]),
+                         C.c_int(nh), C.c_int(nkv), C.c_int(hd), C.c_int(hd), C.c_int(pos), C.c_float(eps), C.c_int(1 if c["neox"] else 0),
                          C.c_int(n))
-                hip.call("ilt_attn_rows", S, P(self.q), P(L["kc"]), P(L["vc"]), P(self.att), C.c_int(nh), C.c_int(nkv), C.c_int(hd),
-                         C.c_int(self.pos), C.c_int(n), P(scratch))
+                yield ("keys", li)
+                hip.call("ilt_attn_rows", S, P(W.q), P(L["kc"]), P(L["vc"]), P(W.att), C.c_int(nh), C.c_int(nkv), C.c_int(hd),
+                         C.c_int(pos), C.c_int(n), P(scratch))
             if n == 1:
-                dense.mv_multi(dev, [(L["wo"], self.x, None)], xf=self.att, acc=True)
-                dense.glu_mul(dev, L["gate"], L["up"], None, self.fa, xf=self.x, norm=(L["ffn_norm"], eps))
-                dense.mv_multi(dev, [(L["down"], self.x, None)], xf=self.fa, acc=True)
+                dense.mv_multi(dev, [(L["wo"], W.x, None)], xf=W.att, acc=True)
+                dense.glu_mul(dev, L["gate"], L["up"], None, W.fa, xf=W.x, norm=(L["ffn_norm"], eps))
+                dense.mv_multi(dev, [(L["down"], W.x, None)], xf=W.fa, acc=True)
             elif fast:
-                mul_fast(li, [("wo", self.x, None)], dense.quantize_act(dev, self.att, self.acts[self.qd], n=n), acc=True)
-                mul_fast(li, [("gate", self.fa, None), ("up", self.fb, None)], dense.rmsnorm_q8(dev, self.x, L["ffn_norm"], self.acts[d], d, eps, n=n))
-                mul_fast(li, [("down", self.x, None)], gated(), acc=True)
+                mul_fast(li, [("wo", W.x, None)], dense.quantize_act(dev, W.att, W.acts[self.qd], n=n), acc=True)
+                mul_fast(li, [("gate", W.fa, None), ("up", W.fb, None)], dense.rmsnorm_q8(dev, W.x, L["ffn_norm"], W.acts[d], d, eps, n=n))
+                mul_fast(li, [("down", W.x, None)], gated(), acc=True)
             else:
-                dense.cmat_mul(dev, L["wo"], dense.quantize_act(dev, self.att, self.acts[self.qd], n=n), self.x, n=n, acc=True)
-                a = dense.rmsnorm_q8(dev, self.x, L["ffn_norm"], self.acts[d], d, eps, n=n)
-                dense.cmat_mul_n(dev, [(L["gate"], self.fa, None), (L["up"], self.fb, None)], a, n)
-                dense.cmat_mul(dev, L["down"], gated(), self.x, n=n, acc=True)
-        self.pos += n
+                dense.cmat_mul(dev, L["wo"], dense.quantize_act(dev, W.att, W.acts[self.qd], n=n), W.x, n=n, acc=True)
+                a = dense.rmsnorm_q8(dev, W.x, L["ffn_norm"], W.acts[d], d, eps, n=n)
+                dense.cmat_mul_n(dev, [(L["gate"], W.fa, None), (L["up"], W.fb, None)], a, n)
+                dense.cmat_mul(dev, L["down"], gated(), W.x, n=n, acc=True)
+            yield ("layer", li)
         if logits:
-            last = hip.DBuf(self.x.ptr + 4 * (n - 1) * d, 4 * d, dev)
+            last = hip.DBuf(W.x.ptr + 4 * (n - 1) * d, 4 * d, dev)
             dense.mv_multi(dev, [(self.output, self.logits, None)], xf=last, norm=(self.output_norm, eps))
-        return self.logits
 
     def decode_greedy(self, ntokens):
         """NTOKENS greedy tokens after what the context holds, the first one picked from self.logits: every token picked
@@ -272,12 +308,58 @@ class DenseModel:
         """Forget the tokens seen: the next one is at position 0 (the caches' rows are overwritten as positions are reached)."""
         self.pos = 0
 
+    def forward_halves(self, tokens, logits=True):
+        """forward_n with TOKENS as two halves side by side, each in buffers and on a stream of its own, the second
+        half a step behind the first: its attention in a layer waits for the first half's keys and values of that
+        layer (an event), and nothing else of the one depends on the other.  A chunk of a few hundred tokens leaves
+        most of its launches with fewer workgroups than the GPU has room for (at 512 tokens V is 64 workgroups, wo and
+        down 160, of 512 that fit); the halves' launches fill each other's gaps.  Every token's results are forward_n's."""
+        n, dev = len(tokens), self.dev
+        na = (n // 2 + 127) // 128 * 128
+        if n < 2 or na >= n or n > self.chunk or self.pos + n > self.nctx or self.pos + n > 8192:
+            return self.forward_n(tokens, logits)
+        if self.work2 is None:
+            import copy
+            dev2 = copy.copy(dev)
+            dev2.stream, dev2.second = hip.hip_stream_create(dev), None
+            self.work2 = self._work_set(dev2, (self.chunk + 1) // 2)
+            self._keys_ev = [hip.hip_event_create(dev) for _ in self.layers]
+            self._side_ev = [hip.hip_event_create(dev) for _ in range(2)]
+        w2 = self.work2
+        hip.hip_event_record(self._side_ev[0], dev.stream)           # the second stream after what this one holds so far
+        hip.hip_stream_wait(w2.dev.stream, self._side_ev[0])
+        a = self._steps(tokens[:na], self.pos, False, self.work)
+        b = self._steps(tokens[na:], self.pos + na, logits, w2)
+        for li in range(len(self.layers)):
+            assert next(a) == ("keys", li)
+            hip.hip_event_record(self._keys_ev[li], dev.stream)
+            assert next(b) == ("keys", li)
+            hip.hip_stream_wait(w2.dev.stream, self._keys_ev[li])
+            assert next(a) == ("layer", li)
+            assert next(b) == ("layer", li)
+        for g in (a, b):
+            for _ in g:
+                pass
+        hip.hip_event_record(self._side_ev[1], w2.dev.stream)
+        hip.hip_stream_wait(dev.stream, self._side_ev[1])
+        self.pos += n
+        return self.logits
+
     def eval_tokens(self, tokens, logits=True):
-        """The prompt in chunks (CUDA-EVAL, cuda-dense.lisp:295-305); the logits of the last token only."""
+        """The prompt in chunks (CUDA-EVAL, cuda-dense.lisp:295-305); the logits of the last token only.  A chunk of
+        HALVES_FROM to HALVES_UPTO tokens, a power of two, goes as two halves side by side (forward_halves)."""
         tokens = list(tokens)
         for i in range(0, len(tokens), self.chunk):
             part = tokens[i:i + self.chunk]
-            self.forward_n(part, logits=logits and i + len(part) >= len(tokens))
+            want = logits and i + len(part) >= len(tokens)
+            npart = len(part)
+            # (measured on the Qwen3-4B shape: 256 tokens 14.6 -> 14.0 ms, 512 18.7 -> 17.9, 1,024 33.0 -> 30.2, 2,048 78.7 -> 75.4;
+            # halves of 384 or 768 tokens lose what they gain or more -- 768 tokens 25.5 -> 27.0 ms --, so powers of two only;
+            # the bf16 products' results depend on how many tokens a launch has: they stay whole)
+            if self.prefill == "exact" and HALVES_FROM <= npart <= HALVES_UPTO and npart & (npart - 1) == 0:
+                self.forward_halves(part, logits=want)
+            else:
+                self.forward_n(part, logits=want)
 
     def argmax(self):
         """The greedy token of self.logits (ARGMAX, model.lisp:464-468: the first of equal ones)."""
@@ -290,9 +372,10 @@ class DenseModel:
         if self.output is not self.embd:
             self.output.free()
         self.embd.free()
-        for b in (self.output_norm, self.rope, self.x, self.q, self.k, self.v, self.att, self.fa, self.fb, self.tokens, self.logits, self.scores):
+        for b in (self.output_norm, self.rope, self.logits):
             hip.hip_free(b)
-        for a in self.acts.values():
-            a.free()
-        for b in list(self.xb.values()) + list(self.wb.values()):
+        self._free_work(self.work)
+        if self.work2 is not None:
+            self._free_work(self.work2)
+        for b in self.wb.values():
             hip.hip_free(b)
