@@ -81,7 +81,7 @@ def _mat(w):
     return _Mat(w.type, w.rows, w.cols, w.qs.ptr, w.d.ptr if w.d else 0)
 
 
-HALVES_FROM, HALVES_UPTO = 256, 2048      # eval_tokens: chunks of so many tokens as two halves on two streams (0, -1: never)
+PARTS_FROM, PARTS_UPTO = 256, 2048      # eval_tokens: chunks of so many tokens as parts side by side on streams of their own (0, -1: never)
 
 
 class _Work:
@@ -137,9 +137,9 @@ class DenseModel:
                     self._kinds.setdefault(cols, set()).add("q8k" if L[nm].kquant_p() else "q8")
         if prefill != "exact" and any("q8" in k for k in self._kinds.values()):
             raise ValueError("the bf16 prefill multiplies K-quant matrices; this model has Q8_0 ones")
-        # the buffers a chunk goes through the layers in (a second set, on a stream of its own, is made when two
-        # halves of a chunk first go side by side: eval_tokens)
-        self.work, self.work2 = self._work_set(dev, chunk), None
+        # the buffers a chunk goes through the layers in (more sets, each on a stream of its own, are made when the
+        # parts of a chunk first go side by side: eval_tokens)
+        self.work, self.more_work, self._keys_ev, self._join_ev = self._work_set(dev, chunk), [], [], []
         w = self.work
         self.x, self.q, self.k, self.v, self.att, self.fa, self.fb = w.x, w.q, w.k, w.v, w.att, w.fa, w.fb
         self.tokens, self.scores, self.acts, self.xb = w.tokens, w.scores, w.acts, w.xb
@@ -308,56 +308,65 @@ class DenseModel:
         """Forget the tokens seen: the next one is at position 0 (the caches' rows are overwritten as positions are reached)."""
         self.pos = 0
 
-    def forward_halves(self, tokens, logits=True):
-        """forward_n with TOKENS as two halves side by side, each in buffers and on a stream of its own, the second
-        half a step behind the first: its attention in a layer waits for the first half's keys and values of that
-        layer (an event), and nothing else of the one depends on the other.  A chunk of a few hundred tokens leaves
+    def forward_parts(self, tokens, logits=True, k=2):
+        """forward_n with TOKENS as K parts side by side, each in buffers and on a stream of its own, every part a step
+        behind the one before it: its attention in a layer waits for the earlier parts' keys and values of that layer
+        (an event each), and nothing else of one part depends on another.  A chunk of a few hundred tokens leaves
         most of its launches with fewer workgroups than the GPU has room for (at 512 tokens V is 64 workgroups, wo and
-        down 160, of 512 that fit); the halves' launches fill each other's gaps.  Every token's results are forward_n's."""
+        down 160, of 512 that fit), and while one part is in its attention (vector ALU) another is in its products
+        (matrix cores): the parts' launches fill each other's gaps.  Every token's results are forward_n's."""
         n, dev = len(tokens), self.dev
-        na = (n // 2 + 127) // 128 * 128
-        if n < 2 or na >= n or n > self.chunk or self.pos + n > self.nctx or self.pos + n > 8192:
+        per = ((n + k - 1) // k + 127) // 128 * 128
+        if k < 2 or per * (k - 1) >= n or n > self.chunk or self.pos + n > self.nctx or self.pos + n > 8192:
             return self.forward_n(tokens, logits)
-        if self.work2 is None:
+        while len(self.more_work) < k - 1:
             import copy
             dev2 = copy.copy(dev)
             dev2.stream, dev2.second = hip.hip_stream_create(dev), None
-            self.work2 = self._work_set(dev2, (self.chunk + 1) // 2)
-            self._keys_ev = [hip.hip_event_create(dev) for _ in self.layers]
-            self._side_ev = [hip.hip_event_create(dev) for _ in range(2)]
-        w2 = self.work2
-        hip.hip_event_record(self._side_ev[0], dev.stream)           # the second stream after what this one holds so far
-        hip.hip_stream_wait(w2.dev.stream, self._side_ev[0])
-        a = self._steps(tokens[:na], self.pos, False, self.work)
-        b = self._steps(tokens[na:], self.pos + na, logits, w2)
+            self.more_work.append(self._work_set(dev2, (self.chunk + 1) // 2))
+        while len(self._keys_ev) < k:
+            self._keys_ev.append([hip.hip_event_create(dev) for _ in self.layers])
+            self._join_ev.append(hip.hip_event_create(dev))
+        works = [self.work] + self.more_work[:k - 1]
+        hip.hip_event_record(self._join_ev[0], dev.stream)            # the other streams after what this one holds so far
+        for w in works[1:]:
+            hip.hip_stream_wait(w.dev.stream, self._join_ev[0])
+        gens = [self._steps(tokens[j * per:(j + 1) * per], self.pos + j * per, logits and j == k - 1, works[j]) for j in range(k)]
         for li in range(len(self.layers)):
-            assert next(a) == ("keys", li)
-            hip.hip_event_record(self._keys_ev[li], dev.stream)
-            assert next(b) == ("keys", li)
-            hip.hip_stream_wait(w2.dev.stream, self._keys_ev[li])
-            assert next(a) == ("layer", li)
-            assert next(b) == ("layer", li)
-        for g in (a, b):
+            for j in range(k):
+                assert next(gens[j]) == ("keys", li)
+                if j < k - 1:
+                    hip.hip_event_record(self._keys_ev[j][li], works[j].dev.stream)
+                for i in range(j):
+                    hip.hip_stream_wait(works[j].dev.stream, self._keys_ev[i][li])
+            for j in range(k):
+                assert next(gens[j]) == ("layer", li)
+        for g in gens:
             for _ in g:
                 pass
-        hip.hip_event_record(self._side_ev[1], w2.dev.stream)
-        hip.hip_stream_wait(dev.stream, self._side_ev[1])
+        for j in range(1, k):
+            hip.hip_event_record(self._join_ev[j], works[j].dev.stream)
+            hip.hip_stream_wait(dev.stream, self._join_ev[j])
         self.pos += n
         return self.logits
 
     def eval_tokens(self, tokens, logits=True):
         """The prompt in chunks (CUDA-EVAL, cuda-dense.lisp:295-305); the logits of the last token only.  A chunk of
-        HALVES_FROM to HALVES_UPTO tokens, a power of two, goes as two halves side by side (forward_halves)."""
+        PARTS_FROM to PARTS_UPTO tokens, a power of two, goes as two or four parts side by side (forward_parts)."""
         tokens = list(tokens)
         for i in range(0, len(tokens), self.chunk):
             part = tokens[i:i + self.chunk]
             want = logits and i + len(part) >= len(tokens)
             npart = len(part)
-            # (measured on the Qwen3-4B shape: 256 tokens 14.6 -> 14.0 ms, 512 18.7 -> 17.9, 1,024 33.0 -> 30.2, 2,048 78.7 -> 75.4;
+            # (measured on the Qwen3-4B shape: 256 tokens 14.6 -> 14.0 ms, 512 18.7 -> 17.9, 1,024 33.0 -> 30.2 as two halves,
+            # 35.4 as four quarters; 2,048 78.8 -> 76.7 as halves, 72.1 as quarters: parts of 512 tokens, or two;
             # halves of 384 or 768 tokens lose what they gain or more -- 768 tokens 25.5 -> 27.0 ms --, so powers of two only;
             # the bf16 products' results depend on how many tokens a launch has: they stay whole)
-            if self.prefill == "exact" and HALVES_FROM <= npart <= HALVES_UPTO and npart & (npart - 1) == 0:
-                self.forward_halves(part, logits=want)
+            # (a chunk of 512 tokens far into a long prompt is mostly attention, and its halves gain nothing: 4,096 tokens in
+            # chunks of 512 256.5 -> 258-266 ms)
+            if (self.prefill == "exact" and PARTS_FROM <= npart <= PARTS_UPTO and npart & (npart - 1) == 0
+                    and (npart >= 1024 or self.pos < 1024)):
+                self.forward_parts(part, logits=want, k=max(2, npart // 512))
             else:
                 self.forward_n(part, logits=want)
 
@@ -375,7 +384,7 @@ class DenseModel:
         for b in (self.output_norm, self.rope, self.logits):
             hip.hip_free(b)
         self._free_work(self.work)
-        if self.work2 is not None:
-            self._free_work(self.work2)
+        for w in self.more_work:
+            self._free_work(w)
         for b in self.wb.values():
             hip.hip_free(b)

@@ -404,23 +404,27 @@ def test_chunk_attention_with_sixteen_scores_and_chains_a_thread(dev, monkeypatc
         hip.hip_free(b)
 
 
-def test_a_chunk_as_two_halves_side_by_side(dev):
-    """forward_halves -- a chunk's two halves on two streams, the second half's attention waiting for the first half's
-    keys layer by layer -- leaves forward_n's logits and caches, bit for bit: halves of 128 + 128, of 256 + 44 (the second
-    half on the products for few tokens), and a second chunk whose halves see the first chunk's positions."""
+def test_a_chunk_as_parts_side_by_side(dev):
+    """forward_parts -- a chunk's halves or quarters on streams of their own, a part's attention waiting for the earlier
+    parts' keys layer by layer -- leaves forward_n's logits and caches, bit for bit: halves of 128 + 128, of 256 + 44 (the
+    second half on the products for few tokens), a second chunk whose halves see the first chunk's positions, and
+    quarters of 128."""
     from illatio_amd import hip, model
     host = model.synth_model(12, d=512, ffn=1024, nh=8, nkv=2, hd=64, nl=3, vocab=700)
     c = host["config"]
     rng = synth.make_rng(77)
     kvd = c["nkv"] * c["hd"]
-    for nprompt, chunk in ((256, 256), (300, 300), (600, 300)):
+    for nprompt, chunk, k in ((256, 256, 2), (300, 300, 2), (600, 300, 2), (512, 512, 4), (1000, 500, 4)):
         prompt = rng.integers(0, c["vocab"], nprompt).tolist()
         res = []
         for halves in (True, False):
             m = model.DenseModel(dev, host, nctx=nprompt + 8, chunk=chunk)
             for i in range(0, nprompt, chunk):
                 part = prompt[i:i + chunk]
-                (m.forward_halves if halves else m.forward_n)(part, logits=i + chunk >= nprompt)
+                if halves:
+                    m.forward_parts(part, logits=i + chunk >= nprompt, k=k)
+                else:
+                    m.forward_n(part, logits=i + chunk >= nprompt)
             hip.hip_sync(dev)
             assert m.pos == nprompt
             res.append([hip.hip_floats(m.logits, c["vocab"])] + [hip.hip_floats(m.layers[li][nm], nprompt * kvd) for li in (0, 2) for nm in ("kc", "vc")])
