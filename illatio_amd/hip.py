@@ -254,6 +254,10 @@ def hip_stream_create(dev):
     return s.value
 
 
+def hip_stream_destroy(stream):
+    call("ilt_stream_destroy", C.c_uint64(stream))
+
+
 def hip_stream_wait(stream, event):
     call("ilt_stream_wait_event", C.c_uint64(stream), C.c_uint64(event))
 

@@ -384,7 +384,15 @@ class DenseModel:
         for b in (self.output_norm, self.rope, self.logits):
             hip.hip_free(b)
         self._free_work(self.work)
-        for w in self.more_work:
+        for w in self.more_work:                      # (hip_free waits for the device: nothing is in flight on these streams)
             self._free_work(w)
+            if getattr(w.dev, "second", None) is not None:
+                hip.hip_stream_destroy(w.dev.second)
+                hip.hip_event_destroy(w.dev.forked)
+                hip.hip_event_destroy(w.dev.joined)
+            hip.hip_stream_destroy(w.dev.stream)
+        for e in [e for evs in self._keys_ev for e in evs] + self._join_ev:
+            hip.hip_event_destroy(e)
+        self.more_work, self._keys_ev, self._join_ev = [], [], []
         for b in self.wb.values():
             hip.hip_free(b)
