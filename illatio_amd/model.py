@@ -81,6 +81,7 @@ def _mat(w):
     return _Mat(w.type, w.rows, w.cols, w.qs.ptr, w.d.ptr if w.d else 0)
 
 
+PARTS_WORK = 1e10
 PARTS_FROM, PARTS_UPTO = 256, 2048      # eval_tokens: chunks of so many tokens as parts side by side on streams of their own (0, -1: never)
 
 
@@ -364,9 +365,16 @@ class DenseModel:
             # the bf16 products' results depend on how many tokens a launch has: they stay whole)
             # (a chunk of 512 tokens far into a long prompt is mostly attention, and its halves gain nothing: 4,096 tokens in
             # chunks of 512 256.5 -> 258-266 ms)
+            # (and a small model's launches are over before the next is queued, so twice as many of them only cost: the
+            # Qwen2.5-0.5B shape's 512-token prompt 7.7 -> 10.6 ms as halves; a part must bring PARTS_WORK products of a
+            # weight and a token to a layer: the Qwen3-4B shape's halves of 128 tokens bring 1.3e10, the 0.5B shape's
+            # halves of 256 tokens 3.8e9)
+            k = max(2, npart // 512)
+            c = self.c
+            layer_weights = c["d"] * (2 * self.qd + 2 * self.kvd + 3 * c["ffn"])
             if (self.prefill == "exact" and PARTS_FROM <= npart <= PARTS_UPTO and npart & (npart - 1) == 0
-                    and (npart >= 1024 or self.pos < 1024)):
-                self.forward_parts(part, logits=want, k=max(2, npart // 512))
+                    and (npart >= 1024 or self.pos < 1024) and (npart // k) * layer_weights >= PARTS_WORK):
+                self.forward_parts(part, logits=want, k=k)
             else:
                 self.forward_n(part, logits=want)
 
