@@ -1405,7 +1405,13 @@ hipError_t ilt_k_attn_rows(const float* q, const float* kc, const float* vc, flo
       // kernel of sixteen lanes a score (tests)
       const char* quad = getenv("ILT_ATTN_QUAD");
       const bool qaligned = ((((uintptr_t)q) | ((uintptr_t)kc)) & 15) == 0;
-      if ((hd == 128 || hd == 64) && qaligned && !(quad && (quad[0] == '0' || quad[0] == 'v'))) {
+      // (either kernel where it fills the GPU: 14 heads of 64 on 512 tokens are 112 workgroups of the values kernel,
+      // and the kernel of a chain a thread, 448 workgroups, takes 59 us for the chunk's attention where this one took 78;
+      // "ILT_ATTN_QUAD=1": whatever the shape)
+      const bool forced = quad && quad[0] == '1';
+      const long long swgs = (long long)nh * ((ctx + 63) / 64) * ((ntok + 63) / 64);
+      const long long vwgs = (long long)nh * ((ntok + (hd == 128 ? 31 : 63)) / (hd == 128 ? 32 : 64));
+      if ((hd == 128 || hd == 64) && qaligned && !(quad && (quad[0] == '0' || quad[0] == 'v')) && (forced || swgs >= 256)) {
         static bool qset[64] = {};
         const size_t qsmem = sizeof(float) * 2 * 64 * (size_t)(hd + 4);
         if (!qset[dev]) {
@@ -1425,7 +1431,7 @@ hipError_t ilt_k_attn_rows(const float* q, const float* kc, const float* vc, flo
       // sixteen chains a thread for heads of 64 or 128 columns (16-byte loads and stores: of scratch, vc and out);
       // "ILT_ATTN_QUAD=0": the kernel of one chain a thread (tests)
       const bool aligned = ((((uintptr_t)scratch) | ((uintptr_t)vc) | ((uintptr_t)out)) & 15) == 0;
-      if ((hd == 128 || hd == 64) && aligned && !(quad && quad[0] == '0')) {
+      if ((hd == 128 || hd == 64) && aligned && !(quad && quad[0] == '0') && (forced || vwgs >= 192)) {
         if (hd == 128)
           hipLaunchKernelGGL(attn_values_quad_kernel<128>, dim3(nh, (ntok + 31) / 32), dim3(256), 0, st, scratch, vc, out, nh, nkv, pos0, ntok, smax);
         else
