@@ -362,17 +362,21 @@ class DenseModel:
             # (measured on the Qwen3-4B shape: 256 tokens 14.6 -> 14.0 ms, 512 18.7 -> 17.9, 1,024 33.0 -> 30.2 as two halves,
             # 35.4 as four quarters; 2,048 78.8 -> 76.7 as halves, 72.1 as quarters: parts of 512 tokens, or two;
             # halves of 384 or 768 tokens lose what they gain or more -- 768 tokens 25.5 -> 27.0 ms --, so powers of two only;
-            # the bf16 products' results depend on how many tokens a launch has: they stay whole)
+            # the bf16 products: below)
             # (a chunk of 512 tokens far into a long prompt is mostly attention, and its halves gain nothing: 4,096 tokens in
             # chunks of 512 256.5 -> 258-266 ms)
             # (and a small model's launches are over before the next is queued, so twice as many of them only cost: the
             # Qwen2.5-0.5B shape's 512-token prompt 7.7 -> 10.6 ms as halves; a part must bring PARTS_WORK products of a
             # weight and a token to a layer: the Qwen3-4B shape's halves of 128 tokens bring 1.3e10, the 0.5B shape's
             # halves of 256 tokens 3.8e9)
-            k = max(2, npart // 512)
+            # (the bf16 products from the quantized matrices: two halves from 1,024 tokens on -- 1,024 tokens 29.5 -> 26.1 ms,
+            # 2,048 66.7 -> 62.7; quarters lose, and so do halves of a 512-token chunk; their sums' order depends on a
+            # launch's token count with or without parts.  From resident copies: 28.4 -> 27.2 and 62.7 -> 62.1, left whole)
+            exact = self.prefill == "exact"
+            k = max(2, npart // 512) if exact else 2
             c = self.c
             layer_weights = c["d"] * (2 * self.qd + 2 * self.kvd + 3 * c["ffn"])
-            if (self.prefill == "exact" and PARTS_FROM <= npart <= PARTS_UPTO and npart & (npart - 1) == 0
+            if ((exact or (self.prefill == "bf16" and npart >= 1024)) and PARTS_FROM <= npart <= PARTS_UPTO and npart & (npart - 1) == 0
                     and (npart >= 1024 or self.pos < 1024) and (npart // k) * layer_weights >= PARTS_WORK):
                 self.forward_parts(part, logits=want, k=k)
             else:

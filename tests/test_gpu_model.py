@@ -433,6 +433,31 @@ def test_a_chunk_as_parts_side_by_side(dev):
             assert np.array_equal(bits(a), bits(b)), (nprompt, chunk)
 
 
+def test_bf16_chunk_as_halves_stays_within_the_bf16_roundings(dev):
+    """The bf16 prefill through forward_parts: the halves' products are other launches (other token counts, so the
+    split over the columns may fall otherwise), not other numbers -- the first layer's caches within a few bf16 roundings of the whole
+    chunk's, the logits within 2e-2 of their spread."""
+    from illatio_amd import hip, model
+    host = model.synth_model(13, d=512, ffn=1024, nh=8, nkv=2, hd=64, nl=3, vocab=700)
+    c = host["config"]
+    rng = synth.make_rng(78)
+    nprompt, kvd = 1024, c["nkv"] * c["hd"]
+    prompt = rng.integers(0, c["vocab"], nprompt).tolist()
+    res = []
+    for parts in (True, False):
+        m = model.DenseModel(dev, host, nctx=nprompt + 8, chunk=nprompt, prefill="bf16")
+        if parts:
+            m.forward_parts(prompt, k=2)
+        else:
+            m.forward_n(prompt)
+        hip.hip_sync(dev)
+        res.append((hip.hip_floats(m.logits, c["vocab"]), hip.hip_floats(m.layers[0]["kc"], nprompt * kvd), hip.hip_floats(m.layers[0]["vc"], nprompt * kvd)))
+        m.free()
+    (la, ka, va), (lb, kb, vb) = res
+    assert np.abs(ka - kb).max() <= 2e-2 * np.abs(kb).max() and np.abs(va - vb).max() <= 2e-2 * np.abs(vb).max()
+    assert np.abs(la - lb).max() <= 2e-2 * lb.std(), (np.abs(la - lb).max(), lb.std())
+
+
 def test_chunk_attention_on_seeded_random_shapes(dev):
     """The same comparison on a dozen seeded shapes: heads of 64 and 128, 1 to 12 query heads on 1 to 4 KV heads, chunks
     of 2 to 300 tokens starting anywhere up to 3,000 positions, and one chunk that ends at position 8,192."""
