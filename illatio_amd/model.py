@@ -82,7 +82,7 @@ def _mat(w):
 
 
 PARTS_WORK = 1e10
-PARTS_FROM, PARTS_UPTO = 256, 2048      # eval_tokens: chunks of so many tokens as parts side by side on streams of their own (0, -1: never)
+PARTS_FROM, PARTS_UPTO = 256, 4096      # eval_tokens: chunks of so many tokens as parts side by side on streams of their own (0, -1: never)
 
 
 class _Work:
@@ -324,7 +324,7 @@ class DenseModel:
             import copy
             dev2 = copy.copy(dev)
             dev2.stream, dev2.second = hip.hip_stream_create(dev), None
-            self.more_work.append(self._work_set(dev2, (self.chunk + 1) // 2))
+            self.more_work.append(self._work_set(dev2, ((self.chunk + 1) // 2 + 127) // 128 * 128))      # (a part: up to half a chunk, rounded up to whole tiles of 128 tokens)
         while len(self._keys_ev) < k:
             self._keys_ev.append([hip.hip_event_create(dev) for _ in self.layers])
             self._join_ev.append(hip.hip_event_create(dev))
@@ -353,31 +353,32 @@ class DenseModel:
 
     def eval_tokens(self, tokens, logits=True):
         """The prompt in chunks (CUDA-EVAL, cuda-dense.lisp:295-305); the logits of the last token only.  A chunk of
-        PARTS_FROM to PARTS_UPTO tokens, a power of two, goes as two or four parts side by side (forward_parts)."""
+        PARTS_FROM to PARTS_UPTO tokens goes as two or four parts side by side where that was measured to gain
+        (forward_parts)."""
         tokens = list(tokens)
         for i in range(0, len(tokens), self.chunk):
             part = tokens[i:i + self.chunk]
             want = logits and i + len(part) >= len(tokens)
             npart = len(part)
-            # (measured on the Qwen3-4B shape: 256 tokens 14.6 -> 14.0 ms, 512 18.7 -> 17.9, 1,024 33.0 -> 30.2 as two halves,
-            # 35.4 as four quarters; 2,048 78.8 -> 76.7 as halves, 72.1 as quarters: parts of 512 tokens, or two;
-            # halves of 384 or 768 tokens lose what they gain or more -- 768 tokens 25.5 -> 27.0 ms --, so powers of two only;
-            # the bf16 products: below)
-            # (a chunk of 512 tokens far into a long prompt is mostly attention, and its halves gain nothing: 4,096 tokens in
-            # chunks of 512 256.5 -> 258-266 ms)
-            # (and a small model's launches are over before the next is queued, so twice as many of them only cost: the
-            # Qwen2.5-0.5B shape's 512-token prompt 7.7 -> 10.6 ms as halves; a part must bring PARTS_WORK products of a
-            # weight and a token to a layer: the Qwen3-4B shape's halves of 128 tokens bring 1.3e10, the 0.5B shape's
-            # halves of 256 tokens 3.8e9)
-            # (the bf16 products from the quantized matrices: two halves from 1,024 tokens on -- 1,024 tokens 29.5 -> 26.1 ms,
-            # 2,048 66.7 -> 62.7; quarters lose, and so do halves of a 512-token chunk; their sums' order depends on a
-            # launch's token count with or without parts.  From resident copies: 28.4 -> 27.2 and 62.7 -> 62.1, left whole)
+            # Parts, measured on the Qwen3-4B shape (whole -> parts): 256 tokens 14.6 -> 14.0 ms, 512 18.7 -> 17.9 as halves;
+            # 900 31.7 -> 28.0, 1,024 33.0 -> 30.2, 1,100 37.6 -> 33.8, 1,280 42.9 -> 40.8, 1,536 53.3 -> 50.4, 1,800 68.2 -> 64.0 as
+            # halves (thirds and quarters of those lose); 2,048 78.8 -> 76.7 as halves, 72.1 as quarters.  Between 256 and 900
+            # tokens only the powers of two gain (384 +8 %, but 448 -2 %, 640 0, 768 -1 to -6 %).  A chunk of 512 tokens far
+            # into a long prompt is mostly attention, and its halves gain nothing (4,096 tokens in chunks of 512: 256.5 ->
+            # 258-266 ms).  The bf16 products from the quantized matrices: two halves from 1,024 tokens on (1,024 tokens
+            # 29.5 -> 26.1 ms, 2,048 66.7 -> 62.7; quarters lose, and so do halves of a 512-token chunk; their sums' order
+            # depends on a launch's token count with or without parts); from resident copies 28.4 -> 27.2 and 62.7 -> 62.1:
+            # left whole.  And a small model's launches are over before the next is queued, so twice as many of them only
+            # cost (the Qwen2.5-0.5B shape's 512-token prompt 7.7 -> 10.6 ms as halves): a part must bring PARTS_WORK products
+            # of a weight and a token to a layer (the Qwen3-4B shape's halves of 128 tokens bring 1.3e10, the 0.5B shape's
+            # halves of 256 tokens 3.8e9).
             exact = self.prefill == "exact"
-            k = max(2, npart // 512) if exact else 2
+            k = 4 if exact and npart >= 2048 else 2
             c = self.c
             layer_weights = c["d"] * (2 * self.qd + 2 * self.kvd + 3 * c["ffn"])
-            if ((exact or (self.prefill == "bf16" and npart >= 1024)) and PARTS_FROM <= npart <= PARTS_UPTO and npart & (npart - 1) == 0
-                    and (npart >= 1024 or self.pos < 1024) and (npart // k) * layer_weights >= PARTS_WORK):
+            fits = npart >= 896 or (npart & (npart - 1) == 0 and self.pos < 1024)
+            if ((exact and fits) or (self.prefill == "bf16" and npart >= 1024)) and PARTS_FROM <= npart <= PARTS_UPTO \
+                    and (npart // k) * layer_weights >= PARTS_WORK:
                 self.forward_parts(part, logits=want, k=k)
             else:
                 self.forward_n(part, logits=want)

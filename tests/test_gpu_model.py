@@ -414,7 +414,7 @@ def test_a_chunk_as_parts_side_by_side(dev):
     c = host["config"]
     rng = synth.make_rng(77)
     kvd = c["nkv"] * c["hd"]
-    for nprompt, chunk, k in ((256, 256, 2), (300, 300, 2), (600, 300, 2), (512, 512, 4), (1000, 500, 4)):
+    for nprompt, chunk, k in ((256, 256, 2), (300, 300, 2), (600, 300, 2), (512, 512, 4), (1000, 500, 4), (1000, 1000, 2)):
         prompt = rng.integers(0, c["vocab"], nprompt).tolist()
         res = []
         for halves in (True, False):
